@@ -1,0 +1,243 @@
+/* qwhip.h - C ABI of libqwhip: the MI355X (gfx950) HIP HAL and quantized-matmul
+ * launchers that stand where the reference's Metal HAL + QWGEMM kernels stand.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers and sizes, returns a
+ * status code (0 = ok), never aborts and never launches partially: all checks
+ * run before the first enqueue (the reference throws its typed errors before
+ * any bind, Sources/Operators/QWGEMM/QWGemm.swift:66-80).  Device pointers are
+ * caller-owned; the library never frees caller memory and allocates nothing
+ * inside a launcher.  Launchers enqueue on the given stream and return; order
+ * inside a stream replaces the reference's encoder barriers.
+ *
+ * Paths cited below are relative to the reference checkout.
+ */
+#ifndef QWHIP_H
+#define QWHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes: map 1:1 onto the Swift error cases ---------------------
+ * QWGemmError {badWeights, badShape, badGeometry, f3Blocked}  (QWGemm.swift:66-80)
+ * QWHalError.kernelMissing / deviceUnavailable               (Sources/Foundation/QWHAL/QWHal.swift:60-77) */
+typedef int32_t qwhip_status;
+enum {
+    QWHIP_OK = 0,
+    QWHIP_E_BAD_WEIGHTS = 1,    /* QWGemmError.badWeights  */
+    QWHIP_E_BAD_SHAPE = 2,      /* QWGemmError.badShape    */
+    QWHIP_E_BAD_GEOMETRY = 3,   /* QWGemmError.badGeometry */
+    QWHIP_E_BLOCKED = 4,        /* QWGemmError.f3Blocked / plan backend .blocked */
+    QWHIP_E_KERNEL_MISSING = 5, /* QWHalError.kernelMissing(name) */
+    QWHIP_E_DEVICE = 6,         /* QWHalError.deviceUnavailable / any HIP runtime failure */
+    QWHIP_E_BASIS = 7,          /* activation basis does not fit the container (QWHal.swift:227-232) */
+    QWHIP_E_NULL = 8,           /* a required pointer is NULL */
+    QWHIP_E_ALLOC = 9           /* qwhip_malloc failed */
+};
+
+/* ---- element types (mirror of QWDType, Sources/Foundation/QWCore/QWDType.swift) */
+enum { QWHIP_F32 = 0, QWHIP_F16 = 1, QWHIP_BF16 = 2, QWHIP_I32 = 3 };
+
+/* ---- container kinds (QWWeightView.ContainerKind, Sources/Foundation/QWAlloc/QWWeightView.swift:11-16) */
+enum {
+    QWHIP_KIND_HQ4_G32_M5 = 0,    /* .incumbentHQ4G32: 20-byte magic-bias blocks, rotated */
+    QWHIP_KIND_ROTATED_HQ = 1,    /* .rotatedHQ(bits, group): bit-stream blocks, rotated  */
+    QWHIP_KIND_NATIVE_AFFINE = 2  /* .nativeAffine(bits, group): bit-stream blocks, standard basis */
+};
+
+/* Non-owning view of one quantized bank [n rows][k/group blocks], row-major
+ * (QWWeightView, QWWeightView.swift:86-118).  `bytes` is what the caller's
+ * region holds from `blocks` on; a view is valid when n > 0, k > 0,
+ * k % group == 0, (bits, group) is a supported pair and
+ * bytes >= n * (k/group) * (4 + group*bits/8). */
+typedef struct qwhip_weight_view {
+    const void* blocks; /* device pointer, >= 4-byte aligned */
+    uint64_t bytes;
+    uint32_t n;
+    uint32_t k;
+    uint32_t kind;  /* QWHIP_KIND_* */
+    uint32_t bits;  /* 4 for HQ4_G32_M5; {2,3,4,6,8} for blocks (kernels: {4, 8}) */
+    uint32_t group; /* 32 for HQ4_G32_M5; {32,64,128,256} for blocks */
+} qwhip_weight_view;
+
+typedef struct qwhip_device_s* qwhip_device_t; /* stands for QWHal */
+typedef struct qwhip_stream_s* qwhip_stream_t; /* stands for an open command encoder */
+typedef struct qwhip_event_s* qwhip_event_t;
+
+typedef struct qwhip_caps {
+    char name[64];
+    char arch[32];         /* "gfx950" */
+    uint32_t compute_units;
+    uint32_t wavefront;    /* 64 */
+    uint32_t lds_bytes;    /* per workgroup */
+    uint32_t l2_bytes;
+    uint64_t hbm_bytes;
+    uint32_t clock_khz;
+    uint32_t has_mfma_f16; /* the reference's caps.isMetal4TensorCapable (QWHal.swift:81-130) */
+} qwhip_caps;
+
+/* ---- HAL: device, streams, memory, events --------------------------------- */
+/* QWHal.init (QWHal.swift:133-232): opens device `ordinal`, refuses a device that is not gfx950. */
+qwhip_status qwhip_device_create(int32_t ordinal, qwhip_device_t* out);
+qwhip_status qwhip_device_destroy(qwhip_device_t dev);
+qwhip_status qwhip_device_caps(qwhip_device_t dev, qwhip_caps* out);
+/* hal.begin() / hal.end() (QWHal.swift:325-378): a stream is the encoder the launchers take. */
+qwhip_status qwhip_stream_create(qwhip_device_t dev, qwhip_stream_t* out);
+qwhip_status qwhip_stream_destroy(qwhip_stream_t s);
+qwhip_status qwhip_stream_sync(qwhip_stream_t s); /* waitUntilCompleted (QWHal.swift:352-360) */
+/* The native hipStream_t behind a stream handle, for callers that time or capture on it. */
+void* qwhip_stream_native(qwhip_stream_t s);
+/* Arena backing store (QWArena, Sources/Foundation/QWAlloc/QWArena.swift:161-193): 256-byte aligned device memory. */
+qwhip_status qwhip_malloc(qwhip_device_t dev, size_t bytes, void** out);
+qwhip_status qwhip_free(qwhip_device_t dev, void* p);
+qwhip_status qwhip_memcpy_h2d(qwhip_stream_t s, void* dst, const void* src, size_t bytes); /* synchronous */
+qwhip_status qwhip_memcpy_d2h(qwhip_stream_t s, void* dst, const void* src, size_t bytes); /* synchronous */
+qwhip_status qwhip_memcpy_d2d(qwhip_stream_t s, void* dst, const void* src, size_t bytes); /* async on s */
+qwhip_status qwhip_fill_u32(qwhip_stream_t s, void* dst, uint32_t value, size_t count);    /* async fill kernel */
+/* GPU timestamps (QWStageCounter, Sources/Foundation/QWHAL/QWStageCounter.swift:1-40). */
+qwhip_status qwhip_event_create(qwhip_device_t dev, qwhip_event_t* out);
+qwhip_status qwhip_event_destroy(qwhip_event_t e);
+qwhip_status qwhip_event_record(qwhip_event_t e, qwhip_stream_t s);
+qwhip_status qwhip_event_elapsed_ms(qwhip_event_t start, qwhip_event_t stop, float* ms); /* syncs on stop */
+/* hal.pipeline(name) (QWHal.swift:291-322): 0 when `name` (a reference kernel name such as
+ * "qwg_gemv_q4g_dx_h16_t4") has a launcher here, else QWHIP_E_KERNEL_MISSING.  `launcher`, when
+ * not NULL, receives the name of the qwhip_* entry point that serves it. */
+qwhip_status qwhip_kernel_lookup(const char* name, const char** launcher);
+/* Text of the last error raised on the calling thread ("" when none). */
+const char* qwhip_last_error(void);
+const char* qwhip_status_name(qwhip_status st);
+
+/* ---- container helpers ---------------------------------------------------- */
+/* QWAQBlock.bytesIfBlockSupported (Sources/Foundation/QWQuant/QWAQBlock.swift:48-86): 0 when unsupported. */
+uint32_t qwhip_block_bytes(uint32_t kind, uint32_t bits, uint32_t group);
+/* QWWeightView.init? (QWWeightView.swift:107-118): QWHIP_OK or QWHIP_E_BAD_WEIGHTS. */
+qwhip_status qwhip_weight_view_validate(const qwhip_weight_view* w);
+
+/* ---- launch flags ---------------------------------------------------------- */
+enum {
+    /* Activations are already in the container's basis (rotated per 32-group for a rotated
+     * container).  Without it the launcher rotates them itself: FWHT-32 in fp32, one f16
+     * rounding, fused into the kernel prologue (QWWeightView.isRotated contract,
+     * QWWeightView.swift:33-38; producer-side rotation Sources/QWMetal/include/qw_dequant.metalh:424-493). */
+    QWHIP_X_PREROTATED = 1u << 0
+};
+
+/* ---- elementwise seams ------------------------------------------------------ */
+/* qwg_fwht32_f16 (Sources/QWMetal/gemm/qwgemm.metal:27-32; QWGemm.encodeFwht32, QWGemm.swift:288-300):
+ * normalized FWHT-32 over consecutive 32-groups, src dtype f16/bf16/f32 -> dst f16 (dst may equal src for f16). */
+qwhip_status qwhip_fwht32(qwhip_stream_t s, const void* src, uint32_t src_dtype, void* dst_f16, uint64_t n);
+/* qwg_cast_f32_to_f16 (QWGemm.encodeCast, QWGemm.swift:305-320). */
+qwhip_status qwhip_cast_f32_to_f16(qwhip_stream_t s, const float* src, void* dst_f16, uint64_t n);
+/* qwg_silu_mul_f16 / qwg_silu_mul_split_f16 (Sources/QWMetal/gemm/qwgemm_batched.metal:58-97;
+ * QWGemmF32.swift:47-115): gu [rows, 2*inter] (gate | up) f16 or f32 -> act [rows, inter] f16 =
+ * f16(FWHT32(silu(g)*u)); the rotation is skipped when `rotate` is 0 or inter % 32 != 0. */
+qwhip_status qwhip_swiglu_fwht(qwhip_stream_t s, const void* gu, uint32_t gu_dtype, void* act_f16,
+                               uint32_t rows, uint32_t inter, uint32_t rotate);
+
+/* ---- dequant side output ---------------------------------------------------- */
+/* Writes the f16 weights the kernels contract, [n, k] row-major in the container's own basis:
+ * RN_f16((1024+q)*scale+bias) for HQ4_G32_M5 (unpack_hq4_word8, qw_dequant.metalh:42-62),
+ * RN_f16(code*scale+bias) for blocks (qwg_aq_frag8, Sources/QWMetal/include/qw_gemm_nax.metalh:29-97). */
+qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_view* w, void* out_f16);
+
+/* ---- decode / verify GEMV: y[m, n] = sum_k W[n, k] * x[m, k] ---------------- */
+/* One launcher for the reference's GEMV doors:
+ *   QWGemm.encode / encodeH16            (QWGemm.swift:137-283)  -> qwg_gemv_q4g_v4, _v4_h16(_dual), qwg_gemv_q4g_dx_h16_t4
+ *   QWGemmAQ.encode / encodeDecodeT4     (QWGemmAQ.swift:192-304) -> qwg_gemv_aq*_v4, qwg_gemv_aq*_dx_h16_t4
+ *   qwg_skinny_m2/m3, qwg_gemv_hq4_rows_r_m_t (M = 2..8 verify)
+ * x: [m, k] row-major, f16 or bf16; m in 1..16; every weight byte is read once for all m rows.
+ * y16 (f16 [m, n]) and/or y32 (f32 [m, n]) receive the result; at least one is required
+ * (both = the reference's dual store).  fp32 accumulation. */
+qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
+                        uint32_t m, uint32_t flags, void* y16, float* y32);
+
+/* gate|up GEMV + SwiGLU (+ FWHT-32 of the result): qwg_gemv_q4g_silu_pair{,_h16,_dx_h16}
+ * (qwgemm.metal:204-379; QWGemm.swift:137-283 epilogue .siluMulPair; EncodeKernels.swift:298-326).
+ * w holds 2*inter rows: [0, inter) gate, [inter, 2*inter) up.  act16 f16 [m, inter] =
+ * f16(FWHT32(silu(g)*u)) with SwiGLU on the fp32 accumulators; `rotate_out` = 0 stores it unrotated. */
+qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
+                                  uint32_t m, uint32_t flags, uint32_t rotate_out, void* act16);
+
+/* ---- prefill GEMM: Y[m, n] = X[m, k] . W^T on f16 MFMA, fp32 accumulate ------ */
+/* gemmBatchedH16 (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:119-154) -> qwg_gemm_q4g_h16 /
+ * qwg_gemm_aq*_h16; QWGemm.encodeNaxF32 (Sources/Operators/QWGEMM/QWGemmF32.swift:366-402).
+ * x: f16 or bf16 [m, ldx]; y: f16, bf16 or f32 [m, ldy]; ldx/ldy in elements (0 = tight).
+ * Requires k % 64 == 0 and n % 16 == 0 else QWHIP_E_BAD_GEOMETRY (the reference's tensor path
+ * requires N, K multiples of 64).  Activations must be in the container's basis
+ * (QWHIP_X_PREROTATED) unless `workspace` holds m*k f16 elements for the rotated copy. */
+qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
+                        uint32_t m, uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags,
+                        void* workspace, uint64_t workspace_bytes);
+
+/* ---- MoE --------------------------------------------------------------------- */
+/* qwg_moe_route (Sources/QWMetal/subsystems/qwrouter.metal:31-169; encodeFnMoeRoute,
+ * Sources/Operators/QWGEMM/QWGemmMoERouter.swift:10-75): fp32 softmax over `experts`, top_k rounds of
+ * argmax with ties to the lower index, optional renormalisation, x routed_scale.
+ * idx i32 [t, top_k] (-1 = none), wts f32 [t, top_k].  experts <= 512, top_k <= 16. */
+qwhip_status qwhip_moe_route(qwhip_stream_t s, const float* logits, uint32_t t, uint32_t experts, uint32_t top_k,
+                             uint32_t norm_topk, float routed_scale, int32_t* idx, float* wts);
+
+/* qwg_router_gemm (qwrouter.metal:460-; encodeFnRouterGemm, QWGemmMoERouter.swift:78-113):
+ * logits[t, e] = sum_h x[t, h] * Wr[e, h]; x f16/bf16/f32, Wr f32/f16/bf16, fp32 accumulate. */
+qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
+                               uint32_t t, uint32_t experts, uint32_t hidden, float* logits);
+
+/* Scratch sizes of the pair sort (MoETilePlan, Sources/Operators/QWGEMM/QWGemmMoE.swift:24-62). */
+uint32_t qwhip_moe_max_tiles(uint32_t experts, uint32_t pairs);
+
+/* qwg_moe_group_pairs_f32 (Sources/QWMetal/gemm/qwgemm_moe_group_f32.metal:10-148;
+ * encodeMoEGroupPairsF32, QWGemmMoE.swift:68-99): counting sort of the (token, route) pairs by expert
+ * id (low 16 bits of ids; negative = skipped), stable in pair order.
+ * expert_off i32 [experts+1]; sorted_pair i32 [pairs]; sorted_tok i32 [pairs] (= pair / top_k);
+ * inv_perm i32 [pairs] (may be NULL; -1 for skipped pairs); tile_e / tile_r i32 [max_tiles] and
+ * tile_count i32 [1] (may be NULL together): 64-row tiles with a compact 16/32/64 tail per expert,
+ * tile_r = (code << 24) | row_block_index (Sources/QWMetal/include/qw_moe_tile.metalh:7-34). */
+qwhip_status qwhip_moe_group_pairs(qwhip_stream_t s, const int32_t* ids, uint32_t experts, uint32_t pairs,
+                                   uint32_t top_k, int32_t* expert_off, int32_t* sorted_pair, int32_t* sorted_tok,
+                                   int32_t* inv_perm, int32_t* tile_e, int32_t* tile_r, int32_t* tile_count,
+                                   uint32_t compact_tail);
+
+/* Grouped expert GEMM over the sorted pairs: encodeMoEGateUpNax / encodeMoENaxSplitF32
+ * (QWGemmMoE.swift:201-296) -> qwg_moe_nax_gemm_body / qwg_moe_nax_split_f32_body
+ * (Sources/QWMetal/include/qw_gemm_nax.metalh:436-504).
+ * w: ONE view over the expert-major bank, n = experts * rows_per_expert.  Row slot p in
+ * [expert_off[e], expert_off[e+1]) uses expert e.  A row of slot p is x[gather[p]] when gather is
+ * not NULL (gate_up: gather = sorted_tok) else x[p] (down).  y [pairs, rows_per_expert]. */
+qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_weight_view* w, uint32_t experts,
+                                    const void* x, uint32_t x_dtype, uint32_t ldx, const int32_t* gather,
+                                    const int32_t* expert_off, const int32_t* tile_e, const int32_t* tile_r,
+                                    const int32_t* tile_count, uint32_t max_tiles, uint32_t pairs,
+                                    void* y, uint32_t y_dtype, uint32_t ldy);
+
+/* qwg_moe_down_reduce_combine_f32 (Sources/QWMetal/gemm/qwgemm_moe_nax_f16.metal:7-126;
+ * encodeMoEDownReduceCombineF32, QWGemmMoE.swift:299-332):
+ * out[t, h] = sum_k wts[t, k] * dn[inv_perm[t*top_k + k], h] (+ shared_gate[t] * shared[t, h]). */
+qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint32_t dn_dtype, const int32_t* inv_perm,
+                               const float* wts, uint32_t t, uint32_t top_k, uint32_t hidden,
+                               const float* shared, const float* shared_gate, void* out, uint32_t out_dtype);
+
+/* Decode / verify (t <= 8) routed experts as GEMVs: encodeMoEGateUpF32R1 + encodeMoEDownSharedCombineF32
+ * (QWGemmMoE.swift:120-199) -> Sources/QWMetal/include/qw_moe_f32_common.metalh:187-452.
+ * gate_up: act16 [t, top_k, inter] = f16(FWHT32(silu(Wg[e].x) * (Wu[e].x))), SwiGLU on fp32 accumulators.
+ * down:    out [t, hidden] = sum_k wts[t,k] * Wd[e_k] . act16[t,k]  (+ shared_gate[t]*shared[t]). */
+qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                     const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
+                                     uint32_t top_k, void* act16);
+qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts,
+                                   const void* act16, const int32_t* idx, const float* wts, uint32_t t,
+                                   uint32_t top_k, const float* shared, const float* shared_gate, void* out,
+                                   uint32_t out_dtype);
+
+/* ---- load-time writer (the step before the path) ----------------------------- */
+/* qwg_quantize_bf16_to_hq4_g32_m5 (Sources/QWMetal/quant/qw_online_quant.metal:17-55), GPU twin of
+ * quant_hq4_blocks (Scripts/quantize/hq4.py:54-123): src [n, k] bf16 or f32 -> 20-byte blocks. */
+qwhip_status qwhip_quantize_hq4_g32(qwhip_stream_t s, const void* src, uint32_t src_dtype, uint32_t n, uint32_t k,
+                                    uint32_t rotate, void* blocks_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QWHIP_H */

@@ -1,0 +1,204 @@
+// Elementwise seams of the quantized matmul path: activation rotation, casts, SwiGLU(+FWHT),
+// and the dequant-to-f16 side output used to check weights bit-for-bit.
+#include "qwhip_common.h"
+
+// ---- FWHT-32 over consecutive 32-groups: src (f16 | bf16 | f32) -> dst f16 ----------------------
+// One lane owns one group: 64/128 bytes in, 64 bytes out, all butterflies in registers.
+template <int DT>
+__global__ __launch_bounds__(256) void qw_fwht32_kernel(const void* __restrict__ src, h1_t* __restrict__ dst,
+                                                         uint64_t groups) {
+    const uint64_t g = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= groups) return;
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) qw_load8_f32<DT>(src, g * 32 + 8 * j, v + 8 * j);
+    qw_fwht32(v);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        h8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (h1_t)v[8 * j + e];
+        *(h8_t*)(dst + g * 32 + 8 * j) = o;
+    }
+}
+
+extern "C" qwhip_status qwhip_fwht32(qwhip_stream_t s, const void* src, uint32_t src_dtype, void* dst_f16, uint64_t n) {
+    QWHIP_REQUIRE(s);
+    if (n == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(src);
+    QWHIP_REQUIRE(dst_f16);
+    if (n % 32 != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "fwht32: n=%llu is not a multiple of 32", (unsigned long long)n);
+    if (((uintptr_t)src & 15u) || ((uintptr_t)dst_f16 & 15u))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "fwht32: buffers must be 16-byte aligned");
+    const uint64_t groups = n / 32;
+    const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
+    switch (src_dtype) {
+        case QWHIP_F16: hipLaunchKernelGGL(qw_fwht32_kernel<QWHIP_F16>, grid, block, 0, s->stream, src, (h1_t*)dst_f16, groups); break;
+        case QWHIP_BF16: hipLaunchKernelGGL(qw_fwht32_kernel<QWHIP_BF16>, grid, block, 0, s->stream, src, (h1_t*)dst_f16, groups); break;
+        case QWHIP_F32: hipLaunchKernelGGL(qw_fwht32_kernel<QWHIP_F32>, grid, block, 0, s->stream, src, (h1_t*)dst_f16, groups); break;
+        default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "fwht32: unsupported source dtype %u", src_dtype);
+    }
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// ---- f32 -> f16 cast ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void qw_cast_f32_f16_kernel(const float* __restrict__ src, h1_t* __restrict__ dst,
+                                                               uint64_t n) {
+    uint64_t i = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i + 8 <= n && (((uintptr_t)(src + i) & 15u) == 0) && (((uintptr_t)(dst + i) & 15u) == 0)) {
+        float v[8];
+        qw_load8_f32<QWHIP_F32>(src, i, v);
+        h8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (h1_t)v[e];
+        *(h8_t*)(dst + i) = o;
+    } else {
+        for (int e = 0; e < 8 && i + e < n; ++e) dst[i + e] = (h1_t)src[i + e];
+    }
+}
+
+extern "C" qwhip_status qwhip_cast_f32_to_f16(qwhip_stream_t s, const float* src, void* dst_f16, uint64_t n) {
+    QWHIP_REQUIRE(s);
+    if (n == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(src);
+    QWHIP_REQUIRE(dst_f16);
+    const uint64_t threads = (n + 7) / 8;
+    hipLaunchKernelGGL(qw_cast_f32_f16_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s->stream, src,
+                       (h1_t*)dst_f16, n);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// ---- SwiGLU (+ FWHT-32): gu [rows, 2I] (gate | up) -> act [rows, I] f16 ---------------------------
+// SwiGLU runs in fp32 on the values as stored (f16 inputs are the rounded values the fused prefill
+// path also sees, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:132-152); rotation in fp32, one
+// f16 rounding on store.
+template <int DT, bool ROT>
+__global__ __launch_bounds__(256) void qw_swiglu_fwht_kernel(const void* __restrict__ gu, h1_t* __restrict__ act,
+                                                              uint32_t rows, uint32_t inter) {
+    const uint32_t gpr = inter / 32;  // groups per row
+    const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (uint64_t)rows * gpr) return;
+    const uint32_t r = (uint32_t)(gid / gpr), g = (uint32_t)(gid % gpr);
+    const uint64_t gbase = (uint64_t)r * 2 * inter + 32 * g;
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float a[8], b[8];
+        qw_load8_f32<DT>(gu, gbase + 8 * j, a);
+        qw_load8_f32<DT>(gu, gbase + inter + 8 * j, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[8 * j + e] = qw_swiglu(a[e], b[e]);
+    }
+    if (ROT) qw_fwht32(v);
+    h1_t* o = act + (uint64_t)r * inter + 32 * g;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        h8_t t;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = (h1_t)v[8 * j + e];
+        *(h8_t*)(o + 8 * j) = t;
+    }
+}
+
+// Ragged tail (inter % 32 != 0): one thread per element, never rotated.
+template <int DT>
+__global__ __launch_bounds__(256) void qw_swiglu_scalar_kernel(const void* __restrict__ gu, h1_t* __restrict__ act,
+                                                                uint32_t rows, uint32_t inter) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (uint64_t)rows * inter) return;
+    const uint32_t r = (uint32_t)(i / inter), c = (uint32_t)(i % inter);
+    const float g = qw_load_f32<DT>(gu, (uint64_t)r * 2 * inter + c);
+    const float u = qw_load_f32<DT>(gu, (uint64_t)r * 2 * inter + inter + c);
+    act[i] = (h1_t)qw_swiglu(g, u);
+}
+
+extern "C" qwhip_status qwhip_swiglu_fwht(qwhip_stream_t s, const void* gu, uint32_t gu_dtype, void* act_f16,
+                                          uint32_t rows, uint32_t inter, uint32_t rotate) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0 || inter == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(gu);
+    QWHIP_REQUIRE(act_f16);
+    if (gu_dtype != QWHIP_F16 && gu_dtype != QWHIP_F32)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "swiglu: gate|up must be f16 or f32, got dtype %u", gu_dtype);
+    h1_t* act = (h1_t*)act_f16;
+    if (inter % 32 != 0 || ((uintptr_t)gu & 15u) || ((uintptr_t)act_f16 & 15u)) {
+        const uint64_t n = (uint64_t)rows * inter;
+        const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+        if (inter % 32 == 0 && rotate)
+            return qwhip_fail(QWHIP_E_BAD_SHAPE, "swiglu: rotated output needs 16-byte aligned buffers");
+        if (gu_dtype == QWHIP_F16) hipLaunchKernelGGL(qw_swiglu_scalar_kernel<QWHIP_F16>, grid, block, 0, s->stream, gu, act, rows, inter);
+        else hipLaunchKernelGGL(qw_swiglu_scalar_kernel<QWHIP_F32>, grid, block, 0, s->stream, gu, act, rows, inter);
+    } else {
+        const uint64_t groups = (uint64_t)rows * (inter / 32);
+        const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
+        if (gu_dtype == QWHIP_F16) {
+            if (rotate) hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F16, true>), grid, block, 0, s->stream, gu, act, rows, inter);
+            else hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F16, false>), grid, block, 0, s->stream, gu, act, rows, inter);
+        } else {
+            if (rotate) hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F32, true>), grid, block, 0, s->stream, gu, act, rows, inter);
+            else hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F32, false>), grid, block, 0, s->stream, gu, act, rows, inter);
+        }
+    }
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// ---- dequant side output: f16 weights [n, k] in the container's own basis ---------------------------
+// HQ4_G32_M5: one thread per u32 word (8 weights).
+__global__ __launch_bounds__(256) void qw_dequant_hq4_kernel(const uint8_t* __restrict__ bank, h1_t* __restrict__ out,
+                                                              uint64_t words) {
+    const uint64_t wi = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (wi >= words) return;
+    const uint64_t blk = wi >> 2;
+    const uint32_t j = (uint32_t)(wi & 3);
+    const qw_hq4_block* b = (const qw_hq4_block*)(bank + blk * 20);
+    const uint32_t hdr = b->hdr;
+    h2_t w[4];
+    qw_unpack_hq4_word(b->qs[j], qw_splat_lo(hdr), qw_splat_hi(hdr), w);
+    h8_t o = {w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
+    *(h8_t*)(out + blk * 32 + 8 * j) = o;
+}
+
+// Bit-stream blocks, any (bits, group): one thread per 8 codes (= `bits` payload bytes).
+__global__ __launch_bounds__(256) void qw_dequant_blk_kernel(const uint8_t* __restrict__ bank, h1_t* __restrict__ out,
+                                                              uint64_t octets, uint32_t bits, uint32_t group) {
+    const uint64_t oi = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (oi >= octets) return;
+    const uint32_t opg = group / 8;  // octets per group
+    const uint64_t blk = oi / opg;
+    const uint32_t o = (uint32_t)(oi % opg);
+    const uint32_t bb = 4 + group * bits / 8;
+    const uint8_t* p = bank + blk * bb;
+    const h1_t sc = __builtin_bit_cast(h1_t, (uint16_t)(p[0] | (p[1] << 8)));
+    const h1_t bi = __builtin_bit_cast(h1_t, (uint16_t)(p[2] | (p[3] << 8)));
+    uint64_t stream = 0;
+    for (uint32_t b = 0; b < bits; ++b) stream |= (uint64_t)p[4 + o * bits + b] << (8 * b);
+    h8_t v;
+    const uint32_t mask = (1u << bits) - 1u;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const h1_t code = (h1_t)(float)((uint32_t)(stream >> (e * bits)) & mask);
+        v[e] = __builtin_fmaf16(code, sc, bi);  // RN_f16(code*scale + bias), single rounding
+    }
+    *(h8_t*)(out + blk * group + 8 * o) = v;
+}
+
+extern "C" qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_view* w, void* out_f16) {
+    QWHIP_REQUIRE(s);
+    qwhip_status st = qwhip_weight_view_validate(w);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(out_f16);
+    if ((uintptr_t)out_f16 & 15u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "dequant: output must be 16-byte aligned");
+    const uint64_t total = (uint64_t)w->n * w->k;
+    const uint64_t threads = total / 8;
+    const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+    if (w->kind == QWHIP_KIND_HQ4_G32_M5)
+        hipLaunchKernelGGL(qw_dequant_hq4_kernel, grid, block, 0, s->stream, (const uint8_t*)w->blocks, (h1_t*)out_f16, threads);
+    else
+        hipLaunchKernelGGL(qw_dequant_blk_kernel, grid, block, 0, s->stream, (const uint8_t*)w->blocks, (h1_t*)out_f16, threads,
+                           w->bits, w->group);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}

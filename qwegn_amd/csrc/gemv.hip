@@ -1,0 +1,464 @@
+// Decode / verify GEMV over quantized banks: y[m, n] = sum_k W[n, k] * x[m, k], m in 1..16.
+//
+// Two kernel families, both HBM-bound streamers that read every weight byte once:
+//
+//  * qw_gemv_hq4_dot2_kernel - HQ4_G32_M5, m = 1.  A 32-lane half-wavefront owns R rows; lane l
+//    owns blocks l, l+32, ... of each row (640 contiguous bytes per half-wave per step).  The rotated
+//    activation lives in LDS (80-byte pitch per 32-group, so 128-bit reads are bank-conflict free) and
+//    is reused across the R rows.  Weights are materialised as exact f16 (one packed f16 FMA) and
+//    contracted with v_dot2_f32_f16 into fp32.
+//
+//  * qw_gemv_mfma_kernel - every container, m = 1..16.  A wavefront owns 16*RT rows; lane (i, c) =
+//    (lane & 15, lane >> 4) owns 32-column slice 4*it + c of row i of each row tile, dequantizes it to
+//    four 8-wide f16 MFMA A operands, and v_mfma_f32_16x16x32_f16 contracts them against the m
+//    activation rows held as B operands (column j = m).  The 4 waves of a workgroup split K and reduce
+//    through LDS.  VALU does only the dequant; accumulation rides on the matrix cores.
+#include "qwhip_common.h"
+
+enum { QW_FMT_M5 = 0, QW_FMT_B4 = 1, QW_FMT_B8 = 2 };
+enum { QW_XM_GLOBAL = 0, QW_XM_LDS_ROT = 1 };
+
+// ------------------------------------------------------------------------------------------------
+// Rotated-activation staging: group g of row m -> 4 x 16 bytes at LDS offset m*pitch + g*gpitch.
+// ------------------------------------------------------------------------------------------------
+template <int XDT>
+__device__ __forceinline__ void qw_stage_group(const void* x, uint64_t elem0, bool rotate, h8_t* dst) {
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) qw_load8_f32<XDT>(x, elem0 + 8 * j, v + 8 * j);
+    if (rotate) qw_fwht32(v);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        h8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (h1_t)v[8 * j + e];
+        dst[j] = o;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Variant A: HQ4_G32_M5, m = 1, dot2.
+// ------------------------------------------------------------------------------------------------
+template <int R, int XDT>
+__global__ __launch_bounds__(256) void qw_gemv_hq4_dot2_kernel(const uint8_t* __restrict__ bank,
+                                                                const void* __restrict__ x, h1_t* __restrict__ y16,
+                                                                float* __restrict__ y32, uint32_t N, uint32_t K,
+                                                                uint32_t rotate) {
+    extern __shared__ h8_t xs[];  // 5 h8 per 32-group (4 used): 80-byte pitch
+    const uint32_t nb = K >> 5;
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t g = tid; g < nb; g += 256) qw_stage_group<XDT>(x, (uint64_t)g * 32, rotate != 0, xs + g * 5);
+    __syncthreads();
+    const uint32_t lane = tid & 31u;
+    const uint32_t row0 = (blockIdx.x * 8u + (tid >> 5)) * R;
+    if (row0 >= N) return;
+    const uint8_t* rp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t row = (row0 + r < N) ? row0 + r : N - 1;
+        rp[r] = bank + (uint64_t)row * nb * 20u;
+    }
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+    for (uint32_t g = lane; g < nb; g += 32) {
+        qw_hq4_block b[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) b[r] = *(const qw_hq4_block*)(rp[r] + g * 20u);
+        h8_t xv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xv[j] = xs[g * 5 + j];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const h2_t s2 = qw_splat_lo(b[r].hdr), b2 = qw_splat_hi(b[r].hdr);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                h2_t w[4];
+                qw_unpack_hq4_word(b[r].qs[j], s2, b2, w);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const h2_t xp = {xv[j][2 * k], xv[j][2 * k + 1]};
+                    acc[r] = __builtin_amdgcn_fdot2(w[k], xp, acc[r], false);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float v = qw_reduce32(acc[r]);
+        if (lane == 0 && row0 + r < N) {
+            if (y32) y32[row0 + r] = v;
+            if (y16) y16[row0 + r] = (h1_t)v;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Variant B: MFMA streamer, all containers, m = 1..16.
+// ------------------------------------------------------------------------------------------------
+template <int FMT>
+struct qw_slice {
+    uint32_t hdr;
+    uint32_t q[FMT == QW_FMT_B8 ? 8 : 4];
+};
+
+struct __attribute__((packed, aligned(4))) qw_words4 { uint32_t q[4]; };
+struct __attribute__((packed, aligned(4))) qw_words8 { uint32_t q[8]; };
+
+// Position e of an A operand holds element perm(e) of the 8-column chunk.
+template <int FMT>
+__device__ __forceinline__ constexpr int qw_perm(int e) {
+    if (FMT == QW_FMT_M5) return e;
+    if (FMT == QW_FMT_B4) return (e >> 1) + 4 * (e & 1);      // 0,4,1,5,2,6,3,7
+    return (e & 4) + ((e & 1) << 1) + ((e >> 1) & 1);         // 0,2,1,3,4,6,5,7
+}
+
+// Loads slice `s` (32 columns) of the row at `rowp`.  gshift = log2(group / 32).
+template <int FMT>
+__device__ __forceinline__ void qw_load_slice(const uint8_t* rowp, uint32_t s, uint32_t gshift, uint32_t bb,
+                                              qw_slice<FMT>& o) {
+    if constexpr (FMT == QW_FMT_M5) {
+        const qw_hq4_block b = *(const qw_hq4_block*)(rowp + s * 20u);
+        o.hdr = b.hdr;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o.q[j] = b.qs[j];
+    } else {
+        const uint8_t* p = rowp + (uint64_t)(s >> gshift) * bb;
+        const uint32_t si = s & ((1u << gshift) - 1u);
+        o.hdr = *(const uint32_t*)p;
+        if constexpr (FMT == QW_FMT_B4) {
+            const qw_words4 w = *(const qw_words4*)(p + 4 + si * 16u);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o.q[j] = w.q[j];
+        } else {
+            const qw_words8 w = *(const qw_words8*)(p + 4 + si * 32u);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o.q[j] = w.q[j];
+        }
+    }
+}
+
+// Dequantizes chunk j (8 columns) of a slice into an MFMA A operand of exact f16 weights:
+// RN_f16((1024+q)*s + b) for HQ4_G32_M5, RN_f16(code*s + b) for bit-stream blocks (the magic 1024 is
+// stripped exactly before the single f16 FMA, as qwg_aq_frag8 does,
+// Sources/QWMetal/include/qw_gemm_nax.metalh:61-71).
+template <int FMT>
+__device__ __forceinline__ h8_t qw_dequant_chunk(const qw_slice<FMT>& sl, int j, h2_t s2, h2_t b2) {
+    h2_t w[4];
+    if constexpr (FMT == QW_FMT_M5) {
+        qw_unpack_hq4_word(sl.q[j], s2, b2, w);
+    } else if constexpr (FMT == QW_FMT_B4) {
+        const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t m = ((sl.q[j] >> (4 * k)) & 0x000F000Fu) | 0x64006400u;
+            w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m) + neg, s2, b2);
+        }
+    } else {
+        const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t q = sl.q[2 * j + h];
+            const uint32_t m0 = (q & 0x00FF00FFu) | 0x64006400u;
+            const uint32_t m1 = ((q >> 8) & 0x00FF00FFu) | 0x64006400u;
+            w[2 * h] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m0) + neg, s2, b2);
+            w[2 * h + 1] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m1) + neg, s2, b2);
+        }
+    }
+    h8_t a = {w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
+    return a;
+}
+
+template <int FMT>
+__device__ __forceinline__ h8_t qw_x_operand(const h8_t* xg, int j) {
+    h8_t b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] = xg[j][qw_perm<FMT>(e)];
+    return b;
+}
+
+// PAIR = 1: gate|up pair mode.  The bank holds 2*N rows ([0, N) gate, [N, 2N) up); both are
+// accumulated and the epilogue stores act[m, n] = f16(FWHT32(silu(g) * u)) (rotation optional).
+template <int FMT, int RT, int XDT, int XM, int PAIR>
+__global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __restrict__ bank, const void* __restrict__ x,
+                                                            h1_t* __restrict__ y16, float* __restrict__ y32, uint32_t N,
+                                                            uint32_t K, uint32_t M, uint32_t gshift, uint32_t bb,
+                                                            uint64_t row_bytes, uint32_t rotate, uint32_t rot_out) {
+    constexpr int NACC = RT * (PAIR ? 2 : 1);
+    extern __shared__ h8_t xs[];
+    __shared__ f4_t red[4][NACC][64];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t i = lane & 15u, c = lane >> 4;
+    const uint32_t nsl = K >> 5;
+    const uint32_t xpitch8 = (K >> 3) + 1;  // LDS row pitch in h8 units: K*2 + 16 bytes
+
+    if constexpr (XM == QW_XM_LDS_ROT) {
+        for (uint32_t idx = tid; idx < M * nsl; idx += 256) {
+            const uint32_t m = idx / nsl, g = idx - m * nsl;
+            qw_stage_group<XDT>(x, (uint64_t)m * K + 32u * g, rotate != 0, xs + m * xpitch8 + g * 4);
+        }
+        __syncthreads();
+    }
+
+    const uint32_t n0 = blockIdx.x * (16u * RT);
+    const uint8_t* rp[NACC];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        uint32_t row = n0 + 16u * t + i;
+        if (row >= N) row = N - 1;
+        rp[t] = bank + (uint64_t)row * row_bytes;
+        if (PAIR) rp[RT + t] = bank + (uint64_t)(row + N) * row_bytes;
+    }
+    f4_t acc[NACC];
+#pragma unroll
+    for (int t = 0; t < NACC; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t iters = (nsl + 3) >> 2;
+    const uint32_t per = (iters + 3) >> 2;
+    const uint32_t it0 = wave * per;
+    const uint32_t it1 = min(it0 + per, iters);
+
+    qw_slice<FMT> cur[NACC], nxt[NACC];
+    if (it0 < it1) {
+        const uint32_t s = min(4u * it0 + c, nsl - 1);
+#pragma unroll
+        for (int t = 0; t < NACC; ++t) qw_load_slice<FMT>(rp[t], s, gshift, bb, cur[t]);
+    }
+    for (uint32_t it = it0; it < it1; ++it) {
+        const uint32_t s = 4u * it + c;
+        const bool valid = s < nsl;
+        if (it + 1 < it1) {
+            const uint32_t sn = min(s + 4u, nsl - 1);
+#pragma unroll
+            for (int t = 0; t < NACC; ++t) qw_load_slice<FMT>(rp[t], sn, gshift, bb, nxt[t]);
+        }
+        // activations of slice s for row m = i
+        h8_t xg[4];
+        if (valid && i < M) {
+            if constexpr (XM == QW_XM_LDS_ROT) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xg[j] = xs[i * xpitch8 + s * 4 + j];
+            } else {
+                qw_stage_group<XDT>(x, (uint64_t)i * K + 32u * s, rotate != 0, xg);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xg[j] = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+        h8_t bop[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bop[j] = qw_x_operand<FMT>(xg, j);
+#pragma unroll
+        for (int t = 0; t < NACC; ++t) {
+            const h2_t s2 = qw_splat_lo(cur[t].hdr), b2 = qw_splat_hi(cur[t].hdr);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const h8_t a = qw_dequant_chunk<FMT>(cur[t], j, s2, b2);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bop[j], acc[t], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NACC; ++t) cur[t] = nxt[t];
+    }
+
+    // split-K reduction: D[row 4c + r][col i] of every wave -> wave 0
+#pragma unroll
+    for (int t = 0; t < NACC; ++t) red[wave][t][lane] = acc[t];
+    __syncthreads();
+    if constexpr (!PAIR) {
+        if (wave != 0) return;
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            f4_t v = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
+            if (i < M) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t n = n0 + 16u * t + 4u * c + r;
+                    if (n < N) {
+                        if (y32) y32[(uint64_t)i * N + n] = v[r];
+                        if (y16) y16[(uint64_t)i * N + n] = (h1_t)v[r];
+                    }
+                }
+            }
+        }
+    } else {
+        // SwiGLU on the fp32 sums, then (RT == 2: the workgroup's 32 rows are one 32-group) FWHT-32.
+        __shared__ float actbuf[16][16 * RT + 1];
+        if (wave == 0) {
+#pragma unroll
+            for (int t = 0; t < RT; ++t) {
+                const f4_t g = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
+                const f4_t u = red[0][RT + t][lane] + red[1][RT + t][lane] + red[2][RT + t][lane] + red[3][RT + t][lane];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) actbuf[i][16 * t + 4 * c + r] = qw_swiglu(g[r], u[r]);
+            }
+        }
+        __syncthreads();
+        if (tid < M) {
+            if constexpr (RT == 2) {
+                float v[32];
+#pragma unroll
+                for (int e = 0; e < 32; ++e) v[e] = actbuf[tid][e];
+                if (rot_out && n0 + 32u <= N) qw_fwht32(v);
+#pragma unroll
+                for (int e = 0; e < 32; ++e)
+                    if (n0 + e < N) y16[(uint64_t)tid * N + n0 + e] = (h1_t)v[e];
+            } else {
+                for (int e = 0; e < 16 * RT; ++e)
+                    if (n0 + e < N) y16[(uint64_t)tid * N + n0 + e] = (h1_t)actbuf[tid][e];
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+struct gemv_args {
+    const uint8_t* bank;
+    const void* x;
+    h1_t* y16;
+    float* y32;
+    uint32_t N, K, M, gshift, bb;
+    uint64_t row_bytes;
+    uint32_t rotate, rot_out;
+};
+
+template <int FMT, int RT, int XDT, int XM, int PAIR>
+void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds) {
+    const dim3 grid(qwhip_cdiv(a.N, 16u * RT)), block(256);
+    hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR>), grid, block, lds, st, a.bank, a.x, a.y16, a.y32, a.N,
+                       a.K, a.M, a.gshift, a.bb, a.row_bytes, a.rotate, a.rot_out);
+}
+
+template <int FMT, int RT, int XDT, int PAIR>
+void launch_mfma_xm(hipStream_t st, const gemv_args& a, int xm, size_t lds) {
+    if (xm == QW_XM_LDS_ROT) launch_mfma<FMT, RT, XDT, QW_XM_LDS_ROT, PAIR>(st, a, lds);
+    else launch_mfma<FMT, RT, XDT, QW_XM_GLOBAL, PAIR>(st, a, 0);
+}
+
+template <int FMT, int RT, int PAIR>
+void launch_mfma_dt(hipStream_t st, const gemv_args& a, uint32_t xdt, int xm, size_t lds) {
+    if (xdt == QWHIP_F16) launch_mfma_xm<FMT, RT, QWHIP_F16, PAIR>(st, a, xm, lds);
+    else launch_mfma_xm<FMT, RT, QWHIP_BF16, PAIR>(st, a, xm, lds);
+}
+
+template <int FMT>
+void launch_mfma_rt(hipStream_t st, const gemv_args& a, uint32_t xdt, int xm, size_t lds, int rt) {
+    if (rt == 1) launch_mfma_dt<FMT, 1, 0>(st, a, xdt, xm, lds);
+    else if (rt == 2) launch_mfma_dt<FMT, 2, 0>(st, a, xdt, xm, lds);
+    else launch_mfma_dt<FMT, 4, 0>(st, a, xdt, xm, lds);
+}
+
+qwhip_status check_common(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
+                          int* fmt) {
+    QWHIP_REQUIRE(s);
+    qwhip_status st = qwhip_weight_view_validate(w);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(x);
+    if (x_dtype != QWHIP_F16 && x_dtype != QWHIP_BF16)
+        return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "activations must be f16 or bf16, got dtype %u", x_dtype);
+    if (m == 0 || m > 16) return qwhip_fail(QWHIP_E_BAD_SHAPE, "gemv handles 1..16 activation rows, got %u", m);
+    if (w->n >= (1u << 30)) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "a bank of %u rows does not fit the row count", w->n);
+    if ((uintptr_t)x & 15u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "activations must be 16-byte aligned");
+    if (w->kind == QWHIP_KIND_HQ4_G32_M5) *fmt = QW_FMT_M5;
+    else if (w->bits == 4) *fmt = QW_FMT_B4;
+    else if (w->bits == 8) *fmt = QW_FMT_B8;
+    else return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no gemv kernel for %u-bit group %u", w->bits, w->group);
+    return QWHIP_OK;
+}
+
+uint32_t log2_u32(uint32_t v) {
+    uint32_t r = 0;
+    while ((1u << r) < v) ++r;
+    return r;
+}
+
+}  // namespace
+
+// flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = mfma);
+// bits 12..15: row tiles per wave for the mfma kernel (0 = automatic).
+extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
+                                   uint32_t m, uint32_t flags, void* y16, float* y32) {
+    int fmt = 0;
+    qwhip_status st = check_common(s, w, x, x_dtype, m, &fmt);
+    if (st != QWHIP_OK) return st;
+    if (!y16 && !y32) return qwhip_fail(QWHIP_E_NULL, "gemv needs y16 and/or y32");
+    const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
+    const uint32_t variant = (flags >> 8) & 0xFu;
+    uint32_t rt = (flags >> 12) & 0xFu;
+
+    gemv_args a;
+    a.bank = (const uint8_t*)w->blocks;
+    a.x = x;
+    a.y16 = (h1_t*)y16;
+    a.y32 = y32;
+    a.N = w->n;
+    a.K = w->k;
+    a.M = m;
+    a.gshift = log2_u32(w->group / 32);
+    a.bb = qwhip_view_block_bytes(w);
+    a.row_bytes = qwhip_view_row_bytes(w);
+    a.rotate = rotate ? 1u : 0u;
+    a.rot_out = 0;
+
+    const size_t lds_dot2 = (size_t)(w->k / 32) * 80u;
+    const bool dot2_ok = fmt == QW_FMT_M5 && m == 1 && lds_dot2 <= 60u * 1024u;
+    if (variant == 1 && !dot2_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "dot2 kernel needs HQ4_G32_M5, m = 1, k <= 24576");
+    if (variant == 1 || (variant == 0 && dot2_ok && false)) {
+        const uint32_t r = (w->n >= 8192) ? 2u : 1u;
+        const dim3 grid(qwhip_cdiv(w->n, 8u * r)), block(256);
+#define QW_DOT2(R, DT) hipLaunchKernelGGL((qw_gemv_hq4_dot2_kernel<R, DT>), grid, block, lds_dot2, s->stream, a.bank, a.x, a.y16, a.y32, a.N, a.K, a.rotate)
+        if (x_dtype == QWHIP_F16) { if (r == 2) QW_DOT2(2, QWHIP_F16); else QW_DOT2(1, QWHIP_F16); }
+        else { if (r == 2) QW_DOT2(2, QWHIP_BF16); else QW_DOT2(1, QWHIP_BF16); }
+#undef QW_DOT2
+        QWHIP_TRY_HIP(hipGetLastError());
+        return QWHIP_OK;
+    }
+
+    // mfma streamer.  Rotation in the prologue (LDS) when the rotated rows fit, else per lane.
+    const size_t lds_x = (size_t)m * ((size_t)w->k * 2u + 16u);
+    const int xm = (rotate && lds_x <= 48u * 1024u) ? QW_XM_LDS_ROT : QW_XM_GLOBAL;
+    if (rt != 1 && rt != 2 && rt != 4) rt = (w->n >= 16384) ? 2u : 1u;
+    const size_t lds = xm == QW_XM_LDS_ROT ? lds_x : 0;
+    if (fmt == QW_FMT_M5) launch_mfma_rt<QW_FMT_M5>(s->stream, a, x_dtype, xm, lds, (int)rt);
+    else if (fmt == QW_FMT_B4) launch_mfma_rt<QW_FMT_B4>(s->stream, a, x_dtype, xm, lds, (int)rt);
+    else launch_mfma_rt<QW_FMT_B8>(s->stream, a, x_dtype, xm, lds, (int)rt);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
+                                             uint32_t m, uint32_t flags, uint32_t rotate_out, void* act16) {
+    int fmt = 0;
+    qwhip_status st = check_common(s, w, x, x_dtype, m, &fmt);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(act16);
+    if (w->n % 2 != 0) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "gate|up bank needs an even row count, got %u", w->n);
+    const uint32_t inter = w->n / 2;
+    const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
+    gemv_args a;
+    a.bank = (const uint8_t*)w->blocks;
+    a.x = x;
+    a.y16 = (h1_t*)act16;
+    a.y32 = nullptr;
+    a.N = inter;
+    a.K = w->k;
+    a.M = m;
+    a.gshift = log2_u32(w->group / 32);
+    a.bb = qwhip_view_block_bytes(w);
+    a.row_bytes = qwhip_view_row_bytes(w);
+    a.rotate = rotate ? 1u : 0u;
+    a.rot_out = (rotate_out && inter % 32 == 0) ? 1u : 0u;
+    const size_t lds_x = (size_t)m * ((size_t)w->k * 2u + 16u);
+    const int xm = (rotate && lds_x <= 48u * 1024u) ? QW_XM_LDS_ROT : QW_XM_GLOBAL;
+    const size_t lds = xm == QW_XM_LDS_ROT ? lds_x : 0;
+    if (fmt == QW_FMT_M5) launch_mfma_dt<QW_FMT_M5, 2, 1>(s->stream, a, x_dtype, xm, lds);
+    else if (fmt == QW_FMT_B4) launch_mfma_dt<QW_FMT_B4, 2, 1>(s->stream, a, x_dtype, xm, lds);
+    else launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}

@@ -1,0 +1,153 @@
+// Shared host/device definitions of libqwhip (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qwhip.h"
+
+struct qwhip_device_s {
+    int ordinal;
+    hipDeviceProp_t prop;
+};
+struct qwhip_stream_s {
+    qwhip_device_s* dev;
+    hipStream_t stream;
+};
+struct qwhip_event_s {
+    qwhip_device_s* dev;
+    hipEvent_t ev;
+};
+
+// ---- host-side error plumbing (hal.hip) ------------------------------------
+qwhip_status qwhip_fail(qwhip_status st, const char* fmt, ...);
+qwhip_status qwhip_hip_check(hipError_t e, const char* what);
+#define QWHIP_TRY_HIP(expr)                                        \
+    do {                                                           \
+        hipError_t _e = (expr);                                    \
+        if (_e != hipSuccess) return qwhip_hip_check(_e, #expr);   \
+    } while (0)
+#define QWHIP_REQUIRE(p)                                                       \
+    do {                                                                       \
+        if ((p) == nullptr) return qwhip_fail(QWHIP_E_NULL, "%s is NULL", #p); \
+    } while (0)
+
+static inline uint32_t qwhip_cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+// Block bytes of a validated view.
+static inline uint32_t qwhip_view_block_bytes(const qwhip_weight_view* w) { return 4u + w->group * w->bits / 8u; }
+static inline uint64_t qwhip_view_row_bytes(const qwhip_weight_view* w) {
+    return (uint64_t)(w->k / w->group) * qwhip_view_block_bytes(w);
+}
+static inline bool qwhip_view_rotated(const qwhip_weight_view* w) { return w->kind != QWHIP_KIND_NATIVE_AFFINE; }
+
+// ---- device-side types -------------------------------------------------------
+typedef _Float16 h1_t;
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef float f16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+
+#define QW_INV_SQRT32 0.17677669529663689f /* f32(1/sqrt(32)) = 0x3E3504F3 */
+
+// One HQ4_G32_M5 block: [f16 scale][f16 bias][u32 qs[4]], 4-byte aligned in a bank.
+struct __attribute__((packed, aligned(4))) qw_hq4_block {
+    uint32_t hdr;
+    uint32_t qs[4];
+};
+
+__device__ __forceinline__ float qw_bf16_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+
+// f32 -> bf16 bits, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ uint16_t qw_f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// Load element i of a typed activation array as fp32.
+template <int DT>
+__device__ __forceinline__ float qw_load_f32(const void* p, uint64_t i) {
+    if constexpr (DT == QWHIP_F16) return (float)((const h1_t*)p)[i];
+    else if constexpr (DT == QWHIP_BF16) return qw_bf16_to_f32(((const uint16_t*)p)[i]);
+    else return ((const float*)p)[i];
+}
+
+// Loads 8 consecutive elements (16-byte aligned for 2-byte types) as fp32.
+template <int DT>
+__device__ __forceinline__ void qw_load8_f32(const void* p, uint64_t i, float* out) {
+    if constexpr (DT == QWHIP_F16) {
+        h8_t v = *(const h8_t*)((const h1_t*)p + i);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) out[j] = (float)v[j];
+    } else if constexpr (DT == QWHIP_BF16) {
+        u4_t v = *(const u4_t*)((const uint16_t*)p + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            out[2 * j] = __uint_as_float(v[j] << 16);
+            out[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+        }
+    } else {
+        const f4_t* q = (const f4_t*)((const float*)p + i);
+        f4_t a = q[0], b = q[1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            out[j] = a[j];
+            out[4 + j] = b[j];
+        }
+    }
+}
+
+// In-register orthonormal FWHT-32: butterflies h = 1..16 writing (u+v, u-v) to (i, i+h), then one
+// multiply by f32(1/sqrt(32)) - the operation order of fwht32_ortho (Scripts/quantize/hq4.py:26-51,
+// Sources/Foundation/QWQuant/QWQuant+DequantMath.swift:93-112), so results are bit-identical.
+__device__ __forceinline__ void qw_fwht32(float* v) {
+#pragma unroll
+    for (int h = 1; h < 32; h <<= 1) {
+#pragma unroll
+        for (int i0 = 0; i0 < 32; i0 += 2 * h) {
+#pragma unroll
+            for (int j = 0; j < h; ++j) {
+                const float a = v[i0 + j], b = v[i0 + j + h];
+                v[i0 + j] = a + b;
+                v[i0 + j + h] = a - b;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) v[i] = v[i] * QW_INV_SQRT32;
+}
+
+// SwiGLU on fp32: silu(g) * u = g / (1 + exp(-g)) * u  (qwg_swiglu_mul, plain branch,
+// Sources/QWMetal/include/qw_weight_basis.metalh:50-63).
+__device__ __forceinline__ float qw_swiglu(float g, float u) { return (g / (1.0f + __expf(-g))) * u; }
+
+// 8 HQ4_G32_M5 weights of one u32 word as four half2 (elements 0..7 in order): the nibble of element
+// 8w+j sits at bit 4*(j>>1) + 16*(j&1), so ((word >> 4k) & 0x000F000F) | 0x64006400 viewed as half2 is
+// (1024+q[2k], 1024+q[2k+1]); one packed f16 FMA with (scale, bias) gives RN_f16((1024+q)*s + b)
+// (unpack_hq4_word8, Sources/QWMetal/include/qw_dequant.metalh:42-62).
+__device__ __forceinline__ void qw_unpack_hq4_word(uint32_t word, h2_t s2, h2_t b2, h2_t* w) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t m = ((word >> (4 * k)) & 0x000F000Fu) | 0x64006400u;
+        w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m), s2, b2);
+    }
+}
+
+__device__ __forceinline__ h2_t qw_splat_lo(uint32_t hdr) { return __builtin_bit_cast(h2_t, (hdr & 0xFFFFu) * 0x10001u); }
+__device__ __forceinline__ h2_t qw_splat_hi(uint32_t hdr) { return __builtin_bit_cast(h2_t, (hdr >> 16) * 0x10001u); }
+
+// Sum over the 32 lanes of a half-wavefront (xor butterflies stay inside each aligned 32-lane half).
+__device__ __forceinline__ float qw_reduce32(float v) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float qw_reduce64(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}

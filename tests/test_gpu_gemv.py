@@ -1,0 +1,158 @@
+"""GPU parity of the elementwise seams, the dequant side output and the decode / verify GEMV
+(through the C ABI) against the CPU oracle.  Bars: bit-exact for rotated activations and
+dequantized f16 weights; normalized error <= 2e-3 against the fp64 evaluation of
+dequant + matmul for outputs."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import qworacle as qo
+from qwegn_amd import qwhip
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return qwhip.Device(0)
+
+
+def _bf16(x32):
+    return qo.f32_to_bf16_bits(x32)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+def test_fwht32_bit_exact(dev, dtype):
+    x = H.make_x(7, 640, 1)
+    if dtype == "f16":
+        host, code, ref_in = x.astype(np.float16), qwhip.F16, x.astype(np.float16).astype(np.float32)
+    elif dtype == "bf16":
+        host, code, ref_in = _bf16(x), qwhip.BF16, qo.round_bf16(x)
+    else:
+        host, code, ref_in = x, qwhip.F32, x
+    src = dev.put(host)
+    dst = dev.alloc(x.size * 2)
+    qwhip.check(dev.lib.qwhip_fwht32(dev.stream.handle, src.ptr, code, dst.ptr, x.size))
+    got = dst.download(np.float16, x.shape)
+    want = qo.fwht32_ortho(ref_in).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("fmt", list(H.FORMATS))
+def test_dequant_f16_bit_exact(dev, fmt):
+    n, k = 24, 512
+    blocks, w16 = H.make_bank(fmt, n, k, seed=3)
+    bank = dev.put(blocks)
+    out = dev.alloc(n * k * 2)
+    view = H.view_of(dev, bank, fmt, n, k)
+    qwhip.check(dev.lib.qwhip_dequant_f16(dev.stream.handle, C.byref(view), out.ptr))
+    got = out.download(np.float16, (n, k))
+    assert np.array_equal(got.view(np.uint16), w16.view(np.uint16))
+
+
+def _run_gemv(dev, fmt, n, k, m, *, prerot, xdtype="f16", variant=0, rt=0, seed=0, outliers=False):
+    blocks, w16 = H.make_bank(fmt, n, k, seed=seed)
+    x32 = H.make_x(m, k, seed + 100, outliers=outliers)
+    if xdtype == "f16":
+        x_host, code = x32.astype(np.float16), qwhip.F16
+        x_val = x_host.astype(np.float32)
+    else:
+        x_host, code = _bf16(x32), qwhip.BF16
+        x_val = qo.round_bf16(x32)
+    rotate = H.FORMATS[fmt][4]
+    x_basis = (qo.fwht32_ortho(x_val) if rotate else x_val).astype(np.float16)   # what the kernel contracts
+    if prerot:
+        x_dev_host, code = x_basis, qwhip.F16
+    else:
+        x_dev_host = x_host
+    bank = dev.put(blocks)
+    xb = dev.put(x_dev_host)
+    y16 = dev.alloc(m * n * 2)
+    y32 = dev.alloc(m * n * 4)
+    view = H.view_of(dev, bank, fmt, n, k)
+    flags = (qwhip.X_PREROTATED if prerot else 0) | (variant << 8) | (rt << 12)
+    qwhip.check(dev.lib.qwhip_gemv(dev.stream.handle, C.byref(view), xb.ptr, code, m, flags, y16.ptr, y32.ptr))
+    dev.stream.sync()
+    g16 = y16.download(np.float16, (m, n))
+    g32 = y32.download(np.float32, (m, n))
+    ref = qo.matmul_ref_f64(x_basis, w16)
+    for b in (bank, xb, y16, y32):
+        b.free()
+    return g16, g32, ref
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("prerot", [False, True])
+@pytest.mark.parametrize("n,k", [(256, 5120), (1000, 1024), (37, 96), (64, 32)])
+def test_gemv_hq4_m1(dev, variant, prerot, n, k):
+    g16, g32, ref = _run_gemv(dev, "hq4_g32_m5", n, k, 1, prerot=prerot, variant=variant, outliers=True)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("rt", [1, 2, 4])
+@pytest.mark.parametrize("xdtype", ["f16", "bf16"])
+def test_gemv_hq4_mfma_row_tiles_and_dtypes(dev, rt, xdtype):
+    g16, g32, ref = _run_gemv(dev, "hq4_g32_m5", 200, 2048, 1, prerot=False, xdtype=xdtype, variant=2, rt=rt)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["aq4_g32", "hq4_g32", "hq4_g64", "hq4_g128", "hq8_g32", "hq8_g64", "aq8_g256"])
+@pytest.mark.parametrize("m", [1, 2, 3, 8, 16])
+def test_gemv_blocks_small_m(dev, fmt, m):
+    g16, g32, ref = _run_gemv(dev, fmt, 272, 1536, m, prerot=False, seed=5)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("m", [2, 16])
+def test_gemv_rotation_per_lane_path(dev, m):
+    """m*k too large for the LDS staging: rotation runs per lane from global memory."""
+    g16, g32, ref = _run_gemv(dev, "hq4_g64", 96, 17408, m, prerot=False, seed=6)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+
+
+def test_gemv_affine_known_answer(dev):
+    """Code 1, scale 1.0, bias 0.25, x = one-hot: every output is exactly 1.25 - the -1024 must be
+    stripped before the FMA, not folded into an f16 bias
+    (Tests/QWGEMMTests/QWAQBatchedGemmTests.swift:194-205)."""
+    n, k = 64, 128
+    blocks = np.zeros((n, k // 32, 20), dtype=np.uint8)
+    blocks[..., 0:2] = np.array([1.0], dtype=np.float16).view(np.uint8)
+    blocks[..., 2:4] = np.array([0.25], dtype=np.float16).view(np.uint8)
+    blocks[..., 4:] = 0x11
+    x = np.zeros((1, k), dtype=np.float16)
+    x[0, 5] = 1.0
+    bank, xb, y32 = dev.put(blocks), dev.put(x), dev.alloc(n * 4)
+    view = dev.view(bank, n, k, qwhip.KIND_NATIVE_AFFINE, 4, 32)
+    qwhip.check(dev.lib.qwhip_gemv(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, 1, 0, None, y32.ptr))
+    got = y32.download(np.float32, (n,))
+    assert np.all(got == np.float32(1.25))
+
+
+def test_gemv_full_size_decode_config(dev):
+    """HQ4_G32 decode GEMV at its benchmark shape (K = 5120, N = 17408, outliers, fused rotation)."""
+    for variant in (1, 2):
+        g16, g32, ref = _run_gemv(dev, "hq4_g32_m5", 17408, 5120, 1, prerot=False, variant=variant, outliers=True, seed=0)
+        assert qo.normalized_error(g32, ref) <= 2e-5
+        assert qo.normalized_error(g16, ref) <= TOL
+
+
+def test_gemv_rejects_bad_inputs_before_launch(dev):
+    blocks, _ = H.make_bank("hq4_g32_m5", 8, 64, 0)
+    bank, xb, y = dev.put(blocks), dev.put(np.zeros(64, np.float16)), dev.alloc(64)
+    lib, st = dev.lib, dev.stream.handle
+    short = dev.view(bank, 8, 64, qwhip.KIND_HQ4_G32_M5, nbytes=8 * 2 * 20 - 1)
+    assert lib.qwhip_gemv(st, C.byref(short), xb.ptr, qwhip.F16, 1, 0, y.ptr, None) == qwhip.E_BAD_WEIGHTS
+    badk = dev.view(bank, 8, 48, qwhip.KIND_HQ4_G32_M5)
+    assert lib.qwhip_gemv(st, C.byref(badk), xb.ptr, qwhip.F16, 1, 0, y.ptr, None) == qwhip.E_BAD_WEIGHTS
+    good = dev.view(bank, 8, 64, qwhip.KIND_HQ4_G32_M5)
+    assert lib.qwhip_gemv(st, C.byref(good), xb.ptr, qwhip.F32, 1, 0, y.ptr, None) == qwhip.E_BAD_WEIGHTS
+    assert lib.qwhip_gemv(st, C.byref(good), xb.ptr, qwhip.F16, 17, 0, y.ptr, None) == qwhip.E_BAD_SHAPE
+    assert lib.qwhip_gemv(st, C.byref(good), xb.ptr, qwhip.F16, 1, 0, None, None) == qwhip.E_NULL
+    assert lib.qwhip_gemv(st, C.byref(good), xb.ptr, qwhip.F16, 1, 0, y.ptr, None) == qwhip.OK
+    dev.stream.sync()
