@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void qw_dequant_hq4_kernel(const uint8_t* __re
     const qw_hq4_block* b = (const qw_hq4_block*)(bank + blk * 20);
     const uint32_t hdr = b->hdr;
     h2_t w[4];
-    qw_unpack_hq4_word(b->qs[j], qw_splat_lo(hdr), qw_splat_hi(hdr), w);
+    qw_unpack_hq4_word(b->qs[j], qw_splat_lo(hdr), qw_splat_hi(hdr), qw_vgpr_const(0x64006400u), w);
     h8_t o = {w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
     *(h8_t*)(out + blk * 32 + 8 * j) = o;
 }

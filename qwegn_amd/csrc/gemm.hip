@@ -1,0 +1,507 @@
+// Prefill GEMM and MoE grouped GEMM: Y[m, n] = X[m, k] . W_deq[n, k]^T on the f16 matrix cores.
+//
+// One templated kernel.  A workgroup of WVM x WVN wavefronts owns a BM x BN output tile
+// (BM = 32*WM*WVM tokens, BN = 32*WN*WVN weight rows) and walks K in steps of 64:
+//   * activations: global (f16 | bf16) -> registers -> f16 LDS tile [BM][64] (144-byte pitch, so the
+//     128-bit MFMA operand reads of 16 consecutive rows hit 64 distinct banks);
+//   * weights: packed blocks global -> registers -> dequantized to the exact f16 weight
+//     (RN_f16((1024+q)*s+b) / RN_f16(code*s+b), one packed f16 FMA) -> f16 LDS tile [BN][64];
+//   * v_mfma_f32_32x32x16_f16, A = activations (rows i = tokens), B = weights (columns j = weight rows),
+//     fp32 accumulators, f16 / bf16 / f32 store with n contiguous across lanes.
+// The next K-step's global loads are issued before the current step's MFMAs, so HBM/L2 latency hides
+// behind the matrix cores; LDS is single-buffered (two barriers per step).
+//
+// Dense launches map workgroups to tiles XCD-aware: the eight XCDs have private L2s and hardware deals
+// workgroups round-robin, so workgroup w is re-labelled (w % 8) * per_xcd + w / 8 and consecutive labels
+// walk a 4-tile-tall column band: the 32 tiles resident on one XCD share 4 activation panels and 8
+// weight panels through its L2.
+//
+// Grouped launches (MoE) take the tile list of the pair sort: tile t = (expert e, row block) over the
+// expert-major slot range [expert_off[e], expert_off[e+1]); slot rows are gathered through `gather`.
+#include "qwhip_common.h"
+
+enum { QG_FMT_M5 = 0, QG_FMT_B4 = 1, QG_FMT_B8 = 2 };
+
+struct qw_gemm_params {
+    const uint8_t* bank;
+    const void* x;
+    void* y;
+    uint32_t M, N, K;
+    uint32_t ldx, ldy;
+    uint32_t gshift, bb;
+    uint64_t row_bytes;
+    uint32_t tiles_m, tiles_n;
+    // grouped
+    const int32_t* gather;
+    const int32_t* expert_off;
+    const int32_t* tile_e;
+    const int32_t* tile_r;
+    const int32_t* tile_count;
+    uint32_t rows_per_expert;
+};
+
+struct __attribute__((packed, aligned(4))) qg_words4 { uint32_t q[4]; };
+struct __attribute__((packed, aligned(4))) qg_words8 { uint32_t q[8]; };
+
+template <int FMT>
+struct qg_slice {
+    uint32_t hdr;
+    uint32_t q[FMT == QG_FMT_B8 ? 8 : 4];
+};
+
+template <int FMT>
+__device__ __forceinline__ void qg_load_slice(const uint8_t* rowp, uint32_t s, uint32_t gshift, uint32_t bb, qg_slice<FMT>& o) {
+    if constexpr (FMT == QG_FMT_M5) {
+        const qw_hq4_block b = *(const qw_hq4_block*)(rowp + s * 20u);
+        o.hdr = b.hdr;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o.q[j] = b.qs[j];
+    } else {
+        const uint8_t* p = rowp + (uint64_t)(s >> gshift) * bb;
+        const uint32_t si = s & ((1u << gshift) - 1u);
+        o.hdr = *(const uint32_t*)p;
+        if constexpr (FMT == QG_FMT_B4) {
+            const qg_words4 w = *(const qg_words4*)(p + 4 + si * 16u);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o.q[j] = w.q[j];
+        } else {
+            const qg_words8 w = *(const qg_words8*)(p + 4 + si * 32u);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o.q[j] = w.q[j];
+        }
+    }
+}
+
+// 8 consecutive columns (chunk j of the slice) in natural order, as exact f16 weights.
+template <int FMT>
+__device__ __forceinline__ h8_t qg_dequant_chunk(const qg_slice<FMT>& sl, int j, h2_t s2, h2_t b2, uint32_t magic) {
+    h2_t w[4];
+    if constexpr (FMT == QG_FMT_M5) {
+        qw_unpack_hq4_word(sl.q[j], s2, b2, magic, w);
+    } else if constexpr (FMT == QG_FMT_B4) {
+        // bit stream: element e of the word at bit 4e.  lo = even elements, hi = odd elements, one byte each.
+        const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
+        const uint32_t lo = sl.q[j] & 0x0F0F0F0Fu;         // e0 e2 e4 e6
+        const uint32_t hi = (sl.q[j] >> 4) & 0x0F0F0F0Fu;  // e1 e3 e5 e7
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            // bytes: [lo.b_k, 0, hi.b_k, 0]
+            const uint32_t sel = 0x0C000C00u | (uint32_t)k | ((uint32_t)(4 + k) << 16);
+            const uint32_t m = __builtin_amdgcn_perm(hi, lo, sel) | 0x64006400u;
+            w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m) + neg, s2, b2);
+        }
+    } else {
+        const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t q = sl.q[2 * j + h];  // e0 e1 e2 e3 (bytes)
+            const uint32_t m0 = __builtin_amdgcn_perm(q, q, 0x0C010C00u) | 0x64006400u;
+            const uint32_t m1 = __builtin_amdgcn_perm(q, q, 0x0C030C02u) | 0x64006400u;
+            w[2 * h] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m0) + neg, s2, b2);
+            w[2 * h + 1] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m1) + neg, s2, b2);
+        }
+    }
+    h8_t a = {w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
+    return a;
+}
+
+template <int XDT>
+__device__ __forceinline__ h8_t qg_to_f16x8(u4_t raw) {
+    if constexpr (XDT == QWHIP_F16) {
+        return __builtin_bit_cast(h8_t, raw);
+    } else {
+        h8_t o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            o[2 * j] = (h1_t)__uint_as_float(raw[j] << 16);
+            o[2 * j + 1] = (h1_t)__uint_as_float(raw[j] & 0xFFFF0000u);
+        }
+        return o;
+    }
+}
+
+template <int YDT>
+__device__ __forceinline__ void qg_store(void* y, uint64_t idx, float v) {
+    if constexpr (YDT == QWHIP_F32) ((float*)y)[idx] = v;
+    else if constexpr (YDT == QWHIP_F16) ((h1_t*)y)[idx] = (h1_t)v;
+    else ((uint16_t*)y)[idx] = qw_f32_to_bf16(v);
+}
+
+template <int WM, int WN, int WVM, int WVN, int FMT, int XDT, int YDT, bool GROUPED>
+__global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm_kernel(const qw_gemm_params p) {
+    constexpr int NT = WVM * WVN * 64;
+    constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 64;
+    constexpr int PITCH = BK + 8;                   // halves: 144 bytes
+    constexpr int A_CHUNKS = BM * 8;                // 16-byte chunks per K-step
+    constexpr int A_PER = (A_CHUNKS + NT - 1) / NT;
+    constexpr int B_ITEMS = BN * 2;                 // (row, 32-column slice) items per K-step
+    constexpr int B_PER = (B_ITEMS + NT - 1) / NT;
+
+    extern __shared__ h1_t lds[];
+    h1_t* la = lds;
+    h1_t* lb = lds + BM * PITCH;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t wm = wave / WVN, wn = wave % WVN;
+
+    // ---- tile coordinates -------------------------------------------------------------------------
+    uint32_t m0, n0, rows_valid;
+    const uint8_t* bank = p.bank;
+    if constexpr (GROUPED) {
+        const uint32_t t = blockIdx.y;
+        if ((int32_t)t >= p.tile_count[0]) return;
+        const uint32_t e = (uint32_t)p.tile_e[t];
+        const uint32_t packed = (uint32_t)p.tile_r[t];
+        const uint32_t code = packed >> 24;
+        const uint32_t bm = code == 1u ? 16u : (code == 2u ? 32u : 64u);
+        const uint32_t start = (uint32_t)p.expert_off[e] + (packed & 0xFFFFFFu) * bm;
+        const uint32_t end = (uint32_t)p.expert_off[e + 1];
+        m0 = start;
+        rows_valid = min((uint32_t)BM, min(bm, end - start));
+        n0 = blockIdx.x * BN;
+        bank += (uint64_t)e * p.rows_per_expert * p.row_bytes;
+    } else {
+        const uint32_t total = p.tiles_m * p.tiles_n;
+        const uint32_t per_xcd = (total + 7u) / 8u;
+        const uint32_t label = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (label >= total) return;
+        constexpr uint32_t G = 4;
+        const uint32_t band = label / (G * p.tiles_n);
+        const uint32_t band_rows = min(G, p.tiles_m - band * G);
+        const uint32_t in_band = label - band * G * p.tiles_n;
+        const uint32_t tm = band * G + in_band % band_rows;
+        const uint32_t tn = in_band / band_rows;
+        m0 = tm * BM;
+        n0 = tn * BN;
+        rows_valid = min((uint32_t)BM, p.M - m0);
+    }
+
+    // ---- per-thread copy assignments ---------------------------------------------------------------
+    const uint8_t* a_src[A_PER];
+    bool a_ok[A_PER];
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+        const uint32_t c = tid + i * NT;
+        const uint32_t row = c >> 3, kc = c & 7u;
+        a_ok[i] = (c < (uint32_t)A_CHUNKS) && (row < rows_valid);
+        uint64_t src_row = m0 + row;
+        if constexpr (GROUPED) {
+            if (a_ok[i] && p.gather) src_row = (uint32_t)p.gather[m0 + row];
+        }
+        a_src[i] = (const uint8_t*)p.x + (a_ok[i] ? (src_row * p.ldx + kc * 8u) * 2u : 0u);
+    }
+    const uint8_t* b_src[B_PER];
+    uint32_t b_sl[B_PER];
+#pragma unroll
+    for (int i = 0; i < B_PER; ++i) {
+        const uint32_t it = tid + i * NT;
+        uint32_t n = n0 + (it >> 1);
+        if (n >= p.N) n = p.N - 1;
+        b_sl[i] = it & 1u;
+        b_src[i] = bank + (uint64_t)n * p.row_bytes;
+    }
+
+    f16_t acc[WM][WN];
+#pragma unroll
+    for (int a = 0; a < WM; ++a)
+#pragma unroll
+        for (int b = 0; b < WN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    const uint32_t nk = p.K / BK;
+    u4_t a_reg[A_PER];
+    qg_slice<FMT> b_reg[B_PER];
+
+    auto issue_loads = [&](uint32_t kt) {
+#pragma unroll
+        for (int i = 0; i < A_PER; ++i) {
+            if (a_ok[i]) a_reg[i] = *(const u4_t*)(a_src[i] + (uint64_t)kt * (BK * 2));
+            else a_reg[i] = u4_t{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < B_PER; ++i) {
+            if (tid + i * NT < (uint32_t)B_ITEMS) qg_load_slice<FMT>(b_src[i], kt * 2u + b_sl[i], p.gshift, p.bb, b_reg[i]);
+        }
+    };
+
+    issue_loads(0);
+    const uint32_t a_row_l = lane & 31u, k_half = lane >> 5;
+    for (uint32_t kt = 0; kt < nk; ++kt) {
+        __syncthreads();
+        // registers -> LDS
+#pragma unroll
+        for (int i = 0; i < A_PER; ++i) {
+            const uint32_t c = tid + i * NT;
+            if (c < (uint32_t)A_CHUNKS) *(h8_t*)(la + (c >> 3) * PITCH + (c & 7u) * 8u) = qg_to_f16x8<XDT>(a_reg[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < B_PER; ++i) {
+            const uint32_t it = tid + i * NT;
+            if (it < (uint32_t)B_ITEMS) {
+                const h2_t s2 = qw_splat_lo(b_reg[i].hdr), b2 = qw_splat_hi(b_reg[i].hdr);
+                h1_t* dst = lb + (it >> 1) * PITCH + (it & 1u) * 32u;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) *(h8_t*)(dst + 8 * j) = qg_dequant_chunk<FMT>(b_reg[i], j, s2, b2, magic);
+            }
+        }
+        __syncthreads();
+        if (kt + 1 < nk) issue_loads(kt + 1);
+        // MFMA over the 64-wide step: 4 x k16
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            h8_t af[WM], bf[WN];
+#pragma unroll
+            for (int a = 0; a < WM; ++a)
+                af[a] = *(const h8_t*)(la + ((wm * WM + a) * 32 + a_row_l) * PITCH + ks * 16 + k_half * 8);
+#pragma unroll
+            for (int b = 0; b < WN; ++b)
+                bf[b] = *(const h8_t*)(lb + ((wn * WN + b) * 32 + a_row_l) * PITCH + ks * 16 + k_half * 8);
+#pragma unroll
+            for (int a = 0; a < WM; ++a)
+#pragma unroll
+                for (int b = 0; b < WN; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
+        }
+    }
+
+    // ---- store: lane holds column j = lane & 31, rows i = 8*(r/4) + 4*(lane >> 5) + (r & 3) -----------
+#pragma unroll
+    for (int a = 0; a < WM; ++a) {
+#pragma unroll
+        for (int b = 0; b < WN; ++b) {
+            const uint32_t n = n0 + (wn * WN + b) * 32 + (lane & 31u);
+            if (n < p.N) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+uint32_t log2_u32(uint32_t v) {
+    uint32_t r = 0;
+    while ((1u << r) < v) ++r;
+    return r;
+}
+
+template <int WM, int WN, int WVM, int WVN, int FMT, int XDT, int YDT, bool GROUPED>
+hipError_t launch_cfg(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
+    constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
+    constexpr size_t lds = (size_t)(BM + BN) * 72 * 2;
+    auto kern = qw_gemm_kernel<WM, WN, WVM, WVN, FMT, XDT, YDT, GROUPED>;
+    static bool attr_done = false;  // per instantiation
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(WVM * WVN * 64), lds, st, p);
+    return hipGetLastError();
+}
+
+// tile configurations
+enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_64x256 = 3, CFG_256x128 = 4 };
+
+template <int FMT, int XDT, int YDT>
+hipError_t launch_dense(hipStream_t st, qw_gemm_params& p, int cfg) {
+    uint32_t bm, bn;
+    switch (cfg) {
+        case CFG_256x320: bm = 256; bn = 320; break;
+        case CFG_256x256: bm = 256; bn = 256; break;
+        case CFG_256x128: bm = 256; bn = 128; break;
+        default: bm = 128; bn = 128; break;
+    }
+    p.tiles_m = qwhip_cdiv(p.M, bm);
+    p.tiles_n = qwhip_cdiv(p.N, bn);
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const dim3 grid(((total + 7u) / 8u) * 8u);
+    switch (cfg) {
+        case CFG_256x320: return launch_cfg<4, 5, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
+        case CFG_256x256: return launch_cfg<4, 4, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
+        case CFG_256x128: return launch_cfg<4, 2, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
+        default: return launch_cfg<2, 2, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
+    }
+}
+
+template <int FMT, int XDT>
+hipError_t launch_dense_y(hipStream_t st, qw_gemm_params& p, int cfg, uint32_t ydt) {
+    if (ydt == QWHIP_F16) return launch_dense<FMT, XDT, QWHIP_F16>(st, p, cfg);
+    if (ydt == QWHIP_BF16) return launch_dense<FMT, XDT, QWHIP_BF16>(st, p, cfg);
+    return launch_dense<FMT, XDT, QWHIP_F32>(st, p, cfg);
+}
+
+template <int FMT>
+hipError_t launch_dense_xy(hipStream_t st, qw_gemm_params& p, int cfg, uint32_t xdt, uint32_t ydt) {
+    if (xdt == QWHIP_F16) return launch_dense_y<FMT, QWHIP_F16>(st, p, cfg, ydt);
+    return launch_dense_y<FMT, QWHIP_BF16>(st, p, cfg, ydt);
+}
+
+// waste-aware choice among the tile shapes: time ~ rounds of tiles over 256 CUs x per-tile cost
+int choose_cfg(uint32_t M, uint32_t N) {
+    struct cand { int cfg; uint32_t bm, bn; double eff; };
+    // eff: relative MFMA efficiency of the shape (bigger wave tiles feed the matrix cores with fewer LDS reads)
+    const cand cands[] = {{CFG_256x320, 256, 320, 1.00}, {CFG_256x256, 256, 256, 0.97}, {CFG_256x128, 256, 128, 0.85},
+                          {CFG_128x128, 128, 128, 0.70}};
+    double best = 1e300;
+    int best_cfg = CFG_128x128;
+    for (const cand& c : cands) {
+        const double tiles = (double)qwhip_cdiv(M, c.bm) * qwhip_cdiv(N, c.bn);
+        const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
+        const double cost = rounds * c.bm * c.bn / c.eff;
+        if (cost < best) {
+            best = cost;
+            best_cfg = c.cfg;
+        }
+    }
+    return best_cfg;
+}
+
+qwhip_status gemm_checks(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, void* y,
+                         uint32_t y_dtype, int* fmt) {
+    QWHIP_REQUIRE(s);
+    qwhip_status st = qwhip_weight_view_validate(w);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(x);
+    QWHIP_REQUIRE(y);
+    if (x_dtype != QWHIP_F16 && x_dtype != QWHIP_BF16)
+        return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "activations must be f16 or bf16, got dtype %u", x_dtype);
+    if (y_dtype != QWHIP_F16 && y_dtype != QWHIP_BF16 && y_dtype != QWHIP_F32)
+        return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "output must be f16, bf16 or f32, got dtype %u", y_dtype);
+    if (w->k % 64 != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "tensor GEMM needs k %% 64 == 0, got k=%u", w->k);
+    if ((uintptr_t)x & 15u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "activations must be 16-byte aligned");
+    if (w->kind == QWHIP_KIND_HQ4_G32_M5) *fmt = QG_FMT_M5;
+    else if (w->bits == 4) *fmt = QG_FMT_B4;
+    else if (w->bits == 8) *fmt = QG_FMT_B8;
+    else return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no tensor GEMM kernel for %u-bit group %u", w->bits, w->group);
+    return QWHIP_OK;
+}
+
+}  // namespace
+
+// flags bits 8..11: tile shape override for tuning and tests (0 = automatic, 1 + CFG_*).
+extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
+                                   uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags, void* workspace,
+                                   uint64_t workspace_bytes) {
+    int fmt = 0;
+    qwhip_status st = gemm_checks(s, w, x, x_dtype, y, y_dtype, &fmt);
+    if (st != QWHIP_OK) return st;
+    if (m == 0) return QWHIP_OK;
+    if (w->n % 16 != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "tensor GEMM needs n %% 16 == 0, got n=%u", w->n);
+    if (ldx == 0) ldx = w->k;
+    if (ldy == 0) ldy = w->n;
+    if (ldx < w->k || ldy < w->n || (ldx % 8) != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions ldx=%u ldy=%u for k=%u n=%u", ldx, ldy, w->k, w->n);
+
+    const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
+    const void* xin = x;
+    uint32_t xdt = x_dtype;
+    if (rotate) {
+        // rotated f16 copy of the activations in the caller's workspace, then the GEMM reads that
+        const uint64_t need = (uint64_t)m * w->k * 2u;
+        if (!workspace || workspace_bytes < need)
+            return qwhip_fail(QWHIP_E_BASIS,
+                              "activations are not in the rotated basis and the workspace holds %llu bytes, %llu needed",
+                              (unsigned long long)workspace_bytes, (unsigned long long)need);
+        if (ldx != w->k) return qwhip_fail(QWHIP_E_BAD_SHAPE, "rotation pre-pass needs tightly packed activations");
+        st = qwhip_fwht32(s, x, x_dtype, workspace, (uint64_t)m * w->k);
+        if (st != QWHIP_OK) return st;
+        xin = workspace;
+        xdt = QWHIP_F16;
+    }
+
+    qw_gemm_params p = {};
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = xin;
+    p.y = y;
+    p.M = m;
+    p.N = w->n;
+    p.K = w->k;
+    p.ldx = ldx;
+    p.ldy = ldy;
+    p.gshift = log2_u32(w->group / 32);
+    p.bb = qwhip_view_block_bytes(w);
+    p.row_bytes = qwhip_view_row_bytes(w);
+    const uint32_t ov = (flags >> 8) & 0xFu;
+    const int cfg = ov ? (int)ov - 1 : choose_cfg(m, w->n);
+    hipError_t e;
+    if (fmt == QG_FMT_M5) e = launch_dense_xy<QG_FMT_M5>(s->stream, p, cfg, xdt, y_dtype);
+    else if (fmt == QG_FMT_B4) e = launch_dense_xy<QG_FMT_B4>(s->stream, p, cfg, xdt, y_dtype);
+    else e = launch_dense_xy<QG_FMT_B8>(s->stream, p, cfg, xdt, y_dtype);
+    QWHIP_TRY_HIP(e);
+    return QWHIP_OK;
+}
+
+// ---- grouped (MoE) -----------------------------------------------------------------------------
+namespace {
+template <int FMT, int XDT>
+hipError_t launch_grouped_y(hipStream_t st, const qw_gemm_params& p, dim3 grid, uint32_t ydt) {
+    if (ydt == QWHIP_F16) return launch_cfg<2, 2, 1, 4, FMT, XDT, QWHIP_F16, true>(st, p, grid);
+    if (ydt == QWHIP_BF16) return launch_cfg<2, 2, 1, 4, FMT, XDT, QWHIP_BF16, true>(st, p, grid);
+    return launch_cfg<2, 2, 1, 4, FMT, XDT, QWHIP_F32, true>(st, p, grid);
+}
+template <int FMT>
+hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid, uint32_t xdt, uint32_t ydt) {
+    if (xdt == QWHIP_F16) return launch_grouped_y<FMT, QWHIP_F16>(st, p, grid, ydt);
+    return launch_grouped_y<FMT, QWHIP_BF16>(st, p, grid, ydt);
+}
+}  // namespace
+
+extern "C" qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_weight_view* w, uint32_t experts, const void* x,
+                                               uint32_t x_dtype, uint32_t ldx, const int32_t* gather,
+                                               const int32_t* expert_off, const int32_t* tile_e, const int32_t* tile_r,
+                                               const int32_t* tile_count, uint32_t max_tiles, uint32_t pairs, void* y,
+                                               uint32_t y_dtype, uint32_t ldy) {
+    int fmt = 0;
+    qwhip_status st = gemm_checks(s, w, x, x_dtype, y, y_dtype, &fmt);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(expert_off);
+    QWHIP_REQUIRE(tile_e);
+    QWHIP_REQUIRE(tile_r);
+    QWHIP_REQUIRE(tile_count);
+    if (experts == 0 || experts > 512 || w->n % experts != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "grouped GEMM: %u rows do not split over %u experts (<= 512)", w->n, experts);
+    if (pairs == 0 || max_tiles == 0) return QWHIP_OK;
+    const uint32_t rows_per_expert = w->n / experts;
+    if (rows_per_expert % 16 != 0)
+        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "grouped GEMM needs rows per expert %% 16 == 0, got %u", rows_per_expert);
+    if (ldx == 0) ldx = w->k;
+    if (ldy == 0) ldy = rows_per_expert;
+    if (ldx < w->k || ldy < rows_per_expert || (ldx % 8) != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions ldx=%u ldy=%u", ldx, ldy);
+    qw_gemm_params p = {};
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = x;
+    p.y = y;
+    p.M = pairs;
+    p.N = rows_per_expert;
+    p.K = w->k;
+    p.ldx = ldx;
+    p.ldy = ldy;
+    p.gshift = log2_u32(w->group / 32);
+    p.bb = qwhip_view_block_bytes(w);
+    p.row_bytes = qwhip_view_row_bytes(w);
+    p.gather = gather;
+    p.expert_off = expert_off;
+    p.tile_e = tile_e;
+    p.tile_r = tile_r;
+    p.tile_count = tile_count;
+    p.rows_per_expert = rows_per_expert;
+    const dim3 grid(qwhip_cdiv(rows_per_expert, 256u), max_tiles);
+    hipError_t e;
+    if (fmt == QG_FMT_M5) e = launch_grouped_xy<QG_FMT_M5>(s->stream, p, grid, x_dtype, y_dtype);
+    else if (fmt == QG_FMT_B4) e = launch_grouped_xy<QG_FMT_B4>(s->stream, p, grid, x_dtype, y_dtype);
+    else e = launch_grouped_xy<QG_FMT_B8>(s->stream, p, grid, x_dtype, y_dtype);
+    QWHIP_TRY_HIP(e);
+    return QWHIP_OK;
+}

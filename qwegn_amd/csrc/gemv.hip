@@ -38,8 +38,13 @@ __device__ __forceinline__ void qw_stage_group(const void* x, uint64_t elem0, bo
 
 // ------------------------------------------------------------------------------------------------
 // Variant A: HQ4_G32_M5, m = 1, dot2.
+// Order of issue matters more than instruction count here: the whole kernel is one "breath" of about
+// ten microseconds, loads return in order, and nothing can be contracted before the rotated activation
+// is in LDS.  So: the activation loads go first, then every weight load of the wave (NB blocks per lane
+// per row, all in flight at once), then the FWHT, the barrier, and the contraction as data arrive.
+// NB = 0 selects the looped form for rows longer than 8192 columns.
 // ------------------------------------------------------------------------------------------------
-template <int R, int XDT>
+template <int R, int NB, int XDT>
 __global__ __launch_bounds__(256) void qw_gemv_hq4_dot2_kernel(const uint8_t* __restrict__ bank,
                                                                 const void* __restrict__ x, h1_t* __restrict__ y16,
                                                                 float* __restrict__ y32, uint32_t N, uint32_t K,
@@ -47,24 +52,55 @@ __global__ __launch_bounds__(256) void qw_gemv_hq4_dot2_kernel(const uint8_t* __
     extern __shared__ h8_t xs[];  // 5 h8 per 32-group (4 used): 80-byte pitch
     const uint32_t nb = K >> 5;
     const uint32_t tid = threadIdx.x;
-    for (uint32_t g = tid; g < nb; g += 256) qw_stage_group<XDT>(x, (uint64_t)g * 32, rotate != 0, xs + g * 5);
-    __syncthreads();
     const uint32_t lane = tid & 31u;
     const uint32_t row0 = (blockIdx.x * 8u + (tid >> 5)) * R;
-    if (row0 >= N) return;
+
+    // 1. activation loads (first group of this thread)
+    float xv32[32];
+    const bool xact = tid < nb;
+    if (xact) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qw_load8_f32<XDT>(x, (uint64_t)tid * 32 + 8 * j, xv32 + 8 * j);
+    }
+    // 2. weight loads
     const uint8_t* rp[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const uint32_t row = (row0 + r < N) ? row0 + r : N - 1;
         rp[r] = bank + (uint64_t)row * nb * 20u;
     }
+    constexpr int NBH = NB > 0 ? NB : 1;
+    qw_hq4_block hb[NBH][R];
+    if constexpr (NB > 0) {
+#pragma unroll
+        for (int it = 0; it < NB; ++it) {
+            uint32_t g = lane + 32u * it;
+            if (g >= nb) g = nb - 1;
+#pragma unroll
+            for (int r = 0; r < R; ++r) hb[it][r] = *(const qw_hq4_block*)(rp[r] + g * 20u);
+        }
+    }
+    // 3. rotation into LDS
+    if (xact) {
+        if (rotate) qw_fwht32(xv32);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            h8_t o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (h1_t)xv32[8 * j + e];
+            xs[tid * 5 + j] = o;
+        }
+    }
+    for (uint32_t g = tid + 256; g < nb; g += 256) qw_stage_group<XDT>(x, (uint64_t)g * 32, rotate != 0, xs + g * 5);
+    __syncthreads();
+    if (row0 >= N) return;
+
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.0f;
-    for (uint32_t g = lane; g < nb; g += 32) {
-        qw_hq4_block b[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) b[r] = *(const qw_hq4_block*)(rp[r] + g * 20u);
+
+    auto contract = [&](const qw_hq4_block* b, uint32_t g) {
         h8_t xv[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) xv[j] = xs[g * 5 + j];
@@ -74,13 +110,27 @@ __global__ __launch_bounds__(256) void qw_gemv_hq4_dot2_kernel(const uint8_t* __
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 h2_t w[4];
-                qw_unpack_hq4_word(b[r].qs[j], s2, b2, w);
+                qw_unpack_hq4_word(b[r].qs[j], s2, b2, magic, w);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const h2_t xp = {xv[j][2 * k], xv[j][2 * k + 1]};
                     acc[r] = __builtin_amdgcn_fdot2(w[k], xp, acc[r], false);
                 }
             }
+        }
+    };
+    if constexpr (NB > 0) {
+#pragma unroll
+        for (int it = 0; it < NB; ++it) {
+            const uint32_t g = lane + 32u * it;
+            if (g < nb) contract(hb[it], g);
+        }
+    } else {
+        for (uint32_t g = lane; g < nb; g += 32) {
+            qw_hq4_block b[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) b[r] = *(const qw_hq4_block*)(rp[r] + g * 20u);
+            contract(b, g);
         }
     }
 #pragma unroll
@@ -143,15 +193,15 @@ __device__ __forceinline__ void qw_load_slice(const uint8_t* rowp, uint32_t s, u
 // stripped exactly before the single f16 FMA, as qwg_aq_frag8 does,
 // Sources/QWMetal/include/qw_gemm_nax.metalh:61-71).
 template <int FMT>
-__device__ __forceinline__ h8_t qw_dequant_chunk(const qw_slice<FMT>& sl, int j, h2_t s2, h2_t b2) {
+__device__ __forceinline__ h8_t qw_dequant_chunk(const qw_slice<FMT>& sl, int j, h2_t s2, h2_t b2, uint32_t magic) {
     h2_t w[4];
     if constexpr (FMT == QW_FMT_M5) {
-        qw_unpack_hq4_word(sl.q[j], s2, b2, w);
+        qw_unpack_hq4_word(sl.q[j], s2, b2, magic, w);
     } else if constexpr (FMT == QW_FMT_B4) {
         const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const uint32_t m = ((sl.q[j] >> (4 * k)) & 0x000F000Fu) | 0x64006400u;
+            const uint32_t m = qw_and_or(sl.q[j] >> (4 * k), 0x000F000Fu, magic);
             w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m) + neg, s2, b2);
         }
     } else {
@@ -159,8 +209,8 @@ __device__ __forceinline__ h8_t qw_dequant_chunk(const qw_slice<FMT>& sl, int j,
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const uint32_t q = sl.q[2 * j + h];
-            const uint32_t m0 = (q & 0x00FF00FFu) | 0x64006400u;
-            const uint32_t m1 = ((q >> 8) & 0x00FF00FFu) | 0x64006400u;
+            const uint32_t m0 = qw_and_or(q, 0x00FF00FFu, magic);
+            const uint32_t m1 = qw_and_or(q >> 8, 0x00FF00FFu, magic);
             w[2 * h] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m0) + neg, s2, b2);
             w[2 * h + 1] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m1) + neg, s2, b2);
         }
@@ -219,7 +269,8 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __rest
     const uint32_t it0 = wave * per;
     const uint32_t it1 = min(it0 + per, iters);
 
-    qw_slice<FMT> cur[NACC], nxt[NACC];
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    qw_slice<FMT> cur[NACC] = {}, nxt[NACC] = {};
     if (it0 < it1) {
         const uint32_t s = min(4u * it0 + c, nsl - 1);
 #pragma unroll
@@ -254,7 +305,7 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __rest
             const h2_t s2 = qw_splat_lo(cur[t].hdr), b2 = qw_splat_hi(cur[t].hdr);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const h8_t a = qw_dequant_chunk<FMT>(cur[t], j, s2, b2);
+                const h8_t a = qw_dequant_chunk<FMT>(cur[t], j, s2, b2, magic);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bop[j], acc[t], 0, 0, 0);
             }
         }
@@ -408,12 +459,19 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     const size_t lds_dot2 = (size_t)(w->k / 32) * 80u;
     const bool dot2_ok = fmt == QW_FMT_M5 && m == 1 && lds_dot2 <= 60u * 1024u;
     if (variant == 1 && !dot2_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "dot2 kernel needs HQ4_G32_M5, m = 1, k <= 24576");
-    if (variant == 1 || (variant == 0 && dot2_ok && false)) {
-        const uint32_t r = (w->n >= 8192) ? 2u : 1u;
-        const dim3 grid(qwhip_cdiv(w->n, 8u * r)), block(256);
-#define QW_DOT2(R, DT) hipLaunchKernelGGL((qw_gemv_hq4_dot2_kernel<R, DT>), grid, block, lds_dot2, s->stream, a.bank, a.x, a.y16, a.y32, a.N, a.K, a.rotate)
-        if (x_dtype == QWHIP_F16) { if (r == 2) QW_DOT2(2, QWHIP_F16); else QW_DOT2(1, QWHIP_F16); }
-        else { if (r == 2) QW_DOT2(2, QWHIP_BF16); else QW_DOT2(1, QWHIP_BF16); }
+    if (variant == 1 || (variant == 0 && dot2_ok)) {
+        const uint32_t nbl = qwhip_cdiv(w->k / 32, 32);  // blocks per lane
+        const dim3 grid(qwhip_cdiv(w->n, 8u)), block(256);
+        const uint32_t nbt = nbl <= 8 ? nbl : 0;
+#define QW_DOT2(NBV, DT) hipLaunchKernelGGL((qw_gemv_hq4_dot2_kernel<1, NBV, DT>), grid, block, lds_dot2, s->stream, a.bank, a.x, a.y16, a.y32, a.N, a.K, a.rotate)
+#define QW_DOT2_NB(DT)                                                                                                   \
+        switch (nbt) {                                                                                                   \
+            case 1: QW_DOT2(1, DT); break; case 2: QW_DOT2(2, DT); break; case 3: QW_DOT2(3, DT); break;                 \
+            case 4: QW_DOT2(4, DT); break; case 5: QW_DOT2(5, DT); break; case 6: QW_DOT2(6, DT); break;                 \
+            case 7: QW_DOT2(7, DT); break; case 8: QW_DOT2(8, DT); break; default: QW_DOT2(0, DT); break;                \
+        }
+        if (x_dtype == QWHIP_F16) { QW_DOT2_NB(QWHIP_F16) } else { QW_DOT2_NB(QWHIP_BF16) }
+#undef QW_DOT2_NB
 #undef QW_DOT2
         QWHIP_TRY_HIP(hipGetLastError());
         return QWHIP_OK;

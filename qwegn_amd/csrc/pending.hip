@@ -4,8 +4,6 @@
 
 #define QW_PENDING(name) return qwhip_fail(QWHIP_E_BLOCKED, name ": no kernel in this build")
 
-extern "C" qwhip_status qwhip_gemm(qwhip_stream_t, const qwhip_weight_view*, const void*, uint32_t, uint32_t, uint32_t, void*,
-                                   uint32_t, uint32_t, uint32_t, void*, uint64_t) { QW_PENDING("qwhip_gemm"); }
 extern "C" qwhip_status qwhip_moe_route(qwhip_stream_t, const float*, uint32_t, uint32_t, uint32_t, uint32_t, float, int32_t*,
                                         float*) { QW_PENDING("qwhip_moe_route"); }
 extern "C" qwhip_status qwhip_router_gemm(qwhip_stream_t, const void*, uint32_t, const void*, uint32_t, uint32_t, uint32_t,
@@ -17,9 +15,6 @@ extern "C" uint32_t qwhip_moe_max_tiles(uint32_t experts, uint32_t pairs) {
 }
 extern "C" qwhip_status qwhip_moe_group_pairs(qwhip_stream_t, const int32_t*, uint32_t, uint32_t, uint32_t, int32_t*, int32_t*,
                                               int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, uint32_t) { QW_PENDING("qwhip_moe_group_pairs"); }
-extern "C" qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t, const qwhip_weight_view*, uint32_t, const void*, uint32_t, uint32_t,
-                                               const int32_t*, const int32_t*, const int32_t*, const int32_t*, const int32_t*,
-                                               uint32_t, uint32_t, void*, uint32_t, uint32_t) { QW_PENDING("qwhip_moe_grouped_gemm"); }
 extern "C" qwhip_status qwhip_moe_combine(qwhip_stream_t, const void*, uint32_t, const int32_t*, const float*, uint32_t, uint32_t,
                                           uint32_t, const float*, const float*, void*, uint32_t) { QW_PENDING("qwhip_moe_combine"); }
 extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t, const qwhip_weight_view*, uint32_t, const void*, uint32_t, uint32_t,

@@ -125,14 +125,27 @@ __device__ __forceinline__ void qw_fwht32(float* v) {
 // Sources/QWMetal/include/qw_weight_basis.metalh:50-63).
 __device__ __forceinline__ float qw_swiglu(float g, float u) { return (g / (1.0f + __expf(-g))) * u; }
 
+// A constant pinned in a VGPR (v_and_or_b32 is VOP3: on gfx9 it takes no literal and one scalar operand,
+// so one of mask / magic has to live in a vector register to get the single-instruction form).
+__device__ __forceinline__ uint32_t qw_vgpr_const(uint32_t c) {
+    uint32_t v = c;
+    asm volatile("" : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ uint32_t qw_and_or(uint32_t a, uint32_t mask_s, uint32_t magic_v) {
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask_s), "v"(magic_v));
+    return d;
+}
+
 // 8 HQ4_G32_M5 weights of one u32 word as four half2 (elements 0..7 in order): the nibble of element
 // 8w+j sits at bit 4*(j>>1) + 16*(j&1), so ((word >> 4k) & 0x000F000F) | 0x64006400 viewed as half2 is
 // (1024+q[2k], 1024+q[2k+1]); one packed f16 FMA with (scale, bias) gives RN_f16((1024+q)*s + b)
-// (unpack_hq4_word8, Sources/QWMetal/include/qw_dequant.metalh:42-62).
-__device__ __forceinline__ void qw_unpack_hq4_word(uint32_t word, h2_t s2, h2_t b2, h2_t* w) {
+// (unpack_hq4_word8, Sources/QWMetal/include/qw_dequant.metalh:42-62).  `magic` = qw_vgpr_const(0x64006400).
+__device__ __forceinline__ void qw_unpack_hq4_word(uint32_t word, h2_t s2, h2_t b2, uint32_t magic, h2_t* w) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const uint32_t m = ((word >> (4 * k)) & 0x000F000Fu) | 0x64006400u;
+        const uint32_t m = qw_and_or(word >> (4 * k), 0x000F000Fu, magic);
         w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m), s2, b2);
     }
 }

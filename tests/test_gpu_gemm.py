@@ -1,0 +1,119 @@
+"""GPU parity of the prefill GEMM (f16 MFMA, fp32 accumulate) against the fp64 oracle, through the C ABI.
+Bar: normalized error <= 2e-3 (bf16 / f16 stores); fp32 stores are held to 2e-5."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import qworacle as qo
+from qwegn_amd import qwhip
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return qwhip.Device(0)
+
+
+def run_gemm(dev, fmt, m, n, k, *, xdtype="bf16", ydtype="bf16", prerot=True, cfg=0, seed=0, workspace=True):
+    blocks, w16 = H.make_bank(fmt, n, k, seed=seed)
+    x32 = H.make_x(m, k, seed + 7)
+    rotate = H.FORMATS[fmt][4]
+    if xdtype == "bf16":
+        x_val, x_host, xcode = qo.round_bf16(x32), qo.f32_to_bf16_bits(x32), qwhip.BF16
+    else:
+        x_host, xcode = x32.astype(np.float16), qwhip.F16
+        x_val = x_host.astype(np.float32)
+    if prerot or not rotate:
+        # activations arrive in the container's basis; the kernel converts them to f16
+        x_basis = x_val.astype(np.float16)
+        flags = qwhip.X_PREROTATED
+    else:
+        x_basis = qo.fwht32_ortho(x_val).astype(np.float16)
+        flags = 0
+    flags |= (cfg << 8)
+    ysize = {"bf16": 2, "f16": 2, "f32": 4}[ydtype]
+    ycode = {"bf16": qwhip.BF16, "f16": qwhip.F16, "f32": qwhip.F32}[ydtype]
+    bank, xb, yb = dev.put(blocks), dev.put(x_host), dev.alloc(m * n * ysize)
+    ws = dev.alloc(m * k * 2) if workspace else None
+    view = H.view_of(dev, bank, fmt, n, k)
+    st = dev.lib.qwhip_gemm(dev.stream.handle, C.byref(view), xb.ptr, xcode, m, 0, yb.ptr, ycode, 0, flags,
+                            ws.ptr if ws else None, ws.nbytes if ws else 0)
+    out = None
+    if st == qwhip.OK:
+        dev.stream.sync()
+        if ydtype == "bf16":
+            out = qo.bf16_bits_to_f32(yb.download(np.uint16, (m, n)))
+        elif ydtype == "f16":
+            out = yb.download(np.float16, (m, n)).astype(np.float32)
+        else:
+            out = yb.download(np.float32, (m, n))
+    for b in (bank, xb, yb, ws):
+        if b is not None:
+            b.free()
+    ref = qo.matmul_ref_f64(x_basis, w16)
+    return st, out, ref
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 5])
+def test_gemm_hq4_tile_shapes_f32_out(dev, cfg):
+    st, out, ref = run_gemm(dev, "hq4_g32_m5", 512, 640, 1024, ydtype="f32", cfg=cfg)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= 2e-5
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 16, 64), (37, 48, 128), (300, 336, 192), (257, 1040, 320)])
+def test_gemm_ragged_shapes(dev, m, n, k):
+    st, out, ref = run_gemm(dev, "hq4_g32_m5", m, n, k, ydtype="f32")
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= 2e-5
+
+
+@pytest.mark.parametrize("fmt", ["aq4_g32", "hq4_g64", "hq8_g32", "hq4_g128", "aq8_g256"])
+@pytest.mark.parametrize("xdtype,ydtype", [("f16", "f16"), ("bf16", "bf16")])
+def test_gemm_block_formats(dev, fmt, xdtype, ydtype):
+    st, out, ref = run_gemm(dev, fmt, 192, 256, 768, xdtype=xdtype, ydtype=ydtype, seed=3)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= TOL
+
+
+def test_gemm_rotation_prepass_with_workspace(dev):
+    st, out, ref = run_gemm(dev, "hq4_g32_m5", 130, 256, 512, prerot=False, ydtype="f32")
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= 2e-5
+    st, _, _ = run_gemm(dev, "hq4_g32_m5", 130, 256, 512, prerot=False, workspace=False)
+    assert st == qwhip.E_BASIS
+
+
+def test_gemm_geometry_errors(dev):
+    st, _, _ = run_gemm(dev, "hq4_g32_m5", 8, 24, 64)      # n % 16 != 0
+    assert st == qwhip.E_BAD_GEOMETRY
+    st, _, _ = run_gemm(dev, "hq4_g32_m5", 8, 32, 96)      # k % 64 != 0
+    assert st == qwhip.E_BAD_GEOMETRY
+
+
+def test_gemm_matches_per_row_gemv(dev):
+    """Kernel-vs-kernel: batched GEMM against the per-row GEMV, max |diff| in f16 < 0.05
+    (Tests/QWGEMMTests/QWBatchedGemmTests.swift:130-139)."""
+    fmt, m, n, k = "hq4_g32_m5", 16, 512, 1024
+    blocks, _ = H.make_bank(fmt, n, k, seed=9)
+    x16 = H.make_x(m, k, 10).astype(np.float16)
+    bank, xb = dev.put(blocks), dev.put(x16)
+    yg, yv = dev.alloc(m * n * 2), dev.alloc(m * n * 2)
+    view = H.view_of(dev, bank, fmt, n, k)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_gemm(st, C.byref(view), xb.ptr, qwhip.F16, m, 0, yg.ptr, qwhip.F16, 0, qwhip.X_PREROTATED, None, 0))
+    qwhip.check(lib.qwhip_gemv(st, C.byref(view), xb.ptr, qwhip.F16, m, qwhip.X_PREROTATED, yv.ptr, None))
+    a = yg.download(np.float16, (m, n)).astype(np.float32)
+    b = yv.download(np.float16, (m, n)).astype(np.float32)
+    assert np.max(np.abs(a - b)) < 0.05
+
+
+def test_gemm_full_size_prefill_config(dev):
+    """HQ4_G32 prefill GEMM at its benchmark shape: M = 4096, K = 5120, N = 5120, bf16 in / bf16 out."""
+    st, out, ref = run_gemm(dev, "hq4_g32_m5", 4096, 5120, 5120, xdtype="bf16", ydtype="bf16")
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= TOL
