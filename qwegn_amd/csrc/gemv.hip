@@ -227,49 +227,18 @@ __device__ __forceinline__ h8_t qw_x_operand(const h8_t* xg, int j) {
     return b;
 }
 
-// PAIR = 1: gate|up pair mode.  The bank holds 2*N rows ([0, N) gate, [N, 2N) up); both are
-// accumulated and the epilogue stores act[m, n] = f16(FWHT32(silu(g) * u)) (rotation optional).
-template <int FMT, int RT, int XDT, int XM, int PAIR>
-__global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __restrict__ bank, const void* __restrict__ x,
-                                                            h1_t* __restrict__ y16, float* __restrict__ y32, uint32_t N,
-                                                            uint32_t K, uint32_t M, uint32_t gshift, uint32_t bb,
-                                                            uint64_t row_bytes, uint32_t rotate, uint32_t rot_out) {
-    constexpr int NACC = RT * (PAIR ? 2 : 1);
-    extern __shared__ h8_t xs[];
-    __shared__ f4_t red[4][NACC][64];
-    const uint32_t tid = threadIdx.x;
-    const uint32_t wave = tid >> 6, lane = tid & 63u;
-    const uint32_t i = lane & 15u, c = lane >> 4;
+// The K loop of one wavefront: rows rp[0..NACC) (one 16-row tile each, this lane's row already folded
+// in), K range of this wave (a quarter of the iterations), activations from LDS (XM = LDS_ROT) or
+// global memory.  acc[t] += W_t . x over the wave's K range.
+template <int FMT, int NACC, int XDT, int XM>
+__device__ __forceinline__ void qw_stream_rows(const uint8_t* const* rp, const void* x, const h8_t* xs, uint32_t xpitch8,
+                                               uint32_t K, uint32_t M, uint32_t gshift, uint32_t bb, bool rotate,
+                                               uint32_t wave, uint32_t i, uint32_t c, uint32_t magic, f4_t* acc) {
     const uint32_t nsl = K >> 5;
-    const uint32_t xpitch8 = (K >> 3) + 1;  // LDS row pitch in h8 units: K*2 + 16 bytes
-
-    if constexpr (XM == QW_XM_LDS_ROT) {
-        for (uint32_t idx = tid; idx < M * nsl; idx += 256) {
-            const uint32_t m = idx / nsl, g = idx - m * nsl;
-            qw_stage_group<XDT>(x, (uint64_t)m * K + 32u * g, rotate != 0, xs + m * xpitch8 + g * 4);
-        }
-        __syncthreads();
-    }
-
-    const uint32_t n0 = blockIdx.x * (16u * RT);
-    const uint8_t* rp[NACC];
-#pragma unroll
-    for (int t = 0; t < RT; ++t) {
-        uint32_t row = n0 + 16u * t + i;
-        if (row >= N) row = N - 1;
-        rp[t] = bank + (uint64_t)row * row_bytes;
-        if (PAIR) rp[RT + t] = bank + (uint64_t)(row + N) * row_bytes;
-    }
-    f4_t acc[NACC];
-#pragma unroll
-    for (int t = 0; t < NACC; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
-
     const uint32_t iters = (nsl + 3) >> 2;
     const uint32_t per = (iters + 3) >> 2;
     const uint32_t it0 = wave * per;
     const uint32_t it1 = min(it0 + per, iters);
-
-    const uint32_t magic = qw_vgpr_const(0x64006400u);
     qw_slice<FMT> cur[NACC] = {}, nxt[NACC] = {};
     if (it0 < it1) {
         const uint32_t s = min(4u * it0 + c, nsl - 1);
@@ -284,14 +253,13 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __rest
 #pragma unroll
             for (int t = 0; t < NACC; ++t) qw_load_slice<FMT>(rp[t], sn, gshift, bb, nxt[t]);
         }
-        // activations of slice s for row m = i
         h8_t xg[4];
         if (valid && i < M) {
             if constexpr (XM == QW_XM_LDS_ROT) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) xg[j] = xs[i * xpitch8 + s * 4 + j];
             } else {
-                qw_stage_group<XDT>(x, (uint64_t)i * K + 32u * s, rotate != 0, xg);
+                qw_stage_group<XDT>(x, (uint64_t)i * K + 32u * s, rotate, xg);
             }
         } else {
 #pragma unroll
@@ -312,6 +280,79 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __rest
 #pragma unroll
         for (int t = 0; t < NACC; ++t) cur[t] = nxt[t];
     }
+}
+
+struct qw_gemv_params {
+    const uint8_t* bank;
+    const void* x;
+    h1_t* y16;
+    float* y32;
+    uint32_t N, K, M, gshift, bb;
+    uint64_t row_bytes;
+    uint32_t rotate, rot_out;
+    // routed (MoE decode) modes
+    const int32_t* idx;
+    const float* wts;
+    uint32_t top_k;
+    uint64_t expert_bytes;  // bytes of one expert's sub-bank
+    const float* shared;
+    const float* shared_gate;
+    void* out;
+};
+
+// PAIR = 1: gate|up pair mode.  The bank holds 2*N rows ([0, N) gate, [N, 2N) up); both are accumulated
+// and the epilogue stores act[m, n] = f16(FWHT32(silu(g) * u)) (rotation optional).
+// ROUTED = 1 (with PAIR): blockIdx.y is a (token, route) pair; the expert's sub-bank is picked through
+// idx[pair], the activation row is the pair's token, the output row is the pair.
+template <int FMT, int RT, int XDT, int XM, int PAIR, int ROUTED>
+__global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const qw_gemv_params p) {
+    constexpr int NACC = RT * (PAIR ? 2 : 1);
+    extern __shared__ h8_t xs[];
+    __shared__ f4_t red[4][NACC][64];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t i = lane & 15u, c = lane >> 4;
+    const uint32_t N = p.N, K = p.K, M = p.M;
+    const uint32_t nsl = K >> 5;
+    const uint32_t xpitch8 = (K >> 3) + 1;  // LDS row pitch in h8 units: K*2 + 16 bytes
+    const uint32_t n0 = blockIdx.x * (16u * RT);
+
+    const uint8_t* bank = p.bank;
+    const void* x = p.x;
+    h1_t* y16 = p.y16;
+    if constexpr (ROUTED) {
+        const uint32_t pair = blockIdx.y;
+        const int32_t e = p.idx[pair];
+        y16 += (uint64_t)pair * N;
+        if (e < 0) {  // no expert: the pair contributes nothing
+            for (uint32_t n = n0 + tid; n < min(n0 + 16u * RT, N); n += 256) y16[n] = (h1_t)0.0f;
+            return;
+        }
+        bank += (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
+        x = (const uint8_t*)x + (uint64_t)(pair / p.top_k) * K * 2u;
+    }
+
+    if constexpr (XM == QW_XM_LDS_ROT) {
+        for (uint32_t idx = tid; idx < M * nsl; idx += 256) {
+            const uint32_t m = idx / nsl, g = idx - m * nsl;
+            qw_stage_group<XDT>(x, (uint64_t)m * K + 32u * g, p.rotate != 0, xs + m * xpitch8 + g * 4);
+        }
+        __syncthreads();
+    }
+
+    const uint8_t* rp[NACC];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        uint32_t row = n0 + 16u * t + i;
+        if (row >= N) row = N - 1;
+        rp[t] = bank + (uint64_t)row * p.row_bytes;
+        if (PAIR) rp[RT + t] = bank + (uint64_t)(row + N) * p.row_bytes;
+    }
+    f4_t acc[NACC];
+#pragma unroll
+    for (int t = 0; t < NACC; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    qw_stream_rows<FMT, NACC, XDT, XM>(rp, x, xs, xpitch8, K, M, p.gshift, p.bb, p.rotate != 0, wave, i, c, magic, acc);
 
     // split-K reduction: D[row 4c + r][col i] of every wave -> wave 0
 #pragma unroll
@@ -327,7 +368,7 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __rest
                 for (int r = 0; r < 4; ++r) {
                     const uint32_t n = n0 + 16u * t + 4u * c + r;
                     if (n < N) {
-                        if (y32) y32[(uint64_t)i * N + n] = v[r];
+                        if (p.y32) p.y32[(uint64_t)i * N + n] = v[r];
                         if (y16) y16[(uint64_t)i * N + n] = (h1_t)v[r];
                     }
                 }
@@ -351,7 +392,7 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __rest
                 float v[32];
 #pragma unroll
                 for (int e = 0; e < 32; ++e) v[e] = actbuf[tid][e];
-                if (rot_out && n0 + 32u <= N) qw_fwht32(v);
+                if (p.rot_out && n0 + 32u <= N) qw_fwht32(v);
 #pragma unroll
                 for (int e = 0; e < 32; ++e)
                     if (n0 + e < N) y16[(uint64_t)tid * N + n0 + e] = (h1_t)v[e];
@@ -363,38 +404,96 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const uint8_t* __rest
     }
 }
 
+// Routed down projection of the decode path: blockIdx.y is a token; the workgroup's 16*RT output rows
+// accumulate sum_k wts[t, k] * (W_down[e_k] . act[t, k]) over the token's routes, add the gated shared
+// expert, and store.  Activations (SwiGLU output) are already in the rotated basis.
+template <int FMT, int RT, int ODT>
+__global__ __launch_bounds__(256) void qw_moe_down_decode_kernel(const qw_gemv_params p) {
+    __shared__ f4_t red[4][RT][64];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t i = lane & 15u, c = lane >> 4;
+    const uint32_t N = p.N, K = p.K;
+    const uint32_t n0 = blockIdx.x * (16u * RT);
+    const uint32_t tok = blockIdx.y;
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    f4_t total[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) total[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+    for (uint32_t k = 0; k < p.top_k; ++k) {
+        const uint32_t pair = tok * p.top_k + k;
+        const int32_t e = p.idx[pair];
+        if (e < 0) continue;
+        const float wk = p.wts[pair];
+        const uint8_t* bank = p.bank + (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
+        const uint8_t* rp[RT];
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            uint32_t row = n0 + 16u * t + i;
+            if (row >= N) row = N - 1;
+            rp[t] = bank + (uint64_t)row * p.row_bytes;
+        }
+        f4_t acc[RT];
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+        const void* x = (const uint8_t*)p.x + (uint64_t)pair * K * 2u;
+        qw_stream_rows<FMT, RT, QWHIP_F16, QW_XM_GLOBAL>(rp, x, nullptr, 0, K, 1, p.gshift, p.bb, false, wave, i, c, magic, acc);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) total[t] += acc[t] * wk;
+    }
+#pragma unroll
+    for (int t = 0; t < RT; ++t) red[wave][t][lane] = total[t];
+    __syncthreads();
+    if (wave != 0 || i != 0) return;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const f4_t v = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t n = n0 + 16u * t + 4u * c + r;
+            if (n < N) {
+                float o = v[r];
+                const uint64_t at = (uint64_t)tok * N + n;
+                if (p.shared) o = fmaf(p.shared_gate ? p.shared_gate[tok] : 1.0f, p.shared[at], o);
+                if constexpr (ODT == QWHIP_F32) ((float*)p.out)[at] = o;
+                else if constexpr (ODT == QWHIP_F16) ((h1_t*)p.out)[at] = (h1_t)o;
+                else ((uint16_t*)p.out)[at] = qw_f32_to_bf16(o);
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-struct gemv_args {
-    const uint8_t* bank;
-    const void* x;
-    h1_t* y16;
-    float* y32;
-    uint32_t N, K, M, gshift, bb;
-    uint64_t row_bytes;
-    uint32_t rotate, rot_out;
-};
+typedef qw_gemv_params gemv_args;
 
 template <int FMT, int RT, int XDT, int XM, int PAIR>
-void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds) {
-    const dim3 grid(qwhip_cdiv(a.N, 16u * RT)), block(256);
-    hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR>), grid, block, lds, st, a.bank, a.x, a.y16, a.y32, a.N,
-                       a.K, a.M, a.gshift, a.bb, a.row_bytes, a.rotate, a.rot_out);
+void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds, uint32_t routed_pairs = 0) {
+    const dim3 block(256);
+    if (routed_pairs) {
+        if constexpr (PAIR) {
+            const dim3 grid(qwhip_cdiv(a.N, 16u * RT), routed_pairs);
+            hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1>), grid, block, lds, st, a);
+        }
+    } else {
+        const dim3 grid(qwhip_cdiv(a.N, 16u * RT));
+        hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0>), grid, block, lds, st, a);
+    }
 }
 
 template <int FMT, int RT, int XDT, int PAIR>
-void launch_mfma_xm(hipStream_t st, const gemv_args& a, int xm, size_t lds) {
-    if (xm == QW_XM_LDS_ROT) launch_mfma<FMT, RT, XDT, QW_XM_LDS_ROT, PAIR>(st, a, lds);
-    else launch_mfma<FMT, RT, XDT, QW_XM_GLOBAL, PAIR>(st, a, 0);
+void launch_mfma_xm(hipStream_t st, const gemv_args& a, int xm, size_t lds, uint32_t routed_pairs = 0) {
+    if (xm == QW_XM_LDS_ROT) launch_mfma<FMT, RT, XDT, QW_XM_LDS_ROT, PAIR>(st, a, lds, routed_pairs);
+    else launch_mfma<FMT, RT, XDT, QW_XM_GLOBAL, PAIR>(st, a, 0, routed_pairs);
 }
 
 template <int FMT, int RT, int PAIR>
-void launch_mfma_dt(hipStream_t st, const gemv_args& a, uint32_t xdt, int xm, size_t lds) {
-    if (xdt == QWHIP_F16) launch_mfma_xm<FMT, RT, QWHIP_F16, PAIR>(st, a, xm, lds);
-    else launch_mfma_xm<FMT, RT, QWHIP_BF16, PAIR>(st, a, xm, lds);
+void launch_mfma_dt(hipStream_t st, const gemv_args& a, uint32_t xdt, int xm, size_t lds, uint32_t routed_pairs = 0) {
+    if (xdt == QWHIP_F16) launch_mfma_xm<FMT, RT, QWHIP_F16, PAIR>(st, a, xm, lds, routed_pairs);
+    else launch_mfma_xm<FMT, RT, QWHIP_BF16, PAIR>(st, a, xm, lds, routed_pairs);
 }
 
 template <int FMT>
@@ -442,7 +541,7 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     const uint32_t variant = (flags >> 8) & 0xFu;
     uint32_t rt = (flags >> 12) & 0xFu;
 
-    gemv_args a;
+    gemv_args a = {};
     a.bank = (const uint8_t*)w->blocks;
     a.x = x;
     a.y16 = (h1_t*)y16;
@@ -498,7 +597,7 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     if (w->n % 2 != 0) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "gate|up bank needs an even row count, got %u", w->n);
     const uint32_t inter = w->n / 2;
     const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
-    gemv_args a;
+    gemv_args a = {};
     a.bank = (const uint8_t*)w->blocks;
     a.x = x;
     a.y16 = (h1_t*)act16;
@@ -517,6 +616,95 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     if (fmt == QW_FMT_M5) launch_mfma_dt<QW_FMT_M5, 2, 1>(s->stream, a, x_dtype, xm, lds);
     else if (fmt == QW_FMT_B4) launch_mfma_dt<QW_FMT_B4, 2, 1>(s->stream, a, x_dtype, xm, lds);
     else launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// ---- MoE decode / verify (t <= 8): routed experts as GEMVs -----------------------------------------
+extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                                const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
+                                                uint32_t top_k, void* act16) {
+    int fmt = 0;
+    qwhip_status st = check_common(s, w_gate_up, x, x_dtype, 1, &fmt);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(act16);
+    if (t == 0 || top_k == 0) return QWHIP_OK;
+    if (experts == 0 || experts > 512 || w_gate_up->n % (2 * experts) != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "gate|up bank of %u rows does not split over %u experts", w_gate_up->n, experts);
+    if ((uint64_t)t * top_k > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "decode path holds at most 65535 (token, route) pairs");
+    const uint32_t inter = w_gate_up->n / (2 * experts);
+    const bool rotate = qwhip_view_rotated(w_gate_up) && !(flags & QWHIP_X_PREROTATED);
+    gemv_args a = {};
+    a.bank = (const uint8_t*)w_gate_up->blocks;
+    a.x = x;
+    a.y16 = (h1_t*)act16;
+    a.N = inter;
+    a.K = w_gate_up->k;
+    a.M = 1;
+    a.gshift = log2_u32(w_gate_up->group / 32);
+    a.bb = qwhip_view_block_bytes(w_gate_up);
+    a.row_bytes = qwhip_view_row_bytes(w_gate_up);
+    a.rotate = rotate ? 1u : 0u;
+    a.rot_out = (qwhip_view_rotated(w_gate_up) && inter % 32 == 0) ? 1u : 0u;
+    a.idx = idx;
+    a.top_k = top_k;
+    a.expert_bytes = (uint64_t)2 * inter * a.row_bytes;
+    const size_t lds_x = (size_t)w_gate_up->k * 2u + 16u;
+    const int xm = (rotate && lds_x <= 48u * 1024u) ? QW_XM_LDS_ROT : QW_XM_GLOBAL;
+    const size_t lds = xm == QW_XM_LDS_ROT ? lds_x : 0;
+    const uint32_t pairs = t * top_k;
+    if (fmt == QW_FMT_M5) launch_mfma_dt<QW_FMT_M5, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs);
+    else if (fmt == QW_FMT_B4) launch_mfma_dt<QW_FMT_B4, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs);
+    else launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts,
+                                              const void* act16, const int32_t* idx, const float* wts, uint32_t t, uint32_t top_k,
+                                              const float* shared, const float* shared_gate, void* out, uint32_t out_dtype) {
+    int fmt = 0;
+    qwhip_status st = check_common(s, w_down, act16, QWHIP_F16, 1, &fmt);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(wts);
+    QWHIP_REQUIRE(out);
+    if (t == 0 || top_k == 0) return QWHIP_OK;
+    if (experts == 0 || experts > 512 || w_down->n % experts != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "down bank of %u rows does not split over %u experts", w_down->n, experts);
+    if (t > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "decode path holds at most 65535 tokens");
+    if ((w_down->k * 2u) % 16u != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "activation rows must be 16-byte multiples");
+    const uint32_t hidden = w_down->n / experts;
+    gemv_args a = {};
+    a.bank = (const uint8_t*)w_down->blocks;
+    a.x = act16;
+    a.N = hidden;
+    a.K = w_down->k;
+    a.M = 1;
+    a.gshift = log2_u32(w_down->group / 32);
+    a.bb = qwhip_view_block_bytes(w_down);
+    a.row_bytes = qwhip_view_row_bytes(w_down);
+    a.idx = idx;
+    a.wts = wts;
+    a.top_k = top_k;
+    a.expert_bytes = (uint64_t)hidden * a.row_bytes;
+    a.shared = shared;
+    a.shared_gate = shared_gate;
+    a.out = out;
+    const dim3 grid(qwhip_cdiv(hidden, 16u)), block(256);
+    const dim3 g2(grid.x, t);
+#define QW_DD(F, OD) hipLaunchKernelGGL((qw_moe_down_decode_kernel<F, 1, OD>), g2, block, 0, s->stream, a)
+#define QW_DD_O(F)                                                                                          \
+    switch (out_dtype) {                                                                                    \
+        case QWHIP_F32: QW_DD(F, QWHIP_F32); break;                                                         \
+        case QWHIP_F16: QW_DD(F, QWHIP_F16); break;                                                         \
+        case QWHIP_BF16: QW_DD(F, QWHIP_BF16); break;                                                       \
+        default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe down: unsupported output dtype %u", out_dtype);  \
+    }
+    if (fmt == QW_FMT_M5) { QW_DD_O(QW_FMT_M5) } else if (fmt == QW_FMT_B4) { QW_DD_O(QW_FMT_B4) } else { QW_DD_O(QW_FMT_B8) }
+#undef QW_DD_O
+#undef QW_DD
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }

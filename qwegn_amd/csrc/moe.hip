@@ -1,0 +1,369 @@
+// MoE plumbing around the grouped GEMM: router logits, softmax top-k routing, the expert-major pair sort
+// with its tile list, and the weighted combine.
+#include "qwhip_common.h"
+
+// ------------------------------------------------------------------------------------------------
+// Router logits: logits[t, e] = sum_h x[t, h] * Wr[e, h], fp32 accumulate.
+// A workgroup owns 8 token rows (staged as fp32 in LDS) so each router row is read once per 8 tokens;
+// a wavefront owns experts wave, wave+4, ...; lanes stride the hidden dimension.
+// ------------------------------------------------------------------------------------------------
+template <int XDT, int WDT>
+__global__ __launch_bounds__(256) void qw_router_gemm_kernel(const void* __restrict__ x, const void* __restrict__ wr,
+                                                              float* __restrict__ logits, uint32_t T, uint32_t E, uint32_t H) {
+    constexpr int TT = 8;
+    extern __shared__ float xs[];  // [TT][H]
+    const uint32_t t0 = blockIdx.x * TT;
+    const uint32_t nt = min((uint32_t)TT, T - t0);
+    for (uint32_t i = threadIdx.x; i < TT * H; i += 256) {
+        const uint32_t r = i / H, h = i - r * H;
+        xs[i] = r < nt ? qw_load_f32<XDT>(x, (uint64_t)(t0 + r) * H + h) : 0.0f;
+    }
+    __syncthreads();
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    for (uint32_t e = wave; e < E; e += 4) {
+        float acc[TT];
+#pragma unroll
+        for (int r = 0; r < TT; ++r) acc[r] = 0.0f;
+        for (uint32_t h = lane; h < H; h += 64) {
+            const float w = qw_load_f32<WDT>(wr, (uint64_t)e * H + h);
+#pragma unroll
+            for (int r = 0; r < TT; ++r) acc[r] = fmaf(w, xs[r * H + h], acc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < TT; ++r) {
+            const float v = qw_reduce64(acc[r]);
+            if (lane == 0 && (uint32_t)r < nt) logits[(uint64_t)(t0 + r) * E + e] = v;
+        }
+    }
+}
+
+extern "C" qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
+                                          uint32_t t, uint32_t experts, uint32_t hidden, float* logits) {
+    QWHIP_REQUIRE(s);
+    if (t == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(x);
+    QWHIP_REQUIRE(wr);
+    QWHIP_REQUIRE(logits);
+    if (experts == 0 || hidden == 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: empty experts or hidden");
+    const size_t lds = (size_t)8 * hidden * 4;
+    if (lds > 64u * 1024u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: hidden %u exceeds the staged tile (<= 2048)", hidden);
+    const dim3 grid(qwhip_cdiv(t, 8)), block(256);
+#define QW_RG(XD, WD) hipLaunchKernelGGL((qw_router_gemm_kernel<XD, WD>), grid, block, lds, s->stream, x, wr, logits, t, experts, hidden)
+#define QW_RG_W(XD)                                                   \
+    switch (w_dtype) {                                                \
+        case QWHIP_F32: QW_RG(XD, QWHIP_F32); break;                  \
+        case QWHIP_F16: QW_RG(XD, QWHIP_F16); break;                  \
+        case QWHIP_BF16: QW_RG(XD, QWHIP_BF16); break;                \
+        default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: unsupported weight dtype %u", w_dtype); \
+    }
+    switch (x_dtype) {
+        case QWHIP_F32: QW_RG_W(QWHIP_F32) break;
+        case QWHIP_F16: QW_RG_W(QWHIP_F16) break;
+        case QWHIP_BF16: QW_RG_W(QWHIP_BF16) break;
+        default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: unsupported activation dtype %u", x_dtype);
+    }
+#undef QW_RG_W
+#undef QW_RG
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Routing: one wavefront per token row; lane l holds experts l, l+64, ... (E <= 512 -> <= 8 each).
+// fp32 softmax (max-subtracted), top_k rounds of argmax with ties to the lower index, optional
+// renormalisation by the sum of the selected, times the routed scale.  Non-finite logits never win.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ bool qw_finite(float v) { return (__float_as_uint(v) & 0x7F800000u) != 0x7F800000u; }
+
+__global__ __launch_bounds__(64) void qw_moe_route_kernel(const float* __restrict__ logits, int32_t* __restrict__ idx,
+                                                           float* __restrict__ wts, uint32_t E, uint32_t K, uint32_t norm,
+                                                           float routed_scale) {
+    const uint32_t t = blockIdx.x, lane = threadIdx.x;
+    const uint32_t JN = (E + 63u) >> 6;
+    float p[8];
+    bool ok[8];
+    float mx = -3.4e38f;
+    bool any_finite = false;
+#pragma unroll
+    for (uint32_t j = 0; j < 8; ++j) {
+        const uint32_t id = lane + 64u * j;
+        float v = 0.0f;
+        ok[j] = false;
+        if (j < JN && id < E) {
+            v = logits[(uint64_t)t * E + id];
+            ok[j] = qw_finite(v);
+            if (ok[j]) {
+                mx = any_finite ? fmaxf(mx, v) : v;
+                any_finite = true;
+            }
+        }
+        p[j] = v;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float total = 0.0f;
+#pragma unroll
+    for (uint32_t j = 0; j < 8; ++j) {
+        p[j] = ok[j] ? expf(p[j] - mx) : 0.0f;
+        total += p[j];
+    }
+    total = qw_reduce64(total);
+#pragma unroll
+    for (uint32_t j = 0; j < 8; ++j) {
+        ok[j] = ok[j] && total > 0.0f;
+        p[j] = ok[j] ? p[j] / total : -1e30f;
+    }
+    float wsel = 0.0f;  // lane r keeps the weight of rank r (K <= 16 < 64)
+    int32_t isel = -1;
+    for (uint32_t r = 0; r < K; ++r) {
+        float bv = -3.4e38f;
+        uint32_t bi = 0xFFFFFFFFu;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t id = lane + 64u * j;
+            if (ok[j] && (bi == 0xFFFFFFFFu || p[j] > bv)) {  // ascending id within the lane: strict > keeps the lower id
+                bv = p[j];
+                bi = id;
+            }
+        }
+        // wave argmax, ties to the lower id
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const uint32_t oi = __shfl_xor(bi, off, 64);
+            if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi))) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if (bi != 0xFFFFFFFFu && (bi & 63u) == lane) {
+#pragma unroll
+            for (uint32_t j = 0; j < 8; ++j)
+                if (j == (bi >> 6)) ok[j] = false;
+        }
+        if (lane == r) {
+            wsel = bi != 0xFFFFFFFFu ? bv : 0.0f;
+            isel = bi != 0xFFFFFFFFu ? (int32_t)bi : -1;
+        }
+    }
+    // sum of the selected in rank order (lane 0 .. K-1), as the reference's serial loop
+    float acc = 0.0f;
+    for (uint32_t r = 0; r < K; ++r) acc += __shfl(wsel, (int)r, 64);
+    if (lane < K) {
+        float w = wsel;
+        if (norm) w = acc > 0.0f ? w / acc : 0.0f;
+        idx[(uint64_t)t * K + lane] = isel;
+        wts[(uint64_t)t * K + lane] = w * routed_scale;
+    }
+}
+
+extern "C" qwhip_status qwhip_moe_route(qwhip_stream_t s, const float* logits, uint32_t t, uint32_t experts, uint32_t top_k,
+                                        uint32_t norm_topk, float routed_scale, int32_t* idx, float* wts) {
+    QWHIP_REQUIRE(s);
+    if (t == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(logits);
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(wts);
+    if (experts == 0 || experts > 512) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: experts must be 1..512, got %u", experts);
+    if (top_k == 0 || top_k > 16) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: top_k must be 1..16, got %u", top_k);
+    const float scale = routed_scale > 0.0f ? routed_scale : 1.0f;
+    hipLaunchKernelGGL(qw_moe_route_kernel, dim3(t), dim3(64), 0, s->stream, logits, idx, wts, experts, top_k,
+                       norm_topk ? 1u : 0u, scale);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Expert-major pair sort: counting sort by expert id in one 1024-thread workgroup, plus the tile list.
+// ------------------------------------------------------------------------------------------------
+extern "C" uint32_t qwhip_moe_max_tiles(uint32_t experts, uint32_t pairs) {
+    const uint32_t a = experts < pairs ? experts : pairs;
+    const uint32_t b = a + (pairs + 63u) / 64u;
+    return pairs < b ? pairs : b;
+}
+
+__device__ __forceinline__ int qw_moe_tile_block(int c) { return c <= 16 ? 16 : (c <= 32 ? 32 : 64); }
+__device__ __forceinline__ int qw_moe_pack_tile_r(int tid_y, int bm) {
+    const int code = (bm == 16) ? 1 : ((bm == 32) ? 2 : 3);
+    return (code << 24) | (tid_y & 0xFFFFFF);
+}
+
+__global__ __launch_bounds__(1024) void qw_moe_group_pairs_kernel(const int32_t* __restrict__ ids, uint32_t experts,
+                                                                   uint32_t pairs, uint32_t top_k, int32_t* __restrict__ expert_off,
+                                                                   int32_t* __restrict__ sorted_pair, int32_t* __restrict__ sorted_tok,
+                                                                   int32_t* __restrict__ inv_perm, int32_t* __restrict__ tile_e,
+                                                                   int32_t* __restrict__ tile_r, int32_t* __restrict__ tile_count,
+                                                                   uint32_t compact_tail) {
+    __shared__ int cnt[512];
+    __shared__ int off[513];
+    __shared__ int cursor[512];
+    __shared__ int tile_off[513];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t e = tid; e < experts; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < pairs; i += 1024) {
+        const int32_t raw = ids[i];
+        if (raw >= 0) {
+            const uint32_t e = (uint32_t)raw & 0xFFFFu;
+            if (e < experts) atomicAdd(&cnt[e], 1);
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        // serial scan over <= 512 experts: rows and tiles
+        int c = 0, t = 0;
+        for (uint32_t e = 0; e < experts; ++e) {
+            off[e] = c;
+            tile_off[e] = t;
+            const int n = cnt[e];
+            c += n;
+            if (n > 0) {
+                if (compact_tail) t += (n >> 6) + ((n & 63) ? 1 : 0);
+                else {
+                    const int bm = qw_moe_tile_block(n);
+                    t += (n + bm - 1) / bm;
+                }
+            }
+        }
+        off[experts] = c;
+        tile_off[experts] = t;
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e <= experts; e += 1024) {
+        expert_off[e] = off[e];
+        if (e < experts) cursor[e] = off[e];
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < pairs; i += 1024) {
+        const int32_t raw = ids[i];
+        bool placed = false;
+        if (raw >= 0) {
+            const uint32_t e = (uint32_t)raw & 0xFFFFu;
+            if (e < experts) {
+                const int at = atomicAdd(&cursor[e], 1);
+                sorted_pair[at] = (int32_t)i;
+                sorted_tok[at] = (int32_t)(i / top_k);
+                if (inv_perm) inv_perm[i] = at;
+                placed = true;
+            }
+        }
+        if (!placed && inv_perm) inv_perm[i] = -1;
+    }
+    if (tile_e) {
+        for (uint32_t e = tid; e < experts; e += 1024) {
+            const int n = cnt[e];
+            int t = tile_off[e];
+            if (n <= 0) continue;
+            if (compact_tail) {
+                const int q = n >> 6, rem = n & 63;
+                for (int r = 0; r < q; ++r) {
+                    tile_e[t] = (int32_t)e;
+                    tile_r[t] = qw_moe_pack_tile_r(r, 64);
+                    ++t;
+                }
+                if (rem > 0) {
+                    const int bm = qw_moe_tile_block(rem);
+                    tile_e[t] = (int32_t)e;
+                    tile_r[t] = qw_moe_pack_tile_r((q * 64) / bm, bm);
+                }
+            } else {
+                const int bm = qw_moe_tile_block(n);
+                for (int r = 0; r * bm < n; ++r) {
+                    tile_e[t] = (int32_t)e;
+                    tile_r[t] = qw_moe_pack_tile_r(r, bm);
+                    ++t;
+                }
+            }
+        }
+        if (tid == 0) tile_count[0] = tile_off[experts];
+    }
+}
+
+extern "C" qwhip_status qwhip_moe_group_pairs(qwhip_stream_t s, const int32_t* ids, uint32_t experts, uint32_t pairs,
+                                              uint32_t top_k, int32_t* expert_off, int32_t* sorted_pair, int32_t* sorted_tok,
+                                              int32_t* inv_perm, int32_t* tile_e, int32_t* tile_r, int32_t* tile_count,
+                                              uint32_t compact_tail) {
+    QWHIP_REQUIRE(s);
+    QWHIP_REQUIRE(ids);
+    QWHIP_REQUIRE(expert_off);
+    QWHIP_REQUIRE(sorted_pair);
+    QWHIP_REQUIRE(sorted_tok);
+    if (experts == 0 || experts > 512)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "the expert-sorted pair order holds 512 experts, got %u", experts);
+    if (top_k == 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe group pairs: top_k must be positive");
+    const bool tiles = tile_e || tile_r || tile_count;
+    if (tiles && !(tile_e && tile_r && tile_count))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe group pairs: tile_e, tile_r and tile_count come together");
+    hipLaunchKernelGGL(qw_moe_group_pairs_kernel, dim3(1), dim3(1024), 0, s->stream, ids, experts, pairs, top_k, expert_off,
+                       sorted_pair, sorted_tok, inv_perm, tile_e, tile_r, tile_count, compact_tail ? 1u : 0u);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Combine: out[t, h] = sum_k wts[t, k] * dn[inv_perm[t*K + k], h] (+ shared_gate[t] * shared[t, h]).
+// One thread per 4 consecutive h; fp32 accumulation in rank order.
+// ------------------------------------------------------------------------------------------------
+template <int DDT, int ODT>
+__global__ __launch_bounds__(256) void qw_moe_combine_kernel(const void* __restrict__ dn, const int32_t* __restrict__ inv_perm,
+                                                              const float* __restrict__ wts, uint32_t T, uint32_t K, uint32_t H,
+                                                              const float* __restrict__ shared, const float* __restrict__ shared_gate,
+                                                              void* __restrict__ out) {
+    const uint32_t t = blockIdx.y;
+    const uint32_t h = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (h >= H) return;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t k = 0; k < K; ++k) {
+        const int32_t slot = inv_perm[(uint64_t)t * K + k];
+        if (slot < 0) continue;
+        const float w = wts[(uint64_t)t * K + k];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (h + j < H) acc[j] = fmaf(w, qw_load_f32<DDT>(dn, (uint64_t)slot * H + h + j), acc[j]);
+    }
+    if (shared) {
+        const float g = shared_gate ? shared_gate[t] : 1.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (h + j < H) acc[j] = fmaf(g, shared[(uint64_t)t * H + h + j], acc[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (h + j < H) {
+            const uint64_t o = (uint64_t)t * H + h + j;
+            if constexpr (ODT == QWHIP_F32) ((float*)out)[o] = acc[j];
+            else if constexpr (ODT == QWHIP_F16) ((h1_t*)out)[o] = (h1_t)acc[j];
+            else ((uint16_t*)out)[o] = qw_f32_to_bf16(acc[j]);
+        }
+    }
+}
+
+extern "C" qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint32_t dn_dtype, const int32_t* inv_perm,
+                                          const float* wts, uint32_t t, uint32_t top_k, uint32_t hidden, const float* shared,
+                                          const float* shared_gate, void* out, uint32_t out_dtype) {
+    QWHIP_REQUIRE(s);
+    if (t == 0 || hidden == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(dn);
+    QWHIP_REQUIRE(inv_perm);
+    QWHIP_REQUIRE(wts);
+    QWHIP_REQUIRE(out);
+    const dim3 grid(qwhip_cdiv(hidden, 1024), t), block(256);
+#define QW_CB(DD, OD) hipLaunchKernelGGL((qw_moe_combine_kernel<DD, OD>), grid, block, 0, s->stream, dn, inv_perm, wts, t, top_k, hidden, shared, shared_gate, out)
+#define QW_CB_O(DD)                                                   \
+    switch (out_dtype) {                                              \
+        case QWHIP_F32: QW_CB(DD, QWHIP_F32); break;                  \
+        case QWHIP_F16: QW_CB(DD, QWHIP_F16); break;                  \
+        case QWHIP_BF16: QW_CB(DD, QWHIP_BF16); break;                \
+        default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine: unsupported output dtype %u", out_dtype); \
+    }
+    switch (dn_dtype) {
+        case QWHIP_F32: QW_CB_O(QWHIP_F32) break;
+        case QWHIP_F16: QW_CB_O(QWHIP_F16) break;
+        case QWHIP_BF16: QW_CB_O(QWHIP_BF16) break;
+        default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine: unsupported input dtype %u", dn_dtype);
+    }
+#undef QW_CB_O
+#undef QW_CB
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}

@@ -1,0 +1,214 @@
+"""GPU parity of the MoE pieces (router, routing, pair sort + tile list, grouped GEMM, combine, decode
+GEMVs) and of the whole routed block against the CPU oracle, through the C ABI."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import qworacle as qo
+from qwegn_amd import qwhip
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return qwhip.Device(0)
+
+
+def _route(dev, logits, k, norm=True, scale=1.0):
+    t, e = logits.shape
+    lb, ib, wb = dev.put(logits.astype(np.float32)), dev.alloc(t * k * 4), dev.alloc(t * k * 4)
+    qwhip.check(dev.lib.qwhip_moe_route(dev.stream.handle, lb.ptr, t, e, k, 1 if norm else 0, scale, ib.ptr, wb.ptr))
+    return ib.download(np.int32, (t, k)), wb.download(np.float32, (t, k))
+
+
+@pytest.mark.parametrize("t,e,k", [(64, 128, 8), (5, 8, 2), (33, 512, 16), (7, 100, 3)])
+def test_moe_route_matches_oracle(dev, t, e, k):
+    rng = np.random.default_rng(e + k)
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    idx, wts = _route(dev, logits, k, norm=True, scale=2.5)
+    ridx, rwts = qo.moe_route(logits, k, norm_topk=True, routed_scale=2.5)
+    assert np.array_equal(idx, ridx)
+    np.testing.assert_allclose(wts, rwts, rtol=2e-6, atol=1e-9)
+    idx2, wts2 = _route(dev, logits, k, norm=False)
+    ridx2, rwts2 = qo.moe_route(logits, k, norm_topk=False)
+    assert np.array_equal(idx2, ridx2)
+    np.testing.assert_allclose(wts2, rwts2, rtol=2e-6, atol=1e-9)
+
+
+def test_moe_route_ties_and_non_finite(dev):
+    logits = np.zeros((3, 64), dtype=np.float32)          # all tied: lowest indices win, in order
+    logits[1, 10] = np.inf                                 # non-finite never wins
+    logits[1, 11] = np.nan
+    logits[2, :] = -np.inf                                 # nothing to select
+    logits[2, 5] = 1.0
+    idx, wts = _route(dev, logits, 4)
+    assert idx[0].tolist() == [0, 1, 2, 3]
+    assert 10 not in idx[1] and 11 not in idx[1] and idx[1].tolist() == [0, 1, 2, 3]
+    assert idx[2].tolist() == [5, -1, -1, -1]
+    assert wts[2].tolist() == [1.0, 0.0, 0.0, 0.0]
+    np.testing.assert_allclose(wts[0], 0.25, rtol=1e-6)
+
+
+@pytest.mark.parametrize("xdt", ["f32", "bf16", "f16"])
+def test_router_gemm(dev, xdt):
+    t, e, h = 19, 128, 2048
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((t, h)).astype(np.float32)
+    wr = (rng.standard_normal((e, h)) * 0.05).astype(np.float32)
+    if xdt == "f32":
+        xh, code, xv = x, qwhip.F32, x
+    elif xdt == "bf16":
+        xh, code, xv = qo.f32_to_bf16_bits(x), qwhip.BF16, qo.round_bf16(x)
+    else:
+        xh, code = x.astype(np.float16), qwhip.F16
+        xv = xh.astype(np.float32)
+    xb, wb, lb = dev.put(xh), dev.put(wr), dev.alloc(t * e * 4)
+    qwhip.check(dev.lib.qwhip_router_gemm(dev.stream.handle, xb.ptr, code, wb.ptr, qwhip.F32, t, e, h, lb.ptr))
+    got = lb.download(np.float32, (t, e))
+    ref = xv.astype(np.float64) @ wr.astype(np.float64).T
+    assert qo.normalized_error(got, ref) <= 1e-5
+
+
+def _group(dev, ids, experts, top_k, compact=True):
+    pairs = ids.size
+    mt = max(1, dev.lib.qwhip_moe_max_tiles(experts, pairs))
+    b = dict(ids=dev.put(ids.astype(np.int32)), off=dev.alloc((experts + 1) * 4), sp=dev.alloc(pairs * 4), stok=dev.alloc(pairs * 4),
+             inv=dev.alloc(pairs * 4), te=dev.alloc(mt * 4), tr=dev.alloc(mt * 4), tc=dev.alloc(16))
+    qwhip.check(dev.lib.qwhip_moe_group_pairs(dev.stream.handle, b["ids"].ptr, experts, pairs, top_k, b["off"].ptr, b["sp"].ptr,
+                                              b["stok"].ptr, b["inv"].ptr, b["te"].ptr, b["tr"].ptr, b["tc"].ptr, 1 if compact else 0))
+    dev.stream.sync()
+    out = dict(off=b["off"].download(np.int32, (experts + 1,)), sp=b["sp"].download(np.int32, (pairs,)),
+               stok=b["stok"].download(np.int32, (pairs,)), inv=b["inv"].download(np.int32, (pairs,)),
+               tc=int(b["tc"].download(np.int32, (1,))[0]))
+    out["te"] = b["te"].download(np.int32, (mt,))[: out["tc"]]
+    out["tr"] = b["tr"].download(np.int32, (mt,))[: out["tc"]]
+    out["bufs"], out["max_tiles"] = b, mt
+    return out
+
+
+@pytest.mark.parametrize("t,e,k,compact", [(300, 128, 8, True), (300, 128, 8, False), (3, 16, 2, True), (2048, 128, 8, True), (50, 512, 16, True)])
+def test_moe_group_pairs_invariants_and_tiles(dev, t, e, k, compact):
+    """Sort invariants (Tests/QWFlashNextMetalTests/MoE/FNMetalMoEGroupTests.swift:80-92) and the tile list
+    against the closed forms of QWGemmMoE.swift:24-62 / qw_moe_tile.metalh."""
+    rng = np.random.default_rng(t + e)
+    ids = np.stack([rng.choice(e, size=k, replace=False) for _ in range(t)]).astype(np.int32)
+    ids[rng.random(ids.shape) < 0.02] = -1                     # a few empty routes
+    g = _group(dev, ids, e, k, compact)
+    ref = qo.moe_group_pairs(ids, e, k, compact_tail=compact)
+    valid = int((ids >= 0).sum())
+    assert g["off"][0] == 0 and g["off"][e] == valid and np.all(np.diff(g["off"]) >= 0)
+    assert np.array_equal(g["off"], ref["expertOff"])
+    sp = g["sp"][:valid]
+    assert np.array_equal(np.sort(sp), np.flatnonzero(ids.ravel() >= 0))           # each valid pair exactly once
+    assert np.array_equal(g["stok"][:valid], sp // k)
+    assert np.array_equal(g["inv"][sp], np.arange(valid))                           # invPerm o sortedPairIdx = id
+    assert np.all(g["inv"][ids.ravel() < 0] == -1)
+    flat = ids.ravel()
+    for ex in range(e):                                                             # slots of expert ex hold its pairs
+        assert np.all(flat[sp[g["off"][ex]:g["off"][ex + 1]]] == ex)
+    assert g["tc"] == ref["tileCount"] <= g["max_tiles"]
+    assert np.array_equal(g["te"], ref["tileE"]) and np.array_equal(g["tr"], ref["tileR"])
+
+
+def _moe_banks(experts, hidden, inter, seed, fmt="hq4_g32_m5"):
+    gu_blocks, gu16 = H.make_bank(fmt, experts * 2 * inter, hidden, seed)
+    dn_blocks, dn16 = H.make_bank(fmt, experts * hidden, inter, seed + 1)
+    return gu_blocks, gu16.reshape(experts, 2 * inter, hidden), dn_blocks, dn16.reshape(experts, hidden, inter)
+
+
+@pytest.mark.parametrize("t,experts,hidden,inter,k", [(40, 8, 256, 128, 2), (130, 16, 512, 192, 4)])
+def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
+    """route -> pair sort -> grouped gate_up GEMM -> SwiGLU+FWHT -> grouped down GEMM -> combine."""
+    fmt = "hq4_g32_m5"
+    gu_blocks, gu16, dn_blocks, dn16 = _moe_banks(experts, hidden, inter, seed=11)
+    rng = np.random.default_rng(5)
+    x16 = qo.rotate_activation_f16(rng.standard_normal((t, hidden)).astype(np.float32))     # rotated f16 hidden
+    logits = rng.standard_normal((t, experts)).astype(np.float32)
+    idx, wts = _route(dev, logits, k)
+    g = _group(dev, idx, experts, k)
+    pairs = t * k
+    lib, st, b = dev.lib, dev.stream.handle, g["bufs"]
+    gub, dnb, xb = dev.put(gu_blocks), dev.put(dn_blocks), dev.put(x16)
+    gu_out, act, dn_out, out = dev.alloc(pairs * 2 * inter * 2), dev.alloc(pairs * inter * 2), dev.alloc(pairs * hidden * 4), dev.alloc(t * hidden * 4)
+    wb = dev.put(wts)
+    vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
+    vdn = H.view_of(dev, dnb, fmt, experts * hidden, inter)
+    qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, b["stok"].ptr, b["off"].ptr, b["te"].ptr,
+                                           b["tr"].ptr, b["tc"].ptr, g["max_tiles"], pairs, gu_out.ptr, qwhip.F16, 0))
+    qwhip.check(lib.qwhip_swiglu_fwht(st, gu_out.ptr, qwhip.F16, act.ptr, pairs, inter, 1))
+    qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vdn), experts, act.ptr, qwhip.F16, 0, None, b["off"].ptr, b["te"].ptr,
+                                           b["tr"].ptr, b["tc"].ptr, g["max_tiles"], pairs, dn_out.ptr, qwhip.F32, 0))
+    qwhip.check(lib.qwhip_moe_combine(st, dn_out.ptr, qwhip.F32, b["inv"].ptr, wb.ptr, t, k, hidden, None, None, out.ptr, qwhip.F32))
+    dev.stream.sync()
+    got = out.download(np.float32, (t, hidden))
+    ref = qo.moe_forward_f64(x16, idx, wts, gu16, dn16, act_f16=True, rotate_act=True)
+    assert qo.normalized_error(got, ref) <= TOL
+
+
+@pytest.mark.parametrize("t", [1, 3, 8])
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+def test_moe_decode_chain_matches_oracle(dev, t, xdt):
+    """Decode / verify path: routed gate_up GEMV (+SwiGLU+FWHT) and routed down GEMV with weighted combine,
+    un-rotated activations in, fused rotation."""
+    fmt, experts, hidden, inter, k = "hq4_g32_m5", 16, 512, 192, 4
+    gu_blocks, gu16, dn_blocks, dn16 = _moe_banks(experts, hidden, inter, seed=21)
+    rng = np.random.default_rng(6)
+    x32 = rng.standard_normal((t, hidden)).astype(np.float32)
+    if xdt == "f16":
+        xh, code, xv = x32.astype(np.float16), qwhip.F16, x32.astype(np.float16).astype(np.float32)
+    else:
+        xh, code, xv = qo.f32_to_bf16_bits(x32), qwhip.BF16, qo.round_bf16(x32)
+    logits = rng.standard_normal((t, experts)).astype(np.float32)
+    idx, wts = _route(dev, logits, k)
+    idx[0, k - 1] = -1                                         # an empty route is skipped
+    shared = rng.standard_normal((t, hidden)).astype(np.float32)
+    gate = rng.random(t).astype(np.float32)
+    lib, st = dev.lib, dev.stream.handle
+    gub, dnb, xb, ib, wb = dev.put(gu_blocks), dev.put(dn_blocks), dev.put(xh), dev.put(idx), dev.put(wts)
+    sb, gb = dev.put(shared), dev.put(gate)
+    act, out = dev.alloc(t * k * inter * 2), dev.alloc(t * hidden * 4)
+    vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
+    vdn = H.view_of(dev, dnb, fmt, experts * hidden, inter)
+    qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(vgu), experts, xb.ptr, code, 0, ib.ptr, t, k, act.ptr))
+    qwhip.check(lib.qwhip_moe_down_decode(st, C.byref(vdn), experts, act.ptr, ib.ptr, wb.ptr, t, k, sb.ptr, gb.ptr, out.ptr, qwhip.F32))
+    dev.stream.sync()
+    got = out.download(np.float32, (t, hidden))
+    x_rot = qo.fwht32_ortho(xv).astype(np.float16)
+    ref = qo.moe_forward_f64(x_rot, idx, wts, gu16, dn16, act_f16=True, rotate_act=True) + gate[:, None].astype(np.float64) * shared
+    assert qo.normalized_error(got, ref) <= TOL
+    a = act.download(np.float16, (t, k, inter))
+    assert np.all(a[0, k - 1] == 0)
+
+
+def test_online_quantizer_writes_the_packers_bytes(dev):
+    """Device HQ4_G32_M5 quantizer vs the oracle's restatement of the packer, byte-identical
+    (Tests/QWFlashNextMetalTests/QUANT/FNMetalOnlineQuantTests.swift:243), bf16 and f32 sources, rotate on/off."""
+    w = H.make_weights(96, 1024, seed=4)
+    w[3, :32] = 0.0
+    w[5, 7] = 3.0
+    for src_kind in ("f32", "bf16"):
+        if src_kind == "bf16":
+            host, code, val = qo.f32_to_bf16_bits(w), qwhip.BF16, qo.round_bf16(w)
+        else:
+            host, code, val = w, qwhip.F32, w
+        for rotate in (1, 0):
+            sb, ob = dev.put(host), dev.alloc(96 * 32 * 20)
+            qwhip.check(dev.lib.qwhip_quantize_hq4_g32(dev.stream.handle, sb.ptr, code, 96, 1024, rotate, ob.ptr))
+            got = ob.download(np.uint8, (96, 32, 20))
+            assert np.array_equal(got, qo.quant_hq4_blocks(val, rotate=bool(rotate)))
+
+
+def test_swiglu_fwht_matches_oracle(dev):
+    rng = np.random.default_rng(2)
+    rows, inter = 9, 160
+    gu = (rng.standard_normal((rows, 2 * inter)) * 2).astype(np.float16)
+    gb, ab = dev.put(gu), dev.alloc(rows * inter * 2)
+    for rotate in (1, 0):
+        qwhip.check(dev.lib.qwhip_swiglu_fwht(dev.stream.handle, gb.ptr, qwhip.F16, ab.ptr, rows, inter, rotate))
+        got = ab.download(np.float16, (rows, inter)).astype(np.float32)
+        want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=bool(rotate)).astype(np.float32)
+        assert np.max(np.abs(got - want)) <= 2e-3 * max(1.0, float(np.max(np.abs(want))))

@@ -1,0 +1,228 @@
+"""Pins the oracle on what the mathematics fixes, independent of the golden vectors: closed forms,
+invariants, brute force on tiny inputs and scalar restatements of the reference's host readers.  Each
+check is chosen so a plausible mistake (wrong nibble order, wrong rounding mode, a dropped term, a
+transposed butterfly) fails it."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from oracle import qworacle as qo
+
+
+def test_fwht_is_the_dense_hadamard_and_self_inverse():
+    # Sylvester H32 built by Kronecker products; natural (Hadamard) order is what the (i, i+h) butterflies give
+    h = np.array([[1.0]])
+    for _ in range(5):
+        h = np.block([[h, h], [h, -h]])
+    x = np.random.default_rng(0).standard_normal((5, 64)).astype(np.float32)
+    want = (x.reshape(-1, 32).astype(np.float64) @ h.T / np.sqrt(32.0)).reshape(x.shape)
+    got = qo.fwht32_ortho(x)
+    assert np.max(np.abs(got - want)) < 1e-5
+    assert np.max(np.abs(qo.fwht32_ortho(got) - x)) < 1e-5
+    # unit vectors: column i of H/sqrt(32), exactly +-f32(1/sqrt(32))
+    e = np.eye(32, dtype=np.float32)
+    col = qo.fwht32_ortho(e)
+    assert np.all(np.abs(col) == qo.INV_SQRT32)
+    assert np.array_equal(np.sign(col), np.sign(h))
+    assert qo.INV_SQRT32.view(np.uint32) == 0x3E3504F3
+
+
+def _rn_f16(frac: Fraction) -> np.float16:
+    """Exact round-to-nearest-even of a rational to binary16 (brute force over the two neighbours)."""
+    f = float(frac)                       # doubles hold these values exactly (checked by the caller)
+    assert Fraction(f) == frac
+    lo = np.float16(f)
+    # np.float16(double) is correctly rounded; confirm against the neighbours with exact arithmetic
+    cands = [lo, np.nextafter(lo, np.float16(np.inf)), np.nextafter(lo, np.float16(-np.inf))]
+    cands = [c for c in cands if np.isfinite(c)]
+    best = min(cands, key=lambda c: (abs(Fraction(float(c)) - frac), int(c.view(np.uint16)) & 1))
+    return best
+
+
+def test_f16_weight_closed_form_brute_force():
+    """RN_f16((1024+q)*s + b) and RN_f16(code*s + b) against exact rational arithmetic."""
+    rng = np.random.default_rng(1)
+    scales = np.concatenate([rng.uniform(1e-4, 0.2, 40), [6e-8, 3.0e-5, 63.46875]]).astype(np.float16)
+    for s16 in scales:
+        b16 = np.float16(np.float32(-1032.0) * np.float32(s16))
+        blocks = np.zeros((1, 1, 20), dtype=np.uint8)
+        blocks[0, 0, 0:2] = np.array([s16]).view(np.uint8)
+        blocks[0, 0, 2:4] = np.array([b16]).view(np.uint8)
+        q = np.arange(32) % 16
+        blocks[0, 0, 4:] = qo.hq4_interleave(q[None, :]).view(np.uint8).reshape(16)
+        w16 = qo.weights_f16_exact(blocks, 4, 32, True)[0]
+        for i in range(16):
+            exact = (1024 + int(q[i])) * Fraction(float(s16)) + Fraction(float(b16))
+            assert w16[i] == _rn_f16(exact), (s16, i)
+        # block family: code*s + b with an unrelated bias
+        bias = np.float16(-7.5 * float(s16))
+        blk = np.zeros((1, 1, 36), dtype=np.uint8)
+        blk[0, 0, 0:2] = np.array([s16]).view(np.uint8)
+        blk[0, 0, 2:4] = np.array([bias]).view(np.uint8)
+        codes = (np.arange(32) * 37 + 11) % 256
+        blk[0, 0, 4:] = codes
+        w8 = qo.weights_f16_exact(blk, 8, 32, False)[0]
+        for i in range(32):
+            exact = int(codes[i]) * Fraction(float(s16)) + Fraction(float(bias))
+            assert w8[i] == _rn_f16(exact), (s16, i)
+
+
+def test_hq4_nibble_order_matches_the_scalar_reader():
+    """Element 8w+j sits at bit 4*(j>>1) + 16*(j&1) of word w (QWAQProducer.swift:85-87; reader shifts
+    0,16,4,20,8,24,12,28 in QWQuant+DequantMath.swift:82-89)."""
+    q = np.arange(32) % 16
+    words = qo.hq4_interleave(q[None, :])[0]
+    for w in range(4):
+        for j in range(8):
+            shift = 4 * (j >> 1) + 16 * (j & 1)
+            assert (int(words[w]) >> shift) & 0xF == q[8 * w + j]
+    blocks = np.zeros((1, 1, 20), dtype=np.uint8)
+    blocks[0, 0, 4:] = words.view(np.uint8)
+    assert np.array_equal(qo.hq4_codes(blocks)[0, 0], q)
+
+
+def test_hq4_quantizer_invariants():
+    rng = np.random.default_rng(2)
+    w = (rng.standard_normal((16, 256)) * 0.02).astype(np.float32)
+    w[0, :32] = 0.0                                       # scale 0 -> code 8 everywhere, bias -0
+    blocks = qo.quant_hq4_blocks(w, rotate=False)
+    s = np.ascontiguousarray(blocks[..., 0:2]).view(np.float16)[..., 0]
+    b = np.ascontiguousarray(blocks[..., 2:4]).view(np.float16)[..., 0]
+    assert np.array_equal(b, (np.float32(-1032.0) * s.astype(np.float32)).astype(np.float16))     # bias law
+    codes = qo.hq4_codes(blocks)
+    assert np.all(codes[0, 0] == 8) and s[0, 0] == 0
+    v = w.reshape(16, 8, 32)
+    deq = qo.dequant_hq4_rot(blocks).reshape(16, 8, 32)
+    sf = s.astype(np.float32)[..., None]
+    inner = (codes > 0) & (codes < 15)
+    assert np.all(np.abs(deq - v)[inner] <= (0.5 * sf * 1.01 + 1e-9).repeat(32, -1)[inner])          # brackets v within scale/2
+    for g in range(8):                                                                           # code monotone in v
+        order = np.argsort(v[3, g], kind="stable")
+        assert np.all(np.diff(codes[3, g][order].astype(int)) >= 0)
+    amax = np.abs(v).max(-1)
+    assert np.array_equal(s, np.minimum(amax / np.float32(7.5), np.float32(63.46875)).astype(np.float16))
+    # the scale clamp
+    big = np.full((1, 32), 1000.0, dtype=np.float32)
+    sb = np.ascontiguousarray(qo.quant_hq4_blocks(big, rotate=False)[..., 0:2]).view(np.float16)
+    assert float(sb[0, 0, 0]) == 63.46875
+
+
+def _read_bits_scalar(payload: bytes, bits: int, index: int) -> int:
+    """Scalar restatement of QWAQBlock.readBits (QWAQBlock.swift:115-126)."""
+    bit = index * bits
+    byte, off = bit >> 3, bit & 7
+    v = payload[byte] >> off
+    taken = 8 - off
+    if taken < bits:
+        v |= payload[byte + 1] << taken
+    return v & ((1 << bits) - 1)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
+@pytest.mark.parametrize("group", [32, 64, 128, 256])
+def test_bitstream_layout_and_size_law(bits, group):
+    assert qo.hq_block_bytes(bits, group) == 4 + group * bits // 8
+    rng = np.random.default_rng(bits * 1000 + group)
+    q = rng.integers(0, 1 << bits, size=(3, group))
+    payload = qo.pack_bitstream(q, bits)
+    assert payload.shape == (3, group * bits // 8)
+    for r in range(3):
+        raw = payload[r].tobytes()
+        assert [_read_bits_scalar(raw, bits, i) for i in range(group)] == q[r].tolist()
+    assert np.array_equal(qo.unpack_bitstream(payload, bits, group), q)
+
+
+def test_block_quantizer_invariants():
+    rng = np.random.default_rng(3)
+    w = (rng.standard_normal((8, 256)) * 0.02).astype(np.float32)
+    w[1, 64:128] = 0.5                                          # constant group: scale 0, codes 0, bias = value
+    for bits, group in [(4, 32), (4, 64), (8, 32)]:
+        blocks, eff = qo.quant_hq_blocks(w, bits=bits, group=group, rotate=False)
+        assert eff == group and blocks.shape == (8, 256 // group, 4 + group * bits // 8)
+        s, b = qo.hq_block_header(blocks)
+        v = w.reshape(8, 256 // group, group)
+        assert np.array_equal(b, v.min(-1).astype(np.float16).astype(np.float32))
+        qmax = (1 << bits) - 1
+        assert np.array_equal(s, ((v.max(-1) - v.min(-1)) / np.float32(qmax)).astype(np.float16).astype(np.float32))
+        codes = qo.hq_block_codes(blocks, bits, group)
+        const = (v.max(-1) == v.min(-1))
+        assert np.all(codes[const] == 0)
+        deq = qo.dequant_hq_blocks_rot(blocks, bits, group).reshape(v.shape)
+        inner = (codes > 0) & (codes < qmax)
+        tol = 0.5 * s[..., None] * 1.01 + 1e-9
+        assert np.all(np.abs(deq - v)[inner] <= np.broadcast_to(tol, v.shape)[inner])
+    # round-half-even, not half-up: (w - b)/s = 0.5 and 1.5 and 2.5 -> 0, 2, 2
+    g = np.zeros((1, 32), dtype=np.float32)
+    g[0, :4] = [0.0, 0.5, 1.5, 2.5]
+    g[0, 31] = 15.0                                            # min 0, max 15 -> scale 1, bias 0 (4-bit)
+    blk, _ = qo.quant_hq_blocks(g, bits=4, group=32, rotate=False)
+    assert qo.hq_block_codes(blk, 4, 32)[0, 0, :4].tolist() == [0, 0, 2, 2]
+    with pytest.raises(ValueError):
+        qo.resolve_group_size(48, 32)
+    assert qo.resolve_group_size(96, 64) == 32                  # gcd clamp (hq_blocks.py:106-114)
+
+
+def test_rotation_preserves_products():
+    """(x H)(W H)^T = x W^T: the whole point of rotating both sides."""
+    rng = np.random.default_rng(4)
+    w = rng.standard_normal((6, 128)).astype(np.float32)
+    x = rng.standard_normal((2, 128)).astype(np.float32)
+    a = x.astype(np.float64) @ w.astype(np.float64).T
+    b = qo.fwht32_ortho(x).astype(np.float64) @ qo.fwht32_ortho(w).astype(np.float64).T
+    assert np.max(np.abs(a - b)) < 1e-4
+
+
+def test_route_is_textbook_softmax_topk():
+    rng = np.random.default_rng(5)
+    logits = rng.standard_normal((20, 24)).astype(np.float32)
+    idx, wts = qo.moe_route(logits, 4, norm_topk=True)
+    p = np.exp(logits.astype(np.float64) - logits.max(1, keepdims=True))
+    p /= p.sum(1, keepdims=True)
+    want_idx = np.argsort(-p, axis=1, kind="stable")[:, :4]
+    assert np.array_equal(idx, want_idx)
+    sel = np.take_along_axis(p, want_idx, 1)
+    np.testing.assert_allclose(wts, sel / sel.sum(1, keepdims=True), rtol=1e-5)
+    np.testing.assert_allclose(wts.sum(1), 1.0, rtol=1e-6)
+    idx2, w2 = qo.moe_route(np.zeros((1, 8), np.float32), 3, norm_topk=False)
+    assert idx2[0].tolist() == [0, 1, 2] and np.allclose(w2, 1 / 8)
+
+
+def test_group_pairs_brute_force_and_tile_closed_forms():
+    rng = np.random.default_rng(6)
+    for t, e, k in [(1, 4, 2), (9, 8, 3), (200, 16, 4), (70, 4, 1)]:
+        ids = np.stack([rng.choice(e, size=k, replace=False) for _ in range(t)]).astype(np.int32)
+        ids[rng.random(ids.shape) < 0.1] = -1
+        for compact in (True, False):
+            g = qo.moe_group_pairs(ids, e, k, compact_tail=compact)
+            flat = ids.ravel()
+            valid = np.flatnonzero(flat >= 0)
+            assert g["expertOff"][0] == 0 and g["expertOff"][e] == valid.size
+            assert sorted(g["sortedPairIdx"].tolist()) == valid.tolist()
+            assert np.array_equal(g["invPerm"][g["sortedPairIdx"]], np.arange(valid.size))
+            assert np.array_equal(g["sortedTok"], g["sortedPairIdx"] // k)
+            covered = np.zeros(valid.size, dtype=int)
+            for te, tr in zip(g["tileE"], g["tileR"]):
+                code, rb = tr >> 24, tr & 0xFFFFFF
+                bm = {1: 16, 2: 32, 3: 64}[code]
+                lo = g["expertOff"][te] + rb * bm
+                hi = min(lo + bm, g["expertOff"][te + 1])
+                assert lo < hi
+                covered[lo:hi] += 1
+            assert np.all(covered == 1)                         # tiles partition the slots exactly
+            assert g["tileCount"] <= qo.moe_max_tiles(e, ids.size) or ids.size == 0
+    # closed forms (qw_moe_tile.metalh:7-16, QWGemmMoE.swift:24-26)
+    assert [qo.moe_tile_block(c) for c in (1, 16, 17, 32, 33, 64, 1000)] == [16, 16, 32, 32, 64, 64, 64]
+    assert qo.moe_pack_tile_r(5, 16) == (1 << 24) | 5 and qo.moe_pack_tile_r(2, 64) == (3 << 24) | 2
+    assert qo.moe_max_tiles(128, 16384) == 128 + 256 and qo.moe_max_tiles(128, 3) == 3
+    # 70 rows of one expert with compact tail: one 64-row tile + one 16-row tail at row 64 = block index 4
+    g = qo.moe_group_pairs(np.zeros(70, np.int32), 4, 1, compact_tail=True)
+    assert g["tileR"].tolist() == [qo.moe_pack_tile_r(0, 64), qo.moe_pack_tile_r(4, 16)]
+
+
+def test_swiglu_closed_form():
+    g = np.array([0.0, 1.0, -2.0, 30.0, -30.0], dtype=np.float32)
+    u = np.array([3.0, 2.0, 0.5, 1.0, 1.0], dtype=np.float32)
+    want = g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u
+    np.testing.assert_allclose(qo.swiglu(g, u), want, rtol=1e-6, atol=1e-12)
+    assert qo.swiglu_fwht_f16(np.ones((1, 48), np.float32), np.ones((1, 48), np.float32)).shape == (1, 48)  # I % 32 != 0: not rotated
