@@ -42,6 +42,33 @@ extern "C" qwhip_status qwhip_fwht32(qwhip_stream_t s, const void* src, uint32_t
     return QWHIP_OK;
 }
 
+// ---- any -> f16 convert, 8 elements per lane (n % 8 == 0, 16-byte aligned) ----------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void qw_convert_f16_kernel(const void* __restrict__ src, h1_t* __restrict__ dst, uint64_t n8) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    float v[8];
+    qw_load8_f32<DT>(src, i * 8, v);
+    h8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (h1_t)v[e];
+    *(h8_t*)(dst + i * 8) = o;
+}
+
+qwhip_status qw_convert_to_f16(qwhip_stream_t s, const void* src, uint32_t src_dtype, void* dst_f16, uint64_t n) {
+    if (n % 8 != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "convert: n=%llu is not a multiple of 8", (unsigned long long)n);
+    const uint64_t n8 = n / 8;
+    const dim3 grid((unsigned)((n8 + 255) / 256)), block(256);
+    switch (src_dtype) {
+        case QWHIP_F16: hipLaunchKernelGGL(qw_convert_f16_kernel<QWHIP_F16>, grid, block, 0, s->stream, src, (h1_t*)dst_f16, n8); break;
+        case QWHIP_BF16: hipLaunchKernelGGL(qw_convert_f16_kernel<QWHIP_BF16>, grid, block, 0, s->stream, src, (h1_t*)dst_f16, n8); break;
+        case QWHIP_F32: hipLaunchKernelGGL(qw_convert_f16_kernel<QWHIP_F32>, grid, block, 0, s->stream, src, (h1_t*)dst_f16, n8); break;
+        default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "convert: unsupported source dtype %u", src_dtype);
+    }
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
 // ---- f32 -> f16 cast ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void qw_cast_f32_f16_kernel(const float* __restrict__ src, h1_t* __restrict__ dst,
                                                                uint64_t n) {

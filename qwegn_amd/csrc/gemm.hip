@@ -285,6 +285,210 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm_kernel(const qw_gemm_pa
 }
 
 // ------------------------------------------------------------------------------------------------
+// Pipelined kernel (f16 activations): the activation tile goes global -> LDS by the DMA path
+// (global_load_lds_dwordx4: no VGPRs, no VALU, no ds_write), LDS is double-buffered with an XOR
+// swizzle instead of padding (16-byte slot = k-chunk ^ ((row >> 1) & 7): the 16 rows one MFMA operand
+// read touches land on 16 distinct slots of a 256-byte bank row), and each K-step needs one barrier:
+//   iteration k:  DMA A(k+1) -> stage (k+1)&1 | global loads B(k+2) -> registers
+//                 dequant B(k+1) registers -> stage (k+1)&1
+//                 MFMAs on stage k&1
+//                 wait DMA, barrier
+// ------------------------------------------------------------------------------------------------
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED>
+__global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_params p) {
+    constexpr int NT = WVM * WVN * 64;
+    constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 64;
+    constexpr int A_PER = BM * 8 / NT;  // DMA instructions per thread and K-step
+    static_assert((BM * 8) % NT == 0, "activation tile must split evenly over the workgroup");
+    constexpr int B_ITEMS = BN * 2;
+    constexpr int B_PER = (B_ITEMS + NT - 1) / NT;
+    constexpr int B_VMEM = B_PER * (FMT == QG_FMT_B8 ? 3 : 2);  // VMEM loads per thread and K-step for the weights
+    constexpr uint32_t A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds2[];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t wm = wave / WVN, wn = wave % WVN;
+
+    uint32_t m0, n0, rows_valid;
+    const uint8_t* bank = p.bank;
+    if constexpr (GROUPED) {
+        const uint32_t t = blockIdx.y;
+        if ((int32_t)t >= p.tile_count[0]) return;
+        const uint32_t e = (uint32_t)p.tile_e[t];
+        const uint32_t packed = (uint32_t)p.tile_r[t];
+        const uint32_t code = packed >> 24;
+        const uint32_t bm = code == 1u ? 16u : (code == 2u ? 32u : 64u);
+        const uint32_t start = (uint32_t)p.expert_off[e] + (packed & 0xFFFFFFu) * bm;
+        const uint32_t end = (uint32_t)p.expert_off[e + 1];
+        m0 = start;
+        rows_valid = min((uint32_t)BM, min(bm, end - start));
+        n0 = blockIdx.x * BN;
+        bank += (uint64_t)e * p.rows_per_expert * p.row_bytes;
+    } else {
+        const uint32_t total = p.tiles_m * p.tiles_n;
+        const uint32_t per_xcd = (total + 7u) / 8u;
+        const uint32_t label = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (label >= total) return;
+        constexpr uint32_t G = 4;
+        const uint32_t band = label / (G * p.tiles_n);
+        const uint32_t band_rows = min(G, p.tiles_m - band * G);
+        const uint32_t in_band = label - band * G * p.tiles_n;
+        const uint32_t tm = band * G + in_band % band_rows;
+        const uint32_t tn = in_band / band_rows;
+        m0 = tm * BM;
+        n0 = tn * BN;
+        rows_valid = min((uint32_t)BM, p.M - m0);
+    }
+
+    // ---- DMA sources: chunk c = i*NT + tid -> LDS row c >> 3, slot c & 7 (linear in c, as the DMA writes it) ----
+    const uint8_t* a_src[A_PER];
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+        const uint32_t c = tid + i * NT;
+        uint32_t row = c >> 3;
+        const uint32_t kc = (c & 7u) ^ ((row >> 1) & 7u);
+        if (row >= rows_valid) row = rows_valid - 1;  // tail rows re-read a valid row; their outputs are never stored
+        uint64_t src_row = m0 + row;
+        if constexpr (GROUPED) {
+            if (p.gather) src_row = (uint32_t)p.gather[m0 + row];
+        }
+        a_src[i] = (const uint8_t*)p.x + (src_row * p.ldx + kc * 8u) * 2u;
+    }
+    const uint8_t* b_src[B_PER];
+    uint32_t b_dst[B_PER];  // LDS byte offset of the row inside the B tile, and the slice's slot base
+    uint32_t b_sw[B_PER];
+#pragma unroll
+    for (int i = 0; i < B_PER; ++i) {
+        // every thread owns B_PER items; the surplus ones repeat the last item (same bytes to the same LDS slot), which
+        // keeps the K loop free of branches so the dequant can be scheduled into the MFMA shadow
+        const uint32_t it = min(tid + i * NT, (uint32_t)B_ITEMS - 1u);
+        const uint32_t nl = it >> 1;
+        uint32_t n = n0 + nl;
+        if (n >= p.N) n = p.N - 1;
+        b_src[i] = bank + (uint64_t)n * p.row_bytes;
+        b_dst[i] = nl * 128u;
+        b_sw[i] = ((nl >> 1) & 7u) | ((it & 1u) << 8);  // swizzle key | slice bit
+    }
+
+    f16_t acc[WM][WN];
+#pragma unroll
+    for (int a = 0; a < WM; ++a)
+#pragma unroll
+        for (int b = 0; b < WN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    const uint32_t nk = p.K / BK;
+    qg_slice<FMT> b_reg[B_PER];
+
+    auto dma_a = [&](uint32_t kt, uint32_t stage) {
+#pragma unroll
+        for (int i = 0; i < A_PER; ++i) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[i] + (uint64_t)kt * 128u),
+                                             (__attribute__((address_space(3))) void*)(lds2 + stage * STAGE + (i * NT + wave * 64) * 16),
+                                             16, 0, 0);
+        }
+    };
+    auto load_b = [&](uint32_t kt) {
+#pragma unroll
+        for (int i = 0; i < B_PER; ++i) qg_load_slice<FMT>(b_src[i], kt * 2u + (b_sw[i] >> 8), p.gshift, p.bb, b_reg[i]);
+    };
+    auto store_b = [&](uint32_t stage) {
+#pragma unroll
+        for (int i = 0; i < B_PER; ++i) {
+            const h2_t s2 = qw_splat_lo(b_reg[i].hdr), b2 = qw_splat_hi(b_reg[i].hdr);
+            uint8_t* row = lds2 + stage * STAGE + A_BYTES + b_dst[i];
+            const uint32_t sw = b_sw[i] & 7u, sl4 = (b_sw[i] >> 8) * 4u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *(h8_t*)(row + (((sl4 + j) ^ sw) * 16u)) = qg_dequant_chunk<FMT>(b_reg[i], j, s2, b2, magic);
+        }
+    };
+
+    // ---- prologue: tile 0 in stage 0, weights of tile 1 in registers ----
+    dma_a(0, 0);
+    load_b(0);
+    store_b(0);
+    load_b(nk > 1 ? 1u : 0u);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(B_VMEM) : "memory");
+    __syncthreads();
+
+    const uint32_t fr_row = lane & 31u, fr_sw = (fr_row >> 1) & 7u, k_half = lane >> 5;
+    uint32_t a_off[WM], b_off[WN];
+#pragma unroll
+    for (int a = 0; a < WM; ++a) a_off[a] = ((wm * WM + a) * 32 + fr_row) * 128u;
+#pragma unroll
+    for (int b = 0; b < WN; ++b) b_off[b] = A_BYTES + ((wn * WN + b) * 32 + fr_row) * 128u;
+
+    auto mfma_step = [&](const uint8_t* st_base) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint32_t slot = ((ks * 2u + k_half) ^ fr_sw) * 16u;
+            h8_t af[WM], bf[WN];
+#pragma unroll
+            for (int a = 0; a < WM; ++a) af[a] = *(const h8_t*)(st_base + a_off[a] + slot);
+#pragma unroll
+            for (int b = 0; b < WN; ++b) bf[b] = *(const h8_t*)(st_base + b_off[b] + slot);
+#pragma unroll
+            for (int a = 0; a < WM; ++a)
+#pragma unroll
+                for (int b = 0; b < WN; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
+        }
+    };
+
+    // steady state: branch-free body so the scheduler can interleave the dequant VALU and the LDS traffic of
+    // tile kt+1 with the MFMAs of tile kt
+    for (uint32_t kt = 0; kt + 1 < nk; ++kt) {
+        const uint32_t cur = kt & 1u, nxt = cur ^ 1u;
+        dma_a(kt + 1, nxt);
+        mfma_step(lds2 + cur * STAGE);
+        store_b(nxt);                                  // registers hold the weights of tile kt + 1
+        load_b(min(kt + 2, nk - 1));                   // (the last one re-reads tile nk-1; never used)
+        // Issue order of the block above.  LDS reads (stage cur) stay ahead of LDS writes (stage nxt) - the compiler
+        // cannot prove the two stages disjoint - so: DMA, the first operand reads, then one MFMA at a time with the
+        // dequant VALU in its shadow, operand reads while they last, then the writes, and the weight loads last.
+        {
+            constexpr int NMFMA = WM * WN * 4, NREAD = (WM + WN) * 4, NWRITE = B_PER * 4;
+            constexpr int VALU_PER = 4;
+            __builtin_amdgcn_sched_group_barrier(0x010, A_PER, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, WM + WN, 0);
+#pragma unroll
+            for (int i = 0; i < NMFMA; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER, 0);
+                if (i < NREAD - (WM + WN)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                else if (i - (NREAD - (WM + WN)) < NWRITE) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x010, B_VMEM, 0);
+        }
+        // the DMA of tile kt+1 is older than the register loads just issued: wait for it alone
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(B_VMEM) : "memory");
+        __syncthreads();
+    }
+    mfma_step(lds2 + ((nk - 1) & 1u) * STAGE);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+#pragma unroll
+    for (int a = 0; a < WM; ++a) {
+#pragma unroll
+        for (int b = 0; b < WN; ++b) {
+            const uint32_t n = n0 + (wn * WN + b) * 32 + (lane & 31u);
+            if (n < p.N) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -310,58 +514,74 @@ hipError_t launch_cfg(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-// tile configurations
-enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_64x256 = 3, CFG_256x128 = 4 };
-
-template <int FMT, int XDT, int YDT>
-hipError_t launch_dense(hipStream_t st, qw_gemm_params& p, int cfg) {
-    uint32_t bm, bn;
-    switch (cfg) {
-        case CFG_256x320: bm = 256; bn = 320; break;
-        case CFG_256x256: bm = 256; bn = 256; break;
-        case CFG_256x128: bm = 256; bn = 128; break;
-        default: bm = 128; bn = 128; break;
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED>
+hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
+    constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
+    constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
+    auto kern = qw_gemm2_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED>;
+    static bool attr_done = false;  // per instantiation
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_done = true;
     }
-    p.tiles_m = qwhip_cdiv(p.M, bm);
-    p.tiles_n = qwhip_cdiv(p.N, bn);
+    hipLaunchKernelGGL(kern, grid, dim3(WVM * WVN * 64), lds, st, p);
+    return hipGetLastError();
+}
+
+// tile shapes of the pipelined kernel
+enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_256x128 = 3, CFG_COUNT = 4 };
+static const uint32_t kCfgBM[CFG_COUNT] = {256, 256, 128, 256};
+static const uint32_t kCfgBN[CFG_COUNT] = {320, 256, 128, 128};
+
+template <int FMT, int YDT>
+hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
+    p.tiles_m = qwhip_cdiv(p.M, kCfgBM[cfg]);
+    p.tiles_n = qwhip_cdiv(p.N, kCfgBN[cfg]);
     const uint32_t total = p.tiles_m * p.tiles_n;
     const dim3 grid(((total + 7u) / 8u) * 8u);
     switch (cfg) {
-        case CFG_256x320: return launch_cfg<4, 5, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
-        case CFG_256x256: return launch_cfg<4, 4, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
-        case CFG_256x128: return launch_cfg<4, 2, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
-        default: return launch_cfg<2, 2, 2, 2, FMT, XDT, YDT, false>(st, p, grid);
+        case CFG_256x320: return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
+        case CFG_256x256: return launch_cfg2<2, 4, 4, 2, FMT, YDT, false>(st, p, grid);
+        case CFG_256x128: return launch_cfg2<2, 2, 4, 2, FMT, YDT, false>(st, p, grid);
+        default: return launch_cfg2<2, 2, 2, 2, FMT, YDT, false>(st, p, grid);
     }
 }
 
-template <int FMT, int XDT>
-hipError_t launch_dense_y(hipStream_t st, qw_gemm_params& p, int cfg, uint32_t ydt) {
-    if (ydt == QWHIP_F16) return launch_dense<FMT, XDT, QWHIP_F16>(st, p, cfg);
-    if (ydt == QWHIP_BF16) return launch_dense<FMT, XDT, QWHIP_BF16>(st, p, cfg);
-    return launch_dense<FMT, XDT, QWHIP_F32>(st, p, cfg);
-}
-
 template <int FMT>
-hipError_t launch_dense_xy(hipStream_t st, qw_gemm_params& p, int cfg, uint32_t xdt, uint32_t ydt) {
-    if (xdt == QWHIP_F16) return launch_dense_y<FMT, QWHIP_F16>(st, p, cfg, ydt);
-    return launch_dense_y<FMT, QWHIP_BF16>(st, p, cfg, ydt);
+hipError_t launch_dense2_y(hipStream_t st, qw_gemm_params& p, int cfg, uint32_t ydt) {
+    if (ydt == QWHIP_F16) return launch_dense2<FMT, QWHIP_F16>(st, p, cfg);
+    if (ydt == QWHIP_BF16) return launch_dense2<FMT, QWHIP_BF16>(st, p, cfg);
+    return launch_dense2<FMT, QWHIP_F32>(st, p, cfg);
 }
 
-// waste-aware choice among the tile shapes: time ~ rounds of tiles over 256 CUs x per-tile cost
+// fallback (bf16 activations converted inside the kernel, no workspace): 128 x 128 tiles only
+template <int FMT, int XDT>
+hipError_t launch_dense1_y(hipStream_t st, qw_gemm_params& p, uint32_t ydt) {
+    p.tiles_m = qwhip_cdiv(p.M, 128u);
+    p.tiles_n = qwhip_cdiv(p.N, 128u);
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const dim3 grid(((total + 7u) / 8u) * 8u);
+    if (ydt == QWHIP_F16) return launch_cfg<2, 2, 2, 2, FMT, XDT, QWHIP_F16, false>(st, p, grid);
+    if (ydt == QWHIP_BF16) return launch_cfg<2, 2, 2, 2, FMT, XDT, QWHIP_BF16, false>(st, p, grid);
+    return launch_cfg<2, 2, 2, 2, FMT, XDT, QWHIP_F32, false>(st, p, grid);
+}
+
+// waste-aware choice among the tile shapes: time ~ rounds of tiles over the CUs x per-tile cost / shape efficiency
 int choose_cfg(uint32_t M, uint32_t N) {
-    struct cand { int cfg; uint32_t bm, bn; double eff; };
-    // eff: relative MFMA efficiency of the shape (bigger wave tiles feed the matrix cores with fewer LDS reads)
-    const cand cands[] = {{CFG_256x320, 256, 320, 1.00}, {CFG_256x256, 256, 256, 0.97}, {CFG_256x128, 256, 128, 0.85},
-                          {CFG_128x128, 128, 128, 0.70}};
+    // relative matrix-core efficiency of each shape (measured on M = 4096, N = K = 5120) and workgroups resident per CU
+    const double eff[CFG_COUNT] = {1.00, 0.95, 0.70, 0.85};
+    const double resident[CFG_COUNT] = {1, 1, 2, 1};
     double best = 1e300;
     int best_cfg = CFG_128x128;
-    for (const cand& c : cands) {
-        const double tiles = (double)qwhip_cdiv(M, c.bm) * qwhip_cdiv(N, c.bn);
-        const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
-        const double cost = rounds * c.bm * c.bn / c.eff;
+    for (int c = 0; c < CFG_COUNT; ++c) {
+        const double tiles = (double)qwhip_cdiv(M, kCfgBM[c]) * qwhip_cdiv(N, kCfgBN[c]);
+        const double slots = 256.0 * resident[c];
+        const double rounds = (double)(uint64_t)((tiles + slots - 1.0) / slots);
+        const double cost = rounds * resident[c] * kCfgBM[c] * kCfgBN[c] / eff[c];
         if (cost < best) {
             best = cost;
-            best_cfg = c.cfg;
+            best_cfg = c;
         }
     }
     return best_cfg;
@@ -389,7 +609,7 @@ qwhip_status gemm_checks(qwhip_stream_t s, const qwhip_weight_view* w, const voi
 
 }  // namespace
 
-// flags bits 8..11: tile shape override for tuning and tests (0 = automatic, 1 + CFG_*).
+// flags bits 8..11: tile shape override for tuning and tests (0 = automatic, 1 + CFG_*; 15 = the unpipelined kernel).
 extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                    uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags, void* workspace,
                                    uint64_t workspace_bytes) {
@@ -404,17 +624,24 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions ldx=%u ldy=%u for k=%u n=%u", ldx, ldy, w->k, w->n);
 
     const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
+    const uint64_t ws_need = (uint64_t)m * w->k * 2u;
+    const bool ws_ok = workspace && workspace_bytes >= ws_need && ldx == w->k && ((uintptr_t)workspace & 15u) == 0;
     const void* xin = x;
     uint32_t xdt = x_dtype;
     if (rotate) {
         // rotated f16 copy of the activations in the caller's workspace, then the GEMM reads that
-        const uint64_t need = (uint64_t)m * w->k * 2u;
-        if (!workspace || workspace_bytes < need)
+        if (!workspace || workspace_bytes < ws_need)
             return qwhip_fail(QWHIP_E_BASIS,
                               "activations are not in the rotated basis and the workspace holds %llu bytes, %llu needed",
-                              (unsigned long long)workspace_bytes, (unsigned long long)need);
-        if (ldx != w->k) return qwhip_fail(QWHIP_E_BAD_SHAPE, "rotation pre-pass needs tightly packed activations");
+                              (unsigned long long)workspace_bytes, (unsigned long long)ws_need);
+        if (!ws_ok) return qwhip_fail(QWHIP_E_BAD_SHAPE, "rotation pre-pass needs tightly packed activations and a 16-byte aligned workspace");
         st = qwhip_fwht32(s, x, x_dtype, workspace, (uint64_t)m * w->k);
+        if (st != QWHIP_OK) return st;
+        xin = workspace;
+        xdt = QWHIP_F16;
+    } else if (x_dtype == QWHIP_BF16 && ws_ok) {
+        // one bf16 -> f16 pass instead of a conversion in every tile of the GEMM
+        st = qw_convert_to_f16(s, x, x_dtype, workspace, (uint64_t)m * w->k);
         if (st != QWHIP_OK) return st;
         xin = workspace;
         xdt = QWHIP_F16;
@@ -433,11 +660,23 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     p.bb = qwhip_view_block_bytes(w);
     p.row_bytes = qwhip_view_row_bytes(w);
     const uint32_t ov = (flags >> 8) & 0xFu;
-    const int cfg = ov ? (int)ov - 1 : choose_cfg(m, w->n);
     hipError_t e;
-    if (fmt == QG_FMT_M5) e = launch_dense_xy<QG_FMT_M5>(s->stream, p, cfg, xdt, y_dtype);
-    else if (fmt == QG_FMT_B4) e = launch_dense_xy<QG_FMT_B4>(s->stream, p, cfg, xdt, y_dtype);
-    else e = launch_dense_xy<QG_FMT_B8>(s->stream, p, cfg, xdt, y_dtype);
+    if (xdt != QWHIP_F16 || ov == 15u) {
+        if (xdt == QWHIP_F16) {
+            if (fmt == QG_FMT_M5) e = launch_dense1_y<QG_FMT_M5, QWHIP_F16>(s->stream, p, y_dtype);
+            else if (fmt == QG_FMT_B4) e = launch_dense1_y<QG_FMT_B4, QWHIP_F16>(s->stream, p, y_dtype);
+            else e = launch_dense1_y<QG_FMT_B8, QWHIP_F16>(s->stream, p, y_dtype);
+        } else {
+            if (fmt == QG_FMT_M5) e = launch_dense1_y<QG_FMT_M5, QWHIP_BF16>(s->stream, p, y_dtype);
+            else if (fmt == QG_FMT_B4) e = launch_dense1_y<QG_FMT_B4, QWHIP_BF16>(s->stream, p, y_dtype);
+            else e = launch_dense1_y<QG_FMT_B8, QWHIP_BF16>(s->stream, p, y_dtype);
+        }
+    } else {
+        const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : choose_cfg(m, w->n);
+        if (fmt == QG_FMT_M5) e = launch_dense2_y<QG_FMT_M5>(s->stream, p, cfg, y_dtype);
+        else if (fmt == QG_FMT_B4) e = launch_dense2_y<QG_FMT_B4>(s->stream, p, cfg, y_dtype);
+        else e = launch_dense2_y<QG_FMT_B8>(s->stream, p, cfg, y_dtype);
+    }
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
 }
@@ -452,7 +691,11 @@ hipError_t launch_grouped_y(hipStream_t st, const qw_gemm_params& p, dim3 grid, 
 }
 template <int FMT>
 hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid, uint32_t xdt, uint32_t ydt) {
-    if (xdt == QWHIP_F16) return launch_grouped_y<FMT, QWHIP_F16>(st, p, grid, ydt);
+    if (xdt == QWHIP_F16) {  // pipelined kernel, 64 x 256 tiles
+        if (ydt == QWHIP_F16) return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F16, true>(st, p, grid);
+        if (ydt == QWHIP_BF16) return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_BF16, true>(st, p, grid);
+        return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F32, true>(st, p, grid);
+    }
     return launch_grouped_y<FMT, QWHIP_BF16>(st, p, grid, ydt);
 }
 }  // namespace

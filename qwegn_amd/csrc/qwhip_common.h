@@ -31,6 +31,9 @@ qwhip_status qwhip_hip_check(hipError_t e, const char* what);
         if ((p) == nullptr) return qwhip_fail(QWHIP_E_NULL, "%s is NULL", #p); \
     } while (0)
 
+// elementwise.hip: src (f16 | bf16 | f32) -> f16, no rotation (internal helper of the GEMM pre-pass)
+qwhip_status qw_convert_to_f16(qwhip_stream_t s, const void* src, uint32_t src_dtype, void* dst_f16, uint64_t n);
+
 static inline uint32_t qwhip_cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
 // Block bytes of a validated view.
@@ -133,9 +136,9 @@ __device__ __forceinline__ uint32_t qw_vgpr_const(uint32_t c) {
     return v;
 }
 __device__ __forceinline__ uint32_t qw_and_or(uint32_t a, uint32_t mask_s, uint32_t magic_v) {
-    uint32_t d;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask_s), "v"(magic_v));
-    return d;
+    // plain C on purpose: with the magic in a VGPR the compiler selects v_and_or_b32 itself, and unlike an
+    // inline-asm statement the result stays visible to the instruction scheduler as an ordinary VALU op
+    return (a & mask_s) | magic_v;
 }
 
 // 8 HQ4_G32_M5 weights of one u32 word as four half2 (elements 0..7 in order): the nibble of element

@@ -58,7 +58,7 @@ def run_gemm(dev, fmt, m, n, k, *, xdtype="bf16", ydtype="bf16", prerot=True, cf
     return st, out, ref
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 5])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 15])
 def test_gemm_hq4_tile_shapes_f32_out(dev, cfg):
     st, out, ref = run_gemm(dev, "hq4_g32_m5", 512, 640, 1024, ydtype="f32", cfg=cfg)
     assert st == qwhip.OK
