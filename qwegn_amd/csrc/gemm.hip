@@ -38,7 +38,16 @@ struct qw_gemm_params {
     const int32_t* tile_r;
     const int32_t* tile_count;
     uint32_t rows_per_expert;
+#ifdef QW_GEMM_TIMING
+    unsigned long long* tlog;  // probe builds only: per-phase cycle stamps of workgroup 0, wave 0
+#endif
 };
+
+#ifdef QW_GEMM_TIMING
+#define QW_TSTAMP(slot) do { if (blockIdx.x == 8 && threadIdx.x == 0 && kt < 64) p.tlog[kt * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define QW_TSTAMP(slot) do { } while (0)
+#endif
 
 struct __attribute__((packed, aligned(4))) qg_words4 { uint32_t q[4]; };
 struct __attribute__((packed, aligned(4))) qg_words8 { uint32_t q[8]; };
@@ -408,12 +417,11 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
         }
     };
 
-    // ---- prologue: tile 0 in stage 0, weights of tile 1 in registers ----
+    // ---- prologue: tile 0 in stage 0 ----
     dma_a(0, 0);
     load_b(0);
     store_b(0);
-    load_b(nk > 1 ? 1u : 0u);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(B_VMEM) : "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     const uint32_t fr_row = lane & 31u, fr_sw = (fr_row >> 1) & 7u, k_half = lane >> 5;
@@ -440,34 +448,28 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
         }
     };
 
-    // steady state: branch-free body so the scheduler can interleave the dequant VALU and the LDS traffic of
-    // tile kt+1 with the MFMAs of tile kt
+    // steady state, branch-free: the DMA of the next activation tile and the loads of the next weight slices are
+    // issued first, the MFMAs of the current tile hide their latency, then the weights are dequantized into the
+    // other stage.  No loaded value is carried across the back edge (a loop-carried destination register makes the
+    // compiler wait on the load right where it is issued).
     for (uint32_t kt = 0; kt + 1 < nk; ++kt) {
         const uint32_t cur = kt & 1u, nxt = cur ^ 1u;
+        QW_TSTAMP(0);
+#ifndef QW_PROBE_SKIP_ADMA
         dma_a(kt + 1, nxt);
+#endif
+#ifndef QW_PROBE_SKIP_BLOAD
+        load_b(kt + 1);
+#endif
+        __builtin_amdgcn_sched_barrier(0);             // keep the loads at the top: their latency hides behind the MFMAs
         mfma_step(lds2 + cur * STAGE);
-        store_b(nxt);                                  // registers hold the weights of tile kt + 1
-        load_b(min(kt + 2, nk - 1));                   // (the last one re-reads tile nk-1; never used)
-        // Issue order of the block above.  LDS reads (stage cur) stay ahead of LDS writes (stage nxt) - the compiler
-        // cannot prove the two stages disjoint - so: DMA, the first operand reads, then one MFMA at a time with the
-        // dequant VALU in its shadow, operand reads while they last, then the writes, and the weight loads last.
-        {
-            constexpr int NMFMA = WM * WN * 4, NREAD = (WM + WN) * 4, NWRITE = B_PER * 4;
-            constexpr int VALU_PER = 4;
-            __builtin_amdgcn_sched_group_barrier(0x010, A_PER, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, WM + WN, 0);
-#pragma unroll
-            for (int i = 0; i < NMFMA; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER, 0);
-                if (i < NREAD - (WM + WN)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                else if (i - (NREAD - (WM + WN)) < NWRITE) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x010, B_VMEM, 0);
-        }
-        // the DMA of tile kt+1 is older than the register loads just issued: wait for it alone
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(B_VMEM) : "memory");
+        QW_TSTAMP(1);
+        store_b(nxt);
+        QW_TSTAMP(2);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        QW_TSTAMP(3);
         __syncthreads();
+        QW_TSTAMP(4);
     }
     mfma_step(lds2 + ((nk - 1) & 1u) * STAGE);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -570,7 +572,7 @@ hipError_t launch_dense1_y(hipStream_t st, qw_gemm_params& p, uint32_t ydt) {
 // waste-aware choice among the tile shapes: time ~ rounds of tiles over the CUs x per-tile cost / shape efficiency
 int choose_cfg(uint32_t M, uint32_t N) {
     // relative matrix-core efficiency of each shape (measured on M = 4096, N = K = 5120) and workgroups resident per CU
-    const double eff[CFG_COUNT] = {1.00, 0.95, 0.70, 0.85};
+    const double eff[CFG_COUNT] = {1.00, 0.82, 0.78, 0.75};
     const double resident[CFG_COUNT] = {1, 1, 2, 1};
     double best = 1e300;
     int best_cfg = CFG_128x128;
