@@ -54,5 +54,21 @@ def build_lib(jobs: int = 8, verbose: bool = False) -> pathlib.Path:
     return LIB_PATH
 
 
+HOST_TESTS = PKG / "host" / "host_tests"
+
+
+def build_host_tests(verbose: bool = False) -> pathlib.Path:
+    """Compiles the C++ host operator layer's test program (plain host C++ through hipcc's clang) against libqwhip.so."""
+    cmd = [_hipcc(), "-x", "c++", "-std=c++17", "-O2", str(PKG / "host" / "host_tests.cpp"), "-x", "none", "-o", str(HOST_TESTS),
+           "-L", str(LIB_DIR), "-lqwhip", "-Wl,-rpath,$ORIGIN/../lib"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"host_tests build failed:\n{res.stderr[-6000:]}")
+    if verbose:
+        print(f"built {HOST_TESTS}")
+    return HOST_TESTS
+
+
 if __name__ == "__main__":
     build_lib(verbose=True)
+    build_host_tests(verbose=True)

@@ -1,0 +1,329 @@
+// Tests of the host operator layer (qwhost.hpp).  `--cpu`: plan table, failable views, error mapping, no device.
+// `--gpu`: the operators run on the device and are checked against host formulas restated from the reference's own
+// self-contained tests (splitmix64 HQ4 GEMV: Tests/QWGEMMTests/QWHQ4GEMVTests.swift:16-50,108-133; closed-form MoE:
+// Tests/QWGEMMTests/QWMoEReuseTests.swift:18-127).  Exit code 0 = all passed.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "qwhost.hpp"
+
+using namespace qw;
+
+static int g_failed = 0, g_checks = 0;
+#define CHECK(cond)                                                                  \
+    do {                                                                             \
+        ++g_checks;                                                                  \
+        if (!(cond)) {                                                               \
+            ++g_failed;                                                              \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);            \
+        }                                                                            \
+    } while (0)
+#define CHECK_THROWS(expr, ErrT, kindv)                                              \
+    do {                                                                             \
+        ++g_checks;                                                                  \
+        bool ok_ = false;                                                            \
+        try { expr; } catch (const ErrT& e_) { ok_ = e_.kind == kindv; } catch (...) {} \
+        if (!ok_) { ++g_failed; std::printf("FAILED %s:%d: %s did not throw %s\n", __FILE__, __LINE__, #expr, #kindv); } \
+    } while (0)
+
+static uint16_t f2h(float f) { _Float16 h = (_Float16)f; uint16_t b; std::memcpy(&b, &h, 2); return b; }
+static float h2f(uint16_t b) { _Float16 h; std::memcpy(&h, &b, 2); return (float)h; }
+
+// ---------------------------------------------------------------------------------------------------------------
+static void test_plan_table() {
+    using B = QWGemmPlan::Backend;
+    // decode GEMV families and outputs (QWGemm.swift:92-133)
+    auto p = QWGemm::plan({1, 17408, 5120}, QWDType::q4g, QWEpilogue::none, QWDType::f16);
+    CHECK(p.backend == B::handQ4gV4H16 && p.kernel == "qwg_gemv_q4g_v4_h16" && p.family == QWGemmFamily::f1DecodeGemv);
+    p = QWGemm::plan({1, 17408, 5120}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::handQ4gV4 && p.kernel == "qwg_gemv_q4g_v4");
+    p = QWGemm::plan({1, 248320, 5120}, QWDType::q4g, QWEpilogue::none, QWDType::f32, 248320);
+    CHECK(p.family == QWGemmFamily::f2LmHeadGemv && p.backend == B::handQ4gV4);
+    p = QWGemm::plan({1, 34816, 5120}, QWDType::q4g, QWEpilogue::siluMulPair, QWDType::f16);
+    CHECK(p.backend == B::handQ4gSiluPairH16 && p.kernel == "qwg_gemv_q4g_silu_pair_h16");
+    p = QWGemm::plan({3, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::handQ4gSkinny && p.kernel == "qwg_skinny_m3" && p.family == QWGemmFamily::f5SkinnyGemm);
+    p = QWGemm::plan({4096, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::mfmaGemmF16 && p.family == QWGemmFamily::f3PrefillGemm);
+    p = QWGemm::plan({4096, 5120, 5100}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::blocked);
+    p = QWGemm::plan({1, 64, 64}, QWDType::f32, QWEpilogue::none);
+    CHECK(p.backend == B::blocked);
+    CHECK((QWGemmShape{100, 8, 8}.family() == QWGemmFamily::f4AttentionTiles));
+}
+
+static void test_weight_view() {
+    std::vector<uint8_t> buf(8 * 2 * 36);
+    QWTensorValue blocks = QWTensorValue::make(buf.data(), buf.size(), QWDType::q4g);
+    // QWWeightView.init? (QWWeightView.swift:107-118)
+    CHECK(QWWeightView::make(blocks, 8, 64, 4, 32, true).has_value());
+    CHECK(QWWeightView::make(blocks, 8, 64, 4, 32, true)->containerKind.isIncumbentContainer());
+    CHECK(QWWeightView::make(blocks, 8, 64, 4, 32, true)->formatName() == "HQ4_G32");
+    CHECK(!QWWeightView::make(blocks, 0, 64, 4, 32, true).has_value());
+    CHECK(!QWWeightView::make(blocks, 8, 48, 4, 32, true).has_value());
+    CHECK(!QWWeightView::make(blocks, 8, 64, 5, 32, true).has_value());
+    CHECK(!QWWeightView::make(blocks, 8, 64, 4, 32, false, true).has_value());   // incumbent must be rotated
+    auto v8 = QWWeightView::make(blocks, 8, 64, 8, 32, true);
+    CHECK(v8.has_value() && v8->rowBytes() == 72 && v8->requiredBytes() == 576 && v8->formatName() == "HQ8_G32" && v8->isRotated());
+    auto a4 = QWWeightView::make(blocks, 8, 64, 4, 64, false);
+    CHECK(a4.has_value() && a4->formatName() == "AQ4_G64" && !a4->isRotated() && a4->rowBytes() == 36);
+    // the 4-bit G32 pair has two containers of the same size but different kinds (QWAQBlock.swift:14-16)
+    auto blk = QWWeightView::make(blocks, 8, 64, 4, 32, true, false);
+    CHECK(blk.has_value() && !blk->containerKind.isIncumbentContainer() && blk->rowBytes() == 40);
+    QWTensorValue small = QWTensorValue::make(buf.data(), 8 * 2 * 20 - 1, QWDType::q4g);
+    CHECK(!QWWeightView::make(small, 8, 64, 4, 32, true).has_value());
+    CHECK(v8->subview(blocks, 4, 64).has_value());
+}
+
+static void test_hal_refuses_without_device() {
+    // no device: the HAL refuses to open (no CPU fallback)
+    CHECK_THROWS(QWHal hal(0), QWHalError, QWHalError::deviceUnavailable);
+}
+
+static void test_error_mapping() {
+    CHECK_THROWS(throwIfFailed(QWHIP_E_BAD_GEOMETRY), QWGemmError, QWGemmError::badGeometry);
+    CHECK_THROWS(throwIfFailed(QWHIP_E_KERNEL_MISSING), QWHalError, QWHalError::kernelMissing);
+    CHECK(QWGemm::moeMaxTiles(128, 16384) == 384 && QWGemm::moeMaxTiles(128, 5) == 5);
+    CHECK(QWGemmAQ::kernelName(8, 32).value_or("") == "qwg_gemv_aq8_g32_v4" && !QWGemmAQ::kernelName(3, 32).has_value());
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+static uint64_t splitmix64(uint64_t x) {
+    uint64_t z = x + 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+static const int kNibbleShift[8] = {0, 16, 4, 20, 8, 24, 12, 28};  // QWAQProducer.hq4NibbleBitOffset
+
+struct DeviceBuf {
+    QWHal& hal;
+    void* p;
+    size_t bytes;
+    DeviceBuf(QWHal& h, size_t n) : hal(h), p(h.alloc(n ? n : 256)), bytes(n) {}
+    ~DeviceBuf() { hal.free(p); }
+};
+static void upload(QWHipEncoder& e, DeviceBuf& b, const void* src, size_t n) { throwIfFailed(qwhip_memcpy_h2d(e.stream, b.p, src, n)); }
+static void download(QWHipEncoder& e, void* dst, DeviceBuf& b, size_t n) { throwIfFailed(qwhip_memcpy_d2h(e.stream, dst, b.p, n)); }
+
+static void test_gpu_hq4_gemv(QWHal& hal) {
+    const int rows = 64, cols = 256, groups = cols / 32;
+    std::vector<uint8_t> bank((size_t)rows * groups * 20);
+    for (int r = 0; r < rows; ++r)
+        for (int g = 0; g < groups; ++g) {
+            const uint64_t s = splitmix64((uint64_t)r * 0x00000001000003B3ull + (uint64_t)g * 0x9E3779B97F4A7C15ull);
+            const double unit = (double)(splitmix64(s + 0x5DEECE66Dull) % 1000000) / 1000000.0;
+            const uint16_t sc = f2h((float)(unit * 0.02 + 0.001));
+            const uint16_t bi = f2h(-1032.0f * h2f(sc));
+            uint8_t* o = &bank[((size_t)r * groups + g) * 20];
+            std::memcpy(o, &sc, 2);
+            std::memcpy(o + 2, &bi, 2);
+            for (int w = 0; w < 4; ++w) {
+                uint32_t word = 0;
+                for (int j = 0; j < 8; ++j) word |= (uint32_t)(splitmix64(s + (uint64_t)(8 * w + j)) & 0xF) << kNibbleShift[j];
+                std::memcpy(o + 4 + 4 * w, &word, 4);
+            }
+        }
+    std::vector<uint16_t> xs(cols);
+    for (int i = 0; i < cols; ++i) xs[i] = f2h((float)((double)(splitmix64((uint64_t)i * 0x9E3779B97F4A7C15ull) % 2000001) / 1000000.0 - 1.0));
+
+    QWHipEncoder enc = hal.begin();
+    DeviceBuf dbank(hal, bank.size()), dx(hal, cols * 2), dy16(hal, rows * 2), dy32(hal, rows * 4);
+    upload(enc, dbank, bank.data(), bank.size());
+    upload(enc, dx, xs.data(), cols * 2);
+    auto view = QWWeightView::make(QWTensorValue::make(dbank.p, bank.size(), QWDType::q4g), rows, cols, 4, 32, true);
+    CHECK(view.has_value());
+    const QWTensorValue x = QWTensorValue::make(dx.p, cols, QWDType::f16);
+    const QWTensorValue y16 = QWTensorValue::make(dy16.p, rows, QWDType::f16), y32 = QWTensorValue::make(dy32.p, rows, QWDType::f32);
+    const QWGemmPlan plan = QWGemm::plan({1, rows, cols}, QWDType::q4g, QWEpilogue::none, QWDType::f16);
+    QWGemm::encodeH16(enc, hal, plan, x, *view, y16, &y32);   // dual store
+    std::vector<float> got(rows);
+    download(enc, got.data(), dy32, rows * 4);
+    std::vector<uint16_t> got16(rows);
+    download(enc, got16.data(), dy16, rows * 2);
+    for (int r = 0; r < rows; ++r) {
+        double value = 0, magnitude = 0;
+        for (int g = 0; g < groups; ++g) {
+            const uint8_t* o = &bank[((size_t)r * groups + g) * 20];
+            uint16_t sc, bi;
+            std::memcpy(&sc, o, 2);
+            std::memcpy(&bi, o + 2, 2);
+            for (int w = 0; w < 4; ++w) {
+                uint32_t word;
+                std::memcpy(&word, o + 4 + 4 * w, 4);
+                for (int j = 0; j < 8; ++j) {
+                    const float nib = (float)((word >> kNibbleShift[j]) & 0xF);
+                    const float v = h2f(f2h((1024.0f + nib) * h2f(sc) + h2f(bi)));
+                    const double prod = (double)v * (double)h2f(xs[g * 32 + w * 8 + j]);
+                    value += prod;
+                    magnitude += std::fabs(prod);
+                }
+            }
+        }
+        const double scale = std::fmax(std::fmax(std::fabs(value), magnitude), 1e-6);
+        CHECK(std::fabs((double)got[r] - value) / scale <= 1e-3);
+        CHECK(std::fabs((double)h2f(got16[r]) - value) / scale <= 2e-3);
+    }
+    // errors surface before any launch and leave the stream usable (Tests/QWGEMMTests/QWGEMMTests.swift:246-247)
+    const QWTensorValue shortX = QWTensorValue::make(dx.p, cols - 1, QWDType::f16);
+    CHECK_THROWS(QWGemm::encodeH16(enc, hal, plan, shortX, *view, y16), QWGemmError, QWGemmError::badWeights);
+    const QWTensorValue wrongY = QWTensorValue::make(dy16.p, rows / 2, QWDType::f32);
+    CHECK_THROWS(QWGemm::encodeH16(enc, hal, plan, x, *view, wrongY), QWGemmError, QWGemmError::badWeights);
+    CHECK_THROWS(hal.pipeline("qwg_gemv_shvq4_g32_v4"), QWHalError, QWHalError::kernelMissing);
+    const QWGemmPlan blocked = QWGemm::plan({1, rows, cols}, QWDType::f32, QWEpilogue::none);
+    CHECK_THROWS(QWGemm::encode(enc, hal, blocked, x, *view, y32), QWGemmError, QWGemmError::f3Blocked);
+    QWGemm::encodeH16(enc, hal, plan, x, *view, y16);
+    hal.end(enc);
+}
+
+// closed-form bank: code (r*7 + c*3 + 5) % 16, scale 1/16, HQ4_G32 block -> weight (code - 8)/16
+static double cf_weight(int row, int col) { return ((double)((row * 7 + col * 3 + 5) % 16) - 8.0) / 16.0; }
+static std::vector<uint8_t> cf_bank(int rows, int cols) {
+    std::vector<uint8_t> bank((size_t)rows * (cols / 32) * 20);
+    const uint16_t sc = f2h(1.0f / 16), bi = f2h(-1032.0f / 16);
+    for (int r = 0; r < rows; ++r)
+        for (int g = 0; g < cols / 32; ++g) {
+            uint8_t* o = &bank[((size_t)r * (cols / 32) + g) * 20];
+            std::memcpy(o, &sc, 2);
+            std::memcpy(o + 2, &bi, 2);
+            for (int w = 0; w < 4; ++w) {
+                uint32_t word = 0;
+                for (int j = 0; j < 8; ++j) word |= (uint32_t)((r * 7 + (g * 32 + w * 8 + j) * 3 + 5) % 16) << kNibbleShift[j];
+                std::memcpy(o + 4 + 4 * w, &word, 4);
+            }
+        }
+    return bank;
+}
+static void fwht32(double* p) {
+    for (int h = 1; h < 32; h <<= 1)
+        for (int i0 = 0; i0 < 32; i0 += 2 * h)
+            for (int j = 0; j < h; ++j) {
+                const double u = p[i0 + j], v = p[i0 + j + h];
+                p[i0 + j] = u + v;
+                p[i0 + j + h] = u - v;
+            }
+    for (int i = 0; i < 32; ++i) p[i] /= std::sqrt(32.0);
+}
+
+static void test_gpu_moe_resident(QWHal& hal, int rows) {
+    const int E = 16, K = 3, H = 64, I = 64;
+    const std::vector<uint8_t> gu = cf_bank(E * 2 * I, H), dn = cf_bank(E * H, I);
+    std::vector<float> router((size_t)E * H);
+    for (int e = 0; e < E; ++e)
+        for (int h = 0; h < H; ++h) router[(size_t)e * H + h] = (float)(((e * 5 + h * 11) % 17) - 8) / 32.0f;
+    std::vector<uint16_t> x((size_t)rows * H);
+    std::vector<double> xd((size_t)rows * H);
+    for (int t = 0; t < rows; ++t)
+        for (int h = 0; h < H; ++h) {
+            const float v = (float)(((t * 13 + h * 7) % 19) - 9) / 8.0f;
+            x[(size_t)t * H + h] = f2h(v);
+            xd[(size_t)t * H + h] = h2f(f2h(v));
+        }
+    // host reference: routing (softmax top-k, ties to the lower index, renormalised), experts in double, act rounded to f16 after rotation
+    std::vector<double> ref((size_t)rows * H, 0.0);
+    for (int t = 0; t < rows; ++t) {
+        std::vector<double> logit(E), p(E);
+        double mx = -1e300, tot = 0;
+        for (int e = 0; e < E; ++e) {
+            double s = 0;
+            for (int h = 0; h < H; ++h) s += (double)router[(size_t)e * H + h] * xd[(size_t)t * H + h];
+            logit[e] = (double)(float)s;
+            mx = std::fmax(mx, logit[e]);
+        }
+        for (int e = 0; e < E; ++e) { p[e] = std::exp(logit[e] - mx); tot += p[e]; }
+        std::vector<int> chosen;
+        std::vector<bool> taken(E, false);
+        double wsum = 0;
+        for (int r = 0; r < K; ++r) {
+            int best = -1;
+            for (int e = 0; e < E; ++e)
+                if (!taken[e] && (best < 0 || p[e] > p[best])) best = e;
+            taken[best] = true;
+            chosen.push_back(best);
+            wsum += p[best] / tot;
+        }
+        for (int r = 0; r < K; ++r) {
+            const int e = chosen[r];
+            const double wk = (p[e] / tot) / wsum;
+            std::vector<double> act(I);
+            for (int i = 0; i < I; ++i) {
+                double g = 0, u = 0;
+                for (int h = 0; h < H; ++h) {
+                    g += cf_weight(e * 2 * I + i, h) * xd[(size_t)t * H + h];
+                    u += cf_weight(e * 2 * I + I + i, h) * xd[(size_t)t * H + h];
+                }
+                act[i] = g / (1 + std::exp(-g)) * u;
+            }
+            for (int o = 0; o < I; o += 32) fwht32(&act[o]);
+            for (int i = 0; i < I; ++i) act[i] = h2f(f2h((float)act[i]));
+            for (int h = 0; h < H; ++h) {
+                double d = 0;
+                for (int i = 0; i < I; ++i) d += cf_weight(e * H + h, i) * act[i];
+                ref[(size_t)t * H + h] += wk * d;
+            }
+        }
+    }
+    QWHipEncoder enc = hal.begin();
+    const int pairs = rows * K, mt = QWGemm::moeMaxTiles(E, pairs);
+    DeviceBuf dgu(hal, gu.size()), ddn(hal, dn.size()), dr(hal, router.size() * 4), dx(hal, x.size() * 2), dout(hal, (size_t)rows * H * 4);
+    DeviceBuf dlog(hal, (size_t)rows * E * 4), didx(hal, pairs * 4), dw(hal, pairs * 4), dact(hal, (size_t)pairs * I * 2);
+    DeviceBuf doff(hal, (E + 1) * 4), dsp(hal, pairs * 4), dst(hal, pairs * 4), dinv(hal, pairs * 4), dte(hal, mt * 4), dtr(hal, mt * 4), dtc(hal, 16);
+    DeviceBuf dgu16(hal, (size_t)pairs * 2 * I * 2), ddnhi(hal, (size_t)pairs * H * 4);
+    upload(enc, dgu, gu.data(), gu.size());
+    upload(enc, ddn, dn.data(), dn.size());
+    upload(enc, dr, router.data(), router.size() * 4);
+    upload(enc, dx, x.data(), x.size() * 2);
+    QWMoEOperator::Weights w;
+    w.router = QWTensorValue::make(dr.p, router.size(), QWDType::f32);
+    w.gateUp = *QWWeightView::make(QWTensorValue::make(dgu.p, gu.size(), QWDType::q4g), E * 2 * I, H, 4, 32, true);
+    w.down = *QWWeightView::make(QWTensorValue::make(ddn.p, dn.size(), QWDType::q4g), E * H, I, 4, 32, true);
+    w.hidden = H; w.experts = E; w.topK = K; w.intermediate = I;
+    QWMoEOperator::Scratch s;
+    s.logits = QWTensorValue::make(dlog.p, (size_t)rows * E, QWDType::f32);
+    s.idx = QWTensorValue::make(didx.p, pairs, QWDType::i32);
+    s.wts = QWTensorValue::make(dw.p, pairs, QWDType::f32);
+    s.act16 = QWTensorValue::make(dact.p, (size_t)pairs * I, QWDType::f16);
+    s.expOff = QWTensorValue::make(doff.p, E + 1, QWDType::i32);
+    s.sortedPair = QWTensorValue::make(dsp.p, pairs, QWDType::i32);
+    s.sortedTok = QWTensorValue::make(dst.p, pairs, QWDType::i32);
+    s.invPerm = QWTensorValue::make(dinv.p, pairs, QWDType::i32);
+    s.tileE = QWTensorValue::make(dte.p, mt, QWDType::i32);
+    s.tileR = QWTensorValue::make(dtr.p, mt, QWDType::i32);
+    s.tileCount = QWTensorValue::make(dtc.p, 4, QWDType::i32);
+    s.gu16 = QWTensorValue::make(dgu16.p, (size_t)pairs * 2 * I, QWDType::f16);
+    s.dnHi = QWTensorValue::make(ddnhi.p, (size_t)pairs * H, QWDType::f32);
+    const QWTensorValue xt = QWTensorValue::make(dx.p, x.size(), QWDType::f16);
+    const QWTensorValue out = QWTensorValue::make(dout.p, (size_t)rows * H, QWDType::f32);
+    // the test feeds the same rows to the router and the experts (the closed-form bank is taken as given in its basis)
+    QWMoEOperator::encodeResident(enc, hal, w, s, xt, xt, out, rows);
+    std::vector<float> got((size_t)rows * H);
+    download(enc, got.data(), dout, got.size() * 4);
+    double num = 0, den = 0;
+    for (size_t i = 0; i < got.size(); ++i) { num += ((double)got[i] - ref[i]) * ((double)got[i] - ref[i]); den += ref[i] * ref[i]; }
+    const double err = std::sqrt(num / std::fmax(den, 1e-30));
+    std::printf("moe encodeResident rows=%d normalized error %.3e\n", rows, err);
+    CHECK(err <= 2e-3);
+    hal.end(enc);
+}
+
+int main(int argc, char** argv) {
+    const bool gpu = argc > 1 && std::strcmp(argv[1], "--gpu") == 0;
+    test_plan_table();
+    test_weight_view();
+    const bool nodevice = argc > 1 && std::strcmp(argv[1], "--cpu-nodevice") == 0;
+    if (!gpu) {
+        test_error_mapping();
+        if (nodevice) test_hal_refuses_without_device();
+    } else {
+        QWHal hal(0);
+        std::printf("device: %s (%s), %u CUs\n", hal.caps.name, hal.caps.arch, hal.caps.compute_units);
+        test_gpu_hq4_gemv(hal);
+        test_gpu_moe_resident(hal, 3);    // decode / verify path
+        test_gpu_moe_resident(hal, 40);   // grouped prefill path
+    }
+    std::printf("%d checks, %d failed\n", g_checks, g_failed);
+    return g_failed ? 1 : 0;
+}

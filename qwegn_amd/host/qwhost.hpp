@@ -1,0 +1,526 @@
+// qwhost.hpp - host-side operator layer above the libqwhip C ABI, mirroring the reference's Swift operator API
+// for the quantized matmul path name for name: QWHal, QWTensorValue, QWWeightView, QWGemm, QWGemmAQ, QWMoEOperator.
+// Argument meaning and error behaviour follow the cited Swift sources: every check runs before the first launch
+// and failures surface as the same typed errors (QWGemmError / QWHalError), so a failed encode leaves the stream
+// untouched.  Header-only C++17; link against libqwhip.so.
+//
+// Paths cited below are relative to the reference checkout.
+#pragma once
+#include <cstdint>
+#include <cstring>
+#include <optional>
+#include <stdexcept>
+#include <string>
+
+#include "../../include/qwhip.h"
+
+namespace qw {
+
+// ---- QWDType (Sources/Foundation/QWCore/QWDType.swift) -----------------------------------------------------------
+enum class QWDType { f32, f16, bf16, i32, q4g };
+inline size_t dtypeBytes(QWDType d) { return d == QWDType::f32 || d == QWDType::i32 ? 4 : (d == QWDType::q4g ? 1 : 2); }
+inline uint32_t abiDType(QWDType d) {
+    switch (d) {
+        case QWDType::f32: return QWHIP_F32;
+        case QWDType::f16: return QWHIP_F16;
+        case QWDType::bf16: return QWHIP_BF16;
+        default: return QWHIP_I32;
+    }
+}
+
+// ---- errors (QWGemm.swift:66-80, Sources/Foundation/QWHAL/QWHal.swift:60-77) ---------------------------------------
+struct QWGemmError : std::runtime_error {
+    enum Kind { f3Blocked, badWeights, badShape, badGeometry } kind;
+    QWGemmError(Kind k, const std::string& s) : std::runtime_error(prefix(k) + s), kind(k) {}
+    static std::string prefix(Kind k) {
+        switch (k) {
+            case f3Blocked: return "QWGEMM: F3 prefill path blocked - ";
+            case badWeights: return "QWGEMM: weight view invalid - ";
+            case badShape: return "QWGEMM: shape invalid - ";
+            default: return "QWGEMM: geometry invalid - ";
+        }
+    }
+};
+struct QWHalError : std::runtime_error {
+    enum Kind { deviceUnavailable, kernelMissing } kind;
+    QWHalError(Kind k, const std::string& s) : std::runtime_error(s), kind(k) {}
+};
+
+// Maps a C-ABI status onto the Swift error cases; QWHIP_OK passes.
+inline void throwIfFailed(qwhip_status st) {
+    if (st == QWHIP_OK) return;
+    const std::string msg = qwhip_last_error();
+    switch (st) {
+        case QWHIP_E_BAD_WEIGHTS: case QWHIP_E_NULL: case QWHIP_E_BASIS: throw QWGemmError(QWGemmError::badWeights, msg);
+        case QWHIP_E_BAD_SHAPE: throw QWGemmError(QWGemmError::badShape, msg);
+        case QWHIP_E_BAD_GEOMETRY: throw QWGemmError(QWGemmError::badGeometry, msg);
+        case QWHIP_E_BLOCKED: throw QWGemmError(QWGemmError::f3Blocked, msg);
+        case QWHIP_E_KERNEL_MISSING: throw QWHalError(QWHalError::kernelMissing, msg);
+        default: throw QWHalError(QWHalError::deviceUnavailable, msg);
+    }
+}
+
+// ---- QWTensorShape / QWTensorValue (Sources/Foundation/QWAlloc/QWArena.swift:36-151): non-owning typed region ----
+struct QWTensorShape {
+    size_t elementCount = 0;
+    QWDType dtype = QWDType::f16;
+};
+struct QWTensorValue {
+    void* base = nullptr;  // device pointer of the arena region
+    size_t offset = 0;     // byte offset of this tensor inside the region
+    size_t bytes = 0;      // bytes available from offset on
+    QWTensorShape shape;
+    void* ptr() const { return (uint8_t*)base + offset; }
+    // x.slice(byteOffset:count:dtype:) (QWArena.swift:120-151)
+    QWTensorValue slice(size_t byteOffset, size_t count, QWDType dtype) const {
+        QWTensorValue t = *this;
+        t.offset += byteOffset;
+        t.bytes = bytes >= byteOffset ? bytes - byteOffset : 0;
+        t.shape = {count, dtype};
+        return t;
+    }
+    static QWTensorValue make(void* base, size_t count, QWDType dtype, size_t offset = 0) {
+        return {base, offset, count * dtypeBytes(dtype), {count, dtype}};
+    }
+};
+
+// ---- QWWeightView (Sources/Foundation/QWAlloc/QWWeightView.swift:9-152) -------------------------------------------
+struct QWWeightView {
+    struct ContainerKind {
+        enum Tag { incumbentHQ4G32, rotatedHQ, nativeAffine } tag = incumbentHQ4G32;
+        int bitsV = 4, groupV = 32;
+        static ContainerKind incumbent() { return {incumbentHQ4G32, 4, 32}; }
+        static ContainerKind rotated(int bits, int group) { return {rotatedHQ, bits, group}; }
+        static ContainerKind affine(int bits, int group) { return {nativeAffine, bits, group}; }
+        int bits() const { return bitsV; }
+        int groupSize() const { return groupV; }
+        bool isRotated() const { return tag != nativeAffine; }
+        bool isIncumbentContainer() const { return tag == incumbentHQ4G32; }
+        uint32_t abiKind() const { return tag == incumbentHQ4G32 ? QWHIP_KIND_HQ4_G32_M5 : (tag == rotatedHQ ? QWHIP_KIND_ROTATED_HQ : QWHIP_KIND_NATIVE_AFFINE); }
+        std::string formatName() const {
+            if (tag == incumbentHQ4G32) return "HQ4_G32";
+            return std::string(tag == rotatedHQ ? "HQ" : "AQ") + std::to_string(bitsV) + "_G" + std::to_string(groupV);
+        }
+        int groupBytes() const { return (int)qwhip_block_bytes(abiKind(), (uint32_t)bitsV, (uint32_t)groupV); }  // 0 = unsupported
+        size_t rowBytes(int k) const { return (size_t)(k / groupV) * (size_t)groupBytes(); }
+    };
+
+    QWTensorValue blocks;
+    int n = 0, k = 0;
+    ContainerKind containerKind;
+
+    int bits() const { return containerKind.bits(); }
+    int groupSize() const { return containerKind.groupSize(); }
+    bool isRotated() const { return containerKind.isRotated(); }
+    size_t rowBytes() const { return containerKind.rowBytes(k); }
+    size_t requiredBytes() const { return rowBytes() * (size_t)n; }
+    std::string formatName() const { return containerKind.formatName(); }
+
+    // init?(blocks:n:k:containerKind:) - nullopt unless n > 0, k > 0, k % group == 0, the pair is supported and the bytes fit
+    static std::optional<QWWeightView> make(const QWTensorValue& blocks, int n, int k, ContainerKind kind) {
+        if (n <= 0 || k <= 0 || kind.groupSize() <= 0 || k % kind.groupSize() != 0) return std::nullopt;
+        const int gb = kind.groupBytes();
+        if (gb == 0) return std::nullopt;
+        if (blocks.bytes < (size_t)n * (size_t)(k / kind.groupSize()) * (size_t)gb) return std::nullopt;
+        QWWeightView v;
+        v.blocks = blocks;
+        v.n = n;
+        v.k = k;
+        v.containerKind = kind;
+        return v;
+    }
+    // init?(blocks:n:k:bits:groupSize:isRotated:) - isRotated has no default: every construction states the basis
+    static std::optional<QWWeightView> make(const QWTensorValue& blocks, int n, int k, int bits, int groupSize, bool isRotated,
+                                            std::optional<bool> isIncumbentContainer = std::nullopt) {
+        const bool incumbent = isIncumbentContainer.value_or(isRotated && bits == 4 && groupSize == 32);
+        if (incumbent) {
+            if (!(isRotated && bits == 4 && groupSize == 32)) return std::nullopt;
+            return make(blocks, n, k, ContainerKind::incumbent());
+        }
+        return make(blocks, n, k, isRotated ? ContainerKind::rotated(bits, groupSize) : ContainerKind::affine(bits, groupSize));
+    }
+    std::optional<QWWeightView> subview(const QWTensorValue& b, int n2, int k2) const { return make(b, n2, k2, containerKind); }
+
+    qwhip_weight_view abi() const {
+        qwhip_weight_view w;
+        w.blocks = blocks.ptr();
+        w.bytes = blocks.bytes;
+        w.n = (uint32_t)n;
+        w.k = (uint32_t)k;
+        w.kind = containerKind.abiKind();
+        w.bits = (uint32_t)bits();
+        w.group = (uint32_t)groupSize();
+        return w;
+    }
+};
+
+// ---- QWHal (Sources/Foundation/QWHAL/QWHal.swift:81-398): device + encoder (= stream) -----------------------------
+struct QWHipEncoder {
+    qwhip_stream_t stream = nullptr;
+};
+class QWHal {
+public:
+    explicit QWHal(int ordinal = 0) {
+        qwhip_status st = qwhip_device_create(ordinal, &dev_);
+        if (st != QWHIP_OK) throw QWHalError(QWHalError::deviceUnavailable, qwhip_last_error());
+        qwhip_device_caps(dev_, &caps);
+    }
+    ~QWHal() {
+        if (dev_) qwhip_device_destroy(dev_);
+    }
+    QWHal(const QWHal&) = delete;
+    QWHal& operator=(const QWHal&) = delete;
+    qwhip_caps caps{};
+    // hal.pipeline(name): throws QWHalError.kernelMissing(name) (QWHal.swift:291-322); returns the serving launcher's name
+    const char* pipeline(const char* name) const {
+        const char* launcher = nullptr;
+        if (qwhip_kernel_lookup(name, &launcher) != QWHIP_OK) throw QWHalError(QWHalError::kernelMissing, qwhip_last_error());
+        return launcher;
+    }
+    QWHipEncoder begin() {  // hal.begin(): opens an encoder (QWHal.swift:325-350)
+        QWHipEncoder e;
+        throwIfFailed(qwhip_stream_create(dev_, &e.stream));
+        return e;
+    }
+    void end(QWHipEncoder& e) {  // hal.end(): commit and wait (QWHal.swift:352-378)
+        throwIfFailed(qwhip_stream_sync(e.stream));
+        qwhip_stream_destroy(e.stream);
+        e.stream = nullptr;
+    }
+    void* alloc(size_t bytes) {
+        void* p = nullptr;
+        throwIfFailed(qwhip_malloc(dev_, bytes, &p));
+        return p;
+    }
+    void free(void* p) { qwhip_free(dev_, p); }
+    qwhip_device_t device() const { return dev_; }
+
+private:
+    qwhip_device_t dev_ = nullptr;
+};
+
+// ---- QWGemm (Sources/Operators/QWGEMM/QWGemm.swift) ---------------------------------------------------------------
+enum class QWGemmFamily { f1DecodeGemv, f2LmHeadGemv, f3PrefillGemm, f4AttentionTiles, f5SkinnyGemm };
+enum class QWEpilogue { none, siluMulPair };
+
+struct QWGemmShape {
+    int m, n, k;
+    QWGemmFamily family(std::optional<int> vocab = std::nullopt) const {  // QWGemm.swift:27-33
+        if (m == 1 && vocab && n == *vocab) return QWGemmFamily::f2LmHeadGemv;
+        if (m == 1) return QWGemmFamily::f1DecodeGemv;
+        if (m >= 512) return QWGemmFamily::f3PrefillGemm;
+        if (m <= 8) return QWGemmFamily::f5SkinnyGemm;
+        return QWGemmFamily::f4AttentionTiles;
+    }
+};
+
+struct QWGemmPlan {
+    // The reference's backends, with the prefill winner re-pointed at the MFMA kernel this library ships and the
+    // skinny window widened: the streaming GEMV takes M = 2..16 in one pass (the reference's F5 window is M in {2,3}).
+    enum class Backend { handQ4gV4, handQ4gV4H16, handQ4gSiluPair, handQ4gSiluPairH16, handQ4gSkinny, mfmaGemmF16, blocked };
+    Backend backend;
+    std::string kernel;  // the reference's kernel name: the key hal.pipeline() resolves
+    int threadsPerTG;
+    QWGemmFamily family;
+    QWEpilogue epilogue;
+};
+
+struct QWGemm {
+    // Pure table lookup (QWGemm.swift:92-133).
+    static QWGemmPlan plan(const QWGemmShape& shape, QWDType dtype, QWEpilogue epi, QWDType outDtype = QWDType::f32,
+                           std::optional<int> vocab = std::nullopt) {
+        using B = QWGemmPlan::Backend;
+        const QWGemmFamily fam = shape.family(vocab);
+        if (dtype != QWDType::q4g) return {B::blocked, "", 0, fam, epi};
+        if (epi == QWEpilogue::siluMulPair)
+            return outDtype == QWDType::f16 ? QWGemmPlan{B::handQ4gSiluPairH16, "qwg_gemv_q4g_silu_pair_h16", 256, fam, epi}
+                                            : QWGemmPlan{B::handQ4gSiluPair, "qwg_gemv_q4g_silu_pair", 256, fam, epi};
+        switch (fam) {
+            case QWGemmFamily::f1DecodeGemv:
+            case QWGemmFamily::f2LmHeadGemv:
+                return outDtype == QWDType::f16 ? QWGemmPlan{B::handQ4gV4H16, "qwg_gemv_q4g_v4_h16", 256, fam, epi}
+                                                : QWGemmPlan{B::handQ4gV4, "qwg_gemv_q4g_v4", 256, fam, epi};
+            case QWGemmFamily::f5SkinnyGemm:
+                if (shape.m >= 2) return {B::handQ4gSkinny, shape.m == 3 ? "qwg_skinny_m3" : "qwg_skinny_m2", 256, fam, epi};
+                return {B::blocked, "", 0, fam, epi};
+            case QWGemmFamily::f3PrefillGemm:
+                if (shape.k % 64 == 0) return {B::mfmaGemmF16, "qwg_gemm_q4g_h16", 256, fam, epi};
+                return {B::blocked, "", 0, fam, epi};
+            default:
+                if (shape.m <= 16) return {B::handQ4gSkinny, "qwg_skinny_m2", 256, fam, epi};
+                if (shape.k % 64 == 0) return {B::mfmaGemmF16, "qwg_gemm_q4g_h16", 256, fam, epi};
+                return {B::blocked, "", 0, fam, epi};
+        }
+    }
+
+    // Activations given to these doors are in the container's basis (the reference's producers rotate; pass
+    // `rotateInKernel` to let the GEMV rotate un-rotated activations in its prologue instead).
+
+    // QWGemm.encode (QWGemm.swift:218-283): f32 output; .siluMulPair needs even N and stores f16 activations.
+    static void encode(QWHipEncoder& enc, const QWHal& hal, const QWGemmPlan& plan, const QWTensorValue& x, const QWWeightView& wQ4,
+                       const QWTensorValue& y, int rows = 1, bool rotateInKernel = false) {
+        using B = QWGemmPlan::Backend;
+        if (plan.backend == B::blocked) {
+            if (plan.family == QWGemmFamily::f5SkinnyGemm) throw QWGemmError(QWGemmError::badWeights, "F5 window: run F1 per row");
+            throw QWGemmError(QWGemmError::f3Blocked, "no winner raced for this family");
+        }
+        if (plan.backend == B::mfmaGemmF16) throw QWGemmError(QWGemmError::f3Blocked, "plan resolved to the tensor GEMM - use gemmBatchedH16");
+        if (plan.epilogue == QWEpilogue::siluMulPair && wQ4.n % 2 != 0) throw QWGemmError(QWGemmError::badWeights, "silu_pair needs even N");
+        if (x.shape.dtype != QWDType::f16 && x.shape.dtype != QWDType::bf16) throw QWGemmError(QWGemmError::badWeights, "activations must be f16");
+        if (x.shape.elementCount < (size_t)rows * (size_t)wQ4.k) throw QWGemmError(QWGemmError::badWeights, "activations are short");
+        hal.pipeline(plan.kernel.c_str());
+        const qwhip_weight_view w = wQ4.abi();
+        const uint32_t flags = rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED;
+        if (plan.epilogue == QWEpilogue::siluMulPair) {
+            if (y.shape.dtype != QWDType::f16 || y.shape.elementCount < (size_t)rows * (size_t)(wQ4.n / 2))
+                throw QWGemmError(QWGemmError::badWeights, "silu_pair output must be f16 [rows, N/2]");
+            throwIfFailed(qwhip_gemv_silu_pair(enc.stream, &w, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows, flags, 1, y.ptr()));
+            return;
+        }
+        if (y.shape.dtype != QWDType::f32 || y.shape.elementCount < (size_t)rows * (size_t)wQ4.n)
+            throw QWGemmError(QWGemmError::badWeights, "output must be f32 [rows, N]");
+        throwIfFailed(qwhip_gemv(enc.stream, &w, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows, flags, nullptr, (float*)y.ptr()));
+    }
+
+    // QWGemm.encodeH16 (QWGemm.swift:137-214): direct f16 store, optional dual f32 store.
+    static void encodeH16(QWHipEncoder& enc, const QWHal& hal, const QWGemmPlan& plan, const QWTensorValue& x, const QWWeightView& wQ4,
+                          const QWTensorValue& y16, const QWTensorValue* y32 = nullptr, int rows = 1, bool rotateInKernel = false) {
+        using B = QWGemmPlan::Backend;
+        if (plan.backend != B::handQ4gV4H16 && plan.backend != B::handQ4gSiluPairH16 && plan.backend != B::handQ4gSkinny)
+            throw QWGemmError(QWGemmError::badWeights, "encodeH16 requires handQ4gV4H16 or handQ4gSiluPairH16");
+        if (y16.shape.dtype != QWDType::f16) throw QWGemmError(QWGemmError::badWeights, "y16 must have dtype .f16");
+        if (plan.epilogue == QWEpilogue::siluMulPair) {
+            encode(enc, hal, plan, x, wQ4, y16, rows, rotateInKernel);
+            return;
+        }
+        if (x.shape.dtype != QWDType::f16 && x.shape.dtype != QWDType::bf16) throw QWGemmError(QWGemmError::badWeights, "activations must be f16");
+        if (x.shape.elementCount < (size_t)rows * (size_t)wQ4.k) throw QWGemmError(QWGemmError::badWeights, "activations are short");
+        if (y16.shape.elementCount < (size_t)rows * (size_t)wQ4.n) throw QWGemmError(QWGemmError::badWeights, "y16 is short");
+        if (y32 && (y32->shape.dtype != QWDType::f32 || y32->shape.elementCount < (size_t)rows * (size_t)wQ4.n))
+            throw QWGemmError(QWGemmError::badWeights, "y32 must be f32 [rows, N]");
+        hal.pipeline(plan.kernel.c_str());
+        const qwhip_weight_view w = wQ4.abi();
+        const uint32_t flags = rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED;
+        throwIfFailed(qwhip_gemv(enc.stream, &w, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows, flags, y16.ptr(),
+                                 y32 ? (float*)y32->ptr() : nullptr));
+    }
+
+    // QWGemm.encodeFwht32 (QWGemm.swift:288-300): in-place normalized FWHT-32 over f16 elements.
+    static void encodeFwht32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, std::optional<size_t> count = std::nullopt) {
+        const size_t n = count.value_or(x.shape.elementCount);
+        if (x.shape.dtype != QWDType::f16 || n == 0 || n % 32 != 0)
+            throw QWGemmError(QWGemmError::badWeights, "fwht32 f16: n must be > 0 and divisible by 32");
+        hal.pipeline("qwg_fwht32_f16");
+        throwIfFailed(qwhip_fwht32(enc.stream, x.ptr(), QWHIP_F16, x.ptr(), n));
+    }
+
+    // QWGemm.encodeCast (QWGemm.swift:305-320): the f32 -> f16 seam.
+    static void encodeCast(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x32, const QWTensorValue& y16,
+                           std::optional<size_t> count = std::nullopt) {
+        const size_t n = count.value_or(x32.shape.elementCount);
+        if (x32.shape.dtype != QWDType::f32 || y16.shape.dtype != QWDType::f16 || n == 0 || x32.shape.elementCount < n ||
+            y16.shape.elementCount < n || n % 8 != 0)
+            throw QWGemmError(QWGemmError::badWeights, "cast f32->f16: n must fit buffers and divide 8");
+        hal.pipeline("qwg_cast_f32_to_f16");
+        throwIfFailed(qwhip_cast_f32_to_f16(enc.stream, (const float*)x32.ptr(), y16.ptr(), n));
+    }
+
+    // gemmBatchedH16 (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:119-154) / QWGemm.encodeNaxF32
+    // (Sources/Operators/QWGEMM/QWGemmF32.swift:366-402): Y[rows, n] = X[rows, k] . W^T on the matrix cores.
+    static void gemmBatchedH16(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWWeightView& w, const QWTensorValue& y,
+                               int rows, const QWTensorValue* workspace = nullptr, bool rotateInPrepass = false) {
+        if (rows <= 0) throw QWGemmError(QWGemmError::badShape, "rows must be positive");
+        if (w.n % 64 != 0 || w.k % 64 != 0) throw QWGemmError(QWGemmError::badGeometry, "tensor GEMM needs N and K multiples of 64");
+        if (x.shape.elementCount < (size_t)rows * (size_t)w.k) throw QWGemmError(QWGemmError::badWeights, "activations are short");
+        if (y.shape.elementCount < (size_t)rows * (size_t)w.n) throw QWGemmError(QWGemmError::badWeights, "output is short");
+        hal.pipeline(w.containerKind.isIncumbentContainer() ? "qwg_gemm_q4g_h16" : ("qwg_gemm_aq" + std::to_string(w.bits()) + "_g" + std::to_string(w.groupSize()) + "_h16").c_str());
+        const qwhip_weight_view v = w.abi();
+        throwIfFailed(qwhip_gemm(enc.stream, &v, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows, 0, y.ptr(), abiDType(y.shape.dtype), 0,
+                                 rotateInPrepass ? 0u : (uint32_t)QWHIP_X_PREROTATED, workspace ? workspace->ptr() : nullptr,
+                                 workspace ? workspace->bytes : 0));
+    }
+
+    // QWGemm.encodeSiluMulF16 / encodeSiluMulSplitF16 (QWGemmF32.swift:47-115): SwiGLU (+FWHT-32) over gate|up rows.
+    static void encodeSiluMulSplitF16(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& gu, const QWTensorValue& act16, int rows,
+                                      int inter, bool rotate = true) {
+        if (act16.shape.dtype != QWDType::f16 || act16.shape.elementCount < (size_t)rows * (size_t)inter ||
+            gu.shape.elementCount < (size_t)rows * 2 * (size_t)inter)
+            throw QWGemmError(QWGemmError::badShape, "silu_mul: buffers do not fit rows x intermediate");
+        hal.pipeline("qwg_silu_mul_split_f16");
+        throwIfFailed(qwhip_swiglu_fwht(enc.stream, gu.ptr(), abiDType(gu.shape.dtype), act16.ptr(), (uint32_t)rows, (uint32_t)inter, rotate ? 1 : 0));
+    }
+
+    // ---- MoE encoders (Sources/Operators/QWGEMM/QWGemmMoE.swift, QWGemmMoERouter.swift) ----------------------------
+    static int moeMaxTiles(int experts, int pairs) { return (int)qwhip_moe_max_tiles((uint32_t)experts, (uint32_t)pairs); }  // QWGemmMoE.swift:24-26
+
+    // encodeFnRouterGemm (QWGemmMoERouter.swift:78-113)
+    static void encodeFnRouterGemm(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWTensorValue& router,
+                                   const QWTensorValue& logits, int rows, int experts, int hidden) {
+        if (logits.shape.dtype != QWDType::f32 || logits.shape.elementCount < (size_t)rows * (size_t)experts)
+            throw QWGemmError(QWGemmError::badShape, "router logits must be f32 [rows, experts]");
+        hal.pipeline("qwg_router_gemm");
+        throwIfFailed(qwhip_router_gemm(enc.stream, x.ptr(), abiDType(x.shape.dtype), router.ptr(), abiDType(router.shape.dtype), (uint32_t)rows,
+                                        (uint32_t)experts, (uint32_t)hidden, (float*)logits.ptr()));
+    }
+    // encodeFnMoeRoute (QWGemmMoERouter.swift:10-75)
+    static void encodeFnMoeRoute(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& logits, const QWTensorValue& idx,
+                                 const QWTensorValue& wts, int rows, int experts, int topK, bool normTopK, float routedScale = 1.0f) {
+        if (experts > 512 || topK > 16 || topK <= 0) throw QWGemmError(QWGemmError::badShape, "router holds 512 experts and 16 routes");
+        if (idx.shape.elementCount < (size_t)rows * (size_t)topK || wts.shape.elementCount < (size_t)rows * (size_t)topK)
+            throw QWGemmError(QWGemmError::badShape, "router outputs are short");
+        hal.pipeline("qwg_moe_route");
+        throwIfFailed(qwhip_moe_route(enc.stream, (const float*)logits.ptr(), (uint32_t)rows, (uint32_t)experts, (uint32_t)topK, normTopK ? 1 : 0,
+                                      routedScale, (int32_t*)idx.ptr(), (float*)wts.ptr()));
+    }
+    // encodeMoEGroupPairsF32 (QWGemmMoE.swift:68-99)
+    static void encodeMoEGroupPairsF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& ids, const QWTensorValue& expertOff,
+                                       const QWTensorValue& sortedPairIdx, const QWTensorValue& sortedTok, int experts, int totalPairs,
+                                       int routes, const QWTensorValue* invPerm = nullptr, const QWTensorValue* tileE = nullptr,
+                                       const QWTensorValue* tileR = nullptr, const QWTensorValue* tileCount = nullptr, bool compactTail = true) {
+        if (experts > 512) throw QWGemmError(QWGemmError::badShape, "the expert-sorted pair order holds 512 experts");
+        const bool hasTiles = tileE && tileR && tileCount;
+        if (hasTiles && (tileE->shape.elementCount < (size_t)moeMaxTiles(experts, totalPairs) ||
+                         tileR->shape.elementCount < (size_t)moeMaxTiles(experts, totalPairs)))
+            throw QWGemmError(QWGemmError::badShape, "moe group pairs: tile scratch does not fit the tile plan");
+        hal.pipeline("qwg_moe_group_pairs_f32");
+        throwIfFailed(qwhip_moe_group_pairs(enc.stream, (const int32_t*)ids.ptr(), (uint32_t)experts, (uint32_t)totalPairs, (uint32_t)routes,
+                                            (int32_t*)expertOff.ptr(), (int32_t*)sortedPairIdx.ptr(), (int32_t*)sortedTok.ptr(),
+                                            invPerm ? (int32_t*)invPerm->ptr() : nullptr, hasTiles ? (int32_t*)tileE->ptr() : nullptr,
+                                            hasTiles ? (int32_t*)tileR->ptr() : nullptr, hasTiles ? (int32_t*)tileCount->ptr() : nullptr,
+                                            compactTail ? 1 : 0));
+    }
+    // encodeMoEGateUpNax / encodeMoENaxSplitF32 (QWGemmMoE.swift:201-296): grouped expert GEMM over the sorted pairs
+    static void encodeMoEGroupedGemm(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& w, int experts, const QWTensorValue& x,
+                                     const QWTensorValue* gather, const QWTensorValue& expertOff, const QWTensorValue& tileE,
+                                     const QWTensorValue& tileR, const QWTensorValue& tileCount, int pairs, const QWTensorValue& y) {
+        hal.pipeline(gather ? "qwg_moe_nax_gemm" : "qwg_moe_nax_split_f32");
+        const qwhip_weight_view v = w.abi();
+        throwIfFailed(qwhip_moe_grouped_gemm(enc.stream, &v, (uint32_t)experts, x.ptr(), abiDType(x.shape.dtype), 0,
+                                             gather ? (const int32_t*)gather->ptr() : nullptr, (const int32_t*)expertOff.ptr(),
+                                             (const int32_t*)tileE.ptr(), (const int32_t*)tileR.ptr(), (const int32_t*)tileCount.ptr(),
+                                             (uint32_t)moeMaxTiles(experts, pairs), (uint32_t)pairs, y.ptr(), abiDType(y.shape.dtype), 0));
+    }
+    // encodeMoEDownReduceCombineF32 (QWGemmMoE.swift:299-332)
+    static void encodeMoEDownReduceCombineF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& dn, const QWTensorValue& invPerm,
+                                              const QWTensorValue& wts, int rows, int topK, int hidden, const QWTensorValue* shared,
+                                              const QWTensorValue* sharedGate, const QWTensorValue& out) {
+        hal.pipeline("qwg_moe_down_reduce_combine_f32");
+        throwIfFailed(qwhip_moe_combine(enc.stream, dn.ptr(), abiDType(dn.shape.dtype), (const int32_t*)invPerm.ptr(), (const float*)wts.ptr(),
+                                        (uint32_t)rows, (uint32_t)topK, (uint32_t)hidden, shared ? (const float*)shared->ptr() : nullptr,
+                                        sharedGate ? (const float*)sharedGate->ptr() : nullptr, out.ptr(), abiDType(out.shape.dtype)));
+    }
+    // encodeMoEGateUpF32R1 / encodeMoEDownSharedCombineF32 (QWGemmMoE.swift:120-199): decode / verify, rows <= 8
+    static void encodeMoEGateUpF32R1(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& gateUp, int experts, const QWTensorValue& x,
+                                     const QWTensorValue& idx, int rows, int topK, const QWTensorValue& act16, bool rotateInKernel = false) {
+        hal.pipeline("qwg_moe_gateup_q4g_f32_r1");
+        const qwhip_weight_view v = gateUp.abi();
+        throwIfFailed(qwhip_moe_gateup_decode(enc.stream, &v, (uint32_t)experts, x.ptr(), abiDType(x.shape.dtype),
+                                              rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED, (const int32_t*)idx.ptr(), (uint32_t)rows,
+                                              (uint32_t)topK, act16.ptr()));
+    }
+    static void encodeMoEDownSharedCombineF32(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& down, int experts,
+                                              const QWTensorValue& act16, const QWTensorValue& idx, const QWTensorValue& wts, int rows, int topK,
+                                              const QWTensorValue* shared, const QWTensorValue* sharedGate, const QWTensorValue& out) {
+        hal.pipeline("qwg_moe_down_shared_combine_q4g_f32");
+        const qwhip_weight_view v = down.abi();
+        throwIfFailed(qwhip_moe_down_decode(enc.stream, &v, (uint32_t)experts, act16.ptr(), (const int32_t*)idx.ptr(), (const float*)wts.ptr(),
+                                            (uint32_t)rows, (uint32_t)topK, shared ? (const float*)shared->ptr() : nullptr,
+                                            sharedGate ? (const float*)sharedGate->ptr() : nullptr, out.ptr(), abiDType(out.shape.dtype)));
+    }
+};
+
+// ---- QWGemmAQ (Sources/Operators/QWGEMM/QWGemmAQ.swift:192-304): the bit-stream block family ----------------------
+struct QWGemmAQ {
+    static std::optional<std::string> kernelName(int bits, int group) {
+        if (!(bits == 4 || bits == 8)) return std::nullopt;
+        if (!(group == 32 || group == 64 || group == 128 || group == 256)) return std::nullopt;
+        return "qwg_gemv_aq" + std::to_string(bits) + "_g" + std::to_string(group) + "_v4";
+    }
+    // QWGemmAQ.encode: f16 activations [rows, k] -> f32 y [rows, n]; every weight byte read once for up to 16 rows a pass
+    static void encode(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& blocks, const QWTensorValue& x, const QWTensorValue& y,
+                       int n, int k, int bits, int group, int rows = 1, bool isRotated = true, bool rotateInKernel = false) {
+        const auto name = kernelName(bits, group);
+        if (!name) throw QWGemmError(QWGemmError::badWeights, "no affine-quantised kernel for this pair");
+        if (k % group != 0 || n <= 0 || rows <= 0) throw QWGemmError(QWGemmError::badWeights, "k must be a multiple of the group and n positive");
+        const auto view = QWWeightView::make(blocks, n, k, bits, group, isRotated, false);
+        if (!view) throw QWGemmError(QWGemmError::badWeights, "block bank is short for n rows");
+        if (x.shape.dtype != QWDType::f16) throw QWGemmError(QWGemmError::badWeights, "activations must be f16");
+        if (x.shape.elementCount < (size_t)rows * (size_t)k) throw QWGemmError(QWGemmError::badWeights, "activations are short");
+        if (y.shape.dtype != QWDType::f32) throw QWGemmError(QWGemmError::badWeights, "output must be f32");
+        if (y.shape.elementCount < (size_t)rows * (size_t)n) throw QWGemmError(QWGemmError::badWeights, "output is short");
+        if (n >= (rows > 1 ? (1 << 24) : (1 << 30))) throw QWGemmError(QWGemmError::badWeights, "bank does not fit the row-count flags");
+        hal.pipeline(name->c_str());
+        const qwhip_weight_view w = view->abi();
+        const uint32_t flags = rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED;
+        for (int r0 = 0; r0 < rows; r0 += 16) {  // the reference chunks at 8 rows; one pass here holds 16
+            const int chunk = rows - r0 < 16 ? rows - r0 : 16;
+            const QWTensorValue xc = x.slice((size_t)r0 * k * 2, (size_t)chunk * k, QWDType::f16);
+            const QWTensorValue yc = y.slice((size_t)r0 * n * 4, (size_t)chunk * n, QWDType::f32);
+            throwIfFailed(qwhip_gemv(enc.stream, &w, xc.ptr(), QWHIP_F16, (uint32_t)chunk, flags, nullptr, (float*)yc.ptr()));
+        }
+    }
+    // QWGemmAQ.encodeDecodeT4: f16 in, f16 out, one row
+    static void encodeDecodeT4(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& blocks, const QWTensorValue& x, const QWTensorValue& y16,
+                               int n, int k, int bits, int group, bool isRotated = true, bool rotateInKernel = false) {
+        const auto name = kernelName(bits, group);
+        if (!name) throw QWGemmError(QWGemmError::badWeights, "no affine-quantised decode kernel for this pair");
+        if (k % group != 0 || n <= 0) throw QWGemmError(QWGemmError::badWeights, "k must be a multiple of the group and n positive");
+        if (n >= (1 << 24)) throw QWGemmError(QWGemmError::badWeights, "bank does not fit the row-count flags");
+        const auto view = QWWeightView::make(blocks, n, k, bits, group, isRotated, false);
+        if (!view) throw QWGemmError(QWGemmError::badWeights, "block bank is short for n rows");
+        if (x.shape.dtype != QWDType::f16 || x.shape.elementCount < (size_t)k) throw QWGemmError(QWGemmError::badWeights, "activations must be f16 [k]");
+        if (y16.shape.dtype != QWDType::f16 || y16.shape.elementCount < (size_t)n) throw QWGemmError(QWGemmError::badWeights, "output must be f16 [n]");
+        hal.pipeline(("qwg_gemv_aq" + std::to_string(bits) + "_g" + std::to_string(group) + "_dx_h16_t4").c_str());
+        const qwhip_weight_view w = view->abi();
+        throwIfFailed(qwhip_gemv(enc.stream, &w, x.ptr(), QWHIP_F16, 1, rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED, y16.ptr(), nullptr));
+    }
+};
+
+// ---- QWMoEOperator.encodeResident (Sources/Operators/QWGEMM/QWMoEOperator.swift:57-442) ---------------------------
+struct QWMoEOperator {
+    struct Weights {
+        QWTensorValue router;  // [experts, hidden] f32 / f16 / bf16
+        QWWeightView gateUp;   // n = experts * 2 * intermediate, k = hidden
+        QWWeightView down;     // n = experts * hidden, k = intermediate
+        int hidden = 0, experts = 0, topK = 0, intermediate = 0;
+        bool normTopK = true;
+        float routedScale = 1.0f;
+    };
+    struct Scratch {  // caller-owned; sizes in elements
+        QWTensorValue logits;      // f32 [rows, experts]
+        QWTensorValue idx;         // i32 [rows, topK]
+        QWTensorValue wts;         // f32 [rows, topK]
+        QWTensorValue act16;       // f16 [rows * topK, intermediate]
+        // prefill only (rows > 8)
+        QWTensorValue expOff, sortedPair, sortedTok, invPerm, tileE, tileR, tileCount;  // i32
+        QWTensorValue gu16;        // f16 [rows * topK, 2 * intermediate]
+        QWTensorValue dnHi;        // f32 or f16 [rows * topK, hidden]
+    };
+    // x: f16 hidden rows in the experts' basis; xPlain: the un-rotated rows the router reads (may equal x for a standard-basis bank).
+    // out = sum_k w_k * expert_k(x) (+ sharedGate * shared when given).  Prefill (rows > 8) runs the grouped path:
+    // router -> route -> pair sort -> gate_up GEMM -> SwiGLU+FWHT -> down GEMM -> combine; decode / verify runs the routed GEMVs.
+    static void encodeResident(QWHipEncoder& enc, const QWHal& hal, const Weights& w, const Scratch& s, const QWTensorValue& x,
+                               const QWTensorValue& xPlain, const QWTensorValue& out, int rows, const QWTensorValue* shared = nullptr,
+                               const QWTensorValue* sharedGate = nullptr) {
+        const int H = w.hidden, E = w.experts, K = w.topK, I = w.intermediate;
+        if (E > 512 || E <= 0 || K <= 0 || K > 16) throw QWGemmError(QWGemmError::badShape, "moe: experts <= 512, routes <= 16");
+        if (w.gateUp.n != E * 2 * I || w.gateUp.k != H || w.down.n != E * H || w.down.k != I)
+            throw QWGemmError(QWGemmError::badShape, "moe: expert banks do not match (experts, hidden, intermediate)");
+        QWGemm::encodeFnRouterGemm(enc, hal, xPlain, w.router, s.logits, rows, E, H);
+        QWGemm::encodeFnMoeRoute(enc, hal, s.logits, s.idx, s.wts, rows, E, K, w.normTopK, w.routedScale);
+        const bool grouped = rows > 8 && s.expOff.base && s.gu16.base && s.dnHi.base && H % 64 == 0 && I % 64 == 0;
+        if (grouped) {
+            const int pairs = rows * K;
+            QWGemm::encodeMoEGroupPairsF32(enc, hal, s.idx, s.expOff, s.sortedPair, s.sortedTok, E, pairs, K, &s.invPerm, &s.tileE, &s.tileR, &s.tileCount);
+            QWGemm::encodeMoEGroupedGemm(enc, hal, w.gateUp, E, x, &s.sortedTok, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.gu16);
+            QWGemm::encodeSiluMulSplitF16(enc, hal, s.gu16, s.act16, pairs, I, w.down.isRotated());
+            QWGemm::encodeMoEGroupedGemm(enc, hal, w.down, E, s.act16, nullptr, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.dnHi);
+            QWGemm::encodeMoEDownReduceCombineF32(enc, hal, s.dnHi, s.invPerm, s.wts, rows, K, H, shared, sharedGate, out);
+        } else {
+            QWGemm::encodeMoEGateUpF32R1(enc, hal, w.gateUp, E, x, s.idx, rows, K, s.act16);
+            QWGemm::encodeMoEDownSharedCombineF32(enc, hal, w.down, E, s.act16, s.idx, s.wts, rows, K, shared, sharedGate, out);
+        }
+    }
+};
+
+}  // namespace qw
