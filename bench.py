@@ -73,7 +73,11 @@ def run_gemv(args, fmt, n, k, m, label, outliers):
     views = [H.view_of(dev, b, fmt, n, k) for b in banks]
     xb = dev.put(x16)
     y16 = dev.alloc(m * n * 2)
-    flags = (args.variant << 8) | (args.rt << 12)
+    prerot = bool(rotate) and (args.prerot or m > 1)     # verify (m > 1) activations arrive rotated by their producer
+    x_basis = H.x_in_basis(x16, fmt)
+    if prerot:
+        xb = dev.put(x_basis)
+    flags = (args.variant << 8) | (args.rt << 12) | (qwhip.X_PREROTATED if prerot else 0)
     lib, st = dev.lib, dev.stream.handle
 
     def launch(i):
@@ -94,7 +98,6 @@ def run_gemv(args, fmt, n, k, m, label, outliers):
     us_per = ms * 1e3 / args.steps
 
     got = y16.download(np.float16, (m, n))
-    x_basis = H.x_in_basis(x16, fmt)
     err = qo.normalized_error(got, qo.matmul_ref_f64(x_basis, w16))
     if not err <= 2e-3:
         _fail(f"bench: output failed parity (normalized error {err:.3e})")
@@ -106,7 +109,7 @@ def run_gemv(args, fmt, n, k, m, label, outliers):
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": label, "format": fmt, "M": m, "N": n, "K": k, "fused_fwht": bool(rotate),
+        "config": {"workload": label, "format": fmt, "M": m, "N": n, "K": k, "fused_fwht": bool(rotate) and not prerot,
                    "cache": "hot" if args.hot else f"cold ring of {ring_n} banks ({ring_n * bank_bytes / 1e6:.0f} MB)"},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
@@ -210,6 +213,7 @@ def main() -> None:
     ap.add_argument("--variant", type=int, default=0, help="gemv kernel override (0 auto, 1 dot2, 2 mfma)")
     ap.add_argument("--rt", type=int, default=0, help="row tiles per wave for the mfma gemv (0 auto)")
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
+    ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=4096)
     args = ap.parse_args()

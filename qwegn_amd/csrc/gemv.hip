@@ -606,8 +606,12 @@ uint32_t log2_u32(uint32_t v) {
 
 }  // namespace
 
-// flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = mfma);
-// bits 12..15: row tiles per wave for the mfma kernel (0 = automatic).
+// stream.hip
+bool qw_stream_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m, bool rotate,
+                    void* y16, float* y32, uint32_t kw_override, hipError_t* err);
+
+// flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer);
+// bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer (0 = automatic).
 extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                                    uint32_t m, uint32_t flags, void* y16, float* y32) {
     int fmt = 0;
@@ -635,6 +639,17 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     const size_t lds_dot2 = (size_t)(w->k / 32) * 80u;
     const bool dot2_ok = fmt == QW_FMT_M5 && m == 1 && lds_dot2 <= 60u * 1024u;
     if (variant == 1 && !dot2_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "dot2 kernel needs HQ4_G32_M5, m = 1, k <= 24576");
+    // automatic choice: the DMA streamer where it measured faster than the direct-load kernel (few row tiles, short rows,
+    // one or two activation rows), the direct-load kernel otherwise
+    const bool stream_auto = !dot2_ok && m <= 2 && w->n <= 8192 && w->k <= 8192;
+    if (variant == 3 || (variant == 0 && stream_auto)) {
+        hipError_t e = hipSuccess;
+        if (qw_stream_gemv(s->stream, w, x, x_dtype, m, rotate, y16, y32, rt, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+        if (variant == 3) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the DMA streamer does not take this shape");
+    }
     if (variant == 1 || (variant == 0 && dot2_ok)) {
         const uint32_t nbl = qwhip_cdiv(w->k / 32, 32);  // blocks per lane
         const dim3 grid(qwhip_cdiv(w->n, 8u)), block(256);

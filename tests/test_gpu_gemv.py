@@ -93,6 +93,27 @@ def test_gemv_hq4_m1(dev, variant, prerot, n, k):
     assert qo.normalized_error(g16, ref) <= TOL
 
 
+@pytest.mark.parametrize("kw", [0, 2, 4])
+@pytest.mark.parametrize("prerot,xdtype", [(False, "f16"), (False, "bf16"), (True, "f16")])
+@pytest.mark.parametrize("n,k,m", [(256, 5120, 1), (1000, 1024, 1), (72, 128, 2), (300, 2048, 5)])
+def test_gemv_hq4_dma_streamer(dev, kw, prerot, xdtype, n, k, m):
+    """The DMA streamer on HQ4_G32_M5: K-splits, fused rotation, ragged N, a ragged last step (k = 128 is half a step)."""
+    g16, g32, ref = _run_gemv(dev, "hq4_g32_m5", n, k, m, prerot=prerot, xdtype=xdtype, variant=3, rt=kw, outliers=True, seed=n)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["aq4_g32", "hq4_g64", "hq4_g128", "hq8_g32", "hq8_g64"])
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_gemv_blocks_dma_streamer_staged_activations(dev, fmt, m):
+    """Pre-rotated f16 activations, m up to 16: per-step activation panels staged once per workgroup; few workgroups
+    (deep prefetch ring) and many workgroups."""
+    for n, k in [(200, 2048), (4096, 512)]:
+        g16, g32, ref = _run_gemv(dev, fmt, n, k, m, prerot=True, variant=3, seed=m)
+        assert qo.normalized_error(g32, ref) <= 2e-5
+        assert qo.normalized_error(g16, ref) <= TOL
+
+
 @pytest.mark.parametrize("rt", [1, 2, 4])
 @pytest.mark.parametrize("xdtype", ["f16", "bf16"])
 def test_gemv_hq4_mfma_row_tiles_and_dtypes(dev, rt, xdtype):
@@ -136,7 +157,7 @@ def test_gemv_affine_known_answer(dev):
 
 def test_gemv_full_size_decode_config(dev):
     """HQ4_G32 decode GEMV at its benchmark shape (K = 5120, N = 17408, outliers, fused rotation)."""
-    for variant in (1, 2):
+    for variant in (1, 2, 3):
         g16, g32, ref = _run_gemv(dev, "hq4_g32_m5", 17408, 5120, 1, prerot=False, variant=variant, outliers=True, seed=0)
         assert qo.normalized_error(g32, ref) <= 2e-5
         assert qo.normalized_error(g16, ref) <= TOL
