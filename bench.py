@@ -35,26 +35,42 @@ def _fail(msg: str) -> None:
     sys.exit(2)
 
 
-def cpu_baseline_gemv(blocks, x_rot16, bits, group, is_m5, algo_bytes_full, rows_sample):
-    """Reference CPU oracle form on a row sample: dequant whole sample to fp32 (f16-rounded), then sgemv."""
-    from oracle import qworacle as qo
-    sample = blocks[:rows_sample]
-    frac = sample.shape[0] / blocks.shape[0]
+def _oracle_clib():
+    """The oracle's C restatement (built by __graft_entry__.build(); compiled here with gcc when missing)."""
+    from oracle import build_oracle
+    if not build_oracle.LIB.exists():
+        build_oracle.build()
+    return C.CDLL(str(build_oracle.LIB))
+
+
+def cpu_baseline_gemv(blocks, x_basis16, bits, group, is_m5, algo_bytes_full, rows_sample):
+    """Reference CPU oracle form (dequantize the bank to f16-rounded fp32, then one fp32 matrix-vector product:
+    Scripts/oracle/gen_s1_q4_fixtures.py:28-31) in the oracle's C restatement, OpenMP over rows, on a row sample."""
+    lib = _oracle_clib()
+    sample = np.ascontiguousarray(blocks[:rows_sample])
+    n_s, k = sample.shape[0], x_basis16.shape[-1]
+    frac = n_s / blocks.shape[0]
+    x = np.ascontiguousarray(x_basis16.reshape(-1, k)[0]).view(np.uint16)
+    scratch, xf, y = np.empty((n_s, k), np.float32), np.empty(k, np.float32), np.empty(n_s, np.float32)
+    vp = lambda a: a.ctypes.data_as(C.c_void_p)
+
+    def once():
+        if is_m5:
+            lib.qwo_oracle_gemv_hq4(vp(sample), vp(x), C.c_int64(n_s), C.c_int64(k), vp(scratch), vp(xf), vp(y))
+        else:
+            lib.qwo_oracle_gemv_blocks(vp(sample), vp(x), C.c_int64(n_s), C.c_int64(k), bits, group, vp(scratch), vp(xf), vp(y))
+
+    once()
     reps, t_total = 0, 0.0
-    while t_total < 10.0 and reps < 50:
+    while t_total < 10.0 and reps < 200:
         t0 = time.perf_counter()
-        qo.cpu_oracle_gemv(sample, x_rot16, bits, group, is_m5)
+        once()
         t_total += time.perf_counter() - t0
         reps += 1
     sec = t_total / reps
-    try:
-        import threadpoolctl
-        cores = max(int(i.get("num_threads", 1)) for i in threadpoolctl.threadpool_info()) if threadpoolctl.threadpool_info() else 1
-    except Exception:
-        cores = 1
-    return {"value": round(algo_bytes_full * frac / sec / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"{sample.shape[0]} of {blocks.shape[0]} rows, numpy dequant-to-fp32 + fp32 product, "
-                      f"{reps} reps, {sec * 1e3:.1f} ms each"}
+    return {"value": round(algo_bytes_full * frac / sec / 1e9, 3), "unit": "GB/s", "cores": int(lib.qwo_threads()), "kind": "port",
+            "sample": f"{n_s} of {blocks.shape[0]} rows, one activation row, C restatement of the oracle form (dequantize to fp32, "
+                      f"then sgemv; OpenMP), {reps} reps, {sec * 1e3:.1f} ms each"}
 
 
 def run_gemv(args, fmt, n, k, m, label, outliers):
@@ -183,11 +199,162 @@ def run_gemm(args, fmt, n, k, m, label):
     return out
 
 
+class _LazyExpertBank:
+    """Dequantizes one expert's exact f16 weights on demand from the host copy of a bank (oracle side of the parity check)."""
+
+    def __init__(self, blocks, experts, rows, k):
+        self.blocks, self.shape, self._cache = blocks.reshape(experts, rows, k // 32, 20), (experts, rows, k), {}
+
+    def __getitem__(self, e):
+        from oracle import qworacle as qo
+        if e not in self._cache:
+            self._cache[e] = qo.weights_f16_exact(self.blocks[e], 4, 32, True)
+        return self._cache[e]
+
+
+def run_moe(args, t, label):
+    """C4: 128 experts, top-8, hidden 2048, intermediate 768, HQ4_G32 banks.  One step = the whole routed-expert
+    operator on t tokens from router logits to the combined output.  t <= 8: routed GEMVs (HBM bound, bf16 hidden
+    un-rotated, rotation fused); t > 8: pair sort + grouped GEMMs (MFMA bound, f16 hidden in the experts' basis)."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+
+    E, K, Hd, I = 128, 8, 2048, 768
+    dev = qwhip.Device(0)
+    lib, st = dev.lib, dev.stream.handle
+    rng = np.random.default_rng(0)
+    gub, dnb = dev.alloc(E * 2 * I * (Hd // 32) * 20), dev.alloc(E * Hd * (I // 32) * 20)
+    src = dev.alloc(2 * I * Hd * 4)
+    check_e0 = None
+    for e in range(E):                       # banks are written by the device quantizer (byte-identical to the packer)
+        wg = rng.standard_normal((2 * I, Hd), dtype=np.float32) * np.float32(0.02)
+        src.upload(wg)
+        qwhip.check(lib.qwhip_quantize_hq4_g32(st, src.ptr, qwhip.F32, 2 * I, Hd, 1, gub.ptr + e * 2 * I * (Hd // 32) * 20))
+        wd = rng.standard_normal((Hd, I), dtype=np.float32) * np.float32(0.02)
+        src.upload(wd)
+        qwhip.check(lib.qwhip_quantize_hq4_g32(st, src.ptr, qwhip.F32, Hd, I, 1, dnb.ptr + e * Hd * (I // 32) * 20))
+        if e == 0:
+            check_e0 = (wg, wd)
+    dev.stream.sync()
+    gu_blocks = gub.download(np.uint8, (E * 2 * I, Hd // 32, 20))
+    dn_blocks = dnb.download(np.uint8, (E * Hd, I // 32, 20))
+    if not (np.array_equal(gu_blocks[:2 * I], qo.quant_hq4_blocks(check_e0[0])) and np.array_equal(dn_blocks[:Hd], qo.quant_hq4_blocks(check_e0[1]))):
+        _fail("bench: device quantizer bytes differ from the oracle's")
+    vgu = dev.view(gub, E * 2 * I, Hd, qwhip.KIND_HQ4_G32_M5)
+    vdn = dev.view(dnb, E * Hd, I, qwhip.KIND_HQ4_G32_M5)
+
+    x32 = rng.standard_normal((t, Hd), dtype=np.float32)
+    logits = rng.standard_normal((t, E), dtype=np.float32)
+    pairs = t * K
+    lb, ib, wb = dev.put(logits), dev.alloc(pairs * 4), dev.alloc(pairs * 4)
+    act, out = dev.alloc(pairs * I * 2), dev.alloc(t * Hd * 4)
+    decode = t <= 8
+    if decode:
+        xv = qo.round_bf16(x32)
+        xb = dev.put(qo.f32_to_bf16_bits(x32))
+        x_basis = qo.fwht32_ortho(xv).astype(np.float16)
+
+        def gate_up():
+            qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, 0, ib.ptr, t, K, act.ptr))
+
+        def chain():
+            qwhip.check(lib.qwhip_moe_route(st, lb.ptr, t, E, K, 1, 1.0, ib.ptr, wb.ptr))
+            gate_up()
+            qwhip.check(lib.qwhip_moe_down_decode(st, C.byref(vdn), E, act.ptr, ib.ptr, wb.ptr, t, K, None, None, out.ptr, qwhip.F32))
+    else:
+        x_basis = qo.rotate_activation_f16(x32)
+        xb = dev.put(x_basis)
+        mt = max(1, lib.qwhip_moe_max_tiles(E, pairs))
+        off, sp, stok, inv = dev.alloc((E + 1) * 4), dev.alloc(pairs * 4), dev.alloc(pairs * 4), dev.alloc(pairs * 4)
+        te, tr, tc = dev.alloc(mt * 4), dev.alloc(mt * 4), dev.alloc(16)
+        gu_out, dn_out = dev.alloc(pairs * 2 * I * 2), dev.alloc(pairs * Hd * 2)
+
+        def gate_up():
+            qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), E, xb.ptr, qwhip.F16, 0, stok.ptr, off.ptr, te.ptr, tr.ptr, tc.ptr,
+                                                   mt, pairs, gu_out.ptr, qwhip.F16, 0))
+
+        def chain():
+            qwhip.check(lib.qwhip_moe_route(st, lb.ptr, t, E, K, 1, 1.0, ib.ptr, wb.ptr))
+            qwhip.check(lib.qwhip_moe_group_pairs(st, ib.ptr, E, pairs, K, off.ptr, sp.ptr, stok.ptr, inv.ptr, te.ptr, tr.ptr, tc.ptr, 1))
+            gate_up()
+            qwhip.check(lib.qwhip_swiglu_fwht(st, gu_out.ptr, qwhip.F16, act.ptr, pairs, I, 1))
+            qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vdn), E, act.ptr, qwhip.F16, 0, None, off.ptr, te.ptr, tr.ptr, tc.ptr,
+                                                   mt, pairs, dn_out.ptr, qwhip.F16, 0))
+            qwhip.check(lib.qwhip_moe_combine(st, dn_out.ptr, qwhip.F16, inv.ptr, wb.ptr, t, K, Hd, None, None, out.ptr, qwhip.F32))
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        dev.stream.sync()
+        e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+        e0.record(dev.stream)
+        for _ in range(steps):
+            fn()
+        e1.record(dev.stream)
+        dev.stream.sync()
+        return e0.elapsed_ms(e1) * 1e3 / steps
+
+    us_chain = timed(chain, args.steps, args.warmup)
+    us_gu = timed(gate_up, args.steps, max(2, args.warmup // 4))      # the dominant kernel alone, same inputs
+    got = out.download(np.float32, (t, Hd))
+    idx, wts = ib.download(np.int32, (t, K)), wb.download(np.float32, (t, K))
+    ridx, rwts = qo.moe_route(logits, K, True, 1.0)
+    if not (np.array_equal(idx, ridx) and np.allclose(wts, rwts, rtol=1e-5, atol=1e-7)):
+        _fail("bench: routing differs from the oracle's")
+    rows = np.arange(0, t, max(1, t // 6))[:6]
+    ref = qo.moe_forward_f64(x_basis[rows], idx[rows], wts[rows], _LazyExpertBank(gu_blocks, E, 2 * I, Hd),
+                             _LazyExpertBank(dn_blocks, E, Hd, I), act_f16=True, rotate_act=True)
+    err = qo.normalized_error(got[rows], ref)
+    if not err <= 2e-3:
+        _fail(f"bench: MoE output failed parity (normalized error {err:.3e})")
+
+    base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us_chain / 1e3, 6), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)", "normalized_error": err}
+    cfg = {"workload": label, "format": "hq4_g32_m5", "tokens": t, "experts": E, "top_k": K, "hidden": Hd, "intermediate": I}
+    if decode:
+        used = len({int(e) for e in idx.ravel() if e >= 0})
+        w_bytes = used * (2 * I * (Hd // 32) * 20 + Hd * (I // 32) * 20)
+        algo = w_bytes + t * Hd * 2 + t * Hd * 4 + t * E * 4
+        gu_bytes = used * 2 * I * (Hd // 32) * 20 + t * Hd * 2 + pairs * I * 2
+        gbs, gu_gbs = algo / (us_chain * 1e-6) / 1e9, gu_bytes / (us_gu * 1e-6) / 1e9
+        cfg["cache"] = "hot (the routed experts repeat between steps; 23.6 MB of the 377 MB banks per token)"
+        base.update({"value": round(gbs, 2), "unit": "GB/s", "config": cfg,
+                     "roofline": {"bound": "hbm", "kernel": "routed gate_up GEMV", "achieved": round(gu_gbs, 2), "peak": HBM_PEAK_GBS,
+                                  "unit": "GB/s", "frac": round(gu_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                                  "algorithmic_bytes": gu_bytes, "kernel_us": round(us_gu, 3)}})
+    else:
+        valid = int((idx >= 0).sum())
+        flops = valid * (2.0 * 2 * I * Hd + 2.0 * Hd * I)
+        gu_flops = valid * 2.0 * 2 * I * Hd
+        tf, gu_tf = flops / (us_chain * 1e-6) / 1e12, gu_flops / (us_gu * 1e-6) / 1e12
+        base.update({"value": round(tf, 2), "unit": "TFLOP/s", "config": cfg,
+                     "roofline": {"bound": "mfma", "kernel": "grouped gate_up GEMM", "achieved": round(gu_tf, 2), "peak": MFMA_PEAK_TFLOPS,
+                                  "unit": "TFLOP/s", "frac": round(gu_tf / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                                  "algorithmic_flops": gu_flops, "kernel_us": round(us_gu, 3)}})
+    if not args.no_cpu:
+        rows_c = np.arange(min(t, 2))
+        t0 = time.perf_counter()
+        qo.moe_forward_f64(x_basis[rows_c], idx[rows_c], wts[rows_c], _LazyExpertBank(gu_blocks, E, 2 * I, Hd),
+                           _LazyExpertBank(dn_blocks, E, Hd, I), act_f16=True, rotate_act=True)
+        sec = time.perf_counter() - t0
+        per_tok = sec / len(rows_c)
+        if decode:
+            v, u = (K * (2 * I * (Hd // 32) * 20 + Hd * (I // 32) * 20)) / per_tok / 1e9, "GB/s"
+        else:
+            v, u = K * (2.0 * 2 * I * Hd + 2.0 * Hd * I) / per_tok / 1e12, "TFLOP/s"
+        base["cpu_baseline"] = {"value": round(v, 5), "unit": u, "cores": 1, "kind": "port",
+                                "sample": f"{len(rows_c)} token(s): numpy oracle (dequantize the routed experts, fp64 products), {sec:.1f} s"}
+    return base
+
+
 WORKLOADS = {
     # label: (runner kind, fmt, n, k, m, outliers)
     "c1": ("gemv", "aq4_g32", 4096, 4096, 1, False),
     "c2": ("gemv", "hq4_g32_m5", 17408, 5120, 1, True),
     "c3": ("gemm", "hq4_g32_m5", 5120, 5120, 4096, False),
+    "c4_decode": ("moe", None, None, None, 1, False),
+    "c4_prefill": ("moe", None, None, None, 2048, False),
     "c5_qkv": ("gemv", "hq8_g32", 7168, 5120, None, False),
     "c5_down": ("gemv", "hq4_g64", 5120, 17408, None, False),
 }
@@ -195,6 +362,8 @@ LABELS = {
     "c1": "C1 AQ4_G32 affine GEMV N=4096 K=4096",
     "c2": "C2 HQ4_G32 decode GEMV M=1 K=5120 N=17408 fused FWHT",
     "c3": "C3 HQ4_G32 prefill GEMM M=4096 K=5120 N=5120",
+    "c4_decode": "C4 MoE decode T=1 E=128 top-8 H=2048 I=768",
+    "c4_prefill": "C4 MoE prefill T=2048 E=128 top-8 H=2048 I=768",
     "c5_qkv": "C5 verify GEMM HQ8_G32 K=5120 N=7168",
     "c5_down": "C5 verify GEMM HQ4_G64 K=17408 N=5120",
 }
@@ -215,7 +384,7 @@ def main() -> None:
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--cpu-rows", type=int, default=4096)
+    ap.add_argument("--cpu-rows", type=int, default=1 << 30, help="rows of the bank the CPU baseline runs over (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         _fail("bench.py: this build measures one GPU only (every box has one); run with --gpus 1")
@@ -233,7 +402,9 @@ def main() -> None:
     kind, fmt, n, k, m, outliers = WORKLOADS[args.workload]
     if m is None:
         m = args.m
-    if kind == "gemm":
+    if kind == "moe":
+        out = run_moe(args, m, LABELS[args.workload])
+    elif kind == "gemm":
         out = run_gemm(args, fmt, n, k, m, LABELS[args.workload])
     else:
         out = run_gemv(args, fmt, n, k, m, LABELS[args.workload] + (f" M={m}" if args.workload.startswith("c5") else ""), outliers)

@@ -13,6 +13,18 @@
 #include <math.h>
 #include <stdint.h>
 #include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* threads the parallel loops below run on (reported beside the CPU baseline) */
+int qwo_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
 
 /* IEEE binary16 <-> binary32, round to nearest even, subnormals kept (gcc 11 on x86 has no _Float16). */
 static inline float h2f(uint16_t h) {
@@ -167,5 +179,13 @@ void qwo_oracle_gemv_hq4(const uint8_t* blocks, const uint16_t* x_rot_f16, int64
                          float* y) {
     qwo_dequant_hq4_rot(blocks, n, k, 1, scratch);
     for (int64_t c = 0; c < k; ++c) xf[c] = h2f(x_rot_f16[c]);
+    qwo_sgemv(scratch, xf, n, k, y);
+}
+
+/* Same form for a bit-stream container (scratch [n, k] fp32, xf [k] fp32). */
+void qwo_oracle_gemv_blocks(const uint8_t* blocks, const uint16_t* x_f16, int64_t n, int64_t k, int bits, int group,
+                            float* scratch, float* xf, float* y) {
+    qwo_dequant_blocks_rot(blocks, n, k, bits, group, 1, scratch);
+    for (int64_t c = 0; c < k; ++c) xf[c] = h2f(x_f16[c]);
     qwo_sgemv(scratch, xf, n, k, y);
 }

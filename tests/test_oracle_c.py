@@ -72,3 +72,16 @@ def test_c_oracle_gemv_matches_numpy_form(clib):
     np.testing.assert_allclose(y, want, rtol=2e-4, atol=2e-5)
     ref = qo.matmul_ref_f64(x16[None, :], qo.weights_f16_exact(blocks, 4, 32, True))[0]
     assert qo.normalized_error(y, ref) < 1e-5
+
+
+@pytest.mark.parametrize("bits,group,rotate", [(4, 32, False), (8, 32, True), (4, 64, True)])
+def test_c_oracle_gemv_blocks_matches_f64(clib, bits, group, rotate):
+    n, k = 128, 512
+    w = (np.random.default_rng(3).standard_normal((n, k)) * 0.02).astype(np.float32)
+    blocks, _ = qo.quant_hq_blocks(w, bits=bits, group=group, rotate=rotate)
+    x16 = np.random.default_rng(4).standard_normal(k).astype(np.float16)
+    scratch, xf, y = np.empty((n, k), np.float32), np.empty(k, np.float32), np.empty(n, np.float32)
+    clib.qwo_oracle_gemv_blocks(_p(blocks), _p(x16.view(np.uint16)), C.c_int64(n), C.c_int64(k), bits, group, _p(scratch), _p(xf), _p(y))
+    ref = qo.matmul_ref_f64(x16[None, :], qo.weights_f16_exact(blocks, bits, group, False))[0]
+    assert qo.normalized_error(y, ref) < 1e-5
+    assert clib.qwo_threads() >= 1
