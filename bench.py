@@ -29,6 +29,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense f16/bf16 MFMA, published
 
+# HBM bytes per launch of the dominant kernel under its automatic configuration, from rocprofv3 --pmc passes
+# (FETCH_SIZE KiB x 1024 x 2.000 + WRITE_SIZE KiB x 1024 x 1.000; the factors come from a streaming kernel of known
+# size).  The counter passes and the calibration are recorded as text under profiles/.
+MEASURED_TRAFFIC = {"c2": 55_947_878, "c3": 195_355_648}
+
 
 def _fail(msg: str) -> None:
     print(msg, file=sys.stderr)
@@ -62,7 +67,7 @@ def cpu_baseline_gemv(blocks, x_basis16, bits, group, is_m5, algo_bytes_full, ro
 
     once()
     reps, t_total = 0, 0.0
-    while t_total < 10.0 and reps < 200:
+    while t_total < 10.0 and reps < 2000:
         t0 = time.perf_counter()
         once()
         t_total += time.perf_counter() - t0
@@ -73,7 +78,7 @@ def cpu_baseline_gemv(blocks, x_basis16, bits, group, is_m5, algo_bytes_full, ro
                       f"then sgemv; OpenMP), {reps} reps, {sec * 1e3:.1f} ms each"}
 
 
-def run_gemv(args, fmt, n, k, m, label, outliers):
+def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None):
     from oracle import qworacle as qo
     from qwegn_amd import qwhip
     from tests import helpers as H
@@ -128,7 +133,8 @@ def run_gemv(args, fmt, n, k, m, label, outliers):
         "config": {"workload": label, "format": fmt, "M": m, "N": n, "K": k, "fused_fwht": bool(rotate) and not prerot,
                    "cache": "hot" if args.hot else f"cold ring of {ring_n} banks ({ring_n * bank_bytes / 1e6:.0f} MB)"},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": traffic if (args.variant == 0 and args.rt == 0 and not args.prerot) else None,
                      "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
         "normalized_error": err, "wall_ms_per_step": round(wall * 1e3 / args.steps, 6),
     }
@@ -138,7 +144,7 @@ def run_gemv(args, fmt, n, k, m, label, outliers):
     return out
 
 
-def run_gemm(args, fmt, n, k, m, label):
+def run_gemm(args, fmt, n, k, m, label, traffic=None):
     """Prefill GEMM: X bf16 [m, k] in the container's basis -> Y bf16 [m, n]; one step = one launch."""
     from oracle import qworacle as qo
     from qwegn_amd import qwhip
@@ -168,6 +174,18 @@ def run_gemm(args, fmt, n, k, m, label):
     e1.record(dev.stream)
     dev.stream.sync()
     us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    # the GEMM kernel alone (f16 activations already in the workspace, no conversion pass): the roofline's duration
+    def launch_kernel_only():
+        qwhip.check(lib.qwhip_gemm(st, C.byref(view), ws.ptr, qwhip.F16, m, 0, yb.ptr, qwhip.BF16, 0, flags, None, 0))
+
+    launch_kernel_only()
+    dev.stream.sync()
+    e0.record(dev.stream)
+    for _ in range(args.steps):
+        launch_kernel_only()
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_kernel = e0.elapsed_ms(e1) * 1e3 / args.steps
     # parity on a row sample (full-size parity is a test)
     rows = np.arange(0, m, max(1, m // 64))[:64]
     got = qo.bf16_bits_to_f32(yb.download(np.uint16, (m, n)))[rows]
@@ -177,15 +195,17 @@ def run_gemm(args, fmt, n, k, m, label):
         _fail(f"bench: GEMM output failed parity (normalized error {err:.3e})")
     flops = 2.0 * m * n * k
     tf = flops / (us_per * 1e-6) / 1e12
+    tf_k = flops / (us_kernel * 1e-6) / 1e12
     out = {
         "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
         "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": label, "format": fmt, "M": m, "N": n, "K": k, "x": "bf16 (in the weight basis)", "y": "bf16"},
-        "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tf / MFMA_PEAK_TFLOPS, 4), "traffic": None, "algorithmic_flops": flops,
-                     "kernel_us": round(us_per, 3)},
+        "roofline": {"bound": "mfma", "kernel": "quantized GEMM kernel alone (f16 activations; the step adds one bf16->f16 pass)",
+                     "achieved": round(tf_k, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf_k / MFMA_PEAK_TFLOPS, 4), "traffic": traffic if args.cfg == 0 else None,
+                     "algorithmic_flops": flops, "kernel_us": round(us_kernel, 3)},
         "normalized_error": err,
     }
     if not args.no_cpu:
@@ -348,6 +368,30 @@ def run_moe(args, t, label):
     return base
 
 
+def run_calibration(args):
+    """A plain streaming kernel of known size (f32 -> f16 cast of 2^26 elements: reads 256 MiB, writes 128 MiB), the
+    reference point the FETCH_SIZE / WRITE_SIZE counter readings of the other workloads are scaled by."""
+    from qwegn_amd import qwhip
+    dev = qwhip.Device(0)
+    n = 1 << 26
+    src, dst = dev.alloc(n * 4), dev.alloc(n * 2)
+    qwhip.check(dev.lib.qwhip_fill_u32(dev.stream.handle, src.ptr, 0x3F800000, n))
+    for _ in range(args.warmup):
+        qwhip.check(dev.lib.qwhip_cast_f32_to_f16(dev.stream.handle, src.ptr, dst.ptr, n))
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for _ in range(args.steps):
+        qwhip.check(dev.lib.qwhip_cast_f32_to_f16(dev.stream.handle, src.ptr, dst.ptr, n))
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us = e0.elapsed_ms(e1) * 1e3 / args.steps
+    if not np.all(dst.download(np.float16, (1024,)) == np.float16(1.0)):
+        _fail("bench: calibration kernel wrote wrong values")
+    return {"workload": "calibration cast f32->f16", "read_bytes": n * 4, "write_bytes": n * 2, "kernel_us": round(us, 3),
+            "GB/s": round(n * 6 / (us * 1e-6) / 1e9, 1)}
+
+
 WORKLOADS = {
     # label: (runner kind, fmt, n, k, m, outliers)
     "c1": ("gemv", "aq4_g32", 4096, 4096, 1, False),
@@ -374,7 +418,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS) + ["headline"],
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS) + ["headline", "calib"],
                     help="headline = c2 (the bench line) with the c3 prefill GEMM summarised under 'prefill_gemm'")
     ap.add_argument("--m", type=int, default=8, help="activation rows for the c5 workloads")
     ap.add_argument("--hot", action="store_true", help="single bank (Infinity-Cache resident) instead of the cold ring")
@@ -388,13 +432,16 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         _fail("bench.py: this build measures one GPU only (every box has one); run with --gpus 1")
+    if args.workload == "calib":
+        print(json.dumps(run_calibration(args)))
+        return
     if args.workload == "headline":
         kind, fmt, n, k, m, outliers = WORKLOADS["c2"]
-        out = run_gemv(args, fmt, n, k, m, LABELS["c2"], outliers)
+        out = run_gemv(args, fmt, n, k, m, LABELS["c2"], outliers, MEASURED_TRAFFIC["c2"])
         gargs = argparse.Namespace(**vars(args))
         gargs.steps, gargs.warmup, gargs.no_cpu = max(10, args.steps // 10), max(3, args.warmup // 4), True
         kind, fmt, n, k, m, outliers = WORKLOADS["c3"]
-        g = run_gemm(gargs, fmt, n, k, m, LABELS["c3"])
+        g = run_gemm(gargs, fmt, n, k, m, LABELS["c3"], MEASURED_TRAFFIC["c3"])
         out["prefill_gemm"] = {"value": g["value"], "unit": g["unit"], "ms_per_step": g["ms_per_step"], "steps": g["steps"],
                                "config": g["config"], "roofline": g["roofline"], "normalized_error": g["normalized_error"]}
         print(json.dumps(out))
@@ -405,9 +452,10 @@ def main() -> None:
     if kind == "moe":
         out = run_moe(args, m, LABELS[args.workload])
     elif kind == "gemm":
-        out = run_gemm(args, fmt, n, k, m, LABELS[args.workload])
+        out = run_gemm(args, fmt, n, k, m, LABELS[args.workload], MEASURED_TRAFFIC.get(args.workload))
     else:
-        out = run_gemv(args, fmt, n, k, m, LABELS[args.workload] + (f" M={m}" if args.workload.startswith("c5") else ""), outliers)
+        out = run_gemv(args, fmt, n, k, m, LABELS[args.workload] + (f" M={m}" if args.workload.startswith("c5") else ""), outliers,
+                       MEASURED_TRAFFIC.get(args.workload))
     print(json.dumps(out))
 
 
