@@ -37,71 +37,6 @@ __device__ __forceinline__ void qw_stage_group(const void* x, uint64_t elem0, bo
 }
 
 // ------------------------------------------------------------------------------------------------
-// FWHT-32 on the matrix cores.  For 16 consecutive 32-groups, rot[g][i] = sum_k H[i][k] x[g][k] is one
-// 16x16x32 MFMA per half of the outputs: A = H rows (entries +-1, exact in f16), B = the activations
-// (column j = group, lane (j, c) holds x[g_j][8c .. 8c+7] straight from one 16-byte load), fp32
-// accumulate; the 1/sqrt(32) is applied in fp32 afterwards and the result is rounded once to f16.
-// The products are exact and the sum is an fp32 sum of 32 terms, so the result can differ from the
-// butterfly order only in the last fp32 bit before the f16 rounding.  VALU cost per wave and 16
-// groups: ~20 instructions instead of ~260 for the in-register butterflies, and the work spreads
-// over all four SIMDs of the workgroup.
-// ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ h8_t qw_hadamard_rows(uint32_t i, uint32_t c) {
-    // H[i][8c + e], e = 0..7: sign = parity(i & (8c + e)) = parity(i & 8c) ^ parity(i & e)
-    const uint32_t pc = __popc(i & (8u * c)) & 1u;
-    u4_t bits;
-#pragma unroll
-    for (int pr = 0; pr < 4; ++pr) {
-        const uint32_t p0 = (pc ^ __popc(i & (uint32_t)(2 * pr))) & 1u;
-        const uint32_t p1 = (pc ^ __popc(i & (uint32_t)(2 * pr + 1))) & 1u;
-        bits[pr] = (0x3C00u | (p0 << 15)) | ((0x3C00u | (p1 << 15)) << 16);
-    }
-    return __builtin_bit_cast(h8_t, bits);
-}
-
-template <int XDT>
-__device__ __forceinline__ h8_t qw_load_x8_f16(const void* x, uint64_t elem) {
-    if constexpr (XDT == QWHIP_F16) {
-        return *(const h8_t*)((const h1_t*)x + elem);
-    } else {
-        const u4_t raw = *(const u4_t*)((const uint16_t*)x + elem);
-        h8_t o;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            o[2 * j] = (h1_t)__uint_as_float(raw[j] << 16);
-            o[2 * j + 1] = (h1_t)__uint_as_float(raw[j] & 0xFFFF0000u);
-        }
-        return o;
-    }
-}
-
-// Rotates (or just converts) the 16 groups of tile `gt` from the operand `xb` this lane loaded and writes
-// them to LDS (80-byte pitch per group).
-__device__ __forceinline__ void qw_rotate_tile_to_lds(h8_t xb, uint32_t gt, uint32_t nb, uint32_t lane, bool rotate,
-                                                      h8_t h_lo, h8_t h_hi, h8_t* xs) {
-    const uint32_t j = lane & 15u, c = lane >> 4;
-    const uint32_t g = gt * 16u + j;
-    h1_t* base = (h1_t*)xs + (uint64_t)g * 40u;
-    if (rotate) {
-        f4_t d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
-        d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(h_lo, xb, d0, 0, 0, 0);
-        d1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(h_hi, xb, d1, 0, 0, 0);
-        if (g < nb) {
-            h4_t o0, o1;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                o0[r] = (h1_t)(d0[r] * QW_INV_SQRT32);
-                o1[r] = (h1_t)(d1[r] * QW_INV_SQRT32);
-            }
-            *(h4_t*)(base + 4u * c) = o0;
-            *(h4_t*)(base + 16u + 4u * c) = o1;
-        }
-    } else if (g < nb) {
-        *(h8_t*)(base + 8u * c) = xb;
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // Variant A: HQ4_G32_M5, m = 1, dot2.
 // Order of issue matters more than instruction count here: the whole kernel is one "breath" of about
 // ten microseconds, loads return in order, and nothing can be contracted before the rotated activation
@@ -610,8 +545,14 @@ uint32_t log2_u32(uint32_t v) {
 bool qw_stream_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m, bool rotate,
                     void* y16, float* y32, uint32_t kw_override, hipError_t* err);
 
-// flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer);
-// bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer (0 = automatic).
+// gemv_col.hip
+bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
+                 float* y32, uint32_t tune, hipError_t* err);
+
+// flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer,
+// 4 = column-stationary persistent kernel);
+// bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer / tuning code of the
+// column-stationary kernel (0 = automatic).
 extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                                    uint32_t m, uint32_t flags, void* y16, float* y32) {
     int fmt = 0;
@@ -649,6 +590,14 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
             return QWHIP_OK;
         }
         if (variant == 3) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the DMA streamer does not take this shape");
+    }
+    if (variant == 4 || (variant == 0 && fmt == QW_FMT_M5 && m == 1)) {
+        hipError_t e = hipSuccess;
+        if (fmt == QW_FMT_M5 && m == 1 && qw_col_gemv(s->stream, w, x, x_dtype, rotate, y16, y32, rt, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+        if (variant == 4) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the column-stationary kernel needs HQ4_G32_M5, m = 1, k <= 24576");
     }
     if (variant == 1 || (variant == 0 && dot2_ok)) {
         const uint32_t nbl = qwhip_cdiv(w->k / 32, 32);  // blocks per lane

@@ -1,0 +1,230 @@
+// Decode GEMV (m = 1) over an HQ4_G32_M5 bank, column-stationary persistent form.
+//
+// The launch is a fixed population of workgroups that together walk the bank once, top to bottom: row slot s of
+// workgroup w is bank row s * gridDim.x + w, so at any moment the whole grid is fetching one contiguous band of rows
+// (what the HBM channels like) and every workgroup has the same number of rows to within one.
+//
+// Inside a workgroup a 32-lane half-wavefront (set, chunk) owns block columns 32*chunk .. 32*chunk + 31 of the rows
+// set, set + SETS, ... of the workgroup.  A lane therefore multiplies the same 32 activations for the whole kernel and
+// keeps them in registers (16 packed pairs); the main loop has no LDS reads, only a rolling window of D block loads
+// per lane, the nibble unpack, 16 v_dot2_f32_f16 and a half-wave reduction per row.
+//
+// Arithmetic.  A block dequantizes as w = (1024 + q) * s + b (unpack_hq4_word8, Sources/QWMetal/include/
+// qw_dequant.metalh:42-62).  The kernel never forms w: the masked nibble pairs are used directly as f16 operands -
+// bits 0..3 / 16..19 of a word read as two f16 subnormals q * 2^-24, bits 4..7 / 20..23 as 16 q * 2^-24
+// (v_dot2_f32_f16 honours f16 subnormals; products are exact, accumulation is fp32) - and the affine part is applied once
+// per block:  sum_i w_i x_i = s * (sum_i q_i x_i + 1024 S) + b * S,  S = sum_i x_i,
+// the same factorisation the reference's bit-stream GEMVs use (qwg_aq_slice_dot, qw_dequant_multi.metalh:205-208).
+// The activations are the f16-rounded rotated values the reference's producers would have stored.
+#include "qwhip_common.h"
+
+namespace {
+
+// Rows i and i + 16 (i = lane & 15) of the 32-point Hadamard matrix, columns 8c .. 8c + 7 (c = lane >> 4), as f16 +-1:
+// sign(i, k) = parity(i & k); for i < 16 that is parity(i & 8c) ^ parity(i & e) with only bit 3 of i meeting 8c, and
+// row i + 16 flips the sign where k >= 16.
+__device__ __forceinline__ void qc_hadamard_pair(uint32_t i, uint32_t c, h8_t& lo, h8_t& hi) {
+    const uint32_t b0 = i & 1u, b1 = (i >> 1) & 1u, b2 = (i >> 2) & 1u;
+    const uint32_t pc = (c & 1u) & ((i >> 3) & 1u);
+    const uint32_t s0 = pc, s1 = pc ^ b0, s2 = pc ^ b1, s3 = s1 ^ b1, s4 = pc ^ b2, s5 = s1 ^ b2, s6 = s2 ^ b2, s7 = s3 ^ b2;
+    u4_t w;
+    w[0] = 0x3C003C00u | (s0 << 15) | (s1 << 31);
+    w[1] = 0x3C003C00u | (s2 << 15) | (s3 << 31);
+    w[2] = 0x3C003C00u | (s4 << 15) | (s5 << 31);
+    w[3] = 0x3C003C00u | (s6 << 15) | (s7 << 31);
+    lo = __builtin_bit_cast(h8_t, w);
+    const uint32_t flip = (c >= 2u) ? 0x80008000u : 0u;
+    const u4_t v = {w[0] ^ flip, w[1] ^ flip, w[2] ^ flip, w[3] ^ flip};
+    hi = __builtin_bit_cast(h8_t, v);
+}
+
+// Sum over each aligned 32-lane half; the result is valid in lanes 16..31 (half 0) and 48..63 (half 1).
+__device__ __forceinline__ float qc_reduce32(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, true));  // row_bcast15 into rows 1, 3
+    return v;
+}
+
+struct qc_params {
+    const uint8_t* bank;
+    const void* x;
+    h1_t* y16;
+    float* y32;
+    uint32_t N, nb, cpr, rotate;
+};
+
+// SETS row sets per workgroup, D blocks in flight per lane, D0 of them issued before the activation prologue.
+// blockDim.x = 32 * cpr * SETS; dynamic LDS = nb * 80 + rows-per-workgroup * cpr * 4 bytes.
+template <int XDT, int SETS, int D, int D0>
+__global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
+    constexpr int XT = SETS == 1 ? 4 : (SETS == 2 ? 2 : 1);   // 16-group activation tiles per wave: ceil(2 cpr / waves)
+    extern __shared__ h8_t qc_lds[];
+    const uint32_t nb = p.nb, cpr = p.cpr, N = p.N;
+    h8_t* xs = qc_lds;                                 // 80 bytes per 32-group (64 used)
+    float* part = (float*)(qc_lds + (size_t)nb * 5);   // [row slot][chunk] partial sums
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 31u, hw = tid >> 5;
+    const uint32_t wave = tid >> 6, l64 = tid & 63u;
+    const uint32_t nw = (blockDim.x + 63u) >> 6;
+    const uint32_t set = hw / cpr, chunk = hw - set * cpr;
+    const uint32_t g0 = chunk * 32u + lane;
+    const bool gvalid = g0 < nb;
+    const uint32_t g = gvalid ? g0 : nb - 1u;
+    const uint32_t G = gridDim.x;
+    if (blockIdx.x >= N) return;
+    const uint32_t nrows = (N - blockIdx.x + G - 1u) / G;   // row slots of this workgroup
+    const uint32_t nmax = (nrows + SETS - 1u) / SETS;        // trip count, uniform over the workgroup
+    const uint32_t row_bytes = nb * 20u;
+    const uint32_t step = G * SETS * row_bytes;              // bytes between consecutive rows of one set
+    const uint32_t mine = nrows > set ? (nrows - set + SETS - 1u) / SETS : 0u;
+    uint32_t off = ((mine ? set : 0u) * G + blockIdx.x) * row_bytes + g * 20u;
+    const uint32_t off_max = off + (mine ? mine - 1u : 0u) * step;   // loads past the set's last row re-read it
+
+    // 1. activation loads go first: loads return in order, and the rotation must not queue behind the weight prefetch
+    h8_t xv[XT];
+#pragma unroll
+    for (int t = 0; t < XT; ++t) {
+        const uint32_t gt = wave + nw * t;
+        const uint32_t gg = min(gt * 16u + (l64 & 15u), nb - 1u);
+        xv[t] = qw_load_x8_f16<XDT>(p.x, (uint64_t)gg * 32u + 8u * (l64 >> 4));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // 2. first weight rows
+    qw_hq4_block buf[D];
+    auto issue = [&](int slot) {
+        buf[slot] = *(const qw_hq4_block*)(p.bank + off);
+        off = min(off + step, off_max);
+    };
+#pragma unroll
+    for (int j = 0; j < D0; ++j) issue(j);
+    __builtin_amdgcn_sched_barrier(0);
+    // 3. rotation on the matrix cores into the shared image
+    {
+        h8_t h_lo, h_hi;
+        qc_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
+#pragma unroll
+        for (int t = 0; t < XT; ++t) qw_rotate_tile_to_lds(xv[t], wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs);
+    }
+    __syncthreads();
+    // 4. this lane's column: 16 operand pairs and the group sum S
+    h2_t xo[16];
+    float S;
+    {
+        const h8_t* src = xs + g * 5;
+        const h2_t one = {(h1_t)1.0f, (h1_t)1.0f};
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const h8_t v = src[j];
+#pragma unroll
+            for (int e2 = 0; e2 < 4; ++e2) {
+                const h2_t pr = {v[2 * e2], v[2 * e2 + 1]};
+                if (e2 & 1) s1 = __builtin_amdgcn_fdot2(pr, one, s1, false);
+                else s0 = __builtin_amdgcn_fdot2(pr, one, s0, false);
+                xo[4 * j + e2] = pr;
+            }
+        }
+        S = s0 + s1;
+    }
+    const float c1 = 1024.0f * S;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = D0; j < D; ++j) issue(j);
+    __builtin_amdgcn_sched_barrier(0);
+
+    uint32_t rslot = set;   // row slot being consumed
+    for (uint32_t ib = 0; ib < nmax; ib += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            if (ib + j >= nmax) break;
+            const qw_hq4_block b = buf[j];
+            float lo0 = 0.f, lo1 = 0.f, hi0 = 0.f, hi1 = 0.f;
+#pragma unroll
+            for (int w4 = 0; w4 < 4; ++w4) {
+                const uint32_t w = b.qs[w4], w8 = w >> 8;
+                const uint32_t m0 = w & 0x000F000Fu, m1 = w & 0x00F000F0u, m2 = w8 & 0x000F000Fu, m3 = w8 & 0x00F000F0u;
+                lo0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m0), xo[4 * w4 + 0], lo0, false);
+                hi0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m1), xo[4 * w4 + 1], hi0, false);
+                lo1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m2), xo[4 * w4 + 2], lo1, false);
+                hi1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m3), xo[4 * w4 + 3], hi1, false);
+            }
+            issue(j);
+            const h2_t hd = __builtin_bit_cast(h2_t, b.hdr);
+            float q = __builtin_fmaf(lo0 + lo1, 16777216.0f, c1);   // sum q x + 1024 S
+            q = __builtin_fmaf(hi0 + hi1, 1048576.0f, q);
+            float v = __builtin_fmaf((float)hd[0], q, (float)hd[1] * S);
+            v = gvalid ? v : 0.0f;
+            v = qc_reduce32(v);
+            if (lane == 31u && rslot < nrows) part[rslot * cpr + chunk] = v;
+            rslot += SETS;
+        }
+    }
+    __syncthreads();
+    // 5. fixed-order sum of the chunk partials of each row
+    for (uint32_t s = tid; s < nrows; s += blockDim.x) {
+        float v = 0.f;
+        for (uint32_t c = 0; c < cpr; ++c) v += part[s * cpr + c];
+        const uint32_t row = s * G + blockIdx.x;
+        if (p.y32) p.y32[row] = v;
+        if (p.y16) p.y16[row] = (h1_t)v;
+    }
+}
+
+template <int XDT, int SETS>
+hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t threads, size_t lds, uint32_t depth) {
+    if (depth == 2) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 1>), dim3(wgs), dim3(threads), lds, st, p);
+    else if (depth == 4) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 4, 1>), dim3(wgs), dim3(threads), lds, st, p);
+    else hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 3, 1>), dim3(wgs), dim3(threads), lds, st, p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// Tries the column-stationary kernel for a validated m = 1 HQ4_G32_M5 call; false when the shape is outside its envelope.
+// `tune`: 0 = automatic; else bits 0..1 pick the prefetch depth (1 -> 2, 2 -> 3, 3 -> 4) and bits 2..3 scale the grid
+// (1 -> half, 2 -> double).
+bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
+                 float* y32, uint32_t tune, hipError_t* err) {
+    if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
+    const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u;
+    if (cpr > 32u) return false;
+    if ((uint64_t)w->n * nb * 20u >= (1ull << 32)) return false;   // 32-bit offsets inside the bank
+    if (((uintptr_t)x & 15u) != 0) return false;
+    const uint32_t sets = cpr <= 3u ? 4u : (cpr <= 12u ? 2u : 1u);
+    const uint32_t threads = 32u * cpr * sets;
+    const uint32_t waves = (threads + 63u) / 64u;
+    // about 20 waves per compute unit, at least four rows per set, at most 128 row slots per workgroup
+    uint32_t wgs = (256u * 20u + waves / 2u) / waves;
+    if ((tune >> 2 & 3u) == 1u) wgs /= 2u;
+    if ((tune >> 2 & 3u) == 2u) wgs *= 2u;
+    wgs = min(wgs, max(1u, w->n / (sets * 4u)));
+    wgs = max(wgs, qwhip_cdiv(w->n, 128u));
+    const uint32_t rows_per_wg = qwhip_cdiv(w->n, wgs);
+    const size_t lds = (size_t)nb * 80u + (size_t)rows_per_wg * cpr * 4u;
+    if (lds > 60u * 1024u) return false;
+    const uint32_t depth = (tune & 3u) ? (tune & 3u) + 1u : 2u;
+    qc_params p;
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = x;
+    p.y16 = (h1_t*)y16;
+    p.y32 = y32;
+    p.N = w->n;
+    p.nb = nb;
+    p.cpr = cpr;
+    p.rotate = rotate ? 1u : 0u;
+    hipError_t e;
+    if (x_dtype == QWHIP_F16) {
+        e = sets == 4 ? qc_launch<QWHIP_F16, 4>(st, p, wgs, threads, lds, depth)
+          : sets == 2 ? qc_launch<QWHIP_F16, 2>(st, p, wgs, threads, lds, depth)
+                      : qc_launch<QWHIP_F16, 1>(st, p, wgs, threads, lds, depth);
+    } else {
+        e = sets == 4 ? qc_launch<QWHIP_BF16, 4>(st, p, wgs, threads, lds, depth)
+          : sets == 2 ? qc_launch<QWHIP_BF16, 2>(st, p, wgs, threads, lds, depth)
+                      : qc_launch<QWHIP_BF16, 1>(st, p, wgs, threads, lds, depth);
+    }
+    *err = e;
+    return true;
+}
