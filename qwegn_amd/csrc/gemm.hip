@@ -19,6 +19,7 @@
 // Grouped launches (MoE) take the tile list of the pair sort: tile t = (expert e, row block) over the
 // expert-major slot range [expert_off[e], expert_off[e+1]); slot rows are gathered through `gather`.
 #include "qwhip_common.h"
+#include "qw_mfma_2x5.h"
 
 enum { QG_FMT_M5 = 0, QG_FMT_B4 = 1, QG_FMT_B8 = 2 };
 
@@ -38,6 +39,7 @@ struct qw_gemm_params {
     const int32_t* tile_r;
     const int32_t* tile_count;
     uint32_t rows_per_expert;
+    uint32_t force_gemm2;  // tuning / tests: keep the DMA-fed kernel for the 256 x 320 shape
 #ifdef QW_GEMM_TIMING
     unsigned long long* tlog;  // probe builds only: per-phase cycle stamps of workgroup 0, wave 0
 #endif
@@ -491,6 +493,263 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 }
 
 // ------------------------------------------------------------------------------------------------
+// Ping-pong kernel (f16 activations, 8 waves): the waves of a workgroup form two groups of four, one wave of each group
+// per SIMD.  Every K-step both groups read tile k from one LDS stage and write tile k+1 into the other, but in opposite
+// order: group 0 multiplies first and fills afterwards, group 1 fills first and multiplies afterwards, so for most of a
+// K-step one wave of each SIMD feeds the matrix pipe while the other dequantizes.  One barrier per K-step.  Activations
+// and packed weights travel global -> registers one K-step ahead (loads issued before the MFMAs, consumed after them).
+// The MFMA phase of the 2 x 5 fragment wave tile is hand-scheduled (qw_mfma_2x5.h).
+// ------------------------------------------------------------------------------------------------
+
+#define QG3_BAR_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#define QG3_BAR_ALL() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED>
+__global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_params p) {
+    static_assert(WVM * WVN == 8, "two groups of four waves");
+    constexpr int NT = WVM * WVN * 64;
+    constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 64;
+    constexpr int B_ITEMS = BN * 2;
+    constexpr int B_PER = (B_ITEMS + NT - 1) / NT;
+    constexpr uint32_t A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds2[];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u;
+    const uint32_t wm = wave / WVN, wn = wave % WVN;
+    const uint32_t group = wave >> 2;
+
+    uint32_t m0, n0, rows_valid;
+    const uint8_t* bank = p.bank;
+    if constexpr (GROUPED) {
+        const uint32_t t = blockIdx.y;
+        if ((int32_t)t >= p.tile_count[0]) return;
+        const uint32_t e = (uint32_t)p.tile_e[t];
+        const uint32_t packed = (uint32_t)p.tile_r[t];
+        const uint32_t code = packed >> 24;
+        const uint32_t bm = code == 1u ? 16u : (code == 2u ? 32u : 64u);
+        const uint32_t start = (uint32_t)p.expert_off[e] + (packed & 0xFFFFFFu) * bm;
+        const uint32_t end = (uint32_t)p.expert_off[e + 1];
+        m0 = start;
+        rows_valid = min((uint32_t)BM, min(bm, end - start));
+        n0 = blockIdx.x * BN;
+        bank += (uint64_t)e * p.rows_per_expert * p.row_bytes;
+    } else {
+        const uint32_t total = p.tiles_m * p.tiles_n;
+        const uint32_t per_xcd = (total + 7u) / 8u;
+        const uint32_t label = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (label >= total) return;
+        constexpr uint32_t G = 4;
+        const uint32_t band = label / (G * p.tiles_n);
+        const uint32_t band_rows = min(G, p.tiles_m - band * G);
+        const uint32_t in_band = label - band * G * p.tiles_n;
+        const uint32_t tm = band * G + in_band % band_rows;
+        const uint32_t tn = in_band / band_rows;
+        m0 = tm * BM;
+        n0 = tn * BN;
+        rows_valid = min((uint32_t)BM, p.M - m0);
+    }
+
+    // ---- activation tile: chunk c = tid + i * NT -> tile row (tid >> 3) + (NT / 8) * i, 16-byte k-chunk tid & 7.
+    // Global -> registers one K-step ahead (coalesced 128-byte rows), registers -> LDS slot (k-chunk ^ ((row >> 1) & 7)).
+    // Dense: one per-thread offset, the row block (NT / 8 rows) is a wave-uniform term; blocks past the tile's rows
+    // re-read block 0 (their outputs are never stored), so M must be a multiple of NT / 8 = 64.
+    constexpr int A_LD = BM * 8 / NT;
+    static_assert((BM * 8) % NT == 0, "activation tile must split evenly over the workgroup");
+    constexpr uint32_t A_BLK = NT / 8;
+    uint32_t a_voff[GROUPED ? A_LD : 1];
+    const uint32_t a_lds0 = (tid >> 3) * 128u + (((tid & 7u) ^ ((tid >> 4) & 7u)) << 4);   // + i * A_BLK * 128 (swizzle key unchanged)
+    if constexpr (GROUPED) {
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) {
+            const uint32_t row = (tid >> 3) + A_BLK * i;
+            const uint32_t r = row < rows_valid ? row : rows_valid - 1;
+            const uint32_t src_row = p.gather ? (uint32_t)p.gather[m0 + r] : m0 + r;
+            a_voff[i] = src_row * p.ldx * 2u + (tid & 7u) * 16u;    // activations < 4 GiB (checked by the launcher)
+        }
+    } else {
+        a_voff[0] = (tid >> 3) * p.ldx * 2u + (tid & 7u) * 16u;
+    }
+    const uint64_t a_tile_base = GROUPED ? 0ull : (uint64_t)m0 * p.ldx * 2u;
+    const uint64_t a_blk_stride = (uint64_t)A_BLK * p.ldx * 2u;
+    const uint32_t a_blocks = rows_valid / A_BLK;
+
+    // ---- weight tile: item = (tile row, 32-column slice); thread items tid and NT + (tid % (B_ITEMS - NT)) (items past
+    // the tile are done redundantly by several threads: identical bytes to the same slot) ----
+    static_assert(B_ITEMS >= NT && B_ITEMS <= NT + NT / 2, "the second weight items are covered by group 0 alone");
+    uint32_t b_off32[B_PER], b_meta[B_PER];   // byte offset of the row inside the tile's bank rows; LDS row offset | swizzle key << 16 | slice << 20
+    const uint8_t* b_tile = bank + (uint64_t)n0 * p.row_bytes;
+#pragma unroll
+    for (int i = 0; i < B_PER; ++i) {
+        const uint32_t it = i == 0 ? tid : NT + (B_ITEMS > NT ? tid % (uint32_t)(B_ITEMS > NT ? B_ITEMS - NT : 1) : 0u);
+        const uint32_t nl = it >> 1;
+        const uint32_t n = min(n0 + nl, p.N - 1u) - n0;
+        b_off32[i] = n * (uint32_t)p.row_bytes;                     // a tile's rows span < 4 GiB
+        b_meta[i] = (nl * 128u) | (((nl >> 1) & 7u) << 16) | ((it & 1u) << 20);
+    }
+
+    f16_t acc[WM][WN];
+#pragma unroll
+    for (int a = 0; a < WM; ++a)
+#pragma unroll
+        for (int b = 0; b < WN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    const uint32_t nk = p.K / BK;
+
+    auto load_a = [&](uint32_t kt, u4_t* a_reg) {
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) {
+            if constexpr (GROUPED) {
+                a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
+            } else {
+                const uint32_t blk = (uint32_t)i < a_blocks ? (uint32_t)i : 0u;
+                a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + blk * a_blk_stride + (uint64_t)kt * 128u + a_voff[0]);
+            }
+        }
+    };
+    auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) *(u4_t*)(lds2 + stage * STAGE + a_lds0 + i * (A_BLK * 128u)) = a_reg[i];
+    };
+    auto load_b = [&](uint32_t kt, qg_slice<FMT>* b_reg, int nitems) {
+#pragma unroll
+        for (int i = 0; i < B_PER; ++i) if (i < nitems) qg_load_slice<FMT>(b_tile + b_off32[i], kt * 2u + (b_meta[i] >> 20), p.gshift, p.bb, b_reg[i]);
+    };
+    auto store_b = [&](uint32_t stage, const qg_slice<FMT>* b_reg, int nitems) {
+#pragma unroll
+        for (int i = 0; i < B_PER; ++i) {
+            if (i >= nitems) break;
+            const h2_t s2 = qw_splat_lo(b_reg[i].hdr), b2 = qw_splat_hi(b_reg[i].hdr);
+            uint8_t* row = lds2 + stage * STAGE + A_BYTES + (b_meta[i] & 0xFFFFu);
+            const uint32_t sw = (b_meta[i] >> 16) & 7u, sl4 = (b_meta[i] >> 20) * 4u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *(h8_t*)(row + (((sl4 + j) ^ sw) * 16u)) = qg_dequant_chunk<FMT>(b_reg[i], j, s2, b2, magic);
+        }
+    };
+
+    const uint32_t fr_row = lane & 31u, fr_sw = (fr_row >> 1) & 7u, k_half = lane >> 5;
+    // byte address of (row, 16-byte slot) = row * 128 + ((2 ks + k_half) ^ fr_sw) * 16 = (row * 128 | t) ^ (32 ks), t = (k_half ^ fr_sw) * 16
+    const uint32_t a_bt = (wm * WM * 32 + fr_row) * 128u + ((k_half ^ fr_sw) << 4);
+    const uint32_t b_bt = A_BYTES + (wn * WN * 32 + fr_row) * 128u + ((k_half ^ fr_sw) << 4);
+
+    // MFMAs of one K-step.  Operands of sub-step ks+1 are fetched while sub-step ks runs: the activation fragments are
+    // double-buffered, each weight fragment is reloaded right after the two MFMAs that consume it (b-major order), so
+    // every LDS read has ten MFMAs of distance to its use.
+    auto mfma_step = [&](const uint8_t* st_base) {
+        if constexpr (WM == 2 && WN == 5) {
+            const uint32_t sb = (uint32_t)(st_base - lds2);
+            qg3_mfma_2x5(acc, a_bt + sb + (uint32_t)(uintptr_t)lds2, b_bt + sb + (uint32_t)(uintptr_t)lds2);
+            return;
+        }
+        h8_t af[2][WM], bf[WN];
+        {
+            #pragma unroll
+            for (int a = 0; a < WM; ++a) af[0][a] = *(const h8_t*)(st_base + a_bt + a * 4096);
+#pragma unroll
+            for (int b = 0; b < WN; ++b) bf[b] = *(const h8_t*)(st_base + b_bt + b * 4096);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            const uint32_t a_nx = a_bt ^ (32u * (ks + 1)), b_nx = b_bt ^ (32u * (ks + 1));
+            if (ks < 3) {
+#pragma unroll
+                for (int a = 0; a < WM; ++a) af[nxt][a] = *(const h8_t*)(st_base + a_nx + a * 4096);
+                __builtin_amdgcn_sched_group_barrier(0x100, WM, 0);
+            }
+#pragma unroll
+            for (int b = 0; b < WN; ++b) {
+#pragma unroll
+                for (int a = 0; a < WM; ++a)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][a], bf[b], acc[a][b], 0, 0, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, WM, 0);
+                if (ks < 3) {
+                    bf[b] = *(const h8_t*)(st_base + b_nx + b * 4096);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+            }
+        }
+    };
+
+    // ---- prologue: stage 0 ----
+    {
+        qg_slice<FMT> b_reg[B_PER];
+        u4_t a_reg[A_LD];
+        load_a(0, a_reg);
+        load_b(0, b_reg, B_PER);
+        store_a(0, a_reg);
+        store_b(0, b_reg, B_PER);
+    }
+    QG3_BAR_ALL();
+
+    const uint32_t last = nk - 1u;
+    // Both groups run  { load tile k+1 (group 0) / k+2 (group 1) into registers; MFMAs of step k; barrier; registers -> LDS
+    // stage; barrier }, group 1 half a K-step behind group 0: while one group multiplies, the other fills the next stage.
+    if (group == 0) {
+        for (uint32_t kt = 0; kt < nk; ++kt) {
+            qg_slice<FMT> b_reg[B_PER];
+            u4_t a_reg[A_LD];
+            load_a(min(kt + 1u, last), a_reg);
+            load_b(min(kt + 1u, last), b_reg, B_PER);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(3);
+            mfma_step(lds2 + (kt & 1u) * STAGE);
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+            store_a((kt + 1u) & 1u, a_reg);
+            store_b((kt + 1u) & 1u, b_reg, B_PER);
+            QG3_BAR_LDS();
+        }
+    } else {
+        {
+            qg_slice<FMT> b_reg[B_PER];
+            u4_t a_reg[A_LD];
+            load_a(min(1u, last), a_reg);
+            load_b(min(1u, last), b_reg, 1);
+            store_a(1u, a_reg);
+            store_b(1u, b_reg, 1);
+        }
+        for (uint32_t kt = 0; kt < nk; ++kt) {
+            qg_slice<FMT> b_reg[B_PER];
+            u4_t a_reg[A_LD];
+            load_a(min(kt + 2u, last), a_reg);
+            load_b(min(kt + 2u, last), b_reg, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(3);
+            mfma_step(lds2 + (kt & 1u) * STAGE);
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+            QG3_BAR_LDS();
+            if (kt + 1u < nk) {
+                store_a(kt & 1u, a_reg);         // stage (k+2)&1
+                store_b(kt & 1u, b_reg, 1);
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+#pragma unroll
+    for (int a = 0; a < WM; ++a) {
+#pragma unroll
+        for (int b = 0; b < WN; ++b) {
+            const uint32_t n = n0 + (wn * WN + b) * 32 + (lane & 31u);
+            if (n < p.N) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -531,6 +790,21 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT>
+hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
+    constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
+    constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, false>;
+    static bool attr_done = false;  // per instantiation
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(WVM * WVN * 64), lds, st, p);
+    return hipGetLastError();
+}
+
 // tile shapes of the pipelined kernel
 enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_256x128 = 3, CFG_COUNT = 4 };
 static const uint32_t kCfgBM[CFG_COUNT] = {256, 256, 128, 256};
@@ -543,7 +817,10 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     const uint32_t total = p.tiles_m * p.tiles_n;
     const dim3 grid(((total + 7u) / 8u) * 8u);
     switch (cfg) {
-        case CFG_256x320: return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
+        case CFG_256x320:
+            // the ping-pong kernel takes whole 64-row activation blocks; ragged M stays on the DMA-fed kernel
+            if (p.M % 64u == 0 && !p.force_gemm2) return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
+            return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x256: return launch_cfg2<2, 4, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x128: return launch_cfg2<2, 2, 4, 2, FMT, YDT, false>(st, p, grid);
         default: return launch_cfg2<2, 2, 2, 2, FMT, YDT, false>(st, p, grid);
@@ -611,7 +888,8 @@ qwhip_status gemm_checks(qwhip_stream_t s, const qwhip_weight_view* w, const voi
 
 }  // namespace
 
-// flags bits 8..11: tile shape override for tuning and tests (0 = automatic, 1 + CFG_*; 15 = the unpipelined kernel).
+// flags bits 8..11: tile shape override for tuning and tests (0 = automatic, 1 + CFG_*; 14 = 256 x 320 on the DMA-fed
+// kernel instead of the ping-pong kernel; 15 = the unpipelined kernel).
 extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                    uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags, void* workspace,
                                    uint64_t workspace_bytes) {
@@ -674,7 +952,8 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
             else e = launch_dense1_y<QG_FMT_B8, QWHIP_BF16>(s->stream, p, y_dtype);
         }
     } else {
-        const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : choose_cfg(m, w->n);
+        const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n));
+        p.force_gemm2 = ov == 14u ? 1u : 0u;
         if (fmt == QG_FMT_M5) e = launch_dense2_y<QG_FMT_M5>(s->stream, p, cfg, y_dtype);
         else if (fmt == QG_FMT_B4) e = launch_dense2_y<QG_FMT_B4>(s->stream, p, cfg, y_dtype);
         else e = launch_dense2_y<QG_FMT_B8>(s->stream, p, cfg, y_dtype);
