@@ -58,7 +58,7 @@ def run_gemm(dev, fmt, m, n, k, *, xdtype="bf16", ydtype="bf16", prerot=True, cf
     return st, out, ref
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 15])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 14, 15])
 def test_gemm_hq4_tile_shapes_f32_out(dev, cfg):
     st, out, ref = run_gemm(dev, "hq4_g32_m5", 512, 640, 1024, ydtype="f32", cfg=cfg)
     assert st == qwhip.OK
@@ -76,6 +76,18 @@ def test_gemm_ragged_shapes(dev, m, n, k):
 @pytest.mark.parametrize("xdtype,ydtype", [("f16", "f16"), ("bf16", "bf16")])
 def test_gemm_block_formats(dev, fmt, xdtype, ydtype):
     st, out, ref = run_gemm(dev, fmt, 192, 256, 768, xdtype=xdtype, ydtype=ydtype, seed=3)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "aq4_g32", "hq8_g32", "hq4_g64"])
+def test_gemm_pingpong_kernel_ragged_tiles(dev, fmt):
+    """The 8-wave ping-pong kernel (256 x 320 tiles, whole 64-row activation blocks) on a shape whose last tile row
+    holds one 64-row block and whose last tile column is ragged, for every weight format family."""
+    st, out, ref = run_gemm(dev, fmt, 320, 400, 640, xdtype="f16", ydtype="f32", cfg=1, seed=5)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= 2e-5
+    st, out, ref = run_gemm(dev, fmt, 64, 320, 64, xdtype="bf16", ydtype="bf16", cfg=1, seed=6)   # a single K-step
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= TOL
 
