@@ -245,10 +245,10 @@ __device__ __forceinline__ h8_t qw_x_operand(const h8_t* xg, int j) {
 template <int FMT, int NACC, int XDT, int XM>
 __device__ __forceinline__ void qw_stream_rows(const uint8_t* const* rp, const void* x, const h8_t* xs, uint32_t xpitch8,
                                                uint32_t K, uint32_t M, uint32_t gshift, uint32_t bb, bool rotate,
-                                               uint32_t wave, uint32_t i, uint32_t c, uint32_t magic, f4_t* acc) {
+                                               uint32_t wave, uint32_t i, uint32_t c, uint32_t magic, f4_t* acc, uint32_t nw = 4) {
     const uint32_t nsl = K >> 5;
     const uint32_t iters = (nsl + 3) >> 2;
-    const uint32_t per = (iters + 3) >> 2;
+    const uint32_t per = (iters + nw - 1u) / nw;
     const uint32_t it0 = wave * per;
     const uint32_t it1 = min(it0 + per, iters);
     qw_slice<FMT> cur[NACC] = {}, nxt[NACC] = {};
@@ -316,11 +316,12 @@ struct qw_gemv_params {
 // and the epilogue stores act[m, n] = f16(FWHT32(silu(g) * u)) (rotation optional).
 // ROUTED = 1 (with PAIR): blockIdx.y is a (token, route) pair; the expert's sub-bank is picked through
 // idx[pair], the activation row is the pair's token, the output row is the pair.
-template <int FMT, int RT, int XDT, int XM, int PAIR, int ROUTED>
-__global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const qw_gemv_params p) {
+template <int FMT, int RT, int XDT, int XM, int PAIR, int ROUTED, int NWV = 4>
+__global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_params p) {
+    constexpr uint32_t NTH = 64 * NWV;
     constexpr int NACC = RT * (PAIR ? 2 : 1);
     extern __shared__ h8_t xs[];
-    __shared__ f4_t red[4][NACC][64];
+    __shared__ f4_t red[NWV][NACC][64];
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = tid >> 6, lane = tid & 63u;
     const uint32_t i = lane & 15u, c = lane >> 4;
@@ -337,7 +338,7 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const qw_gemv_params 
         const int32_t e = p.idx[pair];
         y16 += (uint64_t)pair * N;
         if (e < 0) {  // no expert: the pair contributes nothing
-            for (uint32_t n = n0 + tid; n < min(n0 + 16u * RT, N); n += 256) y16[n] = (h1_t)0.0f;
+            for (uint32_t n = n0 + tid; n < min(n0 + 16u * RT, N); n += NTH) y16[n] = (h1_t)0.0f;
             return;
         }
         bank += (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const qw_gemv_params 
     }
 
     if constexpr (XM == QW_XM_LDS_ROT) {
-        for (uint32_t idx = tid; idx < M * nsl; idx += 256) {
+        for (uint32_t idx = tid; idx < M * nsl; idx += NTH) {
             const uint32_t m = idx / nsl, g = idx - m * nsl;
             qw_stage_group<XDT>(x, (uint64_t)m * K + 32u * g, p.rotate != 0, xs + m * xpitch8 + g * 4);
         }
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const qw_gemv_params 
 #pragma unroll
     for (int t = 0; t < NACC; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
     const uint32_t magic = qw_vgpr_const(0x64006400u);
-    qw_stream_rows<FMT, NACC, XDT, XM>(rp, x, xs, xpitch8, K, M, p.gshift, p.bb, p.rotate != 0, wave, i, c, magic, acc);
+    qw_stream_rows<FMT, NACC, XDT, XM>(rp, x, xs, xpitch8, K, M, p.gshift, p.bb, p.rotate != 0, wave, i, c, magic, acc, NWV);
 
     // split-K reduction: D[row 4c + r][col i] of every wave -> wave 0
 #pragma unroll
@@ -374,7 +375,9 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const qw_gemv_params 
         if (wave != 0) return;
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
-            f4_t v = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
+            f4_t v = red[0][t][lane];
+#pragma unroll
+            for (int w2 = 1; w2 < NWV; ++w2) v += red[w2][t][lane];
             if (i < M) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -392,8 +395,12 @@ __global__ __launch_bounds__(256) void qw_gemv_mfma_kernel(const qw_gemv_params 
         if (wave == 0) {
 #pragma unroll
             for (int t = 0; t < RT; ++t) {
-                const f4_t g = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
-                const f4_t u = red[0][RT + t][lane] + red[1][RT + t][lane] + red[2][RT + t][lane] + red[3][RT + t][lane];
+                f4_t g = red[0][t][lane], u = red[0][RT + t][lane];
+#pragma unroll
+                for (int w2 = 1; w2 < NWV; ++w2) {
+                    g += red[w2][t][lane];
+                    u += red[w2][RT + t][lane];
+                }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) actbuf[i][16 * t + 4 * c + r] = qw_swiglu(g[r], u[r]);
             }
@@ -476,6 +483,103 @@ __global__ __launch_bounds__(256) void qw_moe_down_decode_kernel(const qw_gemv_p
 }
 
 // ------------------------------------------------------------------------------------------------
+// Variant C: column-stationary MFMA kernel, all containers, m = 1..16, activations already in the container's basis,
+// rows of at most 40 K-iterations (k <= 5120).
+// One workgroup of 8 waves per compute unit walks the row tiles (16 rows) blockIdx.x, blockIdx.x + gridDim.x, ... so
+// the whole grid reads one contiguous band of rows at a time.  Wave w owns K-iterations [w * IPW, (w + 1) * IPW)
+// (an iteration = 4 slices of 32 columns; lane (i, c) holds slice 4*it + c of row i) for every row tile, so its
+// activation operands - the B operands of v_mfma_f32_16x16x32_f16, column j = activation row - are loaded once and
+// stay in registers: no activation traffic in the row loop, whatever m is.  The packed blocks of the next row tile
+// are fetched while the current one is dequantized and contracted; the 8 partial 16 x 16 tiles meet in LDS.
+// What bounds it today: the MFMA operand layout makes consecutive lanes hold different rows, so every load
+// instruction touches 16 rows (about 40 cache lines) and the address unit, not HBM, sets the pace (16 us on
+// N = 7168, K = 5120 in 36-byte blocks; the same bytes stream in about 7 us when lanes read consecutive blocks).
+// ------------------------------------------------------------------------------------------------
+template <int FMT, int XDT, int IPW>
+__global__ __launch_bounds__(512) void qw_gemv_colm_kernel(const qw_gemv_params p) {
+    __shared__ float red[2][8][64][4];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t i = lane & 15u, c = lane >> 4;
+    const uint32_t N = p.N, K = p.K, M = p.M;
+    const uint32_t nsl = K >> 5;
+    const uint32_t tiles = (N + 15u) >> 4;
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+
+    // ---- this wave's activation operands: xop[u][j] = columns 8j..8j+7 of slice 4*(wave*IPW + u) + c of row i.
+    // Their loads go out first, the first row tile's loads right behind them (issued before any of the activation
+    // data is touched), so the prologue costs one memory round trip, not two.
+    h8_t xraw[IPW][4], xop[IPW][4];
+    uint32_t sl[IPW];   // slice index per iteration (clamped; invalid slices carry zero operands)
+#pragma unroll
+    for (int u = 0; u < IPW; ++u) {
+        sl[u] = min(4u * (wave * IPW + u) + c, nsl - 1u);
+        const uint64_t at = (uint64_t)min(i, M - 1u) * K + 32u * sl[u];   // clamped address: no branches around the loads
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xraw[u][j] = qw_load_x8_f16<XDT>(p.x, at + 8u * j);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    auto load_tile = [&](uint32_t t, qw_slice<FMT>* blk) {
+        const uint32_t row = min(16u * min(t, tiles - 1u) + i, N - 1u);
+        const uint8_t* rowp = p.bank + (uint64_t)row * p.row_bytes;
+#pragma unroll
+        for (int u = 0; u < IPW; ++u) qw_load_slice<FMT>(rowp, sl[u], p.gshift, p.bb, blk[u]);
+    };
+    auto compute_tile = [&](uint32_t t, const qw_slice<FMT>* blk, uint32_t buf) {
+        f4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < IPW; ++u) {
+            const h2_t s2 = qw_splat_lo(blk[u].hdr), b2 = qw_splat_hi(blk[u].hdr);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const h8_t a = qw_dequant_chunk<FMT>(blk[u], j, s2, b2, magic);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xop[u][j], acc, 0, 0, 0);
+            }
+        }
+        // lane (j = activation row, c) holds rows 4c + r of the tile
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[buf][wave][lane][r] = acc[r];
+        __syncthreads();
+        if (tid < 256u && t < tiles) {
+            const uint32_t rr = tid & 15u, m = tid >> 4;   // consecutive lanes -> consecutive output rows
+            const uint32_t slot = m + 16u * (rr >> 2), comp = rr & 3u;
+            float v = 0.f;
+#pragma unroll
+            for (int w2 = 0; w2 < 8; ++w2) v += red[buf][w2][slot][comp];
+            const uint32_t n = 16u * t + rr;
+            if (m < M && n < N) {
+                if (p.y32) p.y32[(uint64_t)m * N + n] = v;
+                if (p.y16) p.y16[(uint64_t)m * N + n] = (h1_t)v;
+            }
+        }
+    };
+
+    // ---- row tiles, two per trip so the register buffers keep static names ----
+    const uint32_t G = gridDim.x;
+    qw_slice<FMT> bufA[IPW], bufB[IPW];
+    uint32_t t = blockIdx.x;
+    load_tile(t, bufA);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < IPW; ++u) {
+        const bool ok = 4u * (wave * IPW + u) + c < nsl && i < M;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const h8_t v = qw_x_operand<FMT>(xraw[u], j);
+            const u4_t raw = __builtin_bit_cast(u4_t, v);
+            const u4_t z = {ok ? raw[0] : 0u, ok ? raw[1] : 0u, ok ? raw[2] : 0u, ok ? raw[3] : 0u};
+            xop[u][j] = __builtin_bit_cast(h8_t, z);
+        }
+    }
+    for (; t < tiles; t += 2u * G) {
+        load_tile(t + G, bufB);
+        compute_tile(t, bufA, 0);
+        load_tile(t + 2u * G, bufA);
+        compute_tile(t + G, bufB, 1);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -484,6 +588,20 @@ typedef qw_gemv_params gemv_args;
 
 template <int FMT, int RT, int XDT, int XM, int PAIR>
 void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds, uint32_t routed_pairs = 0) {
+    if constexpr (!PAIR && RT == 1) {
+        // Few row tiles, long rows and one or two activation rows: more waves per workgroup split K further, so
+        // that the launch keeps enough loads in flight to cover HBM latency (measured on K = 17408, N = 5120:
+        // 33.6 -> 26.0 us at m = 1; with more activation rows the extra waves multiply the activation traffic instead).
+        if (!routed_pairs && a.M <= 2u) {
+            const uint32_t tiles = qwhip_cdiv(a.N, 16u);
+            const uint32_t iters = qwhip_cdiv(a.K >> 5, 4u);
+            uint32_t nw = 4;
+            while (nw < 16u && tiles * nw < 4096u && iters >= 4u * nw) nw *= 2u;
+            const dim3 grid(tiles);
+            if (nw == 16u) { hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0, 16>), grid, dim3(1024), lds, st, a); return; }
+            if (nw == 8u) { hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0, 8>), grid, dim3(512), lds, st, a); return; }
+        }
+    }
     const dim3 block(256);
     if (routed_pairs) {
         if constexpr (PAIR) {
@@ -513,6 +631,26 @@ void launch_mfma_rt(hipStream_t st, const gemv_args& a, uint32_t xdt, int xm, si
     if (rt == 1) launch_mfma_dt<FMT, 1, 0>(st, a, xdt, xm, lds);
     else if (rt == 2) launch_mfma_dt<FMT, 2, 0>(st, a, xdt, xm, lds);
     else launch_mfma_dt<FMT, 4, 0>(st, a, xdt, xm, lds);
+}
+
+// Column-stationary kernel (variant C): false when the call is outside its envelope.
+template <int FMT>
+bool launch_colm(hipStream_t st, const gemv_args& a, uint32_t xdt) {
+    const uint32_t iters = qwhip_cdiv(a.K >> 5, 4u);
+    if (iters > 40u || a.rotate) return false;
+    const uint32_t ipw = qwhip_cdiv(iters, 8u);
+    const uint32_t tiles = qwhip_cdiv(a.N, 16u);
+    const dim3 grid(min(tiles, 256u)), block(512);
+#define QW_COLM(DT, I) hipLaunchKernelGGL((qw_gemv_colm_kernel<FMT, DT, I>), grid, block, 0, st, a)
+#define QW_COLM_I(DT)                                                                                  \
+    switch (ipw) {                                                                                     \
+        case 1: QW_COLM(DT, 1); break; case 2: QW_COLM(DT, 2); break; case 3: QW_COLM(DT, 3); break;   \
+        case 4: QW_COLM(DT, 4); break; default: QW_COLM(DT, 5); break;                                 \
+    }
+    if (xdt == QWHIP_F16) { QW_COLM_I(QWHIP_F16) } else { QW_COLM_I(QWHIP_BF16) }
+#undef QW_COLM_I
+#undef QW_COLM
+    return true;
 }
 
 qwhip_status check_common(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
@@ -550,7 +688,7 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
                  float* y32, uint32_t tune, hipError_t* err);
 
 // flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer,
-// 4 = column-stationary persistent kernel);
+// 4 = column-stationary persistent kernel, 5 = column-stationary MFMA kernel);
 // bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer / tuning code of the
 // column-stationary kernel (0 = automatic).
 extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
@@ -582,7 +720,7 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     if (variant == 1 && !dot2_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "dot2 kernel needs HQ4_G32_M5, m = 1, k <= 24576");
     // automatic choice: the DMA streamer where it measured faster than the direct-load kernel (few row tiles, short rows,
     // one or two activation rows), the direct-load kernel otherwise
-    const bool stream_auto = !dot2_ok && m <= 2 && w->n <= 8192 && w->k <= 8192;
+    const bool stream_auto = !dot2_ok && m <= 2 && w->n <= 4096 && w->k <= 8192;
     if (variant == 3 || (variant == 0 && stream_auto)) {
         hipError_t e = hipSuccess;
         if (qw_stream_gemv(s->stream, w, x, x_dtype, m, rotate, y16, y32, rt, &e)) {
@@ -617,10 +755,23 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
         return QWHIP_OK;
     }
 
+    // column-stationary MFMA kernel: activations already in the basis (verify rows, standard-basis containers), k <= 5120
+    if (variant == 5 || (variant == 0 && !rotate)) {
+        bool done = false;
+        if (fmt == QW_FMT_M5) done = launch_colm<QW_FMT_M5>(s->stream, a, x_dtype);
+        else if (fmt == QW_FMT_B4) done = launch_colm<QW_FMT_B4>(s->stream, a, x_dtype);
+        else done = launch_colm<QW_FMT_B8>(s->stream, a, x_dtype);
+        if (done) {
+            QWHIP_TRY_HIP(hipGetLastError());
+            return QWHIP_OK;
+        }
+        if (variant == 5) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the column-stationary MFMA kernel needs activations in the basis and k <= 5120");
+    }
     // mfma streamer.  Rotation in the prologue (LDS) when the rotated rows fit, else per lane.
     const size_t lds_x = (size_t)m * ((size_t)w->k * 2u + 16u);
     const int xm = (rotate && lds_x <= 48u * 1024u) ? QW_XM_LDS_ROT : QW_XM_GLOBAL;
-    if (rt != 1 && rt != 2 && rt != 4) rt = (w->n >= 16384) ? 2u : 1u;
+    // two row tiles per wave halve the activation traffic per weight byte: it pays from eight activation rows on
+    if (rt != 1 && rt != 2 && rt != 4) rt = (w->n >= 16384 || m >= 8) ? 2u : 1u;
     const size_t lds = xm == QW_XM_LDS_ROT ? lds_x : 0;
     if (fmt == QW_FMT_M5) launch_mfma_rt<QW_FMT_M5>(s->stream, a, x_dtype, xm, lds, (int)rt);
     else if (fmt == QW_FMT_B4) launch_mfma_rt<QW_FMT_B4>(s->stream, a, x_dtype, xm, lds, (int)rt);
