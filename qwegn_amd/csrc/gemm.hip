@@ -733,16 +733,60 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
+    if constexpr (YDT != QWHIP_F32) {
+        // 2-byte outputs: each wave transposes its 32-row slabs through a private LDS region (the operand stages are
+        // dead by now) and stores 16-byte row chunks; a lane's accumulators are one column of 16 rows, and 2-byte
+        // stores from that layout cost one address per element. The host side guarantees 16-byte aligned output rows.
+        constexpr uint32_t EP_PITCH = WN * 64 + 16;    // 4 rows apart land 16 banks apart
+        constexpr uint32_t EP_CH = WN * 4;             // 16-byte chunks per slab row
+        static_assert(8u * 32u * EP_PITCH <= 2u * STAGE, "epilogue slabs must fit the operand stages");
+        __syncthreads();
+        uint8_t* ep = lds2 + wave * (32u * EP_PITCH);
+        const uint32_t w_off = (4u * (lane >> 5)) * EP_PITCH + (lane & 31u) * 2u;
 #pragma unroll
-    for (int a = 0; a < WM; ++a) {
+        for (int a = 0; a < WM; ++a) {
 #pragma unroll
-        for (int b = 0; b < WN; ++b) {
-            const uint32_t n = n0 + (wn * WN + b) * 32 + (lane & 31u);
-            if (n < p.N) {
+            for (int b = 0; b < WN; ++b) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const uint32_t row = (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                for (int r = 0; r < 16; r += 2) {
+                    const uint32_t o = w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH + b * 64u;
+                    uint32_t pk;
+                    if constexpr (YDT == QWHIP_BF16) {
+                        typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+                        typedef float fl2_t __attribute__((ext_vector_type(2)));
+                        const fl2_t v = {acc[a][b][r], acc[a][b][r + 1]};
+                        pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2_t));
+                    } else {
+                        const h2_t v = {(h1_t)acc[a][b][r], (h1_t)acc[a][b][r + 1]};
+                        pk = __builtin_bit_cast(uint32_t, v);
+                    }
+                    *(uint16_t*)(ep + o) = (uint16_t)pk;
+                    *(uint16_t*)(ep + o + EP_PITCH) = (uint16_t)(pk >> 16);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < WN * 2; ++q) {
+                const uint32_t c = q * 64u + lane;
+                const uint32_t row = c / EP_CH, cc = c - row * EP_CH;
+                const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
+                const uint32_t grow = (wm * WM + a) * 32u + row;
+                const uint32_t n = n0 + wn * (WN * 32u) + cc * 8u;
+                if (grow < rows_valid && n < p.N)
+                    *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int a = 0; a < WM; ++a) {
+#pragma unroll
+            for (int b = 0; b < WN; ++b) {
+                const uint32_t n = n0 + (wn * WN + b) * 32 + (lane & 31u);
+                if (n < p.N) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t row = (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                        if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                    }
                 }
             }
         }
@@ -819,7 +863,9 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     switch (cfg) {
         case CFG_256x320:
             // the ping-pong kernel takes whole 64-row activation blocks; ragged M stays on the DMA-fed kernel
-            if (p.M % 64u == 0 && !p.force_gemm2) return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
+            if (p.M % 64u == 0 && !p.force_gemm2 &&
+                (YDT == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0)))
+                return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
             return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x256: return launch_cfg2<2, 4, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x128: return launch_cfg2<2, 2, 4, 2, FMT, YDT, false>(st, p, grid);

@@ -245,14 +245,18 @@ __device__ __forceinline__ h8_t qw_x_operand(const h8_t* xg, int j) {
 template <int FMT, int NACC, int XDT, int XM>
 __device__ __forceinline__ void qw_stream_rows(const uint8_t* const* rp, const void* x, const h8_t* xs, uint32_t xpitch8,
                                                uint32_t K, uint32_t M, uint32_t gshift, uint32_t bb, bool rotate,
-                                               uint32_t wave, uint32_t i, uint32_t c, uint32_t magic, f4_t* acc, uint32_t nw = 4) {
+                                               uint32_t wave, uint32_t i, uint32_t c, uint32_t magic, f4_t* acc, uint32_t nw = 4,
+                                               const qw_slice<FMT>* first = nullptr) {
     const uint32_t nsl = K >> 5;
     const uint32_t iters = (nsl + 3) >> 2;
     const uint32_t per = (iters + nw - 1u) / nw;
     const uint32_t it0 = wave * per;
     const uint32_t it1 = min(it0 + per, iters);
     qw_slice<FMT> cur[NACC] = {}, nxt[NACC] = {};
-    if (it0 < it1) {
+    if (first) {
+#pragma unroll
+        for (int t = 0; t < NACC; ++t) cur[t] = first[t];
+    } else if (it0 < it1) {
         const uint32_t s = min(4u * it0 + c, nsl - 1);
 #pragma unroll
         for (int t = 0; t < NACC; ++t) qw_load_slice<FMT>(rp[t], s, gshift, bb, cur[t]);
@@ -294,6 +298,19 @@ __device__ __forceinline__ void qw_stream_rows(const uint8_t* const* rp, const v
     }
 }
 
+// The first iteration's loads of qw_stream_rows, for callers that want them in flight before their own prologue ends
+// (the slice index is clamped: a wave with no iterations loads a valid slice it never uses).
+template <int FMT, int NACC>
+__device__ __forceinline__ void qw_stream_first(const uint8_t* const* rp, uint32_t K, uint32_t gshift, uint32_t bb, uint32_t wave,
+                                                uint32_t c, uint32_t nw, qw_slice<FMT>* first) {
+    const uint32_t nsl = K >> 5;
+    const uint32_t iters = (nsl + 3) >> 2;
+    const uint32_t per = (iters + nw - 1u) / nw;
+    const uint32_t s = min(4u * wave * per + c, nsl - 1);
+#pragma unroll
+    for (int t = 0; t < NACC; ++t) qw_load_slice<FMT>(rp[t], s, gshift, bb, first[t]);
+}
+
 struct qw_gemv_params {
     const uint8_t* bank;
     const void* x;
@@ -333,24 +350,28 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_pa
     const uint8_t* bank = p.bank;
     const void* x = p.x;
     h1_t* y16 = p.y16;
+    // Order of the prologue's memory traffic: the route's expert id first, the activation staging (which does not
+    // need it) behind it, then the first weight slices, and only then the barrier that publishes the staged
+    // activations: the three round trips overlap instead of queueing.
+    int32_t e = 0;
     if constexpr (ROUTED) {
         const uint32_t pair = blockIdx.y;
-        const int32_t e = p.idx[pair];
+        e = p.idx[pair];
         y16 += (uint64_t)pair * N;
-        if (e < 0) {  // no expert: the pair contributes nothing
-            for (uint32_t n = n0 + tid; n < min(n0 + 16u * RT, N); n += NTH) y16[n] = (h1_t)0.0f;
-            return;
-        }
-        bank += (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
         x = (const uint8_t*)x + (uint64_t)(pair / p.top_k) * K * 2u;
     }
-
     if constexpr (XM == QW_XM_LDS_ROT) {
         for (uint32_t idx = tid; idx < M * nsl; idx += NTH) {
             const uint32_t m = idx / nsl, g = idx - m * nsl;
             qw_stage_group<XDT>(x, (uint64_t)m * K + 32u * g, p.rotate != 0, xs + m * xpitch8 + g * 4);
         }
-        __syncthreads();
+    }
+    if constexpr (ROUTED) {
+        if (e < 0) {  // no expert: the pair contributes nothing (uniform over the workgroup, before any barrier)
+            for (uint32_t n = n0 + tid; n < min(n0 + 16u * RT, N); n += NTH) y16[n] = (h1_t)0.0f;
+            return;
+        }
+        bank += (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
     }
 
     const uint8_t* rp[NACC];
@@ -361,11 +382,14 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_pa
         rp[t] = bank + (uint64_t)row * p.row_bytes;
         if (PAIR) rp[RT + t] = bank + (uint64_t)(row + N) * p.row_bytes;
     }
+    qw_slice<FMT> first[NACC];
+    qw_stream_first<FMT, NACC>(rp, K, p.gshift, p.bb, wave, c, NWV, first);
+    if constexpr (XM == QW_XM_LDS_ROT) __syncthreads();
     f4_t acc[NACC];
 #pragma unroll
     for (int t = 0; t < NACC; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
     const uint32_t magic = qw_vgpr_const(0x64006400u);
-    qw_stream_rows<FMT, NACC, XDT, XM>(rp, x, xs, xpitch8, K, M, p.gshift, p.bb, p.rotate != 0, wave, i, c, magic, acc, NWV);
+    qw_stream_rows<FMT, NACC, XDT, XM>(rp, x, xs, xpitch8, K, M, p.gshift, p.bb, p.rotate != 0, wave, i, c, magic, acc, NWV, first);
 
     // split-K reduction: D[row 4c + r][col i] of every wave -> wave 0
 #pragma unroll
@@ -426,11 +450,14 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_pa
 // Routed down projection of the decode path: blockIdx.y is a token; the workgroup's 16*RT output rows
 // accumulate sum_k wts[t, k] * (W_down[e_k] . act[t, k]) over the token's routes, add the gated shared
 // expert, and store.  Activations (SwiGLU output) are already in the rotated basis.
+// Wave w takes routes w, w + 8, ... whole (every route is a short row: its loads are all in flight at once and the
+// routes of a token stream side by side instead of one after the other); the route partials meet in LDS and are
+// summed in wave order.
 template <int FMT, int RT, int ODT>
-__global__ __launch_bounds__(256) void qw_moe_down_decode_kernel(const qw_gemv_params p) {
-    __shared__ f4_t red[4][RT][64];
+__global__ __launch_bounds__(512) void qw_moe_down_decode_kernel(const qw_gemv_params p) {
+    __shared__ f4_t red[8][RT][64];
     const uint32_t tid = threadIdx.x;
-    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u;
     const uint32_t i = lane & 15u, c = lane >> 4;
     const uint32_t N = p.N, K = p.K;
     const uint32_t n0 = blockIdx.x * (16u * RT);
@@ -439,7 +466,7 @@ __global__ __launch_bounds__(256) void qw_moe_down_decode_kernel(const qw_gemv_p
     f4_t total[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) total[t] = f4_t{0.f, 0.f, 0.f, 0.f};
-    for (uint32_t k = 0; k < p.top_k; ++k) {
+    for (uint32_t k = wave; k < p.top_k; k += 8u) {
         const uint32_t pair = tok * p.top_k + k;
         const int32_t e = p.idx[pair];
         if (e < 0) continue;
@@ -456,7 +483,7 @@ __global__ __launch_bounds__(256) void qw_moe_down_decode_kernel(const qw_gemv_p
 #pragma unroll
         for (int t = 0; t < RT; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
         const void* x = (const uint8_t*)p.x + (uint64_t)pair * K * 2u;
-        qw_stream_rows<FMT, RT, QWHIP_F16, QW_XM_GLOBAL>(rp, x, nullptr, 0, K, 1, p.gshift, p.bb, false, wave, i, c, magic, acc);
+        qw_stream_rows<FMT, RT, QWHIP_F16, QW_XM_GLOBAL>(rp, x, nullptr, 0, K, 1, p.gshift, p.bb, false, 0u, i, c, magic, acc, 1u);
 #pragma unroll
         for (int t = 0; t < RT; ++t) total[t] += acc[t] * wk;
     }
@@ -466,7 +493,9 @@ __global__ __launch_bounds__(256) void qw_moe_down_decode_kernel(const qw_gemv_p
     if (wave != 0 || i != 0) return;
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
-        const f4_t v = red[0][t][lane] + red[1][t][lane] + red[2][t][lane] + red[3][t][lane];
+        f4_t v = red[0][t][lane];
+#pragma unroll
+        for (int w2 = 1; w2 < 8; ++w2) v += red[w2][t][lane];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const uint32_t n = n0 + 16u * t + 4u * c + r;
@@ -605,8 +634,12 @@ void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds, uint32_t routed
     const dim3 block(256);
     if (routed_pairs) {
         if constexpr (PAIR) {
+            // one short row set per (route, tile): eight waves split K so that each holds two or more iterations in flight
             const dim3 grid(qwhip_cdiv(a.N, 16u * RT), routed_pairs);
-            hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1>), grid, block, lds, st, a);
+            if (qwhip_cdiv(a.K >> 5, 4u) >= 16u)
+                hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1, 8>), grid, dim3(512), lds, st, a);
+            else
+                hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1>), grid, block, lds, st, a);
         }
     } else {
         const dim3 grid(qwhip_cdiv(a.N, 16u * RT));
@@ -884,7 +917,7 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
     a.shared = shared;
     a.shared_gate = shared_gate;
     a.out = out;
-    const dim3 grid(qwhip_cdiv(hidden, 16u)), block(256);
+    const dim3 grid(qwhip_cdiv(hidden, 16u)), block(512);
     const dim3 g2(grid.x, t);
 #define QW_DD(F, OD) hipLaunchKernelGGL((qw_moe_down_decode_kernel<F, 1, OD>), g2, block, 0, s->stream, a)
 #define QW_DD_O(F)                                                                                          \

@@ -113,42 +113,50 @@ __global__ __launch_bounds__(64) void qw_moe_route_kernel(const float* __restric
         ok[j] = ok[j] && total > 0.0f;
         p[j] = ok[j] ? p[j] / total : -1e30f;
     }
+    // Selection rounds on the scalar unit: the wave maximum comes from four DPP steps inside each row of 16 lanes and
+    // four lane reads, the owner of the maximum from ballots in ascending expert order (ties go to the lower id).
+    // Cross-lane permutes through LDS would put two dependent ~100-clock round trips on every one of the 6 x top_k steps.
+    float cand[8];
+#pragma unroll
+    for (uint32_t j = 0; j < 8; ++j) cand[j] = ok[j] ? p[j] : -1.0f;   // probabilities are >= 0
     float wsel = 0.0f;  // lane r keeps the weight of rank r (K <= 16 < 64)
     int32_t isel = -1;
     for (uint32_t r = 0; r < K; ++r) {
-        float bv = -3.4e38f;
+        float lm = cand[0];
+#pragma unroll
+        for (uint32_t j = 1; j < 8; ++j) lm = fmaxf(lm, cand[j]);
+        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0xB1, 0xF, 0xF, true)));
+        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0x4E, 0xF, 0xF, true)));
+        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0x141, 0xF, 0xF, true)));
+        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0x140, 0xF, 0xF, true)));
+        const int lmi = __builtin_bit_cast(int, lm);
+        const float wm = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 0)),
+                                     __builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 16))),
+                               fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 32)),
+                                     __builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 48))));
         uint32_t bi = 0xFFFFFFFFu;
+        if (wm >= 0.0f) {
 #pragma unroll
-        for (uint32_t j = 0; j < 8; ++j) {
-            const uint32_t id = lane + 64u * j;
-            if (ok[j] && (bi == 0xFFFFFFFFu || p[j] > bv)) {  // ascending id within the lane: strict > keeps the lower id
-                bv = p[j];
-                bi = id;
-            }
-        }
-        // wave argmax, ties to the lower id
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(bv, off, 64);
-            const uint32_t oi = __shfl_xor(bi, off, 64);
-            if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi))) {
-                bv = ov;
-                bi = oi;
+            for (uint32_t j = 0; j < 8; ++j) {
+                const unsigned long long m = __ballot(cand[j] == wm);
+                if (bi == 0xFFFFFFFFu && m != 0ull) bi = 64u * j + (uint32_t)__builtin_ctzll(m);
             }
         }
         if (bi != 0xFFFFFFFFu && (bi & 63u) == lane) {
 #pragma unroll
             for (uint32_t j = 0; j < 8; ++j)
-                if (j == (bi >> 6)) ok[j] = false;
+                if (j == (bi >> 6)) cand[j] = -1.0f;
         }
         if (lane == r) {
-            wsel = bi != 0xFFFFFFFFu ? bv : 0.0f;
+            wsel = bi != 0xFFFFFFFFu ? wm : 0.0f;
             isel = bi != 0xFFFFFFFFu ? (int32_t)bi : -1;
         }
     }
     // sum of the selected in rank order (lane 0 .. K-1), as the reference's serial loop
     float acc = 0.0f;
-    for (uint32_t r = 0; r < K; ++r) acc += __shfl(wsel, (int)r, 64);
+#pragma unroll
+    for (uint32_t r = 0; r < 16; ++r)
+        if (r < K) acc += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsel), r));
     if (lane < K) {
         float w = wsel;
         if (norm) w = acc > 0.0f ? w / acc : 0.0f;
