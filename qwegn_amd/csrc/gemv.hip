@@ -716,6 +716,13 @@ uint32_t log2_u32(uint32_t v) {
 bool qw_stream_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m, bool rotate,
                     void* y16, float* y32, uint32_t kw_override, hipError_t* err);
 
+// moe_col.hip
+bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
+                       bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err);
+bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* act16, const int32_t* idx,
+                     const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
+                     uint32_t out_dtype, hipError_t* err);
+
 // gemv_col.hip
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
                  float* y32, uint32_t tune, hipError_t* err);
@@ -860,6 +867,15 @@ extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_we
     if ((uint64_t)t * top_k > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "decode path holds at most 65535 (token, route) pairs");
     const uint32_t inter = w_gate_up->n / (2 * experts);
     const bool rotate = qwhip_view_rotated(w_gate_up) && !(flags & QWHIP_X_PREROTATED);
+    // HQ4_G32_M5 banks take the column-stationary kernel (flags bits 8..11 = 2 keep the general one, for tests)
+    if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
+        hipError_t e = hipSuccess;
+        if (qw_moe_gateup_col(s->stream, w_gate_up, experts, x, x_dtype, rotate, qwhip_view_rotated(w_gate_up) && inter % 32 == 0,
+                              idx, t * top_k, top_k, act16, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+    }
     gemv_args a = {};
     a.bank = (const uint8_t*)w_gate_up->blocks;
     a.x = x;
@@ -901,6 +917,13 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
     if (t > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "decode path holds at most 65535 tokens");
     if ((w_down->k * 2u) % 16u != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "activation rows must be 16-byte multiples");
     const uint32_t hidden = w_down->n / experts;
+    if (fmt == QW_FMT_M5) {
+        hipError_t e = hipSuccess;
+        if (qw_moe_down_col(s->stream, w_down, experts, act16, idx, wts, t, top_k, shared, shared_gate, out, out_dtype, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+    }
     gemv_args a = {};
     a.bank = (const uint8_t*)w_down->blocks;
     a.x = act16;

@@ -20,34 +20,6 @@
 
 namespace {
 
-// Rows i and i + 16 (i = lane & 15) of the 32-point Hadamard matrix, columns 8c .. 8c + 7 (c = lane >> 4), as f16 +-1:
-// sign(i, k) = parity(i & k); for i < 16 that is parity(i & 8c) ^ parity(i & e) with only bit 3 of i meeting 8c, and
-// row i + 16 flips the sign where k >= 16.
-__device__ __forceinline__ void qc_hadamard_pair(uint32_t i, uint32_t c, h8_t& lo, h8_t& hi) {
-    const uint32_t b0 = i & 1u, b1 = (i >> 1) & 1u, b2 = (i >> 2) & 1u;
-    const uint32_t pc = (c & 1u) & ((i >> 3) & 1u);
-    const uint32_t s0 = pc, s1 = pc ^ b0, s2 = pc ^ b1, s3 = s1 ^ b1, s4 = pc ^ b2, s5 = s1 ^ b2, s6 = s2 ^ b2, s7 = s3 ^ b2;
-    u4_t w;
-    w[0] = 0x3C003C00u | (s0 << 15) | (s1 << 31);
-    w[1] = 0x3C003C00u | (s2 << 15) | (s3 << 31);
-    w[2] = 0x3C003C00u | (s4 << 15) | (s5 << 31);
-    w[3] = 0x3C003C00u | (s6 << 15) | (s7 << 31);
-    lo = __builtin_bit_cast(h8_t, w);
-    const uint32_t flip = (c >= 2u) ? 0x80008000u : 0u;
-    const u4_t v = {w[0] ^ flip, w[1] ^ flip, w[2] ^ flip, w[3] ^ flip};
-    hi = __builtin_bit_cast(h8_t, v);
-}
-
-// Sum over each aligned 32-lane half; the result is valid in lanes 16..31 (half 0) and 48..63 (half 1).
-__device__ __forceinline__ float qc_reduce32(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, true));  // row_bcast15 into rows 1, 3
-    return v;
-}
-
 struct qc_params {
     const uint8_t* bank;
     const void* x;
@@ -104,7 +76,7 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
     // 3. rotation on the matrix cores into the shared image
     {
         h8_t h_lo, h_hi;
-        qc_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
+        qw_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
 #pragma unroll
         for (int t = 0; t < XT; ++t) qw_rotate_tile_to_lds(xv[t], wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs);
     }
@@ -157,7 +129,7 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
             q = __builtin_fmaf(hi0 + hi1, 1048576.0f, q);
             float v = __builtin_fmaf((float)hd[0], q, (float)hd[1] * S);
             v = gvalid ? v : 0.0f;
-            v = qc_reduce32(v);
+            v = qw_reduce32_dpp(v);
             if (lane == 31u && rslot < nrows) part[rslot * cpr + chunk] = v;
             rslot += SETS;
         }

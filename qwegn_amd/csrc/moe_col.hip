@@ -1,0 +1,300 @@
+// MoE decode (a handful of tokens) over HQ4_G32_M5 expert banks, column-stationary form.
+//
+// Both routed projections of the decode path (encodeMoEGateUpF32R1 / encodeMoEDownSharedCombineF32,
+// Sources/Operators/QWGEMM/QWGemmMoE.swift:120-199) read a few short rows from each routed expert: the launch is
+// latency bound, so what matters is that every byte is requested at once, by loads whose lanes read consecutive
+// blocks.  A lane owns one block column for the whole kernel, keeps its 32 activations in registers as 16 f16 pairs
+// and contracts the masked nibble pairs directly as f16 subnormal operands of v_dot2_f32_f16:
+//     sum_i w_i x_i = s * (sum_i q_i x_i + 1024 S) + b * S,   S = sum_i x_i      (w = (1024 + q) s + b,
+// unpack_hq4_word8, Sources/QWMetal/include/qw_dequant.metalh:42-62).  A half-wavefront covers 32 block columns of a
+// row and reduces with DPP; the per-chunk partial sums meet in LDS and are added in chunk order.
+#include "qwhip_common.h"
+
+namespace {
+
+// 16 operand pairs and their sum from the 32 activations v[0..3] of one block column.
+__device__ __forceinline__ float qmc_operands(const h8_t* v, h2_t* xo) {
+    const h2_t one = {(h1_t)1.0f, (h1_t)1.0f};
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+            const h2_t pr = {v[j][2 * e2], v[j][2 * e2 + 1]};
+            if (e2 & 1) s1 = __builtin_amdgcn_fdot2(pr, one, s1, false);
+            else s0 = __builtin_amdgcn_fdot2(pr, one, s0, false);
+            xo[4 * j + e2] = pr;
+        }
+    }
+    return s0 + s1;
+}
+
+// One block against the lane's operands: s * (sum q x + 1024 S) + b * S.
+__device__ __forceinline__ float qmc_block_dot(const qw_hq4_block& b, const h2_t* xo, float S, float c1) {
+    float lo0 = 0.f, lo1 = 0.f, hi0 = 0.f, hi1 = 0.f;
+#pragma unroll
+    for (int w4 = 0; w4 < 4; ++w4) {
+        const uint32_t w = b.qs[w4], w8 = w >> 8;
+        const uint32_t m0 = w & 0x000F000Fu, m1 = w & 0x00F000F0u, m2 = w8 & 0x000F000Fu, m3 = w8 & 0x00F000F0u;
+        lo0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m0), xo[4 * w4 + 0], lo0, false);
+        hi0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m1), xo[4 * w4 + 1], hi0, false);
+        lo1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m2), xo[4 * w4 + 2], lo1, false);
+        hi1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m3), xo[4 * w4 + 3], hi1, false);
+    }
+    const h2_t hd = __builtin_bit_cast(h2_t, b.hdr);
+    float q = __builtin_fmaf(lo0 + lo1, 16777216.0f, c1);   // the low nibbles read as q * 2^-24, the high ones as 16 q * 2^-24
+    q = __builtin_fmaf(hi0 + hi1, 1048576.0f, q);
+    return __builtin_fmaf((float)hd[0], q, (float)hd[1] * S);
+}
+
+// ------------------------------------------------------------------------------------------------
+// gate|up: grid (ceil(I / 32), pairs).  A workgroup owns 32 gate rows and the 32 matching up rows of the pair's expert
+// (row slot s: up = s >> 5, n = n0 + (s & 31)); set j of SETS takes slots j * R .. j * R + R - 1, R = 64 / SETS.
+// Epilogue: act[pair, n] = f16(FWHT32(silu(g) * u)) over the 32 outputs of the workgroup (rotation optional).
+// blockDim.x = 32 * cpr * SETS; dynamic LDS = nb * 80 + 64 * cpr * 4 bytes.
+// ------------------------------------------------------------------------------------------------
+struct qmc_gu_params {
+    const uint8_t* bank;
+    const void* x;
+    h1_t* act;
+    const int32_t* idx;
+    uint32_t I, nb, cpr, top_k, rotate, rot_out;
+    uint64_t expert_bytes;
+};
+
+template <int XDT, int SETS>
+__global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_params p) {
+    constexpr int R = 64 / SETS;
+    constexpr int D = R < 8 ? R : 8;             // rows in flight per lane
+    constexpr int XT = SETS == 2 ? 2 : 1;        // 16-group activation tiles per wave: ceil(2 cpr / (cpr * SETS / 2))
+    extern __shared__ h8_t qmc_lds[];
+    const uint32_t nb = p.nb, cpr = p.cpr, I = p.I;
+    h8_t* xs = qmc_lds;
+    float* part = (float*)(qmc_lds + (size_t)nb * 5);   // [64 row slots][cpr]
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 31u, hw = tid >> 5;
+    const uint32_t wave = tid >> 6, l64 = tid & 63u;
+    const uint32_t nw = blockDim.x >> 6;
+    const uint32_t set = hw / cpr, chunk = hw - set * cpr;
+    const uint32_t g0 = chunk * 32u + lane;
+    const bool gvalid = g0 < nb;
+    const uint32_t g = gvalid ? g0 : nb - 1u;
+    const uint32_t pair = blockIdx.y, n0 = blockIdx.x * 32u;
+    const uint32_t row_bytes = nb * 20u;
+
+    // memory order: the route's expert id, the token's activations, the first weight rows; the rotation runs under them
+    const int32_t e = p.idx[pair];
+    const uint8_t* x = (const uint8_t*)p.x + (uint64_t)(pair / p.top_k) * nb * 64u;
+    h8_t xv[XT];
+#pragma unroll
+    for (int t = 0; t < XT; ++t) {
+        const uint32_t gg = min((wave + nw * t) * 16u + (l64 & 15u), nb - 1u);
+        xv[t] = qw_load_x8_f16<XDT>(x, (uint64_t)gg * 32u + 8u * (l64 >> 4));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    h1_t* act = p.act + (uint64_t)pair * I;
+    if (e < 0) {   // no expert: the pair contributes nothing (uniform over the workgroup)
+        if (tid < 32u && n0 + tid < I) act[n0 + tid] = (h1_t)0.0f;
+        return;
+    }
+    const uint8_t* bank = p.bank + (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
+    auto row_off = [&](uint32_t r) {   // r-th row of this set
+        const uint32_t s = set * R + min(r, (uint32_t)R - 1u);
+        const uint32_t n = min(n0 + (s & 31u), I - 1u);
+        return ((s >> 5) * I + n) * row_bytes + g * 20u;
+    };
+    qw_hq4_block buf[D];
+#pragma unroll
+    for (int j = 0; j < D; ++j) buf[j] = *(const qw_hq4_block*)(bank + row_off(j));
+    __builtin_amdgcn_sched_barrier(0);
+    {
+        h8_t h_lo, h_hi;
+        qw_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
+#pragma unroll
+        for (int t = 0; t < XT; ++t) qw_rotate_tile_to_lds(xv[t], wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs);
+    }
+    __syncthreads();
+    h2_t xo[16];
+    const float S = qmc_operands(xs + g * 5, xo);
+    const float c1 = 1024.0f * S;
+#pragma unroll
+    for (int r0 = 0; r0 < R; r0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const qw_hq4_block b = buf[j];
+            if (r0 + D + j < R) buf[j] = *(const qw_hq4_block*)(bank + row_off(r0 + D + j));
+            float v = qmc_block_dot(b, xo, S, c1);
+            v = gvalid ? v : 0.0f;
+            v = qw_reduce32_dpp(v);
+            if (lane == 31u) part[(set * R + r0 + j) * cpr + chunk] = v;
+        }
+    }
+    __syncthreads();
+    if (tid < 32u) {
+        float gsum = 0.f, usum = 0.f;
+        for (uint32_t c = 0; c < cpr; ++c) {
+            gsum += part[tid * cpr + c];
+            usum += part[(32u + tid) * cpr + c];
+        }
+        float a = qw_swiglu(gsum, usum);
+        if (p.rot_out && n0 + 32u <= I) {
+            // the butterfly order of the serial transform (pairs h apart: lower = a + b, upper = a - b), across lanes
+#pragma unroll
+            for (int h = 1; h < 32; h <<= 1) {
+                const float o = __shfl_xor(a, h, 64);
+                a = (tid & (uint32_t)h) ? o - a : a + o;
+            }
+            a *= QW_INV_SQRT32;
+        }
+        if (n0 + tid < I) act[n0 + tid] = (h1_t)a;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// down + combine: grid (ceil(H / (SETS * D)), tokens).  The token's routes are laid side by side as one virtual row of
+// top_k * nbI blocks: virtual block v belongs to route k = v / nbI, block b = v % nbI of that expert's row, so a lane's
+// column fixes its expert, its 32 activations (act[token, k, 32 b ..]) and its route weight.
+//   out[token, n] = sum_k wts[k] * (W_down[e_k][n, :] . act[k, :]) (+ shared_gate * shared[n])
+// blockDim.x = 32 * cprv * SETS, cprv = ceil(top_k * nbI / 32); set j takes rows n0 + j * D .. + D - 1.
+// ------------------------------------------------------------------------------------------------
+struct qmc_dn_params {
+    const uint8_t* bank;
+    const h1_t* act;
+    const int32_t* idx;
+    const float* wts;
+    const float* shared;
+    const float* shared_gate;
+    void* out;
+    uint32_t H, nbI, nbv, cprv, top_k, sets;
+    uint64_t expert_bytes;
+};
+
+template <int ODT, int D>
+__global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_params p) {
+    __shared__ float part[1024];   // [sets * D rows][cprv]
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 31u, hw = tid >> 5;
+    const uint32_t cprv = p.cprv, H = p.H;
+    const uint32_t set = hw / cprv, chunk = hw - set * cprv;
+    const uint32_t tok = blockIdx.y, n0 = blockIdx.x * (p.sets * D);
+    const uint32_t v0 = chunk * 32u + lane;
+    const bool vvalid = v0 < p.nbv;
+    const uint32_t v = vvalid ? v0 : 0u;
+    const uint32_t k = v / p.nbI, b = v - k * p.nbI;
+    const uint32_t pair = tok * p.top_k + k;
+    const int32_t e = p.idx[pair];
+    const float wk = p.wts[pair];
+    const bool valid = vvalid && e >= 0;
+    const uint32_t row_bytes = p.nbI * 20u;
+    // activations do not wait for the expert id; the weight rows follow as soon as it is known
+    h8_t xr[4];
+    const h8_t* xsrc = (const h8_t*)(p.act + ((uint64_t)pair * p.nbI + b) * 32u);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xr[j] = xsrc[j];
+    const uint8_t* base = p.bank + (uint64_t)(valid ? ((uint32_t)e & 0xFFFFu) : 0u) * p.expert_bytes + b * 20u;
+    qw_hq4_block buf[D];
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        const uint32_t n = min(n0 + set * D + j, H - 1u);
+        buf[j] = *(const qw_hq4_block*)(base + (uint64_t)n * row_bytes);
+    }
+    h2_t xo[16];
+    const float S = qmc_operands(xr, xo);
+    const float c1 = 1024.0f * S;
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        float r = qmc_block_dot(buf[j], xo, S, c1) * wk;
+        r = valid ? r : 0.0f;
+        r = qw_reduce32_dpp(r);
+        if (lane == 31u) part[(set * D + j) * cprv + chunk] = r;
+    }
+    __syncthreads();
+    if (tid < p.sets * D) {
+        const uint32_t n = n0 + tid;
+        if (n < H) {
+            float o = 0.f;
+            for (uint32_t c = 0; c < cprv; ++c) o += part[tid * cprv + c];
+            const uint64_t at = (uint64_t)tok * H + n;
+            if (p.shared) o = fmaf(p.shared_gate ? p.shared_gate[tok] : 1.0f, p.shared[at], o);
+            if constexpr (ODT == QWHIP_F32) ((float*)p.out)[at] = o;
+            else if constexpr (ODT == QWHIP_F16) ((h1_t*)p.out)[at] = (h1_t)o;
+            else ((uint16_t*)p.out)[at] = qw_f32_to_bf16(o);
+        }
+    }
+}
+
+}  // namespace
+
+// Routed gate|up projection with the SwiGLU (+ rotation) epilogue for a validated HQ4_G32_M5 bank; false when the shape
+// is outside the kernel's envelope (the caller then takes the general kernel).
+bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
+                       bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err) {
+    if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
+    const uint32_t inter = w->n / (2u * experts);
+    const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u;
+    if (cpr > 16u || pairs > 65535u) return false;
+    if ((uint64_t)2u * inter * nb * 20u >= (1ull << 32)) return false;   // 32-bit offsets inside an expert's sub-bank
+    const uint32_t sets = cpr <= 4u ? 8u : (cpr <= 8u ? 4u : 2u);
+    const size_t lds = (size_t)nb * 80u + (size_t)64u * cpr * 4u;
+    if (lds > 60u * 1024u) return false;
+    qmc_gu_params p;
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = x;
+    p.act = (h1_t*)act16;
+    p.idx = idx;
+    p.I = inter;
+    p.nb = nb;
+    p.cpr = cpr;
+    p.top_k = top_k;
+    p.rotate = rotate ? 1u : 0u;
+    p.rot_out = rot_out ? 1u : 0u;
+    p.expert_bytes = (uint64_t)2u * inter * nb * 20u;
+    const dim3 grid(qwhip_cdiv(inter, 32u), pairs), block(32u * cpr * sets);
+#define QMC_GU(DT, S) hipLaunchKernelGGL((qw_moe_gateup_col_kernel<DT, S>), grid, block, lds, st, p)
+    if (x_dtype == QWHIP_F16) {
+        if (sets == 8u) QMC_GU(QWHIP_F16, 8); else if (sets == 4u) QMC_GU(QWHIP_F16, 4); else QMC_GU(QWHIP_F16, 2);
+    } else {
+        if (sets == 8u) QMC_GU(QWHIP_BF16, 8); else if (sets == 4u) QMC_GU(QWHIP_BF16, 4); else QMC_GU(QWHIP_BF16, 2);
+    }
+#undef QMC_GU
+    *err = hipGetLastError();
+    return true;
+}
+
+// Routed down projection + weighted combine (+ gated shared expert) for a validated HQ4_G32_M5 bank; false when the
+// shape is outside the kernel's envelope.
+bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* act16, const int32_t* idx,
+                     const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
+                     uint32_t out_dtype, hipError_t* err) {
+    if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
+    const uint32_t hidden = w->n / experts;
+    const uint32_t nbI = w->k / 32u;
+    const uint32_t nbv = top_k * nbI, cprv = (nbv + 31u) / 32u;
+    if (cprv > 32u || t > 65535u) return false;
+    if (((uintptr_t)act16 & 15u) != 0) return false;
+    uint32_t sets = 1;
+    while (sets < 8u && 32u * cprv * sets * 2u <= 1024u) sets *= 2u;
+    constexpr int D = 2;
+    qmc_dn_params p;
+    p.bank = (const uint8_t*)w->blocks;
+    p.act = (const h1_t*)act16;
+    p.idx = idx;
+    p.wts = wts;
+    p.shared = shared;
+    p.shared_gate = shared_gate;
+    p.out = out;
+    p.H = hidden;
+    p.nbI = nbI;
+    p.nbv = nbv;
+    p.cprv = cprv;
+    p.top_k = top_k;
+    p.sets = sets;
+    p.expert_bytes = (uint64_t)hidden * nbI * 20u;
+    const dim3 grid(qwhip_cdiv(hidden, sets * D), t), block(32u * cprv * sets);
+    if (out_dtype == QWHIP_F32) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_F32, D>), grid, block, 0, st, p);
+    else if (out_dtype == QWHIP_F16) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_F16, D>), grid, block, 0, st, p);
+    else if (out_dtype == QWHIP_BF16) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_BF16, D>), grid, block, 0, st, p);
+    else return false;
+    *err = hipGetLastError();
+    return true;
+}

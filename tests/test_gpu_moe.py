@@ -149,13 +149,16 @@ def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
     assert qo.normalized_error(got, ref) <= TOL
 
 
+# (format, gate_up kernel override): HQ4_G32_M5 runs the column-stationary kernels, override 2 keeps its gate_up on the
+# general kernel; the bit-stream container runs the general kernels for both projections.
+@pytest.mark.parametrize("fmt,gu_flags", [("hq4_g32_m5", 0), ("hq4_g32_m5", 2 << 8), ("hq4_g32", 0)])
+@pytest.mark.parametrize("experts,hidden,inter,k", [(16, 512, 192, 4), (8, 1280, 96, 3), (4, 2048, 768, 4)])
 @pytest.mark.parametrize("t", [1, 3, 8])
 @pytest.mark.parametrize("xdt", ["f16", "bf16"])
-def test_moe_decode_chain_matches_oracle(dev, t, xdt):
+def test_moe_decode_chain_matches_oracle(dev, t, xdt, experts, hidden, inter, k, fmt, gu_flags):
     """Decode / verify path: routed gate_up GEMV (+SwiGLU+FWHT) and routed down GEMV with weighted combine,
-    un-rotated activations in, fused rotation."""
-    fmt, experts, hidden, inter, k = "hq4_g32_m5", 16, 512, 192, 4
-    gu_blocks, gu16, dn_blocks, dn16 = _moe_banks(experts, hidden, inter, seed=21)
+    un-rotated activations in, fused rotation; shapes with partial 32-block chunks and ragged row tiles."""
+    gu_blocks, gu16, dn_blocks, dn16 = _moe_banks(experts, hidden, inter, seed=21, fmt=fmt)
     rng = np.random.default_rng(6)
     x32 = rng.standard_normal((t, hidden)).astype(np.float32)
     if xdt == "f16":
@@ -173,7 +176,7 @@ def test_moe_decode_chain_matches_oracle(dev, t, xdt):
     act, out = dev.alloc(t * k * inter * 2), dev.alloc(t * hidden * 4)
     vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
     vdn = H.view_of(dev, dnb, fmt, experts * hidden, inter)
-    qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(vgu), experts, xb.ptr, code, 0, ib.ptr, t, k, act.ptr))
+    qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(vgu), experts, xb.ptr, code, gu_flags, ib.ptr, t, k, act.ptr))
     qwhip.check(lib.qwhip_moe_down_decode(st, C.byref(vdn), experts, act.ptr, ib.ptr, wb.ptr, t, k, sb.ptr, gb.ptr, out.ptr, qwhip.F32))
     dev.stream.sync()
     got = out.download(np.float32, (t, hidden))
