@@ -75,21 +75,39 @@ extern "C" qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint3
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ bool qw_finite(float v) { return (__float_as_uint(v) & 0x7F800000u) != 0x7F800000u; }
 
+// Wave-wide maximum / sum, uniform result: four DPP steps inside each row of 16 lanes, then four lane reads.
+#define QW_DPP_F32(v, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true))
+#define QW_LANE_F32(v, l) __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l))
+__device__ __forceinline__ float qw_wave_max(float v) {
+    v = fmaxf(v, QW_DPP_F32(v, 0xB1));
+    v = fmaxf(v, QW_DPP_F32(v, 0x4E));
+    v = fmaxf(v, QW_DPP_F32(v, 0x141));
+    v = fmaxf(v, QW_DPP_F32(v, 0x140));
+    return fmaxf(fmaxf(QW_LANE_F32(v, 0), QW_LANE_F32(v, 16)), fmaxf(QW_LANE_F32(v, 32), QW_LANE_F32(v, 48)));
+}
+__device__ __forceinline__ float qw_wave_sum(float v) {
+    v += QW_DPP_F32(v, 0xB1);
+    v += QW_DPP_F32(v, 0x4E);
+    v += QW_DPP_F32(v, 0x141);
+    v += QW_DPP_F32(v, 0x140);
+    return (QW_LANE_F32(v, 0) + QW_LANE_F32(v, 16)) + (QW_LANE_F32(v, 32) + QW_LANE_F32(v, 48));
+}
+
+template <int JN>   // experts per lane: E <= 64 * JN
 __global__ __launch_bounds__(64) void qw_moe_route_kernel(const float* __restrict__ logits, int32_t* __restrict__ idx,
                                                            float* __restrict__ wts, uint32_t E, uint32_t K, uint32_t norm,
                                                            float routed_scale) {
     const uint32_t t = blockIdx.x, lane = threadIdx.x;
-    const uint32_t JN = (E + 63u) >> 6;
-    float p[8];
-    bool ok[8];
+    float p[JN];
+    bool ok[JN];
     float mx = -3.4e38f;
     bool any_finite = false;
 #pragma unroll
-    for (uint32_t j = 0; j < 8; ++j) {
+    for (uint32_t j = 0; j < JN; ++j) {
         const uint32_t id = lane + 64u * j;
         float v = 0.0f;
         ok[j] = false;
-        if (j < JN && id < E) {
+        if (id < E) {
             v = logits[(uint64_t)t * E + id];
             ok[j] = qw_finite(v);
             if (ok[j]) {
@@ -99,52 +117,43 @@ __global__ __launch_bounds__(64) void qw_moe_route_kernel(const float* __restric
         }
         p[j] = v;
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = qw_wave_max(mx);
     float total = 0.0f;
 #pragma unroll
-    for (uint32_t j = 0; j < 8; ++j) {
+    for (uint32_t j = 0; j < JN; ++j) {
         p[j] = ok[j] ? expf(p[j] - mx) : 0.0f;
         total += p[j];
     }
-    total = qw_reduce64(total);
+    total = qw_wave_sum(total);
 #pragma unroll
-    for (uint32_t j = 0; j < 8; ++j) {
+    for (uint32_t j = 0; j < JN; ++j) {
         ok[j] = ok[j] && total > 0.0f;
         p[j] = ok[j] ? p[j] / total : -1e30f;
     }
     // Selection rounds on the scalar unit: the wave maximum comes from four DPP steps inside each row of 16 lanes and
     // four lane reads, the owner of the maximum from ballots in ascending expert order (ties go to the lower id).
     // Cross-lane permutes through LDS would put two dependent ~100-clock round trips on every one of the 6 x top_k steps.
-    float cand[8];
+    float cand[JN];
 #pragma unroll
-    for (uint32_t j = 0; j < 8; ++j) cand[j] = ok[j] ? p[j] : -1.0f;   // probabilities are >= 0
+    for (uint32_t j = 0; j < JN; ++j) cand[j] = ok[j] ? p[j] : -1.0f;   // probabilities are >= 0
     float wsel = 0.0f;  // lane r keeps the weight of rank r (K <= 16 < 64)
     int32_t isel = -1;
     for (uint32_t r = 0; r < K; ++r) {
         float lm = cand[0];
 #pragma unroll
-        for (uint32_t j = 1; j < 8; ++j) lm = fmaxf(lm, cand[j]);
-        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0xB1, 0xF, 0xF, true)));
-        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0x4E, 0xF, 0xF, true)));
-        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0x141, 0xF, 0xF, true)));
-        lm = fmaxf(lm, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, lm), 0x140, 0xF, 0xF, true)));
-        const int lmi = __builtin_bit_cast(int, lm);
-        const float wm = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 0)),
-                                     __builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 16))),
-                               fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 32)),
-                                     __builtin_bit_cast(float, __builtin_amdgcn_readlane(lmi, 48))));
+        for (uint32_t j = 1; j < JN; ++j) lm = fmaxf(lm, cand[j]);
+        const float wm = qw_wave_max(lm);
         uint32_t bi = 0xFFFFFFFFu;
         if (wm >= 0.0f) {
 #pragma unroll
-            for (uint32_t j = 0; j < 8; ++j) {
+            for (uint32_t j = 0; j < JN; ++j) {
                 const unsigned long long m = __ballot(cand[j] == wm);
                 if (bi == 0xFFFFFFFFu && m != 0ull) bi = 64u * j + (uint32_t)__builtin_ctzll(m);
             }
         }
         if (bi != 0xFFFFFFFFu && (bi & 63u) == lane) {
 #pragma unroll
-            for (uint32_t j = 0; j < 8; ++j)
+            for (uint32_t j = 0; j < JN; ++j)
                 if (j == (bi >> 6)) cand[j] = -1.0f;
         }
         if (lane == r) {
@@ -175,8 +184,13 @@ extern "C" qwhip_status qwhip_moe_route(qwhip_stream_t s, const float* logits, u
     if (experts == 0 || experts > 512) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: experts must be 1..512, got %u", experts);
     if (top_k == 0 || top_k > 16) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: top_k must be 1..16, got %u", top_k);
     const float scale = routed_scale > 0.0f ? routed_scale : 1.0f;
-    hipLaunchKernelGGL(qw_moe_route_kernel, dim3(t), dim3(64), 0, s->stream, logits, idx, wts, experts, top_k,
-                       norm_topk ? 1u : 0u, scale);
+#define QW_ROUTE(J) hipLaunchKernelGGL(qw_moe_route_kernel<J>, dim3(t), dim3(64), 0, s->stream, logits, idx, wts, experts, top_k, \
+                                       norm_topk ? 1u : 0u, scale)
+    if (experts <= 64) QW_ROUTE(1);
+    else if (experts <= 128) QW_ROUTE(2);
+    else if (experts <= 256) QW_ROUTE(4);
+    else QW_ROUTE(8);
+#undef QW_ROUTE
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
