@@ -222,7 +222,8 @@ qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint32_t dn_dty
 /* Decode / verify (t <= 8) routed experts as GEMVs: encodeMoEGateUpF32R1 + encodeMoEDownSharedCombineF32
  * (QWGemmMoE.swift:120-199) -> Sources/QWMetal/include/qw_moe_f32_common.metalh:187-452.
  * gate_up: act16 [t, top_k, inter] = f16(FWHT32(silu(Wg[e].x) * (Wu[e].x))), SwiGLU on fp32 accumulators.
- * down:    out [t, hidden] = sum_k wts[t,k] * Wd[e_k] . act16[t,k]  (+ shared_gate[t]*shared[t]). */
+ * down:    out [t, hidden] = sum_k wts[t,k] * Wd[e_k] . act16[t,k]  (+ shared_gate[t]*shared[t]).
+ * gate_up flags: QWHIP_X_PREROTATED; bits 8..11 = 2 keep an HQ4_G32_M5 bank on the general kernel (tests). */
 qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
                                      const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
                                      uint32_t top_k, void* act16);
