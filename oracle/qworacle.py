@@ -334,6 +334,23 @@ def weights_f16_exact(blocks: np.ndarray, bits: int, group: int, is_m5: bool) ->
     return (q * s.astype(np.float64)[..., None] + b.astype(np.float64)[..., None]).astype(np.float16).reshape(n, nb * group)
 
 
+def weights_affine_f64(blocks: np.ndarray, bits: int, group: int, is_m5: bool) -> np.ndarray:
+    """The un-rounded real weights (q+1024)*s + b (M5) / code*s + b (blocks) in float64: what the reference's
+    factorised GEMVs contract, scale * sum(code * x) + bias * sum(x) per slice (qwg_aq_slice_dot,
+    Sources/QWMetal/include/qw_dequant_multi.metalh:205-208).  Differs from `weights_f16_exact` only by the f16
+    rounding of each weight; pinned through it (same codes, same headers)."""
+    if is_m5:
+        n, g, _ = blocks.shape
+        s = np.ascontiguousarray(blocks[..., 0:2]).view(np.float16).astype(np.float64)
+        b = np.ascontiguousarray(blocks[..., 2:4]).view(np.float16).astype(np.float64)
+        q = hq4_codes(blocks).astype(np.float64)
+        return ((q + 1024.0) * s + b).reshape(n, g * GROUP)
+    n, nb, _ = blocks.shape
+    s, b = hq_block_header(blocks)
+    q = hq_block_codes(blocks, bits, group).astype(np.float64)
+    return (q * s.astype(np.float64)[..., None] + b.astype(np.float64)[..., None]).reshape(n, nb * group)
+
+
 # --------------------------------------------------------------------------- #
 # planar HQ8_G32_M5  (pinned: golden selfpack_hq8.qwp + .dq8rot.f32.bin, hq_blocks_golden hq8_planar)
 # --------------------------------------------------------------------------- #

@@ -15,7 +15,6 @@
 //    through LDS.  VALU does only the dequant; accumulation rides on the matrix cores.
 #include "qwhip_common.h"
 
-enum { QW_FMT_M5 = 0, QW_FMT_B4 = 1, QW_FMT_B8 = 2 };
 enum { QW_XM_GLOBAL = 0, QW_XM_LDS_ROT = 1 };
 
 // ------------------------------------------------------------------------------------------------
@@ -723,12 +722,17 @@ bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expert
                      const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
                      uint32_t out_dtype, hipError_t* err);
 
+// gemv_colx.hip
+bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                  const void* x, uint32_t x_dtype, uint32_t m, bool rotate, void* y16, float* y32, uint32_t tune,
+                  hipError_t* err);
+
 // gemv_col.hip
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
                  float* y32, uint32_t tune, hipError_t* err);
 
 // flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer,
-// 4 = column-stationary persistent kernel, 5 = column-stationary MFMA kernel);
+// 4 = column-stationary persistent kernel, 5 = column-stationary MFMA kernel, 6 = column-stationary small-M kernel);
 // bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer / tuning code of the
 // column-stationary kernel (0 = automatic).
 extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
@@ -758,6 +762,20 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     const size_t lds_dot2 = (size_t)(w->k / 32) * 80u;
     const bool dot2_ok = fmt == QW_FMT_M5 && m == 1 && lds_dot2 <= 60u * 1024u;
     if (variant == 1 && !dot2_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "dot2 kernel needs HQ4_G32_M5, m = 1, k <= 24576");
+    // column-stationary small-M kernel: one row (rotation fused where needed), or up to eight rows already in the basis.
+    // Its VALU work grows with m (16 dot2 per slice and row): from five rows on, short rows go to the column-stationary
+    // MFMA kernel below, which measured faster there (N = 7168, K = 5120, m = 8: 16.5 against 20.1 us).
+    // HQ4_G32_M5 at m = 1 has its own kernel.
+    const bool colx_shape = (m == 1 || !rotate) && m <= 8;
+    if (variant == 6 || (variant == 0 && colx_shape && !(fmt == QW_FMT_M5 && m == 1) && (m <= 4 || w->k > 5120u))) {
+        hipError_t e = hipSuccess;
+        if (colx_shape && qw_colx_gemv(s->stream, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, rotate, y16, y32, rt, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+        if (variant == 6)
+            return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the column-stationary small-M kernel takes m = 1, or m <= 8 rows already in the basis, on rows that fit one workgroup");
+    }
     // automatic choice: the DMA streamer where it measured faster than the direct-load kernel (few row tiles, short rows,
     // one or two activation rows), the direct-load kernel otherwise
     const bool stream_auto = !dot2_ok && m <= 2 && w->n <= 4096 && w->k <= 8192;

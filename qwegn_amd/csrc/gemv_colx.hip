@@ -1,0 +1,300 @@
+// Small-M GEMV over any 4- or 8-bit container, column-stationary persistent form: m = 1..8 activation rows already in
+// the container's basis, or one row with the FWHT-32 fused in front.
+//
+// Same launch shape as the m = 1 HQ4 kernel of gemv_col.hip: a fixed population of workgroups walks the bank once
+// (row slot s of workgroup w is bank row s * gridDim.x + w, so the grid reads one contiguous band of rows at a time);
+// a 32-lane half-wavefront (set, chunk) owns slice columns 32 * chunk .. + 31 (a slice = 32 columns) of the rows
+// set, set + sets, ...  Consecutive lanes read consecutive slices of a row: every load instruction covers a
+// contiguous run of the bank.  A lane keeps its 32 activations of each of the MR activation rows in registers
+// (16 f16 pairs per row), so the row loop has no activation traffic and its cost per weight byte grows only by
+// 16 v_dot2_f32_f16 per extra activation row.
+//
+// Arithmetic.  The packed codes are used directly as f16 operands: a 4-bit code masked in place at bits 0..3 / 16..19
+// of a word reads as the f16 subnormal q * 2^-24 (at bits 4..7 / 20..23 as 16 q * 2^-24), an 8-bit code at bits
+// 0..7 / 16..23 likewise (v_dot2_f32_f16 honours f16 subnormals; products are exact, accumulation is fp32).  The affine
+// part is applied once per slice:  sum_i w_i x_i = s * sum_i q_i x_i + b * S,  S = sum_i x_i  (HQ4_G32_M5:
+// s * (sum_i q_i x_i + 1024 S) + b * S) - the factorisation of the reference's bit-stream GEMVs
+// (qwg_aq_slice_dot, Sources/QWMetal/include/qw_dequant_multi.metalh:205-208).
+// Element order inside a word fixes which activations pair up: HQ4_G32_M5 keeps element 8w + j at bit
+// 4 (j >> 1) + 16 (j & 1) (unpack_hq4_word8, qw_dequant.metalh:42-62), the bit-stream containers element i at bit
+// i * bits, so a masked 4-bit word holds elements (k, k + 4) and a masked 8-bit word elements (k, k + 2).
+#include "qwhip_common.h"
+
+namespace {
+
+struct qcx_params {
+    const uint8_t* bank;
+    const void* x;
+    h1_t* y16;
+    float* y32;
+    uint32_t N, K, M, nsl, cpr, sets, gshift, bb, row_bytes;
+};
+
+struct __attribute__((packed, aligned(4))) qcx_words4 { uint32_t q[4]; };
+struct __attribute__((packed, aligned(4))) qcx_words8 { uint32_t q[8]; };
+
+template <int FMT>
+struct qcx_slice {
+    uint32_t hdr;
+    uint32_t q[FMT == QW_FMT_B8 ? 8 : 4];
+};
+
+// The 16 operand pairs of one activation row for this lane's slice, in the order the masked code words come out.
+template <int FMT>
+__device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
+    const h2_t one = {(h1_t)1.0f, (h1_t)1.0f};
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            h2_t pr;
+            if constexpr (FMT == QW_FMT_M5) pr = h2_t{v[j][2 * k], v[j][2 * k + 1]};
+            else if constexpr (FMT == QW_FMT_B4) pr = h2_t{v[j][k], v[j][k + 4]};
+            else pr = h2_t{v[j][4 * (k >> 1) + (k & 1)], v[j][4 * (k >> 1) + (k & 1) + 2]};
+            if (k & 1) s1 = __builtin_amdgcn_fdot2(pr, one, s1, false);
+            else s0 = __builtin_amdgcn_fdot2(pr, one, s0, false);
+            xo[4 * j + k] = pr;
+        }
+    }
+    return s0 + s1;
+}
+
+// MR activation rows, D slices in flight per lane.  blockDim.x = 32 * cpr * sets;
+// dynamic LDS = rows-per-workgroup * cpr * MR * 4 bytes (+ nsl * 80 bytes in front with ROT).
+// ROT (MR = 1 only): the activation row arrives un-rotated; the FWHT-32 of its groups runs on the matrix cores into
+// an LDS image (16 groups per wave and tile), and each lane then reads its own column from there.
+template <int FMT, int XDT, int MR, int D, int LB, bool ROT>
+__global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
+    static_assert(!ROT || MR == 1, "fused rotation is built for one activation row");
+    extern __shared__ h8_t qcx_lds[];
+    h8_t* xs = qcx_lds;                                                     // ROT: 80 bytes per 32-group (64 used)
+    float* qcx_part = (float*)(qcx_lds + (ROT ? (size_t)p.nsl * 5 : 0));    // [row slot][chunk][MR]
+    const uint32_t cpr = p.cpr, N = p.N, sets = p.sets;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 31u, hw = tid >> 5;
+    const uint32_t set = hw / cpr, chunk = hw - set * cpr;
+    const uint32_t g0 = chunk * 32u + lane;
+    const bool gvalid = g0 < p.nsl;
+    const uint32_t g = gvalid ? g0 : p.nsl - 1u;
+    const uint32_t G = gridDim.x;
+    if (blockIdx.x >= N) return;
+    const uint32_t nrows = (N - blockIdx.x + G - 1u) / G;   // row slots of this workgroup
+    const uint32_t nmax = (nrows + sets - 1u) / sets;       // trip count, uniform over the workgroup
+    const uint32_t step = G * sets * p.row_bytes;            // bytes between consecutive rows of one set
+    const uint32_t mine = nrows > set ? (nrows - set + sets - 1u) / sets : 0u;
+    uint32_t hdr_off, pay_off;
+    if constexpr (FMT == QW_FMT_M5) {
+        hdr_off = g * 20u;
+        pay_off = hdr_off + 4u;
+    } else {
+        hdr_off = (g >> p.gshift) * p.bb;
+        pay_off = hdr_off + 4u + (g & ((1u << p.gshift) - 1u)) * (FMT == QW_FMT_B8 ? 32u : 16u);
+    }
+    uint32_t off = ((mine ? set : 0u) * G + blockIdx.x) * p.row_bytes;
+    const uint32_t off_max = off + (mine ? mine - 1u : 0u) * step;   // loads past the set's last row re-read it
+
+    // 1. activation loads first (they return in order, ahead of the weight prefetch); rows past M re-read row M - 1
+    u4_t xraw[MR][4];   // 8 two-byte activations per register quad, converted one activation row at a time below
+    constexpr int XT = 5;                                  // rotation tiles per wave: covers 2 * cpr tiles over cpr / 2 waves
+    h8_t xv[ROT ? XT : 1];
+    const uint32_t wave = tid >> 6, l64 = tid & 63u, nwf = blockDim.x >> 6;   // full waves only take rotation tiles
+    if constexpr (ROT) {
+#pragma unroll
+        for (int t = 0; t < XT; ++t) {
+            const uint32_t gg = min((wave + nwf * t) * 16u + (l64 & 15u), p.nsl - 1u);
+            xv[t] = qw_load_x8_f16<XDT>(p.x, (uint64_t)gg * 32u + 8u * (l64 >> 4));
+        }
+    } else {
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const uint64_t at = (uint64_t)min((uint32_t)m, p.M - 1u) * p.K + (uint64_t)g * 32u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xraw[m][j] = *(const u4_t*)((const uint16_t*)p.x + at + 8u * j);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // 2. first weight rows
+    qcx_slice<FMT> buf[D];
+    auto issue = [&](int slot) {
+        const uint8_t* rp = p.bank + off;
+        buf[slot].hdr = *(const uint32_t*)(rp + hdr_off);
+        if constexpr (FMT == QW_FMT_B8) {
+            const qcx_words8 w = *(const qcx_words8*)(rp + pay_off);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) buf[slot].q[j] = w.q[j];
+        } else {
+            const qcx_words4 w = *(const qcx_words4*)(rp + pay_off);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) buf[slot].q[j] = w.q[j];
+        }
+        off = min(off + step, off_max);
+    };
+#pragma unroll
+    for (int j = 0; j < D; ++j) issue(j);
+    __builtin_amdgcn_sched_barrier(0);
+    // 3. this lane's operands
+    if constexpr (ROT) {
+        if (wave < nwf) {
+            h8_t h_lo, h_hi;
+            qw_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
+#pragma unroll
+            for (int t = 0; t < XT; ++t) qw_rotate_tile_to_lds(xv[t], wave + nwf * t, p.nsl, l64, true, h_lo, h_hi, xs);
+        }
+        __syncthreads();
+    }
+    h2_t xo[MR][16];
+    float S[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        h8_t xr[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (ROT) {
+                xr[j] = xs[g * 5u + j];
+            } else if constexpr (XDT == QWHIP_F16) {
+                xr[j] = __builtin_bit_cast(h8_t, xraw[m][j]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    xr[j][2 * e] = (h1_t)__uint_as_float(xraw[m][j][e] << 16);
+                    xr[j][2 * e + 1] = (h1_t)__uint_as_float(xraw[m][j][e] & 0xFFFF0000u);
+                }
+            }
+        }
+        S[m] = qcx_operands<FMT>(xr, xo[m]);
+        __builtin_amdgcn_sched_barrier(0);   // keeps the conversion of row m + 1 from overlapping row m's registers
+    }
+
+    uint32_t rslot = set;   // row slot being consumed
+    for (uint32_t ib = 0; ib < nmax; ib += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            if (ib + j >= nmax) break;
+            const qcx_slice<FMT> b = buf[j];
+            issue(j);
+            uint32_t ow[16];   // masked code words, operand order
+            if constexpr (FMT == QW_FMT_B8) {
+#pragma unroll
+                for (int w = 0; w < 8; ++w) {
+                    ow[2 * w] = b.q[w] & 0x00FF00FFu;
+                    ow[2 * w + 1] = (b.q[w] >> 8) & 0x00FF00FFu;
+                }
+            } else {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t q = b.q[w], q8 = q >> 8;
+                    ow[4 * w + 0] = q & 0x000F000Fu;
+                    ow[4 * w + 1] = q & 0x00F000F0u;
+                    ow[4 * w + 2] = q8 & 0x000F000Fu;
+                    ow[4 * w + 3] = q8 & 0x00F000F0u;
+                }
+            }
+            const h2_t hd = __builtin_bit_cast(h2_t, b.hdr);
+            const float sc = (float)hd[0], bi = (float)hd[1];
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+                for (int i = 0; i < 16; i += 4) {
+                    a0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 0]), xo[m][i + 0], a0, false);
+                    a1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 1]), xo[m][i + 1], a1, false);
+                    a2 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 2]), xo[m][i + 2], a2, false);
+                    a3 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 3]), xo[m][i + 3], a3, false);
+                }
+                float q;
+                if constexpr (FMT == QW_FMT_B8) {
+                    q = ((a0 + a1) + (a2 + a3)) * 16777216.0f;
+                } else {
+                    q = __builtin_fmaf(a0 + a2, 16777216.0f, FMT == QW_FMT_M5 ? 1024.0f * S[m] : 0.0f);   // codes at bits 0..3
+                    q = __builtin_fmaf(a1 + a3, 1048576.0f, q);                                           // codes at bits 4..7
+                }
+                float v = __builtin_fmaf(sc, q, bi * S[m]);
+                v = gvalid ? v : 0.0f;
+                v = qw_reduce32_dpp(v);
+                if (lane == 31u && rslot < nrows) qcx_part[(rslot * cpr + chunk) * MR + m] = v;
+            }
+            rslot += sets;
+        }
+    }
+    __syncthreads();
+    // 4. fixed-order sum of the chunk partials of each (row, activation row)
+    for (uint32_t t = tid; t < nrows * p.M; t += blockDim.x) {
+        const uint32_t m = t / nrows, s = t - m * nrows;
+        float v = 0.f;
+        for (uint32_t c = 0; c < cpr; ++c) v += qcx_part[(s * cpr + c) * MR + m];
+        const uint64_t at = (uint64_t)m * N + s * G + blockIdx.x;
+        if (p.y32) p.y32[at] = v;
+        if (p.y16) p.y16[at] = (h1_t)v;
+    }
+}
+
+template <int FMT, int XDT, int MR, int D, int LB, bool ROT = false>
+void qcx_launch1(hipStream_t st, const qcx_params& p, uint32_t wgs, uint32_t threads, size_t lds) {
+    hipLaunchKernelGGL((qw_gemv_colx_kernel<FMT, XDT, MR, D, LB, ROT>), dim3(wgs), dim3(threads), lds, st, p);
+}
+
+template <int FMT, int XDT>
+void qcx_launch_m(hipStream_t st, const qcx_params& p, uint32_t mr, bool rotate, uint32_t wgs, uint32_t threads, size_t lds) {
+    if (rotate) qcx_launch1<FMT, XDT, 1, 2, 1024, true>(st, p, wgs, threads, lds);
+    else if (mr == 1) qcx_launch1<FMT, XDT, 1, 2, 1024>(st, p, wgs, threads, lds);
+    else if (mr == 2) qcx_launch1<FMT, XDT, 2, 2, 1024>(st, p, wgs, threads, lds);
+    else if (mr == 4) qcx_launch1<FMT, XDT, 4, 3, 576>(st, p, wgs, threads, lds);
+    else qcx_launch1<FMT, XDT, 8, 3, 512>(st, p, wgs, threads, lds);
+}
+
+}  // namespace
+
+// Tries the column-stationary small-M kernel for a validated call; false when the shape is outside its envelope:
+// up to eight activation rows already in the container's basis, or one row to rotate (`rotate`).
+// fmt: QW_FMT_M5 / QW_FMT_B4 / QW_FMT_B8.  `tune`: 0 = automatic; bits 0..1 scale the grid (1 -> half, 2 -> double).
+bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                  const void* x, uint32_t x_dtype, uint32_t m, bool rotate, void* y16, float* y32, uint32_t tune,
+                  hipError_t* err) {
+    if (m == 0 || m > 8 || (rotate && m != 1)) return false;
+    const uint32_t mr = m <= 1 ? 1u : (m <= 2 ? 2u : (m <= 4 ? 4u : 8u));
+    const uint32_t nsl = w->k / 32u, cpr = (nsl + 31u) / 32u;
+    // threads per workgroup follow the register budget: 128 VGPRs up to two activation rows, 170 for four, 256 for eight
+    const uint32_t lb = mr <= 2 ? 1024u : (mr == 4 ? 576u : 512u);
+    const uint32_t waves_cu = mr <= 2 ? 16u : (mr == 4 ? 12u : 8u);
+    if (32u * cpr > lb) return false;
+    if ((uint64_t)w->n * row_bytes >= (1ull << 32)) return false;   // 32-bit offsets inside the bank
+    if (((uintptr_t)x & 15u) != 0) return false;
+    uint32_t sets = lb / (32u * cpr);
+    sets = min(sets, 8u);
+    const uint32_t threads = 32u * cpr * sets;
+    const uint32_t waves = (threads + 63u) / 64u;
+    uint32_t wgs = 256u * max(1u, waves_cu / waves);
+    if ((tune & 3u) == 1u) wgs /= 2u;
+    if ((tune & 3u) == 2u) wgs *= 2u;
+    wgs = min(wgs, max(1u, w->n / sets));
+    const uint32_t rows_per_wg = qwhip_cdiv(w->n, wgs);
+    if (rotate && (threads >> 6) * 5u * 16u < nsl) return false;   // rotation tiles: five per full wave
+    const size_t lds = (size_t)rows_per_wg * cpr * mr * 4u + (rotate ? (size_t)nsl * 80u : 0u);
+    if (lds > 60u * 1024u) return false;
+    qcx_params p;
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = x;
+    p.y16 = (h1_t*)y16;
+    p.y32 = y32;
+    p.N = w->n;
+    p.K = w->k;
+    p.M = m;
+    p.nsl = nsl;
+    p.cpr = cpr;
+    p.sets = sets;
+    p.gshift = gshift;
+    p.bb = bb;
+    p.row_bytes = (uint32_t)row_bytes;
+    if (x_dtype == QWHIP_F16) {
+        if (fmt == QW_FMT_M5) qcx_launch_m<QW_FMT_M5, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B4) qcx_launch_m<QW_FMT_B4, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
+        else qcx_launch_m<QW_FMT_B8, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
+    } else {
+        if (fmt == QW_FMT_M5) qcx_launch_m<QW_FMT_M5, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B4) qcx_launch_m<QW_FMT_B4, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
+        else qcx_launch_m<QW_FMT_B8, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
+    }
+    *err = hipGetLastError();
+    return true;
+}

@@ -53,6 +53,9 @@ typedef float f16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
 
+// GEMV container families: HQ4_G32_M5 20-byte blocks, 4-bit and 8-bit bit-stream blocks.
+enum { QW_FMT_M5 = 0, QW_FMT_B4 = 1, QW_FMT_B8 = 2 };
+
 #define QW_INV_SQRT32 0.17677669529663689f /* f32(1/sqrt(32)) = 0x3E3504F3 */
 
 // One HQ4_G32_M5 block: [f16 scale][f16 bias][u32 qs[4]], 4-byte aligned in a bank.

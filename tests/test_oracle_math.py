@@ -68,6 +68,26 @@ def test_f16_weight_closed_form_brute_force():
             assert w8[i] == _rn_f16(exact), (s16, i)
 
 
+def test_affine_weights_are_the_exact_values_behind_the_f16_weights():
+    """weights_affine_f64 is the un-rounded (q+1024)*s + b / code*s + b: exact rational arithmetic on a few blocks,
+    and rounding it to f16 reproduces weights_f16_exact on seeded banks of every container family."""
+    s16, b16 = np.float16(0.0123), np.float16(-0.071)
+    blk = np.zeros((1, 1, 36), dtype=np.uint8)
+    blk[0, 0, 0:2] = np.array([s16]).view(np.uint8)
+    blk[0, 0, 2:4] = np.array([b16]).view(np.uint8)
+    codes = (np.arange(32) * 29 + 3) % 256
+    blk[0, 0, 4:] = codes
+    w = qo.weights_affine_f64(blk, 8, 32, False)[0]
+    for i in range(32):
+        assert Fraction(float(w[i])) == int(codes[i]) * Fraction(float(s16)) + Fraction(float(b16))
+    rng = np.random.default_rng(3)
+    wsrc = (rng.standard_normal((8, 256)) * 0.02).astype(np.float32)
+    for bits, group, is_m5 in [(4, 32, True), (4, 32, False), (4, 64, False), (8, 32, False), (8, 128, False)]:
+        blocks, _ = qo.quant_hq_blocks(wsrc, bits=bits, group=group, is_m5=is_m5, rotate=True)
+        exact = qo.weights_affine_f64(blocks, bits, group, is_m5)
+        assert np.array_equal(exact.astype(np.float16), qo.weights_f16_exact(blocks, bits, group, is_m5))
+
+
 def test_hq4_nibble_order_matches_the_scalar_reader():
     """Element 8w+j sits at bit 4*(j>>1) + 16*(j&1) of word w (QWAQProducer.swift:85-87; reader shifts
     0,16,4,20,8,24,12,28 in QWQuant+DequantMath.swift:82-89)."""
