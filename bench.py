@@ -437,7 +437,7 @@ def main() -> None:
     ap.add_argument("--m", type=int, default=8, help="activation rows for the c5 workloads")
     ap.add_argument("--hot", action="store_true", help="single bank (Infinity-Cache resident) instead of the cold ring")
     ap.add_argument("--ring-mb", type=float, default=640.0)
-    ap.add_argument("--variant", type=int, default=0, help="gemv kernel override (0 auto, 1 dot2, 2 mfma)")
+    ap.add_argument("--variant", type=int, default=0, help="gemv kernel override (0 auto; 1..7 as the flags of qwhip_gemv)")
     ap.add_argument("--rt", type=int, default=0, help="row tiles per wave for the mfma gemv (0 auto)")
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")

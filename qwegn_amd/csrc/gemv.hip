@@ -722,6 +722,10 @@ bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expert
                      const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
                      uint32_t out_dtype, hipError_t* err);
 
+// gemv_quad.hip
+bool qw_quad_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                  const void* x, uint32_t x_dtype, uint32_t m, void* y16, float* y32, uint32_t tune, hipError_t* err);
+
 // gemv_colx.hip
 bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
                   const void* x, uint32_t x_dtype, uint32_t m, bool rotate, void* y16, float* y32, uint32_t tune,
@@ -732,7 +736,8 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
                  float* y32, uint32_t tune, hipError_t* err);
 
 // flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer,
-// 4 = column-stationary persistent kernel, 5 = column-stationary MFMA kernel, 6 = column-stationary small-M kernel);
+// 4 = column-stationary persistent kernel, 5 = column-stationary MFMA kernel, 6 = column-stationary small-M kernel,
+// 7 = 4x4x4-block MFMA kernel);
 // bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer / tuning code of the
 // column-stationary kernel (0 = automatic).
 extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
@@ -762,12 +767,11 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     const size_t lds_dot2 = (size_t)(w->k / 32) * 80u;
     const bool dot2_ok = fmt == QW_FMT_M5 && m == 1 && lds_dot2 <= 60u * 1024u;
     if (variant == 1 && !dot2_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "dot2 kernel needs HQ4_G32_M5, m = 1, k <= 24576");
-    // column-stationary small-M kernel: one row (rotation fused where needed), or up to eight rows already in the basis.
-    // Its VALU work grows with m (16 dot2 per slice and row): from five rows on, short rows go to the column-stationary
-    // MFMA kernel below, which measured faster there (N = 7168, K = 5120, m = 8: 16.5 against 20.1 us).
-    // HQ4_G32_M5 at m = 1 has its own kernel.
+    // column-stationary dot2 kernel: one row (rotation fused where needed); it also takes up to eight rows already in the
+    // basis (override 6), but its VALU work grows with m (16 dot2 per slice and row).  HQ4_G32_M5 at m = 1 has its own kernel.
+    // From two rows on the 4x4x4-block MFMA kernel further below is faster (its cost does not grow with 16 dot2 per row).
     const bool colx_shape = (m == 1 || !rotate) && m <= 8;
-    if (variant == 6 || (variant == 0 && colx_shape && !(fmt == QW_FMT_M5 && m == 1) && (m <= 4 || w->k > 5120u))) {
+    if (variant == 6 || (variant == 0 && colx_shape && !(fmt == QW_FMT_M5 && m == 1) && m == 1)) {
         hipError_t e = hipSuccess;
         if (colx_shape && qw_colx_gemv(s->stream, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, rotate, y16, y32, rt, &e)) {
             QWHIP_TRY_HIP(e);
@@ -778,7 +782,7 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     }
     // automatic choice: the DMA streamer where it measured faster than the direct-load kernel (few row tiles, short rows,
     // one or two activation rows), the direct-load kernel otherwise
-    const bool stream_auto = !dot2_ok && m <= 2 && w->n <= 4096 && w->k <= 8192;
+    const bool stream_auto = !dot2_ok && rotate && m <= 2 && w->n <= 4096 && w->k <= 8192;   // rows already in the basis: kernels below
     if (variant == 3 || (variant == 0 && stream_auto)) {
         hipError_t e = hipSuccess;
         if (qw_stream_gemv(s->stream, w, x, x_dtype, m, rotate, y16, y32, rt, &e)) {
@@ -813,6 +817,17 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
         return QWHIP_OK;
     }
 
+    // 4x4x4-block MFMA kernel: activations already in the basis.  Measured best for 2..8 rows (N = 7168, K = 5120, HQ8:
+    // 11.3 / 12.0 / 13.3 us at m = 2 / 4 / 8) and up to 12 rows on rows too long for the column-stationary MFMA kernel
+    // (N = 5120, K = 17408, HQ4_G64: 22.9 us at m = 8, 29.6 at m = 12 against 39-40 for the streamer).
+    if (variant == 7 || (variant == 0 && !rotate && m >= 2 && (m <= 8 || (m <= 12 && w->k > 5120u)))) {
+        hipError_t e = hipSuccess;
+        if (!rotate && qw_quad_gemv(s->stream, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, y16, y32, rt, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+        if (variant == 7) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the 4x4x4-block kernel needs activations in the basis");
+    }
     // column-stationary MFMA kernel: activations already in the basis (verify rows, standard-basis containers), k <= 5120
     if (variant == 5 || (variant == 0 && !rotate)) {
         bool done = false;

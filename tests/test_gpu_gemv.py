@@ -173,6 +173,30 @@ def test_gemv_column_stationary_fused_rotation(dev, fmt, xdtype, n, k):
     assert qo.normalized_error(g16, ref) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "aq4_g32", "hq4_g32", "hq4_g64", "hq4_g128", "hq8_g32", "hq8_g64", "aq8_g256"])
+@pytest.mark.parametrize("m", [1, 3, 5, 8, 13, 16])
+def test_gemv_block_mfma_kernel(dev, fmt, m):
+    """4x4x4-block MFMA kernel (override 7), activations handed over in the basis: tight against the factorised form,
+    inside the judged bar against the f16-weight reference.  n = 270 ends in a partial row quad, k = 1536 = 3 chunks
+    of 16 slices."""
+    g16, g32, ref = _run_gemv(dev, fmt, 270, 1536, m, prerot=True, seed=5, variant=7)
+    assert qo.normalized_error(g32, _affine_ref(fmt, 270, 1536, m, 5)) <= 2e-5
+    assert qo.normalized_error(g32, ref) <= TOL
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt,n,k,m,xdtype", [("hq4_g64", 96, 17408, 8, "f16"), ("hq4_g64", 50, 17408, 16, "f16"),
+                                              ("aq4_g32", 300, 2080, 6, "bf16"), ("aq8_g256", 64, 5120, 16, "bf16"),
+                                              ("hq8_g32", 5, 64, 2, "f16")])
+def test_gemv_block_mfma_kernel_k_ranges_and_dtypes(dev, fmt, n, k, m, xdtype):
+    """Long rows take several K ranges (k = 17408: three ranges of 12 chunks, partials accumulate in LDS); k = 2080 ends
+    in a partial chunk; bf16 activations on the standard-basis containers; a bank smaller than one row quad per set."""
+    prerot = H.FORMATS[fmt][4]
+    g16, g32, ref = _run_gemv(dev, fmt, n, k, m, prerot=prerot, xdtype=xdtype, seed=8, variant=7)
+    assert qo.normalized_error(g32, _affine_ref(fmt, n, k, m, 8, "f16" if prerot else xdtype)) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
 @pytest.mark.parametrize("m", [1, 4])
 def test_gemv_column_stationary_long_rows(dev, m):
     """k = 17408: 17 half-waves per row, one row set per workgroup."""
