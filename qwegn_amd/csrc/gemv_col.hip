@@ -147,16 +147,18 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
 
 template <int XDT, int SETS>
 hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t threads, size_t lds, uint32_t depth) {
-    if (depth == 2) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 1>), dim3(wgs), dim3(threads), lds, st, p);
-    else if (depth == 4) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 4, 1>), dim3(wgs), dim3(threads), lds, st, p);
-    else hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 3, 1>), dim3(wgs), dim3(threads), lds, st, p);
+    if (depth == 1) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 1>), dim3(wgs), dim3(threads), lds, st, p);
+    else if (depth == 3) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 3, 3>), dim3(wgs), dim3(threads), lds, st, p);
+    else if (depth == 4) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 4, 4>), dim3(wgs), dim3(threads), lds, st, p);
+    else hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 2>), dim3(wgs), dim3(threads), lds, st, p);
     return hipGetLastError();
 }
 
 }  // namespace
 
 // Tries the column-stationary kernel for a validated m = 1 HQ4_G32_M5 call; false when the shape is outside its envelope.
-// `tune`: 0 = automatic; else bits 0..1 pick the prefetch depth (1 -> 2, 2 -> 3, 3 -> 4) and bits 2..3 scale the grid
+// `tune`: 0 = automatic (two rows in flight, both issued ahead of the prologue); bits 0..1 pick the prefetch
+// (1 -> two rows, one ahead of the prologue; 2 -> three rows; 3 -> four rows) and bits 2..3 scale the grid
 // (1 -> half, 2 -> double).
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
                  float* y32, uint32_t tune, hipError_t* err) {
@@ -168,8 +170,10 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     const uint32_t sets = cpr <= 3u ? 4u : (cpr <= 12u ? 2u : 1u);
     const uint32_t threads = 32u * cpr * sets;
     const uint32_t waves = (threads + 63u) / 64u;
-    // about 20 waves per compute unit, at least four rows per set, at most 128 row slots per workgroup
-    uint32_t wgs = (256u * 20u + waves / 2u) / waves;
+    // about 10 waves per compute unit with both prefetch rows issued ahead of the activation prologue (measured on
+    // N = 17408, K = 5120: 11.3 us, against 11.5 with 20 waves and one row ahead, 12.2 with three rows in flight and
+    // 13.5+ with 5 waves); at least four rows per set, at most 128 row slots per workgroup
+    uint32_t wgs = (256u * 10u + waves / 2u) / waves;
     if ((tune >> 2 & 3u) == 1u) wgs /= 2u;
     if ((tune >> 2 & 3u) == 2u) wgs *= 2u;
     wgs = min(wgs, max(1u, w->n / (sets * 4u)));
@@ -177,7 +181,7 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     const uint32_t rows_per_wg = qwhip_cdiv(w->n, wgs);
     const size_t lds = (size_t)nb * 80u + (size_t)rows_per_wg * cpr * 4u;
     if (lds > 60u * 1024u) return false;
-    const uint32_t depth = (tune & 3u) ? (tune & 3u) + 1u : 2u;
+    const uint32_t depth = (tune & 3u) == 1u ? 1u : ((tune & 3u) ? (tune & 3u) + 1u : 2u);
     qc_params p;
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
