@@ -10,7 +10,7 @@ kernel measured with HIP events on the launch stream, and the CPU baseline (the 
 oracle form - dequantize the bank to fp32, then one fp32 product - restated in numpy and timed
 on this box's host cores over a bounded sample).
 
-Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down (see WORKLOADS).
+Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up (see WORKLOADS).
 """
 from __future__ import annotations
 
@@ -154,6 +154,58 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None):
         out["cpu_baseline"] = cpu_baseline_gemv(blocks, x_basis, bits, group, is_m5, algo_bytes,
                                                 rows_sample=min(n, args.cpu_rows))
     return out
+
+
+def run_silu_pair(args, fmt, inter, k, m, label):
+    """Dense MLP gate|up GEMV with the SwiGLU + rotation epilogue: act[m, inter] from a [2*inter, k] bank; one step = one launch."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+    from tests import helpers as H
+
+    dev = qwhip.Device(0)
+    blocks, w16 = H.make_bank(fmt, 2 * inter, k, seed=0)
+    x16 = H.make_x(m, k, 100).astype(np.float16)
+    ring_n = max(2, int(np.ceil(args.ring_mb * 1e6 / blocks.nbytes))) if not args.hot else 1
+    banks = [dev.put(blocks) for _ in range(ring_n)]
+    views = [H.view_of(dev, b, fmt, 2 * inter, k) for b in banks]
+    xb, act = dev.put(x16), dev.alloc(m * inter * 2)
+    flags = args.variant << 8
+    lib, st = dev.lib, dev.stream.handle
+
+    def launch(i):
+        qwhip.check(lib.qwhip_gemv_silu_pair(st, C.byref(views[i % ring_n]), xb.ptr, qwhip.F16, m, flags, 1, act.ptr))
+
+    _spin_up(dev, launch)
+    for i in range(args.warmup):
+        launch(i)
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        launch(i)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    got = act.download(np.float16, (m, inter)).astype(np.float32)
+    gu = qo.matmul_ref_f64(H.x_in_basis(x16, fmt), w16)
+    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=True).astype(np.float32)
+    err = qo.normalized_error(got, want)
+    if not err <= 2e-3:
+        _fail(f"bench: SwiGLU pair output failed parity (normalized error {err:.3e})")
+    algo_bytes = blocks.nbytes + m * k * 2 + m * inter * 2
+    gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": label, "format": fmt, "M": m, "N": 2 * inter, "K": k, "fused_fwht": True,
+                   "cache": "hot" if args.hot else f"cold ring of {ring_n} banks ({ring_n * blocks.nbytes / 1e6:.0f} MB)"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": algo_bytes,
+                     "kernel_us": round(us_per, 3)},
+        "normalized_error": err,
+    }
 
 
 def run_gemm(args, fmt, n, k, m, label, traffic=None):
@@ -415,6 +467,7 @@ WORKLOADS = {
     "c4_prefill": ("moe", None, None, None, 2048, False),
     "c5_qkv": ("gemv", "hq8_g32", 7168, 5120, None, False),
     "c5_down": ("gemv", "hq4_g64", 5120, 17408, None, False),
+    "mlp_gate_up": ("pair", "hq4_g32_m5", 17408, 5120, 1, False),      # n = intermediate size: the bank has 2n rows
 }
 LABELS = {
     "c1": "C1 AQ4_G32 affine GEMV N=4096 K=4096",
@@ -424,6 +477,7 @@ LABELS = {
     "c4_prefill": "C4 MoE prefill T=2048 E=128 top-8 H=2048 I=768",
     "c5_qkv": "C5 verify GEMM HQ8_G32 K=5120 N=7168",
     "c5_down": "C5 verify GEMM HQ4_G64 K=17408 N=5120",
+    "mlp_gate_up": "dense MLP gate|up GEMV + SwiGLU + FWHT, HQ4_G32 M=1 K=5120 I=17408",
 }
 
 
@@ -465,6 +519,8 @@ def main() -> None:
         m = args.m
     if kind == "moe":
         out = run_moe(args, m, LABELS[args.workload])
+    elif kind == "pair":
+        out = run_silu_pair(args, fmt, n, k, m, LABELS[args.workload])
     elif kind == "gemm":
         out = run_gemm(args, fmt, n, k, m, LABELS[args.workload], MEASURED_TRAFFIC.get(args.workload))
     else:

@@ -862,6 +862,15 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     if (w->n % 2 != 0) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "gate|up bank needs an even row count, got %u", w->n);
     const uint32_t inter = w->n / 2;
     const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
+    // HQ4_G32_M5: the column-stationary gate|up kernel of the MoE decode path, as one dense bank with one "route" per
+    // activation row (flags bits 8..11 = 2 keep the general kernel, for tests)
+    if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
+        hipError_t e = hipSuccess;
+        if (qw_moe_gateup_col(s->stream, w, 1, x, x_dtype, rotate, rotate_out && inter % 32 == 0, nullptr, m, 1, act16, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+    }
     gemv_args a = {};
     a.bank = (const uint8_t*)w->blocks;
     a.x = x;

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
     const uint32_t row_bytes = nb * 20u;
 
     // memory order: the route's expert id, the token's activations, the first weight rows; the rotation runs under them
-    const int32_t e = p.idx[pair];
+    const int32_t e = p.idx ? p.idx[pair] : 0;   // no route list: one dense gate|up bank
     const uint8_t* x = (const uint8_t*)p.x + (uint64_t)(pair / p.top_k) * nb * 64u;
     h8_t xv[XT];
 #pragma unroll

@@ -212,6 +212,31 @@ def test_gemv_rotation_per_lane_path(dev, m):
     assert qo.normalized_error(g32, ref) <= 2e-5
 
 
+@pytest.mark.parametrize("fmt,flags", [("hq4_g32_m5", 0), ("hq4_g32_m5", 2 << 8), ("hq4_g64", 0), ("aq8_g256", 0)])
+@pytest.mark.parametrize("m", [1, 3])
+@pytest.mark.parametrize("prerot,rot_out", [(False, 1), (True, 1), (True, 0)])
+def test_gemv_silu_pair_matches_oracle(dev, fmt, flags, m, prerot, rot_out):
+    """gate|up GEMV with the SwiGLU epilogue (EncodeKernels.swift:298-326): act = f16(FWHT32(silu(Wg.x) * (Wu.x))) on
+    fp32 accumulators; HQ4_G32_M5 on the column-stationary kernel and (override 2) on the general one."""
+    inter, k = 160, 1536
+    kind, bits, group, is_m5, rotate = H.FORMATS[fmt]
+    blocks, w16 = H.make_bank(fmt, 2 * inter, k, seed=12)
+    x16 = H.make_x(m, k, 112).astype(np.float16)
+    x_basis = H.x_in_basis(x16, fmt)
+    xb = dev.put(x_basis if prerot else x16)
+    bank, act = dev.put(blocks), dev.alloc(m * inter * 2)
+    view = H.view_of(dev, bank, fmt, 2 * inter, k)
+    fl = (qwhip.X_PREROTATED if prerot else 0) | flags
+    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, m, fl, rot_out, act.ptr))
+    dev.stream.sync()
+    got = act.download(np.float16, (m, inter)).astype(np.float32)
+    gu = qo.matmul_ref_f64(x_basis, w16)
+    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=bool(rot_out)).astype(np.float32)
+    assert qo.normalized_error(got, want) <= TOL
+    for b in (bank, xb, act):
+        b.free()
+
+
 def test_gemv_affine_known_answer(dev):
     """Code 1, scale 1.0, bias 0.25, x = one-hot: every output is exactly 1.25 - the -1024 must be
     stripped before the FMA, not folded into an f16 bias
