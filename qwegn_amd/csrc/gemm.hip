@@ -619,6 +619,10 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 #pragma unroll
         for (int i = 0; i < B_PER; ++i) if (i < nitems) qg_load_slice<FMT>(b_tile + b_off32[i], kt * 2u + (b_meta[i] >> 20), p.gshift, p.bb, b_reg[i]);
     };
+    // When the second items number a quarter of the workgroup, each is shared by the two group-0 threads tid and
+    // tid + NT / 4: one dequantizes its chunks 0..1, the other 2..3 (half the second pass instead of doing it twice).
+    constexpr bool SPLIT2 = (B_ITEMS - NT) * 4 == NT;
+    const bool hi_half = (tid & (NT / 4)) != 0;
     auto store_b = [&](uint32_t stage, const qg_slice<FMT>* b_reg, int nitems) {
 #pragma unroll
         for (int i = 0; i < B_PER; ++i) {
@@ -626,9 +630,20 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
             const h2_t s2 = qw_splat_lo(b_reg[i].hdr), b2 = qw_splat_hi(b_reg[i].hdr);
             uint8_t* row = lds2 + stage * STAGE + A_BYTES + (b_meta[i] & 0xFFFFu);
             const uint32_t sw = (b_meta[i] >> 16) & 7u, sl4 = (b_meta[i] >> 20) * 4u;
+            if (SPLIT2 && i == 1) {
+                constexpr int WPC = FMT == QG_FMT_B8 ? 2 : 1;   // code words per 8-column chunk
+                qg_slice<FMT> half;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                *(h8_t*)(row + (((sl4 + j) ^ sw) * 16u)) = qg_dequant_chunk<FMT>(b_reg[i], j, s2, b2, magic);
+                for (int w = 0; w < 2 * WPC; ++w) half.q[w] = hi_half ? b_reg[i].q[2 * WPC + w] : b_reg[i].q[w];
+                const uint32_t j0 = hi_half ? 2u : 0u;
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    *(h8_t*)(row + (((sl4 + j0 + j) ^ sw) * 16u)) = qg_dequant_chunk<FMT>(half, j, s2, b2, magic);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    *(h8_t*)(row + (((sl4 + j) ^ sw) * 16u)) = qg_dequant_chunk<FMT>(b_reg[i], j, s2, b2, magic);
+            }
         }
     };
 
