@@ -326,6 +326,8 @@ struct qw_gemv_params {
     const float* shared;
     const float* shared_gate;
     void* out;
+    // transposing kernel: waves per row set, row sets per workgroup, K ranges
+    uint32_t wpr, sets, nkr;
 };
 
 // PAIR = 1: gate|up pair mode.  The bank holds 2*N rows ([0, N) gate, [N, 2N) up); both are accumulated
@@ -608,6 +610,158 @@ __global__ __launch_bounds__(512) void qw_gemv_colm_kernel(const qw_gemv_params 
 }
 
 // ------------------------------------------------------------------------------------------------
+// Variant D: transposing MFMA kernel, all containers, m = 1..16, activations already in the container's basis.
+// The contraction is variant C's (lane (i, c) dequantizes slice 4u + c of row i to exact f16 weights, four
+// v_mfma_f32_16x16x32_f16 per group of four slices against activation operands held in registers), but the bank is
+// read the way memory likes it and turned into that layout on chip: a wave owns a chunk of 16 consecutive slices;
+// per tile of 16 rows it issues four loads whose lanes (b = lane >> 2, r = lane & 3) read slice b of rows 4q + r
+// (four contiguous runs of the bank per instruction instead of sixteen), parks them in a wave-private LDS region
+// (row pitch = 16 slices + one 16-byte pad: conflict-free 16-byte reads down a column of rows) and reads each
+// lane's (row, slice) back.  The loads of the next tile are in flight while the current one is contracted; no
+// workgroup barrier until the end.  Launch shape as the other persistent kernels: grid-stride over row tiles,
+// wave wv of a row set owns chunk kr * wpr + wv in K range kr, the 16 x 16 partial tiles accumulate in LDS per
+// (tile slot, wave) across K ranges and are summed in wave order at the end.
+// ------------------------------------------------------------------------------------------------
+template <int FMT, int XDT>
+__global__ __launch_bounds__(768) void qw_gemv_colt_kernel(const qw_gemv_params p) {
+    constexpr uint32_t PW = FMT == QW_FMT_B8 ? 8 : 4;     // payload dwords per slice
+    constexpr uint32_t RS = 16 * PW + 4;                   // row pitch of the payload image, dwords
+    constexpr uint32_t HS = 17;                            // row pitch of the header image, dwords
+    constexpr uint32_t WAVE_DW = 16 * RS + 16 * HS + 16;   // per-wave region (16-byte multiple)
+    extern __shared__ __attribute__((aligned(16))) uint32_t ct_lds[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u;
+    const uint32_t nwaves = blockDim.x >> 6;
+    const uint32_t wpr = p.wpr, sets = p.sets;
+    const uint32_t set = wave / wpr, wv = wave - set * wpr;
+    const uint32_t lb = lane >> 2, lr = lane & 3u;      // load role: slice of the chunk, row of the quad
+    const uint32_t i = lane & 15u, c = lane >> 4;       // contraction role
+    const uint32_t N = p.N, K = p.K, M = p.M;
+    const uint32_t nsl = K >> 5;
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    uint32_t* pay = ct_lds + wave * WAVE_DW;
+    uint32_t* hdr = pay + 16 * RS;
+    f4_t* part = (f4_t*)(ct_lds + nwaves * WAVE_DW);    // [tile slot][wave of the set][lane]
+
+    const uint32_t G = gridDim.x;
+    const uint32_t tiles = (N + 15u) >> 4;
+    if (blockIdx.x >= tiles) return;
+    const uint32_t nt = (tiles - blockIdx.x + G - 1u) / G;   // tile slots of this workgroup
+    const uint32_t nmax = (nt + sets - 1u) / sets;            // trip count, uniform over the workgroup
+    const uint32_t mine = nt > set ? (nt - set + sets - 1u) / sets : 0u;
+    const uint32_t t_first = (mine ? set : 0u) * G + blockIdx.x;
+    const uint32_t t_last = t_first + (mine ? mine - 1u : 0u) * G * sets;
+    const uint32_t row_bytes = (uint32_t)p.row_bytes;
+
+    for (uint32_t kr = 0; kr < p.nkr; ++kr) {
+        const uint32_t chunk = kr * wpr + wv;
+        // ---- activation operands of this chunk (issued first), then the first tile's loads ----
+        h8_t xraw[4][4], xop[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t sx = min(chunk * 16u + 4u * u + c, nsl - 1u);
+            const uint64_t at = (uint64_t)min(i, M - 1u) * K + 32u * sx;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xraw[u][j] = qw_load_x8_f16<XDT>(p.x, at + 8u * j);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t gl = min(chunk * 16u + lb, nsl - 1u);   // this lane's slice in the load role
+        uint32_t hdr_off, pay_off;
+        if constexpr (FMT == QW_FMT_M5) {
+            hdr_off = gl * 20u;
+            pay_off = hdr_off + 4u;
+        } else {
+            hdr_off = (gl >> p.gshift) * p.bb;
+            pay_off = hdr_off + 4u + (gl & ((1u << p.gshift) - 1u)) * (PW * 4u);
+        }
+        qw_slice<FMT> ld[4];
+        auto issue = [&](uint32_t t) {   // rows 16 t + 4 q + r, clamped into the bank (clamped rows are never stored)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint8_t* rp = p.bank + min(16u * t + 4u * q + lr, N - 1u) * row_bytes;
+                ld[q].hdr = *(const uint32_t*)(rp + hdr_off);
+                if constexpr (FMT == QW_FMT_B8) {
+                    const qw_words8 w = *(const qw_words8*)(rp + pay_off);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) ld[q].q[k] = w.q[k];
+                } else {
+                    const qw_words4 w = *(const qw_words4*)(rp + pay_off);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) ld[q].q[k] = w.q[k];
+                }
+            }
+        };
+        uint32_t t = t_first;
+        issue(t);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const bool ok = chunk * 16u + 4u * u + c < nsl && i < M;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const u4_t raw = __builtin_bit_cast(u4_t, qw_x_operand<FMT>(xraw[u], j));
+                const u4_t z = {ok ? raw[0] : 0u, ok ? raw[1] : 0u, ok ? raw[2] : 0u, ok ? raw[3] : 0u};
+                xop[u][j] = __builtin_bit_cast(h8_t, z);
+            }
+        }
+
+        uint32_t slot = set;
+        for (uint32_t ib = 0; ib < nmax; ++ib) {
+            // registers -> LDS image (the previous tile's reads are done: LDS operations of a wave complete in order)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t r = 4u * q + lr;
+                hdr[r * HS + lb] = ld[q].hdr;
+#pragma unroll
+                for (uint32_t k = 0; k < PW; k += 4) {
+                    const u4_t v = {ld[q].q[k], ld[q].q[k + 1], ld[q].q[k + 2], ld[q].q[k + 3]};
+                    *(u4_t*)(pay + r * RS + lb * PW + k) = v;
+                }
+            }
+            t = min(t + G * sets, t_last);
+            issue(t);   // next tile (the set's last tile again past the end)
+            f4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                qw_slice<FMT> blk;
+                blk.hdr = hdr[i * HS + 4u * u + c];
+#pragma unroll
+                for (uint32_t k = 0; k < PW; k += 4) {
+                    const u4_t v = *(const u4_t*)(pay + i * RS + (4u * u + c) * PW + k);
+                    blk.q[k] = v[0]; blk.q[k + 1] = v[1]; blk.q[k + 2] = v[2]; blk.q[k + 3] = v[3];
+                }
+                const h2_t s2 = qw_splat_lo(blk.hdr), b2 = qw_splat_hi(blk.hdr);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const h8_t a = qw_dequant_chunk<FMT>(blk, j, s2, b2, magic);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xop[u][j], acc, 0, 0, 0);
+                }
+            }
+            // lane (j = activation row, c) holds rows 4c + r of the tile
+            if (slot < nt) {
+                f4_t* dst = part + (size_t)(slot * wpr + wv) * 64u + lane;
+                if (kr == 0) *dst = acc;
+                else *dst += acc;
+            }
+            slot += sets;
+        }
+    }
+    __syncthreads();
+    // fixed-order sum over the waves of a row set; consecutive threads -> consecutive output rows
+    for (uint32_t e = tid; e < nt * 16u * M; e += blockDim.x) {
+        const uint32_t rr = e & 15u, sm = e >> 4;
+        const uint32_t s = sm / M, m = sm - s * M;
+        const uint32_t n = 16u * (s * G + blockIdx.x) + rr;
+        if (n >= N) continue;
+        const uint32_t src = m + 16u * (rr >> 2), comp = rr & 3u;
+        float v = 0.f;
+        for (uint32_t w2 = 0; w2 < wpr; ++w2) v += part[(size_t)(s * wpr + w2) * 64u + src][comp];
+        if (p.y32) p.y32[(uint64_t)m * N + n] = v;
+        if (p.y16) p.y16[(uint64_t)m * N + n] = (h1_t)v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -685,6 +839,45 @@ bool launch_colm(hipStream_t st, const gemv_args& a, uint32_t xdt) {
     return true;
 }
 
+// Transposing kernel (variant D): false when the call is outside its envelope.
+template <int FMT, int XDT>
+bool launch_colt_1(hipStream_t st, gemv_args a, hipError_t* err) {
+    constexpr uint32_t PW = FMT == QW_FMT_B8 ? 8 : 4;
+    constexpr uint32_t WAVE_DW = 16 * (16 * PW + 4) + 16 * 17 + 16;
+    if ((uint64_t)a.N * a.row_bytes >= (1ull << 32)) return false;   // 32-bit offsets inside the bank
+    const uint32_t nsl = a.K >> 5, nch = qwhip_cdiv(nsl, 16u);
+    // at most 12 waves per row set (768 threads); longer rows take several K ranges
+    a.nkr = qwhip_cdiv(nch, 12u);
+    a.wpr = qwhip_cdiv(nch, a.nkr);
+    a.sets = max(1u, 12u / a.wpr);
+    const uint32_t waves = a.wpr * a.sets;
+    const uint32_t tiles = qwhip_cdiv(a.N, 16u);
+    uint32_t wgs = min(256u, max(1u, tiles / a.sets));
+    size_t lds = 0;
+    for (;;) {
+        lds = (size_t)waves * WAVE_DW * 4u + (size_t)qwhip_cdiv(tiles, wgs) * a.wpr * 1024u;
+        if (lds <= 150u * 1024u || wgs >= tiles) break;
+        wgs = min(wgs * 2u, tiles);
+    }
+    if (lds > 150u * 1024u) return false;
+    auto kern = qw_gemv_colt_kernel<FMT, XDT>;
+    static size_t attr_lds = 0;   // per instantiation
+    if (lds > attr_lds) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        if (e != hipSuccess) { *err = e; return true; }
+        attr_lds = 150u * 1024u;
+    }
+    hipLaunchKernelGGL(kern, dim3(wgs), dim3(64u * waves), lds, st, a);
+    *err = hipGetLastError();
+    return true;
+}
+
+template <int FMT>
+bool launch_colt(hipStream_t st, const gemv_args& a, uint32_t xdt, hipError_t* err) {
+    if (a.rotate) return false;
+    return xdt == QWHIP_F16 ? launch_colt_1<FMT, QWHIP_F16>(st, a, err) : launch_colt_1<FMT, QWHIP_BF16>(st, a, err);
+}
+
 qwhip_status check_common(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                           int* fmt) {
     QWHIP_REQUIRE(s);
@@ -737,7 +930,7 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
 
 // flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer,
 // 4 = column-stationary persistent kernel, 5 = column-stationary MFMA kernel, 6 = column-stationary small-M kernel,
-// 7 = 4x4x4-block MFMA kernel);
+// 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel);
 // bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer / tuning code of the
 // column-stationary kernel (0 = automatic).
 extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
@@ -817,6 +1010,21 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
         return QWHIP_OK;
     }
 
+    // transposing MFMA kernel: activations already in the basis.  Its cost barely grows with m: measured best from 13 rows
+    // on (N = 7168, K = 5120, HQ8: 16.9 us at m = 16 against 18.6 for the column-stationary MFMA kernel and 23.9 for the
+    // 4x4x4-block kernel; N = 5120, K = 17408, HQ4_G64: 34.8 against 40.8 for the streamer) and from 9 on short rows.
+    if (variant == 8 || (variant == 0 && !rotate && (m >= 13 || (m >= 9 && w->k <= 5120u)))) {
+        hipError_t e = hipSuccess;
+        bool done = false;
+        if (fmt == QW_FMT_M5) done = launch_colt<QW_FMT_M5>(s->stream, a, x_dtype, &e);
+        else if (fmt == QW_FMT_B4) done = launch_colt<QW_FMT_B4>(s->stream, a, x_dtype, &e);
+        else done = launch_colt<QW_FMT_B8>(s->stream, a, x_dtype, &e);
+        if (done) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+        if (variant == 8) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the transposing MFMA kernel needs activations in the basis");
+    }
     // 4x4x4-block MFMA kernel: activations already in the basis.  Measured best for 2..8 rows (N = 7168, K = 5120, HQ8:
     // 11.3 / 12.0 / 13.3 us at m = 2 / 4 / 8) and up to 12 rows on rows too long for the column-stationary MFMA kernel
     // (N = 5120, K = 17408, HQ4_G64: 22.9 us at m = 8, 29.6 at m = 12 against 39-40 for the streamer).

@@ -197,6 +197,28 @@ def test_gemv_block_mfma_kernel_k_ranges_and_dtypes(dev, fmt, n, k, m, xdtype):
     assert qo.normalized_error(g16, ref) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "aq4_g32", "hq4_g32", "hq4_g64", "hq4_g128", "hq8_g32", "hq8_g64", "aq8_g256"])
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_gemv_transposing_mfma_kernel(dev, fmt, m):
+    """Transposing MFMA kernel (override 8): coalesced loads parked in LDS, exact f16 weights on the matrix cores.
+    n = 270 ends in a partial 16-row tile, k = 1536 = 3 chunks of 16 slices."""
+    g16, g32, ref = _run_gemv(dev, fmt, 270, 1536, m, prerot=True, seed=5, variant=8)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt,n,k,m,xdtype", [("hq4_g64", 96, 17408, 16, "f16"), ("aq4_g32", 300, 2080, 6, "bf16"),
+                                              ("aq8_g256", 64, 5120, 16, "bf16"), ("hq8_g32", 5, 64, 2, "f16"),
+                                              ("hq8_g32", 1000, 5120, 13, "f16")])
+def test_gemv_transposing_mfma_kernel_k_ranges_and_dtypes(dev, fmt, n, k, m, xdtype):
+    """Long rows take several K ranges (partial tiles accumulate in LDS), a partial last chunk, bf16 activations, a bank
+    smaller than one tile, several tile slots per workgroup."""
+    prerot = H.FORMATS[fmt][4]
+    g16, g32, ref = _run_gemv(dev, fmt, n, k, m, prerot=prerot, xdtype=xdtype, seed=8, variant=8)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
 @pytest.mark.parametrize("m", [1, 4])
 def test_gemv_column_stationary_long_rows(dev, m):
     """k = 17408: 17 half-waves per row, one row set per workgroup."""
