@@ -32,7 +32,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense f16/bf16 MFMA, published
 # HBM bytes per launch of the dominant kernel under its automatic configuration, from rocprofv3 --pmc passes
 # (FETCH_SIZE KiB x 1024 x 2.000 + WRITE_SIZE KiB x 1024 x 1.000; the factors come from a streaming kernel of known
 # size).  The counter passes and the calibration are recorded as text under profiles/.
-MEASURED_TRAFFIC = {"c2": 56_124_468, "c3": 191_582_251}
+MEASURED_TRAFFIC = {"c2": 56_129_590, "c3": 191_578_172}
 
 
 def _fail(msg: str) -> None:
