@@ -19,8 +19,9 @@
 //
 // Launch shape: persistent, grid-stride over row quads (quad slot s of workgroup w is quad s * gridDim.x + w, so the
 // grid reads one contiguous band of the bank at a time).  Wave wv of a row set owns slice chunk kr * wpr + wv
-// (16 slices) in K range kr; long rows take several K ranges, the activations of one range in registers at a time,
-// partial sums accumulating in LDS per (quad slot, wave, 16-lane row) and summed in a fixed order at the end.
+// (16 slices) in K range kr; long rows take several K ranges, the activations of one range in registers at a time
+// (the next range's fetched meanwhile, the weight prefetch running on across the boundary), partial sums
+// accumulating in LDS per (quad slot, wave, 16-lane row) and summed in a fixed order at the end.
 #include "qwhip_common.h"
 
 namespace {
@@ -64,11 +65,14 @@ __global__ __launch_bounds__(LB) void qw_gemv_quad_kernel(const qq_params p) {
     const uint32_t W16 = wpr * 4u;
     const uint32_t step = G * sets * 4u * p.row_bytes;      // bytes between consecutive quads of one set
 
-    for (uint32_t kr = 0; kr < p.nkr; ++kr) {
-        const uint32_t g0 = (kr * wpr + wv) * 16u + b;
-        const bool gvalid = g0 < p.nsl;
-        const uint32_t g = gvalid ? g0 : p.nsl - 1u;
-        uint32_t hdr_off, pay_off;
+    // this lane's bank row inside a quad is j (the A role); rows past the bank re-read its last row (never stored)
+    const uint32_t q_first = (mine ? set : 0u) * G + blockIdx.x;
+    const uint32_t off_first = min(4u * q_first + j, N - 1u) * p.row_bytes;
+    const uint32_t last_quad = q_first + (mine ? mine - 1u : 0u) * G * sets;
+    const uint32_t off_max = min(4u * last_quad + j, N - 1u) * p.row_bytes;   // loads past the set's last quad re-read it
+    // slice of this lane in K range kr (clamped into the row) and its byte offsets inside a bank row
+    auto slice_of = [&](uint32_t kr, uint32_t& hdr_off, uint32_t& pay_off) {
+        const uint32_t g = min((kr * wpr + wv) * 16u + b, p.nsl - 1u);
         if constexpr (FMT == QW_FMT_M5) {
             hdr_off = g * 20u;
             pay_off = hdr_off + 4u;
@@ -76,40 +80,57 @@ __global__ __launch_bounds__(LB) void qw_gemv_quad_kernel(const qq_params p) {
             hdr_off = (g >> p.gshift) * p.bb;
             pay_off = hdr_off + 4u + (g & ((1u << p.gshift) - 1u)) * (FMT == QW_FMT_B8 ? 32u : 16u);
         }
-        // this lane's bank row inside a quad is j (the A role); rows past the bank re-read its last row (never stored)
-        const uint32_t q_first = (mine ? set : 0u) * G + blockIdx.x;
-        const uint32_t r_first = min(4u * q_first + j, N - 1u);
-        uint32_t off = r_first * p.row_bytes;
-        const uint32_t last_quad = q_first + (mine ? mine - 1u : 0u) * G * sets;
-        const uint32_t off_max = min(4u * last_quad + j, N - 1u) * p.row_bytes;   // loads past the set's last quad re-read it
-
-        // 1. activation loads of this K range first, then the first row quads
-        u4_t xraw[MG][4];
+        return g;
+    };
+    // The weight prefetch runs ahead of the consumer across K ranges: after the last quad of a range it goes on with
+    // the first quad of the next one, so a range boundary costs no memory round trip.
+    uint32_t i_kr = 0, i_left = nmax, i_off = off_first, i_hdr, i_pay;
+    slice_of(0, i_hdr, i_pay);
+    qq_slice<FMT> buf[D];
+    auto issue = [&](int slot) {
+        const uint8_t* rp = p.bank + i_off;
+        buf[slot].hdr = *(const uint32_t*)(rp + i_hdr);
+        if constexpr (FMT == QW_FMT_B8) {
+            const qq_words8 w = *(const qq_words8*)(rp + i_pay);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) buf[slot].q[c] = w.q[c];
+        } else {
+            const qq_words4 w = *(const qq_words4*)(rp + i_pay);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) buf[slot].q[c] = w.q[c];
+        }
+        i_off = min(i_off + step, off_max);
+        if (--i_left == 0u) {   // uniform over the workgroup
+            i_kr = min(i_kr + 1u, p.nkr - 1u);   // past the last range: its data again, never consumed
+            slice_of(i_kr, i_hdr, i_pay);
+            i_off = off_first;
+            i_left = nmax;
+        }
+    };
+    // Activations of a K range: with up to eight activation rows the next range's are fetched while this one is
+    // contracted (they share the registers of the raw loads); with more rows they are loaded at the range's start.
+    constexpr bool XPF = MG <= 2;
+    u4_t xraw[MG][4];
+    auto load_x = [&](uint32_t kr) {
+        uint32_t ho, po;
+        const uint32_t g = slice_of(kr, ho, po);
 #pragma unroll
         for (int mg = 0; mg < MG; ++mg) {
             const uint64_t at = (uint64_t)min(4u * mg + j, p.M - 1u) * p.K + (uint64_t)g * 32u;
 #pragma unroll
             for (int c = 0; c < 4; ++c) xraw[mg][c] = *(const u4_t*)((const uint16_t*)p.x + at + 8u * c);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        qq_slice<FMT> buf[D];
-        auto issue = [&](int slot) {
-            const uint8_t* rp = p.bank + off;
-            buf[slot].hdr = *(const uint32_t*)(rp + hdr_off);
-            if constexpr (FMT == QW_FMT_B8) {
-                const qq_words8 w = *(const qq_words8*)(rp + pay_off);
+    };
+    // 1. activation loads of the first K range first, then the first row quads
+    if (XPF) load_x(0);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int c = 0; c < 8; ++c) buf[slot].q[c] = w.q[c];
-            } else {
-                const qq_words4 w = *(const qq_words4*)(rp + pay_off);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) buf[slot].q[c] = w.q[c];
-            }
-            off = min(off + step, off_max);
-        };
-#pragma unroll
-        for (int d = 0; d < D; ++d) issue(d);
-        __builtin_amdgcn_sched_barrier(0);
+    for (int d = 0; d < D; ++d) issue(d);
+    __builtin_amdgcn_sched_barrier(0);
+
+    for (uint32_t kr = 0; kr < p.nkr; ++kr) {
+        const bool gvalid = (kr * wpr + wv) * 16u + b < p.nsl;
+        if (!XPF) load_x(kr);
         // 2. B operands: pairs in the order the masked code words come out, zero for slices past the row's end
         h4_t xb[MG][8];
         float S[MG];
@@ -156,6 +177,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_quad_kernel(const qq_params p) {
             __builtin_amdgcn_sched_barrier(0);
         }
 
+        if (XPF && kr + 1u < p.nkr) load_x(kr + 1u);
         uint32_t qslot = set;   // quad slot being consumed
         for (uint32_t ib = 0; ib < nmax; ib += D) {
 #pragma unroll
@@ -224,6 +246,16 @@ __global__ __launch_bounds__(LB) void qw_gemv_quad_kernel(const qq_params p) {
                 qslot += sets;
             }
         }
+        // the next range's first quads are already in flight, in the slots after the last one consumed: turn the
+        // window so that they sit in slots 0, 1, ... again
+        if (kr + 1u < p.nkr) {
+            for (uint32_t k = nmax % D; k > 0u; --k) {
+                const qq_slice<FMT> first = buf[0];
+#pragma unroll
+                for (int d = 0; d + 1 < D; ++d) buf[d] = buf[d + 1];
+                buf[D - 1] = first;
+            }
+        }
     }
     __syncthreads();
     // fixed-order sum of the partials of each (quad slot, activation row, bank row)
@@ -246,7 +278,7 @@ void qq_launch1(hipStream_t st, const qq_params& p, uint32_t wgs, uint32_t threa
     auto kern = qw_gemv_quad_kernel<FMT, XDT, MG, D, 768>;
     static bool attr_done = false;   // per instantiation
     if (!attr_done) {
-        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
         attr_done = true;
     }
     hipLaunchKernelGGL(kern, dim3(wgs), dim3(threads), lds, st, p);
@@ -285,10 +317,10 @@ bool qw_quad_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t 
     size_t lds = 0;
     for (;;) {
         lds = (size_t)qwhip_cdiv(nquads, wgs) * (wpr * 4u) * (4u * mg) * 16u;
-        if (lds <= 48u * 1024u || wgs >= nquads) break;
+        if (lds <= 96u * 1024u || wgs >= nquads) break;   // more workgroups re-read the activations: one per CU while it fits
         wgs = min(wgs * 2u, nquads);
     }
-    if (lds > 64u * 1024u) return false;
+    if (lds > 96u * 1024u) return false;
     qq_params p;
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
