@@ -661,6 +661,26 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
             qg3_mfma_2x5(acc, a_bt + sb + (uint32_t)(uintptr_t)lds2, b_bt + sb + (uint32_t)(uintptr_t)lds2);
             return;
         }
+        if constexpr (WM * WN <= 4) {
+            // small wave tile: two or four MFMAs per sub-step cannot cover an LDS round trip, so every fragment of the
+            // K-step is requested first (48 registers at most) and the MFMAs then run back to back
+            h8_t af[4][WM], bf[4][WN];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                for (int a = 0; a < WM; ++a) af[ks][a] = *(const h8_t*)(st_base + (a_bt ^ (32u * ks)) + a * 4096);
+#pragma unroll
+                for (int b = 0; b < WN; ++b) bf[ks][b] = *(const h8_t*)(st_base + (b_bt ^ (32u * ks)) + b * 4096);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int b = 0; b < WN; ++b)
+#pragma unroll
+                    for (int a = 0; a < WM; ++a)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks][a], bf[ks][b], acc[a][b], 0, 0, 0);
+            return;
+        }
         h8_t af[2][WM], bf[WN];
         {
             #pragma unroll
@@ -849,11 +869,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED = false>
 hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, false>;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1033,7 +1053,15 @@ hipError_t launch_grouped_y(hipStream_t st, const qw_gemm_params& p, dim3 grid, 
 }
 template <int FMT>
 hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid, uint32_t xdt, uint32_t ydt) {
-    if (xdt == QWHIP_F16) {  // pipelined kernel, 64 x 256 tiles
+    if (xdt == QWHIP_F16 && !p.force_gemm2 && (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0))) {
+        // ping-pong kernel on the 64 x 256 tiles: 8 waves, one of each group per SIMD, so one dequantizes while the other
+        // multiplies (measured on T = 2048, E = 128, top-8: gate_up 257 -> 221 us; pairing two list entries of an expert
+        // into a 128-row tile, or loading two K-steps ahead, measured no faster)
+        if (ydt == QWHIP_F16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F16, true>(st, p, grid);
+        if (ydt == QWHIP_BF16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_BF16, true>(st, p, grid);
+        return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F32, true>(st, p, grid);
+    }
+    if (xdt == QWHIP_F16) {  // DMA-fed pipelined kernel, 64 x 256 tiles
         if (ydt == QWHIP_F16) return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F16, true>(st, p, grid);
         if (ydt == QWHIP_BF16) return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_BF16, true>(st, p, grid);
         return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F32, true>(st, p, grid);
