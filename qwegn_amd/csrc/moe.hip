@@ -215,61 +215,141 @@ __global__ __launch_bounds__(1024) void qw_moe_group_pairs_kernel(const int32_t*
                                                                    int32_t* __restrict__ sorted_pair, int32_t* __restrict__ sorted_tok,
                                                                    int32_t* __restrict__ inv_perm, int32_t* __restrict__ tile_e,
                                                                    int32_t* __restrict__ tile_r, int32_t* __restrict__ tile_count,
-                                                                   uint32_t compact_tail) {
+                                                                   uint32_t compact_tail, uint32_t stage_lds) {
+    extern __shared__ int32_t lds_sorted[];   // [pairs] when stage_lds
+    // Per-wave histograms and cursors: LDS atomics of the 16 waves on one shared set of counters serialize on the few
+    // hot addresses (16,384 pairs over 128 experts: 32 us); privately they meet only their own 64 lanes.
+    __shared__ int cnt_w[16][512];
     __shared__ int cnt[512];
     __shared__ int off[513];
-    __shared__ int cursor[512];
     __shared__ int tile_off[513];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t e = tid; e < experts; e += 1024) cnt[e] = 0;
+    const uint32_t wave = tid >> 6;
+    for (uint32_t e = tid; e < 16u * 512u; e += 1024) (&cnt_w[0][0])[e] = 0;
     __syncthreads();
-    for (uint32_t i = tid; i < pairs; i += 1024) {
-        const int32_t raw = ids[i];
-        if (raw >= 0) {
-            const uint32_t e = (uint32_t)raw & 0xFFFFu;
-            if (e < experts) atomicAdd(&cnt[e], 1);
+    // ids in batches of 16 per thread: the loads of a batch are issued together (a load per atomic would pay one memory
+    // round trip per pair and thread)
+    for (uint32_t base = 0; base < pairs; base += 16u * 1024u) {
+        int32_t raw[16];
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const uint32_t i = base + tid + 1024u * c;
+            raw[c] = ids[min(i, pairs - 1u)];
+            if (i >= pairs) raw[c] = -1;
+        }
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            if (raw[c] >= 0) {
+                const uint32_t e = (uint32_t)raw[c] & 0xFFFFu;
+                if (e < experts) atomicAdd(&cnt_w[wave][e], 1);
+            }
         }
     }
     __syncthreads();
-    if (tid == 0) {
-        // serial scan over <= 512 experts: rows and tiles
-        int c = 0, t = 0;
-        for (uint32_t e = 0; e < experts; ++e) {
-            off[e] = c;
-            tile_off[e] = t;
-            const int n = cnt[e];
-            c += n;
+    for (uint32_t e = tid; e < experts; e += 1024) {
+        int c = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) c += cnt_w[w][e];
+        cnt[e] = c;
+    }
+    __syncthreads();
+    if (tid < 64u) {
+        // exclusive scans over <= 512 experts (rows and tiles) by one wave: lane l owns experts 8 l .. 8 l + 7
+        int rows8[8], tiles8[8], rsum = 0, tsum = 0;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint32_t e = 8u * tid + q;
+            const int n = e < experts ? cnt[e] : 0;
+            int t = 0;
             if (n > 0) {
-                if (compact_tail) t += (n >> 6) + ((n & 63) ? 1 : 0);
+                if (compact_tail) t = (n >> 6) + ((n & 63) ? 1 : 0);
                 else {
                     const int bm = qw_moe_tile_block(n);
-                    t += (n + bm - 1) / bm;
+                    t = (n + bm - 1) / bm;
                 }
             }
+            rows8[q] = rsum;
+            tiles8[q] = tsum;
+            rsum += n;
+            tsum += t;
         }
-        off[experts] = c;
-        tile_off[experts] = t;
+        int rinc = rsum, tinc = tsum;   // inclusive scan over the lanes
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int ro = __shfl_up(rinc, d, 64), to = __shfl_up(tinc, d, 64);
+            if ((int)tid >= d) {
+                rinc += ro;
+                tinc += to;
+            }
+        }
+        const int rbase = rinc - rsum, tbase = tinc - tsum;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint32_t e = 8u * tid + q;
+            if (e < experts) {
+                off[e] = rbase + rows8[q];
+                tile_off[e] = tbase + tiles8[q];
+            }
+        }
+        if (tid == 63u) {
+            off[experts] = rinc;
+            tile_off[experts] = tinc;
+        }
     }
     __syncthreads();
     for (uint32_t e = tid; e <= experts; e += 1024) {
         expert_off[e] = off[e];
-        if (e < experts) cursor[e] = off[e];
-    }
-    __syncthreads();
-    for (uint32_t i = tid; i < pairs; i += 1024) {
-        const int32_t raw = ids[i];
-        bool placed = false;
-        if (raw >= 0) {
-            const uint32_t e = (uint32_t)raw & 0xFFFFu;
-            if (e < experts) {
-                const int at = atomicAdd(&cursor[e], 1);
-                sorted_pair[at] = (int32_t)i;
-                sorted_tok[at] = (int32_t)(i / top_k);
-                if (inv_perm) inv_perm[i] = at;
-                placed = true;
+        if (e < experts) {   // the waves' slices of the expert's slot range, in wave order: counts become cursors
+            int c = off[e];
+#pragma unroll
+            for (int w = 0; w < 16; ++w) {
+                const int n = cnt_w[w][e];
+                cnt_w[w][e] = c;
+                c += n;
             }
         }
-        if (!placed && inv_perm) inv_perm[i] = -1;
+    }
+    __syncthreads();
+    for (uint32_t base = 0; base < pairs; base += 16u * 1024u) {
+        int32_t raw[16];
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const uint32_t i = base + tid + 1024u * c;
+            raw[c] = ids[min(i, pairs - 1u)];
+            if (i >= pairs) raw[c] = -2;   // past the list: nothing to place, nothing to mark
+        }
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const uint32_t i = base + tid + 1024u * c;
+            if (raw[c] == -2) continue;
+            bool placed = false;
+            if (raw[c] >= 0) {
+                const uint32_t e = (uint32_t)raw[c] & 0xFFFFu;
+                if (e < experts) {
+                    const int at = atomicAdd(&cnt_w[wave][e], 1);
+                    if (stage_lds) {
+                        lds_sorted[at] = (int32_t)i;          // written out in slot order below
+                    } else {
+                        sorted_pair[at] = (int32_t)i;
+                        sorted_tok[at] = (int32_t)(i / top_k);
+                    }
+                    if (inv_perm) inv_perm[i] = at;
+                    placed = true;
+                }
+            }
+            if (!placed && inv_perm) inv_perm[i] = -1;
+        }
+    }
+    if (stage_lds) {
+        // the sorted list was built in LDS: stores in slot order are whole lines (scattered 4-byte stores from the one
+        // CU this kernel runs on cost an address cycle each: 2 x 16,384 of them were most of its time)
+        __syncthreads();
+        const uint32_t total = (uint32_t)off[experts];
+        for (uint32_t j = tid; j < total; j += 1024) {
+            const int32_t sp = lds_sorted[j];
+            sorted_pair[j] = sp;
+            sorted_tok[j] = (int32_t)((uint32_t)sp / top_k);
+        }
     }
     if (tile_e) {
         for (uint32_t e = tid; e < experts; e += 1024) {
@@ -316,8 +396,16 @@ extern "C" qwhip_status qwhip_moe_group_pairs(qwhip_stream_t s, const int32_t* i
     const bool tiles = tile_e || tile_r || tile_count;
     if (tiles && !(tile_e && tile_r && tile_count))
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe group pairs: tile_e, tile_r and tile_count come together");
-    hipLaunchKernelGGL(qw_moe_group_pairs_kernel, dim3(1), dim3(1024), 0, s->stream, ids, experts, pairs, top_k, expert_off,
-                       sorted_pair, sorted_tok, inv_perm, tile_e, tile_r, tile_count, compact_tail ? 1u : 0u);
+    // up to 24,576 pairs the sorted list is staged in LDS (96 KB beside the 38 KB of counters)
+    const uint32_t stage = pairs <= 24576u ? 1u : 0u;
+    const size_t lds = stage ? (size_t)pairs * 4u : 0u;
+    static bool attr_done = false;
+    if (!attr_done) {
+        QWHIP_TRY_HIP(hipFuncSetAttribute((const void*)qw_moe_group_pairs_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(qw_moe_group_pairs_kernel, dim3(1), dim3(1024), lds, s->stream, ids, experts, pairs, top_k, expert_off,
+                       sorted_pair, sorted_tok, inv_perm, tile_e, tile_r, tile_count, compact_tail ? 1u : 0u, stage);
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
@@ -326,7 +414,7 @@ extern "C" qwhip_status qwhip_moe_group_pairs(qwhip_stream_t s, const int32_t* i
 // Combine: out[t, h] = sum_k wts[t, k] * dn[inv_perm[t*K + k], h] (+ shared_gate[t] * shared[t, h]).
 // One thread per 4 consecutive h; fp32 accumulation in rank order.
 // ------------------------------------------------------------------------------------------------
-template <int DDT, int ODT>
+template <int DDT, int ODT, int KMAX>   // KMAX: unrolled route slots of the vector path (8 or 16)
 __global__ __launch_bounds__(256) void qw_moe_combine_kernel(const void* __restrict__ dn, const int32_t* __restrict__ inv_perm,
                                                               const float* __restrict__ wts, uint32_t T, uint32_t K, uint32_t H,
                                                               const float* __restrict__ shared, const float* __restrict__ shared_gate,
@@ -335,6 +423,41 @@ __global__ __launch_bounds__(256) void qw_moe_combine_kernel(const void* __restr
     const uint32_t h = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (h >= H) return;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (K <= (uint32_t)KMAX && (H & 3u) == 0u) {
+        // every route's slot and weight first, then all the rows' four columns as one load each: the loads of a thread
+        // are independent of each other, only the additions keep the rank order
+        int32_t slot[KMAX];
+        float w[KMAX];
+#pragma unroll
+        for (uint32_t k = 0; k < (uint32_t)KMAX; ++k) {
+            slot[k] = k < K ? inv_perm[(uint64_t)t * K + k] : -1;
+            w[k] = k < K ? wts[(uint64_t)t * K + k] : 0.0f;
+        }
+        float v[KMAX][4];
+#pragma unroll
+        for (uint32_t k = 0; k < (uint32_t)KMAX; ++k) {
+            const uint64_t at = (uint64_t)(slot[k] < 0 ? 0 : slot[k]) * H + h;   // an empty route reads row 0 and is not added
+            if constexpr (DDT == QWHIP_F32) {
+                const f4_t x = *(const f4_t*)((const float*)dn + at);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[k][j] = x[j];
+            } else {
+                const u2_t x = *(const u2_t*)((const uint16_t*)dn + at);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint16_t b = (uint16_t)(x[j >> 1] >> (16 * (j & 1)));
+                    v[k][j] = DDT == QWHIP_F16 ? (float)__builtin_bit_cast(h1_t, b) : qw_bf16_to_f32(b);
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < (uint32_t)KMAX; ++k) {
+            if (slot[k] >= 0) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = fmaf(w[k], v[k][j], acc[j]);
+            }
+        }
+    } else
     for (uint32_t k = 0; k < K; ++k) {
         const int32_t slot = inv_perm[(uint64_t)t * K + k];
         if (slot < 0) continue;
@@ -370,7 +493,13 @@ extern "C" qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint
     QWHIP_REQUIRE(wts);
     QWHIP_REQUIRE(out);
     const dim3 grid(qwhip_cdiv(hidden, 1024), t), block(256);
-#define QW_CB(DD, OD) hipLaunchKernelGGL((qw_moe_combine_kernel<DD, OD>), grid, block, 0, s->stream, dn, inv_perm, wts, t, top_k, hidden, shared, shared_gate, out)
+#define QW_CB(DD, OD)                                                                                                          \
+    do {                                                                                                                       \
+        if (top_k <= 8) hipLaunchKernelGGL((qw_moe_combine_kernel<DD, OD, 8>), grid, block, 0, s->stream, dn, inv_perm, wts, t, \
+                                           top_k, hidden, shared, shared_gate, out);                                           \
+        else hipLaunchKernelGGL((qw_moe_combine_kernel<DD, OD, 16>), grid, block, 0, s->stream, dn, inv_perm, wts, t, top_k,    \
+                                hidden, shared, shared_gate, out);                                                             \
+    } while (0)
 #define QW_CB_O(DD)                                                   \
     switch (out_dtype) {                                              \
         case QWHIP_F32: QW_CB(DD, QWHIP_F32); break;                  \
