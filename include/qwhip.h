@@ -150,7 +150,14 @@ qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_view* w, voi
  *   qwg_skinny_m2/m3, qwg_gemv_hq4_rows_r_m_t (M = 2..8 verify)
  * x: [m, k] row-major, f16 or bf16; m in 1..16; every weight byte is read once for all m rows.
  * y16 (f16 [m, n]) and/or y32 (f32 [m, n]) receive the result; at least one is required
- * (both = the reference's dual store).  fp32 accumulation. */
+ * (both = the reference's dual store).  fp32 accumulation.
+ * Arithmetic: the kernels chosen for rows already in the container's basis and for m = 1 contract the factorised form
+ * of the reference's own GEMVs, scale * sum(code * x) + bias * sum(x) per slice (qwg_aq_slice_dot,
+ * Sources/QWMetal/include/qw_dequant_multi.metalh:205-208); the others contract the f16 weights of qwhip_dequant_f16.
+ * flags: QWHIP_X_PREROTATED; bits 8..11 pick one kernel for tuning and tests (0 = automatic, 1 = half-wave dot2,
+ * 2 = MFMA streamer, 3 = DMA streamer, 4 = column-stationary HQ4 kernel, 5 = column-stationary MFMA kernel,
+ * 6 = column-stationary dot2 kernel, 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel; a kernel that does not
+ * take the shape returns QWHIP_E_BAD_GEOMETRY); bits 12..15 its tuning code. */
 qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                         uint32_t m, uint32_t flags, void* y16, float* y32);
 
