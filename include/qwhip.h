@@ -245,6 +245,23 @@ qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_
 qwhip_status qwhip_quantize_hq4_g32(qwhip_stream_t s, const void* src, uint32_t src_dtype, uint32_t n, uint32_t k,
                                     uint32_t rotate, void* blocks_out);
 
+/* qwg_repack_mlx_affine_to_aq_m5 / qwg_repack_mlx_affine_switch_gate_up_to_aq_m5
+ * (Sources/QWMetal/quant/qw_online_quant.metal:56-178; QWAQRepack.repackMLXAffine / repackMLXAffineSwitchGateUp,
+ * Sources/Foundation/QWLoad/AQRepack.swift:108-250): an MLX affine checkpoint (packed codes u32, scales and biases
+ * bf16 or f16, one pair per group) becomes AQ blocks [f16 scale][f16 bias][payload] at the same byte count; the
+ * switch variant interleaves gate_proj and up_proj [experts, inter, cols] into one [experts, 2*inter, cols] bank.
+ * A header that f16 does not hold exactly (values below 2^-14 excepted) is written as the f16 NaN 0x7e00 and counted
+ * in *refused (a device word the caller zeroes first and reads after the stream has drained; the reference door
+ * throws headersNotExact when it is not zero). */
+qwhip_status qwhip_repack_mlx_affine(qwhip_stream_t s, const void* mlx_w, const void* mlx_scales, const void* mlx_biases,
+                                     uint32_t scale_dtype, uint32_t rows, uint32_t cols, uint32_t bits, uint32_t group,
+                                     void* dst_blocks, uint32_t* refused);
+qwhip_status qwhip_repack_mlx_affine_switch_gate_up(qwhip_stream_t s, const void* gate_w, const void* gate_scales,
+                                                    const void* gate_biases, const void* up_w, const void* up_scales,
+                                                    const void* up_biases, uint32_t scale_dtype, uint32_t experts,
+                                                    uint32_t inter, uint32_t cols, uint32_t bits, uint32_t group,
+                                                    void* dst_blocks, uint32_t* refused);
+
 #ifdef __cplusplus
 }
 #endif

@@ -334,6 +334,55 @@ def weights_f16_exact(blocks: np.ndarray, bits: int, group: int, is_m5: bool) ->
     return (q * s.astype(np.float64)[..., None] + b.astype(np.float64)[..., None]).astype(np.float16).reshape(n, nb * group)
 
 
+def f16_header_holds(raw: np.ndarray, stored: np.ndarray) -> np.ndarray:
+    """qwg_f16_header_holds (Sources/QWMetal/quant/qw_online_quant.metal:62-69): `stored = half(raw)` holds `raw` when it
+    converts back to it, or when both are finite and |raw| < 2^-14 (the subnormal range of f16, where the nearest
+    2^-24 step is accepted)."""
+    raw = np.asarray(raw, dtype=np.float32)
+    back = np.asarray(stored, dtype=np.float16).astype(np.float32)
+    with np.errstate(invalid="ignore"):
+        same = back == raw
+        small = np.isfinite(raw) & np.isfinite(back) & (np.abs(raw) < np.float32(6.103515625e-5))
+    return same | small
+
+
+def _mlx_header_f32(bits16: np.ndarray, is_f16: bool) -> np.ndarray:
+    b = np.ascontiguousarray(bits16, dtype=np.uint16)
+    return b.view(np.float16).astype(np.float32) if is_f16 else bf16_bits_to_f32(b)
+
+
+def repack_mlx_affine(mlx_w: np.ndarray, scales16: np.ndarray, biases16: np.ndarray, rows: int, cols: int, bits: int,
+                      group: int, scale_is_f16: bool):
+    """qwg_repack_mlx_affine_to_aq_m5 (qw_online_quant.metal:71-122): MLX packed codes [rows, cols*bits/8] bytes and one
+    bf16/f16 (scale, bias) pair per group -> AQ blocks [rows, cols/group, 4 + group*bits/8] at the same byte count.
+    Payload bytes are copied; a header f16 does not hold is the f16 NaN 0x7e00 in both halves and is counted.
+    Returns (blocks u8, refused count)."""
+    groups, payload = cols // group, group * bits // 8
+    w = np.ascontiguousarray(mlx_w).view(np.uint8).reshape(rows, groups, payload)
+    with np.errstate(over="ignore"):
+        rs = _mlx_header_f32(scales16, scale_is_f16).reshape(rows, groups)
+        rb = _mlx_header_f32(biases16, scale_is_f16).reshape(rows, groups)
+        hs, hb = rs.astype(np.float16), rb.astype(np.float16)
+    exact = f16_header_holds(rs, hs) & f16_header_holds(rb, hb)
+    blocks = np.empty((rows, groups, 4 + payload), dtype=np.uint8)
+    poison = np.uint16(0x7E00)
+    blocks[..., 0:2] = np.where(exact, hs.view(np.uint16), poison).astype(np.uint16)[..., None].view(np.uint8)
+    blocks[..., 2:4] = np.where(exact, hb.view(np.uint16), poison).astype(np.uint16)[..., None].view(np.uint8)
+    blocks[..., 4:] = w
+    return blocks, int((~exact).sum())
+
+
+def repack_mlx_affine_switch_gate_up(gate_w, gate_s, gate_b, up_w, up_s, up_b, experts: int, inter: int, cols: int, bits: int,
+                                     group: int, scale_is_f16: bool):
+    """qwg_repack_mlx_affine_switch_gate_up_to_aq_m5 (qw_online_quant.metal:124-178): gate_proj and up_proj
+    [experts, inter, cols] interleaved per expert into one [experts, 2*inter, cols] AQ bank (gate rows, then up rows)."""
+    g, rg = repack_mlx_affine(gate_w, gate_s, gate_b, experts * inter, cols, bits, group, scale_is_f16)
+    u, ru = repack_mlx_affine(up_w, up_s, up_b, experts * inter, cols, bits, group, scale_is_f16)
+    nb, bb = g.shape[1], g.shape[2]
+    out = np.concatenate([g.reshape(experts, inter, nb, bb), u.reshape(experts, inter, nb, bb)], axis=1)
+    return out.reshape(experts * 2 * inter, nb, bb), rg + ru
+
+
 def weights_affine_f64(blocks: np.ndarray, bits: int, group: int, is_m5: bool) -> np.ndarray:
     """The un-rounded real weights (q+1024)*s + b (M5) / code*s + b (blocks) in float64: what the reference's
     factorised GEMVs contract, scale * sum(code * x) + bias * sum(x) per slice (qwg_aq_slice_dot,

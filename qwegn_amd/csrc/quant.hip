@@ -58,3 +58,123 @@ extern "C" qwhip_status qwhip_quantize_hq4_g32(qwhip_stream_t s, const void* src
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// MLX affine checkpoint -> AQ blocks at the same byte count (qwg_repack_mlx_affine_to_aq_m5 and its switch gate|up
+// variant, Sources/QWMetal/quant/qw_online_quant.metal:56-178; doors Sources/Foundation/QWLoad/AQRepack.swift:108-250).
+// A block is [f16 scale][f16 bias][payload]: the payload bytes are the checkpoint's, the header is the checkpoint's
+// bf16 / f16 scale and bias as f16.  A header that f16 does not hold (overflow, or a value lost in the normal range;
+// below 2^-14 the nearest subnormal is accepted) is poisoned with the f16 NaN 0x7e00 and counted in `refused`.
+// One thread per output dword (header word or payload word), so both streams are read and written in whole lines.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float qw_read_scale(const uint16_t* p, uint32_t is_f16, uint64_t i) {
+    const uint16_t b = p[i];
+    return is_f16 ? (float)__builtin_bit_cast(h1_t, b) : qw_bf16_to_f32(b);
+}
+
+__device__ __forceinline__ bool qw_f16_header_holds(float raw, h1_t stored) {
+    const float back = (float)stored;
+    if (back == raw) return true;
+    const bool fin = (__float_as_uint(raw) & 0x7F800000u) != 0x7F800000u && (__float_as_uint(back) & 0x7F800000u) != 0x7F800000u;
+    return fin && fabsf(raw) < 6.103515625e-5f;
+}
+
+// SWITCH: source rows come from two [experts, inter, cols] tensors interleaved per expert as [gate rows | up rows].
+template <bool SWITCH>
+__global__ __launch_bounds__(256) void qw_repack_mlx_kernel(const uint32_t* __restrict__ w0, const uint16_t* __restrict__ s0,
+                                                            const uint16_t* __restrict__ b0, const uint32_t* __restrict__ w1,
+                                                            const uint16_t* __restrict__ s1, const uint16_t* __restrict__ b1,
+                                                            uint32_t* __restrict__ dst, uint64_t blocks, uint32_t groups,
+                                                            uint32_t pay_words, uint32_t inter, uint32_t is_f16,
+                                                            uint32_t* __restrict__ refused) {
+    const uint32_t W = pay_words + 1u;
+    const uint64_t d = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (d >= blocks * W) return;
+    const uint64_t b = d / W;
+    const uint32_t j = (uint32_t)(d - b * W);
+    uint64_t src_group = b;
+    const uint32_t* w = w0;
+    const uint16_t* sc = s0;
+    const uint16_t* bi = b0;
+    if constexpr (SWITCH) {
+        const uint64_t out_row = b / groups;
+        const uint32_t g = (uint32_t)(b - out_row * groups);
+        const uint64_t e = out_row / (2u * inter);
+        const uint32_t local = (uint32_t)(out_row - e * (2u * inter));
+        const bool up = local >= inter;
+        src_group = (e * inter + (up ? local - inter : local)) * groups + g;
+        if (up) {
+            w = w1;
+            sc = s1;
+            bi = b1;
+        }
+    }
+    if (j == 0u) {
+        const float rs = qw_read_scale(sc, is_f16, src_group), rb = qw_read_scale(bi, is_f16, src_group);
+        const h1_t hs = (h1_t)rs, hb = (h1_t)rb;
+        const bool exact = qw_f16_header_holds(rs, hs) && qw_f16_header_holds(rb, hb);
+        if (!exact) atomicAdd(refused, 1u);
+        const uint32_t lo = exact ? (uint32_t)__builtin_bit_cast(uint16_t, hs) : 0x7E00u;
+        const uint32_t hi = exact ? (uint32_t)__builtin_bit_cast(uint16_t, hb) : 0x7E00u;
+        dst[d] = lo | (hi << 16);
+    } else {
+        dst[d] = w[src_group * pay_words + (j - 1u)];
+    }
+}
+
+namespace {
+qwhip_status repack_checks(qwhip_stream_t s, uint32_t scale_dtype, uint64_t rows, uint32_t cols, uint32_t bits, uint32_t group,
+                           const void* dst, const uint32_t* refused) {
+    QWHIP_REQUIRE(s);
+    QWHIP_REQUIRE(dst);
+    QWHIP_REQUIRE(refused);
+    if (scale_dtype != QWHIP_BF16 && scale_dtype != QWHIP_F16)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "MLX scales and biases are bf16 or f16, got dtype %u", scale_dtype);
+    if (rows == 0 || cols == 0 || bits == 0 || bits > 8 || group == 0 || cols % group != 0 || (group * bits) % 32 != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "invalid MLX group layout (rows=%llu cols=%u bits=%u group=%u)",
+                          (unsigned long long)rows, cols, bits, group);
+    if (((uintptr_t)dst & 3u) != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "the AQ plane must be 4-byte aligned");
+    return QWHIP_OK;
+}
+}  // namespace
+
+extern "C" qwhip_status qwhip_repack_mlx_affine(qwhip_stream_t s, const void* mlx_w, const void* mlx_scales, const void* mlx_biases,
+                                                uint32_t scale_dtype, uint32_t rows, uint32_t cols, uint32_t bits, uint32_t group,
+                                                void* dst_blocks, uint32_t* refused) {
+    qwhip_status st = repack_checks(s, scale_dtype, rows, cols, bits, group, dst_blocks, refused);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(mlx_w);
+    QWHIP_REQUIRE(mlx_scales);
+    QWHIP_REQUIRE(mlx_biases);
+    const uint32_t groups = cols / group, pay_words = group * bits / 32u;
+    const uint64_t blocks = (uint64_t)rows * groups, total = blocks * (pay_words + 1u);
+    const dim3 grid((unsigned)((total + 255u) / 256u)), block(256);
+    hipLaunchKernelGGL(qw_repack_mlx_kernel<false>, grid, block, 0, s->stream, (const uint32_t*)mlx_w, (const uint16_t*)mlx_scales,
+                       (const uint16_t*)mlx_biases, nullptr, nullptr, nullptr, (uint32_t*)dst_blocks, blocks, groups, pay_words, 0u,
+                       scale_dtype == QWHIP_F16 ? 1u : 0u, refused);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+extern "C" qwhip_status qwhip_repack_mlx_affine_switch_gate_up(qwhip_stream_t s, const void* gate_w, const void* gate_scales,
+                                                               const void* gate_biases, const void* up_w, const void* up_scales,
+                                                               const void* up_biases, uint32_t scale_dtype, uint32_t experts,
+                                                               uint32_t inter, uint32_t cols, uint32_t bits, uint32_t group,
+                                                               void* dst_blocks, uint32_t* refused) {
+    qwhip_status st = repack_checks(s, scale_dtype, (uint64_t)experts * 2u * inter, cols, bits, group, dst_blocks, refused);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(gate_w);
+    QWHIP_REQUIRE(gate_scales);
+    QWHIP_REQUIRE(gate_biases);
+    QWHIP_REQUIRE(up_w);
+    QWHIP_REQUIRE(up_scales);
+    QWHIP_REQUIRE(up_biases);
+    const uint32_t groups = cols / group, pay_words = group * bits / 32u;
+    const uint64_t blocks = (uint64_t)experts * 2u * inter * groups, total = blocks * (pay_words + 1u);
+    const dim3 grid((unsigned)((total + 255u) / 256u)), block(256);
+    hipLaunchKernelGGL(qw_repack_mlx_kernel<true>, grid, block, 0, s->stream, (const uint32_t*)gate_w, (const uint16_t*)gate_scales,
+                       (const uint16_t*)gate_biases, (const uint32_t*)up_w, (const uint16_t*)up_scales, (const uint16_t*)up_biases,
+                       (uint32_t*)dst_blocks, blocks, groups, pay_words, inter, scale_dtype == QWHIP_F16 ? 1u : 0u, refused);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}

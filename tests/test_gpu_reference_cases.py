@@ -146,3 +146,70 @@ def test_small_tiles_match_the_64_row_tiles_bit_for_bit(dev):
         order = inv.download(np.int32, (pairs,))
         outs.append(got[order])                    # back to pair order: slot order inside an expert is arbitrary
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+
+
+def _mlx_checkpoint(rng, rows, cols, bits, group, f16):
+    """A synthetic MLX affine tensor: packed codes, and one (scale, bias) pair per group in bf16 or f16."""
+    groups, payload = cols // group, group * bits // 8
+    w = rng.integers(0, 256, size=(rows, groups * payload), dtype=np.uint8)
+    sc = (rng.uniform(1e-3, 0.05, size=rows * groups)).astype(np.float32)
+    bi = (-sc * rng.uniform(2, 9, size=rows * groups)).astype(np.float32)
+    if f16:
+        return w, sc.astype(np.float16).view(np.uint16), bi.astype(np.float16).view(np.uint16)
+    return w, qo.f32_to_bf16_bits(sc), qo.f32_to_bf16_bits(bi)
+
+
+@pytest.mark.parametrize("bits,group", [(4, 32), (4, 64), (8, 32), (8, 128), (3, 32), (2, 64)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_mlx_repack_writes_the_oracles_bytes(dev, bits, group, f16):
+    """qwhip_repack_mlx_affine vs the oracle's restatement of qwg_repack_mlx_affine_to_aq_m5, byte for byte, with
+    headers f16 cannot hold (too large, NaN, infinite, below 2^-14) in the mix: poisoned and counted, or accepted."""
+    rng = np.random.default_rng(bits * 100 + group + f16)
+    rows, cols = 37, 4 * group
+    w, s16, b16 = _mlx_checkpoint(rng, rows, cols, bits, group, f16)
+    if not f16:
+        s16[3], b16[7], s16[11], b16[20] = 0x7F00, 0x7FC0, 0x7F80, 0x0080     # 1.7e38, NaN, +inf, 1.2e-38 (bf16)
+    else:
+        s16[3], b16[7] = 0x7E00, 0x0001                                         # NaN, smallest subnormal (f16)
+    want, refused = qo.repack_mlx_affine(w, s16, b16, rows, cols, bits, group, scale_is_f16=f16)
+    wb, sb, bb_ = dev.put(w), dev.put(s16), dev.put(b16)
+    out = dev.alloc(want.nbytes)
+    cnt = dev.put(np.zeros(1, np.uint32))
+    qwhip.check(dev.lib.qwhip_repack_mlx_affine(dev.stream.handle, wb.ptr, sb.ptr, bb_.ptr, qwhip.F16 if f16 else qwhip.BF16,
+                                                rows, cols, bits, group, out.ptr, cnt.ptr))
+    dev.stream.sync()
+    assert np.array_equal(out.download(np.uint8, want.shape), want)
+    assert int(cnt.download(np.uint32, (1,))[0]) == refused and refused >= 1
+
+
+def test_mlx_repack_switch_gate_up_interleaves_experts(dev):
+    """qwhip_repack_mlx_affine_switch_gate_up: [experts, inter, cols] gate and up tensors -> one [experts, 2*inter, cols]
+    bank, byte for byte; the bank then multiplies like any other AQ4_G64 bank."""
+    rng = np.random.default_rng(77)
+    experts, inter, cols, bits, group = 3, 40, 256, 4, 64
+    gw, gs, gb = _mlx_checkpoint(rng, experts * inter, cols, bits, group, False)
+    uw, us, ub = _mlx_checkpoint(rng, experts * inter, cols, bits, group, False)
+    want, refused = qo.repack_mlx_affine_switch_gate_up(gw, gs, gb, uw, us, ub, experts, inter, cols, bits, group, False)
+    bufs = [dev.put(a) for a in (gw, gs, gb, uw, us, ub)]
+    out, cnt = dev.alloc(want.nbytes), dev.put(np.zeros(1, np.uint32))
+    qwhip.check(dev.lib.qwhip_repack_mlx_affine_switch_gate_up(dev.stream.handle, *[b.ptr for b in bufs], qwhip.BF16, experts, inter,
+                                                               cols, bits, group, out.ptr, cnt.ptr))
+    dev.stream.sync()
+    assert refused == 0 and int(cnt.download(np.uint32, (1,))[0]) == 0
+    assert np.array_equal(out.download(np.uint8, want.shape), want)
+    n = experts * 2 * inter
+    x16 = rng.standard_normal((1, cols)).astype(np.float16)
+    xb, y32 = dev.put(x16), dev.alloc(n * 4)
+    view = dev.view(out, n, cols, qwhip.KIND_NATIVE_AFFINE, bits, group)
+    qwhip.check(dev.lib.qwhip_gemv(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, 1, 0, None, y32.ptr))
+    dev.stream.sync()
+    ref = qo.matmul_ref_f64(x16, qo.weights_f16_exact(want, bits, group, False))
+    assert qo.normalized_error(y32.download(np.float32, (1, n)), ref) <= 2e-3
+
+
+def test_mlx_repack_rejects_bad_layouts_before_launch(dev):
+    z = dev.put(np.zeros(64, np.uint8))
+    st = dev.stream.handle
+    assert dev.lib.qwhip_repack_mlx_affine(st, z.ptr, z.ptr, z.ptr, qwhip.F32, 1, 64, 4, 32, z.ptr, z.ptr) == qwhip.E_BAD_SHAPE
+    assert dev.lib.qwhip_repack_mlx_affine(st, z.ptr, z.ptr, z.ptr, qwhip.BF16, 1, 48, 4, 32, z.ptr, z.ptr) == qwhip.E_BAD_SHAPE
+    assert dev.lib.qwhip_repack_mlx_affine(st, z.ptr, z.ptr, z.ptr, qwhip.BF16, 1, 64, 4, 32, z.ptr, None) == qwhip.E_NULL

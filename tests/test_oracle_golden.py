@@ -81,6 +81,48 @@ def test_aq_block_unpack_matches_mlx_witness(golden_dir):
         assert np.max(np.abs(got - values)) < 1e-5
 
 
+def test_mlx_repack_keeps_the_witness_codes_and_values(golden_dir):
+    """aq_repack_golden.json through the repacker: the payload of every block is the MLX packed bytes, the header the
+    f16 of the (bf16-rounded) MLX scale and bias, and the dequantized block is the witness's value wherever the header
+    is exact in bf16 and f16 alike."""
+    doc = json.loads((golden_dir / "aq_repack_golden.json").read_text())
+    rows, cols, group, bits = doc["rows"], doc["cols"], doc["group"], doc["bits"]
+    packed = np.frombuffer(bytes.fromhex(doc["packed"]), dtype=np.uint8).reshape(rows, cols * bits // 8)
+    scales = np.frombuffer(bytes.fromhex(doc["scales"]), dtype=np.float32)
+    biases = np.frombuffer(bytes.fromhex(doc["biases"]), dtype=np.float32)
+    values = np.frombuffer(bytes.fromhex(doc["values"]), dtype=np.float32).reshape(rows, cols)
+    s16, b16 = qo.f32_to_bf16_bits(scales), qo.f32_to_bf16_bits(biases)
+    blocks, refused = qo.repack_mlx_affine(packed, s16, b16, rows, cols, bits, group, scale_is_f16=False)
+    assert refused == 0 and blocks.shape == (rows, cols // group, qo.hq_block_bytes(bits, group))
+    assert np.array_equal(blocks[..., 4:].reshape(rows, -1), packed)
+    hs, hb = qo.hq_block_header(blocks)
+    assert np.array_equal(hs.ravel(), qo.bf16_bits_to_f32(s16).astype(np.float16).astype(np.float32))
+    got = qo.dequant_hq_blocks_rot(blocks, bits, group)
+    exact = (qo.bf16_bits_to_f32(s16) == scales) & (qo.bf16_bits_to_f32(b16) == biases)
+    cols_ok = np.repeat(exact.reshape(rows, -1), group, axis=1)
+    if cols_ok.any():
+        assert np.max(np.abs(got[cols_ok] - values[cols_ok])) < 1e-5
+
+
+def test_f16_header_rule_on_every_bf16_value():
+    """The exactness rule against first principles on all 65,536 bf16 patterns: a finite bf16 value is held by f16 iff it
+    is 0, or 2^-14 <= |v| <= 65504 (8 significant bits always fit f16's 11); smaller magnitudes are accepted by the
+    rule anyway, larger ones overflow and are refused; infinities convert back to themselves; NaN never does."""
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    v = qo.bf16_bits_to_f32(bits)
+    with np.errstate(over="ignore", invalid="ignore"):
+        holds = qo.f16_header_holds(v, v.astype(np.float16))
+    with np.errstate(invalid="ignore"):
+        a = np.abs(v.astype(np.float64))
+    want = np.where(np.isnan(v), False, np.where(np.isinf(v), True, a <= 65504.0 + 16.0 - 1e-9))
+    # |v| in (65504, 65520) would round down to 65504 and be refused by the round trip; bf16 has no value there
+    assert not np.any((a > 65504.0) & (a < 65536.0))
+    assert np.array_equal(holds, want)
+    blocks, refused = qo.repack_mlx_affine(np.zeros((1, 16), np.uint8), np.array([0x7F00], np.uint16), np.array([0x3F80], np.uint16),
+                                           1, 32, 4, 32, scale_is_f16=False)       # scale 1.7e38: refused, both halves poisoned
+    assert refused == 1 and bytes(blocks[0, 0, :4]) == b"\x00\x7e\x00\x7e"
+
+
 CASES = [
     ("aq4_g32_std", 4, 32, False, False),
     ("hq4_g32_blk", 4, 32, False, True),
