@@ -213,3 +213,42 @@ def test_mlx_repack_rejects_bad_layouts_before_launch(dev):
     assert dev.lib.qwhip_repack_mlx_affine(st, z.ptr, z.ptr, z.ptr, qwhip.F32, 1, 64, 4, 32, z.ptr, z.ptr) == qwhip.E_BAD_SHAPE
     assert dev.lib.qwhip_repack_mlx_affine(st, z.ptr, z.ptr, z.ptr, qwhip.BF16, 1, 48, 4, 32, z.ptr, z.ptr) == qwhip.E_BAD_SHAPE
     assert dev.lib.qwhip_repack_mlx_affine(st, z.ptr, z.ptr, z.ptr, qwhip.BF16, 1, 64, 4, 32, z.ptr, None) == qwhip.E_NULL
+
+
+def test_pack_plane_mover_feeds_the_kernels(dev, golden_dir, tmp_path):
+    """selfpack.qwp through the plane mover: the device bank dequantizes to the f16 weights of the pack's own blocks
+    (bit-exact), and multiplies like them.  A synthetic expert stack becomes one [E * N, K] bank."""
+    from qwegn_amd import pack as qp
+    from tests.test_pack import write_pack
+
+    p = qp.Pack(golden_dir / "selfpack.qwp")
+    buf, view = p.upload(dev, "w_test", chunk_bytes=50_000)        # several chunks
+    n, k = view.n, view.k
+    blocks = np.asarray(p.plane("w_test")[1]).reshape(n, k // 32, 20)
+    w16 = qo.weights_f16_exact(blocks, 4, 32, True)
+    out = dev.alloc(n * k * 2)
+    qwhip.check(dev.lib.qwhip_dequant_f16(dev.stream.handle, C.byref(view), out.ptr))
+    dev.stream.sync()
+    assert np.array_equal(out.download(np.float16, (n, k)).view(np.uint16), w16.view(np.uint16))
+    x16 = np.random.default_rng(4).standard_normal((1, k)).astype(np.float16)
+    xb, y32 = dev.put(x16), dev.alloc(n * 4)
+    qwhip.check(dev.lib.qwhip_gemv(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, 1, 0, None, y32.ptr))
+    dev.stream.sync()
+    ref = qo.matmul_ref_f64(qo.rotate_activation_f16(x16), w16)
+    assert qo.normalized_error(y32.download(np.float32, (1, n)), ref) <= 2e-3
+    raw_buf, raw_view = p.upload(dev, "norm_test")
+    assert raw_view is None and np.array_equal(raw_buf.download(np.uint8, (512,)), np.asarray(p.plane("norm_test")[1]))
+
+    rng = np.random.default_rng(1)
+    experts, rows, kk = 4, 16, 256
+    w = (rng.standard_normal((experts * rows, kk)) * 0.02).astype(np.float32)
+    hq4 = qo.quant_hq4_blocks(w)
+    write_pack(tmp_path / "e.qwp", {"mlp.experts.down": ({"shape": [experts, rows, kk], "experts": experts,
+                                                           "e_hq4": rows * (kk // 32) * 20}, hq4.tobytes(), "hq4_off")})
+    ebuf, eview = qp.Pack(tmp_path / "e.qwp").upload(dev, "mlp.experts.down")
+    assert (eview.n, eview.k, eview.kind) == (experts * rows, kk, qwhip.KIND_HQ4_G32_M5)
+    eout = dev.alloc(experts * rows * kk * 2)
+    qwhip.check(dev.lib.qwhip_dequant_f16(dev.stream.handle, C.byref(eview), eout.ptr))
+    dev.stream.sync()
+    assert np.array_equal(eout.download(np.float16, (experts * rows, kk)).view(np.uint16),
+                          qo.weights_f16_exact(hq4, 4, 32, True).view(np.uint16))
