@@ -10,7 +10,7 @@ kernel measured with HIP events on the launch stream, and the CPU baseline (the 
 oracle form - dequantize the bank to fp32, then one fp32 product - restated in numpy and timed
 on this box's host cores over a bounded sample).
 
-Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up (see WORKLOADS).
+Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up|norm_prefill|norm_decode (see WORKLOADS).
 """
 from __future__ import annotations
 
@@ -205,6 +205,55 @@ def run_silu_pair(args, fmt, inter, k, m, label):
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": algo_bytes,
                      "kernel_us": round(us_per, 3)},
         "normalized_error": err,
+    }
+
+
+def run_norm(args, rows, hidden, label):
+    """RMSNorm + rotation producer with the fused residual update: one step = one launch over [rows, hidden] f16.
+    Algorithmic bytes: x read, residual read and written, y written, gamma read."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+
+    dev = qwhip.Device(0)
+    rng = np.random.default_rng(0)
+    x16 = rng.standard_normal((rows, hidden)).astype(np.float16)
+    gam = (rng.standard_normal(hidden) * 0.1).astype(np.float16)
+    res0 = rng.standard_normal((rows, hidden)).astype(np.float16)
+    xb, gb, rb, yb = dev.put(x16), dev.put(gam), dev.put(res0), dev.alloc(rows * hidden * 2)
+    lib, st = dev.lib, dev.stream.handle
+
+    def launch(i):
+        qwhip.check(lib.qwhip_rmsnorm(st, xb.ptr, gb.ptr, rb.ptr, rows, hidden, 1e-6, 1, yb.ptr))
+
+    launch(0)
+    dev.stream.sync()
+    want, want_res = qo.rmsnorm_rot_f16(x16, gam, 1e-6, residual16=res0)
+    got = yb.download(np.float16, (rows, hidden))
+    err = float(np.max(np.abs(got.astype(np.float32) - want.astype(np.float32))))
+    if not (err <= 1e-3 * max(1.0, float(np.max(np.abs(want)))) and np.array_equal(rb.download(np.float16, (rows, hidden)), want_res)):
+        _fail(f"bench: norm output failed parity (max abs error {err:.3e})")
+    _spin_up(dev, launch)
+    for i in range(args.warmup):
+        launch(i)
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        launch(i)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    algo_bytes = rows * hidden * 2 * 4 + hidden * 2
+    gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": label, "rows": rows, "hidden": hidden, "residual": True, "rotate": True},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
+        "max_abs_error": err,
     }
 
 
@@ -468,6 +517,8 @@ WORKLOADS = {
     "c5_qkv": ("gemv", "hq8_g32", 7168, 5120, None, False),
     "c5_down": ("gemv", "hq4_g64", 5120, 17408, None, False),
     "mlp_gate_up": ("pair", "hq4_g32_m5", 17408, 5120, 1, False),      # n = intermediate size: the bank has 2n rows
+    "norm_prefill": ("norm", None, 5120, None, 4096, False),           # n = hidden, m = rows
+    "norm_decode": ("norm", None, 5120, None, 1, False),
 }
 LABELS = {
     "c1": "C1 AQ4_G32 affine GEMV N=4096 K=4096",
@@ -478,6 +529,8 @@ LABELS = {
     "c5_qkv": "C5 verify GEMM HQ8_G32 K=5120 N=7168",
     "c5_down": "C5 verify GEMM HQ4_G64 K=17408 N=5120",
     "mlp_gate_up": "dense MLP gate|up GEMV + SwiGLU + FWHT, HQ4_G32 M=1 K=5120 I=17408",
+    "norm_prefill": "RMSNorm + residual + FWHT producer, 4096 rows x 5120",
+    "norm_decode": "RMSNorm + residual + FWHT producer, 1 row x 5120",
 }
 
 
@@ -519,6 +572,8 @@ def main() -> None:
         m = args.m
     if kind == "moe":
         out = run_moe(args, m, LABELS[args.workload])
+    elif kind == "norm":
+        out = run_norm(args, m, n, LABELS[args.workload])
     elif kind == "pair":
         out = run_silu_pair(args, fmt, n, k, m, LABELS[args.workload])
     elif kind == "gemm":

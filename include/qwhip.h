@@ -129,6 +129,13 @@ enum {
 /* qwg_fwht32_f16 (Sources/QWMetal/gemm/qwgemm.metal:27-32; QWGemm.encodeFwht32, QWGemm.swift:288-300):
  * normalized FWHT-32 over consecutive 32-groups, src dtype f16/bf16/f32 -> dst f16 (dst may equal src for f16). */
 qwhip_status qwhip_fwht32(qwhip_stream_t s, const void* src, uint32_t src_dtype, void* dst_f16, uint64_t n);
+/* qwg_rmsnorm / qwg_rmsnorm_residual (Sources/QWMetal/mlp_norm_rope/qwnorm.metal:27-79, 127-189; encodeRMSNormFast /
+ * encodeRMSNormResidualFast, Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:339-404): the producer in front of the
+ * projections.  y [rows, hidden] f16 = f16(FWHT32(x * rsqrt(mean(x^2) + eps) * (1 + gamma))), fp32 inside, gamma stored raw
+ * (plus-one law); with `residual_f16` (in/out, may be NULL) the row normalized is residual <- f16(residual + x), stored
+ * back bit-exactly.  hidden % 256 == 0 (the reference driver's contract); `rotate` = 0 leaves the row in the standard basis. */
+qwhip_status qwhip_rmsnorm(qwhip_stream_t s, const void* x_f16, const void* gamma_f16, void* residual_f16, uint32_t rows,
+                           uint32_t hidden, float eps, uint32_t rotate, void* y_f16);
 /* qwg_cast_f32_to_f16 (QWGemm.encodeCast, QWGemm.swift:305-320). */
 qwhip_status qwhip_cast_f32_to_f16(qwhip_stream_t s, const float* src, void* dst_f16, uint64_t n);
 /* qwg_silu_mul_f16 / qwg_silu_mul_split_f16 (Sources/QWMetal/gemm/qwgemm_batched.metal:58-97;

@@ -455,6 +455,28 @@ def rotate_activation_f16(x: np.ndarray) -> np.ndarray:
     return fwht32_ortho(np.asarray(x).astype(np.float32)).astype(np.float16)
 
 
+def rmsnorm_rot_f16(x16: np.ndarray, gamma16: np.ndarray, eps: float, rotate: bool = True, residual16: np.ndarray | None = None):
+    """qwg_rmsnorm / qwg_rmsnorm_residual (Sources/QWMetal/mlp_norm_rope/qwnorm.metal:27-79, 127-189):
+    y = f16(fwht32(x * rsqrt(mean(x^2) + eps) * (1 + gamma))), gamma stored raw (plus-one law), fp32 products in the
+    kernel's order ((x * rstd) * (gamma + 1)), fp32 transform in the butterfly order of fwht32_f32_inplace
+    (qw_dequant.metalh:442-478, the order of `fwht32_ortho`), one f16 rounding at the end.  With `residual16` the row
+    normalized is f16(f32(residual) + f32(x)), which is also returned (the kernel stores it back).
+    The mean of squares is evaluated in float64 and rounded to fp32 (the kernel's fp32 summation order is not part of
+    the contract).  Returns (y f16, residual_out f16 or None)."""
+    x = np.asarray(x16, dtype=np.float16)
+    res_out = None
+    if residual16 is not None:
+        x = (x.astype(np.float32) + np.asarray(residual16, dtype=np.float16).astype(np.float32)).astype(np.float16)
+        res_out = x
+    xf = x.astype(np.float32)
+    ms = (xf.astype(np.float64) ** 2).mean(axis=-1, keepdims=True)
+    rstd = (1.0 / np.sqrt(ms + np.float64(np.float32(eps)))).astype(np.float32)
+    f = (xf * rstd) * (np.asarray(gamma16, dtype=np.float16).astype(np.float32) + np.float32(1.0))
+    if rotate:
+        f = fwht32_ortho(f)
+    return f.astype(np.float16), res_out
+
+
 def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     """silu(g)*u = g/(1+exp(-g))*u in fp32 (Sources/QWMetal/include/qw_weight_basis.metalh:50-63,
     plain SwiGLU branch; Scripts/oracle/gen_mlp_fixtures.py:79)."""

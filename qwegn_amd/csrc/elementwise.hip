@@ -229,3 +229,118 @@ extern "C" qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_v
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// RMSNorm with the rotation fused (the producer in front of every projection of a decode layer):
+//   y = f16( FWHT32( x * rsqrt(mean(x^2) + eps) * (1 + gamma) ) ),  optionally after  residual <- f16(residual + x)
+// (qwg_rmsnorm / qwg_rmsnorm_residual, Sources/QWMetal/mlp_norm_rope/qwnorm.metal:27-79, 127-189; doors
+// encodeRMSNormFast / encodeRMSNormResidualFast, Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:339-404).
+// Plus-one law: gamma is stored raw and applied as (1 + gamma) in fp32; sum of squares in fp32; the 32-point
+// transform in fp32 in the butterfly order of fwht32_f32_inplace (qw_dequant.metalh:442-478: strides 1, 2, 4 inside a
+// lane's 8 values, 8 and 16 across 4 lanes, times 1/sqrt(32)); one f16 rounding at the store.
+// One workgroup per row; a thread owns 8 consecutive values per 2048-column sweep (16-byte loads, the row stays in
+// registers up to 16384 columns); four neighbouring lanes hold one 32-group.
+// ------------------------------------------------------------------------------------------------
+template <bool RESIDUAL>
+__global__ __launch_bounds__(256) void qw_rmsnorm_kernel(const h1_t* __restrict__ x, const h1_t* __restrict__ gamma,
+                                                         h1_t* __restrict__ residual, h1_t* __restrict__ y, uint32_t hidden,
+                                                         float eps, uint32_t rotate) {
+    constexpr int SW = 8;   // sweeps held in registers
+    __shared__ float wsum[4];
+    const uint32_t tid = threadIdx.x;
+    const uint64_t row = (uint64_t)blockIdx.x * hidden;
+    h8_t v[SW];
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < SW; ++k) {
+        const uint32_t c = (k * 256u + tid) * 8u;
+        if (c < hidden) {
+            h8_t xv = *(const h8_t*)(x + row + c);
+            if constexpr (RESIDUAL) {
+                const h8_t rv = *(const h8_t*)(residual + row + c);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[i] = (h1_t)((float)xv[i] + (float)rv[i]);
+                *(h8_t*)(residual + row + c) = xv;
+            }
+            v[k] = xv;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float t = (float)xv[i];
+                acc = fmaf(t, t, acc);
+            }
+        }
+    }
+    acc = qw_reduce64(acc);
+    if ((tid & 63u) == 0u) wsum[tid >> 6] = acc;
+    __syncthreads();
+    const float total = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+    const float rstd = 1.0f / sqrtf(total / (float)hidden + eps);
+#pragma unroll
+    for (int k = 0; k < SW; ++k) {
+        const uint32_t c = (k * 256u + tid) * 8u;
+        if (c >= hidden) continue;   // whole quads of lanes leave together: hidden is a multiple of 32
+        const h8_t gv = *(const h8_t*)(gamma + c);
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)v[k][i] * rstd * ((float)gv[i] + 1.0f);
+        if (rotate) {
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                const float a = f[i], b = f[i + 1];
+                f[i] = a + b;
+                f[i + 1] = a - b;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i += 4) {
+                const float a0 = f[i], a1 = f[i + 1], b0 = f[i + 2], b1 = f[i + 3];
+                f[i] = a0 + b0;
+                f[i + 1] = a1 + b1;
+                f[i + 2] = a0 - b0;
+                f[i + 3] = a1 - b1;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float a = f[i], b = f[i + 4];
+                f[i] = a + b;
+                f[i + 4] = a - b;
+            }
+            const bool neg1 = (tid & 1u) != 0u, neg2 = (tid & 2u) != 0u;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, f[i]), 0xB1, 0xF, 0xF, true));
+                f[i] = neg1 ? (p - f[i]) : (f[i] + p);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, f[i]), 0x4E, 0xF, 0xF, true));
+                f[i] = (neg2 ? (p - f[i]) : (f[i] + p)) * QW_INV_SQRT32;
+            }
+        }
+        h8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (h1_t)f[i];
+        *(h8_t*)(y + row + c) = o;
+    }
+}
+
+extern "C" qwhip_status qwhip_rmsnorm(qwhip_stream_t s, const void* x_f16, const void* gamma_f16, void* residual_f16, uint32_t rows,
+                                      uint32_t hidden, float eps, uint32_t rotate, void* y_f16) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(x_f16);
+    QWHIP_REQUIRE(gamma_f16);
+    QWHIP_REQUIRE(y_f16);
+    if (hidden == 0 || hidden % 256u != 0u)
+        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the norm family needs a hidden that is a multiple of 256, got %u", hidden);
+    if (hidden > 16384u) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the norm kernel holds rows of at most 16384 columns, got %u", hidden);
+    if (((uintptr_t)x_f16 | (uintptr_t)gamma_f16 | (uintptr_t)y_f16 | (uintptr_t)residual_f16) & 15u)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "the norm kernel needs 16-byte aligned rows");
+    if (residual_f16)
+        hipLaunchKernelGGL(qw_rmsnorm_kernel<true>, dim3(rows), dim3(256), 0, s->stream, (const h1_t*)x_f16, (const h1_t*)gamma_f16,
+                           (h1_t*)residual_f16, (h1_t*)y_f16, hidden, eps, rotate ? 1u : 0u);
+    else
+        hipLaunchKernelGGL(qw_rmsnorm_kernel<false>, dim3(rows), dim3(256), 0, s->stream, (const h1_t*)x_f16, (const h1_t*)gamma_f16,
+                           (h1_t*)nullptr, (h1_t*)y_f16, hidden, eps, rotate ? 1u : 0u);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}

@@ -84,6 +84,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
         b"qwg_moe_down_reduce_combine_f32": b"qwhip_moe_combine", b"qwg_moe_gateup_q4g_f32_r1": b"qwhip_moe_gateup_decode",
         b"qwg_moe_down_shared_combine_q4g_f32": b"qwhip_moe_down_decode", b"qwg_fwht32_f16": b"qwhip_fwht32",
         b"qwg_quantize_bf16_to_hq4_g32_m5": b"qwhip_quantize_hq4_g32",
+        b"qwg_rmsnorm": b"qwhip_rmsnorm", b"qwg_rmsnorm_residual": b"qwhip_rmsnorm",
         b"qwg_repack_mlx_affine_to_aq_m5": b"qwhip_repack_mlx_affine",
         b"qwg_repack_mlx_affine_switch_gate_up_to_aq_m5": b"qwhip_repack_mlx_affine_switch_gate_up",
     }

@@ -252,3 +252,38 @@ def test_pack_plane_mover_feeds_the_kernels(dev, golden_dir, tmp_path):
     dev.stream.sync()
     assert np.array_equal(eout.download(np.float16, (experts * rows, kk)).view(np.uint16),
                           qo.weights_f16_exact(hq4, 4, 32, True).view(np.uint16))
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 5120), (7, 2048), (33, 256), (4, 16384)])
+@pytest.mark.parametrize("residual", [False, True])
+@pytest.mark.parametrize("rotate", [1, 0])
+def test_rmsnorm_with_rotation_matches_oracle(dev, rows, hidden, residual, rotate):
+    """qwhip_rmsnorm vs the oracle's restatement of qwg_rmsnorm / qwg_rmsnorm_residual: max |diff| <= 1e-3 on the f16
+    output (the reference's own bar, Tests/QWNormTests/QWNormTests.swift:8-10), at most one f16 ulp (or 2e-6 absolute)
+    anywhere (the kernel's fp32 sum of squares runs in another order), and the residual update bit-exact."""
+    rng = np.random.default_rng(rows * 7 + hidden)
+    x16 = (rng.standard_normal((rows, hidden)) * 1.5).astype(np.float16)
+    gam = (rng.standard_normal(hidden) * 0.1).astype(np.float16)
+    res = (rng.standard_normal((rows, hidden)) * 2.0).astype(np.float16) if residual else None
+    eps = 1e-6
+    want, want_res = qo.rmsnorm_rot_f16(x16, gam, eps, rotate=bool(rotate), residual16=res)
+    xb, gb, yb = dev.put(x16), dev.put(gam), dev.alloc(rows * hidden * 2)
+    rb = dev.put(res) if residual else None
+    qwhip.check(dev.lib.qwhip_rmsnorm(dev.stream.handle, xb.ptr, gb.ptr, rb.ptr if residual else None, rows, hidden, eps, rotate, yb.ptr))
+    dev.stream.sync()
+    got = yb.download(np.float16, (rows, hidden))
+    assert np.max(np.abs(got.astype(np.float32) - want.astype(np.float32))) <= 1e-3 * max(1.0, float(np.max(np.abs(want))))
+    ulp = np.abs(got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
+    diff = np.abs(got.astype(np.float32) - want.astype(np.float32))
+    assert np.all((ulp <= 1) | (diff <= 2e-6))     # coefficients that cancel to ~1e-5 carry the fp32 error of their terms
+    assert np.mean(ulp == 0) >= 0.98
+    if residual:
+        assert np.array_equal(rb.download(np.float16, (rows, hidden)).view(np.uint16), want_res.view(np.uint16))
+
+
+def test_rmsnorm_refuses_the_geometries_the_reference_driver_refuses(dev):
+    z = dev.put(np.zeros(4096, np.float16))
+    st = dev.stream.handle
+    assert dev.lib.qwhip_rmsnorm(st, z.ptr, z.ptr, None, 1, 1000, 1e-6, 1, z.ptr) == qwhip.E_BAD_GEOMETRY     # hidden % 256
+    assert dev.lib.qwhip_rmsnorm(st, z.ptr, None, None, 1, 1024, 1e-6, 1, z.ptr) == qwhip.E_NULL
+    assert dev.lib.qwhip_rmsnorm(st, z.ptr, z.ptr, None, 0, 1024, 1e-6, 1, z.ptr) == qwhip.OK                 # no rows: nothing to do

@@ -246,3 +246,32 @@ def test_swiglu_closed_form():
     want = g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u
     np.testing.assert_allclose(qo.swiglu(g, u), want, rtol=1e-6, atol=1e-12)
     assert qo.swiglu_fwht_f16(np.ones((1, 48), np.float32), np.ones((1, 48), np.float32)).shape == (1, 48)  # I % 32 != 0: not rotated
+
+
+def test_rmsnorm_closed_forms():
+    """The norm restatement against what the mathematics fixes: a constant row (one non-zero coefficient per 32-group,
+    c * rstd * (1 + g) * sqrt(32)), the plus-one law at gamma = 0 on a unit-RMS row (y = FWHT32(x)), Parseval between the
+    rotated and the standard-basis output, and the exact residual update."""
+    h, eps = 512, 1e-6
+    c, g = np.float16(0.75), np.float16(0.125)
+    y, _ = qo.rmsnorm_rot_f16(np.full((2, h), c, np.float16), np.full(h, g, np.float16), eps)
+    want0 = float(c) / np.sqrt(float(c) ** 2 + eps) * (1.0 + float(g)) * np.sqrt(32.0)
+    yv = y.astype(np.float64).reshape(2, h // 32, 32)
+    assert np.allclose(yv[..., 0], want0, rtol=1e-3) and np.all(yv[..., 1:] == 0.0)
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((3, h)).astype(np.float32)
+    x16 = (x / np.sqrt((x ** 2).mean(axis=1, keepdims=True))).astype(np.float16)          # unit RMS up to f16 rounding
+    y, _ = qo.rmsnorm_rot_f16(x16, np.zeros(h, np.float16), 0.0)
+    rms = np.sqrt((x16.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+    assert np.max(np.abs(y.astype(np.float64) - qo.fwht32_ortho((x16.astype(np.float64) / rms).astype(np.float32)))) <= 2e-3
+    gam = (rng.standard_normal(h) * 0.1).astype(np.float16)
+    yr, _ = qo.rmsnorm_rot_f16(x16, gam, eps, rotate=True)
+    yp, _ = qo.rmsnorm_rot_f16(x16, gam, eps, rotate=False)
+    assert np.allclose((yr.astype(np.float64) ** 2).sum(axis=1), (yp.astype(np.float64) ** 2).sum(axis=1), rtol=2e-3)
+    # transpose check: the rotated output is the transform of the plain one (up to the one f16 rounding each)
+    assert np.max(np.abs(qo.fwht32_ortho(yp.astype(np.float32)) - yr.astype(np.float32))) <= 4e-3
+    res = rng.standard_normal((3, h)).astype(np.float16)
+    y2, res_out = qo.rmsnorm_rot_f16(x16, gam, eps, residual16=res)
+    assert np.array_equal(res_out, (x16.astype(np.float32) + res.astype(np.float32)).astype(np.float16))
+    y3, _ = qo.rmsnorm_rot_f16(res_out, gam, eps)
+    assert np.array_equal(y2.view(np.uint16), y3.view(np.uint16))
