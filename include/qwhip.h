@@ -175,6 +175,15 @@ qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void
 qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                                   uint32_t m, uint32_t flags, uint32_t rotate_out, void* act16);
 
+/* LM head for greedy decoding (QWGemmAQ.encodeHeadArgmax, QWGemmAQ.swift:306-349; qwg_head_gemv_q4g_argmax,
+ * qwg_gemv_*_f32_v4_am with the fold of qw_gemm_f32_common.metalh:30-58): logits [m, n] f32 = W . x (as qwhip_gemv), then
+ * tokens[m] = argmax with the reference's key rule: floats compared through qw_sortable_f32_u32 (NaN never wins against
+ * a number), ties to the lower row.  `logits` is required and kept (the reference's writeLogits); the reference's key
+ * scratch is not needed.  qwhip_argmax_f32 is the fold alone, over any [rows, n] f32 logits. */
+qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
+                               uint32_t flags, float* logits, int32_t* tokens);
+qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);
+
 /* ---- prefill GEMM: Y[m, n] = X[m, k] . W^T on f16 MFMA, fp32 accumulate ------ */
 /* gemmBatchedH16 (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:119-154) -> qwg_gemm_q4g_h16 /
  * qwg_gemm_aq*_h16; QWGemm.encodeNaxF32 (Sources/Operators/QWGEMM/QWGemmF32.swift:366-402).

@@ -477,6 +477,24 @@ def rmsnorm_rot_f16(x16: np.ndarray, gamma16: np.ndarray, eps: float, rotate: bo
     return f.astype(np.float16), res_out
 
 
+def sortable_f32_u32(x: np.ndarray) -> np.ndarray:
+    """qw_sortable_f32_u32 (Sources/QWMetal/include/qw_fastmath_safe.metalh:21-25): float bits made monotone as
+    unsigned integers, NaN -> 0."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    key = np.where(u & np.uint32(0x80000000), ~u, u ^ np.uint32(0x80000000))
+    return np.where((u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000), np.uint32(0), key).astype(np.uint32)
+
+
+def head_argmax(logits: np.ndarray) -> np.ndarray:
+    """The fold of the head's argmax epilogue (qwg_gemv_am_fold4 / qwg_gemv_am_reduce4,
+    Sources/QWMetal/include/qw_gemm_f32_common.metalh:30-58): per row the largest (sortable(v), ~row) pair wins, so ties
+    go to the lower row and NaN never beats a number."""
+    keys = sortable_f32_u32(np.atleast_2d(logits)).astype(np.uint64) << np.uint64(32)
+    rows = np.arange(keys.shape[-1], dtype=np.uint64)
+    keys = keys | ((~rows) & np.uint64(0xFFFFFFFF))
+    return (~(keys.max(axis=-1) & np.uint64(0xFFFFFFFF)) & np.uint64(0xFFFFFFFF)).astype(np.int32)
+
+
 def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     """silu(g)*u = g/(1+exp(-g))*u in fp32 (Sources/QWMetal/include/qw_weight_basis.metalh:50-63,
     plain SwiGLU branch; Scripts/oracle/gen_mlp_fixtures.py:79)."""

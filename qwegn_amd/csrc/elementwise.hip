@@ -344,3 +344,59 @@ extern "C" qwhip_status qwhip_rmsnorm(qwhip_stream_t s, const void* x_f16, const
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// Greedy-decoding argmax over logits rows, with the reference's key rule (qw_sortable_f32_u32,
+// Sources/QWMetal/include/qw_fastmath_safe.metalh:21-25; fold in qwg_gemv_am_fold4 / qwg_gemv_am_reduce4,
+// Sources/QWMetal/include/qw_gemm_f32_common.metalh:30-58): key hi = the float's bits made monotone (NaN -> 0, so it
+// never wins against a number), key lo = ~row, larger (hi, lo) wins: ties go to the lower row.
+// One workgroup per logits row; 16-byte loads; wave fold with DPP row steps and lane reads, then LDS across waves.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t qw_sortable_f32(float x) {
+    const uint32_t u = __float_as_uint(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0u;
+    return (u & 0x80000000u) ? ~u : (u ^ 0x80000000u);
+}
+
+__global__ __launch_bounds__(1024) void qw_argmax_rows_kernel(const float* __restrict__ logits, uint32_t n, int32_t* __restrict__ tokens) {
+    __shared__ unsigned long long best_w[16];
+    const uint32_t tid = threadIdx.x;
+    const float* row = logits + (uint64_t)blockIdx.x * n;
+    unsigned long long best = 0ull;   // (hi << 32) | lo; every real candidate has lo = ~row > 0 for row < 2^32 - 1
+    const uint32_t n4 = (((uintptr_t)row & 15u) == 0u) ? (n & ~3u) : 0u;
+    for (uint32_t i = tid * 4u; i < n4; i += 4096u) {
+        const f4_t v = *(const f4_t*)(row + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned long long key = ((unsigned long long)qw_sortable_f32(v[j]) << 32) | (uint32_t)~(i + j);
+            best = key > best ? key : best;
+        }
+    }
+    for (uint32_t i = n4 + tid; i < n; i += 1024u) {
+        const unsigned long long key = ((unsigned long long)qw_sortable_f32(row[i]) << 32) | (uint32_t)~i;
+        best = key > best ? key : best;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(best, off, 64);
+        best = o > best ? o : best;
+    }
+    if ((tid & 63u) == 0u) best_w[tid >> 6] = best;
+    __syncthreads();
+    if (tid == 0u) {
+#pragma unroll
+        for (int w = 1; w < 16; ++w) best = best_w[w] > best ? best_w[w] : best;
+        tokens[blockIdx.x] = (int32_t)~(uint32_t)best;
+    }
+}
+
+extern "C" qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(logits);
+    QWHIP_REQUIRE(tokens);
+    if (n == 0 || n >= (1u << 30)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "argmax over %u logits does not fit the row-count flags", n);
+    hipLaunchKernelGGL(qw_argmax_rows_kernel, dim3(rows), dim3(1024), 0, s->stream, logits, n, tokens);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}

@@ -1206,3 +1206,17 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
+
+// LM head for greedy decoding: logits = W . x over the vocabulary rows, then the argmax of each activation row with the
+// reference's key rule (QWGemmAQ.encodeHeadArgmax, Sources/Operators/QWGEMM/QWGemmAQ.swift:306-349; qwg_head_gemv_*_argmax,
+// qwg_gemv_*_f32_v4_am).  Two launches on the stream: the GEMV of qwhip_gemv into `logits` (which the caller keeps, as
+// with the reference's writeLogits), and one workgroup per row folding it.
+extern "C" qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);
+extern "C" qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
+                                          uint32_t flags, float* logits, int32_t* tokens) {
+    QWHIP_REQUIRE(logits);
+    QWHIP_REQUIRE(tokens);
+    qwhip_status st = qwhip_gemv(s, w, x, x_dtype, m, flags, nullptr, logits);
+    if (st != QWHIP_OK) return st;
+    return qwhip_argmax_f32(s, logits, m, w->n, tokens);
+}

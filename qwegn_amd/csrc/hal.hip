@@ -269,6 +269,8 @@ static const qw_kernel_entry g_kernels[] = {
     {"qwg_moe_gateup_q4g_f32_r1", "qwhip_moe_gateup_decode"},
     {"qwg_moe_down_shared_combine_q4g_f32", "qwhip_moe_down_decode"},
     {"qwg_quantize_bf16_to_hq4_g32_m5", "qwhip_quantize_hq4_g32"},
+    {"qwg_head_gemv_q4g_argmax", "qwhip_head_argmax"},
+    {"qwg_gemv_q4g_f32_v4_am", "qwhip_head_argmax"},
     {"qwg_rmsnorm", "qwhip_rmsnorm"},
     {"qwg_rmsnorm_residual", "qwhip_rmsnorm"},
     {"qwg_rmsnorm_residual_wide", "qwhip_rmsnorm"},

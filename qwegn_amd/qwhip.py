@@ -82,6 +82,8 @@ SIGNATURES = {
     "qwhip_moe_gateup_decode": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _U32, _U32, _P]),
     "qwhip_moe_down_decode": (C.c_int32, [_P, _WV, _U32, _P, _P, _P, _U32, _U32, _P, _P, _P, _U32]),
     "qwhip_quantize_hq4_g32": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, _P]),
+    "qwhip_head_argmax": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _P, _P]),
+    "qwhip_argmax_f32": (C.c_int32, [_P, _P, _U32, _U32, _P]),
     "qwhip_rmsnorm": (C.c_int32, [_P, _P, _P, _P, _U32, _U32, C.c_float, _U32, _P]),
     "qwhip_repack_mlx_affine": (C.c_int32, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _P, _P]),
     "qwhip_repack_mlx_affine_switch_gate_up": (C.c_int32, [_P, _P, _P, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _P, _P]),

@@ -85,6 +85,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
         b"qwg_moe_down_shared_combine_q4g_f32": b"qwhip_moe_down_decode", b"qwg_fwht32_f16": b"qwhip_fwht32",
         b"qwg_quantize_bf16_to_hq4_g32_m5": b"qwhip_quantize_hq4_g32",
         b"qwg_rmsnorm": b"qwhip_rmsnorm", b"qwg_rmsnorm_residual": b"qwhip_rmsnorm",
+        b"qwg_head_gemv_q4g_argmax": b"qwhip_head_argmax", b"qwg_gemv_q4g_f32_v4_am": b"qwhip_head_argmax",
         b"qwg_repack_mlx_affine_to_aq_m5": b"qwhip_repack_mlx_affine",
         b"qwg_repack_mlx_affine_switch_gate_up_to_aq_m5": b"qwhip_repack_mlx_affine_switch_gate_up",
     }
@@ -92,7 +93,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
         assert lib.qwhip_kernel_lookup(name, C.byref(launcher)) == qwhip.OK, name
         assert launcher.value == want
         assert hasattr(lib, want.decode())
-    for missing in (b"qwg_gemv_shvq4_g32_v4", b"qwg_gemv_aq3_g32_v4", b"qwg_head_gemv_q4g_argmax", b"nope"):
+    for missing in (b"qwg_gemv_shvq4_g32_v4", b"qwg_gemv_aq3_g32_v4", b"qwg_head_gemv_shvq4_g32_argmax", b"nope"):
         assert lib.qwhip_kernel_lookup(missing, None) == qwhip.E_KERNEL_MISSING
         assert missing in lib.qwhip_last_error()
 

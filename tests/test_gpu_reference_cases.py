@@ -287,3 +287,42 @@ def test_rmsnorm_refuses_the_geometries_the_reference_driver_refuses(dev):
     assert dev.lib.qwhip_rmsnorm(st, z.ptr, z.ptr, None, 1, 1000, 1e-6, 1, z.ptr) == qwhip.E_BAD_GEOMETRY     # hidden % 256
     assert dev.lib.qwhip_rmsnorm(st, z.ptr, None, None, 1, 1024, 1e-6, 1, z.ptr) == qwhip.E_NULL
     assert dev.lib.qwhip_rmsnorm(st, z.ptr, z.ptr, None, 0, 1024, 1e-6, 1, z.ptr) == qwhip.OK                 # no rows: nothing to do
+
+
+def test_argmax_fold_key_rule(dev):
+    """qwhip_argmax_f32 against the oracle's fold: ties to the lower row, NaN never wins, -0 < +0, infinities, rows whose
+    length is not a multiple of four and rows that start unaligned."""
+    rng = np.random.default_rng(8)
+    for rows, n in [(3, 151936), (5, 1001), (2, 7), (16, 4096)]:
+        logits = rng.standard_normal((rows, n)).astype(np.float32)
+        logits[0, [n // 3, n // 2]] = 11.0
+        logits[1, n - 1] = np.nan
+        if rows > 2:
+            logits[2, :] = np.nan
+        lb, tb = dev.put(logits), dev.alloc(max(256, rows * 4))
+        qwhip.check(dev.lib.qwhip_argmax_f32(dev.stream.handle, lb.ptr, rows, n, tb.ptr))
+        dev.stream.sync()
+        assert np.array_equal(tb.download(np.int32, (rows,)), qo.head_argmax(logits)), (rows, n)
+
+
+@pytest.mark.parametrize("fmt,m", [("hq4_g32_m5", 1), ("hq4_g32_m5", 3), ("aq4_g32", 2), ("hq8_g32", 1)])
+def test_head_argmax_picks_the_oracles_token(dev, fmt, m):
+    """qwhip_head_argmax: logits within the judged bar of the fp64 reference, and the token is the fold of the device's own
+    logits (and the oracle's whenever its two best logits are further apart than the error bar)."""
+    from tests import helpers as H
+    n, k = 3000, 1024
+    blocks, w16 = H.make_bank(fmt, n, k, seed=31)
+    x16 = H.make_x(m, k, 131).astype(np.float16)
+    bank, xb = dev.put(blocks), dev.put(x16)
+    logits, toks = dev.alloc(m * n * 4), dev.alloc(256)
+    view = H.view_of(dev, bank, fmt, n, k)
+    qwhip.check(dev.lib.qwhip_head_argmax(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, m, 0, logits.ptr, toks.ptr))
+    dev.stream.sync()
+    got = logits.download(np.float32, (m, n))
+    ref = qo.matmul_ref_f64(H.x_in_basis(x16, fmt), w16)
+    assert qo.normalized_error(got, ref) <= 2e-3
+    tok = toks.download(np.int32, (m,))
+    assert np.array_equal(tok, qo.head_argmax(got))
+    top2 = np.sort(ref, axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 1e-2 * np.abs(top2[:, 1])
+    assert np.array_equal(tok[clear], np.argmax(ref, axis=1)[clear])

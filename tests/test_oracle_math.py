@@ -275,3 +275,21 @@ def test_rmsnorm_closed_forms():
     assert np.array_equal(res_out, (x16.astype(np.float32) + res.astype(np.float32)).astype(np.float16))
     y3, _ = qo.rmsnorm_rot_f16(res_out, gam, eps)
     assert np.array_equal(y2.view(np.uint16), y3.view(np.uint16))
+
+
+def test_head_argmax_key_rule():
+    """The sortable key is monotone on every finite float and the infinities, NaN maps to 0; the fold is numpy's first
+    maximum whenever no NaN is the only candidate."""
+    rng = np.random.default_rng(2)
+    v = np.concatenate([rng.standard_normal(4000).astype(np.float32) * 1e3, np.array([-0.0, 0.0, np.inf, -np.inf, 1e-45, -1e-45], np.float32)])
+    order = np.argsort(v, kind="stable")
+    k = qo.sortable_f32_u32(v)[order].astype(np.int64)
+    assert np.all(np.diff(k) >= 0) and qo.sortable_f32_u32(np.array([-0.0], np.float32))[0] < qo.sortable_f32_u32(np.array([0.0], np.float32))[0]
+    assert qo.sortable_f32_u32(np.array([np.nan], np.float32))[0] == 0
+    logits = rng.standard_normal((5, 1000)).astype(np.float32)
+    assert np.array_equal(qo.head_argmax(logits), np.argmax(logits, axis=1))
+    logits[0, [7, 300]] = 9.0                  # tie: the lower row
+    logits[1, 5] = np.nan                      # NaN never wins
+    logits[2, :] = np.nan                      # nothing but NaN: row 0
+    logits[3, 999] = np.inf
+    assert list(qo.head_argmax(logits)[:4]) == [7, int(np.nanargmax(logits[1])), 0, 999]
