@@ -892,6 +892,9 @@ qwhip_status check_common(qwhip_stream_t s, const qwhip_weight_view* w, const vo
     if (w->kind == QWHIP_KIND_HQ4_G32_M5) *fmt = QW_FMT_M5;
     else if (w->bits == 4) *fmt = QW_FMT_B4;
     else if (w->bits == 8) *fmt = QW_FMT_B8;
+    else if (w->bits == 2) *fmt = QW_FMT_B2;
+    else if (w->bits == 3) *fmt = QW_FMT_B3;
+    else if (w->bits == 6) *fmt = QW_FMT_B6;
     else return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no gemv kernel for %u-bit group %u", w->bits, w->group);
     return QWHIP_OK;
 }
@@ -957,6 +960,21 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     a.rotate = rotate ? 1u : 0u;
     a.rot_out = 0;
 
+    // 2-, 3- and 6-bit streams: the column-stationary dot2 kernel is their one decode kernel (eight rows per launch)
+    if (fmt >= QW_FMT_B2) {
+        if (rotate && m > 1)
+            return qwhip_fail(QWHIP_E_BASIS, "a rotated %u-bit container takes one un-rotated row, or rows already in its basis", w->bits);
+        for (uint32_t m0 = 0; m0 < m; m0 += 8u) {
+            hipError_t e = hipSuccess;
+            const uint32_t mm = min(8u, m - m0);
+            if (!qw_colx_gemv(s->stream, w, fmt, a.gshift, a.bb, a.row_bytes, (const uint8_t*)x + (size_t)m0 * w->k * 2u, x_dtype, mm,
+                              rotate, y16 ? (void*)((h1_t*)y16 + (size_t)m0 * w->n) : nullptr, y32 ? y32 + (size_t)m0 * w->n : nullptr,
+                              rt, &e))
+                return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "no %u-bit decode kernel for n=%u k=%u m=%u", w->bits, w->n, w->k, m);
+            QWHIP_TRY_HIP(e);
+        }
+        return QWHIP_OK;
+    }
     const size_t lds_dot2 = (size_t)(w->k / 32) * 80u;
     const bool dot2_ok = fmt == QW_FMT_M5 && m == 1 && lds_dot2 <= 60u * 1024u;
     if (variant == 1 && !dot2_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "dot2 kernel needs HQ4_G32_M5, m = 1, k <= 24576");
@@ -1066,6 +1084,7 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     int fmt = 0;
     qwhip_status st = check_common(s, w, x, x_dtype, m, &fmt);
     if (st != QWHIP_OK) return st;
+    if (fmt >= QW_FMT_B2) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no gate|up kernel for %u-bit group %u", w->bits, w->group);
     QWHIP_REQUIRE(act16);
     if (w->n % 2 != 0) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "gate|up bank needs an even row count, got %u", w->n);
     const uint32_t inter = w->n / 2;
@@ -1109,6 +1128,7 @@ extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_we
     int fmt = 0;
     qwhip_status st = check_common(s, w_gate_up, x, x_dtype, 1, &fmt);
     if (st != QWHIP_OK) return st;
+    if (fmt >= QW_FMT_B2) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no routed kernel for %u-bit group %u", w_gate_up->bits, w_gate_up->group);
     QWHIP_REQUIRE(idx);
     QWHIP_REQUIRE(act16);
     if (t == 0 || top_k == 0) return QWHIP_OK;
@@ -1158,6 +1178,7 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
     int fmt = 0;
     qwhip_status st = check_common(s, w_down, act16, QWHIP_F16, 1, &fmt);
     if (st != QWHIP_OK) return st;
+    if (fmt >= QW_FMT_B2) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no routed kernel for %u-bit group %u", w_down->bits, w_down->group);
     QWHIP_REQUIRE(idx);
     QWHIP_REQUIRE(wts);
     QWHIP_REQUIRE(out);

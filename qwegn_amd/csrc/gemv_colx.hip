@@ -17,7 +17,8 @@
 // (qwg_aq_slice_dot, Sources/QWMetal/include/qw_dequant_multi.metalh:205-208).
 // Element order inside a word fixes which activations pair up: HQ4_G32_M5 keeps element 8w + j at bit
 // 4 (j >> 1) + 16 (j & 1) (unpack_hq4_word8, qw_dequant.metalh:42-62), the bit-stream containers element i at bit
-// i * bits, so a masked 4-bit word holds elements (k, k + 4) and a masked 8-bit word elements (k, k + 2).
+// i * bits, so a masked 4-bit word holds elements (k, k + 4) and a masked 8-bit word elements (k, k + 2).  The 2-, 3- and
+// 6-bit streams have no such in-place pairs: their codes are cut out one by one and paired as neighbours.
 #include "qwhip_common.h"
 
 namespace {
@@ -30,13 +31,21 @@ struct qcx_params {
     uint32_t N, K, M, nsl, cpr, sets, gshift, bb, row_bytes;
 };
 
+// payload dwords of one 32-column slice: bits * 32 / 32 (HQ4_G32_M5 and 4-bit streams: 4)
+template <int FMT>
+struct qcx_fmt {
+    static constexpr int BITS = FMT == QW_FMT_B8 ? 8 : (FMT == QW_FMT_B2 ? 2 : (FMT == QW_FMT_B3 ? 3 : (FMT == QW_FMT_B6 ? 6 : 4)));
+    static constexpr int PW = BITS;
+    static constexpr bool GENERIC = FMT == QW_FMT_B2 || FMT == QW_FMT_B3 || FMT == QW_FMT_B6;
+};
+
 struct __attribute__((packed, aligned(4))) qcx_words4 { uint32_t q[4]; };
 struct __attribute__((packed, aligned(4))) qcx_words8 { uint32_t q[8]; };
 
 template <int FMT>
 struct qcx_slice {
     uint32_t hdr;
-    uint32_t q[FMT == QW_FMT_B8 ? 8 : 4];
+    uint32_t q[qcx_fmt<FMT>::PW];
 };
 
 // The 16 operand pairs of one activation row for this lane's slice, in the order the masked code words come out.
@@ -49,7 +58,7 @@ __device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             h2_t pr;
-            if constexpr (FMT == QW_FMT_M5) pr = h2_t{v[j][2 * k], v[j][2 * k + 1]};
+            if constexpr (FMT == QW_FMT_M5 || qcx_fmt<FMT>::GENERIC) pr = h2_t{v[j][2 * k], v[j][2 * k + 1]};
             else if constexpr (FMT == QW_FMT_B4) pr = h2_t{v[j][k], v[j][k + 4]};
             else pr = h2_t{v[j][4 * (k >> 1) + (k & 1)], v[j][4 * (k >> 1) + (k & 1) + 2]};
             if (k & 1) s1 = __builtin_amdgcn_fdot2(pr, one, s1, false);
@@ -89,7 +98,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
         pay_off = hdr_off + 4u;
     } else {
         hdr_off = (g >> p.gshift) * p.bb;
-        pay_off = hdr_off + 4u + (g & ((1u << p.gshift) - 1u)) * (FMT == QW_FMT_B8 ? 32u : 16u);
+        pay_off = hdr_off + 4u + (g & ((1u << p.gshift) - 1u)) * (4u * qcx_fmt<FMT>::PW);
     }
     uint32_t off = ((mine ? set : 0u) * G + blockIdx.x) * p.row_bytes;
     const uint32_t off_max = off + (mine ? mine - 1u : 0u) * step;   // loads past the set's last row re-read it
@@ -119,7 +128,10 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
     auto issue = [&](int slot) {
         const uint8_t* rp = p.bank + off;
         buf[slot].hdr = *(const uint32_t*)(rp + hdr_off);
-        if constexpr (FMT == QW_FMT_B8) {
+        if constexpr (qcx_fmt<FMT>::GENERIC) {
+#pragma unroll
+            for (int j = 0; j < qcx_fmt<FMT>::PW; ++j) buf[slot].q[j] = *(const uint32_t*)(rp + pay_off + 4 * j);
+        } else if constexpr (FMT == QW_FMT_B8) {
             const qcx_words8 w = *(const qcx_words8*)(rp + pay_off);
 #pragma unroll
             for (int j = 0; j < 8; ++j) buf[slot].q[j] = w.q[j];
@@ -174,7 +186,21 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
             const qcx_slice<FMT> b = buf[j];
             issue(j);
             uint32_t ow[16];   // masked code words, operand order
-            if constexpr (FMT == QW_FMT_B8) {
+            if constexpr (qcx_fmt<FMT>::GENERIC) {
+                // 2-, 3- and 6-bit streams: element e at bit e * bits.  Each code is cut out of the stream (compile-time
+                // positions, at most two words) and two neighbours share an operand word as integers, i.e. as the f16
+                // subnormals code * 2^-24.
+                constexpr int BITS = qcx_fmt<FMT>::BITS;
+                constexpr uint32_t MASK = (1u << BITS) - 1u;
+                auto code = [&](int e) {
+                    const int off = e * BITS, wd = off >> 5, sh = off & 31;
+                    uint32_t c = b.q[wd] >> sh;
+                    if (sh + BITS > 32) c |= b.q[wd + 1] << (32 - sh);
+                    return c & MASK;
+                };
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ow[i] = code(2 * i) | (code(2 * i + 1) << 16);
+            } else if constexpr (FMT == QW_FMT_B8) {
 #pragma unroll
                 for (int w = 0; w < 8; ++w) {
                     ow[2 * w] = b.q[w] & 0x00FF00FFu;
@@ -203,7 +229,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
                     a3 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 3]), xo[m][i + 3], a3, false);
                 }
                 float q;
-                if constexpr (FMT == QW_FMT_B8) {
+                if constexpr (FMT == QW_FMT_B8 || qcx_fmt<FMT>::GENERIC) {
                     q = ((a0 + a1) + (a2 + a3)) * 16777216.0f;
                 } else {
                     q = __builtin_fmaf(a0 + a2, 16777216.0f, FMT == QW_FMT_M5 ? 1024.0f * S[m] : 0.0f);   // codes at bits 0..3
@@ -247,7 +273,7 @@ void qcx_launch_m(hipStream_t st, const qcx_params& p, uint32_t mr, bool rotate,
 
 // Tries the column-stationary small-M kernel for a validated call; false when the shape is outside its envelope:
 // up to eight activation rows already in the container's basis, or one row to rotate (`rotate`).
-// fmt: QW_FMT_M5 / QW_FMT_B4 / QW_FMT_B8.  `tune`: 0 = automatic; bits 0..1 scale the grid (1 -> half, 2 -> double).
+// fmt: QW_FMT_M5 / QW_FMT_B4 / QW_FMT_B8, and the 2-, 3- and 6-bit streams QW_FMT_B2 / B3 / B6.  `tune`: 0 = automatic; bits 0..1 scale the grid (1 -> half, 2 -> double).
 bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
                   const void* x, uint32_t x_dtype, uint32_t m, bool rotate, void* y16, float* y32, uint32_t tune,
                   hipError_t* err) {
@@ -289,11 +315,17 @@ bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t 
     if (x_dtype == QWHIP_F16) {
         if (fmt == QW_FMT_M5) qcx_launch_m<QW_FMT_M5, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
         else if (fmt == QW_FMT_B4) qcx_launch_m<QW_FMT_B4, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
-        else qcx_launch_m<QW_FMT_B8, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B8) qcx_launch_m<QW_FMT_B8, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B2) qcx_launch_m<QW_FMT_B2, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B3) qcx_launch_m<QW_FMT_B3, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
+        else qcx_launch_m<QW_FMT_B6, QWHIP_F16>(st, p, mr, rotate, wgs, threads, lds);
     } else {
         if (fmt == QW_FMT_M5) qcx_launch_m<QW_FMT_M5, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
         else if (fmt == QW_FMT_B4) qcx_launch_m<QW_FMT_B4, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
-        else qcx_launch_m<QW_FMT_B8, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B8) qcx_launch_m<QW_FMT_B8, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B2) qcx_launch_m<QW_FMT_B2, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
+        else if (fmt == QW_FMT_B3) qcx_launch_m<QW_FMT_B3, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
+        else qcx_launch_m<QW_FMT_B6, QWHIP_BF16>(st, p, mr, rotate, wgs, threads, lds);
     }
     *err = hipGetLastError();
     return true;

@@ -297,7 +297,8 @@ static bool qw_parse_aq_name(const char* name, const char** launcher) {
         lau = "qwhip_moe_down_decode";
     }
     if (!lau) return false;
-    if (!(bits == 4 || bits == 8)) return false;
+    const bool decode_gemv = !strcmp(lau, "qwhip_gemv");   // the 2-, 3- and 6-bit streams have the decode GEMV only
+    if (!(bits == 4 || bits == 8 || (decode_gemv && (bits == 2 || bits == 3 || bits == 6)))) return false;
     if (!(group == 32 || group == 64 || group == 128 || group == 256)) return false;
     if (launcher) *launcher = lau;
     return true;

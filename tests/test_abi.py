@@ -77,6 +77,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
     table = {
         b"qwg_gemv_q4g_dx_h16_t4": b"qwhip_gemv", b"qwg_gemv_q4g_v4": b"qwhip_gemv", b"qwg_skinny_m3": b"qwhip_gemv",
         b"qwg_gemv_aq8_g32_v4": b"qwhip_gemv", b"qwg_gemv_aq4_g64_dx_h16_t4": b"qwhip_gemv",
+        b"qwg_gemv_aq3_g32_v4": b"qwhip_gemv", b"qwg_gemv_aq6_g128_dx_h16_t4": b"qwhip_gemv", b"qwg_gemv_aq2_g64_v4": b"qwhip_gemv",
         b"qwg_gemv_q4g_silu_pair_dx_h16": b"qwhip_gemv_silu_pair", b"qwg_gemv_aq4_g32_silu_pair_dx_h16": b"qwhip_gemv_silu_pair",
         b"qwg_gemm_q4g_h16": b"qwhip_gemm", b"qwg_gemm_aq8_g32_h16": b"qwhip_gemm", b"qwg_gemm_aq4_g64_nax_f32": b"qwhip_gemm",
         b"qwg_moe_route": b"qwhip_moe_route", b"qwg_moe_group_pairs_f32": b"qwhip_moe_group_pairs",
@@ -93,7 +94,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
         assert lib.qwhip_kernel_lookup(name, C.byref(launcher)) == qwhip.OK, name
         assert launcher.value == want
         assert hasattr(lib, want.decode())
-    for missing in (b"qwg_gemv_shvq4_g32_v4", b"qwg_gemv_aq3_g32_v4", b"qwg_head_gemv_shvq4_g32_argmax", b"nope"):
+    for missing in (b"qwg_gemv_shvq4_g32_v4", b"qwg_gemm_aq3_g32_h16", b"qwg_gemv_aq5_g32_v4", b"qwg_head_gemv_shvq4_g32_argmax", b"nope"):
         assert lib.qwhip_kernel_lookup(missing, None) == qwhip.E_KERNEL_MISSING
         assert missing in lib.qwhip_last_error()
 

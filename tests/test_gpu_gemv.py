@@ -219,6 +219,34 @@ def test_gemv_transposing_mfma_kernel_k_ranges_and_dtypes(dev, fmt, n, k, m, xdt
     assert qo.normalized_error(g16, ref) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["aq2_g64", "hq3_g32", "hq6_g32", "aq6_g128"])
+@pytest.mark.parametrize("m", [1, 3, 8, 12])
+def test_gemv_narrow_and_six_bit_streams(dev, fmt, m):
+    """2-, 3- and 6-bit containers (QWAQBlock.supported, QWAQBlock.swift:17-23) on the column-stationary dot2 kernel:
+    rows already in the basis, eight per launch; tight against the factorised form, inside the judged bar against the
+    f16-weight reference."""
+    g16, g32, ref = _run_gemv(dev, fmt, 272, 1536, m, prerot=True, seed=5)
+    assert qo.normalized_error(g32, _affine_ref(fmt, 272, 1536, m, 5)) <= 2e-5
+    assert qo.normalized_error(g32, ref) <= TOL
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["hq3_g32", "hq6_g32"])
+@pytest.mark.parametrize("xdtype", ["f16", "bf16"])
+def test_gemv_narrow_streams_fused_rotation_and_basis_errors(dev, fmt, xdtype):
+    """One un-rotated row is rotated in the prologue; several un-rotated rows are refused (QWHIP_E_BASIS) before any
+    launch, as are the doors that have no kernel for these widths."""
+    g16, g32, ref = _run_gemv(dev, fmt, 100, 2048, 1, prerot=False, xdtype=xdtype, seed=7)
+    assert qo.normalized_error(g32, _affine_ref(fmt, 100, 2048, 1, 7, xdtype)) <= 2e-5
+    blocks, _ = H.make_bank(fmt, 64, 256, seed=1)
+    bank, xb, yb = dev.put(blocks), dev.put(np.zeros((4, 256), np.float16)), dev.alloc(4 * 64 * 4)
+    view = H.view_of(dev, bank, fmt, 64, 256)
+    st = dev.stream.handle
+    assert dev.lib.qwhip_gemv(st, C.byref(view), xb.ptr, qwhip.F16, 4, 0, None, yb.ptr) == qwhip.E_BASIS
+    assert dev.lib.qwhip_gemv_silu_pair(st, C.byref(view), xb.ptr, qwhip.F16, 1, 0, 1, yb.ptr) == qwhip.E_BAD_WEIGHTS
+    assert dev.lib.qwhip_gemm(st, C.byref(view), xb.ptr, qwhip.F16, 4, 0, yb.ptr, qwhip.F32, 0, qwhip.X_PREROTATED, None, 0) != qwhip.OK
+
+
 @pytest.mark.parametrize("m", [1, 4])
 def test_gemv_column_stationary_long_rows(dev, m):
     """k = 17408: 17 half-waves per row, one row set per workgroup."""
