@@ -10,7 +10,7 @@ kernel measured with HIP events on the launch stream, and the CPU baseline (the 
 oracle form - dequantize the bank to fp32, then one fp32 product - restated in numpy and timed
 on this box's host cores over a bounded sample).
 
-Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up|norm_prefill|norm_decode (see WORKLOADS).
+Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up|head|f32_decode|f32_verify4|repack|norm_prefill|norm_decode (see WORKLOADS).
 """
 from __future__ import annotations
 
@@ -205,6 +205,151 @@ def run_silu_pair(args, fmt, inter, k, m, label):
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": algo_bytes,
                      "kernel_us": round(us_per, 3)},
         "normalized_error": err,
+    }
+
+
+def run_head(args, fmt, n, k, label):
+    """LM head for greedy decoding: GEMV over the vocabulary rows into f32 logits + per-row argmax fold; one step = both
+    launches.  Algorithmic bytes: the bank, x, the logits written and read back once."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+    from tests import helpers as H
+
+    dev = qwhip.Device(0)
+    blocks, w16 = H.make_bank(fmt, n, k, seed=0)
+    x16 = H.make_x(1, k, 100).astype(np.float16)
+    bank, xb = dev.put(blocks), dev.put(x16)
+    logits, tok = dev.alloc(n * 4), dev.alloc(256)
+    view = H.view_of(dev, bank, fmt, n, k)
+    lib, st = dev.lib, dev.stream.handle
+
+    def launch(i):
+        qwhip.check(lib.qwhip_head_argmax(st, C.byref(view), xb.ptr, qwhip.F16, 1, 0, logits.ptr, tok.ptr))
+
+    launch(0)
+    dev.stream.sync()
+    got = logits.download(np.float32, (1, n))
+    err = qo.normalized_error(got, qo.matmul_ref_f64(H.x_in_basis(x16, fmt), w16))
+    if not (err <= 2e-3 and int(tok.download(np.int32, (1,))[0]) == int(qo.head_argmax(got)[0])):
+        _fail(f"bench: head argmax failed parity (normalized error {err:.3e})")
+    _spin_up(dev, launch)
+    for i in range(args.warmup):
+        launch(i)
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        launch(i)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    algo_bytes = blocks.nbytes + k * 2 + 2 * n * 4
+    gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": label, "format": fmt, "M": 1, "N": n, "K": k, "cache": "one bank (larger than the Infinity Cache)"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
+        "normalized_error": err,
+    }
+
+
+def run_gemv_f32(args, fmt, n, k, m, label):
+    """f32-activation GEMV (fp32 arithmetic, epilogue 0): one step = one pass over the bank for all m rows."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+    from tests import helpers as H
+
+    dev = qwhip.Device(0)
+    _, bits, group, is_m5, _ = H.FORMATS[fmt]
+    blocks, _ = H.make_bank(fmt, n, k, seed=0)
+    x = H.make_x(m, k, 100)
+    bank, xb, yb = dev.put(blocks), dev.put(x), dev.alloc(m * n * 4)
+    view = H.view_of(dev, bank, fmt, n, k)
+    lib, st = dev.lib, dev.stream.handle
+
+    def launch(i):
+        qwhip.check(lib.qwhip_gemv_f32(st, C.byref(view), xb.ptr, m, 0, 1.0, yb.ptr))
+
+    launch(0)
+    dev.stream.sync()
+    sample = min(n, 512)
+    err = qo.normalized_error(yb.download(np.float32, (m, n))[:, :sample], qo.gemv_f32(blocks[:sample], x, bits, group, is_m5))
+    if not err <= 2e-5:
+        _fail(f"bench: f32 gemv failed parity (normalized error {err:.3e})")
+    _spin_up(dev, launch)
+    for i in range(args.warmup):
+        launch(i)
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        launch(i)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    algo_bytes = blocks.nbytes + m * k * 4 + m * n * 4
+    gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": label, "format": fmt, "M": m, "N": n, "K": k},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
+        "normalized_error": err,
+    }
+
+
+def run_repack(args, rows, cols, bits, group, label):
+    """Load-time MLX affine -> AQ repack: one step = one launch.  Algorithmic bytes: codes and headers read, blocks written."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+
+    dev = qwhip.Device(0)
+    rng = np.random.default_rng(0)
+    groups, payload = cols // group, group * bits // 8
+    w = rng.integers(0, 256, size=(rows, groups * payload), dtype=np.uint8)
+    sc = qo.f32_to_bf16_bits(rng.uniform(1e-3, 0.05, size=rows * groups).astype(np.float32))
+    bi = qo.f32_to_bf16_bits((-rng.uniform(1e-2, 0.3, size=rows * groups)).astype(np.float32))
+    wb, sb, bb_ = dev.put(w), dev.put(sc), dev.put(bi)
+    out, cnt = dev.alloc(rows * groups * (4 + payload)), dev.put(np.zeros(1, np.uint32))
+    lib, st = dev.lib, dev.stream.handle
+
+    def launch(i):
+        qwhip.check(lib.qwhip_repack_mlx_affine(st, wb.ptr, sb.ptr, bb_.ptr, qwhip.BF16, rows, cols, bits, group, out.ptr, cnt.ptr))
+
+    launch(0)
+    dev.stream.sync()
+    sample = min(rows, 64)
+    want, refused = qo.repack_mlx_affine(w[:sample], sc[:sample * groups], bi[:sample * groups], sample, cols, bits, group, False)
+    if not (np.array_equal(out.download(np.uint8, (rows, groups, 4 + payload))[:sample], want) and int(cnt.download(np.uint32, (1,))[0]) == 0):
+        _fail("bench: repacked blocks differ from the oracle's")
+    _spin_up(dev, launch)
+    for i in range(args.warmup):
+        launch(i)
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        launch(i)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    algo_bytes = rows * groups * (payload + 4) * 2
+    gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": label, "rows": rows, "cols": cols, "bits": bits, "group": group},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
     }
 
 
@@ -517,6 +662,10 @@ WORKLOADS = {
     "c5_qkv": ("gemv", "hq8_g32", 7168, 5120, None, False),
     "c5_down": ("gemv", "hq4_g64", 5120, 17408, None, False),
     "mlp_gate_up": ("pair", "hq4_g32_m5", 17408, 5120, 1, False),      # n = intermediate size: the bank has 2n rows
+    "head": ("head", "hq4_g32_m5", 151936, 5120, 1, False),
+    "f32_decode": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 1, False),
+    "f32_verify4": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 4, False),
+    "repack": ("repack", None, 34816, 5120, None, False),              # MLX 4-bit group 64, gate|up sized
     "norm_prefill": ("norm", None, 5120, None, 4096, False),           # n = hidden, m = rows
     "norm_decode": ("norm", None, 5120, None, 1, False),
 }
@@ -529,6 +678,10 @@ LABELS = {
     "c5_qkv": "C5 verify GEMM HQ8_G32 K=5120 N=7168",
     "c5_down": "C5 verify GEMM HQ4_G64 K=17408 N=5120",
     "mlp_gate_up": "dense MLP gate|up GEMV + SwiGLU + FWHT, HQ4_G32 M=1 K=5120 I=17408",
+    "head": "LM head GEMV + argmax, HQ4_G32 M=1 K=5120 N=151936",
+    "f32_decode": "f32-activation GEMV, HQ4_G32 M=1 K=5120 N=17408",
+    "f32_verify4": "f32-activation GEMV, HQ4_G32 M=4 K=5120 N=17408",
+    "repack": "MLX affine -> AQ4_G64 repack, 34816 x 5120",
     "norm_prefill": "RMSNorm + residual + FWHT producer, 4096 rows x 5120",
     "norm_decode": "RMSNorm + residual + FWHT producer, 1 row x 5120",
 }
@@ -572,6 +725,12 @@ def main() -> None:
         m = args.m
     if kind == "moe":
         out = run_moe(args, m, LABELS[args.workload])
+    elif kind == "gemv_f32":
+        out = run_gemv_f32(args, fmt, n, k, m, LABELS[args.workload])
+    elif kind == "head":
+        out = run_head(args, fmt, n, k, LABELS[args.workload])
+    elif kind == "repack":
+        out = run_repack(args, n, k, 4, 64, LABELS[args.workload])
     elif kind == "norm":
         out = run_norm(args, m, n, LABELS[args.workload])
     elif kind == "pair":

@@ -175,11 +175,29 @@ qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void
 qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                                   uint32_t m, uint32_t flags, uint32_t rotate_out, void* act16);
 
+/* fp32-activation GEMV with a scalar epilogue: QWGemm.encodeHQ4F32V4 and, for the row counts the reference hands to its
+ * batched form, encodeHQ4F32BM (Sources/Operators/QWGEMM/QWGemmF32.swift:178-199,311-350; kernels qwg_gemv_*_f32_v4,
+ * qwg_gemm_*_f32_bm, bodies Sources/QWMetal/include/qw_gemm_f32_common.metalh:59-225).
+ * x: f32 [m, k] already in the container's basis (the reference rotates it with qwg_h32_f32 first); y: f32 [m, n];
+ * every container width (2, 3, 4, 6, 8 bits and HQ4_G32_M5).  All arithmetic in fp32: weights are code * scale + bias
+ * without the f16 rounding of qwhip_dequant_f16, as in the reference's f32 dequant (qw_dequant_f32.metalh:1-24).
+ * epi: 0 none, 1 silu(y / scale), 2 sigmoid(y), 3 silu(y / scale) followed by the FWHT-32 over each 32 consecutive outputs
+ * (a last partial group is padded with zeros).  Four activation rows share one pass over the bank. */
+qwhip_status qwhip_gemv_f32(qwhip_stream_t s, const qwhip_weight_view* w, const float* x, uint32_t m, uint32_t epi,
+                            float scale, float* y);
+
+/* out f32 [rows, hidden] = FWHT-32 of every 32-column group of x, scaled by 1/sqrt(32): QWGemm.encodeH32F32
+ * (QWGemmF32.swift:46-54; qwg_h32_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:191-201; butterfly order of
+ * qwg_fwht32_lane_f32, Sources/QWMetal/include/qw_weight_basis.metalh:31-38).  out may be x. */
+qwhip_status qwhip_h32_f32(qwhip_stream_t s, const float* x, float* out, uint32_t rows, uint32_t hidden);
+
 /* LM head for greedy decoding (QWGemmAQ.encodeHeadArgmax, QWGemmAQ.swift:306-349; qwg_head_gemv_q4g_argmax,
  * qwg_gemv_*_f32_v4_am with the fold of qw_gemm_f32_common.metalh:30-58): logits [m, n] f32 = W . x (as qwhip_gemv), then
  * tokens[m] = argmax with the reference's key rule: floats compared through qw_sortable_f32_u32 (NaN never wins against
  * a number), ties to the lower row.  `logits` is required and kept (the reference's writeLogits); the reference's key
- * scratch is not needed.  qwhip_argmax_f32 is the fold alone, over any [rows, n] f32 logits. */
+ * scratch is not needed.  x_dtype QWHIP_F32 takes fp32 activations already in the container's basis (the logits are then
+ * those of qwhip_gemv_f32 with epilogue 0, and `flags` is unused).  qwhip_argmax_f32 is the fold alone, over any [rows, n]
+ * f32 logits. */
 qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                uint32_t flags, float* logits, int32_t* tokens);
 qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);

@@ -495,6 +495,42 @@ def head_argmax(logits: np.ndarray) -> np.ndarray:
     return (~(keys.max(axis=-1) & np.uint64(0xFFFFFFFF)) & np.uint64(0xFFFFFFFF)).astype(np.int32)
 
 
+def v4_epilogue_f64(y: np.ndarray, epi: int, scale: float) -> np.ndarray:
+    """The scalar epilogue of the f32 GEMV/GEMM family in float64: 0 none, 1 and 3 silu(y / scale), 2 sigmoid(y)
+    (qwg_apply_v4_epi_f32, Sources/QWMetal/include/qw_gemm_f32_common.metalh:15-19; the batched body :131-132)."""
+    y = np.asarray(y, dtype=np.float64)
+    if epi in (1, 3):
+        z = y / float(scale)
+        return z / (1.0 + np.exp(-z))
+    if epi == 2:
+        return 1.0 / (1.0 + np.exp(-y))
+    return y
+
+
+def h32_groups_f64(y: np.ndarray) -> np.ndarray:
+    """Normalised 32-point Walsh-Hadamard transform of every 32 consecutive outputs of each row in float64; a last partial
+    group is padded with zeros, as epilogue 3 of the v4 kernel reads rows past N
+    (Sources/QWMetal/include/qw_gemm_f32_common.metalh:171-196; qwg_fwht32_lane_f32, qw_weight_basis.metalh:31-38)."""
+    y = np.atleast_2d(np.asarray(y, dtype=np.float64))
+    rows, n = y.shape
+    padded = np.zeros((rows, (n + 31) // 32 * 32))
+    padded[:, :n] = y
+    i = np.arange(32)
+    signs = np.array([[1.0 - 2.0 * (bin(a & b).count("1") & 1) for b in i] for a in i])   # Sylvester order
+    out = padded.reshape(rows, -1, 32) @ signs.T / np.sqrt(32.0)
+    return out.reshape(rows, -1)[:, :n]
+
+
+def gemv_f32(blocks: np.ndarray, x_f32: np.ndarray, bits: int, group: int, is_m5: bool, epi: int = 0, scale: float = 1.0) -> np.ndarray:
+    """f32-activation GEMV with epilogue (QWGemm.encodeHQ4F32V4 / encodeHQ4F32BM, Sources/Operators/QWGEMM/QWGemmF32.swift:
+    178-199,311-350) in float64: y = epilogue(x . W^T) over the un-rounded affine weights code * scale + bias
+    (qwg_unpack_hq4_word8_f32, Sources/QWMetal/include/qw_dequant_f32.metalh:10-24), epilogue 3 adding the FWHT-32 over
+    consecutive outputs.  x is already in the container's basis."""
+    w = weights_affine_f64(blocks, bits, group, is_m5)
+    y = v4_epilogue_f64(np.atleast_2d(np.asarray(x_f32, dtype=np.float64)) @ w.T, epi, scale)
+    return h32_groups_f64(y) if epi == 3 else y
+
+
 def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     """silu(g)*u = g/(1+exp(-g))*u in fp32 (Sources/QWMetal/include/qw_weight_basis.metalh:50-63,
     plain SwiGLU branch; Scripts/oracle/gen_mlp_fixtures.py:79)."""

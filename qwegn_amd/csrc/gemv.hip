@@ -1228,6 +1228,58 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
     return QWHIP_OK;
 }
 
+// gemv_f32.hip
+uint32_t qw_f32_gemv_rows(const qwhip_weight_view* w, uint64_t row_bytes);
+void qw_f32_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                 const float* x, uint32_t m, uint32_t epi, float scale, float* y);
+void qw_h32_f32_launch(hipStream_t st, const float* x, float* out, uint32_t rows, uint32_t hidden);
+
+// fp32 activations in the container's basis -> fp32 outputs with the scalar epilogues of the reference's f32 family
+// (QWGemm.encodeHQ4F32V4 / encodeHQ4F32BM, Sources/Operators/QWGEMM/QWGemmF32.swift:178-199,311-350): the rows go through
+// the column-stationary fp32 kernel four (long rows: two, one) at a time, as the reference's v4 door walks them.
+extern "C" qwhip_status qwhip_gemv_f32(qwhip_stream_t s, const qwhip_weight_view* w, const float* x, uint32_t m, uint32_t epi,
+                                       float scale, float* y) {
+    QWHIP_REQUIRE(s);
+    qwhip_status st = qwhip_weight_view_validate(w);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(x);
+    QWHIP_REQUIRE(y);
+    int fmt = 0;
+    st = check_common(s, w, x, QWHIP_F16, 1, &fmt);   // format lookup, alignment and row-count limits
+    if (st != QWHIP_OK) return st;
+    if (m == 0 || m > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "the f32 gemv takes 1..65535 activation rows, got %u", m);
+    if (epi > 3u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "epilogue %u is not one of 0 none, 1 silu(y/scale), 2 sigmoid, 3 silu(y/scale) + H32", epi);
+    if ((epi == 1u || epi == 3u) && !(scale != 0.0f && scale == scale))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "epilogue %u divides by its scale, which must be a non-zero number", epi);
+    const uint64_t row_bytes = qwhip_view_row_bytes(w);
+    const uint32_t per = qw_f32_gemv_rows(w, row_bytes);
+    if (per == 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "no f32 gemv kernel for n=%u k=%u (rows up to 32768 columns, banks under 1 GiB)", w->n, w->k);
+    const uint32_t gshift = log2_u32(w->group / 32), bb = qwhip_view_block_bytes(w);
+    for (uint32_t m0 = 0; m0 < m; m0 += per) {
+        const uint32_t mm = min(per, m - m0);
+        qw_f32_gemv(s->stream, w, fmt, gshift, bb, row_bytes, x + (size_t)m0 * w->k, mm, epi, scale, y + (size_t)m0 * w->n);
+        QWHIP_TRY_HIP(hipGetLastError());
+    }
+    if (epi == 3u) {
+        qw_h32_f32_launch(s->stream, y, y, m, w->n);
+        QWHIP_TRY_HIP(hipGetLastError());
+    }
+    return QWHIP_OK;
+}
+
+// out f32 [rows, hidden] = FWHT-32 of x in the normalised Walsh-Hadamard domain (QWGemm.encodeH32F32,
+// Sources/Operators/QWGEMM/QWGemmF32.swift:46-54; qwg_h32_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:191-201); in place allowed.
+extern "C" qwhip_status qwhip_h32_f32(qwhip_stream_t s, const float* x, float* out, uint32_t rows, uint32_t hidden) {
+    QWHIP_REQUIRE(s);
+    QWHIP_REQUIRE(x);
+    QWHIP_REQUIRE(out);
+    if (rows == 0 || rows > 65535u || hidden == 0 || hidden % 32u != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "the rotation needs 1..65535 rows of a multiple of 32 columns (rows=%u hidden=%u)", rows, hidden);
+    qw_h32_f32_launch(s->stream, x, out, rows, hidden);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
 // LM head for greedy decoding: logits = W . x over the vocabulary rows, then the argmax of each activation row with the
 // reference's key rule (QWGemmAQ.encodeHeadArgmax, Sources/Operators/QWGEMM/QWGemmAQ.swift:306-349; qwg_head_gemv_*_argmax,
 // qwg_gemv_*_f32_v4_am).  Two launches on the stream: the GEMV of qwhip_gemv into `logits` (which the caller keeps, as
@@ -1237,7 +1289,8 @@ extern "C" qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_v
                                           uint32_t flags, float* logits, int32_t* tokens) {
     QWHIP_REQUIRE(logits);
     QWHIP_REQUIRE(tokens);
-    qwhip_status st = qwhip_gemv(s, w, x, x_dtype, m, flags, nullptr, logits);
+    qwhip_status st = x_dtype == QWHIP_F32 ? qwhip_gemv_f32(s, w, (const float*)x, m, 0u, 1.0f, logits)
+                                           : qwhip_gemv(s, w, x, x_dtype, m, flags, nullptr, logits);
     if (st != QWHIP_OK) return st;
     return qwhip_argmax_f32(s, logits, m, w->n, tokens);
 }

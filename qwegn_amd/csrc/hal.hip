@@ -271,6 +271,11 @@ static const qw_kernel_entry g_kernels[] = {
     {"qwg_quantize_bf16_to_hq4_g32_m5", "qwhip_quantize_hq4_g32"},
     {"qwg_head_gemv_q4g_argmax", "qwhip_head_argmax"},
     {"qwg_gemv_q4g_f32_v4_am", "qwhip_head_argmax"},
+    {"qwg_gemv_q4g_f32_v4_am2", "qwhip_head_argmax"},
+    {"qwg_gemv_q4g_f32_v4", "qwhip_gemv_f32"},
+    {"qwg_gemm_q4g_f32_bm", "qwhip_gemv_f32"},
+    {"qwg_gemm_q4g_f32_bm32", "qwhip_gemv_f32"},
+    {"qwg_h32_f32", "qwhip_h32_f32"},
     {"qwg_rmsnorm", "qwhip_rmsnorm"},
     {"qwg_rmsnorm_residual", "qwhip_rmsnorm"},
     {"qwg_rmsnorm_residual_wide", "qwhip_rmsnorm"},
@@ -285,9 +290,12 @@ static bool qw_parse_aq_name(const char* name, const char** launcher) {
     const char* lau = nullptr;
     if (sscanf(name, "qwg_gemv_aq%u_g%u_%63s", &bits, &group, suffix) == 3) {
         if (!strcmp(suffix, "v4") || !strcmp(suffix, "dx_h16_t4")) lau = "qwhip_gemv";
+        else if (!strcmp(suffix, "f32_v4")) lau = "qwhip_gemv_f32";
+        else if (!strcmp(suffix, "f32_v4_am") || !strcmp(suffix, "f32_v4_am2")) lau = "qwhip_head_argmax";
         else if (!strcmp(suffix, "silu_pair_dx_h16")) lau = "qwhip_gemv_silu_pair";
     } else if (sscanf(name, "qwg_gemm_aq%u_g%u_%63s", &bits, &group, suffix) == 3) {
         if (!strcmp(suffix, "h16") || !strcmp(suffix, "nax_f32")) lau = "qwhip_gemm";
+        else if (!strcmp(suffix, "f32_bm") || !strcmp(suffix, "f32_bm32")) lau = "qwhip_gemv_f32";
     } else if (sscanf(name, "qwg_moe_nax_gemm_aq%u_g%u", &bits, &group) == 2 ||
                sscanf(name, "qwg_moe_nax_split_f32_aq%u_g%u", &bits, &group) == 2) {
         lau = "qwhip_moe_grouped_gemm";
@@ -297,7 +305,8 @@ static bool qw_parse_aq_name(const char* name, const char** launcher) {
         lau = "qwhip_moe_down_decode";
     }
     if (!lau) return false;
-    const bool decode_gemv = !strcmp(lau, "qwhip_gemv");   // the 2-, 3- and 6-bit streams have the decode GEMV only
+    // the 2-, 3- and 6-bit streams have the decode GEMVs only (f16/bf16 and f32 activations, and the head built on them)
+    const bool decode_gemv = !strcmp(lau, "qwhip_gemv") || !strcmp(lau, "qwhip_gemv_f32") || !strcmp(lau, "qwhip_head_argmax");
     if (!(bits == 4 || bits == 8 || (decode_gemv && (bits == 2 || bits == 3 || bits == 6)))) return false;
     if (!(group == 32 || group == 64 || group == 128 || group == 256)) return false;
     if (launcher) *launcher = lau;

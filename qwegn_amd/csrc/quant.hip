@@ -65,7 +65,7 @@ extern "C" qwhip_status qwhip_quantize_hq4_g32(qwhip_stream_t s, const void* src
 // A block is [f16 scale][f16 bias][payload]: the payload bytes are the checkpoint's, the header is the checkpoint's
 // bf16 / f16 scale and bias as f16.  A header that f16 does not hold (overflow, or a value lost in the normal range;
 // below 2^-14 the nearest subnormal is accepted) is poisoned with the f16 NaN 0x7e00 and counted in `refused`.
-// One thread per output dword (header word or payload word), so both streams are read and written in whole lines.
+// Threads walk the output dwords (header word or payload word) in order, so both streams are read and written in whole lines.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ float qw_read_scale(const uint16_t* p, uint32_t is_f16, uint64_t i) {
     const uint16_t b = p[i];
@@ -80,46 +80,86 @@ __device__ __forceinline__ bool qw_f16_header_holds(float raw, h1_t stored) {
 }
 
 // SWITCH: source rows come from two [experts, inter, cols] tensors interleaved per expert as [gate rows | up rows].
-template <bool SWITCH>
+// IDX is the type the dword index is divided in: u32 whenever the plane has fewer than 2^32 dwords.  A thread owns four
+// consecutive output dwords (one 16-byte store when VEC): one division finds the first dword's block, the others step.
+template <bool SWITCH, typename IDX, bool VEC>
 __global__ __launch_bounds__(256) void qw_repack_mlx_kernel(const uint32_t* __restrict__ w0, const uint16_t* __restrict__ s0,
                                                             const uint16_t* __restrict__ b0, const uint32_t* __restrict__ w1,
                                                             const uint16_t* __restrict__ s1, const uint16_t* __restrict__ b1,
-                                                            uint32_t* __restrict__ dst, uint64_t blocks, uint32_t groups,
+                                                            uint32_t* __restrict__ dst, uint64_t total, uint32_t groups,
                                                             uint32_t pay_words, uint32_t inter, uint32_t is_f16,
                                                             uint32_t* __restrict__ refused) {
     const uint32_t W = pay_words + 1u;
-    const uint64_t d = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-    if (d >= blocks * W) return;
-    const uint64_t b = d / W;
-    const uint32_t j = (uint32_t)(d - b * W);
-    uint64_t src_group = b;
-    const uint32_t* w = w0;
-    const uint16_t* sc = s0;
-    const uint16_t* bi = b0;
-    if constexpr (SWITCH) {
-        const uint64_t out_row = b / groups;
-        const uint32_t g = (uint32_t)(b - out_row * groups);
-        const uint64_t e = out_row / (2u * inter);
-        const uint32_t local = (uint32_t)(out_row - e * (2u * inter));
-        const bool up = local >= inter;
-        src_group = (e * inter + (up ? local - inter : local)) * groups + g;
-        if (up) {
-            w = w1;
-            sc = s1;
-            bi = b1;
+    const IDX d0 = ((IDX)blockIdx.x * 256u + threadIdx.x) * 4u;
+    if ((uint64_t)d0 >= total) return;
+    IDX b = d0 / (IDX)W;
+    uint32_t j = (uint32_t)(d0 - b * (IDX)W);
+    uint32_t out[4];
+    uint32_t bad = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        out[t] = 0u;
+        if ((uint64_t)d0 + (uint32_t)t < total) {
+            IDX src_group = b;
+            const uint32_t* w = w0;
+            const uint16_t* sc = s0;
+            const uint16_t* bi = b0;
+            if constexpr (SWITCH) {
+                const IDX out_row = b / (IDX)groups;
+                const uint32_t g = (uint32_t)(b - out_row * (IDX)groups);
+                const IDX e = out_row / (IDX)(2u * inter);
+                const uint32_t local = (uint32_t)(out_row - e * (IDX)(2u * inter));
+                const bool up = local >= inter;
+                src_group = (e * (IDX)inter + (up ? local - inter : local)) * (IDX)groups + g;
+                if (up) {
+                    w = w1;
+                    sc = s1;
+                    bi = b1;
+                }
+            }
+            if (j == 0u) {
+                const float rs = qw_read_scale(sc, is_f16, src_group), rb = qw_read_scale(bi, is_f16, src_group);
+                const h1_t hs = (h1_t)rs, hb = (h1_t)rb;
+                const bool exact = qw_f16_header_holds(rs, hs) && qw_f16_header_holds(rb, hb);
+                bad += exact ? 0u : 1u;
+                const uint32_t lo = exact ? (uint32_t)__builtin_bit_cast(uint16_t, hs) : 0x7E00u;
+                const uint32_t hi = exact ? (uint32_t)__builtin_bit_cast(uint16_t, hb) : 0x7E00u;
+                out[t] = lo | (hi << 16);
+            } else {
+                out[t] = w[(uint64_t)src_group * pay_words + (j - 1u)];
+            }
+        }
+        if (++j == W) {
+            j = 0u;
+            ++b;
         }
     }
-    if (j == 0u) {
-        const float rs = qw_read_scale(sc, is_f16, src_group), rb = qw_read_scale(bi, is_f16, src_group);
-        const h1_t hs = (h1_t)rs, hb = (h1_t)rb;
-        const bool exact = qw_f16_header_holds(rs, hs) && qw_f16_header_holds(rb, hb);
-        if (!exact) atomicAdd(refused, 1u);
-        const uint32_t lo = exact ? (uint32_t)__builtin_bit_cast(uint16_t, hs) : 0x7E00u;
-        const uint32_t hi = exact ? (uint32_t)__builtin_bit_cast(uint16_t, hb) : 0x7E00u;
-        dst[d] = lo | (hi << 16);
+    if (bad) atomicAdd(refused, bad);
+    if (VEC && (uint64_t)d0 + 4u <= total) {
+        *(u4_t*)(dst + d0) = u4_t{out[0], out[1], out[2], out[3]};
     } else {
-        dst[d] = w[src_group * pay_words + (j - 1u)];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if ((uint64_t)d0 + (uint32_t)t < total) dst[(uint64_t)d0 + (uint32_t)t] = out[t];
     }
+}
+
+template <bool SWITCH>
+static void qw_repack_launch(hipStream_t st, const void* w0, const void* s0, const void* b0, const void* w1, const void* s1,
+                             const void* b1, void* dst, uint64_t total, uint32_t groups, uint32_t pay_words, uint32_t inter,
+                             uint32_t is_f16, uint32_t* refused) {
+    const dim3 grid((unsigned)((total + 1023u) / 1024u)), block(256);
+    const bool vec = ((uintptr_t)dst & 15u) == 0;
+    const bool narrow = total + 4u < (1ull << 32);
+#define QW_REPACK_GO(IDX, VEC)                                                                                                   \
+    hipLaunchKernelGGL((qw_repack_mlx_kernel<SWITCH, IDX, VEC>), grid, block, 0, st, (const uint32_t*)w0, (const uint16_t*)s0,   \
+                       (const uint16_t*)b0, (const uint32_t*)w1, (const uint16_t*)s1, (const uint16_t*)b1, (uint32_t*)dst, total, \
+                       groups, pay_words, inter, is_f16, refused)
+    if (narrow && vec) QW_REPACK_GO(uint32_t, true);
+    else if (narrow) QW_REPACK_GO(uint32_t, false);
+    else if (vec) QW_REPACK_GO(uint64_t, true);
+    else QW_REPACK_GO(uint64_t, false);
+#undef QW_REPACK_GO
 }
 
 namespace {
@@ -147,11 +187,9 @@ extern "C" qwhip_status qwhip_repack_mlx_affine(qwhip_stream_t s, const void* ml
     QWHIP_REQUIRE(mlx_scales);
     QWHIP_REQUIRE(mlx_biases);
     const uint32_t groups = cols / group, pay_words = group * bits / 32u;
-    const uint64_t blocks = (uint64_t)rows * groups, total = blocks * (pay_words + 1u);
-    const dim3 grid((unsigned)((total + 255u) / 256u)), block(256);
-    hipLaunchKernelGGL(qw_repack_mlx_kernel<false>, grid, block, 0, s->stream, (const uint32_t*)mlx_w, (const uint16_t*)mlx_scales,
-                       (const uint16_t*)mlx_biases, nullptr, nullptr, nullptr, (uint32_t*)dst_blocks, blocks, groups, pay_words, 0u,
-                       scale_dtype == QWHIP_F16 ? 1u : 0u, refused);
+    const uint64_t total = (uint64_t)rows * groups * (pay_words + 1u);
+    qw_repack_launch<false>(s->stream, mlx_w, mlx_scales, mlx_biases, nullptr, nullptr, nullptr, dst_blocks, total, groups, pay_words,
+                            0u, scale_dtype == QWHIP_F16 ? 1u : 0u, refused);
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
@@ -170,11 +208,9 @@ extern "C" qwhip_status qwhip_repack_mlx_affine_switch_gate_up(qwhip_stream_t s,
     QWHIP_REQUIRE(up_scales);
     QWHIP_REQUIRE(up_biases);
     const uint32_t groups = cols / group, pay_words = group * bits / 32u;
-    const uint64_t blocks = (uint64_t)experts * 2u * inter * groups, total = blocks * (pay_words + 1u);
-    const dim3 grid((unsigned)((total + 255u) / 256u)), block(256);
-    hipLaunchKernelGGL(qw_repack_mlx_kernel<true>, grid, block, 0, s->stream, (const uint32_t*)gate_w, (const uint16_t*)gate_scales,
-                       (const uint16_t*)gate_biases, (const uint32_t*)up_w, (const uint16_t*)up_scales, (const uint16_t*)up_biases,
-                       (uint32_t*)dst_blocks, blocks, groups, pay_words, inter, scale_dtype == QWHIP_F16 ? 1u : 0u, refused);
+    const uint64_t total = (uint64_t)experts * 2u * inter * groups * (pay_words + 1u);
+    qw_repack_launch<true>(s->stream, gate_w, gate_scales, gate_biases, up_w, up_scales, up_biases, dst_blocks, total, groups,
+                           pay_words, inter, scale_dtype == QWHIP_F16 ? 1u : 0u, refused);
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }

@@ -1,0 +1,118 @@
+"""GPU parity of the f32-activation GEMV family (through the C ABI) against the CPU oracle: fp32 activations in the
+container's basis, fp32 outputs, epilogues 0..3.  Bar: the arithmetic is fp32 throughout, so outputs sit within 2e-5
+normalized error of the float64 evaluation (the judged bar for outputs is 2e-3); the standalone rotation is bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import qworacle as qo
+from qwegn_amd import qwhip
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-5
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return qwhip.Device(0)
+
+
+def _run(dev, fmt, n, k, m, epi, scale, seed=0):
+    _, bits, group, is_m5, _ = H.FORMATS[fmt]
+    blocks, _ = H.make_bank(fmt, n, k, seed=seed)
+    x = H.make_x(m, k, seed + 100)
+    bank, xb, yb = dev.put(blocks), dev.put(x), dev.alloc(max(256, m * n * 4))
+    view = H.view_of(dev, bank, fmt, n, k)
+    qwhip.check(dev.lib.qwhip_gemv_f32(dev.stream.handle, C.byref(view), xb.ptr, m, epi, scale, yb.ptr))
+    dev.stream.sync()
+    return yb.download(np.float32, (m, n)), qo.gemv_f32(blocks, x, bits, group, is_m5, epi, scale), (view, xb, bank)
+
+
+@pytest.mark.parametrize("fmt", list(H.FORMATS))
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_gemv_f32_matches_the_oracle(dev, fmt, m):
+    got, want, _ = _run(dev, fmt, 200, 1024, m, 0, 1.0, seed=m)
+    assert qo.normalized_error(got, want) <= TOL
+
+
+@pytest.mark.parametrize("epi,scale", [(1, 1.0), (1, 0.05), (2, 1.0), (3, 0.05), (3, 2.0)])
+@pytest.mark.parametrize("fmt,n", [("hq4_g32_m5", 256), ("aq8_g256", 200), ("hq4_g64", 77)])
+def test_gemv_f32_epilogues(dev, fmt, n, epi, scale):
+    """silu(y / scale), sigmoid, and silu + FWHT-32 over consecutive outputs (n = 200 and 77 end in a zero-padded group)."""
+    got, want, _ = _run(dev, fmt, n, 512, 3, epi, scale, seed=7)
+    assert qo.normalized_error(got, want) <= TOL
+
+
+@pytest.mark.parametrize("fmt,n,k,m", [
+    ("hq4_g32_m5", 300, 17408, 5),      # long rows: two activation rows per pass
+    ("hq4_g32_m5", 64, 32768, 2),       # longest rows the kernel takes: one per pass
+    ("aq4_g32", 5000, 2048, 9),         # three passes of 4 + 4 + 1
+    ("hq8_g32", 33, 32, 4),             # a single slice per row
+    ("hq4_g128", 1, 256, 1),            # one bank row
+])
+def test_gemv_f32_shapes(dev, fmt, n, k, m):
+    got, want, _ = _run(dev, fmt, n, k, m, 0, 1.0, seed=11)
+    assert qo.normalized_error(got, want) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq8_g32"])
+def test_epilogue3_rows_together_equal_rows_alone(dev, fmt):
+    """The reference's own check (Tests/QWGEMMTests/QWGemmEpi3MultiRowTests.swift:71-113): 2..5 rows in one call against
+    the same rows one call each, epilogue 3, scale 2.  Here the per-row arithmetic does not depend on the row count: equal bits."""
+    n, k = 128, 512
+    _, bits, group, is_m5, _ = H.FORMATS[fmt]
+    blocks, _ = H.make_bank(fmt, n, k, seed=3)
+    x = (((np.arange(5 * k) % 23) - 11) * 0.08).astype(np.float32).reshape(5, k)
+    bank, xb = dev.put(blocks), dev.put(x)
+    y_multi, y_one = dev.alloc(5 * n * 4), dev.alloc(5 * n * 4)
+    view = H.view_of(dev, bank, fmt, n, k)
+    st = dev.stream.handle
+    for rows in (2, 3, 4, 5):
+        qwhip.check(dev.lib.qwhip_gemv_f32(st, C.byref(view), xb.ptr, rows, 3, 2.0, y_multi.ptr))
+        for r in range(rows):
+            qwhip.check(dev.lib.qwhip_gemv_f32(st, C.byref(view), xb.ptr + r * k * 4, 1, 3, 2.0, y_one.ptr + r * n * 4))
+        dev.stream.sync()
+        a, b = y_multi.download(np.float32, (5, n))[:rows], y_one.download(np.float32, (5, n))[:rows]
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), rows
+        assert qo.normalized_error(a, qo.gemv_f32(blocks, x[:rows], bits, group, is_m5, 3, 2.0)) <= TOL
+
+
+def test_h32_f32_is_the_reference_butterfly(dev):
+    """qwhip_h32_f32 against the golden-pinned fp32 FWHT (same butterfly order: equal bits), out of place and in place."""
+    x = H.make_x(9, 1280, 5)
+    xb, ob = dev.put(x), dev.alloc(x.size * 4)
+    qwhip.check(dev.lib.qwhip_h32_f32(dev.stream.handle, xb.ptr, ob.ptr, 9, 1280))
+    qwhip.check(dev.lib.qwhip_h32_f32(dev.stream.handle, xb.ptr, xb.ptr, 9, 1280))
+    dev.stream.sync()
+    want = qo.fwht32_ortho(x)
+    assert np.array_equal(ob.download(np.float32, x.shape).view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(xb.download(np.float32, x.shape).view(np.uint32), want.view(np.uint32))
+
+
+def test_head_argmax_takes_f32_activations(dev):
+    fmt, n, k, m = "hq4_g32_m5", 3000, 1024, 2
+    _, bits, group, is_m5, _ = H.FORMATS[fmt]
+    blocks, _ = H.make_bank(fmt, n, k, seed=31)
+    x = H.make_x(m, k, 131)
+    bank, xb = dev.put(blocks), dev.put(x)
+    logits, toks = dev.alloc(m * n * 4), dev.alloc(256)
+    view = H.view_of(dev, bank, fmt, n, k)
+    qwhip.check(dev.lib.qwhip_head_argmax(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F32, m, 0, logits.ptr, toks.ptr))
+    dev.stream.sync()
+    got = logits.download(np.float32, (m, n))
+    assert qo.normalized_error(got, qo.gemv_f32(blocks, x, bits, group, is_m5)) <= TOL
+    assert np.array_equal(toks.download(np.int32, (m,)), qo.head_argmax(got))
+
+
+def test_gemv_f32_refusals(dev):
+    blocks, _ = H.make_bank("hq4_g32_m5", 8, 64, seed=1)
+    bank, xb, yb = dev.put(blocks), dev.put(np.zeros((1, 64), np.float32)), dev.alloc(256)
+    view = H.view_of(dev, bank, "hq4_g32_m5", 8, 64)
+    st = dev.stream.handle
+    assert dev.lib.qwhip_gemv_f32(st, C.byref(view), xb.ptr, 1, 4, 1.0, yb.ptr) == qwhip.E_BAD_SHAPE
+    assert dev.lib.qwhip_gemv_f32(st, C.byref(view), xb.ptr, 1, 1, 0.0, yb.ptr) == qwhip.E_BAD_SHAPE
+    assert dev.lib.qwhip_gemv_f32(st, C.byref(view), xb.ptr, 0, 0, 1.0, yb.ptr) == qwhip.E_BAD_SHAPE
+    assert dev.lib.qwhip_gemv_f32(st, C.byref(view), None, 1, 0, 1.0, yb.ptr) == qwhip.E_NULL
+    assert dev.lib.qwhip_h32_f32(st, xb.ptr, yb.ptr, 1, 48) == qwhip.E_BAD_SHAPE

@@ -293,3 +293,36 @@ def test_head_argmax_key_rule():
     logits[2, :] = np.nan                      # nothing but NaN: row 0
     logits[3, 999] = np.inf
     assert list(qo.head_argmax(logits)[:4]) == [7, int(np.nanargmax(logits[1])), 0, 999]
+
+
+def test_f32_gemv_family_closed_forms():
+    """The f32-activation GEMV restatement, pinned without retyping it: one-hot activations read single weights back (codes
+    and headers are pinned on the golden blocks), the epilogues obey sigmoid(v) + sigmoid(-v) = 1 and silu(z) - silu(-z) = z,
+    and epilogue 3's rotation is the golden-pinned fp32 FWHT (an involution; an impulse gives a +-1/sqrt(32) row)."""
+    rng = np.random.default_rng(5)
+    for bits, group, is_m5 in ((4, 32, True), (4, 64, False), (8, 32, False), (3, 32, False)):
+        w = rng.standard_normal((40, 128)).astype(np.float32) * 0.02
+        blocks, _ = qo.quant_hq_blocks(w, bits=bits, group=group, is_m5=is_m5, rotate=False)
+        s, b = qo.hq_block_header(blocks) if not is_m5 else (
+            np.ascontiguousarray(blocks[..., 0:2]).view(np.float16)[..., 0], np.ascontiguousarray(blocks[..., 2:4]).view(np.float16)[..., 0])
+        codes = (qo.hq4_codes(blocks).reshape(40, 128).astype(np.int64) + 1024) if is_m5 else qo.hq_block_codes(blocks, bits, group).reshape(40, 128)
+        for col in (0, 37, 127):
+            x = np.zeros((1, 128), np.float32)
+            x[0, col] = 1.0
+            want = codes[:, col].astype(np.float64) * s[:, col // group].astype(np.float64) + b[:, col // group].astype(np.float64)
+            assert np.array_equal(qo.gemv_f32(blocks, x, bits, group, is_m5)[0], want)
+        x = rng.standard_normal((3, 128)).astype(np.float32)
+        y = qo.gemv_f32(blocks, x, bits, group, is_m5)
+        assert np.allclose(qo.gemv_f32(blocks, x, bits, group, is_m5, 2) + qo.gemv_f32(blocks, -x, bits, group, is_m5, 2), 1.0, atol=1e-15)
+        assert np.allclose(qo.gemv_f32(blocks, x, bits, group, is_m5, 1, 0.25) - qo.gemv_f32(blocks, -x, bits, group, is_m5, 1, 0.25), y / 0.25, atol=1e-12)
+        y3 = qo.gemv_f32(blocks, x, bits, group, is_m5, 3, 2.0)           # 40 outputs: one whole group and a padded one
+        y1 = qo.gemv_f32(blocks, x, bits, group, is_m5, 1, 2.0)
+        padded = np.zeros((3, 64))
+        padded[:, :40] = y1
+        assert np.allclose(y3, qo.fwht32_ortho(padded.astype(np.float32))[:, :40], atol=1e-6)
+        assert np.allclose(qo.h32_groups_f64(qo.h32_groups_f64(padded)), padded, atol=1e-14)
+    e = np.zeros((1, 32))
+    e[0, 5] = 1.0
+    row = qo.h32_groups_f64(e)[0] * np.sqrt(32.0)
+    assert np.allclose(np.abs(row), 1.0) and row[0] == 1.0 and row[5] == np.float64((-1) ** bin(5).count("1"))
+    assert qo.v4_epilogue_f64(np.array([0.0]), 2, 1.0)[0] == 0.5 and qo.v4_epilogue_f64(np.array([0.0]), 1, 3.0)[0] == 0.0
