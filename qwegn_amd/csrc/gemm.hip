@@ -897,10 +897,13 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     const dim3 grid(((total + 7u) / 8u) * 8u);
     switch (cfg) {
         case CFG_256x320:
-            // the ping-pong kernel takes whole 64-row activation blocks; ragged M stays on the DMA-fed kernel
-            if (p.M % 64u == 0 && !p.force_gemm2 &&
-                (YDT == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0)))
-                return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
+            // the ping-pong kernel takes whole 64-row activation blocks; ragged M stays on the DMA-fed kernel, and so do the
+            // 8-bit containers: their wider weight items do not fit the ping-pong kernel's register budget at this tile
+            if constexpr (FMT != QG_FMT_B8) {
+                if (p.M % 64u == 0 && !p.force_gemm2 &&
+                    (YDT == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0)))
+                    return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
+            }
             return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x256: return launch_cfg2<2, 4, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x128: return launch_cfg2<2, 2, 4, 2, FMT, YDT, false>(st, p, grid);
