@@ -546,17 +546,16 @@ def run_moe(args, t, label):
         mt = max(1, lib.qwhip_moe_max_tiles(E, pairs))
         off, sp, stok, inv = dev.alloc((E + 1) * 4), dev.alloc(pairs * 4), dev.alloc(pairs * 4), dev.alloc(pairs * 4)
         te, tr, tc = dev.alloc(mt * 4), dev.alloc(mt * 4), dev.alloc(16)
-        gu_out, dn_out = dev.alloc(pairs * 2 * I * 2), dev.alloc(pairs * Hd * 2)
+        dn_out = dev.alloc(pairs * Hd * 2)
 
-        def gate_up():
-            qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), E, xb.ptr, qwhip.F16, 0, stok.ptr, off.ptr, te.ptr, tr.ptr, tc.ptr,
-                                                   mt, pairs, gu_out.ptr, qwhip.F16, 0))
+        def gate_up():   # grouped gate|up GEMM with the SwiGLU + FWHT-32 epilogue fused
+            qwhip.check(lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(vgu), E, xb.ptr, qwhip.F16, 0, stok.ptr, off.ptr, te.ptr, tr.ptr,
+                                                          tc.ptr, mt, pairs, 1, act.ptr, 0))
 
         def chain():
             qwhip.check(lib.qwhip_moe_route(st, lb.ptr, t, E, K, 1, 1.0, ib.ptr, wb.ptr))
             qwhip.check(lib.qwhip_moe_group_pairs(st, ib.ptr, E, pairs, K, off.ptr, sp.ptr, stok.ptr, inv.ptr, te.ptr, tr.ptr, tc.ptr, 1))
             gate_up()
-            qwhip.check(lib.qwhip_swiglu_fwht(st, gu_out.ptr, qwhip.F16, act.ptr, pairs, I, 1))
             qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vdn), E, act.ptr, qwhip.F16, 0, None, off.ptr, te.ptr, tr.ptr, tc.ptr,
                                                    mt, pairs, dn_out.ptr, qwhip.F16, 0))
             qwhip.check(lib.qwhip_moe_combine(st, dn_out.ptr, qwhip.F16, inv.ptr, wb.ptr, t, K, Hd, None, None, out.ptr, qwhip.F32))

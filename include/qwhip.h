@@ -253,6 +253,19 @@ qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_weight_view* w
                                     const int32_t* tile_count, uint32_t max_tiles, uint32_t pairs,
                                     void* y, uint32_t y_dtype, uint32_t ldy);
 
+/* The gate_up grouped GEMM with the SwiGLU (+ FWHT-32) epilogue fused: act f16 [pairs, inter] in sorted-pair order,
+ * inter = rows_per_expert / 2, an expert's rows being [gate | up].  Bit-identical to qwhip_moe_grouped_gemm with f16 output
+ * followed by qwhip_swiglu_fwht (both accumulators are rounded to f16 first, SwiGLU and the rotation run in fp32, one f16
+ * rounding on store), without writing and re-reading the [pairs, 2 inter] matrix.  The reference fuses the same epilogue
+ * into its dense gate_up GEMM (qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167; kernel
+ * qwg_gemm_q4g_h16_swiglu) and runs encodeSiluMul* after the grouped one (QWMoEOperator.swift).
+ * f16 activations only; inter % 32 == 0; act 16-byte aligned with ldact % 8 == 0 (0 = inter). */
+qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, uint32_t experts,
+                                           const void* x, uint32_t x_dtype, uint32_t ldx, const int32_t* gather,
+                                           const int32_t* expert_off, const int32_t* tile_e, const int32_t* tile_r,
+                                           const int32_t* tile_count, uint32_t max_tiles, uint32_t pairs,
+                                           uint32_t rotate_act, void* act_f16, uint32_t ldact);
+
 /* qwg_moe_down_reduce_combine_f32 (Sources/QWMetal/gemm/qwgemm_moe_nax_f16.metal:7-126;
  * encodeMoEDownReduceCombineF32, QWGemmMoE.swift:299-332):
  * out[t, h] = sum_k wts[t, k] * dn[inv_perm[t*top_k + k], h] (+ shared_gate[t] * shared[t, h]). */

@@ -39,6 +39,7 @@ struct qw_gemm_params {
     const int32_t* tile_r;
     const int32_t* tile_count;
     uint32_t rows_per_expert;
+    uint32_t inter, rotate_act;  // fused SwiGLU epilogue: gate rows [0, inter), up rows [inter, 2 inter) of an expert; FWHT-32 on the result
     uint32_t force_gemm2;  // tuning / tests: keep the DMA-fed kernel for the 256 x 320 shape
 #ifdef QW_GEMM_TIMING
     unsigned long long* tlog;  // probe builds only: per-phase cycle stamps of workgroup 0, wave 0
@@ -504,9 +505,16 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 #define QG3_BAR_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define QG3_BAR_ALL() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED>
+// SWIGLU (grouped, 64 x 256 tiles, f16 out): a tile's 256 weight rows are 128 gate rows and the 128 up rows of the same
+// outputs, laid out so that each wave's two fragments are (gate, up) of the same 32 outputs: tile column 64 w + 32 b + j is
+// expert row b * inter + 128 * blockIdx.x + 32 w + j.  The epilogue rounds both accumulators to f16 (the values the
+// unfused chain stores), applies SwiGLU and the FWHT-32 in fp32 and stores act f16 [pair, inter]: the arithmetic of
+// qwhip_swiglu_fwht on the f16 gate|up matrix, without writing it (the reference's fused form for its dense path:
+// qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167).
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED, bool SWIGLU = false>
 __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_params p) {
     static_assert(WVM * WVN == 8, "two groups of four waves");
+    static_assert(!SWIGLU || (GROUPED && WM == 1 && WN == 2 && WVN == 4 && YDT == QWHIP_F16), "fused SwiGLU: grouped 64 x 256 tiles, f16 out");
     constexpr int NT = WVM * WVN * 64;
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 64;
     constexpr int B_ITEMS = BN * 2;
@@ -533,7 +541,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
         const uint32_t end = (uint32_t)p.expert_off[e + 1];
         m0 = start;
         rows_valid = min((uint32_t)BM, min(bm, end - start));
-        n0 = blockIdx.x * BN;
+        n0 = blockIdx.x * (SWIGLU ? BN / 2 : BN);
         bank += (uint64_t)e * p.rows_per_expert * p.row_bytes;
     } else {
         const uint32_t total = p.tiles_m * p.tiles_n;
@@ -579,12 +587,18 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     // the tile are done redundantly by several threads: identical bytes to the same slot) ----
     static_assert(B_ITEMS >= NT && B_ITEMS <= NT + NT / 2, "the second weight items are covered by group 0 alone");
     uint32_t b_off32[B_PER], b_meta[B_PER];   // byte offset of the row inside the tile's bank rows; LDS row offset | swizzle key << 16 | slice << 20
-    const uint8_t* b_tile = bank + (uint64_t)n0 * p.row_bytes;
+    const uint8_t* b_tile = bank + (SWIGLU ? 0ull : (uint64_t)n0 * p.row_bytes);
 #pragma unroll
     for (int i = 0; i < B_PER; ++i) {
         const uint32_t it = i == 0 ? tid : NT + (B_ITEMS > NT ? tid % (uint32_t)(B_ITEMS > NT ? B_ITEMS - NT : 1) : 0u);
         const uint32_t nl = it >> 1;
-        const uint32_t n = min(n0 + nl, p.N - 1u) - n0;
+        uint32_t n;
+        if constexpr (SWIGLU) {
+            // n0 counts act columns here and b_tile is the expert's first row
+            n = ((nl & 32u) ? p.inter : 0u) + min(n0 + 32u * (nl >> 6) + (nl & 31u), p.inter - 1u);
+        } else {
+            n = min(n0 + nl, p.N - 1u) - n0;
+        }
         b_off32[i] = n * (uint32_t)p.row_bytes;                     // a tile's rows span < 4 GiB
         b_meta[i] = (nl * 128u) | (((nl >> 1) & 7u) << 16) | ((it & 1u) << 20);
     }
@@ -768,7 +782,38 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    if constexpr (YDT != QWHIP_F32) {
+    if constexpr (SWIGLU) {
+        // lane (lane & 31) holds output column c = n0 + 32 wn + (lane & 31) of 16 rows: gate in acc[0][0], up in acc[0][1]
+        constexpr uint32_t EP_PITCH = 64 + 16;
+        __syncthreads();
+        uint8_t* ep = lds2 + wave * (32u * EP_PITCH);
+        const uint32_t j = lane & 31u;
+        const uint32_t w_off = (4u * (lane >> 5)) * EP_PITCH + j * 2u;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float g = (float)(h1_t)acc[0][0][r], u = (float)(h1_t)acc[0][1][r];
+            float v = qw_swiglu(g, u);
+            if (p.rotate_act) {
+#pragma unroll
+                for (uint32_t h = 1; h < 32u; h <<= 1) {
+                    const float o = __shfl_xor(v, (int)h, 32);
+                    v = (j & h) == 0u ? v + o : o - v;
+                }
+                v *= QW_INV_SQRT32;
+            }
+            *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
+        }
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t c = q * 64u + lane;
+            const uint32_t row = c >> 2, cc = c & 3u;
+            const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
+            const uint32_t grow = wm * 32u + row;
+            const uint32_t n = n0 + wn * 32u + cc * 8u;
+            if (grow < rows_valid && n < p.inter)
+                *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+        }
+    } else if constexpr (YDT != QWHIP_F32) {
         // 2-byte outputs: each wave transposes its 32-row slabs through a private LDS region (the operand stages are
         // dead by now) and stores 16-byte row chunks; a lane's accumulators are one column of 16 rows, and 2-byte
         // stores from that layout cost one address per element. The host side guarantees 16-byte aligned output rows.
@@ -869,11 +914,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED = false>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED = false, bool SWIGLU = false>
 hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED>;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED, SWIGLU>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1118,6 +1163,61 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_wei
     if (fmt == QG_FMT_M5) e = launch_grouped_xy<QG_FMT_M5>(s->stream, p, grid, x_dtype, y_dtype);
     else if (fmt == QG_FMT_B4) e = launch_grouped_xy<QG_FMT_B4>(s->stream, p, grid, x_dtype, y_dtype);
     else e = launch_grouped_xy<QG_FMT_B8>(s->stream, p, grid, x_dtype, y_dtype);
+    QWHIP_TRY_HIP(e);
+    return QWHIP_OK;
+}
+
+// Grouped gate|up GEMM with the SwiGLU (+ FWHT-32) epilogue fused: act f16 [pairs, inter] in sorted-pair order, bit-identical
+// to qwhip_moe_grouped_gemm (f16 out) followed by qwhip_swiglu_fwht, without the [pairs, 2 inter] matrix in between.
+extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, uint32_t experts, const void* x,
+                                                      uint32_t x_dtype, uint32_t ldx, const int32_t* gather,
+                                                      const int32_t* expert_off, const int32_t* tile_e, const int32_t* tile_r,
+                                                      const int32_t* tile_count, uint32_t max_tiles, uint32_t pairs,
+                                                      uint32_t rotate_act, void* act_f16, uint32_t ldact) {
+    int fmt = 0;
+    qwhip_status st = gemm_checks(s, w, x, x_dtype, act_f16, QWHIP_F16, &fmt);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(expert_off);
+    QWHIP_REQUIRE(tile_e);
+    QWHIP_REQUIRE(tile_r);
+    QWHIP_REQUIRE(tile_count);
+    if (x_dtype != QWHIP_F16)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "the fused gate_up GEMM takes f16 activations (bf16: qwhip_moe_grouped_gemm + qwhip_swiglu_fwht)");
+    if (experts == 0 || experts > 512 || w->n % experts != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "grouped GEMM: %u rows do not split over %u experts (<= 512)", w->n, experts);
+    if (pairs == 0 || max_tiles == 0) return QWHIP_OK;
+    const uint32_t rows_per_expert = w->n / experts, inter = rows_per_expert / 2u;
+    if (rows_per_expert % 64u != 0)
+        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "fused gate_up needs an intermediate size %% 32 == 0, got %u rows per expert", rows_per_expert);
+    if (ldx == 0) ldx = w->k;
+    if (ldact == 0) ldact = inter;
+    if (ldx < w->k || ldact < inter || (ldx % 8) != 0 || (ldact % 8) != 0 || ((uintptr_t)act_f16 & 15u) != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions or alignment (ldx=%u ldact=%u, act 16-byte aligned)", ldx, ldact);
+    qw_gemm_params p = {};
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = x;
+    p.y = act_f16;
+    p.M = pairs;
+    p.N = rows_per_expert;
+    p.K = w->k;
+    p.ldx = ldx;
+    p.ldy = ldact;
+    p.gshift = log2_u32(w->group / 32);
+    p.bb = qwhip_view_block_bytes(w);
+    p.row_bytes = qwhip_view_row_bytes(w);
+    p.gather = gather;
+    p.expert_off = expert_off;
+    p.tile_e = tile_e;
+    p.tile_r = tile_r;
+    p.tile_count = tile_count;
+    p.rows_per_expert = rows_per_expert;
+    p.inter = inter;
+    p.rotate_act = rotate_act ? 1u : 0u;
+    const dim3 grid(qwhip_cdiv(inter, 128u), max_tiles);
+    hipError_t e;
+    if (fmt == QG_FMT_M5) e = launch_cfg3<1, 2, 2, 4, QG_FMT_M5, QWHIP_F16, true, true>(s->stream, p, grid);
+    else if (fmt == QG_FMT_B4) e = launch_cfg3<1, 2, 2, 4, QG_FMT_B4, QWHIP_F16, true, true>(s->stream, p, grid);
+    else e = launch_cfg3<1, 2, 2, 4, QG_FMT_B8, QWHIP_F16, true, true>(s->stream, p, grid);
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
 }

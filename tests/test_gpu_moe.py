@@ -149,6 +149,53 @@ def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
     assert qo.normalized_error(got, ref) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32"])
+@pytest.mark.parametrize("t,experts,hidden,inter,k,rot", [(40, 8, 256, 128, 2, 1), (130, 16, 512, 192, 4, 1), (300, 4, 128, 64, 2, 0),
+                                                          (64, 8, 192, 448, 3, 1)])
+def test_fused_gate_up_swiglu_equals_the_two_step_chain(dev, fmt, t, experts, hidden, inter, k, rot):
+    """qwhip_moe_grouped_gemm_swiglu == qwhip_moe_grouped_gemm (f16 out) + qwhip_swiglu_fwht, bit for bit, on the rows of the
+    sorted list (intermediate sizes with a partial 128-column tile included), and the chain built on it meets the oracle."""
+    gu_blocks, gu16, dn_blocks, dn16 = _moe_banks(experts, hidden, inter, seed=13, fmt=fmt)
+    rng = np.random.default_rng(9)
+    x16 = rng.standard_normal((t, hidden)).astype(np.float16)
+    logits = rng.standard_normal((t, experts)).astype(np.float32)
+    idx, wts = _route(dev, logits, k)
+    g = _group(dev, idx, experts, k)
+    pairs = t * k
+    lib, st, b = dev.lib, dev.stream.handle, g["bufs"]
+    gub, xb = dev.put(gu_blocks), dev.put(x16)
+    gu_out = dev.alloc(pairs * 2 * inter * 2)
+    act2, act1 = dev.put(np.zeros((pairs, inter), np.float16)), dev.put(np.zeros((pairs, inter), np.float16))
+    vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
+    qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, b["stok"].ptr, b["off"].ptr, b["te"].ptr,
+                                           b["tr"].ptr, b["tc"].ptr, g["max_tiles"], pairs, gu_out.ptr, qwhip.F16, 0))
+    qwhip.check(lib.qwhip_swiglu_fwht(st, gu_out.ptr, qwhip.F16, act2.ptr, pairs, inter, rot))
+    qwhip.check(lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, b["stok"].ptr, b["off"].ptr,
+                                                  b["te"].ptr, b["tr"].ptr, b["tc"].ptr, g["max_tiles"], pairs, rot, act1.ptr, 0))
+    dev.stream.sync()
+    valid = int(g["off"][experts])
+    two, one = act2.download(np.float16, (pairs, inter))[:valid], act1.download(np.float16, (pairs, inter))[:valid]
+    assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
+    # against the oracle: act of sorted slot p = swiglu(x[tok] . gate_e, x[tok] . up_e), rotated
+    e_of = np.repeat(np.arange(experts), np.diff(g["off"]))
+    xs = x16[g["stok"][:valid]].astype(np.float64)
+    gu = np.einsum("pk,pnk->pn", xs, gu16[e_of].astype(np.float64)).astype(np.float16).astype(np.float32)
+    want = qo.swiglu_fwht_f16(gu[:, :inter], gu[:, inter:], rotate=bool(rot)).astype(np.float32)
+    assert qo.normalized_error(one.astype(np.float32), want) <= TOL
+
+
+def test_fused_gate_up_swiglu_refusals(dev):
+    blocks, _ = H.make_bank("hq4_g32_m5", 4 * 2 * 48, 64, 1)
+    bank, xb, act = dev.put(blocks), dev.put(np.zeros((4, 64), np.float16)), dev.alloc(4096)
+    z = dev.put(np.zeros(64, np.int32))
+    lib, st = dev.lib, dev.stream.handle
+    v = H.view_of(dev, bank, "hq4_g32_m5", 4 * 2 * 48, 64)
+    args = (z.ptr, z.ptr, z.ptr, z.ptr, 4, 4, 1, act.ptr, 0)
+    assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v), 4, xb.ptr, qwhip.F16, 0, None, *args) == qwhip.E_BAD_GEOMETRY   # inter = 48
+    v2 = H.view_of(dev, bank, "hq4_g32_m5", 4 * 2 * 48, 64)
+    assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v2), 3, xb.ptr, qwhip.BF16, 0, None, *args) == qwhip.E_BAD_SHAPE     # bf16 activations
+
+
 # (format, gate_up kernel override): HQ4_G32_M5 runs the column-stationary kernels, override 2 keeps its gate_up on the
 # general kernel; the bit-stream container runs the general kernels for both projections.
 @pytest.mark.parametrize("fmt,gu_flags", [("hq4_g32_m5", 0), ("hq4_g32_m5", 2 << 8), ("hq4_g32", 0)])
