@@ -9,8 +9,8 @@
 //
 // Arithmetic: all in fp32.  The reference dequantises one weight as fma(float(code [+ 1024]), scale, bias) in fp32 and
 // feeds an fp32 FMA chain (qwg_unpack_hq4_word8_f32 / qwg_dot_hq4_block_f32_reg, qw_dequant_f32.metalh:10-58); here the
-// affine part is applied once per slice, sum_i w_i x_i = scale * sum_i code_i x_i + bias * sum_i x_i (HQ4_G32_M5:
-// scale * (sum_i code_i x_i + 1024 S) + bias * S), codes converted to fp32 exactly.  Both differ from the exact sum only by
+// affine part is applied once per slice, sum_i w_i x_i = scale * sum_i code_i x_i + bias * sum_i x_i (HQ4_G32_M5: bias stands
+// for fma(1024, scale, bias), rounded once), codes converted to fp32 exactly.  Both differ from the exact sum only by
 // fp32 rounding.
 #include "qwhip_common.h"
 
@@ -134,7 +134,10 @@ __global__ __launch_bounds__(LB) void qw_gemv_f32_kernel(const qf_params p) {
             for (int t = 0; t < PW; ++t) qq[t] = q[j][t];
             const h2_t hd = __builtin_bit_cast(h2_t, hdr[j]);
             issue(j);
-            const float sc = (float)hd[0], bi = (float)hd[1];
+            const float sc = (float)hd[0];
+            // HQ4_G32_M5: weight = (1024 + code) * scale + bias = code * scale + (1024 * scale + bias); the bracket is formed with
+            // one rounding, so the large terms cancel before they meet the activations
+            const float bi = FMT == QW_FMT_M5 ? __builtin_fmaf(1024.0f, sc, (float)hd[1]) : (float)hd[1];
             float acc[MR][4];
 #pragma unroll
             for (int m = 0; m < MR; ++m) acc[m][0] = acc[m][1] = acc[m][2] = acc[m][3] = 0.f;
@@ -171,8 +174,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_f32_kernel(const qf_params p) {
             }
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
-                float qs = (acc[m][0] + acc[m][1]) + (acc[m][2] + acc[m][3]);
-                if constexpr (FMT == QW_FMT_M5) qs = __builtin_fmaf(1024.0f, S[m], qs);
+                const float qs = (acc[m][0] + acc[m][1]) + (acc[m][2] + acc[m][3]);
                 float v = __builtin_fmaf(sc, qs, bi * S[m]);
                 v = gvalid ? v : 0.0f;
                 v = qw_reduce32_dpp(v);

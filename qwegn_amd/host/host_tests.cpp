@@ -309,6 +309,67 @@ static void test_gpu_moe_resident(QWHal& hal, int rows) {
     hal.end(enc);
 }
 
+// f32-activation doors and the head: encodeHQ4F32V4 (epilogues 0 and 3), encodeH32F32, encodeHeadArgmax on the closed-form bank
+static void test_gpu_f32_doors(QWHal& hal) {
+    const int N = 96, Kc = 128, rows = 3;
+    const std::vector<uint8_t> bank = cf_bank(N, Kc);
+    std::vector<float> x((size_t)rows * Kc);
+    for (int t = 0; t < rows; ++t)
+        for (int c = 0; c < Kc; ++c) x[(size_t)t * Kc + c] = (float)(((t * 29 + c * 5) % 23) - 11) * 0.08f;
+    std::vector<double> y0((size_t)rows * N);
+    for (int t = 0; t < rows; ++t)
+        for (int n = 0; n < N; ++n) {
+            double s = 0;
+            for (int c = 0; c < Kc; ++c) s += cf_weight(n, c) * (double)x[(size_t)t * Kc + c];
+            y0[(size_t)t * N + n] = s;
+        }
+    QWHipEncoder enc = hal.begin();
+    DeviceBuf dbank(hal, bank.size()), dx(hal, x.size() * 4), dy(hal, y0.size() * 4), dtok(hal, 64);
+    upload(enc, dbank, bank.data(), bank.size());
+    upload(enc, dx, x.data(), x.size() * 4);
+    const auto view = QWWeightView::make(QWTensorValue::make(dbank.p, bank.size(), QWDType::q4g), N, Kc, 4, 32, true);
+    CHECK(view.has_value());
+    const QWTensorValue xt = QWTensorValue::make(dx.p, x.size(), QWDType::f32), yt = QWTensorValue::make(dy.p, y0.size(), QWDType::f32);
+    std::vector<float> got(y0.size());
+    QWGemm::encodeHQ4F32V4(enc, hal, *view, xt, yt, rows);
+    download(enc, got.data(), dy, got.size() * 4);
+    for (size_t i = 0; i < got.size(); ++i) CHECK(std::fabs((double)got[i] - y0[i]) <= 1e-4 * std::fmax(1.0, std::fabs(y0[i])));
+    // epilogue 3: silu(y / 2) then the rotation over each 32 consecutive outputs
+    QWGemm::encodeHQ4F32V4(enc, hal, *view, xt, yt, rows, 3, 2.0f);
+    download(enc, got.data(), dy, got.size() * 4);
+    for (int t = 0; t < rows; ++t)
+        for (int g = 0; g < N / 32; ++g) {
+            double v[32];
+            for (int i = 0; i < 32; ++i) {
+                const double z = y0[(size_t)t * N + g * 32 + i] / 2.0;
+                v[i] = z / (1.0 + std::exp(-z));
+            }
+            fwht32(v);
+            for (int i = 0; i < 32; ++i) CHECK(std::fabs((double)got[(size_t)t * N + g * 32 + i] - v[i]) <= 1e-4 * std::fmax(1.0, std::fabs(v[i])));
+        }
+    // the standalone rotation is an involution
+    QWGemm::encodeHQ4F32V4(enc, hal, *view, xt, yt, rows);
+    QWGemm::encodeH32F32(enc, hal, yt, yt, rows, N);
+    QWGemm::encodeH32F32(enc, hal, yt, yt, rows, N);
+    download(enc, got.data(), dy, got.size() * 4);
+    for (size_t i = 0; i < got.size(); ++i) CHECK(std::fabs((double)got[i] - y0[i]) <= 1e-4 * std::fmax(1.0, std::fabs(y0[i])));
+    // head: the token is the first maximum of the logits it leaves behind
+    QWGemmAQ::encodeHeadArgmax(enc, hal, *view, xt, yt, QWTensorValue::make(dtok.p, 16, QWDType::i32), rows);
+    download(enc, got.data(), dy, got.size() * 4);
+    int32_t tok[16];
+    download(enc, tok, dtok, 64);
+    for (int t = 0; t < rows; ++t) {
+        int best = 0;
+        for (int n = 1; n < N; ++n)
+            if (got[(size_t)t * N + n] > got[(size_t)t * N + best]) best = n;
+        CHECK(tok[t] == best);
+    }
+    const QWTensorValue x16 = QWTensorValue::make(dx.p, x.size(), QWDType::f16);
+    CHECK_THROWS(QWGemm::encodeHQ4F32V4(enc, hal, *view, x16, yt, rows), QWGemmError, QWGemmError::badWeights);
+    CHECK_THROWS(QWGemm::encodeHQ4F32V4(enc, hal, *view, xt, yt, rows, 7), QWGemmError, QWGemmError::badShape);
+    hal.end(enc);
+}
+
 int main(int argc, char** argv) {
     const bool gpu = argc > 1 && std::strcmp(argv[1], "--gpu") == 0;
     test_plan_table();
@@ -322,7 +383,8 @@ int main(int argc, char** argv) {
         std::printf("device: %s (%s), %u CUs\n", hal.caps.name, hal.caps.arch, hal.caps.compute_units);
         test_gpu_hq4_gemv(hal);
         test_gpu_moe_resident(hal, 3);    // decode / verify path
-        test_gpu_moe_resident(hal, 40);   // grouped prefill path
+        test_gpu_moe_resident(hal, 40);   // grouped prefill path (fused gate_up + SwiGLU)
+        test_gpu_f32_doors(hal);
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed ? 1 : 0;

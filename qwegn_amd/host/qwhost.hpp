@@ -350,6 +350,44 @@ struct QWGemm {
         throwIfFailed(qwhip_swiglu_fwht(enc.stream, gu.ptr(), abiDType(gu.shape.dtype), act16.ptr(), (uint32_t)rows, (uint32_t)inter, rotate ? 1 : 0));
     }
 
+    // QWGemm.encodeHQ4F32V4 / encodeHQ4F32BM (Sources/Operators/QWGEMM/QWGemmF32.swift:178-199,311-350): f32 activations in the
+    // container's basis -> f32 outputs; epi 0 none, 1 silu(y/scale), 2 sigmoid, 3 silu(y/scale) + H_32.
+    static void encodeHQ4F32V4(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& w, const QWTensorValue& x, const QWTensorValue& y,
+                               int rows = 1, uint32_t epi = 0, float scale = 1.0f) {
+        if (rows <= 0) throw QWGemmError(QWGemmError::badShape, "rows must be positive");
+        if (x.shape.dtype != QWDType::f32 || y.shape.dtype != QWDType::f32 || x.shape.elementCount < (size_t)rows * (size_t)w.k ||
+            y.shape.elementCount < (size_t)rows * (size_t)w.n)
+            throw QWGemmError(QWGemmError::badWeights, "f32 v4: x f32 [rows, K], y f32 [rows, N]");
+        hal.pipeline(w.containerKind.isIncumbentContainer()
+                         ? "qwg_gemv_q4g_f32_v4"
+                         : ("qwg_gemv_aq" + std::to_string(w.bits()) + "_g" + std::to_string(w.groupSize()) + "_f32_v4").c_str());
+        const qwhip_weight_view v = w.abi();
+        throwIfFailed(qwhip_gemv_f32(enc.stream, &v, (const float*)x.ptr(), (uint32_t)rows, epi, scale, (float*)y.ptr()));
+    }
+
+    // QWGemm.encodeH32F32 (QWGemmF32.swift:46-54): out f32 [rows, hidden] = rotate(x) in the normalised Walsh-Hadamard domain.
+    static void encodeH32F32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWTensorValue& out, int rows, int hidden) {
+        if (x.shape.dtype != QWDType::f32 || out.shape.dtype != QWDType::f32 || rows <= 0 || hidden <= 0 || hidden % 32 != 0 ||
+            x.shape.elementCount < (size_t)rows * (size_t)hidden || out.shape.elementCount < (size_t)rows * (size_t)hidden)
+            throw QWGemmError(QWGemmError::badShape, "h32 f32: f32 [rows, hidden], hidden % 32 == 0");
+        hal.pipeline("qwg_h32_f32");
+        throwIfFailed(qwhip_h32_f32(enc.stream, (const float*)x.ptr(), (float*)out.ptr(), (uint32_t)rows, (uint32_t)hidden));
+    }
+
+    // encodeRMSNormFast / encodeRMSNormResidualFast (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:339-404): y16 = rotate?(
+    // rmsnorm(x [+ residual]) * (1 + gamma)); with `residual` the sum is written back to it.
+    static void encodeRMSNormFast(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWTensorValue& gamma,
+                                  const QWTensorValue& y, int rows, int hidden, float eps, bool rotate = true,
+                                  const QWTensorValue* residual = nullptr) {
+        if (x.shape.dtype != QWDType::f16 || gamma.shape.dtype != QWDType::f16 || y.shape.dtype != QWDType::f16 ||
+            (residual && residual->shape.dtype != QWDType::f16) || rows <= 0 || x.shape.elementCount < (size_t)rows * (size_t)hidden ||
+            y.shape.elementCount < (size_t)rows * (size_t)hidden || gamma.shape.elementCount < (size_t)hidden)
+            throw QWGemmError(QWGemmError::badShape, "rmsnorm: f16 [rows, hidden] in and out, f16 gamma [hidden]");
+        hal.pipeline(residual ? "qwg_rmsnorm_residual" : "qwg_rmsnorm");
+        throwIfFailed(qwhip_rmsnorm(enc.stream, x.ptr(), gamma.ptr(), residual ? residual->ptr() : nullptr, (uint32_t)rows, (uint32_t)hidden,
+                                    eps, rotate ? 1u : 0u, y.ptr()));
+    }
+
     // ---- MoE encoders (Sources/Operators/QWGEMM/QWGemmMoE.swift, QWGemmMoERouter.swift) ----------------------------
     static int moeMaxTiles(int experts, int pairs) { return (int)qwhip_moe_max_tiles((uint32_t)experts, (uint32_t)pairs); }  // QWGemmMoE.swift:24-26
 
@@ -399,6 +437,24 @@ struct QWGemm {
                                              gather ? (const int32_t*)gather->ptr() : nullptr, (const int32_t*)expertOff.ptr(),
                                              (const int32_t*)tileE.ptr(), (const int32_t*)tileR.ptr(), (const int32_t*)tileCount.ptr(),
                                              (uint32_t)moeMaxTiles(experts, pairs), (uint32_t)pairs, y.ptr(), abiDType(y.shape.dtype), 0));
+    }
+    // The prefill pair encodeMoEGateUpNax + encodeSiluMul* as one launch: act16 [pairs, inter] = FWHT32(silu(g) * u) of the sorted
+    // pairs, bit-identical to the two encoders above (f16 activations; inter % 32 == 0).
+    static void encodeMoEGateUpSwiglu(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& w, int experts, const QWTensorValue& x,
+                                      const QWTensorValue& gather, const QWTensorValue& expertOff, const QWTensorValue& tileE,
+                                      const QWTensorValue& tileR, const QWTensorValue& tileCount, int pairs, const QWTensorValue& act16,
+                                      bool rotate = true) {
+        if (x.shape.dtype != QWDType::f16 || act16.shape.dtype != QWDType::f16)
+            throw QWGemmError(QWGemmError::badShape, "fused gate_up: f16 activations in, f16 act out");
+        if (experts <= 0 || w.n % experts != 0 || act16.shape.elementCount < (size_t)pairs * (size_t)(w.n / experts / 2))
+            throw QWGemmError(QWGemmError::badShape, "fused gate_up: act does not fit pairs x intermediate");
+        hal.pipeline("qwg_moe_nax_gemm");
+        hal.pipeline("qwg_silu_mul_f16");
+        const qwhip_weight_view v = w.abi();
+        throwIfFailed(qwhip_moe_grouped_gemm_swiglu(enc.stream, &v, (uint32_t)experts, x.ptr(), QWHIP_F16, 0, (const int32_t*)gather.ptr(),
+                                                    (const int32_t*)expertOff.ptr(), (const int32_t*)tileE.ptr(), (const int32_t*)tileR.ptr(),
+                                                    (const int32_t*)tileCount.ptr(), (uint32_t)moeMaxTiles(experts, pairs), (uint32_t)pairs,
+                                                    rotate ? 1u : 0u, act16.ptr(), 0));
     }
     // encodeMoEDownReduceCombineF32 (QWGemmMoE.swift:299-332)
     static void encodeMoEDownReduceCombineF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& dn, const QWTensorValue& invPerm,
@@ -474,6 +530,21 @@ struct QWGemmAQ {
         const qwhip_weight_view w = view->abi();
         throwIfFailed(qwhip_gemv(enc.stream, &w, x.ptr(), QWHIP_F16, 1, rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED, y16.ptr(), nullptr));
     }
+    // QWGemmAQ.encodeHeadArgmax (QWGemmAQ.swift:306-349): logits f32 [rows, n] = W . x, tokens i32 [rows] = greedy argmax (ties to
+    // the lower row); f16 activations (rotated in the kernel when asked) or f32 activations already in the basis.
+    static void encodeHeadArgmax(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& w, const QWTensorValue& x, const QWTensorValue& logits,
+                                 const QWTensorValue& tokens, int rows = 1, bool rotateInKernel = false) {
+        if (rows <= 0 || rows > 16) throw QWGemmError(QWGemmError::badShape, "head argmax takes 1..16 rows");
+        if ((x.shape.dtype != QWDType::f16 && x.shape.dtype != QWDType::f32) || x.shape.elementCount < (size_t)rows * (size_t)w.k)
+            throw QWGemmError(QWGemmError::badWeights, "head activations must be f16 or f32 [rows, k]");
+        if (logits.shape.dtype != QWDType::f32 || logits.shape.elementCount < (size_t)rows * (size_t)w.n || tokens.shape.dtype != QWDType::i32 ||
+            tokens.shape.elementCount < (size_t)rows)
+            throw QWGemmError(QWGemmError::badWeights, "head argmax: logits f32 [rows, n], tokens i32 [rows]");
+        hal.pipeline(w.containerKind.isIncumbentContainer() ? "qwg_head_gemv_q4g_argmax" : "qwg_gemv_q4g_f32_v4_am");
+        const qwhip_weight_view v = w.abi();
+        throwIfFailed(qwhip_head_argmax(enc.stream, &v, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows,
+                                        rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED, (float*)logits.ptr(), (int32_t*)tokens.ptr()));
+    }
 };
 
 // ---- QWMoEOperator.encodeResident (Sources/Operators/QWGEMM/QWMoEOperator.swift:57-442) ---------------------------
@@ -493,7 +564,7 @@ struct QWMoEOperator {
         QWTensorValue act16;       // f16 [rows * topK, intermediate]
         // prefill only (rows > 8)
         QWTensorValue expOff, sortedPair, sortedTok, invPerm, tileE, tileR, tileCount;  // i32
-        QWTensorValue gu16;        // f16 [rows * topK, 2 * intermediate]
+        QWTensorValue gu16;        // f16 [rows * topK, 2 * intermediate]; bf16 activations only (f16 rows run the fused gate_up)
         QWTensorValue dnHi;        // f32 or f16 [rows * topK, hidden]
     };
     // x: f16 hidden rows in the experts' basis; xPlain: the un-rotated rows the router reads (may equal x for a standard-basis bank).
@@ -508,12 +579,18 @@ struct QWMoEOperator {
             throw QWGemmError(QWGemmError::badShape, "moe: expert banks do not match (experts, hidden, intermediate)");
         QWGemm::encodeFnRouterGemm(enc, hal, xPlain, w.router, s.logits, rows, E, H);
         QWGemm::encodeFnMoeRoute(enc, hal, s.logits, s.idx, s.wts, rows, E, K, w.normTopK, w.routedScale);
-        const bool grouped = rows > 8 && s.expOff.base && s.gu16.base && s.dnHi.base && H % 64 == 0 && I % 64 == 0;
+        const bool fused = x.shape.dtype == QWDType::f16;   // gate_up GEMM + SwiGLU in one launch: gu16 is not needed
+        const bool grouped = rows > 8 && s.expOff.base && (fused || s.gu16.base) && s.dnHi.base && H % 64 == 0 && I % 64 == 0;
         if (grouped) {
             const int pairs = rows * K;
             QWGemm::encodeMoEGroupPairsF32(enc, hal, s.idx, s.expOff, s.sortedPair, s.sortedTok, E, pairs, K, &s.invPerm, &s.tileE, &s.tileR, &s.tileCount);
-            QWGemm::encodeMoEGroupedGemm(enc, hal, w.gateUp, E, x, &s.sortedTok, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.gu16);
-            QWGemm::encodeSiluMulSplitF16(enc, hal, s.gu16, s.act16, pairs, I, w.down.isRotated());
+            if (fused) {
+                QWGemm::encodeMoEGateUpSwiglu(enc, hal, w.gateUp, E, x, s.sortedTok, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.act16,
+                                              w.down.isRotated());
+            } else {
+                QWGemm::encodeMoEGroupedGemm(enc, hal, w.gateUp, E, x, &s.sortedTok, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.gu16);
+                QWGemm::encodeSiluMulSplitF16(enc, hal, s.gu16, s.act16, pairs, I, w.down.isRotated());
+            }
             QWGemm::encodeMoEGroupedGemm(enc, hal, w.down, E, s.act16, nullptr, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.dnHi);
             QWGemm::encodeMoEDownReduceCombineF32(enc, hal, s.dnHi, s.invPerm, s.wts, rows, K, H, shared, sharedGate, out);
         } else {
