@@ -350,7 +350,7 @@ extern "C" qwhip_status qwhip_rmsnorm(qwhip_stream_t s, const void* x_f16, const
 // Sources/QWMetal/include/qw_fastmath_safe.metalh:21-25; fold in qwg_gemv_am_fold4 / qwg_gemv_am_reduce4,
 // Sources/QWMetal/include/qw_gemm_f32_common.metalh:30-58): key hi = the float's bits made monotone (NaN -> 0, so it
 // never wins against a number), key lo = ~row, larger (hi, lo) wins: ties go to the lower row.
-// One workgroup per logits row; 16-byte loads; wave fold with DPP row steps and lane reads, then LDS across waves.
+// One workgroup per logits row; 16-byte loads, eight in flight per thread; wave fold by lane exchanges, then LDS across waves.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t qw_sortable_f32(float x) {
     const uint32_t u = __float_as_uint(x);
@@ -358,36 +358,71 @@ __device__ __forceinline__ uint32_t qw_sortable_f32(float x) {
     return (u & 0x80000000u) ? ~u : (u ^ 0x80000000u);
 }
 
+// One workgroup's vector ALU and its loads in flight bound the fold, so the sweep keeps a float maximum and its first row
+// per thread (a strict "greater" per element; NaN is never greater) and builds the 64-bit keys only to combine the 1024
+// thread results.  That is exact unless the row's maximum is a zero (+0.0 beats -0.0 in the key order, they are equal as
+// floats) or no element is greater than -inf (only -inf and NaN): those rows take the key sweep over every element.
 __global__ __launch_bounds__(1024) void qw_argmax_rows_kernel(const float* __restrict__ logits, uint32_t n, int32_t* __restrict__ tokens) {
     __shared__ unsigned long long best_w[16];
+    __shared__ uint32_t slow_path;
+    constexpr uint32_t U = 8;   // 16-byte loads in flight per thread
     const uint32_t tid = threadIdx.x;
     const float* row = logits + (uint64_t)blockIdx.x * n;
-    unsigned long long best = 0ull;   // (hi << 32) | lo; every real candidate has lo = ~row > 0 for row < 2^32 - 1
     const uint32_t n4 = (((uintptr_t)row & 15u) == 0u) ? (n & ~3u) : 0u;
-    for (uint32_t i = tid * 4u; i < n4; i += 4096u) {
-        const f4_t v = *(const f4_t*)(row + i);
+    float mx = -__builtin_inff();
+    uint32_t at = 0xFFFFFFFFu;   // no element yet
+    for (uint32_t i0 = tid * 4u; i0 < n4; i0 += U * 4096u) {
+        f4_t v[U];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const unsigned long long key = ((unsigned long long)qw_sortable_f32(v[j]) << 32) | (uint32_t)~(i + j);
-            best = key > best ? key : best;
+        for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t i = i0 + u * 4096u;
+            v[u] = *(const f4_t*)(row + (i < n4 ? i : i0));   // past the end: the batch's first chunk again (never greater)
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool gt = v[u][j] > mx;
+                mx = gt ? v[u][j] : mx;
+                at = gt ? i0 + u * 4096u + j : at;
+            }
         }
     }
     for (uint32_t i = n4 + tid; i < n; i += 1024u) {
-        const unsigned long long key = ((unsigned long long)qw_sortable_f32(row[i]) << 32) | (uint32_t)~i;
-        best = key > best ? key : best;
+        const float x = row[i];
+        const bool gt = x > mx;
+        mx = gt ? x : mx;
+        at = gt ? i : at;
     }
+    // a thread without an element (or whose elements are all -inf / NaN) offers the key of a NaN at row 0: it loses to any number
+    unsigned long long best = at == 0xFFFFFFFFu ? 0xFFFFFFFFull : (((unsigned long long)qw_sortable_f32(mx) << 32) | (uint32_t)~at);
+    auto fold = [&]() {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const unsigned long long o = __shfl_xor(best, off, 64);
-        best = o > best ? o : best;
-    }
-    if ((tid & 63u) == 0u) best_w[tid >> 6] = best;
-    __syncthreads();
-    if (tid == 0u) {
+        for (int off = 32; off > 0; off >>= 1) {
+            const unsigned long long o = __shfl_xor(best, off, 64);
+            best = o > best ? o : best;
+        }
+        if ((tid & 63u) == 0u) best_w[tid >> 6] = best;
+        __syncthreads();
+        best = best_w[0];
 #pragma unroll
         for (int w = 1; w < 16; ++w) best = best_w[w] > best ? best_w[w] : best;
-        tokens[blockIdx.x] = (int32_t)~(uint32_t)best;
+    };
+    fold();
+    const uint32_t hi = (uint32_t)(best >> 32);
+    // maximum +0.0 / -0.0 (keys 0x80000000 / 0x7FFFFFFF), or nothing above -inf (hi 0): decide over every element's key
+    if (tid == 0u) slow_path = (hi == 0x80000000u || hi == 0x7FFFFFFFu || hi == 0u) ? 1u : 0u;
+    __syncthreads();
+    if (slow_path) {
+        best = 0ull;
+        for (uint32_t i = tid; i < n; i += 1024u) {
+            const unsigned long long key = ((unsigned long long)qw_sortable_f32(row[i]) << 32) | (uint32_t)~i;
+            best = key > best ? key : best;
+        }
+        __syncthreads();   // best_w is reused
+        fold();
     }
+    if (tid == 0u) tokens[blockIdx.x] = (int32_t)~(uint32_t)best;
 }
 
 extern "C" qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens) {

@@ -326,3 +326,25 @@ def test_head_argmax_picks_the_oracles_token(dev, fmt, m):
     top2 = np.sort(ref, axis=1)[:, -2:]
     clear = (top2[:, 1] - top2[:, 0]) > 1e-2 * np.abs(top2[:, 1])
     assert np.array_equal(tok[clear], np.argmax(ref, axis=1)[clear])
+
+
+def test_argmax_rows_whose_maximum_is_a_zero_or_nothing_above_minus_infinity(dev):
+    """The rows the fast sweep cannot decide by float compares alone: maximum +-0.0 (the key order puts +0.0 above -0.0, rows in
+    either order, also split over threads), only -inf and NaN, and a long row (several chunks per thread) with a late tie."""
+    n = 70000
+    rng = np.random.default_rng(3)
+    base = -np.abs(rng.standard_normal((6, n)).astype(np.float32)) - 1.0
+    base[0, [5, 40000]] = [-0.0, 0.0]            # +0.0 wins although it comes later
+    base[1, [7, 4103]] = [0.0, -0.0]             # the same thread sees both: the earlier +0.0 wins
+    base[2, :] = -np.inf
+    base[2, 100] = np.nan                        # nothing above -inf: the first -inf
+    base[3, :] = np.nan
+    base[3, 65000] = -np.inf                     # a single number among NaNs
+    base[4, [69999, 33333]] = 7.5                # late tie: the lower row
+    base[5, [12, 13]] = [-0.0, -0.0]             # only negative zeros at the top
+    lb, tb = dev.put(base), dev.alloc(256)
+    qwhip.check(dev.lib.qwhip_argmax_f32(dev.stream.handle, lb.ptr, 6, n, tb.ptr))
+    dev.stream.sync()
+    got = tb.download(np.int32, (6,))
+    assert list(got) == [40000, 7, 0, 65000, 33333, 12]
+    assert np.array_equal(got, qo.head_argmax(base))
