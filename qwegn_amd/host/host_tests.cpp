@@ -370,6 +370,34 @@ static void test_gpu_f32_doors(QWHal& hal) {
     hal.end(enc);
 }
 
+// encodeDenseProjF32: 64 rows take the cast + matrix-core GEMM, 5 rows the f32 GEMV; both against the closed-form bank
+static void test_gpu_dense_proj_f32(QWHal& hal) {
+    const int N = 128, Kc = 128;
+    const std::vector<uint8_t> bank = cf_bank(N, Kc);
+    QWHipEncoder enc = hal.begin();
+    DeviceBuf dbank(hal, bank.size()), dx(hal, 64 * Kc * 4), dx16(hal, 64 * Kc * 2), dy(hal, 64 * N * 4);
+    upload(enc, dbank, bank.data(), bank.size());
+    const auto view = QWWeightView::make(QWTensorValue::make(dbank.p, bank.size(), QWDType::q4g), N, Kc, 4, 32, true);
+    CHECK(view.has_value());
+    for (int rows : {64, 5}) {
+        std::vector<float> x((size_t)rows * Kc);
+        for (int t = 0; t < rows; ++t)
+            for (int c = 0; c < Kc; ++c) x[(size_t)t * Kc + c] = (float)(((t * 31 + c * 7) % 29) - 14) / 16.0f;   // exact in f16
+        upload(enc, dx, x.data(), x.size() * 4);
+        const QWTensorValue xt = QWTensorValue::make(dx.p, x.size(), QWDType::f32), yt = QWTensorValue::make(dy.p, (size_t)rows * N, QWDType::f32);
+        QWGemm::encodeDenseProjF32(enc, hal, *view, xt, yt, QWTensorValue::make(dx16.p, 64 * Kc, QWDType::f16), rows);
+        std::vector<float> got((size_t)rows * N);
+        download(enc, got.data(), dy, got.size() * 4);
+        for (int t = 0; t < rows; ++t)
+            for (int n = 0; n < N; ++n) {
+                double s = 0;
+                for (int c = 0; c < Kc; ++c) s += cf_weight(n, c) * (double)x[(size_t)t * Kc + c];
+                CHECK(std::fabs((double)got[(size_t)t * N + n] - s) <= 1e-3 * std::fmax(1.0, std::fabs(s)));
+            }
+    }
+    hal.end(enc);
+}
+
 int main(int argc, char** argv) {
     const bool gpu = argc > 1 && std::strcmp(argv[1], "--gpu") == 0;
     test_plan_table();
@@ -385,6 +413,7 @@ int main(int argc, char** argv) {
         test_gpu_moe_resident(hal, 3);    // decode / verify path
         test_gpu_moe_resident(hal, 40);   // grouped prefill path (fused gate_up + SwiGLU)
         test_gpu_f32_doors(hal);
+        test_gpu_dense_proj_f32(hal);
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed ? 1 : 0;

@@ -365,6 +365,30 @@ struct QWGemm {
         throwIfFailed(qwhip_gemv_f32(enc.stream, &v, (const float*)x.ptr(), (uint32_t)rows, epi, scale, (float*)y.ptr()));
     }
 
+    // QWGemm.encodeDenseProjF32 (QWGemmF32.swift:413-440): the unified dense projection over `rows` f32 activations in the
+    // container's basis.  rows >= minNaxRows with no epilogue: cast to f16 in `naxX16` (rows * k halves, or the caller's
+    // `x16Precast`) and run the matrix-core GEMM into the f32 output; otherwise the f32 GEMV family (its batched form for
+    // 32 rows and more is the same four-rows-per-pass kernel here).
+    static void encodeDenseProjF32(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& w, const QWTensorValue& x, const QWTensorValue& y,
+                                   const QWTensorValue& naxX16, int rows, uint32_t epi = 0, float scale = 1.0f,
+                                   const QWTensorValue* x16Precast = nullptr, int minNaxRows = 64) {
+        const int effectiveMinNax = minNaxRows > 64 ? minNaxRows : 64;
+        if (rows >= effectiveMinNax && epi == 0 && scale == 1.0f && w.n % 64 == 0 && w.k % 64 == 0 && w.bits() != 2 && w.bits() != 3 &&
+            w.bits() != 6) {
+            const size_t count = (size_t)rows * (size_t)w.k;
+            if (x16Precast) {
+                gemmBatchedH16(enc, hal, x16Precast->slice(0, count, QWDType::f16), w, y, rows);
+            } else {
+                if (naxX16.shape.elementCount < count) throw QWGemmError(QWGemmError::badWeights, "dense proj: the f16 staging buffer is short");
+                const QWTensorValue xHi = naxX16.slice(0, count, QWDType::f16);
+                encodeCast(enc, hal, x, xHi, count);
+                gemmBatchedH16(enc, hal, xHi, w, y, rows);
+            }
+        } else {
+            encodeHQ4F32V4(enc, hal, w, x, y, rows, epi, scale);
+        }
+    }
+
     // QWGemm.encodeH32F32 (QWGemmF32.swift:46-54): out f32 [rows, hidden] = rotate(x) in the normalised Walsh-Hadamard domain.
     static void encodeH32F32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWTensorValue& out, int rows, int hidden) {
         if (x.shape.dtype != QWDType::f32 || out.shape.dtype != QWDType::f32 || rows <= 0 || hidden <= 0 || hidden % 32 != 0 ||
