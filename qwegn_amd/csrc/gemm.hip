@@ -531,8 +531,17 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     uint32_t m0, n0, rows_valid;
     const uint8_t* bank = p.bank;
     if constexpr (GROUPED) {
-        const uint32_t t = blockIdx.y;
-        if ((int32_t)t >= p.tile_count[0]) return;
+        // One-dimensional grid, XCD-aware: workgroup L runs on XCD L % 8 (round-robin dispatch), and each XCD takes one
+        // contiguous eighth of the tile list (the list is sorted by expert), walking (tile, column tile) with the column
+        // fastest.  The row tiles of an expert and the column tiles of a row tile then run side by side under one L2: an
+        // expert's weights and a tile's gathered rows are fetched once instead of once per XCD that happens to use them.
+        const uint32_t ncol = p.tiles_n;
+        const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+        const uint32_t tc = (uint32_t)max(p.tile_count[0], 0);
+        const uint32_t per_xcd = (tc + 7u) >> 3;
+        const uint32_t ti = slot / ncol, col = slot - ti * ncol;
+        const uint32_t t = xcd * per_xcd + ti;
+        if (ti >= per_xcd || t >= tc) return;
         const uint32_t e = (uint32_t)p.tile_e[t];
         const uint32_t packed = (uint32_t)p.tile_r[t];
         const uint32_t code = packed >> 24;
@@ -541,7 +550,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
         const uint32_t end = (uint32_t)p.expert_off[e + 1];
         m0 = start;
         rows_valid = min((uint32_t)BM, min(bm, end - start));
-        n0 = blockIdx.x * (SWIGLU ? BN / 2 : BN);
+        n0 = col * (SWIGLU ? BN / 2 : BN);
         bank += (uint64_t)e * p.rows_per_expert * p.row_bytes;
     } else {
         const uint32_t total = p.tiles_m * p.tiles_n;
@@ -1105,9 +1114,12 @@ hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid,
         // ping-pong kernel on the 64 x 256 tiles: 8 waves, one of each group per SIMD, so one dequantizes while the other
         // multiplies (measured on T = 2048, E = 128, top-8: gate_up 257 -> 221 us; pairing two list entries of an expert
         // into a 128-row tile, or loading two K-steps ahead, measured no faster)
-        if (ydt == QWHIP_F16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F16, true>(st, p, grid);
-        if (ydt == QWHIP_BF16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_BF16, true>(st, p, grid);
-        return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F32, true>(st, p, grid);
+        qw_gemm_params q = p;
+        q.tiles_n = grid.x;
+        const dim3 grid1(8u * qwhip_cdiv(grid.y, 8u) * grid.x);   // XCD-aware one-dimensional grid over (tile, column tile)
+        if (ydt == QWHIP_F16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F16, true>(st, q, grid1);
+        if (ydt == QWHIP_BF16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_BF16, true>(st, q, grid1);
+        return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F32, true>(st, q, grid1);
     }
     if (xdt == QWHIP_F16) {  // DMA-fed pipelined kernel, 64 x 256 tiles
         if (ydt == QWHIP_F16) return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F16, true>(st, p, grid);
@@ -1213,7 +1225,8 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     p.rows_per_expert = rows_per_expert;
     p.inter = inter;
     p.rotate_act = rotate_act ? 1u : 0u;
-    const dim3 grid(qwhip_cdiv(inter, 128u), max_tiles);
+    p.tiles_n = qwhip_cdiv(inter, 128u);
+    const dim3 grid(8u * qwhip_cdiv(max_tiles, 8u) * p.tiles_n);   // XCD-aware one-dimensional grid over (tile, column tile)
     hipError_t e;
     if (fmt == QG_FMT_M5) e = launch_cfg3<1, 2, 2, 4, QG_FMT_M5, QWHIP_F16, true, true>(s->stream, p, grid);
     else if (fmt == QG_FMT_B4) e = launch_cfg3<1, 2, 2, 4, QG_FMT_B4, QWHIP_F16, true, true>(s->stream, p, grid);
