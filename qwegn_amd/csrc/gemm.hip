@@ -505,16 +505,9 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 #define QG3_BAR_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define QG3_BAR_ALL() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
-// SWIGLU (grouped, 64 x 256 tiles, f16 out): a tile's 256 weight rows are 128 gate rows and the 128 up rows of the same
-// outputs, laid out so that each wave's two fragments are (gate, up) of the same 32 outputs: tile column 64 w + 32 b + j is
-// expert row b * inter + 128 * blockIdx.x + 32 w + j.  The epilogue rounds both accumulators to f16 (the values the
-// unfused chain stores), applies SwiGLU and the FWHT-32 in fp32 and stores act f16 [pair, inter]: the arithmetic of
-// qwhip_swiglu_fwht on the f16 gate|up matrix, without writing it (the reference's fused form for its dense path:
-// qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167).
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED, bool SWIGLU = false>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED>
 __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_params p) {
     static_assert(WVM * WVN == 8, "two groups of four waves");
-    static_assert(!SWIGLU || (GROUPED && WM == 1 && WN == 2 && WVN == 4 && YDT == QWHIP_F16), "fused SwiGLU: grouped 64 x 256 tiles, f16 out");
     constexpr int NT = WVM * WVN * 64;
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 64;
     constexpr int B_ITEMS = BN * 2;
@@ -550,7 +543,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
         const uint32_t end = (uint32_t)p.expert_off[e + 1];
         m0 = start;
         rows_valid = min((uint32_t)BM, min(bm, end - start));
-        n0 = col * (SWIGLU ? BN / 2 : BN);
+        n0 = col * BN;
         bank += (uint64_t)e * p.rows_per_expert * p.row_bytes;
     } else {
         const uint32_t total = p.tiles_m * p.tiles_n;
@@ -596,18 +589,12 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     // the tile are done redundantly by several threads: identical bytes to the same slot) ----
     static_assert(B_ITEMS >= NT && B_ITEMS <= NT + NT / 2, "the second weight items are covered by group 0 alone");
     uint32_t b_off32[B_PER], b_meta[B_PER];   // byte offset of the row inside the tile's bank rows; LDS row offset | swizzle key << 16 | slice << 20
-    const uint8_t* b_tile = bank + (SWIGLU ? 0ull : (uint64_t)n0 * p.row_bytes);
+    const uint8_t* b_tile = bank + (uint64_t)n0 * p.row_bytes;
 #pragma unroll
     for (int i = 0; i < B_PER; ++i) {
         const uint32_t it = i == 0 ? tid : NT + (B_ITEMS > NT ? tid % (uint32_t)(B_ITEMS > NT ? B_ITEMS - NT : 1) : 0u);
         const uint32_t nl = it >> 1;
-        uint32_t n;
-        if constexpr (SWIGLU) {
-            // n0 counts act columns here and b_tile is the expert's first row
-            n = ((nl & 32u) ? p.inter : 0u) + min(n0 + 32u * (nl >> 6) + (nl & 31u), p.inter - 1u);
-        } else {
-            n = min(n0 + nl, p.N - 1u) - n0;
-        }
+        const uint32_t n = min(n0 + nl, p.N - 1u) - n0;
         b_off32[i] = n * (uint32_t)p.row_bytes;                     // a tile's rows span < 4 GiB
         b_meta[i] = (nl * 128u) | (((nl >> 1) & 7u) << 16) | ((it & 1u) << 20);
     }
@@ -791,38 +778,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    if constexpr (SWIGLU) {
-        // lane (lane & 31) holds output column c = n0 + 32 wn + (lane & 31) of 16 rows: gate in acc[0][0], up in acc[0][1]
-        constexpr uint32_t EP_PITCH = 64 + 16;
-        __syncthreads();
-        uint8_t* ep = lds2 + wave * (32u * EP_PITCH);
-        const uint32_t j = lane & 31u;
-        const uint32_t w_off = (4u * (lane >> 5)) * EP_PITCH + j * 2u;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float g = (float)(h1_t)acc[0][0][r], u = (float)(h1_t)acc[0][1][r];
-            float v = qw_swiglu(g, u);
-            if (p.rotate_act) {
-#pragma unroll
-                for (uint32_t h = 1; h < 32u; h <<= 1) {
-                    const float o = __shfl_xor(v, (int)h, 32);
-                    v = (j & h) == 0u ? v + o : o - v;
-                }
-                v *= QW_INV_SQRT32;
-            }
-            *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
-        }
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const uint32_t c = q * 64u + lane;
-            const uint32_t row = c >> 2, cc = c & 3u;
-            const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
-            const uint32_t grow = wm * 32u + row;
-            const uint32_t n = n0 + wn * 32u + cc * 8u;
-            if (grow < rows_valid && n < p.inter)
-                *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
-        }
-    } else if constexpr (YDT != QWHIP_F32) {
+    if constexpr (YDT != QWHIP_F32) {
         // 2-byte outputs: each wave transposes its 32-row slabs through a private LDS region (the operand stages are
         // dead by now) and stores 16-byte row chunks; a lane's accumulators are one column of 16 rows, and 2-byte
         // stores from that layout cost one address per element. The host side guarantees 16-byte aligned output rows.
@@ -883,6 +839,218 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 }
 
 // ------------------------------------------------------------------------------------------------
+// Grouped kernel with the weights fed straight into the matrix cores' operand registers (f16 activations, 4 waves,
+// 64 x 256 tiles of the sorted pair list).  With 64-row tiles the LDS-staged kernels above spend most of their LDS
+// bandwidth on weights (written once as f16, read back by both row halves).  Here wave w owns tile columns
+// [64 w, 64 w + 64) for all 64 rows (2 x 2 fragments of v_mfma_f32_32x32x16_f16): lane (n = lane & 31, h = lane >> 5)
+// loads the 32-column slice 2 kt + h of weight row n of each of its two column fragments - one block per lane and
+// fragment, the same loads the staged kernels issue - and dequantizes chunk ks of it (8 columns, exact f16 weights) as
+// the second operand of sub-step ks.  The K order inside a K-step is thereby permuted (sub-step ks contracts columns
+// 32 h + 8 ks .. + 7); the activation fragments are read from LDS in the same order (16-byte chunk 4 h + ks of the
+// row), so only the 64 x 64 activation tile goes through LDS: 8 KB written and 32 KB read per K-step instead of
+// 40 KB and 96 KB.  Two LDS stages, one barrier per K-step; blocks and activations travel global -> registers two
+// K-steps ahead (a K-step is short here: one step of distance left the waves waiting on memory).
+// Grid: one-dimensional and XCD-aware - workgroup L runs on XCD L % 8 (round-robin dispatch), each XCD takes one contiguous
+// eighth of the expert-sorted tile list and walks (tile, column tile) column-fastest, so the row tiles of an expert and
+// the column tiles of a row tile run side by side under one L2.
+// SWIGLU (f16 out): a tile's 256 weight rows are 128 gate rows and the 128 up rows of the same outputs, ordered so that a
+// wave's two column fragments are (gate, up) of the same 32 outputs: fragment b, column j of wave w is expert row
+// b * inter + 128 * column tile + 32 w + j.  The epilogue rounds both accumulators to f16 (the values the two-step chain
+// stores), applies SwiGLU and the FWHT-32 (five lane exchanges) in fp32 and stores act f16 [pair, inter]: the arithmetic of
+// qwhip_swiglu_fwht on the f16 gate|up matrix without writing it (the reference's fused form for its dense path:
+// qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167).
+// ------------------------------------------------------------------------------------------------
+template <int FMT, int YDT, bool SWIGLU>
+__global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
+    static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
+    constexpr uint32_t BM = 64, BN = 256, STAGE = BM * 128u;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds4[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u;
+
+    const uint32_t ncol = p.tiles_n;
+    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const uint32_t tc = (uint32_t)max(p.tile_count[0], 0);
+    const uint32_t per_xcd = (tc + 7u) >> 3;
+    const uint32_t ti = slot / ncol, col = slot - ti * ncol;
+    const uint32_t t = xcd * per_xcd + ti;
+    if (ti >= per_xcd || t >= tc) return;
+    const uint32_t e = (uint32_t)p.tile_e[t];
+    const uint32_t packed = (uint32_t)p.tile_r[t];
+    const uint32_t code = packed >> 24;
+    const uint32_t bm = code == 1u ? 16u : (code == 2u ? 32u : 64u);
+    const uint32_t m0 = (uint32_t)p.expert_off[e] + (packed & 0xFFFFFFu) * bm;
+    const uint32_t rows_valid = min(BM, min(bm, (uint32_t)p.expert_off[e + 1] - m0));
+    const uint32_t n0 = col * (SWIGLU ? BN / 2 : BN);
+    const uint8_t* bank = p.bank + (uint64_t)e * p.rows_per_expert * p.row_bytes;
+
+    // activation tile: chunk (row = (tid >> 3) + 32 i, 16-byte k-chunk tid & 7) -> LDS slot k-chunk ^ ((row >> 1) & 7)
+    uint32_t a_voff[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t row = (tid >> 3) + 32u * i;
+        const uint32_t r = row < rows_valid ? row : rows_valid - 1u;
+        const uint32_t src_row = p.gather ? (uint32_t)p.gather[m0 + r] : m0 + r;
+        a_voff[i] = src_row * p.ldx * 2u + (tid & 7u) * 16u;    // activations < 4 GiB (checked by the launcher)
+    }
+    const uint32_t a_lds0 = (tid >> 3) * 128u + (((tid & 7u) ^ ((tid >> 4) & 7u)) << 4);   // + i * 4096 (swizzle key unchanged)
+
+    // this lane's weight rows (one per column fragment) and K half
+    const uint32_t j = lane & 31u, kh = lane >> 5;
+    const uint8_t* b_row[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        uint32_t n;
+        if constexpr (SWIGLU) n = (b ? p.inter : 0u) + min(n0 + 32u * wave + j, p.inter - 1u);
+        else n = min(n0 + 64u * wave + 32u * b + j, p.N - 1u);
+        b_row[b] = bank + (uint64_t)n * p.row_bytes;
+    }
+    // fragment reads: row j (+ 32 a), logical chunk 4 kh + ks -> byte ((4 kh + ks) ^ key) * 16, key = (row >> 1) & 7 (same for a = 0, 1)
+    const uint32_t fr_key = (j >> 1) & 7u;
+    const uint32_t a_rd = j * 128u;
+
+    f16_t acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    const uint32_t nk = p.K / 64u;
+
+    auto load_a = [&](uint32_t kt, u4_t* a_reg) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
+    };
+    auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *(u4_t*)(lds4 + stage * STAGE + a_lds0 + i * 4096u) = a_reg[i];
+    };
+    auto load_b = [&](uint32_t kt, qg_slice<FMT>* blk) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) qg_load_slice<FMT>(b_row[b], kt * 2u + kh, p.gshift, p.bb, blk[b]);
+    };
+    auto mfma_step = [&](const uint8_t* st, const qg_slice<FMT>* blk) {
+        const h2_t s0 = qw_splat_lo(blk[0].hdr), c0 = qw_splat_hi(blk[0].hdr);
+        const h2_t s1 = qw_splat_lo(blk[1].hdr), c1 = qw_splat_hi(blk[1].hdr);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint32_t off = a_rd + (((4u * kh + (uint32_t)ks) ^ fr_key) << 4);
+            const h8_t a0 = *(const h8_t*)(st + off), a1 = *(const h8_t*)(st + off + 4096u);
+            const h8_t w0 = qg_dequant_chunk<FMT>(blk[0], ks, s0, c0, magic);
+            const h8_t w1 = qg_dequant_chunk<FMT>(blk[1], ks, s1, c1, magic);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, w0, acc[0][0], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, w0, acc[1][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, w1, acc[0][1], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, w1, acc[1][1], 0, 0, 0);
+        }
+    };
+
+    // Register pipeline two K-steps deep: at step kt the blocks of kt are contracted, those of kt + 1 are in flight or
+    // landed, those of kt + 2 are issued; the activation chunks of kt + 1 (issued a step ago) go to LDS at the end of the
+    // step and those of kt + 2 are issued at its start.  Six steps per trip keep every buffer index a constant.
+    const uint32_t last = nk - 1u;
+    qg_slice<FMT> blk[3][2];
+    u4_t a_reg[2][2];
+    load_a(0, a_reg[0]);
+    load_b(0, blk[0]);
+    load_a(min(1u, last), a_reg[1]);
+    load_b(min(1u, last), blk[1]);
+    store_a(0, a_reg[0]);
+    __syncthreads();
+    for (uint32_t kt0 = 0; kt0 < nk; kt0 += 6u) {
+#pragma unroll
+        for (int u = 0; u < 6; ++u) {
+            const uint32_t kt = kt0 + (uint32_t)u;
+            if (kt >= nk) break;
+            load_a(min(kt + 2u, last), a_reg[u & 1]);
+            load_b(min(kt + 2u, last), blk[(u + 2) % 3]);
+            mfma_step(lds4 + (uint32_t)(u & 1) * STAGE, blk[u % 3]);
+            store_a((uint32_t)((u + 1) & 1), a_reg[(u + 1) & 1]);
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: per wave, rows 32 a .. + 31 through a private LDS slab, 16-byte row chunks out ----
+    if constexpr (SWIGLU) {
+        constexpr uint32_t EP_PITCH = 64 + 16;
+        __syncthreads();
+        uint8_t* ep = lds4 + wave * (32u * EP_PITCH);
+        const uint32_t w_off = (4u * kh) * EP_PITCH + j * 2u;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float g = (float)(h1_t)acc[a][0][r], u = (float)(h1_t)acc[a][1][r];
+                float v = qw_swiglu(g, u);
+                if (p.rotate_act) {
+#pragma unroll
+                    for (uint32_t h = 1; h < 32u; h <<= 1) {
+                        const float o = __shfl_xor(v, (int)h, 32);
+                        v = (j & h) == 0u ? v + o : o - v;
+                    }
+                    v *= QW_INV_SQRT32;
+                }
+                *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
+            }
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const uint32_t c = q * 64u + lane;
+                const uint32_t row = c >> 2, cc = c & 3u;
+                const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
+                const uint32_t grow = 32u * a + row;
+                const uint32_t n = n0 + wave * 32u + cc * 8u;
+                if (grow < rows_valid && n < p.inter)
+                    *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+            }
+        }
+    } else if constexpr (YDT != QWHIP_F32) {
+        constexpr uint32_t EP_PITCH = 2 * 64 + 16;
+        __syncthreads();
+        uint8_t* ep = lds4 + wave * (32u * EP_PITCH);
+        const uint32_t w_off = (4u * kh) * EP_PITCH + j * 2u;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t o = w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH + b * 64u;
+                    if constexpr (YDT == QWHIP_BF16) *(uint16_t*)(ep + o) = qw_f32_to_bf16(acc[a][b][r]);
+                    else *(h1_t*)(ep + o) = (h1_t)acc[a][b][r];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t c = q * 64u + lane;
+                const uint32_t row = c >> 3, cc = c & 7u;
+                const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
+                const uint32_t grow = 32u * a + row;
+                const uint32_t n = n0 + wave * 64u + cc * 8u;
+                if (grow < rows_valid && n < p.N)
+                    *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const uint32_t n = n0 + wave * 64u + 32u * b + j;
+                if (n < p.N) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t row = 32u * a + 8 * (r >> 2) + 4 * kh + (r & 3);
+                        if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -923,11 +1091,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED = false, bool SWIGLU = false>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED = false>
 hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED, SWIGLU>;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -935,6 +1103,15 @@ hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
         attr_done = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(WVM * WVN * 64), lds, st, p);
+    return hipGetLastError();
+}
+
+template <int FMT, int YDT, bool SWIGLU>
+hipError_t launch_cfg4(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
+    // two activation stages, or the four epilogue slabs (32 rows x (128 + 16) bytes each) when they are larger
+    constexpr size_t lds = 4u * 32u * 144u;
+    static_assert(lds >= 2u * 64u * 128u, "the stages fit the slab allocation");
+    hipLaunchKernelGGL((qw_gemm4_kernel<FMT, YDT, SWIGLU>), grid, dim3(256), lds, st, p);
     return hipGetLastError();
 }
 
@@ -1111,15 +1288,15 @@ hipError_t launch_grouped_y(hipStream_t st, const qw_gemm_params& p, dim3 grid, 
 template <int FMT>
 hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid, uint32_t xdt, uint32_t ydt) {
     if (xdt == QWHIP_F16 && !p.force_gemm2 && (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0))) {
-        // ping-pong kernel on the 64 x 256 tiles: 8 waves, one of each group per SIMD, so one dequantizes while the other
-        // multiplies (measured on T = 2048, E = 128, top-8: gate_up 257 -> 221 us; pairing two list entries of an expert
-        // into a 128-row tile, or loading two K-steps ahead, measured no faster)
+        // direct-operand kernel on the 64 x 256 tiles (weights dequantized straight into MFMA operand registers, only the
+        // activation tile in LDS); it measured level with the 8-wave ping-pong kernel it replaced (gate_up 211 vs 215 us
+        // on T = 2048, E = 128, top-8) at a quarter of the LDS traffic
         qw_gemm_params q = p;
         q.tiles_n = grid.x;
         const dim3 grid1(8u * qwhip_cdiv(grid.y, 8u) * grid.x);   // XCD-aware one-dimensional grid over (tile, column tile)
-        if (ydt == QWHIP_F16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F16, true>(st, q, grid1);
-        if (ydt == QWHIP_BF16) return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_BF16, true>(st, q, grid1);
-        return launch_cfg3<1, 2, 2, 4, FMT, QWHIP_F32, true>(st, q, grid1);
+        if (ydt == QWHIP_F16) return launch_cfg4<FMT, QWHIP_F16, false>(st, q, grid1);
+        if (ydt == QWHIP_BF16) return launch_cfg4<FMT, QWHIP_BF16, false>(st, q, grid1);
+        return launch_cfg4<FMT, QWHIP_F32, false>(st, q, grid1);
     }
     if (xdt == QWHIP_F16) {  // DMA-fed pipelined kernel, 64 x 256 tiles
         if (ydt == QWHIP_F16) return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F16, true>(st, p, grid);
@@ -1152,6 +1329,8 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_wei
     if (ldy == 0) ldy = rows_per_expert;
     if (ldx < w->k || ldy < rows_per_expert || (ldx % 8) != 0)
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions ldx=%u ldy=%u", ldx, ldy);
+    if ((uint64_t)pairs * ldx * 2u >= (1ull << 32))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "grouped GEMM addresses its activation rows with 32-bit offsets: %u rows of %u do not fit", pairs, ldx);
     qw_gemm_params p = {};
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
@@ -1205,6 +1384,8 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     if (ldact == 0) ldact = inter;
     if (ldx < w->k || ldact < inter || (ldx % 8) != 0 || (ldact % 8) != 0 || ((uintptr_t)act_f16 & 15u) != 0)
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions or alignment (ldx=%u ldact=%u, act 16-byte aligned)", ldx, ldact);
+    if ((uint64_t)pairs * ldx * 2u >= (1ull << 32))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "grouped GEMM addresses its activation rows with 32-bit offsets: %u rows of %u do not fit", pairs, ldx);
     qw_gemm_params p = {};
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
@@ -1228,9 +1409,9 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     p.tiles_n = qwhip_cdiv(inter, 128u);
     const dim3 grid(8u * qwhip_cdiv(max_tiles, 8u) * p.tiles_n);   // XCD-aware one-dimensional grid over (tile, column tile)
     hipError_t e;
-    if (fmt == QG_FMT_M5) e = launch_cfg3<1, 2, 2, 4, QG_FMT_M5, QWHIP_F16, true, true>(s->stream, p, grid);
-    else if (fmt == QG_FMT_B4) e = launch_cfg3<1, 2, 2, 4, QG_FMT_B4, QWHIP_F16, true, true>(s->stream, p, grid);
-    else e = launch_cfg3<1, 2, 2, 4, QG_FMT_B8, QWHIP_F16, true, true>(s->stream, p, grid);
+    if (fmt == QG_FMT_M5) e = launch_cfg4<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid);
+    else if (fmt == QG_FMT_B4) e = launch_cfg4<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
+    else e = launch_cfg4<QG_FMT_B8, QWHIP_F16, true>(s->stream, p, grid);
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
 }
