@@ -505,7 +505,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 #define QG3_BAR_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define QG3_BAR_ALL() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT>
 __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_params p) {
     static_assert(WVM * WVN == 8, "two groups of four waves");
     constexpr int NT = WVM * WVN * 64;
@@ -523,65 +523,30 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 
     uint32_t m0, n0, rows_valid;
     const uint8_t* bank = p.bank;
-    if constexpr (GROUPED) {
-        // One-dimensional grid, XCD-aware: workgroup L runs on XCD L % 8 (round-robin dispatch), and each XCD takes one
-        // contiguous eighth of the tile list (the list is sorted by expert), walking (tile, column tile) with the column
-        // fastest.  The row tiles of an expert and the column tiles of a row tile then run side by side under one L2: an
-        // expert's weights and a tile's gathered rows are fetched once instead of once per XCD that happens to use them.
-        const uint32_t ncol = p.tiles_n;
-        const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-        const uint32_t tc = (uint32_t)max(p.tile_count[0], 0);
-        const uint32_t per_xcd = (tc + 7u) >> 3;
-        const uint32_t ti = slot / ncol, col = slot - ti * ncol;
-        const uint32_t t = xcd * per_xcd + ti;
-        if (ti >= per_xcd || t >= tc) return;
-        const uint32_t e = (uint32_t)p.tile_e[t];
-        const uint32_t packed = (uint32_t)p.tile_r[t];
-        const uint32_t code = packed >> 24;
-        const uint32_t bm = code == 1u ? 16u : (code == 2u ? 32u : 64u);
-        const uint32_t start = (uint32_t)p.expert_off[e] + (packed & 0xFFFFFFu) * bm;
-        const uint32_t end = (uint32_t)p.expert_off[e + 1];
-        m0 = start;
-        rows_valid = min((uint32_t)BM, min(bm, end - start));
-        n0 = col * BN;
-        bank += (uint64_t)e * p.rows_per_expert * p.row_bytes;
-    } else {
-        const uint32_t total = p.tiles_m * p.tiles_n;
-        const uint32_t per_xcd = (total + 7u) / 8u;
-        const uint32_t label = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-        if (label >= total) return;
-        constexpr uint32_t G = 4;
-        const uint32_t band = label / (G * p.tiles_n);
-        const uint32_t band_rows = min(G, p.tiles_m - band * G);
-        const uint32_t in_band = label - band * G * p.tiles_n;
-        const uint32_t tm = band * G + in_band % band_rows;
-        const uint32_t tn = in_band / band_rows;
-        m0 = tm * BM;
-        n0 = tn * BN;
-        rows_valid = min((uint32_t)BM, p.M - m0);
-    }
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const uint32_t per_xcd = (total + 7u) / 8u;
+    const uint32_t label = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if (label >= total) return;
+    constexpr uint32_t G = 4;
+    const uint32_t band = label / (G * p.tiles_n);
+    const uint32_t band_rows = min(G, p.tiles_m - band * G);
+    const uint32_t in_band = label - band * G * p.tiles_n;
+    const uint32_t tm = band * G + in_band % band_rows;
+    const uint32_t tn = in_band / band_rows;
+    m0 = tm * BM;
+    n0 = tn * BN;
+    rows_valid = min((uint32_t)BM, p.M - m0);
 
     // ---- activation tile: chunk c = tid + i * NT -> tile row (tid >> 3) + (NT / 8) * i, 16-byte k-chunk tid & 7.
     // Global -> registers one K-step ahead (coalesced 128-byte rows), registers -> LDS slot (k-chunk ^ ((row >> 1) & 7)).
-    // Dense: one per-thread offset, the row block (NT / 8 rows) is a wave-uniform term; blocks past the tile's rows
+    // One per-thread offset, the row block (NT / 8 rows) is a wave-uniform term; blocks past the tile's rows
     // re-read block 0 (their outputs are never stored), so M must be a multiple of NT / 8 = 64.
     constexpr int A_LD = BM * 8 / NT;
     static_assert((BM * 8) % NT == 0, "activation tile must split evenly over the workgroup");
     constexpr uint32_t A_BLK = NT / 8;
-    uint32_t a_voff[GROUPED ? A_LD : 1];
     const uint32_t a_lds0 = (tid >> 3) * 128u + (((tid & 7u) ^ ((tid >> 4) & 7u)) << 4);   // + i * A_BLK * 128 (swizzle key unchanged)
-    if constexpr (GROUPED) {
-#pragma unroll
-        for (int i = 0; i < A_LD; ++i) {
-            const uint32_t row = (tid >> 3) + A_BLK * i;
-            const uint32_t r = row < rows_valid ? row : rows_valid - 1;
-            const uint32_t src_row = p.gather ? (uint32_t)p.gather[m0 + r] : m0 + r;
-            a_voff[i] = src_row * p.ldx * 2u + (tid & 7u) * 16u;    // activations < 4 GiB (checked by the launcher)
-        }
-    } else {
-        a_voff[0] = (tid >> 3) * p.ldx * 2u + (tid & 7u) * 16u;
-    }
-    const uint64_t a_tile_base = GROUPED ? 0ull : (uint64_t)m0 * p.ldx * 2u;
+    const uint32_t a_voff = (tid >> 3) * p.ldx * 2u + (tid & 7u) * 16u;
+    const uint64_t a_tile_base = (uint64_t)m0 * p.ldx * 2u;
     const uint64_t a_blk_stride = (uint64_t)A_BLK * p.ldx * 2u;
     const uint32_t a_blocks = rows_valid / A_BLK;
 
@@ -613,12 +578,8 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     auto load_a = [&](uint32_t kt, u4_t* a_reg) {
 #pragma unroll
         for (int i = 0; i < A_LD; ++i) {
-            if constexpr (GROUPED) {
-                a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
-            } else {
-                const uint32_t blk = (uint32_t)i < a_blocks ? (uint32_t)i : 0u;
-                a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + blk * a_blk_stride + (uint64_t)kt * 128u + a_voff[0]);
-            }
+            const uint32_t blk = (uint32_t)i < a_blocks ? (uint32_t)i : 0u;
+            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + blk * a_blk_stride + (uint64_t)kt * 128u + a_voff);
         }
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
@@ -1091,11 +1052,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool GROUPED = false>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT>
 hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED>;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
