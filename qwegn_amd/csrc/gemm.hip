@@ -1012,6 +1012,234 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// The direct-operand grouped kernel with the bank read the way memory likes it (HQ4_G32_M5, K % 128 == 0, bank 16-byte
+// aligned).  In qw_gemm4_kernel every lane fetches its own 20-byte block: 64 runs of the bank per load instruction, at
+// 4-byte alignment - the address unit is what bounds it.  Here the 256 weight rows of a tile are copied raw, 128 columns
+// (four blocks = 80 bytes per row) at a time: consecutive threads copy consecutive 16-byte chunks of a row (five per row),
+// global -> registers -> LDS, the LDS image being the same bytes in the same order; each lane then reads its block
+// (five dwords) from the image for the K-step at hand and dequantizes it into the MFMA operand as before.  Per K-step
+// that is 2.5 coalesced load instructions per wave instead of four scattered ones.
+// LDS: two activation stages (8 KB each) and one raw stage (256 rows at a pitch of 88 bytes, 22 KB): 38 KB per workgroup,
+// four workgroups per CU.  The raw image of K pair kp + 1 is in flight (registers) during K pair kp and replaces the
+// stage between two barriers at its end.
+// ------------------------------------------------------------------------------------------------
+template <int YDT, bool SWIGLU>
+__global__ __launch_bounds__(256) void qw_gemm5_kernel(const qw_gemm_params p) {
+    static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
+    constexpr int FMT = QG_FMT_M5;
+    // raw image: row pitch 88 bytes (22 dwords: the 64 lanes of a block read fall on 64 different banks), one stage
+    constexpr uint32_t BM = 64, BN = 256, A_STAGE = BM * 128u, RAW_PITCH = 88u, RAW_OFF = 2u * A_STAGE;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds5[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u;
+
+    const uint32_t ncol = p.tiles_n;
+    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const uint32_t tc = (uint32_t)max(p.tile_count[0], 0);
+    const uint32_t per_xcd = (tc + 7u) >> 3;
+    const uint32_t ti = slot / ncol, col = slot - ti * ncol;
+    const uint32_t t = xcd * per_xcd + ti;
+    if (ti >= per_xcd || t >= tc) return;
+    const uint32_t e = (uint32_t)p.tile_e[t];
+    const uint32_t packed = (uint32_t)p.tile_r[t];
+    const uint32_t code = packed >> 24;
+    const uint32_t bm = code == 1u ? 16u : (code == 2u ? 32u : 64u);
+    const uint32_t m0 = (uint32_t)p.expert_off[e] + (packed & 0xFFFFFFu) * bm;
+    const uint32_t rows_valid = min(BM, min(bm, (uint32_t)p.expert_off[e + 1] - m0));
+    const uint32_t n0 = col * (SWIGLU ? BN / 2 : BN);
+    const uint8_t* bank = p.bank + (uint64_t)e * p.rows_per_expert * p.row_bytes;
+
+    // activation tile: chunk (row = (tid >> 3) + 32 i, 16-byte k-chunk tid & 7) -> LDS slot k-chunk ^ ((row >> 1) & 7)
+    uint32_t a_voff[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t row = (tid >> 3) + 32u * i;
+        const uint32_t r = row < rows_valid ? row : rows_valid - 1u;
+        const uint32_t src_row = p.gather ? (uint32_t)p.gather[m0 + r] : m0 + r;
+        a_voff[i] = src_row * p.ldx * 2u + (tid & 7u) * 16u;    // activations < 4 GiB (checked by the launcher)
+    }
+    const uint32_t a_lds0 = (tid >> 3) * 128u + (((tid & 7u) ^ ((tid >> 4) & 7u)) << 4);   // + i * 4096 (swizzle key unchanged)
+
+    // tile row nl (0..255) = 64 wave + 32 fragment + column -> weight row of the expert
+    auto bank_row = [&](uint32_t nl) -> uint32_t {
+        const uint32_t w = nl >> 6, b = (nl >> 5) & 1u, jj = nl & 31u;
+        if constexpr (SWIGLU) return (b ? p.inter : 0u) + min(n0 + 32u * w + jj, p.inter - 1u);
+        else return min(n0 + 64u * w + 32u * b + jj, p.N - 1u);
+    };
+    // raw copy role: 16-byte chunk q = tid + 256 i of the tile's 256 x 80-byte K-pair image
+    uint32_t raw_goff[5], raw_loff[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+        const uint32_t q = tid + 256u * i, nl = q / 5u, c = q - 5u * nl;
+        raw_goff[i] = bank_row(nl) * (uint32_t)p.row_bytes + c * 16u;     // an expert's rows span < 4 GiB
+        raw_loff[i] = RAW_OFF + nl * RAW_PITCH + c * 16u;                 // 8-byte aligned
+    }
+    // contraction role: lane (j, kh) reads block 2 s + kh of tile rows 64 wave + 32 b + j in K-step s of the pair
+    const uint32_t j = lane & 31u, kh = lane >> 5;
+    const uint32_t rd0 = RAW_OFF + (64u * wave + j) * RAW_PITCH + kh * 20u;   // + 32 rows for the second fragment
+    const uint32_t fr_key = (j >> 1) & 7u;
+    const uint32_t a_rd = j * 128u;
+
+    f16_t acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+    const uint32_t magic = qw_vgpr_const(0x64006400u);
+    const uint32_t nk = p.K / 64u, nkp = nk >> 1;
+
+    auto load_a = [&](uint32_t kt, u4_t* a_reg) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
+    };
+    auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *(u4_t*)(lds5 + stage * A_STAGE + a_lds0 + i * 4096u) = a_reg[i];
+    };
+    auto load_raw = [&](uint32_t kp, u4_t* raw) {
+#pragma unroll
+        for (int i = 0; i < 5; ++i) raw[i] = *(const u4_t*)(bank + raw_goff[i] + (uint64_t)kp * 80u);
+    };
+    auto store_raw = [&](const u4_t* raw) {
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            *(u2_t*)(lds5 + raw_loff[i]) = u2_t{raw[i][0], raw[i][1]};
+            *(u2_t*)(lds5 + raw_loff[i] + 8u) = u2_t{raw[i][2], raw[i][3]};
+        }
+    };
+    auto read_blk = [&](uint32_t s2, qg_slice<FMT>* blk) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const uint32_t* src = (const uint32_t*)(lds5 + rd0 + b * (32u * RAW_PITCH) + s2 * 40u);
+            blk[b].hdr = src[0];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) blk[b].q[w] = src[1 + w];
+        }
+    };
+    auto mfma_step = [&](const uint8_t* st, const qg_slice<FMT>* blk) {
+        const h2_t s0 = qw_splat_lo(blk[0].hdr), c0 = qw_splat_hi(blk[0].hdr);
+        const h2_t s1 = qw_splat_lo(blk[1].hdr), c1 = qw_splat_hi(blk[1].hdr);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint32_t off = a_rd + (((4u * kh + (uint32_t)ks) ^ fr_key) << 4);
+            const h8_t a0 = *(const h8_t*)(st + off), a1 = *(const h8_t*)(st + off + 4096u);
+            const h8_t w0 = qg_dequant_chunk<FMT>(blk[0], ks, s0, c0, magic);
+            const h8_t w1 = qg_dequant_chunk<FMT>(blk[1], ks, s1, c1, magic);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, w0, acc[0][0], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, w0, acc[1][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, w1, acc[0][1], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, w1, acc[1][1], 0, 0, 0);
+        }
+    };
+
+    const uint32_t last = nk - 1u, lastp = nkp - 1u;
+    u4_t raw[5], a_reg[2][2];
+    load_raw(0, raw);
+    load_a(0, a_reg[0]);
+    load_a(min(1u, last), a_reg[1]);
+    store_raw(raw);
+    load_raw(min(1u, lastp), raw);
+    store_a(0, a_reg[0]);
+    __syncthreads();
+    for (uint32_t kp = 0; kp < nkp; ++kp) {
+        const uint32_t kt = 2u * kp;
+        qg_slice<FMT> blk[2];
+        // K-step 2 kp: activations in stage 0
+        load_a(min(kt + 2u, last), a_reg[0]);
+        read_blk(0u, blk);
+        mfma_step(lds5, blk);
+        store_a(1u, a_reg[1]);
+        __syncthreads();
+        // K-step 2 kp + 1: activations in stage 1
+        load_a(min(kt + 3u, last), a_reg[1]);
+        read_blk(1u, blk);
+        mfma_step(lds5 + A_STAGE, blk);
+        store_a(0u, a_reg[0]);
+        __syncthreads();          // every wave has read its blocks of this pair: the single raw stage can be replaced
+        store_raw(raw);
+        load_raw(min(kp + 2u, lastp), raw);
+        __syncthreads();
+    }
+
+    // ---- epilogue (as qw_gemm4_kernel): per wave, rows 32 a .. + 31 through a private LDS slab, 16-byte row chunks out ----
+    if constexpr (SWIGLU) {
+        constexpr uint32_t EP_PITCH = 64 + 16;
+        uint8_t* ep = lds5 + wave * (32u * EP_PITCH);
+        const uint32_t w_off = (4u * kh) * EP_PITCH + j * 2u;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float g = (float)(h1_t)acc[a][0][r], u = (float)(h1_t)acc[a][1][r];
+                float v = qw_swiglu(g, u);
+                if (p.rotate_act) {
+#pragma unroll
+                    for (uint32_t h = 1; h < 32u; h <<= 1) {
+                        const float o = __shfl_xor(v, (int)h, 32);
+                        v = (j & h) == 0u ? v + o : o - v;
+                    }
+                    v *= QW_INV_SQRT32;
+                }
+                *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
+            }
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const uint32_t c = q * 64u + lane;
+                const uint32_t row = c >> 2, cc = c & 3u;
+                const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
+                const uint32_t grow = 32u * a + row;
+                const uint32_t n = n0 + wave * 32u + cc * 8u;
+                if (grow < rows_valid && n < p.inter)
+                    *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+            }
+        }
+    } else if constexpr (YDT != QWHIP_F32) {
+        constexpr uint32_t EP_PITCH = 2 * 64 + 16;
+        uint8_t* ep = lds5 + wave * (32u * EP_PITCH);
+        const uint32_t w_off = (4u * kh) * EP_PITCH + j * 2u;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t o = w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH + b * 64u;
+                    if constexpr (YDT == QWHIP_BF16) *(uint16_t*)(ep + o) = qw_f32_to_bf16(acc[a][b][r]);
+                    else *(h1_t*)(ep + o) = (h1_t)acc[a][b][r];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t c = q * 64u + lane;
+                const uint32_t row = c >> 3, cc = c & 7u;
+                const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
+                const uint32_t grow = 32u * a + row;
+                const uint32_t n = n0 + wave * 64u + cc * 8u;
+                if (grow < rows_valid && n < p.N)
+                    *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const uint32_t n = n0 + wave * 64u + 32u * b + j;
+                if (n < p.N) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t row = 32u * a + 8 * (r >> 2) + 4 * kh + (r & 3);
+                        if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -1074,6 +1302,17 @@ hipError_t launch_cfg4(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     static_assert(lds >= 2u * 64u * 128u, "the stages fit the slab allocation");
     hipLaunchKernelGGL((qw_gemm4_kernel<FMT, YDT, SWIGLU>), grid, dim3(256), lds, st, p);
     return hipGetLastError();
+}
+
+template <int YDT, bool SWIGLU>
+hipError_t launch_cfg5(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
+    constexpr size_t lds = 2u * 64u * 128u + 256u * 88u;   // two activation stages + one raw K-pair image (38,912 bytes)
+    hipLaunchKernelGGL((qw_gemm5_kernel<YDT, SWIGLU>), grid, dim3(256), lds, st, p);
+    return hipGetLastError();
+}
+// the raw-copy kernel takes HQ4_G32_M5 banks whose rows are whole 80-byte K pairs at 16-byte aligned addresses
+inline bool gemm5_takes(const qw_gemm_params& p, int fmt) {
+    return fmt == QG_FMT_M5 && p.K % 128u == 0 && ((uintptr_t)p.bank & 15u) == 0;
 }
 
 // tile shapes of the pipelined kernel
@@ -1255,6 +1494,11 @@ hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid,
         qw_gemm_params q = p;
         q.tiles_n = grid.x;
         const dim3 grid1(8u * qwhip_cdiv(grid.y, 8u) * grid.x);   // XCD-aware one-dimensional grid over (tile, column tile)
+        if (gemm5_takes(q, FMT)) {
+            if (ydt == QWHIP_F16) return launch_cfg5<QWHIP_F16, false>(st, q, grid1);
+            if (ydt == QWHIP_BF16) return launch_cfg5<QWHIP_BF16, false>(st, q, grid1);
+            return launch_cfg5<QWHIP_F32, false>(st, q, grid1);
+        }
         if (ydt == QWHIP_F16) return launch_cfg4<FMT, QWHIP_F16, false>(st, q, grid1);
         if (ydt == QWHIP_BF16) return launch_cfg4<FMT, QWHIP_BF16, false>(st, q, grid1);
         return launch_cfg4<FMT, QWHIP_F32, false>(st, q, grid1);
@@ -1370,7 +1614,8 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     p.tiles_n = qwhip_cdiv(inter, 128u);
     const dim3 grid(8u * qwhip_cdiv(max_tiles, 8u) * p.tiles_n);   // XCD-aware one-dimensional grid over (tile, column tile)
     hipError_t e;
-    if (fmt == QG_FMT_M5) e = launch_cfg4<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid);
+    if (gemm5_takes(p, fmt)) e = launch_cfg5<QWHIP_F16, true>(s->stream, p, grid);
+    else if (fmt == QG_FMT_M5) e = launch_cfg4<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid);
     else if (fmt == QG_FMT_B4) e = launch_cfg4<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
     else e = launch_cfg4<QG_FMT_B8, QWHIP_F16, true>(s->stream, p, grid);
     QWHIP_TRY_HIP(e);
