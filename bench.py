@@ -536,9 +536,9 @@ def run_moe(args, t, label):
         def gate_up():
             qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, 0, ib.ptr, t, K, act.ptr))
 
-        def chain():
-            qwhip.check(lib.qwhip_moe_route(st, lb.ptr, t, E, K, 1, 1.0, ib.ptr, wb.ptr))
-            gate_up()
+        def chain():   # routing happens inside the gate_up launch
+            qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, 0, lb.ptr, t, K, 1, 1.0, ib.ptr, wb.ptr,
+                                                          act.ptr))
             qwhip.check(lib.qwhip_moe_down_decode(st, C.byref(vdn), E, act.ptr, ib.ptr, wb.ptr, t, K, None, None, out.ptr, qwhip.F32))
     else:
         x_basis = qo.rotate_activation_f16(x32)

@@ -281,6 +281,15 @@ qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint32_t dn_dty
 qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
                                      const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
                                      uint32_t top_k, void* act16);
+/* qwhip_moe_route + qwhip_moe_gateup_decode as one launch for the decode step (an HQ4_G32_M5 bank routes inside the gate_up
+ * kernel: every workgroup repeats the token's top-k from its router logits with the arithmetic of qwhip_moe_route and
+ * leaves idx / wts [t, top_k] for the down projection; other containers run the two launches).  Same results as the two
+ * calls; one kernel launch less on a path that is bound by launch latency.  The reference runs encodeFnMoeRoute and
+ * encodeMoEGateUpF32R1 back to back (QWMoEOperator.swift); arguments as in those two doors. */
+qwhip_status qwhip_moe_route_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                           const void* x, uint32_t x_dtype, uint32_t flags, const float* logits, uint32_t t,
+                                           uint32_t top_k, uint32_t norm_topk, float routed_scale, int32_t* idx, float* wts,
+                                           void* act16);
 qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts,
                                    const void* act16, const int32_t* idx, const float* wts, uint32_t t,
                                    uint32_t top_k, const float* shared, const float* shared_gate, void* out,

@@ -913,7 +913,9 @@ bool qw_stream_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, u
 
 // moe_col.hip
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
-                       bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err);
+                       bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
+                       const float* logits = nullptr, int32_t* idx_out = nullptr, float* wts_out = nullptr, uint32_t norm_topk = 0,
+                       float routed_scale = 1.0f);
 bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* act16, const int32_t* idx,
                      const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
                      uint32_t out_dtype, hipError_t* err);
@@ -1119,6 +1121,43 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     else launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds);
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
+}
+
+// ---- MoE decode / verify: routing + routed gate|up in one launch -------------------------------------
+extern "C" qwhip_status qwhip_moe_route(qwhip_stream_t s, const float* logits, uint32_t t, uint32_t experts, uint32_t top_k,
+                                        uint32_t norm_topk, float routed_scale, int32_t* idx, float* wts);
+extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                                const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
+                                                uint32_t top_k, void* act16);
+extern "C" qwhip_status qwhip_moe_route_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                                      const void* x, uint32_t x_dtype, uint32_t flags, const float* logits, uint32_t t,
+                                                      uint32_t top_k, uint32_t norm_topk, float routed_scale, int32_t* idx, float* wts,
+                                                      void* act16) {
+    int fmt = 0;
+    qwhip_status st = check_common(s, w_gate_up, x, x_dtype, 1, &fmt);
+    if (st != QWHIP_OK) return st;
+    QWHIP_REQUIRE(logits);
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(wts);
+    QWHIP_REQUIRE(act16);
+    if (t == 0 || top_k == 0) return QWHIP_OK;
+    if (experts == 0 || experts > 512) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: experts must be 1..512, got %u", experts);
+    if (top_k > 16) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: top_k must be 1..16, got %u", top_k);
+    const float scale = routed_scale > 0.0f ? routed_scale : 1.0f;
+    if (fmt == QW_FMT_M5 && w_gate_up->n % (2 * experts) == 0 && (uint64_t)t * top_k <= 65535u) {
+        const uint32_t inter = w_gate_up->n / (2 * experts);
+        const bool rotate = qwhip_view_rotated(w_gate_up) && !(flags & QWHIP_X_PREROTATED);
+        hipError_t e = hipSuccess;
+        if (qw_moe_gateup_col(s->stream, w_gate_up, experts, x, x_dtype, rotate, qwhip_view_rotated(w_gate_up) && inter % 32 == 0, nullptr,
+                              t * top_k, top_k, act16, &e, logits, idx, wts, norm_topk ? 1u : 0u, scale)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+    }
+    // other containers and shapes: the two launches
+    st = qwhip_moe_route(s, logits, t, experts, top_k, norm_topk, routed_scale, idx, wts);
+    if (st != QWHIP_OK) return st;
+    return qwhip_moe_gateup_decode(s, w_gate_up, experts, x, x_dtype, flags, idx, t, top_k, act16);
 }
 
 // ---- MoE decode / verify (t <= 8): routed experts as GEMVs -----------------------------------------

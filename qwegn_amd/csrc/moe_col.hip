@@ -9,6 +9,7 @@
 // unpack_hq4_word8, Sources/QWMetal/include/qw_dequant.metalh:42-62).  A half-wavefront covers 32 block columns of a
 // row and reduces with DPP; the per-chunk partial sums meet in LDS and are added in chunk order.
 #include "qwhip_common.h"
+#include "qwhip_route.h"
 
 namespace {
 
@@ -60,9 +61,17 @@ struct qmc_gu_params {
     const int32_t* idx;
     uint32_t I, nb, cpr, top_k, rotate, rot_out;
     uint64_t expert_bytes;
+    // JN > 0: the routing is done here.  Every wave routes the pair's token from its router logits (the arithmetic of
+    // qw_moe_route_kernel, so the same experts and weights) and takes rank pair % top_k; the workgroups of the first row
+    // block leave the pair's expert and weight in idx_out / wts_out for the down projection.
+    const float* logits;
+    int32_t* idx_out;
+    float* wts_out;
+    uint32_t experts, norm;
+    float routed_scale;
 };
 
-template <int XDT, int SETS>
+template <int XDT, int SETS, int JN = 0>
 __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_params p) {
     constexpr int R = 64 / SETS;
     constexpr int D = R < 8 ? R : 8;             // rows in flight per lane
@@ -83,8 +92,10 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
     const uint32_t row_bytes = nb * 20u;
 
     // memory order: the route's expert id, the token's activations, the first weight rows; the rotation runs under them
-    const int32_t e = p.idx ? p.idx[pair] : 0;   // no route list: one dense gate|up bank
-    const uint8_t* x = (const uint8_t*)p.x + (uint64_t)(pair / p.top_k) * nb * 64u;
+    int32_t e = 0;                               // no route list: one dense gate|up bank
+    if constexpr (JN == 0) e = p.idx ? p.idx[pair] : 0;
+    const uint32_t token = pair / p.top_k;
+    const uint8_t* x = (const uint8_t*)p.x + (uint64_t)token * nb * 64u;
     h8_t xv[XT];
 #pragma unroll
     for (int t = 0; t < XT; ++t) {
@@ -92,6 +103,17 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
         xv[t] = qw_load_x8_f16<XDT>(x, (uint64_t)gg * 32u + 8u * (l64 >> 4));
     }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (JN > 0) {
+        int32_t isel;
+        float wsel;
+        qw_route_wave<JN>(p.logits + (uint64_t)token * p.experts, p.experts, p.top_k, p.norm, p.routed_scale, l64, isel, wsel);
+        const uint32_t rank = pair - token * p.top_k;
+        e = __builtin_amdgcn_readlane(isel, rank);
+        if (blockIdx.x == 0 && wave == 0 && l64 == rank) {
+            p.idx_out[pair] = isel;
+            p.wts_out[pair] = wsel;
+        }
+    }
     h1_t* act = p.act + (uint64_t)pair * I;
     if (e < 0) {   // no expert: the pair contributes nothing (uniform over the workgroup)
         if (tid < 32u && n0 + tid < I) act[n0 + tid] = (h1_t)0.0f;
@@ -228,7 +250,8 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
 // Routed gate|up projection with the SwiGLU (+ rotation) epilogue for a validated HQ4_G32_M5 bank; false when the shape
 // is outside the kernel's envelope (the caller then takes the general kernel).
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
-                       bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err) {
+                       bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
+                       const float* logits, int32_t* idx_out, float* wts_out, uint32_t norm_topk, float routed_scale) {
     if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
     const uint32_t inter = w->n / (2u * experts);
     const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u;
@@ -249,13 +272,26 @@ bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expe
     p.rotate = rotate ? 1u : 0u;
     p.rot_out = rot_out ? 1u : 0u;
     p.expert_bytes = (uint64_t)2u * inter * nb * 20u;
+    p.logits = logits;
+    p.idx_out = idx_out;
+    p.wts_out = wts_out;
+    p.experts = experts;
+    p.norm = norm_topk;
+    p.routed_scale = routed_scale;
     const dim3 grid(qwhip_cdiv(inter, 32u), pairs), block(32u * cpr * sets);
-#define QMC_GU(DT, S) hipLaunchKernelGGL((qw_moe_gateup_col_kernel<DT, S>), grid, block, lds, st, p)
-    if (x_dtype == QWHIP_F16) {
-        if (sets == 8u) QMC_GU(QWHIP_F16, 8); else if (sets == 4u) QMC_GU(QWHIP_F16, 4); else QMC_GU(QWHIP_F16, 2);
+#define QMC_GU(DT, S, J) hipLaunchKernelGGL((qw_moe_gateup_col_kernel<DT, S, J>), grid, block, lds, st, p)
+#define QMC_GU_S(DT, J)                                                                                     \
+    do {                                                                                                    \
+        if (sets == 8u) QMC_GU(DT, 8, J); else if (sets == 4u) QMC_GU(DT, 4, J); else QMC_GU(DT, 2, J);     \
+    } while (0)
+    if (!logits) {
+        if (x_dtype == QWHIP_F16) QMC_GU_S(QWHIP_F16, 0); else QMC_GU_S(QWHIP_BF16, 0);
+    } else if (experts <= 128u) {   // routing in the kernel: two experts per lane cover the usual 64 / 128, eight cover up to 512
+        if (x_dtype == QWHIP_F16) QMC_GU_S(QWHIP_F16, 2); else QMC_GU_S(QWHIP_BF16, 2);
     } else {
-        if (sets == 8u) QMC_GU(QWHIP_BF16, 8); else if (sets == 4u) QMC_GU(QWHIP_BF16, 4); else QMC_GU(QWHIP_BF16, 2);
+        if (x_dtype == QWHIP_F16) QMC_GU_S(QWHIP_F16, 8); else QMC_GU_S(QWHIP_BF16, 8);
     }
+#undef QMC_GU_S
 #undef QMC_GU
     *err = hipGetLastError();
     return true;

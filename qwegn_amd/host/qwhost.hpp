@@ -489,6 +489,21 @@ struct QWGemm {
                                         (uint32_t)rows, (uint32_t)topK, (uint32_t)hidden, shared ? (const float*)shared->ptr() : nullptr,
                                         sharedGate ? (const float*)sharedGate->ptr() : nullptr, out.ptr(), abiDType(out.shape.dtype)));
     }
+    // encodeFnMoeRoute + encodeMoEGateUpF32R1 as one launch (decode / verify): idx / wts are left for the down projection
+    static void encodeMoERouteGateUp(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& gateUp, int experts, const QWTensorValue& x,
+                                     const QWTensorValue& logits, const QWTensorValue& idx, const QWTensorValue& wts, int rows, int topK,
+                                     bool normTopK, float routedScale, const QWTensorValue& act16, bool rotateInKernel = false) {
+        if (logits.shape.dtype != QWDType::f32 || logits.shape.elementCount < (size_t)rows * (size_t)experts ||
+            idx.shape.elementCount < (size_t)rows * (size_t)topK || wts.shape.elementCount < (size_t)rows * (size_t)topK)
+            throw QWGemmError(QWGemmError::badShape, "moe route: logits f32 [rows, experts], idx / wts [rows, topK]");
+        hal.pipeline("qwg_moe_route");
+        hal.pipeline("qwg_moe_gateup_q4g_f32_r1");
+        const qwhip_weight_view v = gateUp.abi();
+        throwIfFailed(qwhip_moe_route_gateup_decode(enc.stream, &v, (uint32_t)experts, x.ptr(), abiDType(x.shape.dtype),
+                                                    rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED, (const float*)logits.ptr(), (uint32_t)rows,
+                                                    (uint32_t)topK, normTopK ? 1 : 0, routedScale, (int32_t*)idx.ptr(), (float*)wts.ptr(),
+                                                    act16.ptr()));
+    }
     // encodeMoEGateUpF32R1 / encodeMoEDownSharedCombineF32 (QWGemmMoE.swift:120-199): decode / verify, rows <= 8
     static void encodeMoEGateUpF32R1(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& gateUp, int experts, const QWTensorValue& x,
                                      const QWTensorValue& idx, int rows, int topK, const QWTensorValue& act16, bool rotateInKernel = false) {
@@ -602,11 +617,11 @@ struct QWMoEOperator {
         if (w.gateUp.n != E * 2 * I || w.gateUp.k != H || w.down.n != E * H || w.down.k != I)
             throw QWGemmError(QWGemmError::badShape, "moe: expert banks do not match (experts, hidden, intermediate)");
         QWGemm::encodeFnRouterGemm(enc, hal, xPlain, w.router, s.logits, rows, E, H);
-        QWGemm::encodeFnMoeRoute(enc, hal, s.logits, s.idx, s.wts, rows, E, K, w.normTopK, w.routedScale);
         const bool fused = x.shape.dtype == QWDType::f16;   // gate_up GEMM + SwiGLU in one launch: gu16 is not needed
         const bool grouped = rows > 8 && s.expOff.base && (fused || s.gu16.base) && s.dnHi.base && H % 64 == 0 && I % 64 == 0;
         if (grouped) {
             const int pairs = rows * K;
+            QWGemm::encodeFnMoeRoute(enc, hal, s.logits, s.idx, s.wts, rows, E, K, w.normTopK, w.routedScale);
             QWGemm::encodeMoEGroupPairsF32(enc, hal, s.idx, s.expOff, s.sortedPair, s.sortedTok, E, pairs, K, &s.invPerm, &s.tileE, &s.tileR, &s.tileCount);
             if (fused) {
                 QWGemm::encodeMoEGateUpSwiglu(enc, hal, w.gateUp, E, x, s.sortedTok, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.act16,
@@ -618,7 +633,7 @@ struct QWMoEOperator {
             QWGemm::encodeMoEGroupedGemm(enc, hal, w.down, E, s.act16, nullptr, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.dnHi);
             QWGemm::encodeMoEDownReduceCombineF32(enc, hal, s.dnHi, s.invPerm, s.wts, rows, K, H, shared, sharedGate, out);
         } else {
-            QWGemm::encodeMoEGateUpF32R1(enc, hal, w.gateUp, E, x, s.idx, rows, K, s.act16);
+            QWGemm::encodeMoERouteGateUp(enc, hal, w.gateUp, E, x, s.logits, s.idx, s.wts, rows, K, w.normTopK, w.routedScale, s.act16);
             QWGemm::encodeMoEDownSharedCombineF32(enc, hal, w.down, E, s.act16, s.idx, s.wts, rows, K, shared, sharedGate, out);
         }
     }

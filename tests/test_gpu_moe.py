@@ -234,6 +234,33 @@ def test_moe_decode_chain_matches_oracle(dev, t, xdt, experts, hidden, inter, k,
     assert np.all(a[0, k - 1] == 0)
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g32"])
+@pytest.mark.parametrize("t,experts,hidden,inter,k", [(1, 128, 512, 96, 8), (3, 16, 1280, 192, 4), (8, 200, 256, 64, 3)])
+def test_fused_route_gateup_decode_equals_the_two_launches(dev, fmt, t, experts, hidden, inter, k):
+    """qwhip_moe_route_gateup_decode leaves the ids, weights and activations of qwhip_moe_route + qwhip_moe_gateup_decode, bit
+    for bit (the HQ4_G32_M5 bank routes inside the gate_up kernel, the bit-stream bank runs the two launches)."""
+    gu_blocks, _, _, _ = _moe_banks(experts, hidden, inter, seed=23, fmt=fmt)
+    rng = np.random.default_rng(8)
+    xh = rng.standard_normal((t, hidden)).astype(np.float16)
+    logits = rng.standard_normal((t, experts)).astype(np.float32)
+    logits[0, 3] = np.inf                                      # a non-finite logit never wins
+    logits[t - 1, 5] = logits[t - 1, 9]                        # a tie goes to the lower id
+    lib, st = dev.lib, dev.stream.handle
+    gub, xb, lb = dev.put(gu_blocks), dev.put(xh), dev.put(logits)
+    vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
+    i2, w2, a2 = dev.alloc(t * k * 4 + 256), dev.alloc(t * k * 4 + 256), dev.alloc(t * k * inter * 2)
+    i1, w1, a1 = dev.alloc(t * k * 4 + 256), dev.alloc(t * k * 4 + 256), dev.alloc(t * k * inter * 2)
+    qwhip.check(lib.qwhip_moe_route(st, lb.ptr, t, experts, k, 1, 2.5, i2.ptr, w2.ptr))
+    qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, i2.ptr, t, k, a2.ptr))
+    qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, lb.ptr, t, k, 1, 2.5, i1.ptr, w1.ptr, a1.ptr))
+    dev.stream.sync()
+    assert np.array_equal(i1.download(np.int32, (t, k)), i2.download(np.int32, (t, k)))
+    assert np.array_equal(w1.download(np.uint32, (t, k)), w2.download(np.uint32, (t, k)))
+    assert np.array_equal(a1.download(np.uint16, (t, k, inter)), a2.download(np.uint16, (t, k, inter)))
+    ref_idx, ref_w = qo.moe_route(logits, k, True, 2.5)
+    assert np.array_equal(i1.download(np.int32, (t, k)), ref_idx)
+
+
 def test_online_quantizer_writes_the_packers_bytes(dev):
     """Device HQ4_G32_M5 quantizer vs the oracle's restatement of the packer, byte-identical
     (Tests/QWFlashNextMetalTests/QUANT/FNMetalOnlineQuantTests.swift:243), bf16 and f32 sources, rotate on/off."""
