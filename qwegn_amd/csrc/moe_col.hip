@@ -61,9 +61,9 @@ struct qmc_gu_params {
     const int32_t* idx;
     uint32_t I, nb, cpr, top_k, rotate, rot_out;
     uint64_t expert_bytes;
-    // JN > 0: the routing is done here.  Every wave routes the pair's token from its router logits (the arithmetic of
-    // qw_moe_route_kernel, so the same experts and weights) and takes rank pair % top_k; the workgroups of the first row
-    // block leave the pair's expert and weight in idx_out / wts_out for the down projection.
+    // JN > 0: the routing is done here.  The first wave of every workgroup routes the pair's token from its router logits
+    // (the arithmetic of qw_moe_route_kernel, so the same experts and weights) and the workgroup takes rank pair % top_k;
+    // the workgroups of the first row block leave the pair's expert and weight in idx_out / wts_out for the down projection.
     const float* logits;
     int32_t* idx_out;
     float* wts_out;
@@ -104,15 +104,22 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (JN > 0) {
-        int32_t isel;
-        float wsel;
-        qw_route_wave<JN>(p.logits + (uint64_t)token * p.experts, p.experts, p.top_k, p.norm, p.routed_scale, l64, isel, wsel);
-        const uint32_t rank = pair - token * p.top_k;
-        e = __builtin_amdgcn_readlane(isel, rank);
-        if (blockIdx.x == 0 && wave == 0 && l64 == rank) {
-            p.idx_out[pair] = isel;
-            p.wts_out[pair] = wsel;
+        __shared__ int32_t e_route;
+        if (wave == 0) {   // one wave routes (the others would only compete for the same SIMDs), the workgroup reads its result
+            int32_t isel;
+            float wsel;
+            qw_route_wave<JN>(p.logits + (uint64_t)token * p.experts, p.experts, p.top_k, p.norm, p.routed_scale, l64, isel, wsel);
+            const uint32_t rank = pair - token * p.top_k;
+            if (l64 == rank) {
+                e_route = isel;
+                if (blockIdx.x == 0) {
+                    p.idx_out[pair] = isel;
+                    p.wts_out[pair] = wsel;
+                }
+            }
         }
+        __syncthreads();
+        e = e_route;
     }
     h1_t* act = p.act + (uint64_t)pair * I;
     if (e < 0) {   // no expert: the pair contributes nothing (uniform over the workgroup)
