@@ -1012,8 +1012,8 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// The direct-operand grouped kernel with the bank read the way memory likes it (HQ4_G32_M5, K % 128 == 0, bank 16-byte
-// aligned).  In qw_gemm4_kernel every lane fetches its own 20-byte block: 64 runs of the bank per load instruction, at
+// The direct-operand grouped kernel with the bank read the way memory likes it (banks of 20-byte blocks: HQ4_G32_M5 and
+// the 4-bit group-32 bit streams; K % 128 == 0, bank 16-byte aligned).  In qw_gemm4_kernel every lane fetches its own 20-byte block: 64 runs of the bank per load instruction, at
 // 4-byte alignment - the address unit is what bounds it.  Here the 256 weight rows of a tile are copied raw, 128 columns
 // (four blocks = 80 bytes per row) at a time: consecutive threads copy consecutive 16-byte chunks of a row (five per row),
 // global -> registers -> LDS, the LDS image being the same bytes in the same order; each lane then reads its block
@@ -1023,10 +1023,10 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 // four workgroups per CU.  The raw image of K pair kp + 1 is in flight (registers) during K pair kp and replaces the
 // stage between two barriers at its end.
 // ------------------------------------------------------------------------------------------------
-template <int YDT, bool SWIGLU>
+template <int FMT, int YDT, bool SWIGLU>
 __global__ __launch_bounds__(256) void qw_gemm5_kernel(const qw_gemm_params p) {
     static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
-    constexpr int FMT = QG_FMT_M5;
+    static_assert(FMT == QG_FMT_M5 || FMT == QG_FMT_B4, "20-byte blocks: HQ4_G32_M5 and the 4-bit group-32 bit streams");
     // raw image: row pitch 88 bytes (22 dwords: the 64 lanes of a block read fall on 64 different banks), one stage
     constexpr uint32_t BM = 64, BN = 256, A_STAGE = BM * 128u, RAW_PITCH = 88u, RAW_OFF = 2u * A_STAGE;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds5[];
@@ -1304,15 +1304,20 @@ hipError_t launch_cfg4(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int YDT, bool SWIGLU>
+template <int FMT, int YDT, bool SWIGLU>
 hipError_t launch_cfg5(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr size_t lds = 2u * 64u * 128u + 256u * 88u;   // two activation stages + one raw K-pair image (38,912 bytes)
-    hipLaunchKernelGGL((qw_gemm5_kernel<YDT, SWIGLU>), grid, dim3(256), lds, st, p);
-    return hipGetLastError();
+    if constexpr (FMT == QG_FMT_M5 || FMT == QG_FMT_B4) {
+        hipLaunchKernelGGL((qw_gemm5_kernel<FMT, YDT, SWIGLU>), grid, dim3(256), lds, st, p);
+        return hipGetLastError();
+    } else {
+        return hipErrorInvalidValue;   // not reached: gemm5_takes() refuses the 8-bit containers
+    }
 }
-// the raw-copy kernel takes HQ4_G32_M5 banks whose rows are whole 80-byte K pairs at 16-byte aligned addresses
+// the raw-copy kernel takes banks of 20-byte blocks (HQ4_G32_M5, 4-bit group 32) whose rows are whole 80-byte K pairs at
+// 16-byte aligned addresses
 inline bool gemm5_takes(const qw_gemm_params& p, int fmt) {
-    return fmt == QG_FMT_M5 && p.K % 128u == 0 && ((uintptr_t)p.bank & 15u) == 0;
+    return (fmt == QG_FMT_M5 || (fmt == QG_FMT_B4 && p.gshift == 0)) && p.K % 128u == 0 && ((uintptr_t)p.bank & 15u) == 0;
 }
 
 // tile shapes of the pipelined kernel
@@ -1495,9 +1500,9 @@ hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid,
         q.tiles_n = grid.x;
         const dim3 grid1(8u * qwhip_cdiv(grid.y, 8u) * grid.x);   // XCD-aware one-dimensional grid over (tile, column tile)
         if (gemm5_takes(q, FMT)) {
-            if (ydt == QWHIP_F16) return launch_cfg5<QWHIP_F16, false>(st, q, grid1);
-            if (ydt == QWHIP_BF16) return launch_cfg5<QWHIP_BF16, false>(st, q, grid1);
-            return launch_cfg5<QWHIP_F32, false>(st, q, grid1);
+            if (ydt == QWHIP_F16) return launch_cfg5<FMT, QWHIP_F16, false>(st, q, grid1);
+            if (ydt == QWHIP_BF16) return launch_cfg5<FMT, QWHIP_BF16, false>(st, q, grid1);
+            return launch_cfg5<FMT, QWHIP_F32, false>(st, q, grid1);
         }
         if (ydt == QWHIP_F16) return launch_cfg4<FMT, QWHIP_F16, false>(st, q, grid1);
         if (ydt == QWHIP_BF16) return launch_cfg4<FMT, QWHIP_BF16, false>(st, q, grid1);
@@ -1614,7 +1619,8 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     p.tiles_n = qwhip_cdiv(inter, 128u);
     const dim3 grid(8u * qwhip_cdiv(max_tiles, 8u) * p.tiles_n);   // XCD-aware one-dimensional grid over (tile, column tile)
     hipError_t e;
-    if (gemm5_takes(p, fmt)) e = launch_cfg5<QWHIP_F16, true>(s->stream, p, grid);
+    if (gemm5_takes(p, fmt)) e = fmt == QG_FMT_M5 ? launch_cfg5<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid)
+                                                  : launch_cfg5<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
     else if (fmt == QG_FMT_M5) e = launch_cfg4<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid);
     else if (fmt == QG_FMT_B4) e = launch_cfg4<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
     else e = launch_cfg4<QG_FMT_B8, QWHIP_F16, true>(s->stream, p, grid);

@@ -149,7 +149,7 @@ def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
     assert qo.normalized_error(got, ref) <= TOL
 
 
-@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32"])
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g32", "hq4_g64", "hq8_g32"])
 @pytest.mark.parametrize("t,experts,hidden,inter,k,rot", [(40, 8, 256, 128, 2, 1), (130, 16, 512, 192, 4, 1), (300, 4, 128, 64, 2, 0),
                                                           (64, 8, 192, 448, 3, 1)])
 def test_fused_gate_up_swiglu_equals_the_two_step_chain(dev, fmt, t, experts, hidden, inter, k, rot):
