@@ -10,7 +10,7 @@ kernel measured with HIP events on the launch stream, and the CPU baseline (the 
 oracle form - dequantize the bank to fp32, then one fp32 product - restated in numpy and timed
 on this box's host cores over a bounded sample).
 
-Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up|head|f32_decode|f32_verify4|repack|norm_prefill|norm_decode (see WORKLOADS).
+Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up|mlp_prefill|head|f32_decode|f32_verify4|repack|norm_prefill|norm_decode (see WORKLOADS).
 """
 from __future__ import annotations
 
@@ -301,6 +301,70 @@ def run_gemv_f32(args, fmt, n, k, m, label):
         "config": {"workload": label, "format": fmt, "M": m, "N": n, "K": k},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": None, "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
+        "normalized_error": err,
+    }
+
+
+def run_mlp_prefill(args, inter, k, m, label):
+    """Dense MLP prefill gate|up: X f16 [m, k] in the weight basis -> act f16 [m, inter] through the GEMM with the SwiGLU + FWHT-32
+    epilogue fused; one step = one launch.  The bank is written by the device quantizer; parity on a sample of outputs."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+
+    dev = qwhip.Device(0)
+    lib, st = dev.lib, dev.stream.handle
+    rng = np.random.default_rng(0)
+    n = 2 * inter
+    bank = dev.alloc(n * (k // 32) * 20)
+    for r0 in range(0, n, 4096):           # weights N(0, 0.02), quantized on the device chunk by chunk
+        rows_here = min(4096, n - r0)
+        wsrc = dev.put((rng.standard_normal((rows_here, k), dtype=np.float32) * np.float32(0.02)))
+        qwhip.check(lib.qwhip_quantize_hq4_g32(st, wsrc.ptr, qwhip.F32, rows_here, k, 0, bank.ptr + r0 * (k // 32) * 20))
+        dev.stream.sync()
+    view = dev.view(bank, n, k, qwhip.KIND_HQ4_G32_M5)
+    x16 = rng.standard_normal((m, k), dtype=np.float32).astype(np.float16)
+    xb, act = dev.put(x16), dev.alloc(m * inter * 2)
+
+    def launch(i):
+        qwhip.check(lib.qwhip_gemm_swiglu(st, C.byref(view), xb.ptr, qwhip.F16, m, 0, 1, act.ptr, 0, qwhip.X_PREROTATED, None, 0))
+
+    launch(0)
+    dev.stream.sync()
+    # parity: the first 64 outputs (two rotation groups) of 64 sampled rows against the oracle on the downloaded blocks
+    blocks = bank.download(np.uint8, (n, k // 32, 20))
+    cols = np.arange(64)
+    wg = qo.weights_f16_exact(blocks[cols], 4, 32, True)
+    wu = qo.weights_f16_exact(blocks[inter + cols], 4, 32, True)
+    rows = np.arange(0, m, max(1, m // 64))[:64]
+    g = qo.matmul_ref_f64(x16[rows], wg).astype(np.float16).astype(np.float32)
+    u = qo.matmul_ref_f64(x16[rows], wu).astype(np.float16).astype(np.float32)
+    want = qo.swiglu_fwht_f16(g, u, rotate=True).astype(np.float32)
+    got = act.download(np.float16, (m, inter))[rows][:, :64].astype(np.float32)
+    err = qo.normalized_error(got, want)
+    if not err <= 2e-3:
+        _fail(f"bench: fused gate_up output failed parity (normalized error {err:.3e})")
+    _spin_up(dev, launch, 300.0)
+    for i in range(args.warmup):
+        launch(i)
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        launch(i)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    flops = 2.0 * m * n * k
+    tf = flops / (us_per * 1e-6) / 1e12
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": label, "format": "hq4_g32_m5", "M": m, "N": n, "K": k, "x": "f16 (in the weight basis)", "act": "f16 [M, N/2]"},
+        "roofline": {"bound": "mfma", "kernel": "gate|up GEMM with the SwiGLU + FWHT-32 epilogue", "achieved": round(tf, 2),
+                     "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "algorithmic_flops": flops, "kernel_us": round(us_per, 3)},
         "normalized_error": err,
     }
 
@@ -661,6 +725,7 @@ WORKLOADS = {
     "c5_qkv": ("gemv", "hq8_g32", 7168, 5120, None, False),
     "c5_down": ("gemv", "hq4_g64", 5120, 17408, None, False),
     "mlp_gate_up": ("pair", "hq4_g32_m5", 17408, 5120, 1, False),      # n = intermediate size: the bank has 2n rows
+    "mlp_prefill": ("mlp_prefill", "hq4_g32_m5", 17408, 5120, 4096, False),   # n = intermediate size
     "head": ("head", "hq4_g32_m5", 151936, 5120, 1, False),
     "f32_decode": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 1, False),
     "f32_verify4": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 4, False),
@@ -677,6 +742,7 @@ LABELS = {
     "c5_qkv": "C5 verify GEMM HQ8_G32 K=5120 N=7168",
     "c5_down": "C5 verify GEMM HQ4_G64 K=17408 N=5120",
     "mlp_gate_up": "dense MLP gate|up GEMV + SwiGLU + FWHT, HQ4_G32 M=1 K=5120 I=17408",
+    "mlp_prefill": "dense MLP prefill gate|up GEMM + SwiGLU + FWHT fused, HQ4_G32 M=4096 K=5120 I=17408",
     "head": "LM head GEMV + argmax, HQ4_G32 M=1 K=5120 N=151936",
     "f32_decode": "f32-activation GEMV, HQ4_G32 M=1 K=5120 N=17408",
     "f32_verify4": "f32-activation GEMV, HQ4_G32 M=4 K=5120 N=17408",
@@ -726,6 +792,8 @@ def main() -> None:
         out = run_moe(args, m, LABELS[args.workload])
     elif kind == "gemv_f32":
         out = run_gemv_f32(args, fmt, n, k, m, LABELS[args.workload])
+    elif kind == "mlp_prefill":
+        out = run_mlp_prefill(args, n, k, m, LABELS[args.workload])
     elif kind == "head":
         out = run_head(args, fmt, n, k, LABELS[args.workload])
     elif kind == "repack":

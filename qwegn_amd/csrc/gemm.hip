@@ -505,9 +505,17 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 #define QG3_BAR_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define QG3_BAR_ALL() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT>
+// SWIGLU (f16 out, two wave columns): the bank is a dense gate|up bank of 2 * inter rows.  A tile's BN weight rows are
+// BN / 2 gate rows (wave column 0) and the BN / 2 up rows of the same outputs (wave column 1); the epilogue rounds the
+// accumulators to f16 (the values the two-step chain stores) into the waves' LDS slabs, and each pair of waves then reads
+// gate and up chunks of the same outputs, applies SwiGLU and the FWHT-32 in fp32 (three stages inside a lane's eight
+// columns, two across the four lanes of a 32-column group) and stores act f16 [m, inter]: the reference's fused dense
+// gate_up kernel (qwg_gemm_q4g_h16_swiglu: qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167),
+// bit-identical to qwhip_gemm with f16 output followed by qwhip_swiglu_fwht.
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false>
 __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_params p) {
     static_assert(WVM * WVN == 8, "two groups of four waves");
+    static_assert(!SWIGLU || (WVN == 2 && YDT == QWHIP_F16), "fused SwiGLU: gate and up wave columns, f16 out");
     constexpr int NT = WVM * WVN * 64;
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN, BK = 64;
     constexpr int B_ITEMS = BN * 2;
@@ -534,7 +542,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     const uint32_t tm = band * G + in_band % band_rows;
     const uint32_t tn = in_band / band_rows;
     m0 = tm * BM;
-    n0 = tn * BN;
+    n0 = tn * (SWIGLU ? BN / 2 : BN);    // SWIGLU: n0 counts act columns
     rows_valid = min((uint32_t)BM, p.M - m0);
 
     // ---- activation tile: chunk c = tid + i * NT -> tile row (tid >> 3) + (NT / 8) * i, 16-byte k-chunk tid & 7.
@@ -554,12 +562,18 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     // the tile are done redundantly by several threads: identical bytes to the same slot) ----
     static_assert(B_ITEMS >= NT && B_ITEMS <= NT + NT / 2, "the second weight items are covered by group 0 alone");
     uint32_t b_off32[B_PER], b_meta[B_PER];   // byte offset of the row inside the tile's bank rows; LDS row offset | swizzle key << 16 | slice << 20
-    const uint8_t* b_tile = bank + (uint64_t)n0 * p.row_bytes;
+    const uint8_t* b_tile = bank + (SWIGLU ? 0ull : (uint64_t)n0 * p.row_bytes);
 #pragma unroll
     for (int i = 0; i < B_PER; ++i) {
         const uint32_t it = i == 0 ? tid : NT + (B_ITEMS > NT ? tid % (uint32_t)(B_ITEMS > NT ? B_ITEMS - NT : 1) : 0u);
         const uint32_t nl = it >> 1;
-        const uint32_t n = min(n0 + nl, p.N - 1u) - n0;
+        uint32_t n;
+        if constexpr (SWIGLU) {
+            const uint32_t up = nl >= (uint32_t)(BN / 2) ? 1u : 0u;
+            n = up * p.inter + min(n0 + nl - up * (BN / 2), p.inter - 1u);   // whole bank < 4 GiB (checked by the launcher)
+        } else {
+            n = min(n0 + nl, p.N - 1u) - n0;
+        }
         b_off32[i] = n * (uint32_t)p.row_bytes;                     // a tile's rows span < 4 GiB
         b_meta[i] = (nl * 128u) | (((nl >> 1) & 7u) << 16) | ((it & 1u) << 20);
     }
@@ -770,15 +784,62 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
                     *(uint16_t*)(ep + o + EP_PITCH) = (uint16_t)(pk >> 16);
                 }
             }
+            if constexpr (SWIGLU) {
+                __syncthreads();   // the partner wave's slab is complete
+                const uint8_t* gs = lds2 + (wm * WVN) * (32u * EP_PITCH);
+                const uint8_t* us = gs + 32u * EP_PITCH;
+                const uint32_t l4 = lane & 3u;
 #pragma unroll
-            for (int q = 0; q < WN * 2; ++q) {
-                const uint32_t c = q * 64u + lane;
-                const uint32_t row = c / EP_CH, cc = c - row * EP_CH;
-                const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
-                const uint32_t grow = (wm * WM + a) * 32u + row;
-                const uint32_t n = n0 + wn * (WN * 32u) + cc * 8u;
-                if (grow < rows_valid && n < p.N)
-                    *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+                for (int it = 0; it < (int)(32u * EP_CH / 128u); ++it) {
+                    const uint32_t q = (uint32_t)it * 128u + wn * 64u + lane;     // 16-byte chunk of the pair's 32 x (WN * 32) outputs
+                    const uint32_t row = q / EP_CH, cc = q - row * EP_CH;
+                    const h8_t g8 = *(const h8_t*)(gs + row * EP_PITCH + cc * 16u);
+                    const h8_t u8 = *(const h8_t*)(us + row * EP_PITCH + cc * 16u);
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] = qw_swiglu((float)g8[e], (float)u8[e]);
+                    if (p.rotate_act) {
+#pragma unroll
+                        for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+                            for (int i0 = 0; i0 < 8; i0 += 2 * h)
+#pragma unroll
+                                for (int jj = 0; jj < h; ++jj) {
+                                    const float x0 = v[i0 + jj], x1 = v[i0 + jj + h];
+                                    v[i0 + jj] = x0 + x1;
+                                    v[i0 + jj + h] = x0 - x1;
+                                }
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {   // columns 8 apart: the neighbouring lane; 16 apart: two lanes on
+                            const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v[e]), 0xB1, 0xF, 0xF, true));
+                            v[e] = (l4 & 1u) == 0u ? v[e] + o : o - v[e];
+                        }
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v[e]), 0x4E, 0xF, 0xF, true));
+                            v[e] = ((l4 & 2u) == 0u ? v[e] + o : o - v[e]) * QW_INV_SQRT32;
+                        }
+                    }
+                    h8_t o8;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o8[e] = (h1_t)v[e];
+                    const uint32_t grow = (wm * WM + a) * 32u + row;
+                    const uint32_t n = n0 + cc * 8u;
+                    if (grow < rows_valid && n < p.inter)
+                        *(h8_t*)((h1_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = o8;
+                }
+                __syncthreads();   // both waves are done with the slabs before the next row block overwrites them
+            } else {
+#pragma unroll
+                for (int q = 0; q < WN * 2; ++q) {
+                    const uint32_t c = q * 64u + lane;
+                    const uint32_t row = c / EP_CH, cc = c - row * EP_CH;
+                    const u4_t v = *(const u4_t*)(ep + row * EP_PITCH + cc * 16u);
+                    const uint32_t grow = (wm * WM + a) * 32u + row;
+                    const uint32_t n = n0 + wn * (WN * 32u) + cc * 8u;
+                    if (grow < rows_valid && n < p.N)
+                        *(u4_t*)((uint16_t*)p.y + (uint64_t)(m0 + grow) * p.ldy + n) = v;
+                }
             }
         }
     } else {
@@ -1280,11 +1341,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false>
 hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT>;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, SWIGLU>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1478,6 +1539,66 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
         else if (fmt == QG_FMT_B4) e = launch_dense2_y<QG_FMT_B4>(s->stream, p, cfg, y_dtype);
         else e = launch_dense2_y<QG_FMT_B8>(s->stream, p, cfg, y_dtype);
     }
+    QWHIP_TRY_HIP(e);
+    return QWHIP_OK;
+}
+
+// Dense gate|up GEMM with the SwiGLU (+ FWHT-32) epilogue fused: act f16 [m, inter], inter = n / 2, the bank's rows being
+// [gate | up].  Runs the ping-pong kernel's fused form; shapes it does not take are refused (the caller then runs
+// qwhip_gemm into a [m, 2 inter] buffer and qwhip_swiglu_fwht).
+extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
+                                          uint32_t ldx, uint32_t rotate_act, void* act_f16, uint32_t ldact, uint32_t flags,
+                                          void* workspace, size_t workspace_bytes) {
+    int fmt = 0;
+    qwhip_status st = gemm_checks(s, w, x, x_dtype, act_f16, QWHIP_F16, &fmt);
+    if (st != QWHIP_OK) return st;
+    if (m == 0) return QWHIP_OK;
+    const uint32_t inter = w->n / 2u;
+    if (w->n % 64u != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "fused gate_up needs an intermediate size %% 32 == 0, got %u rows", w->n);
+    if (fmt == QG_FMT_B8 || m % 64u != 0)
+        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the fused gate_up GEMM takes 4-bit containers and m %% 64 == 0 (m=%u): run qwhip_gemm + qwhip_swiglu_fwht", m);
+    if (ldx == 0) ldx = w->k;
+    if (ldact == 0) ldact = inter;
+    if (ldx < w->k || ldact < inter || (ldx % 8) != 0 || (ldact % 8) != 0 || ((uintptr_t)act_f16 & 15u) != 0)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions or alignment (ldx=%u ldact=%u, act 16-byte aligned)", ldx, ldact);
+    if ((uint64_t)w->n * qwhip_view_row_bytes(w) >= (1ull << 32))
+        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the fused gate_up GEMM addresses the bank with 32-bit offsets (bank under 4 GiB)");
+    const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
+    const uint64_t ws_need = (uint64_t)m * w->k * 2u;
+    const bool ws_ok = workspace && workspace_bytes >= ws_need && ldx == w->k && ((uintptr_t)workspace & 15u) == 0;
+    const void* xin = x;
+    if (rotate) {
+        if (!ws_ok)
+            return qwhip_fail(QWHIP_E_BASIS, "activations are not in the rotated basis: a 16-byte aligned workspace of %llu bytes and packed rows are needed",
+                              (unsigned long long)ws_need);
+        st = qwhip_fwht32(s, x, x_dtype, workspace, (uint64_t)m * w->k);
+        if (st != QWHIP_OK) return st;
+        xin = workspace;
+    } else if (x_dtype == QWHIP_BF16) {
+        if (!ws_ok) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "bf16 activations need the f16 workspace (%llu bytes, packed rows)", (unsigned long long)ws_need);
+        st = qw_convert_to_f16(s, x, x_dtype, workspace, (uint64_t)m * w->k);
+        if (st != QWHIP_OK) return st;
+        xin = workspace;
+    }
+    qw_gemm_params p = {};
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = xin;
+    p.y = act_f16;
+    p.M = m;
+    p.N = w->n;
+    p.K = w->k;
+    p.ldx = ldx;
+    p.ldy = ldact;
+    p.gshift = log2_u32(w->group / 32);
+    p.bb = qwhip_view_block_bytes(w);
+    p.row_bytes = qwhip_view_row_bytes(w);
+    p.inter = inter;
+    p.rotate_act = rotate_act ? 1u : 0u;
+    p.tiles_m = qwhip_cdiv(m, 256u);
+    p.tiles_n = qwhip_cdiv(inter, 160u);
+    const dim3 grid(((p.tiles_m * p.tiles_n + 7u) / 8u) * 8u);
+    const hipError_t e = fmt == QG_FMT_M5 ? launch_cfg3<2, 5, 4, 2, QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid)
+                                          : launch_cfg3<2, 5, 4, 2, QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
 }

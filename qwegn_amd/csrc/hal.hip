@@ -255,6 +255,7 @@ static const qw_kernel_entry g_kernels[] = {
     {"qwg_gemv_q4g_silu_pair_dx_h16", "qwhip_gemv_silu_pair"},
     {"qwg_gemm_q4g_h16", "qwhip_gemm"},
     {"qwg_gemm_q4g_nax_f32", "qwhip_gemm"},
+    {"qwg_gemm_q4g_h16_swiglu", "qwhip_gemm_swiglu"},
     {"qwg_silu_mul_f16", "qwhip_swiglu_fwht"},
     {"qwg_silu_mul_f32", "qwhip_swiglu_fwht"},
     {"qwg_silu_mul_split_f16", "qwhip_swiglu_fwht"},
@@ -296,6 +297,7 @@ static bool qw_parse_aq_name(const char* name, const char** launcher) {
     } else if (sscanf(name, "qwg_gemm_aq%u_g%u_%63s", &bits, &group, suffix) == 3) {
         if (!strcmp(suffix, "h16") || !strcmp(suffix, "nax_f32")) lau = "qwhip_gemm";
         else if (!strcmp(suffix, "f32_bm") || !strcmp(suffix, "f32_bm32")) lau = "qwhip_gemv_f32";
+        else if (!strcmp(suffix, "h16_swiglu")) lau = "qwhip_gemm_swiglu";
     } else if (sscanf(name, "qwg_moe_nax_gemm_aq%u_g%u", &bits, &group) == 2 ||
                sscanf(name, "qwg_moe_nax_split_f32_aq%u_g%u", &bits, &group) == 2) {
         lau = "qwhip_moe_grouped_gemm";

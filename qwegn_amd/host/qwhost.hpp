@@ -340,6 +340,25 @@ struct QWGemm {
                                  workspace ? workspace->bytes : 0));
     }
 
+    // gemmBatchedH16SwiGLU (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:156-190, kernel qwg_gemm_*_h16_swiglu):
+    // act16 [rows, inter] = FWHT32(silu(x . Wg^T) * (x . Wu^T)) from a [2 * inter, k] gate|up bank; false when the shape is outside
+    // the fused kernel (the caller then runs gemmBatchedH16 + encodeSiluMulSplitF16).
+    static bool gemmBatchedH16SwiGLU(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWWeightView& w, const QWTensorValue& act16,
+                                     int rows, bool rotate = true, const QWTensorValue* workspace = nullptr, bool rotateInPrepass = false) {
+        if (rows <= 0) throw QWGemmError(QWGemmError::badShape, "rows must be positive");
+        if (act16.shape.dtype != QWDType::f16 || act16.shape.elementCount < (size_t)rows * (size_t)(w.n / 2) ||
+            x.shape.elementCount < (size_t)rows * (size_t)w.k)
+            throw QWGemmError(QWGemmError::badWeights, "fused gate_up: x [rows, k], act f16 [rows, n / 2]");
+        if (w.bits() != 4 || rows % 64 != 0 || w.n % 64 != 0 || w.k % 64 != 0) return false;
+        hal.pipeline(w.containerKind.isIncumbentContainer() ? "qwg_gemm_q4g_h16_swiglu"
+                                                            : ("qwg_gemm_aq4_g" + std::to_string(w.groupSize()) + "_h16_swiglu").c_str());
+        const qwhip_weight_view v = w.abi();
+        throwIfFailed(qwhip_gemm_swiglu(enc.stream, &v, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows, 0, rotate ? 1u : 0u, act16.ptr(), 0,
+                                        rotateInPrepass ? 0u : (uint32_t)QWHIP_X_PREROTATED, workspace ? workspace->ptr() : nullptr,
+                                        workspace ? workspace->bytes : 0));
+        return true;
+    }
+
     // QWGemm.encodeSiluMulF16 / encodeSiluMulSplitF16 (QWGemmF32.swift:47-115): SwiGLU (+FWHT-32) over gate|up rows.
     static void encodeSiluMulSplitF16(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& gu, const QWTensorValue& act16, int rows,
                                       int inter, bool rotate = true) {

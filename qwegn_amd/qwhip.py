@@ -78,6 +78,7 @@ SIGNATURES = {
     "qwhip_moe_max_tiles": (_U32, [_U32, _U32]),
     "qwhip_moe_group_pairs": (C.c_int32, [_P, _P, _U32, _U32, _U32, _P, _P, _P, _P, _P, _P, _P, _U32]),
     "qwhip_moe_grouped_gemm": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _P, _P, _P, _P, _U32, _U32, _P, _U32, _U32]),
+    "qwhip_gemm_swiglu": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _U32, _P, _U32, _U32, _P, C.c_size_t]),
     "qwhip_moe_grouped_gemm_swiglu": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _P, _P, _P, _P, _U32, _U32, _U32, _P, _U32]),
     "qwhip_moe_combine": (C.c_int32, [_P, _P, _U32, _P, _P, _U32, _U32, _U32, _P, _P, _P, _U32]),
     "qwhip_moe_gateup_decode": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _U32, _U32, _P]),

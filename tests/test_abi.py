@@ -81,6 +81,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
         b"qwg_gemm_aq4_g32_f32_bm": b"qwhip_gemv_f32", b"qwg_gemv_aq3_g32_f32_v4_am": b"qwhip_head_argmax", b"qwg_h32_f32": b"qwhip_h32_f32",
         b"qwg_gemv_aq3_g32_v4": b"qwhip_gemv", b"qwg_gemv_aq6_g128_dx_h16_t4": b"qwhip_gemv", b"qwg_gemv_aq2_g64_v4": b"qwhip_gemv",
         b"qwg_gemv_q4g_silu_pair_dx_h16": b"qwhip_gemv_silu_pair", b"qwg_gemv_aq4_g32_silu_pair_dx_h16": b"qwhip_gemv_silu_pair",
+        b"qwg_gemm_q4g_h16_swiglu": b"qwhip_gemm_swiglu", b"qwg_gemm_aq4_g64_h16_swiglu": b"qwhip_gemm_swiglu",
         b"qwg_gemm_q4g_h16": b"qwhip_gemm", b"qwg_gemm_aq8_g32_h16": b"qwhip_gemm", b"qwg_gemm_aq4_g64_nax_f32": b"qwhip_gemm",
         b"qwg_moe_route": b"qwhip_moe_route", b"qwg_moe_group_pairs_f32": b"qwhip_moe_group_pairs",
         b"qwg_moe_nax_gemm": b"qwhip_moe_grouped_gemm", b"qwg_moe_nax_split_f32_aq4_g64": b"qwhip_moe_grouped_gemm",

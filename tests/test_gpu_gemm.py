@@ -129,3 +129,50 @@ def test_gemm_full_size_prefill_config(dev):
     st, out, ref = run_gemm(dev, "hq4_g32_m5", 4096, 5120, 5120, xdtype="bf16", ydtype="bf16")
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt,xdtype,prerot", [("hq4_g32_m5", "f16", True), ("hq4_g32_m5", "bf16", True), ("hq4_g64", "f16", False),
+                                               ("aq4_g32", "f16", True)])
+@pytest.mark.parametrize("m,inter,k,rot", [(64, 160, 128, 1), (256, 352, 256, 1), (320, 1024, 192, 0), (576, 96, 64, 1)])
+def test_gemm_swiglu_equals_gemm_then_swiglu(dev, fmt, xdtype, prerot, m, inter, k, rot):
+    """qwhip_gemm_swiglu == qwhip_gemm (f16 out) + qwhip_swiglu_fwht, bit for bit (column tiles of 160 outputs with a partial
+    last one, several row tiles, bf16 and un-rotated activations through the workspace), and within the bar of the oracle."""
+    n = 2 * inter
+    blocks, w16 = H.make_bank(fmt, n, k, seed=5)
+    x32 = H.make_x(m, k, 12)
+    rotate = H.FORMATS[fmt][4]
+    if xdtype == "bf16":
+        x_val, x_host, xcode = qo.round_bf16(x32), qo.f32_to_bf16_bits(x32), qwhip.BF16
+    else:
+        x_host, xcode = x32.astype(np.float16), qwhip.F16
+        x_val = x_host.astype(np.float32)
+    flags = qwhip.X_PREROTATED if (prerot or not rotate) else 0
+    x_basis = x_val.astype(np.float16) if flags else qo.fwht32_ortho(x_val).astype(np.float16)
+    bank, xb = dev.put(blocks), dev.put(x_host)
+    gu, act2, act1 = dev.alloc(m * n * 2), dev.put(np.zeros((m, inter), np.float16)), dev.put(np.zeros((m, inter), np.float16))
+    ws = dev.alloc(m * k * 2)
+    view = H.view_of(dev, bank, fmt, n, k)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_gemm(st, C.byref(view), xb.ptr, xcode, m, 0, gu.ptr, qwhip.F16, 0, flags, ws.ptr, ws.nbytes))
+    qwhip.check(lib.qwhip_swiglu_fwht(st, gu.ptr, qwhip.F16, act2.ptr, m, inter, rot))
+    qwhip.check(lib.qwhip_gemm_swiglu(st, C.byref(view), xb.ptr, xcode, m, 0, rot, act1.ptr, 0, flags, ws.ptr, ws.nbytes))
+    dev.stream.sync()
+    one, two = act1.download(np.float16, (m, inter)), act2.download(np.float16, (m, inter))
+    assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
+    g = qo.matmul_ref_f64(x_basis, w16).astype(np.float16).astype(np.float32)
+    want = qo.swiglu_fwht_f16(g[:, :inter], g[:, inter:], rotate=bool(rot)).astype(np.float32)
+    assert qo.normalized_error(one.astype(np.float32), want) <= TOL
+
+
+def test_gemm_swiglu_refusals(dev):
+    blocks, _ = H.make_bank("hq8_g32", 128, 64, seed=1)
+    bank, xb, act = dev.put(blocks), dev.put(np.zeros((64, 64), np.float16)), dev.alloc(64 * 64 * 2)
+    v8 = H.view_of(dev, bank, "hq8_g32", 128, 64)
+    lib, st = dev.lib, dev.stream.handle
+    assert lib.qwhip_gemm_swiglu(st, C.byref(v8), xb.ptr, qwhip.F16, 64, 0, 1, act.ptr, 0, qwhip.X_PREROTATED, None, 0) == qwhip.E_BAD_GEOMETRY
+    blocks4, _ = H.make_bank("hq4_g32_m5", 128, 64, seed=1)
+    bank4 = dev.put(blocks4)
+    v4 = H.view_of(dev, bank4, "hq4_g32_m5", 128, 64)
+    assert lib.qwhip_gemm_swiglu(st, C.byref(v4), xb.ptr, qwhip.F16, 37, 0, 1, act.ptr, 0, qwhip.X_PREROTATED, None, 0) == qwhip.E_BAD_GEOMETRY
+    assert lib.qwhip_gemm_swiglu(st, C.byref(v4), xb.ptr, qwhip.F16, 64, 0, 1, act.ptr, 0, 0, None, 0) == qwhip.E_BASIS   # rotation needs the workspace
+    assert lib.qwhip_gemm_swiglu(st, C.byref(v4), xb.ptr, qwhip.BF16, 64, 0, 1, act.ptr, 0, qwhip.X_PREROTATED, None, 0) == qwhip.E_BAD_GEOMETRY
