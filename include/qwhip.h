@@ -59,7 +59,7 @@ typedef struct qwhip_weight_view {
     uint32_t n;
     uint32_t k;
     uint32_t kind;  /* QWHIP_KIND_* */
-    uint32_t bits;  /* 4 for HQ4_G32_M5; {2,3,4,6,8} for blocks (kernels: {4, 8}) */
+    uint32_t bits;  /* 4 for HQ4_G32_M5; {2,3,4,6,8} for blocks */
     uint32_t group; /* 32 for HQ4_G32_M5; {32,64,128,256} for blocks */
 } qwhip_weight_view;
 

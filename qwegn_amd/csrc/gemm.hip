@@ -21,7 +21,13 @@
 #include "qwhip_common.h"
 #include "qw_mfma_2x5.h"
 
-enum { QG_FMT_M5 = 0, QG_FMT_B4 = 1, QG_FMT_B8 = 2 };
+enum { QG_FMT_M5 = 0, QG_FMT_B4 = 1, QG_FMT_B8 = 2, QG_FMT_B2 = 3, QG_FMT_B3 = 4, QG_FMT_B6 = 5 };
+
+// code words of one 32-column slice: 32 * bits / 32
+template <int FMT>
+__host__ __device__ constexpr int qg_slice_words() {
+    return FMT == QG_FMT_B8 ? 8 : FMT == QG_FMT_B2 ? 2 : FMT == QG_FMT_B3 ? 3 : FMT == QG_FMT_B6 ? 6 : 4;
+}
 
 struct qw_gemm_params {
     const uint8_t* bank;
@@ -54,11 +60,13 @@ struct qw_gemm_params {
 
 struct __attribute__((packed, aligned(4))) qg_words4 { uint32_t q[4]; };
 struct __attribute__((packed, aligned(4))) qg_words8 { uint32_t q[8]; };
+template <int W>
+struct __attribute__((packed, aligned(4))) qg_words_n { uint32_t q[W]; };
 
 template <int FMT>
 struct qg_slice {
     uint32_t hdr;
-    uint32_t q[FMT == QG_FMT_B8 ? 8 : 4];
+    uint32_t q[qg_slice_words<FMT>()];
 };
 
 template <int FMT>
@@ -76,10 +84,26 @@ __device__ __forceinline__ void qg_load_slice(const uint8_t* rowp, uint32_t s, u
             const qg_words4 w = *(const qg_words4*)(p + 4 + si * 16u);
 #pragma unroll
             for (int j = 0; j < 4; ++j) o.q[j] = w.q[j];
-        } else {
+        } else if constexpr (FMT == QG_FMT_B8) {
             const qg_words8 w = *(const qg_words8*)(p + 4 + si * 32u);
 #pragma unroll
             for (int j = 0; j < 8; ++j) o.q[j] = w.q[j];
+        } else {
+            // 2-, 3- and 6-bit streams: a slice is `bits` words, at a 4-byte aligned offset of the block
+            constexpr int W = qg_slice_words<FMT>();
+            const uint8_t* src = p + 4 + si * (4u * W);
+            if constexpr (W == 6) {   // 24 bytes as 16 + 8: one aggregate of six words is left in scratch memory by the compiler
+                const qg_words4 w0 = *(const qg_words4*)src;
+                const qg_words_n<2> w1 = *(const qg_words_n<2>*)(src + 16);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o.q[j] = w0.q[j];
+                o.q[4] = w1.q[0];
+                o.q[5] = w1.q[1];
+            } else {
+                const qg_words_n<W> w = *(const qg_words_n<W>*)src;
+#pragma unroll
+                for (int j = 0; j < W; ++j) o.q[j] = w.q[j];
+            }
         }
     }
 }
@@ -100,6 +124,29 @@ __device__ __forceinline__ h8_t qg_dequant_chunk(const qg_slice<FMT>& sl, int j,
             // bytes: [lo.b_k, 0, hi.b_k, 0]
             const uint32_t sel = 0x0C000C00u | (uint32_t)k | ((uint32_t)(4 + k) << 16);
             const uint32_t m = __builtin_amdgcn_perm(hi, lo, sel) | 0x64006400u;
+            w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m) + neg, s2, b2);
+        }
+    } else if constexpr (FMT == QG_FMT_B2 || FMT == QG_FMT_B3 || FMT == QG_FMT_B6) {
+        // bit stream of W-bit codes: the chunk's 8 codes are the 8 W bits from bit 8 W j of the slice.  j is a constant
+        // after unrolling at every call site, so the word picks and shifts fold.
+        constexpr int W = qg_slice_words<FMT>();
+        const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
+        const int o = 8 * W * j, wi = o >> 5, sh = o & 31;
+        // word picks as select chains over constant indices: they fold to one register for a constant j and never turn
+        // into an indexed (scratch memory) access
+        uint32_t lo32 = 0, hi32 = 0;
+#pragma unroll
+        for (int t = 0; t < W; ++t) {
+            lo32 = wi == t ? sl.q[t] : lo32;
+            hi32 = wi + 1 == t ? sl.q[t] : hi32;
+        }
+        const uint64_t lo = lo32, hi = hi32;
+        const uint64_t win = (lo | (hi << 32)) >> sh;
+        constexpr uint32_t mask = (1u << W) - 1u;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t c0 = (uint32_t)(win >> (2 * k * W)) & mask, c1 = (uint32_t)(win >> ((2 * k + 1) * W)) & mask;
+            const uint32_t m = c0 | (c1 << 16) | 0x64006400u;
             w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m) + neg, s2, b2);
         }
     } else {
@@ -1395,8 +1442,9 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     switch (cfg) {
         case CFG_256x320:
             // the ping-pong kernel takes whole 64-row activation blocks; ragged M stays on the DMA-fed kernel, and so do the
-            // 8-bit containers: their wider weight items do not fit the ping-pong kernel's register budget at this tile
-            if constexpr (FMT != QG_FMT_B8) {
+            // 8-bit containers: their wider weight items do not fit the ping-pong kernel's register budget at this tile; the
+            // 2-, 3- and 6-bit streams stay there too (the ping-pong kernel splits a slice's words between two stores)
+            if constexpr (FMT == QG_FMT_M5 || FMT == QG_FMT_B4) {
                 if (p.M % 64u == 0 && !p.force_gemm2 &&
                     (YDT == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0)))
                     return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
@@ -1463,9 +1511,24 @@ qwhip_status gemm_checks(qwhip_stream_t s, const qwhip_weight_view* w, const voi
     if (w->kind == QWHIP_KIND_HQ4_G32_M5) *fmt = QG_FMT_M5;
     else if (w->bits == 4) *fmt = QG_FMT_B4;
     else if (w->bits == 8) *fmt = QG_FMT_B8;
+    else if (w->bits == 2) *fmt = QG_FMT_B2;
+    else if (w->bits == 3) *fmt = QG_FMT_B3;
+    else if (w->bits == 6) *fmt = QG_FMT_B6;
     else return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no tensor GEMM kernel for %u-bit group %u", w->bits, w->group);
     return QWHIP_OK;
 }
+
+// runs EXPR with F bound to the container format as a constant
+#define QG_FOR_FMT(fmt, e, EXPR)                                                  \
+    switch (fmt) {                                                                \
+        case QG_FMT_M5: { constexpr int F = QG_FMT_M5; e = (EXPR); } break;       \
+        case QG_FMT_B4: { constexpr int F = QG_FMT_B4; e = (EXPR); } break;       \
+        case QG_FMT_B8: { constexpr int F = QG_FMT_B8; e = (EXPR); } break;       \
+        case QG_FMT_B2: { constexpr int F = QG_FMT_B2; e = (EXPR); } break;       \
+        case QG_FMT_B3: { constexpr int F = QG_FMT_B3; e = (EXPR); } break;       \
+        case QG_FMT_B6: { constexpr int F = QG_FMT_B6; e = (EXPR); } break;       \
+        default: e = hipErrorInvalidValue;                                        \
+    }
 
 }  // namespace
 
@@ -1524,20 +1587,14 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     hipError_t e;
     if (xdt != QWHIP_F16 || ov == 15u) {
         if (xdt == QWHIP_F16) {
-            if (fmt == QG_FMT_M5) e = launch_dense1_y<QG_FMT_M5, QWHIP_F16>(s->stream, p, y_dtype);
-            else if (fmt == QG_FMT_B4) e = launch_dense1_y<QG_FMT_B4, QWHIP_F16>(s->stream, p, y_dtype);
-            else e = launch_dense1_y<QG_FMT_B8, QWHIP_F16>(s->stream, p, y_dtype);
+            QG_FOR_FMT(fmt, e, (launch_dense1_y<F, QWHIP_F16>(s->stream, p, y_dtype)))
         } else {
-            if (fmt == QG_FMT_M5) e = launch_dense1_y<QG_FMT_M5, QWHIP_BF16>(s->stream, p, y_dtype);
-            else if (fmt == QG_FMT_B4) e = launch_dense1_y<QG_FMT_B4, QWHIP_BF16>(s->stream, p, y_dtype);
-            else e = launch_dense1_y<QG_FMT_B8, QWHIP_BF16>(s->stream, p, y_dtype);
+            QG_FOR_FMT(fmt, e, (launch_dense1_y<F, QWHIP_BF16>(s->stream, p, y_dtype)))
         }
     } else {
         const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n));
         p.force_gemm2 = ov == 14u ? 1u : 0u;
-        if (fmt == QG_FMT_M5) e = launch_dense2_y<QG_FMT_M5>(s->stream, p, cfg, y_dtype);
-        else if (fmt == QG_FMT_B4) e = launch_dense2_y<QG_FMT_B4>(s->stream, p, cfg, y_dtype);
-        else e = launch_dense2_y<QG_FMT_B8>(s->stream, p, cfg, y_dtype);
+        QG_FOR_FMT(fmt, e, (launch_dense2_y<F>(s->stream, p, cfg, y_dtype)))
     }
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
@@ -1555,7 +1612,7 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     if (m == 0) return QWHIP_OK;
     const uint32_t inter = w->n / 2u;
     if (w->n % 64u != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "fused gate_up needs an intermediate size %% 32 == 0, got %u rows", w->n);
-    if (fmt == QG_FMT_B8 || m % 64u != 0)
+    if ((fmt != QG_FMT_M5 && fmt != QG_FMT_B4) || m % 64u != 0)
         return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the fused gate_up GEMM takes 4-bit containers and m %% 64 == 0 (m=%u): run qwhip_gemm + qwhip_swiglu_fwht", m);
     if (ldx == 0) ldx = w->k;
     if (ldact == 0) ldact = inter;
@@ -1682,9 +1739,7 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_wei
     p.rows_per_expert = rows_per_expert;
     const dim3 grid(qwhip_cdiv(rows_per_expert, 256u), max_tiles);
     hipError_t e;
-    if (fmt == QG_FMT_M5) e = launch_grouped_xy<QG_FMT_M5>(s->stream, p, grid, x_dtype, y_dtype);
-    else if (fmt == QG_FMT_B4) e = launch_grouped_xy<QG_FMT_B4>(s->stream, p, grid, x_dtype, y_dtype);
-    else e = launch_grouped_xy<QG_FMT_B8>(s->stream, p, grid, x_dtype, y_dtype);
+    QG_FOR_FMT(fmt, e, (launch_grouped_xy<F>(s->stream, p, grid, x_dtype, y_dtype)))
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
 }
@@ -1742,9 +1797,9 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     hipError_t e;
     if (gemm5_takes(p, fmt)) e = fmt == QG_FMT_M5 ? launch_cfg5<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid)
                                                   : launch_cfg5<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
-    else if (fmt == QG_FMT_M5) e = launch_cfg4<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid);
-    else if (fmt == QG_FMT_B4) e = launch_cfg4<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
-    else e = launch_cfg4<QG_FMT_B8, QWHIP_F16, true>(s->stream, p, grid);
+    else {
+        QG_FOR_FMT(fmt, e, (launch_cfg4<F, QWHIP_F16, true>(s->stream, p, grid)))
+    }
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
 }

@@ -157,19 +157,27 @@ __global__ __launch_bounds__(256) void qw_gemv_hq4_dot2_kernel(const uint8_t* __
 // ------------------------------------------------------------------------------------------------
 // Variant B: MFMA streamer, all containers, m = 1..16.
 // ------------------------------------------------------------------------------------------------
+// code words of one 32-column slice (= the bit width)
+template <int FMT>
+__host__ __device__ constexpr int qw_slice_words() {
+    return FMT == QW_FMT_B8 ? 8 : FMT == QW_FMT_B2 ? 2 : FMT == QW_FMT_B3 ? 3 : FMT == QW_FMT_B6 ? 6 : 4;
+}
+
 template <int FMT>
 struct qw_slice {
     uint32_t hdr;
-    uint32_t q[FMT == QW_FMT_B8 ? 8 : 4];
+    uint32_t q[qw_slice_words<FMT>()];
 };
 
 struct __attribute__((packed, aligned(4))) qw_words4 { uint32_t q[4]; };
 struct __attribute__((packed, aligned(4))) qw_words8 { uint32_t q[8]; };
+template <int W>
+struct __attribute__((packed, aligned(4))) qw_words_n { uint32_t q[W]; };
 
 // Position e of an A operand holds element perm(e) of the 8-column chunk.
 template <int FMT>
 __device__ __forceinline__ constexpr int qw_perm(int e) {
-    if (FMT == QW_FMT_M5) return e;
+    if (FMT == QW_FMT_M5 || FMT >= QW_FMT_B2) return e;        // 2-, 3- and 6-bit streams are cut out in natural order
     if (FMT == QW_FMT_B4) return (e >> 1) + 4 * (e & 1);      // 0,4,1,5,2,6,3,7
     return (e & 4) + ((e & 1) << 1) + ((e >> 1) & 1);         // 0,2,1,3,4,6,5,7
 }
@@ -191,10 +199,26 @@ __device__ __forceinline__ void qw_load_slice(const uint8_t* rowp, uint32_t s, u
             const qw_words4 w = *(const qw_words4*)(p + 4 + si * 16u);
 #pragma unroll
             for (int j = 0; j < 4; ++j) o.q[j] = w.q[j];
-        } else {
+        } else if constexpr (FMT == QW_FMT_B8) {
             const qw_words8 w = *(const qw_words8*)(p + 4 + si * 32u);
 #pragma unroll
             for (int j = 0; j < 8; ++j) o.q[j] = w.q[j];
+        } else {
+            // 2-, 3- and 6-bit streams: a slice is `bits` words at a 4-byte aligned offset of the block
+            constexpr int W = qw_slice_words<FMT>();
+            const uint8_t* src = p + 4 + si * (4u * W);
+            if constexpr (W == 6) {
+                const qw_words4 w0 = *(const qw_words4*)src;
+                const qw_words_n<2> w1 = *(const qw_words_n<2>*)(src + 16);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o.q[j] = w0.q[j];
+                o.q[4] = w1.q[0];
+                o.q[5] = w1.q[1];
+            } else {
+                const qw_words_n<W> w = *(const qw_words_n<W>*)src;
+#pragma unroll
+                for (int j = 0; j < W; ++j) o.q[j] = w.q[j];
+            }
         }
     }
 }
@@ -214,6 +238,25 @@ __device__ __forceinline__ h8_t qw_dequant_chunk(const qw_slice<FMT>& sl, int j,
         for (int k = 0; k < 4; ++k) {
             const uint32_t m = qw_and_or(sl.q[j] >> (4 * k), 0x000F000Fu, magic);
             w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, m) + neg, s2, b2);
+        }
+    } else if constexpr (FMT >= QW_FMT_B2) {
+        // the chunk's 8 codes are the 8 W bits from bit 8 W j of the slice; j is a constant after unrolling, and the word
+        // picks are select chains over constant indices so that they never become an indexed (scratch memory) access
+        constexpr int W = qw_slice_words<FMT>();
+        const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
+        const int o = 8 * W * j, wi = o >> 5, sh = o & 31;
+        uint32_t lo32 = 0, hi32 = 0;
+#pragma unroll
+        for (int t = 0; t < W; ++t) {
+            lo32 = wi == t ? sl.q[t] : lo32;
+            hi32 = wi + 1 == t ? sl.q[t] : hi32;
+        }
+        const uint64_t win = ((uint64_t)lo32 | ((uint64_t)hi32 << 32)) >> sh;
+        constexpr uint32_t mask = (1u << W) - 1u;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t c0 = (uint32_t)(win >> (2 * k * W)) & mask, c1 = (uint32_t)(win >> ((2 * k + 1) * W)) & mask;
+            w[k] = __builtin_elementwise_fma(__builtin_bit_cast(h2_t, c0 | (c1 << 16) | magic) + neg, s2, b2);
         }
     } else {
         const h2_t neg = {(h1_t)-1024.0f, (h1_t)-1024.0f};
@@ -1086,7 +1129,6 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     int fmt = 0;
     qwhip_status st = check_common(s, w, x, x_dtype, m, &fmt);
     if (st != QWHIP_OK) return st;
-    if (fmt >= QW_FMT_B2) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no gate|up kernel for %u-bit group %u", w->bits, w->group);
     QWHIP_REQUIRE(act16);
     if (w->n % 2 != 0) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "gate|up bank needs an even row count, got %u", w->n);
     const uint32_t inter = w->n / 2;
@@ -1116,9 +1158,14 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     const size_t lds_x = (size_t)m * ((size_t)w->k * 2u + 16u);
     const int xm = (rotate && lds_x <= 48u * 1024u) ? QW_XM_LDS_ROT : QW_XM_GLOBAL;
     const size_t lds = xm == QW_XM_LDS_ROT ? lds_x : 0;
-    if (fmt == QW_FMT_M5) launch_mfma_dt<QW_FMT_M5, 2, 1>(s->stream, a, x_dtype, xm, lds);
-    else if (fmt == QW_FMT_B4) launch_mfma_dt<QW_FMT_B4, 2, 1>(s->stream, a, x_dtype, xm, lds);
-    else launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds);
+    switch (fmt) {
+        case QW_FMT_M5: launch_mfma_dt<QW_FMT_M5, 2, 1>(s->stream, a, x_dtype, xm, lds); break;
+        case QW_FMT_B4: launch_mfma_dt<QW_FMT_B4, 2, 1>(s->stream, a, x_dtype, xm, lds); break;
+        case QW_FMT_B8: launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds); break;
+        case QW_FMT_B2: launch_mfma_dt<QW_FMT_B2, 2, 1>(s->stream, a, x_dtype, xm, lds); break;
+        case QW_FMT_B3: launch_mfma_dt<QW_FMT_B3, 2, 1>(s->stream, a, x_dtype, xm, lds); break;
+        default: launch_mfma_dt<QW_FMT_B6, 2, 1>(s->stream, a, x_dtype, xm, lds); break;
+    }
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
@@ -1167,7 +1214,6 @@ extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_we
     int fmt = 0;
     qwhip_status st = check_common(s, w_gate_up, x, x_dtype, 1, &fmt);
     if (st != QWHIP_OK) return st;
-    if (fmt >= QW_FMT_B2) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no routed kernel for %u-bit group %u", w_gate_up->bits, w_gate_up->group);
     QWHIP_REQUIRE(idx);
     QWHIP_REQUIRE(act16);
     if (t == 0 || top_k == 0) return QWHIP_OK;
@@ -1204,9 +1250,14 @@ extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_we
     const int xm = (rotate && lds_x <= 48u * 1024u) ? QW_XM_LDS_ROT : QW_XM_GLOBAL;
     const size_t lds = xm == QW_XM_LDS_ROT ? lds_x : 0;
     const uint32_t pairs = t * top_k;
-    if (fmt == QW_FMT_M5) launch_mfma_dt<QW_FMT_M5, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs);
-    else if (fmt == QW_FMT_B4) launch_mfma_dt<QW_FMT_B4, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs);
-    else launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs);
+    switch (fmt) {
+        case QW_FMT_M5: launch_mfma_dt<QW_FMT_M5, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs); break;
+        case QW_FMT_B4: launch_mfma_dt<QW_FMT_B4, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs); break;
+        case QW_FMT_B8: launch_mfma_dt<QW_FMT_B8, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs); break;
+        case QW_FMT_B2: launch_mfma_dt<QW_FMT_B2, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs); break;
+        case QW_FMT_B3: launch_mfma_dt<QW_FMT_B3, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs); break;
+        default: launch_mfma_dt<QW_FMT_B6, 2, 1>(s->stream, a, x_dtype, xm, lds, pairs); break;
+    }
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
@@ -1217,7 +1268,6 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
     int fmt = 0;
     qwhip_status st = check_common(s, w_down, act16, QWHIP_F16, 1, &fmt);
     if (st != QWHIP_OK) return st;
-    if (fmt >= QW_FMT_B2) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "no routed kernel for %u-bit group %u", w_down->bits, w_down->group);
     QWHIP_REQUIRE(idx);
     QWHIP_REQUIRE(wts);
     QWHIP_REQUIRE(out);
@@ -1260,7 +1310,8 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
         case QWHIP_BF16: QW_DD(F, QWHIP_BF16); break;                                                       \
         default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe down: unsupported output dtype %u", out_dtype);  \
     }
-    if (fmt == QW_FMT_M5) { QW_DD_O(QW_FMT_M5) } else if (fmt == QW_FMT_B4) { QW_DD_O(QW_FMT_B4) } else { QW_DD_O(QW_FMT_B8) }
+    if (fmt == QW_FMT_M5) { QW_DD_O(QW_FMT_M5) } else if (fmt == QW_FMT_B4) { QW_DD_O(QW_FMT_B4) } else if (fmt == QW_FMT_B8) { QW_DD_O(QW_FMT_B8) }
+    else if (fmt == QW_FMT_B2) { QW_DD_O(QW_FMT_B2) } else if (fmt == QW_FMT_B3) { QW_DD_O(QW_FMT_B3) } else { QW_DD_O(QW_FMT_B6) }
 #undef QW_DD_O
 #undef QW_DD
     QWHIP_TRY_HIP(hipGetLastError());

@@ -307,9 +307,9 @@ static bool qw_parse_aq_name(const char* name, const char** launcher) {
         lau = "qwhip_moe_down_decode";
     }
     if (!lau) return false;
-    // the 2-, 3- and 6-bit streams have the decode GEMVs only (f16/bf16 and f32 activations, and the head built on them)
-    const bool decode_gemv = !strcmp(lau, "qwhip_gemv") || !strcmp(lau, "qwhip_gemv_f32") || !strcmp(lau, "qwhip_head_argmax");
-    if (!(bits == 4 || bits == 8 || (decode_gemv && (bits == 2 || bits == 3 || bits == 6)))) return false;
+    // every door takes the five widths except the fused dense gate|up GEMM (the ping-pong kernel's 4- and 8-bit name space)
+    const bool narrow_ok = strcmp(lau, "qwhip_gemm_swiglu") != 0;
+    if (!(bits == 4 || bits == 8 || (narrow_ok && (bits == 2 || bits == 3 || bits == 6)))) return false;
     if (!(group == 32 || group == 64 || group == 128 || group == 256)) return false;
     if (launcher) *launcher = lau;
     return true;

@@ -54,7 +54,7 @@ typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
 
 // GEMV container families: HQ4_G32_M5 20-byte blocks, 4-bit and 8-bit bit-stream blocks.
-enum { QW_FMT_M5 = 0, QW_FMT_B4 = 1, QW_FMT_B8 = 2, QW_FMT_B2 = 3, QW_FMT_B3 = 4, QW_FMT_B6 = 5 };   // B2/B3/B6: decode kernels only
+enum { QW_FMT_M5 = 0, QW_FMT_B4 = 1, QW_FMT_B8 = 2, QW_FMT_B2 = 3, QW_FMT_B3 = 4, QW_FMT_B6 = 5 };   // B2/B3/B6: 2-, 3- and 6-bit streams
 
 #define QW_INV_SQRT32 0.17677669529663689f /* f32(1/sqrt(32)) = 0x3E3504F3 */
 

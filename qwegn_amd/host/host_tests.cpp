@@ -87,7 +87,8 @@ static void test_error_mapping() {
     CHECK_THROWS(throwIfFailed(QWHIP_E_BAD_GEOMETRY), QWGemmError, QWGemmError::badGeometry);
     CHECK_THROWS(throwIfFailed(QWHIP_E_KERNEL_MISSING), QWHalError, QWHalError::kernelMissing);
     CHECK(QWGemm::moeMaxTiles(128, 16384) == 384 && QWGemm::moeMaxTiles(128, 5) == 5);
-    CHECK(QWGemmAQ::kernelName(8, 32).value_or("") == "qwg_gemv_aq8_g32_v4" && !QWGemmAQ::kernelName(3, 32).has_value());
+    CHECK(QWGemmAQ::kernelName(8, 32).value_or("") == "qwg_gemv_aq8_g32_v4" && QWGemmAQ::kernelName(3, 32).value_or("") == "qwg_gemv_aq3_g32_v4" &&
+          !QWGemmAQ::kernelName(5, 32).has_value() && !QWGemmAQ::kernelName(4, 48).has_value());
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -392,8 +392,7 @@ struct QWGemm {
                                    const QWTensorValue& naxX16, int rows, uint32_t epi = 0, float scale = 1.0f,
                                    const QWTensorValue* x16Precast = nullptr, int minNaxRows = 64) {
         const int effectiveMinNax = minNaxRows > 64 ? minNaxRows : 64;
-        if (rows >= effectiveMinNax && epi == 0 && scale == 1.0f && w.n % 64 == 0 && w.k % 64 == 0 && w.bits() != 2 && w.bits() != 3 &&
-            w.bits() != 6) {
+        if (rows >= effectiveMinNax && epi == 0 && scale == 1.0f && w.n % 64 == 0 && w.k % 64 == 0) {
             const size_t count = (size_t)rows * (size_t)w.k;
             if (x16Precast) {
                 gemmBatchedH16(enc, hal, x16Precast->slice(0, count, QWDType::f16), w, y, rows);
@@ -546,7 +545,7 @@ struct QWGemm {
 // ---- QWGemmAQ (Sources/Operators/QWGEMM/QWGemmAQ.swift:192-304): the bit-stream block family ----------------------
 struct QWGemmAQ {
     static std::optional<std::string> kernelName(int bits, int group) {
-        if (!(bits == 4 || bits == 8)) return std::nullopt;
+        if (!(bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8)) return std::nullopt;   // QWAQBlock.swift:17-23
         if (!(group == 32 || group == 64 || group == 128 || group == 256)) return std::nullopt;
         return "qwg_gemv_aq" + std::to_string(bits) + "_g" + std::to_string(group) + "_v4";
     }

@@ -16,7 +16,7 @@ FORMATS = {
     "hq8_g32": (qwhip.KIND_ROTATED_HQ, 8, 32, False, True),
     "hq8_g64": (qwhip.KIND_ROTATED_HQ, 8, 64, False, True),
     "aq8_g256": (qwhip.KIND_NATIVE_AFFINE, 8, 256, False, False),
-    # 2-, 3- and 6-bit streams: decode GEMV only
+    # 2-, 3- and 6-bit streams
     "aq2_g64": (qwhip.KIND_NATIVE_AFFINE, 2, 64, False, False),
     "hq3_g32": (qwhip.KIND_ROTATED_HQ, 3, 32, False, True),
     "hq6_g32": (qwhip.KIND_ROTATED_HQ, 6, 32, False, True),

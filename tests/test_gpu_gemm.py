@@ -72,12 +72,22 @@ def test_gemm_ragged_shapes(dev, m, n, k):
     assert qo.normalized_error(out, ref) <= 2e-5
 
 
-@pytest.mark.parametrize("fmt", ["aq4_g32", "hq4_g64", "hq8_g32", "hq4_g128", "aq8_g256"])
+@pytest.mark.parametrize("fmt", ["aq4_g32", "hq4_g64", "hq8_g32", "hq4_g128", "aq8_g256", "aq2_g64", "hq3_g32", "hq6_g32", "aq6_g128"])
 @pytest.mark.parametrize("xdtype,ydtype", [("f16", "f16"), ("bf16", "bf16")])
 def test_gemm_block_formats(dev, fmt, xdtype, ydtype):
     st, out, ref = run_gemm(dev, fmt, 192, 256, 768, xdtype=xdtype, ydtype=ydtype, seed=3)
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["aq2_g64", "hq3_g32", "hq6_g32", "aq6_g128"])
+@pytest.mark.parametrize("cfg,xdtype,workspace", [(15, "f16", True), (0, "bf16", False), (1, "f16", True), (2, "f16", True), (3, "f16", True)])
+def test_gemm_narrow_and_six_bit_streams_on_every_kernel(dev, fmt, cfg, xdtype, workspace):
+    """2-, 3- and 6-bit streams (codes cut out of the slice's words, also across word boundaries) on the unpipelined kernel
+    (f16, and bf16 converted in the tile) and on the DMA-fed kernel's tile shapes, fp32 out, ragged in both directions."""
+    st, out, ref = run_gemm(dev, fmt, 300, 336, 384, xdtype=xdtype, ydtype="f32", cfg=cfg, seed=11, workspace=workspace)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= 2e-5
 
 
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "aq4_g32", "hq8_g32", "hq4_g64"])

@@ -149,7 +149,7 @@ def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
     assert qo.normalized_error(got, ref) <= TOL
 
 
-@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g32", "hq4_g64", "hq8_g32"])
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g32", "hq4_g64", "hq8_g32", "aq2_g64", "hq3_g32", "hq6_g32"])
 @pytest.mark.parametrize("t,experts,hidden,inter,k,rot", [(40, 8, 256, 128, 2, 1), (130, 16, 512, 192, 4, 1), (300, 4, 128, 64, 2, 0),
                                                           (64, 8, 192, 448, 3, 1)])
 def test_fused_gate_up_swiglu_equals_the_two_step_chain(dev, fmt, t, experts, hidden, inter, k, rot):
@@ -198,7 +198,7 @@ def test_fused_gate_up_swiglu_refusals(dev):
 
 # (format, gate_up kernel override): HQ4_G32_M5 runs the column-stationary kernels, override 2 keeps its gate_up on the
 # general kernel; the bit-stream container runs the general kernels for both projections.
-@pytest.mark.parametrize("fmt,gu_flags", [("hq4_g32_m5", 0), ("hq4_g32_m5", 2 << 8), ("hq4_g32", 0)])
+@pytest.mark.parametrize("fmt,gu_flags", [("hq4_g32_m5", 0), ("hq4_g32_m5", 2 << 8), ("hq4_g32", 0), ("hq3_g32", 0), ("hq6_g32", 0)])
 @pytest.mark.parametrize("experts,hidden,inter,k", [(16, 512, 192, 4), (8, 1280, 96, 3), (4, 2048, 768, 4)])
 @pytest.mark.parametrize("t", [1, 3, 8])
 @pytest.mark.parametrize("xdt", ["f16", "bf16"])
