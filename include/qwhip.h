@@ -225,6 +225,12 @@ qwhip_status qwhip_moe_route(qwhip_stream_t s, const float* logits, uint32_t t, 
  * logits[t, e] = sum_h x[t, h] * Wr[e, h]; x f16/bf16/f32, Wr f32/f16/bf16, fp32 accumulate. */
 qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
                                uint32_t t, uint32_t experts, uint32_t hidden, float* logits);
+/* The same launch with the shared-expert gate column (encodeFnRouterGemm's shGateWeight / shGateOut,
+ * QWGemmMoERouter.swift:78-113; qwrouter.metal:467-483,566-574,587-633): sh_gate_out[t] = sigmoid(x[t] . sh_gate_w),
+ * sh_gate_w fp32 [hidden].  Both pointers, or neither (then it is qwhip_router_gemm).  hidden <= 16384. */
+qwhip_status qwhip_router_gemm_shared_gate(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
+                                           uint32_t t, uint32_t experts, uint32_t hidden, float* logits,
+                                           const float* sh_gate_w, float* sh_gate_out);
 
 /* Scratch sizes of the pair sort (MoETilePlan, Sources/Operators/QWGEMM/QWGemmMoE.swift:24-62). */
 uint32_t qwhip_moe_max_tiles(uint32_t experts, uint32_t pairs);

@@ -552,6 +552,13 @@ def swiglu_fwht_f16(gate, up, rotate: bool = True) -> np.ndarray:
 # --------------------------------------------------------------------------- #
 # MoE router  (pinned: golden fn_sparse_moe_golden.json end to end; math: textbook softmax/top-k, tie rule)
 # --------------------------------------------------------------------------- #
+def router_shared_gate_f64(x: np.ndarray, sh_gate_w: np.ndarray) -> np.ndarray:
+    """Shared-expert gate of the router launch: sigmoid(x[t] . w), one scalar per token row
+    (Sources/QWMetal/subsystems/qwrouter.metal:566-574,633; QWGemmMoERouter.swift:69-113 shGateWeight / shGateOut)."""
+    v = np.asarray(x, dtype=np.float64) @ np.asarray(sh_gate_w, dtype=np.float64).reshape(-1)
+    return 1.0 / (1.0 + np.exp(-v))
+
+
 def moe_route(logits: np.ndarray, top_k: int, norm_topk: bool = True, routed_scale: float = 1.0):
     """f32 softmax (max-subtracted) -> K rounds of argmax, ties to the LOWER index ->
     weights renormalised by the sum of the selected -> x routed scale.

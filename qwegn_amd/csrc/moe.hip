@@ -5,13 +5,16 @@
 
 // ------------------------------------------------------------------------------------------------
 // Router logits: logits[t, e] = sum_h x[t, h] * Wr[e, h], fp32 accumulate.
-// A workgroup owns 8 token rows (staged as fp32 in LDS) so each router row is read once per 8 tokens;
-// a wavefront owns experts wave, wave+4, ...; lanes stride the hidden dimension.
+// A workgroup owns TT token rows (staged as fp32 in LDS; 8 rows up to hidden = 2048, fewer on wider rows so the tile
+// stays within 64 KiB) so each router row is read once per TT tokens; a wavefront owns experts wave, wave+4, ...;
+// lanes stride the hidden dimension.  With a shared-expert gate row (fp32 [hidden]) the workgroup also writes
+// sh_out[t] = sigmoid(x[t] . sh_w), the extra output column of the reference's router kernels
+// (Sources/QWMetal/subsystems/qwrouter.metal:467-483,566-574,587-633).
 // ------------------------------------------------------------------------------------------------
-template <int XDT, int WDT>
+template <int XDT, int WDT, int TT>
 __global__ __launch_bounds__(256) void qw_router_gemm_kernel(const void* __restrict__ x, const void* __restrict__ wr,
-                                                              float* __restrict__ logits, uint32_t T, uint32_t E, uint32_t H) {
-    constexpr int TT = 8;
+                                                              float* __restrict__ logits, uint32_t T, uint32_t E, uint32_t H,
+                                                              const float* __restrict__ sh_w, float* __restrict__ sh_out) {
     extern __shared__ float xs[];  // [TT][H]
     const uint32_t t0 = blockIdx.x * TT;
     const uint32_t nt = min((uint32_t)TT, T - t0);
@@ -21,40 +24,59 @@ __global__ __launch_bounds__(256) void qw_router_gemm_kernel(const void* __restr
     }
     __syncthreads();
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    for (uint32_t e = wave; e < E; e += 4) {
+    const uint32_t rows = E + (sh_w ? 1u : 0u);
+    for (uint32_t e = wave; e < rows; e += 4) {
+        const bool gate_row = e == E;   // wave-uniform
         float acc[TT];
 #pragma unroll
         for (int r = 0; r < TT; ++r) acc[r] = 0.0f;
         for (uint32_t h = lane; h < H; h += 64) {
-            const float w = qw_load_f32<WDT>(wr, (uint64_t)e * H + h);
+            const float w = gate_row ? sh_w[h] : qw_load_f32<WDT>(wr, (uint64_t)e * H + h);
 #pragma unroll
             for (int r = 0; r < TT; ++r) acc[r] = fmaf(w, xs[r * H + h], acc[r]);
         }
 #pragma unroll
         for (int r = 0; r < TT; ++r) {
             const float v = qw_reduce64(acc[r]);
-            if (lane == 0 && (uint32_t)r < nt) logits[(uint64_t)(t0 + r) * E + e] = v;
+            if (lane == 0 && (uint32_t)r < nt) {
+                if (gate_row) sh_out[t0 + r] = 1.0f / (1.0f + expf(-v));
+                else logits[(uint64_t)(t0 + r) * E + e] = v;
+            }
         }
     }
 }
 
-extern "C" qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
-                                          uint32_t t, uint32_t experts, uint32_t hidden, float* logits) {
+extern "C" qwhip_status qwhip_router_gemm_shared_gate(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
+                                                      uint32_t t, uint32_t experts, uint32_t hidden, float* logits,
+                                                      const float* sh_gate_w, float* sh_gate_out) {
     QWHIP_REQUIRE(s);
     if (t == 0) return QWHIP_OK;
     QWHIP_REQUIRE(x);
     QWHIP_REQUIRE(wr);
     QWHIP_REQUIRE(logits);
+    if ((sh_gate_w != nullptr) != (sh_gate_out != nullptr))
+        return qwhip_fail(QWHIP_E_NULL, "router gemm: the shared-expert gate needs both its weight row and its output");
     if (experts == 0 || hidden == 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: empty experts or hidden");
-    const size_t lds = (size_t)8 * hidden * 4;
-    if (lds > 64u * 1024u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: hidden %u exceeds the staged tile (<= 2048)", hidden);
-    const dim3 grid(qwhip_cdiv(t, 8)), block(256);
-#define QW_RG(XD, WD) hipLaunchKernelGGL((qw_router_gemm_kernel<XD, WD>), grid, block, lds, s->stream, x, wr, logits, t, experts, hidden)
+    // token rows per workgroup: the fp32 tile stays within 64 KiB
+    uint32_t tt = 8;
+    while (tt > 1u && (size_t)tt * hidden * 4u > 64u * 1024u) tt >>= 1;
+    const size_t lds = (size_t)tt * hidden * 4u;
+    if (lds > 64u * 1024u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: hidden %u exceeds the staged row (<= 16384)", hidden);
+    const dim3 grid(qwhip_cdiv(t, tt)), block(256);
+#define QW_RG(XD, WD, TT) \
+    hipLaunchKernelGGL((qw_router_gemm_kernel<XD, WD, TT>), grid, block, lds, s->stream, x, wr, logits, t, experts, hidden, sh_gate_w, sh_gate_out)
+#define QW_RG_T(XD, WD)                       \
+    switch (tt) {                             \
+        case 8: QW_RG(XD, WD, 8); break;      \
+        case 4: QW_RG(XD, WD, 4); break;      \
+        case 2: QW_RG(XD, WD, 2); break;      \
+        default: QW_RG(XD, WD, 1); break;     \
+    }
 #define QW_RG_W(XD)                                                   \
     switch (w_dtype) {                                                \
-        case QWHIP_F32: QW_RG(XD, QWHIP_F32); break;                  \
-        case QWHIP_F16: QW_RG(XD, QWHIP_F16); break;                  \
-        case QWHIP_BF16: QW_RG(XD, QWHIP_BF16); break;                \
+        case QWHIP_F32: QW_RG_T(XD, QWHIP_F32) break;                 \
+        case QWHIP_F16: QW_RG_T(XD, QWHIP_F16) break;                 \
+        case QWHIP_BF16: QW_RG_T(XD, QWHIP_BF16) break;               \
         default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: unsupported weight dtype %u", w_dtype); \
     }
     switch (x_dtype) {
@@ -64,9 +86,15 @@ extern "C" qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint3
         default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: unsupported activation dtype %u", x_dtype);
     }
 #undef QW_RG_W
+#undef QW_RG_T
 #undef QW_RG
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
+}
+
+extern "C" qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
+                                          uint32_t t, uint32_t experts, uint32_t hidden, float* logits) {
+    return qwhip_router_gemm_shared_gate(s, x, x_dtype, wr, w_dtype, t, experts, hidden, logits, nullptr, nullptr);
 }
 
 // ------------------------------------------------------------------------------------------------

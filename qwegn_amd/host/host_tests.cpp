@@ -307,6 +307,21 @@ static void test_gpu_moe_resident(QWHal& hal, int rows) {
     const double err = std::sqrt(num / std::fmax(den, 1e-30));
     std::printf("moe encodeResident rows=%d normalized error %.3e\n", rows, err);
     CHECK(err <= 2e-3);
+    // shared-expert gate column of the router door: with router row 0 as the gate row, gate[t] = sigmoid(logits[t, 0])
+    {
+        DeviceBuf dgate(hal, (size_t)rows * 4);
+        const QWTensorValue shw = QWTensorValue::make(dr.p, (size_t)H, QWDType::f32);
+        const QWTensorValue shout = QWTensorValue::make(dgate.p, (size_t)rows, QWDType::f32);
+        QWGemm::encodeFnRouterGemm(enc, hal, xt, w.router, s.logits, rows, E, H, &shw, &shout);
+        std::vector<float> lg((size_t)rows * E), gate((size_t)rows);
+        download(enc, lg.data(), dlog, lg.size() * 4);
+        download(enc, gate.data(), dgate, gate.size() * 4);
+        for (int t = 0; t < rows; ++t) CHECK(std::fabs(gate[t] - 1.0 / (1.0 + std::exp(-(double)lg[(size_t)t * E]))) <= 2e-6);
+        bool threw = false;
+        const QWTensorValue shw16 = QWTensorValue::make(dr.p, (size_t)H, QWDType::f16);
+        try { QWGemm::encodeFnRouterGemm(enc, hal, xt, w.router, s.logits, rows, E, H, &shw16, &shout); } catch (const QWGemmError&) { threw = true; }
+        CHECK(threw);
+    }
     hal.end(enc);
 }
 

@@ -434,13 +434,21 @@ struct QWGemm {
     static int moeMaxTiles(int experts, int pairs) { return (int)qwhip_moe_max_tiles((uint32_t)experts, (uint32_t)pairs); }  // QWGemmMoE.swift:24-26
 
     // encodeFnRouterGemm (QWGemmMoERouter.swift:78-113)
+    // shGateWeight f32 [hidden] + shGateOut f32 [rows]: the shared-expert gate sigmoid(x . w) as an extra output column
     static void encodeFnRouterGemm(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWTensorValue& router,
-                                   const QWTensorValue& logits, int rows, int experts, int hidden) {
+                                   const QWTensorValue& logits, int rows, int experts, int hidden,
+                                   const QWTensorValue* shGateWeight = nullptr, const QWTensorValue* shGateOut = nullptr) {
         if (logits.shape.dtype != QWDType::f32 || logits.shape.elementCount < (size_t)rows * (size_t)experts)
             throw QWGemmError(QWGemmError::badShape, "router logits must be f32 [rows, experts]");
+        const bool hasShGate = shGateWeight && shGateOut;   // as the reference: one without the other means no gate column
+        if (hasShGate && (shGateWeight->shape.dtype != QWDType::f32 || shGateWeight->shape.elementCount < (size_t)hidden ||
+                          shGateOut->shape.dtype != QWDType::f32 || shGateOut->shape.elementCount < (size_t)rows))
+            throw QWGemmError(QWGemmError::badShape, "shared-expert gate: f32 weight [hidden] and f32 output [rows]");
         hal.pipeline("qwg_router_gemm");
-        throwIfFailed(qwhip_router_gemm(enc.stream, x.ptr(), abiDType(x.shape.dtype), router.ptr(), abiDType(router.shape.dtype), (uint32_t)rows,
-                                        (uint32_t)experts, (uint32_t)hidden, (float*)logits.ptr()));
+        throwIfFailed(qwhip_router_gemm_shared_gate(enc.stream, x.ptr(), abiDType(x.shape.dtype), router.ptr(), abiDType(router.shape.dtype),
+                                                    (uint32_t)rows, (uint32_t)experts, (uint32_t)hidden, (float*)logits.ptr(),
+                                                    hasShGate ? (const float*)shGateWeight->ptr() : nullptr,
+                                                    hasShGate ? (float*)shGateOut->ptr() : nullptr));
     }
     // encodeFnMoeRoute (QWGemmMoERouter.swift:10-75)
     static void encodeFnMoeRoute(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& logits, const QWTensorValue& idx,

@@ -73,6 +73,35 @@ def test_router_gemm(dev, xdt):
     assert qo.normalized_error(got, ref) <= 1e-5
 
 
+@pytest.mark.parametrize("t,e,h,wdt", [(19, 128, 2048, "f32"), (5, 64, 4096, "bf16"), (33, 40, 5120, "f32"), (3, 8, 16384, "f16")])
+def test_router_gemm_shared_gate_and_wide_rows(dev, t, e, h, wdt):
+    """The shared-expert gate column sigmoid(x . w) beside the logits, on hidden sizes that take 8, 4, 2 and 1 token rows
+    per workgroup; the logits are those of the plain door bit for bit."""
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((t, h)).astype(np.float32)
+    wr = (rng.standard_normal((e, h)) * 0.05).astype(np.float32)
+    shw = (rng.standard_normal(h) * 0.03).astype(np.float32)
+    if wdt == "f32":
+        wh, wcode, wv = wr, qwhip.F32, wr
+    elif wdt == "bf16":
+        wh, wcode, wv = qo.f32_to_bf16_bits(wr), qwhip.BF16, qo.round_bf16(wr)
+    else:
+        wh, wcode = wr.astype(np.float16), qwhip.F16
+        wv = wh.astype(np.float32)
+    xb, wb, sb = dev.put(x), dev.put(wh), dev.put(shw)
+    l1, l2, go = dev.alloc(t * e * 4), dev.alloc(t * e * 4), dev.alloc(t * 4)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_router_gemm_shared_gate(st, xb.ptr, qwhip.F32, wb.ptr, wcode, t, e, h, l1.ptr, sb.ptr, go.ptr))
+    qwhip.check(lib.qwhip_router_gemm(st, xb.ptr, qwhip.F32, wb.ptr, wcode, t, e, h, l2.ptr))
+    dev.stream.sync()
+    got, plain, gate = l1.download(np.float32, (t, e)), l2.download(np.float32, (t, e)), go.download(np.float32, (t,))
+    assert np.array_equal(got.view(np.uint32), plain.view(np.uint32))
+    assert qo.normalized_error(got, x.astype(np.float64) @ wv.astype(np.float64).T) <= 1e-5
+    np.testing.assert_allclose(gate, qo.router_shared_gate_f64(x, shw), rtol=0, atol=2e-6)
+    assert lib.qwhip_router_gemm_shared_gate(st, xb.ptr, qwhip.F32, wb.ptr, wcode, t, e, h, l1.ptr, sb.ptr, None) == qwhip.E_NULL
+    assert lib.qwhip_router_gemm(st, xb.ptr, qwhip.F32, wb.ptr, wcode, t, e, 16388, l1.ptr) == qwhip.E_BAD_SHAPE
+
+
 def _group(dev, ids, experts, top_k, compact=True):
     pairs = ids.size
     mt = max(1, dev.lib.qwhip_moe_max_tiles(experts, pairs))

@@ -326,3 +326,22 @@ def test_f32_gemv_family_closed_forms():
     row = qo.h32_groups_f64(e)[0] * np.sqrt(32.0)
     assert np.allclose(np.abs(row), 1.0) and row[0] == 1.0 and row[5] == np.float64((-1) ** bin(5).count("1"))
     assert qo.v4_epilogue_f64(np.array([0.0]), 2, 1.0)[0] == 0.5 and qo.v4_epilogue_f64(np.array([0.0]), 1, 3.0)[0] == 0.0
+
+
+def test_router_shared_gate_closed_forms():
+    """sigmoid(x . w): zero weights give exactly 1/2, negating the weight row gives the complement, a one-hot weight row
+    reads sigmoid of one activation (against math.exp), and large dots saturate to 0 / 1 without overflow warnings."""
+    import math
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((7, 96)).astype(np.float32)
+    w = rng.standard_normal(96).astype(np.float32)
+    assert np.array_equal(qo.router_shared_gate_f64(x, np.zeros(96, np.float32)), np.full(7, 0.5))
+    g, gn = qo.router_shared_gate_f64(x, w), qo.router_shared_gate_f64(x, -w)
+    np.testing.assert_allclose(g + gn, 1.0, rtol=0, atol=1e-15)
+    onehot = np.zeros(96, np.float32)
+    onehot[11] = 2.0
+    want = [1.0 / (1.0 + math.exp(-2.0 * float(v))) for v in x[:, 11]]
+    np.testing.assert_allclose(qo.router_shared_gate_f64(x, onehot), want, rtol=1e-15)
+    with np.errstate(over="ignore"):
+        big = qo.router_shared_gate_f64(np.array([[1e4], [-1e4]], np.float32), np.array([1.0], np.float32))
+    assert big[0] == 1.0 and big[1] == 0.0
