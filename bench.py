@@ -766,6 +766,8 @@ def main() -> None:
     ap.add_argument("--rt", type=int, default=0, help="row tiles per wave for the mfma gemv (0 auto)")
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
+    ap.add_argument("--format", default=None,
+                    help="container override for the gemv / gemm / pair workloads, e.g. hq3_g32, aq6_g128 (the workload's shape is kept)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=1 << 30, help="rows of the bank the CPU baseline runs over (default: all)")
     args = ap.parse_args()
@@ -788,6 +790,13 @@ def main() -> None:
     kind, fmt, n, k, m, outliers = WORKLOADS[args.workload]
     if m is None:
         m = args.m
+    label, traffic = LABELS[args.workload], MEASURED_TRAFFIC.get(args.workload)
+    if args.format and args.format != fmt:
+        from tests import helpers as H
+        if kind not in ("gemv", "gemm", "pair") or args.format not in H.FORMATS:
+            ap.error(f"--format takes one of {sorted(H.FORMATS)} on a gemv, gemm or pair workload")
+        fmt, traffic = args.format, None
+        label += f" [container {fmt}]"
     if kind == "moe":
         out = run_moe(args, m, LABELS[args.workload])
     elif kind == "gemv_f32":
@@ -801,12 +810,11 @@ def main() -> None:
     elif kind == "norm":
         out = run_norm(args, m, n, LABELS[args.workload])
     elif kind == "pair":
-        out = run_silu_pair(args, fmt, n, k, m, LABELS[args.workload])
+        out = run_silu_pair(args, fmt, n, k, m, label)
     elif kind == "gemm":
-        out = run_gemm(args, fmt, n, k, m, LABELS[args.workload], MEASURED_TRAFFIC.get(args.workload))
+        out = run_gemm(args, fmt, n, k, m, label, traffic)
     else:
-        out = run_gemv(args, fmt, n, k, m, LABELS[args.workload] + (f" M={m}" if args.workload.startswith("c5") else ""), outliers,
-                       MEASURED_TRAFFIC.get(args.workload))
+        out = run_gemv(args, fmt, n, k, m, label + (f" M={m}" if args.workload.startswith("c5") else ""), outliers, traffic)
     print(json.dumps(out))
 
 

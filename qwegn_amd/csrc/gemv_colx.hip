@@ -17,8 +17,10 @@
 // (qwg_aq_slice_dot, Sources/QWMetal/include/qw_dequant_multi.metalh:205-208).
 // Element order inside a word fixes which activations pair up: HQ4_G32_M5 keeps element 8w + j at bit
 // 4 (j >> 1) + 16 (j & 1) (unpack_hq4_word8, qw_dequant.metalh:42-62), the bit-stream containers element i at bit
-// i * bits, so a masked 4-bit word holds elements (k, k + 4) and a masked 8-bit word elements (k, k + 2).  The 2-, 3- and
-// 6-bit streams have no such in-place pairs: their codes are cut out one by one and paired as neighbours.
+// i * bits, so a masked 4-bit word holds elements (k, k + 4), a masked 8-bit word elements (k, k + 2) and a masked 2-bit
+// word elements (k, k + 8) (sixteen codes a word; the four mask positions of a byte read as q, 4 q, 16 q and 64 q times
+// 2^-24 and get one accumulator each).  The 3- and 6-bit streams have no such in-place pairs: their codes are cut out
+// one by one and paired as neighbours.
 #include "qwhip_common.h"
 
 namespace {
@@ -36,7 +38,7 @@ template <int FMT>
 struct qcx_fmt {
     static constexpr int BITS = FMT == QW_FMT_B8 ? 8 : (FMT == QW_FMT_B2 ? 2 : (FMT == QW_FMT_B3 ? 3 : (FMT == QW_FMT_B6 ? 6 : 4)));
     static constexpr int PW = BITS;
-    static constexpr bool GENERIC = FMT == QW_FMT_B2 || FMT == QW_FMT_B3 || FMT == QW_FMT_B6;
+    static constexpr bool GENERIC = FMT == QW_FMT_B3 || FMT == QW_FMT_B6;   // codes cut out of the stream one by one
 };
 
 struct __attribute__((packed, aligned(4))) qcx_words4 { uint32_t q[4]; };
@@ -60,6 +62,7 @@ __device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
             h2_t pr;
             if constexpr (FMT == QW_FMT_M5 || qcx_fmt<FMT>::GENERIC) pr = h2_t{v[j][2 * k], v[j][2 * k + 1]};
             else if constexpr (FMT == QW_FMT_B4) pr = h2_t{v[j][k], v[j][k + 4]};
+            else if constexpr (FMT == QW_FMT_B2) pr = h2_t{v[2 * (j >> 1)][4 * (j & 1) + k], v[2 * (j >> 1) + 1][4 * (j & 1) + k]};
             else pr = h2_t{v[j][4 * (k >> 1) + (k & 1)], v[j][4 * (k >> 1) + (k & 1) + 2]};
             if (k & 1) s1 = __builtin_amdgcn_fdot2(pr, one, s1, false);
             else s0 = __builtin_amdgcn_fdot2(pr, one, s0, false);
@@ -128,7 +131,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
     auto issue = [&](int slot) {
         const uint8_t* rp = p.bank + off;
         buf[slot].hdr = *(const uint32_t*)(rp + hdr_off);
-        if constexpr (qcx_fmt<FMT>::GENERIC) {
+        if constexpr (qcx_fmt<FMT>::GENERIC || FMT == QW_FMT_B2) {
 #pragma unroll
             for (int j = 0; j < qcx_fmt<FMT>::PW; ++j) buf[slot].q[j] = *(const uint32_t*)(rp + pay_off + 4 * j);
         } else if constexpr (FMT == QW_FMT_B8) {
@@ -200,6 +203,21 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
                 };
 #pragma unroll
                 for (int i = 0; i < 16; ++i) ow[i] = code(2 * i) | (code(2 * i + 1) << 16);
+            } else if constexpr (FMT == QW_FMT_B2) {
+                // operand 8 w + j: elements (16 w + j, 16 w + j + 8), masked in place at bits 2 (j & 3) of the bytes 0 / 2 of the
+                // word (j < 4) or of the word shifted down a byte (j >= 4)
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    const uint32_t q = b.q[w], q8 = q >> 8;
+                    ow[8 * w + 0] = q & 0x00030003u;
+                    ow[8 * w + 1] = q & 0x000C000Cu;
+                    ow[8 * w + 2] = q & 0x00300030u;
+                    ow[8 * w + 3] = q & 0x00C000C0u;
+                    ow[8 * w + 4] = q8 & 0x00030003u;
+                    ow[8 * w + 5] = q8 & 0x000C000Cu;
+                    ow[8 * w + 6] = q8 & 0x00300030u;
+                    ow[8 * w + 7] = q8 & 0x00C000C0u;
+                }
             } else if constexpr (FMT == QW_FMT_B8) {
 #pragma unroll
                 for (int w = 0; w < 8; ++w) {
@@ -231,6 +249,10 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
                 float q;
                 if constexpr (FMT == QW_FMT_B8 || qcx_fmt<FMT>::GENERIC) {
                     q = ((a0 + a1) + (a2 + a3)) * 16777216.0f;
+                } else if constexpr (FMT == QW_FMT_B2) {
+                    q = __builtin_fmaf(a1, 4194304.0f, a0 * 16777216.0f);     // codes at bits 0..1 and 2..3 of a byte
+                    q = __builtin_fmaf(a2, 1048576.0f, q);                    // bits 4..5
+                    q = __builtin_fmaf(a3, 262144.0f, q);                     // bits 6..7
                 } else {
                     q = __builtin_fmaf(a0 + a2, 16777216.0f, FMT == QW_FMT_M5 ? 1024.0f * S[m] : 0.0f);   // codes at bits 0..3
                     q = __builtin_fmaf(a1 + a3, 1048576.0f, q);                                           // codes at bits 4..7
