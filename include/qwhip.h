@@ -202,6 +202,14 @@ qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, con
                                uint32_t flags, float* logits, int32_t* tokens);
 qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);
 
+/* Embedding gather over a block table (QWGemmAQ.encodeEmbedAQ, Sources/Operators/QWGEMM/QWGemmAQ.swift:147-187 ->
+ * qwg_embed_aq_f32, Sources/QWMetal/gemm/qwgemm_aq_embed.metal:14-52): `table` is the [vocab = n, hidden = k] bank;
+ * out f32 [rows, hc, hidden] = the row of tokens[r], value = code * scale + bias in fp32 in the container's own basis,
+ * written hc times.  A negative token reads row 0 (as the reference), a token >= n the last row.  Every container
+ * (HQ4_G32_M5 too: (q + 1024) * scale + bias).  out 16-byte aligned, rows <= 65535. */
+qwhip_status qwhip_embed_aq_f32(qwhip_stream_t s, const qwhip_weight_view* table, const int32_t* tokens, uint32_t rows,
+                                uint32_t hc, float* out);
+
 /* ---- prefill GEMM: Y[m, n] = X[m, k] . W^T on f16 MFMA, fp32 accumulate ------ */
 /* gemmBatchedH16 (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:119-154) -> qwg_gemm_q4g_h16 /
  * qwg_gemm_aq*_h16; QWGemm.encodeNaxF32 (Sources/Operators/QWGEMM/QWGemmF32.swift:366-402).

@@ -311,6 +311,15 @@ def dequant_hq_blocks_rot(blocks: np.ndarray, bits: int = 4, group: int = 32, is
     return w.reshape(n, nb * group)
 
 
+def embed_aq_f32(blocks: np.ndarray, tokens, hc: int = 1, bits: int = 4, group: int = 32, is_m5: bool = False) -> np.ndarray:
+    """Embedding gather over a block table [vocab, K/group, block bytes] -> f32 [rows, hc, hidden]: the token's row decoded
+    with the container's own law (code*scale + bias in fp32, block domain), written hc times; a negative token reads row 0
+    (Sources/QWMetal/gemm/qwgemm_aq_embed.metal:14-52; QWGemmAQ.swift:147-187)."""
+    tok = np.maximum(np.asarray(tokens, dtype=np.int64), 0)
+    rows = dequant_hq_blocks_rot(np.asarray(blocks)[tok], bits, group, is_m5)
+    return np.repeat(rows[:, None, :], hc, axis=1).astype(np.float32)
+
+
 def dequant_hq_blocks(blocks, bits=4, group=32, is_m5=False, f16_round=False) -> np.ndarray:
     """Standard-domain dequant of a ROTATED bank (hq_blocks.py:545-561)."""
     return fwht32_ortho(dequant_hq_blocks_rot(blocks, bits, group, is_m5, f16_round))

@@ -230,6 +230,78 @@ extern "C" qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_v
     return QWHIP_OK;
 }
 
+// ---- embedding gather over a block table: the token's row decoded to fp32, written hc times ---------
+// (qwg_embed_aq_f32, Sources/QWMetal/gemm/qwgemm_aq_embed.metal:14-52; door QWGemmAQ.encodeEmbedAQ,
+// Sources/Operators/QWGEMM/QWGemmAQ.swift:147-187).  value = code * scale + bias in fp32 (product rounded, then the sum:
+// the law of the container's host twin), in the container's own basis; a negative token reads row 0 as the reference
+// does, and a token past the table reads its last row instead of memory outside it.
+// One thread per 8 codes of the row (`bits` payload bytes; HQ4_G32_M5: one code word), blockIdx.y = output row.
+template <bool M5>
+__global__ __launch_bounds__(256) void qw_embed_kernel(const uint8_t* __restrict__ bank, const int32_t* __restrict__ tokens,
+                                                        float* __restrict__ out, uint32_t vocab, uint32_t hidden, uint32_t hc,
+                                                        uint32_t bits, uint32_t group, uint32_t row_bytes) {
+    const uint32_t oi = blockIdx.x * 256u + threadIdx.x;   // octet of the row
+    if (oi * 8u >= hidden) return;
+    const uint32_t r = blockIdx.y;
+    const uint32_t tok = min((uint32_t)max(tokens[r], 0), vocab - 1u);
+    const uint8_t* rowp = bank + (uint64_t)tok * row_bytes;
+    float v[8];
+    if constexpr (M5) {
+        const qw_hq4_block* b = (const qw_hq4_block*)(rowp + (oi >> 2) * 20u);
+        const h2_t hd = __builtin_bit_cast(h2_t, b->hdr);
+        const float sc = (float)hd[0], bi = (float)hd[1];
+        const uint32_t q = b->qs[oi & 3u];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {   // element e of the word sits at bit 4 (e >> 1) + 16 (e & 1)
+            const float code = (float)(((q >> (4 * (e >> 1) + 16 * (e & 1))) & 0xFu) + 1024u);
+            v[e] = __fadd_rn(__fmul_rn(code, sc), bi);
+        }
+    } else {
+        const uint32_t opg = group / 8u;
+        const uint8_t* p = rowp + (uint64_t)(oi / opg) * (4u + group * bits / 8u);
+        const uint32_t o = oi % opg;
+        const float sc = (float)__builtin_bit_cast(h1_t, (uint16_t)(p[0] | (p[1] << 8)));
+        const float bi = (float)__builtin_bit_cast(h1_t, (uint16_t)(p[2] | (p[3] << 8)));
+        uint64_t stream = 0;
+        for (uint32_t b = 0; b < bits; ++b) stream |= (uint64_t)p[4 + o * bits + b] << (8 * b);
+        const uint32_t mask = (1u << bits) - 1u;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = __fadd_rn(__fmul_rn((float)((uint32_t)(stream >> (e * bits)) & mask), sc), bi);
+    }
+    const f4_t lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+    for (uint32_t c = 0; c < hc; ++c) {
+        float* dst = out + ((uint64_t)r * hc + c) * hidden + oi * 8u;
+        *(f4_t*)dst = lo;
+        *(f4_t*)(dst + 4) = hi;
+    }
+}
+
+extern "C" qwhip_status qwhip_embed_aq_f32(qwhip_stream_t s, const qwhip_weight_view* table, const int32_t* tokens, uint32_t rows,
+                                           uint32_t hc, float* out) {
+    QWHIP_REQUIRE(s);
+    qwhip_status st = qwhip_weight_view_validate(table);
+    if (st != QWHIP_OK) return st;
+    if (rows == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(tokens);
+    QWHIP_REQUIRE(out);
+    if (hc == 0) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "the embedding gather needs a positive shape");
+    if (rows > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "the embedding gather takes at most 65535 rows a launch, got %u", rows);
+    if ((uintptr_t)out & 15u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "embedding output must be 16-byte aligned");
+    const uint32_t hidden = table->k;
+    const uint32_t bb = qwhip_block_bytes(table->kind, table->bits, table->group);
+    const uint64_t row_bytes = (uint64_t)(hidden / table->group) * bb;
+    if (row_bytes >= (1ull << 32)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "embedding rows of %llu bytes are not addressable", (unsigned long long)row_bytes);
+    const dim3 grid(qwhip_cdiv(hidden / 8u, 256u), rows), block(256);
+    if (table->kind == QWHIP_KIND_HQ4_G32_M5)
+        hipLaunchKernelGGL(qw_embed_kernel<true>, grid, block, 0, s->stream, (const uint8_t*)table->blocks, tokens, out, table->n, hidden, hc,
+                           table->bits, table->group, (uint32_t)row_bytes);
+    else
+        hipLaunchKernelGGL(qw_embed_kernel<false>, grid, block, 0, s->stream, (const uint8_t*)table->blocks, tokens, out, table->n, hidden, hc,
+                           table->bits, table->group, (uint32_t)row_bytes);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
 // ------------------------------------------------------------------------------------------------
 // RMSNorm with the rotation fused (the producer in front of every projection of a decode layer):
 //   y = f16( FWHT32( x * rsqrt(mean(x^2) + eps) * (1 + gamma) ) ),  optionally after  residual <- f16(residual + x)

@@ -262,6 +262,7 @@ static const qw_kernel_entry g_kernels[] = {
     {"qwg_moe_route", "qwhip_moe_route"},
     {"qwg_moe_route_decode", "qwhip_moe_route"},
     {"qwg_router_gemm", "qwhip_router_gemm"},
+    {"qwg_embed_aq_f32", "qwhip_embed_aq_f32"},
     {"qwg_router_nax", "qwhip_router_gemm"},
     {"qwg_moe_group_pairs_f32", "qwhip_moe_group_pairs"},
     {"qwg_moe_nax_gemm", "qwhip_moe_grouped_gemm"},

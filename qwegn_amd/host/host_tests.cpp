@@ -387,6 +387,48 @@ static void test_gpu_f32_doors(QWHal& hal) {
 }
 
 // encodeDenseProjF32: 64 rows take the cast + matrix-core GEMM, 5 rows the f32 GEMV; both against the closed-form bank
+// QWGemmAQ.encodeEmbedAQ on the reference's own table (Tests/QWGEMMTests/QWAQEmbedGatherTests.swift:52-99): 8-bit group 64,
+// code of column i of group g of row r = (3 i + 7 r + 13 g) mod 256, header 1025/4096 and -683/4096
+static void test_gpu_embed(QWHal& hal) {
+    const int hidden = 256, vocab = 8, hc = 3, bits = 8, group = 64, rows = 3;
+    const int bb = 4 + group * bits / 8, groups = hidden / group;
+    std::vector<uint8_t> table((size_t)vocab * groups * bb);
+    const uint16_t hs = f2h(1025.0f / 4096.0f), hb = f2h(-683.0f / 4096.0f);
+    for (int r = 0; r < vocab; ++r)
+        for (int g = 0; g < groups; ++g) {
+            uint8_t* p = &table[((size_t)r * groups + g) * bb];
+            std::memcpy(p, &hs, 2);
+            std::memcpy(p + 2, &hb, 2);
+            for (int i = 0; i < group; ++i) p[4 + i] = (uint8_t)((i * 3 + r * 7 + g * 13) % 256);
+        }
+    const int32_t tokens[rows] = {0, 3, 7};
+    QWHipEncoder enc = hal.begin();
+    DeviceBuf dt(hal, table.size()), dtok(hal, sizeof(tokens)), dout(hal, (size_t)rows * hc * hidden * 4);
+    upload(enc, dt, table.data(), table.size());
+    upload(enc, dtok, tokens, sizeof(tokens));
+    const QWTensorValue blocks = QWTensorValue::make(dt.p, table.size() / 2, QWDType::f16);
+    const QWTensorValue tok = QWTensorValue::make(dtok.p, rows, QWDType::i32);
+    const QWTensorValue out = QWTensorValue::make(dout.p, (size_t)rows * hc * hidden, QWDType::f32);
+    QWGemmAQ::encodeEmbedAQ(enc, hal, blocks, tok, out, hidden, hc, bits, group, rows);
+    std::vector<float> got((size_t)rows * hc * hidden);
+    download(enc, got.data(), dout, got.size() * 4);
+    const double sc = h2f(hs), bi = h2f(hb), ulp = 0.000000059604644775390625;
+    for (int t = 0; t < rows; ++t)
+        for (int d = 0; d < hidden; ++d) {
+            const double code = (double)(((d % group) * 3 + tokens[t] * 7 + (d / group) * 13) % 256);
+            const double want = code * sc + bi;
+            const double tol = std::fabs(code * sc) * ulp + std::fmax(std::fabs(want), std::fabs(bi)) * ulp + 1e-30;
+            for (int c = 0; c < hc; ++c) CHECK(std::fabs((double)got[((size_t)t * hc + c) * hidden + d] - want) <= tol);
+        }
+    bool threw = false;
+    try { QWGemmAQ::encodeEmbedAQ(enc, hal, blocks, tok, out, hidden, hc, 5, group, rows); } catch (const QWGemmError&) { threw = true; }
+    CHECK(threw);
+    threw = false;
+    try { QWGemmAQ::encodeEmbedAQ(enc, hal, blocks, tok, out, 96, hc, bits, group, rows); } catch (const QWGemmError&) { threw = true; }
+    CHECK(threw);
+    hal.end(enc);
+}
+
 static void test_gpu_dense_proj_f32(QWHal& hal) {
     const int N = 128, Kc = 128;
     const std::vector<uint8_t> bank = cf_bank(N, Kc);
@@ -430,6 +472,7 @@ int main(int argc, char** argv) {
         test_gpu_moe_resident(hal, 40);   // grouped prefill path (fused gate_up + SwiGLU)
         test_gpu_f32_doors(hal);
         test_gpu_dense_proj_f32(hal);
+        test_gpu_embed(hal);
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed ? 1 : 0;

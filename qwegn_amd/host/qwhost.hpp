@@ -580,6 +580,29 @@ struct QWGemmAQ {
             throwIfFailed(qwhip_gemv(enc.stream, &w, xc.ptr(), QWHIP_F16, (uint32_t)chunk, flags, nullptr, (float*)yc.ptr()));
         }
     }
+    // QWGemmAQ.encodeEmbedAQ (QWGemmAQ.swift:147-187): the token's row of a block table decoded to f32, written hc times
+    static void encodeEmbedAQ(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& blocks, const QWTensorValue& token, const QWTensorValue& out,
+                              int hidden, int hc, int bits, int group, int rows = 1) {
+        if (hidden <= 0 || hc <= 0 || rows <= 0) throw QWGemmError(QWGemmError::badWeights, "the embedding gather needs a positive shape");
+        const uint32_t bb = qwhip_block_bytes(QWHIP_KIND_NATIVE_AFFINE, (uint32_t)bits, (uint32_t)group);
+        if (bb == 0) throw QWGemmError(QWGemmError::badWeights, "no affine-quantised container for this pair");
+        if (hidden % group != 0) throw QWGemmError(QWGemmError::badWeights, "hidden must be a multiple of the group");
+        const size_t rowBytes = (size_t)(hidden / group) * bb;
+        if (blocks.bytes < rowBytes) throw QWGemmError(QWGemmError::badWeights, "the table is shorter than one row");
+        if (token.shape.elementCount < (size_t)rows) throw QWGemmError(QWGemmError::badWeights, "the token tensor is short");
+        if (out.shape.dtype != QWDType::f32 || out.shape.elementCount < (size_t)rows * (size_t)hidden * (size_t)hc)
+            throw QWGemmError(QWGemmError::badWeights, "the output must hold rows * hidden * hc f32 values");
+        hal.pipeline("qwg_embed_aq_f32");
+        qwhip_weight_view w = {};
+        w.blocks = blocks.ptr();
+        w.n = (uint32_t)(blocks.bytes / rowBytes);   // the rows the table holds: a token past them reads the last one
+        w.k = (uint32_t)hidden;
+        w.kind = QWHIP_KIND_NATIVE_AFFINE;             // the gather decodes in the container's own basis: the tag is not used
+        w.bits = (uint32_t)bits;
+        w.group = (uint32_t)group;
+        w.bytes = (uint64_t)w.n * rowBytes;
+        throwIfFailed(qwhip_embed_aq_f32(enc.stream, &w, (const int32_t*)token.ptr(), (uint32_t)rows, (uint32_t)hc, (float*)out.ptr()));
+    }
     // QWGemmAQ.encodeDecodeT4: f16 in, f16 out, one row
     static void encodeDecodeT4(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& blocks, const QWTensorValue& x, const QWTensorValue& y16,
                                int n, int k, int bits, int group, bool isRotated = true, bool rotateInKernel = false) {

@@ -348,3 +348,66 @@ def test_argmax_rows_whose_maximum_is_a_zero_or_nothing_above_minus_infinity(dev
     got = tb.download(np.int32, (6,))
     assert list(got) == [40000, 7, 0, 65000, 33333, 12]
     assert np.array_equal(got, qo.head_argmax(base))
+
+
+def _embed_table(bits, group, vocab, hidden):
+    """The table of the reference's gather test (Tests/QWGEMMTests/QWAQEmbedGatherTests.swift:52-66): code of column i of
+    group g of row r = (3 i + 7 r + 13 g) mod 2^bits, header 1025/4096, -683/4096 (f16-exact, not powers of two)."""
+    i = np.arange(group)[None, None, :]
+    r = np.arange(vocab)[:, None, None]
+    g = np.arange(hidden // group)[None, :, None]
+    codes = ((3 * i + 7 * r + 13 * g) % (1 << bits)).astype(np.uint8)
+    hdr = np.array([1025.0 / 4096.0, -683.0 / 4096.0], np.float16).view(np.uint8)
+    blocks = np.empty((vocab, hidden // group, 4 + group * bits // 8), np.uint8)
+    blocks[..., :4] = hdr
+    blocks[..., 4:] = qo.pack_bitstream(codes, bits)
+    return blocks, codes.reshape(vocab, hidden)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
+@pytest.mark.parametrize("group", [32, 64, 128, 256])
+def test_embed_gather_every_pair(dev, bits, group):
+    """The reference's own gather cases (QWAQEmbedGatherTests.swift:101-168): hidden 256, vocab 8, tokens 0, 3, 7 written
+    three times, and one copy of row 2; checked against code * scale + bias in f64 within the reference's tolerance
+    (product ulp + result ulp) and bit for bit against the oracle; a negative token reads row 0, one past the table its last row."""
+    hidden, vocab = 256, 8
+    blocks, codes = _embed_table(bits, group, vocab, hidden)
+    kind = qwhip.KIND_NATIVE_AFFINE
+    bank = dev.put(blocks)
+    view = dev.view(bank, vocab, hidden, kind, bits, group)
+    sc, bi = float(np.float16(1025.0 / 4096.0)), float(np.float16(-683.0 / 4096.0))
+    for tokens, hc in (([0, 3, 7], 3), ([2], 1), ([-5, 8, 1], 2)):
+        tb, ob = dev.put(np.array(tokens, np.int32)), dev.alloc(len(tokens) * hc * hidden * 4)
+        qwhip.check(dev.lib.qwhip_embed_aq_f32(dev.stream.handle, C.byref(view), tb.ptr, len(tokens), hc, ob.ptr))
+        dev.stream.sync()
+        got = ob.download(np.float32, (len(tokens), hc, hidden))
+        rows = np.clip(np.array(tokens), 0, vocab - 1)
+        code = codes[rows].astype(np.float64)
+        want = code * sc + bi
+        ulp = 2.0 ** -24
+        tol = np.abs(code * sc) * ulp + np.maximum(np.abs(want), abs(bi)) * ulp + 1e-30
+        assert np.all(np.abs(got.astype(np.float64) - want[:, None, :]) <= tol[:, None, :])
+        oracle = qo.embed_aq_f32(blocks, rows, hc, bits, group)
+        assert np.array_equal(got.view(np.uint32), oracle.view(np.uint32))
+        tb.free(); ob.free()
+    bank.free()
+
+
+def test_embed_gather_hq4_m5_and_errors(dev):
+    """HQ4_G32_M5 tables decode with (q + 1024) * scale + bias, bit for bit the oracle's fp32 dequant; shape errors."""
+    from tests import helpers as H
+    vocab, hidden = 40, 512
+    blocks, _ = H.make_bank("hq4_g32_m5", vocab, hidden, seed=31)
+    bank = dev.put(blocks)
+    view = H.view_of(dev, bank, "hq4_g32_m5", vocab, hidden)
+    tokens = np.array([39, 0, 17, 17], np.int32)
+    tb, ob = dev.put(tokens), dev.alloc(4 * 2 * hidden * 4)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_embed_aq_f32(st, C.byref(view), tb.ptr, 4, 2, ob.ptr))
+    dev.stream.sync()
+    got = ob.download(np.float32, (4, 2, hidden))
+    want = qo.embed_aq_f32(blocks, tokens, 2, 4, 32, True)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert lib.qwhip_embed_aq_f32(st, C.byref(view), tb.ptr, 4, 0, ob.ptr) == qwhip.E_BAD_WEIGHTS
+    assert lib.qwhip_embed_aq_f32(st, C.byref(view), None, 4, 1, ob.ptr) == qwhip.E_NULL
+    assert lib.qwhip_embed_aq_f32(st, C.byref(view), tb.ptr, 0, 1, None) == qwhip.OK

@@ -345,3 +345,29 @@ def test_router_shared_gate_closed_forms():
     with np.errstate(over="ignore"):
         big = qo.router_shared_gate_f64(np.array([[1e4], [-1e4]], np.float32), np.array([1.0], np.float32))
     assert big[0] == 1.0 and big[1] == 0.0
+
+
+def test_embed_gather_reads_the_token_row():
+    """The gather against the reference's own recipe (Tests/QWGEMMTests/QWAQEmbedGatherTests.swift:52-99): known codes and a
+    header that is f16-exact but no power of two; the f64 law within product ulp + result ulp, hc copies equal, negative
+    tokens read row 0, and the M5 container reads (q + 1024) * scale + bias of its own element order."""
+    for bits, group in ((2, 64), (3, 32), (6, 128), (8, 256), (4, 32)):
+        hidden, vocab = 256, 8
+        i = np.arange(group)[None, None, :]
+        r = np.arange(vocab)[:, None, None]
+        g = np.arange(hidden // group)[None, :, None]
+        codes = ((3 * i + 7 * r + 13 * g) % (1 << bits)).astype(np.uint8)
+        blocks = np.empty((vocab, hidden // group, 4 + group * bits // 8), np.uint8)
+        blocks[..., :4] = np.array([1025.0 / 4096.0, -683.0 / 4096.0], np.float16).view(np.uint8)
+        blocks[..., 4:] = qo.pack_bitstream(codes, bits)
+        out = qo.embed_aq_f32(blocks, [0, 3, 7, -2], 3, bits, group)
+        assert out.shape == (4, 3, hidden) and out.dtype == np.float32
+        code = codes.reshape(vocab, hidden)[[0, 3, 7, 0]].astype(np.float64)
+        want = code * (1025.0 / 4096.0) + (-683.0 / 4096.0)
+        tol = np.abs(code * 1025.0 / 4096.0) * 2.0 ** -24 + np.maximum(np.abs(want), 683.0 / 4096.0) * 2.0 ** -24
+        assert np.all(np.abs(out[:, 0].astype(np.float64) - want) <= tol)
+        assert np.array_equal(out[:, 0], out[:, 1]) and np.array_equal(out[:, 0], out[:, 2])
+    w = (np.random.default_rng(2).standard_normal((6, 64)) * 0.02).astype(np.float32)
+    m5, _ = qo.quant_hq_blocks(w, bits=4, group=32, is_m5=True, rotate=True)
+    got = qo.embed_aq_f32(m5, [5, 1], 1, 4, 32, True)[:, 0]
+    assert np.array_equal(got, qo.dequant_hq4_rot(m5)[[5, 1]])
