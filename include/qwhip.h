@@ -202,6 +202,24 @@ qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, con
                                uint32_t flags, float* logits, int32_t* tokens);
 qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);
 
+/* ---- fp32 seams of the MoE operator chain ------------------------------------ */
+/* QWGemm.encodeSiluMulF32 (Sources/Operators/QWGEMM/QWGemmF32.swift:83-94) -> qwg_silu_mul_f32
+ * (Sources/QWMetal/gemm/qwgemm_f32.metal:291-317): act f32 [rows, inter] = FWHT32(silu(gate) * up), gu f32 [rows, 2 inter],
+ * inter % 32 == 0.  (The door's f16 output is qwhip_swiglu_fwht with an f32 gate|up.) */
+qwhip_status qwhip_silu_mul_f32(qwhip_stream_t s, const float* gu, float* act, uint32_t rows, uint32_t inter);
+/* QWGemm.encodeMoEBridgeF16ToF32 (Sources/Operators/QWGEMM/QWGemmMoE.swift:337-377) -> qwg_moe_bridge_f16_to_f32
+ * (Sources/QWMetal/gemm/qwmoe_bridge_f32.metal:16-78): the f16 normed hidden (rotated basis) -> x_rot32 (widened; NULL =
+ * the door's skipRot32) and x_plain32 (un-rotated in fp32 through the f16 hi/lo split).  hidden % 256 == 0. */
+qwhip_status qwhip_moe_bridge_f16_to_f32(qwhip_stream_t s, const void* x_f16, float* x_rot32, float* x_plain32, uint32_t rows,
+                                         uint32_t hidden);
+/* QWGemm.encodeLatentNormH32F32 (QWGemmF32.swift:57-80) -> qwg_latent_norm_h32_f32 (qwgemm_f32.metal:203-288): optional
+ * RMSNorm with the plus-one law (gamma f16 [latent], NULL = none) and the 32-point transform on f32 [rows, latent];
+ * out32 and / or out16 (NULL = not written; at least one).  latent % 32 == 0. */
+qwhip_status qwhip_latent_norm_h32_f32(qwhip_stream_t s, const float* x, const void* gamma_f16, float* out32, void* out16,
+                                       uint32_t rows, uint32_t latent, float eps);
+/* QWGemm.encodeAddF32 (QWGemmF32.swift:108-115) -> qwg_add_f32: out = a + b over count f32 values. */
+qwhip_status qwhip_add_f32(qwhip_stream_t s, const float* a, const float* b, float* out, uint64_t count);
+
 /* Embedding gather over a block table (QWGemmAQ.encodeEmbedAQ, Sources/Operators/QWGEMM/QWGemmAQ.swift:147-187 ->
  * qwg_embed_aq_f32, Sources/QWMetal/gemm/qwgemm_aq_embed.metal:14-52): `table` is the [vocab = n, hidden = k] bank;
  * out f32 [rows, hc, hidden] = the row of tokens[r], value = code * scale + bias in fp32 in the container's own basis,

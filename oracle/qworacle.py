@@ -558,6 +558,39 @@ def swiglu_fwht_f16(gate, up, rotate: bool = True) -> np.ndarray:
     return a.astype(np.float16)
 
 
+def silu_mul_f32(gu: np.ndarray) -> np.ndarray:
+    """f32 gate|up [rows, 2 I] -> FWHT32(silu(g) * u) in fp32 [rows, I]
+    (qwg_silu_mul_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:291-317; I % 32 == 0)."""
+    gu = np.asarray(gu, dtype=np.float32)
+    inter = gu.shape[-1] // 2
+    return fwht32_ortho(swiglu(gu[..., :inter], gu[..., inter:]))
+
+
+def moe_bridge_f16_to_f32(x16: np.ndarray):
+    """The f32 bridge in front of the MoE chain (Sources/QWMetal/gemm/qwmoe_bridge_f32.metal:16-78): the f16 hidden in the
+    rotated basis -> (rotated f32 copy = a widening, un-rotated f32 copy = the transform again in fp32, taken through the
+    f16 hi/lo split: f32(hi) + f32(lo), hi = f16(v), lo = f16(v - f32(hi)))."""
+    rot = np.asarray(x16, dtype=np.float16).astype(np.float32)
+    v = fwht32_ortho(rot)
+    hi = v.astype(np.float16)
+    lo = (v - hi.astype(np.float32)).astype(np.float16)
+    return rot, hi.astype(np.float32) + lo.astype(np.float32)
+
+
+def latent_norm_h32_f32(x: np.ndarray, gamma16=None, eps: float = 1e-6) -> np.ndarray:
+    """Optional RMSNorm with the plus-one law, then FWHT-32, on f32 [rows, L] -> f32
+    (qwg_latent_norm_h32_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:203-288): v = (x * rstd) * (1 + gamma),
+    rstd = rsqrt(mean(x^2) + eps); the mean of squares in float64 rounded to fp32 (the kernel's summation order is not
+    part of the contract).  No gamma: the transform alone."""
+    x = np.asarray(x, dtype=np.float32)
+    if gamma16 is None:
+        return fwht32_ortho(x)
+    ms = (x.astype(np.float64) ** 2).mean(axis=-1, keepdims=True)
+    rstd = (1.0 / np.sqrt(ms + np.float64(np.float32(eps)))).astype(np.float32)
+    g1 = np.float32(1.0) + np.asarray(gamma16, dtype=np.float16).astype(np.float32)
+    return fwht32_ortho((x * rstd) * g1)
+
+
 # --------------------------------------------------------------------------- #
 # MoE router  (pinned: golden fn_sparse_moe_golden.json end to end; math: textbook softmax/top-k, tie rule)
 # --------------------------------------------------------------------------- #

@@ -230,6 +230,182 @@ extern "C" qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_v
     return QWHIP_OK;
 }
 
+// ---- fp32 seams of the MoE operator chain ----------------------------------------------------------
+// One thread per 32-group, the group in registers, the fp32 butterfly of qw_fwht32 (strides 1, 2, 4, 8, 16, then one
+// multiply by 1/sqrt(32): the order of fwht32_f32_inplace, Sources/QWMetal/include/qw_dequant.metalh:442-478).
+
+// silu(gate) * up in fp32, then the 32-point transform, fp32 out (qwg_silu_mul_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:291-317;
+// door QWGemm.encodeSiluMulF32, Sources/Operators/QWGEMM/QWGemmF32.swift:83-94).  gu fp32 [rows, 2 inter], inter % 32 == 0.
+__global__ __launch_bounds__(256) void qw_silu_mul_f32_kernel(const float* __restrict__ gu, float* __restrict__ act, uint32_t rows,
+                                                               uint32_t inter) {
+    const uint64_t gi = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint32_t gpr = inter / 32u;
+    if (gi >= (uint64_t)rows * gpr) return;
+    const uint32_t r = (uint32_t)(gi / gpr), g = (uint32_t)(gi % gpr);
+    const f4_t* gp = (const f4_t*)(gu + (uint64_t)r * 2u * inter + 32u * g);
+    const f4_t* up = (const f4_t*)(gu + (uint64_t)r * 2u * inter + inter + 32u * g);
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const f4_t a = gp[j], b = up[j];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[4 * j + e] = qw_swiglu(a[e], b[e]);
+    }
+    qw_fwht32(v);
+    f4_t* o = (f4_t*)(act + (uint64_t)r * inter + 32u * g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = f4_t{v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
+}
+
+extern "C" qwhip_status qwhip_silu_mul_f32(qwhip_stream_t s, const float* gu, float* act, uint32_t rows, uint32_t inter) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(gu);
+    QWHIP_REQUIRE(act);
+    if (inter == 0 || inter % 32u != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "f32 silu-mul needs intermediate %% 32 == 0, got %u", inter);
+    if (((uintptr_t)gu | (uintptr_t)act) & 15u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "f32 silu-mul needs 16-byte aligned buffers");
+    const uint64_t groups = (uint64_t)rows * (inter / 32u);
+    hipLaunchKernelGGL(qw_silu_mul_f32_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s->stream, gu, act, rows, inter);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// The f32 bridge in front of the MoE chain (qwg_moe_bridge_f16_to_f32, Sources/QWMetal/gemm/qwmoe_bridge_f32.metal:16-78; door
+// QWGemm.encodeMoEBridgeF16ToF32, Sources/Operators/QWGEMM/QWGemmMoE.swift:337-377): the f16 normed hidden in the rotated
+// basis becomes the rotated fp32 copy (a plain widening; skipped when x_rot32 is null) and the un-rotated fp32 copy the
+// router reads - the transform again (it is its own inverse) in fp32, taken through the f16 hi/lo split of the reference's
+// helper: plain = f32(hi) + f32(lo), hi = f16(v), lo = f16(v - f32(hi)).
+__global__ __launch_bounds__(256) void qw_moe_bridge_kernel(const h1_t* __restrict__ x, float* __restrict__ rot32, float* __restrict__ plain32,
+                                                             uint64_t groups) {
+    const uint64_t gi = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gi >= groups) return;
+    const h8_t* xp = (const h8_t*)(x + 32u * gi);
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const h8_t a = xp[j];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[8 * j + e] = (float)a[e];
+    }
+    if (rot32) {
+        f4_t* o = (f4_t*)(rot32 + 32u * gi);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = f4_t{v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
+    }
+    qw_fwht32(v);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const h1_t hi = (h1_t)v[i];
+        const h1_t lo = (h1_t)(v[i] - (float)hi);
+        v[i] = (float)hi + (float)lo;
+    }
+    f4_t* o = (f4_t*)(plain32 + 32u * gi);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = f4_t{v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
+}
+
+extern "C" qwhip_status qwhip_moe_bridge_f16_to_f32(qwhip_stream_t s, const void* x_f16, float* x_rot32, float* x_plain32, uint32_t rows,
+                                                    uint32_t hidden) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0 || hidden == 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "moe bridge: rows=%u hidden=%u", rows, hidden);
+    if (hidden % 256u != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "moe bridge: hidden %u must be a multiple of 256", hidden);
+    QWHIP_REQUIRE(x_f16);
+    QWHIP_REQUIRE(x_plain32);
+    if (((uintptr_t)x_f16 | (uintptr_t)x_rot32 | (uintptr_t)x_plain32) & 15u)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe bridge needs 16-byte aligned buffers");
+    const uint64_t groups = (uint64_t)rows * (hidden / 32u);
+    hipLaunchKernelGGL(qw_moe_bridge_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s->stream, (const h1_t*)x_f16, x_rot32,
+                       x_plain32, groups);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// Optional RMSNorm (1 + gamma) and the 32-point transform on fp32 [rows, latent], fp32 and / or f16 out
+// (qwg_latent_norm_h32_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:203-288; door QWGemm.encodeLatentNormH32F32,
+// Sources/Operators/QWGEMM/QWGemmF32.swift:57-80): v = x * rsqrt(mean(x^2) + eps) * (1 + gamma) (gamma f16; no gamma: v = x),
+// then the transform; one workgroup per row.
+__global__ __launch_bounds__(256) void qw_latent_norm_kernel(const float* __restrict__ x, const h1_t* __restrict__ gamma,
+                                                              float* __restrict__ out32, h1_t* __restrict__ out16, uint32_t latent, float eps) {
+    __shared__ float wsum[4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const float* xr = x + (uint64_t)blockIdx.x * latent;
+    float rstd = 1.0f;
+    if (gamma) {
+        float ss = 0.0f;
+        for (uint32_t c = tid * 4u; c < latent; c += 1024u) {
+            const f4_t a = *(const f4_t*)(xr + c);
+            ss = fmaf(a[0], a[0], ss);
+            ss = fmaf(a[1], a[1], ss);
+            ss = fmaf(a[2], a[2], ss);
+            ss = fmaf(a[3], a[3], ss);
+        }
+        ss = qw_reduce64(ss);
+        if (lane == 0) wsum[wave] = ss;
+        __syncthreads();
+        rstd = rsqrtf(((wsum[0] + wsum[1]) + (wsum[2] + wsum[3])) / (float)latent + eps);
+    }
+    for (uint32_t g = tid; g < latent / 32u; g += 256u) {
+        float v[32];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const f4_t a = *(const f4_t*)(xr + 32u * g + 4 * j);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[4 * j + e] = a[e];
+        }
+        if (gamma) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) v[i] = (v[i] * rstd) * (1.0f + (float)gamma[32u * g + i]);
+        }
+        qw_fwht32(v);
+        const uint64_t at = (uint64_t)blockIdx.x * latent + 32u * g;
+        if (out32) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) *(f4_t*)(out32 + at + 4 * j) = f4_t{v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
+        }
+        if (out16) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                h8_t o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = (h1_t)v[8 * j + e];
+                *(h8_t*)(out16 + at + 8 * j) = o;
+            }
+        }
+    }
+}
+
+extern "C" qwhip_status qwhip_latent_norm_h32_f32(qwhip_stream_t s, const float* x, const void* gamma_f16, float* out32, void* out16,
+                                                  uint32_t rows, uint32_t latent, float eps) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(x);
+    if (!out32 && !out16) return qwhip_fail(QWHIP_E_NULL, "latent norm needs out32 and/or out16");
+    if (latent == 0 || latent % 32u != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent norm H32 needs latent %% 32 == 0, got %u", latent);
+    if (((uintptr_t)x | (uintptr_t)out32 | (uintptr_t)out16) & 15u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent norm needs 16-byte aligned buffers");
+    hipLaunchKernelGGL(qw_latent_norm_kernel, dim3(rows), dim3(256), 0, s->stream, x, (const h1_t*)gamma_f16, out32, (h1_t*)out16, latent, eps);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// out = a + b over count fp32 values (qwg_add_f32, qwgemm_f32.metal:319-326; QWGemm.encodeAddF32, QWGemmF32.swift:108-115)
+__global__ __launch_bounds__(256) void qw_add_f32_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
+                                                          uint64_t count) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) out[i] = a[i] + b[i];
+}
+
+extern "C" qwhip_status qwhip_add_f32(qwhip_stream_t s, const float* a, const float* b, float* out, uint64_t count) {
+    QWHIP_REQUIRE(s);
+    if (count == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(a);
+    QWHIP_REQUIRE(b);
+    QWHIP_REQUIRE(out);
+    if (count > (1ull << 39)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "add: %llu values are more than one launch takes", (unsigned long long)count);
+    hipLaunchKernelGGL(qw_add_f32_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s->stream, a, b, out, count);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
 // ---- embedding gather over a block table: the token's row decoded to fp32, written hc times ---------
 // (qwg_embed_aq_f32, Sources/QWMetal/gemm/qwgemm_aq_embed.metal:14-52; door QWGemmAQ.encodeEmbedAQ,
 // Sources/Operators/QWGEMM/QWGemmAQ.swift:147-187).  value = code * scale + bias in fp32 (product rounded, then the sum:

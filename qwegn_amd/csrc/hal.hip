@@ -257,12 +257,15 @@ static const qw_kernel_entry g_kernels[] = {
     {"qwg_gemm_q4g_nax_f32", "qwhip_gemm"},
     {"qwg_gemm_q4g_h16_swiglu", "qwhip_gemm_swiglu"},
     {"qwg_silu_mul_f16", "qwhip_swiglu_fwht"},
-    {"qwg_silu_mul_f32", "qwhip_swiglu_fwht"},
     {"qwg_silu_mul_split_f16", "qwhip_swiglu_fwht"},
     {"qwg_moe_route", "qwhip_moe_route"},
     {"qwg_moe_route_decode", "qwhip_moe_route"},
     {"qwg_router_gemm", "qwhip_router_gemm"},
     {"qwg_embed_aq_f32", "qwhip_embed_aq_f32"},
+    {"qwg_silu_mul_f32", "qwhip_silu_mul_f32"},
+    {"qwg_moe_bridge_f16_to_f32", "qwhip_moe_bridge_f16_to_f32"},
+    {"qwg_latent_norm_h32_f32", "qwhip_latent_norm_h32_f32"},
+    {"qwg_add_f32", "qwhip_add_f32"},
     {"qwg_router_nax", "qwhip_router_gemm"},
     {"qwg_moe_group_pairs_f32", "qwhip_moe_group_pairs"},
     {"qwg_moe_nax_gemm", "qwhip_moe_grouped_gemm"},

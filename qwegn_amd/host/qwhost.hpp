@@ -369,6 +369,59 @@ struct QWGemm {
         throwIfFailed(qwhip_swiglu_fwht(enc.stream, gu.ptr(), abiDType(gu.shape.dtype), act16.ptr(), (uint32_t)rows, (uint32_t)inter, rotate ? 1 : 0));
     }
 
+    // QWGemm.encodeSiluMulF32 (QWGemmF32.swift:83-94): f32 gate|up -> silu(g) * u + H_32, f32 out, or f16 out when act16 is given
+    static void encodeSiluMulF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& gu, const QWTensorValue& act, int rows, int inter,
+                                 const QWTensorValue* act16 = nullptr) {
+        if (inter % 32 != 0) throw QWGemmError(QWGemmError::badShape, "f32 silu-mul needs intermediate % 32 == 0");
+        if (gu.shape.dtype != QWDType::f32 || gu.shape.elementCount < (size_t)rows * 2 * (size_t)inter)
+            throw QWGemmError(QWGemmError::badShape, "f32 silu-mul: gate|up must be f32 [rows, 2 intermediate]");
+        hal.pipeline("qwg_silu_mul_f32");
+        if (act16) {
+            if (act16->shape.dtype != QWDType::f16 || act16->shape.elementCount < (size_t)rows * (size_t)inter)
+                throw QWGemmError(QWGemmError::badShape, "f32 silu-mul: act16 must be f16 [rows, intermediate]");
+            throwIfFailed(qwhip_swiglu_fwht(enc.stream, gu.ptr(), QWHIP_F32, act16->ptr(), (uint32_t)rows, (uint32_t)inter, 1));
+        } else {
+            if (act.shape.dtype != QWDType::f32 || act.shape.elementCount < (size_t)rows * (size_t)inter)
+                throw QWGemmError(QWGemmError::badShape, "f32 silu-mul: act must be f32 [rows, intermediate]");
+            throwIfFailed(qwhip_silu_mul_f32(enc.stream, (const float*)gu.ptr(), (float*)act.ptr(), (uint32_t)rows, (uint32_t)inter));
+        }
+    }
+    // QWGemm.encodeAddF32 (QWGemmF32.swift:108-115)
+    static void encodeAddF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& a, const QWTensorValue& b, const QWTensorValue& out, size_t count) {
+        if (a.shape.elementCount < count || b.shape.elementCount < count || out.shape.elementCount < count || a.shape.dtype != QWDType::f32 ||
+            b.shape.dtype != QWDType::f32 || out.shape.dtype != QWDType::f32)
+            throw QWGemmError(QWGemmError::badShape, "add: f32 buffers of at least count values");
+        hal.pipeline("qwg_add_f32");
+        throwIfFailed(qwhip_add_f32(enc.stream, (const float*)a.ptr(), (const float*)b.ptr(), (float*)out.ptr(), (uint64_t)count));
+    }
+    // QWGemm.encodeLatentNormH32F32 (QWGemmF32.swift:57-80): optional RMSNorm (1 + gamma) + H_32 on f32 [rows, latent] -> f32 and/or f16
+    static void encodeLatentNormH32F32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWTensorValue* gamma,
+                                       const QWTensorValue& out32, const QWTensorValue* out16, int rows, int latent, float eps = 1e-6f,
+                                       bool skipOut32 = false) {
+        if (latent <= 0 || latent % 32 != 0) throw QWGemmError(QWGemmError::badShape, "latent norm H32 needs latent % 32 == 0");
+        const size_t need = (size_t)rows * (size_t)latent;
+        if (x.shape.dtype != QWDType::f32 || x.shape.elementCount < need || (gamma && (gamma->shape.dtype != QWDType::f16 || gamma->shape.elementCount < (size_t)latent)) ||
+            (!skipOut32 && (out32.shape.dtype != QWDType::f32 || out32.shape.elementCount < need)) ||
+            (out16 && (out16->shape.dtype != QWDType::f16 || out16->shape.elementCount < need)))
+            throw QWGemmError(QWGemmError::badShape, "latent norm: buffers do not fit rows x latent");
+        hal.pipeline("qwg_latent_norm_h32_f32");
+        throwIfFailed(qwhip_latent_norm_h32_f32(enc.stream, (const float*)x.ptr(), gamma ? gamma->ptr() : nullptr, skipOut32 ? nullptr : (float*)out32.ptr(),
+                                                out16 ? out16->ptr() : nullptr, (uint32_t)rows, (uint32_t)latent, eps));
+    }
+    // QWGemm.encodeMoEBridgeF16ToF32 (QWGemmMoE.swift:337-377): f16 normed hidden -> rotated f32 copy + un-rotated f32 copy
+    static void encodeMoEBridgeF16ToF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& x, const QWTensorValue& xRot32,
+                                        const QWTensorValue& xPlain32, int rows, int hidden, bool skipRot32 = false) {
+        if (rows <= 0 || hidden <= 0) throw QWGemmError(QWGemmError::badGeometry, "moe bridge: rows and hidden must be positive");
+        if (hidden % 256 != 0) throw QWGemmError(QWGemmError::badGeometry, "moe bridge: hidden must be a multiple of 256");
+        const size_t need = (size_t)rows * (size_t)hidden;
+        if (x.shape.dtype != QWDType::f16 || xRot32.shape.dtype != QWDType::f32 || xPlain32.shape.dtype != QWDType::f32 ||
+            x.shape.elementCount < need || xRot32.shape.elementCount < need || xPlain32.shape.elementCount < need)
+            throw QWGemmError(QWGemmError::badShape, "moe bridge: rows x hidden do not fit the buffers");
+        hal.pipeline("qwg_moe_bridge_f16_to_f32");
+        throwIfFailed(qwhip_moe_bridge_f16_to_f32(enc.stream, x.ptr(), skipRot32 ? nullptr : (float*)xRot32.ptr(), (float*)xPlain32.ptr(),
+                                                  (uint32_t)rows, (uint32_t)hidden));
+    }
+
     // QWGemm.encodeHQ4F32V4 / encodeHQ4F32BM (Sources/Operators/QWGEMM/QWGemmF32.swift:178-199,311-350): f32 activations in the
     // container's basis -> f32 outputs; epi 0 none, 1 silu(y/scale), 2 sigmoid, 3 silu(y/scale) + H_32.
     static void encodeHQ4F32V4(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& w, const QWTensorValue& x, const QWTensorValue& y,

@@ -75,6 +75,10 @@ SIGNATURES = {
     "qwhip_gemm": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _P, _U32, _U32, _U32, _P, _U64]),
     "qwhip_moe_route": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, C.c_float, _P, _P]),
     "qwhip_router_gemm": (C.c_int32, [_P, _P, _U32, _P, _U32, _U32, _U32, _U32, _P]),
+    "qwhip_silu_mul_f32": (C.c_int32, [_P, _P, _P, _U32, _U32]),
+    "qwhip_moe_bridge_f16_to_f32": (C.c_int32, [_P, _P, _P, _P, _U32, _U32]),
+    "qwhip_latent_norm_h32_f32": (C.c_int32, [_P, _P, _P, _P, _P, _U32, _U32, C.c_float]),
+    "qwhip_add_f32": (C.c_int32, [_P, _P, _P, _P, C.c_uint64]),
     "qwhip_embed_aq_f32": (C.c_int32, [_P, _P, _P, _U32, _U32, _P]),
     "qwhip_router_gemm_shared_gate": (C.c_int32, [_P, _P, _U32, _P, _U32, _U32, _U32, _U32, _P, _P, _P]),
     "qwhip_moe_max_tiles": (_U32, [_U32, _U32]),

@@ -116,3 +116,78 @@ def test_gemv_f32_refusals(dev):
     assert dev.lib.qwhip_gemv_f32(st, C.byref(view), xb.ptr, 0, 0, 1.0, yb.ptr) == qwhip.E_BAD_SHAPE
     assert dev.lib.qwhip_gemv_f32(st, C.byref(view), None, 1, 0, 1.0, yb.ptr) == qwhip.E_NULL
     assert dev.lib.qwhip_h32_f32(st, xb.ptr, yb.ptr, 1, 48) == qwhip.E_BAD_SHAPE
+
+
+def test_silu_mul_f32_matches_oracle(dev):
+    """qwhip_silu_mul_f32: FWHT32(silu(g) * u) in fp32 (QWGemmF32.swift:83-94); 1e-5 of the row's scale (the device's exp
+    differs from numpy's in the last bits), and the f16 door agrees with it after one rounding."""
+    rows, inter = 37, 416
+    rng = np.random.default_rng(5)
+    gu = (rng.standard_normal((rows, 2 * inter)) * 2.0).astype(np.float32)
+    gb, ab, hb = dev.put(gu), dev.alloc(rows * inter * 4), dev.alloc(rows * inter * 2)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_silu_mul_f32(st, gb.ptr, ab.ptr, rows, inter))
+    qwhip.check(lib.qwhip_swiglu_fwht(st, gb.ptr, qwhip.F32, hb.ptr, rows, inter, 1))
+    dev.stream.sync()
+    got, got16 = ab.download(np.float32, (rows, inter)), hb.download(np.float16, (rows, inter))
+    want = qo.silu_mul_f32(gu)
+    assert qo.normalized_error(got, want) <= 1e-6
+    assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+    assert np.array_equal(got.astype(np.float16).view(np.uint16), got16.view(np.uint16))
+    assert lib.qwhip_silu_mul_f32(st, gb.ptr, ab.ptr, rows, 40) == qwhip.E_BAD_SHAPE
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 256), (5, 2048), (40, 768)])
+def test_moe_bridge_matches_oracle(dev, rows, hidden):
+    """qwhip_moe_bridge_f16_to_f32 (QWGemmMoE.swift:337-377): the widened copy is exact; the un-rotated copy is the oracle's
+    bit for bit (fp32 butterfly in the same order, the same hi/lo split); NULL skips the rotated copy; hidden % 256."""
+    rng = np.random.default_rng(rows)
+    x16 = rng.standard_normal((rows, hidden)).astype(np.float16)
+    xb, rb, pb = dev.put(x16), dev.put(np.full((rows, hidden), 7.0, np.float32)), dev.alloc(rows * hidden * 4)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_moe_bridge_f16_to_f32(st, xb.ptr, rb.ptr, pb.ptr, rows, hidden))
+    dev.stream.sync()
+    rot, plain = qo.moe_bridge_f16_to_f32(x16)
+    assert np.array_equal(rb.download(np.float32, (rows, hidden)), rot)
+    assert np.array_equal(pb.download(np.float32, (rows, hidden)).view(np.uint32), plain.view(np.uint32))
+    rb2 = dev.put(np.full((rows, hidden), 7.0, np.float32))
+    qwhip.check(lib.qwhip_moe_bridge_f16_to_f32(st, xb.ptr, None, pb.ptr, rows, hidden))
+    dev.stream.sync()
+    assert np.all(rb2.download(np.float32, (rows, hidden)) == 7.0)
+    assert lib.qwhip_moe_bridge_f16_to_f32(st, xb.ptr, rb.ptr, pb.ptr, rows, hidden - 32) == qwhip.E_BAD_GEOMETRY
+
+
+@pytest.mark.parametrize("rows,latent", [(3, 96), (17, 1024), (2, 4128)])
+@pytest.mark.parametrize("norm", [True, False])
+def test_latent_norm_h32_matches_oracle(dev, rows, latent, norm):
+    """qwhip_latent_norm_h32_f32 (QWGemmF32.swift:57-80): with and without gamma, f32 and f16 outputs, either alone."""
+    rng = np.random.default_rng(latent)
+    x = (rng.standard_normal((rows, latent)) * 3.0).astype(np.float32)
+    gamma = (rng.standard_normal(latent) * 0.2).astype(np.float16)
+    xb, gb = dev.put(x), dev.put(gamma)
+    o32, o16 = dev.alloc(rows * latent * 4), dev.alloc(rows * latent * 2)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_latent_norm_h32_f32(st, xb.ptr, gb.ptr if norm else None, o32.ptr, o16.ptr, rows, latent, 1e-6))
+    dev.stream.sync()
+    want = qo.latent_norm_h32_f32(x, gamma if norm else None, 1e-6)
+    got32, got16 = o32.download(np.float32, (rows, latent)), o16.download(np.float16, (rows, latent))
+    if norm:
+        assert np.max(np.abs(got32 - want)) <= 2e-6 * np.max(np.abs(want))
+    else:
+        assert np.array_equal(got32.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(got16.view(np.uint16), got32.astype(np.float16).view(np.uint16))
+    o16b = dev.put(np.zeros((rows, latent), np.float16))
+    qwhip.check(lib.qwhip_latent_norm_h32_f32(st, xb.ptr, gb.ptr if norm else None, None, o16b.ptr, rows, latent, 1e-6))
+    dev.stream.sync()
+    assert np.array_equal(o16b.download(np.float16, (rows, latent)).view(np.uint16), got16.view(np.uint16))
+    assert lib.qwhip_latent_norm_h32_f32(st, xb.ptr, None, None, None, rows, latent, 1e-6) == qwhip.E_NULL
+    assert lib.qwhip_latent_norm_h32_f32(st, xb.ptr, None, o32.ptr, None, rows, 40, 1e-6) == qwhip.E_BAD_SHAPE
+
+
+def test_add_f32(dev):
+    rng = np.random.default_rng(1)
+    a, b = rng.standard_normal(100003).astype(np.float32), rng.standard_normal(100003).astype(np.float32)
+    ab, bb, ob = dev.put(a), dev.put(b), dev.alloc(a.size * 4)
+    qwhip.check(dev.lib.qwhip_add_f32(dev.stream.handle, ab.ptr, bb.ptr, ob.ptr, a.size))
+    dev.stream.sync()
+    assert np.array_equal(ob.download(np.float32, (a.size,)), a + b)

@@ -371,3 +371,38 @@ def test_embed_gather_reads_the_token_row():
     m5, _ = qo.quant_hq_blocks(w, bits=4, group=32, is_m5=True, rotate=True)
     got = qo.embed_aq_f32(m5, [5, 1], 1, 4, 32, True)[:, 0]
     assert np.array_equal(got, qo.dequant_hq4_rot(m5)[[5, 1]])
+
+
+def test_f32_seams_closed_forms():
+    """silu_mul_f32: a constant gate|up row gives sqrt(32) * silu(g) * u in column 0 of every group and zeros elsewhere;
+    bridge: the un-rotated copy of a rotated one-hot-in-standard-basis row is that one-hot (involution), the rotated copy
+    is the input widened, and the split keeps ~21 bits; latent norm: constant row with gamma 0 -> sqrt(32) * sign in column
+    0, gamma = 1 doubles it (plus-one law), no gamma = the bare transform, Parseval for the normalized row."""
+    import math
+    g, u = 0.75, -1.5
+    gu = np.concatenate([np.full((2, 64), g, np.float32), np.full((2, 64), u, np.float32)], axis=1)
+    out = qo.silu_mul_f32(gu)
+    want0 = math.sqrt(32.0) * (g / (1.0 + math.exp(-g))) * u
+    np.testing.assert_allclose(out[:, ::32], want0, rtol=2e-6)
+    mask = np.ones(64, bool)
+    mask[::32] = False
+    assert np.all(np.abs(out[:, mask]) <= 1e-6)
+    e = np.zeros((1, 256), np.float32)
+    e[0, 37] = 1.0
+    x16 = qo.fwht32_ortho(e).astype(np.float16)          # +-1/sqrt(32): f16-exact up to its rounding
+    rot, plain = qo.moe_bridge_f16_to_f32(x16)
+    assert np.array_equal(rot, x16.astype(np.float32))
+    np.testing.assert_allclose(plain, e, atol=2e-3 * 0.18)
+    rng = np.random.default_rng(8)
+    y16 = rng.standard_normal((3, 256)).astype(np.float16)
+    rot, plain = qo.moe_bridge_f16_to_f32(y16)
+    np.testing.assert_allclose(plain, qo.fwht32_ortho(y16.astype(np.float32)), rtol=0, atol=4 * 2.0 ** -21)   # hi/lo keeps 21+ bits
+    c = np.full((2, 96), -3.0, np.float32)
+    n0 = qo.latent_norm_h32_f32(c, np.zeros(96, np.float16), eps=0.0)
+    np.testing.assert_allclose(n0[:, ::32], -math.sqrt(32.0), rtol=1e-6)
+    n1 = qo.latent_norm_h32_f32(c, np.ones(96, np.float16), eps=0.0)
+    np.testing.assert_allclose(n1, 2.0 * n0, rtol=1e-6, atol=1e-6)
+    r = rng.standard_normal((4, 128)).astype(np.float32)
+    assert np.array_equal(qo.latent_norm_h32_f32(r), qo.fwht32_ortho(r))
+    nr = qo.latent_norm_h32_f32(r, np.zeros(128, np.float16), eps=0.0)
+    np.testing.assert_allclose((nr.astype(np.float64) ** 2).mean(axis=1), 1.0, rtol=1e-5)
