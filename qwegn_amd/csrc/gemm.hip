@@ -1612,8 +1612,19 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     if (m == 0) return QWHIP_OK;
     const uint32_t inter = w->n / 2u;
     if (w->n % 64u != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "fused gate_up needs an intermediate size %% 32 == 0, got %u rows", w->n);
-    if ((fmt != QG_FMT_M5 && fmt != QG_FMT_B4) || m % 64u != 0)
-        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the fused gate_up GEMM takes 4-bit containers and m %% 64 == 0 (m=%u): run qwhip_gemm + qwhip_swiglu_fwht", m);
+    if ((fmt != QG_FMT_M5 && fmt != QG_FMT_B4) || m % 64u != 0) {
+        // other containers and row counts: the two launches inside the door, through the caller's workspace
+        // ([m, 2 inter] f16 first, the rest for qwhip_gemm's own copy of the activations); same bits as the two doors
+        const uint64_t gu_bytes = (uint64_t)m * w->n * 2u;
+        if (!workspace || ((uintptr_t)workspace & 15u) || workspace_bytes < gu_bytes || (ldact != 0 && ldact != inter) || ((uintptr_t)act_f16 & 15u))
+            return qwhip_fail(QWHIP_E_BAD_GEOMETRY,
+                              "the fused gate_up GEMM takes 4-bit containers and m %% 64 == 0 in one launch (m=%u); other calls need a 16-byte "
+                              "aligned workspace of m * n * 2 bytes (plus m * k * 2 for bf16 or un-rotated activations) and packed act rows", m);
+        const uint64_t rest = workspace_bytes - gu_bytes;
+        st = qwhip_gemm(s, w, x, x_dtype, m, ldx, workspace, QWHIP_F16, 0, flags & QWHIP_X_PREROTATED, rest ? (uint8_t*)workspace + gu_bytes : nullptr, rest);
+        if (st != QWHIP_OK) return st;
+        return qwhip_swiglu_fwht(s, workspace, QWHIP_F16, act_f16, m, inter, rotate_act ? 1u : 0u);
+    }
     if (ldx == 0) ldx = w->k;
     if (ldact == 0) ldact = inter;
     if (ldx < w->k || ldact < inter || (ldx % 8) != 0 || (ldact % 8) != 0 || ((uintptr_t)act_f16 & 15u) != 0)

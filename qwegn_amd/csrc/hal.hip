@@ -311,9 +311,7 @@ static bool qw_parse_aq_name(const char* name, const char** launcher) {
         lau = "qwhip_moe_down_decode";
     }
     if (!lau) return false;
-    // every door takes the five widths except the fused dense gate|up GEMM (the ping-pong kernel's 4- and 8-bit name space)
-    const bool narrow_ok = strcmp(lau, "qwhip_gemm_swiglu") != 0;
-    if (!(bits == 4 || bits == 8 || (narrow_ok && (bits == 2 || bits == 3 || bits == 6)))) return false;
+    if (!(bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8)) return false;
     if (!(group == 32 || group == 64 || group == 128 || group == 256)) return false;
     if (launcher) *launcher = lau;
     return true;

@@ -100,7 +100,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
         assert lib.qwhip_kernel_lookup(name, C.byref(launcher)) == qwhip.OK, name
         assert launcher.value == want
         assert hasattr(lib, want.decode())
-    for missing in (b"qwg_gemv_shvq4_g32_v4", b"qwg_gemm_aq3_g32_h16_swiglu", b"qwg_gemv_aq5_g32_v4", b"qwg_head_gemv_shvq4_g32_argmax", b"nope"):
+    for missing in (b"qwg_gemv_shvq4_g32_v4", b"qwg_gemm_aq7_g32_h16_swiglu", b"qwg_gemv_aq5_g32_v4", b"qwg_head_gemv_shvq4_g32_argmax", b"nope"):
         assert lib.qwhip_kernel_lookup(missing, None) == qwhip.E_KERNEL_MISSING
         assert missing in lib.qwhip_last_error()
 

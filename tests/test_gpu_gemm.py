@@ -174,6 +174,38 @@ def test_gemm_swiglu_equals_gemm_then_swiglu(dev, fmt, xdtype, prerot, m, inter,
     assert qo.normalized_error(one.astype(np.float32), want) <= TOL
 
 
+@pytest.mark.parametrize("fmt,m", [("hq8_g32", 128), ("hq3_g32", 64), ("aq6_g128", 75), ("hq4_g32_m5", 37), ("aq2_g64", 200)])
+@pytest.mark.parametrize("xdtype,prerot", [("f16", True), ("bf16", False)])
+def test_gemm_swiglu_two_launch_form_through_the_workspace(dev, fmt, m, xdtype, prerot):
+    """Containers and row counts the one-launch kernel does not take run qwhip_gemm + qwhip_swiglu_fwht inside the door when
+    the workspace holds the [m, 2 inter] matrix: the same bits as the two doors called one after the other."""
+    inter, k = 224, 384
+    n = 2 * inter
+    rotate = H.FORMATS[fmt][4]
+    blocks, _ = H.make_bank(fmt, n, k, seed=4)
+    x32 = H.make_x(m, k, 13)
+    if xdtype == "bf16":
+        x_host, xcode = qo.f32_to_bf16_bits(x32), qwhip.BF16
+    else:
+        x_host, xcode = x32.astype(np.float16), qwhip.F16
+    flags = qwhip.X_PREROTATED if (prerot or not rotate) else 0
+    bank, xb = dev.put(blocks), dev.put(x_host)
+    gu, act2, act1 = dev.alloc(m * n * 2), dev.put(np.zeros((m, inter), np.float16)), dev.put(np.zeros((m, inter), np.float16))
+    ws1, ws2 = dev.alloc(m * k * 2), dev.alloc(m * n * 2 + m * k * 2)
+    view = H.view_of(dev, bank, fmt, n, k)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_gemm(st, C.byref(view), xb.ptr, xcode, m, 0, gu.ptr, qwhip.F16, 0, flags, ws1.ptr, ws1.nbytes))
+    qwhip.check(lib.qwhip_swiglu_fwht(st, gu.ptr, qwhip.F16, act2.ptr, m, inter, 1))
+    qwhip.check(lib.qwhip_gemm_swiglu(st, C.byref(view), xb.ptr, xcode, m, 0, 1, act1.ptr, 0, flags, ws2.ptr, ws2.nbytes))
+    dev.stream.sync()
+    one, two = act1.download(np.float16, (m, inter)), act2.download(np.float16, (m, inter))
+    assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
+    assert np.any(one != 0)
+    # a workspace that holds only the activation copy is refused, as before
+    assert lib.qwhip_gemm_swiglu(st, C.byref(view), xb.ptr, xcode, m, 0, 1, act1.ptr, 0, flags, ws1.ptr, ws1.nbytes) == (
+        qwhip.E_BAD_GEOMETRY if m * n * 2 > ws1.nbytes else qwhip.OK)
+
+
 def test_gemm_swiglu_refusals(dev):
     blocks, _ = H.make_bank("hq8_g32", 128, 64, seed=1)
     bank, xb, act = dev.put(blocks), dev.put(np.zeros((64, 64), np.float16)), dev.alloc(64 * 64 * 2)
