@@ -19,8 +19,13 @@
 // 4 (j >> 1) + 16 (j & 1) (unpack_hq4_word8, qw_dequant.metalh:42-62), the bit-stream containers element i at bit
 // i * bits, so a masked 4-bit word holds elements (k, k + 4), a masked 8-bit word elements (k, k + 2) and a masked 2-bit
 // word elements (k, k + 8) (sixteen codes a word; the four mask positions of a byte read as q, 4 q, 16 q and 64 q times
-// 2^-24 and get one accumulator each).  The 3- and 6-bit streams have no such in-place pairs: their codes are cut out
-// one by one and paired as neighbours.
+// 2^-24 and get one accumulator each).  A 3-bit stream has no two codes 16 bits apart, but any 32-bit window of it holds a
+// code start within bits 0..2 of each half: six windows of the slice's 96 bits (one funnel shift each), placed so that the
+// low half's codes start at bit 1 and the high half's at bit 0, give 15 pairs under three masks (fields at bits 1/0, 4/3,
+// 7/6: the values read as 2 q, q; 16 q, 8 q; 128 q, 64 q times 2^-24); the low activation of each pair is halved once in
+// the prologue so that both halves of a pair share a scale, and each mask gets its own accumulator.  Codes 30 and 31
+// are cut out the plain way.  The 6-bit stream has no in-place pairs: its codes are cut out one by one and paired as
+// neighbours.
 #include "qwhip_common.h"
 
 namespace {
@@ -38,7 +43,7 @@ template <int FMT>
 struct qcx_fmt {
     static constexpr int BITS = FMT == QW_FMT_B8 ? 8 : (FMT == QW_FMT_B2 ? 2 : (FMT == QW_FMT_B3 ? 3 : (FMT == QW_FMT_B6 ? 6 : 4)));
     static constexpr int PW = BITS;
-    static constexpr bool GENERIC = FMT == QW_FMT_B3 || FMT == QW_FMT_B6;   // codes cut out of the stream one by one
+    static constexpr bool GENERIC = FMT == QW_FMT_B6;   // codes cut out of the stream one by one
 };
 
 struct __attribute__((packed, aligned(4))) qcx_words4 { uint32_t q[4]; };
@@ -51,10 +56,33 @@ struct qcx_slice {
 };
 
 // The 16 operand pairs of one activation row for this lane's slice, in the order the masked code words come out.
+// 3-bit streams: operand i pairs the elements (QCX_B3_LO[i], QCX_B3_HI[i]); operands 0..6 sit under the first mask
+// (6 = codes 30, 31, cut out the plain way), 7..12 under the second, 13..15 under the third
+__device__ constexpr int QCX_B3_LO[16] = {0, 3, 10, 13, 20, 23, 30, 1, 4, 11, 14, 21, 24, 2, 12, 22};
+__device__ constexpr int QCX_B3_HI[16] = {5, 8, 15, 18, 25, 28, 31, 6, 9, 16, 19, 26, 29, 7, 17, 27};
+
 template <int FMT>
 __device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
     const h2_t one = {(h1_t)1.0f, (h1_t)1.0f};
     float s0 = 0.f, s1 = 0.f;
+    if constexpr (FMT == QW_FMT_B3) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const h2_t nat = {v[j][2 * k], v[j][2 * k + 1]};
+                if (k & 1) s1 = __builtin_amdgcn_fdot2(nat, one, s1, false);
+                else s0 = __builtin_amdgcn_fdot2(nat, one, s0, false);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int lo = QCX_B3_LO[i], hi = QCX_B3_HI[i];
+            const h1_t xl = v[lo >> 3][lo & 7], xh = v[hi >> 3][hi & 7];
+            xo[i] = h2_t{i == 6 ? xl : xl * (h1_t)0.5f, xh};   // the windows' low fields read twice their code
+        }
+        return s0 + s1;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -131,7 +159,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
     auto issue = [&](int slot) {
         const uint8_t* rp = p.bank + off;
         buf[slot].hdr = *(const uint32_t*)(rp + hdr_off);
-        if constexpr (qcx_fmt<FMT>::GENERIC || FMT == QW_FMT_B2) {
+        if constexpr (qcx_fmt<FMT>::GENERIC || FMT == QW_FMT_B2 || FMT == QW_FMT_B3) {
 #pragma unroll
             for (int j = 0; j < qcx_fmt<FMT>::PW; ++j) buf[slot].q[j] = *(const uint32_t*)(rp + pay_off + 4 * j);
         } else if constexpr (FMT == QW_FMT_B8) {
@@ -203,6 +231,33 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
                 };
 #pragma unroll
                 for (int i = 0; i < 16; ++i) ow[i] = code(2 * i) | (code(2 * i + 1) << 16);
+            } else if constexpr (FMT == QW_FMT_B3) {
+                // windows of the 96-bit slice at bits -1, 8, 29, 38, 59, 68: low-half codes start at window bit 1, high-half
+                // codes at bit 16 (elements: QCX_B3_LO / QCX_B3_HI)
+                const uint32_t w0 = b.q[0], w1 = b.q[1], w2 = b.q[2];
+                const uint32_t wa = w0 << 1;
+                const uint32_t wb = __builtin_amdgcn_alignbit(w1, w0, 8);
+                const uint32_t wc = __builtin_amdgcn_alignbit(w1, w0, 29);
+                const uint32_t wd = __builtin_amdgcn_alignbit(w2, w1, 6);
+                const uint32_t we = __builtin_amdgcn_alignbit(w2, w1, 27);
+                const uint32_t wf = w2 >> 4;
+                constexpr uint32_t M0 = 0x0007000Eu, M1 = 0x00380070u, M2 = 0x01C00380u;
+                ow[0] = wa & M0;
+                ow[1] = wb & M0;
+                ow[2] = wc & M0;
+                ow[3] = wd & M0;
+                ow[4] = we & M0;
+                ow[5] = wf & M0;
+                ow[6] = ((w2 >> 26) & 7u) | ((w2 >> 13) & 0x00070000u);   // codes 30 and 31
+                ow[7] = wa & M1;
+                ow[8] = wb & M1;
+                ow[9] = wc & M1;
+                ow[10] = wd & M1;
+                ow[11] = we & M1;
+                ow[12] = wf & M1;
+                ow[13] = wa & M2;
+                ow[14] = wc & M2;
+                ow[15] = we & M2;
             } else if constexpr (FMT == QW_FMT_B2) {
                 // operand 8 w + j: elements (16 w + j, 16 w + j + 8), masked in place at bits 2 (j & 3) of the bytes 0 / 2 of the
                 // word (j < 4) or of the word shifted down a byte (j >= 4)
@@ -239,15 +294,31 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
                 float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+                if constexpr (FMT == QW_FMT_B3) {
+                    // a0, a1: the first mask's seven operands; a2: the second mask's six; a3: the third mask's three
 #pragma unroll
-                for (int i = 0; i < 16; i += 4) {
-                    a0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 0]), xo[m][i + 0], a0, false);
-                    a1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 1]), xo[m][i + 1], a1, false);
-                    a2 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 2]), xo[m][i + 2], a2, false);
-                    a3 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 3]), xo[m][i + 3], a3, false);
+                    for (int i = 0; i < 7; ++i) {
+                        if (i & 1) a1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i]), xo[m][i], a1, false);
+                        else a0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i]), xo[m][i], a0, false);
+                    }
+#pragma unroll
+                    for (int i = 7; i < 13; ++i) a2 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i]), xo[m][i], a2, false);
+#pragma unroll
+                    for (int i = 13; i < 16; ++i) a3 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i]), xo[m][i], a3, false);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; i += 4) {
+                        a0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 0]), xo[m][i + 0], a0, false);
+                        a1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 1]), xo[m][i + 1], a1, false);
+                        a2 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 2]), xo[m][i + 2], a2, false);
+                        a3 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 3]), xo[m][i + 3], a3, false);
+                    }
                 }
                 float q;
-                if constexpr (FMT == QW_FMT_B8 || qcx_fmt<FMT>::GENERIC) {
+                if constexpr (FMT == QW_FMT_B3) {
+                    q = __builtin_fmaf(a2, 2097152.0f, (a0 + a1) * 16777216.0f);   // fields at bits 4 / 3 of the halves: 8 q
+                    q = __builtin_fmaf(a3, 262144.0f, q);                          // bits 7 / 6: 64 q
+                } else if constexpr (FMT == QW_FMT_B8 || qcx_fmt<FMT>::GENERIC) {
                     q = ((a0 + a1) + (a2 + a3)) * 16777216.0f;
                 } else if constexpr (FMT == QW_FMT_B2) {
                     q = __builtin_fmaf(a1, 4194304.0f, a0 * 16777216.0f);     // codes at bits 0..1 and 2..3 of a byte
