@@ -24,8 +24,9 @@
 // low half's codes start at bit 1 and the high half's at bit 0, give 15 pairs under three masks (fields at bits 1/0, 4/3,
 // 7/6: the values read as 2 q, q; 16 q, 8 q; 128 q, 64 q times 2^-24); the low activation of each pair is halved once in
 // the prologue so that both halves of a pair share a scale, and each mask gets its own accumulator.  Codes 30 and 31
-// are cut out the plain way.  The 6-bit stream has no in-place pairs: its codes are cut out one by one and paired as
-// neighbours.
+// are cut out the plain way.  A 6-bit stream works the same way with one pair a window: the window at bit 6 e holds code e
+// at bits 0..5 and code e + 3 at bits 18..23 (four times its value: the high activation of the pair is quartered in the
+// prologue), fifteen windows for the pairs (e, e + 3) and codes 30, 31 cut out the plain way, one scale class.
 #include "qwhip_common.h"
 
 namespace {
@@ -43,7 +44,6 @@ template <int FMT>
 struct qcx_fmt {
     static constexpr int BITS = FMT == QW_FMT_B8 ? 8 : (FMT == QW_FMT_B2 ? 2 : (FMT == QW_FMT_B3 ? 3 : (FMT == QW_FMT_B6 ? 6 : 4)));
     static constexpr int PW = BITS;
-    static constexpr bool GENERIC = FMT == QW_FMT_B6;   // codes cut out of the stream one by one
 };
 
 struct __attribute__((packed, aligned(4))) qcx_words4 { uint32_t q[4]; };
@@ -65,6 +65,24 @@ template <int FMT>
 __device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
     const h2_t one = {(h1_t)1.0f, (h1_t)1.0f};
     float s0 = 0.f, s1 = 0.f;
+    if constexpr (FMT == QW_FMT_B6) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const h2_t nat = {v[j][2 * k], v[j][2 * k + 1]};
+                if (k & 1) s1 = __builtin_amdgcn_fdot2(nat, one, s1, false);
+                else s0 = __builtin_amdgcn_fdot2(nat, one, s0, false);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 15; ++i) {   // operand i: elements (e, e + 3), e = 6 (i / 3) + i % 3
+            const int lo = 6 * (i / 3) + i % 3, hi = lo + 3;
+            xo[i] = h2_t{v[lo >> 3][lo & 7], v[hi >> 3][hi & 7] * (h1_t)0.25f};
+        }
+        xo[15] = h2_t{v[3][6], v[3][7]};
+        return s0 + s1;
+    }
     if constexpr (FMT == QW_FMT_B3) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -88,7 +106,7 @@ __device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             h2_t pr;
-            if constexpr (FMT == QW_FMT_M5 || qcx_fmt<FMT>::GENERIC) pr = h2_t{v[j][2 * k], v[j][2 * k + 1]};
+            if constexpr (FMT == QW_FMT_M5) pr = h2_t{v[j][2 * k], v[j][2 * k + 1]};
             else if constexpr (FMT == QW_FMT_B4) pr = h2_t{v[j][k], v[j][k + 4]};
             else if constexpr (FMT == QW_FMT_B2) pr = h2_t{v[2 * (j >> 1)][4 * (j & 1) + k], v[2 * (j >> 1) + 1][4 * (j & 1) + k]};
             else pr = h2_t{v[j][4 * (k >> 1) + (k & 1)], v[j][4 * (k >> 1) + (k & 1) + 2]};
@@ -159,7 +177,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
     auto issue = [&](int slot) {
         const uint8_t* rp = p.bank + off;
         buf[slot].hdr = *(const uint32_t*)(rp + hdr_off);
-        if constexpr (qcx_fmt<FMT>::GENERIC || FMT == QW_FMT_B2 || FMT == QW_FMT_B3) {
+        if constexpr (FMT == QW_FMT_B2 || FMT == QW_FMT_B3 || FMT == QW_FMT_B6) {
 #pragma unroll
             for (int j = 0; j < qcx_fmt<FMT>::PW; ++j) buf[slot].q[j] = *(const uint32_t*)(rp + pay_off + 4 * j);
         } else if constexpr (FMT == QW_FMT_B8) {
@@ -217,20 +235,16 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
             const qcx_slice<FMT> b = buf[j];
             issue(j);
             uint32_t ow[16];   // masked code words, operand order
-            if constexpr (qcx_fmt<FMT>::GENERIC) {
-                // 2-, 3- and 6-bit streams: element e at bit e * bits.  Each code is cut out of the stream (compile-time
-                // positions, at most two words) and two neighbours share an operand word as integers, i.e. as the f16
-                // subnormals code * 2^-24.
-                constexpr int BITS = qcx_fmt<FMT>::BITS;
-                constexpr uint32_t MASK = (1u << BITS) - 1u;
-                auto code = [&](int e) {
-                    const int off = e * BITS, wd = off >> 5, sh = off & 31;
-                    uint32_t c = b.q[wd] >> sh;
-                    if (sh + BITS > 32) c |= b.q[wd + 1] << (32 - sh);
-                    return c & MASK;
-                };
+            if constexpr (FMT == QW_FMT_B6) {
+                // window i at bit 6 e of the 192-bit slice, e = 6 (i / 3) + i % 3: code e at bits 0..5, code e + 3 at bits 18..23
+                constexpr uint32_t M = 0x00FC003Fu;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) ow[i] = code(2 * i) | (code(2 * i + 1) << 16);
+                for (int i = 0; i < 15; ++i) {
+                    const int bit = 6 * (6 * (i / 3) + i % 3), wd = bit >> 5, sh = bit & 31;
+                    const uint32_t win = sh == 0 ? b.q[wd] : __builtin_amdgcn_alignbit(b.q[wd + 1], b.q[wd], sh);
+                    ow[i] = win & M;
+                }
+                ow[15] = ((b.q[5] >> 20) & 0x3Fu) | ((b.q[5] >> 10) & 0x003F0000u);   // codes 30 and 31
             } else if constexpr (FMT == QW_FMT_B3) {
                 // windows of the 96-bit slice at bits -1, 8, 29, 38, 59, 68: low-half codes start at window bit 1, high-half
                 // codes at bit 16 (elements: QCX_B3_LO / QCX_B3_HI)
@@ -318,7 +332,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
                 if constexpr (FMT == QW_FMT_B3) {
                     q = __builtin_fmaf(a2, 2097152.0f, (a0 + a1) * 16777216.0f);   // fields at bits 4 / 3 of the halves: 8 q
                     q = __builtin_fmaf(a3, 262144.0f, q);                          // bits 7 / 6: 64 q
-                } else if constexpr (FMT == QW_FMT_B8 || qcx_fmt<FMT>::GENERIC) {
+                } else if constexpr (FMT == QW_FMT_B8 || FMT == QW_FMT_B6) {
                     q = ((a0 + a1) + (a2 + a3)) * 16777216.0f;
                 } else if constexpr (FMT == QW_FMT_B2) {
                     q = __builtin_fmaf(a1, 4194304.0f, a0 * 16777216.0f);     // codes at bits 0..1 and 2..3 of a byte
