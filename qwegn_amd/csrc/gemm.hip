@@ -663,10 +663,17 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
             uint8_t* row = lds2 + stage * STAGE + A_BYTES + (b_meta[i] & 0xFFFFu);
             const uint32_t sw = (b_meta[i] >> 16) & 7u, sl4 = (b_meta[i] >> 20) * 4u;
             if (SPLIT2 && i == 1) {
-                constexpr int WPC = FMT == QG_FMT_B8 ? 2 : 1;   // code words per 8-column chunk
+                // the half of the slice this thread dequantizes (chunks 0..1 or 2..3) moved to the front of a slice of its own
                 qg_slice<FMT> half;
+                if constexpr (FMT == QG_FMT_B3) {   // 24-bit chunks: the second pair starts in the middle of word 1
+                    half.q[0] = hi_half ? __builtin_amdgcn_alignbit(b_reg[i].q[2], b_reg[i].q[1], 16) : b_reg[i].q[0];
+                    half.q[1] = hi_half ? b_reg[i].q[2] >> 16 : b_reg[i].q[1];
+                    half.q[2] = 0;
+                } else {
+                    constexpr int HW = qg_slice_words<FMT>() / 2;   // code words of two 8-column chunks
 #pragma unroll
-                for (int w = 0; w < 2 * WPC; ++w) half.q[w] = hi_half ? b_reg[i].q[2 * WPC + w] : b_reg[i].q[w];
+                    for (int w = 0; w < HW; ++w) half.q[w] = hi_half ? b_reg[i].q[HW + w] : b_reg[i].q[w];
+                }
                 const uint32_t j0 = hi_half ? 2u : 0u;
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
@@ -1442,9 +1449,9 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     switch (cfg) {
         case CFG_256x320:
             // the ping-pong kernel takes whole 64-row activation blocks; ragged M stays on the DMA-fed kernel, and so do the
-            // 8-bit containers: their wider weight items do not fit the ping-pong kernel's register budget at this tile; the
-            // 2-, 3- and 6-bit streams stay there too (the ping-pong kernel splits a slice's words between two stores)
-            if constexpr (FMT == QG_FMT_M5 || FMT == QG_FMT_B4) {
+            // 8-bit containers: their wider weight items do not fit the ping-pong kernel's register budget at this tile (the
+            // 6-bit streams spill three to five registers there and still run a sixth faster than on the DMA-fed kernel)
+            if constexpr (FMT != QG_FMT_B8) {
                 if (p.M % 64u == 0 && !p.force_gemm2 &&
                     (YDT == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0)))
                     return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
@@ -1612,13 +1619,13 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     if (m == 0) return QWHIP_OK;
     const uint32_t inter = w->n / 2u;
     if (w->n % 64u != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "fused gate_up needs an intermediate size %% 32 == 0, got %u rows", w->n);
-    if ((fmt != QG_FMT_M5 && fmt != QG_FMT_B4) || m % 64u != 0) {
+    if (fmt == QG_FMT_B8 || fmt == QG_FMT_B6 || m % 64u != 0) {   // the 6- and 8-bit weight items do not fit the fused kernel's registers
         // other containers and row counts: the two launches inside the door, through the caller's workspace
         // ([m, 2 inter] f16 first, the rest for qwhip_gemm's own copy of the activations); same bits as the two doors
         const uint64_t gu_bytes = (uint64_t)m * w->n * 2u;
         if (!workspace || ((uintptr_t)workspace & 15u) || workspace_bytes < gu_bytes || (ldact != 0 && ldact != inter) || ((uintptr_t)act_f16 & 15u))
             return qwhip_fail(QWHIP_E_BAD_GEOMETRY,
-                              "the fused gate_up GEMM takes 4-bit containers and m %% 64 == 0 in one launch (m=%u); other calls need a 16-byte "
+                              "the fused gate_up GEMM takes 2-, 3- and 4-bit containers and m %% 64 == 0 in one launch (m=%u); other calls need a 16-byte "
                               "aligned workspace of m * n * 2 bytes (plus m * k * 2 for bf16 or un-rotated activations) and packed act rows", m);
         const uint64_t rest = workspace_bytes - gu_bytes;
         st = qwhip_gemm(s, w, x, x_dtype, m, ldx, workspace, QWHIP_F16, 0, flags & QWHIP_X_PREROTATED, rest ? (uint8_t*)workspace + gu_bytes : nullptr, rest);
@@ -1665,8 +1672,14 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     p.tiles_m = qwhip_cdiv(m, 256u);
     p.tiles_n = qwhip_cdiv(inter, 160u);
     const dim3 grid(((p.tiles_m * p.tiles_n + 7u) / 8u) * 8u);
-    const hipError_t e = fmt == QG_FMT_M5 ? launch_cfg3<2, 5, 4, 2, QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid)
-                                          : launch_cfg3<2, 5, 4, 2, QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
+    hipError_t e;
+    switch (fmt) {
+        case QG_FMT_M5: e = launch_cfg3<2, 5, 4, 2, QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid); break;
+        case QG_FMT_B4: e = launch_cfg3<2, 5, 4, 2, QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid); break;
+        case QG_FMT_B2: e = launch_cfg3<2, 5, 4, 2, QG_FMT_B2, QWHIP_F16, true>(s->stream, p, grid); break;
+        case QG_FMT_B3: e = launch_cfg3<2, 5, 4, 2, QG_FMT_B3, QWHIP_F16, true>(s->stream, p, grid); break;
+        default: e = hipErrorInvalidValue;
+    }
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
 }
