@@ -1074,9 +1074,9 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     }
 
     // transposing MFMA kernel: activations already in the basis.  Its cost barely grows with m: measured best from 13 rows
-    // on (N = 7168, K = 5120, HQ8: 16.9 us at m = 16 against 18.6 for the column-stationary MFMA kernel and 23.9 for the
-    // 4x4x4-block kernel; N = 5120, K = 17408, HQ4_G64: 34.8 against 40.8 for the streamer) and from 9 on short rows.
-    if (variant == 8 || (variant == 0 && !rotate && (m >= 13 || (m >= 9 && w->k <= 5120u)))) {
+    // on (N = 7168, K = 5120, HQ8: 16.0 / 16.9 us at m = 13 / 16 against 16.6 / 17.9 for the 4x4x4-block kernel and 18.6 for
+    // the column-stationary MFMA kernel; N = 5120, K = 17408, HQ4_G64: level with the 4x4x4-block kernel, 31.5 / 34.6 us).
+    if (variant == 8 || (variant == 0 && !rotate && m >= 13)) {
         hipError_t e = hipSuccess;
         bool done = false;
         if (fmt == QW_FMT_M5) done = launch_colt<QW_FMT_M5>(s->stream, a, x_dtype, &e);
@@ -1088,10 +1088,10 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
         }
         if (variant == 8) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the transposing MFMA kernel needs activations in the basis");
     }
-    // 4x4x4-block MFMA kernel: activations already in the basis.  Measured best for 2..8 rows (N = 7168, K = 5120, HQ8:
-    // 11.3 / 12.0 / 13.3 us at m = 2 / 4 / 8) and up to 12 rows on rows too long for the column-stationary MFMA kernel
-    // (N = 5120, K = 17408, HQ4_G64: 22.9 us at m = 8, 29.6 at m = 12 against 39-40 for the streamer).
-    if (variant == 7 || (variant == 0 && !rotate && m >= 2 && (m <= 8 || (m <= 12 && w->k > 5120u)))) {
+    // 4x4x4-block MFMA kernel: activations already in the basis.  Measured best for 2..12 rows (N = 7168, K = 5120, HQ8:
+    // 11.0 / 11.9 / 13.2 us at m = 2 / 4 / 8, 14.4 / 15.7 at m = 9 / 12 against 15.2 / 16.0 for the transposing kernel;
+    // N = 5120, K = 17408, HQ4_G64: 23.4 us at m = 8, 25.9 / 27.9 at m = 9 / 12 against 28.1 / 31.1).
+    if (variant == 7 || (variant == 0 && !rotate && m >= 2 && m <= 12)) {
         hipError_t e = hipSuccess;
         if (!rotate && qw_quad_gemv(s->stream, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, y16, y32, rt, &e)) {
             QWHIP_TRY_HIP(e);
