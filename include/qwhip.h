@@ -228,6 +228,11 @@ qwhip_status qwhip_add_f32(qwhip_stream_t s, const float* a, const float* b, flo
 qwhip_status qwhip_embed_aq_f32(qwhip_stream_t s, const qwhip_weight_view* table, const int32_t* tokens, uint32_t rows,
                                 uint32_t hc, float* out);
 
+/* The same gather from a raw bf16 table [vocab, hidden] (QWGemm.encodeEmbedBf16F32, Sources/Operators/QWGEMM/QWGemmF32.swift:352-363
+ * -> qwg_embed_bf16_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:102-116): out f32 [rows, hc, hidden], exact. */
+qwhip_status qwhip_embed_bf16_f32(qwhip_stream_t s, const void* table_bf16, uint32_t vocab, uint32_t hidden, const int32_t* tokens,
+                                  uint32_t rows, uint32_t hc, float* out);
+
 /* ---- prefill GEMM: Y[m, n] = X[m, k] . W^T on f16 MFMA, fp32 accumulate ------ */
 /* gemmBatchedH16 (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:119-154) -> qwg_gemm_q4g_h16 /
  * qwg_gemm_aq*_h16; QWGemm.encodeNaxF32 (Sources/Operators/QWGEMM/QWGemmF32.swift:366-402).

@@ -478,6 +478,34 @@ extern "C" qwhip_status qwhip_embed_aq_f32(qwhip_stream_t s, const qwhip_weight_
     return QWHIP_OK;
 }
 
+// The same gather from a raw bf16 table (qwg_embed_bf16_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:102-116; door
+// QWGemm.encodeEmbedBf16F32, Sources/Operators/QWGEMM/QWGemmF32.swift:352-363): a widening, exact.
+__global__ __launch_bounds__(256) void qw_embed_bf16_kernel(const uint16_t* __restrict__ table, const int32_t* __restrict__ tokens,
+                                                             float* __restrict__ out, uint32_t vocab, uint32_t hidden, uint32_t hc) {
+    const uint32_t r = blockIdx.y;
+    const uint32_t tok = min((uint32_t)max(tokens[r], 0), vocab - 1u);
+    const uint16_t* row = table + (uint64_t)tok * hidden;
+    for (uint32_t d = blockIdx.x * 256u + threadIdx.x; d < hidden; d += gridDim.x * 256u) {
+        const float v = __uint_as_float((uint32_t)row[d] << 16);
+        for (uint32_t c = 0; c < hc; ++c) out[((uint64_t)r * hc + c) * hidden + d] = v;
+    }
+}
+
+extern "C" qwhip_status qwhip_embed_bf16_f32(qwhip_stream_t s, const void* table_bf16, uint32_t vocab, uint32_t hidden, const int32_t* tokens,
+                                             uint32_t rows, uint32_t hc, float* out) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(table_bf16);
+    QWHIP_REQUIRE(tokens);
+    QWHIP_REQUIRE(out);
+    if (vocab == 0 || hidden == 0 || hc == 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "the embedding gather needs a positive shape");
+    if (rows > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "the embedding gather takes at most 65535 rows a launch, got %u", rows);
+    const dim3 grid(min(qwhip_cdiv(hidden, 256u), 4096u), rows), block(256);
+    hipLaunchKernelGGL(qw_embed_bf16_kernel, grid, block, 0, s->stream, (const uint16_t*)table_bf16, tokens, out, vocab, hidden, hc);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
 // ------------------------------------------------------------------------------------------------
 // RMSNorm with the rotation fused (the producer in front of every projection of a decode layer):
 //   y = f16( FWHT32( x * rsqrt(mean(x^2) + eps) * (1 + gamma) ) ),  optionally after  residual <- f16(residual + x)

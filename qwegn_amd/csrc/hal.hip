@@ -262,6 +262,7 @@ static const qw_kernel_entry g_kernels[] = {
     {"qwg_moe_route_decode", "qwhip_moe_route"},
     {"qwg_router_gemm", "qwhip_router_gemm"},
     {"qwg_embed_aq_f32", "qwhip_embed_aq_f32"},
+    {"qwg_embed_bf16_f32", "qwhip_embed_bf16_f32"},
     {"qwg_silu_mul_f32", "qwhip_silu_mul_f32"},
     {"qwg_moe_bridge_f16_to_f32", "qwhip_moe_bridge_f16_to_f32"},
     {"qwg_latent_norm_h32_f32", "qwhip_latent_norm_h32_f32"},

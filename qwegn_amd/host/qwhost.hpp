@@ -386,6 +386,16 @@ struct QWGemm {
             throwIfFailed(qwhip_silu_mul_f32(enc.stream, (const float*)gu.ptr(), (float*)act.ptr(), (uint32_t)rows, (uint32_t)inter));
         }
     }
+    // QWGemm.encodeEmbedBf16F32 (QWGemmF32.swift:352-363): the token's row of a raw bf16 table widened to f32, written hc times
+    static void encodeEmbedBf16F32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& table, const QWTensorValue& token, const QWTensorValue& out,
+                                   int hidden, int hc, int rows = 1) {
+        if (hidden <= 0 || hc <= 0 || rows <= 0 || table.shape.dtype != QWDType::bf16 || table.shape.elementCount < (size_t)hidden ||
+            token.shape.elementCount < (size_t)rows || out.shape.dtype != QWDType::f32 || out.shape.elementCount < (size_t)rows * (size_t)hidden * (size_t)hc)
+            throw QWGemmError(QWGemmError::badShape, "bf16 embedding gather: table bf16 [vocab, hidden], out f32 [rows, hc, hidden]");
+        hal.pipeline("qwg_embed_bf16_f32");
+        throwIfFailed(qwhip_embed_bf16_f32(enc.stream, table.ptr(), (uint32_t)(table.shape.elementCount / (size_t)hidden), (uint32_t)hidden,
+                                           (const int32_t*)token.ptr(), (uint32_t)rows, (uint32_t)hc, (float*)out.ptr()));
+    }
     // QWGemm.encodeAddF32 (QWGemmF32.swift:108-115)
     static void encodeAddF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& a, const QWTensorValue& b, const QWTensorValue& out, size_t count) {
         if (a.shape.elementCount < count || b.shape.elementCount < count || out.shape.elementCount < count || a.shape.dtype != QWDType::f32 ||

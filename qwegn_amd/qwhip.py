@@ -79,6 +79,7 @@ SIGNATURES = {
     "qwhip_moe_bridge_f16_to_f32": (C.c_int32, [_P, _P, _P, _P, _U32, _U32]),
     "qwhip_latent_norm_h32_f32": (C.c_int32, [_P, _P, _P, _P, _P, _U32, _U32, C.c_float]),
     "qwhip_add_f32": (C.c_int32, [_P, _P, _P, _P, C.c_uint64]),
+    "qwhip_embed_bf16_f32": (C.c_int32, [_P, _P, _U32, _U32, _P, _U32, _U32, _P]),
     "qwhip_embed_aq_f32": (C.c_int32, [_P, _P, _P, _U32, _U32, _P]),
     "qwhip_router_gemm_shared_gate": (C.c_int32, [_P, _P, _U32, _P, _U32, _U32, _U32, _U32, _P, _P, _P]),
     "qwhip_moe_max_tiles": (_U32, [_U32, _U32]),

@@ -411,3 +411,18 @@ def test_embed_gather_hq4_m5_and_errors(dev):
     assert lib.qwhip_embed_aq_f32(st, C.byref(view), tb.ptr, 4, 0, ob.ptr) == qwhip.E_BAD_WEIGHTS
     assert lib.qwhip_embed_aq_f32(st, C.byref(view), None, 4, 1, ob.ptr) == qwhip.E_NULL
     assert lib.qwhip_embed_aq_f32(st, C.byref(view), tb.ptr, 0, 1, None) == qwhip.OK
+
+
+def test_embed_gather_bf16_table(dev):
+    """Raw bf16 table -> f32, hc copies, exact (QWGemmF32.swift:352-363); negative and out-of-table tokens are clamped."""
+    vocab, hidden, hc = 50, 1000, 2
+    rng = np.random.default_rng(6)
+    table = qo.f32_to_bf16_bits(rng.standard_normal((vocab, hidden)).astype(np.float32))
+    tokens = np.array([49, 0, 7, -1, 50], np.int32)
+    tb, kb, ob = dev.put(table), dev.put(tokens), dev.alloc(tokens.size * hc * hidden * 4)
+    qwhip.check(dev.lib.qwhip_embed_bf16_f32(dev.stream.handle, tb.ptr, vocab, hidden, kb.ptr, tokens.size, hc, ob.ptr))
+    dev.stream.sync()
+    got = ob.download(np.float32, (tokens.size, hc, hidden))
+    want = qo.bf16_bits_to_f32(table)[np.clip(tokens, 0, vocab - 1)]
+    assert np.array_equal(got[:, 0], want) and np.array_equal(got[:, 1], want)
+    assert dev.lib.qwhip_embed_bf16_f32(dev.stream.handle, tb.ptr, vocab, hidden, kb.ptr, 1, 0, ob.ptr) == qwhip.E_BAD_SHAPE
