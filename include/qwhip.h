@@ -252,6 +252,15 @@ qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void
 qwhip_status qwhip_moe_route(qwhip_stream_t s, const float* logits, uint32_t t, uint32_t experts, uint32_t top_k,
                              uint32_t norm_topk, float routed_scale, int32_t* idx, float* wts);
 
+/* The same door with the reference's other routing modes (bias / splitFeature / routedScaleParam of encodeFnMoeRoute,
+ * QWGemmMoERouter.swift:10-58; qwrouter.metal:44-46,63-82,146-159): with a selection bias (f32 [experts]) and / or
+ * split_feature (logits [t, 2 experts]) the score is sigmoid(l) (+ sigmoid(l')), experts are chosen by score + bias and
+ * weighted by the score alone, renormalised by the sum of the selected + 1e-20; scale_param (f32 [experts], may be NULL)
+ * replaces routed_scale per selected expert.  bias = NULL, split_feature = 0: the softmax law of qwhip_moe_route. */
+qwhip_status qwhip_moe_route_ex(qwhip_stream_t s, const float* logits, uint32_t t, uint32_t experts, uint32_t top_k,
+                                uint32_t norm_topk, float routed_scale, uint32_t split_feature, const float* bias,
+                                const float* scale_param, int32_t* idx, float* wts);
+
 /* qwg_router_gemm (qwrouter.metal:460-; encodeFnRouterGemm, QWGemmMoERouter.swift:78-113):
  * logits[t, e] = sum_h x[t, h] * Wr[e, h]; x f16/bf16/f32, Wr f32/f16/bf16, fp32 accumulate. */
 qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,

@@ -639,6 +639,51 @@ def moe_route(logits: np.ndarray, top_k: int, norm_topk: bool = True, routed_sca
     return idx, wts
 
 
+def moe_route_ex(logits: np.ndarray, top_k: int, norm_topk: bool = True, routed_scale: float = 1.0, bias=None,
+                 split_feature: bool = False, scale_param=None):
+    """The router's other modes (Sources/QWMetal/subsystems/qwrouter.metal:44-46,63-82,113-159): with a selection bias and / or
+    split-feature logits [T, 2E] the score is sigmoid(l) (+ sigmoid(l')) in fp32, experts are chosen by score + bias (K rounds
+    of argmax, ties to the lower index; non-finite logits or scores never win) and weighted by the score alone, renormalised
+    by the fp32 sum of the selected (rank order) + 1e-20; a per-expert scale replaces the routed scale.  Without bias and
+    split features it is moe_route (softmax) with the per-expert scale."""
+    lg = np.asarray(logits, dtype=np.float32)
+    if bias is None and not split_feature:
+        idx, wts = moe_route(lg, top_k, norm_topk, 1.0)
+    else:
+        t = lg.shape[0]
+        e = lg.shape[1] // 2 if split_feature else lg.shape[1]
+        idx = np.full((t, top_k), -1, dtype=np.int32)
+        wts = np.zeros((t, top_k), dtype=np.float32)
+        one = np.float32(1.0)
+        with np.errstate(over="ignore", invalid="ignore"):
+            for r in range(t):
+                l0 = lg[r, :e]
+                sc = one / (one + np.exp(-l0).astype(np.float32))
+                ok = np.isfinite(l0)
+                if split_feature:
+                    l1 = lg[r, e:2 * e]
+                    sc = (sc + one / (one + np.exp(-l1).astype(np.float32))).astype(np.float32)
+                    ok &= np.isfinite(l1)
+                score = (sc + np.asarray(bias, dtype=np.float32)).astype(np.float32) if bias is not None else sc
+                ok &= np.isfinite(sc) & np.isfinite(score)
+                order = sorted([i for i in range(e) if ok[i]], key=lambda i: (-float(score[i]), i))[:top_k]
+                sel = np.array([sc[i] for i in order], dtype=np.float32)
+                if norm_topk:
+                    acc = np.float32(0)
+                    for v in sel:
+                        acc = np.float32(acc + v)
+                    acc = np.float32(acc + np.float32(1e-20))
+                    sel = (sel / acc).astype(np.float32) if acc > 0 else np.zeros_like(sel)
+                idx[r, :len(order)] = order
+                wts[r, :len(order)] = sel
+    if scale_param is not None:
+        sp = np.asarray(scale_param, dtype=np.float32)
+        scale = np.where(idx >= 0, sp[np.maximum(idx, 0)], np.float32(1.0)).astype(np.float32)
+    else:
+        scale = np.float32(routed_scale if routed_scale > 0 else 1.0)
+    return idx, (wts * scale).astype(np.float32)
+
+
 # --------------------------------------------------------------------------- #
 # expert-major pair sort and tile list  (pinned: math - permutation invariants, closed-form tile counts)
 # --------------------------------------------------------------------------- #

@@ -137,6 +137,49 @@ extern "C" qwhip_status qwhip_moe_route(qwhip_stream_t s, const float* logits, u
     return QWHIP_OK;
 }
 
+// The routing door with the reference's other modes (encodeFnMoeRoute's bias / splitFeature / routedScaleParam,
+// Sources/Operators/QWGEMM/QWGemmMoERouter.swift:10-58): sigmoid scoring when a selection bias or split-feature logits
+// ([t, 2 experts]) are given, softmax otherwise; a per-expert scale replaces the routed scale when given.
+template <int JN>
+__global__ __launch_bounds__(64) void qw_moe_route_ex_kernel(const float* __restrict__ logits, int32_t* __restrict__ idx,
+                                                              float* __restrict__ wts, uint32_t E, uint32_t K, uint32_t norm,
+                                                              float routed_scale, uint32_t split, const float* __restrict__ bias,
+                                                              const float* __restrict__ scale_param) {
+    const uint32_t t = blockIdx.x, lane = threadIdx.x;
+    const float* row = logits + (uint64_t)t * (split ? 2u * E : E);
+    int32_t isel;
+    float w;
+    if (bias || split) qw_route_wave_sigmoid<JN>(row, E, K, norm, split != 0, bias, lane, isel, w);
+    else qw_route_wave<JN>(row, E, K, norm, 1.0f, lane, isel, w);
+    if (lane < K) {
+        const float scale = (scale_param && isel >= 0) ? scale_param[(uint32_t)isel & 0xFFFFu] : routed_scale;
+        idx[(uint64_t)t * K + lane] = isel;
+        wts[(uint64_t)t * K + lane] = w * scale;
+    }
+}
+
+extern "C" qwhip_status qwhip_moe_route_ex(qwhip_stream_t s, const float* logits, uint32_t t, uint32_t experts, uint32_t top_k,
+                                           uint32_t norm_topk, float routed_scale, uint32_t split_feature, const float* bias,
+                                           const float* scale_param, int32_t* idx, float* wts) {
+    QWHIP_REQUIRE(s);
+    if (t == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(logits);
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(wts);
+    if (experts == 0 || experts > 512) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: experts must be 1..512, got %u", experts);
+    if (top_k == 0 || top_k > 16) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe route: top_k must be 1..16, got %u", top_k);
+    const float scale = routed_scale > 0.0f ? routed_scale : 1.0f;
+#define QW_ROUTE(J) hipLaunchKernelGGL(qw_moe_route_ex_kernel<J>, dim3(t), dim3(64), 0, s->stream, logits, idx, wts, experts, top_k, \
+                                       norm_topk ? 1u : 0u, scale, split_feature ? 1u : 0u, bias, scale_param)
+    if (experts <= 64) QW_ROUTE(1);
+    else if (experts <= 128) QW_ROUTE(2);
+    else if (experts <= 256) QW_ROUTE(4);
+    else QW_ROUTE(8);
+#undef QW_ROUTE
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
 // ------------------------------------------------------------------------------------------------
 // Expert-major pair sort: counting sort by expert id in one 1024-thread workgroup, plus the tile list.
 // ------------------------------------------------------------------------------------------------

@@ -101,3 +101,76 @@ __device__ __forceinline__ void qw_route_wave(const float* __restrict__ row, uin
     isel_out = isel;
     w_out = w * routed_scale;
 }
+
+// Sigmoid scoring of the same routine (the reference's selection-bias and split-feature modes,
+// Sources/QWMetal/subsystems/qwrouter.metal:63-82,113-159): score = sigmoid(l) (+ sigmoid(l') of the row's second half with
+// split features), experts are selected by score + bias (ties to the lower index), the weight of a selected expert is its
+// score without the bias, renormalised by the sum of the selected + 1e-20.  The caller applies the routed scale.
+template <int JN>
+__device__ __forceinline__ void qw_route_wave_sigmoid(const float* __restrict__ row, uint32_t E, uint32_t K, uint32_t norm, bool split,
+                                                      const float* __restrict__ bias, uint32_t lane, int32_t& isel_out, float& w_out) {
+    constexpr float NONE = -3.4e38f;
+    float ex[JN], cand[JN];
+#pragma unroll
+    for (uint32_t j = 0; j < JN; ++j) {
+        const uint32_t id = lane + 64u * j;
+        ex[j] = 0.0f;
+        cand[j] = NONE;
+        if (id < E) {
+            const float l0 = row[id];
+            float sc = 1.0f / (1.0f + expf(-l0));
+            bool okv = qw_finite(l0);
+            if (split) {
+                const float l1 = row[E + id];
+                sc += 1.0f / (1.0f + expf(-l1));
+                okv = okv && qw_finite(l1);
+            }
+            const float score = bias ? sc + bias[id] : sc;
+            okv = okv && qw_finite(sc) && qw_finite(score);
+            ex[j] = sc;
+            if (okv) cand[j] = score;
+        }
+    }
+    float wsel = 0.0f;
+    int32_t isel = -1;
+    for (uint32_t r = 0; r < K; ++r) {
+        float lm = cand[0];
+#pragma unroll
+        for (uint32_t j = 1; j < JN; ++j) lm = fmaxf(lm, cand[j]);
+        const float wm = qw_wave_max(lm);
+        uint32_t bi = 0xFFFFFFFFu;
+        if (wm > NONE) {
+#pragma unroll
+            for (uint32_t j = 0; j < JN; ++j) {
+                const unsigned long long m = __ballot(cand[j] == wm);
+                if (bi == 0xFFFFFFFFu && m != 0ull) bi = 64u * j + (uint32_t)__builtin_ctzll(m);
+            }
+        }
+        bi = __builtin_amdgcn_readfirstlane(bi);
+        float own = 0.0f;
+        if (bi != 0xFFFFFFFFu && (bi & 63u) == lane) {
+#pragma unroll
+            for (uint32_t j = 0; j < JN; ++j)
+                if (j == (bi >> 6)) {
+                    own = ex[j];
+                    cand[j] = NONE;
+                }
+        }
+        const float pw = bi != 0xFFFFFFFFu ? QW_LANE_F32(own, bi & 63u) : 0.0f;
+        if (lane == r) {
+            wsel = pw;
+            isel = bi != 0xFFFFFFFFu ? (int32_t)bi : -1;
+        }
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (uint32_t r = 0; r < 16; ++r)
+        if (r < K) acc += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wsel), r));
+    float w = wsel;
+    if (norm) {
+        acc += 1e-20f;
+        w = acc > 0.0f ? w / acc : 0.0f;
+    }
+    isel_out = isel;
+    w_out = w;
+}

@@ -514,14 +514,28 @@ struct QWGemm {
                                                     hasShGate ? (float*)shGateOut->ptr() : nullptr));
     }
     // encodeFnMoeRoute (QWGemmMoERouter.swift:10-75)
+    // bias (f32 [experts]) and / or splitFeature (logits [rows, 2 experts]) switch to sigmoid scoring; routedScaleParam (f32 [experts])
+    // replaces the routed scale per selected expert
     static void encodeFnMoeRoute(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& logits, const QWTensorValue& idx,
-                                 const QWTensorValue& wts, int rows, int experts, int topK, bool normTopK, float routedScale = 1.0f) {
+                                 const QWTensorValue& wts, int rows, int experts, int topK, bool normTopK, float routedScale = 1.0f,
+                                 const QWTensorValue* bias = nullptr, bool splitFeature = false, const QWTensorValue* routedScaleParam = nullptr) {
         if (experts > 512 || topK > 16 || topK <= 0) throw QWGemmError(QWGemmError::badShape, "router holds 512 experts and 16 routes");
         if (idx.shape.elementCount < (size_t)rows * (size_t)topK || wts.shape.elementCount < (size_t)rows * (size_t)topK)
             throw QWGemmError(QWGemmError::badShape, "router outputs are short");
+        if (logits.shape.elementCount < (size_t)rows * (size_t)experts * (splitFeature ? 2u : 1u) ||
+            (bias && (bias->shape.dtype != QWDType::f32 || bias->shape.elementCount < (size_t)experts)) ||
+            (routedScaleParam && (routedScaleParam->shape.dtype != QWDType::f32 || routedScaleParam->shape.elementCount < (size_t)experts)))
+            throw QWGemmError(QWGemmError::badShape, "router inputs are short");
         hal.pipeline("qwg_moe_route");
-        throwIfFailed(qwhip_moe_route(enc.stream, (const float*)logits.ptr(), (uint32_t)rows, (uint32_t)experts, (uint32_t)topK, normTopK ? 1 : 0,
-                                      routedScale, (int32_t*)idx.ptr(), (float*)wts.ptr()));
+        if (!bias && !splitFeature && !routedScaleParam) {
+            throwIfFailed(qwhip_moe_route(enc.stream, (const float*)logits.ptr(), (uint32_t)rows, (uint32_t)experts, (uint32_t)topK, normTopK ? 1 : 0,
+                                          routedScale, (int32_t*)idx.ptr(), (float*)wts.ptr()));
+        } else {
+            throwIfFailed(qwhip_moe_route_ex(enc.stream, (const float*)logits.ptr(), (uint32_t)rows, (uint32_t)experts, (uint32_t)topK, normTopK ? 1 : 0,
+                                             routedScale, splitFeature ? 1u : 0u, bias ? (const float*)bias->ptr() : nullptr,
+                                             routedScaleParam ? (const float*)routedScaleParam->ptr() : nullptr, (int32_t*)idx.ptr(),
+                                             (float*)wts.ptr()));
+        }
     }
     // encodeMoEGroupPairsF32 (QWGemmMoE.swift:68-99)
     static void encodeMoEGroupPairsF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& ids, const QWTensorValue& expertOff,

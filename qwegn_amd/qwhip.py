@@ -74,6 +74,7 @@ SIGNATURES = {
     "qwhip_gemv_silu_pair": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _U32, _P]),
     "qwhip_gemm": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _P, _U32, _U32, _U32, _P, _U64]),
     "qwhip_moe_route": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, C.c_float, _P, _P]),
+    "qwhip_moe_route_ex": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, C.c_float, _U32, _P, _P, _P, _P]),
     "qwhip_router_gemm": (C.c_int32, [_P, _P, _U32, _P, _U32, _U32, _U32, _U32, _P]),
     "qwhip_silu_mul_f32": (C.c_int32, [_P, _P, _P, _U32, _U32]),
     "qwhip_moe_bridge_f16_to_f32": (C.c_int32, [_P, _P, _P, _P, _U32, _U32]),

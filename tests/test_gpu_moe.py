@@ -102,6 +102,32 @@ def test_router_gemm_shared_gate_and_wide_rows(dev, t, e, h, wdt):
     assert lib.qwhip_router_gemm(st, xb.ptr, qwhip.F32, wb.ptr, wcode, t, e, 16388, l1.ptr) == qwhip.E_BAD_SHAPE
 
 
+@pytest.mark.parametrize("t,e,k", [(33, 128, 8), (5, 40, 4), (9, 512, 16), (7, 100, 3)])
+@pytest.mark.parametrize("mode", ["bias", "split", "bias+split", "softmax+scale"])
+@pytest.mark.parametrize("norm", [0, 1])
+def test_route_modes_match_oracle(dev, t, e, k, mode, norm):
+    """qwhip_moe_route_ex: sigmoid scoring with a selection bias and / or split-feature logits, and the per-expert scale;
+    the choice is the oracle's exactly (ties and non-finite logits included), the weights within 2e-6."""
+    rng = np.random.default_rng(t * 7 + e)
+    split = "split" in mode
+    lg = rng.standard_normal((t, 2 * e if split else e)).astype(np.float32)
+    lg[0, 1] = lg[0, 0]                                        # a tie
+    lg[t - 1, 2] = np.nan
+    lg[t - 1, 3] = -np.inf
+    bias = (rng.standard_normal(e) * 0.5).astype(np.float32) if "bias" in mode else None
+    scale = (rng.random(e) + 0.5).astype(np.float32) if "scale" in mode else None
+    lb, ib, wb = dev.put(lg), dev.alloc(t * k * 4), dev.alloc(t * k * 4)
+    bb = dev.put(bias) if bias is not None else None
+    sb = dev.put(scale) if scale is not None else None
+    qwhip.check(dev.lib.qwhip_moe_route_ex(dev.stream.handle, lb.ptr, t, e, k, norm, 1.5, 1 if split else 0, bb.ptr if bb else None,
+                                           sb.ptr if sb else None, ib.ptr, wb.ptr))
+    dev.stream.sync()
+    idx, wts = ib.download(np.int32, (t, k)), wb.download(np.float32, (t, k))
+    ridx, rwts = qo.moe_route_ex(lg, k, bool(norm), 1.5, bias=bias, split_feature=split, scale_param=scale)
+    assert np.array_equal(idx, ridx)
+    np.testing.assert_allclose(wts, rwts, rtol=2e-6, atol=1e-9)
+
+
 def _group(dev, ids, experts, top_k, compact=True):
     pairs = ids.size
     mt = max(1, dev.lib.qwhip_moe_max_tiles(experts, pairs))

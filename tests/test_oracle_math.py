@@ -406,3 +406,42 @@ def test_f32_seams_closed_forms():
     assert np.array_equal(qo.latent_norm_h32_f32(r), qo.fwht32_ortho(r))
     nr = qo.latent_norm_h32_f32(r, np.zeros(128, np.float16), eps=0.0)
     np.testing.assert_allclose((nr.astype(np.float64) ** 2).mean(axis=1), 1.0, rtol=1e-5)
+
+
+def test_route_modes_closed_forms():
+    """Sigmoid routing: without a bias the choice is the top-k of the logits (sigmoid is monotone) and normalised weights sum
+    to one; a large bias forces an expert in while its weight stays its own small score; split features add two sigmoids;
+    ties go to the lower index; a per-expert scale multiplies the normalised weight; no bias and no split = the softmax door."""
+    import math
+    rng = np.random.default_rng(12)
+    lg = rng.standard_normal((6, 40)).astype(np.float32)
+    idx, w = qo.moe_route_ex(lg, 4, True, 1.0, bias=np.zeros(40, np.float32))
+    for r in range(6):
+        assert sorted(idx[r].tolist()) == sorted(np.argsort(-lg[r], kind="stable")[:4].tolist())
+        assert abs(float(w[r].sum()) - 1.0) < 1e-6
+        assert np.all(np.diff(lg[r, idx[r]]) <= 0)                       # rank order = descending score
+    bias = np.zeros(40, np.float32)
+    bias[17] = 5.0
+    lg2 = lg.copy()
+    lg2[:, 17] = -6.0
+    idx2, w2 = qo.moe_route_ex(lg2, 4, False, 1.0, bias=bias)
+    assert np.all(idx2[:, 0] == 17)
+    np.testing.assert_allclose(w2[:, 0], 1.0 / (1.0 + math.exp(6.0)), rtol=1e-6)      # the score, not score + bias
+    sp = np.concatenate([lg, np.zeros_like(lg)], axis=1)                              # second half: sigmoid(0) = 1/2 everywhere
+    idx3, w3 = qo.moe_route_ex(sp, 4, False, 1.0, split_feature=True)
+    idx1, w1 = qo.moe_route_ex(lg, 4, False, 1.0, bias=np.zeros(40, np.float32))
+    assert np.array_equal(idx3, idx1)
+    np.testing.assert_allclose(w3, w1 + 0.5, rtol=1e-6)
+    tie = np.zeros((1, 8), np.float32)
+    idx4, _ = qo.moe_route_ex(tie, 3, True, 1.0, bias=np.zeros(8, np.float32))
+    assert idx4[0].tolist() == [0, 1, 2]
+    scale = np.arange(40, dtype=np.float32) + 1.0
+    idx5, w5 = qo.moe_route_ex(lg, 4, True, 7.0, bias=np.zeros(40, np.float32), scale_param=scale)
+    np.testing.assert_allclose(w5, w * scale[idx5], rtol=1e-6)
+    a, b = qo.moe_route_ex(lg, 4, True, 2.5), qo.moe_route(lg, 4, True, 2.5)
+    assert np.array_equal(a[0], b[0]) and np.allclose(a[1], b[1], rtol=1e-6)
+    nan = lg.copy()
+    nan[0, 3] = np.nan
+    nan[0, 5] = np.inf
+    idx6, _ = qo.moe_route_ex(nan, 40, False, 1.0, bias=np.zeros(40, np.float32))
+    assert 3 not in idx6[0].tolist() and 5 not in idx6[0].tolist() and (idx6[0] == -1).sum() == 2
