@@ -3,8 +3,11 @@
 This module restates, in numpy, the reference's algorithms for the QWGEMM path:
 the HQ4_G32_M5 and HQ/AQ block quantizers, their dequantizers, the 32-point
 orthonormal Walsh-Hadamard rotation, the oracle matmul forms, SwiGLU, the MoE
-router, the expert-major pair sort with its tile list, and the whole routed MoE
-block.  Only tests, the smoke check and the benchmark's CPU-baseline leg may
+router (softmax and sigmoid / bias / split-feature modes, the shared-expert gate), the
+expert-major pair sort with its tile list, the whole routed MoE block, and the seams
+either side of the path (RMSNorm + rotation, LM-head argmax, the f32 GEMV family, the
+embedding gather, the f32 bridge / SwiGLU / latent norm of the MoE chain, the MLX
+repacker).  Only tests, the smoke check and the benchmark's CPU-baseline leg may
 import it; the product path (libqwhip) never does.
 
 Every function cites the reference file:line it follows (paths relative to the
