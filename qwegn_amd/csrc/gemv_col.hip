@@ -13,7 +13,7 @@
 // qw_dequant.metalh:42-62).  The kernel never forms w: the masked nibble pairs are used directly as f16 operands -
 // bits 0..3 / 16..19 of a word read as two f16 subnormals q * 2^-24, bits 4..7 / 20..23 as 16 q * 2^-24
 // (v_dot2_f32_f16 honours f16 subnormals; products are exact, accumulation is fp32) - and the affine part is applied once
-// per block:  sum_i w_i x_i = s * (sum_i q_i x_i + 1024 S) + b * S,  S = sum_i x_i,
+// per block:  sum_i w_i x_i = s * sum_i q_i x_i + (1024 s + b) * S,  S = sum_i x_i,
 // the same factorisation the reference's bit-stream GEMVs use (qwg_aq_slice_dot, qw_dequant_multi.metalh:205-208).
 // The activations are the f16-rounded rotated values the reference's producers would have stored.
 #include "qwhip_common.h"
@@ -32,7 +32,9 @@ struct qc_params {
 // blockDim.x = 32 * cpr * SETS; dynamic LDS = nb * 80 + rows-per-workgroup * cpr * 4 bytes.
 template <int XDT, int SETS, int D, int D0>
 __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
-    constexpr int XT = SETS == 1 ? 4 : (SETS == 2 ? 2 : 1);   // 16-group activation tiles per wave: ceil(2 cpr / waves)
+    // 16-group activation tiles per full wave: ceil(2 cpr / full waves).  One row set with an odd cpr ends in a half
+    // wave, which takes no tile (its upper lanes do not exist): cpr = 13 leaves 6 full waves for 26 tiles.
+    constexpr int XT = SETS == 1 ? 5 : (SETS == 2 ? 2 : 1);
     extern __shared__ h8_t qc_lds[];
     const uint32_t nb = p.nb, cpr = p.cpr, N = p.N;
     h8_t* xs = qc_lds;                                 // 80 bytes per 32-group (64 used)
@@ -40,7 +42,8 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 31u, hw = tid >> 5;
     const uint32_t wave = tid >> 6, l64 = tid & 63u;
-    const uint32_t nw = (blockDim.x + 63u) >> 6;
+    const uint32_t nw = blockDim.x >> 6;               // full waves
+    const bool tiler = wave < nw;
     const uint32_t set = hw / cpr, chunk = hw - set * cpr;
     const uint32_t g0 = chunk * 32u + lane;
     const bool gvalid = g0 < nb;
@@ -77,8 +80,10 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
     {
         h8_t h_lo, h_hi;
         qw_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
+        if (tiler) {
 #pragma unroll
-        for (int t = 0; t < XT; ++t) qw_rotate_tile_to_lds(xv[t], wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs);
+            for (int t = 0; t < XT; ++t) qw_rotate_tile_to_lds(xv[t], wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs);
+        }
     }
     __syncthreads();
     // 4. this lane's column: 16 operand pairs and the group sum S
@@ -101,7 +106,6 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
         }
         S = s0 + s1;
     }
-    const float c1 = 1024.0f * S;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = D0; j < D; ++j) issue(j);
@@ -125,9 +129,11 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
             }
             issue(j);
             const h2_t hd = __builtin_bit_cast(h2_t, b.hdr);
-            float q = __builtin_fmaf(lo0 + lo1, 16777216.0f, c1);   // sum q x + 1024 S
-            q = __builtin_fmaf(hi0 + hi1, 1048576.0f, q);
-            float v = __builtin_fmaf((float)hd[0], q, (float)hd[1] * S);
+            // s * sum(q x) + (1024 s + b) * S: the header sum is exact in fp32 (two f16 values a factor 1024 / 1032 apart),
+            // so the large terms 1024 s S and b S never meet as rounded fp32 numbers
+            const float sc = (float)hd[0];
+            const float q = __builtin_fmaf(hi0 + hi1, 0.0625f, lo0 + lo1);
+            float v = __builtin_fmaf(sc * 16777216.0f, q, __builtin_fmaf(sc, 1024.0f, (float)hd[1]) * S);
             v = gvalid ? v : 0.0f;
             v = qw_reduce32_dpp(v);
             if (lane == 31u && rslot < nrows) part[rslot * cpr + chunk] = v;
