@@ -244,6 +244,17 @@ qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void
                         uint32_t m, uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags,
                         void* workspace, uint64_t workspace_bytes);
 
+/* qwhip_gemm for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks, kernels and
+ * results as qwhip_gemm; the f16 copy of the activations (rotated, or converted from bf16) goes to a static device array
+ * inside the library instead of the caller's workspace, and the call allocates nothing.  m * k * 2 must not exceed
+ * qwhip_gemm_noalloc_max_bytes() (8 MiB, held by every GPU the library runs on until the process ends), else
+ * QWHIP_E_BAD_SHAPE.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams) race;
+ * calls on one stream do not. */
+qwhip_status qwhip_gemm_noalloc(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
+                                uint32_t m, uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags);
+uint64_t qwhip_gemm_noalloc_max_bytes(void);
+
 /* ---- MoE --------------------------------------------------------------------- */
 /* qwg_moe_route (Sources/QWMetal/subsystems/qwrouter.metal:31-169; encodeFnMoeRoute,
  * Sources/Operators/QWGEMM/QWGemmMoERouter.swift:10-75): fp32 softmax over `experts`, top_k rounds of

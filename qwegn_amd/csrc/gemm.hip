@@ -18,6 +18,8 @@
 //
 // Grouped launches (MoE) take the tile list of the pair sort: tile t = (expert e, row block) over the
 // expert-major slot range [expert_off[e], expert_off[e+1]); slot rows are gathered through `gather`.
+#include <mutex>
+
 #include "qwhip_common.h"
 #include "qw_mfma_2x5.h"
 
@@ -1605,6 +1607,45 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     }
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;
+}
+
+// ---- qwhip_gemm for callers that cannot allocate ------------------------------------------------------------------------
+// The f16 copy of the activations (rotated, or converted from bf16) that qwhip_gemm keeps in the caller's workspace lives
+// here in a file-scope device array instead.  Each GPU holds its own copy of the array at its own address: the address is
+// resolved once per device, with that device current, from qwhip_device_create, and host code only ever uses the resolved
+// pointer (the array's name is not a device address on the host side).
+#define QW_GEMM_SCRATCH_BYTES (8u << 20)
+#define QW_GEMM_SCRATCH_DEVICES 64
+static __device__ __align__(256) uint8_t qw_gemm_scratch[QW_GEMM_SCRATCH_BYTES];
+static void* qw_gemm_scratch_ptr[QW_GEMM_SCRATCH_DEVICES];   // written under qw_gemm_scratch_mu, read after device creation
+static std::mutex qw_gemm_scratch_mu;
+
+// Called by qwhip_device_create with device `ordinal` current.
+qwhip_status qw_gemm_scratch_init(int ordinal) {
+    if (ordinal < 0 || ordinal >= QW_GEMM_SCRATCH_DEVICES) return QWHIP_OK;   // such a device has no static scratch; the entry point says so
+    std::lock_guard<std::mutex> lock(qw_gemm_scratch_mu);
+    if (qw_gemm_scratch_ptr[ordinal]) return QWHIP_OK;
+    void* ptr = nullptr;
+    QWHIP_TRY_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(qw_gemm_scratch)));
+    if (!ptr) return qwhip_fail(QWHIP_E_DEVICE, "hipGetSymbolAddress returned no address for the GEMM scratch array");
+    qw_gemm_scratch_ptr[ordinal] = ptr;
+    return QWHIP_OK;
+}
+
+extern "C" uint64_t qwhip_gemm_noalloc_max_bytes(void) { return QW_GEMM_SCRATCH_BYTES; }
+
+extern "C" qwhip_status qwhip_gemm_noalloc(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
+                                           uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags) {
+    QWHIP_REQUIRE(s);
+    QWHIP_REQUIRE(w);
+    const uint64_t need = (uint64_t)m * w->k * 2u;
+    if (need > QW_GEMM_SCRATCH_BYTES)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "qwhip_gemm_noalloc: m * k * 2 = %llu bytes exceeds the static scratch of %u bytes; use qwhip_gemm with a workspace",
+                          (unsigned long long)need, (unsigned)QW_GEMM_SCRATCH_BYTES);
+    const int ord = s->dev->ordinal;
+    void* scratch = (ord >= 0 && ord < QW_GEMM_SCRATCH_DEVICES) ? qw_gemm_scratch_ptr[ord] : nullptr;
+    if (!scratch) return qwhip_fail(QWHIP_E_DEVICE, "qwhip_gemm_noalloc: device %d has no resolved scratch array", ord);
+    return qwhip_gemm(s, w, x, x_dtype, m, ldx, y, y_dtype, ldy, flags, scratch, QW_GEMM_SCRATCH_BYTES);
 }
 
 // Dense gate|up GEMM with the SwiGLU (+ FWHT-32) epilogue fused: act f16 [m, inter], inter = n / 2, the bank's rows being

@@ -70,6 +70,12 @@ extern "C" qwhip_status qwhip_device_create(int32_t ordinal, qwhip_device_t* out
         delete d;
         return qwhip_hip_check(e, "hipSetDevice");
     }
+    // per-device address of the static GEMM scratch (gemm.hip), resolved while this device is current
+    const qwhip_status sst = qw_gemm_scratch_init(ordinal);
+    if (sst != QWHIP_OK) {
+        delete d;
+        return sst;
+    }
     *out = d;
     return QWHIP_OK;
 }

@@ -34,6 +34,9 @@ qwhip_status qwhip_hip_check(hipError_t e, const char* what);
 // elementwise.hip: src (f16 | bf16 | f32) -> f16, no rotation (internal helper of the GEMM pre-pass)
 qwhip_status qw_convert_to_f16(qwhip_stream_t s, const void* src, uint32_t src_dtype, void* dst_f16, uint64_t n);
 
+// gemm.hip: resolves this device's address of the static scratch array behind qwhip_gemm_noalloc (device `ordinal` current)
+qwhip_status qw_gemm_scratch_init(int ordinal);
+
 static inline uint32_t qwhip_cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
 // Block bytes of a validated view.

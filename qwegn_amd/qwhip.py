@@ -73,6 +73,8 @@ SIGNATURES = {
     "qwhip_gemv": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _P, _P]),
     "qwhip_gemv_silu_pair": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _U32, _P]),
     "qwhip_gemm": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _P, _U32, _U32, _U32, _P, _U64]),
+    "qwhip_gemm_noalloc": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _P, _U32, _U32, _U32]),
+    "qwhip_gemm_noalloc_max_bytes": (_U64, []),
     "qwhip_moe_route": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, C.c_float, _P, _P]),
     "qwhip_moe_route_ex": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, C.c_float, _U32, _P, _P, _P, _P]),
     "qwhip_router_gemm": (C.c_int32, [_P, _P, _U32, _P, _U32, _U32, _U32, _U32, _P]),
