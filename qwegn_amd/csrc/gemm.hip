@@ -49,16 +49,9 @@ struct qw_gemm_params {
     uint32_t rows_per_expert;
     uint32_t inter, rotate_act;  // fused SwiGLU epilogue: gate rows [0, inter), up rows [inter, 2 inter) of an expert; FWHT-32 on the result
     uint32_t force_gemm2;  // tuning / tests: keep the DMA-fed kernel for the 256 x 320 shape
-#ifdef QW_GEMM_TIMING
-    unsigned long long* tlog;  // probe builds only: per-phase cycle stamps of workgroup 0, wave 0
-#endif
+    uint32_t x_bf16;       // ping-pong kernel: activations are bf16, converted while the tile is staged
 };
 
-#ifdef QW_GEMM_TIMING
-#define QW_TSTAMP(slot) do { if (blockIdx.x == 8 && threadIdx.x == 0 && kt < 64) p.tlog[kt * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define QW_TSTAMP(slot) do { } while (0)
-#endif
 
 struct __attribute__((packed, aligned(4))) qg_words4 { uint32_t q[4]; };
 struct __attribute__((packed, aligned(4))) qg_words8 { uint32_t q[8]; };
@@ -171,13 +164,16 @@ __device__ __forceinline__ h8_t qg_to_f16x8(u4_t raw) {
     if constexpr (XDT == QWHIP_F16) {
         return __builtin_bit_cast(h8_t, raw);
     } else {
-        h8_t o;
+        // a bf16 pair widens with one shift and one mask; v_cvt_pk_f16_f32 rounds both to f16 (to nearest even, exact for
+        // every bf16 value f16 holds as a normal number)
+        typedef float fl2_t __attribute__((ext_vector_type(2)));
+        u4_t o;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            o[2 * j] = (h1_t)__uint_as_float(raw[j] << 16);
-            o[2 * j + 1] = (h1_t)__uint_as_float(raw[j] & 0xFFFF0000u);
+            const fl2_t v = {__uint_as_float(raw[j] << 16), __uint_as_float(raw[j] & 0xFFFF0000u)};
+            o[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h2_t));
         }
-        return o;
+        return __builtin_bit_cast(h8_t, o);
     }
 }
 
@@ -506,7 +502,6 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
     // compiler wait on the load right where it is issued).
     for (uint32_t kt = 0; kt + 1 < nk; ++kt) {
         const uint32_t cur = kt & 1u, nxt = cur ^ 1u;
-        QW_TSTAMP(0);
 #ifndef QW_PROBE_SKIP_ADMA
         dma_a(kt + 1, nxt);
 #endif
@@ -515,13 +510,9 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 #endif
         __builtin_amdgcn_sched_barrier(0);             // keep the loads at the top: their latency hides behind the MFMAs
         mfma_step(lds2 + cur * STAGE);
-        QW_TSTAMP(1);
         store_b(nxt);
-        QW_TSTAMP(2);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        QW_TSTAMP(3);
         __syncthreads();
-        QW_TSTAMP(4);
     }
     mfma_step(lds2 + ((nk - 1) & 1u) * STAGE);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -561,7 +552,9 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 // columns, two across the four lanes of a 32-column group) and stores act f16 [m, inter]: the reference's fused dense
 // gate_up kernel (qwg_gemm_q4g_h16_swiglu: qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167),
 // bit-identical to qwhip_gemm with f16 output followed by qwhip_swiglu_fwht.
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false>
+// XDT = bf16: the activation tile is converted to f16 on its way from the load registers into LDS (12 vector operations
+// per 16-byte piece, inside the filling phase), so bf16 activations need no pass of their own and no workspace.
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false, int XDT = QWHIP_F16>
 __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_params p) {
     static_assert(WVM * WVN == 8, "two groups of four waves");
     static_assert(!SWIGLU || (WVN == 2 && YDT == QWHIP_F16), "fused SwiGLU: gate and up wave columns, f16 out");
@@ -647,7 +640,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
-        for (int i = 0; i < A_LD; ++i) *(u4_t*)(lds2 + stage * STAGE + a_lds0 + i * (A_BLK * 128u)) = a_reg[i];
+        for (int i = 0; i < A_LD; ++i) *(h8_t*)(lds2 + stage * STAGE + a_lds0 + i * (A_BLK * 128u)) = qg_to_f16x8<XDT>(a_reg[i]);
     };
     auto load_b = [&](uint32_t kt, qg_slice<FMT>* b_reg, int nitems) {
 #pragma unroll
@@ -1397,11 +1390,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false, int XDT = QWHIP_F16>
 hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, SWIGLU>;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, SWIGLU, XDT>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1442,6 +1435,13 @@ enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_256x128 = 3, CFG_C
 static const uint32_t kCfgBM[CFG_COUNT] = {256, 256, 128, 256};
 static const uint32_t kCfgBN[CFG_COUNT] = {320, 256, 128, 128};
 
+// the ping-pong kernel takes whole 64-row activation blocks on the 256 x 320 tile, every container but the 8-bit ones, and
+// 2-byte outputs whose rows are 16-byte aligned
+inline bool gemm3_takes(const qw_gemm_params& p, int cfg, int fmt, uint32_t ydt) {
+    return cfg == CFG_256x320 && fmt != QG_FMT_B8 && p.M % 64u == 0 && !p.force_gemm2 &&
+           (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0));
+}
+
 template <int FMT, int YDT>
 hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     p.tiles_m = qwhip_cdiv(p.M, kCfgBM[cfg]);
@@ -1454,9 +1454,10 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
             // 8-bit containers: their wider weight items do not fit the ping-pong kernel's register budget at this tile (the
             // 6-bit streams spill three to five registers there and still run a sixth faster than on the DMA-fed kernel)
             if constexpr (FMT != QG_FMT_B8) {
-                if (p.M % 64u == 0 && !p.force_gemm2 &&
-                    (YDT == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0)))
+                if (gemm3_takes(p, cfg, FMT, YDT)) {
+                    if (p.x_bf16) return launch_cfg3<2, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
                     return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
+                }
             }
             return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x256: return launch_cfg2<2, 4, 4, 2, FMT, YDT, false>(st, p, grid);
@@ -1561,7 +1562,20 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     const bool ws_ok = workspace && workspace_bytes >= ws_need && ldx == w->k && ((uintptr_t)workspace & 15u) == 0;
     const void* xin = x;
     uint32_t xdt = x_dtype;
-    if (rotate) {
+    const uint32_t ov = (flags >> 8) & 0xFu;
+    const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n));
+    qw_gemm_params p = {};
+    p.M = m;
+    p.ldy = ldy;
+    p.y = y;
+    p.force_gemm2 = ov == 14u ? 1u : 0u;
+    // bf16 activations already in the basis: the ping-pong kernel converts them while it stages the tile (no pass of its own,
+    // no workspace); flags bit 16 keeps the separate pass, for tests and comparisons
+    const bool direct_bf16 = !rotate && x_dtype == QWHIP_BF16 && ov != 15u && !(flags & (1u << 16)) && gemm3_takes(p, cfg, fmt, y_dtype);
+    if (direct_bf16) {
+        p.x_bf16 = 1u;
+        xdt = QWHIP_F16;   // dispatch as the f16 kernels do; the kernel itself reads bf16
+    } else if (rotate) {
         // rotated f16 copy of the activations in the caller's workspace, then the GEMM reads that
         if (!workspace || workspace_bytes < ws_need)
             return qwhip_fail(QWHIP_E_BASIS,
@@ -1580,19 +1594,14 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
         xdt = QWHIP_F16;
     }
 
-    qw_gemm_params p = {};
     p.bank = (const uint8_t*)w->blocks;
     p.x = xin;
-    p.y = y;
-    p.M = m;
     p.N = w->n;
     p.K = w->k;
     p.ldx = ldx;
-    p.ldy = ldy;
     p.gshift = log2_u32(w->group / 32);
     p.bb = qwhip_view_block_bytes(w);
     p.row_bytes = qwhip_view_row_bytes(w);
-    const uint32_t ov = (flags >> 8) & 0xFu;
     hipError_t e;
     if (xdt != QWHIP_F16 || ov == 15u) {
         if (xdt == QWHIP_F16) {
@@ -1601,8 +1610,6 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
             QG_FOR_FMT(fmt, e, (launch_dense1_y<F, QWHIP_BF16>(s->stream, p, y_dtype)))
         }
     } else {
-        const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n));
-        p.force_gemm2 = ov == 14u ? 1u : 0u;
         QG_FOR_FMT(fmt, e, (launch_dense2_y<F>(s->stream, p, cfg, y_dtype)))
     }
     QWHIP_TRY_HIP(e);
