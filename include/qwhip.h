@@ -371,6 +371,23 @@ qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_
 qwhip_status qwhip_quantize_hq4_g32(qwhip_stream_t s, const void* src, uint32_t src_dtype, uint32_t n, uint32_t k,
                                     uint32_t rotate, void* blocks_out);
 
+/* Bit-stream block writer for the non-M5 containers, the device twin of quant_hq_blocks (Scripts/quantize/hq_blocks.py:436-517; the
+ * packer's own GPU path is the quant_hq_simd shader at :260): src [n, k] bf16 or f32 -> [n, k / group] blocks of
+ * 4 + group * bits / 8 bytes, byte-identical to the packer.  bits in {2, 3, 4, 6, 8}, group in {32, 64, 128, 256} with
+ * k % group == 0 (the packer's gcd rule is the caller's: pass the resolved group); rotate = FWHT-32 over every 32 weights first.
+ * mse_clip: 0 plain min / max, 1 the ten-point shrink search (:409-432), 2 the packer's default (the search for 2 and 3 bits).
+ * Non-finite weights, which the packer refuses, give unspecified blocks. */
+qwhip_status qwhip_quantize_blocks(qwhip_stream_t s, const void* src, uint32_t src_dtype, uint32_t n, uint32_t k,
+                                   uint32_t bits, uint32_t group, uint32_t rotate, uint32_t mse_clip, void* blocks_out);
+
+/* Planar HQ8_G32_M5 (quant_hq8_g32_m5 / dequant_hq8_g32_m5_rot, hq_blocks.py:564-615; host reader dequantHQ8Rot,
+ * Sources/Foundation/QWQuant/QWPack.swift:326-351): int8 codes [n, k] and f16 scales [n, k / 32] as two planes, symmetric,
+ * scale = f16(amax / 127); the dequant writes the rotated-domain fp32 weights code * scale. */
+qwhip_status qwhip_quantize_hq8_planar(qwhip_stream_t s, const void* src, uint32_t src_dtype, uint32_t n, uint32_t k,
+                                       uint32_t rotate, void* qs_out, void* scales_out_f16);
+qwhip_status qwhip_dequant_hq8_planar(qwhip_stream_t s, const void* qs, const void* scales_f16, uint32_t n, uint32_t k,
+                                      float* out_f32);
+
 /* qwg_repack_mlx_affine_to_aq_m5 / qwg_repack_mlx_affine_switch_gate_up_to_aq_m5
  * (Sources/QWMetal/quant/qw_online_quant.metal:56-178; QWAQRepack.repackMLXAffine / repackMLXAffineSwitchGateUp,
  * Sources/Foundation/QWLoad/AQRepack.swift:108-250): an MLX affine checkpoint (packed codes u32, scales and biases

@@ -184,6 +184,26 @@ class Pack:
             raise QWQuantError("badPlane", f"{name}: offset {off} size {nbytes} outside the pack's data")
         return layout, self.raw[off:off + nbytes]
 
+    def hq8_planes(self, name: str) -> tuple[np.ndarray, np.ndarray]:
+        """Planar HQ8_G32_M5 entry: (int8 codes [n, k], f16 scales [n, k / 32]) as views of the mapping
+        (QWQuant.Pack.dequantHQ8Rot reads the same two planes, Sources/Foundation/QWQuant/QWPack.swift:326-351)."""
+        e = self.entry(name)
+        if not e.hq8_quantized or e.hq8_s_off is None or len(e.shape) != 2 or e.shape[1] % GROUP != 0:
+            raise QWQuantError("badPlane", f"{name} is not a 2-D planar HQ8 tensor")
+        n, k = e.shape
+        q_bytes, s_bytes = n * k, n * (k // GROUP) * 2
+        for off, size in ((e.hq8_off, q_bytes), (e.hq8_s_off, s_bytes)):
+            if off < 12 or off + size > self.data_end:
+                raise QWQuantError("badPlane", f"{name}: offset {off} size {size} outside the pack's data")
+        qs = self.raw[e.hq8_off:e.hq8_off + q_bytes].view(np.int8).reshape(n, k)
+        scales = self.raw[e.hq8_s_off:e.hq8_s_off + s_bytes].view(np.float16).reshape(n, k // GROUP)
+        return qs, scales
+
+    def upload_hq8(self, dev: "qwhip.Device", name: str):
+        """Moves a planar HQ8 entry into two device buffers: (codes, scales, n, k); qwhip_dequant_hq8_planar reads them."""
+        qs, scales = self.hq8_planes(name)
+        return dev.put(np.ascontiguousarray(qs)), dev.put(np.ascontiguousarray(scales)), qs.shape[0], qs.shape[1]
+
     def weight_geometry(self, name: str) -> tuple[int, int, int, int, int]:
         """(rows, k, kind, bits, group) of a quantized entry as the weight view wants it: an expert stack
         [E, N, K] is one bank of E * N rows (expert e at row e * N)."""

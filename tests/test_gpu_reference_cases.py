@@ -8,6 +8,7 @@ import pytest
 
 from oracle import qworacle as qo
 from qwegn_amd import qwhip
+from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
 M64 = (1 << 64) - 1
@@ -426,3 +427,91 @@ def test_embed_gather_bf16_table(dev):
     want = qo.bf16_bits_to_f32(table)[np.clip(tokens, 0, vocab - 1)]
     assert np.array_equal(got[:, 0], want) and np.array_equal(got[:, 1], want)
     assert dev.lib.qwhip_embed_bf16_f32(dev.stream.handle, tb.ptr, vocab, hidden, kb.ptr, 1, 0, ob.ptr) == qwhip.E_BAD_SHAPE
+
+
+# ---- load-time writers for the non-M5 containers -----------------------------------------------------------------------
+BLOCK_CASES = [
+    # name in hq_blocks_golden.npz, bits, group, rotate
+    ("aq4_g32_std", 4, 32, False), ("hq4_g32_blk", 4, 32, True), ("hq4_g64", 4, 64, True), ("hq8_g32", 8, 32, True),
+    ("hq8_g64", 8, 64, True), ("hq6_g32", 6, 32, True), ("hq4_g128", 4, 128, True), ("hq8_g256", 8, 256, True),
+    ("hq2_g64", 2, 64, True), ("hq3_g32", 3, 32, True),
+]
+
+
+@pytest.mark.parametrize("name,bits,group,rotate", BLOCK_CASES)
+def test_device_block_quantizer_writes_the_packers_bytes(dev, golden_dir, name, bits, group, rotate):
+    """qwhip_quantize_blocks against the block bytes the reference's quant_hq_blocks wrote for the same input
+    (tests/golden/hq_blocks_golden.npz: an outlier, a constant group, tiny values, ties; the 2- and 3-bit cases run the
+    shrink search), f32 source."""
+    gold = np.load(golden_dir / "hq_blocks_golden.npz")
+    w = gold["w"]
+    want = gold[f"{name}__blocks"]
+    n, k = w.shape
+    src, out = dev.put(w), dev.alloc(want.nbytes)
+    qwhip.check(dev.lib.qwhip_quantize_blocks(dev.stream.handle, src.ptr, qwhip.F32, n, k, bits, group, int(rotate), 2, out.ptr))
+    got = out.download(np.uint8, want.shape)
+    assert np.array_equal(got, want)
+    for b in (src, out):
+        b.free()
+
+
+@pytest.mark.parametrize("fmt", ["aq4_g32", "hq4_g64", "hq8_g32", "hq8_g64", "hq4_g128", "aq8_g256", "hq6_g32", "aq6_g128", "aq2_g64", "hq3_g32"])
+@pytest.mark.parametrize("src_dtype", ["f32", "bf16"])
+def test_device_block_quantizer_matches_the_oracle_on_seeded_weights(dev, fmt, src_dtype):
+    """Every container of the tests on N(0, 0.02) weights: device bytes == the oracle's bytes; bf16 sources are widened
+    exactly.  k = 1536 gives ragged group counts per wave for the wide groups; a bank written on the device dequantizes to the
+    oracle's f16 weights bit for bit."""
+    kind, bits, group, is_m5, rotate = H.FORMATS[fmt]
+    n, k = 40, 1536
+    w = H.make_weights(n, k, seed=17)
+    if src_dtype == "bf16":
+        bits16 = qo.f32_to_bf16_bits(w)
+        w = qo.bf16_bits_to_f32(bits16)
+        src, code = dev.put(bits16), qwhip.BF16
+    else:
+        src, code = dev.put(w), qwhip.F32
+    want, eff = qo.quant_hq_blocks(w, bits=bits, group=group, is_m5=False, rotate=rotate)
+    out = dev.alloc(want.nbytes)
+    qwhip.check(dev.lib.qwhip_quantize_blocks(dev.stream.handle, src.ptr, code, n, k, bits, group, int(rotate), 2, out.ptr))
+    assert np.array_equal(out.download(np.uint8, want.shape), want)
+    deq = dev.alloc(n * k * 2)
+    view = dev.view(out, n, k, kind, bits, group)
+    qwhip.check(dev.lib.qwhip_dequant_f16(dev.stream.handle, C.byref(view), deq.ptr))
+    assert np.array_equal(deq.download(np.float16, (n, k)).view(np.uint16), qo.weights_f16_exact(want, bits, group, False).view(np.uint16))
+    for b in (src, out, deq):
+        b.free()
+
+
+def test_block_quantizer_rejects_bad_calls(dev):
+    src, out = dev.put(np.zeros((4, 96), np.float32)), dev.alloc(4096)
+    lib, st = dev.lib, dev.stream.handle
+    assert lib.qwhip_quantize_blocks(st, src.ptr, qwhip.F32, 4, 96, 5, 32, 1, 2, out.ptr) == qwhip.E_BAD_WEIGHTS     # no 5-bit container
+    assert lib.qwhip_quantize_blocks(st, src.ptr, qwhip.F32, 4, 96, 4, 64, 1, 2, out.ptr) == qwhip.E_BAD_SHAPE       # 96 % 64
+    assert lib.qwhip_quantize_blocks(st, src.ptr, qwhip.F16, 4, 96, 4, 32, 1, 2, out.ptr) == qwhip.E_BAD_SHAPE       # f16 source
+    assert lib.qwhip_quantize_blocks(st, src.ptr, qwhip.F32, 4, 96, 4, 32, 1, 3, out.ptr) == qwhip.E_BAD_SHAPE       # mse_clip
+    assert lib.qwhip_quantize_blocks(st, src.ptr, qwhip.F32, 4, 96, 4, 32, 1, 2, out.ptr) == qwhip.OK
+    dev.stream.sync()
+
+
+def test_planar_hq8_device_writer_and_reader(dev, golden_dir):
+    """qwhip_quantize_hq8_planar writes the reference's planes for the golden input (hq_blocks_golden.npz); the reference's
+    planar pack goes reader -> device planes -> qwhip_dequant_hq8_planar and lands within 1e-6 of selfpack_hq8.qwp.dq8rot.f32.bin
+    (the bar of Tests/QWQuantTests/QWHQ8PackTests.swift:30-44), bit-identical to the oracle's dequant."""
+    from qwegn_amd import pack as qpack
+    gold = np.load(golden_dir / "hq_blocks_golden.npz")
+    w = gold["w"]
+    n, k = w.shape
+    src, qs, sc = dev.put(w), dev.alloc(n * k), dev.alloc(n * (k // 32) * 2)
+    qwhip.check(dev.lib.qwhip_quantize_hq8_planar(dev.stream.handle, src.ptr, qwhip.F32, n, k, 1, qs.ptr, sc.ptr))
+    assert np.array_equal(qs.download(np.int8, (n, k)), gold["hq8_planar__qs"])
+    assert np.array_equal(sc.download(np.uint16, (n, k // 32)), gold["hq8_planar__scales"])
+    pk = qpack.Pack(golden_dir / "selfpack_hq8.qwp")
+    name = next(nm for nm, e in pk.tensors.items() if e.hq8_quantized)
+    dq, ds, pn, pkk = pk.upload_hq8(dev, name)
+    out = dev.alloc(pn * pkk * 4)
+    qwhip.check(dev.lib.qwhip_dequant_hq8_planar(dev.stream.handle, dq.ptr, ds.ptr, pn, pkk, out.ptr))
+    got = out.download(np.float32, (pn, pkk))
+    want = np.frombuffer((golden_dir / "selfpack_hq8.qwp.dq8rot.f32.bin").read_bytes(), dtype=np.float32).reshape(pn, pkk)
+    assert np.max(np.abs(got - want)) <= 1e-6
+    host_q, host_s = pk.hq8_planes(name)
+    assert np.array_equal(got.view(np.uint32), qo.dequant_hq8_planar_rot(np.asarray(host_q), np.asarray(host_s)).view(np.uint32))

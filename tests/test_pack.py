@@ -42,6 +42,12 @@ def test_reads_the_reference_packs(golden_dir):
     p8 = qp.Pack(golden_dir / "selfpack_hq8.qwp")
     e8 = p8.entry("w_test8")
     assert e8.hq8_quantized and not e8.quantized and qp.PlaneLayout.resolve(e8) is None
+    # the planar reader hands out the two planes; their host dequant is the reference's stored answer (<= 1e-6)
+    name8 = next(nm for nm, e in p8.tensors.items() if e.hq8_quantized)
+    qs, sc = p8.hq8_planes(name8)
+    assert qs.dtype == np.int8 and sc.dtype == np.float16 and qs.shape == tuple(e8.shape) and sc.shape == (e8.shape[0], e8.shape[1] // 32)
+    want = np.frombuffer((golden_dir / "selfpack_hq8.qwp.dq8rot.f32.bin").read_bytes(), dtype=np.float32).reshape(qs.shape)
+    assert np.max(np.abs(qo.dequant_hq8_planar_rot(np.asarray(qs), np.asarray(sc)) - want)) <= 1e-6
     with pytest.raises(qp.QWQuantError) as err:
         p8.plane("w_test8")
     assert err.value.case == "badPlane"
