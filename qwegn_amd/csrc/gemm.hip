@@ -20,6 +20,8 @@
 // expert-major slot range [expert_off[e], expert_off[e+1]); slot rows are gathered through `gather`.
 #include <mutex>
 
+#include <atomic>
+
 #include "qwhip_common.h"
 #include "qw_mfma_2x5.h"
 
@@ -1365,11 +1367,11 @@ hipError_t launch_cfg(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)(BM + BN) * 72 * 2;
     auto kern = qw_gemm_kernel<WM, WN, WVM, WVN, FMT, XDT, YDT, GROUPED>;
-    static bool attr_done = false;  // per instantiation
-    if (!attr_done) {
+    static std::atomic<bool> attr_done{false};  // per instantiation
+    if (!attr_done.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        attr_done = true;
+        attr_done.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, grid, dim3(WVM * WVN * 64), lds, st, p);
     return hipGetLastError();
@@ -1380,11 +1382,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
     auto kern = qw_gemm2_kernel<WM, WN, WVM, WVN, FMT, YDT, GROUPED>;
-    static bool attr_done = false;  // per instantiation
-    if (!attr_done) {
+    static std::atomic<bool> attr_done{false};  // per instantiation
+    if (!attr_done.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        attr_done = true;
+        attr_done.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, grid, dim3(WVM * WVN * 64), lds, st, p);
     return hipGetLastError();
@@ -1395,11 +1397,11 @@ hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
     auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, SWIGLU, XDT>;
-    static bool attr_done = false;  // per instantiation
-    if (!attr_done) {
+    static std::atomic<bool> attr_done{false};  // per instantiation
+    if (!attr_done.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        attr_done = true;
+        attr_done.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, grid, dim3(WVM * WVN * 64), lds, st, p);
     return hipGetLastError();

@@ -13,6 +13,8 @@
 //    four 8-wide f16 MFMA A operands, and v_mfma_f32_16x16x32_f16 contracts them against the m
 //    activation rows held as B operands (column j = m).  The 4 waves of a workgroup split K and reduce
 //    through LDS.  VALU does only the dequant; accumulation rides on the matrix cores.
+#include <atomic>
+
 #include "qwhip_common.h"
 
 enum { QW_XM_GLOBAL = 0, QW_XM_LDS_ROT = 1 };
@@ -904,11 +906,11 @@ bool launch_colt_1(hipStream_t st, gemv_args a, hipError_t* err) {
     }
     if (lds > 150u * 1024u) return false;
     auto kern = qw_gemv_colt_kernel<FMT, XDT>;
-    static size_t attr_lds = 0;   // per instantiation
-    if (lds > attr_lds) {
+    static std::atomic<size_t> attr_lds{0};   // per instantiation
+    if (lds > attr_lds.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
         if (e != hipSuccess) { *err = e; return true; }
-        attr_lds = 150u * 1024u;
+        attr_lds.store(150u * 1024u, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, dim3(wgs), dim3(64u * waves), lds, st, a);
     *err = hipGetLastError();

@@ -22,6 +22,8 @@
 // (16 slices) in K range kr; long rows take several K ranges, the activations of one range in registers at a time
 // (the next range's fetched meanwhile, the weight prefetch running on across the boundary), partial sums
 // accumulating in LDS per (quad slot, wave, 16-lane row) and summed in a fixed order at the end.
+#include <atomic>
+
 #include "qwhip_common.h"
 
 namespace {
@@ -276,10 +278,10 @@ template <int FMT, int XDT, int MG>
 void qq_launch1(hipStream_t st, const qq_params& p, uint32_t wgs, uint32_t threads, size_t lds) {
     constexpr int D = FMT == QW_FMT_B8 ? 2 : 3;
     auto kern = qw_gemv_quad_kernel<FMT, XDT, MG, D, 768>;
-    static bool attr_done = false;   // per instantiation
-    if (!attr_done) {
+    static std::atomic<bool> attr_done{false};   // per instantiation
+    if (!attr_done.load(std::memory_order_acquire)) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        attr_done = true;
+        attr_done.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, dim3(wgs), dim3(threads), lds, st, p);
 }

@@ -1,5 +1,7 @@
 // MoE plumbing around the grouped GEMM: router logits, softmax top-k routing, the expert-major pair sort
 // with its tile list, and the weighted combine.
+#include <atomic>
+
 #include "qwhip_common.h"
 #include "qwhip_route.h"
 
@@ -384,10 +386,10 @@ extern "C" qwhip_status qwhip_moe_group_pairs(qwhip_stream_t s, const int32_t* i
     // up to 24,576 pairs the sorted list is staged in LDS (96 KB beside the 38 KB of counters)
     const uint32_t stage = pairs <= 24576u ? 1u : 0u;
     const size_t lds = stage ? (size_t)pairs * 4u : 0u;
-    static bool attr_done = false;
-    if (!attr_done) {
+    static std::atomic<bool> attr_done{false};
+    if (!attr_done.load(std::memory_order_acquire)) {
         QWHIP_TRY_HIP(hipFuncSetAttribute((const void*)qw_moe_group_pairs_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        attr_done = true;
+        attr_done.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(qw_moe_group_pairs_kernel, dim3(1), dim3(1024), lds, s->stream, ids, experts, pairs, top_k, expert_off,
                        sorted_pair, sorted_tok, inv_perm, tile_e, tile_r, tile_count, compact_tail ? 1u : 0u, stage);

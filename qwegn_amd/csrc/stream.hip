@@ -13,6 +13,8 @@
 //     each step's [m, 512] panel is DMA-staged once per workgroup and shared by its 4 row tiles (m up to 16 without
 //     multiplying L2 traffic);
 //   * the 4 waves of a workgroup are RW row tiles x KW K-splits (RW*KW = 4); K-splits reduce through LDS.
+#include <atomic>
+
 #include "qwhip_common.h"
 
 namespace {
@@ -299,11 +301,11 @@ hipError_t qs_launch_fmt(hipStream_t st, const qs_params& p, int kw, int xmode, 
 #define QS_GO(KWV, XM, DT, PFV)                                                                                    \
     do {                                                                                                            \
         auto kern = qw_stream_kernel<BITS, GROUP, M5, KWV, XM, DT, PFV>;                                            \
-        static bool attr_done = false;                                                                              \
-        if (!attr_done) {                                                                                           \
+        static std::atomic<bool> attr_done{false};                                                                              \
+        if (!attr_done.load(std::memory_order_acquire)) {                                                                                           \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024); \
             if (e != hipSuccess) return e;                                                                          \
-            attr_done = true;                                                                                       \
+            attr_done.store(true, std::memory_order_release);                                                                                       \
         }                                                                                                           \
         hipLaunchKernelGGL(kern, grid, block, lds, st, p);                                                          \
         return hipGetLastError();                                                                                   \

@@ -35,24 +35,49 @@ static float h2f(uint16_t b) { _Float16 h; std::memcpy(&h, &b, 2); return (float
 // ---------------------------------------------------------------------------------------------------------------
 static void test_plan_table() {
     using B = QWGemmPlan::Backend;
-    // decode GEMV families and outputs (QWGemm.swift:92-133)
+    // the reference's table row by row (QWGemm.swift:92-133): backend, kernel name, threads per threadgroup
     auto p = QWGemm::plan({1, 17408, 5120}, QWDType::q4g, QWEpilogue::none, QWDType::f16);
-    CHECK(p.backend == B::handQ4gV4H16 && p.kernel == "qwg_gemv_q4g_v4_h16" && p.family == QWGemmFamily::f1DecodeGemv);
+    CHECK(p.backend == B::handQ4gV4H16 && p.kernel == "qwg_gemv_q4g_v4_h16" && p.threadsPerTG == 32 && p.family == QWGemmFamily::f1DecodeGemv);
     p = QWGemm::plan({1, 17408, 5120}, QWDType::q4g, QWEpilogue::none);
-    CHECK(p.backend == B::handQ4gV4 && p.kernel == "qwg_gemv_q4g_v4");
+    CHECK(p.backend == B::handQ4gV4 && p.kernel == "qwg_gemv_q4g_v4" && p.threadsPerTG == 32);
     p = QWGemm::plan({1, 248320, 5120}, QWDType::q4g, QWEpilogue::none, QWDType::f32, 248320);
     CHECK(p.family == QWGemmFamily::f2LmHeadGemv && p.backend == B::handQ4gV4);
     p = QWGemm::plan({1, 34816, 5120}, QWDType::q4g, QWEpilogue::siluMulPair, QWDType::f16);
-    CHECK(p.backend == B::handQ4gSiluPairH16 && p.kernel == "qwg_gemv_q4g_silu_pair_h16");
+    CHECK(p.backend == B::handQ4gSiluPairH16 && p.kernel == "qwg_gemv_q4g_silu_pair_h16" && p.threadsPerTG == 64);
+    p = QWGemm::plan({4096, 34816, 5120}, QWDType::q4g, QWEpilogue::siluMulPair);   // the epilogue rows come first, whatever the family
+    CHECK(p.backend == B::handQ4gSiluPair && p.kernel == "qwg_gemv_q4g_silu_pair" && p.family == QWGemmFamily::f3PrefillGemm);
+    p = QWGemm::plan({2, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::handQ4gSkinny && p.kernel == "qwg_skinny_m2" && p.threadsPerTG == 32);
     p = QWGemm::plan({3, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
     CHECK(p.backend == B::handQ4gSkinny && p.kernel == "qwg_skinny_m3" && p.family == QWGemmFamily::f5SkinnyGemm);
+    p = QWGemm::plan({3, 5120, 65536}, QWDType::q4g, QWEpilogue::none);             // 3 * 65536 * 2 bytes > 256 KiB of constants
+    CHECK(p.backend == B::blocked && p.family == QWGemmFamily::f5SkinnyGemm);
+    p = QWGemm::plan({4, 5120, 5120}, QWDType::q4g, QWEpilogue::none);              // the skinny window is M in {2, 3}
+    CHECK(p.backend == B::blocked && p.kernel.empty() && p.threadsPerTG == 0);
+    p = QWGemm::plan({1, 4096, 4096}, QWDType::f16, QWEpilogue::none);
+    CHECK(p.backend == B::handF16V4 && p.kernel == "qwg_gemv_f16_v4" && p.threadsPerTG == 32);
     p = QWGemm::plan({4096, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
-    CHECK(p.backend == B::mfmaGemmF16 && p.family == QWGemmFamily::f3PrefillGemm);
-    p = QWGemm::plan({4096, 5120, 5100}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::mpsGraphBmmF16 && p.kernel == "mpsgraph_bmm_f16" && p.threadsPerTG == 0 && p.family == QWGemmFamily::f3PrefillGemm);
+    p = QWGemm::plan({4096, 5120, 5100}, QWDType::q4g, QWEpilogue::none);           // K % 32 != 0
     CHECK(p.backend == B::blocked);
+    p = QWGemm::plan({100, 5120, 5120}, QWDType::q4g, QWEpilogue::none);            // F4: nothing raced
+    CHECK(p.backend == B::blocked && p.family == QWGemmFamily::f4AttentionTiles);
     p = QWGemm::plan({1, 64, 64}, QWDType::f32, QWEpilogue::none);
     CHECK(p.backend == B::blocked);
+    p = QWGemm::plan({4096, 64, 64}, QWDType::f16, QWEpilogue::none);
+    CHECK(p.backend == B::blocked);
     CHECK((QWGemmShape{100, 8, 8}.family() == QWGemmFamily::f4AttentionTiles));
+    // this library's routing over the same shapes
+    p = QWGemm::planHip({4, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::handQ4gSkinny);
+    p = QWGemm::planHip({16, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::handQ4gSkinny && p.family == QWGemmFamily::f4AttentionTiles);
+    p = QWGemm::planHip({4096, 5120, 5120}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::mfmaGemmF16 && p.kernel == "qwg_gemm_q4g_h16");
+    p = QWGemm::planHip({4096, 5120, 5100}, QWDType::q4g, QWEpilogue::none);
+    CHECK(p.backend == B::blocked);
+    p = QWGemm::planHip({1, 64, 64}, QWDType::f16, QWEpilogue::none);
+    CHECK(p.backend == B::blocked);
 }
 
 static void test_weight_view() {

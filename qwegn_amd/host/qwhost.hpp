@@ -215,9 +215,10 @@ struct QWGemmShape {
 };
 
 struct QWGemmPlan {
-    // The reference's backends, with the prefill winner re-pointed at the MFMA kernel this library ships and the
-    // skinny window widened: the streaming GEMV takes M = 2..16 in one pass (the reference's F5 window is M in {2,3}).
-    enum class Backend { handQ4gV4, handQ4gV4H16, handQ4gSiluPair, handQ4gSiluPairH16, handQ4gSkinny, mfmaGemmF16, blocked };
+    // The reference's backends (QWGemm.swift:36-61).  `mfmaGemmF16` is the one addition: the prefill door of this library
+    // (planHip only; the reference's own F3 winner is the MPSGraph door `mpsGraphBmmF16`, which has no kernel to encode).
+    enum class Backend { handQ4gV4, handQ4gV4H16, handQ4gSiluPair, handQ4gSiluPairH16, handQ4gSkinny, handF16V4, mpsF16,
+                         mpsGraphBmmF16, blocked, mfmaGemmF16 };
     Backend backend;
     std::string kernel;  // the reference's kernel name: the key hal.pipeline() resolves
     int threadsPerTG;
@@ -226,9 +227,42 @@ struct QWGemmPlan {
 };
 
 struct QWGemm {
-    // Pure table lookup (QWGemm.swift:92-133).
+    static constexpr int maxConstantBytes = 256 * 1024;   // QWGemm.swift:90
+
+    // Pure table lookup, row for row the reference's (QWGemm.swift:92-133): same backend, kernel name and threads per
+    // threadgroup for every (family, dtype, epilogue, output dtype), `.blocked` wherever the reference blocks.
     static QWGemmPlan plan(const QWGemmShape& shape, QWDType dtype, QWEpilogue epi, QWDType outDtype = QWDType::f32,
                            std::optional<int> vocab = std::nullopt) {
+        using B = QWGemmPlan::Backend;
+        using F = QWGemmFamily;
+        const F fam = shape.family(vocab);
+        const QWGemmPlan blocked{B::blocked, "", 0, fam, epi};
+        const bool decode = fam == F::f1DecodeGemv || fam == F::f2LmHeadGemv;
+        if (dtype == QWDType::q4g && epi == QWEpilogue::siluMulPair)
+            return outDtype == QWDType::f16 ? QWGemmPlan{B::handQ4gSiluPairH16, "qwg_gemv_q4g_silu_pair_h16", 64, fam, epi}
+                                            : QWGemmPlan{B::handQ4gSiluPair, "qwg_gemv_q4g_silu_pair", 64, fam, epi};
+        if (epi != QWEpilogue::none) return blocked;
+        if (dtype == QWDType::q4g && decode)
+            return outDtype == QWDType::f16 ? QWGemmPlan{B::handQ4gV4H16, "qwg_gemv_q4g_v4_h16", 32, fam, epi}
+                                            : QWGemmPlan{B::handQ4gV4, "qwg_gemv_q4g_v4", 32, fam, epi};
+        if (dtype == QWDType::q4g && fam == F::f5SkinnyGemm) {
+            if ((shape.m == 2 || shape.m == 3) && shape.m * shape.k * 2 <= maxConstantBytes)
+                return {B::handQ4gSkinny, shape.m == 2 ? "qwg_skinny_m2" : "qwg_skinny_m3", 32, fam, epi};
+            return blocked;
+        }
+        if (dtype == QWDType::f16 && decode) return {B::handF16V4, "qwg_gemv_f16_v4", 32, fam, epi};
+        if (dtype == QWDType::q4g && fam == F::f3PrefillGemm)
+            return shape.k % 32 == 0 ? QWGemmPlan{B::mpsGraphBmmF16, "mpsgraph_bmm_f16", 0, fam, epi} : blocked;
+        return blocked;
+    }
+
+    // This library's routing over the same shapes: where `plan` blocks or names a door that does not exist here, the kernels
+    // of libqwhip take the call.  Differences from `plan`: the streaming GEMV takes every row count 2..16 in one pass (the
+    // reference's skinny window is M in {2, 3}, its other F5 / F4 shapes are blocked), prefill and the remaining F4 shapes go
+    // to the matrix-core GEMM when K % 64 == 0, the f16-weight GEMV and the MPSGraph door have no counterpart, and
+    // threadsPerTG is the 256-thread workgroup of the HIP kernels.  encode / encodeH16 accept either plan.
+    static QWGemmPlan planHip(const QWGemmShape& shape, QWDType dtype, QWEpilogue epi, QWDType outDtype = QWDType::f32,
+                              std::optional<int> vocab = std::nullopt) {
         using B = QWGemmPlan::Backend;
         const QWGemmFamily fam = shape.family(vocab);
         if (dtype != QWDType::q4g) return {B::blocked, "", 0, fam, epi};
@@ -264,7 +298,10 @@ struct QWGemm {
             if (plan.family == QWGemmFamily::f5SkinnyGemm) throw QWGemmError(QWGemmError::badWeights, "F5 window: run F1 per row");
             throw QWGemmError(QWGemmError::f3Blocked, "no winner raced for this family");
         }
-        if (plan.backend == B::mfmaGemmF16) throw QWGemmError(QWGemmError::f3Blocked, "plan resolved to the tensor GEMM - use gemmBatchedH16");
+        if (plan.backend == B::mfmaGemmF16 || plan.backend == B::mpsGraphBmmF16)
+            throw QWGemmError(QWGemmError::f3Blocked, "plan resolved to the tensor GEMM - use gemmBatchedH16");
+        if (plan.backend == B::handF16V4 || plan.backend == B::mpsF16)
+            throw QWGemmError(QWGemmError::badWeights, "the f16-weight doors have no kernel in this library");
         if (plan.epilogue == QWEpilogue::siluMulPair && wQ4.n % 2 != 0) throw QWGemmError(QWGemmError::badWeights, "silu_pair needs even N");
         if (x.shape.dtype != QWDType::f16 && x.shape.dtype != QWDType::bf16) throw QWGemmError(QWGemmError::badWeights, "activations must be f16");
         if (x.shape.elementCount < (size_t)rows * (size_t)wQ4.k) throw QWGemmError(QWGemmError::badWeights, "activations are short");

@@ -240,3 +240,129 @@ class Pack:
         if view_args is None:
             return buf, None
         return buf, dev.view(buf, *view_args, nbytes=int(plane.nbytes))
+
+
+class PackWriter:
+    """Writes a QWP1 pack in the layout the reference's packer gives it (pack_file, Scripts/quantize/pack.py:115-316): magic,
+    the trailer's byte count at offset 4, planes, JSON trailer {"provenance", "tensors"} at the end of the file.  Raw and planar
+    planes start and end on 256-byte boundaries, block planes on 16 KiB boundaries; entries keep the order they were added in
+    and carry exactly the keys the reader's schema knows (shape, kind, raw_off | hq4_off | hq8_off + hq8_s_off, experts, e_hq4, hq).
+    Planes are bytes the caller already holds: quantized with the device writers (`add_weights`) or copied from elsewhere."""
+
+    RAW_ALIGN, BLOCK_ALIGN = 256, 16384
+
+    def __init__(self, path, provenance: dict):
+        self.path = pathlib.Path(path)
+        self.provenance = dict(provenance)
+        self.index: dict[str, dict] = {}
+        self._f = open(self.path, "wb")
+        self._f.write(MAGIC + b"\0" * 8)
+        self._pad(self.RAW_ALIGN)
+
+    def _pad(self, alignment: int) -> int:
+        off = self._f.tell()
+        fill = (-off) % alignment
+        self._f.write(b"\0" * fill)
+        return off + fill
+
+    def _claim(self, name: str) -> None:
+        if self._f is None:
+            raise QWQuantError("badPlane", "the pack is closed")
+        if name in self.index:
+            raise QWQuantError("badPlane", f"duplicate tensor: {name}")
+
+    def add_raw(self, name: str, values: np.ndarray, kind: str = "bf16") -> dict:
+        """A verbatim plane: bf16 bits (u16) or f32 values."""
+        self._claim(name)
+        arr = np.ascontiguousarray(values)
+        if kind == "bf16" and arr.dtype != np.uint16:
+            raise QWQuantError("badPlane", f"{name}: bf16 planes are handed over as their 16-bit patterns")
+        if kind == "f32":
+            arr = arr.astype("<f4", copy=False)
+        elif kind != "bf16":
+            raise QWQuantError("badPlane", f"{name}: raw kind {kind}")
+        entry = {"shape": list(arr.shape), "kind": kind, "raw_off": self._pad(self.RAW_ALIGN)}
+        self._f.write(arr.tobytes())
+        self._pad(self.RAW_ALIGN)
+        self.index[name] = entry
+        return entry
+
+    def add_blocks(self, name: str, shape, blocks: np.ndarray, bits: int = 4, group: int = GROUP, is_m5: bool = True) -> dict:
+        """A block plane for a [N, K] tensor or an expert stack [E, N, K] (stored as one bank of E * N rows, e_hq4 bytes per
+        expert; N even as the packer demands).  `blocks`: the bank's bytes in row order."""
+        self._claim(name)
+        shape = [int(d) for d in shape]
+        if len(shape) not in (2, 3) or shape[-1] % group != 0 or (len(shape) == 3 and shape[1] % 2 != 0):
+            raise QWQuantError("badPlane", f"{name}: shape {shape} does not fit group {group}")
+        m5 = is_m5 and bits == 4 and group == GROUP
+        bb = BLOCK_BYTES if m5 else aq_block_bytes(bits, group)
+        if not m5 and not aq_block_supported(bits, group):
+            raise QWQuantError("badPlane", f"{name}: no container for {bits} bits, group {group}")
+        rows = shape[0] if len(shape) == 2 else shape[0] * shape[1]
+        data = np.ascontiguousarray(blocks).view(np.uint8).ravel()
+        if data.nbytes != rows * (shape[-1] // group) * bb:
+            raise QWQuantError("badPlane", f"{name}: {data.nbytes} bytes for {rows} rows of {(shape[-1] // group) * bb}")
+        entry = {"shape": shape}
+        if len(shape) == 3:
+            entry["experts"] = shape[0]
+            entry["e_hq4"] = shape[1] * (shape[2] // group) * bb
+        entry["hq4_off"] = self._pad(self.BLOCK_ALIGN)
+        if not m5:
+            entry["hq"] = {"bits": int(bits), "group": int(group)}
+        self._f.write(data.tobytes())
+        self._pad(self.BLOCK_ALIGN)
+        self.index[name] = entry
+        return entry
+
+    def add_hq8_planar(self, name: str, qs: np.ndarray, scales: np.ndarray) -> dict:
+        """Planar HQ8_G32_M5: int8 codes [N, K], then f16 scales [N, K / 32], each plane on its own 256-byte boundary."""
+        self._claim(name)
+        qs = np.ascontiguousarray(qs, dtype=np.int8)
+        scales = np.ascontiguousarray(scales, dtype=np.float16)
+        if qs.ndim != 2 or qs.shape[1] % GROUP != 0 or scales.shape != (qs.shape[0], qs.shape[1] // GROUP):
+            raise QWQuantError("badPlane", f"{name}: planar HQ8 wants 2-D codes and one scale per 32 columns")
+        entry = {"shape": list(qs.shape), "hq8_off": self._pad(self.RAW_ALIGN)}
+        self._f.write(qs.tobytes())
+        entry["hq8_s_off"] = self._pad(self.RAW_ALIGN)
+        self._f.write(scales.tobytes())
+        self._pad(self.RAW_ALIGN)
+        self.index[name] = entry
+        return entry
+
+    def add_weights(self, dev: "qwhip.Device", name: str, w: np.ndarray, bits: int = 4, group: int = GROUP, is_m5: bool = True,
+                    rotate: bool = True) -> dict:
+        """Quantizes fp32 weights [N, K] or [E, N, K] on the device (qwhip_quantize_hq4_g32 / qwhip_quantize_blocks, the group
+        resolved as the packer does: gcd(K, requested)) and adds the bank."""
+        import math
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        k = w.shape[-1]
+        rows = int(np.prod(w.shape[:-1], dtype=np.int64))
+        eff = math.gcd(k, group)
+        m5 = is_m5 and bits == 4 and eff == GROUP
+        bb = BLOCK_BYTES if m5 else aq_block_bytes(bits, eff)
+        src, out = dev.put(w), dev.alloc(max(rows * (k // eff) * bb, 256))
+        if m5:
+            qwhip.check(dev.lib.qwhip_quantize_hq4_g32(dev.stream.handle, src.ptr, qwhip.F32, rows, k, int(rotate), out.ptr))
+        else:
+            qwhip.check(dev.lib.qwhip_quantize_blocks(dev.stream.handle, src.ptr, qwhip.F32, rows, k, bits, eff, int(rotate), 2, out.ptr))
+        blocks = out.download(np.uint8, (rows * (k // eff) * bb,))
+        src.free()
+        out.free()
+        return self.add_blocks(name, w.shape, blocks, bits, eff, is_m5)
+
+    def close(self) -> pathlib.Path:
+        trailer = json.dumps({"provenance": self.provenance, "tensors": self.index}).encode()
+        self._f.write(trailer)
+        self._f.seek(4)
+        self._f.write(len(trailer).to_bytes(8, "little"))
+        self._f.close()
+        self._f = None
+        return self.path
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if self._f is not None:
+            self.close()
+        return False

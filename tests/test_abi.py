@@ -128,3 +128,20 @@ def test_device_create_fails_loudly_without_a_gpu():
     assert not h.value
     with pytest.raises(qwhip.QwhipError):
         qwhip.Device(0)
+
+
+def test_swift_shim_resolves_only_kernel_names_the_library_knows():
+    """Every name the Swift shim hands to hal.pipeline() is a key of qwhip_kernel_lookup, so a door of the shim cannot throw
+    kernelMissing for a kernel the library serves; the two plan rows whose doors do not exist here (the f16-weight GEMV and the
+    MPSGraph prefill door of QWGemm.plan) are the only names without a launcher."""
+    import re
+    lib = qwhip.load()
+    text = (ROOT / "qwegn_amd" / "swift" / "QWHipHAL" / "QWHipHAL.swift").read_text()
+    literal = set(re.findall(r'hal\.pipeline\([^"\n]*"([a-z0-9_]+)"', text)) | set(re.findall(r'kernel: "([a-z0-9_]+)"', text))
+    literal |= {m for m in re.findall(r'\? "([a-z0-9_]+)" :', text) if m.startswith("qwg_")}
+    assert len(literal) >= 20
+    missing = {n for n in literal if lib.qwhip_kernel_lookup(n.encode(), None) != qwhip.OK}
+    assert missing == {"mpsgraph_bmm_f16", "qwg_gemv_f16_v4"}
+    for templ in re.findall(r'"(qwg_[a-z0-9_]*\\\(bank\.bits\)_g\\\(bank\.groupSize\)[a-z0-9_]*)"', text):
+        name = templ.replace("\\(bank.bits)", "8").replace("\\(bank.groupSize)", "64")
+        assert lib.qwhip_kernel_lookup(name.encode(), None) == qwhip.OK, name

@@ -515,3 +515,21 @@ def test_planar_hq8_device_writer_and_reader(dev, golden_dir):
     assert np.max(np.abs(got - want)) <= 1e-6
     host_q, host_s = pk.hq8_planes(name)
     assert np.array_equal(got.view(np.uint32), qo.dequant_hq8_planar_rot(np.asarray(host_q), np.asarray(host_s)).view(np.uint32))
+
+
+def test_pack_writer_quantizes_on_the_device_and_round_trips(dev, tmp_path):
+    """PackWriter.add_weights: fp32 weights -> device quantizer -> pack file -> reader -> device bank: the bank's bytes are the
+    oracle's for an HQ4_G32_M5 expert stack and an HQ8_G64 projection (group resolved by gcd as the packer does: 64 stays 64)."""
+    from qwegn_amd import pack as qpack
+    experts, rows, k = 2, 16, 512
+    w3 = H.make_weights(experts * rows, k, seed=41).reshape(experts, rows, k)
+    w2 = H.make_weights(24, k, seed=42)
+    with qpack.PackWriter(tmp_path / "dev.qwp", {"source": "device-writer"}) as wr:
+        wr.add_weights(dev, "mlp.experts.down", w3)
+        wr.add_weights(dev, "o_proj", w2, bits=8, group=64, is_m5=False)
+    pk = qpack.Pack(tmp_path / "dev.qwp")
+    assert np.array_equal(np.asarray(pk.plane("mlp.experts.down")[1]), qo.quant_hq4_blocks(w3.reshape(-1, k)).ravel().view(np.uint8))
+    want, _ = qo.quant_hq_blocks(w2, bits=8, group=64, is_m5=False, rotate=True)
+    buf, view = pk.upload(dev, "o_proj")
+    assert (view.n, view.k, view.bits, view.group) == (24, k, 8, 64)
+    assert np.array_equal(buf.download(np.uint8, (want.nbytes,)), want.ravel().view(np.uint8))

@@ -99,3 +99,44 @@ def test_reader_error_cases(tmp_path):
     with pytest.raises(qp.QWQuantError) as err:
         p.entry("nope")
     assert err.value.case == "unknownTensor"
+
+
+def test_writer_reproduces_the_reference_packs_byte_for_byte(golden_dir, tmp_path):
+    """PackWriter given the reference packs' own planes and provenance writes the same files: header, plane offsets and padding,
+    the trailer's text (Scripts/quantize/pack.py:115-316 wrote tests/golden/selfpack.qwp and selfpack_hq8.qwp)."""
+    src = qp.Pack(golden_dir / "selfpack.qwp")
+    with qp.PackWriter(tmp_path / "again.qwp", src.provenance) as wr:
+        wr.add_raw("norm_test", np.asarray(src.plane("norm_test")[1]).view(np.uint16))
+        wr.add_blocks("w_test", src.entry("w_test").shape, np.asarray(src.plane("w_test")[1]))
+    assert (tmp_path / "again.qwp").read_bytes() == (golden_dir / "selfpack.qwp").read_bytes()
+    src8 = qp.Pack(golden_dir / "selfpack_hq8.qwp")
+    qs, sc = src8.hq8_planes("w_test8")
+    with qp.PackWriter(tmp_path / "again8.qwp", src8.provenance) as wr:
+        wr.add_hq8_planar("w_test8", np.asarray(qs), np.asarray(sc))
+    assert (tmp_path / "again8.qwp").read_bytes() == (golden_dir / "selfpack_hq8.qwp").read_bytes()
+
+
+def test_writer_round_trips_block_families_and_expert_stacks(tmp_path):
+    rng = np.random.default_rng(3)
+    experts, n, k = 2, 6, 256
+    w = (rng.standard_normal((experts * n, k)) * 0.02).astype(np.float32)
+    stack = qo.quant_hq4_blocks(w)
+    blk, _ = qo.quant_hq_blocks(w[:n], bits=6, group=128, is_m5=False, rotate=True)
+    with qp.PackWriter(tmp_path / "w.qwp", {"source": "writer-test"}) as wr:
+        e1 = wr.add_blocks("m.experts.gate_up", (experts, n, k), stack)
+        e2 = wr.add_blocks("proj", (n, k), blk, bits=6, group=128, is_m5=False)
+        e3 = wr.add_raw("gamma", np.arange(k, dtype=np.float32), kind="f32")
+        with pytest.raises(qp.QWQuantError):
+            wr.add_raw("gamma", np.zeros(4, np.float32), kind="f32")          # duplicate name
+        with pytest.raises(qp.QWQuantError):
+            wr.add_blocks("odd", (experts, 5, k), stack[: experts * 5])        # odd rows per expert
+        with pytest.raises(qp.QWQuantError):
+            wr.add_blocks("short", (n, k), blk[:-1], bits=6, group=128, is_m5=False)
+    assert e1["hq4_off"] % 16384 == 0 and e2["hq4_off"] % 16384 == 0 and e3["raw_off"] % 256 == 0
+    assert e1["experts"] == experts and e1["e_hq4"] == n * (k // 32) * 20 and "hq" not in e1 and e2["hq"] == {"bits": 6, "group": 128}
+    p = qp.Pack(tmp_path / "w.qwp")
+    assert np.array_equal(np.asarray(p.plane("m.experts.gate_up")[1]), stack.ravel().view(np.uint8))
+    assert p.weight_geometry("m.experts.gate_up") == (experts * n, k, qp.qwhip.KIND_HQ4_G32_M5, 4, 32)
+    assert p.weight_geometry("proj") == (n, k, qp.qwhip.KIND_ROTATED_HQ, 6, 128)
+    assert np.array_equal(np.asarray(p.plane("proj")[1]), blk.ravel().view(np.uint8))
+    assert np.array_equal(np.asarray(p.plane("gamma")[1]).view(np.float32), np.arange(k, dtype=np.float32))
