@@ -163,8 +163,10 @@ qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_view* w, voi
  * Sources/QWMetal/include/qw_dequant_multi.metalh:205-208); the others contract the f16 weights of qwhip_dequant_f16.
  * flags: QWHIP_X_PREROTATED; bits 8..11 pick one kernel for tuning and tests (0 = automatic, 1 = half-wave dot2,
  * 2 = MFMA streamer, 3 = DMA streamer, 4 = column-stationary HQ4 kernel, 5 = column-stationary MFMA kernel,
- * 6 = column-stationary dot2 kernel, 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel; a kernel that does not
- * take the shape returns QWHIP_E_BAD_GEOMETRY); bits 12..15 its tuning code. */
+ * 6 = column-stationary dot2 kernel, 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel, 9 = split-K MFMA kernel; a
+ * kernel that does not take the shape returns QWHIP_E_BAD_GEOMETRY); bits 12..15 its tuning code (bits 12..18 for the
+ * split-K kernel).  The split-K kernel (automatic for 4-bit banks with k >= 8192 and m >= 6) keeps its partial sums in
+ * the stream's scratch: calls on one stream are ordered; calls on different streams do not share it. */
 qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                         uint32_t m, uint32_t flags, void* y16, float* y32);
 

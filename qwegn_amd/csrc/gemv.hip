@@ -978,11 +978,15 @@ bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t 
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
                  float* y32, uint32_t tune, hipError_t* err);
 
+// gemv_sk.hip
+bool qw_sk_gemv(qwhip_stream_t s, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                const void* x, uint32_t x_dtype, uint32_t m, void* y16, float* y32, uint32_t tune, hipError_t* err);
+
 // flags bits 8..11: kernel override for tuning and tests (0 = automatic, 1 = dot2, 2 = direct-load mfma, 3 = DMA streamer,
 // 4 = column-stationary persistent kernel, 5 = column-stationary MFMA kernel, 6 = column-stationary small-M kernel,
-// 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel);
+// 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel, 9 = split-K MFMA kernel);
 // bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer / tuning code of the
-// column-stationary kernel (0 = automatic).
+// column-stationary kernel (0 = automatic); bits 12..18: tuning code of the split-K kernel.
 extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                                    uint32_t m, uint32_t flags, void* y16, float* y32) {
     int fmt = 0;
@@ -1075,6 +1079,19 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
         return QWHIP_OK;
     }
 
+    // split-K matrix-core kernel: activations already in the basis, 2..16 rows.  Its cost is flat in m (two launches, one
+    // dequantization per weight whatever m is), so it takes over where rows are long and few and m is large: N = 5120,
+    // K = 17408, HQ4_G64 measured 18.7 / 18.7 / 20.7 us at m = 6 / 8 / 16 against 21.2 / 23.2 / 34.9 for the kernels below
+    // (16.7 against 18.6 at m = 4); on K = 5120 banks (N = 7168 HQ8, N = 17408 or 5120 HQ4) the kernels below stay ahead.
+    if (variant == 9 || (variant == 0 && !rotate && m >= 6 && w->k >= 8192 && fmt != QW_FMT_B8)) {
+        hipError_t e = hipSuccess;
+        if (!rotate && qw_sk_gemv(s, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, y16, y32, variant == 9 ? (flags >> 12) & 0x7Fu : 0u, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+        if (variant == 9)
+            return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the split-K kernel takes 2..16 rows already in the basis, k %% 128 == 0, partial sums within the stream's scratch");
+    }
     // transposing MFMA kernel: activations already in the basis.  Its cost barely grows with m: measured best from 13 rows
     // on (N = 7168, K = 5120, HQ8: 16.0 / 16.9 us at m = 13 / 16 against 16.6 / 17.9 for the 4x4x4-block kernel and 18.6 for
     // the column-stationary MFMA kernel; N = 5120, K = 17408, HQ4_G64: level with the 4x4x4-block kernel, 31.5 / 34.6 us).

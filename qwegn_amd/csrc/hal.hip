@@ -114,6 +114,16 @@ extern "C" qwhip_status qwhip_stream_create(qwhip_device_t dev, qwhip_stream_t* 
         delete s;
         return qwhip_hip_check(e, "hipStreamCreateWithFlags");
     }
+    // the stream's split-K scratch: counters zeroed once, here
+    e = hipMalloc((void**)&s->scratch, QWHIP_STREAM_SCRATCH_BYTES);
+    if (e == hipSuccess) e = hipMemset(s->scratch, 0, QWHIP_STREAM_COUNTER_BYTES);
+    if (e != hipSuccess) {
+        if (s->scratch) (void)hipFree(s->scratch);
+        (void)hipStreamDestroy(s->stream);
+        delete s;
+        return qwhip_hip_check(e, "stream scratch");
+    }
+    s->scratch_bytes = QWHIP_STREAM_SCRATCH_BYTES;
     *out = s;
     return QWHIP_OK;
 }
@@ -121,6 +131,7 @@ extern "C" qwhip_status qwhip_stream_create(qwhip_device_t dev, qwhip_stream_t* 
 extern "C" qwhip_status qwhip_stream_destroy(qwhip_stream_t s) {
     if (!s) return QWHIP_OK;
     hipError_t e = hipStreamDestroy(s->stream);
+    if (s->scratch) (void)hipFree(s->scratch);
     delete s;
     return qwhip_hip_check(e, "hipStreamDestroy");
 }

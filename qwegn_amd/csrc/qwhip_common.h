@@ -9,9 +9,17 @@ struct qwhip_device_s {
     int ordinal;
     hipDeviceProp_t prop;
 };
+// Partial-sum scratch of the split-K verify GEMV: owned by the stream (allocated when the stream is created, never inside a
+// launcher), so launches on different streams never share it and launches on one stream use it one after the other.
+// The first QWHIP_STREAM_COUNTER_BYTES hold per-row-tile arrival counters, zero between launches (the last arriver resets
+// its counter), the rest holds fp32 partial outputs.
+#define QWHIP_STREAM_COUNTER_BYTES (64u << 10)
+#define QWHIP_STREAM_SCRATCH_BYTES ((8u << 20) + QWHIP_STREAM_COUNTER_BYTES)
 struct qwhip_stream_s {
     qwhip_device_s* dev;
     hipStream_t stream;
+    uint8_t* scratch;
+    size_t scratch_bytes;
 };
 struct qwhip_event_s {
     qwhip_device_s* dev;

@@ -219,6 +219,53 @@ def test_gemv_transposing_mfma_kernel_k_ranges_and_dtypes(dev, fmt, n, k, m, xdt
     assert qo.normalized_error(g16, ref) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "aq4_g32", "hq4_g32", "hq4_g64", "hq4_g128", "hq8_g32", "hq8_g64", "aq8_g256"])
+@pytest.mark.parametrize("m", [2, 5, 8, 9, 16])
+def test_gemv_split_k_mfma_kernel(dev, fmt, m):
+    """Split-K MFMA kernel (override 9): slices land in LDS straight from the bank, exact f16 weights on the matrix cores.
+    n = 270 ends in a partial 16-row tile; k = 1536 is one K range (outputs stored by the kernel itself)."""
+    g16, g32, ref = _run_gemv(dev, fmt, 270, 1536, m, prerot=True, seed=5, variant=9)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt,n,k,m,xdtype,tune", [
+    ("hq4_g64", 96, 17408, 16, "f16", 0),        # six K ranges, partial sums through the stream's scratch
+    ("hq4_g64", 5120, 17408, 8, "f16", 0),       # the verify down projection: every compute unit busy
+    ("aq4_g32", 300, 2176, 6, "bf16", 0x08),     # 32 KiB image: two ranges, the last one short and not whole windows
+    ("aq8_g256", 64, 5120, 16, "bf16", 0),       # 8-bit stream, sixteen activation rows, four ranges
+    ("hq8_g32", 5, 128, 2, "f16", 0),            # a bank smaller than a tile, a row shorter than one window
+    ("hq4_g32_m5", 1000, 5120, 13, "f16", 3),    # three groups in flight
+    ("hq4_g32_m5", 1000, 5120, 3, "f16", 0x24),  # four groups in flight, four waves per workgroup
+    ("hq4_g128", 333, 4096, 7, "f16", 0x46),     # six groups in flight, two waves per workgroup
+    ("hq8_g64", 700, 8192, 12, "f16", 0x18),     # 128 KiB image
+])
+def test_gemv_split_k_mfma_kernel_k_ranges_and_tunings(dev, fmt, n, k, m, xdtype, tune):
+    prerot = H.FORMATS[fmt][4]
+    g16, g32, ref = _run_gemv(dev, fmt, n, k, m, prerot=prerot, xdtype=xdtype, seed=8, variant=9, rt=tune)
+    assert qo.normalized_error(g32, ref) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
+
+
+def test_gemv_split_k_mfma_kernel_refusals_and_stream_order(dev):
+    """Outside its envelope the override is refused before any launch; two calls in a row on one stream share the scratch of
+    partial sums in stream order (the second, smaller call must not see the first one's sums)."""
+    lib, st = dev.lib, dev.stream.handle
+    blocks, _ = H.make_bank("hq4_g32_m5", 32, 160, 0)
+    bank, xb, y = dev.put(blocks), dev.put(np.zeros((2, 160), np.float16)), dev.alloc(2 * 32 * 2)
+    v = dev.view(bank, 32, 160, qwhip.KIND_HQ4_G32_M5)
+    flags = qwhip.X_PREROTATED | (9 << 8)
+    assert lib.qwhip_gemv(st, C.byref(v), xb.ptr, qwhip.F16, 2, flags, y.ptr, None) == qwhip.E_BAD_GEOMETRY      # k % 128
+    v128 = dev.view(bank, 32, 128, qwhip.KIND_HQ4_G32_M5, nbytes=32 * 4 * 20)
+    assert lib.qwhip_gemv(st, C.byref(v128), xb.ptr, qwhip.F16, 1, flags, y.ptr, None) == qwhip.E_BAD_GEOMETRY   # m = 1
+    assert lib.qwhip_gemv(st, C.byref(v128), xb.ptr, qwhip.F16, 2, 9 << 8, y.ptr, None) == qwhip.E_BAD_GEOMETRY  # not in the basis
+    for b in (bank, xb, y):
+        b.free()
+    for n, k, m in ((640, 17408, 16), (96, 8192, 6)):
+        g16, g32, ref = _run_gemv(dev, "hq4_g32_m5", n, k, m, prerot=True, seed=n, variant=0)     # automatic: k >= 8192, m >= 6
+        assert qo.normalized_error(g32, ref) <= 2e-5
+
+
 @pytest.mark.parametrize("fmt", ["aq2_g64", "hq3_g32", "hq6_g32", "aq6_g128"])
 @pytest.mark.parametrize("m", [1, 3, 8, 12])
 def test_gemv_narrow_and_six_bit_streams(dev, fmt, m):
