@@ -137,6 +137,22 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None):
 
     algo_bytes = bank_bytes + m * k * 2 + m * n * 2
     gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    # the yardstick: a launch that only reads the same banks (four 16-byte loads in flight per thread, one atomic per wave),
+    # timed the same way over the same cold ring; its sum is checked against the host's
+    sum_dev = dev.alloc(256 * 8)
+    qwhip.check(lib.qwhip_fill_u32(st, sum_dev.ptr, 0, 512))
+    qwhip.check(lib.qwhip_plane_checksum(st, banks[0].ptr, bank_bytes, sum_dev.ptr))
+    dev.stream.sync()
+    if int(sum_dev.download(np.uint64, (256,)).sum()) != int(blocks.ravel().view(np.uint32).astype(np.uint64).sum()):
+        _fail("bench: plane checksum differs from the host's")
+    for i in range(args.warmup):
+        lib.qwhip_plane_checksum(st, banks[i % ring_n].ptr, bank_bytes, sum_dev.ptr)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        lib.qwhip_plane_checksum(st, banks[i % ring_n].ptr, bank_bytes, sum_dev.ptr)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    read_us = e0.elapsed_ms(e1) * 1e3 / args.steps
     out = {
         "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -147,7 +163,8 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None):
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": traffic if (args.variant == 0 and args.rt == 0 and not args.prerot) else None,
-                     "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
+                     "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3),
+                     "read_only_launch_us": round(read_us, 3), "read_only_frac": round(bank_bytes / (read_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
         "normalized_error": err, "wall_ms_per_step": round(wall * 1e3 / args.steps, 6),
     }
     if not args.no_cpu:

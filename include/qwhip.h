@@ -97,6 +97,11 @@ qwhip_status qwhip_memcpy_h2d(qwhip_stream_t s, void* dst, const void* src, size
 qwhip_status qwhip_memcpy_d2h(qwhip_stream_t s, void* dst, const void* src, size_t bytes); /* synchronous */
 qwhip_status qwhip_memcpy_d2d(qwhip_stream_t s, void* dst, const void* src, size_t bytes); /* async on s */
 qwhip_status qwhip_fill_u32(qwhip_stream_t s, void* dst, uint32_t value, size_t count);    /* async fill kernel */
+/* Adds the sum of the 32-bit words of a device plane (16-byte aligned, whole 16-byte pieces) into the 256 device words
+ * sum[0..255], which the caller clears first (qwhip_fill_u32, 512 words); the checksum is their total mod 2^64.  No
+ * counterpart in the reference: it is how a loader checks an uploaded plane against the host copy without reading it
+ * back, and - a launch that only reads - the read-bandwidth yardstick bench.py quotes beside the decode GEMV. */
+qwhip_status qwhip_plane_checksum(qwhip_stream_t s, const void* plane, size_t bytes, uint64_t* sum);
 /* GPU timestamps (QWStageCounter, Sources/Foundation/QWHAL/QWStageCounter.swift:1-40). */
 qwhip_status qwhip_event_create(qwhip_device_t dev, qwhip_event_t* out);
 qwhip_status qwhip_event_destroy(qwhip_event_t e);

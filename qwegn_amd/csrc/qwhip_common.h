@@ -205,12 +205,12 @@ __device__ __forceinline__ h8_t qw_hadamard_rows(uint32_t i, uint32_t c) {
     return __builtin_bit_cast(h8_t, bits);
 }
 
+// 8 activations loaded as 16 raw bytes (f16 or bf16) -> f16
 template <int XDT>
-__device__ __forceinline__ h8_t qw_load_x8_f16(const void* x, uint64_t elem) {
+__device__ __forceinline__ h8_t qw_x8_from_raw(u4_t raw) {
     if constexpr (XDT == QWHIP_F16) {
-        return *(const h8_t*)((const h1_t*)x + elem);
+        return __builtin_bit_cast(h8_t, raw);
     } else {
-        const u4_t raw = *(const u4_t*)((const uint16_t*)x + elem);
         h8_t o;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -219,6 +219,11 @@ __device__ __forceinline__ h8_t qw_load_x8_f16(const void* x, uint64_t elem) {
         }
         return o;
     }
+}
+
+template <int XDT>
+__device__ __forceinline__ h8_t qw_load_x8_f16(const void* x, uint64_t elem) {
+    return qw_x8_from_raw<XDT>(*(const u4_t*)((const uint16_t*)x + elem));
 }
 
 // Rows i and i + 16 (i = lane & 15) of the 32-point Hadamard matrix, columns 8c .. 8c + 7 (c = lane >> 4), as f16 +-1:

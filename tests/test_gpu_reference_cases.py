@@ -533,3 +533,27 @@ def test_pack_writer_quantizes_on_the_device_and_round_trips(dev, tmp_path):
     buf, view = pk.upload(dev, "o_proj")
     assert (view.n, view.k, view.bits, view.group) == (24, k, 8, 64)
     assert np.array_equal(buf.download(np.uint8, (want.nbytes,)), want.ravel().view(np.uint8))
+
+
+@pytest.mark.parametrize("nbytes", [16, 4096 + 16, 3 * 1024 * 1024 + 48, 55705600])
+def test_plane_checksum_is_the_hosts_word_sum(dev, nbytes):
+    """The sum of a plane's 32-bit words, exact in 64 bits whatever order the workgroups finish in; it adds into the 256
+    words the caller cleared (two calls double their total); unaligned planes and ragged sizes are refused before any launch."""
+    rng = np.random.default_rng(nbytes)
+    host = rng.integers(0, 1 << 32, size=nbytes // 4, dtype=np.uint64).astype(np.uint32)
+    plane, out = dev.put(host), dev.alloc(256 * 8)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_fill_u32(st, out.ptr, 0, 512))
+    qwhip.check(lib.qwhip_plane_checksum(st, plane.ptr, nbytes, out.ptr))
+    dev.stream.sync()
+    want = int(host.astype(np.uint64).sum())
+    assert int(out.download(np.uint64, (256,)).sum()) == want
+    qwhip.check(lib.qwhip_plane_checksum(st, plane.ptr, nbytes, out.ptr))
+    dev.stream.sync()
+    assert int(out.download(np.uint64, (256,)).sum()) == 2 * want
+    assert lib.qwhip_plane_checksum(st, plane.ptr, nbytes - 4, out.ptr) == qwhip.E_BAD_SHAPE
+    if nbytes > 16:
+        assert lib.qwhip_plane_checksum(st, plane.ptr + 4, nbytes - 16, out.ptr) == qwhip.E_BAD_SHAPE
+    assert lib.qwhip_plane_checksum(st, plane.ptr, 0, out.ptr) == qwhip.OK
+    plane.free()
+    out.free()
