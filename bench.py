@@ -10,7 +10,7 @@ kernel measured with HIP events on the launch stream, and the CPU baseline (the 
 oracle form - dequantize the bank to fp32, then one fp32 product - restated in numpy and timed
 on this box's host cores over a bounded sample).
 
-Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up|mlp_prefill|head|f32_decode|f32_verify4|repack|norm_prefill|norm_decode (see WORKLOADS).
+Other workloads: --workload c1|c2|c3|c4_decode|c4_prefill|c5_qkv|c5_down|mlp_gate_up|mlp_prefill|head|f32_decode|f32_verify4|f32_batched64|repack|norm_prefill|norm_decode (see WORKLOADS).
 """
 from __future__ import annotations
 
@@ -750,6 +750,7 @@ WORKLOADS = {
     "head": ("head", "hq4_g32_m5", 151936, 5120, 1, False),
     "f32_decode": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 1, False),
     "f32_verify4": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 4, False),
+    "f32_batched64": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 64, False),      # 32 rows and more: the matrix-core form
     "repack": ("repack", None, 34816, 5120, None, False),              # MLX 4-bit group 64, gate|up sized
     "norm_prefill": ("norm", None, 5120, None, 4096, False),           # n = hidden, m = rows
     "norm_decode": ("norm", None, 5120, None, 1, False),
@@ -767,6 +768,7 @@ LABELS = {
     "head": "LM head GEMV + argmax, HQ4_G32 M=1 K=5120 N=151936",
     "f32_decode": "f32-activation GEMV, HQ4_G32 M=1 K=5120 N=17408",
     "f32_verify4": "f32-activation GEMV, HQ4_G32 M=4 K=5120 N=17408",
+    "f32_batched64": "f32-activation batched GEMM, HQ4_G32 M=64 K=5120 N=17408",
     "repack": "MLX affine -> AQ4_G64 repack, 34816 x 5120",
     "norm_prefill": "RMSNorm + residual + FWHT producer, 4096 rows x 5120",
     "norm_decode": "RMSNorm + residual + FWHT producer, 1 row x 5120",

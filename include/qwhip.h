@@ -189,7 +189,11 @@ qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, 
  * every container width (2, 3, 4, 6, 8 bits and HQ4_G32_M5).  All arithmetic in fp32: weights are code * scale + bias
  * without the f16 rounding of qwhip_dequant_f16, as in the reference's f32 dequant (qw_dequant_f32.metalh:1-24).
  * epi: 0 none, 1 silu(y / scale), 2 sigmoid(y), 3 silu(y / scale) followed by the FWHT-32 over each 32 consecutive outputs
- * (a last partial group is padded with zeros).  Four activation rows share one pass over the bank. */
+ * (a last partial group is padded with zeros).  Up to 31 rows: four activation rows share one pass over the bank, all
+ * arithmetic in fp32.  From 32 rows on (where the reference switches to its batched kernels) and k % 64 == 0: the
+ * matrix-core form, 64 activation rows per pass over the bank; activations and weights are each split into two f16
+ * numbers (22 bits together) and three products are accumulated in fp32 - the same 2e-5 bar, activations within the
+ * f16 range (|x| <= 65504). */
 qwhip_status qwhip_gemv_f32(qwhip_stream_t s, const qwhip_weight_view* w, const float* x, uint32_t m, uint32_t epi,
                             float scale, float* y);
 

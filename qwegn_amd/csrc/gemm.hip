@@ -1005,7 +1005,7 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 // stage between two barriers at its end.
 // ------------------------------------------------------------------------------------------------
 template <int FMT, int YDT, bool SWIGLU>
-__global__ __launch_bounds__(256) void qw_gemm5_kernel(const qw_gemm_params p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void qw_gemm5_kernel(const qw_gemm_params p) {
     static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
     static_assert(FMT == QG_FMT_M5 || FMT == QG_FMT_B4, "20-byte blocks: HQ4_G32_M5 and the 4-bit group-32 bit streams");
     // raw image: row pitch 88 bytes (22 dwords: the 64 lanes of a block read fall on 64 different banks), one stage

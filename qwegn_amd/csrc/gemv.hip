@@ -1342,10 +1342,15 @@ uint32_t qw_f32_gemv_rows(const qwhip_weight_view* w, uint64_t row_bytes);
 void qw_f32_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
                  const float* x, uint32_t m, uint32_t epi, float scale, float* y);
 void qw_h32_f32_launch(hipStream_t st, const float* x, float* out, uint32_t rows, uint32_t hidden);
+// gemm_f32.hip
+bool qw_f32_gemm(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                 const float* x, uint32_t m, uint32_t epi, float scale, float* y);
 
 // fp32 activations in the container's basis -> fp32 outputs with the scalar epilogues of the reference's f32 family
 // (QWGemm.encodeHQ4F32V4 / encodeHQ4F32BM, Sources/Operators/QWGEMM/QWGemmF32.swift:178-199,311-350): the rows go through
-// the column-stationary fp32 kernel four (long rows: two, one) at a time, as the reference's v4 door walks them.
+// the column-stationary fp32 kernel four (long rows: two, one) at a time, as the reference's v4 door walks them; from 32
+// rows on (where the reference switches to its batched kernels) the matrix-core form of gemm_f32.hip reads the bank once
+// per 64 rows.
 extern "C" qwhip_status qwhip_gemv_f32(qwhip_stream_t s, const qwhip_weight_view* w, const float* x, uint32_t m, uint32_t epi,
                                        float scale, float* y) {
     QWHIP_REQUIRE(s);
@@ -1364,7 +1369,9 @@ extern "C" qwhip_status qwhip_gemv_f32(qwhip_stream_t s, const qwhip_weight_view
     const uint32_t per = qw_f32_gemv_rows(w, row_bytes);
     if (per == 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "no f32 gemv kernel for n=%u k=%u (rows up to 32768 columns, banks under 1 GiB)", w->n, w->k);
     const uint32_t gshift = log2_u32(w->group / 32), bb = qwhip_view_block_bytes(w);
-    for (uint32_t m0 = 0; m0 < m; m0 += per) {
+    const bool batched = m >= 32u && qw_f32_gemm(s->stream, w, fmt, gshift, bb, row_bytes, x, m, epi, scale, y);
+    if (batched) QWHIP_TRY_HIP(hipGetLastError());
+    for (uint32_t m0 = 0; !batched && m0 < m; m0 += per) {
         const uint32_t mm = min(per, m - m0);
         qw_f32_gemv(s->stream, w, fmt, gshift, bb, row_bytes, x + (size_t)m0 * w->k, mm, epi, scale, y + (size_t)m0 * w->n);
         QWHIP_TRY_HIP(hipGetLastError());

@@ -57,6 +57,43 @@ def test_gemv_f32_shapes(dev, fmt, n, k, m):
     assert qo.normalized_error(got, want) <= TOL
 
 
+@pytest.mark.parametrize("fmt", list(H.FORMATS))
+@pytest.mark.parametrize("m", [32, 45, 64, 130])
+def test_batched_f32_form_matches_the_oracle(dev, fmt, m):
+    """From 32 activation rows on (QWGemm.encodeHQ4F32BM, QWGemmF32.swift:311-350) the door runs the matrix-core form:
+    activations and un-rounded affine weights each split into two f16 numbers, three products in fp32 accumulators.  Same
+    bar as the fp32 GEMV form; n = 200 ends in a partial 64-row tile, m = 45 / 130 in partial row tiles."""
+    got, want, _ = _run(dev, fmt, 200, 1024, m, 0, 1.0, seed=m)
+    assert qo.normalized_error(got, want) <= TOL
+
+
+@pytest.mark.parametrize("epi,scale", [(1, 1.0), (1, 0.05), (2, 1.0), (3, 0.05), (3, 2.0)])
+@pytest.mark.parametrize("fmt,n", [("hq4_g32_m5", 256), ("aq8_g256", 200), ("hq4_g64", 77), ("hq3_g32", 96)])
+def test_batched_f32_form_epilogues(dev, fmt, n, epi, scale):
+    got, want, _ = _run(dev, fmt, n, 512, 40, epi, scale, seed=7)
+    assert qo.normalized_error(got, want) <= TOL
+
+
+@pytest.mark.parametrize("fmt,n,k,m", [
+    ("hq4_g32_m5", 17408, 5120, 64),    # the decode MLP bank with 64 rows: 272 x 1 tiles
+    ("hq4_g64", 512, 17408, 33),        # long rows
+    ("aq4_g32", 70, 64, 32),            # one K-step
+    ("hq8_g32", 64, 96, 32),            # K is not whole 64-column steps: the GEMV form takes it
+])
+def test_batched_f32_form_shapes(dev, fmt, n, k, m):
+    got, want, _ = _run(dev, fmt, n, k, m, 0, 1.0, seed=11)
+    assert qo.normalized_error(got, want) <= TOL
+
+
+def test_batched_f32_form_agrees_with_the_row_form(dev):
+    """31 rows go four at a time through the fp32 kernel, 32 rows through the matrix cores: the same rows agree to the
+    oracle's bar with each other (both sit within 2e-5 of the float64 evaluation)."""
+    got32, want32, _ = _run(dev, "hq4_g32_m5", 384, 2048, 32, 0, 1.0, seed=5)
+    got31, want31, _ = _run(dev, "hq4_g32_m5", 384, 2048, 31, 0, 1.0, seed=5)
+    assert np.array_equal(want32[:31], want31)
+    assert qo.normalized_error(got32[:31], got31.astype(np.float64)) <= 2 * TOL
+
+
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq8_g32"])
 def test_epilogue3_rows_together_equal_rows_alone(dev, fmt):
     """The reference's own check (Tests/QWGEMMTests/QWGemmEpi3MultiRowTests.swift:71-113): 2..5 rows in one call against
