@@ -349,7 +349,10 @@ qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_
 
 /* qwg_moe_down_reduce_combine_f32 (Sources/QWMetal/gemm/qwgemm_moe_nax_f16.metal:7-126;
  * encodeMoEDownReduceCombineF32, QWGemmMoE.swift:299-332):
- * out[t, h] = sum_k wts[t, k] * dn[inv_perm[t*top_k + k], h] (+ shared_gate[t] * shared[t, h]). */
+ * out[t, h] = sum_k wts[t, k] * dn[inv_perm[t*top_k + k], h] (+ shared_gate[t] * shared[t, h]).
+ * inv_perm = NULL: route k of token t sits in row t*top_k + k (the door's invPerm: nil); wts = NULL: unit weights (its
+ * unweightedSingle) - with top_k = 1 that is out = dn + shared_gate * shared, the last step of the latent operator.
+ * out may be dn when inv_perm is NULL and top_k = 1. */
 qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint32_t dn_dtype, const int32_t* inv_perm,
                                const float* wts, uint32_t t, uint32_t top_k, uint32_t hidden,
                                const float* shared, const float* shared_gate, void* out, uint32_t out_dtype);

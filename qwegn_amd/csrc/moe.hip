@@ -417,8 +417,8 @@ __global__ __launch_bounds__(256) void qw_moe_combine_kernel(const void* __restr
         float w[KMAX];
 #pragma unroll
         for (uint32_t k = 0; k < (uint32_t)KMAX; ++k) {
-            slot[k] = k < K ? inv_perm[(uint64_t)t * K + k] : -1;
-            w[k] = k < K ? wts[(uint64_t)t * K + k] : 0.0f;
+            slot[k] = k < K ? (inv_perm ? inv_perm[(uint64_t)t * K + k] : (int32_t)(t * K + k)) : -1;
+            w[k] = k < K ? (wts ? wts[(uint64_t)t * K + k] : 1.0f) : 0.0f;
         }
         float v[KMAX][4];
 #pragma unroll
@@ -446,9 +446,9 @@ __global__ __launch_bounds__(256) void qw_moe_combine_kernel(const void* __restr
         }
     } else
     for (uint32_t k = 0; k < K; ++k) {
-        const int32_t slot = inv_perm[(uint64_t)t * K + k];
+        const int32_t slot = inv_perm ? inv_perm[(uint64_t)t * K + k] : (int32_t)(t * K + k);
         if (slot < 0) continue;
-        const float w = wts[(uint64_t)t * K + k];
+        const float w = wts ? wts[(uint64_t)t * K + k] : 1.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             if (h + j < H) acc[j] = fmaf(w, qw_load_f32<DDT>(dn, (uint64_t)slot * H + h + j), acc[j]);
@@ -476,9 +476,8 @@ extern "C" qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint
     QWHIP_REQUIRE(s);
     if (t == 0 || hidden == 0) return QWHIP_OK;
     QWHIP_REQUIRE(dn);
-    QWHIP_REQUIRE(inv_perm);
-    QWHIP_REQUIRE(wts);
     QWHIP_REQUIRE(out);
+    if ((uint64_t)t * top_k >= (1ull << 31)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine: %u x %u route slots", t, top_k);
     const dim3 grid(qwhip_cdiv(hidden, 1024), t), block(256);
 #define QW_CB(DD, OD)                                                                                                          \
     do {                                                                                                                       \

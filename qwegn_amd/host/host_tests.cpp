@@ -350,6 +350,181 @@ static void test_gpu_moe_resident(QWHal& hal, int rows) {
     hal.end(enc);
 }
 
+// QWMoEOperator.encodeResidentLatent on closed-form banks against the chain in double (QWMoEOperator+Latent.swift:17-303):
+// bridge -> router (+ shared gate) -> fc1 -> route -> rotate -> routed experts in the latent width -> latent norm -> fc2,
+// shared expert on the hidden width added under its gate.  rows = 3 takes the routed GEMVs, rows = 40 the grouped GEMMs and
+// the batched f32 projections.
+static void test_gpu_moe_latent(QWHal& hal, int rows) {
+    const int E = 16, K = 3, H = 256, L = 64, I = 64, ISh = 64;
+    const float eps = 1e-6f;
+    const std::vector<uint8_t> fc1 = cf_bank(L, H), fc2 = cf_bank(H, L), gu = cf_bank(E * 2 * I, L), dn = cf_bank(E * L, I);
+    const std::vector<uint8_t> shgu = cf_bank(2 * ISh, H), shdn = cf_bank(H, ISh);
+    std::vector<float> router((size_t)E * H);
+    for (int e = 0; e < E; ++e)
+        for (int h = 0; h < H; ++h) router[(size_t)e * H + h] = (float)(((e * 5 + h * 11) % 17) - 8) / 64.0f;
+    std::vector<uint16_t> gamma(L);
+    for (int l = 0; l < L; ++l) gamma[l] = f2h((float)((l % 5) - 2) / 16.0f);
+    std::vector<uint16_t> x((size_t)rows * H);
+    for (int t = 0; t < rows; ++t)
+        for (int h = 0; h < H; ++h) x[(size_t)t * H + h] = f2h((float)(((t * 13 + h * 7) % 19) - 9) / 8.0f);
+    auto silu = [](double g) { return g / (1 + std::exp(-g)); };
+    std::vector<double> ref((size_t)rows * H, 0.0);
+    for (int t = 0; t < rows; ++t) {
+        std::vector<double> xr(H), xp(H);
+        for (int h = 0; h < H; ++h) xr[h] = xp[h] = h2f(x[(size_t)t * H + h]);
+        for (int o = 0; o < H; o += 32) fwht32(&xp[o]);
+        std::vector<double> logit(E), p(E);
+        double mx = -1e300, tot = 0;
+        for (int e = 0; e < E; ++e) {
+            double a = 0;
+            for (int h = 0; h < H; ++h) a += (double)router[(size_t)e * H + h] * xp[h];
+            logit[e] = a;
+            mx = std::fmax(mx, a);
+        }
+        const double gate = 1.0 / (1.0 + std::exp(-logit[0]));   // the gate row is router row 0
+        for (int e = 0; e < E; ++e) { p[e] = std::exp(logit[e] - mx); tot += p[e]; }
+        std::vector<int> chosen;
+        std::vector<bool> taken(E, false);
+        double wsum = 0;
+        for (int r = 0; r < K; ++r) {
+            int best = -1;
+            for (int e = 0; e < E; ++e)
+                if (!taken[e] && (best < 0 || p[e] > p[best])) best = e;
+            taken[best] = true;
+            chosen.push_back(best);
+            wsum += p[best] / tot;
+        }
+        std::vector<double> lat(L), B(L, 0.0);
+        for (int l = 0; l < L; ++l) {
+            double a = 0;
+            for (int h = 0; h < H; ++h) a += cf_weight(l, h) * xr[h];
+            lat[l] = a;
+        }
+        for (int o = 0; o < L; o += 32) fwht32(&lat[o]);
+        for (int l = 0; l < L; ++l) lat[l] = h2f(f2h((float)lat[l]));
+        for (int r = 0; r < K; ++r) {
+            const int e = chosen[r];
+            const double wk = (p[e] / tot) / wsum;
+            std::vector<double> act(I);
+            for (int i = 0; i < I; ++i) {
+                double g = 0, u = 0;
+                for (int l = 0; l < L; ++l) {
+                    g += cf_weight(e * 2 * I + i, l) * lat[l];
+                    u += cf_weight(e * 2 * I + I + i, l) * lat[l];
+                }
+                act[i] = silu(g) * u;
+            }
+            for (int o = 0; o < I; o += 32) fwht32(&act[o]);
+            for (int i = 0; i < I; ++i) act[i] = h2f(f2h((float)act[i]));
+            for (int l = 0; l < L; ++l) {
+                double d = 0;
+                for (int i = 0; i < I; ++i) d += cf_weight(e * L + l, i) * act[i];
+                B[l] += wk * d;
+            }
+        }
+        double ms = 0;
+        for (int l = 0; l < L; ++l) ms += B[l] * B[l];
+        const double inv = 1.0 / std::sqrt(ms / L + (double)eps);
+        std::vector<double> Cn(L);
+        for (int l = 0; l < L; ++l) Cn[l] = B[l] * inv * (1.0 + (double)h2f(gamma[l]));
+        for (int o = 0; o < L; o += 32) fwht32(&Cn[o]);
+        std::vector<double> sact(ISh);
+        for (int j = 0; j < ISh; ++j) {
+            double g = 0, u = 0;
+            for (int h = 0; h < H; ++h) {
+                g += cf_weight(j, h) * xr[h];
+                u += cf_weight(ISh + j, h) * xr[h];
+            }
+            sact[j] = silu(g) * u;
+        }
+        for (int o = 0; o < ISh; o += 32) fwht32(&sact[o]);
+        for (int h = 0; h < H; ++h) {
+            double a = 0, sh = 0;
+            for (int l = 0; l < L; ++l) a += cf_weight(h, l) * Cn[l];
+            for (int j = 0; j < ISh; ++j) sh += cf_weight(h, j) * sact[j];
+            ref[(size_t)t * H + h] = a + gate * sh;
+        }
+    }
+    QWHipEncoder enc = hal.begin();
+    const int pairs = rows * K, mt = QWGemm::moeMaxTiles(E, pairs);
+    DeviceBuf dfc1(hal, fc1.size()), dfc2(hal, fc2.size()), dgu(hal, gu.size()), ddn(hal, dn.size()), dshgu(hal, shgu.size()), dshdn(hal, shdn.size());
+    DeviceBuf dr(hal, router.size() * 4), dgm(hal, gamma.size() * 2), dx(hal, x.size() * 2), dout(hal, (size_t)rows * H * 4);
+    DeviceBuf dlog(hal, (size_t)rows * E * 4), didx(hal, pairs * 4), dw(hal, pairs * 4), dact(hal, (size_t)pairs * I * 2);
+    DeviceBuf doff(hal, (E + 1) * 4), dsp(hal, pairs * 4), dst(hal, pairs * 4), dinv(hal, pairs * 4), dte(hal, mt * 4), dtr(hal, mt * 4), dtc(hal, 16);
+    DeviceBuf ddnhi(hal, (size_t)pairs * L * 4);
+    DeviceBuf dxr(hal, (size_t)rows * H * 4), dxp(hal, (size_t)rows * H * 4), dA(hal, (size_t)rows * L * 4), dB(hal, (size_t)rows * L * 4);
+    DeviceBuf dB16(hal, (size_t)rows * L * 2), dnax(hal, (size_t)rows * H * 2), dgate(hal, (size_t)rows * 4);
+    DeviceBuf dgush(hal, (size_t)rows * 2 * ISh * 4), dactsh(hal, (size_t)rows * ISh * 4), dshared(hal, (size_t)rows * H * 4);
+    upload(enc, dfc1, fc1.data(), fc1.size());
+    upload(enc, dfc2, fc2.data(), fc2.size());
+    upload(enc, dgu, gu.data(), gu.size());
+    upload(enc, ddn, dn.data(), dn.size());
+    upload(enc, dshgu, shgu.data(), shgu.size());
+    upload(enc, dshdn, shdn.data(), shdn.size());
+    upload(enc, dr, router.data(), router.size() * 4);
+    upload(enc, dgm, gamma.data(), gamma.size() * 2);
+    upload(enc, dx, x.data(), x.size() * 2);
+    auto bankView = [](DeviceBuf& b, int n, int k) { return *QWWeightView::make(QWTensorValue::make(b.p, b.bytes, QWDType::q4g), n, k, 4, 32, true); };
+    QWMoEOperator::LatentWeights lw;
+    lw.routed.router = QWTensorValue::make(dr.p, router.size(), QWDType::f32);
+    lw.routed.gateUp = bankView(dgu, E * 2 * I, L);
+    lw.routed.down = bankView(ddn, E * L, I);
+    lw.routed.hidden = H; lw.routed.experts = E; lw.routed.topK = K; lw.routed.intermediate = I;
+    lw.sharedGateUp = bankView(dshgu, 2 * ISh, H);
+    lw.sharedDown = bankView(dshdn, H, ISh);
+    lw.sharedGateScalar = QWTensorValue::make(dr.p, (size_t)H, QWDType::f32);
+    lw.sharedIntermediate = ISh;
+    QWMoEOperator::LatentBottleneck lb;
+    lb.fc1 = bankView(dfc1, L, H);
+    lb.fc2 = bankView(dfc2, H, L);
+    lb.normGamma = QWTensorValue::make(dgm.p, (size_t)L, QWDType::f16);
+    lb.normEps = eps;
+    lb.latentDim = L;
+    QWMoEOperator::Scratch s;
+    s.logits = QWTensorValue::make(dlog.p, (size_t)rows * E, QWDType::f32);
+    s.idx = QWTensorValue::make(didx.p, pairs, QWDType::i32);
+    s.wts = QWTensorValue::make(dw.p, pairs, QWDType::f32);
+    s.act16 = QWTensorValue::make(dact.p, (size_t)pairs * I, QWDType::f16);
+    s.expOff = QWTensorValue::make(doff.p, E + 1, QWDType::i32);
+    s.sortedPair = QWTensorValue::make(dsp.p, pairs, QWDType::i32);
+    s.sortedTok = QWTensorValue::make(dst.p, pairs, QWDType::i32);
+    s.invPerm = QWTensorValue::make(dinv.p, pairs, QWDType::i32);
+    s.tileE = QWTensorValue::make(dte.p, mt, QWDType::i32);
+    s.tileR = QWTensorValue::make(dtr.p, mt, QWDType::i32);
+    s.tileCount = QWTensorValue::make(dtc.p, 4, QWDType::i32);
+    s.dnHi = QWTensorValue::make(ddnhi.p, (size_t)pairs * L, QWDType::f32);
+    QWMoEOperator::LatentScratch ls;
+    ls.xRot32 = QWTensorValue::make(dxr.p, (size_t)rows * H, QWDType::f32);
+    ls.xPlain32 = QWTensorValue::make(dxp.p, (size_t)rows * H, QWDType::f32);
+    ls.bufA32 = QWTensorValue::make(dA.p, (size_t)rows * L, QWDType::f32);
+    ls.bufB32 = QWTensorValue::make(dB.p, (size_t)rows * L, QWDType::f32);
+    ls.bufB16 = QWTensorValue::make(dB16.p, (size_t)rows * L, QWDType::f16);
+    ls.naxX16 = QWTensorValue::make(dnax.p, (size_t)rows * H, QWDType::f16);
+    ls.gate = QWTensorValue::make(dgate.p, (size_t)rows, QWDType::f32);
+    ls.guSh32 = QWTensorValue::make(dgush.p, (size_t)rows * 2 * ISh, QWDType::f32);
+    ls.actSh32 = QWTensorValue::make(dactsh.p, (size_t)rows * ISh, QWDType::f32);
+    ls.shared = QWTensorValue::make(dshared.p, (size_t)rows * H, QWDType::f32);
+    const QWTensorValue xt = QWTensorValue::make(dx.p, x.size(), QWDType::f16);
+    const QWTensorValue out = QWTensorValue::make(dout.p, (size_t)rows * H, QWDType::f32);
+    QWMoEOperator::encodeResidentLatent(enc, hal, lw, lb, s, ls, xt, out, rows);
+    std::vector<float> got((size_t)rows * H);
+    download(enc, got.data(), dout, got.size() * 4);
+    double num = 0, den = 0;
+    for (size_t i = 0; i < got.size(); ++i) { num += ((double)got[i] - ref[i]) * ((double)got[i] - ref[i]); den += ref[i] * ref[i]; }
+    const double err = std::sqrt(num / std::fmax(den, 1e-30));
+    std::printf("moe encodeResidentLatent rows=%d normalized error %.3e\n", rows, err);
+    CHECK(err <= 2e-3);
+    // geometry checks of the door: a latent width the banks do not have is refused before any launch
+    {
+        QWMoEOperator::LatentBottleneck bad = lb;
+        bad.latentDim = L + 32;
+        bool threw = false;
+        try { QWMoEOperator::encodeResidentLatent(enc, hal, lw, bad, s, ls, xt, out, rows); } catch (const QWGemmError&) { threw = true; }
+        CHECK(threw);
+    }
+    hal.end(enc);
+}
+
 // f32-activation doors and the head: encodeHQ4F32V4 (epilogues 0 and 3), encodeH32F32, encodeHeadArgmax on the closed-form bank
 static void test_gpu_f32_doors(QWHal& hal) {
     const int N = 96, Kc = 128, rows = 3;
@@ -495,6 +670,8 @@ int main(int argc, char** argv) {
         test_gpu_hq4_gemv(hal);
         test_gpu_moe_resident(hal, 3);    // decode / verify path
         test_gpu_moe_resident(hal, 40);   // grouped prefill path (fused gate_up + SwiGLU)
+        test_gpu_moe_latent(hal, 3);      // latent bottleneck, routed GEMVs
+        test_gpu_moe_latent(hal, 40);     // latent bottleneck, grouped GEMMs and batched f32 projections
         test_gpu_f32_doors(hal);
         test_gpu_dense_proj_f32(hal);
         test_gpu_embed(hal);

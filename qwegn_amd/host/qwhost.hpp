@@ -629,6 +629,18 @@ struct QWGemm {
                                         (uint32_t)rows, (uint32_t)topK, (uint32_t)hidden, shared ? (const float*)shared->ptr() : nullptr,
                                         sharedGate ? (const float*)sharedGate->ptr() : nullptr, out.ptr(), abiDType(out.shape.dtype)));
     }
+    // the door's invPerm: nil + unweightedSingle form (QWGemmMoE.swift:299-332): out = dn + sharedGate * shared, one row per token
+    static void encodeMoEAddSharedF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& dn, int rows, int hidden,
+                                      const QWTensorValue& shared, const QWTensorValue* sharedGate, const QWTensorValue& out) {
+        const size_t need = (size_t)rows * (size_t)hidden;
+        if (dn.shape.elementCount < need || shared.shape.dtype != QWDType::f32 || shared.shape.elementCount < need ||
+            out.shape.elementCount < need || (sharedGate && (sharedGate->shape.dtype != QWDType::f32 || sharedGate->shape.elementCount < (size_t)rows)))
+            throw QWGemmError(QWGemmError::badShape, "moe shared add: buffers do not fit rows x hidden");
+        hal.pipeline("qwg_moe_down_reduce_combine_f32");
+        throwIfFailed(qwhip_moe_combine(enc.stream, dn.ptr(), abiDType(dn.shape.dtype), nullptr, nullptr, (uint32_t)rows, 1u, (uint32_t)hidden,
+                                        (const float*)shared.ptr(), sharedGate ? (const float*)sharedGate->ptr() : nullptr, out.ptr(),
+                                        abiDType(out.shape.dtype)));
+    }
     // encodeFnMoeRoute + encodeMoEGateUpF32R1 as one launch (decode / verify): idx / wts are left for the down projection
     static void encodeMoERouteGateUp(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& gateUp, int experts, const QWTensorValue& x,
                                      const QWTensorValue& logits, const QWTensorValue& idx, const QWTensorValue& wts, int rows, int topK,
@@ -799,6 +811,78 @@ struct QWMoEOperator {
             QWGemm::encodeMoERouteGateUp(enc, hal, w.gateUp, E, x, s.logits, s.idx, s.wts, rows, K, w.normTopK, w.routedScale, s.act16);
             QWGemm::encodeMoEDownSharedCombineF32(enc, hal, w.down, E, s.act16, s.idx, s.wts, rows, K, shared, sharedGate, out);
         }
+    }
+
+    // ---- latent-bottleneck sparse MoE (QWMoEOperator+Latent.swift:17-303): fc1 -> routed experts in the latent width ->
+    // latent norm -> fc2, with the shared expert on the full hidden width ---------------------------------------------------
+    struct LatentBottleneck {
+        QWWeightView fc1;                       // n = latentDim, k = hidden
+        QWWeightView fc2;                       // n = hidden, k = latentDim
+        std::optional<QWTensorValue> normGamma; // f16 [latentDim], plus-one law; none = rotation only
+        float normEps = 1e-6f;
+        int latentDim = 0;
+    };
+    struct LatentWeights {
+        Weights routed;                         // gateUp: n = experts * 2 * intermediate, k = latentDim; down: n = experts * latentDim, k = intermediate
+        std::optional<QWWeightView> sharedGateUp;   // n = 2 * sharedIntermediate, k = hidden
+        std::optional<QWWeightView> sharedDown;     // n = hidden, k = sharedIntermediate
+        std::optional<QWTensorValue> sharedGateScalar;   // f32 [hidden]: gate = sigmoid(x . w), a column of the router launch
+        int sharedIntermediate = 0;
+        std::optional<QWTensorValue> routerBias, routedScaleParam;   // f32 [experts]
+        bool splitFeatureRouting = false;
+    };
+    struct LatentScratch {   // caller-owned
+        QWTensorValue xRot32, xPlain32;         // f32 [rows, hidden]
+        QWTensorValue bufA32, bufB32;           // f32 [rows, latentDim]
+        QWTensorValue bufB16;                   // f16 [rows, latentDim]: what the routed experts read
+        QWTensorValue naxX16;                   // f16 staging of the dense projections: rows * max(hidden, latentDim, sharedIntermediate)
+        QWTensorValue gate;                     // f32 [rows]
+        QWTensorValue guSh32, actSh32, shared;  // f32 [rows, 2 ISh], [rows, ISh], [rows, hidden]
+    };
+    // x16: f16 normed hidden rows in the rotated basis (the operator's .f16Normed input).  `s.dnHi` holds [rows * topK, latentDim].
+    // As in the reference the routed experts read the latent rows as f16 on the grouped path; here the decode path does too.
+    static void encodeResidentLatent(QWHipEncoder& enc, const QWHal& hal, const LatentWeights& lw, const LatentBottleneck& latent, const Scratch& s,
+                                     const LatentScratch& ls, const QWTensorValue& x16, const QWTensorValue& out32, int rows) {
+        const Weights& w = lw.routed;
+        const int H = w.hidden, L = latent.latentDim, E = w.experts, K = w.topK, I = w.intermediate, ISh = lw.sharedIntermediate;
+        if (E > 512 || E <= 0 || K <= 0 || K > 16) throw QWGemmError(QWGemmError::badShape, "latent moe: experts <= 512, routes <= 16");
+        if (L <= 0 || L % 32 != 0 || latent.fc1.n != L || latent.fc1.k != H || latent.fc2.n != H || latent.fc2.k != L)
+            throw QWGemmError(QWGemmError::badShape, "latent moe: fc1 is [latent, hidden], fc2 [hidden, latent], latent % 32 == 0");
+        if (w.gateUp.n != E * 2 * I || w.gateUp.k != L || w.down.n != E * L || w.down.k != I)
+            throw QWGemmError(QWGemmError::badShape, "latent moe: expert banks do not match (experts, latent, intermediate)");
+        const bool hasShared = ISh > 0 && lw.sharedGateUp && lw.sharedDown;
+        if (hasShared && (lw.sharedGateUp->n != 2 * ISh || lw.sharedGateUp->k != H || lw.sharedDown->n != H || lw.sharedDown->k != ISh))
+            throw QWGemmError(QWGemmError::badShape, "latent moe: shared expert banks do not match (hidden, shared intermediate)");
+        const int routerCols = lw.splitFeatureRouting ? 2 * E : E;
+        QWGemm::encodeMoEBridgeF16ToF32(enc, hal, x16, ls.xRot32, ls.xPlain32, rows, H);
+        const bool hasGate = hasShared && lw.sharedGateScalar;
+        QWGemm::encodeFnRouterGemm(enc, hal, ls.xPlain32, w.router, s.logits, rows, routerCols, H, hasGate ? &*lw.sharedGateScalar : nullptr,
+                           hasGate ? &ls.gate : nullptr);
+        QWGemm::encodeDenseProjF32(enc, hal, latent.fc1, ls.xRot32, ls.bufA32, ls.naxX16, rows);
+        QWGemm::encodeFnMoeRoute(enc, hal, s.logits, s.idx, s.wts, rows, E, K, w.normTopK, w.routedScale, lw.routerBias ? &*lw.routerBias : nullptr,
+                         lw.splitFeatureRouting, lw.routedScaleParam ? &*lw.routedScaleParam : nullptr);
+        QWGemm::encodeLatentNormH32F32(enc, hal, ls.bufA32, nullptr, ls.bufB32, &ls.bufB16, rows, L, latent.normEps, true);
+        if (hasShared) {
+            QWGemm::encodeDenseProjF32(enc, hal, *lw.sharedGateUp, ls.xRot32, ls.guSh32, ls.naxX16, rows);
+            QWGemm::encodeSiluMulF32(enc, hal, ls.guSh32, ls.actSh32, rows, ISh);
+            QWGemm::encodeDenseProjF32(enc, hal, *lw.sharedDown, ls.actSh32, ls.shared, ls.naxX16, rows);
+        }
+        const int pairs = rows * K;
+        const QWTensorValue xLat16 = ls.bufB16.slice(0, (size_t)rows * (size_t)L, QWDType::f16);
+        const bool grouped = rows > 8 && s.expOff.base && s.dnHi.base && L % 64 == 0 && I % 64 == 0;
+        if (grouped) {
+            QWGemm::encodeMoEGroupPairsF32(enc, hal, s.idx, s.expOff, s.sortedPair, s.sortedTok, E, pairs, K, &s.invPerm, &s.tileE, &s.tileR, &s.tileCount);
+            QWGemm::encodeMoEGateUpSwiglu(enc, hal, w.gateUp, E, xLat16, s.sortedTok, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.act16,
+                                  w.down.isRotated());
+            QWGemm::encodeMoEGroupedGemm(enc, hal, w.down, E, s.act16, nullptr, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.dnHi);
+            QWGemm::encodeMoEDownReduceCombineF32(enc, hal, s.dnHi, s.invPerm, s.wts, rows, K, L, nullptr, nullptr, ls.bufA32);
+        } else {
+            QWGemm::encodeMoEGateUpF32R1(enc, hal, w.gateUp, E, xLat16, s.idx, rows, K, s.act16);
+            QWGemm::encodeMoEDownSharedCombineF32(enc, hal, w.down, E, s.act16, s.idx, s.wts, rows, K, nullptr, nullptr, ls.bufA32);
+        }
+        QWGemm::encodeLatentNormH32F32(enc, hal, ls.bufA32, latent.normGamma ? &*latent.normGamma : nullptr, ls.bufB32, nullptr, rows, L, latent.normEps);
+        QWGemm::encodeDenseProjF32(enc, hal, latent.fc2, ls.bufB32, out32, ls.naxX16, rows);
+        if (hasShared) QWGemm::encodeMoEAddSharedF32(enc, hal, out32, rows, H, ls.shared, hasGate ? &ls.gate : nullptr, out32);
     }
 };
 
