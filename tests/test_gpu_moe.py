@@ -355,3 +355,41 @@ def test_moe_full_size_operator(t):
     import bench
     out = bench.run_moe(argparse.Namespace(steps=2, warmup=1, no_cpu=True), t, "full-size parity")
     assert out["normalized_error"] <= TOL
+
+
+@pytest.mark.parametrize("hidden", [256, 1000])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_combine_identity_slots_and_unit_weights(dev, hidden, dtype):
+    """The door's invPerm: nil and unweightedSingle forms (encodeMoEDownReduceCombineF32, QWGemmMoE.swift:299-332): without
+    a permutation route k of token t is row t * top_k + k, without weights every route counts once; with one route that is
+    out = dn + gate * shared (the last step of the latent operator), in place when the types agree."""
+    rng = np.random.default_rng(hidden)
+    t, k = 5, 3
+    dn = rng.standard_normal((t * k, hidden)).astype(np.float32)
+    dn_h = dn.astype(np.float16) if dtype == "f16" else dn
+    wts = rng.random((t, k)).astype(np.float32)
+    shared = rng.standard_normal((t, hidden)).astype(np.float32)
+    gate = rng.random(t).astype(np.float32)
+    lib, st = dev.lib, dev.stream.handle
+    code = qwhip.F16 if dtype == "f16" else qwhip.F32
+    d_dn, d_w, d_sh, d_g, d_out = dev.put(dn_h), dev.put(wts), dev.put(shared), dev.put(gate), dev.alloc(t * hidden * 4)
+    base = dn_h.astype(np.float64).reshape(t, k, hidden)
+    # identity slots with weights
+    qwhip.check(lib.qwhip_moe_combine(st, d_dn.ptr, code, None, d_w.ptr, t, k, hidden, None, None, d_out.ptr, qwhip.F32))
+    dev.stream.sync()
+    want = (base * wts[:, :, None].astype(np.float64)).sum(1)
+    assert np.max(np.abs(d_out.download(np.float32, (t, hidden)) - want)) <= 1e-5 * np.abs(want).max()
+    # unit weights with the gated shared rows
+    qwhip.check(lib.qwhip_moe_combine(st, d_dn.ptr, code, None, None, t, k, hidden, d_sh.ptr, d_g.ptr, d_out.ptr, qwhip.F32))
+    dev.stream.sync()
+    want = base.sum(1) + gate[:, None].astype(np.float64) * shared
+    assert np.max(np.abs(d_out.download(np.float32, (t, hidden)) - want)) <= 1e-5 * np.abs(want).max()
+    if dtype == "f32":   # one route, in place: dn += gate * shared
+        rows = dev.put(dn[:t])
+        qwhip.check(lib.qwhip_moe_combine(st, rows.ptr, qwhip.F32, None, None, t, 1, hidden, d_sh.ptr, d_g.ptr, rows.ptr, qwhip.F32))
+        dev.stream.sync()
+        want = dn[:t].astype(np.float64) + gate[:, None].astype(np.float64) * shared
+        assert np.max(np.abs(rows.download(np.float32, (t, hidden)) - want)) <= 1e-6 * np.abs(want).max()
+        rows.free()
+    for b in (d_dn, d_w, d_sh, d_g, d_out):
+        b.free()
