@@ -208,7 +208,9 @@ qwhip_status qwhip_h32_f32(qwhip_stream_t s, const float* x, float* out, uint32_
  * a number), ties to the lower row.  `logits` is required and kept (the reference's writeLogits); the reference's key
  * scratch is not needed.  x_dtype QWHIP_F32 takes fp32 activations already in the container's basis (the logits are then
  * those of qwhip_gemv_f32 with epilogue 0, and `flags` is unused).  qwhip_argmax_f32 is the fold alone, over any [rows, n]
- * f32 logits. */
+ * f32 logits.  One row (m = 1, f16 / bf16) over an HQ4_G32_M5 bank folds inside the GEMV's epilogue, as the reference's head
+ * kernels do: every workgroup leaves one key in the stream's scratch and the second launch is the one-workgroup fold of those
+ * keys (qwg_head_argmax_fin); the token is the same. */
 qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                uint32_t flags, float* logits, int32_t* tokens);
 qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);

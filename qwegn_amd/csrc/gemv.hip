@@ -976,7 +976,8 @@ bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t 
 
 // gemv_col.hip
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
-                 float* y32, uint32_t tune, hipError_t* err);
+                 float* y32, uint32_t tune, hipError_t* err, unsigned long long* keys, uint32_t keys_cap, int32_t* token,
+                 bool* folded);
 
 // gemv_sk.hip
 bool qw_sk_gemv(qwhip_stream_t s, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
@@ -987,8 +988,9 @@ bool qw_sk_gemv(qwhip_stream_t s, const qwhip_weight_view* w, int fmt, uint32_t 
 // 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel, 9 = split-K MFMA kernel);
 // bits 12..15: row tiles per wave for the direct-load mfma kernel / K-split of the streamer / tuning code of the
 // column-stationary kernel (0 = automatic); bits 12..18: tuning code of the split-K kernel.
-extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
-                                   uint32_t m, uint32_t flags, void* y16, float* y32) {
+// `token` (head door only): where the column-stationary kernel's fused fold leaves the argmax; *folded tells whether it ran
+static qwhip_status qw_gemv_impl(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
+                                 uint32_t flags, void* y16, float* y32, int32_t* token, bool* folded) {
     int fmt = 0;
     qwhip_status st = check_common(s, w, x, x_dtype, m, &fmt);
     if (st != QWHIP_OK) return st;
@@ -1055,7 +1057,9 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     }
     if (variant == 4 || (variant == 0 && fmt == QW_FMT_M5 && m == 1)) {
         hipError_t e = hipSuccess;
-        if (fmt == QW_FMT_M5 && m == 1 && qw_col_gemv(s->stream, w, x, x_dtype, rotate, y16, y32, rt, &e)) {
+        unsigned long long* keys = token && s->scratch ? (unsigned long long*)s->scratch : nullptr;   // the stream's counter area
+        if (fmt == QW_FMT_M5 && m == 1 &&
+            qw_col_gemv(s->stream, w, x, x_dtype, rotate, y16, y32, rt, &e, keys, QWHIP_STREAM_COUNTER_BYTES / 8u, token, folded)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }
@@ -1141,6 +1145,11 @@ extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w,
     else launch_mfma_rt<QW_FMT_B8>(s->stream, a, x_dtype, xm, lds, (int)rt);
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
+}
+
+extern "C" qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
+                                   uint32_t m, uint32_t flags, void* y16, float* y32) {
+    return qw_gemv_impl(s, w, x, x_dtype, m, flags, y16, y32, nullptr, nullptr);
 }
 
 extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
@@ -1399,14 +1408,18 @@ extern "C" qwhip_status qwhip_h32_f32(qwhip_stream_t s, const float* x, float* o
 // LM head for greedy decoding: logits = W . x over the vocabulary rows, then the argmax of each activation row with the
 // reference's key rule (QWGemmAQ.encodeHeadArgmax, Sources/Operators/QWGEMM/QWGemmAQ.swift:306-349; qwg_head_gemv_*_argmax,
 // qwg_gemv_*_f32_v4_am).  Two launches on the stream: the GEMV of qwhip_gemv into `logits` (which the caller keeps, as
-// with the reference's writeLogits), and one workgroup per row folding it.
+// with the reference's writeLogits), and one workgroup per row folding it.  One un-rotated or rotated row over an
+// HQ4_G32_M5 bank folds inside the GEMV's epilogue, as the reference's head kernels do (a key per workgroup in the stream's
+// scratch), and the second launch is the one-workgroup fold of those keys (the reference's qwg_head_argmax_fin).
 extern "C" qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);
 extern "C" qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                           uint32_t flags, float* logits, int32_t* tokens) {
     QWHIP_REQUIRE(logits);
     QWHIP_REQUIRE(tokens);
+    bool folded = false;
     qwhip_status st = x_dtype == QWHIP_F32 ? qwhip_gemv_f32(s, w, (const float*)x, m, 0u, 1.0f, logits)
-                                           : qwhip_gemv(s, w, x, x_dtype, m, flags, nullptr, logits);
+                                           : qw_gemv_impl(s, w, x, x_dtype, m, flags, nullptr, logits, m == 1u ? tokens : nullptr, &folded);
     if (st != QWHIP_OK) return st;
+    if (folded) return QWHIP_OK;
     return qwhip_argmax_f32(s, logits, m, w->n, tokens);
 }

@@ -26,7 +26,16 @@ struct qc_params {
     h1_t* y16;
     float* y32;
     uint32_t N, nb, cpr, rotate;
+    unsigned long long* keys;   // NULL, or [gridDim.x]: the workgroup's argmax key (monotone float bits << 32 | ~row) over its rows
 };
+
+// A float's bits made monotone as an unsigned number; NaN -> 0, so it never wins (qw_sortable_f32_u32,
+// Sources/QWMetal/include/qw_fastmath_safe.metalh:21-25).
+__device__ __forceinline__ uint32_t qc_sortable_f32(float x) {
+    const uint32_t u = __float_as_uint(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0u;
+    return (u & 0x80000000u) ? ~u : (u ^ 0x80000000u);
+}
 
 // SETS row sets per workgroup, D blocks in flight per lane, D0 of them issued before the activation prologue.
 // blockDim.x = 32 * cpr * SETS; dynamic LDS = nb * 80 + rows-per-workgroup * cpr * 4 bytes.
@@ -141,13 +150,52 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
         }
     }
     __syncthreads();
-    // 5. fixed-order sum of the chunk partials of each row
+    // 5. fixed-order sum of the chunk partials of each row; with `keys` also the greedy-decoding fold of the reference's
+    // head kernels (qwg_gemv_am_fold4 / qwg_gemv_am_reduce4, Sources/QWMetal/include/qw_gemm_f32_common.metalh:30-58):
+    // larger (monotone bits, ~row) wins, so ties go to the lower row
+    unsigned long long best = 0ull;
     for (uint32_t s = tid; s < nrows; s += blockDim.x) {
         float v = 0.f;
         for (uint32_t c = 0; c < cpr; ++c) v += part[s * cpr + c];
         const uint32_t row = s * G + blockIdx.x;
         if (p.y32) p.y32[row] = v;
         if (p.y16) p.y16[row] = (h1_t)v;
+        const unsigned long long key = ((unsigned long long)qc_sortable_f32(v) << 32) | (uint32_t)~row;
+        best = key > best ? key : best;
+    }
+    if (p.keys) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const unsigned long long other = __shfl_xor(best, o, 64);
+            best = other > best ? other : best;
+        }
+        __syncthreads();                                   // the partial sums are read: their LDS is free
+        unsigned long long* wbest = (unsigned long long*)part;
+        if ((tid & 63u) == 0u) wbest[tid >> 6] = best;
+        __syncthreads();
+        if (tid == 0u) {
+            const uint32_t nwaves = (blockDim.x + 63u) >> 6;
+            for (uint32_t wv = 1; wv < nwaves; ++wv) best = wbest[wv] > best ? wbest[wv] : best;
+            p.keys[blockIdx.x] = best;
+        }
+    }
+}
+
+// Folds the workgroups' keys into the token: one workgroup.
+__global__ __launch_bounds__(256) void qw_col_keys_fin_kernel(const unsigned long long* __restrict__ keys, uint32_t count, int32_t* token) {
+    __shared__ unsigned long long wbest[4];
+    unsigned long long best = 0ull;
+    for (uint32_t i = threadIdx.x; i < count; i += 256u) best = keys[i] > best ? keys[i] : best;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(best, o, 64);
+        best = other > best ? other : best;
+    }
+    if ((threadIdx.x & 63u) == 0u) wbest[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0u) {
+        for (int wv = 1; wv < 4; ++wv) best = wbest[wv] > best ? wbest[wv] : best;
+        *token = (int32_t)~(uint32_t)best;
     }
 }
 
@@ -166,8 +214,11 @@ hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t 
 // `tune`: 0 = automatic (two rows in flight, both issued ahead of the prologue); bits 0..1 pick the prefetch
 // (1 -> two rows, one ahead of the prologue; 2 -> three rows; 3 -> four rows) and bits 2..3 scale the grid
 // (1 -> half, 2 -> double).
+// `keys` (NULL, or room for `keys_cap` entries) + `token`: the head's greedy-decoding fold rides in the epilogue and a second,
+// one-workgroup launch writes *token; a grid larger than keys_cap drops the fold (*folded = false) and the caller folds the logits.
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
-                 float* y32, uint32_t tune, hipError_t* err) {
+                 float* y32, uint32_t tune, hipError_t* err, unsigned long long* keys, uint32_t keys_cap, int32_t* token,
+                 bool* folded) {
     if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
     const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u;
     if (cpr > 32u) return false;
@@ -197,6 +248,9 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     p.nb = nb;
     p.cpr = cpr;
     p.rotate = rotate ? 1u : 0u;
+    const bool fold = keys && token && wgs <= keys_cap && (size_t)rows_per_wg * cpr * 4u >= 8u * waves;
+    p.keys = fold ? keys : nullptr;
+    if (folded) *folded = fold;
     hipError_t e;
     if (x_dtype == QWHIP_F16) {
         e = sets == 4 ? qc_launch<QWHIP_F16, 4>(st, p, wgs, threads, lds, depth)
@@ -206,6 +260,10 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
         e = sets == 4 ? qc_launch<QWHIP_BF16, 4>(st, p, wgs, threads, lds, depth)
           : sets == 2 ? qc_launch<QWHIP_BF16, 2>(st, p, wgs, threads, lds, depth)
                       : qc_launch<QWHIP_BF16, 1>(st, p, wgs, threads, lds, depth);
+    }
+    if (e == hipSuccess && fold) {
+        hipLaunchKernelGGL(qw_col_keys_fin_kernel, dim3(1), dim3(256), 0, st, keys, wgs, token);
+        e = hipGetLastError();
     }
     *err = e;
     return true;

@@ -329,6 +329,48 @@ def test_head_argmax_picks_the_oracles_token(dev, fmt, m):
     assert np.array_equal(tok[clear], np.argmax(ref, axis=1)[clear])
 
 
+@pytest.mark.parametrize("n,k,prerot", [(50021, 1024, False), (151936, 512, True), (4100, 5120, False)])
+def test_head_argmax_fold_inside_the_gemv_epilogue(dev, n, k, prerot):
+    """One row over an HQ4_G32_M5 bank: the fold rides in the GEMV's epilogue (a key per workgroup, then a one-workgroup
+    fold).  The token equals the fold of the logits the same call wrote, and the tie rule holds through it: the winning
+    bank row is copied to a higher and (where there is room) a lower row - equal logits, the lowest of them wins."""
+    from tests import helpers as H
+    fmt = "hq4_g32_m5"
+    blocks, _ = H.make_bank(fmt, n, k, seed=n % 97)
+    x16 = H.make_x(1, k, 17).astype(np.float16)
+    xin = H.x_in_basis(x16, fmt) if prerot else x16
+    flags = qwhip.X_PREROTATED if prerot else 0
+    lib, st = dev.lib, dev.stream.handle
+    bank, xb = dev.put(blocks), dev.put(xin)
+    logits, tok = dev.alloc(n * 4), dev.alloc(256)
+    view = H.view_of(dev, bank, fmt, n, k)
+    qwhip.check(lib.qwhip_head_argmax(st, C.byref(view), xb.ptr, qwhip.F16, 1, flags, logits.ptr, tok.ptr))
+    dev.stream.sync()
+    got = logits.download(np.float32, (1, n))
+    first = int(tok.download(np.int32, (1,))[0])
+    assert first == int(qo.head_argmax(got)[0])
+    # duplicate the winner
+    rows = blocks.reshape(n, -1).copy()
+    lower = first - 3 if first >= 3 else None
+    rows[min(first + 5, n - 1)] = rows[first]
+    if lower is not None:
+        rows[lower] = rows[first]
+    bank2 = dev.put(rows)
+    view2 = H.view_of(dev, bank2, fmt, n, k)
+    qwhip.check(lib.qwhip_head_argmax(st, C.byref(view2), xb.ptr, qwhip.F16, 1, flags, logits.ptr, tok.ptr))
+    dev.stream.sync()
+    got2 = logits.download(np.float32, (1, n))
+    want = lower if lower is not None else first
+    assert got2[0, want] == got2[0, first] == got[0, first]
+    assert int(tok.download(np.int32, (1,))[0]) == want == int(qo.head_argmax(got2)[0])
+    # the standalone fold over the same logits agrees
+    qwhip.check(lib.qwhip_argmax_f32(st, logits.ptr, 1, n, tok.ptr))
+    dev.stream.sync()
+    assert int(tok.download(np.int32, (1,))[0]) == want
+    for b in (bank, bank2, xb, logits, tok):
+        b.free()
+
+
 def test_argmax_rows_whose_maximum_is_a_zero_or_nothing_above_minus_infinity(dev):
     """The rows the fast sweep cannot decide by float compares alone: maximum +-0.0 (the key order puts +0.0 above -0.0, rows in
     either order, also split over threads), only -inf and NaN, and a long row (several chunks per thread) with a late tie."""
