@@ -920,20 +920,14 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
         __syncthreads();
         uint8_t* ep = lds4 + wave * (32u * EP_PITCH);
         const uint32_t w_off = (4u * kh) * EP_PITCH + j * 2u;
+        const qw_fwht32_signs fw_signs = qw_fwht32_lane_signs(j);
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float g = (float)(h1_t)acc[a][0][r], u = (float)(h1_t)acc[a][1][r];
                 float v = qw_swiglu(g, u);
-                if (p.rotate_act) {
-#pragma unroll
-                    for (uint32_t h = 1; h < 32u; h <<= 1) {
-                        const float o = __shfl_xor(v, (int)h, 32);
-                        v = (j & h) == 0u ? v + o : o - v;
-                    }
-                    v *= QW_INV_SQRT32;
-                }
+                if (p.rotate_act) v = qw_fwht32_lanes(v, fw_signs) * QW_INV_SQRT32;
                 *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
             }
 #pragma unroll
@@ -1149,20 +1143,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         constexpr uint32_t EP_PITCH = 64 + 16;
         uint8_t* ep = lds5 + wave * (32u * EP_PITCH);
         const uint32_t w_off = (4u * kh) * EP_PITCH + j * 2u;
+        const qw_fwht32_signs fw_signs = qw_fwht32_lane_signs(j);
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float g = (float)(h1_t)acc[a][0][r], u = (float)(h1_t)acc[a][1][r];
                 float v = qw_swiglu(g, u);
-                if (p.rotate_act) {
-#pragma unroll
-                    for (uint32_t h = 1; h < 32u; h <<= 1) {
-                        const float o = __shfl_xor(v, (int)h, 32);
-                        v = (j & h) == 0u ? v + o : o - v;
-                    }
-                    v *= QW_INV_SQRT32;
-                }
+                if (p.rotate_act) v = qw_fwht32_lanes(v, fw_signs) * QW_INV_SQRT32;
                 *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
             }
 #pragma unroll

@@ -142,6 +142,45 @@ __device__ __forceinline__ void qw_fwht32(float* v) {
 // Sources/QWMetal/include/qw_weight_basis.metalh:50-63).
 __device__ __forceinline__ float qw_swiglu(float g, float u) { return (g / (1.0f + __expf(-g))) * u; }
 
+// FWHT-32 over the 32 lanes of a half wavefront (lane j = lane & 31 holds element j), un-normalised, stage order
+// h = 1, 2, 4, 8, 16 with v' = (j & h) == 0 ? v + o : o - v, o = the value of lane j ^ h: the arithmetic of the butterfly
+// written with lane exchanges through LDS (ds_bpermute), bit for bit, but the partners come by DPP (quad permutes, row
+// mirrors: j ^ 4 = half-mirror then quad-reverse, j ^ 8 = mirror then half-mirror) and, across the two 16-lane rows, by
+// v_permlane16_swap_b32 - no LDS round trip per stage.  `sg[t]` = (j & (1 << t)) ? -1 : +1.
+struct qw_fwht32_signs {
+    float sg[5];
+    bool odd_row;
+};
+__device__ __forceinline__ qw_fwht32_signs qw_fwht32_lane_signs(uint32_t lane) {
+    qw_fwht32_signs s;
+#pragma unroll
+    for (int t = 0; t < 5; ++t) s.sg[t] = (lane & (1u << t)) ? -1.0f : 1.0f;
+    s.odd_row = (lane & 16u) != 0u;
+    return s;
+}
+#define QW_DPP_F32(v, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true))
+__device__ __forceinline__ float qw_fwht32_lanes(float v, const qw_fwht32_signs& s) {
+    v = QW_DPP_F32(v, 0xB1) + s.sg[0] * v;                       // quad_perm [1,0,3,2]: lane ^ 1
+    v = QW_DPP_F32(v, 0x4E) + s.sg[1] * v;                       // quad_perm [2,3,0,1]: lane ^ 2
+    {
+        const float m = QW_DPP_F32(v, 0x141);                    // row_half_mirror: lane ^ 7
+        v = QW_DPP_F32(m, 0x1B) + s.sg[2] * v;                   // quad_perm [3,2,1,0]: ^ 3 -> lane ^ 4
+    }
+    {
+        const float m = QW_DPP_F32(v, 0x140);                    // row_mirror: lane ^ 15
+        v = QW_DPP_F32(m, 0x141) + s.sg[3] * v;                  // row_half_mirror: ^ 7 -> lane ^ 8
+    }
+    {
+        // (the compiler's builtin for this instruction returns its first result twice: written out)
+        float a = v, b = v;
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        // a = rows (0, 0, 2, 2) of v, b = rows (1, 1, 3, 3): the partner row is b for an even row, a for an odd one
+        const float o = s.odd_row ? a : b;
+        v = o + s.sg[4] * v;
+    }
+    return v;
+}
+
 // A constant pinned in a VGPR (v_and_or_b32 is VOP3: on gfx9 it takes no literal and one scalar operand,
 // so one of mask / magic has to live in a vector register to get the single-instruction form).
 __device__ __forceinline__ uint32_t qw_vgpr_const(uint32_t c) {
