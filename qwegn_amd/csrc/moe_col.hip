@@ -159,23 +159,19 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
         }
     }
     __syncthreads();
-    if (tid < 32u) {
+    if (tid < 64u) {
+        // the whole first wave runs the transform (its upper half repeats the lower half's outputs: the cross-row exchange
+        // wants every row of the wave live); the lower half stores
+        const uint32_t o32 = tid & 31u;
         float gsum = 0.f, usum = 0.f;
         for (uint32_t c = 0; c < cpr; ++c) {
-            gsum += part[tid * cpr + c];
-            usum += part[(32u + tid) * cpr + c];
+            gsum += part[o32 * cpr + c];
+            usum += part[(32u + o32) * cpr + c];
         }
         float a = qw_swiglu(gsum, usum);
-        if (p.rot_out && n0 + 32u <= I) {
-            // the butterfly order of the serial transform (pairs h apart: lower = a + b, upper = a - b), across lanes
-#pragma unroll
-            for (int h = 1; h < 32; h <<= 1) {
-                const float o = __shfl_xor(a, h, 64);
-                a = (tid & (uint32_t)h) ? o - a : a + o;
-            }
-            a *= QW_INV_SQRT32;
-        }
-        if (n0 + tid < I) act[n0 + tid] = (h1_t)a;
+        // the butterfly order of the serial transform (pairs h apart: lower = a + b, upper = a - b), across lanes by DPP
+        if (p.rot_out && n0 + 32u <= I) a = qw_fwht32_lanes(a, qw_fwht32_lane_signs(o32)) * QW_INV_SQRT32;
+        if (tid < 32u && n0 + tid < I) act[n0 + tid] = (h1_t)a;
     }
 }
 
