@@ -201,12 +201,7 @@ __global__ __launch_bounds__(256) void qw_h32_f32_kernel(const float* x, float* 
     if (col >= padded) return;   // padded is a multiple of 32: whole 32-lane groups leave together
     const uint64_t at = (uint64_t)blockIdx.y * hidden + col;
     float v = col < hidden ? x[at] : 0.0f;
-    const uint32_t l = threadIdx.x & 31u;
-#pragma unroll
-    for (uint32_t s = 1; s < 32u; s <<= 1) {
-        const float o = __shfl_xor(v, (int)s, 32);
-        v = (l & s) == 0u ? v + o : o - v;
-    }
+    v = qw_fwht32_lanes(v, qw_fwht32_lane_signs(threadIdx.x & 31u));   // the same stages and sums, partners by DPP
     if (col < hidden) out[at] = v * 0.17677669529663689f;
 }
 
