@@ -288,6 +288,31 @@ public enum QWGemm {
         try hal.pipeline("qwg_add_f32")
         try qwCheck(qwhip_add_f32(enc.stream, a.f32, b.f32, out.f32, UInt64(count)))
     }
+    /// QWGemm.encodeLatentNormH32F32 (QWGemmF32.swift:57-80): optional RMSNorm (1 + gamma) + H_32 on f32 rows -> f32 and / or f16.
+    public static func encodeLatentNormH32F32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, gamma: QWTensorValue?, out32: QWTensorValue?,
+                                              out16: QWTensorValue?, rows: Int, latent: Int, eps: Float = 1e-6) throws {
+        guard latent > 0, latent % 32 == 0, out32 != nil || out16 != nil else { throw QWGemmError.badShape("latent norm H32: latent % 32 == 0, one output") }
+        try hal.pipeline("qwg_latent_norm_h32_f32")
+        try qwCheck(qwhip_latent_norm_h32_f32(enc.stream, x.f32, gamma?.ptr, out32?.f32, out16?.ptr, UInt32(rows), UInt32(latent), eps))
+    }
+    /// QWGemm.encodeMoEBridgeF16ToF32 (QWGemmMoE.swift:337-377): f16 normed hidden -> rotated f32 copy + un-rotated f32 copy.
+    public static func encodeMoEBridgeF16ToF32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, xRot32: QWTensorValue?, xPlain32: QWTensorValue,
+                                               rows: Int, hidden: Int) throws {
+        guard hidden % 256 == 0 else { throw QWGemmError.badGeometry("moe bridge: hidden must be a multiple of 256") }
+        try hal.pipeline("qwg_moe_bridge_f16_to_f32")
+        try qwCheck(qwhip_moe_bridge_f16_to_f32(enc.stream, x.ptr, xRot32?.f32, xPlain32.f32, UInt32(rows), UInt32(hidden)))
+    }
+    /// QWGemm.encodeDenseProjF32 (QWGemmF32.swift:413-440): f32 rows in the container's basis -> f32 outputs; 64 rows and more without
+    /// an epilogue go through one cast and the f16 GEMM, fewer through the f32 door (its batched matrix-core form from 32 rows on).
+    public static func encodeDenseProjF32(_ enc: QWHipEncoder, hal: QWHal, weight: QWWeightView, x: QWTensorValue, y: QWTensorValue,
+                                          naxX16: QWTensorValue, rows: Int, epilogue: Int = 0, scale: Float = 1) throws {
+        if rows >= 64, epilogue == 0, scale == 1, weight.n % 64 == 0, weight.k % 64 == 0, naxX16.elementCount >= rows * weight.k {
+            try encodeCast(enc, hal: hal, src32: x, dst16: naxX16, count: rows * weight.k)
+            try gemmBatchedH16(enc, hal: hal, x: naxX16, w: weight, y: y, rows: rows)
+        } else {
+            try encodeHQ4F32V4(enc, hal: hal, weight: weight, x: x, y: y, rows: rows, epilogue: epilogue, scale: scale)
+        }
+    }
 
     // ---- MoE doors (QWGemmMoE.swift, QWGemmMoERouter.swift) -------------------------------------------------------
     public static func moeMaxTiles(experts: Int, pairs: Int) -> Int { Int(qwhip_moe_max_tiles(UInt32(experts), UInt32(pairs))) }   // QWGemmMoE.swift:24-26
@@ -352,6 +377,21 @@ public enum QWGemm {
         try hal.pipeline("qwg_moe_down_reduce_combine_f32")
         try qwCheck(qwhip_moe_combine(enc.stream, dnAcc.ptr, dnAcc.dtype.rawValue, invPerm.i32, weights.f32, UInt32(tokens), UInt32(routes),
                                       UInt32(hidden), shared?.f32, gate?.f32, out.ptr, out.dtype.rawValue))
+    }
+    /// The same door with invPerm: nil and unweightedSingle (QWGemmMoE.swift:299-332): out = dnAcc + gate * shared, one row per token.
+    public static func encodeMoEAddSharedF32(_ enc: QWHipEncoder, hal: QWHal, dnAcc: QWTensorValue, shared: QWTensorValue, gate: QWTensorValue?,
+                                             out: QWTensorValue, hidden: Int, tokens: Int) throws {
+        try hal.pipeline("qwg_moe_down_reduce_combine_f32")
+        try qwCheck(qwhip_moe_combine(enc.stream, dnAcc.ptr, dnAcc.dtype.rawValue, nil, nil, UInt32(tokens), 1, UInt32(hidden), shared.f32, gate?.f32,
+                                      out.ptr, out.dtype.rawValue))
+    }
+    /// encodeMoEGateUpF32R1 with fuseSiluFwht (QWGemmMoE.swift:120-155): routed gate_up with the ids given.
+    public static func encodeMoEGateUpF32R1(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, experts: Int, ids: QWTensorValue,
+                                            out: QWTensorValue, routes: Int, tokens: Int, xIsRotated: Bool = true) throws {
+        try hal.pipeline(bank.isIncumbent ? "qwg_moe_gateup_q4g_f32_r1" : "qwg_moe_gateup_aq\(bank.bits)_g\(bank.groupSize)_f32_r1")
+        var w = bank.abi
+        try qwCheck(qwhip_moe_gateup_decode(enc.stream, &w, UInt32(experts), x.ptr, x.dtype.rawValue, xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0,
+                                            ids.i32, UInt32(tokens), UInt32(routes), out.ptr))
     }
     /// encodeMoEGateUpF32R1 with fuseSiluFwht (QWGemmMoE.swift:120-155), routing folded into the launch for an HQ4_G32_M5 bank.
     public static func encodeMoERouteGateUp(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, experts: Int,
@@ -481,6 +521,81 @@ public enum QWMoEOperator {
                                             routes: K, tokens: T, normTopK: w.normTopK, routedScale: w.routedScale)
             try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: s.act16, bank: w.down, experts: E, routes: K, weights: s.wts, shared: shared,
                                                      gate: sharedGate, out: out32, ids: s.idx, tokens: T)
+        }
+    }
+
+    // ---- latent-bottleneck sparse MoE (QWMoEOperator+Latent.swift:17-303) ------------------------------------------------
+    public struct LatentBottleneck {
+        public let fc1: QWWeightView           // n = latentDim, k = hidden
+        public let fc2: QWWeightView           // n = hidden, k = latentDim
+        public let normGamma: QWTensorValue?   // f16 [latentDim], plus-one law
+        public let normEps: Float
+        public let latentDim: Int
+    }
+    public struct LatentWeights {
+        public let routed: Weights             // gateUp: k = latentDim; down: n = experts * latentDim
+        public let sharedGateUp: QWWeightView?, sharedDown: QWWeightView?
+        public let sharedGateScalar: QWTensorValue?      // f32 [hidden]
+        public let sharedIntermediate: Int
+        public let routerBias: QWTensorValue?, routedScaleParam: QWTensorValue?
+        public let splitFeatureRouting: Bool
+    }
+    public struct LatentScratch {
+        public let xRot32, xPlain32: QWTensorValue       // f32 [rows, hidden]
+        public let bufA32, bufB32: QWTensorValue         // f32 [rows, latentDim]
+        public let bufB16: QWTensorValue                 // f16 [rows, latentDim]
+        public let naxX16: QWTensorValue                 // f16 staging of the dense projections
+        public let gate: QWTensorValue                   // f32 [rows]
+        public let guSh32, actSh32, shared: QWTensorValue
+    }
+    /// fc1 -> route -> rotate -> routed experts in the latent width -> latent norm -> fc2, the shared expert on the hidden width
+    /// added under its gate.  x16: the operator's .f16Normed input.
+    public static func encodeResidentLatent(_ enc: QWHipEncoder, hal: QWHal, weights lw: LatentWeights, latent: LatentBottleneck, scratch s: Scratch,
+                                            latentScratch ls: LatentScratch, x16: QWTensorValue, out32: QWTensorValue, rows T: Int) throws {
+        let w = lw.routed
+        let (H, L, E, K, I, ISh) = (w.hidden, latent.latentDim, w.experts, w.topK, w.intermediate, lw.sharedIntermediate)
+        guard L > 0, L % 32 == 0, latent.fc1.n == L, latent.fc1.k == H, latent.fc2.n == H, latent.fc2.k == L,
+              w.gateUp.n == E * 2 * I, w.gateUp.k == L, w.down.n == E * L, w.down.k == I else {
+            throw QWGemmError.badShape("latent moe: banks do not match (hidden, latent, experts, intermediate)")
+        }
+        let routerCols = lw.splitFeatureRouting ? 2 * E : E
+        try QWGemm.encodeMoEBridgeF16ToF32(enc, hal: hal, x: x16, xRot32: ls.xRot32, xPlain32: ls.xPlain32, rows: T, hidden: H)
+        let sharedBanks: (QWWeightView, QWWeightView)? = (ISh > 0 && lw.sharedGateUp != nil && lw.sharedDown != nil) ? (lw.sharedGateUp!, lw.sharedDown!) : nil
+        let gateW = sharedBanks != nil ? lw.sharedGateScalar : nil
+        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: ls.xPlain32, y: s.logits, rows: T, n: routerCols, k: H,
+                                      shGateWeight: gateW, shGateOut: gateW != nil ? ls.gate : nil)
+        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: latent.fc1, x: ls.xRot32, y: ls.bufA32, naxX16: ls.naxX16, rows: T)
+        try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
+                                    routedScale: w.routedScale, bias: lw.routerBias, splitFeature: lw.splitFeatureRouting,
+                                    routedScaleParam: lw.routedScaleParam)
+        try QWGemm.encodeLatentNormH32F32(enc, hal: hal, x: ls.bufA32, gamma: nil, out32: nil, out16: ls.bufB16, rows: T, latent: L, eps: latent.normEps)
+        if let (shGU, shDown) = sharedBanks {
+            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shGU, x: ls.xRot32, y: ls.guSh32, naxX16: ls.naxX16, rows: T)
+            try QWGemm.encodeSiluMulF32(enc, hal: hal, gu: ls.guSh32, act: ls.actSh32, rows: T, inter: ISh)
+            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shDown, x: ls.actSh32, y: ls.shared, naxX16: ls.naxX16, rows: T)
+        }
+        let pairs = T * K
+        if T > 8, let expOff = s.expOff, let sortedPair = s.sortedPair, let sortedTok = s.sortedTok, let invPerm = s.invPerm,
+           let tileE = s.tileE, let tileR = s.tileR, let tileCount = s.tileCount, let dnHi = s.dnHi, L % 64 == 0, I % 64 == 0 {
+            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: expOff, sortedPairIdx: sortedPair, sortedTok: sortedTok, experts: E,
+                                              totalPairs: pairs, routes: K, invPerm: invPerm, tileE: tileE, tileR: tileR, tileCount: tileCount)
+            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: ls.bufB16, bank: w.gateUp, experts: E, sortedTok: sortedTok, expertOff: expOff, tileE: tileE,
+                                             tileR: tileR, tileCount: tileCount, act16: s.act16, pairs: pairs, rotateAct: w.down.isRotated)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: s.act16, bank: w.down, experts: E, expertOff: expOff, tileE: tileE, tileR: tileR,
+                                            tileCount: tileCount, y: dnHi, pairs: pairs)
+            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: dnHi, invPerm: invPerm, weights: s.wts, shared: nil, gate: nil,
+                                                     out: ls.bufA32, hidden: L, routes: K, tokens: T)
+        } else {
+            try QWGemm.encodeMoEGateUpF32R1(enc, hal: hal, x: ls.bufB16, bank: w.gateUp, experts: E, ids: s.idx, out: s.act16, routes: K, tokens: T)
+            try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: s.act16, bank: w.down, experts: E, routes: K, weights: s.wts, shared: nil,
+                                                     gate: nil, out: ls.bufA32, ids: s.idx, tokens: T)
+        }
+        try QWGemm.encodeLatentNormH32F32(enc, hal: hal, x: ls.bufA32, gamma: latent.normGamma, out32: ls.bufB32, out16: nil, rows: T, latent: L,
+                                          eps: latent.normEps)
+        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: latent.fc2, x: ls.bufB32, y: out32, naxX16: ls.naxX16, rows: T)
+        if sharedBanks != nil {
+            try QWGemm.encodeMoEAddSharedF32(enc, hal: hal, dnAcc: out32, shared: ls.shared, gate: gateW != nil ? ls.gate : nil, out: out32, hidden: H,
+                                             tokens: T)
         }
     }
 }
