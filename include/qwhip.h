@@ -381,6 +381,47 @@ qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_
                                    uint32_t top_k, const float* shared, const float* shared_gate, void* out,
                                    uint32_t out_dtype);
 
+/* ---- group-latent MoE (QWMoEOperator.encodeResidentGroupLatent, Sources/Operators/QWGEMM/QWMoEOperator+GroupLatent.swift:11-294)
+ * Every expert carries the label of one of num_groups (1..32) latent groups.  A token's routes read D_g . x of their
+ * expert's group (bank latentD [num_groups * latent, hidden]), run the expert in the latent width, are summed by group
+ * with their route weights, and the groups' sums go up through U_g (bank latentU [num_groups * hidden, latent]) and are
+ * added.  The reference carries the group in the high bits of its route ids (qwg_moe_route with latentLabels,
+ * Sources/QWMetal/subsystems/qwrouter.metal:135-165); here the route ids stay plain and the group rules are these doors. */
+
+/* group_ids [t, num_groups] = g where one of the token's routes has labels[idx] == g, else -1 (qwrouter.metal:163-165);
+ * pair_rows [t, top_k] (may be NULL) = t * num_groups + labels[idx[t, k]], the row of route k's latent in a [t, num_groups]
+ * matrix, -1 for an absent route.  labels: i32 [experts]. */
+qwhip_status qwhip_moe_latent_groups(qwhip_stream_t s, const int32_t* idx, const int32_t* labels, uint32_t t, uint32_t top_k,
+                                     uint32_t experts, uint32_t num_groups, int32_t* group_ids, int32_t* pair_rows);
+/* The routed projection without the sum over routes (encodeMoEDownSharedCombineF32 with routeOutput and tokenIndexedX,
+ * QWGemmMoE.swift:157-199): out [t, top_k, n / experts] = wts[t, r] * W[idx[t, r]] . x_row, zeros where idx < 0.
+ * x16: f16 [t, k] when x_per_token != 0 (all routes of a token read its one row), else [t, top_k, k].  wts NULL = 1. */
+qwhip_status qwhip_moe_routed_gemv(qwhip_stream_t s, const qwhip_weight_view* w, uint32_t experts, const void* x16,
+                                   uint32_t x_per_token, const int32_t* idx, const float* wts, uint32_t t, uint32_t top_k,
+                                   void* out, uint32_t out_dtype);
+/* qwhip_moe_gateup_decode with the activation row of every (token, route) pair given: pair p reads x row x_rows[p]
+ * (the reference's packed ids make its gate_up kernel read row token * numGroups + group of xLatent32). */
+qwhip_status qwhip_moe_gateup_decode_rows(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                          const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx,
+                                          const int32_t* x_rows, uint32_t t, uint32_t top_k, void* act16);
+/* The routed down projection summed by group (encodeMoEDownSharedCombineF32 with numGroups, QWGemmMoE.swift:157-199):
+ * out [t, num_groups, n / experts] = sum over routes r with labels[idx[t, r]] == g of wts[t, r] * Wd[idx[t, r]] . act16[t, r],
+ * zeros for a group without routes. */
+qwhip_status qwhip_moe_down_decode_groups(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts,
+                                          const void* act16, const int32_t* idx, const float* wts, const int32_t* labels,
+                                          uint32_t num_groups, uint32_t t, uint32_t top_k, void* out, uint32_t out_dtype);
+/* Prefill: rows_out[p] = slot_of_row[pair_rows[sorted_pair[p]]] for the `pairs` positions of an expert-sorted pair list:
+ * the gather rows of a grouped GEMM whose activations are the (sorted) output of an earlier grouped GEMM over n_rows
+ * (token, group) rows, slot_of_row being that sort's inv_perm (NULL = the rows are in place). */
+qwhip_status qwhip_moe_compose_rows(qwhip_stream_t s, const int32_t* sorted_pair, uint32_t pairs, const int32_t* pair_rows,
+                                    uint32_t n_rows, const int32_t* slot_of_row, int32_t* rows_out);
+/* qwhip_moe_combine summed by group (encodeMoEDownReduceCombineF32 with numGroups, QWGemmMoE.swift:299-332;
+ * qwgemm_moe_nax_f16.metal:51-111): out [t, num_groups, width] = sum over routes k with labels[idx[t, k]] == g of
+ * wts[t, k] * dn[inv_perm[t * top_k + k], :], zeros for a group without routes.  inv_perm / wts NULL as in qwhip_moe_combine. */
+qwhip_status qwhip_moe_combine_groups(qwhip_stream_t s, const void* dn, uint32_t dn_dtype, const int32_t* inv_perm,
+                                      const float* wts, const int32_t* idx, const int32_t* labels, uint32_t t, uint32_t top_k,
+                                      uint32_t num_groups, uint32_t width, void* out, uint32_t out_dtype);
+
 /* ---- load-time writer (the step before the path) ----------------------------- */
 /* qwg_quantize_bf16_to_hq4_g32_m5 (Sources/QWMetal/quant/qw_online_quant.metal:17-55), GPU twin of
  * quant_hq4_blocks (Scripts/quantize/hq4.py:54-123): src [n, k] bf16 or f32 -> 20-byte blocks. */

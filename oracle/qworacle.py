@@ -783,3 +783,66 @@ def moe_forward_f64(x, idx, wts, gate_up_w, down_w, act_f16: bool, rotate_act: b
                 act = a32.astype(np.float16).astype(np.float64)
             out[r] += float(wts[r, k]) * (down_w[ex].astype(np.float64) @ act)
     return out
+
+
+# --------------------------------------------------------------------------- #
+# group-latent routed MoE block  (no golden in the reference: pinned by the identities of tests/test_oracle_math.py -
+# one identity group reduces it to moe_forward_f64, and the per-route expansion by linearity of U_g)
+# --------------------------------------------------------------------------- #
+def moe_latent_groups(idx: np.ndarray, labels: np.ndarray, num_groups: int):
+    """group_ids [t, NG] = g where a route of the token carries label g, else -1; pair_rows [t, k] = t * NG + label of
+    the route, -1 for an absent route (activeMask / groupIds, Sources/QWMetal/subsystems/qwrouter.metal:135-165)."""
+    idx = np.asarray(idx)
+    t, k = idx.shape
+    gids = np.full((t, num_groups), -1, dtype=np.int32)
+    rows = np.full((t, k), -1, dtype=np.int32)
+    for r in range(t):
+        for j in range(k):
+            e = int(idx[r, j])
+            if e < 0:
+                continue
+            g = int(labels[e & 0xFFFF])
+            if 0 <= g < num_groups:
+                gids[r, g] = g
+                rows[r, j] = r * num_groups + g
+    return gids, rows
+
+
+def moe_group_latent_forward_f64(x, idx, wts, labels, latent_d_w, gate_up_w, down_w, latent_u_w, act_f16: bool = True,
+                                 rotate_act: bool = True, latent_f16: bool = True):
+    """out[t] = sum over active groups g of U_g . z_g,  z_g = sum over the token's routes k with labels[e_k] == g of
+    wts[t, k] * W_down[e_k] . SwiGLU(W_gu[e_k] . (D_g . x[t]))
+    (FNSparseMoE.forward, Tests/QWFlashNextTests/Reference/FNSparseMoE.swift:113-139).
+
+    latent_d_w [NG, L, H], gate_up_w [E, 2I, L], down_w [E, L, I], latent_u_w [NG, H, L]: dequantized weights in the
+    basis the kernels contract them in.  latent_f16 rounds D_g . x and z_g to f16, as the kernels hand them on; act_f16 /
+    rotate_act as in moe_forward_f64.  All products in fp64."""
+    x = np.asarray(x, dtype=np.float64)
+    t = x.shape[0]
+    ng, lat, _ = latent_d_w.shape
+    i = gate_up_w.shape[1] // 2
+    out = np.zeros((t, latent_u_w.shape[1]), dtype=np.float64)
+    r16 = (lambda v: v.astype(np.float32).astype(np.float16).astype(np.float64)) if latent_f16 else (lambda v: v)
+    for r in range(t):
+        z = np.zeros((ng, lat), dtype=np.float64)
+        xin = {}
+        for k in range(idx.shape[1]):
+            e = int(idx[r, k])
+            if e < 0:
+                continue
+            e &= 0xFFFF
+            g = int(labels[e])
+            if g not in xin:
+                xin[g] = r16(latent_d_w[g].astype(np.float64) @ x[r])
+            gu = gate_up_w[e].astype(np.float64) @ xin[g]
+            gt, up = gu[:i], gu[i:]
+            act = gt / (1.0 + np.exp(-gt)) * up
+            if act_f16:
+                a32 = act.astype(np.float32)
+                if rotate_act and i % 32 == 0:
+                    a32 = fwht32_ortho(a32)
+                act = a32.astype(np.float16).astype(np.float64)
+            z[g] += float(wts[r, k]) * (down_w[e].astype(np.float64) @ act)
+        for g in xin:
+            out[r] += latent_u_w[g].astype(np.float64) @ r16(z[g])
+    return out

@@ -371,6 +371,10 @@ struct qw_gemv_params {
     const float* shared;
     const float* shared_gate;
     void* out;
+    const int32_t* x_rows;  // gate|up: activation row of every pair (NULL: the pair's token)
+    uint32_t x_div;         // down: pairs that share one activation row (0 and 1: a row per pair)
+    const int32_t* labels;  // down, num_groups > 0: group of every expert; blockIdx.y = token * num_groups + group and
+    uint32_t num_groups;    // only the token's routes into that group are summed
     // transposing kernel: waves per row set, row sets per workgroup, K ranges
     uint32_t wpr, sets, nkr;
 };
@@ -404,7 +408,8 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_pa
         const uint32_t pair = blockIdx.y;
         e = p.idx[pair];
         y16 += (uint64_t)pair * N;
-        x = (const uint8_t*)x + (uint64_t)(pair / p.top_k) * K * 2u;
+        const uint32_t xrow = p.x_rows ? (uint32_t)max(p.x_rows[pair], 0) : pair / p.top_k;
+        x = (const uint8_t*)x + (uint64_t)xrow * K * 2u;
     }
     if constexpr (XM == QW_XM_LDS_ROT) {
         for (uint32_t idx = tid; idx < M * nsl; idx += NTH) {
@@ -507,16 +512,19 @@ __global__ __launch_bounds__(512) void qw_moe_down_decode_kernel(const qw_gemv_p
     const uint32_t i = lane & 15u, c = lane >> 4;
     const uint32_t N = p.N, K = p.K;
     const uint32_t n0 = blockIdx.x * (16u * RT);
-    const uint32_t tok = blockIdx.y;
+    const uint32_t tok = blockIdx.y;   // the output row
+    const uint32_t src = p.num_groups ? tok / p.num_groups : tok;
+    const int32_t grp = p.num_groups ? (int32_t)(tok - src * p.num_groups) : 0;
     const uint32_t magic = qw_vgpr_const(0x64006400u);
     f4_t total[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) total[t] = f4_t{0.f, 0.f, 0.f, 0.f};
     for (uint32_t k = wave; k < p.top_k; k += 8u) {
-        const uint32_t pair = tok * p.top_k + k;
+        const uint32_t pair = src * p.top_k + k;
         const int32_t e = p.idx[pair];
         if (e < 0) continue;
-        const float wk = p.wts[pair];
+        if (p.num_groups && p.labels[(uint32_t)e & 0xFFFFu] != grp) continue;
+        const float wk = p.wts ? p.wts[pair] : 1.0f;
         const uint8_t* bank = p.bank + (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
         const uint8_t* rp[RT];
 #pragma unroll
@@ -528,7 +536,7 @@ __global__ __launch_bounds__(512) void qw_moe_down_decode_kernel(const qw_gemv_p
         f4_t acc[RT];
 #pragma unroll
         for (int t = 0; t < RT; ++t) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
-        const void* x = (const uint8_t*)p.x + (uint64_t)pair * K * 2u;
+        const void* x = (const uint8_t*)p.x + (uint64_t)(p.x_div > 1u ? pair / p.x_div : pair) * K * 2u;
         qw_stream_rows<FMT, RT, QWHIP_F16, QW_XM_GLOBAL>(rp, x, nullptr, 0, K, 1, p.gshift, p.bb, false, 0u, i, c, magic, acc, 1u);
 #pragma unroll
         for (int t = 0; t < RT; ++t) total[t] += acc[t] * wk;
@@ -960,10 +968,11 @@ bool qw_stream_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, u
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
                        bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
                        const float* logits = nullptr, int32_t* idx_out = nullptr, float* wts_out = nullptr, uint32_t norm_topk = 0,
-                       float routed_scale = 1.0f);
+                       float routed_scale = 1.0f, const int32_t* x_rows = nullptr);
 bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* act16, const int32_t* idx,
                      const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
-                     uint32_t out_dtype, hipError_t* err);
+                     uint32_t out_dtype, hipError_t* err, uint32_t x_div = 1, const int32_t* labels = nullptr,
+                     uint32_t num_groups = 0);
 
 // gemv_quad.hip
 bool qw_quad_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
@@ -1236,9 +1245,10 @@ extern "C" qwhip_status qwhip_moe_route_gateup_decode(qwhip_stream_t s, const qw
 }
 
 // ---- MoE decode / verify (t <= 8): routed experts as GEMVs -----------------------------------------
-extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
-                                                const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
-                                                uint32_t top_k, void* act16) {
+// x_rows: the activation row of every (token, route) pair; NULL = the pair's token.
+static qwhip_status qw_moe_gateup_decode_impl(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts, const void* x,
+                                              uint32_t x_dtype, uint32_t flags, const int32_t* idx, const int32_t* x_rows, uint32_t t,
+                                              uint32_t top_k, void* act16) {
     int fmt = 0;
     qwhip_status st = check_common(s, w_gate_up, x, x_dtype, 1, &fmt);
     if (st != QWHIP_OK) return st;
@@ -1254,7 +1264,7 @@ extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_we
     if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
         hipError_t e = hipSuccess;
         if (qw_moe_gateup_col(s->stream, w_gate_up, experts, x, x_dtype, rotate, qwhip_view_rotated(w_gate_up) && inter % 32 == 0,
-                              idx, t * top_k, top_k, act16, &e)) {
+                              idx, t * top_k, top_k, act16, &e, nullptr, nullptr, nullptr, 0, 1.0f, x_rows)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }
@@ -1272,6 +1282,7 @@ extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_we
     a.rotate = rotate ? 1u : 0u;
     a.rot_out = (qwhip_view_rotated(w_gate_up) && inter % 32 == 0) ? 1u : 0u;
     a.idx = idx;
+    a.x_rows = x_rows;
     a.top_k = top_k;
     a.expert_bytes = (uint64_t)2 * inter * a.row_bytes;
     const size_t lds_x = (size_t)w_gate_up->k * 2u + 16u;
@@ -1290,24 +1301,42 @@ extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_we
     return QWHIP_OK;
 }
 
-extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts,
-                                              const void* act16, const int32_t* idx, const float* wts, uint32_t t, uint32_t top_k,
-                                              const float* shared, const float* shared_gate, void* out, uint32_t out_dtype) {
+extern "C" qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                                const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
+                                                uint32_t top_k, void* act16) {
+    return qw_moe_gateup_decode_impl(s, w_gate_up, experts, x, x_dtype, flags, idx, nullptr, t, top_k, act16);
+}
+
+extern "C" qwhip_status qwhip_moe_gateup_decode_rows(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
+                                                     const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx,
+                                                     const int32_t* x_rows, uint32_t t, uint32_t top_k, void* act16) {
+    QWHIP_REQUIRE(x_rows);
+    return qw_moe_gateup_decode_impl(s, w_gate_up, experts, x, x_dtype, flags, idx, x_rows, t, top_k, act16);
+}
+
+// The routed down projection in its three shapes.  rows = output rows (grid.y): tokens, (token, route) pairs with top_k = 1
+// and x_div pairs per activation row, or (token, group) pairs with num_groups > 0 (then only the routes whose expert carries
+// that group's label are summed).  wts NULL = unit weights.
+static qwhip_status qw_moe_down_decode_impl(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts, const void* act16,
+                                            const int32_t* idx, const float* wts, uint32_t t, uint32_t top_k, const float* shared,
+                                            const float* shared_gate, void* out, uint32_t out_dtype, uint32_t x_div,
+                                            const int32_t* labels, uint32_t num_groups) {
     int fmt = 0;
     qwhip_status st = check_common(s, w_down, act16, QWHIP_F16, 1, &fmt);
     if (st != QWHIP_OK) return st;
     QWHIP_REQUIRE(idx);
-    QWHIP_REQUIRE(wts);
     QWHIP_REQUIRE(out);
     if (t == 0 || top_k == 0) return QWHIP_OK;
     if (experts == 0 || experts > 512 || w_down->n % experts != 0)
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "down bank of %u rows does not split over %u experts", w_down->n, experts);
-    if (t > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "decode path holds at most 65535 tokens");
+    const uint64_t out_rows = (uint64_t)t * (num_groups ? num_groups : 1u);
+    if (out_rows > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "decode path holds at most 65535 output rows");
     if ((w_down->k * 2u) % 16u != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "activation rows must be 16-byte multiples");
     const uint32_t hidden = w_down->n / experts;
     if (fmt == QW_FMT_M5) {
         hipError_t e = hipSuccess;
-        if (qw_moe_down_col(s->stream, w_down, experts, act16, idx, wts, t, top_k, shared, shared_gate, out, out_dtype, &e)) {
+        if (qw_moe_down_col(s->stream, w_down, experts, act16, idx, wts, t, top_k, shared, shared_gate, out, out_dtype, &e, x_div, labels,
+                            num_groups)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }
@@ -1328,8 +1357,11 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
     a.shared = shared;
     a.shared_gate = shared_gate;
     a.out = out;
+    a.x_div = x_div;
+    a.labels = labels;
+    a.num_groups = num_groups;
     const dim3 grid(qwhip_cdiv(hidden, 16u)), block(512);
-    const dim3 g2(grid.x, t);
+    const dim3 g2(grid.x, (uint32_t)out_rows);
 #define QW_DD(F, OD) hipLaunchKernelGGL((qw_moe_down_decode_kernel<F, 1, OD>), g2, block, 0, s->stream, a)
 #define QW_DD_O(F)                                                                                          \
     switch (out_dtype) {                                                                                    \
@@ -1344,6 +1376,32 @@ extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weig
 #undef QW_DD
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
+}
+
+extern "C" qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts,
+                                              const void* act16, const int32_t* idx, const float* wts, uint32_t t, uint32_t top_k,
+                                              const float* shared, const float* shared_gate, void* out, uint32_t out_dtype) {
+    return qw_moe_down_decode_impl(s, w_down, experts, act16, idx, wts, t, top_k, shared, shared_gate, out, out_dtype, 1u, nullptr, 0u);
+}
+
+// out[t, r, :] = wts[t, r] * W[idx[t, r]] . x_row, one output row per route (zeros where idx < 0): the routed projection
+// without the sum over routes.
+extern "C" qwhip_status qwhip_moe_routed_gemv(qwhip_stream_t s, const qwhip_weight_view* w, uint32_t experts, const void* x16,
+                                              uint32_t x_per_token, const int32_t* idx, const float* wts, uint32_t t, uint32_t top_k,
+                                              void* out, uint32_t out_dtype) {
+    if ((uint64_t)t * top_k > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "decode path holds at most 65535 (token, route) pairs");
+    return qw_moe_down_decode_impl(s, w, experts, x16, idx, wts, t * top_k, 1u, nullptr, nullptr, out, out_dtype,
+                                   x_per_token ? top_k : 1u, nullptr, 0u);
+}
+
+// out[t, g, :] = sum over the routes r of token t with labels[idx[t, r]] == g of wts[t, r] * W_down[idx[t, r]] . act16[t, r, :]
+// (zeros for a group none of the token's routes falls into).
+extern "C" qwhip_status qwhip_moe_down_decode_groups(qwhip_stream_t s, const qwhip_weight_view* w_down, uint32_t experts,
+                                                     const void* act16, const int32_t* idx, const float* wts, const int32_t* labels,
+                                                     uint32_t num_groups, uint32_t t, uint32_t top_k, void* out, uint32_t out_dtype) {
+    QWHIP_REQUIRE(labels);
+    if (num_groups == 0 || num_groups > 32u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent groups must be 1..32, got %u", num_groups);
+    return qw_moe_down_decode_impl(s, w_down, experts, act16, idx, wts, t, top_k, nullptr, nullptr, out, out_dtype, 1u, labels, num_groups);
 }
 
 // gemv_f32.hip

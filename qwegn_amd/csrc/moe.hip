@@ -504,3 +504,159 @@ extern "C" qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// Group-latent MoE (QWMoEOperator.encodeResidentGroupLatent, Sources/Operators/QWGEMM/QWMoEOperator+GroupLatent.swift:11-294):
+// every expert carries the label of one of num_groups latent groups; a token's routes go through the down-projection D_g of
+// their expert's group, the expert in the latent width, and the up-projection U_g of the sum of the group's routes.
+// ------------------------------------------------------------------------------------------------
+
+// group_ids[t, g] = g when one of the token's routes falls into group g, else -1 (the rule of qwg_moe_route with
+// latentLabels, Sources/QWMetal/subsystems/qwrouter.metal:135-165); pair_rows[t, k] = t * num_groups + label of route k
+// (the row of the route's latent among the [t, num_groups] rows), -1 for an absent route.
+__global__ __launch_bounds__(256) void qw_moe_latent_groups_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ labels,
+                                                                    uint32_t T, uint32_t K, uint32_t E, uint32_t NG,
+                                                                    int32_t* __restrict__ group_ids, int32_t* __restrict__ pair_rows) {
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= T) return;
+    uint32_t mask = 0;
+    for (uint32_t k = 0; k < K; ++k) {
+        const int32_t raw = idx[(uint64_t)t * K + k];
+        int32_t row = -1;
+        if (raw >= 0 && ((uint32_t)raw & 0xFFFFu) < E) {
+            const int32_t g = labels[(uint32_t)raw & 0xFFFFu];
+            if (g >= 0 && (uint32_t)g < NG) {
+                mask |= 1u << g;
+                row = (int32_t)(t * NG + (uint32_t)g);
+            }
+        }
+        if (pair_rows) pair_rows[(uint64_t)t * K + k] = row;
+    }
+    for (uint32_t g = 0; g < NG; ++g) group_ids[(uint64_t)t * NG + g] = (mask >> g) & 1u ? (int32_t)g : -1;
+}
+
+extern "C" qwhip_status qwhip_moe_latent_groups(qwhip_stream_t s, const int32_t* idx, const int32_t* labels, uint32_t t, uint32_t top_k,
+                                                uint32_t experts, uint32_t num_groups, int32_t* group_ids, int32_t* pair_rows) {
+    QWHIP_REQUIRE(s);
+    if (t == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(labels);
+    QWHIP_REQUIRE(group_ids);
+    if (num_groups == 0 || num_groups > 32u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent groups must be 1..32, got %u", num_groups);
+    if (top_k == 0 || experts == 0 || experts > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent groups: top_k %u, experts %u", top_k, experts);
+    if ((uint64_t)t * max(top_k, num_groups) >= (1ull << 31)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent groups: %u tokens", t);
+    hipLaunchKernelGGL(qw_moe_latent_groups_kernel, dim3(qwhip_cdiv(t, 256u)), dim3(256), 0, s->stream, idx, labels, t, top_k, experts,
+                       num_groups, group_ids, pair_rows);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// rows_out[p] = slot_of_row[pair_rows[sorted_pair[p]]]: the gather row of sorted position p when the routes' activations
+// are themselves the output of an earlier grouped GEMM (slot_of_row = that sort's inverse permutation).  Positions whose
+// chain breaks (nothing sorted there, absent route, absent group) read row 0 and are never used.
+__global__ __launch_bounds__(256) void qw_moe_compose_rows_kernel(const int32_t* __restrict__ sorted_pair, uint32_t n,
+                                                                   const int32_t* __restrict__ pair_rows, uint32_t n_rows,
+                                                                   const int32_t* __restrict__ slot_of_row, int32_t* __restrict__ rows_out) {
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    int32_t r = 0;
+    const int32_t sp = sorted_pair[p];
+    if (sp >= 0 && (uint32_t)sp < n) {
+        const int32_t pr = pair_rows[sp];
+        if (pr >= 0 && (uint32_t)pr < n_rows) r = slot_of_row ? max(slot_of_row[pr], 0) : pr;
+    }
+    rows_out[p] = r;
+}
+
+extern "C" qwhip_status qwhip_moe_compose_rows(qwhip_stream_t s, const int32_t* sorted_pair, uint32_t pairs, const int32_t* pair_rows,
+                                               uint32_t n_rows, const int32_t* slot_of_row, int32_t* rows_out) {
+    QWHIP_REQUIRE(s);
+    if (pairs == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(sorted_pair);
+    QWHIP_REQUIRE(pair_rows);
+    QWHIP_REQUIRE(rows_out);
+    if (pairs >= (1u << 31) || n_rows >= (1u << 31)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "compose rows: %u pairs, %u rows", pairs, n_rows);
+    hipLaunchKernelGGL(qw_moe_compose_rows_kernel, dim3(qwhip_cdiv(pairs, 256u)), dim3(256), 0, s->stream, sorted_pair, pairs, pair_rows,
+                       n_rows, slot_of_row, rows_out);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+// out[t * NG + g, :] = sum over the routes k of token t with labels[idx[t, k]] == g of wts[t, k] * dn[inv_perm[t * K + k], :]
+// in rank order, zeros for a group without routes (the numGroups mode of qwg_moe_down_reduce_combine_f32,
+// Sources/QWMetal/gemm/qwgemm_moe_nax_f16.metal:51-111).  One thread per 4 columns.
+template <int DDT, int ODT>
+__global__ __launch_bounds__(256) void qw_moe_combine_groups_kernel(const void* __restrict__ dn, const int32_t* __restrict__ inv_perm,
+                                                                     const float* __restrict__ wts, const int32_t* __restrict__ idx,
+                                                                     const int32_t* __restrict__ labels, uint32_t K, uint32_t NG,
+                                                                     uint32_t W, void* __restrict__ out) {
+    const uint32_t row = blockIdx.y, t = row / NG;
+    const int32_t g = (int32_t)(row - t * NG);
+    const uint32_t c = (blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (c >= W) return;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t k = 0; k < K; ++k) {
+        const int32_t e = idx[(uint64_t)t * K + k];
+        if (e < 0 || labels[(uint32_t)e & 0xFFFFu] != g) continue;
+        const int32_t slot = inv_perm ? inv_perm[(uint64_t)t * K + k] : (int32_t)(t * K + k);
+        if (slot < 0) continue;
+        const float w = wts ? wts[(uint64_t)t * K + k] : 1.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (c + j < W) acc[j] = fmaf(w, qw_load_f32<DDT>(dn, (uint64_t)slot * W + c + j), acc[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (c + j < W) {
+            const uint64_t o = (uint64_t)row * W + c + j;
+            if constexpr (ODT == QWHIP_F32) ((float*)out)[o] = acc[j];
+            else if constexpr (ODT == QWHIP_F16) ((h1_t*)out)[o] = (h1_t)acc[j];
+            else ((uint16_t*)out)[o] = qw_f32_to_bf16(acc[j]);
+        }
+    }
+}
+
+extern "C" qwhip_status qwhip_moe_combine_groups(qwhip_stream_t s, const void* dn, uint32_t dn_dtype, const int32_t* inv_perm,
+                                                 const float* wts, const int32_t* idx, const int32_t* labels, uint32_t t, uint32_t top_k,
+                                                 uint32_t num_groups, uint32_t width, void* out, uint32_t out_dtype) {
+    QWHIP_REQUIRE(s);
+    if (t == 0 || width == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(dn);
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(labels);
+    QWHIP_REQUIRE(out);
+    if (num_groups == 0 || num_groups > 32u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent groups must be 1..32, got %u", num_groups);
+    if ((uint64_t)t * num_groups >= (1ull << 31) || (uint64_t)t * top_k >= (1ull << 31))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine by groups: %u tokens", t);
+    // grid.y holds 65535 rows: more (token, group) rows go in slabs of whole tokens
+    const uint32_t tok_per = 65535u / num_groups;
+    for (uint32_t t0 = 0; t0 < t; t0 += tok_per) {
+        const uint32_t tt = min(tok_per, t - t0);
+        const dim3 grid(qwhip_cdiv(width, 1024), tt * num_groups), block(256);
+        const int32_t* ip = inv_perm ? inv_perm + (uint64_t)t0 * top_k : nullptr;
+        const float* wp = wts ? wts + (uint64_t)t0 * top_k : nullptr;
+        const int32_t* xp = idx + (uint64_t)t0 * top_k;
+        const uint64_t orow = (uint64_t)t0 * num_groups * width;
+        void* op = (uint8_t*)out + orow * (out_dtype == QWHIP_F32 ? 4u : 2u);
+        // identity slots count from the slab's first token: shift the dn base instead
+        const void* dp = inv_perm ? dn : (const void*)((const uint8_t*)dn + (uint64_t)t0 * top_k * width * (dn_dtype == QWHIP_F32 ? 4u : 2u));
+#define QW_CG(DD, OD) hipLaunchKernelGGL((qw_moe_combine_groups_kernel<DD, OD>), grid, block, 0, s->stream, dp, ip, wp, xp, labels, top_k, num_groups, width, op)
+#define QW_CG_O(DD)                                                   \
+        switch (out_dtype) {                                          \
+            case QWHIP_F32: QW_CG(DD, QWHIP_F32); break;              \
+            case QWHIP_F16: QW_CG(DD, QWHIP_F16); break;              \
+            case QWHIP_BF16: QW_CG(DD, QWHIP_BF16); break;            \
+            default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine by groups: unsupported output dtype %u", out_dtype); \
+        }
+        switch (dn_dtype) {
+            case QWHIP_F32: QW_CG_O(QWHIP_F32) break;
+            case QWHIP_F16: QW_CG_O(QWHIP_F16) break;
+            case QWHIP_BF16: QW_CG_O(QWHIP_BF16) break;
+            default: return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine by groups: unsupported input dtype %u", dn_dtype);
+        }
+#undef QW_CG_O
+#undef QW_CG
+        QWHIP_TRY_HIP(hipGetLastError());
+    }
+    return QWHIP_OK;
+}

@@ -59,6 +59,7 @@ struct qmc_gu_params {
     const void* x;
     h1_t* act;
     const int32_t* idx;
+    const int32_t* x_rows;   // activation row of every pair (NULL: the pair's token)
     uint32_t I, nb, cpr, top_k, rotate, rot_out;
     uint64_t expert_bytes;
     // JN > 0: the routing is done here.  The first wave of every workgroup routes the pair's token from its router logits
@@ -95,7 +96,8 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
     int32_t e = 0;                               // no route list: one dense gate|up bank
     if constexpr (JN == 0) e = p.idx ? p.idx[pair] : 0;
     const uint32_t token = pair / p.top_k;
-    const uint8_t* x = (const uint8_t*)p.x + (uint64_t)token * nb * 64u;
+    const uint32_t xrow = (JN == 0 && p.x_rows) ? (uint32_t)max(p.x_rows[pair], 0) : token;
+    const uint8_t* x = (const uint8_t*)p.x + (uint64_t)xrow * nb * 64u;
     h8_t xv[XT];
 #pragma unroll
     for (int t = 0; t < XT; ++t) {
@@ -192,6 +194,9 @@ struct qmc_dn_params {
     void* out;
     uint32_t H, nbI, nbv, cprv, top_k, sets;
     uint64_t expert_bytes;
+    uint32_t x_div;          // pairs that share one activation row (1: a row per pair)
+    const int32_t* labels;   // num_groups > 0: blockIdx.y = token * num_groups + group, and only the token's routes whose
+    uint32_t num_groups;     // expert carries that group's label are summed
 };
 
 template <int ODT, int D>
@@ -201,19 +206,22 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
     const uint32_t lane = tid & 31u, hw = tid >> 5;
     const uint32_t cprv = p.cprv, H = p.H;
     const uint32_t set = hw / cprv, chunk = hw - set * cprv;
-    const uint32_t tok = blockIdx.y, n0 = blockIdx.x * (p.sets * D);
+    const uint32_t tok = blockIdx.y, n0 = blockIdx.x * (p.sets * D);   // tok: the output row
+    const uint32_t src = p.num_groups ? tok / p.num_groups : tok;
+    const int32_t grp = p.num_groups ? (int32_t)(tok - src * p.num_groups) : 0;
     const uint32_t v0 = chunk * 32u + lane;
     const bool vvalid = v0 < p.nbv;
     const uint32_t v = vvalid ? v0 : 0u;
     const uint32_t k = v / p.nbI, b = v - k * p.nbI;
-    const uint32_t pair = tok * p.top_k + k;
+    const uint32_t pair = src * p.top_k + k;
     const int32_t e = p.idx[pair];
-    const float wk = p.wts[pair];
-    const bool valid = vvalid && e >= 0;
+    const float wk = p.wts ? p.wts[pair] : 1.0f;
+    bool valid = vvalid && e >= 0;
+    if (p.num_groups) valid = valid && p.labels[valid ? ((uint32_t)e & 0xFFFFu) : 0u] == grp;
     const uint32_t row_bytes = p.nbI * 20u;
     // activations do not wait for the expert id; the weight rows follow as soon as it is known
     h8_t xr[4];
-    const h8_t* xsrc = (const h8_t*)(p.act + ((uint64_t)pair * p.nbI + b) * 32u);
+    const h8_t* xsrc = (const h8_t*)(p.act + ((uint64_t)(p.x_div > 1u ? pair / p.x_div : pair) * p.nbI + b) * 32u);
 #pragma unroll
     for (int j = 0; j < 4; ++j) xr[j] = xsrc[j];
     const uint8_t* base = p.bank + (uint64_t)(valid ? ((uint32_t)e & 0xFFFFu) : 0u) * p.expert_bytes + b * 20u;
@@ -221,7 +229,8 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
 #pragma unroll
     for (int j = 0; j < D; ++j) {
         const uint32_t n = min(n0 + set * D + j, H - 1u);
-        buf[j] = *(const qw_hq4_block*)(base + (uint64_t)n * row_bytes);
+        buf[j] = qw_hq4_block{};
+        if (valid) buf[j] = *(const qw_hq4_block*)(base + (uint64_t)n * row_bytes);   // lanes of other groups' routes read nothing
     }
     h2_t xo[16];
     const float S = qmc_operands(xr, xo);
@@ -254,7 +263,8 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
 // is outside the kernel's envelope (the caller then takes the general kernel).
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
                        bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
-                       const float* logits, int32_t* idx_out, float* wts_out, uint32_t norm_topk, float routed_scale) {
+                       const float* logits, int32_t* idx_out, float* wts_out, uint32_t norm_topk, float routed_scale,
+                       const int32_t* x_rows) {
     if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
     const uint32_t inter = w->n / (2u * experts);
     const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u;
@@ -268,6 +278,7 @@ bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expe
     p.x = x;
     p.act = (h1_t*)act16;
     p.idx = idx;
+    p.x_rows = x_rows;
     p.I = inter;
     p.nb = nb;
     p.cpr = cpr;
@@ -304,12 +315,13 @@ bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expe
 // shape is outside the kernel's envelope.
 bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* act16, const int32_t* idx,
                      const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
-                     uint32_t out_dtype, hipError_t* err) {
+                     uint32_t out_dtype, hipError_t* err, uint32_t x_div, const int32_t* labels, uint32_t num_groups) {
     if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
     const uint32_t hidden = w->n / experts;
     const uint32_t nbI = w->k / 32u;
     const uint32_t nbv = top_k * nbI, cprv = (nbv + 31u) / 32u;
-    if (cprv > 32u || t > 65535u) return false;
+    const uint32_t out_rows = t * (num_groups ? num_groups : 1u);
+    if (cprv > 32u || out_rows > 65535u) return false;
     if (((uintptr_t)act16 & 15u) != 0) return false;
     uint32_t sets = 1;
     while (sets < 8u && 32u * cprv * sets * 2u <= 1024u) sets *= 2u;
@@ -329,7 +341,10 @@ bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expert
     p.top_k = top_k;
     p.sets = sets;
     p.expert_bytes = (uint64_t)hidden * nbI * 20u;
-    const dim3 grid(qwhip_cdiv(hidden, sets * D), t), block(32u * cprv * sets);
+    p.x_div = x_div;
+    p.labels = labels;
+    p.num_groups = num_groups;
+    const dim3 grid(qwhip_cdiv(hidden, sets * D), out_rows), block(32u * cprv * sets);
     if (out_dtype == QWHIP_F32) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_F32, D>), grid, block, 0, st, p);
     else if (out_dtype == QWHIP_F16) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_F16, D>), grid, block, 0, st, p);
     else if (out_dtype == QWHIP_BF16) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_BF16, D>), grid, block, 0, st, p);

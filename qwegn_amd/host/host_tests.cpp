@@ -525,6 +525,246 @@ static void test_gpu_moe_latent(QWHal& hal, int rows) {
     hal.end(enc);
 }
 
+// Group-latent MoE with the configuration of the reference's own test (FNLatentMoETests.testGroupLatentMoEMatchesCPUAcrossDecodeVerifyAndPrefill,
+// Tests/QWFlashNextTests/FNLatentMoETests.swift:95-189): H = L = I = IS = 64, 4 groups, 32 experts, 4 routes; latent and shared
+// banks 8-bit G32, expert banks 4-bit G64, all rotated bit-stream containers with the test's code formula; the CPU side is the
+// un-rotated restatement of FNSparseMoE.forward (Tests/QWFlashNextTests/Reference/FNSparseMoE.swift:113-156) in fp64 and the
+// pass mark is the test's: max |got - want| / max |want| < 0.002 (0.01 from 64 rows on).
+struct GLMatrix {
+    std::vector<uint8_t> blocks;     // [rows, cols / group] blocks: f16 scale, f16 bias, bit stream
+    std::vector<double> plain;       // [rows, cols]: the weights in the un-rotated basis
+};
+static GLMatrix gl_matrix(int rows, int cols, int bits, int group, int seed, bool foldOutput) {
+    GLMatrix m;
+    const int qmax = (1 << bits) - 1;
+    const float scale = bits == 8 ? 1.0f / 256.0f : 1.0f / 16.0f, bias = -0.5f;
+    const int bb = 4 + group * bits / 8;
+    m.blocks.assign((size_t)rows * (cols / group) * bb, 0);
+    m.plain.assign((size_t)rows * cols, 0.0);
+    for (int r = 0; r < rows; ++r)
+        for (int g = 0; g < cols; g += group) {
+            uint8_t* blk = m.blocks.data() + ((size_t)r * (cols / group) + g / group) * bb;
+            const uint16_t hs = f2h(scale), hb = f2h(bias);
+            std::memcpy(blk, &hs, 2);
+            std::memcpy(blk + 2, &hb, 2);
+            for (int i = 0; i < group; ++i) {
+                const uint32_t code = (uint32_t)(((r * 13 + (g + i) * 7 + seed * 19) & 0xFFFF) % (qmax + 1));
+                const int bit = i * bits;
+                for (int b = 0; b < bits; ++b)
+                    if ((code >> b) & 1u) blk[4 + ((bit + b) >> 3)] |= (uint8_t)(1u << ((bit + b) & 7));
+                m.plain[(size_t)r * cols + g + i] = (double)code * (double)scale + (double)bias;
+            }
+        }
+    for (int r = 0; r < rows; ++r)   // the container holds W . H: un-rotate along the input columns
+        for (int c = 0; c < cols; c += 32) fwht32(&m.plain[(size_t)r * cols + c]);
+    if (foldOutput) {                // and H . W when the output rotation is folded into the rows
+        std::vector<double> col(32);
+        for (int c = 0; c < cols; ++c)
+            for (int r0 = 0; r0 < rows; r0 += 32) {
+                for (int j = 0; j < 32; ++j) col[j] = m.plain[(size_t)(r0 + j) * cols + c];
+                fwht32(col.data());
+                for (int j = 0; j < 32; ++j) m.plain[(size_t)(r0 + j) * cols + c] = col[j];
+            }
+    }
+    return m;
+}
+
+static void test_gpu_moe_group_latent(QWHal& hal, int rows) {
+    const int H = 64, NG = 4, L = 64, E = 32, K = 4, I = 64, IS = 64;
+    std::vector<GLMatrix> dM, uM, guM, dnM;
+    for (int g = 0; g < NG; ++g) dM.push_back(gl_matrix(L, H, 8, 32, 1 + g, true));
+    for (int g = 0; g < NG; ++g) uM.push_back(gl_matrix(H, L, 8, 32, 11 + g, false));
+    for (int e = 0; e < E; ++e) guM.push_back(gl_matrix(2 * I, L, 4, 64, 21 + e, false));
+    for (int e = 0; e < E; ++e) dnM.push_back(gl_matrix(L, I, 4, 64, 61 + e, true));
+    const GLMatrix shGate = gl_matrix(IS, H, 8, 32, 101, false), shUp = gl_matrix(IS, H, 8, 32, 102, false), shDn = gl_matrix(H, IS, 8, 32, 103, false);
+    auto cat = [](const std::vector<GLMatrix>& v) {
+        std::vector<uint8_t> o;
+        for (const GLMatrix& m : v) o.insert(o.end(), m.blocks.begin(), m.blocks.end());
+        return o;
+    };
+    const std::vector<uint8_t> dB = cat(dM), uB = cat(uM), guB = cat(guM), dnB = cat(dnM);
+    std::vector<uint8_t> shguB = shGate.blocks;
+    shguB.insert(shguB.end(), shUp.blocks.begin(), shUp.blocks.end());
+    std::vector<int32_t> labels(E);
+    for (int e = 0; e < E; ++e) labels[e] = e % NG;
+    std::vector<float> gateW((size_t)E * H), shScalar(H);
+    for (int i = 0; i < E * H; ++i) gateW[i] = (float)((i * 17) % 19 - 9) * 0.0625f;
+    for (int h = 0; h < H; ++h) shScalar[h] = (float)((h * 11) % 13 - 6) * 0.0625f;
+    // the operator's input as the reference's test gives it: f32 rows un-rotated and rotated, the f16 copy from 64 rows on
+    std::vector<float> xPlainF((size_t)rows * H), xRotF((size_t)rows * H);
+    std::vector<uint16_t> x16((size_t)rows * H);
+    std::vector<double> xp((size_t)rows * H);
+    for (int t = 0; t < rows; ++t) {
+        std::vector<double> r(H);
+        for (int h = 0; h < H; ++h) {
+            xPlainF[(size_t)t * H + h] = (float)(((t * H + h) * 7 + rows) % 23 - 11) * 0.1f;
+            xp[(size_t)t * H + h] = r[h] = (double)xPlainF[(size_t)t * H + h];
+        }
+        for (int o = 0; o < H; o += 32) fwht32(&r[o]);
+        for (int h = 0; h < H; ++h) { xRotF[(size_t)t * H + h] = (float)r[h]; x16[(size_t)t * H + h] = f2h((float)r[h]); }
+    }
+    auto silu = [](double g) { return g / (1 + std::exp(-g)); };
+    auto linear = [](const double* x, const std::vector<double>& w, int out, int in) {
+        std::vector<double> y(out, 0.0);
+        for (int o = 0; o < out; ++o) {
+            double a = 0;
+            for (int i = 0; i < in; ++i) a += w[(size_t)o * in + i] * x[i];
+            y[o] = a;
+        }
+        return y;
+    };
+    std::vector<double> ref((size_t)rows * H, 0.0);
+    for (int t = 0; t < rows; ++t) {
+        const double* xt = &xp[(size_t)t * H];
+        std::vector<double> logit(E), p(E);
+        double mx = -1e300, tot = 0;
+        for (int e = 0; e < E; ++e) {
+            double a = 0;
+            for (int h = 0; h < H; ++h) a += (double)gateW[(size_t)e * H + h] * xt[h];
+            logit[e] = a;
+            mx = std::fmax(mx, a);
+        }
+        for (int e = 0; e < E; ++e) { p[e] = std::exp(logit[e] - mx); tot += p[e]; }
+        std::vector<int> chosen;
+        std::vector<bool> taken(E, false);
+        double wsum = 0;
+        for (int r = 0; r < K; ++r) {
+            int best = -1;
+            for (int e = 0; e < E; ++e)
+                if (!taken[e] && (best < 0 || p[e] > p[best])) best = e;
+            taken[best] = true;
+            chosen.push_back(best);
+            wsum += p[best] / tot;
+        }
+        std::vector<std::vector<double>> z(NG, std::vector<double>(L, 0.0)), dcache(NG);
+        std::vector<bool> active(NG, false);
+        for (int r = 0; r < K; ++r) {
+            const int e = chosen[r], g = labels[e];
+            if (dcache[g].empty()) dcache[g] = linear(xt, dM[g].plain, L, H);
+            const std::vector<double> gu = linear(dcache[g].data(), guM[e].plain, 2 * I, L);
+            std::vector<double> act(I);
+            for (int i = 0; i < I; ++i) act[i] = silu(gu[i]) * gu[I + i];
+            const std::vector<double> y = linear(act.data(), dnM[e].plain, L, I);
+            const double wk = (p[e] / tot) / wsum;
+            for (int l = 0; l < L; ++l) z[g][l] += wk * y[l];
+            active[g] = true;
+        }
+        std::vector<double> acc(H, 0.0);
+        for (int g = 0; g < NG; ++g) {
+            if (!active[g]) continue;
+            const std::vector<double> y = linear(z[g].data(), uM[g].plain, H, L);
+            for (int h = 0; h < H; ++h) acc[h] += y[h];
+        }
+        const std::vector<double> sg = linear(xt, shGate.plain, IS, H), su = linear(xt, shUp.plain, IS, H);
+        std::vector<double> sh(IS);
+        for (int i = 0; i < IS; ++i) sh[i] = silu(sg[i]) * su[i];
+        const std::vector<double> shared = linear(sh.data(), shDn.plain, H, IS);
+        double gl = 0;
+        for (int h = 0; h < H; ++h) gl += (double)shScalar[h] * xt[h];
+        const double gate = 1.0 / (1.0 + std::exp(-gl));
+        for (int h = 0; h < H; ++h) ref[(size_t)t * H + h] = acc[h] + gate * shared[h];
+    }
+    QWHipEncoder enc = hal.begin();
+    const int pairs = rows * K, gpairs = rows * NG, mt = QWGemm::moeMaxTiles(E, pairs), gmt = QWGemm::moeMaxTiles(NG, gpairs);
+    DeviceBuf dd(hal, dB.size()), du(hal, uB.size()), dgu(hal, guB.size()), ddn(hal, dnB.size()), dshgu(hal, shguB.size()), dshdn(hal, shDn.blocks.size());
+    DeviceBuf dr(hal, gateW.size() * 4), dsc(hal, shScalar.size() * 4), dlab(hal, labels.size() * 4), dx(hal, x16.size() * 2), dout(hal, (size_t)rows * H * 4);
+    DeviceBuf dlog(hal, (size_t)rows * E * 4), didx(hal, pairs * 4), dw(hal, pairs * 4), dact(hal, (size_t)pairs * I * 2);
+    DeviceBuf doff(hal, (E + 1) * 4), dsp(hal, pairs * 4), dst(hal, pairs * 4), dinv(hal, pairs * 4), dte(hal, mt * 4), dtr(hal, mt * 4), dtc(hal, 16);
+    DeviceBuf ddnhi(hal, (size_t)pairs * L * 4);
+    DeviceBuf dxr(hal, (size_t)rows * H * 4), dxpl(hal, (size_t)rows * H * 4), dgid(hal, gpairs * 4), dprow(hal, pairs * 4), dones(hal, gpairs * 4);
+    DeviceBuf dxl(hal, (size_t)gpairs * L * 2), dzl(hal, (size_t)gpairs * L * 2), dnax(hal, (size_t)rows * H * 2), dgate(hal, (size_t)rows * 4);
+    DeviceBuf dgush(hal, (size_t)rows * 2 * IS * 4), dactsh(hal, (size_t)rows * IS * 4), dshared(hal, (size_t)rows * H * 4);
+    DeviceBuf dgoff(hal, (NG + 1) * 4), dgsp(hal, gpairs * 4), dgst(hal, gpairs * 4), dginv(hal, gpairs * 4), dgte(hal, gmt * 4), dgtr(hal, gmt * 4), dgtc(hal, 16);
+    DeviceBuf drows2(hal, pairs * 4), dup(hal, (size_t)gpairs * H * 4), dxe(hal, (size_t)rows * H * 2);
+    upload(enc, dd, dB.data(), dB.size());
+    upload(enc, du, uB.data(), uB.size());
+    upload(enc, dgu, guB.data(), guB.size());
+    upload(enc, ddn, dnB.data(), dnB.size());
+    upload(enc, dshgu, shguB.data(), shguB.size());
+    upload(enc, dshdn, shDn.blocks.data(), shDn.blocks.size());
+    upload(enc, dr, gateW.data(), gateW.size() * 4);
+    upload(enc, dsc, shScalar.data(), shScalar.size() * 4);
+    upload(enc, dlab, labels.data(), labels.size() * 4);
+    upload(enc, dx, x16.data(), x16.size() * 2);
+    upload(enc, dxpl, xPlainF.data(), xPlainF.size() * 4);
+    upload(enc, dxr, xRotF.data(), xRotF.size() * 4);
+    const std::vector<float> ones(gpairs, 1.0f);
+    upload(enc, dones, ones.data(), ones.size() * 4);
+    auto view = [](DeviceBuf& b, int n, int k, int bits, int group) { return *QWWeightView::make(QWTensorValue::make(b.p, b.bytes, QWDType::q4g), n, k, bits, group, true); };
+    auto i32 = [](DeviceBuf& b, size_t n) { return QWTensorValue::make(b.p, n, QWDType::i32); };
+    auto f32 = [](DeviceBuf& b, size_t n) { return QWTensorValue::make(b.p, n, QWDType::f32); };
+    auto f16 = [](DeviceBuf& b, size_t n) { return QWTensorValue::make(b.p, n, QWDType::f16); };
+    QWMoEOperator::GroupLatentWeights gw;
+    gw.routed.router = f32(dr, gateW.size());
+    gw.routed.gateUp = view(dgu, E * 2 * I, L, 4, 64);
+    gw.routed.down = view(ddn, E * L, I, 4, 64);
+    gw.routed.hidden = H; gw.routed.experts = E; gw.routed.topK = K; gw.routed.intermediate = I;
+    gw.latentD = view(dd, NG * L, H, 8, 32);
+    gw.latentU = view(du, NG * H, L, 8, 32);
+    gw.latentLabels = i32(dlab, E);
+    gw.numLatentGroups = NG;
+    gw.latentDim = L;
+    gw.sharedGateUp = view(dshgu, 2 * IS, H, 8, 32);
+    gw.sharedDown = view(dshdn, H, IS, 8, 32);
+    gw.sharedGateScalar = f32(dsc, H);
+    gw.sharedIntermediate = IS;
+    QWMoEOperator::Scratch s;
+    s.logits = f32(dlog, (size_t)rows * E);
+    s.idx = i32(didx, pairs);
+    s.wts = f32(dw, pairs);
+    s.act16 = f16(dact, (size_t)pairs * I);
+    s.expOff = i32(doff, E + 1);
+    s.sortedPair = i32(dsp, pairs);
+    s.sortedTok = i32(dst, pairs);
+    s.invPerm = i32(dinv, pairs);
+    s.tileE = i32(dte, mt);
+    s.tileR = i32(dtr, mt);
+    s.tileCount = i32(dtc, 4);
+    s.dnHi = f32(ddnhi, (size_t)pairs * L);
+    QWMoEOperator::GroupLatentScratch gs;
+    gs.xRot32 = f32(dxr, (size_t)rows * H);
+    gs.xPlain32 = f32(dxpl, (size_t)rows * H);
+    gs.groupIds = i32(dgid, gpairs);
+    gs.pairRows = i32(dprow, pairs);
+    gs.onesRoute = f32(dones, gpairs);
+    gs.xLatent16 = f16(dxl, (size_t)gpairs * L);
+    gs.zLatent16 = f16(dzl, (size_t)gpairs * L);
+    gs.naxX16 = f16(dnax, (size_t)rows * H);
+    gs.gate = f32(dgate, rows);
+    gs.guSh32 = f32(dgush, (size_t)rows * 2 * IS);
+    gs.actSh32 = f32(dactsh, (size_t)rows * IS);
+    gs.shared = f32(dshared, (size_t)rows * H);
+    gs.gExpOff = i32(dgoff, NG + 1);
+    gs.gSortedPair = i32(dgsp, gpairs);
+    gs.gSortedTok = i32(dgst, gpairs);
+    gs.gInvPerm = i32(dginv, gpairs);
+    gs.gTileE = i32(dgte, gmt);
+    gs.gTileR = i32(dgtr, gmt);
+    gs.gTileCount = i32(dgtc, 4);
+    gs.rows2 = i32(drows2, pairs);
+    gs.upAcc = f32(dup, (size_t)gpairs * H);
+    gs.xe16 = f16(dxe, (size_t)rows * H);
+    const QWTensorValue pre16 = f16(dx, x16.size());
+    const QWMoEOperator::Input xt = QWMoEOperator::Input::preRotated(gs.xPlain32, gs.xRot32, rows >= 64 ? &pre16 : nullptr);
+    const QWTensorValue out = f32(dout, (size_t)rows * H);
+    QWMoEOperator::encodeResidentGroupLatent(enc, hal, gw, s, gs, xt, out, rows);
+    std::vector<float> got((size_t)rows * H);
+    download(enc, got.data(), dout, got.size() * 4);
+    double worst = 0, wantMax = 0;
+    for (size_t i = 0; i < got.size(); ++i) { worst = std::fmax(worst, std::fabs((double)got[i] - ref[i])); wantMax = std::fmax(wantMax, std::fabs(ref[i])); }
+    const double rel = worst / std::fmax(1e-6, wantMax);
+    std::printf("moe encodeResidentGroupLatent rows=%d maxAbs %.3e wantMax %.3e rel %.3e\n", rows, worst, wantMax, rel);
+    CHECK(rel < (rows >= 64 ? 0.01 : 0.002));
+    {   // a label table shorter than the experts is refused before any launch
+        QWMoEOperator::GroupLatentWeights bad = gw;
+        bad.latentLabels = i32(dlab, E - 1);
+        bool threw = false;
+        try { QWMoEOperator::encodeResidentGroupLatent(enc, hal, bad, s, gs, xt, out, rows); } catch (const QWGemmError&) { threw = true; }
+        CHECK(threw);
+    }
+    hal.end(enc);
+}
+
 // f32-activation doors and the head: encodeHQ4F32V4 (epilogues 0 and 3), encodeH32F32, encodeHeadArgmax on the closed-form bank
 static void test_gpu_f32_doors(QWHal& hal) {
     const int N = 96, Kc = 128, rows = 3;
@@ -672,6 +912,7 @@ int main(int argc, char** argv) {
         test_gpu_moe_resident(hal, 40);   // grouped prefill path (fused gate_up + SwiGLU)
         test_gpu_moe_latent(hal, 3);      // latent bottleneck, routed GEMVs
         test_gpu_moe_latent(hal, 40);     // latent bottleneck, grouped GEMMs and batched f32 projections
+        for (int rows : {1, 2, 4, 16, 64}) test_gpu_moe_group_latent(hal, rows);   // the row counts of the reference's test
         test_gpu_f32_doors(hal);
         test_gpu_dense_proj_f32(hal);
         test_gpu_embed(hal);

@@ -674,6 +674,71 @@ struct QWGemm {
                                             (uint32_t)rows, (uint32_t)topK, shared ? (const float*)shared->ptr() : nullptr,
                                             sharedGate ? (const float*)sharedGate->ptr() : nullptr, out.ptr(), abiDType(out.shape.dtype)));
     }
+
+    // ---- group-latent doors: the modes of the reference's encoders that carry latentLabels / groupIds / numGroups ----------
+    // encodeFnMoeRoute(latentLabels:groupIds:numGroups:) (QWGemmMoERouter.swift:10-75): the groups a token's routes fall into and
+    // the latent row of every route
+    static void encodeMoELatentGroups(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& idx, const QWTensorValue& labels, int rows, int topK,
+                                      int experts, int numGroups, const QWTensorValue& groupIds, const QWTensorValue* pairRows) {
+        if (numGroups <= 0 || numGroups > 32) throw QWGemmError(QWGemmError::badShape, "group-latent moe: 1..32 latent groups");
+        if (labels.shape.elementCount < (size_t)experts || groupIds.shape.elementCount < (size_t)rows * (size_t)numGroups ||
+            idx.shape.elementCount < (size_t)rows * (size_t)topK || (pairRows && pairRows->shape.elementCount < (size_t)rows * (size_t)topK))
+            throw QWGemmError(QWGemmError::badShape, "group-latent moe: labels [experts], groupIds [rows, groups], pairRows [rows, topK]");
+        hal.pipeline("qwg_moe_route");
+        throwIfFailed(qwhip_moe_latent_groups(enc.stream, (const int32_t*)idx.ptr(), (const int32_t*)labels.ptr(), (uint32_t)rows, (uint32_t)topK,
+                                              (uint32_t)experts, (uint32_t)numGroups, (int32_t*)groupIds.ptr(),
+                                              pairRows ? (int32_t*)pairRows->ptr() : nullptr));
+    }
+    // encodeMoEDownSharedCombineF32(routeOutput: true, tokenIndexedX: true) (QWGemmMoE.swift:157-199): one output row per route
+    static void encodeMoERoutedGemv(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& bank, int experts, const QWTensorValue& x16,
+                                    bool xPerToken, const QWTensorValue& idx, const QWTensorValue* wts, int rows, int routes, const QWTensorValue& out) {
+        hal.pipeline("qwg_moe_down_shared_combine_q4g_f32");
+        const qwhip_weight_view v = bank.abi();
+        throwIfFailed(qwhip_moe_routed_gemv(enc.stream, &v, (uint32_t)experts, x16.ptr(), xPerToken ? 1u : 0u, (const int32_t*)idx.ptr(),
+                                            wts ? (const float*)wts->ptr() : nullptr, (uint32_t)rows, (uint32_t)routes, out.ptr(),
+                                            abiDType(out.shape.dtype)));
+    }
+    // encodeMoEGateUpF32R1 over the latent rows of the routes (the reference's packed ids select row token * numGroups + group)
+    static void encodeMoEGateUpRowsF32R1(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& gateUp, int experts, const QWTensorValue& x,
+                                         const QWTensorValue& idx, const QWTensorValue& xRows, int rows, int topK, const QWTensorValue& act16) {
+        hal.pipeline("qwg_moe_gateup_q4g_f32_r1");
+        const qwhip_weight_view v = gateUp.abi();
+        throwIfFailed(qwhip_moe_gateup_decode_rows(enc.stream, &v, (uint32_t)experts, x.ptr(), abiDType(x.shape.dtype), (uint32_t)QWHIP_X_PREROTATED,
+                                                   (const int32_t*)idx.ptr(), (const int32_t*)xRows.ptr(), (uint32_t)rows, (uint32_t)topK, act16.ptr()));
+    }
+    // encodeMoEDownSharedCombineF32(numGroups:) (QWGemmMoE.swift:157-199): the routed down projection summed by latent group
+    static void encodeMoEDownGroupsF32(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& down, int experts, const QWTensorValue& act16,
+                                       const QWTensorValue& idx, const QWTensorValue& wts, const QWTensorValue& labels, int numGroups, int rows,
+                                       int topK, const QWTensorValue& out) {
+        hal.pipeline("qwg_moe_down_shared_combine_q4g_f32");
+        const qwhip_weight_view v = down.abi();
+        throwIfFailed(qwhip_moe_down_decode_groups(enc.stream, &v, (uint32_t)experts, act16.ptr(), (const int32_t*)idx.ptr(), (const float*)wts.ptr(),
+                                                   (const int32_t*)labels.ptr(), (uint32_t)numGroups, (uint32_t)rows, (uint32_t)topK, out.ptr(),
+                                                   abiDType(out.shape.dtype)));
+    }
+    // the gather rows of a grouped GEMM that reads the sorted output of an earlier one (the reference scatters that output back
+    // to [token, group] rows instead: encodeMoEDownReduceCombineF32(scatterPerRoute: true))
+    static void encodeMoEComposeRows(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& sortedPair, int pairs, const QWTensorValue& pairRows,
+                                     int nRows, const QWTensorValue* slotOfRow, const QWTensorValue& rowsOut) {
+        if (sortedPair.shape.elementCount < (size_t)pairs || pairRows.shape.elementCount < (size_t)pairs || rowsOut.shape.elementCount < (size_t)pairs ||
+            (slotOfRow && slotOfRow->shape.elementCount < (size_t)nRows))
+            throw QWGemmError(QWGemmError::badShape, "moe compose rows: lists are short");
+        hal.pipeline("qwg_moe_group_pairs_f32");
+        throwIfFailed(qwhip_moe_compose_rows(enc.stream, (const int32_t*)sortedPair.ptr(), (uint32_t)pairs, (const int32_t*)pairRows.ptr(), (uint32_t)nRows,
+                                             slotOfRow ? (const int32_t*)slotOfRow->ptr() : nullptr, (int32_t*)rowsOut.ptr()));
+    }
+    // encodeMoEDownReduceCombineF32(numGroups:) (QWGemmMoE.swift:299-332): the sorted down outputs summed by latent group
+    static void encodeMoECombineGroupsF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& dn, const QWTensorValue* invPerm,
+                                          const QWTensorValue* wts, const QWTensorValue& idx, const QWTensorValue& labels, int rows, int topK,
+                                          int numGroups, int width, const QWTensorValue& out) {
+        if (out.shape.elementCount < (size_t)rows * (size_t)numGroups * (size_t)width)
+            throw QWGemmError(QWGemmError::badShape, "moe combine by groups: out [rows, groups, width] is short");
+        hal.pipeline("qwg_moe_down_reduce_combine_f32");
+        throwIfFailed(qwhip_moe_combine_groups(enc.stream, dn.ptr(), abiDType(dn.shape.dtype), invPerm ? (const int32_t*)invPerm->ptr() : nullptr,
+                                               wts ? (const float*)wts->ptr() : nullptr, (const int32_t*)idx.ptr(), (const int32_t*)labels.ptr(),
+                                               (uint32_t)rows, (uint32_t)topK, (uint32_t)numGroups, (uint32_t)width, out.ptr(),
+                                               abiDType(out.shape.dtype)));
+    }
 };
 
 // ---- QWGemmAQ (Sources/Operators/QWGEMM/QWGemmAQ.swift:192-304): the bit-stream block family ----------------------
@@ -883,6 +948,119 @@ struct QWMoEOperator {
         QWGemm::encodeLatentNormH32F32(enc, hal, ls.bufA32, latent.normGamma ? &*latent.normGamma : nullptr, ls.bufB32, nullptr, rows, L, latent.normEps);
         QWGemm::encodeDenseProjF32(enc, hal, latent.fc2, ls.bufB32, out32, ls.naxX16, rows);
         if (hasShared) QWGemm::encodeMoEAddSharedF32(enc, hal, out32, rows, H, ls.shared, hasGate ? &ls.gate : nullptr, out32);
+    }
+
+    // ---- group-latent sparse MoE (QWMoEOperator+GroupLatent.swift:11-294): latentD[g] -> routed experts in the latent width ->
+    // sum by group -> latentU[g], the shared expert on the full hidden width -----------------------------------------------
+    struct GroupLatentWeights {
+        Weights routed;                         // gateUp: n = experts * 2 * intermediate, k = latentDim; down: n = experts * latentDim, k = intermediate
+        QWWeightView latentD;                   // n = numLatentGroups * latentDim, k = hidden (output rotation folded in)
+        QWWeightView latentU;                   // n = numLatentGroups * hidden, k = latentDim
+        QWTensorValue latentLabels;             // i32 [experts]: the group of every expert
+        int numLatentGroups = 0, latentDim = 0;
+        std::optional<QWWeightView> sharedGateUp, sharedDown;
+        std::optional<QWTensorValue> sharedGateScalar;   // f32 [hidden]
+        int sharedIntermediate = 0;
+        std::optional<QWTensorValue> routerBias, routedScaleParam;
+        bool splitFeatureRouting = false;
+    };
+    struct GroupLatentScratch {   // caller-owned
+        QWTensorValue xRot32, xPlain32;         // f32 [rows, hidden]
+        QWTensorValue groupIds;                 // i32 [rows, groups]
+        QWTensorValue pairRows;                 // i32 [rows, topK]
+        QWTensorValue onesRoute;                // f32 [rows, groups], all 1 (the reference's onesRoute)
+        QWTensorValue xLatent16, zLatent16;     // f16 [rows * groups, latentDim]
+        QWTensorValue naxX16;                   // f16 staging of the shared expert's projections
+        QWTensorValue gate;                     // f32 [rows]
+        QWTensorValue guSh32, actSh32, shared;  // f32 [rows, 2 ISh], [rows, ISh], [rows, hidden]
+        // prefill only: the sort of the (token, group) pairs, kept beside the experts' sort in Scratch, and its outputs
+        QWTensorValue gExpOff, gSortedPair, gSortedTok, gInvPerm, gTileE, gTileR, gTileCount;   // i32
+        QWTensorValue rows2;                    // i32 [rows * topK]: gather rows of the experts' gate_up
+        QWTensorValue upAcc;                    // f32 [rows * groups, hidden]
+        QWTensorValue xe16;                     // f16 [rows, hidden]: the cast of an f32 input without a precast copy
+    };
+    // The operator's Input (QWMoEOperator.swift:12-17): f16 normed rows in the rotated basis, or f32 rows given both un-rotated
+    // and rotated (with an optional f16 copy of the rotated rows).
+    struct Input {
+        std::optional<QWTensorValue> f16Normed;
+        std::optional<QWTensorValue> plain32, rotated32, precast16;
+        static Input normed(const QWTensorValue& x16) { Input i; i.f16Normed = x16; return i; }
+        static Input preRotated(const QWTensorValue& plain, const QWTensorValue& rotated, const QWTensorValue* precast = nullptr) {
+            Input i; i.plain32 = plain; i.rotated32 = rotated; if (precast) i.precast16 = *precast; return i;
+        }
+    };
+    // `s.dnHi` holds [rows * topK, latentDim].  The latents travel as f16 between the stages on both paths (the reference's grouped
+    // path does; its decode path keeps them f32).
+    static void encodeResidentGroupLatent(QWHipEncoder& enc, const QWHal& hal, const GroupLatentWeights& gw, const Scratch& s,
+                                          const GroupLatentScratch& gs, const Input& input, const QWTensorValue& out32, int rows) {
+        const Weights& w = gw.routed;
+        const int H = w.hidden, L = gw.latentDim, NG = gw.numLatentGroups, E = w.experts, K = w.topK, I = w.intermediate, ISh = gw.sharedIntermediate;
+        if (E > 512 || E <= 0 || K <= 0 || K > 16) throw QWGemmError(QWGemmError::badShape, "group-latent moe: experts <= 512, routes <= 16");
+        if (NG <= 0 || NG > 32 || L <= 0 || L % 32 != 0 || gw.latentD.n != NG * L || gw.latentD.k != H || gw.latentU.n != NG * H || gw.latentU.k != L)
+            throw QWGemmError(QWGemmError::badShape, "group-latent moe: latentD is [groups * latent, hidden], latentU [groups * hidden, latent], 1..32 groups");
+        if (w.gateUp.n != E * 2 * I || w.gateUp.k != L || w.down.n != E * L || w.down.k != I)
+            throw QWGemmError(QWGemmError::badShape, "group-latent moe: expert banks do not match (experts, latent, intermediate)");
+        const bool hasShared = ISh > 0 && gw.sharedGateUp && gw.sharedDown;
+        if (hasShared && (gw.sharedGateUp->n != 2 * ISh || gw.sharedGateUp->k != H || gw.sharedDown->n != H || gw.sharedDown->k != ISh))
+            throw QWGemmError(QWGemmError::badShape, "group-latent moe: shared expert banks do not match (hidden, shared intermediate)");
+        const int routerCols = gw.splitFeatureRouting ? 2 * E : E;
+        const bool hasGate = hasShared && gw.sharedGateScalar;
+        QWTensorValue x16, xPlain32, xRot32;
+        if (input.f16Normed) {
+            x16 = *input.f16Normed;
+            xPlain32 = gs.xPlain32;
+            xRot32 = gs.xRot32;
+            QWGemm::encodeMoEBridgeF16ToF32(enc, hal, x16, xRot32, xPlain32, rows, H);
+        } else if (input.plain32 && input.rotated32) {
+            xPlain32 = *input.plain32;
+            xRot32 = *input.rotated32;
+            if (input.precast16) {
+                x16 = *input.precast16;
+            } else {
+                if (!gs.xe16.base) throw QWGemmError(QWGemmError::badShape, "group-latent moe: an f32 input without a precast copy needs the xe16 scratch");
+                QWGemm::encodeCast(enc, hal, xRot32, gs.xe16, (size_t)rows * (size_t)H);
+                x16 = gs.xe16;
+            }
+        } else {
+            throw QWGemmError(QWGemmError::badShape, "group-latent moe: input is f16 normed rows or the f32 (plain, rotated) pair");
+        }
+        QWGemm::encodeFnRouterGemm(enc, hal, xPlain32, w.router, s.logits, rows, routerCols, H, hasGate ? &*gw.sharedGateScalar : nullptr,
+                                   hasGate ? &gs.gate : nullptr);
+        QWGemm::encodeFnMoeRoute(enc, hal, s.logits, s.idx, s.wts, rows, E, K, w.normTopK, w.routedScale, gw.routerBias ? &*gw.routerBias : nullptr,
+                                 gw.splitFeatureRouting, gw.routedScaleParam ? &*gw.routedScaleParam : nullptr);
+        QWGemm::encodeMoELatentGroups(enc, hal, s.idx, gw.latentLabels, rows, K, E, NG, gs.groupIds, &gs.pairRows);
+        if (hasShared) {
+            QWGemm::encodeDenseProjF32(enc, hal, *gw.sharedGateUp, xRot32, gs.guSh32, gs.naxX16, rows);
+            QWGemm::encodeSiluMulF32(enc, hal, gs.guSh32, gs.actSh32, rows, ISh);
+            QWGemm::encodeDenseProjF32(enc, hal, *gw.sharedDown, gs.actSh32, gs.shared, gs.naxX16, rows);
+        }
+        const QWTensorValue* shared = hasShared ? &gs.shared : nullptr;
+        const QWTensorValue* gate = hasGate ? &gs.gate : nullptr;
+        const int pairs = rows * K, gpairs = rows * NG;
+        const bool grouped = rows > 8 && s.expOff.base && s.dnHi.base && gs.gExpOff.base && gs.upAcc.base && H % 64 == 0 && L % 64 == 0 && I % 64 == 0;
+        if (grouped) {
+            // (token, group) pairs sorted by group: D_g over the sorted rows, kept in sorted order
+            QWGemm::encodeMoEGroupPairsF32(enc, hal, gs.groupIds, gs.gExpOff, gs.gSortedPair, gs.gSortedTok, NG, gpairs, NG, &gs.gInvPerm, &gs.gTileE,
+                                           &gs.gTileR, &gs.gTileCount);
+            QWGemm::encodeMoEGroupedGemm(enc, hal, gw.latentD, NG, x16, &gs.gSortedTok, gs.gExpOff, gs.gTileE, gs.gTileR, gs.gTileCount, gpairs,
+                                         gs.xLatent16);
+            // the experts' sort; every sorted (token, route) pair reads the sorted latent row of its token and group
+            QWGemm::encodeMoEGroupPairsF32(enc, hal, s.idx, s.expOff, s.sortedPair, s.sortedTok, E, pairs, K, &s.invPerm, &s.tileE, &s.tileR, &s.tileCount);
+            QWGemm::encodeMoEComposeRows(enc, hal, s.sortedPair, pairs, gs.pairRows, gpairs, &gs.gInvPerm, gs.rows2);
+            QWGemm::encodeMoEGateUpSwiglu(enc, hal, w.gateUp, E, gs.xLatent16, gs.rows2, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.act16,
+                                          w.down.isRotated());
+            QWGemm::encodeMoEGroupedGemm(enc, hal, w.down, E, s.act16, nullptr, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.dnHi);
+            QWGemm::encodeMoECombineGroupsF32(enc, hal, s.dnHi, &s.invPerm, &s.wts, s.idx, gw.latentLabels, rows, K, NG, L, gs.zLatent16);
+            // U_g over the groups' sums (rows token * groups + group, gathered in the first sort's order), then the sum over groups
+            QWGemm::encodeMoEGroupedGemm(enc, hal, gw.latentU, NG, gs.zLatent16, &gs.gSortedPair, gs.gExpOff, gs.gTileE, gs.gTileR, gs.gTileCount, gpairs,
+                                         gs.upAcc);
+            QWGemm::encodeMoEDownReduceCombineF32(enc, hal, gs.upAcc, gs.gInvPerm, gs.onesRoute, rows, NG, H, shared, gate, out32);
+        } else {
+            QWGemm::encodeMoERoutedGemv(enc, hal, gw.latentD, NG, x16, true, gs.groupIds, nullptr, rows, NG, gs.xLatent16);
+            QWGemm::encodeMoEGateUpRowsF32R1(enc, hal, w.gateUp, E, gs.xLatent16, s.idx, gs.pairRows, rows, K, s.act16);
+            QWGemm::encodeMoEDownGroupsF32(enc, hal, w.down, E, s.act16, s.idx, s.wts, gw.latentLabels, NG, rows, K, gs.zLatent16);
+            QWGemm::encodeMoEDownSharedCombineF32(enc, hal, gw.latentU, NG, gs.zLatent16, gs.groupIds, gs.onesRoute, rows, NG, shared, gate, out32);
+        }
     }
 };
 

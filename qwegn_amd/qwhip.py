@@ -95,6 +95,12 @@ SIGNATURES = {
     "qwhip_moe_gateup_decode": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _U32, _U32, _P]),
     "qwhip_moe_route_gateup_decode": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _U32, _U32, _U32, C.c_float, _P, _P, _P]),
     "qwhip_moe_down_decode": (C.c_int32, [_P, _WV, _U32, _P, _P, _P, _U32, _U32, _P, _P, _P, _U32]),
+    "qwhip_moe_latent_groups": (C.c_int32, [_P, _P, _P, _U32, _U32, _U32, _U32, _P, _P]),
+    "qwhip_moe_routed_gemv": (C.c_int32, [_P, _WV, _U32, _P, _U32, _P, _P, _U32, _U32, _P, _U32]),
+    "qwhip_moe_gateup_decode_rows": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _P, _U32, _U32, _P]),
+    "qwhip_moe_down_decode_groups": (C.c_int32, [_P, _WV, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _P, _U32]),
+    "qwhip_moe_compose_rows": (C.c_int32, [_P, _P, _U32, _P, _U32, _P, _P]),
+    "qwhip_moe_combine_groups": (C.c_int32, [_P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _P, _U32]),
     "qwhip_quantize_hq4_g32": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, _P]),
     "qwhip_quantize_blocks": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _U32, _P]),
     "qwhip_quantize_hq8_planar": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, _P, _P]),

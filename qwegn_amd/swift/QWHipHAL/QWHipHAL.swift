@@ -412,6 +412,55 @@ public enum QWGemm {
         try qwCheck(qwhip_moe_down_decode(enc.stream, &w, UInt32(experts), x.ptr, ids.i32, weights.f32, UInt32(tokens), UInt32(routes), shared?.f32,
                                           gate?.f32, out.ptr, out.dtype.rawValue))
     }
+
+    // ---- group-latent modes of the same encoders (latentLabels / groupIds / numGroups; the route ids stay plain here) ----
+    /// encodeFnMoeRoute(latentLabels:groupIds:numGroups:) (QWGemmMoERouter.swift:10-75): groups of a token's routes, latent row of every route.
+    public static func encodeMoELatentGroups(_ enc: QWHipEncoder, hal: QWHal, idx: QWTensorValue, labels: QWTensorValue, rows: Int, topK: Int,
+                                             experts: Int, numGroups: Int, groupIds: QWTensorValue, pairRows: QWTensorValue?) throws {
+        guard (1...32).contains(numGroups) else { throw QWGemmError.badShape("group-latent moe: 1..32 latent groups") }
+        try hal.pipeline("qwg_moe_route")
+        try qwCheck(qwhip_moe_latent_groups(enc.stream, idx.i32, labels.i32, UInt32(rows), UInt32(topK), UInt32(experts), UInt32(numGroups),
+                                            groupIds.i32, pairRows?.i32))
+    }
+    /// encodeMoEDownSharedCombineF32(routeOutput: true, tokenIndexedX: true) (QWGemmMoE.swift:157-199): one output row per route.
+    public static func encodeMoERoutedGemv(_ enc: QWHipEncoder, hal: QWHal, bank: QWWeightView, experts: Int, x16: QWTensorValue, xPerToken: Bool,
+                                           ids: QWTensorValue, weights: QWTensorValue?, tokens: Int, routes: Int, out: QWTensorValue) throws {
+        try hal.pipeline(bank.isIncumbent ? "qwg_moe_down_shared_combine_q4g_f32" : "qwg_moe_down_shared_combine_aq\(bank.bits)_g\(bank.groupSize)_f32")
+        var w = bank.abi
+        try qwCheck(qwhip_moe_routed_gemv(enc.stream, &w, UInt32(experts), x16.ptr, xPerToken ? 1 : 0, ids.i32, weights?.f32, UInt32(tokens),
+                                          UInt32(routes), out.ptr, out.dtype.rawValue))
+    }
+    /// encodeMoEGateUpF32R1 over the latent rows of the routes (row token * numGroups + group of the latent matrix).
+    public static func encodeMoEGateUpRowsF32R1(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, experts: Int, ids: QWTensorValue,
+                                                xRows: QWTensorValue, out: QWTensorValue, routes: Int, tokens: Int) throws {
+        try hal.pipeline(bank.isIncumbent ? "qwg_moe_gateup_q4g_f32_r1" : "qwg_moe_gateup_aq\(bank.bits)_g\(bank.groupSize)_f32_r1")
+        var w = bank.abi
+        try qwCheck(qwhip_moe_gateup_decode_rows(enc.stream, &w, UInt32(experts), x.ptr, x.dtype.rawValue, UInt32(QWHIP_X_PREROTATED), ids.i32,
+                                                 xRows.i32, UInt32(tokens), UInt32(routes), out.ptr))
+    }
+    /// encodeMoEDownSharedCombineF32(numGroups:) (QWGemmMoE.swift:157-199): the routed down projection summed by latent group.
+    public static func encodeMoEDownGroupsF32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, experts: Int, ids: QWTensorValue,
+                                              weights: QWTensorValue, labels: QWTensorValue, numGroups: Int, tokens: Int, routes: Int,
+                                              out: QWTensorValue) throws {
+        try hal.pipeline(bank.isIncumbent ? "qwg_moe_down_shared_combine_q4g_f32" : "qwg_moe_down_shared_combine_aq\(bank.bits)_g\(bank.groupSize)_f32")
+        var w = bank.abi
+        try qwCheck(qwhip_moe_down_decode_groups(enc.stream, &w, UInt32(experts), x.ptr, ids.i32, weights.f32, labels.i32, UInt32(numGroups),
+                                                 UInt32(tokens), UInt32(routes), out.ptr, out.dtype.rawValue))
+    }
+    /// Gather rows of a grouped GEMM that reads the sorted output of an earlier one (the reference scatters that output back instead).
+    public static func encodeMoEComposeRows(_ enc: QWHipEncoder, hal: QWHal, sortedPair: QWTensorValue, pairs: Int, pairRows: QWTensorValue,
+                                            rowCount: Int, slotOfRow: QWTensorValue?, rowsOut: QWTensorValue) throws {
+        try hal.pipeline("qwg_moe_group_pairs_f32")
+        try qwCheck(qwhip_moe_compose_rows(enc.stream, sortedPair.i32, UInt32(pairs), pairRows.i32, UInt32(rowCount), slotOfRow?.i32, rowsOut.i32))
+    }
+    /// encodeMoEDownReduceCombineF32(numGroups:) (QWGemmMoE.swift:299-332): the sorted down outputs summed by latent group.
+    public static func encodeMoECombineGroupsF32(_ enc: QWHipEncoder, hal: QWHal, dnAcc: QWTensorValue, invPerm: QWTensorValue?, weights: QWTensorValue?,
+                                                 ids: QWTensorValue, labels: QWTensorValue, tokens: Int, routes: Int, numGroups: Int, width: Int,
+                                                 out: QWTensorValue) throws {
+        try hal.pipeline("qwg_moe_down_reduce_combine_f32")
+        try qwCheck(qwhip_moe_combine_groups(enc.stream, dnAcc.ptr, dnAcc.dtype.rawValue, invPerm?.i32, weights?.f32, ids.i32, labels.i32, UInt32(tokens),
+                                             UInt32(routes), UInt32(numGroups), UInt32(width), out.ptr, out.dtype.rawValue))
+    }
 }
 
 /// QWGemmAQ (Sources/Operators/QWGEMM/QWGemmAQ.swift): the doors over the bit-stream containers.
@@ -596,6 +645,104 @@ public enum QWMoEOperator {
         if sharedBanks != nil {
             try QWGemm.encodeMoEAddSharedF32(enc, hal: hal, dnAcc: out32, shared: ls.shared, gate: gateW != nil ? ls.gate : nil, out: out32, hidden: H,
                                              tokens: T)
+        }
+    }
+
+    // ---- group-latent sparse MoE (QWMoEOperator+GroupLatent.swift:11-294) ------------------------------------------------
+    public struct GroupLatentWeights {
+        public let routed: Weights             // gateUp: k = latentDim; down: n = experts * latentDim
+        public let latentD: QWWeightView       // n = groups * latentDim, k = hidden
+        public let latentU: QWWeightView       // n = groups * hidden, k = latentDim
+        public let latentLabels: QWTensorValue // i32 [experts]
+        public let numLatentGroups: Int, latentDim: Int
+        public let sharedGateUp: QWWeightView?, sharedDown: QWWeightView?
+        public let sharedGateScalar: QWTensorValue?
+        public let sharedIntermediate: Int
+        public let routerBias: QWTensorValue?, routedScaleParam: QWTensorValue?
+        public let splitFeatureRouting: Bool
+    }
+    public struct GroupLatentScratch {
+        public let groupIds: QWTensorValue, pairRows: QWTensorValue     // i32 [rows, groups], [rows, topK]
+        public let onesRoute: QWTensorValue                             // f32 [rows, groups], all 1
+        public let xLatent16, zLatent16: QWTensorValue                  // f16 [rows * groups, latentDim]
+        public let naxX16, xe16: QWTensorValue                          // f16 [rows, hidden]
+        public let xRot32, xPlain32: QWTensorValue, gate: QWTensorValue
+        public let guSh32, actSh32, shared: QWTensorValue
+        public let gExpOff, gSortedPair, gSortedTok, gInvPerm, gTileE, gTileR, gTileCount: QWTensorValue?   // prefill: the (token, group) sort
+        public let rows2: QWTensorValue?, upAcc: QWTensorValue?         // prefill: i32 [rows * topK], f32 [rows * groups, hidden]
+    }
+    /// QWMoEOperator.Input (QWMoEOperator.swift:12-17)
+    public enum Input {
+        case f16Normed(QWTensorValue)
+        case f32PreRotated(plain: QWTensorValue, rotated: QWTensorValue, prefillPrecast16: QWTensorValue?)
+    }
+    public static func encodeResidentGroupLatent(_ enc: QWHipEncoder, hal: QWHal, weights gw: GroupLatentWeights, scratch s: Scratch,
+                                                 groupScratch gs: GroupLatentScratch, input: Input, out32: QWTensorValue, rows T: Int) throws {
+        let w = gw.routed
+        let (H, L, NG, E, K, I, ISh) = (w.hidden, gw.latentDim, gw.numLatentGroups, w.experts, w.topK, w.intermediate, gw.sharedIntermediate)
+        guard (1...32).contains(NG), L > 0, L % 32 == 0, gw.latentD.n == NG * L, gw.latentD.k == H, gw.latentU.n == NG * H, gw.latentU.k == L,
+              w.gateUp.n == E * 2 * I, w.gateUp.k == L, w.down.n == E * L, w.down.k == I else {
+            throw QWGemmError.badShape("group-latent moe: banks do not match (hidden, groups, latent, experts, intermediate)")
+        }
+        let x16: QWTensorValue, xPlain: QWTensorValue, xRot: QWTensorValue
+        switch input {
+        case .f16Normed(let x):
+            try QWGemm.encodeMoEBridgeF16ToF32(enc, hal: hal, x: x, xRot32: gs.xRot32, xPlain32: gs.xPlain32, rows: T, hidden: H)
+            (x16, xPlain, xRot) = (x, gs.xPlain32, gs.xRot32)
+        case .f32PreRotated(let plain, let rotated, let precast16):
+            if let p16 = precast16 { x16 = p16 } else {
+                try QWGemm.encodeCast(enc, hal: hal, src32: rotated, dst16: gs.xe16, count: T * H)
+                x16 = gs.xe16
+            }
+            (xPlain, xRot) = (plain, rotated)
+        }
+        let sharedBanks: (QWWeightView, QWWeightView)? = (ISh > 0 && gw.sharedGateUp != nil && gw.sharedDown != nil) ? (gw.sharedGateUp!, gw.sharedDown!) : nil
+        let gateW = sharedBanks != nil ? gw.sharedGateScalar : nil
+        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: xPlain, y: s.logits, rows: T, n: gw.splitFeatureRouting ? 2 * E : E, k: H,
+                                      shGateWeight: gateW, shGateOut: gateW != nil ? gs.gate : nil)
+        try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
+                                    routedScale: w.routedScale, bias: gw.routerBias, splitFeature: gw.splitFeatureRouting,
+                                    routedScaleParam: gw.routedScaleParam)
+        try QWGemm.encodeMoELatentGroups(enc, hal: hal, idx: s.idx, labels: gw.latentLabels, rows: T, topK: K, experts: E, numGroups: NG,
+                                         groupIds: gs.groupIds, pairRows: gs.pairRows)
+        if let (shGU, shDown) = sharedBanks {
+            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shGU, x: xRot, y: gs.guSh32, naxX16: gs.naxX16, rows: T)
+            try QWGemm.encodeSiluMulF32(enc, hal: hal, gu: gs.guSh32, act: gs.actSh32, rows: T, inter: ISh)
+            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shDown, x: gs.actSh32, y: gs.shared, naxX16: gs.naxX16, rows: T)
+        }
+        let shared = sharedBanks != nil ? gs.shared : nil, gate = gateW != nil ? gs.gate : nil
+        let (pairs, gpairs) = (T * K, T * NG)
+        if T > 8, H % 64 == 0, L % 64 == 0, I % 64 == 0, let expOff = s.expOff, let sortedPair = s.sortedPair, let sortedTok = s.sortedTok,
+           let invPerm = s.invPerm, let tileE = s.tileE, let tileR = s.tileR, let tileCount = s.tileCount, let dnHi = s.dnHi,
+           let gOff = gs.gExpOff, let gPair = gs.gSortedPair, let gTok = gs.gSortedTok, let gInv = gs.gInvPerm, let gTE = gs.gTileE, let gTR = gs.gTileR,
+           let gTC = gs.gTileCount, let rows2 = gs.rows2, let upAcc = gs.upAcc {
+            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: gs.groupIds, expertOff: gOff, sortedPairIdx: gPair, sortedTok: gTok, experts: NG,
+                                              totalPairs: gpairs, routes: NG, invPerm: gInv, tileE: gTE, tileR: gTR, tileCount: gTC)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: x16, bank: gw.latentD, experts: NG, expertOff: gOff, tileE: gTE, tileR: gTR, tileCount: gTC,
+                                            y: gs.xLatent16, pairs: gpairs, sortedTok: gTok)
+            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: expOff, sortedPairIdx: sortedPair, sortedTok: sortedTok, experts: E,
+                                              totalPairs: pairs, routes: K, invPerm: invPerm, tileE: tileE, tileR: tileR, tileCount: tileCount)
+            try QWGemm.encodeMoEComposeRows(enc, hal: hal, sortedPair: sortedPair, pairs: pairs, pairRows: gs.pairRows, rowCount: gpairs, slotOfRow: gInv,
+                                            rowsOut: rows2)
+            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: gs.xLatent16, bank: w.gateUp, experts: E, sortedTok: rows2, expertOff: expOff, tileE: tileE,
+                                             tileR: tileR, tileCount: tileCount, act16: s.act16, pairs: pairs, rotateAct: w.down.isRotated)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: s.act16, bank: w.down, experts: E, expertOff: expOff, tileE: tileE, tileR: tileR,
+                                            tileCount: tileCount, y: dnHi, pairs: pairs)
+            try QWGemm.encodeMoECombineGroupsF32(enc, hal: hal, dnAcc: dnHi, invPerm: invPerm, weights: s.wts, ids: s.idx, labels: gw.latentLabels,
+                                                 tokens: T, routes: K, numGroups: NG, width: L, out: gs.zLatent16)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: gs.zLatent16, bank: gw.latentU, experts: NG, expertOff: gOff, tileE: gTE, tileR: gTR,
+                                            tileCount: gTC, y: upAcc, pairs: gpairs, sortedTok: gPair)
+            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: upAcc, invPerm: gInv, weights: gs.onesRoute, shared: shared, gate: gate,
+                                                     out: out32, hidden: H, routes: NG, tokens: T)
+        } else {
+            try QWGemm.encodeMoERoutedGemv(enc, hal: hal, bank: gw.latentD, experts: NG, x16: x16, xPerToken: true, ids: gs.groupIds, weights: nil,
+                                           tokens: T, routes: NG, out: gs.xLatent16)
+            try QWGemm.encodeMoEGateUpRowsF32R1(enc, hal: hal, x: gs.xLatent16, bank: w.gateUp, experts: E, ids: s.idx, xRows: gs.pairRows, out: s.act16,
+                                                routes: K, tokens: T)
+            try QWGemm.encodeMoEDownGroupsF32(enc, hal: hal, x: s.act16, bank: w.down, experts: E, ids: s.idx, weights: s.wts, labels: gw.latentLabels,
+                                              numGroups: NG, tokens: T, routes: K, out: gs.zLatent16)
+            try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: gs.zLatent16, bank: gw.latentU, experts: NG, routes: NG, weights: gs.onesRoute,
+                                                     shared: shared, gate: gate, out: out32, ids: gs.groupIds, tokens: T)
         }
     }
 }

@@ -393,3 +393,226 @@ def test_combine_identity_slots_and_unit_weights(dev, hidden, dtype):
         rows.free()
     for b in (d_dn, d_w, d_sh, d_g, d_out):
         b.free()
+
+
+# ---- group-latent MoE: the doors and the whole block -------------------------------------------------------------------
+def _latent_routes(rng, t, e, k, ng, hole=True):
+    idx = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+    if hole and t * k > 1:
+        idx[0, k - 1] = -1
+    wts = (rng.random((t, k)) + 0.1).astype(np.float32)
+    labels = rng.integers(0, ng, e).astype(np.int32)
+    return idx, wts, labels
+
+
+@pytest.mark.parametrize("t,e,k,ng", [(1, 32, 4, 4), (7, 100, 8, 8), (300, 128, 8, 32), (5, 16, 2, 1)])
+def test_latent_groups_and_compose_rows(dev, t, e, k, ng):
+    """group ids / latent rows of the routes against the oracle's rule, and the composed gather rows of a second sort."""
+    rng = np.random.default_rng(t + ng)
+    idx, _, labels = _latent_routes(rng, t, e, k, ng)
+    lib, st = dev.lib, dev.stream.handle
+    ib, lb, gb, rb = dev.put(idx), dev.put(labels), dev.alloc(t * ng * 4), dev.alloc(t * k * 4)
+    qwhip.check(lib.qwhip_moe_latent_groups(st, ib.ptr, lb.ptr, t, k, e, ng, gb.ptr, rb.ptr))
+    dev.stream.sync()
+    gids, rows = qo.moe_latent_groups(idx, labels, ng)
+    assert np.array_equal(gb.download(np.int32, (t, ng)), gids)
+    assert np.array_equal(rb.download(np.int32, (t, k)), rows)
+    pairs = t * k
+    sp = rng.permutation(pairs).astype(np.int32)
+    slot = rng.permutation(t * ng).astype(np.int32)
+    slot[gids.ravel() < 0] = -1                                 # rows of absent groups have no slot
+    ob, spb, slb = dev.alloc(pairs * 4), dev.put(sp), dev.put(slot)
+    qwhip.check(lib.qwhip_moe_compose_rows(st, spb.ptr, pairs, rb.ptr, t * ng, slb.ptr, ob.ptr))
+    dev.stream.sync()
+    pr = rows.ravel()[sp]
+    want = np.where(pr >= 0, np.maximum(slot[np.maximum(pr, 0)], 0), 0)
+    assert np.array_equal(ob.download(np.int32, (pairs,)), want)
+    assert lib.qwhip_moe_latent_groups(st, ib.ptr, lb.ptr, t, k, e, 33, gb.ptr, rb.ptr) == qwhip.E_BAD_SHAPE
+
+
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq8_g32", "hq4_g64"])
+@pytest.mark.parametrize("t,ng,lat,hidden", [(1, 4, 64, 256), (3, 8, 96, 512), (8, 4, 40, 1280)])
+def test_routed_gemv_keeps_one_row_per_route(dev, fmt, t, ng, lat, hidden):
+    """out[t, r] = wts * W[idx[t, r]] . x: every route its own output row, one activation row per token or per route, unit
+    weights when none are given, zeros for an absent route."""
+    blocks, w16 = H.make_bank(fmt, ng * lat, hidden, 41)
+    w = w16.reshape(ng, lat, hidden).astype(np.float64)
+    rng = np.random.default_rng(3)
+    ids = np.tile(np.arange(ng, dtype=np.int32), (t, 1))
+    ids[rng.random((t, ng)) < 0.3] = -1
+    wts = (rng.random((t, ng)) + 0.2).astype(np.float32)
+    x_tok = rng.standard_normal((t, hidden)).astype(np.float16)
+    x_rt = rng.standard_normal((t, ng, hidden)).astype(np.float16)
+    lib, st = dev.lib, dev.stream.handle
+    bank, ib, wb = dev.put(blocks), dev.put(ids), dev.put(wts)
+    v = H.view_of(dev, bank, fmt, ng * lat, hidden)
+    for per_token, x, wbuf, odt in ((1, x_tok, None, qwhip.F16), (0, x_rt, wb, qwhip.F32)):
+        out, xb = dev.put(np.full((t, ng, lat), 7, np.float32)), dev.put(x)
+        qwhip.check(lib.qwhip_moe_routed_gemv(st, C.byref(v), ng, xb.ptr, per_token, ib.ptr, wbuf.ptr if wbuf else None, t, ng,
+                                              out.ptr, odt))
+        dev.stream.sync()
+        if odt == qwhip.F16:
+            got = out.download(np.float16, (2 * t * ng * lat,))[: t * ng * lat]
+        else:
+            got = out.download(np.float32, (t * ng * lat,))
+        got = got.reshape(t, ng, lat).astype(np.float64)
+        ref = np.zeros((t, ng, lat))
+        for r in range(t):
+            for g in range(ng):
+                if ids[r, g] >= 0:
+                    xv = (x[r] if per_token else x[r, g]).astype(np.float64)
+                    ref[r, g] = (wts[r, g] if wbuf else 1.0) * (w[ids[r, g]] @ xv)
+        assert qo.normalized_error(got, ref) <= TOL
+        assert np.all(got[ids < 0] == 0)
+
+
+@pytest.mark.parametrize("fmt,gu_flags", [("hq4_g32_m5", 0), ("hq4_g32_m5", 2 << 8), ("hq4_g64", 0)])
+@pytest.mark.parametrize("t,e,k,ng,lat,inter", [(1, 16, 4, 4, 64, 64), (4, 32, 4, 4, 256, 96), (8, 8, 3, 2, 1792, 64)])
+def test_gateup_decode_rows_reads_the_given_rows(dev, fmt, gu_flags, t, e, k, ng, lat, inter):
+    """qwhip_moe_gateup_decode_rows == qwhip_moe_gateup_decode over the gathered rows, bit for bit."""
+    gu_blocks, _ = H.make_bank(fmt, e * 2 * inter, lat, 43)
+    rng = np.random.default_rng(t)
+    idx, _, labels = _latent_routes(rng, t, e, k, ng)
+    _, rows = qo.moe_latent_groups(idx, labels, ng)
+    xl = rng.standard_normal((t * ng, lat)).astype(np.float16)
+    lib, st = dev.lib, dev.stream.handle
+    bank, ib = dev.put(gu_blocks), dev.put(idx)
+    v = H.view_of(dev, bank, fmt, e * 2 * inter, lat)
+    a1, a2 = dev.put(np.full((t * k, inter), 3, np.float16)), dev.put(np.full((t * k, inter), 5, np.float16))
+    flags = qwhip.X_PREROTATED | gu_flags
+    xlb, rwb, gab = dev.put(xl), dev.put(rows), dev.put(xl[np.maximum(rows.ravel(), 0)])
+    qwhip.check(lib.qwhip_moe_gateup_decode_rows(st, C.byref(v), e, xlb.ptr, qwhip.F16, flags, ib.ptr, rwb.ptr, t, k, a1.ptr))
+    qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(v), e, gab.ptr, qwhip.F16, flags, ib.ptr, t * k, 1, a2.ptr))
+    dev.stream.sync()
+    one, two = a1.download(np.float16, (t * k, inter)), a2.download(np.float16, (t * k, inter))
+    assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
+    assert np.any(one != 0) and np.all(one[idx.ravel() < 0] == 0)
+
+
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32"])
+@pytest.mark.parametrize("t,e,k,ng,lat,inter", [(1, 16, 4, 4, 64, 64), (4, 32, 8, 8, 160, 128), (8, 8, 3, 2, 1792, 64)])
+def test_down_decode_groups_sums_the_routes_of_each_group(dev, fmt, t, e, k, ng, lat, inter):
+    dn_blocks, dn16 = H.make_bank(fmt, e * lat, inter, 47)
+    w = dn16.reshape(e, lat, inter).astype(np.float64)
+    rng = np.random.default_rng(ng + t)
+    idx, wts, labels = _latent_routes(rng, t, e, k, ng)
+    act = rng.standard_normal((t, k, inter)).astype(np.float16)
+    lib, st = dev.lib, dev.stream.handle
+    bank = dev.put(dn_blocks)
+    v = H.view_of(dev, bank, fmt, e * lat, inter)
+    out = dev.put(np.full((t, ng, lat), 9, np.float32))
+    ab, ib, wb, lb = dev.put(act), dev.put(idx), dev.put(wts), dev.put(labels)
+    qwhip.check(lib.qwhip_moe_down_decode_groups(st, C.byref(v), e, ab.ptr, ib.ptr, wb.ptr, lb.ptr, ng, t, k, out.ptr, qwhip.F32))
+    dev.stream.sync()
+    got = out.download(np.float32, (t, ng, lat)).astype(np.float64)
+    ref = np.zeros((t, ng, lat))
+    for r in range(t):
+        for j in range(k):
+            if idx[r, j] >= 0:
+                ref[r, labels[idx[r, j]]] += wts[r, j] * (w[idx[r, j]] @ act[r, j].astype(np.float64))
+    assert qo.normalized_error(got, ref) <= TOL
+    gids, _ = qo.moe_latent_groups(idx, labels, ng)
+    assert np.all(got[gids < 0] == 0)
+
+
+@pytest.mark.parametrize("t,k,ng,width,ddt,odt,perm", [(5, 4, 4, 64, "f32", "f16", True), (300, 8, 8, 1792, "f16", "f32", True),
+                                                       (3, 3, 2, 100, "f32", "f32", False)])
+def test_combine_groups(dev, t, k, ng, width, ddt, odt, perm):
+    rng = np.random.default_rng(width)
+    e = 4 * ng
+    idx, wts, labels = _latent_routes(rng, t, e, k, ng)
+    pairs = t * k
+    dn = rng.standard_normal((pairs, width)).astype(np.float32)
+    dnh = dn.astype(np.float16) if ddt == "f16" else dn
+    inv = rng.permutation(pairs).astype(np.int32) if perm else None
+    if perm:
+        inv[idx.ravel() < 0] = -1
+    lib, st = dev.lib, dev.stream.handle
+    out = dev.alloc(t * ng * width * 4)
+    db, pb, wb, ib, lb = dev.put(dnh), (dev.put(inv) if perm else None), dev.put(wts), dev.put(idx), dev.put(labels)
+    qwhip.check(lib.qwhip_moe_combine_groups(st, db.ptr, qwhip.F16 if ddt == "f16" else qwhip.F32, pb.ptr if perm else None,
+                                             wb.ptr, ib.ptr, lb.ptr, t, k, ng, width, out.ptr, qwhip.F16 if odt == "f16" else qwhip.F32))
+    dev.stream.sync()
+    got = out.download(np.float16 if odt == "f16" else np.float32, (t, ng, width)).astype(np.float64)
+    ref = np.zeros((t, ng, width))
+    for r in range(t):
+        for j in range(k):
+            if idx[r, j] < 0:
+                continue
+            slot = int(inv[r * k + j]) if perm else r * k + j
+            ref[r, labels[idx[r, j]]] += float(wts[r, j]) * dnh[slot].astype(np.float64)
+    assert qo.normalized_error(got, ref) <= (2e-3 if odt == "f16" else 1e-6)
+
+
+def _group_latent_block(dev, fmts, t, e, k, ng, hidden, lat, inter, x16, idx, wts, labels, banks):
+    """The block from the doors: decode (t <= 8) through the routed GEMVs, prefill through two pair sorts and the grouped GEMMs."""
+    lib, st = dev.lib, dev.stream.handle
+    f_lat, f_exp = fmts
+    bd, bu, bgu, bdn = dev.put(banks["d"]), dev.put(banks["u"]), dev.put(banks["gu"]), dev.put(banks["dn"])
+    vd = H.view_of(dev, bd, f_lat, ng * lat, hidden)
+    vu = H.view_of(dev, bu, f_lat, ng * hidden, lat)
+    vgu = H.view_of(dev, bgu, f_exp, e * 2 * inter, lat)
+    vdn = H.view_of(dev, bdn, f_exp, e * lat, inter)
+    ones = dev.put(np.ones((t, ng), np.float32))
+    xb, ib, wb, lb = dev.put(x16), dev.put(idx), dev.put(wts), dev.put(labels)
+    gids, rows = dev.alloc(t * ng * 4), dev.alloc(t * k * 4)
+    out = dev.alloc(t * hidden * 4)
+    pairs = t * k
+    qwhip.check(lib.qwhip_moe_latent_groups(st, ib.ptr, lb.ptr, t, k, e, ng, gids.ptr, rows.ptr))
+    act = dev.alloc(pairs * inter * 2)
+    z16 = dev.alloc(t * ng * lat * 2)
+    if t <= 8:
+        xl = dev.alloc(t * ng * lat * 2)
+        qwhip.check(lib.qwhip_moe_routed_gemv(st, C.byref(vd), ng, xb.ptr, 1, gids.ptr, None, t, ng, xl.ptr, qwhip.F16))
+        qwhip.check(lib.qwhip_moe_gateup_decode_rows(st, C.byref(vgu), e, xl.ptr, qwhip.F16, qwhip.X_PREROTATED, ib.ptr, rows.ptr, t, k, act.ptr))
+        qwhip.check(lib.qwhip_moe_down_decode_groups(st, C.byref(vdn), e, act.ptr, ib.ptr, wb.ptr, lb.ptr, ng, t, k, z16.ptr, qwhip.F16))
+        qwhip.check(lib.qwhip_moe_down_decode(st, C.byref(vu), ng, z16.ptr, gids.ptr, ones.ptr, t, ng, None, None, out.ptr, qwhip.F32))
+    else:
+        dev.stream.sync()
+        g1 = _group(dev, gids.download(np.int32, (t, ng)), ng, ng)
+        b1 = g1["bufs"]
+        n1 = t * ng
+        xl = dev.alloc(n1 * lat * 2)
+        qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vd), ng, xb.ptr, qwhip.F16, 0, b1["stok"].ptr, b1["off"].ptr, b1["te"].ptr, b1["tr"].ptr,
+                                               b1["tc"].ptr, g1["max_tiles"], n1, xl.ptr, qwhip.F16, 0))
+        g2 = _group(dev, idx, e, k)
+        b2 = g2["bufs"]
+        rows2 = dev.alloc(pairs * 4)
+        qwhip.check(lib.qwhip_moe_compose_rows(st, b2["sp"].ptr, pairs, rows.ptr, n1, b1["inv"].ptr, rows2.ptr))
+        qwhip.check(lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(vgu), e, xl.ptr, qwhip.F16, 0, rows2.ptr, b2["off"].ptr, b2["te"].ptr, b2["tr"].ptr,
+                                                      b2["tc"].ptr, g2["max_tiles"], pairs, 1, act.ptr, 0))
+        dn = dev.alloc(pairs * lat * 4)
+        qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vdn), e, act.ptr, qwhip.F16, 0, None, b2["off"].ptr, b2["te"].ptr, b2["tr"].ptr,
+                                               b2["tc"].ptr, g2["max_tiles"], pairs, dn.ptr, qwhip.F32, 0))
+        qwhip.check(lib.qwhip_moe_combine_groups(st, dn.ptr, qwhip.F32, b2["inv"].ptr, wb.ptr, ib.ptr, lb.ptr, t, k, ng, lat, z16.ptr, qwhip.F16))
+        yu = dev.alloc(n1 * hidden * 4)
+        qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vu), ng, z16.ptr, qwhip.F16, 0, b1["sp"].ptr, b1["off"].ptr, b1["te"].ptr, b1["tr"].ptr,
+                                               b1["tc"].ptr, g1["max_tiles"], n1, yu.ptr, qwhip.F32, 0))
+        qwhip.check(lib.qwhip_moe_combine(st, yu.ptr, qwhip.F32, b1["inv"].ptr, None, t, ng, hidden, None, None, out.ptr, qwhip.F32))
+    dev.stream.sync()
+    return out.download(np.float32, (t, hidden))
+
+
+@pytest.mark.parametrize("fmts", [("hq8_g32", "hq4_g64"), ("hq4_g32_m5", "hq4_g32_m5")])
+@pytest.mark.parametrize("t,e,k,ng,hidden,lat,inter", [(1, 32, 4, 4, 64, 64, 64), (4, 32, 4, 4, 256, 128, 64), (8, 64, 8, 8, 512, 192, 128),
+                                                       (16, 32, 4, 4, 64, 64, 64), (64, 32, 4, 4, 256, 128, 64), (130, 64, 8, 8, 512, 192, 128)])
+def test_group_latent_block_matches_oracle(dev, fmts, t, e, k, ng, hidden, lat, inter):
+    """latentD -> routed experts in the latent width -> sum by group -> latentU, decode and prefill forms, against
+    moe_group_latent_forward_f64 (the sizes of FNLatentMoETests among them: H = L = I = 64, 32 experts, 4 groups, 4 routes)."""
+    f_lat, f_exp = fmts
+    banks, w = {}, {}
+    banks["d"], w["d"] = H.make_bank(f_lat, ng * lat, hidden, 51)
+    banks["u"], w["u"] = H.make_bank(f_lat, ng * hidden, lat, 52)
+    banks["gu"], w["gu"] = H.make_bank(f_exp, e * 2 * inter, lat, 53)
+    banks["dn"], w["dn"] = H.make_bank(f_exp, e * lat, inter, 54)
+    rng = np.random.default_rng(t * 7 + ng)
+    x16 = qo.rotate_activation_f16(rng.standard_normal((t, hidden)).astype(np.float32))
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    idx, wts = _route(dev, logits, k)
+    labels = (np.arange(e) % ng).astype(np.int32)
+    if t >= 4:
+        labels[idx[1]] = labels[idx[1, 0]]                    # one token with all its routes in one group
+    got = _group_latent_block(dev, fmts, t, e, k, ng, hidden, lat, inter, x16, idx, wts, labels, banks)
+    ref = qo.moe_group_latent_forward_f64(x16, idx, wts, labels, w["d"].reshape(ng, lat, hidden), w["gu"].reshape(e, 2 * inter, lat),
+                                          w["dn"].reshape(e, lat, inter), w["u"].reshape(ng, hidden, lat))
+    assert qo.normalized_error(got, ref) <= TOL

@@ -445,3 +445,54 @@ def test_route_modes_closed_forms():
     nan[0, 5] = np.inf
     idx6, _ = qo.moe_route_ex(nan, 40, False, 1.0, bias=np.zeros(40, np.float32))
     assert 3 not in idx6[0].tolist() and 5 not in idx6[0].tolist() and (idx6[0] == -1).sum() == 2
+
+
+def test_group_latent_block_identities():
+    """moe_group_latent_forward_f64: (1) one group with identity D and U is the plain routed block; (2) without the f16
+    hand-over roundings the grouped sum equals the per-route expansion sum_k w_k U_g(k) down_k(swiglu(gu_k(D_g(k) x)))
+    (U_g is linear, so summing before or after it agrees); (3) swapping the labels of two experts that are not routed
+    changes nothing, relabelling a routed one does; moe_latent_groups marks exactly the labels of the routes."""
+    rng = np.random.default_rng(31)
+    t, e, k, h, lat, inter, ng = 5, 12, 3, 64, 32, 64, 4
+    x = rng.standard_normal((t, h))
+    gu = rng.standard_normal((e, 2 * inter, lat)) * 0.2
+    dn = rng.standard_normal((e, lat, inter)) * 0.2
+    d = rng.standard_normal((ng, lat, h)) * 0.2
+    u = rng.standard_normal((ng, h, lat)) * 0.2
+    idx = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+    idx[1, 2] = -1
+    wts = rng.random((t, k)).astype(np.float32)
+    labels = (np.arange(e) % ng).astype(np.int32)
+    # (1)
+    eye_d, eye_u = np.eye(lat)[None], np.eye(lat)[None]
+    xl = rng.standard_normal((t, lat)).astype(np.float16)
+    one = qo.moe_group_latent_forward_f64(xl, idx, wts, np.zeros(e, np.int32), eye_d, gu, dn, eye_u, latent_f16=False)
+    np.testing.assert_allclose(one, qo.moe_forward_f64(xl, idx, wts, gu, dn, act_f16=True, rotate_act=True), rtol=1e-12, atol=1e-12)
+    # (2)
+    got = qo.moe_group_latent_forward_f64(x, idx, wts, labels, d, gu, dn, u, act_f16=False, rotate_act=False, latent_f16=False)
+    want = np.zeros((t, h))
+    for r in range(t):
+        for j in range(k):
+            ex = int(idx[r, j])
+            if ex < 0:
+                continue
+            g = int(labels[ex])
+            a = gu[ex] @ (d[g] @ x[r])
+            act = a[:inter] / (1.0 + np.exp(-a[:inter])) * a[inter:]
+            want[r] += float(wts[r, j]) * (u[g] @ (dn[ex] @ act))
+    np.testing.assert_allclose(got, want, rtol=1e-10, atol=1e-10)
+    # (3)
+    unused = sorted(set(range(e)) - set(int(v) for v in idx.ravel() if v >= 0))
+    if len(unused) >= 2 and labels[unused[0]] != labels[unused[1]]:
+        l2 = labels.copy()
+        l2[unused[0]], l2[unused[1]] = labels[unused[1]], labels[unused[0]]
+        assert np.array_equal(qo.moe_group_latent_forward_f64(x, idx, wts, l2, d, gu, dn, u), qo.moe_group_latent_forward_f64(x, idx, wts, labels, d, gu, dn, u))
+    l3 = labels.copy()
+    l3[idx[0, 0]] = (labels[idx[0, 0]] + 1) % ng
+    assert not np.allclose(qo.moe_group_latent_forward_f64(x, idx, wts, l3, d, gu, dn, u)[0], qo.moe_group_latent_forward_f64(x, idx, wts, labels, d, gu, dn, u)[0])
+    gids, rows = qo.moe_latent_groups(idx, labels, ng)
+    for r in range(t):
+        have = {int(labels[v]) for v in idx[r] if v >= 0}
+        assert {int(g) for g in gids[r] if g >= 0} == have and all(gids[r, g] in (-1, g) for g in range(ng))
+        for j in range(k):
+            assert rows[r, j] == (-1 if idx[r, j] < 0 else r * ng + labels[idx[r, j]])
