@@ -83,6 +83,17 @@ typedef struct qwhip_caps {
 /* QWHal.init (QWHal.swift:133-232): opens device `ordinal`, refuses a device that is not gfx950. */
 qwhip_status qwhip_device_create(int32_t ordinal, qwhip_device_t* out);
 qwhip_status qwhip_device_destroy(qwhip_device_t dev);
+/* The gated activation every FFN epilogue of this device applies (qwg_swiglu_mul, Sources/QWMetal/include/qw_weight_basis.metalh:48-66),
+ * the counterpart of the reference's pipeline function constants 224 / 228 / 229 that QWHal derives from the model geometry
+ * (QWHal+Constants.swift:60-75): kind 0 = SwiGLU silu(g) * u (the default); 1 = SwiGLU with g <= p0 and |u| <= p0 (swigluLimit);
+ * 2 = the bounded form p0 tanh(g / p0) sigmoid(g) * p1 tanh(u / p1) (activationKind .situ(beta: p0, linearBeta: p1); p1 <= 0
+ * leaves u as it is).  Applies to launches enqueued afterwards on every stream of the device: qwhip_swiglu_fwht,
+ * qwhip_silu_mul_f32, qwhip_gemm_swiglu, qwhip_moe_grouped_gemm_swiglu, qwhip_gemv_silu_pair, qwhip_moe_gateup_decode*
+ * and qwhip_moe_route_gateup_decode.  Set it once after qwhip_device_create, as the reference builds its pipelines once. */
+#define QWHIP_ACT_SWIGLU 0u
+#define QWHIP_ACT_SWIGLU_CLAMPED 1u
+#define QWHIP_ACT_BOUNDED 2u
+qwhip_status qwhip_device_set_gated_activation(qwhip_device_t dev, uint32_t kind, float p0, float p1);
 qwhip_status qwhip_device_caps(qwhip_device_t dev, qwhip_caps* out);
 /* hal.begin() / hal.end() (QWHal.swift:325-378): a stream is the encoder the launchers take. */
 qwhip_status qwhip_stream_create(qwhip_device_t dev, qwhip_stream_t* out);

@@ -846,3 +846,23 @@ def moe_group_latent_forward_f64(x, idx, wts, labels, latent_d_w, gate_up_w, dow
         for g in xin:
             out[r] += latent_u_w[g].astype(np.float64) @ r16(z[g])
     return out
+
+
+# --------------------------------------------------------------------------- #
+# generalized gated FFN activation  (pinned by limits: tests/test_oracle_math.py)
+# --------------------------------------------------------------------------- #
+def gated_act(gate, up, kind: int = 0, p0: float = 0.0, p1: float = 0.0) -> np.ndarray:
+    """qwg_swiglu_mul (Sources/QWMetal/include/qw_weight_basis.metalh:48-66) in fp64: kind 0 silu(g) * u; kind 1 the same
+    with g <= p0 and |u| <= p0 (QW_FC_SWIGLU_LIMIT); kind 2 p0 tanh(g / p0) sigmoid(g) * p1 tanh(u / p1), u as it is when
+    p1 <= 0 (QW_FC_SITU_BETA / QW_FC_SITU_LIN_BETA; the reference's own restatement: situRef,
+    Tests/QWGEMMTests/QWErnie55MoETests.swift:120-125)."""
+    g = np.asarray(gate, dtype=np.float64)
+    u = np.asarray(up, dtype=np.float64)
+    if kind == 2:
+        gg = p0 * np.tanh(g / p0) / (1.0 + np.exp(-g))
+        uu = p1 * np.tanh(u / p1) if p1 > 0 else u
+        return gg * uu
+    if kind == 1:
+        g = np.minimum(g, p0)
+        u = np.clip(u, -p0, p0)
+    return g / (1.0 + np.exp(-g)) * u

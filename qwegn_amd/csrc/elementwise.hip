@@ -103,7 +103,7 @@ extern "C" qwhip_status qwhip_cast_f32_to_f16(qwhip_stream_t s, const float* src
 // f16 rounding on store.
 template <int DT, bool ROT>
 __global__ __launch_bounds__(256) void qw_swiglu_fwht_kernel(const void* __restrict__ gu, h1_t* __restrict__ act,
-                                                              uint32_t rows, uint32_t inter) {
+                                                              uint32_t rows, uint32_t inter, const qw_act ga) {
     const uint32_t gpr = inter / 32;  // groups per row
     const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (uint64_t)rows * gpr) return;
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void qw_swiglu_fwht_kernel(const void* __restr
         qw_load8_f32<DT>(gu, gbase + 8 * j, a);
         qw_load8_f32<DT>(gu, gbase + inter + 8 * j, b);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[8 * j + e] = qw_swiglu(a[e], b[e]);
+        for (int e = 0; e < 8; ++e) v[8 * j + e] = qw_gated(a[e], b[e], ga);
     }
     if (ROT) qw_fwht32(v);
     h1_t* o = act + (uint64_t)r * inter + 32 * g;
@@ -132,13 +132,13 @@ __global__ __launch_bounds__(256) void qw_swiglu_fwht_kernel(const void* __restr
 // Ragged tail (inter % 32 != 0): one thread per element, never rotated.
 template <int DT>
 __global__ __launch_bounds__(256) void qw_swiglu_scalar_kernel(const void* __restrict__ gu, h1_t* __restrict__ act,
-                                                                uint32_t rows, uint32_t inter) {
+                                                                uint32_t rows, uint32_t inter, const qw_act ga) {
     const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (uint64_t)rows * inter) return;
     const uint32_t r = (uint32_t)(i / inter), c = (uint32_t)(i % inter);
     const float g = qw_load_f32<DT>(gu, (uint64_t)r * 2 * inter + c);
     const float u = qw_load_f32<DT>(gu, (uint64_t)r * 2 * inter + inter + c);
-    act[i] = (h1_t)qw_swiglu(g, u);
+    act[i] = (h1_t)qw_gated(g, u, ga);
 }
 
 extern "C" qwhip_status qwhip_swiglu_fwht(qwhip_stream_t s, const void* gu, uint32_t gu_dtype, void* act_f16,
@@ -155,17 +155,17 @@ extern "C" qwhip_status qwhip_swiglu_fwht(qwhip_stream_t s, const void* gu, uint
         const dim3 grid((unsigned)((n + 255) / 256)), block(256);
         if (inter % 32 == 0 && rotate)
             return qwhip_fail(QWHIP_E_BAD_SHAPE, "swiglu: rotated output needs 16-byte aligned buffers");
-        if (gu_dtype == QWHIP_F16) hipLaunchKernelGGL(qw_swiglu_scalar_kernel<QWHIP_F16>, grid, block, 0, s->stream, gu, act, rows, inter);
-        else hipLaunchKernelGGL(qw_swiglu_scalar_kernel<QWHIP_F32>, grid, block, 0, s->stream, gu, act, rows, inter);
+        if (gu_dtype == QWHIP_F16) hipLaunchKernelGGL(qw_swiglu_scalar_kernel<QWHIP_F16>, grid, block, 0, s->stream, gu, act, rows, inter, s->dev->act);
+        else hipLaunchKernelGGL(qw_swiglu_scalar_kernel<QWHIP_F32>, grid, block, 0, s->stream, gu, act, rows, inter, s->dev->act);
     } else {
         const uint64_t groups = (uint64_t)rows * (inter / 32);
         const dim3 grid((unsigned)((groups + 255) / 256)), block(256);
         if (gu_dtype == QWHIP_F16) {
-            if (rotate) hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F16, true>), grid, block, 0, s->stream, gu, act, rows, inter);
-            else hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F16, false>), grid, block, 0, s->stream, gu, act, rows, inter);
+            if (rotate) hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F16, true>), grid, block, 0, s->stream, gu, act, rows, inter, s->dev->act);
+            else hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F16, false>), grid, block, 0, s->stream, gu, act, rows, inter, s->dev->act);
         } else {
-            if (rotate) hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F32, true>), grid, block, 0, s->stream, gu, act, rows, inter);
-            else hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F32, false>), grid, block, 0, s->stream, gu, act, rows, inter);
+            if (rotate) hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F32, true>), grid, block, 0, s->stream, gu, act, rows, inter, s->dev->act);
+            else hipLaunchKernelGGL((qw_swiglu_fwht_kernel<QWHIP_F32, false>), grid, block, 0, s->stream, gu, act, rows, inter, s->dev->act);
         }
     }
     QWHIP_TRY_HIP(hipGetLastError());
@@ -237,7 +237,7 @@ extern "C" qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_v
 // silu(gate) * up in fp32, then the 32-point transform, fp32 out (qwg_silu_mul_f32, Sources/QWMetal/gemm/qwgemm_f32.metal:291-317;
 // door QWGemm.encodeSiluMulF32, Sources/Operators/QWGEMM/QWGemmF32.swift:83-94).  gu fp32 [rows, 2 inter], inter % 32 == 0.
 __global__ __launch_bounds__(256) void qw_silu_mul_f32_kernel(const float* __restrict__ gu, float* __restrict__ act, uint32_t rows,
-                                                               uint32_t inter) {
+                                                               uint32_t inter, const qw_act ga) {
     const uint64_t gi = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     const uint32_t gpr = inter / 32u;
     if (gi >= (uint64_t)rows * gpr) return;
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(256) void qw_silu_mul_f32_kernel(const float* __res
     for (int j = 0; j < 8; ++j) {
         const f4_t a = gp[j], b = up[j];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[4 * j + e] = qw_swiglu(a[e], b[e]);
+        for (int e = 0; e < 4; ++e) v[4 * j + e] = qw_gated(a[e], b[e], ga);
     }
     qw_fwht32(v);
     f4_t* o = (f4_t*)(act + (uint64_t)r * inter + 32u * g);
@@ -265,7 +265,7 @@ extern "C" qwhip_status qwhip_silu_mul_f32(qwhip_stream_t s, const float* gu, fl
     if (inter == 0 || inter % 32u != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "f32 silu-mul needs intermediate %% 32 == 0, got %u", inter);
     if (((uintptr_t)gu | (uintptr_t)act) & 15u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "f32 silu-mul needs 16-byte aligned buffers");
     const uint64_t groups = (uint64_t)rows * (inter / 32u);
-    hipLaunchKernelGGL(qw_silu_mul_f32_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s->stream, gu, act, rows, inter);
+    hipLaunchKernelGGL(qw_silu_mul_f32_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s->stream, gu, act, rows, inter, s->dev->act);
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }

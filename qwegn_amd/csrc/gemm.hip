@@ -43,6 +43,7 @@ struct qw_gemm_params {
     const int32_t* tile_count;
     uint32_t rows_per_expert;
     uint32_t inter, rotate_act;  // fused SwiGLU epilogue: gate rows [0, inter), up rows [inter, 2 inter) of an expert; FWHT-32 on the result
+    qw_act act;                  // the device's gated activation (all zero: SwiGLU)
     uint32_t force_gemm2;  // tuning / tests: keep the DMA-fed kernel for the 256 x 320 shape
     uint32_t x_bf16;       // ping-pong kernel: activations are bf16, converted while the tile is staged
 };
@@ -425,7 +426,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm2_kernel(const qw_gemm_p
 // bit-identical to qwhip_gemm with f16 output followed by qwhip_swiglu_fwht.
 // XDT = bf16: the activation tile is converted to f16 on its way from the load registers into LDS (12 vector operations
 // per 16-byte piece, inside the filling phase), so bf16 activations need no pass of their own and no workspace.
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false, int XDT = QWHIP_F16>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false, int XDT = QWHIP_F16, bool GACT = false>
 __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_params p) {
     static_assert(WVM * WVN == 8, "two groups of four waves");
     static_assert(!SWIGLU || (WVN == 2 && YDT == QWHIP_F16), "fused SwiGLU: gate and up wave columns, f16 out");
@@ -717,7 +718,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
                     const h8_t u8 = *(const h8_t*)(us + row * EP_PITCH + cc * 16u);
                     float v[8];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) v[e] = qw_swiglu((float)g8[e], (float)u8[e]);
+                    for (int e = 0; e < 8; ++e) v[e] = GACT ? qw_gated((float)g8[e], (float)u8[e], p.act) : qw_swiglu((float)g8[e], (float)u8[e]);
                     if (p.rotate_act) {
 #pragma unroll
                         for (int h = 1; h < 8; h <<= 1)
@@ -802,7 +803,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 // qwhip_swiglu_fwht on the f16 gate|up matrix without writing it (the reference's fused form for its dense path:
 // qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167).
 // ------------------------------------------------------------------------------------------------
-template <int FMT, int YDT, bool SWIGLU>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
 __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
     static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
     constexpr uint32_t BM = 64, BN = 256, STAGE = BM * 128u;
@@ -926,7 +927,7 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float g = (float)(h1_t)acc[a][0][r], u = (float)(h1_t)acc[a][1][r];
-                float v = qw_swiglu(g, u);
+                float v = GACT ? qw_gated(g, u, p.act) : qw_swiglu(g, u);
                 if (p.rotate_act) v = qw_fwht32_lanes(v, fw_signs) * QW_INV_SQRT32;
                 *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
             }
@@ -998,7 +999,7 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 // four workgroups per CU.  The raw image of K pair kp + 1 is in flight (registers) during K pair kp and replaces the
 // stage between two barriers at its end.
 // ------------------------------------------------------------------------------------------------
-template <int FMT, int YDT, bool SWIGLU>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void qw_gemm5_kernel(const qw_gemm_params p) {
     static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
     static_assert(FMT == QG_FMT_M5 || FMT == QG_FMT_B4, "20-byte blocks: HQ4_G32_M5 and the 4-bit group-32 bit streams");
@@ -1149,7 +1150,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float g = (float)(h1_t)acc[a][0][r], u = (float)(h1_t)acc[a][1][r];
-                float v = qw_swiglu(g, u);
+                float v = GACT ? qw_gated(g, u, p.act) : qw_swiglu(g, u);
                 if (p.rotate_act) v = qw_fwht32_lanes(v, fw_signs) * QW_INV_SQRT32;
                 *(h1_t*)(ep + w_off + (8u * (r >> 2) + (r & 3)) * EP_PITCH) = (h1_t)v;
             }
@@ -1249,11 +1250,11 @@ hipError_t launch_cfg2(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false, int XDT = QWHIP_F16>
+template <int WM, int WN, int WVM, int WVN, int FMT, int YDT, bool SWIGLU = false, int XDT = QWHIP_F16, bool GACT = false>
 hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr int BM = 32 * WM * WVM, BN = 32 * WN * WVN;
     constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, SWIGLU, XDT>;
+    auto kern = qw_gemm3_kernel<WM, WN, WVM, WVN, FMT, YDT, SWIGLU, XDT, GACT>;
     static std::atomic<bool> attr_done{false};  // per instantiation
     if (!attr_done.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1264,20 +1265,20 @@ hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
-template <int FMT, int YDT, bool SWIGLU>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
 hipError_t launch_cfg4(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     // two activation stages, or the four epilogue slabs (32 rows x (128 + 16) bytes each) when they are larger
     constexpr size_t lds = 4u * 32u * 144u;
     static_assert(lds >= 2u * 64u * 128u, "the stages fit the slab allocation");
-    hipLaunchKernelGGL((qw_gemm4_kernel<FMT, YDT, SWIGLU>), grid, dim3(256), lds, st, p);
+    hipLaunchKernelGGL((qw_gemm4_kernel<FMT, YDT, SWIGLU, GACT>), grid, dim3(256), lds, st, p);
     return hipGetLastError();
 }
 
-template <int FMT, int YDT, bool SWIGLU>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
 hipError_t launch_cfg5(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr size_t lds = 2u * 64u * 128u + 256u * 88u;   // two activation stages + one raw K-pair image (38,912 bytes)
     if constexpr (FMT == QG_FMT_M5 || FMT == QG_FMT_B4) {
-        hipLaunchKernelGGL((qw_gemm5_kernel<FMT, YDT, SWIGLU>), grid, dim3(256), lds, st, p);
+        hipLaunchKernelGGL((qw_gemm5_kernel<FMT, YDT, SWIGLU, GACT>), grid, dim3(256), lds, st, p);
         return hipGetLastError();
     } else {
         return hipErrorInvalidValue;   // not reached: gemm5_takes() refuses the 8-bit containers
@@ -1576,15 +1577,19 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     p.row_bytes = qwhip_view_row_bytes(w);
     p.inter = inter;
     p.rotate_act = rotate_act ? 1u : 0u;
+    p.act = s->dev->act;
     p.tiles_m = qwhip_cdiv(m, 256u);
     p.tiles_n = qwhip_cdiv(inter, 160u);
     const dim3 grid(((p.tiles_m * p.tiles_n + 7u) / 8u) * 8u);
     hipError_t e;
+    // the plain SwiGLU epilogue keeps its own instantiation: the general activation's code costs it 3 % at this size
+    const bool ga = p.act.kind != 0u;
     switch (fmt) {
-        case QG_FMT_M5: e = launch_cfg3<2, 5, 4, 2, QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid); break;
-        case QG_FMT_B4: e = launch_cfg3<2, 5, 4, 2, QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid); break;
-        case QG_FMT_B2: e = launch_cfg3<2, 5, 4, 2, QG_FMT_B2, QWHIP_F16, true>(s->stream, p, grid); break;
-        case QG_FMT_B3: e = launch_cfg3<2, 5, 4, 2, QG_FMT_B3, QWHIP_F16, true>(s->stream, p, grid); break;
+#define QG_SWIGLU3(F) \
+    case F: e = ga ? launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true, QWHIP_F16, true>(s->stream, p, grid) \
+                   : launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true>(s->stream, p, grid); break;
+        QG_SWIGLU3(QG_FMT_M5) QG_SWIGLU3(QG_FMT_B4) QG_SWIGLU3(QG_FMT_B2) QG_SWIGLU3(QG_FMT_B3)
+#undef QG_SWIGLU3
         default: e = hipErrorInvalidValue;
     }
     QWHIP_TRY_HIP(e);
@@ -1723,12 +1728,19 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     p.rows_per_expert = rows_per_expert;
     p.inter = inter;
     p.rotate_act = rotate_act ? 1u : 0u;
+    p.act = s->dev->act;
     p.tiles_n = qwhip_cdiv(inter, 128u);
     const dim3 grid(8u * qwhip_cdiv(max_tiles, 8u) * p.tiles_n);   // XCD-aware one-dimensional grid over (tile, column tile)
     hipError_t e;
-    if (gemm5_takes(p, fmt)) e = fmt == QG_FMT_M5 ? launch_cfg5<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid)
-                                                  : launch_cfg5<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
-    else {
+    const bool ga = p.act.kind != 0u;   // the plain SwiGLU epilogue keeps its own instantiation
+    if (gemm5_takes(p, fmt)) {
+        if (ga) e = fmt == QG_FMT_M5 ? launch_cfg5<QG_FMT_M5, QWHIP_F16, true, true>(s->stream, p, grid)
+                                     : launch_cfg5<QG_FMT_B4, QWHIP_F16, true, true>(s->stream, p, grid);
+        else e = fmt == QG_FMT_M5 ? launch_cfg5<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid)
+                                  : launch_cfg5<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
+    } else if (ga) {
+        QG_FOR_FMT(fmt, e, (launch_cfg4<F, QWHIP_F16, true, true>(s->stream, p, grid)))
+    } else {
         QG_FOR_FMT(fmt, e, (launch_cfg4<F, QWHIP_F16, true>(s->stream, p, grid)))
     }
     QWHIP_TRY_HIP(e);

@@ -375,6 +375,7 @@ struct qw_gemv_params {
     uint32_t x_div;         // down: pairs that share one activation row (0 and 1: a row per pair)
     const int32_t* labels;  // down, num_groups > 0: group of every expert; blockIdx.y = token * num_groups + group and
     uint32_t num_groups;    // only the token's routes into that group are summed
+    qw_act act;             // gate|up pair mode: the device's gated activation (all zero: SwiGLU)
     // transposing kernel: waves per row set, row sets per workgroup, K ranges
     uint32_t wpr, sets, nkr;
 };
@@ -477,7 +478,7 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_pa
                     u += red[w2][RT + t][lane];
                 }
 #pragma unroll
-                for (int r = 0; r < 4; ++r) actbuf[i][16 * t + 4 * c + r] = qw_swiglu(g[r], u[r]);
+                for (int r = 0; r < 4; ++r) actbuf[i][16 * t + 4 * c + r] = qw_gated(g[r], u[r], p.act);
             }
         }
         __syncthreads();
@@ -967,7 +968,7 @@ bool qw_stream_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, u
 // moe_col.hip
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
                        bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
-                       const float* logits = nullptr, int32_t* idx_out = nullptr, float* wts_out = nullptr, uint32_t norm_topk = 0,
+                       const qw_act act, const float* logits = nullptr, int32_t* idx_out = nullptr, float* wts_out = nullptr, uint32_t norm_topk = 0,
                        float routed_scale = 1.0f, const int32_t* x_rows = nullptr);
 bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* act16, const int32_t* idx,
                      const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
@@ -1174,7 +1175,7 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     // activation row (flags bits 8..11 = 2 keep the general kernel, for tests)
     if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
         hipError_t e = hipSuccess;
-        if (qw_moe_gateup_col(s->stream, w, 1, x, x_dtype, rotate, rotate_out && inter % 32 == 0, nullptr, m, 1, act16, &e)) {
+        if (qw_moe_gateup_col(s->stream, w, 1, x, x_dtype, rotate, rotate_out && inter % 32 == 0, nullptr, m, 1, act16, &e, s->dev->act)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }
@@ -1192,6 +1193,7 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     a.row_bytes = qwhip_view_row_bytes(w);
     a.rotate = rotate ? 1u : 0u;
     a.rot_out = (rotate_out && inter % 32 == 0) ? 1u : 0u;
+    a.act = s->dev->act;
     const size_t lds_x = (size_t)m * ((size_t)w->k * 2u + 16u);
     const int xm = (rotate && lds_x <= 48u * 1024u) ? QW_XM_LDS_ROT : QW_XM_GLOBAL;
     const size_t lds = xm == QW_XM_LDS_ROT ? lds_x : 0;
@@ -1233,7 +1235,7 @@ extern "C" qwhip_status qwhip_moe_route_gateup_decode(qwhip_stream_t s, const qw
         const bool rotate = qwhip_view_rotated(w_gate_up) && !(flags & QWHIP_X_PREROTATED);
         hipError_t e = hipSuccess;
         if (qw_moe_gateup_col(s->stream, w_gate_up, experts, x, x_dtype, rotate, qwhip_view_rotated(w_gate_up) && inter % 32 == 0, nullptr,
-                              t * top_k, top_k, act16, &e, logits, idx, wts, norm_topk ? 1u : 0u, scale)) {
+                              t * top_k, top_k, act16, &e, s->dev->act, logits, idx, wts, norm_topk ? 1u : 0u, scale)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }
@@ -1264,7 +1266,7 @@ static qwhip_status qw_moe_gateup_decode_impl(qwhip_stream_t s, const qwhip_weig
     if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
         hipError_t e = hipSuccess;
         if (qw_moe_gateup_col(s->stream, w_gate_up, experts, x, x_dtype, rotate, qwhip_view_rotated(w_gate_up) && inter % 32 == 0,
-                              idx, t * top_k, top_k, act16, &e, nullptr, nullptr, nullptr, 0, 1.0f, x_rows)) {
+                              idx, t * top_k, top_k, act16, &e, s->dev->act, nullptr, nullptr, nullptr, 0, 1.0f, x_rows)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }
@@ -1283,6 +1285,7 @@ static qwhip_status qw_moe_gateup_decode_impl(qwhip_stream_t s, const qwhip_weig
     a.rot_out = (qwhip_view_rotated(w_gate_up) && inter % 32 == 0) ? 1u : 0u;
     a.idx = idx;
     a.x_rows = x_rows;
+    a.act = s->dev->act;
     a.top_k = top_k;
     a.expert_bytes = (uint64_t)2 * inter * a.row_bytes;
     const size_t lds_x = (size_t)w_gate_up->k * 2u + 16u;

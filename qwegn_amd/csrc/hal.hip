@@ -80,6 +80,16 @@ extern "C" qwhip_status qwhip_device_create(int32_t ordinal, qwhip_device_t* out
     return QWHIP_OK;
 }
 
+extern "C" qwhip_status qwhip_device_set_gated_activation(qwhip_device_t dev, uint32_t kind, float p0, float p1) {
+    QWHIP_REQUIRE(dev);
+    if (kind > 2u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "gated activation %u is not one of 0 SwiGLU, 1 clamped SwiGLU, 2 bounded (tanh) form", kind);
+    if (kind != 0u && !(p0 > 0.0f)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "gated activation %u needs a positive first parameter", kind);
+    dev->act.kind = kind;
+    dev->act.p0 = kind ? p0 : 0.0f;
+    dev->act.p1 = kind == 2u ? p1 : 0.0f;
+    return QWHIP_OK;
+}
+
 extern "C" qwhip_status qwhip_device_destroy(qwhip_device_t dev) {
     delete dev;
     return QWHIP_OK;

@@ -60,6 +60,7 @@ struct qmc_gu_params {
     h1_t* act;
     const int32_t* idx;
     const int32_t* x_rows;   // activation row of every pair (NULL: the pair's token)
+    qw_act ga;               // the device's gated activation (all zero: SwiGLU)
     uint32_t I, nb, cpr, top_k, rotate, rot_out;
     uint64_t expert_bytes;
     // JN > 0: the routing is done here.  The first wave of every workgroup routes the pair's token from its router logits
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
             gsum += part[o32 * cpr + c];
             usum += part[(32u + o32) * cpr + c];
         }
-        float a = qw_swiglu(gsum, usum);
+        float a = qw_gated(gsum, usum, p.ga);
         // the butterfly order of the serial transform (pairs h apart: lower = a + b, upper = a - b), across lanes by DPP
         if (p.rot_out && n0 + 32u <= I) a = qw_fwht32_lanes(a, qw_fwht32_lane_signs(o32)) * QW_INV_SQRT32;
         if (tid < 32u && n0 + tid < I) act[n0 + tid] = (h1_t)a;
@@ -199,7 +200,7 @@ struct qmc_dn_params {
     uint32_t num_groups;     // expert carries that group's label are summed
 };
 
-template <int ODT, int D>
+template <int ODT, int D, bool GRP = false>   // GRP: one output row per (token, latent group)
 __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_params p) {
     __shared__ float part[1024];   // [sets * D rows][cprv]
     const uint32_t tid = threadIdx.x;
@@ -207,8 +208,8 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
     const uint32_t cprv = p.cprv, H = p.H;
     const uint32_t set = hw / cprv, chunk = hw - set * cprv;
     const uint32_t tok = blockIdx.y, n0 = blockIdx.x * (p.sets * D);   // tok: the output row
-    const uint32_t src = p.num_groups ? tok / p.num_groups : tok;
-    const int32_t grp = p.num_groups ? (int32_t)(tok - src * p.num_groups) : 0;
+    const uint32_t src = GRP ? tok / p.num_groups : tok;
+    const int32_t grp = GRP ? (int32_t)(tok - src * p.num_groups) : 0;
     const uint32_t v0 = chunk * 32u + lane;
     const bool vvalid = v0 < p.nbv;
     const uint32_t v = vvalid ? v0 : 0u;
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
     const int32_t e = p.idx[pair];
     const float wk = p.wts ? p.wts[pair] : 1.0f;
     bool valid = vvalid && e >= 0;
-    if (p.num_groups) valid = valid && p.labels[valid ? ((uint32_t)e & 0xFFFFu) : 0u] == grp;
+    if constexpr (GRP) valid = valid && p.labels[valid ? ((uint32_t)e & 0xFFFFu) : 0u] == grp;
     const uint32_t row_bytes = p.nbI * 20u;
     // activations do not wait for the expert id; the weight rows follow as soon as it is known
     h8_t xr[4];
@@ -229,8 +230,12 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
 #pragma unroll
     for (int j = 0; j < D; ++j) {
         const uint32_t n = min(n0 + set * D + j, H - 1u);
-        buf[j] = qw_hq4_block{};
-        if (valid) buf[j] = *(const qw_hq4_block*)(base + (uint64_t)n * row_bytes);   // lanes of other groups' routes read nothing
+        if constexpr (GRP) {   // lanes of other groups' routes read nothing
+            buf[j] = qw_hq4_block{};
+            if (valid) buf[j] = *(const qw_hq4_block*)(base + (uint64_t)n * row_bytes);
+        } else {
+            buf[j] = *(const qw_hq4_block*)(base + (uint64_t)n * row_bytes);
+        }
     }
     h2_t xo[16];
     const float S = qmc_operands(xr, xo);
@@ -263,7 +268,7 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
 // is outside the kernel's envelope (the caller then takes the general kernel).
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
                        bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
-                       const float* logits, int32_t* idx_out, float* wts_out, uint32_t norm_topk, float routed_scale,
+                       const qw_act act, const float* logits, int32_t* idx_out, float* wts_out, uint32_t norm_topk, float routed_scale,
                        const int32_t* x_rows) {
     if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
     const uint32_t inter = w->n / (2u * experts);
@@ -279,6 +284,7 @@ bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expe
     p.act = (h1_t*)act16;
     p.idx = idx;
     p.x_rows = x_rows;
+    p.ga = act;
     p.I = inter;
     p.nb = nb;
     p.cpr = cpr;
@@ -345,10 +351,16 @@ bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expert
     p.labels = labels;
     p.num_groups = num_groups;
     const dim3 grid(qwhip_cdiv(hidden, sets * D), out_rows), block(32u * cprv * sets);
-    if (out_dtype == QWHIP_F32) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_F32, D>), grid, block, 0, st, p);
-    else if (out_dtype == QWHIP_F16) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_F16, D>), grid, block, 0, st, p);
-    else if (out_dtype == QWHIP_BF16) hipLaunchKernelGGL((qw_moe_down_col_kernel<QWHIP_BF16, D>), grid, block, 0, st, p);
+#define QMC_DN(OD)                                                                                            \
+    do {                                                                                                      \
+        if (num_groups) hipLaunchKernelGGL((qw_moe_down_col_kernel<OD, D, true>), grid, block, 0, st, p);     \
+        else hipLaunchKernelGGL((qw_moe_down_col_kernel<OD, D, false>), grid, block, 0, st, p);               \
+    } while (0)
+    if (out_dtype == QWHIP_F32) QMC_DN(QWHIP_F32);
+    else if (out_dtype == QWHIP_F16) QMC_DN(QWHIP_F16);
+    else if (out_dtype == QWHIP_BF16) QMC_DN(QWHIP_BF16);
     else return false;
+#undef QMC_DN
     *err = hipGetLastError();
     return true;
 }

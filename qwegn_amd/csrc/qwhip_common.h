@@ -5,9 +5,17 @@
 
 #include "../../include/qwhip.h"
 
+// The gated activation of the FFN epilogues, a device-wide constant like the reference's function constants 224 / 228 / 229
+// (QWHal+Constants.swift:60-75): kind 0 SwiGLU, 1 SwiGLU with gate <= p0 and |up| <= p0, 2 the bounded form
+// p0 tanh(g / p0) sigmoid(g) * p1 tanh(u / p1) (p1 <= 0: up as it is).
+struct qw_act {
+    uint32_t kind;
+    float p0, p1;
+};
 struct qwhip_device_s {
     int ordinal;
     hipDeviceProp_t prop;
+    qw_act act;
 };
 // Partial-sum scratch of the split-K verify GEMV: owned by the stream (allocated when the stream is created, never inside a
 // launcher), so launches on different streams never share it and launches on one stream use it one after the other.
@@ -141,6 +149,20 @@ __device__ __forceinline__ void qw_fwht32(float* v) {
 // SwiGLU on fp32: silu(g) * u = g / (1 + exp(-g)) * u  (qwg_swiglu_mul, plain branch,
 // Sources/QWMetal/include/qw_weight_basis.metalh:50-63).
 __device__ __forceinline__ float qw_swiglu(float g, float u) { return (g / (1.0f + __expf(-g))) * u; }
+// The generalized gated activation (qwg_swiglu_mul, all three branches, Sources/QWMetal/include/qw_weight_basis.metalh:48-66);
+// `a` is uniform over a launch.
+__device__ __forceinline__ float qw_gated(float g, float u, const qw_act a) {
+    if (a.kind == 2u) {
+        const float gg = a.p0 * tanhf(g / a.p0) * (1.0f / (1.0f + __expf(-g)));
+        const float uu = a.p1 > 0.0f ? a.p1 * tanhf(u / a.p1) : u;
+        return gg * uu;
+    }
+    if (a.kind == 1u) {
+        g = fminf(g, a.p0);
+        u = fminf(fmaxf(u, -a.p0), a.p0);
+    }
+    return qw_swiglu(g, u);
+}
 
 // FWHT-32 over the 32 lanes of a half wavefront (lane j = lane & 31 holds element j), un-normalised, stage order
 // h = 1, 2, 4, 8, 16 with v' = (j & h) == 0 ? v + o : o - v, o = the value of lane j ^ h: the arithmetic of the butterfly

@@ -194,6 +194,21 @@ public:
     }
     void free(void* p) { qwhip_free(dev_, p); }
     qwhip_device_t device() const { return dev_; }
+    // The geometry's gated FFN activation, which the reference bakes into its pipelines as function constants 224 / 228 / 229
+    // (QWHal+Constants.swift:60-75; QWModelDescriptor.ActivationKind, QWModelDescriptor+Hybrid.swift:182-186)
+    struct ActivationKind {
+        enum Kind { swiglu, swigluClamped, situ } kind = swiglu;
+        float a = 0.0f, b = 0.0f;   // swigluClamped: the limit; situ: beta, linearBeta
+        static ActivationKind swiGLU() { return {}; }
+        static ActivationKind clamped(float limit) { return {swigluClamped, limit, 0.0f}; }
+        static ActivationKind situAndMul(float beta, float linearBeta) { return {situ, beta, linearBeta}; }
+    };
+    void setActivation(const ActivationKind& k) {
+        throwIfFailed(qwhip_device_set_gated_activation(dev_, k.kind == ActivationKind::situ ? QWHIP_ACT_BOUNDED
+                                                              : k.kind == ActivationKind::swigluClamped ? QWHIP_ACT_SWIGLU_CLAMPED
+                                                                                                        : QWHIP_ACT_SWIGLU,
+                                                        k.a, k.b));
+    }
 
 private:
     qwhip_device_t dev_ = nullptr;

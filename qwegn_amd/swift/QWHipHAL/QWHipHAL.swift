@@ -37,6 +37,16 @@ public final class QWHal: @unchecked Sendable {
         device = d!
         qwhip_device_caps(device, &caps)
     }
+    /// The geometry's gated FFN activation: what QWHal+Constants.swift:60-75 bakes into every pipeline as function constants
+    /// 224 (swigluLimit) and 228 / 229 (activationKind .situ(beta:linearBeta:)) is one device-wide setting here.
+    public convenience init(geometry: QWModelGeometry, ordinal: Int32 = 0) throws {
+        try self.init(ordinal: ordinal)
+        if case let .situ(beta, linearBeta) = geometry.descriptor.activationKind {
+            try qwCheck(qwhip_device_set_gated_activation(device, UInt32(QWHIP_ACT_BOUNDED), beta, linearBeta))
+        } else if let limit = geometry.swigluLimit, limit > 0 {
+            try qwCheck(qwhip_device_set_gated_activation(device, UInt32(QWHIP_ACT_SWIGLU_CLAMPED), Float(limit), 0))
+        }
+    }
     deinit { qwhip_device_destroy(device) }
     /// hal.pipeline(name): the kernel-name table of the library; throws kernelMissing like the metallib lookup.
     public func pipeline(_ name: String) throws { try qwCheck(qwhip_kernel_lookup(name, nil)) }

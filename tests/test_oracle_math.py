@@ -496,3 +496,29 @@ def test_group_latent_block_identities():
         assert {int(g) for g in gids[r] if g >= 0} == have and all(gids[r, g] in (-1, g) for g in range(ng))
         for j in range(k):
             assert rows[r, j] == (-1 if idx[r, j] < 0 else r * ng + labels[idx[r, j]])
+
+
+def test_gated_activation_limits():
+    """gated_act: kind 0 is swiglu; a clamp beyond every input changes nothing, a gate above the limit acts as the limit and up
+    saturates at +-limit; the bounded form tends to SwiGLU for large parameters (x - beta tanh(x / beta) ~ x^3 / (3 beta^2)),
+    is bounded by beta * linear_beta, keeps the sign structure, and equals its textbook value at a hand-computed point."""
+    import math
+    rng = np.random.default_rng(17)
+    g, u = rng.standard_normal(500) * 3, rng.standard_normal(500) * 3
+    base = qo.swiglu(g, u).astype(np.float64)
+    np.testing.assert_allclose(qo.gated_act(g, u), base, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(qo.gated_act(g, u, 1, 100.0), qo.gated_act(g, u), rtol=0, atol=0)
+    lim = 1.5
+    got = qo.gated_act(np.array([0.5, 9.0, 9.0, -4.0]), np.array([7.0, -7.0, 0.25, 0.5]), 1, lim)
+    silu = lambda v: v / (1.0 + math.exp(-v))
+    np.testing.assert_allclose(got, [silu(0.5) * lim, silu(lim) * -lim, silu(lim) * 0.25, silu(-4.0) * 0.5], rtol=1e-12)
+    far = qo.gated_act(g, u, 2, 1e4, 1e4)
+    np.testing.assert_allclose(far, qo.gated_act(g, u), rtol=1e-6, atol=1e-9)
+    b, lb = 4.0, 25.0
+    big = qo.gated_act(np.array([50.0, -50.0, 50.0]), np.array([1e3, 1e3, -1e3]), 2, b, lb)
+    np.testing.assert_allclose(big, [b * lb, 0.0, -b * lb], rtol=1e-9, atol=1e-12)
+    assert np.all(np.abs(qo.gated_act(g * 10, u * 10, 2, b, lb)) <= b * lb)
+    one = qo.gated_act(np.array([2.0]), np.array([-3.0]), 2, b, lb)[0]
+    want = (b * math.tanh(2.0 / b) / (1.0 + math.exp(-2.0))) * (lb * math.tanh(-3.0 / lb))
+    assert abs(one - want) <= 1e-14 and abs(want - (-4.8611)) < 1e-3      # 4 tanh(.5) = 1.8485, sigmoid(2) = .8808, 25 tanh(-.12) = -2.9857: 1.8485 * .8808 * -2.9857
+    np.testing.assert_allclose(qo.gated_act(g, u, 2, b, 0.0), b * np.tanh(g / b) / (1 + np.exp(-g)) * u, rtol=1e-12)
