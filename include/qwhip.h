@@ -392,6 +392,15 @@ qwhip_status qwhip_moe_down_decode(qwhip_stream_t s, const qwhip_weight_view* w_
                                    uint32_t top_k, const float* shared, const float* shared_gate, void* out,
                                    uint32_t out_dtype);
 
+/* encodeFnMoeRoute(expertBudget:) (QWGemmMoERouter.swift:63-75) -> the normTopK & 4 branch of qwg_moe_route_decode
+ * (Sources/QWMetal/subsystems/qwrouter.metal:193-268): after qwhip_moe_route* over a verify window of rows = 2..4 (rows * top_k <= 64),
+ * at most max(top_k, budget) distinct experts stay.  Row 0 keeps its routes; the other (row, route) pairs are admitted expert by
+ * expert in the order of their weights (ties: the lower pair index); the rest get idx -1 and weight 0 (every door skips such a
+ * route), and with norm_topk a later row that lost weight is rescaled to its former sum.  budget 0 or >= rows * top_k: no-op.
+ * In place on idx / wts [rows, top_k]. */
+qwhip_status qwhip_moe_route_budget(qwhip_stream_t s, int32_t* idx, float* wts, uint32_t rows, uint32_t top_k, uint32_t budget,
+                                    uint32_t norm_topk);
+
 /* ---- group-latent MoE (QWMoEOperator.encodeResidentGroupLatent, Sources/Operators/QWGEMM/QWMoEOperator+GroupLatent.swift:11-294)
  * Every expert carries the label of one of num_groups (1..32) latent groups.  A token's routes read D_g . x of their
  * expert's group (bank latentD [num_groups * latent, hidden]), run the expert in the latent width, are summed by group

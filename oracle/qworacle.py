@@ -866,3 +866,59 @@ def gated_act(gate, up, kind: int = 0, p0: float = 0.0, p1: float = 0.0) -> np.n
         g = np.minimum(g, p0)
         u = np.clip(u, -p0, p0)
     return g / (1.0 + np.exp(-g)) * u
+
+
+def moe_route_budget(idx: np.ndarray, wts: np.ndarray, budget: int, norm_topk: bool = True):
+    """Expert budget over a verify window of 2..4 routed rows (the `normTopK & 4` branch of qwg_moe_route_decode,
+    Sources/QWMetal/subsystems/qwrouter.metal:193-268): row 0 keeps its routes, the other pairs are admitted expert by expert
+    in the order of their weights (ties to the lower pair index) until max(top_k, budget) distinct experts are in, the rest
+    get idx -1 and weight 0; with norm_topk a later row that lost weight is rescaled to its former sum (fp32)."""
+    idx = np.array(idx, dtype=np.int32)
+    wts = np.array(wts, dtype=np.float32)
+    m, k = idx.shape
+    total = m * k
+    if budget <= 0 or budget >= total:
+        return idx, wts
+    b = max(k, budget)
+    ids, w = idx.ravel().copy(), wts.ravel().copy()
+    orig = [np.float32(0)] * m
+    for r in range(m):
+        s = np.float32(0)
+        for j in range(k):
+            s = np.float32(s + w[r * k + j])
+        orig[r] = s
+    keep = [p < k for p in range(total)]
+    unique = 0
+    for s in range(k):
+        e = int(ids[s])
+        if e < 0 or any(int(ids[p]) == e for p in range(s)):
+            continue
+        unique += 1
+        for p in range(total):
+            if int(ids[p]) == e:
+                keep[p] = True
+    while unique < b:
+        cand = [float(w[p]) if (not keep[p] and ids[p] >= 0) else -1.0 for p in range(total)]
+        best = max(cand)
+        if best < 0:
+            break
+        win = cand.index(best)
+        for p in range(total):
+            if ids[p] == ids[win]:
+                keep[p] = True
+        unique += 1
+    out_i, out_w = ids.copy(), w.copy()
+    for p in range(total):
+        if not keep[p]:
+            out_i[p], out_w[p] = -1, np.float32(0)
+    if norm_topk:
+        for r in range(1, m):
+            now = np.float32(0)
+            for j in range(k):
+                if out_w[r * k + j] > 0:
+                    now = np.float32(now + out_w[r * k + j])
+            if now > 0 and now < np.float32(orig[r] * np.float32(0.9999)):
+                scale = np.float32(orig[r] / now)
+                for j in range(k):
+                    out_w[r * k + j] = np.float32(out_w[r * k + j] * scale)
+    return out_i.reshape(m, k), out_w.reshape(m, k)

@@ -660,3 +660,83 @@ extern "C" qwhip_status qwhip_moe_combine_groups(qwhip_stream_t s, const void* d
     }
     return QWHIP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// Expert budget over a verify window (the normTopK & 4 branch of qwg_moe_route_decode,
+// Sources/QWMetal/subsystems/qwrouter.metal:193-268; door: encodeFnMoeRoute(expertBudget:), QWGemmMoERouter.swift:63-75):
+// after the routing of 2..4 rows, at most `budget` distinct experts stay.  Row 0 keeps its routes; the other pairs are
+// admitted expert by expert in the order of their weights (ties: the lower pair index) until `budget` distinct experts are in;
+// the rest lose their route (idx -1, weight 0), and with `norm` every later row that lost weight is rescaled to its old sum.
+// One wavefront, lane p = pair p (rows * top_k <= 64).
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void qw_moe_route_budget_kernel(int32_t* __restrict__ idx, float* __restrict__ wts, uint32_t M, uint32_t K,
+                                                                  uint32_t B, uint32_t norm) {
+    __shared__ int32_t ids[64];
+    __shared__ float ws[64];
+    const uint32_t lane = threadIdx.x, total = M * K;
+    const int32_t id = lane < total ? idx[lane] : -1;
+    const float w = lane < total ? wts[lane] : -1.0f;
+    ids[lane] = id;
+    ws[lane] = w;
+    __syncthreads();
+    float orig = 0.0f;   // lane r < M: the row's weight sum before pruning, added in route order
+    if (norm && lane < M)
+        for (uint32_t k = 0; k < K; ++k) orig += ws[lane * K + k];
+    bool keep = lane < K;
+    uint32_t unique = 0;
+    for (uint32_t s = 0; s < K; ++s) {   // uniform over the wave
+        const int32_t e = ids[s];
+        if (e < 0) continue;
+        bool dup = false;
+        for (uint32_t prev = 0; prev < s; ++prev) dup = dup || ids[prev] == e;
+        if (!dup) {
+            ++unique;
+            if (id == e) keep = true;
+        }
+    }
+    while (unique < B) {
+        const float cand = (!keep && id >= 0) ? w : -1.0f;
+        float best = cand;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) best = fmaxf(best, __shfl_xor(best, d, 64));
+        if (best < 0.0f) break;
+        const unsigned long long hit = __ballot(cand == best);
+        const uint32_t win = (uint32_t)__builtin_ctzll(hit);
+        if (win >= total) break;
+        const int32_t we = ids[win];
+        if (id == we) keep = true;
+        ++unique;
+    }
+    const bool pruned = lane < total && !keep;
+    if (pruned) {
+        idx[lane] = -1;
+        wts[lane] = 0.0f;
+    }
+    __syncthreads();
+    ws[lane] = pruned ? 0.0f : w;
+    __syncthreads();
+    if (norm && lane >= 1u && lane < M) {
+        float now = 0.0f;
+        for (uint32_t k = 0; k < K; ++k) {
+            const float v = ws[lane * K + k];
+            if (v > 0.0f) now += v;
+        }
+        if (now > 0.0f && now < orig * 0.9999f) {
+            const float scale = orig / now;
+            for (uint32_t k = 0; k < K; ++k) wts[lane * K + k] = ws[lane * K + k] * scale;
+        }
+    }
+}
+
+extern "C" qwhip_status qwhip_moe_route_budget(qwhip_stream_t s, int32_t* idx, float* wts, uint32_t rows, uint32_t top_k, uint32_t budget,
+                                               uint32_t norm_topk) {
+    QWHIP_REQUIRE(s);
+    QWHIP_REQUIRE(idx);
+    QWHIP_REQUIRE(wts);
+    if (rows < 2u || rows > 4u || top_k == 0 || top_k > 16u || rows * top_k > 64u)
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "expert budget: a window of 2..4 rows of at most 16 routes (rows=%u top_k=%u)", rows, top_k);
+    if (budget == 0 || budget >= rows * top_k) return QWHIP_OK;   // nothing to prune
+    hipLaunchKernelGGL(qw_moe_route_budget_kernel, dim3(1), dim3(64), 0, s->stream, idx, wts, rows, top_k, max(top_k, budget), norm_topk ? 1u : 0u);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}

@@ -570,7 +570,8 @@ struct QWGemm {
     // replaces the routed scale per selected expert
     static void encodeFnMoeRoute(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& logits, const QWTensorValue& idx,
                                  const QWTensorValue& wts, int rows, int experts, int topK, bool normTopK, float routedScale = 1.0f,
-                                 const QWTensorValue* bias = nullptr, bool splitFeature = false, const QWTensorValue* routedScaleParam = nullptr) {
+                                 const QWTensorValue* bias = nullptr, bool splitFeature = false, const QWTensorValue* routedScaleParam = nullptr,
+                                 int expertBudget = 0) {
         if (experts > 512 || topK > 16 || topK <= 0) throw QWGemmError(QWGemmError::badShape, "router holds 512 experts and 16 routes");
         if (idx.shape.elementCount < (size_t)rows * (size_t)topK || wts.shape.elementCount < (size_t)rows * (size_t)topK)
             throw QWGemmError(QWGemmError::badShape, "router outputs are short");
@@ -588,6 +589,10 @@ struct QWGemm {
                                              routedScaleParam ? (const float*)routedScaleParam->ptr() : nullptr, (int32_t*)idx.ptr(),
                                              (float*)wts.ptr()));
         }
+        // the expert budget of a verify window (QWGemmMoERouter.swift:63-75): the door's own condition, silently skipped otherwise
+        if (expertBudget > 0 && rows > 1 && rows <= 4 && expertBudget < rows * topK && rows * topK <= 64)
+            throwIfFailed(qwhip_moe_route_budget(enc.stream, (int32_t*)idx.ptr(), (float*)wts.ptr(), (uint32_t)rows, (uint32_t)topK,
+                                                 (uint32_t)expertBudget, normTopK ? 1 : 0));
     }
     // encodeMoEGroupPairsF32 (QWGemmMoE.swift:68-99)
     static void encodeMoEGroupPairsF32(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& ids, const QWTensorValue& expertOff,

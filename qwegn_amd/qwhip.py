@@ -96,6 +96,7 @@ SIGNATURES = {
     "qwhip_moe_route_gateup_decode": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _U32, _U32, _U32, C.c_float, _P, _P, _P]),
     "qwhip_moe_down_decode": (C.c_int32, [_P, _WV, _U32, _P, _P, _P, _U32, _U32, _P, _P, _P, _U32]),
     "qwhip_device_set_gated_activation": (C.c_int32, [_P, _U32, C.c_float, C.c_float]),
+    "qwhip_moe_route_budget": (C.c_int32, [_P, _P, _P, _U32, _U32, _U32, _U32]),
     "qwhip_moe_latent_groups": (C.c_int32, [_P, _P, _P, _U32, _U32, _U32, _U32, _P, _P]),
     "qwhip_moe_routed_gemv": (C.c_int32, [_P, _WV, _U32, _P, _U32, _P, _P, _U32, _U32, _P, _U32]),
     "qwhip_moe_gateup_decode_rows": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _P, _U32, _U32, _P]),

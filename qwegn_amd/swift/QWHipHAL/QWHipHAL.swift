@@ -342,11 +342,15 @@ public enum QWGemm {
     /// encodeFnMoeRoute (QWGemmMoERouter.swift:10-75): softmax top-k (or the sigmoid / bias / split-feature modes).
     public static func encodeFnMoeRoute(_ enc: QWHipEncoder, hal: QWHal, logits: QWTensorValue, idx: QWTensorValue, wts: QWTensorValue,
                                         rows: Int, experts: Int, topK: Int, normTopK: Bool, routedScale: Float = 1, bias: QWTensorValue? = nil,
-                                        splitFeature: Bool = false, routedScaleParam: QWTensorValue? = nil) throws {
+                                        splitFeature: Bool = false, routedScaleParam: QWTensorValue? = nil, expertBudget: Int = 0) throws {
         precondition(experts <= 512 && topK <= 16, "route: experts <= 512, K <= 16")
         try hal.pipeline("qwg_moe_route")
         try qwCheck(qwhip_moe_route_ex(enc.stream, logits.f32, UInt32(rows), UInt32(experts), UInt32(topK), normTopK ? 1 : 0, routedScale,
                                        splitFeature ? 1 : 0, bias?.f32, routedScaleParam?.f32, idx.i32, wts.f32))
+        if expertBudget > 0 && rows > 1 && rows <= 4 && expertBudget < rows * topK && rows * topK <= 64 {      // QWGemmMoERouter.swift:63-75
+            try hal.pipeline("qwg_moe_route_decode")
+            try qwCheck(qwhip_moe_route_budget(enc.stream, idx.i32, wts.f32, UInt32(rows), UInt32(topK), UInt32(expertBudget), normTopK ? 1 : 0))
+        }
     }
     /// encodeMoEGroupPairsF32 (QWGemmMoE.swift:68-99): counting sort of the (token, route) pairs by expert + tile list.
     public static func encodeMoEGroupPairsF32(_ enc: QWHipEncoder, hal: QWHal, ids: QWTensorValue, expertOff: QWTensorValue,

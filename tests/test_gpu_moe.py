@@ -616,3 +616,30 @@ def test_group_latent_block_matches_oracle(dev, fmts, t, e, k, ng, hidden, lat, 
     ref = qo.moe_group_latent_forward_f64(x16, idx, wts, labels, w["d"].reshape(ng, lat, hidden), w["gu"].reshape(e, 2 * inter, lat),
                                           w["dn"].reshape(e, lat, inter), w["u"].reshape(ng, hidden, lat))
     assert qo.normalized_error(got, ref) <= TOL
+
+
+@pytest.mark.parametrize("m,k,e,budget,norm", [(2, 8, 32, 10, 1), (4, 16, 64, 20, 1), (3, 4, 8, 6, 0), (4, 8, 128, 9, 1), (2, 4, 16, 2, 1), (4, 16, 512, 40, 1)])
+def test_route_budget_matches_oracle(dev, m, k, e, budget, norm):
+    """The expert budget of a verify window: ids identical to the oracle, weights to 1e-6; duplicates across rows, ties and a
+    route already empty included; no-op and refused shapes."""
+    rng = np.random.default_rng(m * 100 + k)
+    lg = rng.standard_normal((m, e)).astype(np.float32)
+    lg[1] = lg[0] + rng.standard_normal(e).astype(np.float32) * 0.05          # row 1 shares most experts with row 0
+    idx, wts = _route(dev, lg, k)
+    if m > 2:
+        idx[2, k - 1], wts[2, k - 1] = -1, 0.0
+        wts[2, 0] = wts[m - 1, 1]                                              # a tie between two candidates
+    ib, wb = dev.put(idx), dev.put(wts)
+    lib, st = dev.lib, dev.stream.handle
+    qwhip.check(lib.qwhip_moe_route_budget(st, ib.ptr, wb.ptr, m, k, budget, norm))
+    dev.stream.sync()
+    gi, gw = ib.download(np.int32, (m, k)), wb.download(np.float32, (m, k))
+    ri, rw = qo.moe_route_budget(idx, wts, budget, bool(norm))
+    assert np.array_equal(gi, ri)
+    np.testing.assert_allclose(gw, rw, rtol=1e-6, atol=0)
+    assert np.array_equal(gi[0], idx[0]) and len({int(v) for v in gi.ravel() if v >= 0}) <= max(k, budget)
+    qwhip.check(lib.qwhip_moe_route_budget(st, ib.ptr, wb.ptr, m, k, m * k, norm))   # nothing to prune
+    dev.stream.sync()
+    assert np.array_equal(ib.download(np.int32, (m, k)), gi)
+    assert lib.qwhip_moe_route_budget(st, ib.ptr, wb.ptr, 5, 4, 3, 1) == qwhip.E_BAD_SHAPE
+    assert lib.qwhip_moe_route_budget(st, ib.ptr, wb.ptr, 1, 4, 3, 1) == qwhip.E_BAD_SHAPE

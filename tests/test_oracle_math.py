@@ -522,3 +522,35 @@ def test_gated_activation_limits():
     want = (b * math.tanh(2.0 / b) / (1.0 + math.exp(-2.0))) * (lb * math.tanh(-3.0 / lb))
     assert abs(one - want) <= 1e-14 and abs(want - (-4.8611)) < 1e-3      # 4 tanh(.5) = 1.8485, sigmoid(2) = .8808, 25 tanh(-.12) = -2.9857: 1.8485 * .8808 * -2.9857
     np.testing.assert_allclose(qo.gated_act(g, u, 2, b, 0.0), b * np.tanh(g / b) / (1 + np.exp(-g)) * u, rtol=1e-12)
+
+
+def test_route_budget_rules():
+    """moe_route_budget: a hand-worked window, the invariants the reference's test asserts (row 0 never pruned, at most `budget`
+    distinct experts, pruned routes weigh nothing: Tests/QWGEMMTests/QWErnie55MoETests.swift:332-343), renormalised rows keep their
+    sum, and the no-op cases."""
+    idx = np.array([[5, 2], [7, 2], [9, 4]], np.int32)
+    wts = np.array([[0.6, 0.4], [0.7, 0.3], [0.55, 0.45]], np.float32)
+    # row 0 holds {5, 2}; budget 3 admits the heaviest other pair: (1, 0) -> expert 7; experts 9 and 4 go
+    i3, w3 = qo.moe_route_budget(idx, wts, 3, norm_topk=False)
+    assert i3.tolist() == [[5, 2], [7, 2], [-1, -1]] and w3.tolist() == [[np.float32(0.6), np.float32(0.4)], [np.float32(0.7), np.float32(0.3)], [0.0, 0.0]]
+    # budget 4: 7 (0.7) then 9 (0.55); expert 4 is pruned and row 2 is rescaled to its old sum 1.0
+    i4, w4 = qo.moe_route_budget(idx, wts, 4, norm_topk=True)
+    assert i4.tolist() == [[5, 2], [7, 2], [9, -1]]
+    np.testing.assert_allclose(w4[2], [1.0, 0.0], rtol=1e-6)
+    np.testing.assert_allclose(w4[:2], wts[:2], rtol=0)
+    # a budget below top_k still keeps row 0 whole
+    i1, _ = qo.moe_route_budget(idx, wts, 1, norm_topk=False)
+    assert i1.tolist() == [[5, 2], [-1, 2], [-1, -1]]
+    rng = np.random.default_rng(2)
+    for m, k, e, b in [(2, 8, 32, 10), (4, 16, 64, 20), (3, 4, 8, 6), (4, 8, 128, 9)]:
+        lg = rng.standard_normal((m, e)).astype(np.float32)
+        ids, w = qo.moe_route(lg, k, True)
+        bi, bw = qo.moe_route_budget(ids, w, b, norm_topk=True)
+        assert np.array_equal(bi[0], ids[0]) and np.array_equal(bw[0], w[0])
+        assert len({int(v) for v in bi.ravel() if v >= 0}) <= max(k, b)
+        assert np.all(bw[bi < 0] == 0) and np.all((bi == ids) | (bi == -1))
+        for r in range(1, m):
+            if np.any(bi[r] >= 0):
+                assert abs(float(bw[r].sum()) - float(w[r].sum())) <= 2e-6
+    same_i, same_w = qo.moe_route_budget(idx, wts, 6)
+    assert np.array_equal(same_i, idx) and np.array_equal(same_w, wts)
