@@ -225,6 +225,13 @@ qwhip_status qwhip_h32_f32(qwhip_stream_t s, const float* x, float* out, uint32_
 qwhip_status qwhip_head_argmax(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                uint32_t flags, float* logits, int32_t* tokens);
 qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens);
+/* QWGemm.encodeArgmaxFin with a QWVariationalAcceptance (QWGemmF32.swift:276-307) -> qwg_head_argmax_fin_variational
+ * (Sources/QWMetal/head_sampling/qwhead.metal:271-345), over the logits of a verify window: row r (r + 1 < total_rows) takes
+ * draft_tokens[r + 1] instead of its argmax when that token is in the vocabulary, differs from the argmax, its logit is
+ * >= max - margin and, for a finite min_log_prob, log softmax(row)[draft] >= min_log_prob (-inf: no probability gate).
+ * margin <= 0 or a single row: the plain argmax, as the door decides.  draft_tokens: u32 [total_rows]. */
+qwhip_status qwhip_argmax_f32_variational(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, const uint32_t* draft_tokens,
+                                          uint32_t total_rows, float margin, float min_log_prob, int32_t* tokens);
 
 /* ---- fp32 seams of the MoE operator chain ------------------------------------ */
 /* QWGemm.encodeSiluMulF32 (Sources/Operators/QWGEMM/QWGemmF32.swift:83-94) -> qwg_silu_mul_f32
@@ -298,6 +305,11 @@ qwhip_status qwhip_moe_route_ex(qwhip_stream_t s, const float* logits, uint32_t 
 
 /* qwg_router_gemm (qwrouter.metal:460-; encodeFnRouterGemm, QWGemmMoERouter.swift:78-113):
  * logits[t, e] = sum_h x[t, h] * Wr[e, h]; x f16/bf16/f32, Wr f32/f16/bf16, fp32 accumulate. */
+/* QWGemm.encodeF32Gemv (QWGemmF32.swift:117-141) -> qwg_f32_gemv / qwg_f32_gemv_bm (qwgemm_f32.metal:120-143): dense fp32
+ * weights w [n, k], fp32 rows x [rows, k]: y[t, n] = epilogue(w[n] . x[t]); epi 0 none, 1 silu(y / scale), 2 sigmoid(y),
+ * 3 2 sigmoid(y / scale).  k up to 16384. */
+qwhip_status qwhip_f32_gemv(qwhip_stream_t s, const float* w, const float* x, uint32_t rows, uint32_t n, uint32_t k,
+                            uint32_t epi, float scale, float* y);
 qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
                                uint32_t t, uint32_t experts, uint32_t hidden, float* logits);
 /* The same launch with the shared-expert gate column (encodeFnRouterGemm's shGateWeight / shGateOut,

@@ -922,3 +922,51 @@ def moe_route_budget(idx: np.ndarray, wts: np.ndarray, budget: int, norm_topk: b
                 for j in range(k):
                     out_w[r * k + j] = np.float32(out_w[r * k + j] * scale)
     return out_i.reshape(m, k), out_w.reshape(m, k)
+
+
+# --------------------------------------------------------------------------- #
+# consumers of the head and the dense fp32 GEMV  (pinned by closed forms: tests/test_oracle_math.py)
+# --------------------------------------------------------------------------- #
+def head_argmax_variational(logits: np.ndarray, draft_tokens, margin: float, min_log_prob: float = -np.inf) -> np.ndarray:
+    """Relaxed acceptance of a draft over a verify window (qwg_head_argmax_fin_variational,
+    Sources/QWMetal/head_sampling/qwhead.metal:271-345): row r takes draft_tokens[r + 1] instead of its argmax when the draft is in
+    the vocabulary, is not the argmax, logit(draft) >= max - margin and - for a finite min_log_prob - its log-probability
+    (logit - max - log sum exp(logits - max)) reaches min_log_prob."""
+    lg = np.asarray(logits, dtype=np.float32)
+    rows, vocab = lg.shape
+    out = head_argmax(lg).astype(np.int64)
+    draft = np.asarray(draft_tokens, dtype=np.int64)
+    if not margin > 0:
+        return out
+    for r in range(rows):
+        if r + 1 >= len(draft):
+            continue
+        d = int(draft[r + 1])
+        if not (0 <= d < vocab) or d == out[r]:
+            continue
+        mx = np.float64(lg[r, out[r]])
+        dl = np.float64(lg[r, d])
+        if not dl >= mx - np.float64(np.float32(margin)):
+            continue
+        if np.isfinite(min_log_prob):
+            finite = lg[r][np.isfinite(lg[r]) | (lg[r] == -np.inf)].astype(np.float64)
+            lp = (dl - mx) - np.log(np.sum(np.exp(finite - mx)))
+            if lp >= min_log_prob:
+                out[r] = d
+        else:
+            out[r] = d
+    return out
+
+
+def f32_gemv(w: np.ndarray, x: np.ndarray, epi: int = 0, scale: float = 1.0) -> np.ndarray:
+    """Dense fp32-weight GEMV with its scalar epilogues in fp64 (qwg_f32_gemv, Sources/QWMetal/gemm/qwgemm_f32.metal:120-143):
+    0 none, 1 silu(y / scale), 2 sigmoid(y), 3 2 sigmoid(y / scale)."""
+    y = np.asarray(x, dtype=np.float64) @ np.asarray(w, dtype=np.float64).T
+    if epi == 1:
+        z = y / scale
+        return z / (1.0 + np.exp(-z))
+    if epi == 2:
+        return 1.0 / (1.0 + np.exp(-y))
+    if epi == 3:
+        return 2.0 / (1.0 + np.exp(-(y / scale)))
+    return y

@@ -638,7 +638,13 @@ __device__ __forceinline__ uint32_t qw_sortable_f32(float x) {
 // per thread (a strict "greater" per element; NaN is never greater) and builds the 64-bit keys only to combine the 1024
 // thread results.  That is exact unless the row's maximum is a zero (+0.0 beats -0.0 in the key order, they are equal as
 // floats) or no element is greater than -inf (only -inf and NaN): those rows take the key sweep over every element.
-__global__ __launch_bounds__(1024) void qw_argmax_rows_kernel(const float* __restrict__ logits, uint32_t n, int32_t* __restrict__ tokens) {
+// VAR: the relaxed acceptance of a draft (qwg_head_argmax_fin_variational, Sources/QWMetal/head_sampling/qwhead.metal:271-345):
+// row r takes draft[r + 1] instead of its argmax when that token's logit is within `margin` of the maximum and, for a finite
+// min_log_prob, log softmax(draft) >= min_log_prob (the sum of exponentials runs only for such a candidate).
+template <bool VAR>
+__global__ __launch_bounds__(1024) void qw_argmax_rows_kernel(const float* __restrict__ logits, uint32_t n, int32_t* __restrict__ tokens,
+                                                               const uint32_t* __restrict__ draft, uint32_t total_rows, float margin,
+                                                               float min_log_prob) {
     __shared__ unsigned long long best_w[16];
     __shared__ uint32_t slow_path;
     constexpr uint32_t U = 8;   // 16-byte loads in flight per thread
@@ -698,7 +704,48 @@ __global__ __launch_bounds__(1024) void qw_argmax_rows_kernel(const float* __res
         __syncthreads();   // best_w is reused
         fold();
     }
-    if (tid == 0u) tokens[blockIdx.x] = (int32_t)~(uint32_t)best;
+    if constexpr (!VAR) {
+        if (tid == 0u) tokens[blockIdx.x] = (int32_t)~(uint32_t)best;
+    } else {
+        __shared__ uint32_t gate, cand;
+        __shared__ float part_w[16];
+        const uint32_t out_tok = ~(uint32_t)best, kh = (uint32_t)(best >> 32);
+        const float mx_logit = __uint_as_float((kh & 0x80000000u) ? (kh ^ 0x80000000u) : ~kh);
+        float draft_logit = 0.0f;
+        if (tid == 0u) {
+            uint32_t tok = out_tok, g = 0u;
+            if (margin > 0.0f && blockIdx.x + 1u < total_rows) {
+                const uint32_t d = draft[blockIdx.x + 1u];
+                if (d < n && d != out_tok) {
+                    draft_logit = row[d];
+                    if (draft_logit >= mx_logit - margin) {
+                        if (__builtin_isfinite(min_log_prob)) {
+                            g = 1u;
+                            cand = d;
+                        } else {
+                            tok = d;
+                        }
+                    }
+                }
+            }
+            gate = g;
+            if (g == 0u) tokens[blockIdx.x] = (int32_t)tok;
+        }
+        __syncthreads();
+        if (gate == 0u) return;   // uniform over the workgroup
+        float part = 0.0f;
+        for (uint32_t i = tid; i < n; i += 1024u) part += expf(row[i] - mx_logit);
+        part = qw_reduce64(part);
+        if ((tid & 63u) == 0u) part_w[tid >> 6] = part;
+        __syncthreads();
+        if (tid == 0u) {
+            float total = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) total += part_w[w];
+            const float log_prob = (draft_logit - mx_logit) - logf(total);
+            tokens[blockIdx.x] = (int32_t)(log_prob >= min_log_prob ? cand : out_tok);
+        }
+    }
 }
 
 extern "C" qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, int32_t* tokens) {
@@ -707,7 +754,24 @@ extern "C" qwhip_status qwhip_argmax_f32(qwhip_stream_t s, const float* logits, 
     QWHIP_REQUIRE(logits);
     QWHIP_REQUIRE(tokens);
     if (n == 0 || n >= (1u << 30)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "argmax over %u logits does not fit the row-count flags", n);
-    hipLaunchKernelGGL(qw_argmax_rows_kernel, dim3(rows), dim3(1024), 0, s->stream, logits, n, tokens);
+    hipLaunchKernelGGL(qw_argmax_rows_kernel<false>, dim3(rows), dim3(1024), 0, s->stream, logits, n, tokens, nullptr, 0u, 0.0f, 0.0f);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
+}
+
+extern "C" qwhip_status qwhip_argmax_f32_variational(qwhip_stream_t s, const float* logits, uint32_t rows, uint32_t n, const uint32_t* draft_tokens,
+                                                     uint32_t total_rows, float margin, float min_log_prob, int32_t* tokens) {
+    QWHIP_REQUIRE(s);
+    if (rows == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(logits);
+    QWHIP_REQUIRE(tokens);
+    if (n == 0 || n >= (1u << 30)) return qwhip_fail(QWHIP_E_BAD_SHAPE, "argmax over %u logits does not fit the row-count flags", n);
+    if (!(margin > 0.0f) || rows < 2u || total_rows < 2u)   // the door's own rule (QWGemmF32.swift:292): plain argmax otherwise
+        return qwhip_argmax_f32(s, logits, rows, n, tokens);
+    QWHIP_REQUIRE(draft_tokens);
+    if (min_log_prob != min_log_prob) return qwhip_fail(QWHIP_E_BAD_SHAPE, "min_log_prob is NaN (-inf switches the probability gate off)");
+    hipLaunchKernelGGL(qw_argmax_rows_kernel<true>, dim3(rows), dim3(1024), 0, s->stream, logits, n, tokens, draft_tokens, total_rows, margin,
+                       min_log_prob);
     QWHIP_TRY_HIP(hipGetLastError());
     return QWHIP_OK;
 }

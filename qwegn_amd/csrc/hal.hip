@@ -324,6 +324,10 @@ static const qw_kernel_entry g_kernels[] = {
     {"qwg_silu_mul_f16", "qwhip_swiglu_fwht"},
     {"qwg_silu_mul_split_f16", "qwhip_swiglu_fwht"},
     {"qwg_moe_route", "qwhip_moe_route"},
+    {"qwg_f32_gemv", "qwhip_f32_gemv"},
+    {"qwg_f32_gemv_bm", "qwhip_f32_gemv"},
+    {"qwg_head_argmax_fin", "qwhip_argmax_f32"},
+    {"qwg_head_argmax_fin_variational", "qwhip_argmax_f32_variational"},
     {"qwg_moe_route_decode", "qwhip_moe_route"},
     {"qwg_router_gemm", "qwhip_router_gemm"},
     {"qwg_embed_aq_f32", "qwhip_embed_aq_f32"},

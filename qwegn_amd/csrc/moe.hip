@@ -13,10 +13,23 @@
 // sh_out[t] = sigmoid(x[t] . sh_w), the extra output column of the reference's router kernels
 // (Sources/QWMetal/subsystems/qwrouter.metal:467-483,566-574,587-633).
 // ------------------------------------------------------------------------------------------------
+// The scalar epilogues of the dense f32 GEMV door (qwg_f32_gemv, Sources/QWMetal/gemm/qwgemm_f32.metal:120-143):
+// 0 none, 1 silu(y / scale), 2 sigmoid(y), 3 2 sigmoid(y / scale).
+__device__ __forceinline__ float qw_f32_gemv_epilogue(float y, uint32_t epi, float scale) {
+    if (epi == 1u) {
+        const float z = y / scale;
+        return z / (1.0f + expf(-z));
+    }
+    if (epi == 2u) return 1.0f / (1.0f + expf(-y));
+    if (epi == 3u) return 2.0f / (1.0f + expf(-(y / scale)));
+    return y;
+}
+
 template <int XDT, int WDT, int TT>
 __global__ __launch_bounds__(256) void qw_router_gemm_kernel(const void* __restrict__ x, const void* __restrict__ wr,
                                                               float* __restrict__ logits, uint32_t T, uint32_t E, uint32_t H,
-                                                              const float* __restrict__ sh_w, float* __restrict__ sh_out) {
+                                                              const float* __restrict__ sh_w, float* __restrict__ sh_out,
+                                                              uint32_t epi, float scale) {
     extern __shared__ float xs[];  // [TT][H]
     const uint32_t t0 = blockIdx.x * TT;
     const uint32_t nt = min((uint32_t)TT, T - t0);
@@ -42,15 +55,15 @@ __global__ __launch_bounds__(256) void qw_router_gemm_kernel(const void* __restr
             const float v = qw_reduce64(acc[r]);
             if (lane == 0 && (uint32_t)r < nt) {
                 if (gate_row) sh_out[t0 + r] = 1.0f / (1.0f + expf(-v));
-                else logits[(uint64_t)(t0 + r) * E + e] = v;
+                else logits[(uint64_t)(t0 + r) * E + e] = qw_f32_gemv_epilogue(v, epi, scale);
             }
         }
     }
 }
 
-extern "C" qwhip_status qwhip_router_gemm_shared_gate(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
-                                                      uint32_t t, uint32_t experts, uint32_t hidden, float* logits,
-                                                      const float* sh_gate_w, float* sh_gate_out) {
+static qwhip_status qw_router_gemm_impl(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype, uint32_t t,
+                                        uint32_t experts, uint32_t hidden, float* logits, const float* sh_gate_w, float* sh_gate_out,
+                                        uint32_t epi, float scale) {
     QWHIP_REQUIRE(s);
     if (t == 0) return QWHIP_OK;
     QWHIP_REQUIRE(x);
@@ -66,7 +79,7 @@ extern "C" qwhip_status qwhip_router_gemm_shared_gate(qwhip_stream_t s, const vo
     if (lds > 64u * 1024u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: hidden %u exceeds the staged row (<= 16384)", hidden);
     const dim3 grid(qwhip_cdiv(t, tt)), block(256);
 #define QW_RG(XD, WD, TT) \
-    hipLaunchKernelGGL((qw_router_gemm_kernel<XD, WD, TT>), grid, block, lds, s->stream, x, wr, logits, t, experts, hidden, sh_gate_w, sh_gate_out)
+    hipLaunchKernelGGL((qw_router_gemm_kernel<XD, WD, TT>), grid, block, lds, s->stream, x, wr, logits, t, experts, hidden, sh_gate_w, sh_gate_out, epi, scale)
 #define QW_RG_T(XD, WD)                       \
     switch (tt) {                             \
         case 8: QW_RG(XD, WD, 8); break;      \
@@ -94,9 +107,26 @@ extern "C" qwhip_status qwhip_router_gemm_shared_gate(qwhip_stream_t s, const vo
     return QWHIP_OK;
 }
 
+extern "C" qwhip_status qwhip_router_gemm_shared_gate(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
+                                                      uint32_t t, uint32_t experts, uint32_t hidden, float* logits,
+                                                      const float* sh_gate_w, float* sh_gate_out) {
+    return qw_router_gemm_impl(s, x, x_dtype, wr, w_dtype, t, experts, hidden, logits, sh_gate_w, sh_gate_out, 0u, 1.0f);
+}
+
 extern "C" qwhip_status qwhip_router_gemm(qwhip_stream_t s, const void* x, uint32_t x_dtype, const void* wr, uint32_t w_dtype,
                                           uint32_t t, uint32_t experts, uint32_t hidden, float* logits) {
-    return qwhip_router_gemm_shared_gate(s, x, x_dtype, wr, w_dtype, t, experts, hidden, logits, nullptr, nullptr);
+    return qw_router_gemm_impl(s, x, x_dtype, wr, w_dtype, t, experts, hidden, logits, nullptr, nullptr, 0u, 1.0f);
+}
+
+// Dense fp32-weight GEMV with the scalar epilogues (QWGemm.encodeF32Gemv, Sources/Operators/QWGEMM/QWGemmF32.swift:117-141 ->
+// qwg_f32_gemv / qwg_f32_gemv_bm): y[t, n] = epilogue(sum_k W[n, k] x[t, k]) on the router kernel (every weight row read once
+// per eight activation rows).
+extern "C" qwhip_status qwhip_f32_gemv(qwhip_stream_t s, const float* w, const float* x, uint32_t rows, uint32_t n, uint32_t k,
+                                       uint32_t epi, float scale, float* y) {
+    if (epi > 3u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "epilogue %u is not one of 0 none, 1 silu(y/scale), 2 sigmoid, 3 2 sigmoid(y/scale)", epi);
+    if ((epi == 1u || epi == 3u) && !(scale != 0.0f && scale == scale))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "epilogue %u divides by its scale, which must be a non-zero number", epi);
+    return qw_router_gemm_impl(s, x, QWHIP_F32, w, QWHIP_F32, rows, n, k, y, nullptr, nullptr, epi, scale);
 }
 
 // ------------------------------------------------------------------------------------------------

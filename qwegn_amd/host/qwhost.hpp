@@ -8,6 +8,7 @@
 #pragma once
 #include <cstdint>
 #include <cstring>
+#include <limits>
 #include <optional>
 #include <stdexcept>
 #include <string>
@@ -546,6 +547,41 @@ struct QWGemm {
     }
 
     // ---- MoE encoders (Sources/Operators/QWGEMM/QWGemmMoE.swift, QWGemmMoERouter.swift) ----------------------------
+    // encodeF32Gemv (QWGemmF32.swift:117-141): dense fp32 weights [n, k], epilogues 0 none, 1 silu(y / scale), 2 sigmoid, 3 2 sigmoid(y / scale)
+    static void encodeF32Gemv(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& weight, const QWTensorValue& x, const QWTensorValue& y,
+                              int rows, int n, int k, uint32_t epilogue, float scale) {
+        if (weight.shape.dtype != QWDType::f32 || x.shape.dtype != QWDType::f32 || y.shape.dtype != QWDType::f32 ||
+            weight.shape.elementCount < (size_t)n * (size_t)k || x.shape.elementCount < (size_t)rows * (size_t)k ||
+            y.shape.elementCount < (size_t)rows * (size_t)n)
+            throw QWGemmError(QWGemmError::badShape, "f32 gemv: f32 weight [n, k], x [rows, k], y [rows, n]");
+        hal.pipeline(rows >= 4 ? "qwg_f32_gemv_bm" : "qwg_f32_gemv");
+        throwIfFailed(qwhip_f32_gemv(enc.stream, (const float*)weight.ptr(), (const float*)x.ptr(), (uint32_t)rows, (uint32_t)n, (uint32_t)k,
+                                     epilogue, scale, (float*)y.ptr()));
+    }
+    // encodeArgmaxFin (QWGemmF32.swift:276-307) over f32 logits [rows, vocab]: the plain fold, or the relaxed acceptance of a draft
+    // (QWVariationalAcceptance: logits, draftTokens u32 [totalRows], margin, minLogProb) when margin > 0 and rows > 1
+    struct QWVariationalAcceptance {
+        QWTensorValue draftTokens;
+        int totalRows = 0;
+        float margin = 0.0f;
+        float minLogProb = -std::numeric_limits<float>::infinity();
+    };
+    static void encodeArgmaxFin(QWHipEncoder& enc, const QWHal& hal, const QWTensorValue& logits, const QWTensorValue& token, int vocab, int rows = 1,
+                                const QWVariationalAcceptance* variational = nullptr) {
+        if (logits.shape.dtype != QWDType::f32 || logits.shape.elementCount < (size_t)rows * (size_t)vocab || token.shape.elementCount < (size_t)rows)
+            throw QWGemmError(QWGemmError::badShape, "argmax-fin: logits f32 [rows, vocab], token [rows]");
+        if (variational && variational->margin > 0 && rows > 1) {
+            if (variational->draftTokens.shape.elementCount < (size_t)variational->totalRows)
+                throw QWGemmError(QWGemmError::badShape, "argmax-fin: draft tokens are short");
+            hal.pipeline("qwg_head_argmax_fin_variational");
+            throwIfFailed(qwhip_argmax_f32_variational(enc.stream, (const float*)logits.ptr(), (uint32_t)rows, (uint32_t)vocab,
+                                                       (const uint32_t*)variational->draftTokens.ptr(), (uint32_t)variational->totalRows,
+                                                       variational->margin, variational->minLogProb, (int32_t*)token.ptr()));
+        } else {
+            hal.pipeline("qwg_head_argmax_fin");
+            throwIfFailed(qwhip_argmax_f32(enc.stream, (const float*)logits.ptr(), (uint32_t)rows, (uint32_t)vocab, (int32_t*)token.ptr()));
+        }
+    }
     static int moeMaxTiles(int experts, int pairs) { return (int)qwhip_moe_max_tiles((uint32_t)experts, (uint32_t)pairs); }  // QWGemmMoE.swift:24-26
 
     // encodeFnRouterGemm (QWGemmMoERouter.swift:78-113)

@@ -109,6 +109,8 @@ SIGNATURES = {
     "qwhip_dequant_hq8_planar": (C.c_int32, [_P, _P, _P, _U32, _U32, _P]),
     "qwhip_head_argmax": (C.c_int32, [_P, _WV, _P, _U32, _U32, _U32, _P, _P]),
     "qwhip_argmax_f32": (C.c_int32, [_P, _P, _U32, _U32, _P]),
+    "qwhip_argmax_f32_variational": (C.c_int32, [_P, _P, _U32, _U32, _P, _U32, C.c_float, C.c_float, _P]),
+    "qwhip_f32_gemv": (C.c_int32, [_P, _P, _P, _U32, _U32, _U32, _U32, C.c_float, _P]),
     "qwhip_gemv_f32": (C.c_int32, [_P, _WV, _P, _U32, _U32, C.c_float, _P]),
     "qwhip_h32_f32": (C.c_int32, [_P, _P, _P, _U32, _U32]),
     "qwhip_rmsnorm": (C.c_int32, [_P, _P, _P, _P, _U32, _U32, C.c_float, _U32, _P]),

@@ -298,6 +298,26 @@ public enum QWGemm {
         try hal.pipeline("qwg_add_f32")
         try qwCheck(qwhip_add_f32(enc.stream, a.f32, b.f32, out.f32, UInt64(count)))
     }
+    /// QWGemm.encodeF32Gemv (QWGemmF32.swift:117-141): dense fp32 weights, epilogue 0 none, 1 silu(y / scale), 2 sigmoid, 3 2 sigmoid(y / scale).
+    public static func encodeF32Gemv(_ enc: QWHipEncoder, hal: QWHal, weight: QWTensorValue, x: QWTensorValue, y: QWTensorValue, rows: Int, n: Int,
+                                     k: Int, epilogue: UInt32, scale: Float) throws {
+        try hal.pipeline(rows >= 4 ? "qwg_f32_gemv_bm" : "qwg_f32_gemv")
+        try qwCheck(qwhip_f32_gemv(enc.stream, weight.f32, x.f32, UInt32(rows), UInt32(n), UInt32(k), epilogue, scale, y.f32))
+    }
+    /// QWGemm.encodeArgmaxFin (QWGemmF32.swift:276-307) over f32 logits: the fold, or the relaxed acceptance of a draft.
+    public struct QWVariationalAcceptance { public let draftTokens: QWTensorValue; public let totalRows: Int; public let margin: Float; public let minLogProb: Float }
+    public static func encodeArgmaxFin(_ enc: QWHipEncoder, hal: QWHal, logits: QWTensorValue, token: QWTensorValue, vocab: Int, rows: Int = 1,
+                                       variational: QWVariationalAcceptance? = nil) throws {
+        if let v = variational, v.margin > 0, rows > 1 {
+            try hal.pipeline("qwg_head_argmax_fin_variational")
+            try qwCheck(qwhip_argmax_f32_variational(enc.stream, logits.f32, UInt32(rows), UInt32(vocab),
+                                                     v.draftTokens.ptr.assumingMemoryBound(to: UInt32.self), UInt32(v.totalRows), v.margin, v.minLogProb,
+                                                     token.i32))
+        } else {
+            try hal.pipeline("qwg_head_argmax_fin")
+            try qwCheck(qwhip_argmax_f32(enc.stream, logits.f32, UInt32(rows), UInt32(vocab), token.i32))
+        }
+    }
     /// QWGemm.encodeLatentNormH32F32 (QWGemmF32.swift:57-80): optional RMSNorm (1 + gamma) + H_32 on f32 rows -> f32 and / or f16.
     public static func encodeLatentNormH32F32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, gamma: QWTensorValue?, out32: QWTensorValue?,
                                               out16: QWTensorValue?, rows: Int, latent: Int, eps: Float = 1e-6) throws {

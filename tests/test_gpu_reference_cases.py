@@ -599,3 +599,56 @@ def test_plane_checksum_is_the_hosts_word_sum(dev, nbytes):
     assert lib.qwhip_plane_checksum(st, plane.ptr, 0, out.ptr) == qwhip.OK
     plane.free()
     out.free()
+
+
+@pytest.mark.parametrize("rows,vocab", [(4, 1000), (3, 151936), (2, 37)])
+def test_argmax_variational_acceptance(dev, rows, vocab):
+    """Relaxed acceptance of a draft over a verify window against the oracle: plain argmax without a margin, the margin rule, the
+    log-probability gate on both sides of its threshold, out-of-vocabulary and last-row drafts."""
+    import math
+    rng = np.random.default_rng(rows + vocab)
+    lg = rng.standard_normal((rows, vocab)).astype(np.float32)
+    top = qo.head_argmax(lg)
+    draft = rng.integers(0, vocab, rows + 1).astype(np.uint32)
+    second = np.argsort(-lg[0], kind="stable")[1]
+    draft[1] = second                                      # a near miss for row 0
+    if rows > 2:
+        draft[3] = vocab + 5                               # not a token
+    lb, db, tb = dev.put(lg), dev.put(draft), dev.alloc(rows * 4)
+    lib, st = dev.lib, dev.stream.handle
+
+    def run(total, margin, min_lp):
+        qwhip.check(lib.qwhip_argmax_f32_variational(st, lb.ptr, rows, vocab, db.ptr, total, margin, min_lp, tb.ptr))
+        dev.stream.sync()
+        return tb.download(np.int32, (rows,))
+
+    assert np.array_equal(run(rows + 1, 0.0, -math.inf), top)
+    gap = float(lg[0, top[0]] - lg[0, second])
+    for margin in (gap * 0.5, gap * 1.5, 100.0):
+        want = qo.head_argmax_variational(lg, draft, margin)
+        assert np.array_equal(run(rows + 1, margin, -math.inf), want)
+    assert run(rows + 1, gap * 1.5, -math.inf)[0] == second and run(rows + 1, gap * 0.5, -math.inf)[0] == top[0]
+    want_short = qo.head_argmax_variational(lg, draft[:rows], 100.0)
+    assert np.array_equal(run(rows, 100.0, -math.inf), want_short) and want_short[rows - 1] == top[rows - 1]
+    mx = lg[0].astype(np.float64).max()
+    lp = float(lg[0, second] - mx - np.log(np.exp(lg[0].astype(np.float64) - mx).sum()))
+    assert run(rows + 1, gap * 1.5, lp - 0.01)[0] == second
+    assert run(rows + 1, gap * 1.5, lp + 0.01)[0] == top[0]
+    for min_lp in (lp - 0.01, lp + 0.01, -3.0):
+        assert np.array_equal(run(rows + 1, 100.0, min_lp), qo.head_argmax_variational(lg, draft, 100.0, min_lp))
+    assert lib.qwhip_argmax_f32_variational(st, lb.ptr, rows, vocab, db.ptr, rows + 1, 1.0, math.nan, tb.ptr) == qwhip.E_BAD_SHAPE
+
+
+@pytest.mark.parametrize("rows,n,k", [(1, 40, 256), (5, 33, 100), (20, 8, 4096)])
+@pytest.mark.parametrize("epi,scale", [(0, 1.0), (1, 2.0), (2, 1.0), (3, 0.5)])
+def test_dense_f32_gemv_with_epilogues(dev, rows, n, k, epi, scale):
+    rng = np.random.default_rng(n + k)
+    w = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    wb, xb, yb = dev.put(w), dev.put(x), dev.alloc(rows * n * 4)
+    qwhip.check(dev.lib.qwhip_f32_gemv(dev.stream.handle, wb.ptr, xb.ptr, rows, n, k, epi, scale, yb.ptr))
+    dev.stream.sync()
+    got = yb.download(np.float32, (rows, n))
+    assert qo.normalized_error(got, qo.f32_gemv(w, x, epi, scale)) <= 2e-6
+    assert dev.lib.qwhip_f32_gemv(dev.stream.handle, wb.ptr, xb.ptr, rows, n, k, 4, 1.0, yb.ptr) == qwhip.E_BAD_SHAPE
+    assert dev.lib.qwhip_f32_gemv(dev.stream.handle, wb.ptr, xb.ptr, rows, n, k, 1, 0.0, yb.ptr) == qwhip.E_BAD_SHAPE

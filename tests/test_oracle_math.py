@@ -554,3 +554,36 @@ def test_route_budget_rules():
                 assert abs(float(bw[r].sum()) - float(w[r].sum())) <= 2e-6
     same_i, same_w = qo.moe_route_budget(idx, wts, 6)
     assert np.array_equal(same_i, idx) and np.array_equal(same_w, wts)
+
+
+def test_variational_acceptance_and_f32_gemv_closed_forms():
+    """head_argmax_variational: no margin = the plain argmax; a margin wider than the spread and no probability gate accepts every
+    valid draft that is not the argmax; the last row and out-of-vocabulary drafts keep the argmax; the probability gate on a
+    two-spike row follows log softmax = -log(1 + e^(a - b) + (v - 2) e^(low - b)).  f32_gemv: identity weights expose the
+    epilogues (silu(x / s), sigmoid, 2 sigmoid(x / s) = 1 + tanh(x / 2s))."""
+    import math
+    rng = np.random.default_rng(4)
+    lg = rng.standard_normal((5, 50)).astype(np.float32)
+    draft = np.array([3, 7, 49, 50, 11, 2], np.int64)
+    assert np.array_equal(qo.head_argmax_variational(lg, draft, 0.0), qo.head_argmax(lg))
+    wide = qo.head_argmax_variational(lg, draft, 100.0)
+    plain = qo.head_argmax(lg)
+    assert wide[0] == 7 and wide[1] == 49 and wide[2] == plain[2] and wide[3] == 11 and wide[4] == 2
+    short = qo.head_argmax_variational(lg, draft[:5], 100.0)
+    assert short[4] == plain[4]
+    a, b, low, v = 5.0, 4.0, -20.0, 50
+    row = np.full((2, v), low, np.float32)
+    row[:, 9], row[:, 17] = a, b
+    lp = -math.log(1.0 + math.exp(a - b) + (v - 2) * math.exp(low - b))
+    d2 = np.array([0, 17, 17], np.int64)
+    assert qo.head_argmax_variational(row, d2, 2.0, lp - 1e-3)[0] == 17
+    assert qo.head_argmax_variational(row, d2, 2.0, lp + 1e-3)[0] == 9
+    assert qo.head_argmax_variational(row, d2, 0.5)[0] == 9           # outside the margin
+    x = rng.standard_normal((3, 6))
+    eye = np.eye(6)
+    np.testing.assert_allclose(qo.f32_gemv(eye, x), x)
+    np.testing.assert_allclose(qo.f32_gemv(eye, x, 1, 2.0), (x / 2) / (1 + np.exp(-x / 2)), rtol=1e-12)
+    np.testing.assert_allclose(qo.f32_gemv(eye, x, 2), 1 / (1 + np.exp(-x)), rtol=1e-12)
+    np.testing.assert_allclose(qo.f32_gemv(eye, x, 3, 2.0), 1 + np.tanh(x / 4), rtol=1e-12)
+    w = rng.standard_normal((4, 6))
+    np.testing.assert_allclose(qo.f32_gemv(w, x), np.einsum("tk,nk->tn", x, w), rtol=1e-12)
