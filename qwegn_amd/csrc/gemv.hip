@@ -15,6 +15,8 @@
 //    through LDS.  VALU does only the dequant; accumulation rides on the matrix cores.
 #include <atomic>
 
+#include <type_traits>
+
 #include "qwhip_common.h"
 
 enum { QW_XM_GLOBAL = 0, QW_XM_LDS_ROT = 1 };
@@ -371,13 +373,18 @@ struct qw_gemv_params {
     const float* shared;
     const float* shared_gate;
     void* out;
+    // transposing kernel: waves per row set, row sets per workgroup, K ranges
+    uint32_t wpr, sets, nkr;
+};
+// What only the gate|up pair and routed kernels read.  They take the longer argument block; the plain GEMV kernels keep
+// the short one (the longer block alone cost the transposing kernel 1.8 % on N = 7168, K = 5120, m = 16 in a same-box
+// comparison).
+struct qw_gemv_params_x : qw_gemv_params {
     const int32_t* x_rows;  // gate|up: activation row of every pair (NULL: the pair's token)
     uint32_t x_div;         // down: pairs that share one activation row (0 and 1: a row per pair)
     const int32_t* labels;  // down, num_groups > 0: group of every expert; blockIdx.y = token * num_groups + group and
     uint32_t num_groups;    // only the token's routes into that group are summed
     qw_act act;             // gate|up pair mode: the device's gated activation (all zero: SwiGLU)
-    // transposing kernel: waves per row set, row sets per workgroup, K ranges
-    uint32_t wpr, sets, nkr;
 };
 
 // PAIR = 1: gate|up pair mode.  The bank holds 2*N rows ([0, N) gate, [N, 2N) up); both are accumulated
@@ -385,7 +392,8 @@ struct qw_gemv_params {
 // ROUTED = 1 (with PAIR): blockIdx.y is a (token, route) pair; the expert's sub-bank is picked through
 // idx[pair], the activation row is the pair's token, the output row is the pair.
 template <int FMT, int RT, int XDT, int XM, int PAIR, int ROUTED, int NWV = 4>
-__global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_params p) {
+__global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(
+    const typename std::conditional<(PAIR || ROUTED), qw_gemv_params_x, qw_gemv_params>::type p) {
     constexpr uint32_t NTH = 64 * NWV;
     constexpr int NACC = RT * (PAIR ? 2 : 1);
     extern __shared__ h8_t xs[];
@@ -506,7 +514,7 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(const qw_gemv_pa
 // routes of a token stream side by side instead of one after the other); the route partials meet in LDS and are
 // summed in wave order.
 template <int FMT, int RT, int ODT>
-__global__ __launch_bounds__(512) void qw_moe_down_decode_kernel(const qw_gemv_params p) {
+__global__ __launch_bounds__(512) void qw_moe_down_decode_kernel(const qw_gemv_params_x p) {
     __shared__ f4_t red[8][RT][64];
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u;
@@ -820,7 +828,7 @@ __global__ __launch_bounds__(768) void qw_gemv_colt_kernel(const qw_gemv_params 
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-typedef qw_gemv_params gemv_args;
+typedef qw_gemv_params_x gemv_args;   // the host side fills the long form; plain kernels are handed its base
 
 template <int FMT, int RT, int XDT, int XM, int PAIR>
 void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds, uint32_t routed_pairs = 0) {

@@ -16,6 +16,8 @@
 // per block:  sum_i w_i x_i = s * sum_i q_i x_i + (1024 s + b) * S,  S = sum_i x_i,
 // the same factorisation the reference's bit-stream GEMVs use (qwg_aq_slice_dot, qw_dequant_multi.metalh:205-208).
 // The activations are the f16-rounded rotated values the reference's producers would have stored.
+#include <type_traits>
+
 #include "qwhip_common.h"
 
 namespace {
@@ -26,8 +28,17 @@ struct qc_params {
     h1_t* y16;
     float* y32;
     uint32_t N, nb, cpr, rotate;
-    unsigned long long* keys;   // NULL, or [gridDim.x]: the workgroup's argmax key (monotone float bits << 32 | ~row) over its rows
 };
+// The head's form of the kernel takes one more argument: keys [gridDim.x], the workgroup's argmax key (monotone float bits
+// << 32 | ~row) over its rows.  It is a second instantiation with its own argument block: the decode kernel's argument
+// block and code stay as they are without it (with the extra member and epilogue in the one kernel the N = 17408, K = 5120
+// launch took 11.6 us instead of 11.3 in a same-box comparison).
+struct qc_params_fold {
+    qc_params base;
+    unsigned long long* keys;
+};
+__device__ __forceinline__ const qc_params& qc_base(const qc_params& p) { return p; }
+__device__ __forceinline__ const qc_params& qc_base(const qc_params_fold& p) { return p.base; }
 
 // A float's bits made monotone as an unsigned number; NaN -> 0, so it never wins (qw_sortable_f32_u32,
 // Sources/QWMetal/include/qw_fastmath_safe.metalh:21-25).
@@ -39,8 +50,10 @@ __device__ __forceinline__ uint32_t qc_sortable_f32(float x) {
 
 // SETS row sets per workgroup, D blocks in flight per lane, D0 of them issued before the activation prologue.
 // blockDim.x = 32 * cpr * SETS; dynamic LDS = nb * 80 + rows-per-workgroup * cpr * 4 bytes.
-template <int XDT, int SETS, int D, int D0>
-__global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
+template <int XDT, int SETS, int D, int D0, typename P = qc_params>
+__global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const P pp) {
+    constexpr bool FOLD = !std::is_same<P, qc_params>::value;
+    const qc_params& p = qc_base(pp);
     // 16-group activation tiles per full wave: ceil(2 cpr / full waves).  One row set with an odd cpr ends in a half
     // wave, which takes no tile (its upper lanes do not exist): cpr = 13 leaves 6 full waves for 26 tiles.
     constexpr int XT = SETS == 1 ? 5 : (SETS == 2 ? 2 : 1);
@@ -160,10 +173,12 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
         const uint32_t row = s * G + blockIdx.x;
         if (p.y32) p.y32[row] = v;
         if (p.y16) p.y16[row] = (h1_t)v;
-        const unsigned long long key = ((unsigned long long)qc_sortable_f32(v) << 32) | (uint32_t)~row;
-        best = key > best ? key : best;
+        if constexpr (FOLD) {
+            const unsigned long long key = ((unsigned long long)qc_sortable_f32(v) << 32) | (uint32_t)~row;
+            best = key > best ? key : best;
+        }
     }
-    if (p.keys) {
+    if constexpr (FOLD) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
             const unsigned long long other = __shfl_xor(best, o, 64);
@@ -176,7 +191,7 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const qc_params p) {
         if (tid == 0u) {
             const uint32_t nwaves = (blockDim.x + 63u) >> 6;
             for (uint32_t wv = 1; wv < nwaves; ++wv) best = wbest[wv] > best ? wbest[wv] : best;
-            p.keys[blockIdx.x] = best;
+            pp.keys[blockIdx.x] = best;
         }
     }
 }
@@ -200,7 +215,14 @@ __global__ __launch_bounds__(256) void qw_col_keys_fin_kernel(const unsigned lon
 }
 
 template <int XDT, int SETS>
-hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t threads, size_t lds, uint32_t depth) {
+hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t threads, size_t lds, uint32_t depth, unsigned long long* keys) {
+    if (keys) {   // the head: automatic prefetch only
+        qc_params_fold pf;
+        pf.base = p;
+        pf.keys = keys;
+        hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 2, qc_params_fold>), dim3(wgs), dim3(threads), lds, st, pf);
+        return hipGetLastError();
+    }
     if (depth == 1) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 1>), dim3(wgs), dim3(threads), lds, st, p);
     else if (depth == 3) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 3, 3>), dim3(wgs), dim3(threads), lds, st, p);
     else if (depth == 4) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 4, 4>), dim3(wgs), dim3(threads), lds, st, p);
@@ -249,17 +271,17 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     p.cpr = cpr;
     p.rotate = rotate ? 1u : 0u;
     const bool fold = keys && token && wgs <= keys_cap && (size_t)rows_per_wg * cpr * 4u >= 8u * waves;
-    p.keys = fold ? keys : nullptr;
+    unsigned long long* fold_keys = fold ? keys : nullptr;
     if (folded) *folded = fold;
     hipError_t e;
     if (x_dtype == QWHIP_F16) {
-        e = sets == 4 ? qc_launch<QWHIP_F16, 4>(st, p, wgs, threads, lds, depth)
-          : sets == 2 ? qc_launch<QWHIP_F16, 2>(st, p, wgs, threads, lds, depth)
-                      : qc_launch<QWHIP_F16, 1>(st, p, wgs, threads, lds, depth);
+        e = sets == 4 ? qc_launch<QWHIP_F16, 4>(st, p, wgs, threads, lds, depth, fold_keys)
+          : sets == 2 ? qc_launch<QWHIP_F16, 2>(st, p, wgs, threads, lds, depth, fold_keys)
+                      : qc_launch<QWHIP_F16, 1>(st, p, wgs, threads, lds, depth, fold_keys);
     } else {
-        e = sets == 4 ? qc_launch<QWHIP_BF16, 4>(st, p, wgs, threads, lds, depth)
-          : sets == 2 ? qc_launch<QWHIP_BF16, 2>(st, p, wgs, threads, lds, depth)
-                      : qc_launch<QWHIP_BF16, 1>(st, p, wgs, threads, lds, depth);
+        e = sets == 4 ? qc_launch<QWHIP_BF16, 4>(st, p, wgs, threads, lds, depth, fold_keys)
+          : sets == 2 ? qc_launch<QWHIP_BF16, 2>(st, p, wgs, threads, lds, depth, fold_keys)
+                      : qc_launch<QWHIP_BF16, 1>(st, p, wgs, threads, lds, depth, fold_keys);
     }
     if (e == hipSuccess && fold) {
         hipLaunchKernelGGL(qw_col_keys_fin_kernel, dim3(1), dim3(256), 0, st, keys, wgs, token);
