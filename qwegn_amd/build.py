@@ -15,6 +15,8 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-ffp-contract=off",
+    # scalar kernel arguments arrive in SGPRs instead of through a load at the start of every wave (see qw_launch_scalar)
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
 ]
 
 

@@ -357,43 +357,39 @@ __device__ __forceinline__ void qw_stream_first(const uint8_t* const* rp, uint32
     for (int t = 0; t < NACC; ++t) qw_load_slice<FMT>(rp[t], s, gshift, bb, first[t]);
 }
 
-struct qw_gemv_params {
-    const uint8_t* bank;
-    const void* x;
-    h1_t* y16;
-    float* y32;
-    uint32_t N, K, M, gshift, bb;
-    uint64_t row_bytes;
-    uint32_t rotate, rot_out;
-    // routed (MoE decode) modes
-    const int32_t* idx;
-    const float* wts;
-    uint32_t top_k;
-    uint64_t expert_bytes;  // bytes of one expert's sub-bank
-    const float* shared;
-    const float* shared_gate;
-    void* out;
-    // transposing kernel: waves per row set, row sets per workgroup, K ranges
-    uint32_t wpr, sets, nkr;
-};
+// idx .. out: the routed (MoE decode) modes; expert_bytes: bytes of one expert's sub-bank.  wpr, sets, nkr: the transposing
+// kernel's waves per row set, row sets per workgroup, K ranges.
+#define QGV_FIELDS(X)                                                                                                        \
+    X(const uint8_t*, bank) X(const void*, x) X(h1_t*, y16) X(float*, y32) X(uint32_t, N) X(uint32_t, K) X(uint32_t, M)          \
+    X(uint32_t, gshift) X(uint32_t, bb) X(uint64_t, row_bytes) X(uint32_t, rotate) X(uint32_t, rot_out) X(const int32_t*, idx)   \
+    X(const float*, wts) X(uint32_t, top_k) X(uint64_t, expert_bytes) X(const float*, shared) X(const float*, shared_gate)       \
+    X(void*, out) X(uint32_t, wpr) X(uint32_t, sets) X(uint32_t, nkr)
+QW_ARG_BLOCK(qw_gemv_params, QGV_FIELDS)
 // What only the gate|up pair and routed kernels read.  They take the longer argument block; the plain GEMV kernels keep
 // the short one (the longer block alone cost the transposing kernel 1.8 % on N = 7168, K = 5120, m = 16 in a same-box
-// comparison).
-struct qw_gemv_params_x : qw_gemv_params {
-    const int32_t* x_rows;  // gate|up: activation row of every pair (NULL: the pair's token)
-    uint32_t x_div;         // down: pairs that share one activation row (0 and 1: a row per pair)
-    const int32_t* labels;  // down, num_groups > 0: group of every expert; blockIdx.y = token * num_groups + group and
-    uint32_t num_groups;    // only the token's routes into that group are summed
-    qw_act act;             // gate|up pair mode: the device's gated activation (all zero: SwiGLU)
-};
+// comparison).  x_rows (gate|up): activation row of every pair (NULL: the pair's token); x_div (down): pairs that share one
+// activation row (0 and 1: a row per pair); labels, num_groups > 0 (down): group of every expert; blockIdx.y = token *
+// num_groups + group and only the token's routes into that group are summed; act (pair mode): the device's gated activation.
+#define QGVX_FIELDS(X) \
+    QGV_FIELDS(X) X(const int32_t*, x_rows) X(uint32_t, x_div) X(const int32_t*, labels) X(uint32_t, num_groups) X(qw_act, act)
+QW_ARG_BLOCK(qw_gemv_params_x, QGVX_FIELDS)
+inline qw_gemv_params qw_gemv_base(const qw_gemv_params_x& a) {
+    qw_gemv_params p;
+#define QGV_TAKE(T, n) p.n = a.n;
+    QGV_FIELDS(QGV_TAKE)
+#undef QGV_TAKE
+    return p;
+}
 
 // PAIR = 1: gate|up pair mode.  The bank holds 2*N rows ([0, N) gate, [N, 2N) up); both are accumulated
 // and the epilogue stores act[m, n] = f16(FWHT32(silu(g) * u)) (rotation optional).
 // ROUTED = 1 (with PAIR): blockIdx.y is a (token, route) pair; the expert's sub-bank is picked through
 // idx[pair], the activation row is the pair's token, the output row is the pair.
 template <int FMT, int RT, int XDT, int XM, int PAIR, int ROUTED, int NWV = 4>
-__global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(
-    const typename std::conditional<(PAIR || ROUTED), qw_gemv_params_x, qw_gemv_params>::type p) {
+struct qw_gemv_mfma_kernel {
+typedef typename std::conditional<(PAIR || ROUTED), qw_gemv_params_x, qw_gemv_params>::type params_t;
+static constexpr int kLaunchBound = 64 * NWV;
+static __device__ __forceinline__ void run(const params_t& p) {
     constexpr uint32_t NTH = 64 * NWV;
     constexpr int NACC = RT * (PAIR ? 2 : 1);
     extern __shared__ h8_t xs[];
@@ -506,6 +502,7 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(
         }
     }
 }
+};
 
 // Routed down projection of the decode path: blockIdx.y is a token; the workgroup's 16*RT output rows
 // accumulate sum_k wts[t, k] * (W_down[e_k] . act[t, k]) over the token's routes, add the gated shared
@@ -514,7 +511,9 @@ __global__ __launch_bounds__(64 * NWV) void qw_gemv_mfma_kernel(
 // routes of a token stream side by side instead of one after the other); the route partials meet in LDS and are
 // summed in wave order.
 template <int FMT, int RT, int ODT>
-__global__ __launch_bounds__(512) void qw_moe_down_decode_kernel(const qw_gemv_params_x p) {
+struct qw_moe_down_decode_kernel {
+static constexpr int kLaunchBound = 512;
+static __device__ __forceinline__ void run(const qw_gemv_params_x& p) {
     __shared__ f4_t red[8][RT][64];
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u;
@@ -573,6 +572,7 @@ __global__ __launch_bounds__(512) void qw_moe_down_decode_kernel(const qw_gemv_p
         }
     }
 }
+};
 
 // ------------------------------------------------------------------------------------------------
 // Variant C: column-stationary MFMA kernel, all containers, m = 1..16, activations already in the container's basis,
@@ -830,6 +830,12 @@ namespace {
 
 typedef qw_gemv_params_x gemv_args;   // the host side fills the long form; plain kernels are handed its base
 
+template <typename K>   // the short argument block for the plain kernel, the long one for the pair / routed forms
+void qw_launch_mfma_k(dim3 grid, dim3 block, size_t lds, hipStream_t st, const gemv_args& a) {
+    if constexpr (std::is_same<typename K::params_t, qw_gemv_params_x>::value) qw_launch_scalar<K>(grid, block, lds, st, a);
+    else qw_launch_scalar<K>(grid, block, lds, st, qw_gemv_base(a));
+}
+
 template <int FMT, int RT, int XDT, int XM, int PAIR>
 void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds, uint32_t routed_pairs = 0) {
     if constexpr (!PAIR && RT == 1) {
@@ -842,8 +848,8 @@ void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds, uint32_t routed
             uint32_t nw = 4;
             while (nw < 16u && tiles * nw < 4096u && iters >= 4u * nw) nw *= 2u;
             const dim3 grid(tiles);
-            if (nw == 16u) { hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0, 16>), grid, dim3(1024), lds, st, a); return; }
-            if (nw == 8u) { hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0, 8>), grid, dim3(512), lds, st, a); return; }
+            if (nw == 16u) { qw_launch_mfma_k<qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0, 16>>(grid, dim3(1024), lds, st, a); return; }
+            if (nw == 8u) { qw_launch_mfma_k<qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0, 8>>(grid, dim3(512), lds, st, a); return; }
         }
     }
     const dim3 block(256);
@@ -852,13 +858,13 @@ void launch_mfma(hipStream_t st, const gemv_args& a, size_t lds, uint32_t routed
             // one short row set per (route, tile): eight waves split K so that each holds two or more iterations in flight
             const dim3 grid(qwhip_cdiv(a.N, 16u * RT), routed_pairs);
             if (qwhip_cdiv(a.K >> 5, 4u) >= 16u)
-                hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1, 8>), grid, dim3(512), lds, st, a);
+                qw_launch_mfma_k<qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1, 8>>(grid, dim3(512), lds, st, a);
             else
-                hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1>), grid, block, lds, st, a);
+                qw_launch_mfma_k<qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 1>>(grid, block, lds, st, a);
         }
     } else {
         const dim3 grid(qwhip_cdiv(a.N, 16u * RT));
-        hipLaunchKernelGGL((qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0>), grid, block, lds, st, a);
+        qw_launch_mfma_k<qw_gemv_mfma_kernel<FMT, RT, XDT, XM, PAIR, 0>>(grid, block, lds, st, a);
     }
 }
 
@@ -889,7 +895,7 @@ bool launch_colm(hipStream_t st, const gemv_args& a, uint32_t xdt) {
     const uint32_t ipw = qwhip_cdiv(iters, 8u);
     const uint32_t tiles = qwhip_cdiv(a.N, 16u);
     const dim3 grid(min(tiles, 256u)), block(512);
-#define QW_COLM(DT, I) hipLaunchKernelGGL((qw_gemv_colm_kernel<FMT, DT, I>), grid, block, 0, st, a)
+#define QW_COLM(DT, I) hipLaunchKernelGGL((qw_gemv_colm_kernel<FMT, DT, I>), grid, block, 0, st, qw_gemv_base(a))
 #define QW_COLM_I(DT)                                                                                  \
     switch (ipw) {                                                                                     \
         case 1: QW_COLM(DT, 1); break; case 2: QW_COLM(DT, 2); break; case 3: QW_COLM(DT, 3); break;   \
@@ -929,7 +935,7 @@ bool launch_colt_1(hipStream_t st, gemv_args a, hipError_t* err) {
         if (e != hipSuccess) { *err = e; return true; }
         attr_lds.store(150u * 1024u, std::memory_order_release);
     }
-    hipLaunchKernelGGL(kern, dim3(wgs), dim3(64u * waves), lds, st, a);
+    hipLaunchKernelGGL(kern, dim3(wgs), dim3(64u * waves), lds, st, qw_gemv_base(a));
     *err = hipGetLastError();
     return true;
 }
@@ -1373,7 +1379,7 @@ static qwhip_status qw_moe_down_decode_impl(qwhip_stream_t s, const qwhip_weight
     a.num_groups = num_groups;
     const dim3 grid(qwhip_cdiv(hidden, 16u)), block(512);
     const dim3 g2(grid.x, (uint32_t)out_rows);
-#define QW_DD(F, OD) hipLaunchKernelGGL((qw_moe_down_decode_kernel<F, 1, OD>), g2, block, 0, s->stream, a)
+#define QW_DD(F, OD) qw_launch_scalar<qw_moe_down_decode_kernel<F, 1, OD>>(g2, block, 0, s->stream, a)
 #define QW_DD_O(F)                                                                                          \
     switch (out_dtype) {                                                                                    \
         case QWHIP_F32: QW_DD(F, QWHIP_F32); break;                                                         \

@@ -22,23 +22,22 @@
 
 namespace {
 
-struct qc_params {
-    const uint8_t* bank;
-    const void* x;
-    h1_t* y16;
-    float* y32;
-    uint32_t N, nb, cpr, rotate;
-};
+#define QC_FIELDS(X) X(const uint8_t*, bank) X(const void*, x) X(h1_t*, y16) X(float*, y32) X(uint32_t, N) X(uint32_t, nb) X(uint32_t, cpr) X(uint32_t, rotate)
+QW_ARG_BLOCK(qc_params, QC_FIELDS)
 // The head's form of the kernel takes one more argument: keys [gridDim.x], the workgroup's argmax key (monotone float bits
 // << 32 | ~row) over its rows.  It is a second instantiation with its own argument block: the decode kernel's argument
 // block and code stay as they are without it (with the extra member and epilogue in the one kernel the N = 17408, K = 5120
 // launch took 11.6 us instead of 11.3 in a same-box comparison).
-struct qc_params_fold {
-    qc_params base;
-    unsigned long long* keys;
-};
+#define QC_FOLD_FIELDS(X) QC_FIELDS(X) X(unsigned long long*, keys)
+QW_ARG_BLOCK(qc_params_fold, QC_FOLD_FIELDS)
 __device__ __forceinline__ const qc_params& qc_base(const qc_params& p) { return p; }
-__device__ __forceinline__ const qc_params& qc_base(const qc_params_fold& p) { return p.base; }
+__device__ __forceinline__ qc_params qc_base(const qc_params_fold& f) {
+    qc_params p;
+#define QC_TAKE(T, n) p.n = f.n;
+    QC_FIELDS(QC_TAKE)
+#undef QC_TAKE
+    return p;
+}
 
 // A float's bits made monotone as an unsigned number; NaN -> 0, so it never wins (qw_sortable_f32_u32,
 // Sources/QWMetal/include/qw_fastmath_safe.metalh:21-25).
@@ -51,7 +50,9 @@ __device__ __forceinline__ uint32_t qc_sortable_f32(float x) {
 // SETS row sets per workgroup, D blocks in flight per lane, D0 of them issued before the activation prologue.
 // blockDim.x = 32 * cpr * SETS; dynamic LDS = nb * 80 + rows-per-workgroup * cpr * 4 bytes.
 template <int XDT, int SETS, int D, int D0, typename P = qc_params>
-__global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const P pp) {
+struct qw_gemv_col_kernel {
+static constexpr int kLaunchBound = 1024;
+static __device__ __forceinline__ void run(const P& pp) {
     constexpr bool FOLD = !std::is_same<P, qc_params>::value;
     const qc_params& p = qc_base(pp);
     // 16-group activation tiles per full wave: ceil(2 cpr / full waves).  One row set with an odd cpr ends in a half
@@ -195,6 +196,7 @@ __global__ __launch_bounds__(1024) void qw_gemv_col_kernel(const P pp) {
         }
     }
 }
+};
 
 // Folds the workgroups' keys into the token: one workgroup.
 __global__ __launch_bounds__(256) void qw_col_keys_fin_kernel(const unsigned long long* __restrict__ keys, uint32_t count, int32_t* token) {
@@ -218,15 +220,17 @@ template <int XDT, int SETS>
 hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t threads, size_t lds, uint32_t depth, unsigned long long* keys) {
     if (keys) {   // the head: automatic prefetch only
         qc_params_fold pf;
-        pf.base = p;
+#define QC_TAKE(T, n) pf.n = p.n;
+        QC_FIELDS(QC_TAKE)
+#undef QC_TAKE
         pf.keys = keys;
-        hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 2, qc_params_fold>), dim3(wgs), dim3(threads), lds, st, pf);
+        qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 2, qc_params_fold>>(dim3(wgs), dim3(threads), lds, st, pf);
         return hipGetLastError();
     }
-    if (depth == 1) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 1>), dim3(wgs), dim3(threads), lds, st, p);
-    else if (depth == 3) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 3, 3>), dim3(wgs), dim3(threads), lds, st, p);
-    else if (depth == 4) hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 4, 4>), dim3(wgs), dim3(threads), lds, st, p);
-    else hipLaunchKernelGGL((qw_gemv_col_kernel<XDT, SETS, 2, 2>), dim3(wgs), dim3(threads), lds, st, p);
+    if (depth == 1) qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 1>>(dim3(wgs), dim3(threads), lds, st, p);
+    else if (depth == 3) qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 3, 3>>(dim3(wgs), dim3(threads), lds, st, p);
+    else if (depth == 4) qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 4, 4>>(dim3(wgs), dim3(threads), lds, st, p);
+    else qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 2>>(dim3(wgs), dim3(threads), lds, st, p);
     return hipGetLastError();
 }
 

@@ -31,13 +31,10 @@
 
 namespace {
 
-struct qcx_params {
-    const uint8_t* bank;
-    const void* x;
-    h1_t* y16;
-    float* y32;
-    uint32_t N, K, M, nsl, cpr, sets, gshift, bb, row_bytes;
-};
+#define QCX_FIELDS(X)                                                                                                       \
+    X(const uint8_t*, bank) X(const void*, x) X(h1_t*, y16) X(float*, y32) X(uint32_t, N) X(uint32_t, K) X(uint32_t, M)         \
+    X(uint32_t, nsl) X(uint32_t, cpr) X(uint32_t, sets) X(uint32_t, gshift) X(uint32_t, bb) X(uint32_t, row_bytes)
+QW_ARG_BLOCK(qcx_params, QCX_FIELDS)
 
 // payload dwords of one 32-column slice: bits * 32 / 32 (HQ4_G32_M5 and 4-bit streams: 4)
 template <int FMT>
@@ -123,7 +120,9 @@ __device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
 // ROT (MR = 1 only): the activation row arrives un-rotated; the FWHT-32 of its groups runs on the matrix cores into
 // an LDS image (16 groups per wave and tile), and each lane then reads its own column from there.
 template <int FMT, int XDT, int MR, int D, int LB, bool ROT>
-__global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
+struct qw_gemv_colx_kernel {
+static constexpr int kLaunchBound = LB;
+static __device__ __forceinline__ void run(const qcx_params& p) {
     static_assert(!ROT || MR == 1, "fused rotation is built for one activation row");
     extern __shared__ h8_t qcx_lds[];
     h8_t* xs = qcx_lds;                                                     // ROT: 80 bytes per 32-group (64 used)
@@ -361,10 +360,11 @@ __global__ __launch_bounds__(LB) void qw_gemv_colx_kernel(const qcx_params p) {
         if (p.y16) p.y16[at] = (h1_t)v;
     }
 }
+};
 
 template <int FMT, int XDT, int MR, int D, int LB, bool ROT = false>
 void qcx_launch1(hipStream_t st, const qcx_params& p, uint32_t wgs, uint32_t threads, size_t lds) {
-    hipLaunchKernelGGL((qw_gemv_colx_kernel<FMT, XDT, MR, D, LB, ROT>), dim3(wgs), dim3(threads), lds, st, p);
+    qw_launch_scalar<qw_gemv_colx_kernel<FMT, XDT, MR, D, LB, ROT>>(dim3(wgs), dim3(threads), lds, st, p);
 }
 
 template <int FMT, int XDT>

@@ -16,13 +16,10 @@
 
 namespace {
 
-struct qf_params {
-    const uint8_t* bank;
-    const float* x;
-    float* y;
-    uint32_t N, K, M, nsl, cpr, sets, gshift, bb, row_bytes, epi;
-    float scale;
-};
+#define QF_FIELDS(X)                                                                                                        \
+    X(const uint8_t*, bank) X(const float*, x) X(float*, y) X(uint32_t, N) X(uint32_t, K) X(uint32_t, M) X(uint32_t, nsl)       \
+    X(uint32_t, cpr) X(uint32_t, sets) X(uint32_t, gshift) X(uint32_t, bb) X(uint32_t, row_bytes) X(uint32_t, epi) X(float, scale)
+QW_ARG_BLOCK(qf_params, QF_FIELDS)
 
 template <int FMT>
 struct qf_fmt {
@@ -69,7 +66,9 @@ __device__ __forceinline__ float qf_epilogue(float v, uint32_t epi, float scale)
 // MR activation rows, three (MR = 4: four) slices in flight per lane.  blockDim.x = 32 * cpr * sets;
 // dynamic LDS = rows-per-workgroup * cpr * MR * 4 bytes.
 template <int FMT, int MR, int LB>
-__global__ __launch_bounds__(LB) void qw_gemv_f32_kernel(const qf_params p) {
+struct qw_gemv_f32_kernel {
+static constexpr int kLaunchBound = LB;
+static __device__ __forceinline__ void run(const qf_params& p) {
     constexpr int D = MR == 4 ? 4 : 3, PW = qf_fmt<FMT>::PW;
     extern __shared__ float qf_part[];   // [row slot][chunk][MR]
     const uint32_t cpr = p.cpr, N = p.N, sets = p.sets;
@@ -192,6 +191,7 @@ __global__ __launch_bounds__(LB) void qw_gemv_f32_kernel(const qf_params p) {
         p.y[(uint64_t)m * N + s * G + blockIdx.x] = qf_epilogue(v, p.epi, p.scale);
     }
 }
+};
 
 // In-place capable FWHT-32 over consecutive groups of 32 outputs of each row, butterfly order and scaling of
 // qwg_fwht32_lane_f32 (Sources/QWMetal/include/qw_weight_basis.metalh:31-38); a last partial group is padded with zeros
@@ -207,9 +207,9 @@ __global__ __launch_bounds__(256) void qw_h32_f32_kernel(const float* x, float* 
 
 template <int FMT>
 void qf_launch(hipStream_t st, const qf_params& p, uint32_t mr, uint32_t wgs, uint32_t threads, size_t lds) {
-    if (mr == 1) hipLaunchKernelGGL((qw_gemv_f32_kernel<FMT, 1, 1024>), dim3(wgs), dim3(threads), lds, st, p);
-    else if (mr == 2) hipLaunchKernelGGL((qw_gemv_f32_kernel<FMT, 2, 768>), dim3(wgs), dim3(threads), lds, st, p);
-    else hipLaunchKernelGGL((qw_gemv_f32_kernel<FMT, 4, 512>), dim3(wgs), dim3(threads), lds, st, p);
+    if (mr == 1) qw_launch_scalar<qw_gemv_f32_kernel<FMT, 1, 1024>>(dim3(wgs), dim3(threads), lds, st, p);
+    else if (mr == 2) qw_launch_scalar<qw_gemv_f32_kernel<FMT, 2, 768>>(dim3(wgs), dim3(threads), lds, st, p);
+    else qw_launch_scalar<qw_gemv_f32_kernel<FMT, 4, 512>>(dim3(wgs), dim3(threads), lds, st, p);
 }
 
 }  // namespace

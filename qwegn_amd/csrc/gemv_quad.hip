@@ -28,13 +28,10 @@
 
 namespace {
 
-struct qq_params {
-    const uint8_t* bank;
-    const void* x;
-    h1_t* y16;
-    float* y32;
-    uint32_t N, K, M, nsl, wpr, sets, nkr, gshift, bb, row_bytes;
-};
+#define QQ_FIELDS(X)                                                                                                        \
+    X(const uint8_t*, bank) X(const void*, x) X(h1_t*, y16) X(float*, y32) X(uint32_t, N) X(uint32_t, K) X(uint32_t, M)         \
+    X(uint32_t, nsl) X(uint32_t, wpr) X(uint32_t, sets) X(uint32_t, nkr) X(uint32_t, gshift) X(uint32_t, bb) X(uint32_t, row_bytes)
+QW_ARG_BLOCK(qq_params, QQ_FIELDS)
 
 struct __attribute__((packed, aligned(4))) qq_words4 { uint32_t q[4]; };
 struct __attribute__((packed, aligned(4))) qq_words8 { uint32_t q[8]; };
@@ -51,7 +48,9 @@ struct qq_slice {
 // MG groups of four activation rows, D row quads in flight per lane.  blockDim.x = 64 * wpr * sets;
 // dynamic LDS = quad-slots-per-workgroup * (4 wpr) * (4 MG) * 16 bytes.
 template <int FMT, int XDT, int MG, int D, int LB>
-__global__ __launch_bounds__(LB) void qw_gemv_quad_kernel(const qq_params p) {
+struct qw_gemv_quad_kernel {
+static constexpr int kLaunchBound = LB;
+static __device__ __forceinline__ void run(const qq_params& p) {
     extern __shared__ f4_t qq_part[];   // [quad slot][wave of the set * 4 + 16-lane row][activation row] -> 4 bank rows
     const uint32_t N = p.N, wpr = p.wpr, sets = p.sets;
     const uint32_t tid = threadIdx.x;
@@ -273,17 +272,18 @@ __global__ __launch_bounds__(LB) void qw_gemv_quad_kernel(const qq_params p) {
         if (p.y16) p.y16[at] = (h1_t)v;
     }
 }
+};
 
 template <int FMT, int XDT, int MG>
 void qq_launch1(hipStream_t st, const qq_params& p, uint32_t wgs, uint32_t threads, size_t lds) {
     constexpr int D = FMT == QW_FMT_B8 ? 2 : 3;
-    auto kern = qw_gemv_quad_kernel<FMT, XDT, MG, D, 768>;
+    using kern = qw_gemv_quad_kernel<FMT, XDT, MG, D, 768>;
     static std::atomic<bool> attr_done{false};   // per instantiation
     if (!attr_done.load(std::memory_order_acquire)) {
-        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        (void)hipFuncSetAttribute(qw_scalar_kernel_ptr<kern>((const qq_params*)nullptr), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
         attr_done.store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL(kern, dim3(wgs), dim3(threads), lds, st, p);
+    qw_launch_scalar<kern>(dim3(wgs), dim3(threads), lds, st, p);
 }
 
 template <int FMT, int XDT>

@@ -30,15 +30,12 @@
 
 namespace {
 
-struct qsk_params {
-    const uint8_t* bank;
-    const void* x;
-    h1_t* y16;
-    float* y32;
-    float* part;      // [K range][activation row][padded bank row]
-    uint32_t N, K, M, nsl, ks, nkr, bands, gshift, bb, ntiles;
-    uint64_t row_bytes;
-};
+// part: [K range][activation row][padded bank row]
+#define QSK_FIELDS(X)                                                                                                       \
+    X(const uint8_t*, bank) X(const void*, x) X(float*, part) X(uint32_t, N) X(uint32_t, K) X(uint32_t, M) X(uint32_t, nsl)     \
+    X(uint32_t, ks) X(uint32_t, nkr) X(uint32_t, bands) X(uint32_t, gshift) X(h1_t*, y16) X(float*, y32) X(uint32_t, bb)        \
+    X(uint32_t, ntiles) X(uint64_t, row_bytes)
+QW_ARG_BLOCK(qsk_params, QSK_FIELDS)
 
 template <int N, int I = 0, class F>
 __device__ __forceinline__ void qw_static_for(F&& f) {
@@ -101,7 +98,9 @@ __device__ __forceinline__ void qsk_take(uint32_t land4, uint32_t land16, uint32
 // MP * 8 activation rows in the LDS image, D slice groups in flight per lane.  blockDim.x = 64 * waves; dynamic LDS =
 // waves * D landing slots (first: their addresses stay below 64 KiB), then the image of ks slices at MP * 640 bytes each.
 template <int FMT, int XDT, int MP, int D>
-__global__ __launch_bounds__(512) void qw_gemv_sk_kernel(const qsk_params p) {
+struct qw_gemv_sk_kernel {
+static constexpr int kLaunchBound = 512;
+static __device__ __forceinline__ void run(const qsk_params& p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t qsk_lds[];
     constexpr uint32_t ACTS = 8u * MP, SLB = ACTS * 80u, SB = qsk_slot_bytes<FMT>();
     const uint32_t tid = threadIdx.x, lane = tid & 63u, W = blockDim.x >> 6;
@@ -228,6 +227,7 @@ __global__ __launch_bounds__(512) void qw_gemv_sk_kernel(const qsk_params p) {
         if (r16 < p.M) *(f4_t*)(p.part + ((uint64_t)(kr * p.M + r16) * n16 + rbase)) = acc;
     }
 }
+};
 
 // Second launch of a split call: y[m][row] = sum over the K ranges of the partials, in range order.
 __global__ __launch_bounds__(256) void qw_gemv_sk_reduce_kernel(const float* __restrict__ part, h1_t* y16, float* y32, uint32_t N,
@@ -262,14 +262,14 @@ hipError_t qsk_launch(hipStream_t st, const qsk_params& p, uint32_t wgs, uint32_
     // one attribute per instantiation: the image may take most of the 160 KiB of a compute unit
 #define QSK_GO(DD)                                                                                                  \
     {                                                                                                               \
-        auto kern = qw_gemv_sk_kernel<FMT, XDT, MP, DD>;                                                            \
+        using kern = qw_gemv_sk_kernel<FMT, XDT, MP, DD>;                                                           \
         static std::atomic<bool> attr_done{false};                                                                  \
         if (!attr_done.load(std::memory_order_acquire)) {                                                           \
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            hipError_t e = hipFuncSetAttribute(qw_scalar_kernel_ptr<kern>((const qsk_params*)nullptr), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
             if (e != hipSuccess) return e;                                                                          \
             attr_done.store(true, std::memory_order_release);                                                       \
         }                                                                                                           \
-        hipLaunchKernelGGL(kern, dim3(wgs), dim3(threads), lds, st, p);                                             \
+        qw_launch_scalar<kern>(dim3(wgs), dim3(threads), lds, st, p);                                               \
     }
     if (depth == 3) QSK_GO(3) else if (depth == 4) QSK_GO(4) else if (depth == 6) QSK_GO(6) else QSK_GO(2)
 #undef QSK_GO

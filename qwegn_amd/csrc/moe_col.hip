@@ -54,27 +54,22 @@ __device__ __forceinline__ float qmc_block_dot(const qw_hq4_block& b, const h2_t
 // Epilogue: act[pair, n] = f16(FWHT32(silu(g) * u)) over the 32 outputs of the workgroup (rotation optional).
 // blockDim.x = 32 * cpr * SETS; dynamic LDS = nb * 80 + 64 * cpr * 4 bytes.
 // ------------------------------------------------------------------------------------------------
-struct qmc_gu_params {
-    const uint8_t* bank;
-    const void* x;
-    h1_t* act;
-    const int32_t* idx;
-    const int32_t* x_rows;   // activation row of every pair (NULL: the pair's token)
-    qw_act ga;               // the device's gated activation (all zero: SwiGLU)
-    uint32_t I, nb, cpr, top_k, rotate, rot_out;
-    uint64_t expert_bytes;
-    // JN > 0: the routing is done here.  The first wave of every workgroup routes the pair's token from its router logits
-    // (the arithmetic of qw_moe_route_kernel, so the same experts and weights) and the workgroup takes rank pair % top_k;
-    // the workgroups of the first row block leave the pair's expert and weight in idx_out / wts_out for the down projection.
-    const float* logits;
-    int32_t* idx_out;
-    float* wts_out;
-    uint32_t experts, norm;
-    float routed_scale;
-};
+// logits, idx_out, wts_out, experts, norm, routed_scale (JN > 0): the routing is done here.  The first wave of every workgroup
+// routes the pair's token from its router logits (the arithmetic of qw_moe_route_kernel, so the same experts and weights) and
+// the workgroup takes rank pair % top_k; the workgroups of the first row block leave the pair's expert and weight in idx_out /
+// wts_out for the down projection.  x_rows: activation row of every pair (NULL: the pair's token).  ga: the device's gated
+// activation (all zero: SwiGLU).
+#define QMC_GU_FIELDS(X)                                                                                                     \
+    X(const uint8_t*, bank) X(const void*, x) X(h1_t*, act) X(const int32_t*, idx) X(const float*, logits) X(uint32_t, top_k)    \
+    X(uint32_t, nb) X(uint32_t, cpr) X(uint32_t, I) X(uint32_t, rotate) X(uint32_t, rot_out) X(uint64_t, expert_bytes)           \
+    X(const int32_t*, x_rows) X(uint32_t, experts) X(int32_t*, idx_out) X(float*, wts_out) X(uint32_t, norm)                     \
+    X(float, routed_scale) X(qw_act, ga)
+QW_ARG_BLOCK(qmc_gu_params, QMC_GU_FIELDS)
 
 template <int XDT, int SETS, int JN = 0>
-__global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_params p) {
+struct qw_moe_gateup_col_kernel {
+static constexpr int kLaunchBound = 1024;
+static __device__ __forceinline__ void run(const qmc_gu_params& p) {
     constexpr int R = 64 / SETS;
     constexpr int D = R < 8 ? R : 8;             // rows in flight per lane
     constexpr int XT = SETS == 2 ? 2 : 1;        // 16-group activation tiles per wave: ceil(2 cpr / (cpr * SETS / 2))
@@ -177,6 +172,7 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
         if (tid < 32u && n0 + tid < I) act[n0 + tid] = (h1_t)a;
     }
 }
+};
 
 // ------------------------------------------------------------------------------------------------
 // down + combine: grid (ceil(H / (SETS * D)), tokens).  The token's routes are laid side by side as one virtual row of
@@ -185,23 +181,18 @@ __global__ __launch_bounds__(1024) void qw_moe_gateup_col_kernel(const qmc_gu_pa
 //   out[token, n] = sum_k wts[k] * (W_down[e_k][n, :] . act[k, :]) (+ shared_gate * shared[n])
 // blockDim.x = 32 * cprv * SETS, cprv = ceil(top_k * nbI / 32); set j takes rows n0 + j * D .. + D - 1.
 // ------------------------------------------------------------------------------------------------
-struct qmc_dn_params {
-    const uint8_t* bank;
-    const h1_t* act;
-    const int32_t* idx;
-    const float* wts;
-    const float* shared;
-    const float* shared_gate;
-    void* out;
-    uint32_t H, nbI, nbv, cprv, top_k, sets;
-    uint64_t expert_bytes;
-    uint32_t x_div;          // pairs that share one activation row (1: a row per pair)
-    const int32_t* labels;   // num_groups > 0: blockIdx.y = token * num_groups + group, and only the token's routes whose
-    uint32_t num_groups;     // expert carries that group's label are summed
-};
+// labels, num_groups > 0: blockIdx.y = token * num_groups + group, and only the token's routes whose expert carries that
+// group's label are summed.  x_div: pairs that share one activation row (1: a row per pair).
+#define QMC_DN_FIELDS(X)                                                                                                     \
+    X(const uint8_t*, bank) X(const h1_t*, act) X(const int32_t*, idx) X(const float*, wts) X(void*, out) X(uint32_t, top_k)     \
+    X(uint32_t, nbI) X(uint32_t, nbv) X(uint32_t, cprv) X(uint32_t, H) X(uint32_t, sets) X(uint64_t, expert_bytes)               \
+    X(const float*, shared) X(const float*, shared_gate) X(const int32_t*, labels) X(uint32_t, num_groups) X(uint32_t, x_div)
+QW_ARG_BLOCK(qmc_dn_params, QMC_DN_FIELDS)
 
 template <int ODT, int D, bool GRP = false>   // GRP: one output row per (token, latent group)
-__global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_params p) {
+struct qw_moe_down_col_kernel {
+static constexpr int kLaunchBound = 1024;
+static __device__ __forceinline__ void run(const qmc_dn_params& p) {
     __shared__ float part[1024];   // [sets * D rows][cprv]
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 31u, hw = tid >> 5;
@@ -261,6 +252,7 @@ __global__ __launch_bounds__(1024) void qw_moe_down_col_kernel(const qmc_dn_para
         }
     }
 }
+};
 
 }  // namespace
 
@@ -299,7 +291,7 @@ bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expe
     p.norm = norm_topk;
     p.routed_scale = routed_scale;
     const dim3 grid(qwhip_cdiv(inter, 32u), pairs), block(32u * cpr * sets);
-#define QMC_GU(DT, S, J) hipLaunchKernelGGL((qw_moe_gateup_col_kernel<DT, S, J>), grid, block, lds, st, p)
+#define QMC_GU(DT, S, J) qw_launch_scalar<qw_moe_gateup_col_kernel<DT, S, J>>(grid, block, lds, st, p)
 #define QMC_GU_S(DT, J)                                                                                     \
     do {                                                                                                    \
         if (sets == 8u) QMC_GU(DT, 8, J); else if (sets == 4u) QMC_GU(DT, 4, J); else QMC_GU(DT, 2, J);     \
@@ -353,8 +345,8 @@ bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expert
     const dim3 grid(qwhip_cdiv(hidden, sets * D), out_rows), block(32u * cprv * sets);
 #define QMC_DN(OD)                                                                                            \
     do {                                                                                                      \
-        if (num_groups) hipLaunchKernelGGL((qw_moe_down_col_kernel<OD, D, true>), grid, block, 0, st, p);     \
-        else hipLaunchKernelGGL((qw_moe_down_col_kernel<OD, D, false>), grid, block, 0, st, p);               \
+        if (num_groups) qw_launch_scalar<qw_moe_down_col_kernel<OD, D, true>>(grid, block, 0, st, p);         \
+        else qw_launch_scalar<qw_moe_down_col_kernel<OD, D, false>>(grid, block, 0, st, p);                   \
     } while (0)
     if (out_dtype == QWHIP_F32) QMC_DN(QWHIP_F32);
     else if (out_dtype == QWHIP_F16) QMC_DN(QWHIP_F16);
