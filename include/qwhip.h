@@ -136,8 +136,9 @@ qwhip_status qwhip_weight_view_validate(const qwhip_weight_view* w);
 enum {
     /* Activations are already in the container's basis (rotated per 32-group for a rotated
      * container).  Without it the launcher rotates them itself: FWHT-32 in fp32, one f16
-     * rounding, fused into the kernel prologue (QWWeightView.isRotated contract,
-     * QWWeightView.swift:33-38; producer-side rotation Sources/QWMetal/include/qw_dequant.metalh:424-493). */
+     * rounding, fused into the kernel prologue for one row, one pass into the stream's scratch
+     * for several (QWWeightView.isRotated contract, QWWeightView.swift:33-38; producer-side
+     * rotation Sources/QWMetal/include/qw_dequant.metalh:424-493). */
     QWHIP_X_PREROTATED = 1u << 0
 };
 

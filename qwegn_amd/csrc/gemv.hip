@@ -1037,6 +1037,21 @@ static qwhip_status qw_gemv_impl(qwhip_stream_t s, const qwhip_weight_view* w, c
     a.rotate = rotate ? 1u : 0u;
     a.rot_out = 0;
 
+    // Several un-rotated rows on a rotated container: one rotation pass (fp32 butterfly, one f16 rounding: what the fused
+    // prologues compute) into the stream's scratch, then the kernels for rows already in the basis, instead of the per-lane
+    // rotation of the MFMA streamer.  Kernel overrides keep their own paths.
+    const size_t xrot_bytes = (size_t)m * w->k * 2u;
+    // two rows whose rotated copy fits the streamers' LDS prologue stay there where that measured level or ahead: the DMA
+    // streamer on small banks, the MFMA streamer on 8-bit banks (N = 7168, K = 5120, HQ8: 11.1 against 11.8 us; HQ4_G32_M5,
+    // N = 17408, K = 5120: 18.3 against 14.6 us with the pass, so the 4-bit banks take the pass)
+    const bool fused_two = fmt < QW_FMT_B2 && m == 2 && ((w->n <= 4096 && w->k <= 8192) || (fmt == QW_FMT_B8 && w->k <= 8192));
+    if (variant == 0 && rotate && m > 1 && !fused_two && s->scratch && s->scratch_bytes >= QWHIP_STREAM_SCRATCH_BYTES &&
+        xrot_bytes <= QWHIP_STREAM_XROT_BYTES) {
+        void* xr = s->scratch + s->scratch_bytes - QWHIP_STREAM_XROT_BYTES;
+        st = qwhip_fwht32(s, x, x_dtype, xr, (uint64_t)m * w->k);
+        if (st != QWHIP_OK) return st;
+        return qw_gemv_impl(s, w, xr, QWHIP_F16, m, flags | QWHIP_X_PREROTATED, y16, y32, token, folded);
+    }
     // 2-, 3- and 6-bit streams: the column-stationary dot2 kernel is their one decode kernel (eight rows per launch)
     if (fmt >= QW_FMT_B2) {
         if (rotate && m > 1)

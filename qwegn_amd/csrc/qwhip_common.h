@@ -25,7 +25,10 @@ struct qwhip_device_s {
 // The first QWHIP_STREAM_COUNTER_BYTES hold per-row-tile arrival counters, zero between launches (the last arriver resets
 // its counter), the rest holds fp32 partial outputs.
 #define QWHIP_STREAM_COUNTER_BYTES (64u << 10)
-#define QWHIP_STREAM_SCRATCH_BYTES ((8u << 20) + QWHIP_STREAM_COUNTER_BYTES)
+// The last QWHIP_STREAM_XROT_BYTES hold the rotated copy of several un-rotated activation rows (qwhip_gemv on a rotated
+// container: one rotation pass, then the kernels for rows already in the basis).
+#define QWHIP_STREAM_XROT_BYTES (1u << 20)
+#define QWHIP_STREAM_SCRATCH_BYTES ((8u << 20) + QWHIP_STREAM_COUNTER_BYTES + QWHIP_STREAM_XROT_BYTES)
 struct qwhip_stream_s {
     qwhip_device_s* dev;
     hipStream_t stream;

@@ -281,15 +281,51 @@ def test_gemv_narrow_and_six_bit_streams(dev, fmt, m):
 @pytest.mark.parametrize("fmt", ["hq3_g32", "hq6_g32"])
 @pytest.mark.parametrize("xdtype", ["f16", "bf16"])
 def test_gemv_narrow_streams_fused_rotation_and_basis_errors(dev, fmt, xdtype):
-    """One un-rotated row is rotated in the prologue; several un-rotated rows are refused (QWHIP_E_BASIS) before any
-    launch."""
+    """One un-rotated row is rotated in the prologue; several un-rotated rows are rotated once into the stream's scratch
+    and then run as rows in the basis; under a kernel override there is no such pass and the rows are refused
+    (QWHIP_E_BASIS) before any launch."""
     g16, g32, ref = _run_gemv(dev, fmt, 100, 2048, 1, prerot=False, xdtype=xdtype, seed=7)
     assert qo.normalized_error(g32, _affine_ref(fmt, 100, 2048, 1, 7, xdtype)) <= 2e-5
+    g16, g32, ref = _run_gemv(dev, fmt, 100, 2048, 11, prerot=False, xdtype=xdtype, seed=8)
+    assert qo.normalized_error(g32, _affine_ref(fmt, 100, 2048, 11, 8, xdtype)) <= 2e-5
+    assert qo.normalized_error(g16, ref) <= TOL
     blocks, _ = H.make_bank(fmt, 64, 256, seed=1)
     bank, xb, yb = dev.put(blocks), dev.put(np.zeros((4, 256), np.float16)), dev.alloc(4 * 64 * 4)
     view = H.view_of(dev, bank, fmt, 64, 256)
     st = dev.stream.handle
-    assert dev.lib.qwhip_gemv(st, C.byref(view), xb.ptr, qwhip.F16, 4, 0, None, yb.ptr) == qwhip.E_BASIS
+    assert dev.lib.qwhip_gemv(st, C.byref(view), xb.ptr, qwhip.F16, 4, 6 << 8, None, yb.ptr) == qwhip.E_BASIS
+
+
+@pytest.mark.parametrize("fmt,n,k", [("hq4_g32_m5", 300, 5120), ("hq8_g32", 272, 1536), ("hq4_g64", 96, 17408), ("hq6_g32", 130, 2048)])
+@pytest.mark.parametrize("m", [2, 5, 16])
+@pytest.mark.parametrize("xdtype", ["f16", "bf16"])
+def test_gemv_several_unrotated_rows_equal_the_rows_rotated_first(dev, fmt, n, k, m, xdtype):
+    """A rotated container given m > 1 un-rotated rows: the launcher's rotation pass + the kernels for rows in the basis.
+    Bit-identical to qwhip_fwht32 followed by the pre-rotated call (the same two steps done by the caller), except where
+    two rows stay on a streamer kernel."""
+    blocks, w16 = H.make_bank(fmt, n, k, seed=21)
+    x32 = H.make_x(m, k, 121)
+    if xdtype == "f16":
+        x_host, code = x32.astype(np.float16), qwhip.F16
+    else:
+        x_host, code = _bf16(x32), qwhip.BF16
+    bank, xb = dev.put(blocks), dev.put(x_host)
+    xr, ya, yb_ = dev.alloc(m * k * 2), dev.alloc(m * n * 4), dev.alloc(m * n * 4)
+    view = H.view_of(dev, bank, fmt, n, k)
+    st = dev.stream.handle
+    qwhip.check(dev.lib.qwhip_gemv(st, C.byref(view), xb.ptr, code, m, 0, None, ya.ptr))
+    qwhip.check(dev.lib.qwhip_fwht32(st, xb.ptr, code, xr.ptr, m * k))
+    qwhip.check(dev.lib.qwhip_gemv(st, C.byref(view), xr.ptr, qwhip.F16, m, qwhip.X_PREROTATED, None, yb_.ptr))
+    dev.stream.sync()
+    a, b = ya.download(np.float32, (m, n)), yb_.download(np.float32, (m, n))
+    x_basis = xr.download(np.float16, (m, k))
+    for buf in (bank, xb, xr, ya, yb_):
+        buf.free()
+    if m == 2 and k <= 8192:   # two rows on a small bank stay on a streamer (rotation in its prologue, exact f16 weights)
+        assert qo.normalized_error(a, b) <= 1e-3
+    else:
+        assert np.array_equal(a, b)
+    assert qo.normalized_error(a, qo.matmul_ref_f64(x_basis, w16)) <= TOL
 
 
 @pytest.mark.parametrize("m", [1, 4])
@@ -302,8 +338,9 @@ def test_gemv_column_stationary_long_rows(dev, m):
 
 @pytest.mark.parametrize("m", [2, 16])
 def test_gemv_rotation_per_lane_path(dev, m):
-    """m*k too large for the LDS staging: rotation runs per lane from global memory."""
-    g16, g32, ref = _run_gemv(dev, "hq4_g64", 96, 17408, m, prerot=False, seed=6)
+    """m*k too large for the LDS staging: on the MFMA streamer (kernel override 2) the rotation runs per lane from global
+    memory."""
+    g16, g32, ref = _run_gemv(dev, "hq4_g64", 96, 17408, m, prerot=False, seed=6, variant=2)
     assert qo.normalized_error(g32, ref) <= 2e-5
 
 
