@@ -461,16 +461,19 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 
     // ---- activation tile: chunk c = tid + i * NT -> tile row (tid >> 3) + (NT / 8) * i, 16-byte k-chunk tid & 7.
     // Global -> registers one K-step ahead (coalesced 128-byte rows), registers -> LDS slot (k-chunk ^ ((row >> 1) & 7)).
-    // One per-thread offset, the row block (NT / 8 rows) is a wave-uniform term; blocks past the tile's rows
-    // re-read block 0 (their outputs are never stored), so M must be a multiple of NT / 8 = 64.
+    // One byte offset per thread and row block; rows past the tile's last one re-read the tile's first row (their
+    // outputs are never stored), so any M is taken.
     constexpr int A_LD = BM * 8 / NT;
     static_assert((BM * 8) % NT == 0, "activation tile must split evenly over the workgroup");
     constexpr uint32_t A_BLK = NT / 8;
     const uint32_t a_lds0 = (tid >> 3) * 128u + (((tid & 7u) ^ ((tid >> 4) & 7u)) << 4);   // + i * A_BLK * 128 (swizzle key unchanged)
-    const uint32_t a_voff = (tid >> 3) * p.ldx * 2u + (tid & 7u) * 16u;
     const uint64_t a_tile_base = (uint64_t)m0 * p.ldx * 2u;
-    const uint64_t a_blk_stride = (uint64_t)A_BLK * p.ldx * 2u;
-    const uint32_t a_blocks = rows_valid / A_BLK;
+    uint64_t a_off[A_LD];
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) {
+        const uint32_t r = (tid >> 3) + (uint32_t)i * A_BLK;
+        a_off[i] = (r < rows_valid ? (uint64_t)r * p.ldx * 2u : 0ull) + (tid & 7u) * 16u;
+    }
 
     // ---- weight tile: item = (tile row, 32-column slice); thread items tid and NT + (tid % (B_ITEMS - NT)) (items past
     // the tile are done redundantly by several threads: identical bytes to the same slot) ----
@@ -505,10 +508,8 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 
     auto load_a = [&](uint32_t kt, u4_t* a_reg) {
 #pragma unroll
-        for (int i = 0; i < A_LD; ++i) {
-            const uint32_t blk = (uint32_t)i < a_blocks ? (uint32_t)i : 0u;
-            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + blk * a_blk_stride + (uint64_t)kt * 128u + a_voff);
-        }
+        for (int i = 0; i < A_LD; ++i)
+            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + a_off[i] + (uint64_t)kt * 128u);
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
@@ -1295,10 +1296,10 @@ enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_256x128 = 3, CFG_C
 static const uint32_t kCfgBM[CFG_COUNT] = {256, 256, 128, 256};
 static const uint32_t kCfgBN[CFG_COUNT] = {320, 256, 128, 128};
 
-// the ping-pong kernel takes whole 64-row activation blocks on the 256 x 320 tile, every container but the 8-bit ones, and
-// 2-byte outputs whose rows are 16-byte aligned
+// the ping-pong kernel takes the 256 x 320 tile at any row count, every container but the 8-bit ones, and 2-byte outputs
+// whose rows are 16-byte aligned
 inline bool gemm3_takes(const qw_gemm_params& p, int cfg, int fmt, uint32_t ydt) {
-    return cfg == CFG_256x320 && fmt != QG_FMT_B8 && p.M % 64u == 0 && !p.force_gemm2 &&
+    return cfg == CFG_256x320 && fmt != QG_FMT_B8 && !p.force_gemm2 &&
            (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0));
 }
 
@@ -1310,9 +1311,9 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     const dim3 grid(((total + 7u) / 8u) * 8u);
     switch (cfg) {
         case CFG_256x320:
-            // the ping-pong kernel takes whole 64-row activation blocks; ragged M stays on the DMA-fed kernel, and so do the
-            // 8-bit containers: their wider weight items do not fit the ping-pong kernel's register budget at this tile (the
-            // 6-bit streams spill three to five registers there and still run a sixth faster than on the DMA-fed kernel)
+            // the 8-bit containers stay on the DMA-fed kernel: their wider weight items do not fit the ping-pong kernel's
+            // register budget at this tile (the 6-bit streams spill three to five registers there and still run a sixth
+            // faster than on the DMA-fed kernel)
             if constexpr (FMT != QG_FMT_B8) {
                 if (gemm3_takes(p, cfg, FMT, YDT)) {
                     if (p.x_bf16) return launch_cfg3<2, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
@@ -1527,13 +1528,13 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     if (m == 0) return QWHIP_OK;
     const uint32_t inter = w->n / 2u;
     if (w->n % 64u != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "fused gate_up needs an intermediate size %% 32 == 0, got %u rows", w->n);
-    if (fmt == QG_FMT_B8 || fmt == QG_FMT_B6 || m % 64u != 0) {   // the 6- and 8-bit weight items do not fit the fused kernel's registers
-        // other containers and row counts: the two launches inside the door, through the caller's workspace
+    if (fmt == QG_FMT_B8 || fmt == QG_FMT_B6) {   // the 6- and 8-bit weight items do not fit the fused kernel's registers
+        // these containers: the two launches inside the door, through the caller's workspace
         // ([m, 2 inter] f16 first, the rest for qwhip_gemm's own copy of the activations); same bits as the two doors
         const uint64_t gu_bytes = (uint64_t)m * w->n * 2u;
         if (!workspace || ((uintptr_t)workspace & 15u) || workspace_bytes < gu_bytes || (ldact != 0 && ldact != inter) || ((uintptr_t)act_f16 & 15u))
             return qwhip_fail(QWHIP_E_BAD_GEOMETRY,
-                              "the fused gate_up GEMM takes 2-, 3- and 4-bit containers and m %% 64 == 0 in one launch (m=%u); other calls need a 16-byte "
+                              "the fused gate_up GEMM takes 2-, 3- and 4-bit containers in one launch (m=%u); the 6- and 8-bit ones need a 16-byte "
                               "aligned workspace of m * n * 2 bytes (plus m * k * 2 for bf16 or un-rotated activations) and packed act rows", m);
         const uint64_t rest = workspace_bytes - gu_bytes;
         st = qwhip_gemm(s, w, x, x_dtype, m, ldx, workspace, QWHIP_F16, 0, flags & QWHIP_X_PREROTATED, rest ? (uint8_t*)workspace + gu_bytes : nullptr, rest);
