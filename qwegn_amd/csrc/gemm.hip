@@ -1292,14 +1292,14 @@ inline bool gemm5_takes(const qw_gemm_params& p, int fmt) {
 }
 
 // tile shapes of the pipelined kernel
-enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_256x128 = 3, CFG_COUNT = 4 };
-static const uint32_t kCfgBM[CFG_COUNT] = {256, 256, 128, 256};
-static const uint32_t kCfgBN[CFG_COUNT] = {320, 256, 128, 128};
+enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_256x128 = 3, CFG_128x320 = 4, CFG_COUNT = 5 };
+static const uint32_t kCfgBM[CFG_COUNT] = {256, 256, 128, 256, 128};
+static const uint32_t kCfgBN[CFG_COUNT] = {320, 256, 128, 128, 320};
 
 // the ping-pong kernel takes the 256 x 320 tile at any row count, every container but the 8-bit ones, and 2-byte outputs
 // whose rows are 16-byte aligned
 inline bool gemm3_takes(const qw_gemm_params& p, int cfg, int fmt, uint32_t ydt) {
-    return cfg == CFG_256x320 && fmt != QG_FMT_B8 && !p.force_gemm2 &&
+    return (cfg == CFG_256x320 || cfg == CFG_128x320) && fmt != QG_FMT_B8 && !p.force_gemm2 &&
            (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0));
 }
 
@@ -1321,6 +1321,14 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
                 }
             }
             return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
+        case CFG_128x320:
+            if constexpr (FMT != QG_FMT_B8) {
+                if (gemm3_takes(p, cfg, FMT, YDT)) {
+                    if (p.x_bf16) return launch_cfg3<1, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
+                    return launch_cfg3<1, 5, 4, 2, FMT, YDT>(st, p, grid);
+                }
+            }
+            return launch_cfg2<1, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x256: return launch_cfg2<2, 4, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x128: return launch_cfg2<2, 2, 4, 2, FMT, YDT, false>(st, p, grid);
         default: return launch_cfg2<2, 2, 2, 2, FMT, YDT, false>(st, p, grid);
@@ -1346,18 +1354,28 @@ hipError_t launch_dense1_y(hipStream_t st, qw_gemm_params& p, uint32_t ydt) {
     return launch_cfg<2, 2, 2, 2, FMT, XDT, QWHIP_F32, false>(st, p, grid);
 }
 
-// waste-aware choice among the tile shapes: time ~ rounds of tiles over the CUs x per-tile cost / shape efficiency
-int choose_cfg(uint32_t M, uint32_t N) {
-    // relative matrix-core efficiency of each shape (measured on M = 4096, N = K = 5120) and workgroups resident per CU
-    const double eff[CFG_COUNT] = {1.00, 0.82, 0.78, 0.75};
-    const double resident[CFG_COUNT] = {1, 1, 2, 1};
+// waste-aware choice among the tile shapes: time ~ rounds of tiles over the CUs x per-tile cost / shape efficiency.
+// `pingpong`: the 256 x 320 and 128 x 320 shapes run the ping-pong kernel (every container but the 8-bit ones), which is 1.4x
+// the DMA-fed kernel on the same tile (188 against 264 us on M = 4096, N = K = 5120); `only_pingpong` keeps the choice to
+// those two shapes (bf16 activations with no workspace to convert into: the other kernels would fall to the unpipelined one).
+int choose_cfg(uint32_t M, uint32_t N, bool pingpong, bool only_pingpong) {
+    // relative matrix-core efficiency of each shape on the DMA-fed kernel (measured on M = 4096, N = K = 5120; the half-height
+    // tile from M = 2048: 256 tiles in 115 us where the 128 tiles of 256 x 320 take 144) and workgroups resident per CU
+    const double eff2[CFG_COUNT] = {1.00, 0.82, 0.78, 0.75, 0.82};
+    const double resident[CFG_COUNT] = {1, 1, 2, 1, 1};
+    // a problem of few tiles is one tile's K loop long whatever the shape, and the small tile's loop is the shortest
+    // (N = K = 5120, f16: M = 64 in 65 us on 128 x 128 against 82 us on the half-height ping-pong tile, M = 256 82 against 85)
+    if ((uint64_t)qwhip_cdiv(M, 128u) * qwhip_cdiv(N, 128u) <= 128u) return CFG_128x128;
     double best = 1e300;
-    int best_cfg = CFG_128x128;
+    int best_cfg = only_pingpong ? CFG_256x320 : CFG_128x128;
     for (int c = 0; c < CFG_COUNT; ++c) {
+        const bool pp = c == CFG_256x320 || c == CFG_128x320;
+        if (only_pingpong && !pp) continue;
+        const double eff = eff2[c] * ((pingpong && !pp) ? 0.71 : 1.0);
         const double tiles = (double)qwhip_cdiv(M, kCfgBM[c]) * qwhip_cdiv(N, kCfgBN[c]);
         const double slots = 256.0 * resident[c];
         const double rounds = (double)(uint64_t)((tiles + slots - 1.0) / slots);
-        const double cost = rounds * resident[c] * kCfgBM[c] * kCfgBN[c] / eff[c];
+        const double cost = rounds * resident[c] * kCfgBM[c] * kCfgBN[c] / eff;
         if (cost < best) {
             best = cost;
             best_cfg = c;
@@ -1424,7 +1442,10 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     const void* xin = x;
     uint32_t xdt = x_dtype;
     const uint32_t ov = (flags >> 8) & 0xFu;
-    const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n));
+    // 2-byte outputs reach the ping-pong kernel with 16-byte aligned rows only (gemm3_takes)
+    const bool pp_ok = fmt != QG_FMT_B8 && (y_dtype == QWHIP_F32 || (ldy % 8u == 0 && ((uintptr_t)y & 15u) == 0));
+    const bool bf16_in_place = pp_ok && !rotate && x_dtype == QWHIP_BF16 && !ws_ok && !(flags & (1u << 16));
+    const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n, pp_ok, bf16_in_place));
     qw_gemm_params p = {};
     p.M = m;
     p.ldy = ldy;

@@ -58,7 +58,7 @@ def run_gemm(dev, fmt, m, n, k, *, xdtype="bf16", ydtype="bf16", prerot=True, cf
     return st, out, ref
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 14, 15])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 14, 15])
 def test_gemm_hq4_tile_shapes_f32_out(dev, cfg):
     st, out, ref = run_gemm(dev, "hq4_g32_m5", 512, 640, 1024, ydtype="f32", cfg=cfg)
     assert st == qwhip.OK
@@ -91,26 +91,37 @@ def test_gemm_narrow_and_six_bit_streams_on_every_kernel(dev, fmt, cfg, xdtype, 
 
 
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "aq4_g32", "hq8_g32", "hq4_g64", "aq2_g64", "hq3_g32", "hq6_g32"])
-def test_gemm_pingpong_kernel_ragged_tiles(dev, fmt):
-    """The 8-wave ping-pong kernel (256 x 320 tiles, whole 64-row activation blocks) on a shape whose last tile row
-    holds one 64-row block and whose last tile column is ragged, for every weight format family."""
-    st, out, ref = run_gemm(dev, fmt, 320, 400, 640, xdtype="f16", ydtype="f32", cfg=1, seed=5)
+@pytest.mark.parametrize("cfg", [1, 5])
+def test_gemm_pingpong_kernel_ragged_tiles(dev, fmt, cfg):
+    """The 8-wave ping-pong kernel (256 x 320 and 128 x 320 tiles; the 8-bit containers run the DMA-fed kernel at these
+    shapes) on a shape whose last tile row holds one 64-row block and whose last tile column is ragged, for every weight
+    format family."""
+    st, out, ref = run_gemm(dev, fmt, 320, 400, 640, xdtype="f16", ydtype="f32", cfg=cfg, seed=5)
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= 2e-5
-    st, out, ref = run_gemm(dev, fmt, 64, 320, 64, xdtype="bf16", ydtype="bf16", cfg=1, seed=6)   # a single K-step
+    st, out, ref = run_gemm(dev, fmt, 64, 320, 64, xdtype="bf16", ydtype="bf16", cfg=cfg, seed=6)   # a single K-step
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= TOL
 
 
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "aq4_g32", "hq4_g64", "aq2_g64", "hq3_g32", "hq6_g32"])
 @pytest.mark.parametrize("m", [1, 37, 100, 257, 333, 575])
-def test_gemm_pingpong_kernel_ragged_rows(dev, fmt, m):
-    """Row counts that are not whole 64-row blocks on the ping-pong kernel: threads whose row lies past the last one re-read
-    the tile's first row and store nothing (a last tile row of 1, 37, 36, 1, 77 and 63 rows; one tile of fewer than 64)."""
-    st, out, ref = run_gemm(dev, fmt, m, 400, 320, xdtype="f16", ydtype="f32", cfg=1, seed=7)
+@pytest.mark.parametrize("cfg", [1, 5])
+def test_gemm_pingpong_kernel_ragged_rows(dev, fmt, m, cfg):
+    """Row counts that are not whole 64-row blocks on the ping-pong kernel (256 x 320 and 128 x 320 tiles): threads whose row
+    lies past the last one re-read the tile's first row and store nothing (last tile rows of 1 to 77 rows; one tile of
+    fewer than 64)."""
+    st, out, ref = run_gemm(dev, fmt, m, 400, 320, xdtype="f16", ydtype="f32", cfg=cfg, seed=7)
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= 2e-5
-    st, out, ref = run_gemm(dev, fmt, m, 336, 192, xdtype="bf16", ydtype="bf16", cfg=1, seed=8)
+    st, out, ref = run_gemm(dev, fmt, m, 336, 192, xdtype="bf16", ydtype="bf16", cfg=cfg, seed=8)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= TOL
+
+
+def test_gemm_half_height_tile_at_2048_rows(dev):
+    """M = 2048 on the benchmark bank: the automatic choice is the ping-pong kernel's 128 x 320 tile (256 tiles)."""
+    st, out, ref = run_gemm(dev, "hq4_g32_m5", 2048, 5120, 5120, xdtype="bf16", ydtype="bf16")
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= TOL
 
