@@ -271,7 +271,11 @@ qwhip_status qwhip_embed_bf16_f32(qwhip_stream_t s, const void* table_bf16, uint
  * x: f16 or bf16 [m, ldx]; y: f16, bf16 or f32 [m, ldy]; ldx/ldy in elements (0 = tight).
  * Requires k % 64 == 0 and n % 16 == 0 else QWHIP_E_BAD_GEOMETRY (the reference's tensor path
  * requires N, K multiples of 64).  Activations must be in the container's basis
- * (QWHIP_X_PREROTATED) unless `workspace` holds m*k f16 elements for the rotated copy. */
+ * (QWHIP_X_PREROTATED) unless `workspace` holds m*k f16 elements for the rotated copy.
+ * A problem of few tiles (about m * n <= 128 * 128 * 320) whose workspace also holds fp32 planes of m * n
+ * elements (after the activation copy, rounded up to 256 bytes, when there is one) runs its K-steps in 2..8
+ * ranges and sums the planes in range order in a second launch; the result depends on the workspace size
+ * only through that choice, never on its contents. */
 qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                         uint32_t m, uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags,
                         void* workspace, uint64_t workspace_bytes);

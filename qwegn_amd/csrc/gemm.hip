@@ -504,12 +504,16 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
 
     const uint32_t magic = qw_vgpr_const(0x64006400u);
-    const uint32_t nk = p.K / BK;
+    // K range: blockIdx.y splits the K-steps (fp32 partial outputs, one [M, ldy] plane per range; gridDim.y = 1 otherwise)
+    const uint32_t nk_all = p.K / BK;
+    const uint32_t nk_per = (nk_all + gridDim.y - 1u) / gridDim.y;
+    const uint32_t kt0 = blockIdx.y * nk_per;
+    const uint32_t nk = min(nk_per, nk_all - kt0);
 
     auto load_a = [&](uint32_t kt, u4_t* a_reg) {
 #pragma unroll
         for (int i = 0; i < A_LD; ++i)
-            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + a_off[i] + (uint64_t)kt * 128u);
+            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + a_off[i] + (uint64_t)(kt0 + kt) * 128u);
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
@@ -517,7 +521,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     };
     auto load_b = [&](uint32_t kt, qg_slice<FMT>* b_reg, int nitems) {
 #pragma unroll
-        for (int i = 0; i < B_PER; ++i) if (i < nitems) qg_load_slice<FMT>(b_tile + b_off32[i], kt * 2u + (b_meta[i] >> 20), p.gshift, p.bb, b_reg[i]);
+        for (int i = 0; i < B_PER; ++i) if (i < nitems) qg_load_slice<FMT>(b_tile + b_off32[i], (kt0 + kt) * 2u + (b_meta[i] >> 20), p.gshift, p.bb, b_reg[i]);
     };
     // When the second items number a quarter of the workgroup, each is shared by the two group-0 threads tid and
     // tid + NT / 4: one dequantizes its chunks 0..1, the other 2..3 (half the second pass instead of doing it twice).
@@ -774,7 +778,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const uint32_t row = (wm * WM + a) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                        if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
+                        if (row < rows_valid) qg_store<YDT>(p.y, (uint64_t)blockIdx.y * p.M * p.ldy + (uint64_t)(m0 + row) * p.ldy + n, acc[a][b][r]);
                     }
                 }
             }
@@ -1266,6 +1270,22 @@ hipError_t launch_cfg3(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     return hipGetLastError();
 }
 
+// ---- split-K for problems of few tiles: fp32 partial planes, summed in range order ---------------------------------------
+template <int YDT>
+__global__ __launch_bounds__(256) void qw_splitk_reduce_kernel(const float* __restrict__ part, uint32_t splits, uint32_t M, uint32_t N,
+                                                               void* __restrict__ y, uint32_t ldy) {
+    const uint32_t n4 = N / 4u;
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= (uint64_t)M * n4) return;
+    const uint32_t row = (uint32_t)(i / n4), c = (uint32_t)(i - (uint64_t)row * n4) * 4u;
+    const uint64_t plane = (uint64_t)M * N;
+    typedef float fl4_t __attribute__((ext_vector_type(4)));
+    fl4_t acc = *(const fl4_t*)(part + (uint64_t)row * N + c);
+    for (uint32_t sidx = 1; sidx < splits; ++sidx) acc += *(const fl4_t*)(part + sidx * plane + (uint64_t)row * N + c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) qg_store<YDT>(y, (uint64_t)row * ldy + c + e, acc[e]);
+}
+
 template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
 hipError_t launch_cfg4(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     // two activation stages, or the four epilogue slabs (32 rows x (128 + 16) bytes each) when they are larger
@@ -1408,6 +1428,29 @@ qwhip_status gemm_checks(qwhip_stream_t s, const qwhip_weight_view* w, const voi
 }
 
 // runs EXPR with F bound to the container format as a constant
+// split-K launch of the half-height ping-pong tile into fp32 planes at `part`, then the sum into y
+template <int FMT>
+hipError_t launch_splitk(hipStream_t st, const qw_gemm_params& p, uint32_t splits, float* part, void* y, uint32_t y_dtype, uint32_t ldy) {
+    if constexpr (FMT == QG_FMT_B8) {
+        return hipErrorInvalidValue;   // the 8-bit containers do not run the ping-pong kernel
+    } else {
+        qw_gemm_params q = p;
+        q.y = part;
+        q.ldy = p.N;
+        q.tiles_m = qwhip_cdiv(p.M, kCfgBM[CFG_128x320]);
+        q.tiles_n = qwhip_cdiv(p.N, kCfgBN[CFG_128x320]);
+        const dim3 grid(((q.tiles_m * q.tiles_n + 7u) / 8u) * 8u, splits);
+        hipError_t e = p.x_bf16 ? launch_cfg3<1, 5, 4, 2, FMT, QWHIP_F32, false, QWHIP_BF16>(st, q, grid)
+                                : launch_cfg3<1, 5, 4, 2, FMT, QWHIP_F32>(st, q, grid);
+        if (e != hipSuccess) return e;
+        const dim3 rgrid((unsigned)(((uint64_t)p.M * (p.N / 4u) + 255u) / 256u));
+        if (y_dtype == QWHIP_F16) hipLaunchKernelGGL(qw_splitk_reduce_kernel<QWHIP_F16>, rgrid, dim3(256), 0, st, part, splits, p.M, p.N, y, ldy);
+        else if (y_dtype == QWHIP_BF16) hipLaunchKernelGGL(qw_splitk_reduce_kernel<QWHIP_BF16>, rgrid, dim3(256), 0, st, part, splits, p.M, p.N, y, ldy);
+        else hipLaunchKernelGGL(qw_splitk_reduce_kernel<QWHIP_F32>, rgrid, dim3(256), 0, st, part, splits, p.M, p.N, y, ldy);
+        return hipGetLastError();
+    }
+}
+
 #define QG_FOR_FMT(fmt, e, EXPR)                                                  \
     switch (fmt) {                                                                \
         case QG_FMT_M5: { constexpr int F = QG_FMT_M5; e = (EXPR); } break;       \
@@ -1485,6 +1528,23 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     p.bb = qwhip_view_block_bytes(w);
     p.row_bytes = qwhip_view_row_bytes(w);
     hipError_t e;
+    // Split-K: a problem of few tiles is one tile's K loop long (80 K-steps of ~1.1 us on K = 5120, whatever M).  When the
+    // workspace also holds fp32 partial planes (after the activation copy, if there is one), the K-steps of a tile are dealt
+    // over 2..8 workgroups and a second launch sums the planes in range order.
+    if (ov == 0u && pp_ok && xdt == QWHIP_F16 && workspace && ((uintptr_t)workspace & 15u) == 0 && w->n % 4u == 0) {
+        const uint32_t tiles = qwhip_cdiv(m, kCfgBM[CFG_128x320]) * qwhip_cdiv(w->n, kCfgBN[CFG_128x320]);
+        const uint32_t nk = w->k / 64u;
+        const uint64_t used = xin == workspace ? ((ws_need + 255u) & ~(uint64_t)255u) : 0u;
+        const uint64_t plane = (uint64_t)m * w->n * 4u;
+        uint32_t splits = min(min(8u, 256u / tiles), nk / 8u);
+        while (splits >= 2u && ((uint64_t)(splits - 1u) * qwhip_cdiv(nk, splits) >= nk || used + splits * plane > workspace_bytes)) --splits;
+        if (splits >= 2u) {
+            float* part = (float*)((uint8_t*)workspace + used);
+            QG_FOR_FMT(fmt, e, (launch_splitk<F>(s->stream, p, splits, part, y, y_dtype, ldy)))
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+    }
     if (xdt != QWHIP_F16 || ov == 15u) {
         if (xdt == QWHIP_F16) {
             QG_FOR_FMT(fmt, e, (launch_dense1_y<F, QWHIP_F16>(s->stream, p, y_dtype)))
@@ -1534,7 +1594,8 @@ extern "C" qwhip_status qwhip_gemm_noalloc(qwhip_stream_t s, const qwhip_weight_
     const int ord = s->dev->ordinal;
     void* scratch = (ord >= 0 && ord < QW_GEMM_SCRATCH_DEVICES) ? qw_gemm_scratch_ptr[ord] : nullptr;
     if (!scratch) return qwhip_fail(QWHIP_E_DEVICE, "qwhip_gemm_noalloc: device %d has no resolved scratch array", ord);
-    return qwhip_gemm(s, w, x, x_dtype, m, ldx, y, y_dtype, ldy, flags, scratch, QW_GEMM_SCRATCH_BYTES);
+    // exactly the bytes of the activation copy: the same launches as qwhip_gemm with a workspace of that size (no split-K planes)
+    return qwhip_gemm(s, w, x, x_dtype, m, ldx, y, y_dtype, ldy, flags, scratch, need);
 }
 
 // Dense gate|up GEMM with the SwiGLU (+ FWHT-32) epilogue fused: act f16 [m, inter], inter = n / 2, the bank's rows being

@@ -18,7 +18,7 @@ def dev():
     return qwhip.Device(0)
 
 
-def run_gemm(dev, fmt, m, n, k, *, xdtype="bf16", ydtype="bf16", prerot=True, cfg=0, seed=0, workspace=True):
+def run_gemm(dev, fmt, m, n, k, *, xdtype="bf16", ydtype="bf16", prerot=True, cfg=0, seed=0, workspace=True, workspace_bytes=None):
     blocks, w16 = H.make_bank(fmt, n, k, seed=seed)
     x32 = H.make_x(m, k, seed + 7)
     rotate = H.FORMATS[fmt][4]
@@ -38,7 +38,7 @@ def run_gemm(dev, fmt, m, n, k, *, xdtype="bf16", ydtype="bf16", prerot=True, cf
     ysize = {"bf16": 2, "f16": 2, "f32": 4}[ydtype]
     ycode = {"bf16": qwhip.BF16, "f16": qwhip.F16, "f32": qwhip.F32}[ydtype]
     bank, xb, yb = dev.put(blocks), dev.put(x_host), dev.alloc(m * n * ysize)
-    ws = dev.alloc(m * k * 2) if workspace else None
+    ws = dev.alloc(workspace_bytes if workspace_bytes else m * k * 2) if workspace else None
     view = H.view_of(dev, bank, fmt, n, k)
     st = dev.lib.qwhip_gemm(dev.stream.handle, C.byref(view), xb.ptr, xcode, m, 0, yb.ptr, ycode, 0, flags,
                             ws.ptr if ws else None, ws.nbytes if ws else 0)
@@ -129,6 +129,27 @@ def test_gemm_half_height_tile_at_2048_rows(dev):
 def test_gemm_ragged_rows_at_the_prefill_shape(dev):
     """M = 4001 on the benchmark bank (automatic dispatch, bf16 in / bf16 out): the last tile row holds 161 rows."""
     st, out, ref = run_gemm(dev, "hq4_g32_m5", 4001, 5120, 5120, xdtype="bf16", ydtype="bf16")
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "aq2_g64", "hq3_g32", "hq6_g32", "hq8_g32"])
+@pytest.mark.parametrize("m,n,k", [(64, 640, 1024), (200, 400, 2048), (37, 336, 1536), (512, 1280, 5120)])
+def test_gemm_split_k_with_a_workspace_for_partial_planes(dev, fmt, m, n, k):
+    """Few tiles and a workspace that holds fp32 partial planes: the K-steps of a tile are dealt over several workgroups and a
+    second launch sums the planes (2 to 8 ranges here, with a short last range at k = 1536: 24 K-steps over 3 ranges of 8,
+    and at k = 2048 behind the rotated copy of un-rotated rows).  Same bar as the one-launch form; the 8-bit containers
+    keep the one launch."""
+    big = 64 << 20
+    st, out, ref = run_gemm(dev, fmt, m, n, k, xdtype="f16", ydtype="f32", seed=9, workspace_bytes=big)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= 2e-5
+    st, out1, _ = run_gemm(dev, fmt, m, n, k, xdtype="f16", ydtype="f32", seed=9, workspace=False)
+    assert qo.normalized_error(out, out1) <= 2e-6          # the ranges only change the order of the fp32 sums
+    st, out, ref = run_gemm(dev, fmt, m, n, k, xdtype="bf16", ydtype="bf16", seed=10, workspace_bytes=big)
+    assert st == qwhip.OK
+    assert qo.normalized_error(out, ref) <= TOL
+    st, out, ref = run_gemm(dev, fmt, m, n, k, xdtype="f16", ydtype="f16", prerot=False, seed=11, workspace_bytes=big)
     assert st == qwhip.OK
     assert qo.normalized_error(out, ref) <= TOL
 
