@@ -499,7 +499,8 @@ def run_gemm(args, fmt, n, k, m, label, traffic=None):
     x32 = H.make_x(m, k, 100)
     xbits = qo.f32_to_bf16_bits(x32)
     bank, xb, yb = dev.put(blocks), dev.put(xbits), dev.alloc(m * n * 2)
-    ws = dev.alloc(m * k * 2)                      # f16 copy of the bf16 activations (one conversion pass per launch, timed)
+    # f16 copy of the bf16 activations (only the kernels that do not convert in place use it), plus what --gemm-ws-mb asks for
+    ws = dev.alloc(max(m * k * 2, getattr(args, "gemm_ws_mb", 0) << 20))
     view = H.view_of(dev, bank, fmt, n, k)
     flags = qwhip.X_PREROTATED | (args.cfg << 8)
     lib, st = dev.lib, dev.stream.handle
@@ -794,6 +795,9 @@ def main() -> None:
     ap.add_argument("--variant", type=int, default=0, help="gemv kernel override (0 auto; 1..7 as the flags of qwhip_gemv)")
     ap.add_argument("--rt", type=int, default=0, help="row tiles per wave for the mfma gemv (0 auto)")
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
+    ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 workload when run by itself (0 = the benchmark's 4096)")
+    ap.add_argument("--gemm-ws-mb", type=int, default=0,
+                    help="workspace handed to qwhip_gemm in MiB (0 = the activation copy only; more lets small row counts split K)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
     ap.add_argument("--format", default=None,
                     help="container override for the gemv / gemm / pair workloads, e.g. hq3_g32, aq6_g128 (the workload's shape is kept)")
@@ -844,6 +848,9 @@ def main() -> None:
     elif kind == "pair":
         out = run_silu_pair(args, fmt, n, k, m, label)
     elif kind == "gemm":
+        if args.gemm_rows:
+            m, traffic = args.gemm_rows, None
+            label += f" [rows {m}, workspace {max(m * k * 2, args.gemm_ws_mb << 20) >> 20} MiB]"
         out = run_gemm(args, fmt, n, k, m, label, traffic)
     else:
         out = run_gemv(args, fmt, n, k, m, label + (f" M={m}" if args.workload.startswith("c5") else ""), outliers, traffic)
