@@ -1494,9 +1494,23 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     p.ldy = ldy;
     p.y = y;
     p.force_gemm2 = ov == 14u ? 1u : 0u;
+    // Split-K: a problem of few tiles is one tile's K loop long (80 K-steps of ~1.1 us on K = 5120, whatever M).  When the
+    // workspace also holds fp32 partial planes (after the activation copy, if there is one), the K-steps of a tile are dealt
+    // over 2..8 workgroups and a second launch sums the planes in range order.
+    uint32_t splits = 0;
+    const bool copy_needed = rotate || (x_dtype == QWHIP_BF16 && (flags & (1u << 16)));   // bf16 rows in the basis are read in place
+    const uint64_t sk_used = copy_needed ? ((ws_need + 255u) & ~(uint64_t)255u) : 0u;
+    if (ov == 0u && pp_ok && workspace && ((uintptr_t)workspace & 15u) == 0 && w->n % 4u == 0 && (!copy_needed || ws_ok)) {
+        const uint32_t tiles = qwhip_cdiv(m, kCfgBM[CFG_128x320]) * qwhip_cdiv(w->n, kCfgBN[CFG_128x320]);
+        const uint32_t nk = w->k / 64u;
+        const uint64_t plane = (uint64_t)m * w->n * 4u;
+        splits = min(min(8u, 256u / tiles), nk / 8u);
+        while (splits >= 2u && ((uint64_t)(splits - 1u) * qwhip_cdiv(nk, splits) >= nk || sk_used + splits * plane > workspace_bytes)) --splits;
+        if (splits < 2u) splits = 0;
+    }
     // bf16 activations already in the basis: the ping-pong kernel converts them while it stages the tile (no pass of its own,
     // no workspace); flags bit 16 keeps the separate pass, for tests and comparisons
-    const bool direct_bf16 = !rotate && x_dtype == QWHIP_BF16 && ov != 15u && !(flags & (1u << 16)) && gemm3_takes(p, cfg, fmt, y_dtype);
+    const bool direct_bf16 = !rotate && x_dtype == QWHIP_BF16 && ov != 15u && !(flags & (1u << 16)) && (splits != 0u || gemm3_takes(p, cfg, fmt, y_dtype));
     if (direct_bf16) {
         p.x_bf16 = 1u;
         xdt = QWHIP_F16;   // dispatch as the f16 kernels do; the kernel itself reads bf16
@@ -1528,22 +1542,11 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     p.bb = qwhip_view_block_bytes(w);
     p.row_bytes = qwhip_view_row_bytes(w);
     hipError_t e;
-    // Split-K: a problem of few tiles is one tile's K loop long (80 K-steps of ~1.1 us on K = 5120, whatever M).  When the
-    // workspace also holds fp32 partial planes (after the activation copy, if there is one), the K-steps of a tile are dealt
-    // over 2..8 workgroups and a second launch sums the planes in range order.
-    if (ov == 0u && pp_ok && xdt == QWHIP_F16 && workspace && ((uintptr_t)workspace & 15u) == 0 && w->n % 4u == 0) {
-        const uint32_t tiles = qwhip_cdiv(m, kCfgBM[CFG_128x320]) * qwhip_cdiv(w->n, kCfgBN[CFG_128x320]);
-        const uint32_t nk = w->k / 64u;
-        const uint64_t used = xin == workspace ? ((ws_need + 255u) & ~(uint64_t)255u) : 0u;
-        const uint64_t plane = (uint64_t)m * w->n * 4u;
-        uint32_t splits = min(min(8u, 256u / tiles), nk / 8u);
-        while (splits >= 2u && ((uint64_t)(splits - 1u) * qwhip_cdiv(nk, splits) >= nk || used + splits * plane > workspace_bytes)) --splits;
-        if (splits >= 2u) {
-            float* part = (float*)((uint8_t*)workspace + used);
-            QG_FOR_FMT(fmt, e, (launch_splitk<F>(s->stream, p, splits, part, y, y_dtype, ldy)))
-            QWHIP_TRY_HIP(e);
-            return QWHIP_OK;
-        }
+    if (splits != 0u && xdt == QWHIP_F16) {
+        float* part = (float*)((uint8_t*)workspace + sk_used);
+        QG_FOR_FMT(fmt, e, (launch_splitk<F>(s->stream, p, splits, part, y, y_dtype, ldy)))
+        QWHIP_TRY_HIP(e);
+        return QWHIP_OK;
     }
     if (xdt != QWHIP_F16 || ov == 15u) {
         if (xdt == QWHIP_F16) {
