@@ -1319,7 +1319,7 @@ static const uint32_t kCfgBN[CFG_COUNT] = {320, 256, 128, 128, 320};
 // the ping-pong kernel takes the 256 x 320 tile at any row count, every container but the 8-bit ones, and 2-byte outputs
 // whose rows are 16-byte aligned
 inline bool gemm3_takes(const qw_gemm_params& p, int cfg, int fmt, uint32_t ydt) {
-    return (cfg == CFG_256x320 || cfg == CFG_128x320) && fmt != QG_FMT_B8 && !p.force_gemm2 &&
+    return ((cfg == CFG_256x320 && fmt != QG_FMT_B8) || cfg == CFG_128x320) && !p.force_gemm2 &&
            (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0));
 }
 
@@ -1331,9 +1331,9 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     const dim3 grid(((total + 7u) / 8u) * 8u);
     switch (cfg) {
         case CFG_256x320:
-            // the 8-bit containers stay on the DMA-fed kernel: their wider weight items do not fit the ping-pong kernel's
-            // register budget at this tile (the 6-bit streams spill three to five registers there and still run a sixth
-            // faster than on the DMA-fed kernel)
+            // the 8-bit containers stay on the DMA-fed kernel at this tile: their wider weight items do not fit the ping-pong
+            // kernel's register budget here (they do on the half-height tile; the 6-bit streams spill three to five registers
+            // here and still run a sixth faster than on the DMA-fed kernel)
             if constexpr (FMT != QG_FMT_B8) {
                 if (gemm3_takes(p, cfg, FMT, YDT)) {
                     if (p.x_bf16) return launch_cfg3<2, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
@@ -1342,11 +1342,9 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
             }
             return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_128x320:
-            if constexpr (FMT != QG_FMT_B8) {
-                if (gemm3_takes(p, cfg, FMT, YDT)) {
-                    if (p.x_bf16) return launch_cfg3<1, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
-                    return launch_cfg3<1, 5, 4, 2, FMT, YDT>(st, p, grid);
-                }
+            if (gemm3_takes(p, cfg, FMT, YDT)) {
+                if (p.x_bf16) return launch_cfg3<1, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
+                return launch_cfg3<1, 5, 4, 2, FMT, YDT>(st, p, grid);
             }
             return launch_cfg2<1, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_256x256: return launch_cfg2<2, 4, 4, 2, FMT, YDT, false>(st, p, grid);
@@ -1375,27 +1373,32 @@ hipError_t launch_dense1_y(hipStream_t st, qw_gemm_params& p, uint32_t ydt) {
 }
 
 // waste-aware choice among the tile shapes: time ~ rounds of tiles over the CUs x per-tile cost / shape efficiency.
-// `pingpong`: the 256 x 320 and 128 x 320 shapes run the ping-pong kernel (every container but the 8-bit ones), which is 1.4x
-// the DMA-fed kernel on the same tile (188 against 264 us on M = 4096, N = K = 5120); `only_pingpong` keeps the choice to
-// those two shapes (bf16 activations with no workspace to convert into: the other kernels would fall to the unpipelined one).
-int choose_cfg(uint32_t M, uint32_t N, bool pingpong, bool only_pingpong) {
-    // relative matrix-core efficiency of each shape on the DMA-fed kernel (measured on M = 4096, N = K = 5120; the half-height
-    // tile from M = 2048: 256 tiles in 115 us where the 128 tiles of 256 x 320 take 144) and workgroups resident per CU
-    const double eff2[CFG_COUNT] = {1.00, 0.82, 0.78, 0.75, 0.82};
+// `pingpong`: the ping-pong kernel is available (2-byte outputs need 16-byte aligned rows): it runs the 256 x 320 and
+// 128 x 320 shapes for every container but the 8-bit ones, whose weight items fit its registers on the half-height tile
+// only.  `only_pingpong` keeps the choice to the shapes it runs (bf16 activations with no workspace to convert into: the
+// other kernels would fall to the unpipelined one).
+int choose_cfg(uint32_t M, uint32_t N, bool eight_bit, bool pingpong, bool only_pingpong) {
+    // efficiency of each shape per tile area, on the scale ping-pong 256 x 320 on a 4-bit container = 1 (188 us a round
+    // on M = 4096, N = K = 5120).  DMA-fed kernel: 264 us on that tile (0.71), the smaller shapes 0.82 / 0.78 / 0.75 of that;
+    // half-height ping-pong tile: 115 us for 256 tiles (0.82); 8-bit containers: 237 us a round on the DMA-fed 256 x 320
+    // (0.79), 132 us on the half-height ping-pong tile (0.71)
+    static const double kEffPp[CFG_COUNT] = {1.00, 0.58, 0.55, 0.53, 0.82};
+    static const double kEffPp8[CFG_COUNT] = {0.79, 0.65, 0.62, 0.59, 0.71};
+    static const double kEffDma[CFG_COUNT] = {0.71, 0.58, 0.55, 0.53, 0.58};
+    const double* eff = !pingpong ? kEffDma : (eight_bit ? kEffPp8 : kEffPp);
     const double resident[CFG_COUNT] = {1, 1, 2, 1, 1};
     // a problem of few tiles is one tile's K loop long whatever the shape, and the small tile's loop is the shortest
     // (N = K = 5120, f16: M = 64 in 65 us on 128 x 128 against 82 us on the half-height ping-pong tile, M = 256 82 against 85)
     if ((uint64_t)qwhip_cdiv(M, 128u) * qwhip_cdiv(N, 128u) <= 128u) return CFG_128x128;
     double best = 1e300;
-    int best_cfg = only_pingpong ? CFG_256x320 : CFG_128x128;
+    int best_cfg = only_pingpong ? CFG_128x320 : CFG_128x128;
     for (int c = 0; c < CFG_COUNT; ++c) {
-        const bool pp = c == CFG_256x320 || c == CFG_128x320;
+        const bool pp = pingpong && (c == CFG_128x320 || (c == CFG_256x320 && !eight_bit));
         if (only_pingpong && !pp) continue;
-        const double eff = eff2[c] * ((pingpong && !pp) ? 0.71 : 1.0);
         const double tiles = (double)qwhip_cdiv(M, kCfgBM[c]) * qwhip_cdiv(N, kCfgBN[c]);
         const double slots = 256.0 * resident[c];
         const double rounds = (double)(uint64_t)((tiles + slots - 1.0) / slots);
-        const double cost = rounds * resident[c] * kCfgBM[c] * kCfgBN[c] / eff;
+        const double cost = rounds * resident[c] * kCfgBM[c] * kCfgBN[c] / eff[c];
         if (cost < best) {
             best = cost;
             best_cfg = c;
@@ -1431,9 +1434,7 @@ qwhip_status gemm_checks(qwhip_stream_t s, const qwhip_weight_view* w, const voi
 // split-K launch of the half-height ping-pong tile into fp32 planes at `part`, then the sum into y
 template <int FMT>
 hipError_t launch_splitk(hipStream_t st, const qw_gemm_params& p, uint32_t splits, float* part, void* y, uint32_t y_dtype, uint32_t ldy) {
-    if constexpr (FMT == QG_FMT_B8) {
-        return hipErrorInvalidValue;   // the 8-bit containers do not run the ping-pong kernel
-    } else {
+    {
         qw_gemm_params q = p;
         q.y = part;
         q.ldy = p.N;
@@ -1486,9 +1487,10 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     uint32_t xdt = x_dtype;
     const uint32_t ov = (flags >> 8) & 0xFu;
     // 2-byte outputs reach the ping-pong kernel with 16-byte aligned rows only (gemm3_takes)
-    const bool pp_ok = fmt != QG_FMT_B8 && (y_dtype == QWHIP_F32 || (ldy % 8u == 0 && ((uintptr_t)y & 15u) == 0));
+    const bool pp_ok = y_dtype == QWHIP_F32 || (ldy % 8u == 0 && ((uintptr_t)y & 15u) == 0);
     const bool bf16_in_place = pp_ok && !rotate && x_dtype == QWHIP_BF16 && !ws_ok && !(flags & (1u << 16));
-    const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n, pp_ok, bf16_in_place));
+    const int cfg = (ov >= 1 && ov <= CFG_COUNT) ? (int)ov - 1
+                                                 : (ov == 14u ? (int)CFG_256x320 : choose_cfg(m, w->n, fmt == QG_FMT_B8, pp_ok, bf16_in_place));
     qw_gemm_params p = {};
     p.M = m;
     p.ldy = ldy;

@@ -138,8 +138,7 @@ def test_gemm_ragged_rows_at_the_prefill_shape(dev):
 def test_gemm_split_k_with_a_workspace_for_partial_planes(dev, fmt, m, n, k):
     """Few tiles and a workspace that holds fp32 partial planes: the K-steps of a tile are dealt over several workgroups and a
     second launch sums the planes (2 to 8 ranges here, with a short last range at k = 1536: 24 K-steps over 3 ranges of 8,
-    and at k = 2048 behind the rotated copy of un-rotated rows).  Same bar as the one-launch form; the 8-bit containers
-    keep the one launch."""
+    and at k = 2048 behind the rotated copy of un-rotated rows).  Same bar as the one-launch form."""
     big = 64 << 20
     st, out, ref = run_gemm(dev, fmt, m, n, k, xdtype="f16", ydtype="f32", seed=9, workspace_bytes=big)
     assert st == qwhip.OK
