@@ -468,11 +468,11 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     constexpr uint32_t A_BLK = NT / 8;
     const uint32_t a_lds0 = (tid >> 3) * 128u + (((tid & 7u) ^ ((tid >> 4) & 7u)) << 4);   // + i * A_BLK * 128 (swizzle key unchanged)
     const uint64_t a_tile_base = (uint64_t)m0 * p.ldx * 2u;
-    uint64_t a_off[A_LD];
+    uint32_t a_off[A_LD];   // inside the tile: under 4 GiB (the launcher checks 256 * ldx * 2)
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) {
         const uint32_t r = (tid >> 3) + (uint32_t)i * A_BLK;
-        a_off[i] = (r < rows_valid ? (uint64_t)r * p.ldx * 2u : 0ull) + (tid & 7u) * 16u;
+        a_off[i] = (r < rows_valid ? r * p.ldx * 2u : 0u) + (tid & 7u) * 16u;
     }
 
     // ---- weight tile: item = (tile row, 32-column slice); thread items tid and NT + (tid % (B_ITEMS - NT)) (items past
@@ -494,6 +494,9 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
         b_off32[i] = n * (uint32_t)p.row_bytes;                     // a tile's rows span < 4 GiB
         b_meta[i] = (nl * 128u) | (((nl >> 1) & 7u) << 16) | ((it & 1u) << 20);
     }
+    uint32_t b_voff[B_PER];   // HQ4_G32_M5: row offset + the slice's block inside a K-step
+#pragma unroll
+    for (int i = 0; i < B_PER; ++i) b_voff[i] = b_off32[i] + (b_meta[i] >> 20) * 20u;
 
     f16_t acc[WM][WN];
 #pragma unroll
@@ -511,9 +514,12 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     const uint32_t nk = min(nk_per, nk_all - kt0);
 
     auto load_a = [&](uint32_t kt, u4_t* a_reg) {
+        const uint8_t* xk = (const uint8_t*)p.x + a_tile_base + (uint64_t)(kt0 + kt) * 128u;   // wave-uniform: scalar base + 32-bit lane offset
 #pragma unroll
-        for (int i = 0; i < A_LD; ++i)
-            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + a_tile_base + a_off[i] + (uint64_t)(kt0 + kt) * 128u);
+        for (int i = 0; i < A_LD; ++i) {
+            asm volatile("" : "+v"(a_off[i]));   // keeps the lane offset a 32-bit register: scalar base + 32-bit offset addressing
+            a_reg[i] = *(const u4_t*)(xk + a_off[i]);
+        }
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
@@ -521,7 +527,15 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     };
     auto load_b = [&](uint32_t kt, qg_slice<FMT>* b_reg, int nitems) {
 #pragma unroll
-        for (int i = 0; i < B_PER; ++i) if (i < nitems) qg_load_slice<FMT>(b_tile + b_off32[i], (kt0 + kt) * 2u + (b_meta[i] >> 20), p.gshift, p.bb, b_reg[i]);
+        for (int i = 0; i < B_PER; ++i) {
+            if (i >= nitems) continue;
+            if constexpr (FMT == QG_FMT_M5) {   // 20-byte blocks: the K-step moves a wave-uniform base, the lane offset is fixed
+                asm volatile("" : "+v"(b_voff[i]));
+                qg_load_slice<FMT>(b_tile + (uint64_t)(kt0 + kt) * 40u + b_voff[i], 0u, p.gshift, p.bb, b_reg[i]);
+            } else {
+                qg_load_slice<FMT>(b_tile + b_off32[i], (kt0 + kt) * 2u + (b_meta[i] >> 20), p.gshift, p.bb, b_reg[i]);
+            }
+        }
     };
     // When the second items number a quarter of the workgroup, each is shared by the two group-0 threads tid and
     // tid + NT / 4: one dequantizes its chunks 0..1, the other 2..3 (half the second pass instead of doing it twice).
@@ -1477,7 +1491,7 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     if (w->n % 16 != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "tensor GEMM needs n %% 16 == 0, got n=%u", w->n);
     if (ldx == 0) ldx = w->k;
     if (ldy == 0) ldy = w->n;
-    if (ldx < w->k || ldy < w->n || (ldx % 8) != 0)
+    if (ldx < w->k || ldy < w->n || (ldx % 8) != 0 || ldx >= (1u << 22))   // a tile's 256 activation rows stay under 4 GiB
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions ldx=%u ldy=%u for k=%u n=%u", ldx, ldy, w->k, w->n);
 
     const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
@@ -1630,7 +1644,7 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     }
     if (ldx == 0) ldx = w->k;
     if (ldact == 0) ldact = inter;
-    if (ldx < w->k || ldact < inter || (ldx % 8) != 0 || (ldact % 8) != 0 || ((uintptr_t)act_f16 & 15u) != 0)
+    if (ldx < w->k || ldact < inter || (ldx % 8) != 0 || ldx >= (1u << 22) || (ldact % 8) != 0 || ((uintptr_t)act_f16 & 15u) != 0)
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions or alignment (ldx=%u ldact=%u, act 16-byte aligned)", ldx, ldact);
     if ((uint64_t)w->n * qwhip_view_row_bytes(w) >= (1ull << 32))
         return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "the fused gate_up GEMM addresses the bank with 32-bit offsets (bank under 4 GiB)");
