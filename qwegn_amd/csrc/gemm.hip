@@ -883,7 +883,10 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 
     auto load_a = [&](uint32_t kt, u4_t* a_reg) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
+        for (int i = 0; i < 2; ++i) {
+            asm volatile("" : "+v"(a_voff[i]));   // scalar base + 32-bit lane offset addressing (see qw_gemm3_kernel)
+            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
+        }
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
@@ -1087,7 +1090,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 
     auto load_a = [&](uint32_t kt, u4_t* a_reg) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
+        for (int i = 0; i < 2; ++i) {
+            asm volatile("" : "+v"(a_voff[i]));   // scalar base + 32-bit lane offset addressing (see qw_gemm3_kernel)
+            a_reg[i] = *(const u4_t*)((const uint8_t*)p.x + (uint64_t)kt * 128u + a_voff[i]);
+        }
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
@@ -1095,7 +1101,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     };
     auto load_raw = [&](uint32_t kp, u4_t* raw) {
 #pragma unroll
-        for (int i = 0; i < 5; ++i) raw[i] = *(const u4_t*)(bank + raw_goff[i] + (uint64_t)kp * 80u);
+        for (int i = 0; i < 5; ++i) {
+            asm volatile("" : "+v"(raw_goff[i]));
+            raw[i] = *(const u4_t*)(bank + (uint64_t)kp * 80u + raw_goff[i]);
+        }
     };
     auto store_raw = [&](const u4_t* raw) {
 #pragma unroll
