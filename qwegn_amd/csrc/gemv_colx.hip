@@ -174,17 +174,18 @@ static __device__ __forceinline__ void run(const qcx_params& p) {
     // 2. first weight rows
     qcx_slice<FMT> buf[D];
     auto issue = [&](int slot) {
-        const uint8_t* rp = p.bank + off;
-        buf[slot].hdr = *(const uint32_t*)(rp + hdr_off);
+        // one 32-bit sum per address (the bank is under 4 GiB): scalar base + 32-bit lane offset addressing
+        const uint32_t o_hdr = (uint32_t)off + hdr_off, o_pay = (uint32_t)off + pay_off;
+        buf[slot].hdr = *(const uint32_t*)(p.bank + o_hdr);
         if constexpr (FMT == QW_FMT_B2 || FMT == QW_FMT_B3 || FMT == QW_FMT_B6) {
 #pragma unroll
-            for (int j = 0; j < qcx_fmt<FMT>::PW; ++j) buf[slot].q[j] = *(const uint32_t*)(rp + pay_off + 4 * j);
+            for (int j = 0; j < qcx_fmt<FMT>::PW; ++j) buf[slot].q[j] = *(const uint32_t*)(p.bank + o_pay + 4 * j);
         } else if constexpr (FMT == QW_FMT_B8) {
-            const qcx_words8 w = *(const qcx_words8*)(rp + pay_off);
+            const qcx_words8 w = *(const qcx_words8*)(p.bank + o_pay);
 #pragma unroll
             for (int j = 0; j < 8; ++j) buf[slot].q[j] = w.q[j];
         } else {
-            const qcx_words4 w = *(const qcx_words4*)(rp + pay_off);
+            const qcx_words4 w = *(const qcx_words4*)(p.bank + o_pay);
 #pragma unroll
             for (int j = 0; j < 4; ++j) buf[slot].q[j] = w.q[j];
         }

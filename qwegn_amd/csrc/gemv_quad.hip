@@ -89,14 +89,15 @@ static __device__ __forceinline__ void run(const qq_params& p) {
     slice_of(0, i_hdr, i_pay);
     qq_slice<FMT> buf[D];
     auto issue = [&](int slot) {
-        const uint8_t* rp = p.bank + i_off;
-        buf[slot].hdr = *(const uint32_t*)(rp + i_hdr);
+        // one 32-bit sum per address (the bank is under 4 GiB): scalar base + 32-bit lane offset addressing
+        const uint32_t o_hdr = i_off + i_hdr, o_pay = i_off + i_pay;
+        buf[slot].hdr = *(const uint32_t*)(p.bank + o_hdr);
         if constexpr (FMT == QW_FMT_B8) {
-            const qq_words8 w = *(const qq_words8*)(rp + i_pay);
+            const qq_words8 w = *(const qq_words8*)(p.bank + o_pay);
 #pragma unroll
             for (int c = 0; c < 8; ++c) buf[slot].q[c] = w.q[c];
         } else {
-            const qq_words4 w = *(const qq_words4*)(rp + i_pay);
+            const qq_words4 w = *(const qq_words4*)(p.bank + o_pay);
 #pragma unroll
             for (int c = 0; c < 4; ++c) buf[slot].q[c] = w.q[c];
         }
