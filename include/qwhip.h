@@ -355,11 +355,9 @@ qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_weight_view* w
  * (qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167; door
  * Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:156-190).  w: [2 * inter, k], rows [gate | up]; act f16 [m, inter]
  * = f16(FWHT32(silu(g) * u)) with g, u rounded to f16 first - bit-identical to qwhip_gemm (f16 out) followed by
- * qwhip_swiglu_fwht, without the [m, 2 inter] matrix.  One launch: 2-, 3- and 4-bit containers, any m, inter % 32 == 0, act
+ * qwhip_swiglu_fwht, without the [m, 2 inter] matrix.  One launch for every container and any m; inter % 32 == 0, act
  * 16-byte aligned with ldact % 8 == 0 (0 = inter); x, flags and workspace as qwhip_gemm (bf16 or un-rotated activations
- * need the workspace).  The 6- and 8-bit containers run the two calls inside the door when the workspace holds the
- * [m, 2 inter] f16 matrix (m * n * 2 bytes, plus m * k * 2 for bf16 or un-rotated activations) and act rows are packed;
- * without it they return QWHIP_E_BAD_GEOMETRY. */
+ * need the workspace: m * k * 2 bytes). */
 qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                uint32_t ldx, uint32_t rotate_act, void* act_f16, uint32_t ldact, uint32_t flags,
                                void* workspace, size_t workspace_bytes);

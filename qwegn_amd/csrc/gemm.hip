@@ -1339,10 +1339,10 @@ enum { CFG_256x320 = 0, CFG_256x256 = 1, CFG_128x128 = 2, CFG_256x128 = 3, CFG_1
 static const uint32_t kCfgBM[CFG_COUNT] = {256, 256, 128, 256, 128};
 static const uint32_t kCfgBN[CFG_COUNT] = {320, 256, 128, 128, 320};
 
-// the ping-pong kernel takes the 256 x 320 tile at any row count, every container but the 8-bit ones, and 2-byte outputs
-// whose rows are 16-byte aligned
+// the ping-pong kernel takes the 256 x 320 and 128 x 320 tiles at any row count, every container, and 2-byte outputs whose
+// rows are 16-byte aligned
 inline bool gemm3_takes(const qw_gemm_params& p, int cfg, int fmt, uint32_t ydt) {
-    return ((cfg == CFG_256x320 && fmt != QG_FMT_B8) || cfg == CFG_128x320) && !p.force_gemm2 &&
+    return (cfg == CFG_256x320 || cfg == CFG_128x320) && !p.force_gemm2 &&
            (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0));
 }
 
@@ -1354,14 +1354,11 @@ hipError_t launch_dense2(hipStream_t st, qw_gemm_params& p, int cfg) {
     const dim3 grid(((total + 7u) / 8u) * 8u);
     switch (cfg) {
         case CFG_256x320:
-            // the 8-bit containers stay on the DMA-fed kernel at this tile: their wider weight items do not fit the ping-pong
-            // kernel's register budget here (they do on the half-height tile; the 6-bit streams spill three to five registers
-            // here and still run a sixth faster than on the DMA-fed kernel)
-            if constexpr (FMT != QG_FMT_B8) {
-                if (gemm3_takes(p, cfg, FMT, YDT)) {
-                    if (p.x_bf16) return launch_cfg3<2, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
-                    return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
-                }
+            // (the 6- and 8-bit containers spill three to five registers on this tile and still run a sixth faster than on the
+            // DMA-fed kernel)
+            if (gemm3_takes(p, cfg, FMT, YDT)) {
+                if (p.x_bf16) return launch_cfg3<2, 5, 4, 2, FMT, YDT, false, QWHIP_BF16>(st, p, grid);
+                return launch_cfg3<2, 5, 4, 2, FMT, YDT>(st, p, grid);
             }
             return launch_cfg2<2, 5, 4, 2, FMT, YDT, false>(st, p, grid);
         case CFG_128x320:
@@ -1396,17 +1393,16 @@ hipError_t launch_dense1_y(hipStream_t st, qw_gemm_params& p, uint32_t ydt) {
 }
 
 // waste-aware choice among the tile shapes: time ~ rounds of tiles over the CUs x per-tile cost / shape efficiency.
-// `pingpong`: the ping-pong kernel is available (2-byte outputs need 16-byte aligned rows): it runs the 256 x 320 and
-// 128 x 320 shapes for every container but the 8-bit ones, whose weight items fit its registers on the half-height tile
-// only.  `only_pingpong` keeps the choice to the shapes it runs (bf16 activations with no workspace to convert into: the
-// other kernels would fall to the unpipelined one).
+// `pingpong`: the ping-pong kernel is available (2-byte outputs need 16-byte aligned rows) for the 256 x 320 and 128 x 320
+// shapes.  `only_pingpong` keeps the choice to those two (bf16 activations with no workspace to convert into: the other
+// kernels would fall to the unpipelined one).
 int choose_cfg(uint32_t M, uint32_t N, bool eight_bit, bool pingpong, bool only_pingpong) {
     // efficiency of each shape per tile area, on the scale ping-pong 256 x 320 on a 4-bit container = 1 (188 us a round
     // on M = 4096, N = K = 5120).  DMA-fed kernel: 264 us on that tile (0.71), the smaller shapes 0.82 / 0.78 / 0.75 of that;
-    // half-height ping-pong tile: 115 us for 256 tiles (0.82); 8-bit containers: 237 us a round on the DMA-fed 256 x 320
-    // (0.79), 132 us on the half-height ping-pong tile (0.71)
+    // half-height ping-pong tile: 115 us for 256 tiles (0.82); 8-bit containers: 206 us a round on the ping-pong 256 x 320
+    // (0.91; 237 - 242 us on the DMA-fed kernel), 132 us on the half-height tile (0.71)
     static const double kEffPp[CFG_COUNT] = {1.00, 0.58, 0.55, 0.53, 0.82};
-    static const double kEffPp8[CFG_COUNT] = {0.79, 0.65, 0.62, 0.59, 0.71};
+    static const double kEffPp8[CFG_COUNT] = {0.91, 0.65, 0.62, 0.59, 0.71};
     static const double kEffDma[CFG_COUNT] = {0.71, 0.58, 0.55, 0.53, 0.58};
     const double* eff = !pingpong ? kEffDma : (eight_bit ? kEffPp8 : kEffPp);
     const double resident[CFG_COUNT] = {1, 1, 2, 1, 1};
@@ -1416,7 +1412,7 @@ int choose_cfg(uint32_t M, uint32_t N, bool eight_bit, bool pingpong, bool only_
     double best = 1e300;
     int best_cfg = only_pingpong ? CFG_128x320 : CFG_128x128;
     for (int c = 0; c < CFG_COUNT; ++c) {
-        const bool pp = pingpong && (c == CFG_128x320 || (c == CFG_256x320 && !eight_bit));
+        const bool pp = pingpong && (c == CFG_128x320 || c == CFG_256x320);
         if (only_pingpong && !pp) continue;
         const double tiles = (double)qwhip_cdiv(M, kCfgBM[c]) * qwhip_cdiv(N, kCfgBN[c]);
         const double slots = 256.0 * resident[c];
@@ -1627,8 +1623,7 @@ extern "C" qwhip_status qwhip_gemm_noalloc(qwhip_stream_t s, const qwhip_weight_
 }
 
 // Dense gate|up GEMM with the SwiGLU (+ FWHT-32) epilogue fused: act f16 [m, inter], inter = n / 2, the bank's rows being
-// [gate | up].  Runs the ping-pong kernel's fused form; shapes it does not take are refused (the caller then runs
-// qwhip_gemm into a [m, 2 inter] buffer and qwhip_swiglu_fwht).
+// [gate | up].  Runs the ping-pong kernel's fused form: every container, any row count, one launch.
 extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                           uint32_t ldx, uint32_t rotate_act, void* act_f16, uint32_t ldact, uint32_t flags,
                                           void* workspace, size_t workspace_bytes) {
@@ -1638,19 +1633,6 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     if (m == 0) return QWHIP_OK;
     const uint32_t inter = w->n / 2u;
     if (w->n % 64u != 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "fused gate_up needs an intermediate size %% 32 == 0, got %u rows", w->n);
-    if (fmt == QG_FMT_B8 || fmt == QG_FMT_B6) {   // the 6- and 8-bit weight items do not fit the fused kernel's registers
-        // these containers: the two launches inside the door, through the caller's workspace
-        // ([m, 2 inter] f16 first, the rest for qwhip_gemm's own copy of the activations); same bits as the two doors
-        const uint64_t gu_bytes = (uint64_t)m * w->n * 2u;
-        if (!workspace || ((uintptr_t)workspace & 15u) || workspace_bytes < gu_bytes || (ldact != 0 && ldact != inter) || ((uintptr_t)act_f16 & 15u))
-            return qwhip_fail(QWHIP_E_BAD_GEOMETRY,
-                              "the fused gate_up GEMM takes 2-, 3- and 4-bit containers in one launch (m=%u); the 6- and 8-bit ones need a 16-byte "
-                              "aligned workspace of m * n * 2 bytes (plus m * k * 2 for bf16 or un-rotated activations) and packed act rows", m);
-        const uint64_t rest = workspace_bytes - gu_bytes;
-        st = qwhip_gemm(s, w, x, x_dtype, m, ldx, workspace, QWHIP_F16, 0, flags & QWHIP_X_PREROTATED, rest ? (uint8_t*)workspace + gu_bytes : nullptr, rest);
-        if (st != QWHIP_OK) return st;
-        return qwhip_swiglu_fwht(s, workspace, QWHIP_F16, act_f16, m, inter, rotate_act ? 1u : 0u);
-    }
     if (ldx == 0) ldx = w->k;
     if (ldact == 0) ldact = inter;
     if (ldx < w->k || ldact < inter || (ldx % 8) != 0 || ldx >= (1u << 22) || (ldact % 8) != 0 || ((uintptr_t)act_f16 & 15u) != 0)
@@ -1699,7 +1681,7 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
 #define QG_SWIGLU3(F) \
     case F: e = ga ? launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true, QWHIP_F16, true>(s->stream, p, grid) \
                    : launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true>(s->stream, p, grid); break;
-        QG_SWIGLU3(QG_FMT_M5) QG_SWIGLU3(QG_FMT_B4) QG_SWIGLU3(QG_FMT_B2) QG_SWIGLU3(QG_FMT_B3)
+        QG_SWIGLU3(QG_FMT_M5) QG_SWIGLU3(QG_FMT_B4) QG_SWIGLU3(QG_FMT_B2) QG_SWIGLU3(QG_FMT_B3) QG_SWIGLU3(QG_FMT_B6) QG_SWIGLU3(QG_FMT_B8)
 #undef QG_SWIGLU3
         default: e = hipErrorInvalidValue;
     }

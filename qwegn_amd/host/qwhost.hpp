@@ -402,7 +402,7 @@ struct QWGemm {
         if (act16.shape.dtype != QWDType::f16 || act16.shape.elementCount < (size_t)rows * (size_t)(w.n / 2) ||
             x.shape.elementCount < (size_t)rows * (size_t)w.k)
             throw QWGemmError(QWGemmError::badWeights, "fused gate_up: x [rows, k], act f16 [rows, n / 2]");
-        if (w.bits() > 4 || w.n % 64 != 0 || w.k % 64 != 0) return false;
+        if (w.n % 64 != 0 || w.k % 64 != 0) return false;
         hal.pipeline(w.containerKind.isIncumbentContainer() ? "qwg_gemm_q4g_h16_swiglu"
                                                             : ("qwg_gemm_aq" + std::to_string(w.bits()) + "_g" + std::to_string(w.groupSize()) + "_h16_swiglu").c_str());
         const qwhip_weight_view v = w.abi();
