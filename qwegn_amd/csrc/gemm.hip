@@ -497,6 +497,16 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     uint32_t b_voff[B_PER];   // HQ4_G32_M5: row offset + the slice's block inside a K-step
 #pragma unroll
     for (int i = 0; i < B_PER; ++i) b_voff[i] = b_off32[i] + (b_meta[i] >> 20) * 20u;
+    // bit-stream blocks: lane offsets of the item's header word and of its code words; what the K-step adds is wave-uniform
+    // (group 32: two blocks per K-step; larger groups: the K-step's block, and the pair of slices inside it)
+    uint32_t b_vh[B_PER], b_vc[B_PER];
+    constexpr uint32_t W4 = 4u * (uint32_t)qg_slice_words<FMT>();
+#pragma unroll
+    for (int i = 0; i < B_PER; ++i) {
+        const uint32_t sl = b_meta[i] >> 20;
+        b_vh[i] = b_off32[i] + (p.gshift == 0u ? sl * p.bb : 0u);
+        b_vc[i] = b_vh[i] + 4u + (p.gshift == 0u ? 0u : sl * W4);
+    }
 
     f16_t acc[WM][WN];
 #pragma unroll
@@ -533,7 +543,11 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
                 asm volatile("" : "+v"(b_voff[i]));
                 qg_load_slice<FMT>(b_tile + (uint64_t)(kt0 + kt) * 40u + b_voff[i], 0u, p.gshift, p.bb, b_reg[i]);
             } else {
-                qg_load_slice<FMT>(b_tile + b_off32[i], (kt0 + kt) * 2u + (b_meta[i] >> 20), p.gshift, p.bb, b_reg[i]);
+                const uint32_t kk = kt0 + kt;
+                const uint32_t u_h = p.gshift == 0u ? 2u * kk * p.bb : (kk >> (p.gshift - 1u)) * p.bb;
+                const uint32_t u_c = p.gshift == 0u ? u_h : u_h + ((2u * kk) & ((1u << p.gshift) - 1u)) * W4;
+                asm volatile("" : "+v"(b_vh[i]), "+v"(b_vc[i]));
+                qg_load_slice_at<FMT>(b_tile + u_h + b_vh[i], b_tile + u_c + b_vc[i], b_reg[i]);
             }
         }
     };

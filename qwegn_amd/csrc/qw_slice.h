@@ -64,6 +64,37 @@ __device__ __forceinline__ void qg_load_slice(const uint8_t* rowp, uint32_t s, u
     }
 }
 
+// The same slice of a bit-stream block from its two addresses: the block's header word and the slice's code words
+// (callers that keep a wave-uniform base and a fixed 32-bit lane offset for each).
+template <int FMT>
+__device__ __forceinline__ void qg_load_slice_at(const uint8_t* hdr_p, const uint8_t* src, qg_slice<FMT>& o) {
+    static_assert(FMT != QG_FMT_M5, "bit-stream blocks");
+    o.hdr = *(const uint32_t*)hdr_p;
+    if constexpr (FMT == QG_FMT_B4) {
+        const qg_words4 w = *(const qg_words4*)src;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o.q[j] = w.q[j];
+    } else if constexpr (FMT == QG_FMT_B8) {
+        const qg_words8 w = *(const qg_words8*)src;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o.q[j] = w.q[j];
+    } else {
+        constexpr int W = qg_slice_words<FMT>();
+        if constexpr (W == 6) {
+            const qg_words4 w0 = *(const qg_words4*)src;
+            const qg_words_n<2> w1 = *(const qg_words_n<2>*)(src + 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o.q[j] = w0.q[j];
+            o.q[4] = w1.q[0];
+            o.q[5] = w1.q[1];
+        } else {
+            const qg_words_n<W> w = *(const qg_words_n<W>*)src;
+#pragma unroll
+            for (int j = 0; j < W; ++j) o.q[j] = w.q[j];
+        }
+    }
+}
+
 // 8 consecutive columns (chunk j of the slice) in natural order, as exact f16 weights.
 template <int FMT>
 __device__ __forceinline__ h8_t qg_dequant_chunk(const qg_slice<FMT>& sl, int j, h2_t s2, h2_t b2, uint32_t magic) {
