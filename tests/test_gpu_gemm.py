@@ -153,6 +153,34 @@ def test_gemm_split_k_with_a_workspace_for_partial_planes(dev, fmt, m, n, k):
     assert qo.normalized_error(out, ref) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32"])
+@pytest.mark.parametrize("m,ws_mb", [(333, 0), (333, 64), (2100, 0)])
+def test_gemm_strided_rows_on_every_ping_pong_form(dev, fmt, m, ws_mb):
+    """Activation rows ldx > k apart and output rows ldy > n apart (both in elements) through the one-launch forms (256 x 320
+    and 128 x 320 tiles, ragged row counts) and the split-K form: padding columns of the output stay untouched."""
+    n, k, ldx, ldy = 656, 1024, 1024 + 64, 656 + 8
+    blocks, w16 = H.make_bank(fmt, n, k, seed=13)
+    x32 = H.make_x(m, k, 17)
+    xp = np.zeros((m, ldx), np.float16)
+    xp[:, :k] = x32.astype(np.float16)
+    xp[:, k:] = np.float16(777.0)                      # never read
+    bank, xb = dev.put(blocks), dev.put(xp)
+    yb = dev.put(np.full((m, ldy), 0x7FC0, np.uint16))  # bf16 NaN pattern in the padding
+    ws = dev.alloc(ws_mb << 20) if ws_mb else None
+    view = H.view_of(dev, bank, fmt, n, k)
+    st = dev.lib.qwhip_gemm(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, m, ldx, yb.ptr, qwhip.BF16, ldy, qwhip.X_PREROTATED,
+                            ws.ptr if ws else None, ws.nbytes if ws else 0)
+    assert st == qwhip.OK
+    dev.stream.sync()
+    raw = yb.download(np.uint16, (m, ldy))
+    for b in (bank, xb, yb, ws):
+        if b is not None:
+            b.free()
+    assert np.all(raw[:, n:] == 0x7FC0)
+    ref = qo.matmul_ref_f64(xp[:, :k], w16)
+    assert qo.normalized_error(qo.bf16_bits_to_f32(raw[:, :n]), ref) <= TOL
+
+
 def test_gemm_rotation_prepass_with_workspace(dev):
     st, out, ref = run_gemm(dev, "hq4_g32_m5", 130, 256, 512, prerot=False, ydtype="f32")
     assert st == qwhip.OK
