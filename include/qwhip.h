@@ -268,7 +268,7 @@ qwhip_status qwhip_embed_bf16_f32(qwhip_stream_t s, const void* table_bf16, uint
 /* ---- prefill GEMM: Y[m, n] = X[m, k] . W^T on f16 MFMA, fp32 accumulate ------ */
 /* gemmBatchedH16 (Sources/Runtime/QWEngine/Driver/EncodeKernels.swift:119-154) -> qwg_gemm_q4g_h16 /
  * qwg_gemm_aq*_h16; QWGemm.encodeNaxF32 (Sources/Operators/QWGEMM/QWGemmF32.swift:366-402).
- * x: f16 or bf16 [m, ldx]; y: f16, bf16 or f32 [m, ldy]; ldx/ldy in elements (0 = tight).
+ * x: f16 or bf16 [m, ldx]; y: f16, bf16 or f32 [m, ldy]; ldx/ldy in elements (0 = tight; ldx % 8 == 0, ldx < 2^22).
  * Requires k % 64 == 0 and n % 16 == 0 else QWHIP_E_BAD_GEOMETRY (the reference's tensor path
  * requires N, K multiples of 64).  Activations must be in the container's basis
  * (QWHIP_X_PREROTATED) unless `workspace` holds m*k f16 elements for the rotated copy.
