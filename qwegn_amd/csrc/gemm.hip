@@ -1762,6 +1762,8 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_wei
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions ldx=%u ldy=%u", ldx, ldy);
     if ((uint64_t)pairs * ldx * 2u >= (1ull << 32))
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "grouped GEMM addresses its activation rows with 32-bit offsets: %u rows of %u do not fit", pairs, ldx);
+    if ((uint64_t)rows_per_expert * qwhip_view_row_bytes(w) >= (1ull << 32))
+        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "grouped GEMM addresses an expert's rows with 32-bit offsets: %u rows do not fit", rows_per_expert);
     qw_gemm_params p = {};
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
@@ -1815,6 +1817,8 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "bad leading dimensions or alignment (ldx=%u ldact=%u, act 16-byte aligned)", ldx, ldact);
     if ((uint64_t)pairs * ldx * 2u >= (1ull << 32))
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "grouped GEMM addresses its activation rows with 32-bit offsets: %u rows of %u do not fit", pairs, ldx);
+    if ((uint64_t)rows_per_expert * qwhip_view_row_bytes(w) >= (1ull << 32))
+        return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "grouped GEMM addresses an expert's rows with 32-bit offsets: %u rows do not fit", rows_per_expert);
     qw_gemm_params p = {};
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
