@@ -251,6 +251,19 @@ def test_fused_gate_up_swiglu_refusals(dev):
     assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v2), 3, xb.ptr, qwhip.BF16, 0, None, *args) == qwhip.E_BAD_SHAPE     # bf16 activations
 
 
+def test_grouped_gemm_refuses_expert_of_4gib(dev):
+    """One expert whose rows span 4 GiB or more is refused by both doors before any launch: the kernels address the rows
+    of an expert with 32-bit offsets. The bank is device memory that nothing reads."""
+    k, rows = 16384, 419456                      # 419456 rows x 10240 bytes = 4.0002 GiB
+    bank = dev.alloc(rows * (k // 32) * 20)
+    xb, out, z = dev.put(np.zeros((4, k), np.float16)), dev.alloc(4096), dev.put(np.zeros(64, np.int32))
+    lib, st = dev.lib, dev.stream.handle
+    v = H.view_of(dev, bank, "hq4_g32_m5", rows, k)
+    tiles = (z.ptr, z.ptr, z.ptr, z.ptr, 4, 4)
+    assert lib.qwhip_moe_grouped_gemm(st, C.byref(v), 1, xb.ptr, qwhip.F16, 0, None, *tiles, out.ptr, qwhip.F16, 0) == qwhip.E_BAD_GEOMETRY
+    assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v), 1, xb.ptr, qwhip.F16, 0, None, *tiles, 1, out.ptr, 0) == qwhip.E_BAD_GEOMETRY
+
+
 # (format, gate_up kernel override): HQ4_G32_M5 runs the column-stationary kernels, override 2 keeps its gate_up on the
 # general kernel; the bit-stream container runs the general kernels for both projections.
 @pytest.mark.parametrize("fmt,gu_flags", [("hq4_g32_m5", 0), ("hq4_g32_m5", 2 << 8), ("hq4_g32", 0), ("hq3_g32", 0), ("hq6_g32", 0)])
