@@ -274,8 +274,8 @@ qwhip_status qwhip_embed_bf16_f32(qwhip_stream_t s, const void* table_bf16, uint
  * (QWHIP_X_PREROTATED) unless `workspace` holds m*k f16 elements for the rotated copy.
  * A problem of few tiles (about m * n <= 128 * 128 * 320) whose workspace also holds fp32 planes of m * n
  * elements (after the activation copy, rounded up to 256 bytes, when there is one) runs its K-steps in 2..8
- * ranges and sums the planes in range order in a second launch; the result depends on the workspace size
- * only through that choice, never on its contents. */
+ * ranges and sums the planes in range order in a second launch, when the K-steps saved outweigh the traffic
+ * of the planes; the result depends on the workspace size only through that choice, never on its contents. */
 qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                         uint32_t m, uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags,
                         void* workspace, uint64_t workspace_bytes);

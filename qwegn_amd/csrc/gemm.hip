@@ -1421,8 +1421,10 @@ int choose_cfg(uint32_t M, uint32_t N, bool eight_bit, bool pingpong, bool only_
     const double* eff = !pingpong ? kEffDma : (eight_bit ? kEffPp8 : kEffPp);
     const double resident[CFG_COUNT] = {1, 1, 2, 1, 1};
     // a problem of few tiles is one tile's K loop long whatever the shape, and the small tile's loop is the shortest
-    // (N = K = 5120, f16: M = 64 in 65 us on 128 x 128 against 82 us on the half-height ping-pong tile, M = 256 82 against 85)
-    if ((uint64_t)qwhip_cdiv(M, 128u) * qwhip_cdiv(N, 128u) <= 128u) return CFG_128x128;
+    // (N = K = 5120, f16: M = 64 in 65 us on 128 x 128 against 82 us on the half-height ping-pong tile, M = 512 81 against 85;
+    // N = K = 2048, M = 2048: 32 against 38).  bf16 rows read in place run the unpipelined kernel on that shape, which holds
+    // up to 128 tiles only (M = 256: 88 us against 87)
+    if ((uint64_t)qwhip_cdiv(M, 128u) * qwhip_cdiv(N, 128u) <= (only_pingpong ? 128u : 256u)) return CFG_128x128;
     double best = 1e300;
     int best_cfg = only_pingpong ? CFG_128x320 : CFG_128x128;
     for (int c = 0; c < CFG_COUNT; ++c) {
@@ -1430,8 +1432,13 @@ int choose_cfg(uint32_t M, uint32_t N, bool eight_bit, bool pingpong, bool only_
         if (only_pingpong && !pp) continue;
         const double tiles = (double)qwhip_cdiv(M, kCfgBM[c]) * qwhip_cdiv(N, kCfgBN[c]);
         const double slots = 256.0 * resident[c];
-        const double rounds = (double)(uint64_t)((tiles + slots - 1.0) / slots);
-        const double cost = rounds * resident[c] * kCfgBM[c] * kCfgBN[c] / eff[c];
+        // The last round is cheaper than a full one: the clocks are power-bound, so tiles on half the CUs or fewer finish in
+        // 0.67 of a full round's time and the cost grows linearly from there (256 x 320 on N = K = 5120: 128 tiles 121 us,
+        // 192 tiles 148 us, 256 tiles 180 us; M = 6144, 384 tiles: 301 us = 180 + 121)
+        const double full = (double)(uint64_t)((tiles - 1.0) / slots);
+        const double f = (tiles - full * slots) / slots;
+        const double last = f <= 0.5 ? 0.67 : 0.67 + 0.66 * (f - 0.5);
+        const double cost = (full + last) * resident[c] * kCfgBM[c] * kCfgBN[c] / eff[c];
         if (cost < best) {
             best = cost;
             best_cfg = c;
@@ -1540,7 +1547,12 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
         const uint32_t nk = w->k / 64u;
         const uint64_t plane = (uint64_t)m * w->n * 4u;
         splits = min(min(8u, 256u / tiles), nk / 8u);
-        while (splits >= 2u && ((uint64_t)(splits - 1u) * qwhip_cdiv(nk, splits) >= nk || sk_used + splits * plane > workspace_bytes)) --splits;
+        // Worth it when the K-steps taken off the tile's loop (0.72 us each) outweigh writing and re-reading the planes
+        // (about 5 TB/s together) and the second launch (4 us).  N = K = 2048 with a workspace: M = 1536 over 3 ranges took
+        // 46 us against 36 us in one launch, M = 2048 over 2 ranges 36 against 32; N = K = 5120, M = 1024 over 2: 71 against 84
+        auto pays = [&](uint32_t sp) { return nk * 0.72 * (1.0 - 1.0 / sp) > sp * (double)plane * 2.0 / 5e6 + 4.0; };
+        while (splits >= 2u && ((uint64_t)(splits - 1u) * qwhip_cdiv(nk, splits) >= nk || sk_used + splits * plane > workspace_bytes || !pays(splits)))
+            --splits;
         if (splits < 2u) splits = 0;
     }
     // bf16 activations already in the basis: the ping-pong kernel converts them while it stages the tile (no pass of its own,
