@@ -1697,7 +1697,9 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     p.inter = inter;
     p.rotate_act = rotate_act ? 1u : 0u;
     p.act = s->dev->act;
-    p.tiles_m = qwhip_cdiv(m, 256u);
+    // up to 128 rows: the half-height tile (its K-step is shorter and no row of it is idle; same sums, same results)
+    const bool half = m <= 128u;
+    p.tiles_m = qwhip_cdiv(m, half ? 128u : 256u);
     p.tiles_n = qwhip_cdiv(inter, 160u);
     const dim3 grid(((p.tiles_m * p.tiles_n + 7u) / 8u) * 8u);
     hipError_t e;
@@ -1705,8 +1707,10 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     const bool ga = p.act.kind != 0u;
     switch (fmt) {
 #define QG_SWIGLU3(F) \
-    case F: e = ga ? launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true, QWHIP_F16, true>(s->stream, p, grid) \
-                   : launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true>(s->stream, p, grid); break;
+    case F: e = half ? (ga ? launch_cfg3<1, 5, 4, 2, F, QWHIP_F16, true, QWHIP_F16, true>(s->stream, p, grid) \
+                           : launch_cfg3<1, 5, 4, 2, F, QWHIP_F16, true>(s->stream, p, grid)) \
+                     : (ga ? launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true, QWHIP_F16, true>(s->stream, p, grid) \
+                           : launch_cfg3<2, 5, 4, 2, F, QWHIP_F16, true>(s->stream, p, grid)); break;
         QG_SWIGLU3(QG_FMT_M5) QG_SWIGLU3(QG_FMT_B4) QG_SWIGLU3(QG_FMT_B2) QG_SWIGLU3(QG_FMT_B3) QG_SWIGLU3(QG_FMT_B6) QG_SWIGLU3(QG_FMT_B8)
 #undef QG_SWIGLU3
         default: e = hipErrorInvalidValue;
