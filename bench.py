@@ -795,7 +795,7 @@ def main() -> None:
     ap.add_argument("--variant", type=int, default=0, help="gemv kernel override (0 auto; 1..7 as the flags of qwhip_gemv)")
     ap.add_argument("--rt", type=int, default=0, help="row tiles per wave for the mfma gemv (0 auto)")
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
-    ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 workload when run by itself (0 = the benchmark's 4096)")
+    ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 or mlp_prefill workload when run by itself (0 = the benchmark's 4096)")
     ap.add_argument("--gemm-ws-mb", type=int, default=0,
                     help="workspace handed to qwhip_gemm in MiB (0 = the activation copy only; more lets small row counts split K)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
@@ -838,7 +838,8 @@ def main() -> None:
     elif kind == "gemv_f32":
         out = run_gemv_f32(args, fmt, n, k, m, LABELS[args.workload])
     elif kind == "mlp_prefill":
-        out = run_mlp_prefill(args, n, k, m, LABELS[args.workload])
+        rows_label = f" [rows {args.gemm_rows}]" if args.gemm_rows else ""
+        out = run_mlp_prefill(args, n, k, args.gemm_rows or m, LABELS[args.workload] + rows_label)
     elif kind == "head":
         out = run_head(args, fmt, n, k, LABELS[args.workload])
     elif kind == "repack":
