@@ -1406,6 +1406,13 @@ hipError_t launch_dense1_y(hipStream_t st, qw_gemm_params& p, uint32_t ydt) {
     return launch_cfg<2, 2, 2, 2, FMT, XDT, QWHIP_F32, false>(st, p, grid);
 }
 
+// Rounds of `tiles` over `slots` resident workgroups, the last one priced by how full it is (see choose_cfg).
+double priced_rounds(double tiles, double slots) {
+    const double full = (double)(uint64_t)((tiles - 1.0) / slots);
+    const double f = (tiles - full * slots) / slots;
+    return full + (f <= 0.5 ? 0.67 : 0.67 + 0.66 * (f - 0.5));
+}
+
 // waste-aware choice among the tile shapes: time ~ rounds of tiles over the CUs x per-tile cost / shape efficiency.
 // `pingpong`: the ping-pong kernel is available (2-byte outputs need 16-byte aligned rows) for the 256 x 320 and 128 x 320
 // shapes.  `only_pingpong` keeps the choice to those two (bf16 activations with no workspace to convert into: the other
@@ -1435,10 +1442,7 @@ int choose_cfg(uint32_t M, uint32_t N, bool eight_bit, bool pingpong, bool only_
         // The last round is cheaper than a full one: the clocks are power-bound, so tiles on half the CUs or fewer finish in
         // 0.67 of a full round's time and the cost grows linearly from there (256 x 320 on N = K = 5120: 128 tiles 121 us,
         // 192 tiles 148 us, 256 tiles 180 us; M = 6144, 384 tiles: 301 us = 180 + 121)
-        const double full = (double)(uint64_t)((tiles - 1.0) / slots);
-        const double f = (tiles - full * slots) / slots;
-        const double last = f <= 0.5 ? 0.67 : 0.67 + 0.66 * (f - 0.5);
-        const double cost = (full + last) * resident[c] * kCfgBM[c] * kCfgBN[c] / eff[c];
+        const double cost = priced_rounds(tiles, slots) * resident[c] * kCfgBM[c] * kCfgBN[c] / eff[c];
         if (cost < best) {
             best = cost;
             best_cfg = c;
@@ -1697,10 +1701,13 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     p.inter = inter;
     p.rotate_act = rotate_act ? 1u : 0u;
     p.act = s->dev->act;
-    // up to 128 rows: the half-height tile (its K-step is shorter and no row of it is idle; same sums, same results)
-    const bool half = m <= 128u;
-    p.tiles_m = qwhip_cdiv(m, half ? 128u : 256u);
+    // The half-height tile where it is the cheaper one by the pricing of choose_cfg (0.82 of the big tile's efficiency per
+    // area, 0.78 on 8-bit containers): up to 128 rows, where the big tile is half idle, and where it fills the chip and
+    // the big tile does not (I = 17408: 129 .. 256 rows).  Same sums, same results either way.
     p.tiles_n = qwhip_cdiv(inter, 160u);
+    const bool half = priced_rounds((double)qwhip_cdiv(m, 128u) * p.tiles_n, 256.0) / (fmt == QG_FMT_B8 ? 0.78 : 0.82)
+                      < 2.0 * priced_rounds((double)qwhip_cdiv(m, 256u) * p.tiles_n, 256.0);
+    p.tiles_m = qwhip_cdiv(m, half ? 128u : 256u);
     const dim3 grid(((p.tiles_m * p.tiles_n + 7u) / 8u) * 8u);
     hipError_t e;
     // the plain SwiGLU epilogue keeps its own instantiation: the general activation's code costs it 3 % at this size
