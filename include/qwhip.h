@@ -357,7 +357,11 @@ qwhip_status qwhip_moe_grouped_gemm(qwhip_stream_t s, const qwhip_weight_view* w
  * = f16(FWHT32(silu(g) * u)) with g, u rounded to f16 first - bit-identical to qwhip_gemm (f16 out) followed by
  * qwhip_swiglu_fwht, without the [m, 2 inter] matrix.  One launch for every container and any m; inter % 32 == 0, act
  * 16-byte aligned with ldact % 8 == 0 (0 = inter); x, flags and workspace as qwhip_gemm (bf16 or un-rotated activations
- * need the workspace: m * k * 2 bytes). */
+ * need the workspace: m * k * 2 bytes).  A problem of few tiles and a long K whose workspace also holds, behind the
+ * activation copy, an f16 image of the gate|up matrix (m * 2 inter * 2 bytes, rounded up to 256) and fp32 planes of
+ * m * 2 inter elements runs as qwhip_gemm does with K ranges and then qwhip_swiglu_fwht from the image, when that is
+ * the faster form (packed act rows only; flags bits 8..11 != 0 keep the one launch); as there, the result depends on
+ * the workspace size only through that choice. */
 qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, uint32_t m,
                                uint32_t ldx, uint32_t rotate_act, void* act_f16, uint32_t ldact, uint32_t flags,
                                void* workspace, size_t workspace_bytes);

@@ -1496,6 +1496,22 @@ hipError_t launch_splitk(hipStream_t st, const qw_gemm_params& p, uint32_t split
     }
 }
 
+// K ranges for a problem of few tiles (0 = one launch): 2..8 ranges of at least 8 K-steps over at most 256 workgroups of
+// 128 x 320 tiles, when `workspace_bytes` holds the fp32 planes behind its first `used` bytes and the ranges pay:
+// K-steps taken off the tile's loop (0.72 us each) against writing and re-reading the planes (about 5 TB/s together) and
+// the second launch (4 us).  N = K = 2048 with a workspace: M = 1536 over 3 ranges took 46 us against 36 us in one launch,
+// M = 2048 over 2 ranges 36 against 32; N = K = 5120, M = 1024 over 2: 71 against 84.
+uint32_t choose_splits(uint32_t m, uint32_t n, uint32_t k, uint64_t used, uint64_t workspace_bytes) {
+    const uint32_t tiles = qwhip_cdiv(m, kCfgBM[CFG_128x320]) * qwhip_cdiv(n, kCfgBN[CFG_128x320]);
+    const uint32_t nk = k / 64u;
+    const uint64_t plane = (uint64_t)m * n * 4u;
+    uint32_t splits = min(min(8u, 256u / tiles), nk / 8u);
+    auto pays = [&](uint32_t sp) { return nk * 0.72 * (1.0 - 1.0 / sp) > sp * (double)plane * 2.0 / 5e6 + 4.0; };
+    while (splits >= 2u && ((uint64_t)(splits - 1u) * qwhip_cdiv(nk, splits) >= nk || used + splits * plane > workspace_bytes || !pays(splits)))
+        --splits;
+    return splits < 2u ? 0u : splits;
+}
+
 #define QG_FOR_FMT(fmt, e, EXPR)                                                  \
     switch (fmt) {                                                                \
         case QG_FMT_M5: { constexpr int F = QG_FMT_M5; e = (EXPR); } break;       \
@@ -1543,22 +1559,11 @@ extern "C" qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w,
     // Split-K: a problem of few tiles is one tile's K loop long (80 K-steps of ~1.1 us on K = 5120, whatever M).  When the
     // workspace also holds fp32 partial planes (after the activation copy, if there is one), the K-steps of a tile are dealt
     // over 2..8 workgroups and a second launch sums the planes in range order.
-    uint32_t splits = 0;
     const bool copy_needed = rotate || (x_dtype == QWHIP_BF16 && (flags & (1u << 16)));   // bf16 rows in the basis are read in place
     const uint64_t sk_used = copy_needed ? ((ws_need + 255u) & ~(uint64_t)255u) : 0u;
-    if (ov == 0u && pp_ok && workspace && ((uintptr_t)workspace & 15u) == 0 && w->n % 4u == 0 && (!copy_needed || ws_ok)) {
-        const uint32_t tiles = qwhip_cdiv(m, kCfgBM[CFG_128x320]) * qwhip_cdiv(w->n, kCfgBN[CFG_128x320]);
-        const uint32_t nk = w->k / 64u;
-        const uint64_t plane = (uint64_t)m * w->n * 4u;
-        splits = min(min(8u, 256u / tiles), nk / 8u);
-        // Worth it when the K-steps taken off the tile's loop (0.72 us each) outweigh writing and re-reading the planes
-        // (about 5 TB/s together) and the second launch (4 us).  N = K = 2048 with a workspace: M = 1536 over 3 ranges took
-        // 46 us against 36 us in one launch, M = 2048 over 2 ranges 36 against 32; N = K = 5120, M = 1024 over 2: 71 against 84
-        auto pays = [&](uint32_t sp) { return nk * 0.72 * (1.0 - 1.0 / sp) > sp * (double)plane * 2.0 / 5e6 + 4.0; };
-        while (splits >= 2u && ((uint64_t)(splits - 1u) * qwhip_cdiv(nk, splits) >= nk || sk_used + splits * plane > workspace_bytes || !pays(splits)))
-            --splits;
-        if (splits < 2u) splits = 0;
-    }
+    uint32_t splits = 0;
+    if (ov == 0u && pp_ok && workspace && ((uintptr_t)workspace & 15u) == 0 && w->n % 4u == 0 && (!copy_needed || ws_ok))
+        splits = choose_splits(m, w->n, w->k, sk_used, workspace_bytes);
     // bf16 activations already in the basis: the ping-pong kernel converts them while it stages the tile (no pass of its own,
     // no workspace); flags bit 16 keeps the separate pass, for tests and comparisons
     const bool direct_bf16 = !rotate && x_dtype == QWHIP_BF16 && ov != 15u && !(flags & (1u << 16)) && (splits != 0u || gemm3_takes(p, cfg, fmt, y_dtype));
@@ -1701,6 +1706,24 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
     p.inter = inter;
     p.rotate_act = rotate_act ? 1u : 0u;
     p.act = s->dev->act;
+    // Few tiles and a workspace with room behind the activation copy for an f16 gate|up image and fp32 planes: the K-steps
+    // of a tile are dealt over 2..8 workgroups as in qwhip_gemm, the planes are summed into the image and the SwiGLU pass
+    // reads that - the two doors called one after the other, from one call.  flags bits 8..11 != 0 keep the one launch.
+    {
+        const uint64_t x_used = xin == workspace ? ((ws_need + 255u) & ~(uint64_t)255u) : 0u;
+        const uint64_t gu_bytes = ((uint64_t)m * w->n * 2u + 255u) & ~(uint64_t)255u;
+        uint32_t splits = 0;
+        if (((flags >> 8) & 0xFu) == 0u && workspace && ((uintptr_t)workspace & 15u) == 0 && ldact == inter && workspace_bytes >= x_used + gu_bytes)
+            splits = choose_splits(m, w->n, w->k, x_used + gu_bytes, workspace_bytes);
+        if (splits != 0u) {
+            void* gu = (uint8_t*)workspace + x_used;
+            float* part = (float*)((uint8_t*)workspace + x_used + gu_bytes);
+            hipError_t e;
+            QG_FOR_FMT(fmt, e, (launch_splitk<F>(s->stream, p, splits, part, gu, QWHIP_F16, w->n)))
+            QWHIP_TRY_HIP(e);
+            return qwhip_swiglu_fwht(s, gu, QWHIP_F16, act_f16, m, inter, rotate_act);
+        }
+    }
     // The half-height tile where it is the cheaper one by the pricing of choose_cfg (0.82 of the big tile's efficiency per
     // area, 0.78 on 8-bit containers): up to 128 rows, where the big tile is half idle, and where it fills the chip and
     // the big tile does not (I = 17408: 129 .. 256 rows).  Same sums, same results either way.

@@ -259,7 +259,8 @@ def test_gemm_swiglu_equals_gemm_then_swiglu(dev, fmt, xdtype, prerot, m, inter,
 @pytest.mark.parametrize("xdtype,prerot", [("f16", True), ("bf16", False)])
 def test_gemm_swiglu_every_container_and_row_count_in_one_launch(dev, fmt, m, xdtype, prerot):
     """The 6- and 8-bit containers and ragged row counts on the fused door (once two launches through the workspace): the same
-    bits as the two doors called one after the other, whatever workspace beyond the activation copy is handed over."""
+    bits as the two doors called one after the other, whatever workspace beyond the activation copy is handed over (K = 384 is
+    too short for K ranges, which a roomy workspace would otherwise bring)."""
     inter, k = 224, 384
     n = 2 * inter
     rotate = H.FORMATS[fmt][4]
@@ -285,6 +286,48 @@ def test_gemm_swiglu_every_container_and_row_count_in_one_launch(dev, fmt, m, xd
     # a workspace that holds only the activation copy is enough: the door is one launch for every container and row count
     assert lib.qwhip_gemm_swiglu(st, C.byref(view), xb.ptr, xcode, m, 0, 1, act1.ptr, 0, flags, ws1.ptr, ws1.nbytes) == qwhip.OK
     dev.stream.sync()
+
+
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32", "hq3_g32"])
+@pytest.mark.parametrize("m,inter,k,xdtype,prerot", [(64, 320, 2048, "f16", True), (100, 480, 1536, "bf16", True), (37, 160, 1024, "f16", False),
+                                                     (128, 800, 5120, "bf16", False)])
+def test_gemm_swiglu_split_k_with_a_roomy_workspace(dev, fmt, m, inter, k, xdtype, prerot):
+    """Few tiles, a long K and a workspace with room for an f16 gate|up image and fp32 planes behind the activation copy: the
+    fused door deals the K-steps over several workgroups, sums the planes and runs the SwiGLU pass - the same bits as qwhip_gemm
+    (which splits the same way when neither workspace binds) followed by qwhip_swiglu_fwht, within the bar of the oracle, and
+    within rounding of its own one-launch form (flags bits 8..11 set keep that)."""
+    n = 2 * inter
+    blocks, w16 = H.make_bank(fmt, n, k, seed=6)
+    x32 = H.make_x(m, k, 14)
+    rotate = H.FORMATS[fmt][4]
+    if xdtype == "bf16":
+        x_val, x_host, xcode = qo.round_bf16(x32), qo.f32_to_bf16_bits(x32), qwhip.BF16
+    else:
+        x_host, xcode = x32.astype(np.float16), qwhip.F16
+        x_val = x_host.astype(np.float32)
+    flags = qwhip.X_PREROTATED if (prerot or not rotate) else 0
+    x_basis = x_val.astype(np.float16) if flags else qo.fwht32_ortho(x_val).astype(np.float16)
+    bank, xb = dev.put(blocks), dev.put(x_host)
+    gu = dev.alloc(m * n * 2)
+    acts = [dev.put(np.zeros((m, inter), np.float16)) for _ in range(3)]
+    ws = dev.alloc(64 << 20)
+    view = H.view_of(dev, bank, fmt, n, k)
+    lib, st = dev.lib, dev.stream.handle
+    # bf16 rows go through the separate conversion pass in both doors (flags bit 16 asks qwhip_gemm for it), so both split alike
+    qwhip.check(lib.qwhip_gemm(st, C.byref(view), xb.ptr, xcode, m, 0, gu.ptr, qwhip.F16, 0, flags | (1 << 16), ws.ptr, ws.nbytes))
+    qwhip.check(lib.qwhip_swiglu_fwht(st, gu.ptr, qwhip.F16, acts[0].ptr, m, inter, 1))
+    qwhip.check(lib.qwhip_gemm_swiglu(st, C.byref(view), xb.ptr, xcode, m, 0, 1, acts[1].ptr, 0, flags, ws.ptr, ws.nbytes))
+    qwhip.check(lib.qwhip_gemm_swiglu(st, C.byref(view), xb.ptr, xcode, m, 0, 1, acts[2].ptr, 0, flags | (1 << 8), ws.ptr, ws.nbytes))
+    dev.stream.sync()
+    two, split, one = (a.download(np.float16, (m, inter)) for a in acts)
+    for b in (bank, xb, gu, ws, *acts):
+        b.free()
+    assert np.array_equal(split.view(np.uint16), two.view(np.uint16))
+    g = qo.matmul_ref_f64(x_basis, w16).astype(np.float16).astype(np.float32)
+    want = qo.swiglu_fwht_f16(g[:, :inter], g[:, inter:], rotate=True).astype(np.float32)
+    assert qo.normalized_error(split.astype(np.float32), want) <= TOL
+    assert qo.normalized_error(one.astype(np.float32), want) <= TOL
+    assert qo.normalized_error(split.astype(np.float32), one.astype(np.float32)) <= TOL
 
 
 def test_gemm_swiglu_refusals(dev):
