@@ -795,6 +795,7 @@ def main() -> None:
     ap.add_argument("--variant", type=int, default=0, help="gemv kernel override (0 auto; 1..7 as the flags of qwhip_gemv)")
     ap.add_argument("--rt", type=int, default=0, help="row tiles per wave for the mfma gemv (0 auto)")
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
+    ap.add_argument("--moe-tokens", type=int, default=0, help="tokens of a c4 workload when run by itself (0 = the benchmark's 1 / 2048)")
     ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 or mlp_prefill workload when run by itself (0 = the benchmark's 4096)")
     ap.add_argument("--gemm-ws-mb", type=int, default=0,
                     help="workspace handed to qwhip_gemm in MiB (0 = the activation copy only; more lets small row counts split K)")
@@ -834,7 +835,8 @@ def main() -> None:
         fmt, traffic = args.format, None
         label += f" [container {fmt}]"
     if kind == "moe":
-        out = run_moe(args, m, LABELS[args.workload])
+        tokens = args.moe_tokens or m
+        out = run_moe(args, tokens, LABELS[args.workload] + (f" [tokens {tokens}]" if args.moe_tokens else ""))
     elif kind == "gemv_f32":
         out = run_gemv_f32(args, fmt, n, k, m, LABELS[args.workload])
     elif kind == "mlp_prefill":
