@@ -1420,9 +1420,10 @@ double priced_rounds(double tiles, double slots) {
 int choose_cfg(uint32_t M, uint32_t N, bool eight_bit, bool pingpong, bool only_pingpong) {
     // efficiency of each shape per tile area, on the scale ping-pong 256 x 320 on a 4-bit container = 1 (188 us a round
     // on M = 4096, N = K = 5120).  DMA-fed kernel: 264 us on that tile (0.71), the smaller shapes 0.82 / 0.78 / 0.75 of that;
-    // half-height ping-pong tile: 115 us for 256 tiles (0.82); 8-bit containers: 206 us a round on the ping-pong 256 x 320
-    // (0.91; 237 - 242 us on the DMA-fed kernel), 132 us on the half-height tile (0.71)
-    static const double kEffPp[CFG_COUNT] = {1.00, 0.58, 0.55, 0.53, 0.82};
+    // half-height ping-pong tile: 115 us for 256 tiles against 90 us for half a round of the big tile (0.78); 8-bit
+    // containers: 206 us a round on the ping-pong 256 x 320 (0.91; 237 - 242 us on the DMA-fed kernel), 132 us on the
+    // half-height tile (0.71)
+    static const double kEffPp[CFG_COUNT] = {1.00, 0.58, 0.55, 0.53, 0.78};
     static const double kEffPp8[CFG_COUNT] = {0.91, 0.65, 0.62, 0.59, 0.71};
     static const double kEffDma[CFG_COUNT] = {0.71, 0.58, 0.55, 0.53, 0.58};
     const double* eff = !pingpong ? kEffDma : (eight_bit ? kEffPp8 : kEffPp);
@@ -1724,11 +1725,11 @@ extern "C" qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_v
             return qwhip_swiglu_fwht(s, gu, QWHIP_F16, act_f16, m, inter, rotate_act);
         }
     }
-    // The half-height tile where it is the cheaper one by the pricing of choose_cfg (0.82 of the big tile's efficiency per
-    // area, 0.78 on 8-bit containers): up to 128 rows, where the big tile is half idle, and where it fills the chip and
+    // The half-height tile where it is the cheaper one by the pricing of choose_cfg (0.78 of the big tile's efficiency per
+    // area): up to 128 rows, where the big tile is half idle, and where it fills the chip and
     // the big tile does not (I = 17408: 129 .. 256 rows).  Same sums, same results either way.
     p.tiles_n = qwhip_cdiv(inter, 160u);
-    const bool half = priced_rounds((double)qwhip_cdiv(m, 128u) * p.tiles_n, 256.0) / (fmt == QG_FMT_B8 ? 0.78 : 0.82)
+    const bool half = priced_rounds((double)qwhip_cdiv(m, 128u) * p.tiles_n, 256.0) / 0.78
                       < 2.0 * priced_rounds((double)qwhip_cdiv(m, 256u) * p.tiles_n, 256.0);
     p.tiles_m = qwhip_cdiv(m, half ? 128u : 256u);
     const dim3 grid(((p.tiles_m * p.tiles_n + 7u) / 8u) * 8u);
