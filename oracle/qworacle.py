@@ -785,6 +785,40 @@ def moe_forward_f64(x, idx, wts, gate_up_w, down_w, act_f16: bool, rotate_act: b
     return out
 
 
+def moe_forward_grouped_f64(x, idx, wts, gate_up_w, down_w, act_f16: bool, rotate_act: bool):
+    """moe_forward_f64 with the work ordered by expert instead of by token: the rows routed to expert e are gathered,
+    contracted with that expert's gate|up and down weights as two fp64 matrix products, and scattered back weighted.
+    Same sums per (token, route) as moe_forward_f64 up to fp64 summation order (pinned against it in
+    tests/test_oracle_math.py); it exists so that a whole prefill batch (thousands of tokens, every expert) can be
+    checked in seconds.  gate_up_w / down_w: anything indexable by expert that returns [2I, H] / [H, I] weights
+    (Tests/QWFlashNextTests/Reference/FNSparseMoE.swift:106-160 is the per-token form)."""
+    x = np.asarray(x, dtype=np.float64)
+    idx = np.asarray(idx)
+    t = x.shape[0]
+    ids = np.where(idx < 0, -1, idx & 0xFFFF)
+    out = None
+    for ex in np.unique(ids[ids >= 0]):
+        rows, slots = np.nonzero(ids == ex)
+        gu_w = np.asarray(gate_up_w[int(ex)], dtype=np.float64)
+        dn_w = np.asarray(down_w[int(ex)], dtype=np.float64)
+        i = gu_w.shape[0] // 2
+        gu = x[rows] @ gu_w.T
+        g, u = gu[:, :i], gu[:, i:]
+        act = g / (1.0 + np.exp(-g)) * u
+        if act_f16:
+            a32 = act.astype(np.float32)
+            if rotate_act and i % 32 == 0:
+                a32 = fwht32_ortho(a32)
+            act = a32.astype(np.float16).astype(np.float64)
+        part = (act @ dn_w.T) * np.asarray(wts, dtype=np.float64)[rows, slots][:, None]
+        if out is None:
+            out = np.zeros((t, dn_w.shape[0]), dtype=np.float64)
+        np.add.at(out, rows, part)
+    if out is None:
+        out = np.zeros((t, np.asarray(down_w[0]).shape[0]), dtype=np.float64)
+    return out
+
+
 # --------------------------------------------------------------------------- #
 # group-latent routed MoE block  (no golden in the reference: pinned by the identities of tests/test_oracle_math.py -
 # one identity group reduces it to moe_forward_f64, and the per-route expansion by linearity of U_g)

@@ -836,7 +836,7 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
 // qwhip_swiglu_fwht on the f16 gate|up matrix without writing it (the reference's fused form for its dense path:
 // qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167).
 // ------------------------------------------------------------------------------------------------
-template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false, int XDT = QWHIP_F16>
 __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
     static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
     constexpr uint32_t BM = 64, BN = 256, STAGE = BM * 128u;
@@ -904,7 +904,7 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *(u4_t*)(lds4 + stage * STAGE + a_lds0 + i * 4096u) = a_reg[i];
+        for (int i = 0; i < 2; ++i) *(h8_t*)(lds4 + stage * STAGE + a_lds0 + i * 4096u) = qg_to_f16x8<XDT>(a_reg[i]);
     };
     auto load_b = [&](uint32_t kt, qg_slice<FMT>* blk) {
 #pragma unroll
@@ -1035,7 +1035,7 @@ __global__ __launch_bounds__(256) void qw_gemm4_kernel(const qw_gemm_params p) {
 // four workgroups per CU.  The raw image of K pair kp + 1 is in flight (registers) during K pair kp and replaces the
 // stage between two barriers at its end.
 // ------------------------------------------------------------------------------------------------
-template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false, int XDT = QWHIP_F16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void qw_gemm5_kernel(const qw_gemm_params p) {
     static_assert(!SWIGLU || YDT == QWHIP_F16, "fused SwiGLU stores f16");
     static_assert(FMT == QG_FMT_M5 || FMT == QG_FMT_B4, "20-byte blocks: HQ4_G32_M5 and the 4-bit group-32 bit streams");
@@ -1111,7 +1111,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     };
     auto store_a = [&](uint32_t stage, const u4_t* a_reg) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *(u4_t*)(lds5 + stage * A_STAGE + a_lds0 + i * 4096u) = a_reg[i];
+        for (int i = 0; i < 2; ++i) *(h8_t*)(lds5 + stage * A_STAGE + a_lds0 + i * 4096u) = qg_to_f16x8<XDT>(a_reg[i]);
     };
     auto load_raw = [&](uint32_t kp, u4_t* raw) {
 #pragma unroll
@@ -1323,20 +1323,20 @@ __global__ __launch_bounds__(256) void qw_splitk_reduce_kernel(const float* __re
     for (int e = 0; e < 4; ++e) qg_store<YDT>(y, (uint64_t)row * ldy + c + e, acc[e]);
 }
 
-template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false, int XDT = QWHIP_F16>
 hipError_t launch_cfg4(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     // two activation stages, or the four epilogue slabs (32 rows x (128 + 16) bytes each) when they are larger
     constexpr size_t lds = 4u * 32u * 144u;
     static_assert(lds >= 2u * 64u * 128u, "the stages fit the slab allocation");
-    hipLaunchKernelGGL((qw_gemm4_kernel<FMT, YDT, SWIGLU, GACT>), grid, dim3(256), lds, st, p);
+    hipLaunchKernelGGL((qw_gemm4_kernel<FMT, YDT, SWIGLU, GACT, XDT>), grid, dim3(256), lds, st, p);
     return hipGetLastError();
 }
 
-template <int FMT, int YDT, bool SWIGLU, bool GACT = false>
+template <int FMT, int YDT, bool SWIGLU, bool GACT = false, int XDT = QWHIP_F16>
 hipError_t launch_cfg5(hipStream_t st, const qw_gemm_params& p, dim3 grid) {
     constexpr size_t lds = 2u * 64u * 128u + 256u * 88u;   // two activation stages + one raw K-pair image (38,912 bytes)
     if constexpr (FMT == QG_FMT_M5 || FMT == QG_FMT_B4) {
-        hipLaunchKernelGGL((qw_gemm5_kernel<FMT, YDT, SWIGLU, GACT>), grid, dim3(256), lds, st, p);
+        hipLaunchKernelGGL((qw_gemm5_kernel<FMT, YDT, SWIGLU, GACT, XDT>), grid, dim3(256), lds, st, p);
         return hipGetLastError();
     } else {
         return hipErrorInvalidValue;   // not reached: gemm5_takes() refuses the 8-bit containers
@@ -1758,23 +1758,27 @@ hipError_t launch_grouped_y(hipStream_t st, const qw_gemm_params& p, dim3 grid, 
     if (ydt == QWHIP_BF16) return launch_cfg<2, 2, 1, 4, FMT, XDT, QWHIP_BF16, true>(st, p, grid);
     return launch_cfg<2, 2, 1, 4, FMT, XDT, QWHIP_F32, true>(st, p, grid);
 }
+// direct-operand kernels on the 64 x 256 tiles of the list (weights dequantized straight into MFMA operand registers, only
+// the activation tile in LDS); bf16 rows become f16 between the load registers and LDS
+template <int FMT, int XDT>
+hipError_t launch_grouped_direct(hipStream_t st, const qw_gemm_params& p, dim3 grid, uint32_t ydt) {
+    qw_gemm_params q = p;
+    q.tiles_n = grid.x;
+    const dim3 grid1(8u * qwhip_cdiv(grid.y, 8u) * grid.x);   // XCD-aware one-dimensional grid over (tile, column tile)
+    if (gemm5_takes(q, FMT)) {
+        if (ydt == QWHIP_F16) return launch_cfg5<FMT, QWHIP_F16, false, false, XDT>(st, q, grid1);
+        if (ydt == QWHIP_BF16) return launch_cfg5<FMT, QWHIP_BF16, false, false, XDT>(st, q, grid1);
+        return launch_cfg5<FMT, QWHIP_F32, false, false, XDT>(st, q, grid1);
+    }
+    if (ydt == QWHIP_F16) return launch_cfg4<FMT, QWHIP_F16, false, false, XDT>(st, q, grid1);
+    if (ydt == QWHIP_BF16) return launch_cfg4<FMT, QWHIP_BF16, false, false, XDT>(st, q, grid1);
+    return launch_cfg4<FMT, QWHIP_F32, false, false, XDT>(st, q, grid1);
+}
 template <int FMT>
 hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid, uint32_t xdt, uint32_t ydt) {
-    if (xdt == QWHIP_F16 && !p.force_gemm2 && (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0))) {
-        // direct-operand kernel on the 64 x 256 tiles (weights dequantized straight into MFMA operand registers, only the
-        // activation tile in LDS); it measured level with the 8-wave ping-pong kernel it replaced (gate_up 211 vs 215 us
-        // on T = 2048, E = 128, top-8) at a quarter of the LDS traffic
-        qw_gemm_params q = p;
-        q.tiles_n = grid.x;
-        const dim3 grid1(8u * qwhip_cdiv(grid.y, 8u) * grid.x);   // XCD-aware one-dimensional grid over (tile, column tile)
-        if (gemm5_takes(q, FMT)) {
-            if (ydt == QWHIP_F16) return launch_cfg5<FMT, QWHIP_F16, false>(st, q, grid1);
-            if (ydt == QWHIP_BF16) return launch_cfg5<FMT, QWHIP_BF16, false>(st, q, grid1);
-            return launch_cfg5<FMT, QWHIP_F32, false>(st, q, grid1);
-        }
-        if (ydt == QWHIP_F16) return launch_cfg4<FMT, QWHIP_F16, false>(st, q, grid1);
-        if (ydt == QWHIP_BF16) return launch_cfg4<FMT, QWHIP_BF16, false>(st, q, grid1);
-        return launch_cfg4<FMT, QWHIP_F32, false>(st, q, grid1);
+    if (!p.force_gemm2 && (ydt == QWHIP_F32 || (p.ldy % 8u == 0 && ((uintptr_t)p.y & 15u) == 0))) {
+        if (xdt == QWHIP_F16) return launch_grouped_direct<FMT, QWHIP_F16>(st, p, grid, ydt);
+        return launch_grouped_direct<FMT, QWHIP_BF16>(st, p, grid, ydt);
     }
     if (xdt == QWHIP_F16) {  // DMA-fed pipelined kernel, 64 x 256 tiles
         if (ydt == QWHIP_F16) return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F16, true>(st, p, grid);
@@ -1782,6 +1786,16 @@ hipError_t launch_grouped_xy(hipStream_t st, const qw_gemm_params& p, dim3 grid,
         return launch_cfg2<2, 2, 1, 4, FMT, QWHIP_F32, true>(st, p, grid);
     }
     return launch_grouped_y<FMT, QWHIP_BF16>(st, p, grid, ydt);
+}
+// fused gate_up: the plain SwiGLU epilogue keeps its own instantiation (GACT = false)
+template <int FMT, int XDT>
+hipError_t launch_grouped_swiglu(hipStream_t st, const qw_gemm_params& p, dim3 grid, bool ga) {
+    if (gemm5_takes(p, FMT)) {
+        if (ga) return launch_cfg5<FMT, QWHIP_F16, true, true, XDT>(st, p, grid);
+        return launch_cfg5<FMT, QWHIP_F16, true, false, XDT>(st, p, grid);
+    }
+    if (ga) return launch_cfg4<FMT, QWHIP_F16, true, true, XDT>(st, p, grid);
+    return launch_cfg4<FMT, QWHIP_F16, true, false, XDT>(st, p, grid);
 }
 }  // namespace
 
@@ -1850,8 +1864,6 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     QWHIP_REQUIRE(tile_e);
     QWHIP_REQUIRE(tile_r);
     QWHIP_REQUIRE(tile_count);
-    if (x_dtype != QWHIP_F16)
-        return qwhip_fail(QWHIP_E_BAD_SHAPE, "the fused gate_up GEMM takes f16 activations (bf16: qwhip_moe_grouped_gemm + qwhip_swiglu_fwht)");
     if (experts == 0 || experts > 512 || w->n % experts != 0)
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "grouped GEMM: %u rows do not split over %u experts (<= 512)", w->n, experts);
     if (pairs == 0 || max_tiles == 0) return QWHIP_OK;
@@ -1890,16 +1902,11 @@ extern "C" qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qw
     p.tiles_n = qwhip_cdiv(inter, 128u);
     const dim3 grid(8u * qwhip_cdiv(max_tiles, 8u) * p.tiles_n);   // XCD-aware one-dimensional grid over (tile, column tile)
     hipError_t e;
-    const bool ga = p.act.kind != 0u;   // the plain SwiGLU epilogue keeps its own instantiation
-    if (gemm5_takes(p, fmt)) {
-        if (ga) e = fmt == QG_FMT_M5 ? launch_cfg5<QG_FMT_M5, QWHIP_F16, true, true>(s->stream, p, grid)
-                                     : launch_cfg5<QG_FMT_B4, QWHIP_F16, true, true>(s->stream, p, grid);
-        else e = fmt == QG_FMT_M5 ? launch_cfg5<QG_FMT_M5, QWHIP_F16, true>(s->stream, p, grid)
-                                  : launch_cfg5<QG_FMT_B4, QWHIP_F16, true>(s->stream, p, grid);
-    } else if (ga) {
-        QG_FOR_FMT(fmt, e, (launch_cfg4<F, QWHIP_F16, true, true>(s->stream, p, grid)))
+    const bool ga = p.act.kind != 0u;
+    if (x_dtype == QWHIP_F16) {
+        QG_FOR_FMT(fmt, e, (launch_grouped_swiglu<F, QWHIP_F16>(s->stream, p, grid, ga)))
     } else {
-        QG_FOR_FMT(fmt, e, (launch_cfg4<F, QWHIP_F16, true>(s->stream, p, grid)))
+        QG_FOR_FMT(fmt, e, (launch_grouped_swiglu<F, QWHIP_BF16>(s->stream, p, grid, ga)))
     }
     QWHIP_TRY_HIP(e);
     return QWHIP_OK;

@@ -198,6 +198,180 @@ static __device__ __forceinline__ void run(const P& pp) {
 }
 };
 
+// The same kernel with the block loads issued and awaited by hand.  A compiled rolling window drains once per trip: the
+// register allocator reuses a load's destination as a temporary, copies the value out at the loop's ends, and every copy
+// waits for its load, so a wave has at most D rows in flight right after a trip's start and none at its end (the loop is
+// one memory round trip per D rows per wave).  Here the loads are `asm volatile` statements whose destination registers
+// are tied in and out ("+v": the same registers all the way round the loop), and each row is consumed behind an
+// s_waitcnt vmcnt(2 (D - 1)): exactly the two loads of the oldest row have to have landed, the D - 1 younger rows stay in
+// flight.  Loads stop with the set's last row (the compiled form re-reads it D times) and the last D rows are consumed
+// behind waits that count down.  The activation loads are issued by hand as well: the compiler does not know of the block
+// loads behind them and would wait for everything (vmcnt(0)) before the rotation.
+// Launch contract: trip count ceil(rows per workgroup / SETS) >= 2 D (the host checks).
+template <int XDT, int SETS, int D>
+struct qw_gemv_colw_kernel {
+static constexpr int kLaunchBound = 1024;
+template <int N>
+static __device__ __forceinline__ void wait_row(uint32_t& hdr, u4_t& q) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(hdr), "+v"(q) : "n"(N));
+}
+template <int U, typename F>
+static __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (U < D) {
+        f(std::integral_constant<int, U>{});
+        static_for<U + 1>(f);
+    }
+}
+static __device__ __forceinline__ void run(const qc_params& p) {
+    constexpr int XT = SETS == 1 ? 5 : (SETS == 2 ? 2 : 1);
+    extern __shared__ h8_t qc_lds[];
+    const uint32_t nb = p.nb, cpr = p.cpr, N = p.N;
+    h8_t* xs = qc_lds;
+    float* part = (float*)(qc_lds + (size_t)nb * 5);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 31u, hw = tid >> 5;
+    const uint32_t wave = tid >> 6, l64 = tid & 63u;
+    const uint32_t threads = 32u * cpr * SETS;   // blockDim.x, without the load from the dispatch packet ahead of the first loads
+    const uint32_t nw = threads >> 6;
+    const bool tiler = wave < nw;
+    const uint32_t set = hw / cpr, chunk = hw - set * cpr;
+    const uint32_t g0 = chunk * 32u + lane;
+    const bool gvalid = g0 < nb;
+    const uint32_t g = gvalid ? g0 : nb - 1u;
+    const uint32_t G = gridDim.x;
+    if (blockIdx.x >= N) return;
+    const uint32_t nrows = (N - blockIdx.x + G - 1u) / G;
+    const uint32_t nmax = (nrows + SETS - 1u) / SETS;
+    const uint32_t row_bytes = nb * 20u;
+    const uint32_t step = G * SETS * row_bytes;
+    const uint32_t mine = nrows > set ? (nrows - set + SETS - 1u) / SETS : 0u;
+    uint32_t off = ((mine ? set : 0u) * G + blockIdx.x) * row_bytes + g * 20u;
+    const uint32_t off_max = off + (mine ? mine - 1u : 0u) * step;   // a set one row short re-reads its last row once
+
+    // 1. activation loads, by hand
+    u4_t xraw[XT];
+#pragma unroll
+    for (int t = 0; t < XT; ++t) {
+        const uint32_t gt = wave + nw * t;
+        const uint32_t gg = min(gt * 16u + (l64 & 15u), nb - 1u);
+        const uint32_t xoff = (gg * 32u + 8u * (l64 >> 4)) * 2u;
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(xraw[t]) : "v"(xoff), "s"(p.x) : "memory");
+    }
+    // 2. the first D rows
+    uint32_t hdr[D];
+    u4_t qv[D];
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        hdr[j] = 0u;
+        qv[j] = u4_t{0u, 0u, 0u, 0u};
+    }
+    auto issue = [&](int slot) {
+        asm volatile("global_load_dword %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:4"
+                     : "+v"(hdr[slot]), "+v"(qv[slot]) : "v"(off), "s"(p.bank) : "memory");
+        off = min(off + step, off_max);
+    };
+#pragma unroll
+    for (int j = 0; j < D; ++j) issue(j);
+    // 3. rotation on the matrix cores into the shared image: the XT activation loads have landed, the 2 D block loads fly on
+#pragma unroll
+    for (int t = 0; t < XT; ++t) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xraw[t]) : "n"(2 * D));
+    {
+        h8_t h_lo, h_hi;
+        qw_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
+        if (tiler) {
+#pragma unroll
+            for (int t = 0; t < XT; ++t)
+                qw_rotate_tile_to_lds(qw_x8_from_raw<XDT>(xraw[t]), wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs);
+        }
+    }
+    __syncthreads();
+    // 4. this lane's column: 16 operand pairs and the group sum S
+    h2_t xo[16];
+    float S;
+    {
+        const h8_t* src = xs + g * 5;
+        const h2_t one = {(h1_t)1.0f, (h1_t)1.0f};
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const h8_t v = src[j];
+#pragma unroll
+            for (int e2 = 0; e2 < 4; ++e2) {
+                const h2_t pr = {v[2 * e2], v[2 * e2 + 1]};
+                if (e2 & 1) s1 = __builtin_amdgcn_fdot2(pr, one, s1, false);
+                else s0 = __builtin_amdgcn_fdot2(pr, one, s0, false);
+                xo[4 * j + e2] = pr;
+            }
+        }
+        S = s0 + s1;
+    }
+
+    uint32_t rslot = set;
+    auto consume = [&](int slot) {
+        const uint32_t h = hdr[slot];
+        float lo0 = 0.f, lo1 = 0.f, hi0 = 0.f, hi1 = 0.f;
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+            const uint32_t w = qv[slot][w4], w8 = w >> 8;
+            const uint32_t m0 = w & 0x000F000Fu, m1 = w & 0x00F000F0u, m2 = w8 & 0x000F000Fu, m3 = w8 & 0x00F000F0u;
+            lo0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m0), xo[4 * w4 + 0], lo0, false);
+            hi0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m1), xo[4 * w4 + 1], hi0, false);
+            lo1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m2), xo[4 * w4 + 2], lo1, false);
+            hi1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m3), xo[4 * w4 + 3], hi1, false);
+        }
+        const h2_t hd = __builtin_bit_cast(h2_t, h);
+        const float sc = (float)hd[0];
+        const float q = __builtin_fmaf(hi0 + hi1, 0.0625f, lo0 + lo1);
+        float v = __builtin_fmaf(sc * 16777216.0f, q, __builtin_fmaf(sc, 1024.0f, (float)hd[1]) * S);
+        v = gvalid ? v : 0.0f;
+        v = qw_reduce32_dpp(v);
+        if (lane == 31u && rslot < nrows) part[rslot * cpr + chunk] = v;
+        rslot += SETS;
+    };
+    // steady state: every consumed row is replaced
+    uint32_t i = 0;
+    for (; i + 2u * D <= nmax; i += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            wait_row<2 * (D - 1)>(hdr[j], qv[j]);
+            consume(j);
+            issue(j);
+        }
+    }
+    // the last rem rows, D <= rem < 2 D: rem - D of them are still replaced, the last D are not
+    const uint32_t rem = nmax - i;
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+        if ((uint32_t)u + D < rem) {
+            wait_row<2 * (D - 1)>(hdr[u], qv[u]);
+            consume(u);
+            issue(u);
+        }
+    }
+    // now exactly D rows are in flight or landed; the oldest sits in slot (rem - D) % D = rem - D
+    const uint32_t first = rem - D;
+    static_for<0>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+#pragma unroll
+        for (int sl = 0; sl < D; ++sl) {
+            if ((first + (uint32_t)u) % D == (uint32_t)sl) {
+                wait_row<2 * (D - 1 - u)>(hdr[sl], qv[sl]);
+                consume(sl);
+            }
+        }
+    });
+    __syncthreads();
+    // 5. fixed-order sum of the chunk partials of each row
+    for (uint32_t s = tid; s < nrows; s += threads) {
+        float v = 0.f;
+        for (uint32_t c = 0; c < cpr; ++c) v += part[s * cpr + c];
+        const uint32_t row = s * G + blockIdx.x;
+        if (p.y32) p.y32[row] = v;
+        if (p.y16) p.y16[row] = (h1_t)v;
+    }
+}
+};
+
 // Folds the workgroups' keys into the token: one workgroup.
 __global__ __launch_bounds__(256) void qw_col_keys_fin_kernel(const unsigned long long* __restrict__ keys, uint32_t count, int32_t* token) {
     __shared__ unsigned long long wbest[4];
@@ -225,6 +399,17 @@ hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t 
 #undef QC_TAKE
         pf.keys = keys;
         qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 2, qc_params_fold>>(dim3(wgs), dim3(threads), lds, st, pf);
+        return hipGetLastError();
+    }
+    if (depth >= 16) {   // hand-issued window of depth - 16 + 1 rows
+        switch (depth - 16u) {
+            case 1: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 2>>(dim3(wgs), dim3(threads), lds, st, p); break;
+            case 2: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 3>>(dim3(wgs), dim3(threads), lds, st, p); break;
+            case 3: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 4>>(dim3(wgs), dim3(threads), lds, st, p); break;
+            case 4: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 5>>(dim3(wgs), dim3(threads), lds, st, p); break;
+            case 5: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 6>>(dim3(wgs), dim3(threads), lds, st, p); break;
+            default: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 8>>(dim3(wgs), dim3(threads), lds, st, p); break;
+        }
         return hipGetLastError();
     }
     if (depth == 1) qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 1>>(dim3(wgs), dim3(threads), lds, st, p);
@@ -264,7 +449,10 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     const uint32_t rows_per_wg = qwhip_cdiv(w->n, wgs);
     const size_t lds = (size_t)nb * 80u + (size_t)rows_per_wg * cpr * 4u;
     if (lds > 60u * 1024u) return false;
-    const uint32_t depth = (tune & 3u) == 1u ? 1u : ((tune & 3u) ? (tune & 3u) + 1u : 2u);
+    uint32_t depth = (tune & 3u) == 1u ? 1u : ((tune & 3u) ? (tune & 3u) + 1u : 2u);
+    const uint32_t wcode = (tune >> 4) & 7u;          // 1..5 -> window of 2..6 rows, 6, 7 -> 8 rows
+    const uint32_t wdepth = wcode == 0u ? 0u : (wcode <= 5u ? wcode + 1u : 8u);
+    if (wdepth && !keys && qwhip_cdiv(w->n / wgs, sets) >= 2u * wdepth) depth = 16u + wcode;
     qc_params p;
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;

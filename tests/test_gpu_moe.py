@@ -175,13 +175,25 @@ def _moe_banks(experts, hidden, inter, seed, fmt="hq4_g32_m5"):
     return gu_blocks, gu16.reshape(experts, 2 * inter, hidden), dn_blocks, dn16.reshape(experts, hidden, inter)
 
 
+def _hidden_rows(rng, t, hidden, xdt):
+    """Hidden rows in the experts' basis as the device takes them (f16 values, or bf16 bit patterns), their dtype code, and
+    the values they hold."""
+    x32 = rng.standard_normal((t, hidden)).astype(np.float32)
+    if xdt == "f16":
+        xh = qo.rotate_activation_f16(x32)
+        return xh, qwhip.F16, xh.astype(np.float32)
+    bits = qo.f32_to_bf16_bits(qo.fwht32_ortho(x32))
+    return bits, qwhip.BF16, qo.bf16_bits_to_f32(bits)
+
+
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
 @pytest.mark.parametrize("t,experts,hidden,inter,k", [(40, 8, 256, 128, 2), (130, 16, 512, 192, 4)])
-def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
-    """route -> pair sort -> grouped gate_up GEMM -> SwiGLU+FWHT -> grouped down GEMM -> combine."""
+def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k, xdt):
+    """route -> pair sort -> grouped gate_up GEMM -> SwiGLU+FWHT -> grouped down GEMM -> combine; f16 and bf16 hidden rows."""
     fmt = "hq4_g32_m5"
     gu_blocks, gu16, dn_blocks, dn16 = _moe_banks(experts, hidden, inter, seed=11)
     rng = np.random.default_rng(5)
-    x16 = qo.rotate_activation_f16(rng.standard_normal((t, hidden)).astype(np.float32))     # rotated f16 hidden
+    x16, xcode, xval = _hidden_rows(rng, t, hidden, xdt)                                     # rotated hidden rows
     logits = rng.standard_normal((t, experts)).astype(np.float32)
     idx, wts = _route(dev, logits, k)
     g = _group(dev, idx, experts, k)
@@ -192,7 +204,7 @@ def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
     wb = dev.put(wts)
     vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
     vdn = H.view_of(dev, dnb, fmt, experts * hidden, inter)
-    qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, b["stok"].ptr, b["off"].ptr, b["te"].ptr,
+    qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), experts, xb.ptr, xcode, 0, b["stok"].ptr, b["off"].ptr, b["te"].ptr,
                                            b["tr"].ptr, b["tc"].ptr, g["max_tiles"], pairs, gu_out.ptr, qwhip.F16, 0))
     qwhip.check(lib.qwhip_swiglu_fwht(st, gu_out.ptr, qwhip.F16, act.ptr, pairs, inter, 1))
     qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vdn), experts, act.ptr, qwhip.F16, 0, None, b["off"].ptr, b["te"].ptr,
@@ -200,19 +212,22 @@ def test_moe_prefill_chain_matches_oracle(dev, t, experts, hidden, inter, k):
     qwhip.check(lib.qwhip_moe_combine(st, dn_out.ptr, qwhip.F32, b["inv"].ptr, wb.ptr, t, k, hidden, None, None, out.ptr, qwhip.F32))
     dev.stream.sync()
     got = out.download(np.float32, (t, hidden))
-    ref = qo.moe_forward_f64(x16, idx, wts, gu16, dn16, act_f16=True, rotate_act=True)
+    ref = qo.moe_forward_f64(xval, idx, wts, gu16, dn16, act_f16=True, rotate_act=True)
     assert qo.normalized_error(got, ref) <= TOL
+    assert np.allclose(qo.moe_forward_grouped_f64(xval, idx, wts, gu16, dn16, act_f16=True, rotate_act=True), ref, rtol=1e-3, atol=1e-5)
 
 
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g32", "hq4_g64", "hq8_g32", "aq2_g64", "hq3_g32", "hq6_g32"])
 @pytest.mark.parametrize("t,experts,hidden,inter,k,rot", [(40, 8, 256, 128, 2, 1), (130, 16, 512, 192, 4, 1), (300, 4, 128, 64, 2, 0),
                                                           (64, 8, 192, 448, 3, 1)])
-def test_fused_gate_up_swiglu_equals_the_two_step_chain(dev, fmt, t, experts, hidden, inter, k, rot):
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+def test_fused_gate_up_swiglu_equals_the_two_step_chain(dev, fmt, t, experts, hidden, inter, k, rot, xdt):
     """qwhip_moe_grouped_gemm_swiglu == qwhip_moe_grouped_gemm (f16 out) + qwhip_swiglu_fwht, bit for bit, on the rows of the
-    sorted list (intermediate sizes with a partial 128-column tile included), and the chain built on it meets the oracle."""
+    sorted list (intermediate sizes with a partial 128-column tile included), and the chain built on it meets the oracle;
+    f16 and bf16 hidden rows on every container."""
     gu_blocks, gu16, dn_blocks, dn16 = _moe_banks(experts, hidden, inter, seed=13, fmt=fmt)
     rng = np.random.default_rng(9)
-    x16 = rng.standard_normal((t, hidden)).astype(np.float16)
+    x16, xcode, xval = _hidden_rows(rng, t, hidden, xdt)
     logits = rng.standard_normal((t, experts)).astype(np.float32)
     idx, wts = _route(dev, logits, k)
     g = _group(dev, idx, experts, k)
@@ -222,10 +237,10 @@ def test_fused_gate_up_swiglu_equals_the_two_step_chain(dev, fmt, t, experts, hi
     gu_out = dev.alloc(pairs * 2 * inter * 2)
     act2, act1 = dev.put(np.zeros((pairs, inter), np.float16)), dev.put(np.zeros((pairs, inter), np.float16))
     vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
-    qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, b["stok"].ptr, b["off"].ptr, b["te"].ptr,
+    qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vgu), experts, xb.ptr, xcode, 0, b["stok"].ptr, b["off"].ptr, b["te"].ptr,
                                            b["tr"].ptr, b["tc"].ptr, g["max_tiles"], pairs, gu_out.ptr, qwhip.F16, 0))
     qwhip.check(lib.qwhip_swiglu_fwht(st, gu_out.ptr, qwhip.F16, act2.ptr, pairs, inter, rot))
-    qwhip.check(lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(vgu), experts, xb.ptr, qwhip.F16, 0, b["stok"].ptr, b["off"].ptr,
+    qwhip.check(lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(vgu), experts, xb.ptr, xcode, 0, b["stok"].ptr, b["off"].ptr,
                                                   b["te"].ptr, b["tr"].ptr, b["tc"].ptr, g["max_tiles"], pairs, rot, act1.ptr, 0))
     dev.stream.sync()
     valid = int(g["off"][experts])
@@ -233,7 +248,7 @@ def test_fused_gate_up_swiglu_equals_the_two_step_chain(dev, fmt, t, experts, hi
     assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
     # against the oracle: act of sorted slot p = swiglu(x[tok] . gate_e, x[tok] . up_e), rotated
     e_of = np.repeat(np.arange(experts), np.diff(g["off"]))
-    xs = x16[g["stok"][:valid]].astype(np.float64)
+    xs = xval[g["stok"][:valid]].astype(np.float64)
     gu = np.einsum("pk,pnk->pn", xs, gu16[e_of].astype(np.float64)).astype(np.float16).astype(np.float32)
     want = qo.swiglu_fwht_f16(gu[:, :inter], gu[:, inter:], rotate=bool(rot)).astype(np.float32)
     assert qo.normalized_error(one.astype(np.float32), want) <= TOL
@@ -248,7 +263,8 @@ def test_fused_gate_up_swiglu_refusals(dev):
     args = (z.ptr, z.ptr, z.ptr, z.ptr, 4, 4, 1, act.ptr, 0)
     assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v), 4, xb.ptr, qwhip.F16, 0, None, *args) == qwhip.E_BAD_GEOMETRY   # inter = 48
     v2 = H.view_of(dev, bank, "hq4_g32_m5", 4 * 2 * 48, 64)
-    assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v2), 3, xb.ptr, qwhip.BF16, 0, None, *args) == qwhip.E_BAD_SHAPE     # bf16 activations
+    assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v2), 3, xb.ptr, qwhip.F32, 0, None, *args) == qwhip.E_BAD_WEIGHTS   # f32 activations
+    assert lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(v2), 5, xb.ptr, qwhip.BF16, 0, None, *args) == qwhip.E_BAD_SHAPE    # 384 rows over 5 experts
 
 
 def test_grouped_gemm_refuses_expert_of_4gib(dev):
@@ -361,13 +377,24 @@ def test_swiglu_fwht_matches_oracle(dev):
 
 @pytest.mark.parametrize("t", [1, 2048])
 def test_moe_full_size_operator(t):
-    """C4 at its real shape (128 experts, top-8, hidden 2048, intermediate 768): device-quantized banks byte-checked
-    against the oracle on expert 0, routing identical, sampled tokens against the fp64 oracle."""
+    """C4 at its real shape (128 experts, top-8, hidden 2048, intermediate 768, bf16 hidden rows): device-quantized banks
+    byte-checked against the oracle on expert 0, routing identical, EVERY token against the fp64 oracle (prefill: the
+    oracle's expert-ordered form, which makes the 155 GFLOP of fp64 products a matter of seconds)."""
     import argparse
 
     import bench
     out = bench.run_moe(argparse.Namespace(steps=2, warmup=1, no_cpu=True), t, "full-size parity")
-    assert out["normalized_error"] <= TOL
+    assert out["normalized_error"] <= TOL and out["tokens_checked"] == t and out["config"]["activations"] == "bf16"
+    assert out["worst_token_error"] <= TOL
+
+
+def test_moe_full_size_operator_f16_rows():
+    """The same prefill batch on f16 hidden rows (the reference's own activation type), every token."""
+    import argparse
+
+    import bench
+    out = bench.run_moe(argparse.Namespace(steps=2, warmup=1, no_cpu=True, moe_f16=True), 2048, "full-size parity, f16 rows")
+    assert out["normalized_error"] <= TOL and out["tokens_checked"] == 2048 and out["config"]["activations"] == "f16"
 
 
 @pytest.mark.parametrize("hidden", [256, 1000])

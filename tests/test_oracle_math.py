@@ -447,6 +447,33 @@ def test_route_modes_closed_forms():
     assert 3 not in idx6[0].tolist() and 5 not in idx6[0].tolist() and (idx6[0] == -1).sum() == 2
 
 
+def test_grouped_moe_forward_equals_the_per_token_form():
+    """moe_forward_grouped_f64 (work ordered by expert, matrix products) against moe_forward_f64 (the golden-pinned per-token
+    loop): empty routes, ids with flag bits above bit 15, an expert nobody routes to, f16 hand-over with and without the
+    rotation.  Without the f16 rounding of the activation the two agree to fp64 summation order; with it, a value that sits
+    on an f16 rounding boundary may round the other way, hence the looser bar there."""
+    rng = np.random.default_rng(77)
+    t, e, k, h, inter = 37, 9, 3, 64, 96
+    x = rng.standard_normal((t, h)).astype(np.float16)
+    gu = (rng.standard_normal((e, 2 * inter, h)) * 0.2).astype(np.float16)
+    dn = (rng.standard_normal((e, h, inter)) * 0.2).astype(np.float16)
+    idx = np.stack([rng.permutation(e - 1)[:k] for _ in range(t)]).astype(np.int32)     # expert e - 1 is never routed
+    idx[2, 1] = -1
+    idx[5] = -1
+    idx[7, 0] |= 3 << 16
+    wts = rng.random((t, k)).astype(np.float32)
+    a = qo.moe_forward_grouped_f64(x, idx, wts, gu, dn, act_f16=False, rotate_act=False)
+    b = qo.moe_forward_f64(x, idx, wts, gu, dn, act_f16=False, rotate_act=False)
+    np.testing.assert_allclose(a, b, rtol=1e-12, atol=1e-12)
+    assert np.all(a[5] == 0)
+    for rot in (False, True):
+        a = qo.moe_forward_grouped_f64(x, idx, wts, gu, dn, act_f16=True, rotate_act=rot)
+        b = qo.moe_forward_f64(x, idx, wts, gu, dn, act_f16=True, rotate_act=rot)
+        assert qo.normalized_error(a, b) <= 1e-6
+    none = qo.moe_forward_grouped_f64(x[:2], np.full((2, k), -1, np.int32), wts[:2], gu, dn, True, True)
+    assert none.shape == (2, h) and np.all(none == 0)
+
+
 def test_group_latent_block_identities():
     """moe_group_latent_forward_f64: (1) one group with identity D and U is the plain routed block; (2) without the f16
     hand-over roundings the grouped sum equals the per-route expansion sum_k w_k U_g(k) down_k(swiglu(gu_k(D_g(k) x)))
