@@ -153,6 +153,24 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None, cpu_later=None):
     e1.record(dev.stream)
     dev.stream.sync()
     read_us = e0.elapsed_ms(e1) * 1e3 / args.steps
+    rows_us = None
+    if fmt == "hq4_g32_m5" and m == 1:
+        # the second yardstick: the decode GEMV's own launch (grid, 20-byte pieces per lane, rows in flight) with the
+        # arithmetic taken out
+        row_bytes = (k // 32) * 20
+        qwhip.check(lib.qwhip_fill_u32(st, sum_dev.ptr, 0, 512))
+        qwhip.check(lib.qwhip_plane_checksum_rows(st, banks[0].ptr, n, row_bytes, sum_dev.ptr))
+        dev.stream.sync()
+        if int(sum_dev.download(np.uint64, (256,)).sum()) != int(blocks.ravel().view(np.uint32).astype(np.uint64).sum()):
+            _fail("bench: row checksum differs from the host's")
+        for i in range(args.warmup):
+            lib.qwhip_plane_checksum_rows(st, banks[i % ring_n].ptr, n, row_bytes, sum_dev.ptr)
+        e0.record(dev.stream)
+        for i in range(args.steps):
+            lib.qwhip_plane_checksum_rows(st, banks[i % ring_n].ptr, n, row_bytes, sum_dev.ptr)
+        e1.record(dev.stream)
+        dev.stream.sync()
+        rows_us = e0.elapsed_ms(e1) * 1e3 / args.steps
     out = {
         "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -164,7 +182,9 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None, cpu_later=None):
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": traffic if (args.variant == 0 and args.rt == 0 and not args.prerot) else None,
                      "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3),
-                     "read_only_launch_us": round(read_us, 3), "read_only_frac": round(bank_bytes / (read_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
+                     "read_only_launch_us": round(read_us, 3), "read_only_frac": round(bank_bytes / (read_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                     "read_only_rows_launch_us": None if rows_us is None else round(rows_us, 3),
+                     "read_only_rows_frac": None if rows_us is None else round(bank_bytes / (rows_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
         "normalized_error": err, "wall_ms_per_step": round(wall * 1e3 / args.steps, 6),
     }
     if not args.no_cpu:

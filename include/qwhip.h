@@ -113,6 +113,11 @@ qwhip_status qwhip_fill_u32(qwhip_stream_t s, void* dst, uint32_t value, size_t 
  * counterpart in the reference: it is how a loader checks an uploaded plane against the host copy without reading it
  * back, and - a launch that only reads - the read-bandwidth yardstick bench.py quotes beside the decode GEMV. */
 qwhip_status qwhip_plane_checksum(qwhip_stream_t s, const void* plane, size_t bytes, uint64_t* sum);
+/* The same word sum over a bank of `rows` rows of `row_bytes` bytes (whole 20-byte pieces, 4-byte aligned, under 4 GiB),
+ * read the way the m = 1 HQ4_G32_M5 decode GEMV reads it: its grid, its 20-byte pieces per lane, its window of rows in
+ * flight, the arithmetic taken out.  No counterpart in the reference: it is the second yardstick bench.py quotes beside the
+ * decode GEMV (what the GEMV's own request pattern costs when nothing is computed). */
+qwhip_status qwhip_plane_checksum_rows(qwhip_stream_t s, const void* plane, uint32_t rows, uint32_t row_bytes, uint64_t* sum);
 /* GPU timestamps (QWStageCounter, Sources/Foundation/QWHAL/QWStageCounter.swift:1-40). */
 qwhip_status qwhip_event_create(qwhip_device_t dev, qwhip_event_t* out);
 qwhip_status qwhip_event_destroy(qwhip_event_t e);
@@ -181,7 +186,8 @@ qwhip_status qwhip_dequant_f16(qwhip_stream_t s, const qwhip_weight_view* w, voi
  * flags: QWHIP_X_PREROTATED; bits 8..11 pick one kernel for tuning and tests (0 = automatic, 1 = half-wave dot2,
  * 2 = MFMA streamer, 3 = DMA streamer, 4 = column-stationary HQ4 kernel, 5 = column-stationary MFMA kernel,
  * 6 = column-stationary dot2 kernel, 7 = 4x4x4-block MFMA kernel, 8 = transposing MFMA kernel, 9 = split-K MFMA kernel; a
- * kernel that does not take the shape returns QWHIP_E_BAD_GEOMETRY); bits 12..15 its tuning code (bits 12..18 for the
+ * kernel that does not take the shape returns QWHIP_E_BAD_GEOMETRY); bits 12..15 its tuning code (bits 12..17 for the
+ * column-stationary HQ4 kernel: window form, grid scale, row sets; bits 12..18 for the
  * split-K kernel).  The split-K kernel (automatic for 4-bit banks with k >= 8192 and m >= 6) keeps its partial sums in
  * the stream's scratch: calls on one stream are ordered; calls on different streams do not share it. */
 qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,

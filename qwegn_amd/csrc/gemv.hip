@@ -1098,7 +1098,7 @@ static qwhip_status qw_gemv_impl(qwhip_stream_t s, const qwhip_weight_view* w, c
         hipError_t e = hipSuccess;
         unsigned long long* keys = token && s->scratch ? (unsigned long long*)s->scratch : nullptr;   // the stream's counter area
         if (fmt == QW_FMT_M5 && m == 1 &&
-            qw_col_gemv(s->stream, w, x, x_dtype, rotate, y16, y32, (flags >> 12) & 0x7Fu, &e, keys, QWHIP_STREAM_COUNTER_BYTES / 8u, token, folded)) {
+            qw_col_gemv(s->stream, w, x, x_dtype, rotate, y16, y32, (flags >> 12) & 0xFFFu, &e, keys, QWHIP_STREAM_COUNTER_BYTES / 8u, token, folded)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }

@@ -198,17 +198,25 @@ static __device__ __forceinline__ void run(const P& pp) {
 }
 };
 
-// The same kernel with the block loads issued and awaited by hand.  A compiled rolling window drains once per trip: the
-// register allocator reuses a load's destination as a temporary, copies the value out at the loop's ends, and every copy
-// waits for its load, so a wave has at most D rows in flight right after a trip's start and none at its end (the loop is
-// one memory round trip per D rows per wave).  Here the loads are `asm volatile` statements whose destination registers
-// are tied in and out ("+v": the same registers all the way round the loop), and each row is consumed behind an
+// The same kernel with the block loads issued and awaited by hand, and with less vector work per row.
+// A compiled rolling window drains once per trip: the register allocator reuses a load's destination as a temporary,
+// copies the value out at the loop's ends, and every copy waits for its load, so a wave has at most D rows in flight right
+// after a trip's start and none at its end.  Here the loads are `asm volatile` statements whose destination registers are
+// tied in and out ("+v": the same registers all the way round the loop), and each row is consumed behind an
 // s_waitcnt vmcnt(2 (D - 1)): exactly the two loads of the oldest row have to have landed, the D - 1 younger rows stay in
-// flight.  Loads stop with the set's last row (the compiled form re-reads it D times) and the last D rows are consumed
-// behind waits that count down.  The activation loads are issued by hand as well: the compiler does not know of the block
-// loads behind them and would wait for everything (vmcnt(0)) before the rotation.
-// Launch contract: trip count ceil(rows per workgroup / SETS) >= 2 D (the host checks).
-template <int XDT, int SETS, int D>
+// flight.  The activation loads are issued by hand as well: the compiler does not know of the block loads behind them and
+// would wait for everything (vmcnt(0)) before the rotation.
+// Rows are consumed in groups of D, slot j of a group after slot j - 1.  The first group is padded at its head with `pad`
+// dummies (row 0 fetched once more, its arithmetic skipped by a scalar branch) so that the last group is whole and every
+// slot index is a constant - a slot picked at run time makes the compiler copy registers whose loads are still in flight.
+// Vector work per row (the SIMDs are nearly as busy as the memory system: a workgroup's waves do not spread evenly over the
+// four SIMDs of a compute unit, and the fullest SIMD sets the pace): the row's address is a scalar base that moves by one
+// row stride per issue plus a lane offset that never changes; the first product of each sum does not accumulate (no
+// register to clear); the sums run at 2^-24 of their value so that the scale is used as the f16 it is loaded as
+// (v' = s q + ((1024 s + b) S 2^-24): the same roundings as fma(s 2^24, q, (1024 s + b) S), a power of two apart) and the
+// factor comes back once per row in the epilogue; lanes past the row's last block multiply zeros instead of being
+// masked; the partial sums of all rows, the one a short set does not have included, go to LDS unconditionally.
+template <int XDT, int SETS, int D, int D0 = D>
 struct qw_gemv_colw_kernel {
 static constexpr int kLaunchBound = 1024;
 template <int N>
@@ -221,6 +229,11 @@ static __device__ __forceinline__ void static_for(F&& f) {
         f(std::integral_constant<int, U>{});
         static_for<U + 1>(f);
     }
+}
+static __device__ __forceinline__ float dot2_first(uint32_t a, h2_t b) {
+    float d;
+    asm("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
 }
 static __device__ __forceinline__ void run(const qc_params& p) {
     constexpr int XT = SETS == 1 ? 5 : (SETS == 2 ? 2 : 1);
@@ -241,12 +254,17 @@ static __device__ __forceinline__ void run(const qc_params& p) {
     const uint32_t G = gridDim.x;
     if (blockIdx.x >= N) return;
     const uint32_t nrows = (N - blockIdx.x + G - 1u) / G;
-    const uint32_t nmax = (nrows + SETS - 1u) / SETS;
+    const uint32_t nmax = (nrows + SETS - 1u) / SETS;        // rows of the fullest set: the trip count, workgroup-uniform
+    const uint32_t ngroups = (nmax + D - 1u) / D;
+    const uint32_t pad = ngroups * D - nmax;                 // dummies at the head of the first group, 0 .. D - 1
     const uint32_t row_bytes = nb * 20u;
-    const uint32_t step = G * SETS * row_bytes;
+    const uint32_t step = G * SETS * row_bytes;              // bytes between consecutive rows of one set
     const uint32_t mine = nrows > set ? (nrows - set + SETS - 1u) / SETS : 0u;
-    uint32_t off = ((mine ? set : 0u) * G + blockIdx.x) * row_bytes + g * 20u;
-    const uint32_t off_max = off + (mine ? mine - 1u : 0u) * step;   // a set one row short re-reads its last row once
+    // lane offset inside a row band (added, unsigned, to the band's scalar base: it can never step back a band); a set
+    // without rows walks set 0's, and a set one row short reads set 0's last row where it has none (set 0 is never short)
+    const uint32_t voff0 = blockIdx.x * row_bytes + g * 20u;
+    const uint32_t voff = mine ? set * G * row_bytes + voff0 : voff0;
+    const uint32_t voff_last = mine < nmax ? voff0 : voff;
 
     // 1. activation loads, by hand
     u4_t xraw[XT];
@@ -265,16 +283,24 @@ static __device__ __forceinline__ void run(const qc_params& p) {
         hdr[j] = 0u;
         qv[j] = u4_t{0u, 0u, 0u, 0u};
     }
+    const uint8_t* rowp = p.bank;                 // scalar: the band of the row the next issue fetches
+    int32_t krow = -(int32_t)pad;                 // its index; the dummies (< 0) fetch row 0
+    const int32_t klast = (int32_t)nmax - 1;
     auto issue = [&](int slot) {
+        // the set's last row always lands in slot D - 1
+        const uint32_t vo = (slot == D - 1 && krow == klast) ? voff_last : voff;
         asm volatile("global_load_dword %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:4"
-                     : "+v"(hdr[slot]), "+v"(qv[slot]) : "v"(off), "s"(p.bank) : "memory");
-        off = min(off + step, off_max);
+                     : "+v"(hdr[slot]), "+v"(qv[slot]) : "v"(vo), "s"(rowp) : "memory");
+        rowp += krow >= 0 ? step : 0u;
+        ++krow;
     };
+    // D0 of the window's D rows go out ahead of the activation prologue, the rest behind it: every load queued here
+    // delays the activation loads of the waves that start later on the same compute unit
 #pragma unroll
-    for (int j = 0; j < D; ++j) issue(j);
-    // 3. rotation on the matrix cores into the shared image: the XT activation loads have landed, the 2 D block loads fly on
+    for (int j = 0; j < D0; ++j) issue(j);
+    // 3. rotation on the matrix cores into the shared image: the XT activation loads have landed, the 2 D0 block loads fly on
 #pragma unroll
-    for (int t = 0; t < XT; ++t) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xraw[t]) : "n"(2 * D));
+    for (int t = 0; t < XT; ++t) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xraw[t]) : "n"(2 * D0));
     {
         h8_t h_lo, h_hi;
         qw_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
@@ -285,12 +311,13 @@ static __device__ __forceinline__ void run(const qc_params& p) {
         }
     }
     __syncthreads();
-    // 4. this lane's column: 16 operand pairs and the group sum S
+    // 4. this lane's column: 16 operand pairs and the group sum S (zeros past the row's last block)
     h2_t xo[16];
-    float S;
+    float Sp;
     {
         const h8_t* src = xs + g * 5;
         const h2_t one = {(h1_t)1.0f, (h1_t)1.0f};
+        const h2_t zero = {(h1_t)0.0f, (h1_t)0.0f};
         float s0 = 0.f, s1 = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -300,74 +327,148 @@ static __device__ __forceinline__ void run(const qc_params& p) {
                 const h2_t pr = {v[2 * e2], v[2 * e2 + 1]};
                 if (e2 & 1) s1 = __builtin_amdgcn_fdot2(pr, one, s1, false);
                 else s0 = __builtin_amdgcn_fdot2(pr, one, s0, false);
-                xo[4 * j + e2] = pr;
+                xo[4 * j + e2] = gvalid ? pr : zero;
             }
         }
-        S = s0 + s1;
+        Sp = gvalid ? (s0 + s1) * 5.9604644775390625e-08f : 0.0f;     // S 2^-24
     }
 
-    uint32_t rslot = set;
+    // partial sums: row slot r of the workgroup at part[r cpr + chunk]
+    uint32_t part_at = (uint32_t)(uintptr_t)part + ((set * cpr + chunk) << 2);
+    const uint32_t part_step = (SETS * cpr) << 2;
     auto consume = [&](int slot) {
-        const uint32_t h = hdr[slot];
-        float lo0 = 0.f, lo1 = 0.f, hi0 = 0.f, hi1 = 0.f;
-#pragma unroll
-        for (int w4 = 0; w4 < 4; ++w4) {
-            const uint32_t w = qv[slot][w4], w8 = w >> 8;
-            const uint32_t m0 = w & 0x000F000Fu, m1 = w & 0x00F000F0u, m2 = w8 & 0x000F000Fu, m3 = w8 & 0x00F000F0u;
-            lo0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m0), xo[4 * w4 + 0], lo0, false);
-            hi0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m1), xo[4 * w4 + 1], hi0, false);
-            lo1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m2), xo[4 * w4 + 2], lo1, false);
-            hi1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, m3), xo[4 * w4 + 3], hi1, false);
-        }
-        const h2_t hd = __builtin_bit_cast(h2_t, h);
+        const uint32_t w0 = qv[slot][0], w1 = qv[slot][1], w2 = qv[slot][2], w3 = qv[slot][3];
+        float lo = dot2_first(w0 & 0x000F000Fu, xo[0]);
+        float hi = dot2_first(w0 & 0x00F000F0u, xo[1]);
+        lo = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, (w0 >> 8) & 0x000F000Fu), xo[2], lo, false);
+        hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, (w0 >> 8) & 0x00F000F0u), xo[3], hi, false);
+#define QCW_WORD(W, B)                                                                                        \
+        lo = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, W & 0x000F000Fu), xo[B + 0], lo, false);         \
+        hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, W & 0x00F000F0u), xo[B + 1], hi, false);         \
+        lo = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, (W >> 8) & 0x000F000Fu), xo[B + 2], lo, false);  \
+        hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, (W >> 8) & 0x00F000F0u), xo[B + 3], hi, false);
+        QCW_WORD(w1, 4)
+        QCW_WORD(w2, 8)
+        QCW_WORD(w3, 12)
+#undef QCW_WORD
+        const h2_t hd = __builtin_bit_cast(h2_t, hdr[slot]);
         const float sc = (float)hd[0];
-        const float q = __builtin_fmaf(hi0 + hi1, 0.0625f, lo0 + lo1);
-        float v = __builtin_fmaf(sc * 16777216.0f, q, __builtin_fmaf(sc, 1024.0f, (float)hd[1]) * S);
-        v = gvalid ? v : 0.0f;
+        const float m = __builtin_fmaf(sc, 1024.0f, (float)hd[1]) * Sp;   // the header sum is exact in fp32
+        const float q = __builtin_fmaf(hi, 0.0625f, lo);
+        float v = __builtin_fmaf(sc, q, m);
         v = qw_reduce32_dpp(v);
-        if (lane == 31u && rslot < nrows) part[rslot * cpr + chunk] = v;
-        rslot += SETS;
+        if (lane == 31u) *(__attribute__((address_space(3))) float*)(uintptr_t)part_at = v;
+        part_at += part_step;
     };
-    // steady state: every consumed row is replaced
-    uint32_t i = 0;
-    for (; i + 2u * D <= nmax; i += D) {
+#pragma unroll
+    for (int j = D0; j < D; ++j) issue(j);
+    int32_t kcons = -(int32_t)pad;                // scalar: the row being consumed; a dummy's arithmetic is skipped
+    for (uint32_t grp = 0; grp + 1u < ngroups; ++grp) {
 #pragma unroll
         for (int j = 0; j < D; ++j) {
             wait_row<2 * (D - 1)>(hdr[j], qv[j]);
+            if (kcons >= 0) consume(j);
+            ++kcons;
+            issue(j);
+        }
+    }
+    static_for<0>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        wait_row<2 * (D - 1 - u)>(hdr[u], qv[u]);
+        if (kcons >= 0) consume(u);
+        ++kcons;
+    });
+    __syncthreads();
+    // 5. fixed-order sum of the chunk partials of each row, back at full scale
+    for (uint32_t s = tid; s < nrows; s += threads) {
+        float v = 0.f;
+        for (uint32_t c = 0; c < cpr; ++c) v += part[s * cpr + c];
+        v *= 16777216.0f;
+        const uint32_t row = s * G + blockIdx.x;
+        if (p.y32) p.y32[row] = v;
+        if (p.y16) p.y16[row] = (h1_t)v;
+    }
+}
+};
+
+// The hand-issued window with the arithmetic taken out: every lane adds up the 32-bit words of the 20-byte pieces it
+// fetches (the rows, the grid, the pieces and the window of qw_gemv_colw_kernel<.., 3, 3>) and a workgroup adds its total into
+// sum[blockIdx.x & 255].  What this launch takes over a bank is what the decode GEMV's own request pattern costs.
+#define QCS_FIELDS(X) X(const uint8_t*, bank) X(unsigned long long*, sum) X(uint32_t, N) X(uint32_t, nb) X(uint32_t, cpr)
+QW_ARG_BLOCK(qcs_params, QCS_FIELDS)
+template <int SETS>
+struct qw_rows_checksum_kernel {
+static constexpr int kLaunchBound = 1024;
+static constexpr int D = 3;
+static __device__ __forceinline__ void run(const qcs_params& p) {
+    __shared__ unsigned long long wsum[16];
+    const uint32_t nb = p.nb, cpr = p.cpr, N = p.N;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 31u, hw = tid >> 5;
+    const uint32_t set = hw / cpr, chunk = hw - set * cpr;
+    const uint32_t g0 = chunk * 32u + lane;
+    const bool gvalid = g0 < nb;
+    const uint32_t g = gvalid ? g0 : nb - 1u;
+    const uint32_t G = gridDim.x;
+    if (blockIdx.x >= N) return;
+    const uint32_t nrows = (N - blockIdx.x + G - 1u) / G;
+    const uint32_t nmax = (nrows + SETS - 1u) / SETS;
+    const uint32_t ngroups = (nmax + D - 1u) / D;
+    const uint32_t pad = ngroups * D - nmax;
+    const uint32_t row_bytes = nb * 20u;
+    const uint32_t step = G * SETS * row_bytes;
+    const uint32_t mine = nrows > set ? (nrows - set + SETS - 1u) / SETS : 0u;
+    const uint32_t voff0 = blockIdx.x * row_bytes + g * 20u;
+    const uint32_t voff = mine ? set * G * row_bytes + voff0 : voff0;
+    const uint32_t voff_last = mine < nmax ? voff0 : voff;
+    uint32_t hdr[D];
+    u4_t qv[D];
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        hdr[j] = 0u;
+        qv[j] = u4_t{0u, 0u, 0u, 0u};
+    }
+    const uint8_t* rowp = p.bank;
+    int32_t krow = -(int32_t)pad;
+    const int32_t klast = (int32_t)nmax - 1;
+    auto issue = [&](int slot) {
+        const uint32_t vo = (slot == D - 1 && krow == klast) ? voff_last : voff;
+        asm volatile("global_load_dword %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:4"
+                     : "+v"(hdr[slot]), "+v"(qv[slot]) : "v"(vo), "s"(rowp) : "memory");
+        rowp += krow >= 0 ? step : 0u;
+        ++krow;
+    };
+#pragma unroll
+    for (int j = 0; j < D; ++j) issue(j);
+    unsigned long long acc = 0ull;
+    int32_t kcons = -(int32_t)pad;
+    auto consume = [&](int slot) {      // a row of this lane's own set only (a short set's last fetch is set 0's row)
+        if (kcons >= 0 && gvalid && (uint32_t)kcons < mine)
+            acc += (unsigned long long)hdr[slot] + qv[slot][0] + qv[slot][1] + qv[slot][2] + qv[slot][3];
+        ++kcons;
+    };
+    for (uint32_t grp = 0; grp + 1u < ngroups; ++grp) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(hdr[j]), "+v"(qv[j]) : "n"(2 * (D - 1)));
             consume(j);
             issue(j);
         }
     }
-    // the last rem rows, D <= rem < 2 D: rem - D of them are still replaced, the last D are not
-    const uint32_t rem = nmax - i;
+    asm volatile("s_waitcnt vmcnt(4)" : "+v"(hdr[0]), "+v"(qv[0]));
+    consume(0);
+    asm volatile("s_waitcnt vmcnt(2)" : "+v"(hdr[1]), "+v"(qv[1]));
+    consume(1);
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(hdr[2]), "+v"(qv[2]));
+    consume(2);
 #pragma unroll
-    for (int u = 0; u < D; ++u) {
-        if ((uint32_t)u + D < rem) {
-            wait_row<2 * (D - 1)>(hdr[u], qv[u]);
-            consume(u);
-            issue(u);
-        }
-    }
-    // now exactly D rows are in flight or landed; the oldest sits in slot (rem - D) % D = rem - D
-    const uint32_t first = rem - D;
-    static_for<0>([&](auto uc) {
-        constexpr int u = decltype(uc)::value;
-#pragma unroll
-        for (int sl = 0; sl < D; ++sl) {
-            if ((first + (uint32_t)u) % D == (uint32_t)sl) {
-                wait_row<2 * (D - 1 - u)>(hdr[sl], qv[sl]);
-                consume(sl);
-            }
-        }
-    });
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if ((tid & 63u) == 0u) wsum[tid >> 6] = acc;
     __syncthreads();
-    // 5. fixed-order sum of the chunk partials of each row
-    for (uint32_t s = tid; s < nrows; s += threads) {
-        float v = 0.f;
-        for (uint32_t c = 0; c < cpr; ++c) v += part[s * cpr + c];
-        const uint32_t row = s * G + blockIdx.x;
-        if (p.y32) p.y32[row] = v;
-        if (p.y16) p.y16[row] = (h1_t)v;
+    if (tid == 0u) {
+        unsigned long long total = 0ull;
+        for (uint32_t wv = 0; wv < ((32u * cpr * SETS + 63u) >> 6); ++wv) total += wsum[wv];
+        atomicAdd(p.sum + (blockIdx.x & 255u), total);
     }
 }
 };
@@ -390,9 +491,11 @@ __global__ __launch_bounds__(256) void qw_col_keys_fin_kernel(const unsigned lon
     }
 }
 
+// kind: 0 = the hand-issued window (three rows, two of them ahead of the prologue), 1 = the compiled window (the head's
+// fold rides in its epilogue), 2..5 = other hand-issued windows for tuning
 template <int XDT, int SETS>
-hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t threads, size_t lds, uint32_t depth, unsigned long long* keys) {
-    if (keys) {   // the head: automatic prefetch only
+hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t threads, size_t lds, uint32_t kind, unsigned long long* keys) {
+    if (keys) {
         qc_params_fold pf;
 #define QC_TAKE(T, n) pf.n = p.n;
         QC_FIELDS(QC_TAKE)
@@ -401,32 +504,26 @@ hipError_t qc_launch(hipStream_t st, const qc_params& p, uint32_t wgs, uint32_t 
         qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 2, qc_params_fold>>(dim3(wgs), dim3(threads), lds, st, pf);
         return hipGetLastError();
     }
-    if (depth >= 16) {   // hand-issued window of depth - 16 + 1 rows
-        switch (depth - 16u) {
-            case 1: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 2>>(dim3(wgs), dim3(threads), lds, st, p); break;
-            case 2: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 3>>(dim3(wgs), dim3(threads), lds, st, p); break;
-            case 3: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 4>>(dim3(wgs), dim3(threads), lds, st, p); break;
-            case 4: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 5>>(dim3(wgs), dim3(threads), lds, st, p); break;
-            case 5: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 6>>(dim3(wgs), dim3(threads), lds, st, p); break;
-            default: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 8>>(dim3(wgs), dim3(threads), lds, st, p); break;
-        }
-        return hipGetLastError();
+    switch (kind) {
+        case 1: qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 2>>(dim3(wgs), dim3(threads), lds, st, p); break;
+        case 2: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 2, 2>>(dim3(wgs), dim3(threads), lds, st, p); break;
+        case 3: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 3, 3>>(dim3(wgs), dim3(threads), lds, st, p); break;
+        case 4: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 4, 2>>(dim3(wgs), dim3(threads), lds, st, p); break;
+        case 5: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 6, 3>>(dim3(wgs), dim3(threads), lds, st, p); break;
+        default: qw_launch_scalar<qw_gemv_colw_kernel<XDT, SETS, 3, 2>>(dim3(wgs), dim3(threads), lds, st, p); break;
     }
-    if (depth == 1) qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 1>>(dim3(wgs), dim3(threads), lds, st, p);
-    else if (depth == 3) qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 3, 3>>(dim3(wgs), dim3(threads), lds, st, p);
-    else if (depth == 4) qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 4, 4>>(dim3(wgs), dim3(threads), lds, st, p);
-    else qw_launch_scalar<qw_gemv_col_kernel<XDT, SETS, 2, 2>>(dim3(wgs), dim3(threads), lds, st, p);
     return hipGetLastError();
 }
 
 }  // namespace
 
 // Tries the column-stationary kernel for a validated m = 1 HQ4_G32_M5 call; false when the shape is outside its envelope.
-// `tune`: 0 = automatic (two rows in flight, both issued ahead of the prologue); bits 0..1 pick the prefetch
-// (1 -> two rows, one ahead of the prologue; 2 -> three rows; 3 -> four rows) and bits 2..3 scale the grid
-// (1 -> half, 2 -> double).
-// `keys` (NULL, or room for `keys_cap` entries) + `token`: the head's greedy-decoding fold rides in the epilogue and a second,
-// one-workgroup launch writes *token; a grid larger than keys_cap drops the fold (*folded = false) and the caller folds the logits.
+// `tune` (tests and tuning): bits 0..2 pick the kernel (0 = automatic: the hand-issued window of three rows, two of them
+// ahead of the prologue; 1 = the compiled window; 2..5 = hand-issued windows of (2, 2), (3, 3), (4, 2), (6, 3) rows), bits
+// 3..4 scale the grid (1 -> half, 2 -> double, 3 -> one and a half), bit 5 asks for four row sets per workgroup.
+// `keys` (NULL, or room for `keys_cap` entries) + `token`: the head's greedy-decoding fold rides in the epilogue (compiled
+// window) and a second, one-workgroup launch writes *token; a grid larger than keys_cap drops the fold (*folded = false) and
+// the caller folds the logits.
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
                  float* y32, uint32_t tune, hipError_t* err, unsigned long long* keys, uint32_t keys_cap, int32_t* token,
                  bool* folded) {
@@ -435,24 +532,28 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     if (cpr > 32u) return false;
     if ((uint64_t)w->n * nb * 20u >= (1ull << 32)) return false;   // 32-bit offsets inside the bank
     if (((uintptr_t)x & 15u) != 0) return false;
-    const uint32_t sets = cpr <= 3u ? 4u : (cpr <= 12u ? 2u : 1u);
+    uint32_t sets = cpr <= 3u ? 4u : (cpr <= 12u ? 2u : 1u);
+    if ((tune & 0x20u) && cpr <= 8u) sets = 4u;
     const uint32_t threads = 32u * cpr * sets;
     const uint32_t waves = (threads + 63u) / 64u;
-    // about 10 waves per compute unit with both prefetch rows issued ahead of the activation prologue (measured on
-    // N = 17408, K = 5120: 11.3 us, against 11.5 with 20 waves and one row ahead, 12.2 with three rows in flight and
-    // 13.5+ with 5 waves); at least four rows per set, at most 128 row slots per workgroup
-    uint32_t wgs = (256u * 10u + waves / 2u) / waves;
-    if ((tune >> 2 & 3u) == 1u) wgs /= 2u;
-    if ((tune >> 2 & 3u) == 2u) wgs *= 2u;
+    const uint32_t kind = keys ? 1u : (tune & 7u);
+    static const uint32_t kWindow[6] = {3u, 0u, 2u, 3u, 4u, 6u};
+    const uint32_t wdepth = kWindow[kind <= 5u ? kind : 0u];       // 0: the compiled window
+    // Waves per compute unit, measured on N = 17408, K = 5120.  Compiled window: 10 (11.2-11.3 us; 11.5 with 20, 13.5+ with
+    // 5).  Hand-issued window: 20 (10.8-10.9 us on 1024 workgroups; 11.4 on 512 with the same window, 11.1 on 768; deeper
+    // windows 11.1-11.9, a window of two 11.3).  At least four rows per set, at most 128 row slots per workgroup.
+    uint32_t wgs = (256u * (wdepth ? 20u : 10u) + waves / 2u) / waves;
+    if ((tune >> 3 & 3u) == 1u) wgs /= 2u;
+    if ((tune >> 3 & 3u) == 2u) wgs *= 2u;
+    if ((tune >> 3 & 3u) == 3u) wgs += wgs / 2u;
     wgs = min(wgs, max(1u, w->n / (sets * 4u)));
     wgs = max(wgs, qwhip_cdiv(w->n, 128u));
     const uint32_t rows_per_wg = qwhip_cdiv(w->n, wgs);
-    const size_t lds = (size_t)nb * 80u + (size_t)rows_per_wg * cpr * 4u;
+    // partial sums: one float per (row slot, chunk); the hand-issued window rounds the trip count up to whole groups and
+    // stores every row slot of every group
+    const size_t part_rows = wdepth ? (size_t)qwhip_cdiv(qwhip_cdiv(rows_per_wg, sets), wdepth) * wdepth * sets : rows_per_wg;
+    const size_t lds = (size_t)nb * 80u + part_rows * cpr * 4u;
     if (lds > 60u * 1024u) return false;
-    uint32_t depth = (tune & 3u) == 1u ? 1u : ((tune & 3u) ? (tune & 3u) + 1u : 2u);
-    const uint32_t wcode = (tune >> 4) & 7u;          // 1..5 -> window of 2..6 rows, 6, 7 -> 8 rows
-    const uint32_t wdepth = wcode == 0u ? 0u : (wcode <= 5u ? wcode + 1u : 8u);
-    if (wdepth && !keys && qwhip_cdiv(w->n / wgs, sets) >= 2u * wdepth) depth = 16u + wcode;
     qc_params p;
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
@@ -467,13 +568,13 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     if (folded) *folded = fold;
     hipError_t e;
     if (x_dtype == QWHIP_F16) {
-        e = sets == 4 ? qc_launch<QWHIP_F16, 4>(st, p, wgs, threads, lds, depth, fold_keys)
-          : sets == 2 ? qc_launch<QWHIP_F16, 2>(st, p, wgs, threads, lds, depth, fold_keys)
-                      : qc_launch<QWHIP_F16, 1>(st, p, wgs, threads, lds, depth, fold_keys);
+        e = sets == 4 ? qc_launch<QWHIP_F16, 4>(st, p, wgs, threads, lds, kind, fold_keys)
+          : sets == 2 ? qc_launch<QWHIP_F16, 2>(st, p, wgs, threads, lds, kind, fold_keys)
+                      : qc_launch<QWHIP_F16, 1>(st, p, wgs, threads, lds, kind, fold_keys);
     } else {
-        e = sets == 4 ? qc_launch<QWHIP_BF16, 4>(st, p, wgs, threads, lds, depth, fold_keys)
-          : sets == 2 ? qc_launch<QWHIP_BF16, 2>(st, p, wgs, threads, lds, depth, fold_keys)
-                      : qc_launch<QWHIP_BF16, 1>(st, p, wgs, threads, lds, depth, fold_keys);
+        e = sets == 4 ? qc_launch<QWHIP_BF16, 4>(st, p, wgs, threads, lds, kind, fold_keys)
+          : sets == 2 ? qc_launch<QWHIP_BF16, 2>(st, p, wgs, threads, lds, kind, fold_keys)
+                      : qc_launch<QWHIP_BF16, 1>(st, p, wgs, threads, lds, kind, fold_keys);
     }
     if (e == hipSuccess && fold) {
         hipLaunchKernelGGL(qw_col_keys_fin_kernel, dim3(1), dim3(256), 0, st, keys, wgs, token);
@@ -481,4 +582,32 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     }
     *err = e;
     return true;
+}
+
+// The word sum of a bank of `rows` rows of `row_bytes` bytes (whole 20-byte pieces), read with the decode GEMV's own launch:
+// see qw_rows_checksum_kernel.  Same 256 caller-cleared sums as qwhip_plane_checksum.
+extern "C" qwhip_status qwhip_plane_checksum_rows(qwhip_stream_t s, const void* plane, uint32_t rows, uint32_t row_bytes, uint64_t* sum) {
+    QWHIP_REQUIRE(s);
+    QWHIP_REQUIRE(sum);
+    if (rows == 0 || row_bytes == 0) return QWHIP_OK;
+    QWHIP_REQUIRE(plane);
+    const uint32_t nb = row_bytes / 20u, cpr = (nb + 31u) / 32u;
+    if (row_bytes % 20u != 0 || ((uintptr_t)plane & 3u) != 0 || cpr > 32u || (uint64_t)rows * row_bytes >= (1ull << 32))
+        return qwhip_fail(QWHIP_E_BAD_SHAPE, "row checksum takes rows of whole 20-byte pieces, at most 1024 of them, under 4 GiB in all; got %u rows of %u bytes", rows, row_bytes);
+    const uint32_t sets = cpr <= 3u ? 4u : (cpr <= 12u ? 2u : 1u);
+    const uint32_t threads = 32u * cpr * sets, waves = (threads + 63u) / 64u;
+    uint32_t wgs = (256u * 20u + waves / 2u) / waves;      // the decode GEMV's grid
+    wgs = min(wgs, max(1u, rows / (sets * 4u)));
+    wgs = max(wgs, qwhip_cdiv(rows, 128u));
+    qcs_params p;
+    p.bank = (const uint8_t*)plane;
+    p.sum = (unsigned long long*)sum;
+    p.N = rows;
+    p.nb = nb;
+    p.cpr = cpr;
+    if (sets == 4) qw_launch_scalar<qw_rows_checksum_kernel<4>>(dim3(wgs), dim3(threads), 0, s->stream, p);
+    else if (sets == 2) qw_launch_scalar<qw_rows_checksum_kernel<2>>(dim3(wgs), dim3(threads), 0, s->stream, p);
+    else qw_launch_scalar<qw_rows_checksum_kernel<1>>(dim3(wgs), dim3(threads), 0, s->stream, p);
+    QWHIP_TRY_HIP(hipGetLastError());
+    return QWHIP_OK;
 }

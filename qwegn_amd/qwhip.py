@@ -58,6 +58,7 @@ SIGNATURES = {
     "qwhip_memcpy_d2d": (C.c_int32, [_P, _P, _P, C.c_size_t]),
     "qwhip_fill_u32": (C.c_int32, [_P, _P, _U32, C.c_size_t]),
     "qwhip_plane_checksum": (C.c_int32, [_P, _P, C.c_size_t, _P]),
+    "qwhip_plane_checksum_rows": (C.c_int32, [_P, _P, C.c_uint32, C.c_uint32, _P]),
     "qwhip_event_create": (C.c_int32, [_P, C.POINTER(_P)]),
     "qwhip_event_destroy": (C.c_int32, [_P]),
     "qwhip_event_record": (C.c_int32, [_P, _P]),

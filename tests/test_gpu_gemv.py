@@ -450,6 +450,23 @@ def test_gemv_hq4_column_stationary_row_lengths(dev, variant, prerot, k):
     assert qo.normalized_error(g16, ref) <= TOL
 
 
+@pytest.mark.parametrize("tune", [0, 1, 2, 3, 4, 5, 0 | (1 << 3), 0 | (2 << 3), 4 | (3 << 3), 0 | (1 << 5), 5 | (1 << 5) | (2 << 3)])
+@pytest.mark.parametrize("n,k,xdtype", [(17408, 5120, "f16"), (300, 5120, "bf16"), (1031, 4096, "f16"), (45, 8192, "f16"), (7, 1024, "f16"),
+                                        (513, 17408, "f16"), (2050, 3104, "bf16")])
+def test_gemv_hq4_column_stationary_windows(dev, tune, n, k, xdtype):
+    """Every form of the m = 1 HQ4_G32_M5 column-stationary kernel (override 4, tuning codes: the hand-issued windows of
+    (3, 2), (2, 2), (3, 3), (4, 2), (6, 3) rows, the compiled window, half / double / one-and-a-half grids, four row sets)
+    on row counts that leave ragged row slots, short sets (a set one row short re-reads), fewer rows than a window, a
+    partly filled last chunk (k = 3104) and a workgroup that ends in a half wave (k = 17408).  The hand-issued forms sum a
+    row's blocks in the same order with the same roundings: equal bits, whatever the window and the grid (the compiled
+    window keeps four partial sums per block where they keep two, so it agrees to rounding only)."""
+    g16, g32, ref = _run_gemv(dev, "hq4_g32_m5", n, k, 1, prerot=False, xdtype=xdtype, variant=4, rt=tune, outliers=True, seed=5)
+    assert qo.normalized_error(g32, ref) <= TOL and qo.normalized_error(g16, ref) <= TOL
+    if tune & 7 != 1:
+        b16, b32, _ = _run_gemv(dev, "hq4_g32_m5", n, k, 1, prerot=False, xdtype=xdtype, variant=4, rt=0, outliers=True, seed=5)
+        assert np.array_equal(g32.view(np.uint32), b32.view(np.uint32)) and np.array_equal(g16.view(np.uint16), b16.view(np.uint16))
+
+
 def test_gemv_full_size_affine_config(dev):
     """C1: AQ4_G32 decode GEMV, N = 4096, K = 4096, automatic dispatch, standard basis."""
     g16, g32, ref = _run_full(dev, "aq4_g32", 4096, 4096, 1, prerot=False)

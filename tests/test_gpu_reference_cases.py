@@ -577,6 +577,24 @@ def test_pack_writer_quantizes_on_the_device_and_round_trips(dev, tmp_path):
     assert np.array_equal(buf.download(np.uint8, (want.nbytes,)), want.ravel().view(np.uint8))
 
 
+
+@pytest.mark.parametrize("rows,row_bytes", [(17408, 3200), (300, 3200), (7, 640), (513, 10880), (45, 5120), (2050, 1940), (1, 20)])
+def test_row_checksum_is_the_hosts_word_sum(dev, rows, row_bytes):
+    """qwhip_plane_checksum_rows (the decode GEMV's launch with the arithmetic taken out) adds every 32-bit word of the
+    bank exactly once: ragged row slots, short sets, fewer rows than a window, a partly filled last chunk of lanes, a
+    workgroup that ends in a half wave; refusals for rows that are not whole 20-byte pieces."""
+    rng = np.random.default_rng(rows)
+    host = rng.integers(0, 1 << 32, size=rows * row_bytes // 4, dtype=np.uint32)
+    lib, st = dev.lib, dev.stream.handle
+    plane, out = dev.put(host), dev.alloc(256 * 8)
+    qwhip.check(lib.qwhip_fill_u32(st, out.ptr, 0, 512))
+    qwhip.check(lib.qwhip_plane_checksum_rows(st, plane.ptr, rows, row_bytes, out.ptr))
+    dev.stream.sync()
+    assert int(out.download(np.uint64, (256,)).sum()) == int(host.astype(np.uint64).sum())
+    assert lib.qwhip_plane_checksum_rows(st, plane.ptr, rows, row_bytes + 4, out.ptr) == qwhip.E_BAD_SHAPE
+    assert lib.qwhip_plane_checksum_rows(st, plane.ptr, 0, row_bytes, out.ptr) == qwhip.OK
+
+
 @pytest.mark.parametrize("nbytes", [16, 4096 + 16, 3 * 1024 * 1024 + 48, 55705600])
 def test_plane_checksum_is_the_hosts_word_sum(dev, nbytes):
     """The sum of a plane's 32-bit words, exact in 64 bits whatever order the workgroups finish in; it adds into the 256
