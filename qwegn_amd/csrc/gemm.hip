@@ -664,7 +664,85 @@ __global__ __launch_bounds__(WVM* WVN * 64) void qw_gemm3_kernel(const qw_gemm_p
     const uint32_t last = nk - 1u;
     // Both groups run  { load tile k+1 (group 0) / k+2 (group 1) into registers; MFMAs of step k; barrier; registers -> LDS
     // stage; barrier }, group 1 half a K-step behind group 0: while one group multiplies, the other fills the next stage.
-    if (group == 0) {
+    // RELOAD (HQ4_G32_M5 banks on the 2 x 5 fragment wave tile): a register is loaded again, for the tile after the one being
+    // filled, right after the filling has read it.  The loads then fly for a whole K-step (a load takes ~1800 clocks here;
+    // issued ahead of the MFMA phase they held the wave for 400 to 900 clocks while the address unit took them one by
+    // one, issued inside it they were ~370 clocks short), spaced by the dequantization between them, and the MFMA phase
+    // issues nothing but matrix instructions and LDS reads.  The loads are asm statements with their destinations tied in
+    // and out, behind one s_waitcnt vmcnt(0) at the start of the filling: the compiler must not move or copy registers
+    // that are in flight across the loop's back edge.
+    constexpr bool RELOAD = FMT == QG_FMT_M5 && WM == 2 && WN == 5 && A_LD == 4 && B_PER == 2;
+    if constexpr (RELOAD) {
+        u4_t a_reg[A_LD], bq[2];
+        uint32_t bh[2];
+        auto first_loads = [&](uint32_t kt, int nitems) {          // compiler-visible loads ahead of the loop
+            qg_slice<FMT> b_reg[B_PER];
+            load_a(kt, a_reg);
+            load_b(kt, b_reg, nitems);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                bh[i] = i < nitems ? b_reg[i].hdr : 0u;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) bq[i][w] = i < nitems ? b_reg[i].q[w] : 0u;
+            }
+        };
+        // fills `stage` from the registers and sends each register off for tile `kn` as soon as it has been read
+        auto fill_reload = [&](uint32_t stage, uint32_t kn, int nitems) {
+            const uint8_t* xk = (const uint8_t*)p.x + a_tile_base + (uint64_t)(kt0 + kn) * 128u;
+            const uint8_t* bk = b_tile + (uint64_t)(kt0 + kn) * 40u;
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(a_reg[0]), "+v"(a_reg[1]), "+v"(a_reg[2]), "+v"(a_reg[3]), "+v"(bh[0]), "+v"(bq[0]), "+v"(bh[1]), "+v"(bq[1]));
+#pragma unroll
+            for (int i = 0; i < A_LD; ++i) {
+                *(h8_t*)(lds2 + stage * STAGE + a_lds0 + i * (A_BLK * 128u)) = qg_to_f16x8<XDT>(a_reg[i]);
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "+v"(a_reg[i]) : "v"(a_off[i]), "s"(xk) : "memory");
+            }
+            qg_slice<FMT> b_reg[B_PER];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                b_reg[i].hdr = bh[i];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) b_reg[i].q[w] = bq[i][w];
+            }
+            store_b(stage, b_reg, nitems);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                if (i >= nitems) break;
+                asm volatile("global_load_dword %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:4"
+                             : "+v"(bh[i]), "+v"(bq[i]) : "v"(b_voff[i]), "s"(bk) : "memory");
+            }
+        };
+        if (group == 0) {
+            first_loads(min(1u, last), B_PER);
+            for (uint32_t kt = 0; kt < nk; ++kt) {
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_setprio(3);
+                mfma_step(lds2 + (kt & 1u) * STAGE);
+                __builtin_amdgcn_s_setprio(0);
+                __builtin_amdgcn_sched_barrier(0);
+                fill_reload((kt + 1u) & 1u, min(kt + 2u, last), B_PER);
+                QG3_BAR_LDS();
+            }
+        } else {
+            {
+                qg_slice<FMT> b_first[B_PER];
+                u4_t a_first[A_LD];
+                load_a(min(1u, last), a_first);
+                load_b(min(1u, last), b_first, 1);
+                store_a(1u, a_first);
+                store_b(1u, b_first, 1);
+            }
+            first_loads(min(2u, last), 1);
+            for (uint32_t kt = 0; kt < nk; ++kt) {
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_setprio(3);
+                mfma_step(lds2 + (kt & 1u) * STAGE);
+                __builtin_amdgcn_s_setprio(0);
+                __builtin_amdgcn_sched_barrier(0);
+                QG3_BAR_LDS();
+                if (kt + 1u < nk) fill_reload(kt & 1u, min(kt + 3u, last), 1);      // stage (k+2)&1
+            }
+        }
+    } else if (group == 0) {
         for (uint32_t kt = 0; kt < nk; ++kt) {
             qg_slice<FMT> b_reg[B_PER];
             u4_t a_reg[A_LD];
