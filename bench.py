@@ -29,10 +29,22 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense f16/bf16 MFMA, published
 
-# HBM bytes per launch of the dominant kernel under its automatic configuration, from rocprofv3 --pmc passes
+# HBM bytes per launch of the dominant kernel under its automatic configuration come from rocprofv3 --pmc passes
 # (FETCH_SIZE KiB x 1024 x 2.000 + WRITE_SIZE KiB x 1024 x 1.000; the factors come from a streaming kernel of known
-# size).  The counter passes and the calibration are recorded as text under profiles/.
-MEASURED_TRAFFIC = {"c2": 56_129_590, "c3": 191_578_172}
+# size).  The passes are recorded as text under profiles/; the figure is read from the summary's line
+# "traffic = <bytes> B per launch", so the bench line cannot drift from the committed profile.
+TRAFFIC_PROFILES = {"c2": "gemv_col__c2_decode_n17408_k5120.txt", "c3": "gemm3_pingpong_256x320__c3_prefill_m4096_n5120_k5120.txt"}
+
+
+def measured_traffic(workload: str):
+    """Bytes per launch from the committed rocprof summary of `workload`, or None when there is none."""
+    import re
+    name = TRAFFIC_PROFILES.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return None
+    m = re.search(r"^\s*traffic\s*=\s*([0-9][0-9,]*)\s*B per launch", open(path).read(), re.M)
+    return int(m.group(1).replace(",", "")) if m else None
 
 
 def _fail(msg: str) -> None:
@@ -59,7 +71,7 @@ def _oracle_clib():
     return C.CDLL(str(build_oracle.LIB))
 
 
-def cpu_baseline_gemv(blocks, x_basis16, bits, group, is_m5, algo_bytes_full, rows_sample):
+def cpu_baseline_gemv(blocks, x_basis16, bits, group, is_m5, algo_bytes_full, rows_sample, budget_s=10.0):
     """Reference CPU oracle form (dequantize the bank to f16-rounded fp32, then one fp32 matrix-vector product:
     Scripts/oracle/gen_s1_q4_fixtures.py:28-31) in the oracle's C restatement, OpenMP over rows, on a row sample."""
     lib = _oracle_clib()
@@ -78,7 +90,7 @@ def cpu_baseline_gemv(blocks, x_basis16, bits, group, is_m5, algo_bytes_full, ro
 
     once()
     reps, t_total = 0, 0.0
-    while t_total < 10.0 and reps < 2000:
+    while t_total < budget_s and reps < 2000:
         t0 = time.perf_counter()
         once()
         t_total += time.perf_counter() - t0
@@ -110,6 +122,8 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None, cpu_later=None):
     if prerot:
         xb = dev.put(x_basis)
     flags = (args.variant << 8) | (args.rt << 12) | (qwhip.X_PREROTATED if prerot else 0)
+    if getattr(args, "invariant", False):
+        flags |= qwhip.GEMV_ROW_INVARIANT
     lib, st = dev.lib, dev.stream.handle
 
     def launch(i):
@@ -180,7 +194,7 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None, cpu_later=None):
                    "cache": "hot" if args.hot else f"cold ring of {ring_n} banks ({ring_n * bank_bytes / 1e6:.0f} MB)"},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": traffic if (args.variant == 0 and args.rt == 0 and not args.prerot) else None,
+                     "traffic": traffic if (args.variant == 0 and args.rt == 0 and not args.prerot and not getattr(args, "invariant", False)) else None,
                      "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3),
                      "read_only_launch_us": round(read_us, 3), "read_only_frac": round(bank_bytes / (read_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                      "read_only_rows_launch_us": None if rows_us is None else round(rows_us, 3),
@@ -194,6 +208,19 @@ def run_gemv(args, fmt, n, k, m, label, outliers, traffic=None, cpu_later=None):
             cpu_later.append(baseline)     # the caller runs it after its GPU legs: ten seconds of host work idle the card
         else:
             out["cpu_baseline"] = baseline()
+    return out
+
+
+def cpu_baseline_c1(budget_s: float = 5.0):
+    """The configuration the reference's CPU oracle path is named for (C1: AQ4_G32 affine GEMV, N = K = 4096): the oracle form
+    in its C restatement on this box's host cores, over the whole bank."""
+    from tests import helpers as H
+    kind, fmt, n, k, m, outliers = WORKLOADS["c1"]
+    _, bits, group, is_m5, _ = H.FORMATS[fmt]
+    blocks, _ = H.make_bank(fmt, n, k, seed=0)
+    x16 = H.make_x(1, k, 100).astype(np.float16)
+    out = cpu_baseline_gemv(blocks, H.x_in_basis(x16, fmt), bits, group, is_m5, blocks.nbytes + k * 2 + n * 2, n, budget_s)
+    out["config"] = LABELS["c1"]
     return out
 
 
@@ -639,22 +666,33 @@ def run_moe(args, t, label):
     vdn = dev.view(dnb, E * Hd, I, qwhip.KIND_HQ4_G32_M5)
 
     x32 = rng.standard_normal((t, Hd), dtype=np.float32)
-    logits = rng.standard_normal((t, E), dtype=np.float32)
     pairs = t * K
-    lb, ib, wb = dev.put(logits), dev.alloc(pairs * 4), dev.alloc(pairs * 4)
-    act, out = dev.alloc(pairs * I * 2), dev.alloc(t * Hd * 4)
     decode = t <= 8
+    # decode: a cycle of E / K steps whose tokens all route to different experts (a strong offset on a step's own K experts
+    # of a random partition), so that consecutive steps read different experts and the cycle walks every expert of both
+    # banks (377 MB, beyond the 256 MB Infinity Cache): cold figures.  Prefill: one batch of plain random logits.
+    cycle = E // K if decode else 1
+    logits_cycle = rng.standard_normal((cycle, t, E), dtype=np.float32)
+    if decode:
+        part = rng.permutation(E).reshape(cycle, K)
+        for i in range(cycle):
+            for j in range(t):
+                logits_cycle[i, j, part[(i * t + j) % cycle]] += np.float32(12.0)
+    logits = logits_cycle[0]
+    lbs = [dev.put(np.ascontiguousarray(logits_cycle[i])) for i in range(cycle)]
+    lb, ib, wb = lbs[0], dev.alloc(pairs * 4), dev.alloc(pairs * 4)
+    act, out = dev.alloc(pairs * I * 2), dev.alloc(t * Hd * 4)
     if decode:
         xv = qo.round_bf16(x32)
         xb = dev.put(qo.f32_to_bf16_bits(x32))
         x_basis = qo.fwht32_ortho(xv).astype(np.float16)
 
-        def gate_up():
-            qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, 0, ib.ptr, t, K, act.ptr))
+        def gate_up(i=0):   # the dominant launch: routing + routed gate|up GEMVs + SwiGLU + rotation
+            qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, 0, lbs[i % cycle].ptr, t, K, 1, 1.0, ib.ptr,
+                                                          wb.ptr, act.ptr))
 
-        def chain():   # routing happens inside the gate_up launch
-            qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, 0, lb.ptr, t, K, 1, 1.0, ib.ptr, wb.ptr,
-                                                          act.ptr))
+        def chain(i=0):
+            gate_up(i)
             qwhip.check(lib.qwhip_moe_down_decode(st, C.byref(vdn), E, act.ptr, ib.ptr, wb.ptr, t, K, None, None, out.ptr, qwhip.F32))
     else:
         if getattr(args, "moe_f16", False):
@@ -668,11 +706,11 @@ def run_moe(args, t, label):
         te, tr, tc = dev.alloc(mt * 4), dev.alloc(mt * 4), dev.alloc(16)
         dn_out = dev.alloc(pairs * Hd * 2)
 
-        def gate_up():   # grouped gate|up GEMM with the SwiGLU + FWHT-32 epilogue fused
+        def gate_up(i=0):   # grouped gate|up GEMM with the SwiGLU + FWHT-32 epilogue fused
             qwhip.check(lib.qwhip_moe_grouped_gemm_swiglu(st, C.byref(vgu), E, xb.ptr, xcode, 0, stok.ptr, off.ptr, te.ptr, tr.ptr,
                                                           tc.ptr, mt, pairs, 1, act.ptr, 0))
 
-        def chain():
+        def chain(i=0):
             qwhip.check(lib.qwhip_moe_route(st, lb.ptr, t, E, K, 1, 1.0, ib.ptr, wb.ptr))
             qwhip.check(lib.qwhip_moe_group_pairs(st, ib.ptr, E, pairs, K, off.ptr, sp.ptr, stok.ptr, inv.ptr, te.ptr, tr.ptr, tc.ptr, 1))
             gate_up()
@@ -680,21 +718,25 @@ def run_moe(args, t, label):
                                                    mt, pairs, dn_out.ptr, qwhip.F16, 0))
             qwhip.check(lib.qwhip_moe_combine(st, dn_out.ptr, qwhip.F16, inv.ptr, wb.ptr, t, K, Hd, None, None, out.ptr, qwhip.F32))
 
-    def timed(fn, steps, warmup):
-        _spin_up(dev, lambda i: fn(), 100.0)
-        for _ in range(warmup):
-            fn()
+    def timed(fn, steps, warmup, hot=False):
+        step = (lambda i: fn(0)) if hot else fn
+        _spin_up(dev, step, 100.0)
+        for i in range(warmup):
+            step(i)
         dev.stream.sync()
         e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
         e0.record(dev.stream)
-        for _ in range(steps):
-            fn()
+        for i in range(steps):
+            step(i)
         e1.record(dev.stream)
         dev.stream.sync()
         return e0.elapsed_ms(e1) * 1e3 / steps
 
     us_chain = timed(chain, args.steps, args.warmup)
     us_gu = timed(gate_up, args.steps, max(2, args.warmup // 4))      # the dominant kernel alone, same inputs
+    us_chain_hot = timed(chain, args.steps, max(2, args.warmup // 4), hot=True) if decode else None
+    chain(0)                                                           # the step that is checked: the cycle's first
+    dev.stream.sync()
     got = out.download(np.float32, (t, Hd))
     idx, wts = ib.download(np.int32, (t, K)), wb.download(np.float32, (t, K))
     ridx, rwts = qo.moe_route(logits, K, True, 1.0)
@@ -723,7 +765,10 @@ def run_moe(args, t, label):
         algo = w_bytes + t * Hd * 2 + t * Hd * 4 + t * E * 4
         gu_bytes = used * 2 * I * (Hd // 32) * 20 + t * Hd * 2 + pairs * I * 2
         gbs, gu_gbs = algo / (us_chain * 1e-6) / 1e9, gu_bytes / (us_gu * 1e-6) / 1e9
-        cfg["cache"] = "hot (the routed experts repeat between steps; 23.6 MB of the 377 MB banks per token)"
+        cfg["cache"] = (f"cold: a cycle of {cycle} steps whose tokens route to different experts walks all {E} experts "
+                        f"({E * (2 * I * (Hd // 32) * 20 + Hd * (I // 32) * 20) / 1e6:.0f} MB of banks)")
+        base["hot_cache"] = {"ms_per_step": round(us_chain_hot / 1e3, 6), "value": round(algo / (us_chain_hot * 1e-6) / 1e9, 2), "unit": "GB/s",
+                             "note": "the same step repeated: its experts (23.6 MB per token) stay in the Infinity Cache"}
         base.update({"value": round(gbs, 2), "unit": "GB/s", "config": cfg,
                      "roofline": {"bound": "hbm", "kernel": "routed gate_up GEMV", "achieved": round(gu_gbs, 2), "peak": HBM_PEAK_GBS,
                                   "unit": "GB/s", "frac": round(gu_gbs / HBM_PEAK_GBS, 4), "traffic": None,
@@ -835,6 +880,7 @@ def main() -> None:
     ap.add_argument("--gemm-ws-mb", type=int, default=0,
                     help="workspace handed to qwhip_gemm in MiB (0 = the activation copy only; more lets small row counts split K)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
+    ap.add_argument("--invariant", action="store_true", help="gemv workloads with QWHIP_GEMV_ROW_INVARIANT (every row as in a call of its own)")
     ap.add_argument("--format", default=None,
                     help="container override for the gemv / gemm / pair workloads, e.g. hq3_g32, aq6_g128 (the workload's shape is kept)")
     ap.add_argument("--no-cpu", action="store_true")
@@ -848,21 +894,23 @@ def main() -> None:
     if args.workload == "headline":
         kind, fmt, n, k, m, outliers = WORKLOADS["c2"]
         later = []
-        out = run_gemv(args, fmt, n, k, m, LABELS["c2"], outliers, MEASURED_TRAFFIC["c2"], cpu_later=later)
+        out = run_gemv(args, fmt, n, k, m, LABELS["c2"], outliers, measured_traffic("c2"), cpu_later=later)
         gargs = argparse.Namespace(**vars(args))
-        gargs.steps, gargs.warmup, gargs.no_cpu = max(10, args.steps // 10), max(3, args.warmup // 4), True
+        gargs.steps, gargs.warmup, gargs.no_cpu = max(50, args.steps // 4), max(5, args.warmup // 2), True
         kind, fmt, n, k, m, outliers = WORKLOADS["c3"]
-        g = run_gemm(gargs, fmt, n, k, m, LABELS["c3"], MEASURED_TRAFFIC["c3"])
+        g = run_gemm(gargs, fmt, n, k, m, LABELS["c3"], measured_traffic("c3"))
         out["prefill_gemm"] = {"value": g["value"], "unit": g["unit"], "ms_per_step": g["ms_per_step"], "steps": g["steps"],
                                "config": g["config"], "roofline": g["roofline"], "normalized_error": g["normalized_error"]}
         for fn in later:
             out["cpu_baseline"] = fn()
+        if not args.no_cpu:
+            out["cpu_baseline_c1"] = cpu_baseline_c1()
         print(json.dumps(out))
         return
     kind, fmt, n, k, m, outliers = WORKLOADS[args.workload]
     if m is None:
         m = args.m
-    label, traffic = LABELS[args.workload], MEASURED_TRAFFIC.get(args.workload)
+    label, traffic = LABELS[args.workload], measured_traffic(args.workload)
     if args.format and args.format != fmt:
         from tests import helpers as H
         if kind not in ("gemv", "gemm", "pair") or args.format not in H.FORMATS:

@@ -144,7 +144,10 @@ enum {
      * rounding, fused into the kernel prologue for one row, one pass into the stream's scratch
      * for several (QWWeightView.isRotated contract, QWWeightView.swift:33-38; producer-side
      * rotation Sources/QWMetal/include/qw_dequant.metalh:424-493). */
-    QWHIP_X_PREROTATED = 1u << 0
+    QWHIP_X_PREROTATED = 1u << 0,
+    /* qwhip_gemv: every activation row gets the bits it would get in a call of its own, whatever m is (one arithmetic for
+     * all row counts: the reference's 1- / 2- / 4- / M-row bodies agree bit for bit, qw_dequant_multi_b.metalh:14,486,533) */
+    QWHIP_GEMV_ROW_INVARIANT = 1u << 1
 };
 
 /* ---- elementwise seams ------------------------------------------------------ */
@@ -288,8 +291,9 @@ qwhip_status qwhip_gemm(qwhip_stream_t s, const qwhip_weight_view* w, const void
 
 /* qwhip_gemm for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks, kernels and
- * results as qwhip_gemm; the f16 copy of the activations (rotated, or converted from bf16) goes to a static device array
- * inside the library instead of the caller's workspace, and the call allocates nothing.  m * k * 2 must not exceed
+ * results as qwhip_gemm; the call allocates nothing.  Rows already in the container's basis (QWHIP_X_PREROTATED, or a
+ * standard-basis container) are read in place, at any size.  Rows that still have to be rotated are copied, rotated, into
+ * a static device array inside the library instead of a caller's workspace: for those m * k * 2 must not exceed
  * qwhip_gemm_noalloc_max_bytes() (8 MiB, held by every GPU the library runs on until the process ends), else
  * QWHIP_E_BAD_SHAPE.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams) race;
  * calls on one stream do not. */
@@ -462,10 +466,12 @@ qwhip_status qwhip_moe_compose_rows(qwhip_stream_t s, const int32_t* sorted_pair
                                     uint32_t n_rows, const int32_t* slot_of_row, int32_t* rows_out);
 /* qwhip_moe_combine summed by group (encodeMoEDownReduceCombineF32 with numGroups, QWGemmMoE.swift:299-332;
  * qwgemm_moe_nax_f16.metal:51-111): out [t, num_groups, width] = sum over routes k with labels[idx[t, k]] == g of
- * wts[t, k] * dn[inv_perm[t * top_k + k], :], zeros for a group without routes.  inv_perm / wts NULL as in qwhip_moe_combine. */
+ * wts[t, k] * dn[inv_perm[t * top_k + k], :], zeros for a group without routes.  inv_perm / wts NULL as in qwhip_moe_combine.
+ * labels holds `experts` entries; a route whose id (low 16 bits) is not below `experts` counts as absent, as in
+ * qwhip_moe_latent_groups and qwhip_moe_down_decode_groups. */
 qwhip_status qwhip_moe_combine_groups(qwhip_stream_t s, const void* dn, uint32_t dn_dtype, const int32_t* inv_perm,
-                                      const float* wts, const int32_t* idx, const int32_t* labels, uint32_t t, uint32_t top_k,
-                                      uint32_t num_groups, uint32_t width, void* out, uint32_t out_dtype);
+                                      const float* wts, const int32_t* idx, const int32_t* labels, uint32_t experts, uint32_t t,
+                                      uint32_t top_k, uint32_t num_groups, uint32_t width, void* out, uint32_t out_dtype);
 
 /* ---- load-time writer (the step before the path) ----------------------------- */
 /* qwg_quantize_bf16_to_hq4_g32_m5 (Sources/QWMetal/quant/qw_online_quant.metal:17-55), GPU twin of

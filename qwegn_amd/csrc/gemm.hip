@@ -1725,6 +1725,10 @@ extern "C" qwhip_status qwhip_gemm_noalloc(qwhip_stream_t s, const qwhip_weight_
                                            uint32_t ldx, void* y, uint32_t y_dtype, uint32_t ldy, uint32_t flags) {
     QWHIP_REQUIRE(s);
     QWHIP_REQUIRE(w);
+    // rows already in the container's basis are read where they lie (bf16 rows are converted while a tile is staged): no
+    // copy, so no limit on their size and nothing of the scratch array is touched
+    if (!(qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED)))
+        return qwhip_gemm(s, w, x, x_dtype, m, ldx, y, y_dtype, ldy, flags, nullptr, 0);
     const uint64_t need = (uint64_t)m * w->k * 2u;
     if (need > QW_GEMM_SCRATCH_BYTES)
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "qwhip_gemm_noalloc: m * k * 2 = %llu bytes exceeds the static scratch of %u bytes; use qwhip_gemm with a workspace",

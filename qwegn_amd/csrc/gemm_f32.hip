@@ -8,8 +8,12 @@
 //   v = hi + lo / 2048,  hi = RN_f16(v),  lo = RN_f16((v - hi) * 2048)     (|v - hi - lo / 2048| <= 2^-22 |v|),
 // and three f16 matrix products are accumulated in fp32: x_hi w_hi into one accumulator, x_hi w_lo + x_lo w_hi into a
 // second one that joins the first scaled by 1 / 2048 at the store; the dropped product x_lo w_lo is below 2^-22 of the
-// largest term.  The scaling by 2048 keeps the low parts out of the f16 subnormal range.  Activations beyond the f16
-// range (|x| > 65504) are outside this form.
+// largest term.  The scaling by 2048 keeps the low parts out of the f16 subnormal range.
+// Any fp32 activation row is taken: a first launch finds the largest magnitude of every row and leaves the power of two
+// that brings it into [2^13, 2^14) (the top of the f16 range, so that elements 2^27 times smaller than the largest still
+// split into normal f16 numbers); the rows are multiplied by it on their way into the split - exactly - and the sums by
+// its reciprocal at the store.  Without it a row with |x| > 65504 became inf - inf = NaN and rows below 2^-14 lost their
+// low parts; the reference's batched f32 kernels (qwg_gemm_*_f32_bm) take any fp32.
 //
 // Launch: a workgroup of four waves owns 64 activation rows x 64 weight rows and walks K in steps of 64: activations
 // global f32 -> registers -> two f16 LDS tiles, packed slices global -> registers -> two f16 LDS tiles (half a slice per
@@ -27,7 +31,30 @@ struct qgf_params {
     uint32_t M, N, K, gshift, bb, epi;
     uint64_t row_bytes;
     float scale;
+    const float* row_down;   // [M] powers of two: row r is contracted as x[r] * row_down[r]
 };
+
+// row_down[r] = 2^-e with 2^e <= max |x[r]| * 2^-13 < 2^(e + 1); 1 for a row of zeros.  e is kept inside the exponents
+// whose powers of two and their reciprocals are normal floats (a row whose largest magnitude is below 2^-113 is scaled
+// by 2^126 only); a row that holds inf or NaN gets a finite factor and stays non-finite.
+__global__ __launch_bounds__(256) void qw_row_scale_kernel(const float* __restrict__ x, uint32_t M, uint32_t K, float* __restrict__ row_down) {
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    if (row >= M) return;
+    const uint32_t* xr = (const uint32_t*)(x + (uint64_t)row * K);
+    uint32_t mx = 0u;
+    for (uint32_t c = lane * 4u; c + 3u < K; c += 256u) {
+        const u4_t v = *(const u4_t*)(xr + c);
+        mx = max(max(mx, v[0] & 0x7FFFFFFFu), max(max(v[1] & 0x7FFFFFFFu, v[2] & 0x7FFFFFFFu), v[3] & 0x7FFFFFFFu));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o, 64));
+    if (lane == 0u) {
+        int e = (int)(mx >> 23) - 127 - 13;
+        e = mx == 0u ? 0 : min(max(e, -126), 126);
+        row_down[row] = __uint_as_float((uint32_t)(127 - e) << 23);
+    }
+}
+
 
 template <int FMT>
 struct qgf_fmt {
@@ -81,11 +108,13 @@ __global__ __launch_bounds__(256) void qw_gemm_f32x_kernel(const qgf_params p) {
     // activation role: four 16-byte pieces per thread (row = c >> 4, piece = c & 15 of the row's 64 columns)
     const float* a_src[4];
     bool a_ok[4];
+    float a_down[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t c = tid + 256u * i, row = c >> 4;
         a_ok[i] = m0 + row < p.M;
         a_src[i] = p.x + (uint64_t)(a_ok[i] ? m0 + row : 0u) * p.K + (c & 15u) * 4u;
+        a_down[i] = p.row_down[a_ok[i] ? m0 + row : 0u];
     }
     // weight role: half `half` (16 columns) of slice `sl` of tile row `wr`
     const uint32_t item = tid & 127u, wr = item >> 1, sl = item & 1u;
@@ -147,7 +176,7 @@ __global__ __launch_bounds__(256) void qw_gemm_f32x_kernel(const qgf_params p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 h1_t h, l;
-                qgf_split(a_reg[i][e], h, l);
+                qgf_split(a_reg[i][e] * a_down[i], h, l);
                 hi[e] = h;
                 lo[e] = l;
             }
@@ -175,7 +204,10 @@ __global__ __launch_bounds__(256) void qw_gemm_f32x_kernel(const qgf_params p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const uint32_t row = m0 + wm * 32u + 8u * (r >> 2) + 4u * k_half + (r & 3);
-            if (row < p.M) p.y[(uint64_t)row * p.N + n] = qgf_epilogue(__builtin_fmaf(acc_lo[r], 1.0f / 2048.0f, acc[r]), p.epi, p.scale);
+            if (row < p.M) {
+                const float up = 1.0f / p.row_down[row];     // a power of two: exact
+                p.y[(uint64_t)row * p.N + n] = qgf_epilogue(__builtin_fmaf(acc_lo[r], 1.0f / 2048.0f, acc[r]) * up, p.epi, p.scale);
+            }
         }
     }
 }
@@ -183,11 +215,14 @@ __global__ __launch_bounds__(256) void qw_gemm_f32x_kernel(const qgf_params p) {
 }  // namespace
 
 // Runs the batched form for a validated call; false when the shape is outside it (K not a multiple of 64).
+// `row_down`: device scratch for m floats (the rows' scaling factors, written by the first of the two launches).
 // Epilogue 3's rotation over the outputs is the caller's second launch, as for the GEMV form.
 bool qw_f32_gemm(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
-                 const float* x, uint32_t m, uint32_t epi, float scale, float* y) {
-    if (w->k % 64u != 0 || ((uintptr_t)x & 15u) != 0) return false;
+                 const float* x, uint32_t m, uint32_t epi, float scale, float* y, float* row_down) {
+    if (w->k % 64u != 0 || ((uintptr_t)x & 15u) != 0 || !row_down) return false;
+    hipLaunchKernelGGL(qw_row_scale_kernel, dim3(qwhip_cdiv(m, 4u)), dim3(256), 0, st, x, m, w->k, row_down);
     qgf_params p;
+    p.row_down = row_down;
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
     p.y = y;

@@ -521,8 +521,10 @@ static __device__ __forceinline__ void run(const qw_gemv_params_x& p) {
     const uint32_t N = p.N, K = p.K;
     const uint32_t n0 = blockIdx.x * (16u * RT);
     const uint32_t tok = blockIdx.y;   // the output row
-    const uint32_t src = p.num_groups ? tok / p.num_groups : tok;
-    const int32_t grp = p.num_groups ? (int32_t)(tok - src * p.num_groups) : 0;
+    // group mode: num_groups carries the group count in its low byte and the expert count (the length of labels) above it
+    const uint32_t ng = p.num_groups & 0xFFu, n_experts = p.num_groups >> 8;
+    const uint32_t src = ng ? tok / ng : tok;
+    const int32_t grp = ng ? (int32_t)(tok - src * ng) : 0;
     const uint32_t magic = qw_vgpr_const(0x64006400u);
     f4_t total[RT];
 #pragma unroll
@@ -531,7 +533,7 @@ static __device__ __forceinline__ void run(const qw_gemv_params_x& p) {
         const uint32_t pair = src * p.top_k + k;
         const int32_t e = p.idx[pair];
         if (e < 0) continue;
-        if (p.num_groups && p.labels[(uint32_t)e & 0xFFFFu] != grp) continue;
+        if (ng && (((uint32_t)e & 0xFFFFu) >= n_experts || p.labels[(uint32_t)e & 0xFFFFu] != grp)) continue;   // an id past the labels is no route
         const float wk = p.wts ? p.wts[pair] : 1.0f;
         const uint8_t* bank = p.bank + (uint64_t)((uint32_t)e & 0xFFFFu) * p.expert_bytes;
         const uint8_t* rp[RT];
@@ -1037,6 +1039,47 @@ static qwhip_status qw_gemv_impl(qwhip_stream_t s, const qwhip_weight_view* w, c
     a.rotate = rotate ? 1u : 0u;
     a.rot_out = 0;
 
+    // Row-count invariance (QWHIP_GEMV_ROW_INVARIANT): every row gets the bits it would get alone, whatever m is - what the
+    // reference gets by compiling its 1-, 2-, 4- and M-row bodies without contraction or reassociation
+    // (Sources/QWMetal/include/qw_dequant_multi_b.metalh:14,486,533), and what lets serial decode and batched verify agree
+    // token for token.  One arithmetic serves every row count: the column-stationary dot2 kernel, whose sums for an
+    // activation row do not depend on how many other rows share its registers (four partial sums per slice in a fixed
+    // order, a fixed half-wave reduction, the chunks of a row in order), nor on the grid.  Un-rotated rows are rotated by
+    // the standalone pass first (m = 1 included), so that every row count contracts the same f16 values.
+    if (flags & QWHIP_GEMV_ROW_INVARIANT) {
+        if (variant != 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "the row-invariant mode picks its own kernel (override %u given)", variant);
+        const void* xin = x;
+        uint32_t xdt = x_dtype;
+        if (rotate) {
+            const size_t need = (size_t)m * w->k * 2u;
+            if (!s->scratch || s->scratch_bytes < QWHIP_STREAM_SCRATCH_BYTES || need > QWHIP_STREAM_XROT_BYTES)
+                return qwhip_fail(QWHIP_E_BASIS, "row-invariant gemv: %u un-rotated rows of %u do not fit the stream's rotation scratch; hand them over rotated", m, w->k);
+            void* xr = s->scratch + s->scratch_bytes - QWHIP_STREAM_XROT_BYTES;
+            st = qwhip_fwht32(s, x, x_dtype, xr, (uint64_t)m * w->k);
+            if (st != QWHIP_OK) return st;
+            xin = xr;
+            xdt = QWHIP_F16;
+        }
+        // one row over an HQ4_G32_M5 bank: the decode kernel, whose arithmetic the multi-row kernel repeats bit for bit
+        if (fmt == QW_FMT_M5 && m == 1) {
+            hipError_t e = hipSuccess;
+            if (qw_col_gemv(s->stream, w, xin, xdt, false, y16, y32, 0u, &e, nullptr, 0u, nullptr, nullptr)) {
+                QWHIP_TRY_HIP(e);
+                return QWHIP_OK;
+            }
+        }
+        const uint32_t cpr = (w->k / 32u + 31u) / 32u;
+        const uint32_t per = 32u * cpr <= 512u ? 8u : (32u * cpr <= 576u ? 4u : 2u);   // rows the kernel holds at this row length
+        for (uint32_t m0 = 0; m0 < m; m0 += per) {
+            hipError_t e = hipSuccess;
+            const uint32_t mm = min(per, m - m0);
+            if (!qw_colx_gemv(s->stream, w, fmt, a.gshift, a.bb, a.row_bytes, (const uint8_t*)xin + (size_t)m0 * w->k * 2u, xdt, mm, false,
+                              y16 ? (void*)((h1_t*)y16 + (size_t)m0 * w->n) : nullptr, y32 ? y32 + (size_t)m0 * w->n : nullptr, 0u, &e))
+                return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "row-invariant gemv: no column-stationary kernel for n=%u k=%u (rows up to 32768 columns, banks under 4 GiB)", w->n, w->k);
+            QWHIP_TRY_HIP(e);
+        }
+        return QWHIP_OK;
+    }
     // Several un-rotated rows on a rotated container: one rotation pass (fp32 butterfly, one f16 rounding: what the fused
     // prologues compute) into the stream's scratch, then the kernels for rows already in the basis, instead of the per-lane
     // rotation of the MFMA streamer.  Kernel overrides keep their own paths.
@@ -1391,7 +1434,7 @@ static qwhip_status qw_moe_down_decode_impl(qwhip_stream_t s, const qwhip_weight
     a.out = out;
     a.x_div = x_div;
     a.labels = labels;
-    a.num_groups = num_groups;
+    a.num_groups = num_groups ? (num_groups | (experts << 8)) : 0u;
     const dim3 grid(qwhip_cdiv(hidden, 16u)), block(512);
     const dim3 g2(grid.x, (uint32_t)out_rows);
 #define QW_DD(F, OD) qw_launch_scalar<qw_moe_down_decode_kernel<F, 1, OD>>(g2, block, 0, s->stream, a)
@@ -1443,7 +1486,7 @@ void qw_f32_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t g
 void qw_h32_f32_launch(hipStream_t st, const float* x, float* out, uint32_t rows, uint32_t hidden);
 // gemm_f32.hip
 bool qw_f32_gemm(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
-                 const float* x, uint32_t m, uint32_t epi, float scale, float* y);
+                 const float* x, uint32_t m, uint32_t epi, float scale, float* y, float* row_down);
 
 // fp32 activations in the container's basis -> fp32 outputs with the scalar epilogues of the reference's f32 family
 // (QWGemm.encodeHQ4F32V4 / encodeHQ4F32BM, Sources/Operators/QWGEMM/QWGemmF32.swift:178-199,311-350): the rows go through
@@ -1468,7 +1511,10 @@ extern "C" qwhip_status qwhip_gemv_f32(qwhip_stream_t s, const qwhip_weight_view
     const uint32_t per = qw_f32_gemv_rows(w, row_bytes);
     if (per == 0) return qwhip_fail(QWHIP_E_BAD_GEOMETRY, "no f32 gemv kernel for n=%u k=%u (rows up to 32768 columns, banks under 1 GiB)", w->n, w->k);
     const uint32_t gshift = log2_u32(w->group / 32), bb = qwhip_view_block_bytes(w);
-    const bool batched = m >= 32u && qw_f32_gemm(s->stream, w, fmt, gshift, bb, row_bytes, x, m, epi, scale, y);
+    // the batched form keeps one scaling factor per activation row (at most 65535 floats) at the head of the stream's
+    // partial-sum scratch: launches on a stream are ordered, and nothing else of this call uses the scratch
+    float* row_down = s->scratch ? (float*)(s->scratch + QWHIP_STREAM_COUNTER_BYTES) : nullptr;
+    const bool batched = m >= 32u && qw_f32_gemm(s->stream, w, fmt, gshift, bb, row_bytes, x, m, epi, scale, y, row_down);
     if (batched) QWHIP_TRY_HIP(hipGetLastError());
     for (uint32_t m0 = 0; !batched && m0 < m; m0 += per) {
         const uint32_t mm = min(per, m - m0);

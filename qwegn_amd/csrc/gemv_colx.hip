@@ -308,6 +308,22 @@ static __device__ __forceinline__ void run(const qcx_params& p) {
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
                 float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+                if constexpr (FMT == QW_FMT_M5) {
+                    // The arithmetic of the m = 1 kernel of gemv_col.hip (qw_gemv_colw_kernel), operation for operation: two
+                    // sums in word order (codes at bits 0..3 / 4..7), s q + ((1024 s + b) S 2^-24) at 2^-24 of full scale,
+                    // the factor back after the chunk sum - so that a row gets the same bits from either kernel.
+#pragma unroll
+                    for (int i = 0; i < 16; i += 2) {
+                        a0 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 0]), xo[m][i + 0], a0, false);
+                        a1 = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, ow[i + 1]), xo[m][i + 1], a1, false);
+                    }
+                    const float mt = __builtin_fmaf(sc, 1024.0f, bi) * (S[m] * 5.9604644775390625e-08f);
+                    float v = __builtin_fmaf(sc, __builtin_fmaf(a1, 0.0625f, a0), mt);
+                    v = gvalid ? v : 0.0f;
+                    v = qw_reduce32_dpp(v);
+                    if (lane == 31u && rslot < nrows) qcx_part[(rslot * cpr + chunk) * MR + m] = v;
+                    continue;
+                }
                 if constexpr (FMT == QW_FMT_B3) {
                     // a0, a1: the first mask's seven operands; a2: the second mask's six; a3: the third mask's three
 #pragma unroll
@@ -356,6 +372,7 @@ static __device__ __forceinline__ void run(const qcx_params& p) {
         const uint32_t m = t / nrows, s = t - m * nrows;
         float v = 0.f;
         for (uint32_t c = 0; c < cpr; ++c) v += qcx_part[(s * cpr + c) * MR + m];
+        if constexpr (FMT == QW_FMT_M5) v *= 16777216.0f;
         const uint64_t at = (uint64_t)m * N + s * G + blockIdx.x;
         if (p.y32) p.y32[at] = v;
         if (p.y16) p.y16[at] = (h1_t)v;

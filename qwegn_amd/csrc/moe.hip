@@ -618,7 +618,7 @@ extern "C" qwhip_status qwhip_moe_compose_rows(qwhip_stream_t s, const int32_t* 
 template <int DDT, int ODT>
 __global__ __launch_bounds__(256) void qw_moe_combine_groups_kernel(const void* __restrict__ dn, const int32_t* __restrict__ inv_perm,
                                                                      const float* __restrict__ wts, const int32_t* __restrict__ idx,
-                                                                     const int32_t* __restrict__ labels, uint32_t K, uint32_t NG,
+                                                                     const int32_t* __restrict__ labels, uint32_t E, uint32_t K, uint32_t NG,
                                                                      uint32_t W, void* __restrict__ out) {
     const uint32_t row = blockIdx.y, t = row / NG;
     const int32_t g = (int32_t)(row - t * NG);
@@ -627,7 +627,7 @@ __global__ __launch_bounds__(256) void qw_moe_combine_groups_kernel(const void* 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (uint32_t k = 0; k < K; ++k) {
         const int32_t e = idx[(uint64_t)t * K + k];
-        if (e < 0 || labels[(uint32_t)e & 0xFFFFu] != g) continue;
+        if (e < 0 || ((uint32_t)e & 0xFFFFu) >= E || labels[(uint32_t)e & 0xFFFFu] != g) continue;   // an id past the labels is no route
         const int32_t slot = inv_perm ? inv_perm[(uint64_t)t * K + k] : (int32_t)(t * K + k);
         if (slot < 0) continue;
         const float w = wts ? wts[(uint64_t)t * K + k] : 1.0f;
@@ -647,8 +647,8 @@ __global__ __launch_bounds__(256) void qw_moe_combine_groups_kernel(const void* 
 }
 
 extern "C" qwhip_status qwhip_moe_combine_groups(qwhip_stream_t s, const void* dn, uint32_t dn_dtype, const int32_t* inv_perm,
-                                                 const float* wts, const int32_t* idx, const int32_t* labels, uint32_t t, uint32_t top_k,
-                                                 uint32_t num_groups, uint32_t width, void* out, uint32_t out_dtype) {
+                                                 const float* wts, const int32_t* idx, const int32_t* labels, uint32_t experts, uint32_t t,
+                                                 uint32_t top_k, uint32_t num_groups, uint32_t width, void* out, uint32_t out_dtype) {
     QWHIP_REQUIRE(s);
     if (t == 0 || width == 0) return QWHIP_OK;
     QWHIP_REQUIRE(dn);
@@ -656,6 +656,7 @@ extern "C" qwhip_status qwhip_moe_combine_groups(qwhip_stream_t s, const void* d
     QWHIP_REQUIRE(labels);
     QWHIP_REQUIRE(out);
     if (num_groups == 0 || num_groups > 32u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "latent groups must be 1..32, got %u", num_groups);
+    if (experts == 0 || experts > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine by groups: labels for 1..65535 experts, got %u", experts);
     if ((uint64_t)t * num_groups >= (1ull << 31) || (uint64_t)t * top_k >= (1ull << 31))
         return qwhip_fail(QWHIP_E_BAD_SHAPE, "moe combine by groups: %u tokens", t);
     // grid.y holds 65535 rows: more (token, group) rows go in slabs of whole tokens
@@ -670,7 +671,7 @@ extern "C" qwhip_status qwhip_moe_combine_groups(qwhip_stream_t s, const void* d
         void* op = (uint8_t*)out + orow * (out_dtype == QWHIP_F32 ? 4u : 2u);
         // identity slots count from the slab's first token: shift the dn base instead
         const void* dp = inv_perm ? dn : (const void*)((const uint8_t*)dn + (uint64_t)t0 * top_k * width * (dn_dtype == QWHIP_F32 ? 4u : 2u));
-#define QW_CG(DD, OD) hipLaunchKernelGGL((qw_moe_combine_groups_kernel<DD, OD>), grid, block, 0, s->stream, dp, ip, wp, xp, labels, top_k, num_groups, width, op)
+#define QW_CG(DD, OD) hipLaunchKernelGGL((qw_moe_combine_groups_kernel<DD, OD>), grid, block, 0, s->stream, dp, ip, wp, xp, labels, experts, top_k, num_groups, width, op)
 #define QW_CG_O(DD)                                                   \
         switch (out_dtype) {                                          \
             case QWHIP_F32: QW_CG(DD, QWHIP_F32); break;              \

@@ -199,8 +199,10 @@ static __device__ __forceinline__ void run(const qmc_dn_params& p) {
     const uint32_t cprv = p.cprv, H = p.H;
     const uint32_t set = hw / cprv, chunk = hw - set * cprv;
     const uint32_t tok = blockIdx.y, n0 = blockIdx.x * (p.sets * D);   // tok: the output row
-    const uint32_t src = GRP ? tok / p.num_groups : tok;
-    const int32_t grp = GRP ? (int32_t)(tok - src * p.num_groups) : 0;
+    // group mode: num_groups carries the group count in its low byte and the expert count (the length of labels) above it
+    const uint32_t ng = p.num_groups & 0xFFu, n_experts = p.num_groups >> 8;
+    const uint32_t src = GRP ? tok / ng : tok;
+    const int32_t grp = GRP ? (int32_t)(tok - src * ng) : 0;
     const uint32_t v0 = chunk * 32u + lane;
     const bool vvalid = v0 < p.nbv;
     const uint32_t v = vvalid ? v0 : 0u;
@@ -209,7 +211,10 @@ static __device__ __forceinline__ void run(const qmc_dn_params& p) {
     const int32_t e = p.idx[pair];
     const float wk = p.wts ? p.wts[pair] : 1.0f;
     bool valid = vvalid && e >= 0;
-    if constexpr (GRP) valid = valid && p.labels[valid ? ((uint32_t)e & 0xFFFFu) : 0u] == grp;
+    if constexpr (GRP) {
+        valid = valid && ((uint32_t)e & 0xFFFFu) < n_experts;       // an id past the labels is no route
+        valid = valid && p.labels[valid ? ((uint32_t)e & 0xFFFFu) : 0u] == grp;
+    }
     const uint32_t row_bytes = p.nbI * 20u;
     // activations do not wait for the expert id; the weight rows follow as soon as it is known
     h8_t xr[4];
@@ -341,7 +346,7 @@ bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expert
     p.expert_bytes = (uint64_t)hidden * nbI * 20u;
     p.x_div = x_div;
     p.labels = labels;
-    p.num_groups = num_groups;
+    p.num_groups = num_groups ? (num_groups | (experts << 8)) : 0u;
     const dim3 grid(qwhip_cdiv(hidden, sets * D), out_rows), block(32u * cprv * sets);
 #define QMC_DN(OD)                                                                                            \
     do {                                                                                                      \

@@ -792,7 +792,7 @@ struct QWGemm {
         hal.pipeline("qwg_moe_down_reduce_combine_f32");
         throwIfFailed(qwhip_moe_combine_groups(enc.stream, dn.ptr(), abiDType(dn.shape.dtype), invPerm ? (const int32_t*)invPerm->ptr() : nullptr,
                                                wts ? (const float*)wts->ptr() : nullptr, (const int32_t*)idx.ptr(), (const int32_t*)labels.ptr(),
-                                               (uint32_t)rows, (uint32_t)topK, (uint32_t)numGroups, (uint32_t)width, out.ptr(),
+                                               (uint32_t)labels.shape.elementCount, (uint32_t)rows, (uint32_t)topK, (uint32_t)numGroups, (uint32_t)width, out.ptr(),
                                                abiDType(out.shape.dtype)));
     }
 };

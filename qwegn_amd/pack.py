@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import dataclasses
 import json
+import os
 import pathlib
 
 import numpy as np
@@ -364,5 +365,15 @@ class PackWriter:
 
     def __exit__(self, exc_type, exc, tb):
         if self._f is not None:
-            self.close()
+            if exc_type is None:
+                self.close()
+            else:
+                # the body failed: no trailer, and the partial file goes (it must not pass for a whole pack of the
+                # tensors added so far)
+                self._f.close()
+                self._f = None
+                try:
+                    os.unlink(self.path)
+                except OSError:
+                    pass
         return False

@@ -17,6 +17,7 @@ E_BAD_WEIGHTS, E_BAD_SHAPE, E_BAD_GEOMETRY, E_BLOCKED, E_KERNEL_MISSING, E_DEVIC
 F32, F16, BF16, I32 = 0, 1, 2, 3
 KIND_HQ4_G32_M5, KIND_ROTATED_HQ, KIND_NATIVE_AFFINE = 0, 1, 2
 X_PREROTATED = 1
+GEMV_ROW_INVARIANT = 2
 
 
 class QwhipError(RuntimeError):
@@ -103,7 +104,7 @@ SIGNATURES = {
     "qwhip_moe_gateup_decode_rows": (C.c_int32, [_P, _WV, _U32, _P, _U32, _U32, _P, _P, _U32, _U32, _P]),
     "qwhip_moe_down_decode_groups": (C.c_int32, [_P, _WV, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _P, _U32]),
     "qwhip_moe_compose_rows": (C.c_int32, [_P, _P, _U32, _P, _U32, _P, _P]),
-    "qwhip_moe_combine_groups": (C.c_int32, [_P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _P, _U32]),
+    "qwhip_moe_combine_groups": (C.c_int32, [_P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _P, _U32]),
     "qwhip_quantize_hq4_g32": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, _P]),
     "qwhip_quantize_blocks": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _U32, _P]),
     "qwhip_quantize_hq8_planar": (C.c_int32, [_P, _P, _U32, _U32, _U32, _U32, _P, _P]),

@@ -492,7 +492,7 @@ public enum QWGemm {
                                                  ids: QWTensorValue, labels: QWTensorValue, tokens: Int, routes: Int, numGroups: Int, width: Int,
                                                  out: QWTensorValue) throws {
         try hal.pipeline("qwg_moe_down_reduce_combine_f32")
-        try qwCheck(qwhip_moe_combine_groups(enc.stream, dnAcc.ptr, dnAcc.dtype.rawValue, invPerm?.i32, weights?.f32, ids.i32, labels.i32, UInt32(tokens),
+        try qwCheck(qwhip_moe_combine_groups(enc.stream, dnAcc.ptr, dnAcc.dtype.rawValue, invPerm?.i32, weights?.f32, ids.i32, labels.i32, UInt32(labels.elementCount), UInt32(tokens),
                                              UInt32(routes), UInt32(numGroups), UInt32(width), out.ptr, out.dtype.rawValue))
     }
 }

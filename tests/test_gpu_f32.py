@@ -94,6 +94,36 @@ def test_batched_f32_form_agrees_with_the_row_form(dev):
     assert qo.normalized_error(got32[:31], got31.astype(np.float64)) <= 2 * TOL
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq8_g32", "aq4_g32"])
+@pytest.mark.parametrize("m", [31, 32, 70])
+def test_f32_forms_take_any_fp32_activation_range(dev, fmt, m):
+    """Rows far outside the f16 range - magnitudes of 1e5 .. 3e9 (beyond 65504), of 1e-9 and of 1e-30, one row of zeros,
+    one row that mixes 1e6 with 1e-3 - give the same answers at 31 rows (fp32 kernel) and at 32 and more (matrix cores:
+    every row is scaled by a power of two ahead of the f16 split and back at the store), both within the fp32 bar of the
+    float64 evaluation, and no value turns non-finite."""
+    n, k = 192, 1024
+    _, bits, group, is_m5, _ = H.FORMATS[fmt]
+    blocks, _ = H.make_bank(fmt, n, k, seed=9)
+    rng = np.random.default_rng(m)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    mags = np.array([1e5, 3e9, 1e-9, 1e-30, 0.0, 1.0, 7e4, 1e20], np.float32)
+    x *= mags[np.arange(m) % len(mags)][:, None]
+    x[5, ::2] *= np.float32(1e6)
+    x[5, 1::2] *= np.float32(1e-3)
+    bank, xb, yb = dev.put(blocks), dev.put(x), dev.alloc(m * n * 4)
+    view = H.view_of(dev, bank, fmt, n, k)
+    qwhip.check(dev.lib.qwhip_gemv_f32(dev.stream.handle, C.byref(view), xb.ptr, m, 0, 1.0, yb.ptr))
+    dev.stream.sync()
+    got = yb.download(np.float32, (m, n))
+    want = qo.gemv_f32(blocks, x, bits, group, is_m5, 0, 1.0)
+    assert np.all(np.isfinite(got))
+    for r in range(m):          # row by row: the rows differ by 50 orders of magnitude
+        if mags[r % len(mags)] == 0.0:
+            assert np.all(got[r] == 0)
+        else:
+            assert qo.normalized_error(got[r:r + 1], want[r:r + 1]) <= TOL, (r, float(mags[r % len(mags)]))
+
+
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq8_g32"])
 def test_epilogue3_rows_together_equal_rows_alone(dev, fmt):
     """The reference's own check (Tests/QWGEMMTests/QWGemmEpi3MultiRowTests.swift:71-113): 2..5 rows in one call against

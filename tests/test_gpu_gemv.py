@@ -467,6 +467,50 @@ def test_gemv_hq4_column_stationary_windows(dev, tune, n, k, xdtype):
         assert np.array_equal(g32.view(np.uint32), b32.view(np.uint32)) and np.array_equal(g16.view(np.uint16), b16.view(np.uint16))
 
 
+@pytest.mark.parametrize("fmt,n,k", [("hq8_g32", 7168, 5120), ("hq4_g64", 5120, 17408), ("hq4_g32_m5", 1000, 5120), ("aq4_g32", 512, 4096),
+                                     ("hq4_g32", 300, 2048), ("hq8_g64", 256, 1024), ("aq2_g64", 256, 2048), ("hq3_g32", 200, 3072),
+                                     ("hq6_g32", 256, 5120), ("hq4_g128", 384, 8192), ("aq8_g256", 128, 16384), ("hq4_g32_m5", 96, 17408)])
+@pytest.mark.parametrize("prerot", [True, False])
+def test_gemv_row_invariant_mode_rows_together_equal_rows_alone(dev, fmt, n, k, prerot):
+    """QWHIP_GEMV_ROW_INVARIANT: for m in {2, 4, 8, 16} every row of the batched call carries the bits of the same row in a
+    call of its own (the reference's 1-row vs 2-row check, Tests/QWGEMMTests/QWGemmAQDecodeTests.swift:150-173, made
+    exact and taken to 16 rows) - on the two verify banks at their real shapes (q/k/v HQ8_G32 7168 x 5120, down HQ4_G64
+    5120 x 17408) and on every container class, rows in the basis and rows the call rotates itself; the results stay
+    inside the judged bar against the f16-weight reference."""
+    rotated = H.FORMATS[fmt][4]
+    if not rotated and not prerot:
+        pytest.skip("a standard-basis container has no rotation to fuse")
+    bank, w16 = _full_bank(dev, fmt, n, k)
+    view = H.view_of(dev, bank, fmt, n, k)
+    x16 = H.make_x(16, k, 77, outliers=True).astype(np.float16)
+    x_basis = H.x_in_basis(x16, fmt)
+    xb = dev.put(x_basis if prerot else x16)
+    flags = qwhip.GEMV_ROW_INVARIANT | (qwhip.X_PREROTATED if prerot else 0)
+    lib, st = dev.lib, dev.stream.handle
+    y_one16, y_one32 = dev.alloc(16 * n * 2), dev.alloc(16 * n * 4)
+    for r in range(16):                                   # every row alone
+        qwhip.check(lib.qwhip_gemv(st, C.byref(view), xb.ptr + r * k * 2, qwhip.F16, 1, flags, y_one16.ptr + r * n * 2, y_one32.ptr + r * n * 4))
+    dev.stream.sync()
+    one16, one32 = y_one16.download(np.uint16, (16, n)), y_one32.download(np.uint32, (16, n))
+    ref = qo.matmul_ref_f64(x_basis, w16)
+    assert qo.normalized_error(one32.view(np.float32), ref) <= TOL
+    y16, y32 = dev.alloc(16 * n * 2), dev.alloc(16 * n * 4)
+    if prerot:      # a plain decode call (no flag) on a row in the basis gives those bits too: decode runs at full speed
+        for r in (0, 5):
+            qwhip.check(lib.qwhip_gemv(st, C.byref(view), xb.ptr + r * k * 2, qwhip.F16, 1, qwhip.X_PREROTATED, y16.ptr, y32.ptr))
+            dev.stream.sync()
+            assert np.array_equal(y32.download(np.uint32, (16, n))[0], one32[r]) and np.array_equal(y16.download(np.uint16, (16, n))[0], one16[r])
+    for m in (2, 4, 8, 16, 3, 13):
+        qwhip.check(lib.qwhip_fill_u32(st, y32.ptr, 0xFFFFFFFF, 16 * n))
+        qwhip.check(lib.qwhip_gemv(st, C.byref(view), xb.ptr, qwhip.F16, m, flags, y16.ptr, y32.ptr))
+        dev.stream.sync()
+        assert np.array_equal(y32.download(np.uint32, (16, n))[:m], one32[:m]), f"m={m}: fp32 rows differ from the rows alone"
+        assert np.array_equal(y16.download(np.uint16, (16, n))[:m], one16[:m]), f"m={m}: f16 rows differ from the rows alone"
+    assert lib.qwhip_gemv(st, C.byref(view), xb.ptr, qwhip.F16, 2, flags | (7 << 8), y16.ptr, y32.ptr) == qwhip.E_BAD_SHAPE   # no override in this mode
+    for b in (xb, y_one16, y_one32, y16, y32):
+        b.free()
+
+
 def test_gemv_full_size_affine_config(dev):
     """C1: AQ4_G32 decode GEMV, N = 4096, K = 4096, automatic dispatch, standard basis."""
     g16, g32, ref = _run_full(dev, "aq4_g32", 4096, 4096, 1, prerot=False)

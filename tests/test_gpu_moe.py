@@ -571,7 +571,7 @@ def test_combine_groups(dev, t, k, ng, width, ddt, odt, perm):
     out = dev.alloc(t * ng * width * 4)
     db, pb, wb, ib, lb = dev.put(dnh), (dev.put(inv) if perm else None), dev.put(wts), dev.put(idx), dev.put(labels)
     qwhip.check(lib.qwhip_moe_combine_groups(st, db.ptr, qwhip.F16 if ddt == "f16" else qwhip.F32, pb.ptr if perm else None,
-                                             wb.ptr, ib.ptr, lb.ptr, t, k, ng, width, out.ptr, qwhip.F16 if odt == "f16" else qwhip.F32))
+                                             wb.ptr, ib.ptr, lb.ptr, e, t, k, ng, width, out.ptr, qwhip.F16 if odt == "f16" else qwhip.F32))
     dev.stream.sync()
     got = out.download(np.float16 if odt == "f16" else np.float32, (t, ng, width)).astype(np.float64)
     ref = np.zeros((t, ng, width))
@@ -582,6 +582,20 @@ def test_combine_groups(dev, t, k, ng, width, ddt, odt, perm):
             slot = int(inv[r * k + j]) if perm else r * k + j
             ref[r, labels[idx[r, j]]] += float(wts[r, j]) * dnh[slot].astype(np.float64)
     assert qo.normalized_error(got, ref) <= (2e-3 if odt == "f16" else 1e-6)
+    # a route whose id is not below the expert count has no label: it counts as absent (nothing past the labels is read)
+    idx2 = idx.copy()
+    idx2[0, 0] = e + 5
+    idx2[t - 1, k - 1] = (7 << 16) | e
+    ib2 = dev.put(idx2)
+    qwhip.check(lib.qwhip_moe_combine_groups(st, db.ptr, qwhip.F16 if ddt == "f16" else qwhip.F32, pb.ptr if perm else None,
+                                             wb.ptr, ib2.ptr, lb.ptr, e, t, k, ng, width, out.ptr, qwhip.F16 if odt == "f16" else qwhip.F32))
+    dev.stream.sync()
+    got2 = out.download(np.float16 if odt == "f16" else np.float32, (t, ng, width)).astype(np.float64)
+    for (r, j) in ((0, 0), (t - 1, k - 1)):
+        if idx[r, j] >= 0:
+            slot = int(inv[r * k + j]) if perm else r * k + j
+            ref[r, labels[idx[r, j]]] -= float(wts[r, j]) * dnh[slot].astype(np.float64)
+    assert qo.normalized_error(got2, ref) <= (2e-3 if odt == "f16" else 1e-5)
 
 
 def _group_latent_block(dev, fmts, t, e, k, ng, hidden, lat, inter, x16, idx, wts, labels, banks):
@@ -624,7 +638,7 @@ def _group_latent_block(dev, fmts, t, e, k, ng, hidden, lat, inter, x16, idx, wt
         dn = dev.alloc(pairs * lat * 4)
         qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vdn), e, act.ptr, qwhip.F16, 0, None, b2["off"].ptr, b2["te"].ptr, b2["tr"].ptr,
                                                b2["tc"].ptr, g2["max_tiles"], pairs, dn.ptr, qwhip.F32, 0))
-        qwhip.check(lib.qwhip_moe_combine_groups(st, dn.ptr, qwhip.F32, b2["inv"].ptr, wb.ptr, ib.ptr, lb.ptr, t, k, ng, lat, z16.ptr, qwhip.F16))
+        qwhip.check(lib.qwhip_moe_combine_groups(st, dn.ptr, qwhip.F32, b2["inv"].ptr, wb.ptr, ib.ptr, lb.ptr, e, t, k, ng, lat, z16.ptr, qwhip.F16))
         yu = dev.alloc(n1 * hidden * 4)
         qwhip.check(lib.qwhip_moe_grouped_gemm(st, C.byref(vu), ng, z16.ptr, qwhip.F16, 0, b1["sp"].ptr, b1["off"].ptr, b1["te"].ptr, b1["tr"].ptr,
                                                b1["tc"].ptr, g1["max_tiles"], n1, yu.ptr, qwhip.F32, 0))

@@ -140,3 +140,17 @@ def test_writer_round_trips_block_families_and_expert_stacks(tmp_path):
     assert p.weight_geometry("proj") == (n, k, qp.qwhip.KIND_ROTATED_HQ, 6, 128)
     assert np.array_equal(np.asarray(p.plane("proj")[1]), blk.ravel().view(np.uint8))
     assert np.array_equal(np.asarray(p.plane("gamma")[1]).view(np.float32), np.arange(k, dtype=np.float32))
+
+
+def test_pack_writer_leaves_no_file_when_its_body_fails(tmp_path):
+    """A with-body that raises must not leave something that reads as a complete pack of the tensors added so far: no
+    trailer is written and the partial file is removed; a clean exit still writes the pack."""
+    path = tmp_path / "partial.qwp"
+    with pytest.raises(RuntimeError):
+        with qp.PackWriter(path, {"source": "writer-test"}) as wr:
+            wr.add_raw("gamma", np.arange(64, dtype=np.float32), kind="f32")
+            raise RuntimeError("quantization failed midway")
+    assert not path.exists()
+    with qp.PackWriter(path, {"source": "writer-test"}) as wr:
+        wr.add_raw("gamma", np.arange(64, dtype=np.float32), kind="f32")
+    assert np.array_equal(np.asarray(qp.Pack(path).plane("gamma")[1]).view(np.float32), np.arange(64, dtype=np.float32))
