@@ -675,9 +675,13 @@ def run_moe(args, t, label):
     logits_cycle = rng.standard_normal((cycle, t, E), dtype=np.float32)
     if decode:
         part = rng.permutation(E).reshape(cycle, K)
+        shared = int(getattr(args, "moe_shared", 0) or 0)      # routes of a step's tokens 1.. that repeat token 0's experts
         for i in range(cycle):
             for j in range(t):
-                logits_cycle[i, j, part[(i * t + j) % cycle]] += np.float32(12.0)
+                own = part[(i * t + j) % cycle].copy()
+                if j > 0 and shared:
+                    own[:shared] = part[(i * t) % cycle][:shared]
+                logits_cycle[i, j, own] += np.float32(12.0)
     logits = logits_cycle[0]
     lbs = [dev.put(np.ascontiguousarray(logits_cycle[i])) for i in range(cycle)]
     lb, ib, wb = lbs[0], dev.alloc(pairs * 4), dev.alloc(pairs * 4)
@@ -760,11 +764,12 @@ def run_moe(args, t, label):
     cfg = {"workload": label, "format": "hq4_g32_m5", "tokens": t, "experts": E, "top_k": K, "hidden": Hd, "intermediate": I,
            "activations": "bf16" if decode or not getattr(args, "moe_f16", False) else "f16"}
     if decode:
-        used = len({int(e) for e in idx.ravel() if e >= 0})
+        used = len({int(e) for e in idx.ravel() if e >= 0})      # bytes are counted once per distinct expert of the step
         w_bytes = used * (2 * I * (Hd // 32) * 20 + Hd * (I // 32) * 20)
         algo = w_bytes + t * Hd * 2 + t * Hd * 4 + t * E * 4
         gu_bytes = used * 2 * I * (Hd // 32) * 20 + t * Hd * 2 + pairs * I * 2
         gbs, gu_gbs = algo / (us_chain * 1e-6) / 1e9, gu_bytes / (us_gu * 1e-6) / 1e9
+        cfg["distinct_experts_per_step"] = used
         cfg["cache"] = (f"cold: a cycle of {cycle} steps whose tokens route to different experts walks all {E} experts "
                         f"({E * (2 * I * (Hd // 32) * 20 + Hd * (I // 32) * 20) / 1e6:.0f} MB of banks)")
         base["hot_cache"] = {"ms_per_step": round(us_chain_hot / 1e3, 6), "value": round(algo / (us_chain_hot * 1e-6) / 1e9, 2), "unit": "GB/s",
@@ -875,6 +880,7 @@ def main() -> None:
     ap.add_argument("--rt", type=int, default=0, help="row tiles per wave for the mfma gemv (0 auto)")
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
     ap.add_argument("--moe-tokens", type=int, default=0, help="tokens of a c4 workload when run by itself (0 = the benchmark's 1 / 2048)")
+    ap.add_argument("--moe-shared", type=int, default=0, help="c4_decode with several tokens: how many of a token's routes repeat token 0's experts (0..8)")
     ap.add_argument("--moe-f16", action="store_true", help="c4_prefill on f16 hidden rows (the reference's own type) instead of bf16")
     ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 or mlp_prefill workload when run by itself (0 = the benchmark's 4096)")
     ap.add_argument("--gemm-ws-mb", type=int, default=0,

@@ -373,8 +373,11 @@ static bool qw_parse_aq_name(const char* name, const char** launcher) {
         else if (!strcmp(suffix, "f32_bm") || !strcmp(suffix, "f32_bm32")) lau = "qwhip_gemv_f32";
         else if (!strcmp(suffix, "h16_swiglu")) lau = "qwhip_gemm_swiglu";
     } else if (sscanf(name, "qwg_moe_nax_gemm_aq%u_g%u", &bits, &group) == 2 ||
-               sscanf(name, "qwg_moe_nax_split_f32_aq%u_g%u", &bits, &group) == 2) {
+               sscanf(name, "qwg_moe_nax_split_f32_aq%u_g%u", &bits, &group) == 2 ||
+               (sscanf(name, "qwg_moe_nax_split_aq%u_g%u_%63s", &bits, &group, suffix) == 3 && !strcmp(suffix, "f32"))) {
         lau = "qwhip_moe_grouped_gemm";
+    } else if (sscanf(name, "qwg_head_gemv_aq%u_g%u_%63s", &bits, &group, suffix) == 3 && !strcmp(suffix, "argmax")) {
+        lau = "qwhip_head_argmax";
     } else if (sscanf(name, "qwg_moe_gateup_aq%u_g%u_f32_r1", &bits, &group) == 2) {
         lau = "qwhip_moe_gateup_decode";
     } else if (sscanf(name, "qwg_moe_down_shared_combine_aq%u_g%u_f32", &bits, &group) == 2) {

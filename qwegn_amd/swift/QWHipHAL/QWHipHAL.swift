@@ -74,7 +74,8 @@ extension qwhip_weight_view {
 }
 
 /// The element types of QWDType that this path uses (Sources/Foundation/QWCore/QWDType.swift).
-public enum QWDType: UInt32 { case f32 = 0, f16 = 1, bf16 = 2, i32 = 3
+/// `.q4g` is the weight tag QWGemm.plan takes (HQ4_G32_M5, 20 B per 32 parameters); it is never the type of a tensor value.
+public enum QWDType: UInt32 { case f32 = 0, f16 = 1, bf16 = 2, i32 = 3, q4g = 0x100
     var bytes: Int { self == .f32 || self == .i32 ? 4 : 2 } }
 
 /// QWTensorValue on this HAL (Sources/Foundation/QWAlloc/QWArena.swift:49-151): a non-owning device region with an element
@@ -86,6 +87,11 @@ public struct QWTensorValue {
     public init(region: QWHipRegion, dtype: QWDType, elementCount: Int) {
         precondition(elementCount * dtype.bytes <= region.bytes, "tensor value exceeds its region")
         self.region = region; self.dtype = dtype; self.elementCount = elementCount
+    }
+    /// Zero-copy sub-view (QWArena.swift:62-66): `count` elements of `dtype` (default: this value's) from `byteOffset`.
+    public func slice(byteOffset: Int, count: Int, dtype: QWDType? = nil) -> QWTensorValue {
+        QWTensorValue(region: QWHipRegion(base: region.base, offset: region.offset + byteOffset, bytes: region.bytes - byteOffset),
+                      dtype: dtype ?? self.dtype, elementCount: count)
     }
     var ptr: UnsafeMutableRawPointer { region.ptr }
     var f32: UnsafeMutablePointer<Float> { region.ptr.assumingMemoryBound(to: Float.self) }
@@ -179,6 +185,11 @@ public enum QWGemm {
         return blocked
     }
 
+    /// QWGemm.plan with the reference's own labels (QWGemm.swift:92-133): dtype .q4g = quantized weights, .f16 = f16 weights.
+    public static func plan(_ shape: QWGemmShape, dtype: QWDType, epi: QWEpilogue, outDtype: QWDType = .f32, vocab: Int? = nil) -> QWGemmPlan {
+        plan(shape, quantized: dtype == .q4g, f16Weights: dtype == .f16, epi: epi, outDtype: outDtype, vocab: vocab)
+    }
+
     /// This library's routing: every row count 2...16 streams the bank once (qwhip_gemv), prefill and the remaining F4
     /// shapes run the matrix-core GEMM when K % 64 == 0.
     public static func planHip(_ shape: QWGemmShape, epi: QWEpilogue, outDtype: QWDType = .f32, vocab: Int? = nil) -> QWGemmPlan {
@@ -195,8 +206,11 @@ public enum QWGemm {
     }
 
     /// QWGemm.encode (QWGemm.swift:218-283): f32 output; .siluMulPair needs even N and stores f16 activations [rows, N / 2].
-    public static func encode(_ enc: QWHipEncoder, hal: QWHal, plan: QWGemmPlan, x: QWTensorValue, wQ4: QWWeightView,
-                              y: QWTensorValue, rows: Int = 1, xIsRotated: Bool = true) throws {
+    /// xGroupSum is taken and not read (the kernels form the group sums of x themselves); rows defaults to what the plan's kernel
+    /// implies (qwg_skinny_m2 / m3 -> 2 / 3, else 1), as the reference derives it.
+    public static func encode(_ enc: QWHipEncoder, hal: QWHal, plan: QWGemmPlan, x: QWTensorValue, xGroupSum: QWTensorValue? = nil,
+                              wQ4: QWWeightView, y: QWTensorValue, rows rowsArg: Int? = nil, xIsRotated: Bool = true) throws {
+        let rows = rowsArg ?? (plan.backend == .handQ4gSkinny ? (plan.kernel == "qwg_skinny_m3" ? 3 : 2) : 1)
         switch plan.backend {
         case .blocked:
             if plan.family == .f5SkinnyGemm { throw QWGemmError.badWeights("F5 window: run F1 per row") }
@@ -220,8 +234,8 @@ public enum QWGemm {
     }
 
     /// QWGemm.encodeH16 (QWGemm.swift:137-214): decode GEMV with direct f16 store (and optional f32 dual store).
-    public static func encodeH16(_ enc: QWHipEncoder, hal: QWHal, plan: QWGemmPlan, x: QWTensorValue, wQ4: QWWeightView,
-                                 y16: QWTensorValue, y32: QWTensorValue? = nil, rows: Int = 1, xIsRotated: Bool = true) throws {
+    public static func encodeH16(_ enc: QWHipEncoder, hal: QWHal, plan: QWGemmPlan, x: QWTensorValue, xGroupSum: QWTensorValue? = nil,
+                                 wQ4: QWWeightView, y16: QWTensorValue, y32: QWTensorValue? = nil, rows: Int = 1, xIsRotated: Bool = true) throws {
         guard plan.backend == .handQ4gV4H16 || plan.backend == .handQ4gSiluPairH16 || plan.backend == .handQ4gSkinny else {
             throw QWGemmError.badWeights("encodeH16 requires handQ4gV4H16 or handQ4gSiluPairH16")
         }
@@ -258,16 +272,18 @@ public enum QWGemm {
     }
 
     /// QWGemm.encodeFwht32 (QWGemm.swift:288-300)
-    public static func encodeFwht32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, count: Int) throws {
-        guard count > 0, count % 32 == 0 else { throw QWGemmError.badWeights("fwht32 f16: n must be > 0 and divisible by 32") }
+    public static func encodeFwht32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, count countArg: Int? = nil) throws {
+        let count = countArg ?? x.elementCount
+        guard x.dtype == .f16, count > 0, count % 32 == 0 else { throw QWGemmError.badWeights("fwht32 f16: n must be > 0 and divisible by 32") }
         try hal.pipeline("qwg_fwht32_f16")
         try qwCheck(qwhip_fwht32(enc.stream, x.ptr, UInt32(QWHIP_F16), x.ptr, UInt64(count)))
     }
     /// QWGemm.encodeCast (QWGemm.swift:305-320)
-    public static func encodeCast(_ enc: QWHipEncoder, hal: QWHal, src32: QWTensorValue, dst16: QWTensorValue, count: Int) throws {
-        guard src32.dtype == .f32, dst16.dtype == .f16, src32.elementCount >= count, dst16.elementCount >= count else { throw QWGemmError.badWeights("cast: f32 -> f16 operands") }
+    public static func encodeCast(_ enc: QWHipEncoder, hal: QWHal, x32: QWTensorValue, y16: QWTensorValue, count countArg: Int? = nil) throws {
+        let count = countArg ?? x32.elementCount
+        guard x32.dtype == .f32, y16.dtype == .f16, count > 0, x32.elementCount >= count, y16.elementCount >= count else { throw QWGemmError.badWeights("cast: f32 -> f16 operands") }
         try hal.pipeline("qwg_cast_f32_to_f16")
-        try qwCheck(qwhip_cast_f32_to_f16(enc.stream, src32.f32, dst16.ptr, UInt64(count)))
+        try qwCheck(qwhip_cast_f32_to_f16(enc.stream, x32.f32, y16.ptr, UInt64(count)))
     }
     /// QWGemm.encodeH32F32 (QWGemmF32.swift:46-54)
     public static func encodeH32F32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, out: QWTensorValue, rows: Int, hidden: Int) throws {
@@ -277,22 +293,27 @@ public enum QWGemm {
     }
     /// QWGemm.encodeHQ4F32V4 / encodeHQ4F32BM (QWGemmF32.swift:178-199, 311-350): fp32 activations, scalar epilogue 0...3.
     public static func encodeHQ4F32V4(_ enc: QWHipEncoder, hal: QWHal, weight: QWWeightView, x: QWTensorValue, y: QWTensorValue,
-                                      rows: Int = 1, epilogue: Int = 0, scale: Float = 1) throws {
+                                      rows: Int = 1, epi: UInt32 = 0, scale: Float = 1) throws {
         guard x.dtype == .f32, y.dtype == .f32, x.elementCount >= rows * weight.k, y.elementCount >= rows * weight.n else { throw QWGemmError.badWeights("f32 GEMV operands") }
         try hal.pipeline("qwg_gemv_q4g_f32_v4")
         var w = weight.abi
-        try qwCheck(qwhip_gemv_f32(enc.stream, &w, x.f32, UInt32(rows), UInt32(epilogue), scale, y.f32))
+        try qwCheck(qwhip_gemv_f32(enc.stream, &w, x.f32, UInt32(rows), epi, scale, y.f32))
     }
     /// QWGemm.encodeSiluMulF32 / encodeSiluMulSplitF16 / encodeAddF32 (QWGemmF32.swift:83-115)
-    public static func encodeSiluMulF32(_ enc: QWHipEncoder, hal: QWHal, gu: QWTensorValue, act: QWTensorValue, rows: Int, inter: Int) throws {
-        guard inter % 32 == 0 else { throw QWGemmError.badShape("silu_mul f32: intermediate % 32 == 0") }
+    /// act16 (optional): the same activations also stored as f16.
+    public static func encodeSiluMulF32(_ enc: QWHipEncoder, hal: QWHal, gu: QWTensorValue, act: QWTensorValue, rows: Int, intermediate: Int,
+                                        act16: QWTensorValue? = nil) throws {
+        guard intermediate % 32 == 0 else { throw QWGemmError.badShape("silu_mul f32: intermediate % 32 == 0") }
         try hal.pipeline("qwg_silu_mul_f32")
-        try qwCheck(qwhip_silu_mul_f32(enc.stream, gu.f32, act.f32, UInt32(rows), UInt32(inter)))
+        try qwCheck(qwhip_silu_mul_f32(enc.stream, gu.f32, act.f32, UInt32(rows), UInt32(intermediate)))
+        if let a16 = act16 { try encodeSiluMulF16(enc, hal: hal, gu: gu, act16: a16, rows: rows, intermediate: intermediate) }
     }
-    public static func encodeSiluMulSplitF16(_ enc: QWHipEncoder, hal: QWHal, gu: QWTensorValue, act16: QWTensorValue, rows: Int, inter: Int,
-                                             rotate: Bool = true) throws {
+    /// One f16 output instead of the reference's outHi / outLo pair (encodeSiluMulSplitF16): the f32 doors of this library split
+    /// their activations inside the GEMM kernel, so no caller needs the halves.
+    public static func encodeSiluMulF16(_ enc: QWHipEncoder, hal: QWHal, gu: QWTensorValue, act16: QWTensorValue, rows: Int, intermediate: Int,
+                                        rotate: Bool = true) throws {
         try hal.pipeline("qwg_silu_mul_split_f16")
-        try qwCheck(qwhip_swiglu_fwht(enc.stream, gu.ptr, gu.dtype.rawValue, act16.ptr, UInt32(rows), UInt32(inter), rotate ? 1 : 0))
+        try qwCheck(qwhip_swiglu_fwht(enc.stream, gu.ptr, gu.dtype.rawValue, act16.ptr, UInt32(rows), UInt32(intermediate), rotate ? 1 : 0))
     }
     public static func encodeAddF32(_ enc: QWHipEncoder, hal: QWHal, a: QWTensorValue, b: QWTensorValue, out: QWTensorValue, count: Int) throws {
         try hal.pipeline("qwg_add_f32")
@@ -320,27 +341,33 @@ public enum QWGemm {
     }
     /// QWGemm.encodeLatentNormH32F32 (QWGemmF32.swift:57-80): optional RMSNorm (1 + gamma) + H_32 on f32 rows -> f32 and / or f16.
     public static func encodeLatentNormH32F32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, gamma: QWTensorValue?, out32: QWTensorValue?,
-                                              out16: QWTensorValue?, rows: Int, latent: Int, eps: Float = 1e-6) throws {
-        guard latent > 0, latent % 32 == 0, out32 != nil || out16 != nil else { throw QWGemmError.badShape("latent norm H32: latent % 32 == 0, one output") }
+                                              out16: QWTensorValue? = nil, rows: Int, latent: Int, eps: Float = 1e-6, skipOut32: Bool = false) throws {
+        let o32 = skipOut32 ? nil : out32
+        guard latent > 0, latent % 32 == 0, o32 != nil || out16 != nil else { throw QWGemmError.badShape("latent norm H32: latent % 32 == 0, one output") }
         try hal.pipeline("qwg_latent_norm_h32_f32")
-        try qwCheck(qwhip_latent_norm_h32_f32(enc.stream, x.f32, gamma?.ptr, out32?.f32, out16?.ptr, UInt32(rows), UInt32(latent), eps))
+        try qwCheck(qwhip_latent_norm_h32_f32(enc.stream, x.f32, gamma?.ptr, o32?.f32, out16?.ptr, UInt32(rows), UInt32(latent), eps))
     }
     /// QWGemm.encodeMoEBridgeF16ToF32 (QWGemmMoE.swift:337-377): f16 normed hidden -> rotated f32 copy + un-rotated f32 copy.
     public static func encodeMoEBridgeF16ToF32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, xRot32: QWTensorValue?, xPlain32: QWTensorValue,
-                                               rows: Int, hidden: Int) throws {
+                                               rows: Int, hidden: Int, skipRot32: Bool = false) throws {
         guard hidden % 256 == 0 else { throw QWGemmError.badGeometry("moe bridge: hidden must be a multiple of 256") }
         try hal.pipeline("qwg_moe_bridge_f16_to_f32")
-        try qwCheck(qwhip_moe_bridge_f16_to_f32(enc.stream, x.ptr, xRot32?.f32, xPlain32.f32, UInt32(rows), UInt32(hidden)))
+        try qwCheck(qwhip_moe_bridge_f16_to_f32(enc.stream, x.ptr, skipRot32 ? nil : xRot32?.f32, xPlain32.f32, UInt32(rows), UInt32(hidden)))
     }
     /// QWGemm.encodeDenseProjF32 (QWGemmF32.swift:413-440): f32 rows in the container's basis -> f32 outputs; 64 rows and more without
     /// an epilogue go through one cast and the f16 GEMM, fewer through the f32 door (its batched matrix-core form from 32 rows on).
+    /// naxY16 and maxTileWidth are taken and not used: the GEMM needs no second f16 plane and has no tile-width limit.
     public static func encodeDenseProjF32(_ enc: QWHipEncoder, hal: QWHal, weight: QWWeightView, x: QWTensorValue, y: QWTensorValue,
-                                          naxX16: QWTensorValue, rows: Int, epilogue: Int = 0, scale: Float = 1) throws {
-        if rows >= 64, epilogue == 0, scale == 1, weight.n % 64 == 0, weight.k % 64 == 0, naxX16.elementCount >= rows * weight.k {
-            try encodeCast(enc, hal: hal, src32: x, dst16: naxX16, count: rows * weight.k)
-            try gemmBatchedH16(enc, hal: hal, x: naxX16, w: weight, y: y, rows: rows)
+                                          naxX16: QWTensorValue, naxY16: QWTensorValue, maxTileWidth: Int, rows: Int, epi: UInt32 = 0,
+                                          scale: Float = 1, x16Precast: QWTensorValue? = nil, minNaxRows: Int = 64) throws {
+        let count = rows * weight.k
+        if rows >= max(64, minNaxRows), epi == 0, scale == 1, weight.n % 64 == 0, weight.k % 64 == 0,
+           (x16Precast?.elementCount ?? naxX16.elementCount) >= count {
+            let x16 = (x16Precast ?? naxX16).slice(byteOffset: 0, count: count, dtype: .f16)
+            if x16Precast == nil { try encodeCast(enc, hal: hal, x32: x, y16: x16, count: count) }
+            try gemmBatchedH16(enc, hal: hal, x: x16, w: weight, y: y, rows: rows)
         } else {
-            try encodeHQ4F32V4(enc, hal: hal, weight: weight, x: x, y: y, rows: rows, epilogue: epilogue, scale: scale)
+            try encodeHQ4F32V4(enc, hal: hal, weight: weight, x: x, y: y, rows: rows, epi: epi, scale: scale)
         }
     }
 
@@ -360,16 +387,29 @@ public enum QWGemm {
         }
     }
     /// encodeFnMoeRoute (QWGemmMoERouter.swift:10-75): softmax top-k (or the sigmoid / bias / split-feature modes).
+    /// guSh / actSh / sharedIntermediate: the shared expert's silu_mul, which the reference folds into this launch, runs after it.
+    /// latentLabels / groupIds / numGroups: the groups of each token's routes; the route ids stay plain (the reference packs the
+    /// group into their high bits).  routedScale (an addition): constant factor on the weights.
     public static func encodeFnMoeRoute(_ enc: QWHipEncoder, hal: QWHal, logits: QWTensorValue, idx: QWTensorValue, wts: QWTensorValue,
-                                        rows: Int, experts: Int, topK: Int, normTopK: Bool, routedScale: Float = 1, bias: QWTensorValue? = nil,
-                                        splitFeature: Bool = false, routedScaleParam: QWTensorValue? = nil, expertBudget: Int = 0) throws {
+                                        rows: Int, experts: Int, topK: Int, normTopK: Bool, guSh: QWTensorValue? = nil, actSh: QWTensorValue? = nil,
+                                        sharedIntermediate: Int = 0, bias: QWTensorValue? = nil, expertBudget: Int = 0,
+                                        splitFeature: Bool = false, routedScaleParam: QWTensorValue? = nil, latentLabels: QWTensorValue? = nil,
+                                        groupIds: QWTensorValue? = nil, numGroups: Int = 0, routedScale: Float = 1) throws {
         precondition(experts <= 512 && topK <= 16, "route: experts <= 512, K <= 16")
+        if let gu = guSh, let act = actSh, sharedIntermediate > 0 {
+            try encodeSiluMulF32(enc, hal: hal, gu: gu, act: act, rows: rows, intermediate: sharedIntermediate)
+        }
+
         try hal.pipeline("qwg_moe_route")
         try qwCheck(qwhip_moe_route_ex(enc.stream, logits.f32, UInt32(rows), UInt32(experts), UInt32(topK), normTopK ? 1 : 0, routedScale,
                                        splitFeature ? 1 : 0, bias?.f32, routedScaleParam?.f32, idx.i32, wts.f32))
         if expertBudget > 0 && rows > 1 && rows <= 4 && expertBudget < rows * topK && rows * topK <= 64 {      // QWGemmMoERouter.swift:63-75
             try hal.pipeline("qwg_moe_route_decode")
             try qwCheck(qwhip_moe_route_budget(enc.stream, idx.i32, wts.f32, UInt32(rows), UInt32(topK), UInt32(expertBudget), normTopK ? 1 : 0))
+        }
+        if let labels = latentLabels, let gids = groupIds, numGroups > 0 {
+            try encodeMoELatentGroups(enc, hal: hal, idx: idx, labels: labels, rows: rows, topK: topK, experts: experts, numGroups: numGroups,
+                                      groupIds: gids, pairRows: nil)
         }
     }
     /// encodeMoEGroupPairsF32 (QWGemmMoE.swift:68-99): counting sort of the (token, route) pairs by expert + tile list.
@@ -405,12 +445,22 @@ public enum QWGemm {
                                                   rotateAct ? 1 : 0, act16.ptr, 0))
     }
     /// encodeMoEDownReduceCombineF32 (QWGemmMoE.swift:299-332)
-    public static func encodeMoEDownReduceCombineF32(_ enc: QWHipEncoder, hal: QWHal, dnAcc: QWTensorValue, invPerm: QWTensorValue,
+    /// out (f32 or f16) and out16 are both stored unless skipOut32; unweightedSingle: unit weights; skipShared drops the shared term.
+    /// The group sum (ids + numGroups) and scatterPerRoute have doors of their own here: encodeMoECombineGroupsF32, and the
+    /// grouped GEMM's gather rows (encodeMoEComposeRows).
+    public static func encodeMoEDownReduceCombineF32(_ enc: QWHipEncoder, hal: QWHal, dnAcc: QWTensorValue, invPerm: QWTensorValue?,
                                                      weights: QWTensorValue, shared: QWTensorValue?, gate: QWTensorValue?, out: QWTensorValue,
-                                                     hidden: Int, routes: Int, tokens: Int) throws {
+                                                     hidden: Int, routes: Int, tokens: Int, out16: QWTensorValue? = nil, skipShared: Bool = false,
+                                                     unweightedSingle: Bool = false, ids: QWTensorValue? = nil, numGroups: Int = 0,
+                                                     scatterPerRoute: Bool = false, skipOut32: Bool = false) throws {
+        guard numGroups == 0, !scatterPerRoute else { throw QWGemmError.badShape("combine: group sums and per-route scatter are encodeMoECombineGroupsF32 / encodeMoEComposeRows") }
+        guard !skipOut32 || out16 != nil else { throw QWGemmError.badShape("combine: skipOut32 needs out16") }
         try hal.pipeline("qwg_moe_down_reduce_combine_f32")
-        try qwCheck(qwhip_moe_combine(enc.stream, dnAcc.ptr, dnAcc.dtype.rawValue, invPerm.i32, weights.f32, UInt32(tokens), UInt32(routes),
-                                      UInt32(hidden), shared?.f32, gate?.f32, out.ptr, out.dtype.rawValue))
+        for dst in [skipOut32 ? nil : out, out16].compactMap({ $0 }) {
+            try qwCheck(qwhip_moe_combine(enc.stream, dnAcc.ptr, dnAcc.dtype.rawValue, invPerm?.i32, unweightedSingle ? nil : weights.f32, UInt32(tokens),
+                                          UInt32(routes), UInt32(hidden), skipShared ? nil : shared?.f32, skipShared ? nil : gate?.f32, dst.ptr,
+                                          dst.dtype.rawValue))
+        }
     }
     /// The same door with invPerm: nil and unweightedSingle (QWGemmMoE.swift:299-332): out = dnAcc + gate * shared, one row per token.
     public static func encodeMoEAddSharedF32(_ enc: QWHipEncoder, hal: QWHal, dnAcc: QWTensorValue, shared: QWTensorValue, gate: QWTensorValue?,
@@ -420,8 +470,15 @@ public enum QWGemm {
                                       out.ptr, out.dtype.rawValue))
     }
     /// encodeMoEGateUpF32R1 with fuseSiluFwht (QWGemmMoE.swift:120-155): routed gate_up with the ids given.
-    public static func encodeMoEGateUpF32R1(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, experts: Int, ids: QWTensorValue,
-                                            out: QWTensorValue, routes: Int, tokens: Int, xIsRotated: Bool = true) throws {
+    /// out: f16 [tokens, routes, rowsPerExpert / 2]; the SwiGLU and the rotation always run inside the launch (fuseSiluFwht: false,
+    /// the reference's separate gu32 matrix, is refused), and so is a cold bank.
+    public static func encodeMoEGateUpF32R1(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, ids: QWTensorValue,
+                                            out: QWTensorValue, rowsPerExpert: Int, routes: Int, tokens: Int, fuseSiluFwht: Bool = false,
+                                            coldBank: QWWeightView? = nil, reuseExpertsAcrossTokens: Bool = true, xIsRotated: Bool = true) throws {
+        guard fuseSiluFwht, coldBank == nil, rowsPerExpert > 0, bank.n % rowsPerExpert == 0 else {
+            throw QWGemmError.badShape("routed gate_up: fuseSiluFwht only, no cold bank, bank.n a multiple of rowsPerExpert")
+        }
+        let experts = bank.n / rowsPerExpert
         try hal.pipeline(bank.isIncumbent ? "qwg_moe_gateup_q4g_f32_r1" : "qwg_moe_gateup_aq\(bank.bits)_g\(bank.groupSize)_f32_r1")
         var w = bank.abi
         try qwCheck(qwhip_moe_gateup_decode(enc.stream, &w, UInt32(experts), x.ptr, x.dtype.rawValue, xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0,
@@ -438,13 +495,28 @@ public enum QWGemm {
                                                   logits.f32, UInt32(tokens), UInt32(routes), normTopK ? 1 : 0, routedScale, idx.i32, wts.f32, out.ptr))
     }
     /// encodeMoEDownSharedCombineF32 (QWGemmMoE.swift:157-199)
-    public static func encodeMoEDownSharedCombineF32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, experts: Int,
+    /// x: f16 [tokens, routes, k] ([tokens, k] with tokenIndexedX).  routeOutput: one output row per route, no sum and no shared
+    /// term.  The group sum (numGroups) is encodeMoEDownGroupsF32, which takes the labels; a cold bank is refused.
+    public static func encodeMoEDownSharedCombineF32(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, rowsPerRoute: Int,
                                                      routes: Int, weights: QWTensorValue, shared: QWTensorValue?, gate: QWTensorValue?,
-                                                     out: QWTensorValue, ids: QWTensorValue, tokens: Int) throws {
+                                                     out: QWTensorValue, ids: QWTensorValue, tokens: Int, out16: QWTensorValue? = nil,
+                                                     coldBank: QWWeightView? = nil, routeOutput: Bool = false, reuseExpertsAcrossTokens: Bool = true,
+                                                     skipShared: Bool = false, numGroups: Int = 0, tokenIndexedX: Bool = false) throws {
+        guard coldBank == nil, numGroups == 0, rowsPerRoute > 0, bank.n % rowsPerRoute == 0, routeOutput || !tokenIndexedX else {
+            throw QWGemmError.badShape("routed down: no cold bank, group sums are encodeMoEDownGroupsF32, bank.n a multiple of rowsPerRoute")
+        }
+        let experts = bank.n / rowsPerRoute
+        if routeOutput {
+            try encodeMoERoutedGemv(enc, hal: hal, bank: bank, experts: experts, x16: x, xPerToken: tokenIndexedX, ids: ids, weights: weights,
+                                    tokens: tokens, routes: routes, out: out)
+            return
+        }
         try hal.pipeline(bank.isIncumbent ? "qwg_moe_down_shared_combine_q4g_f32" : "qwg_moe_down_shared_combine_aq\(bank.bits)_g\(bank.groupSize)_f32")
         var w = bank.abi
-        try qwCheck(qwhip_moe_down_decode(enc.stream, &w, UInt32(experts), x.ptr, ids.i32, weights.f32, UInt32(tokens), UInt32(routes), shared?.f32,
-                                          gate?.f32, out.ptr, out.dtype.rawValue))
+        for dst in [out, out16].compactMap({ $0 }) {
+            try qwCheck(qwhip_moe_down_decode(enc.stream, &w, UInt32(experts), x.ptr, ids.i32, weights.f32, UInt32(tokens), UInt32(routes),
+                                              skipShared ? nil : shared?.f32, skipShared ? nil : gate?.f32, dst.ptr, dst.dtype.rawValue))
+        }
     }
 
     // ---- group-latent modes of the same encoders (latentLabels / groupIds / numGroups; the route ids stay plain here) ----
@@ -500,14 +572,44 @@ public enum QWGemm {
 /// QWGemmAQ (Sources/Operators/QWGEMM/QWGemmAQ.swift): the doors over the bit-stream containers.
 public enum QWGemmAQ {
     static func supported(bits: Int, group: Int) -> Bool { qwhip_block_bytes(UInt32(QWHIP_KIND_NATIVE_AFFINE), UInt32(bits), UInt32(group)) != 0 }
-    public static func kernelName(bits: Int, group: Int) -> String? { supported(bits: bits, group: group) ? "qwg_gemv_aq\(bits)_g\(group)_v4" : nil }        // :22-26
-    public static func decodeKernelName(bits: Int, group: Int) -> String? { supported(bits: bits, group: group) ? "qwg_gemv_aq\(bits)_g\(group)_dx_h16_t4" : nil }   // :28-36
-    public static func rowBytes(bits: Int, group: Int, k: Int) -> Int? {                                                                                  // :135-143
-        guard supported(bits: bits, group: group), k % group == 0 else { return nil }
+    /// The reference's name builders (QWGemmAQ.swift:22-133): nil for an unsupported (bits, group) pair and for every SHVQ
+    /// container, which has no kernel in this library.
+    static func name(_ head: String, _ bits: Int, _ group: Int, _ tail: String, _ isSHVQ: Bool) -> String? {
+        !isSHVQ && supported(bits: bits, group: group) ? "\(head)_aq\(bits)_g\(group)\(tail)" : nil
+    }
+    public static func kernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemv", bits, group, "_v4", isSHVQ) }
+    public static func decodeKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemv", bits, group, "_dx_h16_t4", isSHVQ) }
+    public static func siluPairKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemv", bits, group, "_silu_pair_dx_h16", isSHVQ) }
+    public static func headArgmaxKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_head_gemv", bits, group, "_argmax", isSHVQ) }
+    public static func gemmKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemm", bits, group, "_h16", isSHVQ) }
+    public static func swigluGemmKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemm", bits, group, "_h16_swiglu", isSHVQ) }
+    public static func f32BMKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemm", bits, group, "_f32_bm", isSHVQ) }
+    public static func f32V4KernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemv", bits, group, "_f32_v4", isSHVQ) }
+    public static func f32V4ArgmaxKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemv", bits, group, "_f32_v4_am", isSHVQ) }
+    public static func f32V4Argmax2KernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemv", bits, group, "_f32_v4_am2", isSHVQ) }
+    public static func naxF32KernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_gemm", bits, group, "_nax_f32", isSHVQ) }
+    public static func moeGateUpF32R1KernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_moe_gateup", bits, group, "_f32_r1", isSHVQ) }
+    public static func moeDownSharedCombineF32KernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? {
+        name("qwg_moe_down_shared_combine", bits, group, "_f32", isSHVQ)
+    }
+    public static func moeNaxGemmKernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_moe_nax_gemm", bits, group, "", isSHVQ) }
+    public static func moeNaxSplitF32KernelName(bits: Int, group: Int, isSHVQ: Bool = false) -> String? { name("qwg_moe_nax_split", bits, group, "_f32", isSHVQ) }
+    public static func rowBytes(bits: Int, group: Int, k: Int, isSHVQ: Bool = false) -> Int? {                                                            // :135-143
+        guard !isSHVQ, supported(bits: bits, group: group), k % group == 0 else { return nil }
         return (k / group) * Int(qwhip_block_bytes(UInt32(QWHIP_KIND_NATIVE_AFFINE), UInt32(bits), UInt32(group)))
     }
 
     /// QWGemmAQ.encode (QWGemmAQ.swift:192-249): rows 1...16 against one pass over the bank; f32 output.
+    /// isSHVQ: the vector-quantised container has no kernel here and is refused.  isRotated (an addition): the bank is a rotated
+    /// HQ container, which the reference tells from the weight view's kind before it calls this door.
+    public static func encode(_ enc: QWHipEncoder, hal: QWHal, blocks: QWTensorValue, x: QWTensorValue, y: QWTensorValue,
+                              n: Int, k: Int, bits: Int, group: Int, rows: Int = 1, isSHVQ: Bool = false, isRotated: Bool = false,
+                              xIsRotated: Bool = true) throws {
+        guard !isSHVQ else { throw QWGemmError.badWeights("SHVQ containers have no kernel in this library") }
+        try encode(enc, hal: hal, blocks: blocks.region, x: x, y: y, n: n, k: k, bits: bits, group: group, rows: rows, isRotated: isRotated,
+                   xIsRotated: xIsRotated)
+    }
+    /// The same door over a raw device region.
     public static func encode(_ enc: QWHipEncoder, hal: QWHal, blocks: QWHipRegion, x: QWTensorValue, y: QWTensorValue,
                               n: Int, k: Int, bits: Int, group: Int, rows: Int = 1, isRotated: Bool = false, xIsRotated: Bool = true) throws {
         guard let name = kernelName(bits: bits, group: group) else { throw QWGemmError.badWeights("no affine-quantised kernel for \(bits)-bit group \(group)") }
@@ -522,6 +624,13 @@ public enum QWGemmAQ {
         try qwCheck(qwhip_gemv(enc.stream, &w, x.ptr, x.dtype.rawValue, UInt32(rows), xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0, nil, y.f32))
     }
     /// QWGemmAQ.encodeDecodeT4 (QWGemmAQ.swift:255-304): one f16 row in, f16 out.
+    public static func encodeDecodeT4(_ enc: QWHipEncoder, hal: QWHal, blocks: QWTensorValue, x: QWTensorValue, y16: QWTensorValue,
+                                      n: Int, k: Int, bits: Int, group: Int, isSHVQ: Bool = false, isRotated: Bool = false,
+                                      xIsRotated: Bool = true) throws {
+        guard !isSHVQ else { throw QWGemmError.badWeights("SHVQ containers have no kernel in this library") }
+        try encodeDecodeT4(enc, hal: hal, blocks: blocks.region, x: x, y16: y16, n: n, k: k, bits: bits, group: group, isRotated: isRotated,
+                           xIsRotated: xIsRotated)
+    }
     public static func encodeDecodeT4(_ enc: QWHipEncoder, hal: QWHal, blocks: QWHipRegion, x: QWTensorValue, y16: QWTensorValue,
                                       n: Int, k: Int, bits: Int, group: Int, isRotated: Bool = false, xIsRotated: Bool = true) throws {
         guard let name = decodeKernelName(bits: bits, group: group) else { throw QWGemmError.badWeights("no affine-quantised decode kernel for \(bits)-bit group \(group)") }
@@ -546,6 +655,15 @@ public enum QWGemmAQ {
         try qwCheck(qwhip_head_argmax(enc.stream, &w, x.ptr, x.dtype.rawValue, UInt32(rows), xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0, logits.f32, tokens.i32))
     }
     /// QWGemmAQ.encodeEmbedAQ (QWGemmAQ.swift:147-187): out f32 [rows, hc, hidden] = the token's row, code * scale + bias.
+    public static func encodeEmbedAQ(_ enc: QWHipEncoder, hal: QWHal, blocks: QWTensorValue, token: QWTensorValue, out: QWTensorValue,
+                                     hidden: Int, hc: Int, bits: Int, group: Int, rows: Int = 1) throws {
+        guard let rb = rowBytes(bits: bits, group: group, k: hidden), rb > 0,            // the table's row count is what its region holds
+              let table = QWWeightView(blocks: blocks.region, n: blocks.elementCount * blocks.dtype.bytes / rb, k: hidden,
+                                       kind: .nativeAffine(bits: bits, group: group)) else {
+            throw QWGemmError.badWeights("no embedding kernel for \(bits)-bit group \(group), or an empty table")
+        }
+        try encodeEmbedAQ(enc, hal: hal, table: table, token: token, out: out, rows: rows, hc: hc)
+    }
     public static func encodeEmbedAQ(_ enc: QWHipEncoder, hal: QWHal, table: QWWeightView, token: QWTensorValue, out: QWTensorValue,
                                      rows: Int, hc: Int = 1) throws {
         guard rows > 0, hc > 0, token.elementCount >= rows, out.dtype == .f32, out.elementCount >= rows * hc * table.k else {
@@ -557,226 +675,393 @@ public enum QWGemmAQ {
     }
 }
 
-/// QWMoEOperator.encodeResident (Sources/Operators/QWGEMM/QWMoEOperator.swift:57-442): the routed-expert block on resident banks.
+/// QWMoEOperator (Sources/Operators/QWGEMM/QWMoEOperator.swift:12-442, +Latent.swift:17-303, +GroupLatent.swift:11-294): the
+/// routed-expert block on resident banks.  Types, labels and defaults are the reference's; `Weights.routedScale` and
+/// `Scratch.hip` are additions with defaults, `decodeRouterOverride` has no counterpart (the router is always the library's).
+/// The encoder is a HIP stream: work on it runs in order, so `concurrentBarriers`, `rotateEncoder` and `profileStage` are taken
+/// and have nothing to do.
 public enum QWMoEOperator {
-    public struct Weights {
-        public let router: QWTensorValue       // [experts, hidden] f32 / f16 / bf16
-        public let gateUp: QWWeightView        // n = experts * 2 * intermediate, k = hidden
-        public let down: QWWeightView          // n = experts * hidden, k = intermediate
-        public let hidden: Int, experts: Int, topK: Int, intermediate: Int
-        public let normTopK: Bool
-        public let routedScale: Float
-    }
-    public struct Scratch {                    // caller-owned (the reference's arena scratch, QWMoEOperator.swift:117-192)
-        public let logits: QWTensorValue       // f32 [rows, experts]
-        public let idx: QWTensorValue          // i32 [rows, topK]
-        public let wts: QWTensorValue          // f32 [rows, topK]
-        public let act16: QWTensorValue        // f16 [rows * topK, intermediate]
-        public let expOff, sortedPair, sortedTok, invPerm, tileE, tileR, tileCount: QWTensorValue?   // prefill only, i32
-        public let dnHi: QWTensorValue?        // f32 or f16 [rows * topK, hidden], prefill only
-    }
-    /// x: f16 hidden rows in the experts' basis; xPlain: the un-rotated rows the router reads.  rows > 8 runs the grouped path
-    /// (route -> pair sort -> gate_up GEMM with SwiGLU fused -> down GEMM -> combine), fewer rows the routed GEMVs.
-    public static func encodeResident(_ enc: QWHipEncoder, hal: QWHal, weights w: Weights, scratch s: Scratch, x: QWTensorValue,
-                                      xPlain: QWTensorValue, out32: QWTensorValue, rows T: Int, shared: QWTensorValue? = nil,
-                                      sharedGate: QWTensorValue? = nil) throws {
-        let (H, E, K, I) = (w.hidden, w.experts, w.topK, w.intermediate)
-        guard E > 0, E <= 512, K > 0, K <= 16 else { throw QWGemmError.badShape("moe: experts <= 512, routes <= 16") }
-        guard w.gateUp.n == E * 2 * I, w.gateUp.k == H, w.down.n == E * H, w.down.k == I else {
-            throw QWGemmError.badShape("moe: expert banks do not match (experts, hidden, intermediate)")
-        }
-        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: xPlain, y: s.logits, rows: T, n: E, k: H)
-        if T > 8, let expOff = s.expOff, let sortedPair = s.sortedPair, let sortedTok = s.sortedTok, let invPerm = s.invPerm,
-           let tileE = s.tileE, let tileR = s.tileR, let tileCount = s.tileCount, let dnHi = s.dnHi, H % 64 == 0, I % 64 == 0, x.dtype == .f16 {
-            let pairs = T * K
-            try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
-                                        routedScale: w.routedScale)
-            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: expOff, sortedPairIdx: sortedPair, sortedTok: sortedTok, experts: E,
-                                              totalPairs: pairs, routes: K, invPerm: invPerm, tileE: tileE, tileR: tileR, tileCount: tileCount)
-            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: x, bank: w.gateUp, experts: E, sortedTok: sortedTok, expertOff: expOff, tileE: tileE,
-                                             tileR: tileR, tileCount: tileCount, act16: s.act16, pairs: pairs, rotateAct: w.down.isRotated)
-            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: s.act16, bank: w.down, experts: E, expertOff: expOff, tileE: tileE, tileR: tileR,
-                                            tileCount: tileCount, y: dnHi, pairs: pairs)
-            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: dnHi, invPerm: invPerm, weights: s.wts, shared: shared, gate: sharedGate,
-                                                     out: out32, hidden: H, routes: K, tokens: T)
-        } else {
-            try QWGemm.encodeMoERouteGateUp(enc, hal: hal, x: x, bank: w.gateUp, experts: E, logits: s.logits, idx: s.idx, wts: s.wts, out: s.act16,
-                                            routes: K, tokens: T, normTopK: w.normTopK, routedScale: w.routedScale)
-            try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: s.act16, bank: w.down, experts: E, routes: K, weights: s.wts, shared: shared,
-                                                     gate: sharedGate, out: out32, ids: s.idx, tokens: T)
-        }
-    }
-
-    // ---- latent-bottleneck sparse MoE (QWMoEOperator+Latent.swift:17-303) ------------------------------------------------
-    public struct LatentBottleneck {
-        public let fc1: QWWeightView           // n = latentDim, k = hidden
-        public let fc2: QWWeightView           // n = hidden, k = latentDim
-        public let normGamma: QWTensorValue?   // f16 [latentDim], plus-one law
-        public let normEps: Float
-        public let latentDim: Int
-    }
-    public struct LatentWeights {
-        public let routed: Weights             // gateUp: k = latentDim; down: n = experts * latentDim
-        public let sharedGateUp: QWWeightView?, sharedDown: QWWeightView?
-        public let sharedGateScalar: QWTensorValue?      // f32 [hidden]
-        public let sharedIntermediate: Int
-        public let routerBias: QWTensorValue?, routedScaleParam: QWTensorValue?
-        public let splitFeatureRouting: Bool
-    }
-    public struct LatentScratch {
-        public let xRot32, xPlain32: QWTensorValue       // f32 [rows, hidden]
-        public let bufA32, bufB32: QWTensorValue         // f32 [rows, latentDim]
-        public let bufB16: QWTensorValue                 // f16 [rows, latentDim]
-        public let naxX16: QWTensorValue                 // f16 staging of the dense projections
-        public let gate: QWTensorValue                   // f32 [rows]
-        public let guSh32, actSh32, shared: QWTensorValue
-    }
-    /// fc1 -> route -> rotate -> routed experts in the latent width -> latent norm -> fc2, the shared expert on the hidden width
-    /// added under its gate.  x16: the operator's .f16Normed input.
-    public static func encodeResidentLatent(_ enc: QWHipEncoder, hal: QWHal, weights lw: LatentWeights, latent: LatentBottleneck, scratch s: Scratch,
-                                            latentScratch ls: LatentScratch, x16: QWTensorValue, out32: QWTensorValue, rows T: Int) throws {
-        let w = lw.routed
-        let (H, L, E, K, I, ISh) = (w.hidden, latent.latentDim, w.experts, w.topK, w.intermediate, lw.sharedIntermediate)
-        guard L > 0, L % 32 == 0, latent.fc1.n == L, latent.fc1.k == H, latent.fc2.n == H, latent.fc2.k == L,
-              w.gateUp.n == E * 2 * I, w.gateUp.k == L, w.down.n == E * L, w.down.k == I else {
-            throw QWGemmError.badShape("latent moe: banks do not match (hidden, latent, experts, intermediate)")
-        }
-        let routerCols = lw.splitFeatureRouting ? 2 * E : E
-        try QWGemm.encodeMoEBridgeF16ToF32(enc, hal: hal, x: x16, xRot32: ls.xRot32, xPlain32: ls.xPlain32, rows: T, hidden: H)
-        let sharedBanks: (QWWeightView, QWWeightView)? = (ISh > 0 && lw.sharedGateUp != nil && lw.sharedDown != nil) ? (lw.sharedGateUp!, lw.sharedDown!) : nil
-        let gateW = sharedBanks != nil ? lw.sharedGateScalar : nil
-        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: ls.xPlain32, y: s.logits, rows: T, n: routerCols, k: H,
-                                      shGateWeight: gateW, shGateOut: gateW != nil ? ls.gate : nil)
-        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: latent.fc1, x: ls.xRot32, y: ls.bufA32, naxX16: ls.naxX16, rows: T)
-        try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
-                                    routedScale: w.routedScale, bias: lw.routerBias, splitFeature: lw.splitFeatureRouting,
-                                    routedScaleParam: lw.routedScaleParam)
-        try QWGemm.encodeLatentNormH32F32(enc, hal: hal, x: ls.bufA32, gamma: nil, out32: nil, out16: ls.bufB16, rows: T, latent: L, eps: latent.normEps)
-        if let (shGU, shDown) = sharedBanks {
-            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shGU, x: ls.xRot32, y: ls.guSh32, naxX16: ls.naxX16, rows: T)
-            try QWGemm.encodeSiluMulF32(enc, hal: hal, gu: ls.guSh32, act: ls.actSh32, rows: T, inter: ISh)
-            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shDown, x: ls.actSh32, y: ls.shared, naxX16: ls.naxX16, rows: T)
-        }
-        let pairs = T * K
-        if T > 8, let expOff = s.expOff, let sortedPair = s.sortedPair, let sortedTok = s.sortedTok, let invPerm = s.invPerm,
-           let tileE = s.tileE, let tileR = s.tileR, let tileCount = s.tileCount, let dnHi = s.dnHi, L % 64 == 0, I % 64 == 0 {
-            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: expOff, sortedPairIdx: sortedPair, sortedTok: sortedTok, experts: E,
-                                              totalPairs: pairs, routes: K, invPerm: invPerm, tileE: tileE, tileR: tileR, tileCount: tileCount)
-            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: ls.bufB16, bank: w.gateUp, experts: E, sortedTok: sortedTok, expertOff: expOff, tileE: tileE,
-                                             tileR: tileR, tileCount: tileCount, act16: s.act16, pairs: pairs, rotateAct: w.down.isRotated)
-            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: s.act16, bank: w.down, experts: E, expertOff: expOff, tileE: tileE, tileR: tileR,
-                                            tileCount: tileCount, y: dnHi, pairs: pairs)
-            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: dnHi, invPerm: invPerm, weights: s.wts, shared: nil, gate: nil,
-                                                     out: ls.bufA32, hidden: L, routes: K, tokens: T)
-        } else {
-            try QWGemm.encodeMoEGateUpF32R1(enc, hal: hal, x: ls.bufB16, bank: w.gateUp, experts: E, ids: s.idx, out: s.act16, routes: K, tokens: T)
-            try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: s.act16, bank: w.down, experts: E, routes: K, weights: s.wts, shared: nil,
-                                                     gate: nil, out: ls.bufA32, ids: s.idx, tokens: T)
-        }
-        try QWGemm.encodeLatentNormH32F32(enc, hal: hal, x: ls.bufA32, gamma: latent.normGamma, out32: ls.bufB32, out16: nil, rows: T, latent: L,
-                                          eps: latent.normEps)
-        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: latent.fc2, x: ls.bufB32, y: out32, naxX16: ls.naxX16, rows: T)
-        if sharedBanks != nil {
-            try QWGemm.encodeMoEAddSharedF32(enc, hal: hal, dnAcc: out32, shared: ls.shared, gate: gateW != nil ? ls.gate : nil, out: out32, hidden: H,
-                                             tokens: T)
-        }
-    }
-
-    // ---- group-latent sparse MoE (QWMoEOperator+GroupLatent.swift:11-294) ------------------------------------------------
-    public struct GroupLatentWeights {
-        public let routed: Weights             // gateUp: k = latentDim; down: n = experts * latentDim
-        public let latentD: QWWeightView       // n = groups * latentDim, k = hidden
-        public let latentU: QWWeightView       // n = groups * hidden, k = latentDim
-        public let latentLabels: QWTensorValue // i32 [experts]
-        public let numLatentGroups: Int, latentDim: Int
-        public let sharedGateUp: QWWeightView?, sharedDown: QWWeightView?
-        public let sharedGateScalar: QWTensorValue?
-        public let sharedIntermediate: Int
-        public let routerBias: QWTensorValue?, routedScaleParam: QWTensorValue?
-        public let splitFeatureRouting: Bool
-    }
-    public struct GroupLatentScratch {
-        public let groupIds: QWTensorValue, pairRows: QWTensorValue     // i32 [rows, groups], [rows, topK]
-        public let onesRoute: QWTensorValue                             // f32 [rows, groups], all 1
-        public let xLatent16, zLatent16: QWTensorValue                  // f16 [rows * groups, latentDim]
-        public let naxX16, xe16: QWTensorValue                          // f16 [rows, hidden]
-        public let xRot32, xPlain32: QWTensorValue, gate: QWTensorValue
-        public let guSh32, actSh32, shared: QWTensorValue
-        public let gExpOff, gSortedPair, gSortedTok, gInvPerm, gTileE, gTileR, gTileCount: QWTensorValue?   // prefill: the (token, group) sort
-        public let rows2: QWTensorValue?, upAcc: QWTensorValue?         // prefill: i32 [rows * topK], f32 [rows * groups, hidden]
-    }
     /// QWMoEOperator.Input (QWMoEOperator.swift:12-17)
     public enum Input {
         case f16Normed(QWTensorValue)
         case f32PreRotated(plain: QWTensorValue, rotated: QWTensorValue, prefillPrecast16: QWTensorValue?)
     }
-    public static func encodeResidentGroupLatent(_ enc: QWHipEncoder, hal: QWHal, weights gw: GroupLatentWeights, scratch s: Scratch,
-                                                 groupScratch gs: GroupLatentScratch, input: Input, out32: QWTensorValue, rows T: Int) throws {
-        let w = gw.routed
-        let (H, L, NG, E, K, I, ISh) = (w.hidden, gw.latentDim, gw.numLatentGroups, w.experts, w.topK, w.intermediate, gw.sharedIntermediate)
-        guard (1...32).contains(NG), L > 0, L % 32 == 0, gw.latentD.n == NG * L, gw.latentD.k == H, gw.latentU.n == NG * H, gw.latentU.k == L,
+    /// QWMoEOperator.LatentBottleneck (QWMoEOperator.swift:26-41)
+    public struct LatentBottleneck {
+        public let fc1: QWWeightView           // n = latentDim, k = hidden
+        public let normGamma: QWTensorValue?   // f16 [latentDim], plus-one law
+        public let normEps: Float
+        public let fc2: QWWeightView           // n = hidden, k = latentDim
+        public let latentDim: Int
+        public init(fc1: QWWeightView, normGamma: QWTensorValue?, normEps: Float = 1e-6, fc2: QWWeightView, latentDim: Int) {
+            self.fc1 = fc1; self.normGamma = normGamma; self.normEps = normEps; self.fc2 = fc2; self.latentDim = latentDim
+        }
+    }
+    /// QWMoEOperator.LatentScratch (QWMoEOperator.swift:44-54): f32 [rows, latentDim] twice; bufB16 f16 [rows, latentDim] is
+    /// required here (the routed experts read f16 rows at every row count).
+    public struct LatentScratch {
+        public let bufA32: QWTensorValue, bufB32: QWTensorValue
+        public let bufB16: QWTensorValue?
+        public init(bufA32: QWTensorValue, bufB32: QWTensorValue, bufB16: QWTensorValue? = nil) {
+            self.bufA32 = bufA32; self.bufB32 = bufB32; self.bufB16 = bufB16
+        }
+    }
+    /// QWMoEOperator.Weights (QWMoEOperator.swift:57-128).
+    public struct Weights {
+        public let router: QWTensorValue                 // [experts (x 2 with splitFeatureRouting), hidden] f32 / f16 / bf16
+        public let routerBias: QWTensorValue?, routedScaleParam: QWTensorValue?
+        public let splitFeatureRouting: Bool
+        public let gateUp: QWWeightView                  // n = experts * 2 * intermediate, k = hidden (latentDim on the latent forms)
+        public let down: QWWeightView                    // n = experts * hidden (latentDim), k = intermediate
+        public let coldGateUp: QWWeightView?, coldDown: QWWeightView?      // tiered banks: refused when set
+        public let sharedGateUp: QWWeightView?, sharedDown: QWWeightView?
+        public let sharedGateScalar: QWTensorValue?      // f32 [hidden]
+        public let latent: LatentBottleneck?
+        public let latentD: QWWeightView?, latentU: QWWeightView?          // n = groups * latentDim, k = hidden; n = groups * hidden, k = latentDim
+        public let latentLabels: QWTensorValue?          // i32 [experts]
+        public let numLatentGroups: Int, latentDim: Int
+        public let hidden: Int, experts: Int, topK: Int, intermediate: Int, sharedIntermediate: Int
+        public let normTopK: Bool
+        public let reuseExpertsAcrossTokens: Bool        // taken; the caches already serve an expert shared by verify rows once
+        public let moeSpecExpertBudget: Int
+        public let routedScale: Float
+        public init(router: QWTensorValue, routerBias: QWTensorValue? = nil, routedScaleParam: QWTensorValue? = nil,
+                    splitFeatureRouting: Bool = false, gateUp: QWWeightView, down: QWWeightView,
+                    coldGateUp: QWWeightView? = nil, coldDown: QWWeightView? = nil,
+                    sharedGateUp: QWWeightView? = nil, sharedDown: QWWeightView? = nil, sharedGateScalar: QWTensorValue? = nil,
+                    latent: LatentBottleneck? = nil, latentD: QWWeightView? = nil, latentU: QWWeightView? = nil,
+                    latentLabels: QWTensorValue? = nil, numLatentGroups: Int = 0, latentDim: Int = 0,
+                    hidden: Int, experts: Int, topK: Int, intermediate: Int, sharedIntermediate: Int,
+                    normTopK: Bool = true, reuseExpertsAcrossTokens: Bool = true, moeSpecExpertBudget: Int = 0, routedScale: Float = 1) {
+            self.router = router; self.routerBias = routerBias; self.routedScaleParam = routedScaleParam
+            self.splitFeatureRouting = splitFeatureRouting; self.gateUp = gateUp; self.down = down
+            self.coldGateUp = coldGateUp; self.coldDown = coldDown
+            self.sharedGateUp = sharedGateUp; self.sharedDown = sharedDown; self.sharedGateScalar = sharedGateScalar
+            self.latent = latent; self.latentD = latentD; self.latentU = latentU; self.latentLabels = latentLabels
+            self.numLatentGroups = numLatentGroups; self.latentDim = latentDim
+            self.hidden = hidden; self.experts = experts; self.topK = topK; self.intermediate = intermediate
+            self.sharedIntermediate = sharedIntermediate; self.normTopK = normTopK
+            self.reuseExpertsAcrossTokens = reuseExpertsAcrossTokens; self.moeSpecExpertBudget = moeSpecExpertBudget
+            self.routedScale = routedScale
+        }
+        var isGroupLatent: Bool { numLatentGroups > 0 && latentDim > 0 && latentD != nil && latentU != nil && latentLabels != nil }
+        var sharedBanks: (QWWeightView, QWWeightView)? {
+            if sharedIntermediate > 0, let gu = sharedGateUp, let dn = sharedDown { return (gu, dn) } else { return nil }
+        }
+    }
+    /// What the group-latent prefill needs beyond the reference's scratch: the counting sort of the (token, group) pairs, the
+    /// gather rows of the expert GEMM and the up-projection's rows.  Without it that form runs its row counts eight at a time
+    /// on the routed GEMVs.
+    public struct HipScratch {
+        public let gExpOff, gSortedPair, gSortedTok, gInvPerm, gTileE, gTileR, gTileCount: QWTensorValue   // i32, as expOff ... tileCount
+        public let rows2: QWTensorValue        // i32 [rows * topK]
+        public let upAcc: QWTensorValue        // f32 [rows * groups, hidden]
+        public init(gExpOff: QWTensorValue, gSortedPair: QWTensorValue, gSortedTok: QWTensorValue, gInvPerm: QWTensorValue,
+                    gTileE: QWTensorValue, gTileR: QWTensorValue, gTileCount: QWTensorValue, rows2: QWTensorValue, upAcc: QWTensorValue) {
+            self.gExpOff = gExpOff; self.gSortedPair = gSortedPair; self.gSortedTok = gSortedTok; self.gInvPerm = gInvPerm
+            self.gTileE = gTileE; self.gTileR = gTileR; self.gTileCount = gTileCount; self.rows2 = rows2; self.upAcc = upAcc
+        }
+    }
+    /// QWMoEOperator.Scratch (QWMoEOperator.swift:131-192), field for field.  This library's kernels keep their intermediates in
+    /// f16 and use the reference's regions for them: the SwiGLU activations [rows * topK, intermediate] live in gu16 (else in
+    /// act32), the latent rows of the group form in xLatent16 and zLatent32, the route -> latent-row table in gu32.
+    public struct Scratch {
+        public let xRot32, xPlain32: QWTensorValue       // f32 [rows, hidden]
+        public let logits, idx, wts: QWTensorValue       // f32 [rows, routerCols], i32 [rows, topK], f32 [rows, topK]
+        public let gu32, act32: QWTensorValue            // f32 [rows * topK, 2 * intermediate], [rows * topK, intermediate]
+        public let guSh32, actSh32: QWTensorValue?
+        public let shared, gate: QWTensorValue           // f32 [rows, hidden], f32 [rows]
+        public let expOff, sortedPair, sortedTok, invPerm, tileE, tileR, tileCount: QWTensorValue?   // prefill only, i32
+        public let gu16, dnHi: QWTensorValue?            // prefill only
+        public let dnAcc: QWTensorValue                  // f32 [rows * topK, hidden]
+        public let naxX16, naxY16: QWTensorValue?
+        public let latent: LatentScratch?
+        public let groupIds, onesRoute, xLatent32, xLatent16, zLatent32: QWTensorValue?
+        public let maxTileWidth: Int
+        public let hip: HipScratch?
+        public init(xRot32: QWTensorValue, xPlain32: QWTensorValue, logits: QWTensorValue, idx: QWTensorValue, wts: QWTensorValue,
+                    gu32: QWTensorValue, act32: QWTensorValue, guSh32: QWTensorValue?, actSh32: QWTensorValue?,
+                    shared: QWTensorValue, gate: QWTensorValue, expOff: QWTensorValue?, sortedPair: QWTensorValue?,
+                    sortedTok: QWTensorValue?, invPerm: QWTensorValue?, tileE: QWTensorValue?, tileR: QWTensorValue?,
+                    tileCount: QWTensorValue?, gu16: QWTensorValue?, dnHi: QWTensorValue?, dnAcc: QWTensorValue,
+                    naxX16: QWTensorValue?, naxY16: QWTensorValue? = nil, latent: LatentScratch? = nil,
+                    groupIds: QWTensorValue? = nil, onesRoute: QWTensorValue? = nil, xLatent32: QWTensorValue? = nil,
+                    xLatent16: QWTensorValue? = nil, zLatent32: QWTensorValue? = nil, maxTileWidth: Int, hip: HipScratch? = nil) {
+            self.xRot32 = xRot32; self.xPlain32 = xPlain32; self.logits = logits; self.idx = idx; self.wts = wts
+            self.gu32 = gu32; self.act32 = act32; self.guSh32 = guSh32; self.actSh32 = actSh32; self.shared = shared; self.gate = gate
+            self.expOff = expOff; self.sortedPair = sortedPair; self.sortedTok = sortedTok; self.invPerm = invPerm
+            self.tileE = tileE; self.tileR = tileR; self.tileCount = tileCount; self.gu16 = gu16; self.dnHi = dnHi; self.dnAcc = dnAcc
+            self.naxX16 = naxX16; self.naxY16 = naxY16; self.latent = latent; self.groupIds = groupIds; self.onesRoute = onesRoute
+            self.xLatent32 = xLatent32; self.xLatent16 = xLatent16; self.zLatent32 = zLatent32; self.maxTileWidth = maxTileWidth
+            self.hip = hip
+        }
+        /// f16 [pairs, intermediate] inside gu16 (f16 [pairs, 2 * intermediate]) or act32 (f32 [pairs, intermediate]).
+        func act16(pairs: Int, intermediate: Int) -> QWTensorValue {
+            (gu16 ?? act32).slice(byteOffset: 0, count: pairs * intermediate, dtype: .f16)
+        }
+        /// The prefill sort's arrays, all present or none.
+        var sort: (expOff: QWTensorValue, pair: QWTensorValue, tok: QWTensorValue, inv: QWTensorValue, tileE: QWTensorValue,
+                   tileR: QWTensorValue, count: QWTensorValue, dnHi: QWTensorValue)? {
+            if let a = expOff, let b = sortedPair, let c = sortedTok, let d = invPerm, let e = tileE, let f = tileR, let g = tileCount,
+               let h = dnHi { return (a, b, c, d, e, f, g, h) } else { return nil }
+        }
+    }
+
+    /// The operator's input in the three forms its stages read: f16 rows in the experts' basis, f32 un-rotated rows for the router,
+    /// f32 rows in the basis for the dense shared-expert and latent projections (QWMoEOperator.swift:252-272).
+    static func resolve(_ enc: QWHipEncoder, hal: QWHal, scratch s: Scratch, input: Input, rows T: Int, hidden H: Int,
+                        needRot32: Bool) throws -> (x16: QWTensorValue, plain: QWTensorValue, rot32: QWTensorValue) {
+        switch input {
+        case .f16Normed(let x16):
+            try QWGemm.encodeMoEBridgeF16ToF32(enc, hal: hal, x: x16, xRot32: s.xRot32, xPlain32: s.xPlain32, rows: T, hidden: H,
+                                               skipRot32: !needRot32)
+            return (x16, s.xPlain32, s.xRot32)
+        case .f32PreRotated(let plain, let rotated, let precast16):
+            if let p16 = precast16 { return (p16, plain, rotated) }
+            guard let x16 = s.naxX16, x16.elementCount >= T * H else { throw QWGemmError.badShape("moe: f32 input needs scratch.naxX16 f16 [rows, hidden]") }
+            try QWGemm.encodeCast(enc, hal: hal, x32: rotated, y16: x16, count: T * H)
+            return (x16.slice(byteOffset: 0, count: T * H, dtype: .f16), plain, rotated)
+        }
+    }
+    /// The shared expert on the hidden width (QWMoEOperator.swift:300-340): shared = Wd_sh . silu_mul(Wgu_sh . x).
+    /// The f16 rows of the input serve as the gate|up projection's cast; the down projection stages its cast behind them in
+    /// naxX16 when the input's f16 rows live there (an f32 input without a precast), as the reference's shAct16 alias does.
+    static func encodeShared(_ enc: QWHipEncoder, hal: QWHal, weights w: Weights, scratch s: Scratch,
+                             x r: (x16: QWTensorValue, plain: QWTensorValue, rot32: QWTensorValue), rows T: Int) throws -> Bool {
+        guard let (shGU, shDown) = w.sharedBanks else { return false }
+        guard let guSh = s.guSh32, let actSh = s.actSh32, let nax = s.naxX16 else { throw QWGemmError.badShape("moe: the shared expert needs guSh32, actSh32 and naxX16") }
+        let held = r.x16.region.ptr == nax.region.ptr ? T * w.hidden : 0
+        let stage = nax.slice(byteOffset: held * 2, count: max(0, nax.elementCount - held))
+        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shGU, x: r.rot32, y: guSh, naxX16: stage, naxY16: s.naxY16 ?? stage, maxTileWidth: s.maxTileWidth,
+                                      rows: T, x16Precast: r.x16)
+        try QWGemm.encodeSiluMulF32(enc, hal: hal, gu: guSh, act: actSh, rows: T, intermediate: w.sharedIntermediate)
+        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shDown, x: actSh, y: s.shared, naxX16: stage, naxY16: s.naxY16 ?? stage, maxTileWidth: s.maxTileWidth,
+                                      rows: T)
+        return true
+    }
+    /// out32 / out16 / skipOut32 (QWMoEOperator.swift:200-204): where the last stage stores, and the f16 copy made afterwards.
+    static func finish(_ enc: QWHipEncoder, hal: QWHal, out32: QWTensorValue, out16: QWTensorValue?, wrote: QWTensorValue, count: Int) throws {
+        if let o16 = out16, wrote.dtype == .f32 { try QWGemm.encodeCast(enc, hal: hal, x32: out32, y16: o16, count: count) }
+    }
+
+    /// QWMoEOperator.encodeResident (QWMoEOperator.swift:195-442).  rows > 8 with the sort's scratch present runs the grouped path
+    /// (route -> pair sort -> gate_up GEMM with SwiGLU fused -> down GEMM -> combine); otherwise the routed GEMVs, eight rows a launch.
+    public static func encodeResident(_ enc: inout QWHipEncoder, hal: QWHal, weights w: Weights, scratch s: Scratch, input: Input,
+                                      out32: QWTensorValue, out16: QWTensorValue? = nil, skipOut32: Bool = false, rows T: Int,
+                                      supportsGroupedNaxPrefill: Bool = true, concurrentBarriers: Bool = false,
+                                      rotateEncoder: ((inout QWHipEncoder) throws -> Void)? = nil,
+                                      profileStage: ((String) -> QWHipEncoder?)? = nil) throws {
+        guard w.coldGateUp == nil, w.coldDown == nil else { throw QWGemmError.badWeights("moe: tiered (cold) expert banks have no kernel in this library") }
+        if let latent = w.latent {
+            try encodeResidentLatent(&enc, hal: hal, weights: w, latent: latent, scratch: s, input: input, out32: out32, out16: out16,
+                                     skipOut32: skipOut32, rows: T, supportsGroupedNaxPrefill: supportsGroupedNaxPrefill,
+                                     concurrentBarriers: concurrentBarriers, rotateEncoder: rotateEncoder, profileStage: profileStage)
+            return
+        }
+        if w.isGroupLatent {
+            try encodeResidentGroupLatent(&enc, hal: hal, weights: w, scratch: s, input: input, out32: out32, out16: out16,
+                                          skipOut32: skipOut32, rows: T, supportsGroupedNaxPrefill: supportsGroupedNaxPrefill,
+                                          concurrentBarriers: concurrentBarriers, rotateEncoder: rotateEncoder, profileStage: profileStage)
+            return
+        }
+        let (H, E, K, I) = (w.hidden, w.experts, w.topK, w.intermediate)
+        guard E > 0, E <= 512, K > 0, K <= 16 else { throw QWGemmError.badShape("moe: experts <= 512, routes <= 16") }
+        guard w.gateUp.n == E * 2 * I, w.gateUp.k == H, w.down.n == E * H, w.down.k == I else {
+            throw QWGemmError.badShape("moe: expert banks do not match (experts, hidden, intermediate)")
+        }
+        guard !skipOut32 || out16 != nil else { throw QWGemmError.badShape("moe: skipOut32 needs out16") }
+        let r = try resolve(enc, hal: hal, scratch: s, input: input, rows: T, hidden: H, needRot32: w.sharedBanks != nil)
+        let gateW = w.sharedBanks != nil ? w.sharedGateScalar : nil
+        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: r.plain, y: s.logits, rows: T, n: w.splitFeatureRouting ? 2 * E : E, k: H,
+                                      shGateWeight: gateW, shGateOut: gateW != nil ? s.gate : nil)
+        let hasShared = try encodeShared(enc, hal: hal, weights: w, scratch: s, x: r, rows: T)
+        let shared = hasShared ? s.shared : nil, gate = gateW != nil ? s.gate : nil
+        let dst = skipOut32 ? out16! : out32          // the combine stores either type
+        let pairs = T * K
+        let act16 = s.act16(pairs: pairs, intermediate: I)
+        let plainRoute = w.routerBias == nil && w.routedScaleParam == nil && !w.splitFeatureRouting && w.moeSpecExpertBudget == 0
+        if T > 8, supportsGroupedNaxPrefill, let q = s.sort, H % 64 == 0, I % 64 == 0 {
+            try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
+                                        bias: w.routerBias, splitFeature: w.splitFeatureRouting, routedScaleParam: w.routedScaleParam,
+                                        routedScale: w.routedScale)
+            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: q.expOff, sortedPairIdx: q.pair, sortedTok: q.tok, experts: E,
+                                              totalPairs: pairs, routes: K, invPerm: q.inv, tileE: q.tileE, tileR: q.tileR, tileCount: q.count)
+            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: r.x16, bank: w.gateUp, experts: E, sortedTok: q.tok, expertOff: q.expOff, tileE: q.tileE,
+                                             tileR: q.tileR, tileCount: q.count, act16: act16, pairs: pairs, rotateAct: w.down.isRotated)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: act16, bank: w.down, experts: E, expertOff: q.expOff, tileE: q.tileE, tileR: q.tileR,
+                                            tileCount: q.count, y: q.dnHi, pairs: pairs)
+            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: q.dnHi, invPerm: q.inv, weights: s.wts, shared: shared, gate: gate,
+                                                     out: dst, hidden: H, routes: K, tokens: T)
+        } else {
+            if !plainRoute {
+                try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
+                                            bias: w.routerBias, expertBudget: w.moeSpecExpertBudget, splitFeature: w.splitFeatureRouting,
+                                            routedScaleParam: w.routedScaleParam, routedScale: w.routedScale)
+            }
+            var t0 = 0
+            while t0 < T {                            // the routed GEMVs take at most eight rows a launch
+                let tc = min(8, T - t0)
+                let x = r.x16.slice(byteOffset: t0 * H * 2, count: tc * H)
+                let idx = s.idx.slice(byteOffset: t0 * K * 4, count: tc * K), wts = s.wts.slice(byteOffset: t0 * K * 4, count: tc * K)
+                let act = act16.slice(byteOffset: t0 * K * I * 2, count: tc * K * I)
+                if plainRoute {
+                    let cols = E
+                    try QWGemm.encodeMoERouteGateUp(enc, hal: hal, x: x, bank: w.gateUp, experts: E, logits: s.logits.slice(byteOffset: t0 * cols * 4, count: tc * cols),
+                                                    idx: idx, wts: wts, out: act, routes: K, tokens: tc, normTopK: w.normTopK, routedScale: w.routedScale)
+                } else {
+                    try QWGemm.encodeMoEGateUpF32R1(enc, hal: hal, x: x, bank: w.gateUp, ids: idx, out: act, rowsPerExpert: 2 * I, routes: K, tokens: tc,
+                                                    fuseSiluFwht: true)
+                }
+                try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: act, bank: w.down, rowsPerRoute: H, routes: K, weights: wts,
+                                                         shared: shared?.slice(byteOffset: t0 * H * 4, count: tc * H),
+                                                         gate: gate?.slice(byteOffset: t0 * 4, count: tc),
+                                                         out: dst.slice(byteOffset: t0 * H * dst.dtype.bytes, count: tc * H), ids: idx, tokens: tc)
+                t0 += tc
+            }
+        }
+        try finish(enc, hal: hal, out32: out32, out16: skipOut32 ? nil : out16, wrote: dst, count: T * H)
+    }
+
+    /// QWMoEOperator.encodeResidentLatent (QWMoEOperator+Latent.swift:17-303): fc1 -> route -> rotate -> routed experts in the latent
+    /// width -> latent norm -> fc2, the shared expert on the hidden width added under its gate.  out32 is this form's working
+    /// buffer and is written also under skipOut32.
+    public static func encodeResidentLatent(_ enc: inout QWHipEncoder, hal: QWHal, weights w: Weights, latent: LatentBottleneck, scratch s: Scratch,
+                                            input: Input, out32: QWTensorValue, out16: QWTensorValue?, skipOut32: Bool = false, rows T: Int,
+                                            supportsGroupedNaxPrefill: Bool, concurrentBarriers: Bool,
+                                            rotateEncoder: ((inout QWHipEncoder) throws -> Void)?, profileStage: ((String) -> QWHipEncoder?)?) throws {
+        let (H, L, E, K, I) = (w.hidden, latent.latentDim, w.experts, w.topK, w.intermediate)
+        guard L > 0, L % 32 == 0, latent.fc1.n == L, latent.fc1.k == H, latent.fc2.n == H, latent.fc2.k == L,
+              w.gateUp.n == E * 2 * I, w.gateUp.k == L, w.down.n == E * L, w.down.k == I else {
+            throw QWGemmError.badShape("latent moe: banks do not match (hidden, latent, experts, intermediate)")
+        }
+        guard let ls = s.latent, let bufB16 = ls.bufB16, let nax = s.naxX16 else { throw QWGemmError.badShape("latent moe: scratch.latent (with bufB16) and naxX16 are required") }
+        guard !skipOut32 || out16 != nil else { throw QWGemmError.badShape("moe: skipOut32 needs out16") }
+        let naxY = s.naxY16 ?? nax
+        let r = try resolve(enc, hal: hal, scratch: s, input: input, rows: T, hidden: H, needRot32: true)
+        let gateW = w.sharedBanks != nil ? w.sharedGateScalar : nil
+        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: r.plain, y: s.logits, rows: T, n: w.splitFeatureRouting ? 2 * E : E, k: H,
+                                      shGateWeight: gateW, shGateOut: gateW != nil ? s.gate : nil)
+        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: latent.fc1, x: r.rot32, y: ls.bufA32, naxX16: nax, naxY16: naxY, maxTileWidth: s.maxTileWidth, rows: T,
+                                      x16Precast: r.x16)
+        try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
+                                    bias: w.routerBias, expertBudget: w.moeSpecExpertBudget, splitFeature: w.splitFeatureRouting,
+                                    routedScaleParam: w.routedScaleParam, routedScale: w.routedScale)
+        try QWGemm.encodeLatentNormH32F32(enc, hal: hal, x: ls.bufA32, gamma: nil, out32: ls.bufB32, out16: bufB16, rows: T, latent: L, eps: latent.normEps,
+                                          skipOut32: true)
+        let hasShared = try encodeShared(enc, hal: hal, weights: w, scratch: s, x: r, rows: T)
+        let pairs = T * K
+        let act16 = s.act16(pairs: pairs, intermediate: I)
+        if T > 8, supportsGroupedNaxPrefill, let q = s.sort, L % 64 == 0, I % 64 == 0 {
+            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: q.expOff, sortedPairIdx: q.pair, sortedTok: q.tok, experts: E,
+                                              totalPairs: pairs, routes: K, invPerm: q.inv, tileE: q.tileE, tileR: q.tileR, tileCount: q.count)
+            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: bufB16, bank: w.gateUp, experts: E, sortedTok: q.tok, expertOff: q.expOff, tileE: q.tileE,
+                                             tileR: q.tileR, tileCount: q.count, act16: act16, pairs: pairs, rotateAct: w.down.isRotated)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: act16, bank: w.down, experts: E, expertOff: q.expOff, tileE: q.tileE, tileR: q.tileR,
+                                            tileCount: q.count, y: q.dnHi, pairs: pairs)
+            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: q.dnHi, invPerm: q.inv, weights: s.wts, shared: nil, gate: nil,
+                                                     out: ls.bufA32, hidden: L, routes: K, tokens: T)
+        } else {
+            var t0 = 0
+            while t0 < T {
+                let tc = min(8, T - t0)
+                let idx = s.idx.slice(byteOffset: t0 * K * 4, count: tc * K), act = act16.slice(byteOffset: t0 * K * I * 2, count: tc * K * I)
+                try QWGemm.encodeMoEGateUpF32R1(enc, hal: hal, x: bufB16.slice(byteOffset: t0 * L * 2, count: tc * L), bank: w.gateUp, ids: idx, out: act,
+                                                rowsPerExpert: 2 * I, routes: K, tokens: tc, fuseSiluFwht: true)
+                try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: act, bank: w.down, rowsPerRoute: L, routes: K,
+                                                         weights: s.wts.slice(byteOffset: t0 * K * 4, count: tc * K), shared: nil, gate: nil,
+                                                         out: ls.bufA32.slice(byteOffset: t0 * L * 4, count: tc * L), ids: idx, tokens: tc)
+                t0 += tc
+            }
+        }
+        try QWGemm.encodeLatentNormH32F32(enc, hal: hal, x: ls.bufA32, gamma: latent.normGamma, out32: ls.bufB32, out16: nil, rows: T, latent: L,
+                                          eps: latent.normEps)
+        try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: latent.fc2, x: ls.bufB32, y: out32, naxX16: nax, naxY16: naxY, maxTileWidth: s.maxTileWidth, rows: T)
+        if hasShared {
+            try QWGemm.encodeMoEAddSharedF32(enc, hal: hal, dnAcc: out32, shared: s.shared, gate: gateW != nil ? s.gate : nil, out: out32, hidden: H, tokens: T)
+        }
+        try finish(enc, hal: hal, out32: out32, out16: out16, wrote: out32, count: T * H)
+    }
+
+    /// QWMoEOperator.encodeResidentGroupLatent (QWMoEOperator+GroupLatent.swift:11-294): every token's hidden row goes down to the
+    /// latent of each group its routes touch (latentD), the routed experts run in the latent width, their outputs are summed by
+    /// group and come back up through latentU.
+    public static func encodeResidentGroupLatent(_ enc: inout QWHipEncoder, hal: QWHal, weights w: Weights, scratch s: Scratch, input: Input,
+                                                 out32: QWTensorValue, out16: QWTensorValue?, skipOut32: Bool = false, rows T: Int,
+                                                 supportsGroupedNaxPrefill: Bool, concurrentBarriers: Bool,
+                                                 rotateEncoder: ((inout QWHipEncoder) throws -> Void)?, profileStage: ((String) -> QWHipEncoder?)?) throws {
+        let (H, L, NG, E, K, I) = (w.hidden, w.latentDim, w.numLatentGroups, w.experts, w.topK, w.intermediate)
+        guard let latentD = w.latentD, let latentU = w.latentU, let labels = w.latentLabels else { throw QWGemmError.badWeights("group-latent moe: latentD, latentU and latentLabels") }
+        guard (1...32).contains(NG), L > 0, L % 32 == 0, latentD.n == NG * L, latentD.k == H, latentU.n == NG * H, latentU.k == L,
               w.gateUp.n == E * 2 * I, w.gateUp.k == L, w.down.n == E * L, w.down.k == I else {
             throw QWGemmError.badShape("group-latent moe: banks do not match (hidden, groups, latent, experts, intermediate)")
         }
-        let x16: QWTensorValue, xPlain: QWTensorValue, xRot: QWTensorValue
-        switch input {
-        case .f16Normed(let x):
-            try QWGemm.encodeMoEBridgeF16ToF32(enc, hal: hal, x: x, xRot32: gs.xRot32, xPlain32: gs.xPlain32, rows: T, hidden: H)
-            (x16, xPlain, xRot) = (x, gs.xPlain32, gs.xRot32)
-        case .f32PreRotated(let plain, let rotated, let precast16):
-            if let p16 = precast16 { x16 = p16 } else {
-                try QWGemm.encodeCast(enc, hal: hal, src32: rotated, dst16: gs.xe16, count: T * H)
-                x16 = gs.xe16
-            }
-            (xPlain, xRot) = (plain, rotated)
+        guard let groupIds = s.groupIds, let onesRoute = s.onesRoute, let xLat = s.xLatent16, let zLat32 = s.zLatent32 else {
+            throw QWGemmError.badShape("group-latent moe: scratch groupIds, onesRoute, xLatent16 and zLatent32 are required")
         }
-        let sharedBanks: (QWWeightView, QWWeightView)? = (ISh > 0 && gw.sharedGateUp != nil && gw.sharedDown != nil) ? (gw.sharedGateUp!, gw.sharedDown!) : nil
-        let gateW = sharedBanks != nil ? gw.sharedGateScalar : nil
-        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: xPlain, y: s.logits, rows: T, n: gw.splitFeatureRouting ? 2 * E : E, k: H,
-                                      shGateWeight: gateW, shGateOut: gateW != nil ? gs.gate : nil)
-        try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
-                                    routedScale: w.routedScale, bias: gw.routerBias, splitFeature: gw.splitFeatureRouting,
-                                    routedScaleParam: gw.routedScaleParam)
-        try QWGemm.encodeMoELatentGroups(enc, hal: hal, idx: s.idx, labels: gw.latentLabels, rows: T, topK: K, experts: E, numGroups: NG,
-                                         groupIds: gs.groupIds, pairRows: gs.pairRows)
-        if let (shGU, shDown) = sharedBanks {
-            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shGU, x: xRot, y: gs.guSh32, naxX16: gs.naxX16, rows: T)
-            try QWGemm.encodeSiluMulF32(enc, hal: hal, gu: gs.guSh32, act: gs.actSh32, rows: T, inter: ISh)
-            try QWGemm.encodeDenseProjF32(enc, hal: hal, weight: shDown, x: gs.actSh32, y: gs.shared, naxX16: gs.naxX16, rows: T)
-        }
-        let shared = sharedBanks != nil ? gs.shared : nil, gate = gateW != nil ? gs.gate : nil
+        guard !skipOut32 || out16 != nil else { throw QWGemmError.badShape("moe: skipOut32 needs out16") }
         let (pairs, gpairs) = (T * K, T * NG)
-        if T > 8, H % 64 == 0, L % 64 == 0, I % 64 == 0, let expOff = s.expOff, let sortedPair = s.sortedPair, let sortedTok = s.sortedTok,
-           let invPerm = s.invPerm, let tileE = s.tileE, let tileR = s.tileR, let tileCount = s.tileCount, let dnHi = s.dnHi,
-           let gOff = gs.gExpOff, let gPair = gs.gSortedPair, let gTok = gs.gSortedTok, let gInv = gs.gInvPerm, let gTE = gs.gTileE, let gTR = gs.gTileR,
-           let gTC = gs.gTileCount, let rows2 = gs.rows2, let upAcc = gs.upAcc {
-            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: gs.groupIds, expertOff: gOff, sortedPairIdx: gPair, sortedTok: gTok, experts: NG,
-                                              totalPairs: gpairs, routes: NG, invPerm: gInv, tileE: gTE, tileR: gTR, tileCount: gTC)
-            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: x16, bank: gw.latentD, experts: NG, expertOff: gOff, tileE: gTE, tileR: gTR, tileCount: gTC,
-                                            y: gs.xLatent16, pairs: gpairs, sortedTok: gTok)
-            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: expOff, sortedPairIdx: sortedPair, sortedTok: sortedTok, experts: E,
-                                              totalPairs: pairs, routes: K, invPerm: invPerm, tileE: tileE, tileR: tileR, tileCount: tileCount)
-            try QWGemm.encodeMoEComposeRows(enc, hal: hal, sortedPair: sortedPair, pairs: pairs, pairRows: gs.pairRows, rowCount: gpairs, slotOfRow: gInv,
-                                            rowsOut: rows2)
-            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: gs.xLatent16, bank: w.gateUp, experts: E, sortedTok: rows2, expertOff: expOff, tileE: tileE,
-                                             tileR: tileR, tileCount: tileCount, act16: s.act16, pairs: pairs, rotateAct: w.down.isRotated)
-            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: s.act16, bank: w.down, experts: E, expertOff: expOff, tileE: tileE, tileR: tileR,
-                                            tileCount: tileCount, y: dnHi, pairs: pairs)
-            try QWGemm.encodeMoECombineGroupsF32(enc, hal: hal, dnAcc: dnHi, invPerm: invPerm, weights: s.wts, ids: s.idx, labels: gw.latentLabels,
-                                                 tokens: T, routes: K, numGroups: NG, width: L, out: gs.zLatent16)
-            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: gs.zLatent16, bank: gw.latentU, experts: NG, expertOff: gOff, tileE: gTE, tileR: gTR,
-                                            tileCount: gTC, y: upAcc, pairs: gpairs, sortedTok: gPair)
-            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: upAcc, invPerm: gInv, weights: gs.onesRoute, shared: shared, gate: gate,
-                                                     out: out32, hidden: H, routes: NG, tokens: T)
+        let zLat = zLat32.slice(byteOffset: 0, count: gpairs * L, dtype: .f16)          // f16 [rows * groups, latentDim]
+        let pairRows = s.gu32.slice(byteOffset: 0, count: pairs, dtype: .i32)           // i32 [rows, topK]
+        let r = try resolve(enc, hal: hal, scratch: s, input: input, rows: T, hidden: H, needRot32: w.sharedBanks != nil)
+        let gateW = w.sharedBanks != nil ? w.sharedGateScalar : nil
+        try QWGemm.encodeFnRouterGemm(enc, hal: hal, weight: w.router, x: r.plain, y: s.logits, rows: T, n: w.splitFeatureRouting ? 2 * E : E, k: H,
+                                      shGateWeight: gateW, shGateOut: gateW != nil ? s.gate : nil)
+        try QWGemm.encodeFnMoeRoute(enc, hal: hal, logits: s.logits, idx: s.idx, wts: s.wts, rows: T, experts: E, topK: K, normTopK: w.normTopK,
+                                    bias: w.routerBias, expertBudget: w.moeSpecExpertBudget, splitFeature: w.splitFeatureRouting,
+                                    routedScaleParam: w.routedScaleParam, routedScale: w.routedScale)
+        try QWGemm.encodeMoELatentGroups(enc, hal: hal, idx: s.idx, labels: labels, rows: T, topK: K, experts: E, numGroups: NG,
+                                         groupIds: groupIds, pairRows: pairRows)
+        let hasShared = try encodeShared(enc, hal: hal, weights: w, scratch: s, x: r, rows: T)
+        let shared = hasShared ? s.shared : nil, gate = gateW != nil ? s.gate : nil
+        let dst = skipOut32 ? out16! : out32
+        let act16 = s.act16(pairs: pairs, intermediate: I)
+        if T > 8, supportsGroupedNaxPrefill, H % 64 == 0, L % 64 == 0, I % 64 == 0, let q = s.sort, let g = s.hip {
+            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: groupIds, expertOff: g.gExpOff, sortedPairIdx: g.gSortedPair, sortedTok: g.gSortedTok,
+                                              experts: NG, totalPairs: gpairs, routes: NG, invPerm: g.gInvPerm, tileE: g.gTileE, tileR: g.gTileR,
+                                              tileCount: g.gTileCount)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: r.x16, bank: latentD, experts: NG, expertOff: g.gExpOff, tileE: g.gTileE, tileR: g.gTileR,
+                                            tileCount: g.gTileCount, y: xLat, pairs: gpairs, sortedTok: g.gSortedTok)
+            try QWGemm.encodeMoEGroupPairsF32(enc, hal: hal, ids: s.idx, expertOff: q.expOff, sortedPairIdx: q.pair, sortedTok: q.tok, experts: E,
+                                              totalPairs: pairs, routes: K, invPerm: q.inv, tileE: q.tileE, tileR: q.tileR, tileCount: q.count)
+            try QWGemm.encodeMoEComposeRows(enc, hal: hal, sortedPair: q.pair, pairs: pairs, pairRows: pairRows, rowCount: gpairs, slotOfRow: g.gInvPerm,
+                                            rowsOut: g.rows2)
+            try QWGemm.encodeMoEGateUpSwiglu(enc, hal: hal, xe: xLat, bank: w.gateUp, experts: E, sortedTok: g.rows2, expertOff: q.expOff, tileE: q.tileE,
+                                             tileR: q.tileR, tileCount: q.count, act16: act16, pairs: pairs, rotateAct: w.down.isRotated)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: act16, bank: w.down, experts: E, expertOff: q.expOff, tileE: q.tileE, tileR: q.tileR,
+                                            tileCount: q.count, y: q.dnHi, pairs: pairs)
+            try QWGemm.encodeMoECombineGroupsF32(enc, hal: hal, dnAcc: q.dnHi, invPerm: q.inv, weights: s.wts, ids: s.idx, labels: labels,
+                                                 tokens: T, routes: K, numGroups: NG, width: L, out: zLat)
+            try QWGemm.encodeMoEGroupedGemm(enc, hal: hal, xe: zLat, bank: latentU, experts: NG, expertOff: g.gExpOff, tileE: g.gTileE, tileR: g.gTileR,
+                                            tileCount: g.gTileCount, y: g.upAcc, pairs: gpairs, sortedTok: g.gSortedPair)
+            try QWGemm.encodeMoEDownReduceCombineF32(enc, hal: hal, dnAcc: g.upAcc, invPerm: g.gInvPerm, weights: onesRoute, shared: shared, gate: gate,
+                                                     out: dst, hidden: H, routes: NG, tokens: T)
         } else {
-            try QWGemm.encodeMoERoutedGemv(enc, hal: hal, bank: gw.latentD, experts: NG, x16: x16, xPerToken: true, ids: gs.groupIds, weights: nil,
-                                           tokens: T, routes: NG, out: gs.xLatent16)
-            try QWGemm.encodeMoEGateUpRowsF32R1(enc, hal: hal, x: gs.xLatent16, bank: w.gateUp, experts: E, ids: s.idx, xRows: gs.pairRows, out: s.act16,
-                                                routes: K, tokens: T)
-            try QWGemm.encodeMoEDownGroupsF32(enc, hal: hal, x: s.act16, bank: w.down, experts: E, ids: s.idx, weights: s.wts, labels: gw.latentLabels,
-                                              numGroups: NG, tokens: T, routes: K, out: gs.zLatent16)
-            try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: gs.zLatent16, bank: gw.latentU, experts: NG, routes: NG, weights: gs.onesRoute,
-                                                     shared: shared, gate: gate, out: out32, ids: gs.groupIds, tokens: T)
+            var t0 = 0
+            while t0 < T {
+                let tc = min(8, T - t0)
+                let idx = s.idx.slice(byteOffset: t0 * K * 4, count: tc * K), wts = s.wts.slice(byteOffset: t0 * K * 4, count: tc * K)
+                let gids = groupIds.slice(byteOffset: t0 * NG * 4, count: tc * NG), ones = onesRoute.slice(byteOffset: t0 * NG * 4, count: tc * NG)
+                let act = act16.slice(byteOffset: t0 * K * I * 2, count: tc * K * I)
+                // a chunk's latent rows start at row 0 of its own slices: the route -> row table is rebuilt per chunk
+                let rowsOfChunk = pairRows.slice(byteOffset: t0 * K * 4, count: tc * K)
+                if t0 > 0 {
+                    try QWGemm.encodeMoELatentGroups(enc, hal: hal, idx: idx, labels: labels, rows: tc, topK: K, experts: E, numGroups: NG,
+                                                     groupIds: gids, pairRows: rowsOfChunk)
+                }
+                let xl = xLat.slice(byteOffset: t0 * NG * L * 2, count: tc * NG * L), zl = zLat.slice(byteOffset: t0 * NG * L * 2, count: tc * NG * L)
+                try QWGemm.encodeMoERoutedGemv(enc, hal: hal, bank: latentD, experts: NG, x16: r.x16.slice(byteOffset: t0 * H * 2, count: tc * H),
+                                               xPerToken: true, ids: gids, weights: nil, tokens: tc, routes: NG, out: xl)
+                try QWGemm.encodeMoEGateUpRowsF32R1(enc, hal: hal, x: xl, bank: w.gateUp, experts: E, ids: idx, xRows: rowsOfChunk, out: act,
+                                                    routes: K, tokens: tc)
+                try QWGemm.encodeMoEDownGroupsF32(enc, hal: hal, x: act, bank: w.down, experts: E, ids: idx, weights: wts, labels: labels,
+                                                  numGroups: NG, tokens: tc, routes: K, out: zl)
+                try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: zl, bank: latentU, rowsPerRoute: H, routes: NG, weights: ones,
+                                                         shared: shared?.slice(byteOffset: t0 * H * 4, count: tc * H),
+                                                         gate: gate?.slice(byteOffset: t0 * 4, count: tc),
+                                                         out: dst.slice(byteOffset: t0 * H * dst.dtype.bytes, count: tc * H), ids: gids, tokens: tc)
+                t0 += tc
+            }
         }
+        try finish(enc, hal: hal, out32: out32, out16: skipOut32 ? nil : out16, wrote: dst, count: T * H)
     }
 }

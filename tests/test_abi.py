@@ -88,6 +88,7 @@ def test_kernel_lookup_keys_are_the_reference_kernel_names():
         b"qwg_gemm_q4g_h16": b"qwhip_gemm", b"qwg_gemm_aq8_g32_h16": b"qwhip_gemm", b"qwg_gemm_aq4_g64_nax_f32": b"qwhip_gemm",
         b"qwg_moe_route": b"qwhip_moe_route", b"qwg_moe_group_pairs_f32": b"qwhip_moe_group_pairs",
         b"qwg_moe_nax_gemm": b"qwhip_moe_grouped_gemm", b"qwg_moe_nax_split_f32_aq4_g64": b"qwhip_moe_grouped_gemm",
+        b"qwg_moe_nax_split_aq4_g64_f32": b"qwhip_moe_grouped_gemm", b"qwg_head_gemv_aq4_g32_argmax": b"qwhip_head_argmax",
         b"qwg_moe_down_reduce_combine_f32": b"qwhip_moe_combine", b"qwg_moe_gateup_q4g_f32_r1": b"qwhip_moe_gateup_decode",
         b"qwg_moe_down_shared_combine_q4g_f32": b"qwhip_moe_down_decode", b"qwg_fwht32_f16": b"qwhip_fwht32",
         b"qwg_quantize_bf16_to_hq4_g32_m5": b"qwhip_quantize_hq4_g32",
@@ -144,4 +145,10 @@ def test_swift_shim_resolves_only_kernel_names_the_library_knows():
     assert missing == {"mpsgraph_bmm_f16", "qwg_gemv_f16_v4"}
     for templ in re.findall(r'"(qwg_[a-z0-9_]*\\\(bank\.bits\)_g\\\(bank\.groupSize\)[a-z0-9_]*)"', text):
         name = templ.replace("\\(bank.bits)", "8").replace("\\(bank.groupSize)", "64")
+        assert lib.qwhip_kernel_lookup(name.encode(), None) == qwhip.OK, name
+    # the name builders of QWGemmAQ: name("head", bits, group, "tail", isSHVQ) -> head_aq<bits>_g<group>tail
+    built = re.findall(r'name\("(qwg_[a-z0-9_]+)", bits, group, "([a-z0-9_]*)", isSHVQ\)', text)
+    assert len(built) >= 15
+    for head, tail in built:
+        name = f"{head}_aq6_g128{tail}"
         assert lib.qwhip_kernel_lookup(name.encode(), None) == qwhip.OK, name
