@@ -1169,9 +1169,15 @@ static qwhip_status qw_gemv_impl(qwhip_stream_t s, const qwhip_weight_view* w, c
     // dequantization per weight whatever m is), so it takes over where rows are long and few and m is large: N = 5120,
     // K = 17408, HQ4_G64 measured 18.7 / 18.7 / 20.7 us at m = 6 / 8 / 16 against 21.2 / 23.2 / 34.9 for the kernels below
     // (16.7 against 18.6 at m = 4); on K = 5120 banks (N = 7168 HQ8, N = 17408 or 5120 HQ4) the kernels below stay ahead.
-    if (variant == 9 || (variant == 0 && !rotate && m >= 6 && w->k >= 8192 && fmt != QW_FMT_B8)) {
+    // 13..16 rows on an 8-bit stream of short rows take it too, four waves a workgroup, four groups in flight, the image in
+    // 128 KiB (tuning code 60): two K ranges and the second launch, 15.7 us on N = 7168, K = 5120 against 16.9 for the
+    // transposing kernel and 17.7 for the 4x4x4-block kernel.
+    const bool sk_long = !rotate && m >= 6 && w->k >= 8192 && fmt != QW_FMT_B8;
+    const bool sk_wide8 = !rotate && m >= 13 && w->k < 8192 && fmt == QW_FMT_B8;
+    if (variant == 9 || (variant == 0 && (sk_long || sk_wide8))) {
         hipError_t e = hipSuccess;
-        if (!rotate && qw_sk_gemv(s, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, y16, y32, variant == 9 ? (flags >> 12) & 0x7Fu : 0u, &e)) {
+        const uint32_t sk_tune = variant == 9 ? (flags >> 12) & 0x7Fu : (sk_wide8 ? 60u : 0u);
+        if (!rotate && qw_sk_gemv(s, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, y16, y32, sk_tune, &e)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }

@@ -102,12 +102,13 @@ static __device__ __forceinline__ void run(const qq_params& p) {
             for (int c = 0; c < 4; ++c) buf[slot].q[c] = w.q[c];
         }
         i_off = min(i_off + step, off_max);
-        if (--i_left == 0u) {   // uniform over the workgroup
-            i_kr = min(i_kr + 1u, p.nkr - 1u);   // past the last range: its data again, never consumed
+        if (--i_left == 0u && i_kr + 1u < p.nkr) {   // uniform over the workgroup
+            ++i_kr;
             slice_of(i_kr, i_hdr, i_pay);
             i_off = off_first;
             i_left = nmax;
-        }
+        }   // past the last range i_off stays on the last quad: its slices again (still in the caches, never consumed), where
+            // the range's first quads, read long ago, would come from HBM a second time
     };
     // Activations of a K range: with up to eight activation rows the next range's are fetched while this one is
     // contracted (they share the registers of the raw loads); with more rows they are loaded at the range's start.
