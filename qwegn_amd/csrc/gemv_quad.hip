@@ -193,7 +193,8 @@ static __device__ __forceinline__ void run(const qq_params& p) {
                 if constexpr (FMT == QW_FMT_B8) {
 #pragma unroll
                     for (int w = 0; w < 8; ++w) {
-                        const uint32_t lo = blk.q[w] & 0x00FF00FFu, hi = (blk.q[w] >> 8) & 0x00FF00FFu;
+                        // bytes (0, 2) and (1, 3) of the word as two pairs of f16 subnormals: one mask, one byte permute
+                        const uint32_t lo = blk.q[w] & 0x00FF00FFu, hi = __builtin_amdgcn_perm(blk.q[w], blk.q[w], 0x0C030C01u);
                         const u2_t pk = {lo, hi};
                         aw[w] = __builtin_bit_cast(h4_t, pk);
                     }
@@ -216,6 +217,7 @@ static __device__ __forceinline__ void run(const qq_params& p) {
                     const h2_t hd = __builtin_bit_cast(h2_t, hq[i]);
                     sc[i] = (float)hd[0];
                     bi[i] = (float)hd[1];
+                    if constexpr (FMT == QW_FMT_B8) sc[i] *= 16777216.0f;   // the codes are f16 subnormals code * 2^-24: exact, once per header
                 }
 #pragma unroll
                 for (int mg = 0; mg < MG; ++mg) {
@@ -230,7 +232,7 @@ static __device__ __forceinline__ void run(const qq_params& p) {
                     for (int i = 0; i < 4; ++i) {
                         float q;
                         if constexpr (FMT == QW_FMT_B8) {
-                            q = (a0[i] + a1[i]) * 16777216.0f;
+                            q = a0[i] + a1[i];
                         } else {
                             q = __builtin_fmaf(a0[i], 16777216.0f, FMT == QW_FMT_M5 ? 1024.0f * S[mg] : 0.0f);
                             q = __builtin_fmaf(a1[i], 1048576.0f, q);
