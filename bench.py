@@ -33,7 +33,8 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense f16/bf16 MFMA, published
 # (FETCH_SIZE KiB x 1024 x 2.000 + WRITE_SIZE KiB x 1024 x 1.000; the factors come from a streaming kernel of known
 # size).  The passes are recorded as text under profiles/; the figure is read from the summary's line
 # "traffic = <bytes> B per launch", so the bench line cannot drift from the committed profile.
-TRAFFIC_PROFILES = {"c2": "gemv_col__c2_decode_n17408_k5120.txt", "c3": "gemm3_pingpong_256x320__c3_prefill_m4096_n5120_k5120.txt"}
+TRAFFIC_PROFILES = {"c2": "gemv_col__c2_decode_n17408_k5120.txt", "c3": "gemm3_pingpong_256x320__c3_prefill_m4096_n5120_k5120.txt",
+                    "c4_decode": "moe_decode_col__c4_decode_t1.txt", "c4_prefill": "moe_grouped_gemm__c4_prefill_t2048.txt"}
 
 
 def measured_traffic(workload: str):
@@ -776,7 +777,8 @@ def run_moe(args, t, label):
                              "note": "the same step repeated: its experts (23.6 MB per token) stay in the Infinity Cache"}
         base.update({"value": round(gbs, 2), "unit": "GB/s", "config": cfg,
                      "roofline": {"bound": "hbm", "kernel": "routed gate_up GEMV", "achieved": round(gu_gbs, 2), "peak": HBM_PEAK_GBS,
-                                  "unit": "GB/s", "frac": round(gu_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                                  "unit": "GB/s", "frac": round(gu_gbs / HBM_PEAK_GBS, 4),
+                                  "traffic": measured_traffic("c4_decode") if (t == 1 and not args.moe_tokens and not args.hot) else None,
                                   "algorithmic_bytes": gu_bytes, "kernel_us": round(us_gu, 3)}})
     else:
         valid = int((idx >= 0).sum())
@@ -785,7 +787,8 @@ def run_moe(args, t, label):
         tf, gu_tf = flops / (us_chain * 1e-6) / 1e12, gu_flops / (us_gu * 1e-6) / 1e12
         base.update({"value": round(tf, 2), "unit": "TFLOP/s", "config": cfg,
                      "roofline": {"bound": "mfma", "kernel": "grouped gate_up GEMM", "achieved": round(gu_tf, 2), "peak": MFMA_PEAK_TFLOPS,
-                                  "unit": "TFLOP/s", "frac": round(gu_tf / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                                  "unit": "TFLOP/s", "frac": round(gu_tf / MFMA_PEAK_TFLOPS, 4),
+                                  "traffic": measured_traffic("c4_prefill") if (t == 2048 and not getattr(args, "moe_f16", False)) else None,
                                   "algorithmic_flops": gu_flops, "kernel_us": round(us_gu, 3)}})
     if not args.no_cpu:
         rows_c = np.arange(min(t, 2))
