@@ -213,8 +213,9 @@ qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, 
  * (a last partial group is padded with zeros).  Up to 31 rows: four activation rows share one pass over the bank, all
  * arithmetic in fp32.  From 32 rows on (where the reference switches to its batched kernels) and k % 64 == 0: the
  * matrix-core form, 64 activation rows per pass over the bank; activations and weights are each split into two f16
- * numbers (22 bits together) and three products are accumulated in fp32 - the same 2e-5 bar, activations within the
- * f16 range (|x| <= 65504). */
+ * numbers (22 bits together) and three products are accumulated in fp32 - the same 2e-5 bar.  Every activation row is
+ * scaled by a power of two into the f16 range before its split and back at the store (one small launch into the
+ * stream's scratch), so any finite fp32 row is taken at every row count. */
 qwhip_status qwhip_gemv_f32(qwhip_stream_t s, const qwhip_weight_view* w, const float* x, uint32_t m, uint32_t epi,
                             float scale, float* y);
 
