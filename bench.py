@@ -535,6 +535,52 @@ def run_norm(args, rows, hidden, label):
     }
 
 
+def run_dense_f32(args, rows, n, k, label):
+    """Dense fp32-weight GEMV door with no epilogue: one step = one launch, y[rows, n] = x[rows, k] W[n, k]^T.
+    Algorithmic bytes: the weights once, the activation rows once, the outputs once."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+
+    dev = qwhip.Device(0)
+    rng = np.random.default_rng(0)
+    w = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    wb, xb, yb = dev.put(w), dev.put(x), dev.alloc(rows * n * 4)
+    lib, st = dev.lib, dev.stream.handle
+
+    def launch(i):
+        qwhip.check(lib.qwhip_f32_gemv(st, wb.ptr, xb.ptr, rows, n, k, 0, 1.0, yb.ptr))
+
+    launch(0)
+    dev.stream.sync()
+    err = float(qo.normalized_error(yb.download(np.float32, (rows, n)), qo.f32_gemv(w, x, 0, 1.0)))
+    if not err <= 2e-6:
+        _fail(f"bench: dense f32 gemv failed parity (normalized error {err:.3e})")
+    _spin_up(dev, launch)
+    for i in range(args.warmup):
+        launch(i)
+    dev.stream.sync()
+    e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+    e0.record(dev.stream)
+    for i in range(args.steps):
+        launch(i)
+    e1.record(dev.stream)
+    dev.stream.sync()
+    us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
+    algo_bytes = (n * k + rows * k + rows * n) * 4
+    gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": label, "rows": rows, "n": n, "k": k, "weights": "hot (one resident matrix)"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": algo_bytes, "kernel_us": round(us_per, 3)},
+        "normalized_error": err,
+    }
+
+
 def run_gemm(args, fmt, n, k, m, label, traffic=None):
     """Prefill GEMM: X bf16 [m, k] in the container's basis -> Y bf16 [m, n]; one step = one launch."""
     from oracle import qworacle as qo
@@ -778,7 +824,7 @@ def run_moe(args, t, label):
         base.update({"value": round(gbs, 2), "unit": "GB/s", "config": cfg,
                      "roofline": {"bound": "hbm", "kernel": "routed gate_up GEMV", "achieved": round(gu_gbs, 2), "peak": HBM_PEAK_GBS,
                                   "unit": "GB/s", "frac": round(gu_gbs / HBM_PEAK_GBS, 4),
-                                  "traffic": measured_traffic("c4_decode") if (t == 1 and not args.moe_tokens and not args.hot) else None,
+                                  "traffic": measured_traffic("c4_decode") if (t == 1 and not getattr(args, "moe_tokens", 0) and not getattr(args, "hot", False)) else None,
                                   "algorithmic_bytes": gu_bytes, "kernel_us": round(us_gu, 3)}})
     else:
         valid = int((idx >= 0).sum())
@@ -848,6 +894,8 @@ WORKLOADS = {
     "repack": ("repack", None, 34816, 5120, None, False),              # MLX 4-bit group 64, gate|up sized
     "norm_prefill": ("norm", None, 5120, None, 4096, False),           # n = hidden, m = rows
     "norm_decode": ("norm", None, 5120, None, 1, False),
+    "dense_f32_ba": ("dense_f32", None, 64, 2048, 1, False),           # the gated-delta b|a projection of one token
+    "dense_f32_square": ("dense_f32", None, 5120, 5120, 1, False),
 }
 LABELS = {
     "c1": "C1 AQ4_G32 affine GEMV N=4096 K=4096",
@@ -866,6 +914,8 @@ LABELS = {
     "repack": "MLX affine -> AQ4_G64 repack, 34816 x 5120",
     "norm_prefill": "RMSNorm + residual + FWHT producer, 4096 rows x 5120",
     "norm_decode": "RMSNorm + residual + FWHT producer, 1 row x 5120",
+    "dense_f32_ba": "dense f32 GEMV (qwg_f32_gemv), 1 row, N=64 K=2048",
+    "dense_f32_square": "dense f32 GEMV (qwg_f32_gemv), 1 row, N=5120 K=5120",
 }
 
 
@@ -940,6 +990,8 @@ def main() -> None:
         out = run_repack(args, n, k, 4, 64, LABELS[args.workload])
     elif kind == "norm":
         out = run_norm(args, m, n, LABELS[args.workload])
+    elif kind == "dense_f32":
+        out = run_dense_f32(args, m, n, k, LABELS[args.workload])
     elif kind == "pair":
         out = run_silu_pair(args, fmt, n, k, m, label)
     elif kind == "gemm":

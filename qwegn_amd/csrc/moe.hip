@@ -1,5 +1,6 @@
 // MoE plumbing around the grouped GEMM: router logits, softmax top-k routing, the expert-major pair sort
 // with its tile list, and the weighted combine.
+#include <algorithm>
 #include <atomic>
 
 #include "qwhip_common.h"
@@ -8,8 +9,9 @@
 // ------------------------------------------------------------------------------------------------
 // Router logits: logits[t, e] = sum_h x[t, h] * Wr[e, h], fp32 accumulate.
 // A workgroup owns TT token rows (staged as fp32 in LDS; 8 rows up to hidden = 2048, fewer on wider rows so the tile
-// stays within 64 KiB) so each router row is read once per TT tokens; a wavefront owns experts wave, wave+4, ...;
-// lanes stride the hidden dimension.  With a shared-expert gate row (fp32 [hidden]) the workgroup also writes
+// stays within 64 KiB, and no more than the call has) so each router row is read once per TT tokens; blockIdx.y owns a band of `eb` weight rows
+// (a multiple of 4, so that few token rows still spread over the chip), a wavefront the band's rows wave, wave+4, ...;
+// lanes stride the hidden dimension, so an output's summation order does not depend on the band size.  With a shared-expert gate row (fp32 [hidden]) the workgroup also writes
 // sh_out[t] = sigmoid(x[t] . sh_w), the extra output column of the reference's router kernels
 // (Sources/QWMetal/subsystems/qwrouter.metal:467-483,566-574,587-633).
 // ------------------------------------------------------------------------------------------------
@@ -29,23 +31,36 @@ template <int XDT, int WDT, int TT>
 __global__ __launch_bounds__(256) void qw_router_gemm_kernel(const void* __restrict__ x, const void* __restrict__ wr,
                                                               float* __restrict__ logits, uint32_t T, uint32_t E, uint32_t H,
                                                               const float* __restrict__ sh_w, float* __restrict__ sh_out,
-                                                              uint32_t epi, float scale) {
+                                                              uint32_t epi, float scale, uint32_t eb) {
     extern __shared__ float xs[];  // [TT][H]
     const uint32_t t0 = blockIdx.x * TT;
     const uint32_t nt = min((uint32_t)TT, T - t0);
-    for (uint32_t i = threadIdx.x; i < TT * H; i += 256) {
-        const uint32_t r = i / H, h = i - r * H;
-        xs[i] = r < nt ? qw_load_f32<XDT>(x, (uint64_t)(t0 + r) * H + h) : 0.0f;
-    }
+#pragma unroll
+    for (uint32_t r = 0; r < (uint32_t)TT; ++r)
+        for (uint32_t h = threadIdx.x; h < H; h += 256) xs[r * H + h] = r < nt ? qw_load_f32<XDT>(x, (uint64_t)(t0 + r) * H + h) : 0.0f;
     __syncthreads();
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    const uint32_t rows = E + (sh_w ? 1u : 0u);
-    for (uint32_t e = wave; e < rows; e += 4) {
+    const uint32_t rows = min(E + (sh_w ? 1u : 0u), (blockIdx.y + 1u) * eb);
+    for (uint32_t e = blockIdx.y * eb + wave; e < rows; e += 4) {
         const bool gate_row = e == E;   // wave-uniform
         float acc[TT];
 #pragma unroll
         for (int r = 0; r < TT; ++r) acc[r] = 0.0f;
-        for (uint32_t h = lane; h < H; h += 64) {
+        // eight weight loads in flight per lane, consumed in the order h = lane, lane + 64, ... so the sums do not depend on it
+        uint32_t h = lane;
+        if (!gate_row) {
+            const uint64_t row = (uint64_t)e * H;
+            for (; h + 7u * 64u < H; h += 8u * 64u) {
+                float w[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) w[u] = qw_load_f32<WDT>(wr, row + h + (uint32_t)u * 64u);
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+#pragma unroll
+                    for (int r = 0; r < TT; ++r) acc[r] = fmaf(w[u], xs[r * H + h + (uint32_t)u * 64u], acc[r]);
+            }
+        }
+        for (; h < H; h += 64) {
             const float w = gate_row ? sh_w[h] : qw_load_f32<WDT>(wr, (uint64_t)e * H + h);
 #pragma unroll
             for (int r = 0; r < TT; ++r) acc[r] = fmaf(w, xs[r * H + h], acc[r]);
@@ -74,12 +89,17 @@ static qwhip_status qw_router_gemm_impl(qwhip_stream_t s, const void* x, uint32_
     if (experts == 0 || hidden == 0) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: empty experts or hidden");
     // token rows per workgroup: the fp32 tile stays within 64 KiB
     uint32_t tt = 8;
-    while (tt > 1u && (size_t)tt * hidden * 4u > 64u * 1024u) tt >>= 1;
+    while (tt > 1u && ((size_t)tt * hidden * 4u > 64u * 1024u || tt >= 2u * t)) tt >>= 1;
     const size_t lds = (size_t)tt * hidden * 4u;
     if (lds > 64u * 1024u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: hidden %u exceeds the staged row (<= 16384)", hidden);
-    const dim3 grid(qwhip_cdiv(t, tt)), block(256);
+    // weight rows per workgroup: about 1024 workgroups over the launch, at least one row per wavefront
+    const uint32_t gx = qwhip_cdiv(t, tt), rows_total = experts + (sh_gate_w ? 1u : 0u);
+    const uint32_t gy_want = std::min(qwhip_cdiv(rows_total, 4u), std::max(1u, 1024u / gx));
+    const uint32_t eb = (qwhip_cdiv(rows_total, gy_want) + 3u) & ~3u;
+    const dim3 grid(gx, qwhip_cdiv(rows_total, eb)), block(256);
+    if (grid.y > 65535u) return qwhip_fail(QWHIP_E_BAD_SHAPE, "router gemm: %u weight rows exceed the launch grid", rows_total);
 #define QW_RG(XD, WD, TT) \
-    hipLaunchKernelGGL((qw_router_gemm_kernel<XD, WD, TT>), grid, block, lds, s->stream, x, wr, logits, t, experts, hidden, sh_gate_w, sh_gate_out, epi, scale)
+    hipLaunchKernelGGL((qw_router_gemm_kernel<XD, WD, TT>), grid, block, lds, s->stream, x, wr, logits, t, experts, hidden, sh_gate_w, sh_gate_out, epi, scale, eb)
 #define QW_RG_T(XD, WD)                       \
     switch (tt) {                             \
         case 8: QW_RG(XD, WD, 8); break;      \

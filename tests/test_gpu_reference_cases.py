@@ -657,7 +657,7 @@ def test_argmax_variational_acceptance(dev, rows, vocab):
     assert lib.qwhip_argmax_f32_variational(st, lb.ptr, rows, vocab, db.ptr, rows + 1, 1.0, math.nan, tb.ptr) == qwhip.E_BAD_SHAPE
 
 
-@pytest.mark.parametrize("rows,n,k", [(1, 40, 256), (5, 33, 100), (20, 8, 4096)])
+@pytest.mark.parametrize("rows,n,k", [(1, 40, 256), (5, 33, 100), (20, 8, 4096), (1, 4099, 512), (3000, 7, 64), (9, 1030, 96)])
 @pytest.mark.parametrize("epi,scale", [(0, 1.0), (1, 2.0), (2, 1.0), (3, 0.5)])
 def test_dense_f32_gemv_with_epilogues(dev, rows, n, k, epi, scale):
     rng = np.random.default_rng(n + k)
