@@ -738,9 +738,11 @@ def run_moe(args, t, label):
         xb = dev.put(qo.f32_to_bf16_bits(x32))
         x_basis = qo.fwht32_ortho(xv).astype(np.float16)
 
+        gu_flags = qwhip.MOE_REUSE_EXPERTS if getattr(args, "moe_reuse", False) else 0
+
         def gate_up(i=0):   # the dominant launch: routing + routed gate|up GEMVs + SwiGLU + rotation
-            qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, 0, lbs[i % cycle].ptr, t, K, 1, 1.0, ib.ptr,
-                                                          wb.ptr, act.ptr))
+            qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(vgu), E, xb.ptr, qwhip.BF16, gu_flags, lbs[i % cycle].ptr, t, K, 1, 1.0,
+                                                          ib.ptr, wb.ptr, act.ptr))
 
         def chain(i=0):
             gate_up(i)
@@ -934,6 +936,8 @@ def main() -> None:
     ap.add_argument("--cfg", type=int, default=0, help="gemm tile shape override (0 auto)")
     ap.add_argument("--moe-tokens", type=int, default=0, help="tokens of a c4 workload when run by itself (0 = the benchmark's 1 / 2048)")
     ap.add_argument("--moe-shared", type=int, default=0, help="c4_decode with several tokens: how many of a token's routes repeat token 0's experts (0..8)")
+    ap.add_argument("--moe-reuse", action="store_true",
+                    help="c4_decode with 2..4 tokens: QWHIP_MOE_REUSE_EXPERTS (one workgroup reads a shared expert for all of its tokens)")
     ap.add_argument("--moe-f16", action="store_true", help="c4_prefill on f16 hidden rows (the reference's own type) instead of bf16")
     ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 or mlp_prefill workload when run by itself (0 = the benchmark's 4096)")
     ap.add_argument("--gemm-ws-mb", type=int, default=0,

@@ -147,7 +147,13 @@ enum {
     QWHIP_X_PREROTATED = 1u << 0,
     /* qwhip_gemv: every activation row gets the bits it would get in a call of its own, whatever m is (one arithmetic for
      * all row counts: the reference's 1- / 2- / 4- / M-row bodies agree bit for bit, qw_dequant_multi_b.metalh:14,486,533) */
-    QWHIP_GEMV_ROW_INVARIANT = 1u << 1
+    QWHIP_GEMV_ROW_INVARIANT = 1u << 1,
+    /* qwhip_moe_gateup_decode*, qwhip_moe_route_gateup_decode on an HQ4_G32_M5 bank: an expert that several of the 2..4 tokens
+     * of a verify window (at most 64 routes) route to is read by one workgroup for all of them (encodeMoEGateUpF32R1's
+     * reuseExpertsAcrossTokens, QWGemmMoE.swift:119-132).  Without it every (token, route) pair reads its expert's rows itself,
+     * and rows that share an expert meet in the L2; the outputs are the same bits either way.  Off by default: on this
+     * hardware the launch measured slower with it (the owner of a shared expert runs its tokens one after the other). */
+    QWHIP_MOE_REUSE_EXPERTS = 1u << 2
 };
 
 /* ---- elementwise seams ------------------------------------------------------ */
@@ -404,7 +410,8 @@ qwhip_status qwhip_moe_combine(qwhip_stream_t s, const void* dn, uint32_t dn_dty
  * (QWGemmMoE.swift:120-199) -> Sources/QWMetal/include/qw_moe_f32_common.metalh:187-452.
  * gate_up: act16 [t, top_k, inter] = f16(FWHT32(silu(Wg[e].x) * (Wu[e].x))), SwiGLU on fp32 accumulators.
  * down:    out [t, hidden] = sum_k wts[t,k] * Wd[e_k] . act16[t,k]  (+ shared_gate[t]*shared[t]).
- * gate_up flags: QWHIP_X_PREROTATED; bits 8..11 = 2 keep an HQ4_G32_M5 bank on the general kernel (tests). */
+ * gate_up flags: QWHIP_X_PREROTATED, QWHIP_MOE_REUSE_EXPERTS; bits 8..11 = 2 keep an HQ4_G32_M5 bank on the general
+ * kernel (tests). */
 qwhip_status qwhip_moe_gateup_decode(qwhip_stream_t s, const qwhip_weight_view* w_gate_up, uint32_t experts,
                                      const void* x, uint32_t x_dtype, uint32_t flags, const int32_t* idx, uint32_t t,
                                      uint32_t top_k, void* act16);

@@ -985,7 +985,7 @@ bool qw_stream_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, u
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
                        bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
                        const qw_act act, const float* logits = nullptr, int32_t* idx_out = nullptr, float* wts_out = nullptr, uint32_t norm_topk = 0,
-                       float routed_scale = 1.0f, const int32_t* x_rows = nullptr);
+                       float routed_scale = 1.0f, const int32_t* x_rows = nullptr, uint32_t reuse_tokens = 0);
 bool qw_moe_down_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* act16, const int32_t* idx,
                      const float* wts, uint32_t t, uint32_t top_k, const float* shared, const float* shared_gate, void* out,
                      uint32_t out_dtype, hipError_t* err, uint32_t x_div = 1, const int32_t* labels = nullptr,
@@ -1313,7 +1313,8 @@ extern "C" qwhip_status qwhip_moe_route_gateup_decode(qwhip_stream_t s, const qw
         const bool rotate = qwhip_view_rotated(w_gate_up) && !(flags & QWHIP_X_PREROTATED);
         hipError_t e = hipSuccess;
         if (qw_moe_gateup_col(s->stream, w_gate_up, experts, x, x_dtype, rotate, qwhip_view_rotated(w_gate_up) && inter % 32 == 0, nullptr,
-                              t * top_k, top_k, act16, &e, s->dev->act, logits, idx, wts, norm_topk ? 1u : 0u, scale)) {
+                              t * top_k, top_k, act16, &e, s->dev->act, logits, idx, wts, norm_topk ? 1u : 0u, scale, nullptr,
+                              (flags & QWHIP_MOE_REUSE_EXPERTS) ? t : 0u)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }
@@ -1344,7 +1345,8 @@ static qwhip_status qw_moe_gateup_decode_impl(qwhip_stream_t s, const qwhip_weig
     if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
         hipError_t e = hipSuccess;
         if (qw_moe_gateup_col(s->stream, w_gate_up, experts, x, x_dtype, rotate, qwhip_view_rotated(w_gate_up) && inter % 32 == 0,
-                              idx, t * top_k, top_k, act16, &e, s->dev->act, nullptr, nullptr, nullptr, 0, 1.0f, x_rows)) {
+                              idx, t * top_k, top_k, act16, &e, s->dev->act, nullptr, nullptr, nullptr, 0, 1.0f, x_rows,
+                              (flags & QWHIP_MOE_REUSE_EXPERTS) ? t : 0u)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
         }

@@ -66,17 +66,24 @@ __device__ __forceinline__ float qmc_block_dot(const qw_hq4_block& b, const h2_t
     X(float, routed_scale) X(qw_act, ga)
 QW_ARG_BLOCK(qmc_gu_params, QMC_GU_FIELDS)
 
-template <int XDT, int SETS, int JN = 0>
+// MT > 1 (a verify window of 2 .. MT tokens, at most 64 pairs): an expert that several tokens route to is read once
+// (reuseExpertsAcrossTokens of encodeMoEGateUpF32R1, Sources/Operators/QWGEMM/QWGemmMoE.swift:119-132; the leader / follower scan of
+// Sources/QWMetal/include/qw_moe_f32_common.metalh:213-232).  A pair is primary when it is its token's first route to its
+// expert; a primary pair whose expert an earlier token also routes to leaves (that token's workgroup computes it); the
+// first token's primary pair gathers the primary pairs of the later tokens and runs every row block against all of their
+// activation rows.  A token's second route to one expert runs alone.  Every pair's outputs come from the same operations
+// in the same order as in a launch of its own.  Dynamic LDS = MT * (nb * 80 + 64 * cpr * 4) bytes, blockDim.x <= 512.
+template <int XDT, int SETS, int JN = 0, int MT = 1>
 struct qw_moe_gateup_col_kernel {
-static constexpr int kLaunchBound = 1024;
+static constexpr int kLaunchBound = MT > 1 ? 512 : 1024;
 static __device__ __forceinline__ void run(const qmc_gu_params& p) {
     constexpr int R = 64 / SETS;
     constexpr int D = R < 8 ? R : 8;             // rows in flight per lane
     constexpr int XT = SETS == 2 ? 2 : 1;        // 16-group activation tiles per wave: ceil(2 cpr / (cpr * SETS / 2))
     extern __shared__ h8_t qmc_lds[];
     const uint32_t nb = p.nb, cpr = p.cpr, I = p.I;
-    h8_t* xs = qmc_lds;
-    float* part = (float*)(qmc_lds + (size_t)nb * 5);   // [64 row slots][cpr]
+    h8_t* xs = qmc_lds;                                       // [MT][nb] groups of 80 bytes
+    float* part = (float*)(qmc_lds + (size_t)MT * nb * 5);   // [MT][64 row slots][cpr]
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 31u, hw = tid >> 5;
     const uint32_t wave = tid >> 6, l64 = tid & 63u;
@@ -90,18 +97,86 @@ static __device__ __forceinline__ void run(const qmc_gu_params& p) {
 
     // memory order: the route's expert id, the token's activations, the first weight rows; the rotation runs under them
     int32_t e = 0;                               // no route list: one dense gate|up bank
-    if constexpr (JN == 0) e = p.idx ? p.idx[pair] : 0;
+    if constexpr (JN == 0 && MT == 1) e = p.idx ? p.idx[pair] : 0;
     const uint32_t token = pair / p.top_k;
-    const uint32_t xrow = (JN == 0 && p.x_rows) ? (uint32_t)max(p.x_rows[pair], 0) : token;
-    const uint8_t* x = (const uint8_t*)p.x + (uint64_t)xrow * nb * 64u;
-    h8_t xv[XT];
+    uint32_t xrow = token;
+    if constexpr (MT == 1) xrow = (JN == 0 && p.x_rows) ? (uint32_t)max(p.x_rows[pair], 0) : token;
+    h8_t xv[MT][XT];
+    if constexpr (MT == 1) {
+        const uint8_t* x = (const uint8_t*)p.x + (uint64_t)xrow * nb * 64u;
 #pragma unroll
-    for (int t = 0; t < XT; ++t) {
-        const uint32_t gg = min((wave + nw * t) * 16u + (l64 & 15u), nb - 1u);
-        xv[t] = qw_load_x8_f16<XDT>(x, (uint64_t)gg * 32u + 8u * (l64 >> 4));
+        for (int t = 0; t < XT; ++t) {
+            const uint32_t gg = min((wave + nw * t) * 16u + (l64 & 15u), nb - 1u);
+            xv[0][t] = qw_load_x8_f16<XDT>(x, (uint64_t)gg * 32u + 8u * (l64 >> 4));
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (JN > 0) {
+    uint32_t mcount = 1u;
+    uint32_t slot[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) slot[m] = pair;
+    if constexpr (MT > 1) {
+        // the window's route table: lane l holds pair l's expert (and activation row)
+        __shared__ int32_t tab_e[64];
+        __shared__ float tab_w[64];
+        const uint32_t pairs = gridDim.y, K = p.top_k, ntok = pairs / K;   // pairs <= 64, 2 <= ntok <= MT
+        int32_t my_e = -1;
+        if constexpr (JN > 0) {
+            if (wave < ntok) {   // one wave per token routes it
+                int32_t isel;
+                float wsel;
+                qw_route_wave<JN>(p.logits + (uint64_t)wave * p.experts, p.experts, K, p.norm, p.routed_scale, l64, isel, wsel);
+                if (l64 < K) {
+                    tab_e[wave * K + l64] = isel;
+                    tab_w[wave * K + l64] = wsel;
+                }
+            }
+            __syncthreads();
+            if (l64 < pairs) my_e = tab_e[l64];
+            if (blockIdx.x == 0 && tid == 0) {
+                p.idx_out[pair] = tab_e[pair];
+                p.wts_out[pair] = tab_w[pair];
+            }
+        } else {
+            if (l64 < pairs) my_e = p.idx[l64];
+        }
+        uint32_t my_row = l64 / K;
+        if constexpr (JN == 0) {
+            if (p.x_rows && l64 < pairs) my_row = (uint32_t)max(p.x_rows[l64], 0);
+        }
+        e = __builtin_amdgcn_readlane(my_e, pair);
+        if (e >= 0) {
+            const unsigned long long match = __ballot(my_e == e);   // lanes past the table hold -1
+            const uint32_t kmask = (1u << K) - 1u, rank = pair - token * K;
+            const uint32_t own = (uint32_t)(match >> (token * K)) & kmask;
+            if ((uint32_t)__builtin_ctz(own) == rank) {             // primary: the token's first route to this expert
+                for (uint32_t t2 = 0; t2 < token; ++t2)
+                    if (((uint32_t)(match >> (t2 * K)) & kmask) != 0u) return;   // an earlier token's workgroup computes this pair
+                for (uint32_t t2 = token + 1u; t2 < ntok; ++t2) {
+                    const uint32_t mt = (uint32_t)(match >> (t2 * K)) & kmask;
+                    if (mt != 0u && mcount < (uint32_t)MT) {
+                        const uint32_t sl = t2 * K + (uint32_t)__builtin_ctz(mt);
+#pragma unroll
+                        for (int m = 1; m < MT; ++m)
+                            if ((uint32_t)m == mcount) slot[m] = sl;
+                        ++mcount;
+                    }
+                }
+            }
+        }
+        // every slot's activation row is loaded (a spare slot repeats the pair's own row) so that no load sits under a branch
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const uint32_t xr = (uint32_t)__builtin_amdgcn_readlane((int)my_row, slot[m]);
+            const uint8_t* x = (const uint8_t*)p.x + (uint64_t)xr * nb * 64u;
+#pragma unroll
+            for (int t = 0; t < XT; ++t) {
+                const uint32_t gg = min((wave + nw * t) * 16u + (l64 & 15u), nb - 1u);
+                xv[m][t] = qw_load_x8_f16<XDT>(x, (uint64_t)gg * 32u + 8u * (l64 >> 4));
+            }
+        }
+    }
+    if constexpr (JN > 0 && MT == 1) {
         __shared__ int32_t e_route;
         if (wave == 0) {   // one wave routes (the others would only compete for the same SIMDs), the workgroup reads its result
             int32_t isel;
@@ -138,38 +213,67 @@ static __device__ __forceinline__ void run(const qmc_gu_params& p) {
         h8_t h_lo, h_hi;
         qw_hadamard_pair(l64 & 15u, l64 >> 4, h_lo, h_hi);
 #pragma unroll
-        for (int t = 0; t < XT; ++t) qw_rotate_tile_to_lds(xv[t], wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs);
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int t = 0; t < XT; ++t)
+                qw_rotate_tile_to_lds(xv[m][t], wave + nw * t, nb, l64, p.rotate != 0, h_lo, h_hi, xs + (size_t)m * nb * 5);
     }
     __syncthreads();
+    // The lane's blocks stay in registers while the slots pass over them: slot 0 consumes each block as it lands, the
+    // further slots of a shared expert take their operands from LDS one after the other.
     h2_t xo[16];
     const float S = qmc_operands(xs + g * 5, xo);
     const float c1 = 1024.0f * S;
 #pragma unroll
     for (int r0 = 0; r0 < R; r0 += D) {
+        qw_hq4_block blk[D];
 #pragma unroll
         for (int j = 0; j < D; ++j) {
-            const qw_hq4_block b = buf[j];
+            blk[j] = buf[j];
             if (r0 + D + j < R) buf[j] = *(const qw_hq4_block*)(bank + row_off(r0 + D + j));
-            float v = qmc_block_dot(b, xo, S, c1);
+            float v = qmc_block_dot(blk[j], xo, S, c1);
             v = gvalid ? v : 0.0f;
             v = qw_reduce32_dpp(v);
             if (lane == 31u) part[(set * R + r0 + j) * cpr + chunk] = v;
         }
+        if constexpr (MT > 1) {
+            for (uint32_t m = 1; m < mcount; ++m) {
+                h2_t xm[16];
+                const float Sm = qmc_operands(xs + ((size_t)m * nb + g) * 5, xm);
+                const float cm = 1024.0f * Sm;
+#pragma unroll
+                for (int j = 0; j < D; ++j) {
+                    // the nibble masks are formed again for every slot: hoisted out of this loop they would occupy
+                    // 16 registers per block for the whole kernel
+                    qw_hq4_block b = blk[j];
+                    asm volatile("" : "+v"(b.qs[0]), "+v"(b.qs[1]), "+v"(b.qs[2]), "+v"(b.qs[3]));
+                    float v = qmc_block_dot(b, xm, Sm, cm);
+                    v = gvalid ? v : 0.0f;
+                    v = qw_reduce32_dpp(v);
+                    if (lane == 31u) part[(m * 64u + set * R + r0 + j) * cpr + chunk] = v;
+                }
+            }
+        }
     }
     __syncthreads();
-    if (tid < 64u) {
-        // the whole first wave runs the transform (its upper half repeats the lower half's outputs: the cross-row exchange
+    if (wave < mcount) {
+        // a whole wave runs a slot's transform (its upper half repeats the lower half's outputs: the cross-row exchange
         // wants every row of the wave live); the lower half stores
-        const uint32_t o32 = tid & 31u;
+        const uint32_t o32 = l64 & 31u;
+        const float* pm = part + (size_t)wave * 64u * cpr;
         float gsum = 0.f, usum = 0.f;
         for (uint32_t c = 0; c < cpr; ++c) {
-            gsum += part[o32 * cpr + c];
-            usum += part[(32u + o32) * cpr + c];
+            gsum += pm[o32 * cpr + c];
+            usum += pm[(32u + o32) * cpr + c];
         }
         float a = qw_gated(gsum, usum, p.ga);
         // the butterfly order of the serial transform (pairs h apart: lower = a + b, upper = a - b), across lanes by DPP
         if (p.rot_out && n0 + 32u <= I) a = qw_fwht32_lanes(a, qw_fwht32_lane_signs(o32)) * QW_INV_SQRT32;
-        if (tid < 32u && n0 + tid < I) act[n0 + tid] = (h1_t)a;
+        uint32_t sl = slot[0];
+#pragma unroll
+        for (int m = 1; m < MT; ++m)
+            if ((uint32_t)m == wave) sl = slot[m];
+        if (l64 < 32u && n0 + l64 < I) p.act[(uint64_t)sl * I + n0 + l64] = (h1_t)a;
     }
 }
 };
@@ -266,14 +370,20 @@ static __device__ __forceinline__ void run(const qmc_dn_params& p) {
 bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t experts, const void* x, uint32_t x_dtype, bool rotate,
                        bool rot_out, const int32_t* idx, uint32_t pairs, uint32_t top_k, void* act16, hipError_t* err,
                        const qw_act act, const float* logits, int32_t* idx_out, float* wts_out, uint32_t norm_topk, float routed_scale,
-                       const int32_t* x_rows) {
+                       const int32_t* x_rows, uint32_t reuse_tokens) {
     if (w->kind != QWHIP_KIND_HQ4_G32_M5) return false;
     const uint32_t inter = w->n / (2u * experts);
     const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u;
     if (cpr > 16u || pairs > 65535u) return false;
     if ((uint64_t)2u * inter * nb * 20u >= (1ull << 32)) return false;   // 32-bit offsets inside an expert's sub-bank
-    const uint32_t sets = cpr <= 4u ? 8u : (cpr <= 8u ? 4u : 2u);
-    const size_t lds = (size_t)nb * 80u + (size_t)64u * cpr * 4u;
+    // experts shared by the 2..4 tokens of a verify window are read once when the window's route table fits one wavefront
+    // and four activation rows fit the workgroup's LDS; the workgroup is then at most 512 threads wide
+    constexpr uint32_t kReuseRows = 4;
+    const bool reuse = reuse_tokens >= 2u && reuse_tokens <= kReuseRows && (idx || logits) && top_k >= 1u && top_k <= 16u &&
+                       pairs == reuse_tokens * top_k && pairs <= 64u && cpr <= 8u &&
+                       kReuseRows * ((size_t)nb * 80u + (size_t)64u * cpr * 4u) <= 60u * 1024u;
+    const uint32_t sets = reuse ? (cpr <= 2u ? 8u : (cpr <= 4u ? 4u : 2u)) : (cpr <= 4u ? 8u : (cpr <= 8u ? 4u : 2u));
+    const size_t lds = (reuse ? kReuseRows : 1u) * ((size_t)nb * 80u + (size_t)64u * cpr * 4u);
     if (lds > 60u * 1024u) return false;
     qmc_gu_params p;
     p.bank = (const uint8_t*)w->blocks;
@@ -296,10 +406,14 @@ bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expe
     p.norm = norm_topk;
     p.routed_scale = routed_scale;
     const dim3 grid(qwhip_cdiv(inter, 32u), pairs), block(32u * cpr * sets);
-#define QMC_GU(DT, S, J) qw_launch_scalar<qw_moe_gateup_col_kernel<DT, S, J>>(grid, block, lds, st, p)
-#define QMC_GU_S(DT, J)                                                                                     \
-    do {                                                                                                    \
-        if (sets == 8u) QMC_GU(DT, 8, J); else if (sets == 4u) QMC_GU(DT, 4, J); else QMC_GU(DT, 2, J);     \
+#define QMC_GU(DT, S, J, M) qw_launch_scalar<qw_moe_gateup_col_kernel<DT, S, J, M>>(grid, block, lds, st, p)
+#define QMC_GU_M(DT, J, M)                                                                                              \
+    do {                                                                                                                \
+        if (sets == 8u) QMC_GU(DT, 8, J, M); else if (sets == 4u) QMC_GU(DT, 4, J, M); else QMC_GU(DT, 2, J, M);        \
+    } while (0)
+#define QMC_GU_S(DT, J)                                                            \
+    do {                                                                           \
+        if (reuse) QMC_GU_M(DT, J, (int)kReuseRows); else QMC_GU_M(DT, J, 1);      \
     } while (0)
     if (!logits) {
         if (x_dtype == QWHIP_F16) QMC_GU_S(QWHIP_F16, 0); else QMC_GU_S(QWHIP_BF16, 0);
@@ -309,6 +423,7 @@ bool qw_moe_gateup_col(hipStream_t st, const qwhip_weight_view* w, uint32_t expe
         if (x_dtype == QWHIP_F16) QMC_GU_S(QWHIP_F16, 8); else QMC_GU_S(QWHIP_BF16, 8);
     }
 #undef QMC_GU_S
+#undef QMC_GU_M
 #undef QMC_GU
     *err = hipGetLastError();
     return true;

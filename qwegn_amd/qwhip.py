@@ -18,6 +18,7 @@ F32, F16, BF16, I32 = 0, 1, 2, 3
 KIND_HQ4_G32_M5, KIND_ROTATED_HQ, KIND_NATIVE_AFFINE = 0, 1, 2
 X_PREROTATED = 1
 GEMV_ROW_INVARIANT = 2
+MOE_REUSE_EXPERTS = 4
 
 
 class QwhipError(RuntimeError):

@@ -474,24 +474,29 @@ public enum QWGemm {
     /// the reference's separate gu32 matrix, is refused), and so is a cold bank.
     public static func encodeMoEGateUpF32R1(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, ids: QWTensorValue,
                                             out: QWTensorValue, rowsPerExpert: Int, routes: Int, tokens: Int, fuseSiluFwht: Bool = false,
-                                            coldBank: QWWeightView? = nil, reuseExpertsAcrossTokens: Bool = true, xIsRotated: Bool = true) throws {
+                                            coldBank: QWWeightView? = nil, reuseExpertsAcrossTokens: Bool = false, xIsRotated: Bool = true) throws {
+        // reuseExpertsAcrossTokens: QWHIP_MOE_REUSE_EXPERTS for 2...4 tokens.  The reference defaults to true; here the launch
+        // measured slower with it (rows that share an expert already meet in the L2), so the default is false.  Same bits.
         guard fuseSiluFwht, coldBank == nil, rowsPerExpert > 0, bank.n % rowsPerExpert == 0 else {
             throw QWGemmError.badShape("routed gate_up: fuseSiluFwht only, no cold bank, bank.n a multiple of rowsPerExpert")
         }
         let experts = bank.n / rowsPerExpert
         try hal.pipeline(bank.isIncumbent ? "qwg_moe_gateup_q4g_f32_r1" : "qwg_moe_gateup_aq\(bank.bits)_g\(bank.groupSize)_f32_r1")
         var w = bank.abi
-        try qwCheck(qwhip_moe_gateup_decode(enc.stream, &w, UInt32(experts), x.ptr, x.dtype.rawValue, xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0,
+        let flags = (xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0) | (reuseExpertsAcrossTokens ? UInt32(QWHIP_MOE_REUSE_EXPERTS) : 0)
+        try qwCheck(qwhip_moe_gateup_decode(enc.stream, &w, UInt32(experts), x.ptr, x.dtype.rawValue, flags,
                                             ids.i32, UInt32(tokens), UInt32(routes), out.ptr))
     }
     /// encodeMoEGateUpF32R1 with fuseSiluFwht (QWGemmMoE.swift:120-155), routing folded into the launch for an HQ4_G32_M5 bank.
     public static func encodeMoERouteGateUp(_ enc: QWHipEncoder, hal: QWHal, x: QWTensorValue, bank: QWWeightView, experts: Int,
                                             logits: QWTensorValue, idx: QWTensorValue, wts: QWTensorValue, out: QWTensorValue,
-                                            routes: Int, tokens: Int, normTopK: Bool, routedScale: Float, xIsRotated: Bool = true) throws {
+                                            routes: Int, tokens: Int, normTopK: Bool, routedScale: Float, xIsRotated: Bool = true,
+                                            reuseExpertsAcrossTokens: Bool = false) throws {
         precondition(tokens <= 8, "decode / verify path: at most 8 tokens")
         try hal.pipeline(bank.isIncumbent ? "qwg_moe_gateup_q4g_f32_r1" : "qwg_moe_gateup_aq\(bank.bits)_g\(bank.groupSize)_f32_r1")
         var w = bank.abi
-        try qwCheck(qwhip_moe_route_gateup_decode(enc.stream, &w, UInt32(experts), x.ptr, x.dtype.rawValue, xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0,
+        let flags = (xIsRotated ? UInt32(QWHIP_X_PREROTATED) : 0) | (reuseExpertsAcrossTokens ? UInt32(QWHIP_MOE_REUSE_EXPERTS) : 0)
+        try qwCheck(qwhip_moe_route_gateup_decode(enc.stream, &w, UInt32(experts), x.ptr, x.dtype.rawValue, flags,
                                                   logits.f32, UInt32(tokens), UInt32(routes), normTopK ? 1 : 0, routedScale, idx.i32, wts.f32, out.ptr))
     }
     /// encodeMoEDownSharedCombineF32 (QWGemmMoE.swift:157-199)
@@ -722,7 +727,7 @@ public enum QWMoEOperator {
         public let numLatentGroups: Int, latentDim: Int
         public let hidden: Int, experts: Int, topK: Int, intermediate: Int, sharedIntermediate: Int
         public let normTopK: Bool
-        public let reuseExpertsAcrossTokens: Bool        // taken; the caches already serve an expert shared by verify rows once
+        public let reuseExpertsAcrossTokens: Bool        // QWHIP_MOE_REUSE_EXPERTS on the routed gate_up of 2...4 rows (default false here)
         public let moeSpecExpertBudget: Int
         public let routedScale: Float
         public init(router: QWTensorValue, routerBias: QWTensorValue? = nil, routedScaleParam: QWTensorValue? = nil,
@@ -732,7 +737,7 @@ public enum QWMoEOperator {
                     latent: LatentBottleneck? = nil, latentD: QWWeightView? = nil, latentU: QWWeightView? = nil,
                     latentLabels: QWTensorValue? = nil, numLatentGroups: Int = 0, latentDim: Int = 0,
                     hidden: Int, experts: Int, topK: Int, intermediate: Int, sharedIntermediate: Int,
-                    normTopK: Bool = true, reuseExpertsAcrossTokens: Bool = true, moeSpecExpertBudget: Int = 0, routedScale: Float = 1) {
+                    normTopK: Bool = true, reuseExpertsAcrossTokens: Bool = false, moeSpecExpertBudget: Int = 0, routedScale: Float = 1) {
             self.router = router; self.routerBias = routerBias; self.routedScaleParam = routedScaleParam
             self.splitFeatureRouting = splitFeatureRouting; self.gateUp = gateUp; self.down = down
             self.coldGateUp = coldGateUp; self.coldDown = coldDown
@@ -907,10 +912,11 @@ public enum QWMoEOperator {
                 if plainRoute {
                     let cols = E
                     try QWGemm.encodeMoERouteGateUp(enc, hal: hal, x: x, bank: w.gateUp, experts: E, logits: s.logits.slice(byteOffset: t0 * cols * 4, count: tc * cols),
-                                                    idx: idx, wts: wts, out: act, routes: K, tokens: tc, normTopK: w.normTopK, routedScale: w.routedScale)
+                                                    idx: idx, wts: wts, out: act, routes: K, tokens: tc, normTopK: w.normTopK, routedScale: w.routedScale,
+                                                    reuseExpertsAcrossTokens: w.reuseExpertsAcrossTokens)
                 } else {
                     try QWGemm.encodeMoEGateUpF32R1(enc, hal: hal, x: x, bank: w.gateUp, ids: idx, out: act, rowsPerExpert: 2 * I, routes: K, tokens: tc,
-                                                    fuseSiluFwht: true)
+                                                    fuseSiluFwht: true, reuseExpertsAcrossTokens: w.reuseExpertsAcrossTokens)
                 }
                 try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: act, bank: w.down, rowsPerRoute: H, routes: K, weights: wts,
                                                          shared: shared?.slice(byteOffset: t0 * H * 4, count: tc * H),
@@ -966,7 +972,8 @@ public enum QWMoEOperator {
                 let tc = min(8, T - t0)
                 let idx = s.idx.slice(byteOffset: t0 * K * 4, count: tc * K), act = act16.slice(byteOffset: t0 * K * I * 2, count: tc * K * I)
                 try QWGemm.encodeMoEGateUpF32R1(enc, hal: hal, x: bufB16.slice(byteOffset: t0 * L * 2, count: tc * L), bank: w.gateUp, ids: idx, out: act,
-                                                rowsPerExpert: 2 * I, routes: K, tokens: tc, fuseSiluFwht: true)
+                                                rowsPerExpert: 2 * I, routes: K, tokens: tc, fuseSiluFwht: true,
+                                                reuseExpertsAcrossTokens: w.reuseExpertsAcrossTokens)
                 try QWGemm.encodeMoEDownSharedCombineF32(enc, hal: hal, x: act, bank: w.down, rowsPerRoute: L, routes: K,
                                                          weights: s.wts.slice(byteOffset: t0 * K * 4, count: tc * K), shared: nil, gate: nil,
                                                          out: ls.bufA32.slice(byteOffset: t0 * L * 4, count: tc * L), ids: idx, tokens: tc)

@@ -318,6 +318,52 @@ def test_moe_decode_chain_matches_oracle(dev, t, xdt, experts, hidden, inter, k,
     assert np.all(a[0, k - 1] == 0)
 
 
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,inter", [(256, 96), (2048, 160), (3072, 64), (5120, 40)])
+@pytest.mark.parametrize("t,k,experts", [(2, 8, 12), (3, 4, 6), (4, 8, 40), (4, 16, 20), (4, 8, 8)])
+def test_gateup_decode_reads_a_shared_expert_once_with_the_same_bits(dev, t, k, experts, hidden, inter, xdt):
+    """A verify window of 2..4 tokens whose rows share experts: QWHIP_MOE_REUSE_EXPERTS reads a shared expert once for all
+    of its tokens (encodeMoEGateUpF32R1's reuseExpertsAcrossTokens, QWGemmMoE.swift:119-132; QWMoEReuseTests.swift:46-186 compares
+    the two modes) and must leave the bits of the launch that keeps every (token, route) pair to itself.  Few experts force
+    sharing (with 8 experts and top-8 every token routes to all of them); the list also holds a repeated expert inside one
+    token, an absent route, and the route door is run on the same window."""
+    fmt = "hq4_g32_m5"
+    gu_blocks, _ = H.make_bank(fmt, experts * 2 * inter, hidden, 77)
+    rng = np.random.default_rng(1000 * t + k + hidden)
+    x32 = rng.standard_normal((t, hidden)).astype(np.float32)
+    xh, code = (x32.astype(np.float16), qwhip.F16) if xdt == "f16" else (qo.f32_to_bf16_bits(x32), qwhip.BF16)
+    logits = rng.standard_normal((t, experts)).astype(np.float32)
+    ref_idx, _ = qo.moe_route(logits, min(k, experts), True, 1.0)
+    idx = np.full((t, k), -1, np.int32)
+    idx[:, :ref_idx.shape[1]] = ref_idx
+    if k > ref_idx.shape[1]:
+        idx[:, ref_idx.shape[1]:] = rng.integers(0, experts, (t, k - ref_idx.shape[1]))   # repeats inside a token
+    idx[t - 1, 1] = idx[t - 1, 0]                              # a token's second route to one expert
+    idx[0, k - 1] = -1                                         # an absent route
+    shared_pairs = sum(int(np.isin(idx[r][idx[r] >= 0], idx[:r][idx[:r] >= 0]).sum()) for r in range(1, t))
+    assert shared_pairs > 0
+    lib, st = dev.lib, dev.stream.handle
+    gub, xb, ib = dev.put(gu_blocks), dev.put(xh), dev.put(idx)
+    v = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
+    a1, a2 = dev.put(np.full((t, k, inter), 3, np.float16)), dev.put(np.full((t, k, inter), 5, np.float16))
+    qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(v), experts, xb.ptr, code, qwhip.MOE_REUSE_EXPERTS, ib.ptr, t, k, a1.ptr))
+    qwhip.check(lib.qwhip_moe_gateup_decode(st, C.byref(v), experts, xb.ptr, code, 0, ib.ptr, t, k, a2.ptr))
+    dev.stream.sync()
+    one, two = a1.download(np.uint16, (t, k, inter)), a2.download(np.uint16, (t, k, inter))
+    assert np.array_equal(one, two)
+    assert np.all(one[idx < 0] == 0) and np.any(one != 0)
+    if k <= experts:   # the same window through the door that routes inside the launch
+        i1, w1, i2, w2 = (dev.alloc(t * k * 4 + 256) for _ in range(4))
+        lb = dev.put(logits)
+        qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(v), experts, xb.ptr, code, qwhip.MOE_REUSE_EXPERTS, lb.ptr, t, k, 1, 1.0, i1.ptr, w1.ptr, a1.ptr))
+        qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(v), experts, xb.ptr, code, 0, lb.ptr, t, k, 1, 1.0,
+                                                      i2.ptr, w2.ptr, a2.ptr))
+        dev.stream.sync()
+        assert np.array_equal(i1.download(np.int32, (t, k)), ref_idx) and np.array_equal(i2.download(np.int32, (t, k)), ref_idx)
+        assert np.array_equal(w1.download(np.uint32, (t, k)), w2.download(np.uint32, (t, k)))
+        assert np.array_equal(a1.download(np.uint16, (t, k, inter)), a2.download(np.uint16, (t, k, inter)))
+
+
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g32"])
 @pytest.mark.parametrize("t,experts,hidden,inter,k", [(1, 128, 512, 96, 8), (3, 16, 1280, 192, 4), (8, 200, 256, 64, 3)])
 def test_fused_route_gateup_decode_equals_the_two_launches(dev, fmt, t, experts, hidden, inter, k):
@@ -527,6 +573,12 @@ def test_gateup_decode_rows_reads_the_given_rows(dev, fmt, gu_flags, t, e, k, ng
     one, two = a1.download(np.float16, (t * k, inter)), a2.download(np.float16, (t * k, inter))
     assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
     assert np.any(one != 0) and np.all(one[idx.ravel() < 0] == 0)
+    if 2 <= t <= 4:   # a shared expert read once: every pair still reads its own latent row
+        a3 = dev.put(np.full((t * k, inter), 7, np.float16))
+        qwhip.check(lib.qwhip_moe_gateup_decode_rows(st, C.byref(v), e, xlb.ptr, qwhip.F16, flags | qwhip.MOE_REUSE_EXPERTS, ib.ptr, rwb.ptr, t, k,
+                                                     a3.ptr))
+        dev.stream.sync()
+        assert np.array_equal(a3.download(np.uint16, (t * k, inter)), two.view(np.uint16))
 
 
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32"])
