@@ -389,7 +389,7 @@ qwhip_status qwhip_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, con
  * rounding on store), without writing and re-reading the [pairs, 2 inter] matrix.  The reference fuses the same epilogue
  * into its dense gate_up GEMM (qmm_t_nax_swiglu_impl, Sources/QWMetal/include/qw_gemm_nax_swiglu.metalh:86-167; kernel
  * qwg_gemm_q4g_h16_swiglu) and runs encodeSiluMul* after the grouped one (QWMoEOperator.swift).
- * f16 activations only; inter % 32 == 0; act 16-byte aligned with ldact % 8 == 0 (0 = inter). */
+ * f16 or bf16 activations; inter % 32 == 0; act 16-byte aligned with ldact % 8 == 0 (0 = inter). */
 qwhip_status qwhip_moe_grouped_gemm_swiglu(qwhip_stream_t s, const qwhip_weight_view* w, uint32_t experts,
                                            const void* x, uint32_t x_dtype, uint32_t ldx, const int32_t* gather,
                                            const int32_t* expert_off, const int32_t* tile_e, const int32_t* tile_r,
