@@ -976,8 +976,8 @@ def main() -> None:
     label, traffic = LABELS[args.workload], measured_traffic(args.workload)
     if args.format and args.format != fmt:
         from tests import helpers as H
-        if kind not in ("gemv", "gemm", "pair") or args.format not in H.FORMATS:
-            ap.error(f"--format takes one of {sorted(H.FORMATS)} on a gemv, gemm or pair workload")
+        if kind not in ("gemv", "gemm", "pair", "head") or args.format not in H.FORMATS:
+            ap.error(f"--format takes one of {sorted(H.FORMATS)} on a gemv, gemm, pair or head workload")
         fmt, traffic = args.format, None
         label += f" [container {fmt}]"
     if kind == "moe":
@@ -989,7 +989,7 @@ def main() -> None:
         rows_label = f" [rows {args.gemm_rows}]" if args.gemm_rows else ""
         out = run_mlp_prefill(args, n, k, args.gemm_rows or m, LABELS[args.workload] + rows_label)
     elif kind == "head":
-        out = run_head(args, fmt, n, k, LABELS[args.workload])
+        out = run_head(args, fmt, n, k, label)
     elif kind == "repack":
         out = run_repack(args, n, k, 4, 64, LABELS[args.workload])
     elif kind == "norm":

@@ -22,8 +22,8 @@ struct qwhip_device_s {
 };
 // Partial-sum scratch of the split-K verify GEMV: owned by the stream (allocated when the stream is created, never inside a
 // launcher), so launches on different streams never share it and launches on one stream use it one after the other.
-// The first QWHIP_STREAM_COUNTER_BYTES hold per-row-tile arrival counters, zero between launches (the last arriver resets
-// its counter), the rest holds fp32 partial outputs.
+// The first QWHIP_STREAM_COUNTER_BYTES hold the keys of the head's argmax folds (one per workgroup or row slice), the rest
+// holds fp32 partial outputs.
 #define QWHIP_STREAM_COUNTER_BYTES (64u << 10)
 // The last QWHIP_STREAM_XROT_BYTES hold the rotated copy of several un-rotated activation rows (qwhip_gemv on a rotated
 // container: one rotation pass, then the kernels for rows already in the basis).
