@@ -788,6 +788,28 @@ def run_moe(args, t, label):
     us_chain = timed(chain, args.steps, args.warmup)
     us_gu = timed(gate_up, args.steps, max(2, args.warmup // 4))      # the dominant kernel alone, same inputs
     us_chain_hot = timed(chain, args.steps, max(2, args.warmup // 4), hot=True) if decode else None
+    us_graph = None
+    if decode:
+        # the same cold cycle as one HIP graph (2 * cycle kernel nodes), replayed: what the step costs when the host's launch
+        # calls are out of the way; the last replay's output must equal the eager step's, bit for bit
+        graph = qwhip.Graph(dev.stream, lambda: [chain(i) for i in range(cycle)])
+        reps = max(2, args.steps // cycle)
+        for _ in range(3):
+            graph.launch()
+        dev.stream.sync()
+        g0, g1 = qwhip.Event(dev), qwhip.Event(dev)
+        g0.record(dev.stream)
+        for _ in range(reps):
+            graph.launch()
+        g1.record(dev.stream)
+        dev.stream.sync()
+        us_graph = g0.elapsed_ms(g1) * 1e3 / (reps * cycle)
+        replayed = out.download(np.uint32, (t, Hd))
+        chain(cycle - 1)
+        dev.stream.sync()
+        if not np.array_equal(replayed, out.download(np.uint32, (t, Hd))):
+            _fail("bench: the graph replay's output differs from the eager step's")
+        graph.destroy()
     chain(0)                                                           # the step that is checked: the cycle's first
     dev.stream.sync()
     got = out.download(np.float32, (t, Hd))
@@ -821,6 +843,8 @@ def run_moe(args, t, label):
         cfg["distinct_experts_per_step"] = used
         cfg["cache"] = (f"cold: a cycle of {cycle} steps whose tokens route to different experts walks all {E} experts "
                         f"({E * (2 * I * (Hd // 32) * 20 + Hd * (I // 32) * 20) / 1e6:.0f} MB of banks)")
+        base["graph_replay"] = {"ms_per_step": round(us_graph / 1e3, 6), "value": round(algo / (us_graph * 1e-6) / 1e9, 2), "unit": "GB/s",
+                                "note": f"the cold cycle of {cycle} steps captured as one HIP graph and replayed"}
         base["hot_cache"] = {"ms_per_step": round(us_chain_hot / 1e3, 6), "value": round(algo / (us_chain_hot * 1e-6) / 1e9, 2), "unit": "GB/s",
                              "note": "the same step repeated: its experts (23.6 MB per token) stay in the Infinity Cache"}
         base.update({"value": round(gbs, 2), "unit": "GB/s", "config": cfg,

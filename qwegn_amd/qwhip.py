@@ -206,6 +206,55 @@ class Event:
         return float(ms.value)
 
 
+class Graph:
+    """A HIP graph of the launches a callable puts on a stream (the library's launch doors only enqueue kernels: no
+    allocation, no copy, no clear, so a chain of them can be captured), for callers whose steps are bound by launch
+    latency.  capture() runs `fn` once under stream capture; launch() replays the recorded kernels with the arguments they
+    were recorded with."""
+
+    _hip = None
+
+    @classmethod
+    def _rt(cls) -> C.CDLL:
+        if cls._hip is None:
+            hip = C.CDLL("libamdhip64.so")
+            hip.hipStreamBeginCapture.argtypes = [_P, C.c_int]
+            hip.hipStreamEndCapture.argtypes = [_P, C.POINTER(_P)]
+            hip.hipGraphInstantiate.argtypes = [C.POINTER(_P), _P, _P, _P, C.c_size_t]
+            hip.hipGraphLaunch.argtypes = [_P, _P]
+            hip.hipGraphExecDestroy.argtypes = [_P]
+            hip.hipGraphDestroy.argtypes = [_P]
+            cls._hip = hip
+        return cls._hip
+
+    def __init__(self, stream: Stream, fn):
+        hip = self._rt()
+        self.stream = stream
+        self.native = stream.dev.lib.qwhip_stream_native(stream.handle)
+        graph, self.exe = _P(), _P()
+        if hip.hipStreamBeginCapture(self.native, 1) != 0:          # thread-local capture mode
+            raise RuntimeError("hipStreamBeginCapture failed")
+        try:
+            fn()
+        finally:
+            rc = hip.hipStreamEndCapture(self.native, C.byref(graph))
+        if rc != 0 or not graph.value:
+            raise RuntimeError(f"hipStreamEndCapture failed ({rc})")
+        rc = hip.hipGraphInstantiate(C.byref(self.exe), graph, None, None, 0)
+        hip.hipGraphDestroy(graph)
+        if rc != 0:
+            raise RuntimeError(f"hipGraphInstantiate failed ({rc})")
+
+    def launch(self) -> None:
+        if self._rt().hipGraphLaunch(self.exe, self.native) != 0:
+            raise RuntimeError("hipGraphLaunch failed")
+
+    def destroy(self) -> None:
+        if self.exe.value:
+            self._rt().hipGraphExecDestroy(self.exe)
+            self.exe = _P()
+
+
 class Device:
     def __init__(self, ordinal: int = 0):
         self.lib = load()

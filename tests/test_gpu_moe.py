@@ -364,6 +364,52 @@ def test_gateup_decode_reads_a_shared_expert_once_with_the_same_bits(dev, t, k, 
         assert np.array_equal(a1.download(np.uint16, (t, k, inter)), a2.download(np.uint16, (t, k, inter)))
 
 
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64"])
+@pytest.mark.parametrize("t", [1, 3])
+def test_decode_chain_replays_from_a_hip_graph(dev, fmt, t):
+    """The decode doors only enqueue kernels, so a caller bound by launch latency can capture the chain (routing + gate_up,
+    down + combine) as a HIP graph.  The graph is replayed several times with eager launches and synchronisations of the
+    same doors in between (on other buffers and other inputs), and every replay must leave the eager chain's bits."""
+    experts, hidden, inter, k = 16, 512, 192, 4
+    gu_blocks, _, dn_blocks, _ = _moe_banks(experts, hidden, inter, seed=31, fmt=fmt)
+    rng = np.random.default_rng(12)
+    lib, st = dev.lib, dev.stream.handle
+    gub, dnb = dev.put(gu_blocks), dev.put(dn_blocks)
+    vgu = H.view_of(dev, gub, fmt, experts * 2 * inter, hidden)
+    vdn = H.view_of(dev, dnb, fmt, experts * hidden, inter)
+
+    def buffers():
+        return dict(x=dev.alloc(t * hidden * 2), lg=dev.alloc(t * experts * 4), idx=dev.alloc(t * k * 4 + 256), wts=dev.alloc(t * k * 4 + 256),
+                    act=dev.alloc(t * k * inter * 2), out=dev.alloc(t * hidden * 4))
+
+    def chain(b):
+        qwhip.check(lib.qwhip_moe_route_gateup_decode(st, C.byref(vgu), experts, b["x"].ptr, qwhip.F16, 0, b["lg"].ptr, t, k, 1, 1.0,
+                                                      b["idx"].ptr, b["wts"].ptr, b["act"].ptr))
+        qwhip.check(lib.qwhip_moe_down_decode(st, C.byref(vdn), experts, b["act"].ptr, b["idx"].ptr, b["wts"].ptr, t, k, None, None,
+                                              b["out"].ptr, qwhip.F32))
+
+    def fill(b):
+        b["x"].upload(rng.standard_normal((t, hidden)).astype(np.float16))
+        b["lg"].upload(rng.standard_normal((t, experts)).astype(np.float32))
+
+    g, e = buffers(), buffers()          # the graph's buffers and the eager chain's
+    fill(g)
+    chain(g)                             # the kernels are loaded before the capture
+    dev.stream.sync()
+    graph = qwhip.Graph(dev.stream, lambda: chain(g))
+    for replay in range(4):
+        fill(g)                                            # new inputs in the captured buffers
+        e["x"].upload(g["x"].download(np.float16, (t, hidden)))
+        e["lg"].upload(g["lg"].download(np.float32, (t, experts)))
+        g["out"].upload(np.full((t, hidden), 7.0, np.float32))
+        graph.launch()
+        chain(e)                                           # the same doors, eagerly, behind the replay on the stream
+        dev.stream.sync()
+        assert np.array_equal(g["out"].download(np.uint32, (t, hidden)), e["out"].download(np.uint32, (t, hidden))), replay
+        assert np.array_equal(g["idx"].download(np.int32, (t, k)), e["idx"].download(np.int32, (t, k))), replay
+    graph.destroy()
+
+
 @pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g32"])
 @pytest.mark.parametrize("t,experts,hidden,inter,k", [(1, 128, 512, 96, 8), (3, 16, 1280, 192, 4), (8, 200, 256, 64, 3)])
 def test_fused_route_gateup_decode_equals_the_two_launches(dev, fmt, t, experts, hidden, inter, k):
