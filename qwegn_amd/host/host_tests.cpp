@@ -332,6 +332,14 @@ static void test_gpu_moe_resident(QWHal& hal, int rows) {
     const double err = std::sqrt(num / std::fmax(den, 1e-30));
     std::printf("moe encodeResident rows=%d normalized error %.3e\n", rows, err);
     CHECK(err <= 2e-3);
+    if (rows >= 2 && rows <= 4) {   // a verify window with reuseExpertsAcrossTokens: the same bits
+        QWMoEOperator::Weights wr = w;
+        wr.reuseExpertsAcrossTokens = true;
+        QWMoEOperator::encodeResident(enc, hal, wr, s, xt, xt, out, rows);
+        std::vector<float> again((size_t)rows * H);
+        download(enc, again.data(), dout, again.size() * 4);
+        CHECK(std::memcmp(again.data(), got.data(), got.size() * 4) == 0);
+    }
     // shared-expert gate column of the router door: with router row 0 as the gate row, gate[t] = sigmoid(logits[t, 0])
     {
         DeviceBuf dgate(hal, (size_t)rows * 4);

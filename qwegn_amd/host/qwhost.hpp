@@ -700,7 +700,8 @@ struct QWGemm {
     // encodeFnMoeRoute + encodeMoEGateUpF32R1 as one launch (decode / verify): idx / wts are left for the down projection
     static void encodeMoERouteGateUp(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& gateUp, int experts, const QWTensorValue& x,
                                      const QWTensorValue& logits, const QWTensorValue& idx, const QWTensorValue& wts, int rows, int topK,
-                                     bool normTopK, float routedScale, const QWTensorValue& act16, bool rotateInKernel = false) {
+                                     bool normTopK, float routedScale, const QWTensorValue& act16, bool rotateInKernel = false,
+                                     bool reuseExpertsAcrossTokens = false) {
         if (logits.shape.dtype != QWDType::f32 || logits.shape.elementCount < (size_t)rows * (size_t)experts ||
             idx.shape.elementCount < (size_t)rows * (size_t)topK || wts.shape.elementCount < (size_t)rows * (size_t)topK)
             throw QWGemmError(QWGemmError::badShape, "moe route: logits f32 [rows, experts], idx / wts [rows, topK]");
@@ -708,17 +709,23 @@ struct QWGemm {
         hal.pipeline("qwg_moe_gateup_q4g_f32_r1");
         const qwhip_weight_view v = gateUp.abi();
         throwIfFailed(qwhip_moe_route_gateup_decode(enc.stream, &v, (uint32_t)experts, x.ptr(), abiDType(x.shape.dtype),
-                                                    rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED, (const float*)logits.ptr(), (uint32_t)rows,
+                                                    (rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED) |
+                                                        (reuseExpertsAcrossTokens ? (uint32_t)QWHIP_MOE_REUSE_EXPERTS : 0u),
+                                                    (const float*)logits.ptr(), (uint32_t)rows,
                                                     (uint32_t)topK, normTopK ? 1 : 0, routedScale, (int32_t*)idx.ptr(), (float*)wts.ptr(),
                                                     act16.ptr()));
     }
     // encodeMoEGateUpF32R1 / encodeMoEDownSharedCombineF32 (QWGemmMoE.swift:120-199): decode / verify, rows <= 8
     static void encodeMoEGateUpF32R1(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& gateUp, int experts, const QWTensorValue& x,
-                                     const QWTensorValue& idx, int rows, int topK, const QWTensorValue& act16, bool rotateInKernel = false) {
+                                     const QWTensorValue& idx, int rows, int topK, const QWTensorValue& act16, bool rotateInKernel = false,
+                                     bool reuseExpertsAcrossTokens = false) {
+        // reuseExpertsAcrossTokens (QWGemmMoE.swift:119-132): default true in the reference, false here (same bits, slower launch)
         hal.pipeline("qwg_moe_gateup_q4g_f32_r1");
         const qwhip_weight_view v = gateUp.abi();
         throwIfFailed(qwhip_moe_gateup_decode(enc.stream, &v, (uint32_t)experts, x.ptr(), abiDType(x.shape.dtype),
-                                              rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED, (const int32_t*)idx.ptr(), (uint32_t)rows,
+                                              (rotateInKernel ? 0u : (uint32_t)QWHIP_X_PREROTATED) |
+                                                  (reuseExpertsAcrossTokens ? (uint32_t)QWHIP_MOE_REUSE_EXPERTS : 0u),
+                                              (const int32_t*)idx.ptr(), (uint32_t)rows,
                                               (uint32_t)topK, act16.ptr()));
     }
     static void encodeMoEDownSharedCombineF32(QWHipEncoder& enc, const QWHal& hal, const QWWeightView& down, int experts,
@@ -891,6 +898,7 @@ struct QWMoEOperator {
         int hidden = 0, experts = 0, topK = 0, intermediate = 0;
         bool normTopK = true;
         float routedScale = 1.0f;
+        bool reuseExpertsAcrossTokens = false;   // QWHIP_MOE_REUSE_EXPERTS on the routed gate_up of 2..4 rows
     };
     struct Scratch {  // caller-owned; sizes in elements
         QWTensorValue logits;      // f32 [rows, experts]
@@ -929,7 +937,8 @@ struct QWMoEOperator {
             QWGemm::encodeMoEGroupedGemm(enc, hal, w.down, E, s.act16, nullptr, s.expOff, s.tileE, s.tileR, s.tileCount, pairs, s.dnHi);
             QWGemm::encodeMoEDownReduceCombineF32(enc, hal, s.dnHi, s.invPerm, s.wts, rows, K, H, shared, sharedGate, out);
         } else {
-            QWGemm::encodeMoERouteGateUp(enc, hal, w.gateUp, E, x, s.logits, s.idx, s.wts, rows, K, w.normTopK, w.routedScale, s.act16);
+            QWGemm::encodeMoERouteGateUp(enc, hal, w.gateUp, E, x, s.logits, s.idx, s.wts, rows, K, w.normTopK, w.routedScale, s.act16, false,
+                                         w.reuseExpertsAcrossTokens);
             QWGemm::encodeMoEDownSharedCombineF32(enc, hal, w.down, E, s.act16, s.idx, s.wts, rows, K, shared, sharedGate, out);
         }
     }
