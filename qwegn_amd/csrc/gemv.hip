@@ -1176,7 +1176,9 @@ static qwhip_status qw_gemv_impl(qwhip_stream_t s, const qwhip_weight_view* w, c
     const bool sk_wide8 = !rotate && m >= 13 && w->k < 8192 && fmt == QW_FMT_B8;
     if (variant == 9 || (variant == 0 && (sk_long || sk_wide8))) {
         hipError_t e = hipSuccess;
-        const uint32_t sk_tune = variant == 9 ? (flags >> 12) & 0x7Fu : (sk_wide8 ? 60u : 0u);
+        // long rows, more than eight activation rows (1280 bytes of image per slice): a 128 KiB image halves the K ranges
+        // (N = 5120, K = 17408: twelve -> six, 20.4 -> 19.3 us at m = 16); up to eight rows have six ranges at 64 KiB
+        const uint32_t sk_tune = variant == 9 ? (flags >> 12) & 0x7Fu : (sk_wide8 ? 60u : (m > 8u ? 26u : 0u));
         if (!rotate && qw_sk_gemv(s, w, fmt, a.gshift, a.bb, a.row_bytes, x, x_dtype, m, y16, y32, sk_tune, &e)) {
             QWHIP_TRY_HIP(e);
             return QWHIP_OK;
