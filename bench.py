@@ -581,6 +581,33 @@ def run_dense_f32(args, rows, n, k, label):
     }
 
 
+def vendor_plain_gemm(m, n, k, steps=100):
+    """A yardstick for the matrix pipe, as the read-only launches are for HBM: the vendor library's plain GEMM (PyTorch ->
+    hipBLASLt) Y[m, n] = X[m, k] W[n, k]^T on dense f16 and bf16 operands of the same shape - no quantized bank, no
+    dequantization - after the same spin-up, timed with events.  Nothing of the product is involved."""
+    import torch
+    dev = torch.device("cuda:0")
+    res = {}
+    for name, dt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
+        a = torch.randn(m, k, device=dev, dtype=dt)
+        bt = (torch.randn(n, k, device=dev, dtype=dt) * 0.02).t()
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < 300.0:
+            for _ in range(16):
+                torch.matmul(a, bt)
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            torch.matmul(a, bt)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / steps
+        tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
+        res[name] = {"kernel_us": round(us, 3), "tflops": round(tf, 2), "frac": round(tf / MFMA_PEAK_TFLOPS, 4)}
+    return res
+
+
 def run_gemm(args, fmt, n, k, m, label, traffic=None):
     """Prefill GEMM: X bf16 [m, k] in the container's basis -> Y bf16 [m, n]; one step = one launch."""
     from oracle import qworacle as qo
@@ -653,6 +680,13 @@ def run_gemm(args, fmt, n, k, m, label, traffic=None):
                      "f16_activation_kernel_us": round(us_kernel, 3), "f16_activation_kernel_tflops": round(tf_k, 2)},
         "normalized_error": err,
     }
+    if getattr(args, "vendor_gemm", False):
+        # in a process of its own: PyTorch brings its own HIP runtime, which must not meet the one this library links
+        import subprocess
+        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", "vendor_gemm", "--gemm-rows", str(m)],
+                               capture_output=True, text=True, timeout=600)
+        lines = [ln for ln in child.stdout.splitlines() if ln.startswith("{")]
+        out["roofline"]["vendor_plain_gemm"] = json.loads(lines[-1])["vendor_plain_gemm"] if child.returncode == 0 and lines else None
     if not args.no_cpu:
         sample = min(m, 256)
         xs = qo.round_bf16(x32)[:sample].astype(np.float16)
@@ -950,7 +984,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS) + ["headline", "calib"],
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS) + ["headline", "calib", "vendor_gemm"],
                     help="headline = c2 (the bench line) with the c3 prefill GEMM summarised under 'prefill_gemm'")
     ap.add_argument("--m", type=int, default=8, help="activation rows for the c5 workloads")
     ap.add_argument("--hot", action="store_true", help="single bank (Infinity-Cache resident) instead of the cold ring")
@@ -966,6 +1000,8 @@ def main() -> None:
     ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 or mlp_prefill workload when run by itself (0 = the benchmark's 4096)")
     ap.add_argument("--gemm-ws-mb", type=int, default=0,
                     help="workspace handed to qwhip_gemm in MiB (0 = the activation copy only; more lets small row counts split K)")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="c3: also time the vendor library's plain f16 / bf16 GEMM of the same shape (needs PyTorch; a yardstick, not the product)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
     ap.add_argument("--invariant", action="store_true", help="gemv workloads with QWHIP_GEMV_ROW_INVARIANT (every row as in a call of its own)")
     ap.add_argument("--format", default=None,
@@ -977,6 +1013,11 @@ def main() -> None:
         _fail("bench.py: this build measures one GPU only (every box has one); run with --gpus 1")
     if args.workload == "calib":
         print(json.dumps(run_calibration(args)))
+        return
+    if args.workload == "vendor_gemm":      # PyTorch only: this process never loads the library
+        _, _, n, k, m, _ = WORKLOADS["c3"]
+        m = args.gemm_rows or m
+        print(json.dumps({"workload": f"vendor library plain GEMM M={m} K={k} N={n} (f16, bf16)", "vendor_plain_gemm": vendor_plain_gemm(m, n, k)}))
         return
     if args.workload == "headline":
         kind, fmt, n, k, m, outliers = WORKLOADS["c2"]
