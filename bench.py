@@ -581,6 +581,33 @@ def run_dense_f32(args, rows, n, k, label):
     }
 
 
+def vendor_plain_bmm(batch, m, n, k, steps=50):
+    """The grouped counterpart of vendor_plain_gemm: `batch` independent products [m, k] x [n, k]^T on dense f16 / bf16
+    operands (torch.bmm -> the vendor library's batched GEMM), i.e. an MoE layer's grouped GEMM if every expert got exactly
+    m rows and its weights were ready-made f16 matrices."""
+    import torch
+    dev = torch.device("cuda:0")
+    res = {}
+    for name, dt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
+        a = torch.randn(batch, m, k, device=dev, dtype=dt)
+        bt = (torch.randn(batch, n, k, device=dev, dtype=dt) * 0.02).transpose(1, 2)
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < 300.0:
+            for _ in range(8):
+                torch.bmm(a, bt)
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            torch.bmm(a, bt)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / steps
+        tf = 2.0 * batch * m * n * k / (us * 1e-6) / 1e12
+        res[name] = {"kernel_us": round(us, 3), "tflops": round(tf, 2), "frac": round(tf / MFMA_PEAK_TFLOPS, 4)}
+    return res
+
+
 def vendor_plain_gemm(m, n, k, steps=100):
     """A yardstick for the matrix pipe, as the read-only launches are for HBM: the vendor library's plain GEMM (PyTorch ->
     hipBLASLt) Y[m, n] = X[m, k] W[n, k]^T on dense f16 and bf16 operands of the same shape - no quantized bank, no
@@ -1017,7 +1044,12 @@ def main() -> None:
     if args.workload == "vendor_gemm":      # PyTorch only: this process never loads the library
         _, _, n, k, m, _ = WORKLOADS["c3"]
         m = args.gemm_rows or m
-        print(json.dumps({"workload": f"vendor library plain GEMM M={m} K={k} N={n} (f16, bf16)", "vendor_plain_gemm": vendor_plain_gemm(m, n, k)}))
+        out = {"workload": f"vendor library plain GEMM M={m} K={k} N={n} (f16, bf16)", "vendor_plain_gemm": vendor_plain_gemm(m, n, k)}
+        if args.moe_tokens:                 # the C4 layer's two grouped products with every expert at tokens * 8 / 128 rows
+            rows = args.moe_tokens * 8 // 128
+            out["vendor_plain_bmm"] = {"rows_per_expert": rows, "gate_up_128x[rows,2048]x[1536,2048]^T": vendor_plain_bmm(128, rows, 1536, 2048),
+                                       "down_128x[rows,768]x[2048,768]^T": vendor_plain_bmm(128, rows, 2048, 768)}
+        print(json.dumps(out))
         return
     if args.workload == "headline":
         kind, fmt, n, k, m, outliers = WORKLOADS["c2"]
