@@ -239,10 +239,11 @@ def run_silu_pair(args, fmt, inter, k, m, label):
     views = [H.view_of(dev, b, fmt, 2 * inter, k) for b in banks]
     xb, act = dev.put(x16), dev.alloc(m * inter * 2)
     flags = args.variant << 8
+    rot_out = 0 if getattr(args, "plain_out", False) else 1      # 0: act in the plain basis, the down projection rotates its input itself
     lib, st = dev.lib, dev.stream.handle
 
     def launch(i):
-        qwhip.check(lib.qwhip_gemv_silu_pair(st, C.byref(views[i % ring_n]), xb.ptr, qwhip.F16, m, flags, 1, act.ptr))
+        qwhip.check(lib.qwhip_gemv_silu_pair(st, C.byref(views[i % ring_n]), xb.ptr, qwhip.F16, m, flags, rot_out, act.ptr))
 
     _spin_up(dev, launch)
     for i in range(args.warmup):
@@ -257,7 +258,7 @@ def run_silu_pair(args, fmt, inter, k, m, label):
     us_per = e0.elapsed_ms(e1) * 1e3 / args.steps
     got = act.download(np.float16, (m, inter)).astype(np.float32)
     gu = qo.matmul_ref_f64(H.x_in_basis(x16, fmt), w16)
-    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=True).astype(np.float32)
+    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=bool(rot_out)).astype(np.float32)
     err = qo.normalized_error(got, want)
     if not err <= 2e-3:
         _fail(f"bench: SwiGLU pair output failed parity (normalized error {err:.3e})")
@@ -268,12 +269,78 @@ def run_silu_pair(args, fmt, inter, k, m, label):
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": label, "format": fmt, "M": m, "N": 2 * inter, "K": k, "fused_fwht": True,
+        "config": {"workload": label, "format": fmt, "M": m, "N": 2 * inter, "K": k, "fused_fwht": True, "output_rotation": bool(rot_out),
                    "cache": "hot" if args.hot else f"cold ring of {ring_n} banks ({ring_n * blocks.nbytes / 1e6:.0f} MB)"},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": algo_bytes,
                      "kernel_us": round(us_per, 3)},
         "normalized_error": err,
+    }
+
+
+def run_mlp_decode(args, inter, hidden, label):
+    """Dense MLP decode step on HQ4_G32_M5 banks, one token: gate|up GEMV with the gated activation, then the down GEMV;
+    one step = the two launches.  Two forms of the same step: the reference's (the first launch also rotates act into the
+    down bank's basis) and the one that suits this device (act stays plain, the down GEMV rotates its input in its prologue,
+    which is free at one row, and the gate|up bank is read by the decode GEMV's own kernel).  Both are checked against the
+    fp64 chain."""
+    from oracle import qworacle as qo
+    from qwegn_amd import qwhip
+    from tests import helpers as H
+
+    fmt = "hq4_g32_m5"
+    dev = qwhip.Device(0)
+    gu_blocks, gu16 = H.make_bank(fmt, 2 * inter, hidden, seed=0)
+    dn_blocks, dn16 = H.make_bank(fmt, hidden, inter, seed=1)
+    x16 = H.make_x(1, hidden, 100).astype(np.float16)
+    step_bytes = gu_blocks.nbytes + dn_blocks.nbytes
+    ring_n = max(2, int(np.ceil(args.ring_mb * 1e6 / step_bytes))) if not args.hot else 1
+    gus, dns = [dev.put(gu_blocks) for _ in range(ring_n)], [dev.put(dn_blocks) for _ in range(ring_n)]
+    vgu = [H.view_of(dev, b, fmt, 2 * inter, hidden) for b in gus]
+    vdn = [H.view_of(dev, b, fmt, hidden, inter) for b in dns]
+    xb, act, yb = dev.put(x16), dev.alloc(inter * 2), dev.alloc(hidden * 4)
+    lib, st = dev.lib, dev.stream.handle
+
+    def step(i, plain):
+        qwhip.check(lib.qwhip_gemv_silu_pair(st, C.byref(vgu[i % ring_n]), xb.ptr, qwhip.F16, 1, 0, 0 if plain else 1, act.ptr))
+        qwhip.check(lib.qwhip_gemv(st, C.byref(vdn[i % ring_n]), act.ptr, qwhip.F16, 1, 0 if plain else qwhip.X_PREROTATED, None, yb.ptr))
+
+    gu = qo.matmul_ref_f64(H.x_in_basis(x16, fmt), gu16)
+    act_ref = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=True)
+    want = qo.matmul_ref_f64(act_ref, dn16)
+    res = {}
+    for name, plain in (("reference_form", False), ("plain_act_form", True)):
+        step(0, plain)
+        dev.stream.sync()
+        err = float(qo.normalized_error(yb.download(np.float32, (1, hidden)), want))
+        if not err <= 2e-3:
+            _fail(f"bench: dense MLP decode step ({name}) failed parity (normalized error {err:.3e})")
+        _spin_up(dev, lambda i: step(i, plain))
+        for i in range(args.warmup):
+            step(i, plain)
+        dev.stream.sync()
+        e0, e1 = qwhip.Event(dev), qwhip.Event(dev)
+        e0.record(dev.stream)
+        for i in range(args.steps):
+            step(i, plain)
+        e1.record(dev.stream)
+        dev.stream.sync()
+        res[name] = {"us_per_step": round(e0.elapsed_ms(e1) * 1e3 / args.steps, 3), "normalized_error": err}
+    algo_bytes = step_bytes + hidden * 2 + 2 * inter * 2 + hidden * 4
+    us_per = res["plain_act_form"]["us_per_step"]
+    gbs = algo_bytes / (us_per * 1e-6) / 1e9
+    for v in res.values():
+        v["GB/s"] = round(algo_bytes / (v["us_per_step"] * 1e-6) / 1e9, 2)
+    return {
+        "metric": "HQ4 GEMV GB/s (% HBM peak) at M=1; prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": label, "format": fmt, "M": 1, "hidden": hidden, "intermediate": inter,
+                   "cache": "hot" if args.hot else f"cold ring of {ring_n} bank pairs ({ring_n * step_bytes / 1e6:.0f} MB)"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": algo_bytes, "kernel_us": us_per, "forms": res},
+        "normalized_error": res["plain_act_form"]["normalized_error"],
     }
 
 
@@ -974,6 +1041,7 @@ WORKLOADS = {
     "c5_down": ("gemv", "hq4_g64", 5120, 17408, None, False),
     "mlp_gate_up": ("pair", "hq4_g32_m5", 17408, 5120, 1, False),      # n = intermediate size: the bank has 2n rows
     "mlp_prefill": ("mlp_prefill", "hq4_g32_m5", 17408, 5120, 4096, False),   # n = intermediate size
+    "mlp_decode": ("mlp_decode", "hq4_g32_m5", 17408, 5120, 1, False),         # n = intermediate size, k = hidden
     "head": ("head", "hq4_g32_m5", 151936, 5120, 1, False),
     "f32_decode": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 1, False),
     "f32_verify4": ("gemv_f32", "hq4_g32_m5", 17408, 5120, 4, False),
@@ -994,6 +1062,7 @@ LABELS = {
     "c5_down": "C5 verify GEMM HQ4_G64 K=17408 N=5120",
     "mlp_gate_up": "dense MLP gate|up GEMV + SwiGLU + FWHT, HQ4_G32 M=1 K=5120 I=17408",
     "mlp_prefill": "dense MLP prefill gate|up GEMM + SwiGLU + FWHT fused, HQ4_G32 M=4096 K=5120 I=17408",
+    "mlp_decode": "dense MLP decode step: gate|up GEMV + SwiGLU, down GEMV, HQ4_G32 M=1 H=5120 I=17408",
     "head": "LM head GEMV + argmax, HQ4_G32 M=1 K=5120 N=151936",
     "f32_decode": "f32-activation GEMV, HQ4_G32 M=1 K=5120 N=17408",
     "f32_verify4": "f32-activation GEMV, HQ4_G32 M=4 K=5120 N=17408",
@@ -1027,6 +1096,8 @@ def main() -> None:
     ap.add_argument("--gemm-rows", type=int, default=0, help="activation rows of the c3 or mlp_prefill workload when run by itself (0 = the benchmark's 4096)")
     ap.add_argument("--gemm-ws-mb", type=int, default=0,
                     help="workspace handed to qwhip_gemm in MiB (0 = the activation copy only; more lets small row counts split K)")
+    ap.add_argument("--plain-out", action="store_true",
+                    help="mlp_gate_up: no output rotation (act in the plain basis; the down projection then rotates its input itself)")
     ap.add_argument("--vendor-gemm", action="store_true",
                     help="c3: also time the vendor library's plain f16 / bf16 GEMM of the same shape (needs PyTorch; a yardstick, not the product)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
@@ -1085,6 +1156,8 @@ def main() -> None:
     elif kind == "mlp_prefill":
         rows_label = f" [rows {args.gemm_rows}]" if args.gemm_rows else ""
         out = run_mlp_prefill(args, n, k, args.gemm_rows or m, LABELS[args.workload] + rows_label)
+    elif kind == "mlp_decode":
+        out = run_mlp_decode(args, n, k, LABELS[args.workload])
     elif kind == "head":
         out = run_head(args, fmt, n, k, label)
     elif kind == "repack":

@@ -205,7 +205,11 @@ qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void
 /* gate|up GEMV + SwiGLU (+ FWHT-32 of the result): qwg_gemv_q4g_silu_pair{,_h16,_dx_h16}
  * (qwgemm.metal:204-379; QWGemm.swift:137-283 epilogue .siluMulPair; EncodeKernels.swift:298-326).
  * w holds 2*inter rows: [0, inter) gate, [inter, 2*inter) up.  act16 f16 [m, inter] =
- * f16(FWHT32(silu(g)*u)) with SwiGLU on the fp32 accumulators; `rotate_out` = 0 stores it unrotated. */
+ * f16(FWHT32(silu(g)*u)) with SwiGLU on the fp32 accumulators; `rotate_out` = 0 stores it unrotated.
+ * One row over an HQ4_G32_M5 bank with rotate_out = 0 is read by the decode GEMV's own kernel in a gate|up form (the bank
+ * walked as two moving bands: 20.7 against 25.6 us on 2 x 17408 x 5120): a dense MLP decode step is fastest as this call
+ * followed by qwhip_gemv on the down bank without QWHIP_X_PREROTATED, whose fused rotation costs nothing at one row.
+ * flags bits 8..11 (tests): 2 = the general kernel, 3 = the MoE decode kernel also where the gate|up form would be taken. */
 qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                                   uint32_t m, uint32_t flags, uint32_t rotate_out, void* act16);
 

@@ -1001,6 +1001,8 @@ bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t 
                   hipError_t* err);
 
 // gemv_col.hip
+bool qw_col_pair_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* act16,
+                      const qw_act ga, hipError_t* err);
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
                  float* y32, uint32_t tune, hipError_t* err, unsigned long long* keys, uint32_t keys_cap, int32_t* token,
                  bool* folded);
@@ -1252,7 +1254,16 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     const uint32_t inter = w->n / 2;
     const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
     // HQ4_G32_M5: the column-stationary gate|up kernel of the MoE decode path, as one dense bank with one "route" per
-    // activation row (flags bits 8..11 = 2 keep the general kernel, for tests)
+    // activation row (flags bits 8..11 = 2 keep the general kernel, for tests).  One row without the output rotation takes the
+    // decode GEMV's own kernel in its gate|up form (bits 8..11 = 3 keep the MoE kernel): without the rotation a workgroup
+    // does not need 32 neighbouring channels and the bank is read as two moving bands.
+    if (fmt == QW_FMT_M5 && m == 1u && !(rotate_out && inter % 32 == 0) && ((flags >> 8) & 0xFu) == 0u) {
+        hipError_t e = hipSuccess;
+        if (qw_col_pair_gemv(s->stream, w, x, x_dtype, rotate, act16, s->dev->act, &e)) {
+            QWHIP_TRY_HIP(e);
+            return QWHIP_OK;
+        }
+    }
     if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
         hipError_t e = hipSuccess;
         if (qw_moe_gateup_col(s->stream, w, 1, x, x_dtype, rotate, rotate_out && inter % 32 == 0, nullptr, m, 1, act16, &e, s->dev->act)) {

@@ -30,7 +30,19 @@ QW_ARG_BLOCK(qc_params, QC_FIELDS)
 // launch took 11.6 us instead of 11.3 in a same-box comparison).
 #define QC_FOLD_FIELDS(X) QC_FIELDS(X) X(unsigned long long*, keys)
 QW_ARG_BLOCK(qc_params_fold, QC_FOLD_FIELDS)
+// The gate|up form of the kernel (dense MLP decode without the output rotation): the bank holds I gate rows and then the I up
+// rows of the same channels; row slots 2 c and 2 c + 1 of a workgroup are the gate and the up row of its channel c, so that
+// the gated activation is formed in the epilogue and act f16 [I] is what gets stored (y16).  N = 2 I.
+#define QC_PAIR_FIELDS(X) QC_FIELDS(X) X(qw_act, ga)
+QW_ARG_BLOCK(qc_params_pair, QC_PAIR_FIELDS)
 __device__ __forceinline__ const qc_params& qc_base(const qc_params& p) { return p; }
+__device__ __forceinline__ qc_params qc_base(const qc_params_pair& f) {
+    qc_params p;
+#define QC_TAKE(T, n) p.n = f.n;
+    QC_FIELDS(QC_TAKE)
+#undef QC_TAKE
+    return p;
+}
 __device__ __forceinline__ qc_params qc_base(const qc_params_fold& f) {
     qc_params p;
 #define QC_TAKE(T, n) p.n = f.n;
@@ -53,7 +65,9 @@ template <int XDT, int SETS, int D, int D0, typename P = qc_params>
 struct qw_gemv_col_kernel {
 static constexpr int kLaunchBound = 1024;
 static __device__ __forceinline__ void run(const P& pp) {
-    constexpr bool FOLD = !std::is_same<P, qc_params>::value;
+    constexpr bool FOLD = std::is_same<P, qc_params_fold>::value;
+    constexpr bool PAIR = std::is_same<P, qc_params_pair>::value;
+    static_assert(!PAIR || SETS % 2 == 0, "gate and up rows sit in row sets of opposite parity");
     const qc_params& p = qc_base(pp);
     // 16-group activation tiles per full wave: ceil(2 cpr / full waves).  One row set with an odd cpr ends in a half
     // wave, which takes no tile (its upper lanes do not exist): cpr = 13 leaves 6 full waves for 26 tiles.
@@ -72,13 +86,29 @@ static __device__ __forceinline__ void run(const P& pp) {
     const bool gvalid = g0 < nb;
     const uint32_t g = gvalid ? g0 : nb - 1u;
     const uint32_t G = gridDim.x;
-    if (blockIdx.x >= N) return;
-    const uint32_t nrows = (N - blockIdx.x + G - 1u) / G;   // row slots of this workgroup
-    const uint32_t nmax = (nrows + SETS - 1u) / SETS;        // trip count, uniform over the workgroup
     const uint32_t row_bytes = nb * 20u;
-    const uint32_t step = G * SETS * row_bytes;              // bytes between consecutive rows of one set
-    const uint32_t mine = nrows > set ? (nrows - set + SETS - 1u) / SETS : 0u;
-    uint32_t off = ((mine ? set : 0u) * G + blockIdx.x) * row_bytes + g * 20u;
+    uint32_t nrows, nmax, step, mine, off;
+    if constexpr (PAIR) {
+        // channel c of this workgroup is bank channel c G + blockIdx.x; set j walks the channels c = j / 2, + SETS / 2, ... of
+        // half j & 1 (0: gate rows, 1: up rows, I rows further on), so slot trip * SETS + j is (channel, half) = (slot / 2, slot & 1)
+        constexpr uint32_t H2 = SETS / 2;
+        const uint32_t I = N >> 1;
+        if (blockIdx.x >= I) return;
+        const uint32_t nch = (I - blockIdx.x + G - 1u) / G;      // channels of this workgroup
+        const uint32_t sub = set >> 1, half = set & 1u;
+        nrows = 2u * nch;
+        nmax = (nch + H2 - 1u) / H2;
+        step = G * H2 * row_bytes;
+        mine = nch > sub ? (nch - sub + H2 - 1u) / H2 : 0u;
+        off = (half * I + (mine ? sub : 0u) * G + blockIdx.x) * row_bytes + g * 20u;
+    } else {
+        if (blockIdx.x >= N) return;
+        nrows = (N - blockIdx.x + G - 1u) / G;               // row slots of this workgroup
+        nmax = (nrows + SETS - 1u) / SETS;                   // trip count, uniform over the workgroup
+        step = G * SETS * row_bytes;                         // bytes between consecutive rows of one set
+        mine = nrows > set ? (nrows - set + SETS - 1u) / SETS : 0u;
+        off = ((mine ? set : 0u) * G + blockIdx.x) * row_bytes + g * 20u;
+    }
     const uint32_t off_max = off + (mine ? mine - 1u : 0u) * step;   // loads past the set's last row re-read it
 
     // 1. activation loads go first: loads return in order, and the rotation must not queue behind the weight prefetch
@@ -167,6 +197,17 @@ static __device__ __forceinline__ void run(const P& pp) {
     // 5. fixed-order sum of the chunk partials of each row; with `keys` also the greedy-decoding fold of the reference's
     // head kernels (qwg_gemv_am_fold4 / qwg_gemv_am_reduce4, Sources/QWMetal/include/qw_gemm_f32_common.metalh:30-58):
     // larger (monotone bits, ~row) wins, so ties go to the lower row
+    if constexpr (PAIR) {
+        for (uint32_t c = tid; 2u * c < nrows; c += blockDim.x) {
+            float gsum = 0.f, usum = 0.f;
+            for (uint32_t k = 0; k < cpr; ++k) {
+                gsum += part[(2u * c) * cpr + k];
+                usum += part[(2u * c + 1u) * cpr + k];
+            }
+            p.y16[c * G + blockIdx.x] = (h1_t)qw_gated(gsum, usum, pp.ga);
+        }
+        return;
+    }
     unsigned long long best = 0ull;
     for (uint32_t s = tid; s < nrows; s += blockDim.x) {
         float v = 0.f;
@@ -581,6 +622,47 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
         e = hipGetLastError();
     }
     *err = e;
+    return true;
+}
+
+// Gate|up form of the column-stationary kernel for one activation row over a validated HQ4_G32_M5 gate|up bank (n = 2 I rows):
+// act f16 [I] = gated(Wg . x, Wu . x) on the fp32 sums, no output rotation.  The workgroups walk the gate half and the up half
+// of the bank as two bands, like the decode GEMV walks its one.  false when the shape is outside the envelope (rows longer
+// than 12288 columns take one row set per workgroup, which cannot hold a gate and an up row side by side).
+bool qw_col_pair_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* act16,
+                      const qw_act ga, hipError_t* err) {
+    if (w->kind != QWHIP_KIND_HQ4_G32_M5 || (w->n & 1u)) return false;
+    const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u, inter = w->n / 2u;
+    if (cpr > 12u || inter < 64u) return false;
+    if ((uint64_t)w->n * nb * 20u >= (1ull << 32)) return false;   // 32-bit offsets inside the bank
+    if (((uintptr_t)x & 15u) != 0) return false;
+    const uint32_t sets = cpr <= 3u ? 4u : 2u, h2 = sets / 2u;
+    const uint32_t threads = 32u * cpr * sets;
+    const uint32_t waves = (threads + 63u) / 64u;
+    uint32_t wgs = (256u * 10u + waves / 2u) / waves;              // ten waves per compute unit, as the compiled window of the GEMV
+    wgs = min(wgs, max(1u, inter / (h2 * 4u)));                    // at least four channels per set
+    wgs = max(wgs, qwhip_cdiv(inter, 64u));                        // at most 128 row slots per workgroup
+    const uint32_t ch_per_wg = qwhip_cdiv(inter, wgs);
+    const size_t lds = (size_t)nb * 80u + (size_t)2u * ch_per_wg * cpr * 4u;
+    if (lds > 60u * 1024u) return false;
+    qc_params_pair p;
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = x;
+    p.y16 = (h1_t*)act16;
+    p.y32 = nullptr;
+    p.N = w->n;
+    p.nb = nb;
+    p.cpr = cpr;
+    p.rotate = rotate ? 1u : 0u;
+    p.ga = ga;
+    if (x_dtype == QWHIP_F16) {
+        if (sets == 4u) qw_launch_scalar<qw_gemv_col_kernel<QWHIP_F16, 4, 2, 2, qc_params_pair>>(dim3(wgs), dim3(threads), lds, st, p);
+        else qw_launch_scalar<qw_gemv_col_kernel<QWHIP_F16, 2, 2, 2, qc_params_pair>>(dim3(wgs), dim3(threads), lds, st, p);
+    } else {
+        if (sets == 4u) qw_launch_scalar<qw_gemv_col_kernel<QWHIP_BF16, 4, 2, 2, qc_params_pair>>(dim3(wgs), dim3(threads), lds, st, p);
+        else qw_launch_scalar<qw_gemv_col_kernel<QWHIP_BF16, 2, 2, 2, qc_params_pair>>(dim3(wgs), dim3(threads), lds, st, p);
+    }
+    *err = hipGetLastError();
     return true;
 }
 

@@ -308,7 +308,10 @@ struct QWGemm {
 
     // QWGemm.encode (QWGemm.swift:218-283): f32 output; .siluMulPair needs even N and stores f16 activations.
     static void encode(QWHipEncoder& enc, const QWHal& hal, const QWGemmPlan& plan, const QWTensorValue& x, const QWWeightView& wQ4,
-                       const QWTensorValue& y, int rows = 1, bool rotateInKernel = false) {
+                       const QWTensorValue& y, int rows = 1, bool rotateInKernel = false, bool siluPairPlainOut = false) {
+        // siluPairPlainOut: the .siluMulPair epilogue stores act in the plain basis instead of the next projection's; that
+        // projection then rotates its input itself (rotateInKernel), which costs nothing at one row, and the gate|up bank is
+        // read by the decode GEMV's own kernel (one row, HQ4_G32_M5: 20.7 against 25.6 us on 2 x 17408 x 5120).
         using B = QWGemmPlan::Backend;
         if (plan.backend == B::blocked) {
             if (plan.family == QWGemmFamily::f5SkinnyGemm) throw QWGemmError(QWGemmError::badWeights, "F5 window: run F1 per row");
@@ -327,7 +330,7 @@ struct QWGemm {
         if (plan.epilogue == QWEpilogue::siluMulPair) {
             if (y.shape.dtype != QWDType::f16 || y.shape.elementCount < (size_t)rows * (size_t)(wQ4.n / 2))
                 throw QWGemmError(QWGemmError::badWeights, "silu_pair output must be f16 [rows, N/2]");
-            throwIfFailed(qwhip_gemv_silu_pair(enc.stream, &w, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows, flags, 1, y.ptr()));
+            throwIfFailed(qwhip_gemv_silu_pair(enc.stream, &w, x.ptr(), abiDType(x.shape.dtype), (uint32_t)rows, flags, siluPairPlainOut ? 0u : 1u, y.ptr()));
             return;
         }
         if (y.shape.dtype != QWDType::f32 || y.shape.elementCount < (size_t)rows * (size_t)wQ4.n)

@@ -209,7 +209,10 @@ public enum QWGemm {
     /// xGroupSum is taken and not read (the kernels form the group sums of x themselves); rows defaults to what the plan's kernel
     /// implies (qwg_skinny_m2 / m3 -> 2 / 3, else 1), as the reference derives it.
     public static func encode(_ enc: QWHipEncoder, hal: QWHal, plan: QWGemmPlan, x: QWTensorValue, xGroupSum: QWTensorValue? = nil,
-                              wQ4: QWWeightView, y: QWTensorValue, rows rowsArg: Int? = nil, xIsRotated: Bool = true) throws {
+                              wQ4: QWWeightView, y: QWTensorValue, rows rowsArg: Int? = nil, xIsRotated: Bool = true,
+                              siluPairPlainOut: Bool = false) throws {
+        // siluPairPlainOut: .siluMulPair stores act in the plain basis; the next projection then rotates its input itself
+        // (xIsRotated: false there), free at one row, and the gate|up bank is read by the decode GEMV's own kernel.
         let rows = rowsArg ?? (plan.backend == .handQ4gSkinny ? (plan.kernel == "qwg_skinny_m3" ? 3 : 2) : 1)
         switch plan.backend {
         case .blocked:
@@ -226,7 +229,7 @@ public enum QWGemm {
         if plan.epilogue == .siluMulPair {
             guard wQ4.n % 2 == 0 else { throw QWGemmError.badWeights("silu_pair needs even N") }
             guard y.dtype == .f16, y.elementCount >= rows * (wQ4.n / 2) else { throw QWGemmError.badWeights("silu_pair output must be f16 [rows, N/2]") }
-            try qwCheck(qwhip_gemv_silu_pair(enc.stream, &w, x.ptr, x.dtype.rawValue, UInt32(rows), flags, 1, y.ptr))
+            try qwCheck(qwhip_gemv_silu_pair(enc.stream, &w, x.ptr, x.dtype.rawValue, UInt32(rows), flags, siluPairPlainOut ? 0 : 1, y.ptr))
             return
         }
         guard y.dtype == .f32, y.elementCount >= rows * wQ4.n else { throw QWGemmError.badWeights("output must be f32 [rows, N]") }

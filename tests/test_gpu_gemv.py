@@ -370,6 +370,47 @@ def test_gemv_silu_pair_matches_oracle(dev, fmt, flags, m, prerot, rot_out):
         b.free()
 
 
+@pytest.mark.parametrize("xdt", ["f16", "bf16"])
+@pytest.mark.parametrize("inter,k", [(160, 1536), (100, 5120), (777, 4096), (64, 12288), (2051, 2048)])
+@pytest.mark.parametrize("prerot", [False, True])
+def test_gemv_silu_pair_one_row_without_output_rotation(dev, inter, k, prerot, xdt):
+    """One activation row, no output rotation: the gate|up form of the decode GEMV's kernel (gate and up rows of a channel in
+    neighbouring row slots of one workgroup, the bank walked as two bands).  Against the oracle, and against the MoE decode
+    kernel on the same call (flags bits 8..11 = 3), which sums in another order: both within the bar of the reference and
+    within 1e-3 of each other.  Odd channel counts, channel counts below and above a workgroup's share, rows of 48 to 384
+    blocks, the rotation fused or the row handed over rotated, f16 and bf16 rows."""
+    fmt = "hq4_g32_m5"
+    blocks, w16 = H.make_bank(fmt, 2 * inter, k, seed=inter + k)
+    x32 = H.make_x(1, k, 7)
+    if xdt == "f16":
+        code, x16 = qwhip.F16, x32.astype(np.float16)
+        x_basis = H.x_in_basis(x16, fmt)                        # f16: what the fused rotation leaves, or what is handed over
+        xin = x_basis if prerot else x16
+    else:
+        code = qwhip.BF16
+        if prerot:                                              # the producer's rotation in fp32, one bf16 rounding
+            xin = qo.f32_to_bf16_bits(qo.fwht32_ortho(x32))
+            x_basis = qo.bf16_bits_to_f32(xin)
+        else:
+            xin = qo.f32_to_bf16_bits(x32)
+            x_basis = H.x_in_basis(qo.round_bf16(x32), fmt)
+    xb, bank = dev.put(xin), dev.put(blocks)
+    a1, a2 = dev.put(np.full(inter, 3, np.float16)), dev.put(np.full(inter, 5, np.float16))
+    view = H.view_of(dev, bank, fmt, 2 * inter, k)
+    fl = qwhip.X_PREROTATED if prerot else 0
+    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, code, 1, fl, 0, a1.ptr))
+    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, code, 1, fl | (3 << 8), 0, a2.ptr))
+    dev.stream.sync()
+    one = a1.download(np.float16, (1, inter)).astype(np.float32)
+    two = a2.download(np.float16, (1, inter)).astype(np.float32)
+    gu = qo.matmul_ref_f64(np.asarray(x_basis, np.float32).reshape(1, k), w16)
+    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=False).astype(np.float32)
+    assert qo.normalized_error(one, want) <= TOL and qo.normalized_error(two, want) <= TOL
+    assert qo.normalized_error(one, two) <= 1e-3
+    for b in (bank, xb, a1, a2):
+        b.free()
+
+
 def test_gemv_affine_known_answer(dev):
     """Code 1, scale 1.0, bias 0.25, x = one-hot: every output is exactly 1.25 - the -1024 must be
     stripped before the FMA, not folded into an f16 bias

@@ -85,7 +85,7 @@ def test_the_three_operator_doors_match_label_for_label():
     """QWGemm.encodeH16, QWGemmAQ.encode and QWMoEOperator.encodeResident: the reference's labels are a prefix-preserving
     subsequence, and what the shim adds comes after the last of them or is one of the rotation switches."""
     ref, shim = _load()
-    for name, extras in (("QWGemm.encodeH16", {"rows", "xIsRotated"}), ("QWGemm.encode", {"rows", "xIsRotated"}),
+    for name, extras in (("QWGemm.encodeH16", {"rows", "xIsRotated"}), ("QWGemm.encode", {"rows", "xIsRotated", "siluPairPlainOut"}),
                          ("QWGemmAQ.encode", {"isRotated", "xIsRotated"}), ("QWMoEOperator.encodeResident", set()),
                          ("QWMoEOperator.encodeResidentLatent", set()), ("QWMoEOperator.encodeResidentGroupLatent", set())):
         want = ref[name][0]
