@@ -1167,7 +1167,8 @@ def main() -> None:
     elif kind == "dense_f32":
         out = run_dense_f32(args, m, n, k, LABELS[args.workload])
     elif kind == "pair":
-        out = run_silu_pair(args, fmt, n, k, m, label)
+        rows = args.gemm_rows or m
+        out = run_silu_pair(args, fmt, n, k, rows, label + (f" [rows {rows}]" if args.gemm_rows else ""))
     elif kind == "gemm":
         if args.gemm_rows:
             m, traffic = args.gemm_rows, None

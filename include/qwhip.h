@@ -206,10 +206,13 @@ qwhip_status qwhip_gemv(qwhip_stream_t s, const qwhip_weight_view* w, const void
  * (qwgemm.metal:204-379; QWGemm.swift:137-283 epilogue .siluMulPair; EncodeKernels.swift:298-326).
  * w holds 2*inter rows: [0, inter) gate, [inter, 2*inter) up.  act16 f16 [m, inter] =
  * f16(FWHT32(silu(g)*u)) with SwiGLU on the fp32 accumulators; `rotate_out` = 0 stores it unrotated.
- * One row over an HQ4_G32_M5 bank with rotate_out = 0 is read by the decode GEMV's own kernel in a gate|up form (the bank
- * walked as two moving bands: 20.7 against 25.6 us on 2 x 17408 x 5120): a dense MLP decode step is fastest as this call
+ * One row is read by the one-row GEMV kernels in a gate|up form (the bank walked as two moving bands); with rotate_out the
+ * rotation is a second, small launch over fp32 gated values in the stream's scratch.  Without it the call is 2-3 us shorter
+ * (20.7 against 23.5 us on 2 x 17408 x 5120, HQ4_G32_M5): a dense MLP decode step is fastest as this call with rotate_out = 0
  * followed by qwhip_gemv on the down bank without QWHIP_X_PREROTATED, whose fused rotation costs nothing at one row.
- * flags bits 8..11 (tests): 2 = the general kernel, 3 = the MoE decode kernel also where the gate|up form would be taken. */
+ * Two to sixteen rows run qwhip_gemv over the whole bank into an fp32 image in the stream's scratch and qwhip_swiglu_fwht
+ * over that (calls on one stream are ordered; calls on different streams do not share the scratch).
+ * flags bits 8..11 (tests): 2 = the general kernel, 3 = HQ4_G32_M5 on the MoE decode kernel. */
 qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weight_view* w, const void* x, uint32_t x_dtype,
                                   uint32_t m, uint32_t flags, uint32_t rotate_out, void* act16);
 

@@ -1002,7 +1002,13 @@ bool qw_colx_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t 
 
 // gemv_col.hip
 bool qw_col_pair_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* act16,
-                      const qw_act ga, hipError_t* err);
+                      float* gated32, const qw_act ga, hipError_t* err);
+// gemv_colx.hip
+bool qw_colx_pair_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                       const void* x, uint32_t x_dtype, bool rotate, void* act16, float* gated32, const qw_act ga, hipError_t* err);
+extern "C" qwhip_status qwhip_fwht32(qwhip_stream_t s, const void* src, uint32_t src_dtype, void* dst_f16, uint64_t n);
+extern "C" qwhip_status qwhip_swiglu_fwht(qwhip_stream_t s, const void* gu, uint32_t gu_dtype, void* act_f16, uint32_t rows, uint32_t inter,
+                                          uint32_t rotate);
 bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* y16,
                  float* y32, uint32_t tune, hipError_t* err, unsigned long long* keys, uint32_t keys_cap, int32_t* token,
                  bool* folded);
@@ -1253,17 +1259,46 @@ extern "C" qwhip_status qwhip_gemv_silu_pair(qwhip_stream_t s, const qwhip_weigh
     if (w->n % 2 != 0) return qwhip_fail(QWHIP_E_BAD_WEIGHTS, "gate|up bank needs an even row count, got %u", w->n);
     const uint32_t inter = w->n / 2;
     const bool rotate = qwhip_view_rotated(w) && !(flags & QWHIP_X_PREROTATED);
-    // HQ4_G32_M5: the column-stationary gate|up kernel of the MoE decode path, as one dense bank with one "route" per
-    // activation row (flags bits 8..11 = 2 keep the general kernel, for tests).  One row without the output rotation takes the
-    // decode GEMV's own kernel in its gate|up form (bits 8..11 = 3 keep the MoE kernel): without the rotation a workgroup
-    // does not need 32 neighbouring channels and the bank is read as two moving bands.
-    if (fmt == QW_FMT_M5 && m == 1u && !(rotate_out && inter % 32 == 0) && ((flags >> 8) & 0xFu) == 0u) {
-        hipError_t e = hipSuccess;
-        if (qw_col_pair_gemv(s->stream, w, x, x_dtype, rotate, act16, s->dev->act, &e)) {
-            QWHIP_TRY_HIP(e);
-            return QWHIP_OK;
+    // One activation row: the one-row GEMV kernels in their gate|up form (gate and up row of a channel in neighbouring row
+    // slots of a workgroup, the bank read as two moving bands, the gated activation formed in the epilogue).  With the output
+    // rotation the launch leaves gated(g, u) as fp32 in the stream's scratch and the rotation kernel behind it rounds to f16
+    // once, as the fused epilogues do.  flags bits 8..11 (tests): 2 = the general kernel, 3 = HQ4_G32_M5 on the MoE decode kernel.
+    const bool rot_out = rotate_out && inter % 32 == 0;
+    if (m == 1u && ((flags >> 8) & 0xFu) == 0u) {
+        float* gated32 = nullptr;
+        if (rot_out) {
+            if (s->scratch && s->scratch_bytes >= QWHIP_STREAM_COUNTER_BYTES + (size_t)inter * 4u + QWHIP_STREAM_XROT_BYTES)
+                gated32 = (float*)(s->scratch + QWHIP_STREAM_COUNTER_BYTES);
+        }
+        if (!rot_out || gated32) {
+            hipError_t e = hipSuccess;
+            const bool took = fmt == QW_FMT_M5
+                                  ? qw_col_pair_gemv(s->stream, w, x, x_dtype, rotate, act16, gated32, s->dev->act, &e)
+                                  : qw_colx_pair_gemv(s->stream, w, fmt, log2_u32(w->group / 32), qwhip_view_block_bytes(w), qwhip_view_row_bytes(w), x,
+                                                      x_dtype, rotate, act16, gated32, s->dev->act, &e);
+            if (took) {
+                QWHIP_TRY_HIP(e);
+                return rot_out ? qwhip_fwht32(s, gated32, QWHIP_F32, act16, inter) : QWHIP_OK;
+            }
         }
     }
+    // Two to sixteen rows: the verify GEMV over the whole gate|up bank into an fp32 image [m, 2 I] at the top of the stream's
+    // partial-sum area, then the gated activation (+ rotation) pass over it - every weight is read once whatever m is (the MoE
+    // decode kernel reads the bank once per row: 40 / 70 / 125 us at m = 2 / 4 / 8 on 2 x 17408 x 5120).
+    if (m >= 2u && m <= 16u && ((flags >> 8) & 0xFu) == 0u && s->scratch && (!rot_out || ((uintptr_t)act16 & 15u) == 0)) {
+        const size_t need = (((size_t)m * w->n * 4u) + 255u) & ~(size_t)255u;
+        const size_t area = s->scratch_bytes - QWHIP_STREAM_COUNTER_BYTES - QWHIP_STREAM_XROT_BYTES;
+        if (need <= area / 2u) {
+            float* gu32 = (float*)(s->scratch + QWHIP_STREAM_COUNTER_BYTES + area - need);
+            s->scratch_reserved = need;
+            st = qw_gemv_impl(s, w, x, x_dtype, m, flags & (QWHIP_X_PREROTATED | QWHIP_GEMV_ROW_INVARIANT), nullptr, gu32, nullptr, nullptr);
+            s->scratch_reserved = 0;
+            if (st == QWHIP_OK) return qwhip_swiglu_fwht(s, gu32, QWHIP_F32, act16, m, inter, rot_out ? 1u : 0u);
+            if (st != QWHIP_E_BAD_GEOMETRY) return st;
+        }
+    }
+    // HQ4_G32_M5 (flags bits 8..11 = 3, or a shape the forms above do not take): the column-stationary gate|up kernel of the MoE
+    // decode path, as one dense bank with one "route" per activation row
     if (fmt == QW_FMT_M5 && ((flags >> 8) & 0xFu) != 2u) {
         hipError_t e = hipSuccess;
         if (qw_moe_gateup_col(s->stream, w, 1, x, x_dtype, rotate, rotate_out && inter % 32 == 0, nullptr, m, 1, act16, &e, s->dev->act)) {

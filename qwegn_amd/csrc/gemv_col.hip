@@ -204,7 +204,9 @@ static __device__ __forceinline__ void run(const P& pp) {
                 gsum += part[(2u * c) * cpr + k];
                 usum += part[(2u * c + 1u) * cpr + k];
             }
-            p.y16[c * G + blockIdx.x] = (h1_t)qw_gated(gsum, usum, pp.ga);
+            const float a = qw_gated(gsum, usum, pp.ga);
+            if (p.y32) p.y32[c * G + blockIdx.x] = a;         // fp32 for a rotation pass behind the launch
+            else p.y16[c * G + blockIdx.x] = (h1_t)a;
         }
         return;
     }
@@ -626,11 +628,11 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
 }
 
 // Gate|up form of the column-stationary kernel for one activation row over a validated HQ4_G32_M5 gate|up bank (n = 2 I rows):
-// act f16 [I] = gated(Wg . x, Wu . x) on the fp32 sums, no output rotation.  The workgroups walk the gate half and the up half
+// act f16 [I] = gated(Wg . x, Wu . x) on the fp32 sums, no output rotation (or the same as fp32 into gated32 [I]).  The workgroups walk the gate half and the up half
 // of the bank as two bands, like the decode GEMV walks its one.  false when the shape is outside the envelope (rows longer
 // than 12288 columns take one row set per workgroup, which cannot hold a gate and an up row side by side).
 bool qw_col_pair_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint32_t x_dtype, bool rotate, void* act16,
-                      const qw_act ga, hipError_t* err) {
+                      float* gated32, const qw_act ga, hipError_t* err) {
     if (w->kind != QWHIP_KIND_HQ4_G32_M5 || (w->n & 1u)) return false;
     const uint32_t nb = w->k / 32u, cpr = (nb + 31u) / 32u, inter = w->n / 2u;
     if (cpr > 12u || inter < 64u) return false;
@@ -649,7 +651,7 @@ bool qw_col_pair_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x,
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;
     p.y16 = (h1_t*)act16;
-    p.y32 = nullptr;
+    p.y32 = gated32;                                               // not NULL: gated(g, u) as fp32 [I] instead of act16
     p.N = w->n;
     p.nb = nb;
     p.cpr = cpr;

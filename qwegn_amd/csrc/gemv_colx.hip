@@ -35,6 +35,20 @@ namespace {
     X(const uint8_t*, bank) X(const void*, x) X(h1_t*, y16) X(float*, y32) X(uint32_t, N) X(uint32_t, K) X(uint32_t, M)         \
     X(uint32_t, nsl) X(uint32_t, cpr) X(uint32_t, sets) X(uint32_t, gshift) X(uint32_t, bb) X(uint32_t, row_bytes)
 QW_ARG_BLOCK(qcx_params, QCX_FIELDS)
+// The gate|up form (dense MLP decode, one activation row): the bank holds I gate rows and then the I up rows of the same
+// channels, N = 2 I; row slots 2 c and 2 c + 1 of a workgroup are the gate and the up row of its channel c (row sets of even
+// index walk the gate half of the bank, odd ones the up half), and the epilogue stores gated(g, u) on the fp32 sums:
+// f16 into y16 [I], or fp32 into y32 [I] for a rotation pass behind the launch.
+#define QCX_PAIR_FIELDS(X) QCX_FIELDS(X) X(qw_act, ga)
+QW_ARG_BLOCK(qcx_params_pair, QCX_PAIR_FIELDS)
+__device__ __forceinline__ const qcx_params& qcx_base(const qcx_params& p) { return p; }
+__device__ __forceinline__ qcx_params qcx_base(const qcx_params_pair& f) {
+    qcx_params p;
+#define QCX_TAKE(T, n) p.n = f.n;
+    QCX_FIELDS(QCX_TAKE)
+#undef QCX_TAKE
+    return p;
+}
 
 // payload dwords of one 32-column slice: bits * 32 / 32 (HQ4_G32_M5 and 4-bit streams: 4)
 template <int FMT>
@@ -119,11 +133,14 @@ __device__ __forceinline__ float qcx_operands(const h8_t* v, h2_t* xo) {
 // dynamic LDS = rows-per-workgroup * cpr * MR * 4 bytes (+ nsl * 80 bytes in front with ROT).
 // ROT (MR = 1 only): the activation row arrives un-rotated; the FWHT-32 of its groups runs on the matrix cores into
 // an LDS image (16 groups per wave and tile), and each lane then reads its own column from there.
-template <int FMT, int XDT, int MR, int D, int LB, bool ROT>
+template <int FMT, int XDT, int MR, int D, int LB, bool ROT, typename P = qcx_params>
 struct qw_gemv_colx_kernel {
 static constexpr int kLaunchBound = LB;
-static __device__ __forceinline__ void run(const qcx_params& p) {
+static __device__ __forceinline__ void run(const P& pp) {
+    constexpr bool PAIR = !std::is_same<P, qcx_params>::value;
+    const qcx_params& p = qcx_base(pp);
     static_assert(!ROT || MR == 1, "fused rotation is built for one activation row");
+    static_assert(!PAIR || MR == 1, "the gate|up form is built for one activation row");
     extern __shared__ h8_t qcx_lds[];
     h8_t* xs = qcx_lds;                                                     // ROT: 80 bytes per 32-group (64 used)
     float* qcx_part = (float*)(qcx_lds + (ROT ? (size_t)p.nsl * 5 : 0));    // [row slot][chunk][MR]
@@ -135,11 +152,27 @@ static __device__ __forceinline__ void run(const qcx_params& p) {
     const bool gvalid = g0 < p.nsl;
     const uint32_t g = gvalid ? g0 : p.nsl - 1u;
     const uint32_t G = gridDim.x;
-    if (blockIdx.x >= N) return;
-    const uint32_t nrows = (N - blockIdx.x + G - 1u) / G;   // row slots of this workgroup
-    const uint32_t nmax = (nrows + sets - 1u) / sets;       // trip count, uniform over the workgroup
-    const uint32_t step = G * sets * p.row_bytes;            // bytes between consecutive rows of one set
-    const uint32_t mine = nrows > set ? (nrows - set + sets - 1u) / sets : 0u;
+    uint32_t nrows, nmax, step, mine, first_row;
+    if constexpr (PAIR) {
+        // channel c of this workgroup is bank channel c G + blockIdx.x; set j walks the channels j / 2, + sets / 2, ... of half
+        // j & 1 (sets is even), so row slot trip * sets + j is (channel, half) = (slot / 2, slot & 1)
+        const uint32_t h2 = sets >> 1, I = N >> 1;
+        if (blockIdx.x >= I) return;
+        const uint32_t nch = (I - blockIdx.x + G - 1u) / G;
+        const uint32_t sub = set >> 1, half = set & 1u;
+        nrows = 2u * nch;
+        nmax = (nch + h2 - 1u) / h2;
+        step = G * h2 * p.row_bytes;
+        mine = nch > sub ? (nch - sub + h2 - 1u) / h2 : 0u;
+        first_row = half * I + (mine ? sub : 0u) * G + blockIdx.x;
+    } else {
+        if (blockIdx.x >= N) return;
+        nrows = (N - blockIdx.x + G - 1u) / G;               // row slots of this workgroup
+        nmax = (nrows + sets - 1u) / sets;                   // trip count, uniform over the workgroup
+        step = G * sets * p.row_bytes;                       // bytes between consecutive rows of one set
+        mine = nrows > set ? (nrows - set + sets - 1u) / sets : 0u;
+        first_row = (mine ? set : 0u) * G + blockIdx.x;
+    }
     uint32_t hdr_off, pay_off;
     if constexpr (FMT == QW_FMT_M5) {
         hdr_off = g * 20u;
@@ -148,7 +181,7 @@ static __device__ __forceinline__ void run(const qcx_params& p) {
         hdr_off = (g >> p.gshift) * p.bb;
         pay_off = hdr_off + 4u + (g & ((1u << p.gshift) - 1u)) * (4u * qcx_fmt<FMT>::PW);
     }
-    uint32_t off = ((mine ? set : 0u) * G + blockIdx.x) * p.row_bytes;
+    uint32_t off = first_row * p.row_bytes;
     const uint32_t off_max = off + (mine ? mine - 1u : 0u) * step;   // loads past the set's last row re-read it
 
     // 1. activation loads first (they return in order, ahead of the weight prefetch); rows past M re-read row M - 1
@@ -367,6 +400,23 @@ static __device__ __forceinline__ void run(const qcx_params& p) {
         }
     }
     __syncthreads();
+    if constexpr (PAIR) {
+        for (uint32_t c = tid; 2u * c < nrows; c += blockDim.x) {
+            float gsum = 0.f, usum = 0.f;
+            for (uint32_t k = 0; k < cpr; ++k) {
+                gsum += qcx_part[(2u * c) * cpr + k];
+                usum += qcx_part[(2u * c + 1u) * cpr + k];
+            }
+            if constexpr (FMT == QW_FMT_M5) {
+                gsum *= 16777216.0f;
+                usum *= 16777216.0f;
+            }
+            const float a = qw_gated(gsum, usum, pp.ga);
+            if (p.y32) p.y32[c * G + blockIdx.x] = a;
+            else p.y16[c * G + blockIdx.x] = (h1_t)a;
+        }
+        return;
+    }
     // 4. fixed-order sum of the chunk partials of each (row, activation row)
     for (uint32_t t = tid; t < nrows * p.M; t += blockDim.x) {
         const uint32_t m = t / nrows, s = t - m * nrows;
@@ -395,6 +445,63 @@ void qcx_launch_m(hipStream_t st, const qcx_params& p, uint32_t mr, bool rotate,
 }
 
 }  // namespace
+
+// Gate|up form of the column-stationary kernel for one activation row over a validated gate|up bank of n = 2 I rows (any
+// container the kernel takes): gated(Wg . x, Wu . x) on the fp32 sums, as f16 into act16 [I] or as fp32 into gated32 [I] (for a
+// rotation pass behind the launch).  false when the shape is outside the envelope.
+bool qw_colx_pair_gemv(hipStream_t st, const qwhip_weight_view* w, int fmt, uint32_t gshift, uint32_t bb, uint64_t row_bytes,
+                       const void* x, uint32_t x_dtype, bool rotate, void* act16, float* gated32, const qw_act ga, hipError_t* err) {
+    if (w->n & 1u) return false;
+    const uint32_t inter = w->n / 2u;
+    const uint32_t nsl = w->k / 32u, cpr = (nsl + 31u) / 32u;
+    if (64u * cpr > 1024u || inter < 64u) return false;               // two row sets at least
+    if ((uint64_t)w->n * row_bytes >= (1ull << 32)) return false;     // 32-bit offsets inside the bank
+    if (((uintptr_t)x & 15u) != 0) return false;
+    uint32_t sets = min(8u, max(2u, 512u / (32u * cpr))) & ~1u;       // even, at most eight waves a workgroup where two sets allow
+    const uint32_t h2 = sets / 2u;
+    const uint32_t threads = 32u * cpr * sets;
+    const uint32_t waves = (threads + 63u) / 64u;
+    uint32_t wgs = 256u * max(1u, (16u + waves / 2u) / waves);
+    wgs = min(wgs, max(1u, inter / h2));
+    const uint32_t ch_per_wg = qwhip_cdiv(inter, wgs);
+    if (rotate && (threads >> 6) * 5u * 16u < nsl) return false;      // rotation tiles: five per full wave
+    const size_t lds = (size_t)2u * ch_per_wg * cpr * 4u + (rotate ? (size_t)nsl * 80u : 0u);
+    if (lds > 60u * 1024u) return false;
+    qcx_params_pair p;
+    p.bank = (const uint8_t*)w->blocks;
+    p.x = x;
+    p.y16 = (h1_t*)act16;
+    p.y32 = gated32;
+    p.N = w->n;
+    p.K = w->k;
+    p.M = 1;
+    p.nsl = nsl;
+    p.cpr = cpr;
+    p.sets = sets;
+    p.gshift = gshift;
+    p.bb = bb;
+    p.row_bytes = (uint32_t)row_bytes;
+    p.ga = ga;
+#define QCX_PAIR(F, DT)                                                                                                         \
+    do {                                                                                                                        \
+        if (rotate) qw_launch_scalar<qw_gemv_colx_kernel<F, DT, 1, 2, 1024, true, qcx_params_pair>>(dim3(wgs), dim3(threads), lds, st, p);   \
+        else qw_launch_scalar<qw_gemv_colx_kernel<F, DT, 1, 2, 1024, false, qcx_params_pair>>(dim3(wgs), dim3(threads), lds, st, p);         \
+    } while (0)
+#define QCX_PAIR_F(DT)                                                  \
+    switch (fmt) {                                                      \
+        case QW_FMT_M5: QCX_PAIR(QW_FMT_M5, DT); break;                 \
+        case QW_FMT_B4: QCX_PAIR(QW_FMT_B4, DT); break;                 \
+        case QW_FMT_B8: QCX_PAIR(QW_FMT_B8, DT); break;                 \
+        case QW_FMT_B2: QCX_PAIR(QW_FMT_B2, DT); break;                 \
+        case QW_FMT_B3: QCX_PAIR(QW_FMT_B3, DT); break;                 \
+        default: QCX_PAIR(QW_FMT_B6, DT); break;                        \
+    }
+    if (x_dtype == QWHIP_F16) { QCX_PAIR_F(QWHIP_F16) } else { QCX_PAIR_F(QWHIP_BF16) }
+#undef QCX_PAIR_F
+#undef QCX_PAIR
+    *err = hipGetLastError();
+    return true;
+}
 
 // Tries the column-stationary small-M kernel for a validated call; false when the shape is outside its envelope:
 // up to eight activation rows already in the container's basis, or one row to rotate (`rotate`).

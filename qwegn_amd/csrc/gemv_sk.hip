@@ -315,7 +315,8 @@ bool qw_sk_gemv(qwhip_stream_t s, const qwhip_weight_view* w, int fmt, uint32_t 
     bands = min(bands, qwhip_cdiv(ntiles, waves));
     // partial sums live in the stream's scratch
     const uint64_t part_bytes = nkr > 1u ? (uint64_t)nkr * m * ntiles * 16u * 4u : 0u;
-    if (nkr > 1u && (!s->scratch || part_bytes > s->scratch_bytes - QWHIP_STREAM_COUNTER_BYTES - QWHIP_STREAM_XROT_BYTES)) return false;
+    if (nkr > 1u && (!s->scratch || part_bytes + s->scratch_reserved > s->scratch_bytes - QWHIP_STREAM_COUNTER_BYTES - QWHIP_STREAM_XROT_BYTES))
+        return false;
     qsk_params p;
     p.bank = (const uint8_t*)w->blocks;
     p.x = x;

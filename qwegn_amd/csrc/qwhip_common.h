@@ -34,6 +34,9 @@ struct qwhip_stream_s {
     hipStream_t stream;
     uint8_t* scratch;
     size_t scratch_bytes;
+    // bytes at the top of the partial-sum area that the running call keeps for itself (the gate|up door's fp32 image of a
+    // GEMV it launches): the split-K kernel places its partial sums below them.  Zero between calls.
+    size_t scratch_reserved = 0;
 };
 struct qwhip_event_s {
     qwhip_device_s* dev;

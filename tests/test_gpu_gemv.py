@@ -371,15 +371,17 @@ def test_gemv_silu_pair_matches_oracle(dev, fmt, flags, m, prerot, rot_out):
 
 
 @pytest.mark.parametrize("xdt", ["f16", "bf16"])
-@pytest.mark.parametrize("inter,k", [(160, 1536), (100, 5120), (777, 4096), (64, 12288), (2051, 2048)])
-@pytest.mark.parametrize("prerot", [False, True])
-def test_gemv_silu_pair_one_row_without_output_rotation(dev, inter, k, prerot, xdt):
-    """One activation row, no output rotation: the gate|up form of the decode GEMV's kernel (gate and up rows of a channel in
-    neighbouring row slots of one workgroup, the bank walked as two bands).  Against the oracle, and against the MoE decode
-    kernel on the same call (flags bits 8..11 = 3), which sums in another order: both within the bar of the reference and
-    within 1e-3 of each other.  Odd channel counts, channel counts below and above a workgroup's share, rows of 48 to 384
-    blocks, the rotation fused or the row handed over rotated, f16 and bf16 rows."""
-    fmt = "hq4_g32_m5"
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32", "aq2_g64", "hq3_g32", "aq6_g128"])
+@pytest.mark.parametrize("inter,k", [(160, 1536), (100, 5120), (777, 4096), (64, 12288), (2080, 2048)])
+@pytest.mark.parametrize("prerot,rot_out", [(False, 0), (True, 0), (True, 1)])
+def test_gemv_silu_pair_one_row_forms(dev, fmt, inter, k, prerot, rot_out, xdt):
+    """One activation row: the gate|up forms of the one-row GEMV kernels (gate and up rows of a channel in neighbouring row
+    slots of one workgroup, the bank walked as two bands; with the output rotation a rotation pass over the fp32 gated values
+    behind the launch).  Against the oracle, and against the kernel the door used before on the same call (flags bits 8..11:
+    3 = the MoE decode kernel for HQ4_G32_M5, 2 = the general kernel), which sums in another order: both within the bar of the
+    reference and within 1e-3 of each other.  Odd channel counts, channel counts below and above a workgroup's share, rows of
+    48 to 384 blocks, the input rotation fused or the row handed over rotated, f16 and bf16 rows."""
+    kind, bits, group, is_m5, rotated = H.FORMATS[fmt]
     blocks, w16 = H.make_bank(fmt, 2 * inter, k, seed=inter + k)
     x32 = H.make_x(1, k, 7)
     if xdt == "f16":
@@ -388,7 +390,7 @@ def test_gemv_silu_pair_one_row_without_output_rotation(dev, inter, k, prerot, x
         xin = x_basis if prerot else x16
     else:
         code = qwhip.BF16
-        if prerot:                                              # the producer's rotation in fp32, one bf16 rounding
+        if prerot and rotated:                                  # the producer's rotation in fp32, one bf16 rounding
             xin = qo.f32_to_bf16_bits(qo.fwht32_ortho(x32))
             x_basis = qo.bf16_bits_to_f32(xin)
         else:
@@ -398,13 +400,47 @@ def test_gemv_silu_pair_one_row_without_output_rotation(dev, inter, k, prerot, x
     a1, a2 = dev.put(np.full(inter, 3, np.float16)), dev.put(np.full(inter, 5, np.float16))
     view = H.view_of(dev, bank, fmt, 2 * inter, k)
     fl = qwhip.X_PREROTATED if prerot else 0
-    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, code, 1, fl, 0, a1.ptr))
-    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, code, 1, fl | (3 << 8), 0, a2.ptr))
+    before = (3 << 8) if is_m5 else (2 << 8)
+    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, code, 1, fl, rot_out, a1.ptr))
+    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, code, 1, fl | before, rot_out, a2.ptr))
     dev.stream.sync()
     one = a1.download(np.float16, (1, inter)).astype(np.float32)
     two = a2.download(np.float16, (1, inter)).astype(np.float32)
     gu = qo.matmul_ref_f64(np.asarray(x_basis, np.float32).reshape(1, k), w16)
-    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32), rotate=False).astype(np.float32)
+    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32),
+                              rotate=bool(rot_out) and inter % 32 == 0).astype(np.float32)
+    assert qo.normalized_error(one, want) <= TOL and qo.normalized_error(two, want) <= TOL
+    assert qo.normalized_error(one, two) <= 1e-3
+    for b in (bank, xb, a1, a2):
+        b.free()
+
+
+@pytest.mark.parametrize("fmt", ["hq4_g32_m5", "hq4_g64", "hq8_g32", "aq2_g64"])
+@pytest.mark.parametrize("m", [2, 5, 8, 16])
+@pytest.mark.parametrize("inter,k,prerot,rot_out", [(160, 1536, True, 1), (96, 17408, True, 1), (777, 4096, True, 0), (160, 1536, False, 1)])
+def test_gemv_silu_pair_several_rows_read_the_bank_once(dev, fmt, m, inter, k, prerot, rot_out):
+    """Two to sixteen rows: the verify GEMV over the whole gate|up bank into an fp32 image in the stream's scratch, then the
+    gated activation (+ rotation) pass.  Against the oracle and against the kernel the door used before (flags bits 8..11: 3 /
+    2).  K = 17408 sends the 4-bit banks through the split-K GEMV, whose partial sums share the scratch with the image."""
+    kind, bits, group, is_m5, rotated = H.FORMATS[fmt]
+    if not prerot and not rotated:
+        pytest.skip("plain container: nothing to rotate")
+    blocks, w16 = H.make_bank(fmt, 2 * inter, k, seed=inter + k + m)
+    x16 = H.make_x(m, k, 9).astype(np.float16)
+    x_basis = H.x_in_basis(x16, fmt)
+    xb, bank = dev.put(x_basis if prerot else x16), dev.put(blocks)
+    a1, a2 = dev.put(np.full((m, inter), 3, np.float16)), dev.put(np.full((m, inter), 5, np.float16))
+    view = H.view_of(dev, bank, fmt, 2 * inter, k)
+    fl = qwhip.X_PREROTATED if prerot else 0
+    before = (3 << 8) if is_m5 else (2 << 8)
+    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, m, fl, rot_out, a1.ptr))
+    qwhip.check(dev.lib.qwhip_gemv_silu_pair(dev.stream.handle, C.byref(view), xb.ptr, qwhip.F16, m, fl | before, rot_out, a2.ptr))
+    dev.stream.sync()
+    one = a1.download(np.float16, (m, inter)).astype(np.float32)
+    two = a2.download(np.float16, (m, inter)).astype(np.float32)
+    gu = qo.matmul_ref_f64(x_basis, w16)
+    want = qo.swiglu_fwht_f16(gu[:, :inter].astype(np.float32), gu[:, inter:].astype(np.float32),
+                              rotate=bool(rot_out) and inter % 32 == 0).astype(np.float32)
     assert qo.normalized_error(one, want) <= TOL and qo.normalized_error(two, want) <= TOL
     assert qo.normalized_error(one, two) <= 1e-3
     for b in (bank, xb, a1, a2):
