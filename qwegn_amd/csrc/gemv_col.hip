@@ -586,11 +586,16 @@ bool qw_col_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x, uint
     // 5).  Hand-issued window: 20 (10.8-10.9 us on 1024 workgroups; 11.4 on 512 with the same window, 11.1 on 768; deeper
     // windows 11.1-11.9, a window of two 11.3).  At least four rows per set, at most 128 row slots per workgroup.
     uint32_t wgs = (256u * (wdepth ? 20u : 10u) + waves / 2u) / waves;
+    // whole multiples of the 256 compute units: a grid that leaves some of them a workgroup more than the others was up to
+    // 19 % slower (5120 x 17408: 569 workgroups 13.6 us, 512 workgroups 11.2 us; K = 6144 .. 18432 5-10 %)
+    if (!(tune & 0x40u)) wgs = max(256u, (wgs + 128u) / 256u * 256u);   // tune bit 6 (tests): the unrounded grid
     if ((tune >> 3 & 3u) == 1u) wgs /= 2u;
     if ((tune >> 3 & 3u) == 2u) wgs *= 2u;
     if ((tune >> 3 & 3u) == 3u) wgs += wgs / 2u;
     wgs = min(wgs, max(1u, w->n / (sets * 4u)));
     wgs = max(wgs, qwhip_cdiv(w->n, 128u));
+    if (!(tune & 0x40u) && wgs > 256u && wgs % 256u != 0u && (wgs + 255u) / 256u * 256u <= max(1u, w->n / (sets * 4u)))
+        wgs = (wgs + 255u) / 256u * 256u;                          // the row-slot limit raised the grid: up to the next whole multiple
     const uint32_t rows_per_wg = qwhip_cdiv(w->n, wgs);
     // partial sums: one float per (row slot, chunk); the hand-issued window rounds the trip count up to whole groups and
     // stores every row slot of every group
@@ -642,6 +647,7 @@ bool qw_col_pair_gemv(hipStream_t st, const qwhip_weight_view* w, const void* x,
     const uint32_t threads = 32u * cpr * sets;
     const uint32_t waves = (threads + 63u) / 64u;
     uint32_t wgs = (256u * 10u + waves / 2u) / waves;              // ten waves per compute unit, as the compiled window of the GEMV
+    wgs = max(256u, (wgs + 128u) / 256u * 256u);                   // whole multiples of the compute units
     wgs = min(wgs, max(1u, inter / (h2 * 4u)));                    // at least four channels per set
     wgs = max(wgs, qwhip_cdiv(inter, 64u));                        // at most 128 row slots per workgroup
     const uint32_t ch_per_wg = qwhip_cdiv(inter, wgs);
