@@ -777,10 +777,13 @@ def run_gemm(args, fmt, n, k, m, label, traffic=None):
     if getattr(args, "vendor_gemm", False):
         # in a process of its own: PyTorch brings its own HIP runtime, which must not meet the one this library links
         import subprocess
-        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", "vendor_gemm", "--gemm-rows", str(m)],
-                               capture_output=True, text=True, timeout=600)
-        lines = [ln for ln in child.stdout.splitlines() if ln.startswith("{")]
-        out["roofline"]["vendor_plain_gemm"] = json.loads(lines[-1])["vendor_plain_gemm"] if child.returncode == 0 and lines else None
+        try:
+            child = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", "vendor_gemm", "--gemm-rows", str(m)],
+                                   capture_output=True, text=True, timeout=240)
+            lines = [ln for ln in child.stdout.splitlines() if ln.startswith("{")]
+            out["roofline"]["vendor_plain_gemm"] = json.loads(lines[-1])["vendor_plain_gemm"] if child.returncode == 0 and lines else None
+        except (subprocess.TimeoutExpired, OSError, ValueError, KeyError):
+            out["roofline"]["vendor_plain_gemm"] = None      # no PyTorch here, or it took too long: the yardstick is optional
     if not args.no_cpu:
         sample = min(m, 256)
         xs = qo.round_bf16(x32)[:sample].astype(np.float16)
@@ -1098,6 +1101,7 @@ def main() -> None:
                     help="workspace handed to qwhip_gemm in MiB (0 = the activation copy only; more lets small row counts split K)")
     ap.add_argument("--plain-out", action="store_true",
                     help="mlp_gate_up: no output rotation (act in the plain basis; the down projection then rotates its input itself)")
+    ap.add_argument("--no-vendor", action="store_true", help="headline: leave out the vendor library's plain GEMM beside the C3 figure")
     ap.add_argument("--vendor-gemm", action="store_true",
                     help="c3: also time the vendor library's plain f16 / bf16 GEMM of the same shape (needs PyTorch; a yardstick, not the product)")
     ap.add_argument("--prerot", action="store_true", help="hand the gemv activations already rotated")
@@ -1128,6 +1132,7 @@ def main() -> None:
         out = run_gemv(args, fmt, n, k, m, LABELS["c2"], outliers, measured_traffic("c2"), cpu_later=later)
         gargs = argparse.Namespace(**vars(args))
         gargs.steps, gargs.warmup, gargs.no_cpu = max(50, args.steps // 4), max(5, args.warmup // 2), True
+        gargs.vendor_gemm = not args.no_vendor      # the matrix-pipe yardstick beside the C3 figure (a child process, PyTorch only)
         kind, fmt, n, k, m, outliers = WORKLOADS["c3"]
         g = run_gemm(gargs, fmt, n, k, m, LABELS["c3"], measured_traffic("c3"))
         out["prefill_gemm"] = {"value": g["value"], "unit": g["unit"], "ms_per_step": g["ms_per_step"], "steps": g["steps"],
