@@ -294,10 +294,11 @@ def test_argmax_fold_key_rule(dev):
     """qwhip_argmax_f32 against the oracle's fold: ties to the lower row, NaN never wins, -0 < +0, infinities, rows whose
     length is not a multiple of four and rows that start unaligned."""
     rng = np.random.default_rng(8)
-    for rows, n in [(3, 151936), (5, 1001), (2, 7), (16, 4096)]:
+    for rows, n in [(3, 151936), (5, 1001), (2, 7), (16, 4096), (16, 40001), (17, 33000), (1, 32768)]:   # up to 16 long rows: split over 64 workgroups each
         logits = rng.standard_normal((rows, n)).astype(np.float32)
         logits[0, [n // 3, n // 2]] = 11.0
-        logits[1, n - 1] = np.nan
+        if rows > 1:
+            logits[1, n - 1] = np.nan
         if rows > 2:
             logits[2, :] = np.nan
         lb, tb = dev.put(logits), dev.alloc(max(256, rows * 4))
