@@ -779,7 +779,7 @@ def run_gemm(args, fmt, n, k, m, label, traffic=None):
         import subprocess
         try:
             child = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", "vendor_gemm", "--gemm-rows", str(m)],
-                                   capture_output=True, text=True, timeout=240)
+                                   capture_output=True, text=True, timeout=120)
             lines = [ln for ln in child.stdout.splitlines() if ln.startswith("{")]
             out["roofline"]["vendor_plain_gemm"] = json.loads(lines[-1])["vendor_plain_gemm"] if child.returncode == 0 and lines else None
         except (subprocess.TimeoutExpired, OSError, ValueError, KeyError):
